@@ -1,0 +1,255 @@
+/*
+ * mie.h -- C ABI of libmie_hip.so: masked incremental inference kernels for
+ * AMD MI355X (gfx950).
+ *
+ * Every entry point takes raw device pointers, plain integers and a HIP
+ * stream (passed as void* so that this header needs no HIP include), returns
+ * an int status (MIE_OK == 0, negative on error) and never allocates device
+ * memory, never synchronises with the host and never aborts.  After a
+ * negative status mie_last_error_string() describes the failure (thread
+ * local).  All launches are asynchronous on the given stream and contain no
+ * host-side read of device data (launch bounds come from capacities, kernels
+ * exit early on the device-side counts), so a sequence of calls can be
+ * captured in a HIP graph.
+ *
+ * Layouts.  Delta tensors and reservoirs are fp32 NHWC ("channels_last"):
+ * element (n, y, x, c) lives at ((n*H + y)*W + x)*C + c.  Pixel masks are
+ * uint8 [N, H, W] (1 = the pixel carries a delta).  Filters use the layout
+ * the reference extension takes, [Cin][K][K][Cout] (= weight.permute(1,2,3,0)
+ * of a torch OIHW weight; reference: ext/pointops/pointops_functional.py:13-14).
+ *
+ * Tiles.  The image plane is cut into 8x8 pixel tiles (the output tile of
+ * the reference 3x3 kernel, ext/pointops/_C_ext/pointops/ext_conv.cu:352);
+ * tile id = (n*tiles_y + ty)*tiles_x + tx.  A tile set (mie_tileset) lists
+ * the ids of the tiles that hold at least one active pixel, ascending.
+ *
+ * Clean-delta invariant.  Every delta buffer written by these kernels is
+ * exactly zero outside the active pixels of its tile set, so it can be used
+ * as a dense tensor by the caller.  To keep that invariant without touching
+ * the whole frame, mie_build_mask_tiles also lists the tiles that were
+ * active in the previous step and are not any more ("stale"); every kernel
+ * that writes a delta over a tile set zeroes the stale tiles.
+ */
+#ifndef MIE_H_
+#define MIE_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MIE_OK 0
+#define MIE_ERR_INVALID_ARG (-1)   /* null / misaligned pointer, bad size   */
+#define MIE_ERR_UNSUPPORTED (-2)   /* kernel size / stride / shape not built */
+#define MIE_ERR_CAPACITY (-3)      /* tile set too small for the geometry   */
+#define MIE_ERR_LAUNCH (-4)        /* HIP reported a launch failure         */
+
+#define MIE_TILE 8                 /* tile edge in pixels                   */
+
+/* activation kinds of mie_act_incr / fused conv epilogue */
+#define MIE_ACT_NONE 0
+#define MIE_ACT_RELU 1
+#define MIE_ACT_LEAKY_RELU 2
+#define MIE_ACT_SIGMOID 3
+#define MIE_ACT_TANH 4
+
+/* footprint kinds of mie_build_mask_tiles */
+#define MIE_FOOT_CONV 0    /* out(oy,ox) |= in(oy*s-p+ky, ox*s-p+kx)              */
+#define MIE_FOOT_UP2X 1    /* bilinear x2, align_corners=False, non-zero weights  */
+#define MIE_FOOT_TCONV 2   /* transposed conv: oy = iy*s - p + ky                 */
+
+/* conv code path selection */
+#define MIE_PATH_AUTO 0
+#define MIE_PATH_VALU 1
+#define MIE_PATH_MFMA 2
+
+/* flags of mie_act_incr / mie_mul_incr */
+#define MIE_FLAG_KEEP_RESERVOIR 1  /* compute the delta, leave reservoirs as is */
+
+/* counts[] slots of a tile set */
+#define MIE_CNT_ACTIVE 0
+#define MIE_CNT_STALE 1
+#define MIE_CNT_TICKET 2
+#define MIE_CNT_WORDS 4
+
+/*
+ * A tile set at resolution (n, h, w).  All pointers are device memory owned
+ * by the caller; capacity = mie_tile_capacity(n, h, w) entries.  Zero-fill
+ * counts[] and flags[] once before the first use (and again whenever the
+ * delta buffers written under this tile set are re-zeroed by the caller).
+ */
+typedef struct mie_tileset {
+  int32_t n, h, w;
+  uint8_t* pixmask;   /* [n*h*w]      1 = active pixel                        */
+  int32_t* tiles;     /* [capacity]   active tile ids, ascending              */
+  int32_t* stale;     /* [capacity]   tiles active last step, inactive now    */
+  int32_t* counts;    /* [MIE_CNT_WORDS] active, stale, ticket, reserved      */
+  uint32_t* flags;    /* [capacity]   1 = tile active (scratch of the build)  */
+} mie_tileset;
+
+/* Library version (major*10000 + minor*100 + patch). */
+int mie_version(void);
+
+/* Text of the last error on the calling thread ("" if none). */
+const char* mie_last_error_string(void);
+
+/* Number of 8x8 tiles of an (n, h, w) plane = capacity of its tile set. */
+int mie_tile_capacity(int n, int h, int w);
+
+/*
+ * pixmask[n,y,x] = any_c(|delta[n,y,x,c]| > threshold).
+ * Replaces: the reference's only mask definitions, max-pool of abs(x) against
+ * a threshold with field size 1 (incr_modules/utils.py:22-25,
+ * utils/str_sparse_utils.py:10-11); the dilation by the field is the
+ * MIE_FOOT_CONV footprint of mie_build_mask_tiles.
+ */
+int mie_mask_from_delta(const float* delta, int n, int h, int w, int c,
+                        float threshold, uint8_t* pixmask, void* stream);
+
+/*
+ * Build the output pixel mask and the ordered active-tile list of an op from
+ * the pixel mask(s) of its input(s).
+ *   in_mask / in_mask2: uint8 [n, h_in, w_in]; in_mask NULL = every input
+ *   pixel active; in_mask2 optional second input at the same resolution
+ *   (skip sum / concat), OR-ed with the first.
+ *   foot, k, stride, pad: footprint (MIE_FOOT_*); for MIE_FOOT_UP2X k, stride
+ *   and pad are ignored.  Output resolution is out->h, out->w.
+ * Writes out->pixmask (every pixel), out->flags, out->tiles (ascending ids),
+ * out->stale (tiles that were in out->tiles before this call and are not any
+ * more, ascending) and out->counts[ACTIVE, STALE].
+ * Replaces: the mask argument of conv{1,3,5,7}x*_increment_ext
+ * (ext/pointops/_C_ext/pointops/ops.cpp:27-48), which the reference kernel
+ * never reads (ext_conv.cu:74-76 synthesises a fake one).
+ */
+int mie_build_mask_tiles(const uint8_t* in_mask, const uint8_t* in_mask2,
+                         int h_in, int w_in, int foot, int k, int stride,
+                         int pad, const mie_tileset* out, void* stream);
+
+/*
+ * Masked convolution of a delta: for every active tile of `out`
+ *   acc = conv2d(x (++ x2), filter, bias = none, stride, pad)
+ * and then, with reservoir == NULL:      out_delta  = acc
+ *        with reservoir != NULL:          r0 = reservoir; r1 = r0 + acc;
+ *                                         reservoir = r1;
+ *                                         out_delta = act(r1) - act(r0)
+ * (the fused form of nnConvIncr followed by nnReservedActivation).
+ * Stale tiles of `out` are zeroed in out_delta.  Inactive input pixels are
+ * never read.
+ *   x  : [n, h_in, w_in, c1] delta with pixel mask xmask (NULL = all active),
+ *        feeds filter input channels [0, c1)
+ *   x2 : optional second input [n, h_in, w_in, c2] (NULL, c2 = 0 if absent),
+ *        feeds filter input channels [c1, c1 + c2) -- the concat-free form of
+ *        torch.cat((x, h), 1) in ConvLSTMIncr (incr_modules/e2depth_incr.py:100)
+ *   filter : [cin_total][k][k][cout], c1 + c2 <= cin_total
+ *   k in {1,3,5,7}, stride in {1,2}; out->h/w must equal (h_in+2*pad-k)/stride+1
+ * Replaces: conv{1,3,5,7}x*_increment_ext(x_incr, mask, filter, out_incr, stride)
+ * (ext/pointops/_C_ext/pointops/ops.cpp:51-114, include/ops.h:8-52) and the
+ * F.conv2d fallback the reference actually runs
+ * (incr_modules/mask_incr_modules.py:175-178).
+ */
+int mie_conv_masked(const float* x, const uint8_t* xmask, int c1,
+                    const float* x2, const uint8_t* x2mask, int c2,
+                    int h_in, int w_in, const float* filter, int cin_total,
+                    int k, int stride, int pad, int cout,
+                    const mie_tileset* out, float* out_delta,
+                    float* reservoir, int act_kind, float slope, int path,
+                    void* stream);
+
+/*
+ * Incremental point-wise non-linearity over the active tiles of ts:
+ *   r0 = reservoir; r1 = r0 + in_delta; out_delta = act(r1) - act(r0);
+ *   reservoir = r1   (in place)
+ * in_delta is read at the active pixels of ts->pixmask only.  If
+ * out_pixmask != NULL it receives the refined mask
+ *   out_pixmask = ts->pixmask & any_c(out_delta != 0)   (all n*h*w bytes of
+ * active and stale tiles are written; other tiles are left untouched, so
+ * zero-fill it once), else the input mask is passed through by the caller.
+ * flags & MIE_FLAG_KEEP_RESERVOIR: the reservoir is read only (the form of
+ * NonlinearPointOpIncr.forward without the accumulate).
+ * Replaces: activation_increment(X, in_incr, out_incr)
+ * (ext/pointops/_C_ext/pointops/ops.cpp:8-23, pointop_cuda.cu:17-52) and
+ * NonlinearPointOpIncr._nonlin + IncrementReserve.accumulate
+ * (incr_modules/mask_incr_modules.py:101-103,248-251).
+ */
+int mie_act_incr(int act_kind, float slope, const float* in_delta,
+                 float* reservoir, float* out_delta, int c,
+                 const mie_tileset* ts, uint8_t* out_pixmask, int flags,
+                 void* stream);
+
+/*
+ * Incremental point-wise product (product rule with cached operands):
+ *   out = (d2 + r2) * d1 + r1 * d2;  r1 += d1;  r2 += d2
+ * d1/d2 are read only where their pixel masks m1/m2 (NULL = all active) are
+ * set, ts must be built from the union of the two masks.
+ * flags & MIE_FLAG_KEEP_RESERVOIR: r1, r2 are read only (the bare
+ * IncrPointwiseMultiply of the reference).
+ * Replaces: IncrPointwiseMultiply + nnReservedMultiplication.forward
+ * (incr_modules/mask_incr_functional.py:52-54, mask_incr_modules.py:67-75).
+ */
+int mie_mul_incr(const float* d1, const uint8_t* m1, float* r1,
+                 const float* d2, const uint8_t* m2, float* r2,
+                 float* out_delta, int c, const mie_tileset* ts, int flags,
+                 void* stream);
+
+/*
+ * out = a + b over the active tiles of ts (built from the union of ma, mb).
+ * Replaces: the skip sum / residual sum on deltas
+ * (incr_modules/e2depth_incr.py:220,333).
+ */
+int mie_add_incr(const float* a, const uint8_t* ma, const float* b,
+                 const uint8_t* mb, float* out_delta, int c,
+                 const mie_tileset* ts, void* stream);
+
+/*
+ * Bilinear x2 up-sampling (align_corners = False) of a delta, optionally of
+ * the sum of two deltas: out = up2x(a + b).  `out` is the tile set at the
+ * output resolution (2*h_in, 2*w_in), built with MIE_FOOT_UP2X.
+ * Replaces: interpolate_from_module (incr_modules/mask_incr_functional.py:76-78)
+ * with the skip sum of UNetRecurrentIncr.forward folded in
+ * (incr_modules/e2depth_incr.py:429-431).
+ */
+int mie_upsample2x_incr(const float* a, const uint8_t* ma, const float* b,
+                        const uint8_t* mb, int h_in, int w_in, int c,
+                        const mie_tileset* out, float* out_delta, void* stream);
+
+/*
+ * Fused incremental ConvLSTM gate math for hidden size hid over the active
+ * tiles of ts.  gates_delta is [n,h,w,4*hid] in the reference chunk order
+ * [in, remember, out, cell] (incr_modules/e2depth_incr.py:103).  State kept
+ * by the caller (all [n,h,w,*] fp32, updated in place):
+ *   gates_res [4*hid]  pre-activation gate reservoirs
+ *   cprev_res [hid]    cached previous cell state (operand of m2)
+ *   cell_res  [hid]    cached new cell state (input of tanh2)
+ * cprev_delta (with mask cprev_mask) may be NULL = zero.  Computes, per
+ * element, exactly the chain sigmoid1..3/tanh1 -> m1 + m2 -> tanh2 -> m3 of
+ * ConvLSTMIncr.forward with post-activation operands recomputed from the
+ * pre-activation reservoirs, and writes h_delta, c_delta ([n,h,w,hid]).
+ * Replaces: incr_modules/e2depth_incr.py:103-120 (about 25 ATen launches).
+ */
+int mie_convlstm_gates_incr(const float* gates_delta, float* gates_res,
+                            const float* cprev_delta, const uint8_t* cprev_mask,
+                            float* cprev_res, float* cell_res, float* h_delta,
+                            float* c_delta, int hid, const mie_tileset* ts,
+                            void* stream);
+
+/*
+ * Masked transposed convolution of a delta (stride s, padding p; the output
+ * size out->h/w fixes output_padding): out(oy,ox,co) = sum x(iy,ix,ci) *
+ * filter[ci][ky][kx][co] over oy = iy*s - p + ky, ox = ix*s - p + kx, with
+ * the same reservoir/activation epilogue as mie_conv_masked.  filter is the
+ * torch ConvTranspose2d weight [Cin][Cout][K][K] permuted to [Cin][K][K][Cout].
+ * `out` must be built with MIE_FOOT_TCONV.
+ * Replaces: transposed_conv2d_from_module
+ * (incr_modules/mask_incr_functional.py:64-66).
+ */
+int mie_tconv_masked(const float* x, const uint8_t* xmask, int cin, int h_in,
+                     int w_in, const float* filter, int k, int stride, int pad,
+                     int cout, const mie_tileset* out, float* out_delta,
+                     float* reservoir, int act_kind, float slope, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MIE_H_ */

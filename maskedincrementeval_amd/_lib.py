@@ -1,0 +1,101 @@
+"""ctypes binding of libmie_hip.so (the C ABI declared in include/mie.h).
+
+The library is the only compute path of this package: there is no eager /
+CPU fallback.  If the shared object is missing, `lib()` raises.
+"""
+import ctypes
+import os
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG_DIR, "lib", "libmie_hip.so")
+
+MIE_OK = 0
+MIE_TILE = 8
+
+ACT_NONE, ACT_RELU, ACT_LEAKY_RELU, ACT_SIGMOID, ACT_TANH = 0, 1, 2, 3, 4
+FOOT_CONV, FOOT_UP2X, FOOT_TCONV = 0, 1, 2
+PATH_AUTO, PATH_VALU, PATH_MFMA = 0, 1, 2
+FLAG_KEEP_RESERVOIR = 1
+CNT_ACTIVE, CNT_STALE, CNT_TICKET, CNT_WORDS = 0, 1, 2, 4
+
+# every symbol include/mie.h declares
+EXPORTS = (
+    "mie_version", "mie_last_error_string", "mie_tile_capacity", "mie_mask_from_delta",
+    "mie_build_mask_tiles", "mie_conv_masked", "mie_act_incr", "mie_mul_incr", "mie_add_incr",
+    "mie_upsample2x_incr", "mie_convlstm_gates_incr", "mie_tconv_masked",
+)
+
+
+class MieTileSet(ctypes.Structure):
+    """struct mie_tileset of include/mie.h."""
+    _fields_ = [
+        ("n", ctypes.c_int32), ("h", ctypes.c_int32), ("w", ctypes.c_int32),
+        ("pixmask", ctypes.c_void_p), ("tiles", ctypes.c_void_p), ("stale", ctypes.c_void_p),
+        ("counts", ctypes.c_void_p), ("flags", ctypes.c_void_p),
+    ]
+
+
+class MieError(RuntimeError):
+    """A libmie_hip.so entry point returned a negative status."""
+
+    def __init__(self, code, message):
+        super().__init__("libmie_hip status %d: %s" % (code, message))
+        self.code = code
+
+
+_lib = None
+
+
+def _declare(l):
+    vp, ci, cf = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+    tsp = ctypes.POINTER(MieTileSet)
+    l.mie_version.restype = ci
+    l.mie_version.argtypes = []
+    l.mie_last_error_string.restype = ctypes.c_char_p
+    l.mie_last_error_string.argtypes = []
+    l.mie_tile_capacity.restype = ci
+    l.mie_tile_capacity.argtypes = [ci, ci, ci]
+    l.mie_mask_from_delta.restype = ci
+    l.mie_mask_from_delta.argtypes = [vp, ci, ci, ci, ci, cf, vp, vp]
+    l.mie_build_mask_tiles.restype = ci
+    l.mie_build_mask_tiles.argtypes = [vp, vp, ci, ci, ci, ci, ci, ci, tsp, vp]
+    l.mie_conv_masked.restype = ci
+    l.mie_conv_masked.argtypes = [vp, vp, ci, vp, vp, ci, ci, ci, vp, ci, ci, ci, ci, ci, tsp, vp,
+                                  vp, ci, cf, ci, vp]
+    l.mie_act_incr.restype = ci
+    l.mie_act_incr.argtypes = [ci, cf, vp, vp, vp, ci, tsp, vp, ci, vp]
+    l.mie_mul_incr.restype = ci
+    l.mie_mul_incr.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, tsp, ci, vp]
+    l.mie_add_incr.restype = ci
+    l.mie_add_incr.argtypes = [vp, vp, vp, vp, vp, ci, tsp, vp]
+    l.mie_upsample2x_incr.restype = ci
+    l.mie_upsample2x_incr.argtypes = [vp, vp, vp, vp, ci, ci, ci, tsp, vp, vp]
+    l.mie_convlstm_gates_incr.restype = ci
+    l.mie_convlstm_gates_incr.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, ci, tsp, vp]
+    l.mie_tconv_masked.restype = ci
+    l.mie_tconv_masked.argtypes = [vp, vp, ci, ci, ci, vp, ci, ci, ci, ci, tsp, vp, vp, ci, cf, vp]
+
+
+def lib():
+    """The loaded library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "libmie_hip.so not found at %s -- build it with "
+                "`python -m maskedincrementeval_amd.build` (there is no fallback path)" % LIB_PATH)
+        l = ctypes.CDLL(LIB_PATH)
+        _declare(l)
+        _lib = l
+    return _lib
+
+
+def check(status):
+    """Raise MieError for a negative status code."""
+    if status != MIE_OK:
+        msg = lib().mie_last_error_string()
+        raise MieError(status, msg.decode("utf-8", "replace") if msg else "")
+
+
+def tile_capacity(n, h, w):
+    return ((h + MIE_TILE - 1) // MIE_TILE) * ((w + MIE_TILE - 1) // MIE_TILE) * n

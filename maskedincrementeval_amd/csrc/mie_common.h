@@ -1,0 +1,104 @@
+// Shared host/device helpers of libmie_hip.so (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+// The C ABI is the only thing exported from the library.
+#pragma GCC visibility push(default)
+#include "../../include/mie.h"
+#pragma GCC visibility pop
+
+#define MIE_WAVE 64
+
+// ---- host side: error reporting -------------------------------------------
+void mie_set_error(const char* fmt, ...);
+void mie_clear_error();
+
+#define MIE_REQUIRE(cond, code, ...)        \
+  do {                                      \
+    if (!(cond)) {                          \
+      mie_set_error(__VA_ARGS__);           \
+      return (code);                        \
+    }                                       \
+  } while (0)
+
+// Status of the launch that was just enqueued.
+static inline int mie_check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    mie_set_error("%s: launch failed: %s", what, hipGetErrorString(e));
+    return MIE_ERR_LAUNCH;
+  }
+  return MIE_OK;
+}
+
+static inline bool mie_aligned(const void* p, size_t a) {
+  return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0;
+}
+
+// Validates the pointers and geometry of a tile set (host side only).
+int mie_check_tileset(const mie_tileset* ts, const char* who);
+
+static inline int mie_div_up(int a, int b) { return (a + b - 1) / b; }
+
+// ---- device side ------------------------------------------------------------
+// Plain-old-data view of a tile set passed to kernels by value.
+struct TileSetDev {
+  int n, h, w;
+  int tiles_y, tiles_x;
+  const uint8_t* pixmask;
+  const int32_t* tiles;
+  const int32_t* stale;
+  const int32_t* counts;
+};
+
+static inline TileSetDev mie_dev_tileset(const mie_tileset* ts) {
+  TileSetDev d;
+  d.n = ts->n; d.h = ts->h; d.w = ts->w;
+  d.tiles_y = mie_div_up(ts->h, MIE_TILE);
+  d.tiles_x = mie_div_up(ts->w, MIE_TILE);
+  d.pixmask = ts->pixmask; d.tiles = ts->tiles; d.stale = ts->stale;
+  d.counts = ts->counts;
+  return d;
+}
+
+// Which tile block `b` of a capacity-sized grid works on.
+//   returns 0: nothing to do (b beyond active + stale)
+//           1: active tile   2: stale tile (zero its delta)
+// (n, y0, x0) = batch index and top-left output pixel of the tile.
+__device__ __forceinline__ int mie_pick_tile(const TileSetDev& ts, int b,
+                                             int& n, int& y0, int& x0) {
+  const int n_active = ts.counts[MIE_CNT_ACTIVE];
+  const int n_stale = ts.counts[MIE_CNT_STALE];
+  int tile, kind;
+  if (b < n_active) {
+    tile = ts.tiles[b];
+    kind = 1;
+  } else if (b < n_active + n_stale) {
+    tile = ts.stale[b - n_active];
+    kind = 2;
+  } else {
+    return 0;
+  }
+  const int tx = tile % ts.tiles_x;
+  const int t2 = tile / ts.tiles_x;
+  const int ty = t2 % ts.tiles_y;
+  n = t2 / ts.tiles_y;
+  y0 = ty * MIE_TILE;
+  x0 = tx * MIE_TILE;
+  return kind;
+}
+
+__device__ __forceinline__ float mie_act(int kind, float slope, float v) {
+  switch (kind) {
+    case MIE_ACT_RELU: return v > 0.f ? v : 0.f;
+    // __fmul_rn: keep the product from being contracted into the caller's
+    // subtraction, so act(r1) - act(r0) rounds like two separate IEEE ops
+    case MIE_ACT_LEAKY_RELU: return v > 0.f ? v : __fmul_rn(v, slope);
+    case MIE_ACT_SIGMOID: return 1.f / (1.f + expf(-v));
+    case MIE_ACT_TANH: return tanhf(v);
+    default: return v;
+  }
+}

@@ -1,0 +1,271 @@
+// Pixel masks and ordered active-tile compaction (gfx950).
+//
+// mie_build_mask_tiles is one launch: every wave derives the 64 output-mask
+// bits of one 8x8 tile from the input mask footprint and records whether the
+// tile holds any active pixel (wave ballot); the block that finishes last
+// (ticket counter) turns the per-tile flags into the ascending tile list with
+// a ballot + popcount prefix scan, so the list order is deterministic and no
+// atomics touch the list itself.
+#include "mie_common.h"
+
+#include <string.h>
+
+// ---- error string -----------------------------------------------------------
+static thread_local char g_err[512] = "";
+
+void mie_set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+void mie_clear_error() { g_err[0] = 0; }
+
+extern "C" const char* mie_last_error_string(void) { return g_err; }
+extern "C" int mie_version(void) { return 100; }
+
+extern "C" int mie_tile_capacity(int n, int h, int w) {
+  if (n <= 0 || h <= 0 || w <= 0) return 0;
+  long long cap = (long long)n * mie_div_up(h, MIE_TILE) * mie_div_up(w, MIE_TILE);
+  if (cap > 0x3fffffff) return 0;
+  return (int)cap;
+}
+
+int mie_check_tileset(const mie_tileset* ts, const char* who) {
+  MIE_REQUIRE(ts != nullptr, MIE_ERR_INVALID_ARG, "%s: tile set is NULL", who);
+  MIE_REQUIRE(ts->n > 0 && ts->h > 0 && ts->w > 0, MIE_ERR_INVALID_ARG,
+              "%s: tile set geometry (%d,%d,%d) must be positive", who, ts->n, ts->h, ts->w);
+  MIE_REQUIRE(mie_tile_capacity(ts->n, ts->h, ts->w) > 0, MIE_ERR_CAPACITY,
+              "%s: tile set geometry (%d,%d,%d) too large", who, ts->n, ts->h, ts->w);
+  MIE_REQUIRE((long long)ts->n * ts->h * ts->w < 0x7fffffffLL, MIE_ERR_CAPACITY,
+              "%s: more than 2^31 pixels", who);
+  MIE_REQUIRE(ts->pixmask && ts->tiles && ts->stale && ts->counts && ts->flags,
+              MIE_ERR_INVALID_ARG, "%s: tile set has a NULL buffer", who);
+  MIE_REQUIRE(mie_aligned(ts->tiles, 4) && mie_aligned(ts->stale, 4) &&
+                  mie_aligned(ts->counts, 4) && mie_aligned(ts->flags, 4),
+              MIE_ERR_INVALID_ARG, "%s: tile set buffers must be 4-byte aligned", who);
+  return MIE_OK;
+}
+
+// ---- mask from delta ----------------------------------------------------------
+// One thread per pixel walks its channel vector; C is small (<= 1024) and the
+// vector is contiguous, float4 when the row is 16-byte aligned.
+__global__ __launch_bounds__(256) void k_mask_from_delta(
+    const float* __restrict__ delta, long long npix, int c, float thr,
+    uint8_t* __restrict__ pixmask) {
+  const long long p = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (p >= npix) return;
+  const float* row = delta + p * c;
+  int any = 0;
+  if ((c & 3) == 0) {
+    const float4* r4 = reinterpret_cast<const float4*>(row);
+    for (int i = 0; i < (c >> 2); ++i) {
+      const float4 v = r4[i];
+      any |= (fabsf(v.x) > thr) | (fabsf(v.y) > thr) | (fabsf(v.z) > thr) | (fabsf(v.w) > thr);
+    }
+  } else {
+    for (int i = 0; i < c; ++i) any |= (fabsf(row[i]) > thr);
+  }
+  pixmask[p] = (uint8_t)any;
+}
+
+extern "C" int mie_mask_from_delta(const float* delta, int n, int h, int w, int c,
+                                   float threshold, uint8_t* pixmask, void* stream) {
+  mie_clear_error();
+  MIE_REQUIRE(delta && pixmask, MIE_ERR_INVALID_ARG, "mie_mask_from_delta: NULL pointer");
+  MIE_REQUIRE(n > 0 && h > 0 && w > 0 && c > 0, MIE_ERR_INVALID_ARG,
+              "mie_mask_from_delta: sizes must be positive (n=%d h=%d w=%d c=%d)", n, h, w, c);
+  MIE_REQUIRE(threshold >= 0.f, MIE_ERR_INVALID_ARG, "mie_mask_from_delta: threshold < 0");
+  MIE_REQUIRE(mie_aligned(delta, 16), MIE_ERR_INVALID_ARG,
+              "mie_mask_from_delta: delta must be 16-byte aligned");
+  const long long npix = (long long)n * h * w;
+  MIE_REQUIRE(npix < 0x7fffffffLL, MIE_ERR_CAPACITY, "mie_mask_from_delta: too many pixels");
+  const unsigned blocks = (unsigned)((npix + 255) / 256);
+  hipLaunchKernelGGL(k_mask_from_delta, dim3(blocks), dim3(256), 0, (hipStream_t)stream,
+                     delta, npix, c, threshold, pixmask);
+  return mie_check_launch("mie_mask_from_delta");
+}
+
+// ---- footprint + tile flags + ordered compaction ----------------------------
+struct BuildArgs {
+  const uint8_t* in;
+  const uint8_t* in2;
+  int n, h_in, w_in;
+  int foot, k, s, p;
+  uint8_t* out;
+  int h_out, w_out, tiles_y, tiles_x, cap;
+  int32_t* tiles;
+  int32_t* stale;
+  int32_t* counts;
+  uint32_t* flags;
+};
+
+__device__ __forceinline__ int mask_at(const BuildArgs& a, int n, int iy, int ix) {
+  if (iy < 0 || iy >= a.h_in || ix < 0 || ix >= a.w_in) return 0;
+  const long long o = ((long long)n * a.h_in + iy) * a.w_in + ix;
+  int v = a.in[o];
+  if (a.in2) v |= a.in2[o];
+  return v != 0;
+}
+
+// Source index pair of bilinear x2 (align_corners = False) with non-zero weight.
+__device__ __forceinline__ void up2x_src(int o, int in_size, int& i0, int& i1) {
+  const int j = o >> 1;
+  if (o & 1) {
+    i0 = j;
+    i1 = (j + 1 < in_size) ? j + 1 : j;
+  } else {
+    i0 = (j > 0) ? j - 1 : 0;
+    i1 = j;
+  }
+}
+
+__device__ int footprint_bit(const BuildArgs& a, int n, int oy, int ox) {
+  if (a.in == nullptr) return 1;
+  int bit = 0;
+  if (a.foot == MIE_FOOT_CONV) {
+    const int iy0 = oy * a.s - a.p, ix0 = ox * a.s - a.p;
+    for (int ky = 0; ky < a.k; ++ky)
+      for (int kx = 0; kx < a.k; ++kx) bit |= mask_at(a, n, iy0 + ky, ix0 + kx);
+  } else if (a.foot == MIE_FOOT_UP2X) {
+    int r0, r1, c0, c1;
+    up2x_src(oy, a.h_in, r0, r1);
+    up2x_src(ox, a.w_in, c0, c1);
+    bit = mask_at(a, n, r0, c0) | mask_at(a, n, r0, c1) | mask_at(a, n, r1, c0) |
+          mask_at(a, n, r1, c1);
+  } else {  // MIE_FOOT_TCONV
+    for (int ky = 0; ky < a.k; ++ky) {
+      const int ty = oy + a.p - ky;
+      if (ty < 0 || (ty % a.s) != 0) continue;
+      for (int kx = 0; kx < a.k; ++kx) {
+        const int tx = ox + a.p - kx;
+        if (tx < 0 || (tx % a.s) != 0) continue;
+        bit |= mask_at(a, n, ty / a.s, tx / a.s);
+      }
+    }
+  }
+  return bit;
+}
+
+// Ordered compaction of the ids `id(i)` (i in [0, count)) for which keep(i)
+// holds, by the 256 threads of one block: per wave a ballot gives the 64
+// keep-bits, popcount below the lane gives the rank, the four wave totals are
+// exchanged through LDS and a running base carries across chunks.
+template <typename KeepFn, typename IdFn>
+__device__ int block_compact(int count, KeepFn keep, IdFn id, int32_t* dst, int* s_tot) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int base = 0;
+  for (int start = 0; start < count; start += 256) {
+    const int i = start + threadIdx.x;
+    const bool k = (i < count) && keep(i);
+    const unsigned long long bal = __ballot(k);
+    const int rank = __popcll(bal & ((1ull << lane) - 1ull));
+    if (lane == 0) s_tot[wave] = __popcll(bal);
+    __syncthreads();
+    int off = base;
+    for (int wv = 0; wv < wave; ++wv) off += s_tot[wv];
+    if (k) dst[off + rank] = id(i);
+    base += s_tot[0] + s_tot[1] + s_tot[2] + s_tot[3];
+    __syncthreads();
+  }
+  return base;
+}
+
+__global__ __launch_bounds__(256) void k_build_mask_tiles(BuildArgs a) {
+  __shared__ int s_last;
+  __shared__ int s_tot[4];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = blockIdx.x * 4 + wave;
+  if (tile < a.cap) {
+    const int tx = tile % a.tiles_x;
+    const int t2 = tile / a.tiles_x;
+    const int ty = t2 % a.tiles_y;
+    const int n = t2 / a.tiles_y;
+    const int oy = ty * MIE_TILE + (lane >> 3), ox = tx * MIE_TILE + (lane & 7);
+    int bit = 0;
+    if (oy < a.h_out && ox < a.w_out) {
+      bit = footprint_bit(a, n, oy, ox);
+      a.out[((long long)n * a.h_out + oy) * a.w_out + ox] = (uint8_t)bit;
+    }
+    const unsigned long long bal = __ballot(bit != 0);
+    if (lane == 0) a.flags[tile] = (bal != 0ull) ? 1u : 0u;
+  }
+  // Publish this block's flags, then take a ticket; the last block compacts.
+  __threadfence();
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const int t = atomicAdd(&a.counts[MIE_CNT_TICKET], 1);
+    s_last = (t == (int)gridDim.x - 1);
+  }
+  __syncthreads();
+  if (!s_last) return;
+  __threadfence();
+  const uint32_t* flags = a.flags;
+  auto flag_of = [&](int t) {
+    return __hip_atomic_load(&flags[t], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
+  };
+  // 1) stale = tiles of the previous list that are not active any more.
+  const int n_prev = a.counts[MIE_CNT_ACTIVE];
+  const int32_t* prev = a.tiles;
+  const int n_stale = block_compact(
+      n_prev, [&](int i) { return !flag_of(prev[i]); }, [&](int i) { return prev[i]; },
+      a.stale, s_tot);
+  __syncthreads();
+  // 2) new ascending active list.
+  const int n_act = block_compact(
+      a.cap, [&](int i) { return flag_of(i); }, [&](int i) { return i; }, a.tiles, s_tot);
+  if (threadIdx.x == 0) {
+    a.counts[MIE_CNT_ACTIVE] = n_act;
+    a.counts[MIE_CNT_STALE] = n_stale;
+    a.counts[MIE_CNT_TICKET] = 0;
+  }
+}
+
+extern "C" int mie_build_mask_tiles(const uint8_t* in_mask, const uint8_t* in_mask2,
+                                    int h_in, int w_in, int foot, int k, int stride,
+                                    int pad, const mie_tileset* out, void* stream) {
+  mie_clear_error();
+  int rc = mie_check_tileset(out, "mie_build_mask_tiles");
+  if (rc != MIE_OK) return rc;
+  MIE_REQUIRE(h_in > 0 && w_in > 0, MIE_ERR_INVALID_ARG,
+              "mie_build_mask_tiles: input size (%d,%d) must be positive", h_in, w_in);
+  MIE_REQUIRE(in_mask != nullptr || in_mask2 == nullptr, MIE_ERR_INVALID_ARG,
+              "mie_build_mask_tiles: in_mask2 given without in_mask");
+  MIE_REQUIRE((long long)out->n * h_in * w_in < 0x7fffffffLL, MIE_ERR_CAPACITY,
+              "mie_build_mask_tiles: more than 2^31 input pixels");
+  if (foot == MIE_FOOT_CONV) {
+    MIE_REQUIRE(k >= 1 && k <= 15 && stride >= 1 && stride <= 4 && pad >= 0 && pad < 16,
+                MIE_ERR_UNSUPPORTED, "mie_build_mask_tiles: conv footprint k=%d stride=%d pad=%d",
+                k, stride, pad);
+    const int ho = (h_in + 2 * pad - k) / stride + 1, wo = (w_in + 2 * pad - k) / stride + 1;
+    MIE_REQUIRE(h_in + 2 * pad >= k && w_in + 2 * pad >= k && ho == out->h && wo == out->w,
+                MIE_ERR_INVALID_ARG,
+                "mie_build_mask_tiles: conv output of (%d,%d) k=%d s=%d p=%d is (%d,%d), tile set is (%d,%d)",
+                h_in, w_in, k, stride, pad, ho, wo, out->h, out->w);
+  } else if (foot == MIE_FOOT_UP2X) {
+    MIE_REQUIRE(out->h == 2 * h_in && out->w == 2 * w_in, MIE_ERR_INVALID_ARG,
+                "mie_build_mask_tiles: up2x of (%d,%d) is not (%d,%d)", h_in, w_in, out->h, out->w);
+  } else if (foot == MIE_FOOT_TCONV) {
+    MIE_REQUIRE(k >= 1 && k <= 15 && stride >= 1 && stride <= 4 && pad >= 0 && pad < 16,
+                MIE_ERR_UNSUPPORTED, "mie_build_mask_tiles: tconv footprint k=%d stride=%d pad=%d",
+                k, stride, pad);
+    const int hmin = (h_in - 1) * stride - 2 * pad + k, wmin = (w_in - 1) * stride - 2 * pad + k;
+    MIE_REQUIRE(out->h >= hmin && out->h < hmin + stride && out->w >= wmin && out->w < wmin + stride,
+                MIE_ERR_INVALID_ARG,
+                "mie_build_mask_tiles: tconv output (%d,%d) not in [(%d,%d), +stride)", out->h,
+                out->w, hmin, wmin);
+  } else {
+    MIE_REQUIRE(false, MIE_ERR_UNSUPPORTED, "mie_build_mask_tiles: unknown footprint %d", foot);
+  }
+  BuildArgs a;
+  a.in = in_mask; a.in2 = in_mask2;
+  a.n = out->n; a.h_in = h_in; a.w_in = w_in;
+  a.foot = foot; a.k = k; a.s = stride; a.p = pad;
+  a.out = out->pixmask; a.h_out = out->h; a.w_out = out->w;
+  a.tiles_y = mie_div_up(out->h, MIE_TILE); a.tiles_x = mie_div_up(out->w, MIE_TILE);
+  a.cap = mie_tile_capacity(out->n, out->h, out->w);
+  a.tiles = out->tiles; a.stale = out->stale; a.counts = out->counts; a.flags = out->flags;
+  const unsigned blocks = (unsigned)mie_div_up(a.cap, 4);
+  hipLaunchKernelGGL(k_build_mask_tiles, dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
+  return mie_check_launch("mie_build_mask_tiles");
+}

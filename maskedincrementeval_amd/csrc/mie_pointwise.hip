@@ -1,0 +1,400 @@
+// Point-wise incremental kernels over active tiles (gfx950): activation
+// increment, product rule, sum, bilinear x2 up-sampling and the fused ConvLSTM
+// gate chain.  All of them are HBM-bound: one 256-thread block walks the
+// 64 pixels x C channels of one 8x8 tile with consecutive lanes on consecutive
+// channels of the NHWC row (float4 when C % 4 == 0), so a wave reads whole
+// 8-pixel rows of the tile as contiguous segments.
+#include "mie_common.h"
+
+namespace {
+
+template <int VEC> struct Vec;
+template <> struct Vec<4> {
+  float4 v;
+  __device__ static Vec load(const float* p) { Vec r; r.v = *reinterpret_cast<const float4*>(p); return r; }
+  __device__ void store(float* p) const { *reinterpret_cast<float4*>(p) = v; }
+  __device__ static Vec zero() { Vec r; r.v = make_float4(0.f, 0.f, 0.f, 0.f); return r; }
+  __device__ float& operator[](int i) { return (&v.x)[i]; }
+};
+template <> struct Vec<1> {
+  float v;
+  __device__ static Vec load(const float* p) { Vec r; r.v = *p; return r; }
+  __device__ void store(float* p) const { *p = v; }
+  __device__ static Vec zero() { Vec r; r.v = 0.f; return r; }
+  __device__ float& operator[](int) { return v; }
+};
+
+// Slot walker: calls f(px, pixoff, cq) for every in-bounds (pixel, channel
+// vector) slot of the tile; px in [0,64), pixoff = linear pixel index.
+template <typename F>
+__device__ __forceinline__ void for_tile_slots(const TileSetDev& ts, int n, int y0, int x0,
+                                               int cv, F f) {
+  const int total = 64 * cv;
+  for (int idx = threadIdx.x; idx < total; idx += 256) {
+    const int px = idx / cv, cq = idx - px * cv;
+    const int y = y0 + (px >> 3), x = x0 + (px & 7);
+    if (y >= ts.h || x >= ts.w) continue;
+    const long long pixoff = ((long long)n * ts.h + y) * ts.w + x;
+    f(px, pixoff, cq);
+  }
+}
+
+// ---- activation increment -----------------------------------------------------
+template <int VEC>
+__global__ __launch_bounds__(256) void k_act_incr(TileSetDev ts, int kind, float slope,
+                                                  const float* __restrict__ din,
+                                                  float* __restrict__ res,
+                                                  float* __restrict__ dout, int c,
+                                                  uint8_t* __restrict__ out_mask, int keep) {
+  __shared__ unsigned s_any[64];
+  int n, y0, x0;
+  const int tk = mie_pick_tile(ts, blockIdx.x, n, y0, x0);
+  if (tk == 0) return;
+  if (out_mask) {
+    if (threadIdx.x < 64) s_any[threadIdx.x] = 0u;
+    __syncthreads();
+  }
+  const int cv = c / VEC;
+  for_tile_slots(ts, n, y0, x0, cv, [&](int px, long long pixoff, int cq) {
+    const long long off = pixoff * c + (long long)cq * VEC;
+    Vec<VEC> o = Vec<VEC>::zero();
+    if (tk == 1 && ts.pixmask[pixoff]) {
+      Vec<VEC> d = Vec<VEC>::load(din + off);
+      Vec<VEC> r = Vec<VEC>::load(res + off);
+      unsigned nz = 0u;
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        const float r0 = r[i], r1 = r0 + d[i];
+        const float v = mie_act(kind, slope, r1) - mie_act(kind, slope, r0);
+        o[i] = v;
+        r[i] = r1;
+        nz |= (v != 0.f) ? 1u : 0u;
+      }
+      if (!keep) r.store(res + off);
+      if (out_mask && nz) atomicOr(&s_any[px], 1u);
+    }
+    o.store(dout + off);
+  });
+  if (out_mask) {
+    __syncthreads();
+    if (threadIdx.x < 64) {
+      const int px = threadIdx.x;
+      const int y = y0 + (px >> 3), x = x0 + (px & 7);
+      if (y < ts.h && x < ts.w) {
+        const long long pixoff = ((long long)n * ts.h + y) * ts.w + x;
+        out_mask[pixoff] = (uint8_t)((tk == 1 && s_any[px]) ? 1 : 0);
+      }
+    }
+  }
+}
+
+// ---- product rule ---------------------------------------------------------------
+template <int VEC>
+__global__ __launch_bounds__(256) void k_mul_incr(TileSetDev ts, const float* __restrict__ d1,
+                                                  const uint8_t* __restrict__ m1,
+                                                  float* __restrict__ r1,
+                                                  const float* __restrict__ d2,
+                                                  const uint8_t* __restrict__ m2,
+                                                  float* __restrict__ r2,
+                                                  float* __restrict__ dout, int c, int keep) {
+  int n, y0, x0;
+  const int tk = mie_pick_tile(ts, blockIdx.x, n, y0, x0);
+  if (tk == 0) return;
+  const int cv = c / VEC;
+  for_tile_slots(ts, n, y0, x0, cv, [&](int, long long pixoff, int cq) {
+    const long long off = pixoff * c + (long long)cq * VEC;
+    Vec<VEC> o = Vec<VEC>::zero();
+    if (tk == 1 && ts.pixmask[pixoff]) {
+      const bool a1 = (m1 == nullptr) || m1[pixoff];
+      const bool a2 = (m2 == nullptr) || m2[pixoff];
+      if (a1 || a2) {
+        Vec<VEC> x1 = a1 ? Vec<VEC>::load(d1 + off) : Vec<VEC>::zero();
+        Vec<VEC> x2 = a2 ? Vec<VEC>::load(d2 + off) : Vec<VEC>::zero();
+        Vec<VEC> q1 = Vec<VEC>::load(r1 + off);
+        Vec<VEC> q2 = Vec<VEC>::load(r2 + off);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+          o[i] = (x2[i] + q2[i]) * x1[i] + q1[i] * x2[i];
+          q1[i] += x1[i];
+          q2[i] += x2[i];
+        }
+        if (a1 && !keep) q1.store(r1 + off);
+        if (a2 && !keep) q2.store(r2 + off);
+      }
+    }
+    o.store(dout + off);
+  });
+}
+
+// ---- sum ----------------------------------------------------------------------------
+template <int VEC>
+__global__ __launch_bounds__(256) void k_add_incr(TileSetDev ts, const float* __restrict__ a,
+                                                  const uint8_t* __restrict__ ma,
+                                                  const float* __restrict__ b,
+                                                  const uint8_t* __restrict__ mb,
+                                                  float* __restrict__ dout, int c) {
+  int n, y0, x0;
+  const int tk = mie_pick_tile(ts, blockIdx.x, n, y0, x0);
+  if (tk == 0) return;
+  const int cv = c / VEC;
+  for_tile_slots(ts, n, y0, x0, cv, [&](int, long long pixoff, int cq) {
+    const long long off = pixoff * c + (long long)cq * VEC;
+    Vec<VEC> o = Vec<VEC>::zero();
+    if (tk == 1 && ts.pixmask[pixoff]) {
+      if (ma == nullptr || ma[pixoff]) o = Vec<VEC>::load(a + off);
+      if (mb == nullptr || mb[pixoff]) {
+        Vec<VEC> t = Vec<VEC>::load(b + off);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) o[i] += t[i];
+      }
+    }
+    o.store(dout + off);
+  });
+}
+
+// ---- bilinear x2 ------------------------------------------------------------------
+// Source rows/cols and weights of output index o (align_corners = False,
+// scale 2): src = max(0, o/2 - 0.25).
+__device__ __forceinline__ void up2x_coef(int o, int in_size, int& i0, int& i1, float& l0,
+                                          float& l1) {
+  const int j = o >> 1;
+  if (o & 1) {
+    i0 = j; i1 = (j + 1 < in_size) ? j + 1 : j; l0 = 0.75f; l1 = 0.25f;
+  } else if (j == 0) {
+    i0 = 0; i1 = (1 < in_size) ? 1 : 0; l0 = 1.f; l1 = 0.f;
+  } else {
+    i0 = j - 1; i1 = j; l0 = 0.25f; l1 = 0.75f;
+  }
+}
+
+template <int VEC>
+__global__ __launch_bounds__(256) void k_up2x_incr(TileSetDev ts, const float* __restrict__ a,
+                                                   const uint8_t* __restrict__ ma,
+                                                   const float* __restrict__ b,
+                                                   const uint8_t* __restrict__ mb, int h_in,
+                                                   int w_in, float* __restrict__ dout, int c) {
+  int n, y0, x0;
+  const int tk = mie_pick_tile(ts, blockIdx.x, n, y0, x0);
+  if (tk == 0) return;
+  const int cv = c / VEC;
+  for_tile_slots(ts, n, y0, x0, cv, [&](int px, long long pixoff, int cq) {
+    const long long off = pixoff * c + (long long)cq * VEC;
+    Vec<VEC> o = Vec<VEC>::zero();
+    if (tk == 1 && ts.pixmask[pixoff]) {
+      const int oy = y0 + (px >> 3), ox = x0 + (px & 7);
+      int r[2], q[2];
+      float lr[2], lq[2];
+      up2x_coef(oy, h_in, r[0], r[1], lr[0], lr[1]);
+      up2x_coef(ox, w_in, q[0], q[1], lq[0], lq[1]);
+      // value(i,j) = a + b at source (r[i], q[j]); combine as torch does:
+      // l_r0*(l_c0*v00 + l_c1*v01) + l_r1*(l_c0*v10 + l_c1*v11)
+      Vec<VEC> v[2][2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const long long so = ((long long)n * h_in + r[i]) * w_in + q[j];
+          Vec<VEC> t = Vec<VEC>::zero();
+          if (ma == nullptr || ma[so]) t = Vec<VEC>::load(a + so * c + (long long)cq * VEC);
+          if (b != nullptr && (mb == nullptr || mb[so])) {
+            Vec<VEC> u = Vec<VEC>::load(b + so * c + (long long)cq * VEC);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) t[e] += u[e];
+          }
+          v[i][j] = t;
+        }
+#pragma unroll
+      for (int e = 0; e < VEC; ++e)
+        o[e] = lr[0] * (lq[0] * v[0][0][e] + lq[1] * v[0][1][e]) +
+               lr[1] * (lq[0] * v[1][0][e] + lq[1] * v[1][1][e]);
+    }
+    o.store(dout + off);
+  });
+}
+
+// ---- fused ConvLSTM gates ------------------------------------------------------
+__device__ __forceinline__ float sigm(float v) { return 1.f / (1.f + expf(-v)); }
+
+template <int VEC>
+__global__ __launch_bounds__(256) void k_convlstm_gates(
+    TileSetDev ts, const float* __restrict__ dg, float* __restrict__ gres,
+    const float* __restrict__ dcp, const uint8_t* __restrict__ mcp, float* __restrict__ cpres,
+    float* __restrict__ cres, float* __restrict__ dh, float* __restrict__ dc, int hid) {
+  int n, y0, x0;
+  const int tk = mie_pick_tile(ts, blockIdx.x, n, y0, x0);
+  if (tk == 0) return;
+  const int cv = hid / VEC;
+  for_tile_slots(ts, n, y0, x0, cv, [&](int, long long pixoff, int cq) {
+    const long long off = pixoff * hid + (long long)cq * VEC;
+    Vec<VEC> oh = Vec<VEC>::zero(), oc = Vec<VEC>::zero();
+    if (tk == 1 && ts.pixmask[pixoff]) {
+      const long long goff = pixoff * 4 * hid + (long long)cq * VEC;
+      Vec<VEC> di = Vec<VEC>::load(dg + goff), ri = Vec<VEC>::load(gres + goff);
+      Vec<VEC> df = Vec<VEC>::load(dg + goff + hid), rf = Vec<VEC>::load(gres + goff + hid);
+      Vec<VEC> dO = Vec<VEC>::load(dg + goff + 2 * hid), ro = Vec<VEC>::load(gres + goff + 2 * hid);
+      Vec<VEC> dG = Vec<VEC>::load(dg + goff + 3 * hid), rg = Vec<VEC>::load(gres + goff + 3 * hid);
+      const bool has_cp = (dcp != nullptr) && (mcp == nullptr || mcp[pixoff]);
+      Vec<VEC> dP = has_cp ? Vec<VEC>::load(dcp + off) : Vec<VEC>::zero();
+      Vec<VEC> cp = Vec<VEC>::load(cpres + off);
+      Vec<VEC> cc = Vec<VEC>::load(cres + off);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        const float ri1 = ri[e] + di[e], rf1 = rf[e] + df[e];
+        const float ro1 = ro[e] + dO[e], rg1 = rg[e] + dG[e];
+        const float si0 = sigm(ri[e]), dsi = sigm(ri1) - si0;
+        const float sf0 = sigm(rf[e]), dsf = sigm(rf1) - sf0;
+        const float so0 = sigm(ro[e]), dso = sigm(ro1) - so0;
+        const float tg0 = tanhf(rg[e]), dtg = tanhf(rg1) - tg0;
+        // m1(in_gate, cell_gate) + m2(remember_gate, prev_c), product rule
+        const float m1 = (dtg + tg0) * dsi + si0 * dtg;
+        const float m2 = (dP[e] + cp[e]) * dsf + sf0 * dP[e];
+        const float dcell = m1 + m2;
+        const float c0 = cc[e], c1 = c0 + dcell;
+        const float tc0 = tanhf(c0), dtc = tanhf(c1) - tc0;
+        // m3(out_gate, tanh(cell))
+        oh[e] = (dtc + tc0) * dso + so0 * dtc;
+        oc[e] = dcell;
+        ri[e] = ri1; rf[e] = rf1; ro[e] = ro1; rg[e] = rg1;
+        cp[e] += dP[e];
+        cc[e] = c1;
+      }
+      ri.store(gres + goff); rf.store(gres + goff + hid);
+      ro.store(gres + goff + 2 * hid); rg.store(gres + goff + 3 * hid);
+      if (has_cp) cp.store(cpres + off);
+      cc.store(cres + off);
+    }
+    oh.store(dh + off);
+    oc.store(dc + off);
+  });
+}
+
+int check_pointwise(const char* who, const mie_tileset* ts, int c) {
+  int rc = mie_check_tileset(ts, who);
+  if (rc != MIE_OK) return rc;
+  MIE_REQUIRE(c > 0 && c <= 65536, MIE_ERR_INVALID_ARG, "%s: channel count %d out of range", who, c);
+  return MIE_OK;
+}
+
+#define MIE_PTR16(p, who, name) \
+  MIE_REQUIRE(mie_aligned((p), 16), MIE_ERR_INVALID_ARG, "%s: %s must be 16-byte aligned", who, name)
+
+}  // namespace
+
+extern "C" int mie_act_incr(int act_kind, float slope, const float* in_delta, float* reservoir,
+                            float* out_delta, int c, const mie_tileset* ts,
+                            uint8_t* out_pixmask, int flags, void* stream) {
+  mie_clear_error();
+  const char* who = "mie_act_incr";
+  int rc = check_pointwise(who, ts, c);
+  if (rc != MIE_OK) return rc;
+  MIE_REQUIRE(in_delta && reservoir && out_delta, MIE_ERR_INVALID_ARG, "%s: NULL pointer", who);
+  MIE_REQUIRE(act_kind >= MIE_ACT_NONE && act_kind <= MIE_ACT_TANH, MIE_ERR_UNSUPPORTED,
+              "%s: unknown activation %d", who, act_kind);
+  MIE_PTR16(in_delta, who, "in_delta"); MIE_PTR16(reservoir, who, "reservoir");
+  MIE_PTR16(out_delta, who, "out_delta");
+  const int keep = (flags & MIE_FLAG_KEEP_RESERVOIR) ? 1 : 0;
+  const TileSetDev d = mie_dev_tileset(ts);
+  const unsigned grid = (unsigned)mie_tile_capacity(ts->n, ts->h, ts->w);
+  if ((c & 3) == 0)
+    hipLaunchKernelGGL(k_act_incr<4>, dim3(grid), dim3(256), 0, (hipStream_t)stream, d, act_kind,
+                       slope, in_delta, reservoir, out_delta, c, out_pixmask, keep);
+  else
+    hipLaunchKernelGGL(k_act_incr<1>, dim3(grid), dim3(256), 0, (hipStream_t)stream, d, act_kind,
+                       slope, in_delta, reservoir, out_delta, c, out_pixmask, keep);
+  return mie_check_launch(who);
+}
+
+extern "C" int mie_mul_incr(const float* d1, const uint8_t* m1, float* r1, const float* d2,
+                            const uint8_t* m2, float* r2, float* out_delta, int c,
+                            const mie_tileset* ts, int flags, void* stream) {
+  mie_clear_error();
+  const char* who = "mie_mul_incr";
+  int rc = check_pointwise(who, ts, c);
+  if (rc != MIE_OK) return rc;
+  MIE_REQUIRE(d1 && r1 && d2 && r2 && out_delta, MIE_ERR_INVALID_ARG, "%s: NULL pointer", who);
+  MIE_PTR16(d1, who, "d1"); MIE_PTR16(r1, who, "r1"); MIE_PTR16(d2, who, "d2");
+  MIE_PTR16(r2, who, "r2"); MIE_PTR16(out_delta, who, "out_delta");
+  const int keep = (flags & MIE_FLAG_KEEP_RESERVOIR) ? 1 : 0;
+  const TileSetDev d = mie_dev_tileset(ts);
+  const unsigned grid = (unsigned)mie_tile_capacity(ts->n, ts->h, ts->w);
+  if ((c & 3) == 0)
+    hipLaunchKernelGGL(k_mul_incr<4>, dim3(grid), dim3(256), 0, (hipStream_t)stream, d, d1, m1, r1,
+                       d2, m2, r2, out_delta, c, keep);
+  else
+    hipLaunchKernelGGL(k_mul_incr<1>, dim3(grid), dim3(256), 0, (hipStream_t)stream, d, d1, m1, r1,
+                       d2, m2, r2, out_delta, c, keep);
+  return mie_check_launch(who);
+}
+
+extern "C" int mie_add_incr(const float* a, const uint8_t* ma, const float* b, const uint8_t* mb,
+                            float* out_delta, int c, const mie_tileset* ts, void* stream) {
+  mie_clear_error();
+  const char* who = "mie_add_incr";
+  int rc = check_pointwise(who, ts, c);
+  if (rc != MIE_OK) return rc;
+  MIE_REQUIRE(a && b && out_delta, MIE_ERR_INVALID_ARG, "%s: NULL pointer", who);
+  MIE_PTR16(a, who, "a"); MIE_PTR16(b, who, "b"); MIE_PTR16(out_delta, who, "out_delta");
+  const TileSetDev d = mie_dev_tileset(ts);
+  const unsigned grid = (unsigned)mie_tile_capacity(ts->n, ts->h, ts->w);
+  if ((c & 3) == 0)
+    hipLaunchKernelGGL(k_add_incr<4>, dim3(grid), dim3(256), 0, (hipStream_t)stream, d, a, ma, b,
+                       mb, out_delta, c);
+  else
+    hipLaunchKernelGGL(k_add_incr<1>, dim3(grid), dim3(256), 0, (hipStream_t)stream, d, a, ma, b,
+                       mb, out_delta, c);
+  return mie_check_launch(who);
+}
+
+extern "C" int mie_upsample2x_incr(const float* a, const uint8_t* ma, const float* b,
+                                   const uint8_t* mb, int h_in, int w_in, int c,
+                                   const mie_tileset* out, float* out_delta, void* stream) {
+  mie_clear_error();
+  const char* who = "mie_upsample2x_incr";
+  int rc = check_pointwise(who, out, c);
+  if (rc != MIE_OK) return rc;
+  MIE_REQUIRE(a && out_delta, MIE_ERR_INVALID_ARG, "%s: NULL pointer", who);
+  MIE_REQUIRE(b != nullptr || mb == nullptr, MIE_ERR_INVALID_ARG, "%s: mask of absent input b", who);
+  MIE_REQUIRE(h_in > 0 && w_in > 0 && out->h == 2 * h_in && out->w == 2 * w_in,
+              MIE_ERR_INVALID_ARG, "%s: output (%d,%d) is not twice the input (%d,%d)", who,
+              out->h, out->w, h_in, w_in);
+  MIE_PTR16(a, who, "a"); MIE_PTR16(b, who, "b"); MIE_PTR16(out_delta, who, "out_delta");
+  const TileSetDev d = mie_dev_tileset(out);
+  const unsigned grid = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
+  if ((c & 3) == 0)
+    hipLaunchKernelGGL(k_up2x_incr<4>, dim3(grid), dim3(256), 0, (hipStream_t)stream, d, a, ma, b,
+                       mb, h_in, w_in, out_delta, c);
+  else
+    hipLaunchKernelGGL(k_up2x_incr<1>, dim3(grid), dim3(256), 0, (hipStream_t)stream, d, a, ma, b,
+                       mb, h_in, w_in, out_delta, c);
+  return mie_check_launch(who);
+}
+
+extern "C" int mie_convlstm_gates_incr(const float* gates_delta, float* gates_res,
+                                       const float* cprev_delta, const uint8_t* cprev_mask,
+                                       float* cprev_res, float* cell_res, float* h_delta,
+                                       float* c_delta, int hid, const mie_tileset* ts,
+                                       void* stream) {
+  mie_clear_error();
+  const char* who = "mie_convlstm_gates_incr";
+  int rc = check_pointwise(who, ts, hid);
+  if (rc != MIE_OK) return rc;
+  MIE_REQUIRE(gates_delta && gates_res && cprev_res && cell_res && h_delta && c_delta,
+              MIE_ERR_INVALID_ARG, "%s: NULL pointer", who);
+  MIE_REQUIRE(cprev_delta != nullptr || cprev_mask == nullptr, MIE_ERR_INVALID_ARG,
+              "%s: mask of absent cprev_delta", who);
+  MIE_PTR16(gates_delta, who, "gates_delta"); MIE_PTR16(gates_res, who, "gates_res");
+  MIE_PTR16(cprev_delta, who, "cprev_delta"); MIE_PTR16(cprev_res, who, "cprev_res");
+  MIE_PTR16(cell_res, who, "cell_res"); MIE_PTR16(h_delta, who, "h_delta");
+  MIE_PTR16(c_delta, who, "c_delta");
+  const TileSetDev d = mie_dev_tileset(ts);
+  const unsigned grid = (unsigned)mie_tile_capacity(ts->n, ts->h, ts->w);
+  if ((hid & 3) == 0)
+    hipLaunchKernelGGL(k_convlstm_gates<4>, dim3(grid), dim3(256), 0, (hipStream_t)stream, d,
+                       gates_delta, gates_res, cprev_delta, cprev_mask, cprev_res, cell_res,
+                       h_delta, c_delta, hid);
+  else
+    hipLaunchKernelGGL(k_convlstm_gates<1>, dim3(grid), dim3(256), 0, (hipStream_t)stream, d,
+                       gates_delta, gates_res, cprev_delta, cprev_mask, cprev_res, cell_res,
+                       h_delta, c_delta, hid);
+  return mie_check_launch(who);
+}

@@ -1,0 +1,522 @@
+"""E2Depth / E2VID recurrent UNet in incremental form.
+
+Restates incr_modules/e2depth_incr.py of the reference on the masked kernels:
+same class names, constructor arguments, sub-module names (so state_dict keys
+match) and the forward / forward_refresh_reservoirs pair.  Differences that
+are deliberate:
+
+* conv + activation run as one kernel (`fuse=True`), the ConvLSTM gate chain
+  as one kernel (`fused=True`); the un-fused chains of the reference remain
+  available and are what the fused ones are tested against;
+* skip connections are mask-aware: the skip sum is folded into the bilinear
+  up-sampling kernel (reference :333,429-431 add the tensors);
+* three slips of the reference are not reproduced: `m1(...) + m2(...)`
+  concatenates two lists and drops the m2 term (:113), `self.norm ==
+  ['BN','IN']` is never true (:35), and the per-stage `print_sparsity` calls
+  (:404-437) synchronise with the host inside the hot loop.
+* `BaseE2VID` (an un-vendored dependency of the reference, :4) is replaced
+  by a plain config dict on `E2VIDRecurrentIncr`.
+"""
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import _lib, ops
+from .masked_types import DenseT, Masked, TileMask
+from .mask_incr_functional import IncrementReserve, _unpack
+from .mask_incr_modules import (_IncrBuffers, nnAddIncr, nnBatchNorm2dIncr, nnConvIncr,
+                                nnConvTranspose2dIncr, nnReluIncr, nnReservedActivation,
+                                nnReservedMultiplication, nnSigmoidIncr, nnTanhIncr,
+                                nnUpsample2xIncr, activation_kind)
+
+
+def _mask_of(x_incr):
+    return x_incr[1] if len(x_incr) > 1 else None
+
+
+class ConvLayerIncr(nn.Module):
+    """conv -> [BN] -> activation (reference :12-51)."""
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0,
+                 activation='relu', norm=None, fuse=True):
+        super().__init__()
+        bias = False if norm == 'BN' else True
+        self.conv2d = nnConvIncr(in_channels, out_channels, kernel_size, stride, padding, bias=bias)
+        if activation is not None:
+            op = getattr(torch, activation, 'relu')
+            self.activation = nnReservedActivation(op)
+        else:
+            self.activation = None
+        self.norm = norm
+        if norm == 'BN':
+            self.norm_layer = nnBatchNorm2dIncr(out_channels)
+        elif norm == 'IN':
+            raise NotImplementedError
+        self.fuse = fuse
+
+    def forward(self, x_incr: Masked, x2_incr: Masked = None) -> Masked:
+        if self.fuse and self.activation is not None and self.norm not in ['BN', 'IN']:
+            return self.conv2d.forward_fused(x_incr, self.activation, x2_incr)
+        out_incr = self.conv2d(x_incr, x2_incr)
+        if self.norm in ['BN', 'IN']:
+            out_incr = self.norm_layer(out_incr)
+        if self.activation is not None:
+            out_incr = self.activation(out_incr)
+        return out_incr
+
+    def forward_refresh_reservoirs(self, x: DenseT):
+        out = self.conv2d.forward_refresh_reservoirs(x)
+        if self.norm in ['BN', 'IN']:
+            out = self.norm_layer.forward_refresh_reservoirs(out)
+        if self.activation is not None:
+            out = self.activation.forward_refresh_reservoirs(out)
+        return out
+
+
+class ConvLSTMIncr(nn.Module, _IncrBuffers):
+    """Incremental ConvLSTM cell (reference :54-166).
+
+    fused=True keeps three reservoirs -- gate pre-activations (4*hid channels),
+    previous cell state, new cell state -- and runs the whole gate chain in
+    one kernel after the gates conv; the concat of (input, previous hidden) is
+    never formed (two-pointer conv input, and the hidden half is skipped when
+    no previous-state delta is given).  fused=False runs the reference chain
+    sigmoid1..3 / tanh1 / m1 / m2 / tanh2 / m3 module by module.
+    """
+
+    def __init__(self, input_size: int, hidden_size: int, kernel_size: int,
+                 prev_c_res: IncrementReserve = None, fused: bool = True):
+        super().__init__()
+        self.input_size = input_size
+        self.hidden_size = hidden_size
+        self.kernel_size = kernel_size
+        pad = kernel_size // 2
+        self.zero_tensors = {}
+        self.fused = fused
+        self.Gates = nnConvIncr(input_size + hidden_size, 4 * hidden_size, kernel_size, padding=pad)
+        self.m1 = nnReservedMultiplication()
+        self.m2 = nnReservedMultiplication()
+        self.m3 = nnReservedMultiplication()
+        self.sigmoid1 = nnSigmoidIncr()
+        self.sigmoid2 = nnSigmoidIncr()
+        self.sigmoid3 = nnSigmoidIncr()
+        self.tanh1 = nnTanhIncr()
+        self.tanh2 = nnTanhIncr()
+        self.add_cell = nnAddIncr()
+        # reservoirs of the fused chain
+        self.gates_res = IncrementReserve()
+        self.cprev_res = IncrementReserve()
+        self.cell_res = IncrementReserve()
+
+    def forward(self, input_incr: Masked, prev_state_incr):
+        prev_h_incr = prev_c_incr = None
+        if prev_state_incr is not None:
+            prev_h_incr, prev_c_incr = prev_state_incr
+            if _mask_of(prev_c_incr) is not _mask_of(prev_h_incr):
+                # the tile set of the gates conv must cover the cell delta too
+                prev_h_incr = [prev_h_incr[0], None]
+        if self.fused:
+            return self._forward_fused(input_incr, prev_h_incr, prev_c_incr)
+        return self._forward_chain(input_incr, prev_h_incr, prev_c_incr)
+
+    def _forward_fused(self, input_incr, prev_h_incr, prev_c_incr):
+        if self.gates_res.reservoir is None:
+            raise RuntimeError("ConvLSTMIncr: call forward_refresh_reservoirs first")
+        gates, ts = self.Gates(input_incr, prev_h_incr)
+        n, _, h, w = gates.shape
+        hid = self.hidden_size
+        dh = self._delta_buf("h", (n, hid, h, w), gates.device)
+        dc = self._delta_buf("c", (n, hid, h, w), gates.device)
+        cp = cpm = None
+        if prev_c_incr is not None:
+            cp, cpm, _ = _unpack(prev_c_incr)
+        ops.convlstm_gates_incr(gates, self.gates_res.reservoir, cp, cpm, self.cprev_res.reservoir,
+                                self.cell_res.reservoir, dh, dc, ts)
+        return [dh, ts], [dc, ts]
+
+    def _forward_chain(self, input_incr, prev_h_incr, prev_c_incr):
+        gates_incr = self.Gates(input_incr, prev_h_incr)
+        ts = gates_incr[1]
+        in_gate, remember_gate, out_gate, cell_gate = gates_incr[0].chunk(4, 1)
+        in_gate = self.sigmoid1([in_gate, ts])
+        remember_gate = self.sigmoid2([remember_gate, ts])
+        out_gate = self.sigmoid3([out_gate, ts])
+        cell_gate = self.tanh1([cell_gate, ts])
+        cell = self.m1(in_gate, cell_gate)
+        if prev_c_incr is None:
+            # d(f * c_prev) with dc_prev = 0 is df * c_prev: the product rule with a zero delta
+            zero = self._delta_buf("zero_c", tuple(cell[0].shape), cell[0].device)
+            prev_c_incr = [zero, remember_gate[1]]
+        cell = self.add_cell(cell, self.m2(remember_gate, prev_c_incr))
+        cell_tanh = self.tanh2(cell)
+        hidden = self.m3(out_gate, cell_tanh)
+        return hidden, cell
+
+    def forward_refresh_reservoirs(self, input_, prev_state):
+        batch_size = input_.data.size()[0]
+        spatial_size = input_.data.size()[2:]
+        if prev_state is None:
+            state_size = tuple([batch_size, self.hidden_size] + list(spatial_size))
+            if state_size not in self.zero_tensors:
+                self.zero_tensors[state_size] = (
+                    torch.zeros(state_size, device=input_.device).to(memory_format=torch.channels_last),
+                    torch.zeros(state_size, device=input_.device).to(memory_format=torch.channels_last))
+            prev_state = self.zero_tensors[tuple(state_size)]
+        prev_h, prev_c = prev_state
+        self._reset_incr()
+        stacked_inputs = torch.cat((input_, prev_h), 1)
+        gates = self.Gates.forward_refresh_reservoirs(stacked_inputs)
+        in_gate, remember_gate, out_gate, cell_gate = gates.chunk(4, 1)
+        if self.fused:
+            self.gates_res.update_reservoir(gates)
+            self.cprev_res.update_reservoir(prev_c)
+            in_gate, remember_gate = torch.sigmoid(in_gate), torch.sigmoid(remember_gate)
+            out_gate, cell_gate = torch.sigmoid(out_gate), torch.tanh(cell_gate)
+            cell = in_gate * cell_gate + remember_gate * prev_c
+            self.cell_res.update_reservoir(cell)
+            hidden = out_gate * torch.tanh(cell)
+            return hidden, cell
+        in_gate = self.sigmoid1.forward_refresh_reservoirs(in_gate)
+        remember_gate = self.sigmoid2.forward_refresh_reservoirs(remember_gate)
+        out_gate = self.sigmoid3.forward_refresh_reservoirs(out_gate)
+        cell_gate = self.tanh1.forward_refresh_reservoirs(cell_gate)
+        cell = self.m1.forward_refresh_reservoirs(in_gate, cell_gate) + \
+            self.m2.forward_refresh_reservoirs(remember_gate, prev_c)
+        self.add_cell.forward_refresh_reservoirs(cell, cell)
+        cell_tanh = self.tanh2.forward_refresh_reservoirs(cell)
+        hidden = self.m3.forward_refresh_reservoirs(out_gate, cell_tanh)
+        return hidden, cell
+
+
+class RecurrentConvLayerIncr(nn.Module):
+    """Reference :169-186."""
+
+    def __init__(self, in_channels, out_channels, kernel_size=3, stride=1, padding=0,
+                 recurrent_block_type='convlstm', activation='relu', norm=None, fuse=True):
+        super().__init__()
+        assert recurrent_block_type == 'convlstm'
+        self.conv = ConvLayerIncr(in_channels, out_channels, kernel_size, stride, padding,
+                                  activation, norm, fuse=fuse)
+        self.recurrent_block = ConvLSTMIncr(input_size=out_channels, hidden_size=out_channels,
+                                            kernel_size=3, fused=fuse)
+
+    def forward(self, x_incr, prev_state_incr):
+        x_incr = self.conv(x_incr)
+        state_incr = self.recurrent_block(x_incr, prev_state_incr)
+        x_incr = state_incr[0]
+        return x_incr, state_incr
+
+    def forward_refresh_reservoirs(self, x: DenseT, prev_state):
+        x = self.conv.forward_refresh_reservoirs(x)
+        state = self.recurrent_block.forward_refresh_reservoirs(x, prev_state)
+        x = state[0]
+        return x, state
+
+
+class ResidualBlockIncr(nn.Module):
+    """conv-relu-conv, + residual, relu (reference :189-240)."""
+
+    def __init__(self, in_channels, out_channels, stride=1, downsample=None, norm=None, fuse=True):
+        super().__init__()
+        bias = False if norm == 'BN' else True
+        self.conv1 = nnConvIncr(in_channels, out_channels, kernel_size=3, stride=stride, padding=1, bias=bias)
+        self.norm = norm
+        if norm == 'BN':
+            self.bn1 = nnBatchNorm2dIncr(out_channels)
+            self.bn2 = nnBatchNorm2dIncr(out_channels)
+        elif norm == 'IN':
+            raise NotImplementedError
+        self.relu1 = nnReluIncr()
+        self.conv2 = nnConvIncr(out_channels, out_channels, kernel_size=3, stride=1, padding=1, bias=bias)
+        self.relu2 = nnReluIncr()
+        self.downsample = downsample
+        self.add = nnAddIncr()
+        self.fuse = fuse
+
+    def forward(self, x_incr: Masked) -> Masked:
+        residual_incr = x_incr
+        if self.fuse and self.norm not in ['BN', 'IN']:
+            out_incr = self.conv1.forward_fused(x_incr, self.relu1)
+        else:
+            out_incr = self.conv1(x_incr)
+            if self.norm in ['BN', 'IN']:
+                out_incr = self.bn1(out_incr)
+            out_incr = self.relu1(out_incr)
+        out_incr = self.conv2(out_incr)
+        if self.norm in ['BN', 'IN']:
+            out_incr = self.bn2(out_incr)
+        if self.downsample:
+            residual_incr = self.downsample(x_incr)
+        out_incr = self.add(out_incr, residual_incr)
+        out_incr = self.relu2(out_incr)
+        return out_incr
+
+    def forward_refresh_reservoirs(self, x):
+        residual = x
+        out = self.conv1.forward_refresh_reservoirs(x)
+        if self.norm in ['BN', 'IN']:
+            out = self.bn1.forward_refresh_reservoirs(out)
+        out = self.relu1.forward_refresh_reservoirs(out)
+        out = self.conv2.forward_refresh_reservoirs(out)
+        if self.norm in ['BN', 'IN']:
+            out = self.bn2.forward_refresh_reservoirs(out)
+        if self.downsample:
+            residual = self.downsample.forward_refresh_reservoirs(x)
+        out = self.add.forward_refresh_reservoirs(out, residual)
+        out = self.relu2.forward_refresh_reservoirs(out)
+        return out
+
+
+class TransposedConvLayerIncr(nn.Module):
+    """Transposed conv (stride 2, output_padding 1) -> activation (reference :243-282)."""
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0,
+                 activation='relu', norm=None, fuse=True):
+        super().__init__()
+        bias = False if norm == 'BN' else True
+        self.transposed_conv2d = nnConvTranspose2dIncr(
+            in_channels, out_channels, kernel_size, stride=2, padding=padding, output_padding=1, bias=bias)
+        self.activation = None
+        if activation is not None:
+            op = getattr(torch, activation, 'relu')
+            self.activation = nnReservedActivation(op)
+        self.norm = norm
+        if norm == 'BN':
+            self.norm_layer = nnBatchNorm2dIncr(out_channels)
+        elif norm == 'IN':
+            raise NotImplementedError
+        self.add = nnAddIncr()
+        self.fuse = fuse
+
+    def forward(self, x_incr: Masked, skip_incr: Masked = None) -> Masked:
+        if skip_incr is not None:
+            x_incr = self.add(x_incr, skip_incr)
+        if self.fuse and self.activation is not None and self.norm not in ['BN', 'IN']:
+            kind, slope = activation_kind(self.activation.op)
+            return self.transposed_conv2d(x_incr, self.activation.in_res.reservoir, kind, slope)
+        out_incr = self.transposed_conv2d(x_incr)
+        if self.norm in ['BN', 'IN']:
+            out_incr = self.norm_layer(out_incr)
+        if self.activation is not None:
+            out_incr = self.activation(out_incr)
+        return out_incr
+
+    def forward_refresh_reservoirs(self, x, skip=None):
+        if skip is not None:
+            x = self.add.forward_refresh_reservoirs(x, skip)
+        out = self.transposed_conv2d.forward_refresh_reservoirs(x)
+        if self.norm in ['BN', 'IN']:
+            out = self.norm_layer.forward_refresh_reservoirs(out)
+        if self.activation is not None:
+            out = self.activation.forward_refresh_reservoirs(out)
+        return out
+
+
+class UpsampleConvLayerIncr(nn.Module):
+    """bilinear x2 -> conv -> activation (reference :284-322); the skip sum of the
+    UNet is taken inside the up-sampling kernel."""
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0,
+                 activation='relu', norm=None, fuse=True):
+        super().__init__()
+        bias = False if norm == 'BN' else True
+        self.conv2d = nnConvIncr(in_channels, out_channels, kernel_size, stride, padding, bias=bias)
+        if activation is not None:
+            op = getattr(torch, activation, 'relu')
+            self.activation = nnReservedActivation(op)
+        else:
+            self.activation = None
+        self.norm = norm
+        if norm == 'BN':
+            self.norm_layer = nnBatchNorm2dIncr(out_channels)
+        elif norm == 'IN':
+            raise NotImplementedError
+        self.upsample = nnUpsample2xIncr()
+        self.fuse = fuse
+
+    def forward(self, x_incr: Masked, skip_incr: Masked = None) -> Masked:
+        x_upsampled_incr = self.upsample(x_incr, skip_incr)
+        if self.fuse and self.activation is not None and self.norm not in ['BN', 'IN']:
+            return self.conv2d.forward_fused(x_upsampled_incr, self.activation)
+        out_incr = self.conv2d(x_upsampled_incr)
+        if self.norm in ['BN', 'IN']:
+            out_incr = self.norm_layer(out_incr)
+        if self.activation is not None:
+            out_incr = self.activation(out_incr)
+        return out_incr
+
+    def forward_refresh_reservoirs(self, x, skip=None):
+        x_upsampled = self.upsample.forward_refresh_reservoirs(x, skip)
+        out = self.conv2d.forward_refresh_reservoirs(x_upsampled)
+        if self.norm in ['BN', 'IN']:
+            out = self.norm_layer.forward_refresh_reservoirs(out)
+        if self.activation is not None:
+            out = self.activation.forward_refresh_reservoirs(out)
+        return out
+
+
+class BaseUNetIncr(nn.Module):
+    """Reference :325-377."""
+
+    def __init__(self, num_input_channels, num_output_channels=1, skip_type='sum', activation='sigmoid',
+                 num_encoders=4, base_num_channels=32, num_residual_blocks=2, norm=None,
+                 use_upsample_conv=True, fuse=True):
+        super().__init__()
+        self.num_input_channels = num_input_channels
+        self.num_output_channels = num_output_channels
+        self.skip_type = skip_type
+        if skip_type != 'sum':
+            raise NotImplementedError("E2Depth-incr is built with skip_type='sum'")
+        self.norm = norm
+        self.fuse = fuse
+        self.UpsampleLayer = UpsampleConvLayerIncr if use_upsample_conv else TransposedConvLayerIncr
+        self.num_encoders = num_encoders
+        self.base_num_channels = base_num_channels
+        self.num_residual_blocks = num_residual_blocks
+        self.max_num_channels = self.base_num_channels * pow(2, self.num_encoders)
+        assert self.num_input_channels > 0
+        assert self.num_output_channels > 0
+        self.encoder_input_sizes = [self.base_num_channels * pow(2, i) for i in range(self.num_encoders)]
+        self.encoder_output_sizes = [self.base_num_channels * pow(2, i + 1) for i in range(self.num_encoders)]
+        op = getattr(torch, activation, 'relu')
+        self.activation = nnReservedActivation(op)
+
+    def build_resblocks(self):
+        self.resblocks = nn.ModuleList()
+        for _ in range(self.num_residual_blocks):
+            self.resblocks.append(ResidualBlockIncr(self.max_num_channels, self.max_num_channels,
+                                                    norm=self.norm, fuse=self.fuse))
+
+    def build_decoders(self):
+        decoder_input_sizes = list(reversed([self.base_num_channels * pow(2, i + 1)
+                                             for i in range(self.num_encoders)]))
+        self.decoders = nn.ModuleList()
+        for input_size in decoder_input_sizes:
+            self.decoders.append(self.UpsampleLayer(input_size, input_size // 2, kernel_size=5,
+                                                    padding=2, norm=self.norm, fuse=self.fuse))
+
+    def build_prediction_layer(self):
+        self.pred = ConvLayerIncr(self.base_num_channels, self.num_output_channels, 1,
+                                  activation=None, norm=self.norm, fuse=self.fuse)
+        self.pred_add = nnAddIncr()
+
+
+class UNetRecurrentIncr(BaseUNetIncr):
+    """Recurrent UNet: head, stride-2 conv + ConvLSTM encoders, residual blocks,
+    up-sampling decoders with skip sums, 1x1 prediction + sigmoid (reference :380-468)."""
+
+    def __init__(self, num_input_channels, num_output_channels=1, skip_type='sum',
+                 recurrent_block_type='convlstm', activation='sigmoid', num_encoders=4,
+                 base_num_channels=32, num_residual_blocks=2, norm=None, use_upsample_conv=True,
+                 fuse=True):
+        super().__init__(num_input_channels, num_output_channels, skip_type, activation,
+                         num_encoders, base_num_channels, num_residual_blocks, norm,
+                         use_upsample_conv, fuse)
+        self.head = ConvLayerIncr(self.num_input_channels, self.base_num_channels,
+                                  kernel_size=5, stride=1, padding=2, fuse=fuse)
+        self.encoders = nn.ModuleList()
+        for input_size, output_size in zip(self.encoder_input_sizes, self.encoder_output_sizes):
+            self.encoders.append(RecurrentConvLayerIncr(input_size, output_size, kernel_size=5,
+                                                        stride=2, padding=2,
+                                                        recurrent_block_type=recurrent_block_type,
+                                                        norm=self.norm, fuse=fuse))
+        self.build_resblocks()
+        self.build_decoders()
+        self.build_prediction_layer()
+
+    def forward(self, x_incr: Masked, prev_states_incr):
+        x_incr = self.head(x_incr)
+        head = x_incr
+        if prev_states_incr is None:
+            prev_states_incr = [None] * self.num_encoders
+        blocks = []
+        states_incr = []
+        for i, encoder in enumerate(self.encoders):
+            x_incr, state_incr = encoder(x_incr, prev_states_incr[i])
+            blocks.append(x_incr)
+            states_incr.append(state_incr)
+        for resblock in self.resblocks:
+            x_incr = resblock(x_incr)
+        for i, decoder in enumerate(self.decoders):
+            x_incr = decoder(x_incr, blocks[self.num_encoders - i - 1])
+        pred_incr = self.pred(self.pred_add(x_incr, head))
+        pred_incr = self.activation(pred_incr)
+        return pred_incr, states_incr
+
+    def forward_refresh_reservoirs(self, x: DenseT, prev_states):
+        x = self.head.forward_refresh_reservoirs(x)
+        head = x
+        if prev_states is None:
+            prev_states = [None] * self.num_encoders
+        blocks = []
+        states = []
+        for i, encoder in enumerate(self.encoders):
+            x, state = encoder.forward_refresh_reservoirs(x, prev_states[i])
+            blocks.append(x)
+            states.append(state)
+        for resblock in self.resblocks:
+            x = resblock.forward_refresh_reservoirs(x)
+        for i, decoder in enumerate(self.decoders):
+            x = decoder.forward_refresh_reservoirs(x, blocks[self.num_encoders - i - 1])
+        pred = self.pred.forward_refresh_reservoirs(self.pred_add.forward_refresh_reservoirs(x, head))
+        pred = self.activation.forward_refresh_reservoirs(pred)
+        return pred, states
+
+
+E2DEPTH_DEFAULT_CONFIG = dict(num_bins=5, skip_type='sum', num_encoders=3, base_num_channels=32,
+                              num_residual_blocks=2, norm=None, use_upsample_conv=True,
+                              recurrent_block_type='convlstm')
+
+
+class E2VIDRecurrentIncr(nn.Module, _IncrBuffers):
+    """E2Depth-incr / E2VID-incr (reference :471-498).
+
+    `config` is a dict (keys of E2DEPTH_DEFAULT_CONFIG; missing keys take the
+    defaults, which give the network traced in the reference's todo.txt:34-57).
+    When the input pair carries no mask (the reference drivers pass
+    `(x_t - x_{t-1}, None)`), the pixel mask is derived on the device as
+    any_c(|delta| > mask_threshold).
+    """
+
+    def __init__(self, config=None, fuse=True, mask_threshold: float = 0.0, derive_input_mask=True):
+        super().__init__()
+        cfg = dict(E2DEPTH_DEFAULT_CONFIG)
+        cfg.update(config or {})
+        self.num_bins = int(cfg['num_bins'])
+        self.skip_type = str(cfg['skip_type'])
+        self.num_encoders = int(cfg['num_encoders'])
+        self.base_num_channels = int(cfg['base_num_channels'])
+        self.num_residual_blocks = int(cfg['num_residual_blocks'])
+        self.norm = cfg['norm']
+        self.use_upsample_conv = bool(cfg['use_upsample_conv'])
+        self.recurrent_block_type = str(cfg['recurrent_block_type'])
+        self.mask_threshold = float(mask_threshold)
+        self.derive_input_mask = derive_input_mask
+        self.unetrecurrent = UNetRecurrentIncr(num_input_channels=self.num_bins,
+                                               num_output_channels=1,
+                                               skip_type=self.skip_type,
+                                               recurrent_block_type=self.recurrent_block_type,
+                                               activation='sigmoid',
+                                               num_encoders=self.num_encoders,
+                                               base_num_channels=self.base_num_channels,
+                                               num_residual_blocks=self.num_residual_blocks,
+                                               norm=self.norm,
+                                               use_upsample_conv=self.use_upsample_conv,
+                                               fuse=fuse)
+
+    def input_mask(self, delta: torch.Tensor) -> torch.Tensor:
+        n, _, h, w = delta.shape
+        pix = self._pix_buf("input", n, h, w, delta.device)
+        return ops.mask_from_delta(delta, self.mask_threshold, pix)
+
+    def forward(self, event_tensor: Masked, prev_states):
+        delta = ops.as_nhwc(event_tensor[0])
+        mask = _mask_of(event_tensor)
+        if mask is None and self.derive_input_mask:
+            mask = self.input_mask(delta)
+        img_pred, states = self.unetrecurrent.forward([delta, mask], prev_states)
+        return img_pred, states
+
+    def forward_refresh_reservoirs(self, event_tensor: DenseT, prev_states):
+        img_pred, states = self.unetrecurrent.forward_refresh_reservoirs(event_tensor, prev_states)
+        return img_pred, states

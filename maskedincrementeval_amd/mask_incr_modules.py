@@ -1,0 +1,493 @@
+"""nn.Module surface of the incremental layers.
+
+Drop-in for incr_modules/mask_incr_modules.py of the reference: same class
+names, constructor signatures and the two-forward protocol
+
+    forward(x_incr: Masked) -> Masked          incremental step on [delta, mask]
+    forward_refresh_reservoirs(x) -> dense     dense pass that (re)fills reservoirs
+
+(reference :13-17).  The incremental forwards run the masked HIP kernels of
+libmie_hip.so on persistent per-module buffers; the mask slot of the result
+is a `TileMask`.  The dense refresh uses torch ops on the GPU (it runs once
+every 20-100 frames in the reference drivers).
+"""
+import functools
+from typing import Tuple
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import _lib, ops
+from .masked_types import DenseT, Masked, TileMask
+from .mask_incr_functional import (IncrPointwiseMultiply, IncrementReserve, _square, _unpack,
+                                   bn2d_from_module, conv2d_from_module)
+
+
+class _IncrBuffers:
+    """Persistent per-module device buffers of the incremental path.
+
+    Deltas written by the kernels live in fixed buffers (stable pointers, zero
+    outside the active tiles); `_reset_incr` returns them to the all-zero state
+    a dense refresh implies.
+    """
+
+    def _ib(self):
+        d = self.__dict__.get("_incr_bufs")
+        if d is None:
+            d = {}
+            self.__dict__["_incr_bufs"] = d
+        return d
+
+    def _delta_buf(self, name, shape, device) -> torch.Tensor:
+        key = ("d", name, tuple(shape), str(device))
+        b = self._ib().get(key)
+        if b is None:
+            b = ops.new_nhwc(*shape, device)
+            self._ib()[key] = b
+        return b
+
+    def _tile_set(self, name, n, h, w, device) -> TileMask:
+        key = ("t", name, (n, h, w), str(device))
+        b = self._ib().get(key)
+        if b is None:
+            b = TileMask(n, h, w, device)
+            self._ib()[key] = b
+        return b
+
+    def _pix_buf(self, name, n, h, w, device) -> torch.Tensor:
+        key = ("p", name, (n, h, w), str(device))
+        b = self._ib().get(key)
+        if b is None:
+            b = torch.zeros((n, 1, h, w), dtype=torch.uint8, device=device)
+            self._ib()[key] = b
+        return b
+
+    def _view(self, name, parent: TileMask, pix: torch.Tensor) -> TileMask:
+        key = ("v", name, parent.tiles.data_ptr(), pix.data_ptr())
+        b = self._ib().get(key)
+        if b is None:
+            b = parent.with_pixmask(pix)
+            self._ib()[key] = b
+        return b
+
+    def _reset_incr(self):
+        for key, b in self._ib().items():
+            if key[0] in ("d", "p"):
+                b.zero_()
+            elif key[0] == "t":
+                b.reset()
+
+
+# input output increments: interface for incremental modules
+class IncrementMaskModule(nn.Module, _IncrBuffers):
+
+    def forward_refresh_reservoirs(self, x: DenseT) -> DenseT:
+        return x
+
+
+class KFencedMaskModule(IncrementMaskModule):
+    """Delta quantiser: lets multiples of k through, carries the rest (reference :21-47).
+
+    T = Rd + d;  f = k * floor(0.5 + T / k);  Rd = T - f;  returns [f, None].
+    The reference instantiates it in every nnConvIncr but never calls its
+    forward; it is kept as torch ops on the device.
+    """
+
+    def __init__(self, tp: float = .1):
+        super().__init__()
+        self.delta = IncrementReserve()
+        self.tp = tp
+        self.k = tp
+
+    def floor_by_k(self, T):
+        return self.k * torch.floor(0.5 + T / self.k)
+
+    def forward(self, incr: Masked) -> Masked:
+        T1 = self.delta.reservoir + incr[0]
+        f_delta = self.floor_by_k(T1)
+        self.delta.update_reservoir(T1 - f_delta)
+        return f_delta, None
+
+    def forward_refresh_reservoirs(self, x: DenseT) -> DenseT:
+        self.k = self.tp * torch.norm(x)
+        self.delta.update_reservoir(torch.zeros_like(x))
+        return x
+
+
+class PointwiseMultiplyIncr(IncrementMaskModule):
+    """Product rule on cached operands, reservoirs owned elsewhere (reference :51-64)."""
+
+    def __init__(self, x1res_module: IncrementReserve, x2res_module: IncrementReserve):
+        super().__init__()
+        self.x1_res: IncrementReserve = x1res_module
+        self.x2_res: IncrementReserve = x2res_module
+
+    def forward(self, x1_incr: Masked, x2_incr: Masked) -> Masked:
+        return IncrPointwiseMultiply(x1_incr, self.x1_res, x2_incr, self.x2_res)
+
+    def forward_refresh_reservoirs(self, x1: DenseT, x2: DenseT) -> DenseT:
+        return x1 * x2
+
+
+class nnReservedMultiplication(PointwiseMultiplyIncr):
+    """Product rule + accumulation of both operands, one kernel (reference :67-81)."""
+
+    def __init__(self):
+        super().__init__(IncrementReserve(), IncrementReserve())
+
+    def forward(self, x1_incr: Masked, x2_incr: Masked) -> Masked:
+        d1, p1, t1 = _unpack(x1_incr)
+        d2, p2, t2 = _unpack(x2_incr)
+        if self.x1_res.reservoir is None or self.x2_res.reservoir is None:
+            raise RuntimeError("nnReservedMultiplication: call forward_refresh_reservoirs first")
+        n, c, h, w = d1.shape
+        if t1 is not None and t1.shares_tiles_with(t2) and t1.pixmask is t2.pixmask:
+            ts = t1
+        else:
+            ts = self._tile_set("union", n, h, w, d1.device)
+            ops.build_mask_tiles(p1, p2, n, h, w, _lib.FOOT_CONV, 1, 1, 0, ts)
+        out = self._delta_buf("out", (n, c, h, w), d1.device)
+        ops.mul_incr(d1, p1, self.x1_res.reservoir, d2, p2, self.x2_res.reservoir, out, ts)
+        return [out, ts]
+
+    def forward_refresh_reservoirs(self, x1: DenseT, x2: DenseT) -> DenseT:
+        out = PointwiseMultiplyIncr.forward_refresh_reservoirs(self, x1, x2)
+        self.x1_res.update_reservoir(x1)
+        self.x2_res.update_reservoir(x2)
+        self._reset_incr()
+        return out
+
+
+def activation_kind(op) -> Tuple[int, float]:
+    """Map a unary torch callable onto a kernel activation (kind, negative slope)."""
+    if isinstance(op, functools.partial):
+        kind, slope = activation_kind(op.func)
+        if kind == _lib.ACT_LEAKY_RELU:
+            slope = op.keywords.get("negative_slope", op.args[0] if op.args else slope)
+        return kind, float(slope)
+    if isinstance(op, nn.LeakyReLU):
+        return _lib.ACT_LEAKY_RELU, float(op.negative_slope)
+    if isinstance(op, nn.ReLU) or op in (torch.relu, F.relu, torch.relu_):
+        return _lib.ACT_RELU, 0.0
+    if isinstance(op, nn.Sigmoid) or op in (torch.sigmoid, F.sigmoid):
+        return _lib.ACT_SIGMOID, 0.0
+    if isinstance(op, nn.Tanh) or op in (torch.tanh, F.tanh):
+        return _lib.ACT_TANH, 0.0
+    if op is F.leaky_relu:
+        return _lib.ACT_LEAKY_RELU, 0.01
+    slope = getattr(op, "negative_slope", None)
+    if slope is not None:
+        return _lib.ACT_LEAKY_RELU, float(slope)
+    raise NotImplementedError(
+        "incremental activation for %r has no kernel (supported: relu, leaky_relu, sigmoid, tanh)" % (op,))
+
+
+def leaky_relu_op(negative_slope: float = 0.01):
+    """Unary callable for nnReservedActivation(op=...) that the kernels recognise."""
+    return functools.partial(F.leaky_relu, negative_slope=negative_slope)
+
+
+class NonlinearPointOpIncr(IncrementMaskModule):
+    """out = op(R + d) - op(R); the reservoir is owned by the caller (reference :86-103)."""
+
+    def __init__(self, res_in: IncrementReserve, op=torch.tanh, refine_mask: bool = True):
+        super().__init__()
+        self.reservoir_in = res_in
+        self.op = op
+        self.refine_mask = refine_mask
+
+    def forward(self, x_incr: Masked) -> Masked:
+        return self._nonlin(x_incr, keep_reservoir=True)
+
+    def forward_refresh_reservoirs(self, x: DenseT):
+        return self.op(x)
+
+    def _nonlin(self, x_incr: Masked, keep_reservoir: bool):
+        kind, slope = activation_kind(self.op)
+        d, _, _ = _unpack(x_incr)
+        res = self.reservoir_in.reservoir
+        if res is None:
+            raise RuntimeError("incremental activation: call forward_refresh_reservoirs first")
+        n, c, h, w = d.shape
+        mask = x_incr[1] if len(x_incr) > 1 else None
+        if isinstance(mask, TileMask):
+            ts = mask
+        else:
+            ts = self._tile_set("own", n, h, w, d.device)
+            ops.build_mask_tiles(ops.pixel_mask_of(mask, d), None, n, h, w, _lib.FOOT_CONV, 1, 1, 0, ts)
+        out = self._delta_buf("out", (n, c, h, w), d.device)
+        if self.refine_mask:
+            pix = self._pix_buf("refined", n, h, w, d.device)
+            ops.act_incr(kind, slope, d, res, out, ts, pix, keep_reservoir=keep_reservoir)
+            return [out, self._view("refined", ts, pix)]
+        ops.act_incr(kind, slope, d, res, out, ts, None, keep_reservoir=keep_reservoir)
+        return [out, ts]
+
+
+class nnLinearIncr(nn.Linear):
+    """Fully connected layer on a delta: bias dropped (reference :106-116)."""
+
+    def forward(self, x_incr: Masked) -> Masked:
+        return F.linear(x_incr[0], self.weight, bias=None), None
+
+    def forward_refresh_reservoirs(self, x: DenseT) -> DenseT:
+        return super().forward(x)
+
+
+class _ConvIncrMixin(_IncrBuffers):
+    """Shared body of nnConvIncrBase / nnConvIncr."""
+
+    def _geometry(self):
+        k = _square(self.kernel_size, "kernel_size")
+        s = _square(self.stride, "stride")
+        p = _square(self.padding, "padding")
+        if _square(self.dilation, "dilation") != 1 or self.groups != 1:
+            raise NotImplementedError("incremental conv with dilation / groups")
+        if k not in (1, 3, 5, 7) or s not in (1, 2):
+            raise NotImplementedError("not Implemented convolution for these dimensions!")
+        return k, s, p
+
+    @property
+    def conv2d_weights(self) -> torch.Tensor:
+        """Filter in the kernel layout [Cin, K, K, Cout], rebuilt when the weight changes."""
+        w = self.weight
+        tag = (w.data_ptr(), w._version, str(w.device))
+        cached = self.__dict__.get("_filt_cache")
+        if cached is None or cached[0] != tag:
+            cached = (tag, w.detach().permute(1, 2, 3, 0).contiguous().float())
+            self.__dict__["_filt_cache"] = cached
+        return cached[1]
+
+    def _incr_forward(self, x_incr: Masked, x2_incr: Masked = None, reservoir=None,
+                      act=_lib.ACT_NONE, slope=0.0, path=_lib.PATH_AUTO, out_name="out") -> Masked:
+        k, s, p = self._geometry()
+        x, pix, _ = _unpack(x_incr)
+        x2 = pix2 = None
+        if x2_incr is not None:
+            x2, pix2, _ = _unpack(x2_incr)
+        n, _, h, w = x.shape
+        ho, wo = ops.conv_out_size(h, w, k, s, p)
+        ts = self._tile_set(out_name, n, ho, wo, x.device)
+        out = self._delta_buf(out_name, (n, self.out_channels, ho, wo), x.device)
+        if x2 is None:
+            m1, m2 = pix, None
+        elif pix is None or pix2 is None:      # one input dense -> every tile active
+            m1 = m2 = None
+        else:
+            m1, m2 = pix, pix2
+        ops.build_mask_tiles(m1, m2, n, h, w, _lib.FOOT_CONV, k, s, p, ts)
+        ops.conv_masked(x, pix, x2, pix2, self.conv2d_weights, k, s, p, ts, out, reservoir, act,
+                        slope, path)
+        return [out, ts]
+
+
+class nnConvIncrBase(nn.Conv2d, _ConvIncrMixin):
+    """Reference :122-142."""
+
+    def forward(self, x_incr):
+        return self._incr_forward(x_incr)
+
+    def forward_refresh_reservoirs(self, x):
+        self._reset_incr()
+        return nn.Conv2d.forward(self, x)
+
+
+class nnConvIncr(nn.Conv2d, _ConvIncrMixin):
+    """Incremental conv: forward([d, m]) = [conv2d(d, W, bias=None), tile mask].
+
+    Reference :146-196, where forward always falls back to a dense F.conv2d on
+    the delta (:175-178); here only the active output tiles are computed.
+    `path` selects the kernel (auto / VALU / MFMA), for tests and benchmarks.
+    """
+
+    def __init__(self, in_channels: int, out_channels: int, kernel_size, stride=1, padding=0,
+                 bias=True):
+        nn.Conv2d.__init__(self, in_channels, out_channels, kernel_size, stride, padding, bias=bias)
+        self.kf = KFencedMaskModule(0.3)
+        self.path = _lib.PATH_AUTO
+
+    def load_state_dict(self, state_dict, strict: bool = True):
+        ret = nn.Conv2d.load_state_dict(self, state_dict, strict=strict)
+        self.__dict__.pop("_filt_cache", None)
+        return ret
+
+    def forward(self, x_incr, x2_incr=None):
+        return self._incr_forward(x_incr, x2_incr, path=self.path)
+
+    def forward_fused(self, x_incr, activation: "nnReservedActivation", x2_incr=None):
+        """conv + activation increment in one kernel; updates activation.in_res in place."""
+        kind, slope = activation_kind(activation.op)
+        res = activation.in_res.reservoir
+        if res is None:
+            raise RuntimeError("fused conv+activation: call forward_refresh_reservoirs first")
+        return self._incr_forward(x_incr, x2_incr, reservoir=res, act=kind, slope=slope,
+                                  path=self.path, out_name="out_act")
+
+    def forward_refresh_reservoirs(self, x):
+        # The reference also refreshes self.kf here (:193), a norm and a zero clone
+        # that nothing reads because kf.forward is never called (:166).
+        self._reset_incr()
+        return nn.Conv2d.forward(self, x)
+
+
+class nnConvTranspose2dIncr(nn.ConvTranspose2d, _IncrBuffers):
+    """Incremental transposed conv (named but not defined by the reference,
+    incr_modules/e2depth_incr.py:248; semantics of transposed_conv2d_from_module,
+    mask_incr_functional.py:64-66)."""
+
+    def _filter(self):
+        w = self.weight
+        tag = (w.data_ptr(), w._version, str(w.device))
+        cached = self.__dict__.get("_filt_cache")
+        if cached is None or cached[0] != tag:
+            cached = (tag, w.detach().permute(0, 2, 3, 1).contiguous().float())
+            self.__dict__["_filt_cache"] = cached
+        return cached[1]
+
+    def forward(self, x_incr: Masked, reservoir=None, act=_lib.ACT_NONE, slope=0.0) -> Masked:
+        k = _square(self.kernel_size, "kernel_size")
+        s, p = _square(self.stride, "stride"), _square(self.padding, "padding")
+        op = _square(self.output_padding, "output_padding")
+        if _square(self.dilation, "dilation") != 1 or self.groups != 1:
+            raise NotImplementedError("transposed conv with dilation / groups")
+        x, pix, _ = _unpack(x_incr)
+        n, _, h, w = x.shape
+        ho, wo = (h - 1) * s - 2 * p + k + op, (w - 1) * s - 2 * p + k + op
+        ts = self._tile_set("out", n, ho, wo, x.device)
+        out = self._delta_buf("out", (n, self.out_channels, ho, wo), x.device)
+        ops.build_mask_tiles(pix, None, n, h, w, _lib.FOOT_TCONV, k, s, p, ts)
+        ops.tconv_masked(x, pix, self._filter(), k, s, p, ts, out, reservoir, act, slope)
+        return [out, ts]
+
+    def forward_refresh_reservoirs(self, x):
+        self._reset_incr()
+        return nn.ConvTranspose2d.forward(self, x)
+
+
+class nnBatchNorm2dIncr(nn.BatchNorm2d):
+    """Reference :200-207."""
+
+    def forward(self, x_incr):
+        return bn2d_from_module(x_incr, self)
+
+    def forward_refresh_reservoirs(self, x):
+        return super().forward(x)
+
+
+class nnMaxPool2dIncr(nn.MaxPool2d):
+    """pool(R + d) - pool(R), R += d (reference :210-224); torch ops, not on the hot path."""
+
+    def __init__(self, kernel_size, stride=None, padding=0):
+        nn.MaxPool2d.__init__(self, kernel_size=kernel_size, stride=stride, padding=padding)
+        self.functional = lambda x: F.max_pool2d(x, kernel_size=self.kernel_size,
+                                                 stride=self.stride, padding=self.padding)
+        self.mp_res = IncrementReserve()
+
+    def forward(self, x_incr: Masked) -> Masked:
+        out = self.functional(self.mp_res.reservoir + x_incr[0]) - self.functional(self.mp_res.reservoir)
+        self.mp_res.accumulate(x_incr)
+        return out, None
+
+    def forward_refresh_reservoirs(self, x: DenseT) -> DenseT:
+        self.mp_res.update_reservoir(x)
+        return super().forward(x)
+
+
+class nnAdaptiveAvgPool2dIncr(nn.AdaptiveAvgPool2d):
+    """Reference :228-233."""
+
+    def forward(self, x_incr):
+        return nn.AdaptiveAvgPool2d.forward(self, x_incr[0]), None
+
+    def forward_refresh_reservoirs(self, x):
+        return super().forward(x)
+
+
+class nnSequentialIncr(nn.Sequential):
+    """Reference :236-240."""
+
+    def forward_refresh_reservoirs(self, x):
+        for module in self:
+            x = module.forward_refresh_reservoirs(x)
+        return x
+
+
+class nnReservedActivation(NonlinearPointOpIncr):
+    """Activation increment with its own reservoir, updated in the same kernel
+    (reference :243-256)."""
+
+    def __init__(self, op=torch.relu, refine_mask: bool = True):
+        nn.Module.__init__(self)
+        self.in_res = IncrementReserve()
+        NonlinearPointOpIncr.__init__(self, self.in_res, op, refine_mask)
+
+    def forward(self, x_incr: Masked):
+        return self._nonlin(x_incr, keep_reservoir=False)
+
+    def forward_refresh_reservoirs(self, x: DenseT):
+        out = NonlinearPointOpIncr.forward_refresh_reservoirs(self, x)
+        self.in_res.update_reservoir(x)
+        self._reset_incr()
+        return out
+
+
+class nnReluIncr(nnReservedActivation):
+    def __init__(self):
+        nnReservedActivation.__init__(self, torch.relu)
+
+
+class nnSigmoidIncr(nnReservedActivation):
+    def __init__(self):
+        nnReservedActivation.__init__(self, torch.sigmoid)
+
+
+class nnTanhIncr(nnReservedActivation):
+    def __init__(self):
+        nnReservedActivation.__init__(self, torch.tanh)
+
+
+class nnAddIncr(IncrementMaskModule):
+    """Sum of two deltas with the union of their masks (the skip / residual sum the
+    reference writes as a tensor add, incr_modules/e2depth_incr.py:220,333)."""
+
+    def forward(self, a_incr: Masked, b_incr: Masked) -> Masked:
+        a, pa, _ = _unpack(a_incr)
+        b, pb, _ = _unpack(b_incr)
+        n, c, h, w = a.shape
+        ts = self._tile_set("union", n, h, w, a.device)
+        ops.build_mask_tiles(pa, pb, n, h, w, _lib.FOOT_CONV, 1, 1, 0, ts)
+        out = self._delta_buf("out", (n, c, h, w), a.device)
+        ops.add_incr(a, pa, b, pb, out, ts)
+        return [out, ts]
+
+    def forward_refresh_reservoirs(self, a: DenseT, b: DenseT) -> DenseT:
+        self._reset_incr()
+        return a + b
+
+
+class nnUpsample2xIncr(IncrementMaskModule):
+    """Bilinear x2 of a delta (optionally of the sum of two deltas) on persistent
+    buffers; module form of interpolate_from_module (mask_incr_functional.py:76-78)."""
+
+    def forward(self, x_incr: Masked, skip_incr: Masked = None) -> Masked:
+        a, pa, _ = _unpack(x_incr)
+        b = pb = None
+        if skip_incr is not None:
+            b, pb, _ = _unpack(skip_incr)
+        n, c, h, w = a.shape
+        ts = self._tile_set("out", n, 2 * h, 2 * w, a.device)
+        if skip_incr is not None and (pa is None or pb is None):
+            m1 = m2 = None
+        else:
+            m1, m2 = pa, pb
+        ops.build_mask_tiles(m1, m2, n, h, w, _lib.FOOT_UP2X, 0, 0, 0, ts)
+        out = self._delta_buf("out", (n, c, 2 * h, 2 * w), a.device)
+        ops.upsample2x_incr(a, pa, b, pb, ts, out)
+        return [out, ts]
+
+    def forward_refresh_reservoirs(self, x: DenseT, skip: DenseT = None) -> DenseT:
+        self._reset_incr()
+        if skip is not None:
+            x = x + skip
+        return F.interpolate(x, scale_factor=2, mode="bilinear", align_corners=False)

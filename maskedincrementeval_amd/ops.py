@@ -1,0 +1,219 @@
+"""Tensor-level wrappers over the C ABI of libmie_hip.so.
+
+Each function checks shapes / layouts on the host, pulls raw device pointers
+and the current HIP stream out of torch, and calls one entry point of
+include/mie.h.  torch is used for memory and streams only.
+"""
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import check, lib
+from .masked_types import TileMask
+
+
+def _stream(t: torch.Tensor):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _require_gpu(t: torch.Tensor, name: str):
+    if not t.is_cuda:
+        raise RuntimeError("%s must live on the GPU (got %s); this package has no CPU path"
+                           % (name, t.device))
+
+
+def nhwc_ptr(t: Optional[torch.Tensor], name: str, c: Optional[int] = None):
+    """Device pointer of an (N,C,H,W) fp32 tensor stored channels_last; None -> NULL."""
+    if t is None:
+        return None
+    _require_gpu(t, name)
+    if t.dim() != 4 or t.dtype != torch.float32:
+        raise ValueError("%s must be a 4-D float32 tensor, got %s %s" % (name, tuple(t.shape), t.dtype))
+    if not t.permute(0, 2, 3, 1).is_contiguous():
+        raise ValueError("%s must be channels_last (NHWC in memory); strides %s" % (name, t.stride()))
+    if c is not None and t.shape[1] != c:
+        raise ValueError("%s has %d channels, expected %d" % (name, t.shape[1], c))
+    return t.data_ptr()
+
+
+def as_nhwc(t: torch.Tensor) -> torch.Tensor:
+    """Return t as fp32 channels_last (copies only if the layout / dtype differs)."""
+    if t.dtype != torch.float32:
+        t = t.float()
+    if not t.permute(0, 2, 3, 1).is_contiguous():
+        t = t.contiguous(memory_format=torch.channels_last)
+        if not t.permute(0, 2, 3, 1).is_contiguous():   # C == 1 corner: force the strides
+            t = t.permute(0, 2, 3, 1).contiguous().permute(0, 3, 1, 2)
+    return t
+
+
+def new_nhwc(n, c, h, w, device) -> torch.Tensor:
+    """Zero-filled (N,C,H,W) fp32 tensor with NHWC storage."""
+    return torch.zeros((n, h, w, c), dtype=torch.float32, device=device).permute(0, 3, 1, 2)
+
+
+def pix_ptr(m, n, h, w, name):
+    """Device pointer of a pixel mask: None | TileMask | uint8 (N,1,H,W) tensor."""
+    if m is None:
+        return None
+    t = m.pixmask if isinstance(m, TileMask) else m
+    if t.dtype != torch.uint8 or tuple(t.shape) != (n, 1, h, w) or not t.is_contiguous():
+        raise ValueError("%s must be a contiguous uint8 (%d,1,%d,%d) mask, got %s %s"
+                         % (name, n, h, w, tuple(t.shape), t.dtype))
+    _require_gpu(t, name)
+    return t.data_ptr()
+
+
+def pixel_mask_of(mask, like: torch.Tensor) -> Optional[torch.Tensor]:
+    """Normalise the mask slot of a Masked pair to a uint8 (N,1,H,W) tensor (None = dense)."""
+    if mask is None:
+        return None
+    if isinstance(mask, TileMask):
+        return mask.pixmask
+    n, _, h, w = like.shape
+    m = mask
+    if m.dim() != 4 or m.shape[0] != n or m.shape[2] != h or m.shape[3] != w:
+        raise ValueError("mask shape %s does not match delta %s" % (tuple(m.shape), tuple(like.shape)))
+    if m.shape[1] != 1:
+        m = m.ne(0).any(dim=1, keepdim=True)
+    return m.ne(0).to(torch.uint8).contiguous().to(like.device)
+
+
+# ---- entry points ----------------------------------------------------------------
+def mask_from_delta(delta: torch.Tensor, threshold: float, out: torch.Tensor):
+    n, c, h, w = delta.shape
+    check(lib().mie_mask_from_delta(nhwc_ptr(delta, "delta"), n, h, w, c, float(threshold),
+                                    pix_ptr(out, n, h, w, "out"), _stream(delta)))
+    return out
+
+
+def build_mask_tiles(in_mask, in_mask2, n, h_in, w_in, foot, k, stride, pad, out: TileMask):
+    """in_mask / in_mask2: None | TileMask | uint8 (N,1,H,W)."""
+    p1 = pix_ptr(in_mask, n, h_in, w_in, "in_mask")
+    p2 = pix_ptr(in_mask2, n, h_in, w_in, "in_mask2")
+    if p1 is None and p2 is not None:   # "all active" OR anything = all active
+        p2 = None
+    st = torch.cuda.current_stream(out.device).cuda_stream
+    check(lib().mie_build_mask_tiles(p1, p2, h_in, w_in, foot, k, stride, pad, out.ref, st))
+    return out
+
+
+def conv_masked(x, xmask, x2, x2mask, filt, k, stride, pad, out_ts: TileMask, out_delta,
+                reservoir=None, act=_lib.ACT_NONE, slope=0.0, path=_lib.PATH_AUTO):
+    """filt: [Cin_total, K, K, Cout] contiguous fp32."""
+    n, c1, h, w = x.shape
+    c2 = 0 if x2 is None else x2.shape[1]
+    if x2 is not None and (x2.shape[0] != n or x2.shape[2:] != x.shape[2:]):
+        raise ValueError("x2 shape %s incompatible with x %s" % (tuple(x2.shape), tuple(x.shape)))
+    if filt.dim() != 4 or filt.shape[1] != k or filt.shape[2] != k or not filt.is_contiguous() \
+            or filt.dtype != torch.float32:
+        raise ValueError("filter must be contiguous fp32 [Cin,%d,%d,Cout], got %s" % (k, k, tuple(filt.shape)))
+    _require_gpu(filt, "filter")
+    cin_total, cout = filt.shape[0], filt.shape[3]
+    if tuple(out_delta.shape) != (n, cout, out_ts.h, out_ts.w) or out_ts.n != n:
+        raise ValueError("out_delta shape %s, expected %s" % (tuple(out_delta.shape), (n, cout, out_ts.h, out_ts.w)))
+    if reservoir is not None and reservoir.shape != out_delta.shape:
+        raise ValueError("reservoir shape %s != output %s" % (tuple(reservoir.shape), tuple(out_delta.shape)))
+    check(lib().mie_conv_masked(
+        nhwc_ptr(x, "x"), pix_ptr(xmask, n, h, w, "xmask"), c1,
+        nhwc_ptr(x2, "x2"), pix_ptr(x2mask, n, h, w, "x2mask"), c2, h, w,
+        filt.data_ptr(), cin_total, k, stride, pad, cout, out_ts.ref,
+        nhwc_ptr(out_delta, "out_delta"), nhwc_ptr(reservoir, "reservoir"),
+        act, float(slope), path, _stream(x)))
+    return out_delta
+
+
+def tconv_masked(x, xmask, filt, k, stride, pad, out_ts: TileMask, out_delta, reservoir=None,
+                 act=_lib.ACT_NONE, slope=0.0):
+    """filt: ConvTranspose2d weight permuted to [Cin, K, K, Cout], contiguous fp32."""
+    n, cin, h, w = x.shape
+    if filt.dim() != 4 or filt.shape[0] != cin or filt.shape[1] != k or not filt.is_contiguous():
+        raise ValueError("filter must be contiguous [Cin,%d,%d,Cout], got %s" % (k, k, tuple(filt.shape)))
+    _require_gpu(filt, "filter")
+    cout = filt.shape[3]
+    if tuple(out_delta.shape) != (n, cout, out_ts.h, out_ts.w):
+        raise ValueError("out_delta shape %s" % (tuple(out_delta.shape),))
+    check(lib().mie_tconv_masked(
+        nhwc_ptr(x, "x"), pix_ptr(xmask, n, h, w, "xmask"), cin, h, w, filt.data_ptr(), k, stride,
+        pad, cout, out_ts.ref, nhwc_ptr(out_delta, "out_delta"), nhwc_ptr(reservoir, "reservoir"),
+        act, float(slope), _stream(x)))
+    return out_delta
+
+
+def _same_shape(name, t, ref):
+    if t.shape != ref.shape:
+        raise ValueError("%s shape %s != %s" % (name, tuple(t.shape), tuple(ref.shape)))
+
+
+def act_incr(kind, slope, in_delta, reservoir, out_delta, ts: TileMask, out_pixmask=None,
+             keep_reservoir=False):
+    n, c, h, w = in_delta.shape
+    _same_shape("reservoir", reservoir, in_delta)
+    _same_shape("out_delta", out_delta, in_delta)
+    if (ts.n, ts.h, ts.w) != (n, h, w):
+        raise ValueError("tile set %s does not match delta %s" % ((ts.n, ts.h, ts.w), (n, h, w)))
+    check(lib().mie_act_incr(kind, float(slope), nhwc_ptr(in_delta, "in_delta"),
+                             nhwc_ptr(reservoir, "reservoir"), nhwc_ptr(out_delta, "out_delta"), c,
+                             ts.ref, pix_ptr(out_pixmask, n, h, w, "out_pixmask"),
+                             _lib.FLAG_KEEP_RESERVOIR if keep_reservoir else 0,
+                             _stream(in_delta)))
+    return out_delta
+
+
+def mul_incr(d1, m1, r1, d2, m2, r2, out_delta, ts: TileMask, keep_reservoir=False):
+    n, c, h, w = d1.shape
+    for name, t in (("r1", r1), ("d2", d2), ("r2", r2), ("out_delta", out_delta)):
+        _same_shape(name, t, d1)
+    check(lib().mie_mul_incr(nhwc_ptr(d1, "d1"), pix_ptr(m1, n, h, w, "m1"), nhwc_ptr(r1, "r1"),
+                             nhwc_ptr(d2, "d2"), pix_ptr(m2, n, h, w, "m2"), nhwc_ptr(r2, "r2"),
+                             nhwc_ptr(out_delta, "out_delta"), c, ts.ref,
+                             _lib.FLAG_KEEP_RESERVOIR if keep_reservoir else 0, _stream(d1)))
+    return out_delta
+
+
+def add_incr(a, ma, b, mb, out_delta, ts: TileMask):
+    n, c, h, w = a.shape
+    _same_shape("b", b, a)
+    _same_shape("out_delta", out_delta, a)
+    check(lib().mie_add_incr(nhwc_ptr(a, "a"), pix_ptr(ma, n, h, w, "ma"), nhwc_ptr(b, "b"),
+                             pix_ptr(mb, n, h, w, "mb"), nhwc_ptr(out_delta, "out_delta"), c,
+                             ts.ref, _stream(a)))
+    return out_delta
+
+
+def upsample2x_incr(a, ma, b, mb, out_ts: TileMask, out_delta):
+    n, c, h, w = a.shape
+    if b is not None:
+        _same_shape("b", b, a)
+    if tuple(out_delta.shape) != (n, c, 2 * h, 2 * w):
+        raise ValueError("out_delta shape %s, expected %s" % (tuple(out_delta.shape), (n, c, 2 * h, 2 * w)))
+    check(lib().mie_upsample2x_incr(nhwc_ptr(a, "a"), pix_ptr(ma, n, h, w, "ma"),
+                                    nhwc_ptr(b, "b"), pix_ptr(mb, n, h, w, "mb"), h, w, c,
+                                    out_ts.ref, nhwc_ptr(out_delta, "out_delta"), _stream(a)))
+    return out_delta
+
+
+def convlstm_gates_incr(gates_delta, gates_res, cprev_delta, cprev_mask, cprev_res, cell_res,
+                        h_delta, c_delta, ts: TileMask):
+    n, c4, h, w = gates_delta.shape
+    hid = c4 // 4
+    if c4 != 4 * hid:
+        raise ValueError("gates tensor needs 4*hid channels, got %d" % c4)
+    _same_shape("gates_res", gates_res, gates_delta)
+    for name, t in (("cprev_res", cprev_res), ("cell_res", cell_res), ("h_delta", h_delta),
+                    ("c_delta", c_delta)):
+        if tuple(t.shape) != (n, hid, h, w):
+            raise ValueError("%s shape %s, expected %s" % (name, tuple(t.shape), (n, hid, h, w)))
+    check(lib().mie_convlstm_gates_incr(
+        nhwc_ptr(gates_delta, "gates_delta"), nhwc_ptr(gates_res, "gates_res"),
+        nhwc_ptr(cprev_delta, "cprev_delta"), pix_ptr(cprev_mask, n, h, w, "cprev_mask"),
+        nhwc_ptr(cprev_res, "cprev_res"), nhwc_ptr(cell_res, "cell_res"),
+        nhwc_ptr(h_delta, "h_delta"), nhwc_ptr(c_delta, "c_delta"), hid, ts.ref,
+        _stream(gates_delta)))
+    return h_delta, c_delta
+
+
+def conv_out_size(h, w, k, stride, pad) -> Tuple[int, int]:
+    """Output size formula of the reference wrapper (ext/pointops/pointops_functional.py:25-26)."""
+    return (h + 2 * pad - k) // stride + 1, (w + 2 * pad - k) // stride + 1

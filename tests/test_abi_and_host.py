@@ -1,0 +1,212 @@
+"""CPU-side checks: the C-ABI library loads and exports every symbol include/mie.h
+declares, host-side argument validation returns status codes (no compute call
+reaches a GPU here), and the host logic of the Python surface."""
+import ctypes
+import functools
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from maskedincrementeval_amd import _lib
+from maskedincrementeval_amd import masked_types as mt
+from maskedincrementeval_amd import mask_incr_modules as mm
+from maskedincrementeval_amd import synthetic
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "mie.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mie_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported(mie_lib):
+    declared = _declared_symbols()
+    assert len(declared) >= 12
+    assert sorted(_lib.EXPORTS) == declared
+    for name in declared:
+        assert hasattr(mie_lib, name), name
+    assert mie_lib.mie_version() >= 100
+
+
+def test_tile_capacity(mie_lib):
+    assert mie_lib.mie_tile_capacity(1, 264, 352) == 33 * 44
+    assert mie_lib.mie_tile_capacity(8, 480, 640) == 8 * 60 * 80
+    assert mie_lib.mie_tile_capacity(1, 9, 9) == 4
+    assert mie_lib.mie_tile_capacity(0, 8, 8) == 0
+    assert _lib.tile_capacity(2, 19, 27) == mie_lib.mie_tile_capacity(2, 19, 27)
+
+
+def _fake_tileset(n=1, h=16, w=16, null=None):
+    """Tile set with non-NULL but never dereferenced host pointers (validation only)."""
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.addressof(buf)
+    vals = dict(pixmask=p, tiles=p, stale=p, counts=p, flags=p)
+    if null:
+        vals[null] = None
+    return _lib.MieTileSet(n, h, w, vals["pixmask"], vals["tiles"], vals["stale"], vals["counts"],
+                           vals["flags"]), buf
+
+
+def test_invalid_arguments_return_status_not_abort(mie_lib):
+    # every call below is rejected by host-side validation: nothing is launched
+    ts, keep = _fake_tileset()
+    buf = ctypes.create_string_buffer(4096)
+    p = (ctypes.addressof(buf) + 15) & ~15
+    err = lambda: mie_lib.mie_last_error_string().decode()
+    # NULL tile set
+    assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 16, 16, p, 16, 3, 1, 1, 32, None, p,
+                                   None, 0, 0.0, 0, None) == -1
+    assert "tile set is NULL" in err()
+    # NULL input pointer
+    assert mie_lib.mie_conv_masked(None, None, 16, None, None, 0, 16, 16, p, 16, 3, 1, 1, 32,
+                                   ctypes.byref(ts), p, None, 0, 0.0, 0, None) == -1
+    # unsupported kernel size and stride (the reference throws std::logic_error, ext_conv.cu:366)
+    assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 16, 16, p, 16, 4, 1, 1, 32,
+                                   ctypes.byref(ts), p, None, 0, 0.0, 0, None) == -2
+    assert "kernel size 4" in err()
+    assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 16, 16, p, 16, 3, 3, 1, 32,
+                                   ctypes.byref(ts), p, None, 0, 0.0, 0, None) == -2
+    # output geometry mismatch
+    assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 20, 16, p, 16, 3, 1, 1, 32,
+                                   ctypes.byref(ts), p, None, 0, 0.0, 0, None) == -1
+    assert "tile set is" in err()
+    # misaligned pointer
+    assert mie_lib.mie_conv_masked(p + 4, None, 16, None, None, 0, 16, 16, p, 16, 3, 1, 1, 32,
+                                   ctypes.byref(ts), p, None, 0, 0.0, 0, None) == -1
+    assert "aligned" in err()
+    # MFMA path on a shape it cannot take
+    assert mie_lib.mie_conv_masked(p, None, 5, None, None, 0, 16, 16, p, 5, 3, 1, 1, 32,
+                                   ctypes.byref(ts), p, None, 0, 0.0, _lib.PATH_MFMA, None) == -2
+    # activation without a reservoir
+    assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 16, 16, p, 16, 3, 1, 1, 32,
+                                   ctypes.byref(ts), p, None, _lib.ACT_RELU, 0.0, 0, None) == -1
+    # channels beyond the filter
+    assert mie_lib.mie_conv_masked(p, None, 16, p, None, 16, 16, 16, p, 16, 3, 1, 1, 32,
+                                   ctypes.byref(ts), p, None, 0, 0.0, 0, None) == -1
+    # tile set with a NULL member / zero-sized geometry
+    bad, keep2 = _fake_tileset(null="tiles")
+    assert mie_lib.mie_act_incr(1, 0.0, p, p, p, 8, ctypes.byref(bad), None, 0, None) == -1
+    zero, keep3 = _fake_tileset(n=0)
+    assert mie_lib.mie_act_incr(1, 0.0, p, p, p, 8, ctypes.byref(zero), None, 0, None) == -1
+    assert mie_lib.mie_act_incr(9, 0.0, p, p, p, 8, ctypes.byref(ts), None, 0, None) == -2
+    assert mie_lib.mie_build_mask_tiles(None, None, 16, 16, 7, 3, 1, 1, ctypes.byref(ts), None) == -2
+    assert mie_lib.mie_build_mask_tiles(None, None, 9, 8, _lib.FOOT_UP2X, 0, 0, 0, ctypes.byref(ts), None) == -1
+    assert mie_lib.mie_upsample2x_incr(p, None, None, None, 9, 8, 4, ctypes.byref(ts), p, None) == -1
+    assert mie_lib.mie_mask_from_delta(p, 1, 4, 4, 4, -1.0, p, None) == -1
+    assert mie_lib.mie_convlstm_gates_incr(p, p, None, p, p, p, p, p, 4, ctypes.byref(ts), None) == -1
+    assert mie_lib.mie_tconv_masked(p, None, 4, 9, 9, p, 3, 2, 1, 4, ctypes.byref(ts), p, None, 0, 0.0, None) == -1
+
+
+def test_check_raises_runtime_error(mie_lib):
+    rc = mie_lib.mie_mask_from_delta(None, 1, 4, 4, 4, 0.0, None, None)
+    with pytest.raises(RuntimeError, match="NULL pointer"):
+        _lib.check(rc)
+    assert issubclass(_lib.MieError, RuntimeError)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(RuntimeError, match="no fallback"):
+        _lib.lib()
+
+
+def test_ops_refuse_cpu_tensors():
+    from maskedincrementeval_amd import ops
+    ts = mt.TileMask(1, 16, 16, "cpu")
+    x = torch.zeros(1, 8, 16, 16).contiguous(memory_format=torch.channels_last)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        ops.act_incr(_lib.ACT_RELU, 0.0, x, x.clone(), x.clone(), ts)
+
+
+def test_activation_kind_mapping():
+    assert mm.activation_kind(torch.relu) == (_lib.ACT_RELU, 0.0)
+    assert mm.activation_kind(torch.sigmoid)[0] == _lib.ACT_SIGMOID
+    assert mm.activation_kind(torch.tanh)[0] == _lib.ACT_TANH
+    assert mm.activation_kind(F.leaky_relu) == (_lib.ACT_LEAKY_RELU, 0.01)
+    assert mm.activation_kind(nn.LeakyReLU(0.2)) == (_lib.ACT_LEAKY_RELU, pytest.approx(0.2))
+    assert mm.activation_kind(mm.leaky_relu_op(0.05)) == (_lib.ACT_LEAKY_RELU, pytest.approx(0.05))
+    assert mm.activation_kind(functools.partial(F.leaky_relu, negative_slope=0.3))[1] == pytest.approx(0.3)
+    with pytest.raises(NotImplementedError):
+        mm.activation_kind(torch.exp)
+
+
+def test_module_surface_matches_reference_names():
+    # names the reference exports from incr_modules/mask_incr_modules.py and *_functional.py
+    for name in ("IncrementMaskModule", "KFencedMaskModule", "PointwiseMultiplyIncr",
+                 "nnReservedMultiplication", "NonlinearPointOpIncr", "nnLinearIncr", "nnConvIncrBase",
+                 "nnConvIncr", "nnBatchNorm2dIncr", "nnMaxPool2dIncr", "nnAdaptiveAvgPool2dIncr",
+                 "nnSequentialIncr", "nnReservedActivation", "nnReluIncr", "nnSigmoidIncr", "nnTanhIncr"):
+        assert hasattr(mm, name), name
+    from maskedincrementeval_amd import mask_incr_functional as mf
+    for name in ("AccumStreamManager", "IncrementReserve", "IncrPointwiseMultiply", "conv2d_from_module",
+                 "transposed_conv2d_from_module", "bn2d_from_module", "interpolate_from_module"):
+        assert hasattr(mf, name), name
+    for name in ("Sp", "DenseT", "SpOrDense", "Masked", "_device"):
+        assert hasattr(mt, name), name
+    c = mm.nnConvIncr(3, 5, 3, 1, 1, bias=False)
+    assert set(c.state_dict().keys()) == {"weight"}               # nn.Conv2d keys, as in the reference
+    assert tuple(c.conv2d_weights.shape) == (3, 3, 3, 5)          # [Cin, K, K, Cout]
+    assert torch.equal(c.conv2d_weights, c.weight.detach().permute(1, 2, 3, 0))
+    with torch.no_grad():
+        c.weight.mul_(2.0)
+    assert torch.equal(c.conv2d_weights, c.weight.detach().permute(1, 2, 3, 0))   # follows the weight
+    with pytest.raises(NotImplementedError):
+        mm.nnConvIncr(3, 5, 4)._geometry()
+    with pytest.raises(NotImplementedError):
+        mm.nnConvIncr(3, 5, 3, stride=3)._geometry()
+
+
+def test_e2depth_module_tree_and_shapes():
+    from maskedincrementeval_amd.e2depth_incr import E2VIDRecurrentIncr
+    net = E2VIDRecurrentIncr()
+    sd = net.state_dict()
+    # layer shapes of the reference trace (todo.txt:34-57)
+    u = "unetrecurrent."
+    assert tuple(sd[u + "head.conv2d.weight"].shape) == (32, 5, 5, 5)
+    assert tuple(sd[u + "encoders.0.conv.conv2d.weight"].shape) == (64, 32, 5, 5)
+    assert tuple(sd[u + "encoders.0.recurrent_block.Gates.weight"].shape) == (256, 128, 3, 3)
+    assert tuple(sd[u + "encoders.2.recurrent_block.Gates.weight"].shape) == (1024, 512, 3, 3)
+    assert tuple(sd[u + "resblocks.1.conv2.weight"].shape) == (256, 256, 3, 3)
+    assert tuple(sd[u + "decoders.0.conv2d.weight"].shape) == (128, 256, 5, 5)
+    assert tuple(sd[u + "decoders.2.conv2d.weight"].shape) == (32, 64, 5, 5)
+    assert tuple(sd[u + "pred.conv2d.weight"].shape) == (1, 32, 1, 1)
+    # dense refresh runs on the CPU (torch ops only) and fills the reservoirs
+    synthetic.seed_module_(net, 3)
+    with torch.no_grad():
+        pred, states = net.forward_refresh_reservoirs(torch.randn(1, 5, 16, 24), None)
+    assert pred.shape == (1, 1, 16, 24) and len(states) == 3
+    assert net.unetrecurrent.head.activation.in_res.reservoir.shape == (1, 32, 16, 24)
+    assert net.unetrecurrent.encoders[2].recurrent_block.gates_res.reservoir.shape == (1, 1024, 2, 3)
+
+
+def test_increment_reserve_keeps_pointer():
+    from maskedincrementeval_amd.mask_incr_functional import IncrementReserve
+    r = IncrementReserve(torch.randn(1, 4, 6, 6))
+    assert r.reservoir.permute(0, 2, 3, 1).is_contiguous()       # channels_last, as the reference
+    ptr = r.reservoir.data_ptr()
+    x = torch.randn(1, 4, 6, 6)
+    r.update_reservoir(x)
+    assert r.reservoir.data_ptr() == ptr and torch.equal(r.reservoir, x)
+    r.accumulate([torch.ones(1, 4, 6, 6), None])
+    assert torch.equal(r.reservoir, x + 1)
+
+
+def test_blob_mask_density_and_determinism():
+    for p in (0.01, 0.05, 0.20):
+        m = synthetic.blob_mask(264, 352, p, seed=11)
+        assert m.sum() == round(p * 264 * 352)
+        assert np.array_equal(m, synthetic.blob_mask(264, 352, p, seed=11))
+    d, m = synthetic.gaussian_delta(1, 8, 32, 40, 0.1, 0.1, seed=2)
+    assert (d[:, :, m[0, 0] == 0] == 0).all() and m.dtype == torch.uint8
+    ev, m2 = synthetic.event_voxel_delta(1, 5, 32, 40, 0.05, seed=3)
+    vals = torch.unique(ev * 10).round()
+    assert (ev[:, :, m2[0, 0] == 0] == 0).all() and torch.allclose(ev * 10, (ev * 10).round(), atol=1e-5)
+    assert vals.abs().max() >= 2

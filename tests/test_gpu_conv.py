@@ -1,0 +1,182 @@
+"""GPU parity of the masked convolutions (VALU, MFMA, small-Cout, transposed) against
+the CPU oracle, through the C ABI.  fp32 tolerance: rtol 1e-4, atol 1e-5."""
+import numpy as np
+import pytest
+import torch
+
+from maskedincrementeval_amd import _lib, ops
+from maskedincrementeval_amd.masked_types import TileMask
+from maskedincrementeval_amd.synthetic import blob_mask, gaussian_delta, he_normal_conv_weight
+from oracle import incr_oracle as io
+from oracle import mask_oracle as mo
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+RTOL, ATOL = 1e-4, 1e-5
+
+
+def _dev(t):
+    return ops.as_nhwc(t.to(DEV).contiguous(memory_format=torch.channels_last))
+
+
+def _filt(w_oihw):
+    return w_oihw.permute(1, 2, 3, 0).contiguous().to(DEV)
+
+
+def _close(got, ref, what=""):
+    got = got.cpu()
+    err = (got - ref).abs().max().item()
+    assert torch.allclose(got, ref, rtol=RTOL, atol=ATOL), "%s max|diff| = %.3e" % (what, err)
+
+
+class _Conv:
+    """One masked conv on persistent buffers, as a module would hold them."""
+
+    def __init__(self, n, cin, cout, h, w, k, s, p, seed, path):
+        self.k, self.s, self.p, self.path = k, s, p, path
+        self.w = he_normal_conv_weight(cout, cin, k, seed)
+        self.filt = _filt(self.w)
+        self.ho, self.wo = mo.conv_out_size(h, w, k, s, p)
+        self.ts = TileMask(n, self.ho, self.wo, DEV)
+        self.out = ops.new_nhwc(n, cout, self.ho, self.wo, DEV)
+        self.n, self.h, self.w_in = n, h, w
+
+    def run(self, delta, mask, reservoir=None, act=_lib.ACT_NONE, slope=0.0, x2=None, m2=None):
+        dm = None if mask is None else mask.to(DEV)
+        dm2 = None if m2 is None else m2.to(DEV)
+        both = dm if x2 is None else (None if (dm is None or dm2 is None) else dm)
+        ops.build_mask_tiles(both, dm2 if both is not None else None, self.n, self.h, self.w_in,
+                             _lib.FOOT_CONV, self.k, self.s, self.p, self.ts)
+        ops.conv_masked(_dev(delta), dm, None if x2 is None else _dev(x2), dm2, self.filt, self.k,
+                        self.s, self.p, self.ts, self.out, reservoir, act, slope, self.path)
+        torch.cuda.synchronize()
+        return self.out
+
+
+PATHS = [("valu", _lib.PATH_VALU), ("mfma", _lib.PATH_MFMA)]
+
+
+@pytest.mark.parametrize("pname,path", PATHS)
+@pytest.mark.parametrize("k,s,p", [(1, 1, 0), (3, 1, 1), (3, 2, 1), (5, 1, 2), (5, 2, 2), (7, 1, 3), (7, 2, 3)])
+@pytest.mark.parametrize("cin,cout", [(16, 32), (32, 64)])
+def test_conv_paths_match_oracle(pname, path, k, s, p, cin, cout):
+    n, h, w = 2, 37, 45      # ragged: not multiples of the 8x8 tile
+    d, m = gaussian_delta(n, cin, h, w, 0.06, 0.5, seed=k * 100 + s * 10 + cin)
+    conv = _Conv(n, cin, cout, h, w, k, s, p, seed=3, path=path)
+    got = conv.run(d, m)
+    _close(got, io.conv_incr(d, conv.w, s, p), "%s k%d s%d" % (pname, k, s))
+
+
+@pytest.mark.parametrize("cin,cout,k,s,p", [(5, 32, 5, 1, 2), (3, 5, 3, 1, 1), (7, 70, 3, 2, 1), (32, 1, 1, 1, 0),
+                                            (32, 2, 3, 1, 1), (4, 3, 5, 2, 2), (20, 33, 1, 2, 0)])
+def test_odd_channel_counts_auto_path(cin, cout, k, s, p):
+    # head (Cin=5), prediction (Cout=1), flow heads (Cout=2) and other shapes the MFMA path cannot take
+    n, h, w = 1, 41, 29
+    d, m = gaussian_delta(n, cin, h, w, 0.1, 0.5, seed=cin + cout)
+    conv = _Conv(n, cin, cout, h, w, k, s, p, seed=4, path=_lib.PATH_AUTO)
+    _close(conv.run(d, m), io.conv_incr(d, conv.w, s, p))
+
+
+@pytest.mark.parametrize("pname,path", PATHS)
+def test_all_ones_mask_equals_dense_conv(pname, path):
+    # reference tests/test_pointops.py:25-35, at a shape both paths take
+    n, cin, cout, h, w = 1, 16, 32, 25, 25
+    x = torch.randn(n, cin, h, w, generator=torch.Generator().manual_seed(0))
+    conv = _Conv(n, cin, cout, h, w, 3, 1, 1, seed=5, path=path)
+    ref = io.conv_refresh(x, conv.w, None, 1, 1)
+    _close(conv.run(x, torch.ones(n, 1, h, w, dtype=torch.uint8)), ref)
+    _close(conv.run(x, None), ref)        # mask None = all active
+
+
+@pytest.mark.parametrize("pname,path", PATHS)
+def test_inactive_pixels_are_never_read_and_output_is_clean(pname, path):
+    n, cin, cout, h, w = 1, 32, 32, 64, 72
+    conv = _Conv(n, cin, cout, h, w, 3, 1, 1, seed=6, path=path)
+    for step, dens in enumerate((0.08, 0.02, 0.15, 0.0)):   # fresh masks: tiles go stale, last one empty
+        d, m = gaussian_delta(n, cin, h, w, dens, 0.3, seed=40 + step)
+        poisoned = torch.where(m.bool().expand_as(d), d, torch.full_like(d, float("nan")))
+        got = conv.run(poisoned, m).cpu()
+        ref = io.conv_incr(d, conv.w, 1, 1)
+        assert torch.isfinite(got).all()
+        _close(got, ref, "step %d" % step)
+        # exactly zero outside the footprint of the mask (clean-delta invariant)
+        fp = torch.from_numpy(mo.footprint_conv(m[:, 0].numpy(), 3, 1, 1)).bool().unsqueeze(1)
+        assert torch.count_nonzero(got * (~fp)) == 0
+
+
+@pytest.mark.parametrize("pname,path", PATHS)
+def test_two_pointer_input_equals_concat(pname, path):
+    # ConvLSTM gates: conv over cat(x, h) without forming the concat (e2depth_incr.py:100-101)
+    n, c1, c2, cout, h, w = 1, 32, 32, 128, 33, 44
+    dx, mx = gaussian_delta(n, c1, h, w, 0.05, 0.3, seed=60)
+    dh, mh = gaussian_delta(n, c2, h, w, 0.03, 0.3, seed=61)
+    conv = _Conv(n, c1 + c2, cout, h, w, 3, 1, 1, seed=7, path=path)
+    ref = io.conv_incr(torch.cat((dx, dh), 1), conv.w, 1, 1)
+    _close(conv.run(dx, mx, x2=dh, m2=mh), ref, "x ++ h")
+    # hidden half absent: only the first c1 filter channels are used
+    ref0 = io.conv_incr(torch.cat((dx, torch.zeros_like(dh)), 1), conv.w, 1, 1)
+    _close(conv.run(dx, mx), ref0, "x only")
+
+
+@pytest.mark.parametrize("pname,path", PATHS)
+@pytest.mark.parametrize("act,slope,op", [(_lib.ACT_RELU, 0.0, torch.relu),
+                                          (_lib.ACT_LEAKY_RELU, 0.01, io.leaky_relu),
+                                          (_lib.ACT_SIGMOID, 0.0, torch.sigmoid),
+                                          (_lib.ACT_TANH, 0.0, torch.tanh)])
+def test_fused_conv_activation_epilogue(pname, path, act, slope, op):
+    n, cin, cout, h, w = 1, 16, 32, 40, 48
+    conv = _Conv(n, cin, cout, h, w, 3, 1, 1, seed=8, path=path)
+    r0 = torch.randn(n, cout, h, w, generator=torch.Generator().manual_seed(1))
+    res_gpu = _dev(r0.clone())
+    res_cpu = io.Reserve(r0)
+    for step in range(3):
+        d, m = gaussian_delta(n, cin, h, w, 0.1, 0.5, seed=70 + step)
+        got = conv.run(d, m, reservoir=res_gpu, act=act, slope=slope)
+        ref = io.act_incr(op, res_cpu, io.conv_incr(d, conv.w, 1, 1))
+        _close(got, ref, "delta step %d" % step)
+        _close(res_gpu, res_cpu.reservoir, "reservoir step %d" % step)
+
+
+def test_config1_cached_output_plus_increment_is_dense_conv():
+    # benchmark configuration 1: 1x32x264x352 -> 32, 3x3 s1 p1, He-normal weights, x_prev ~ N(0,1),
+    # 5 % smoothed-threshold mask, delta ~ N(0, 0.1)
+    n, c, h, w = 1, 32, 264, 352
+    g = torch.Generator().manual_seed(0)
+    x_prev = torch.randn(n, c, h, w, generator=g)
+    d, m = gaussian_delta(n, c, h, w, 0.05, 0.1, seed=1000)
+    assert int(m.sum()) == round(0.05 * h * w)
+    for path in (_lib.PATH_VALU, _lib.PATH_MFMA):
+        conv = _Conv(n, c, 32, h, w, 3, 1, 1, seed=0, path=path)
+        cached = io.conv_refresh(x_prev, conv.w, None, 1, 1)
+        got = conv.run(d, m).cpu()
+        dense = io.conv_refresh(x_prev + d, conv.w, None, 1, 1)
+        assert torch.allclose(cached + got, dense, rtol=RTOL, atol=ATOL)
+        tiles = conv.ts.active_tiles().cpu().numpy()
+        assert np.array_equal(tiles, mo.tile_list(mo.footprint_conv(m[:, 0].numpy(), 3, 1, 1)))
+        assert 0 < tiles.size < conv.ts.capacity // 2
+
+
+@pytest.mark.parametrize("k,s,p,op", [(3, 2, 1, 1), (4, 2, 1, 0), (5, 2, 2, 1), (2, 2, 0, 0)])
+def test_tconv_matches_oracle(k, s, p, op):
+    n, cin, cout, h, w = 2, 12, 20, 19, 23
+    d, m = gaussian_delta(n, cin, h, w, 0.08, 0.5, seed=k)
+    wt = torch.randn(cin, cout, k, k, generator=torch.Generator().manual_seed(k)) * 0.2
+    ho, wo = (h - 1) * s - 2 * p + k + op, (w - 1) * s - 2 * p + k + op
+    ts = TileMask(n, ho, wo, DEV)
+    out = ops.new_nhwc(n, cout, ho, wo, DEV)
+    filt = wt.permute(0, 2, 3, 1).contiguous().to(DEV)
+    ref = io.tconv_incr(d, wt, s, p, op)
+    for step in range(2):
+        ops.build_mask_tiles(m.to(DEV), None, n, h, w, _lib.FOOT_TCONV, k, s, p, ts)
+        ops.tconv_masked(_dev(d), m.to(DEV), filt, k, s, p, ts, out)
+        torch.cuda.synchronize()
+        _close(out, ref, "tconv k%d" % k)
+
+
+def test_large_channel_mfma_bottleneck_shapes():
+    # 256 -> 256 3x3 at 33x44 (residual blocks) and 512 -> 1024 gates: K = 2304 / 4608 contractions
+    n, h, w = 1, 33, 44
+    for cin, cout in ((256, 256), (512, 1024)):
+        d, m = gaussian_delta(n, cin, h, w, 0.2, 0.2, seed=cin)
+        conv = _Conv(n, cin, cout, h, w, 3, 1, 1, seed=9, path=_lib.PATH_MFMA)
+        _close(conv.run(d, m), io.conv_incr(d, conv.w, 1, 1), "%d->%d" % (cin, cout))

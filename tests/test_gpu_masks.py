@@ -1,0 +1,129 @@
+"""GPU parity: pixel masks, footprints and ordered active-tile lists are bit-exact
+against the numpy oracle (oracle/mask_oracle.py), through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from maskedincrementeval_amd import _lib, ops
+from maskedincrementeval_amd.masked_types import TileMask
+from maskedincrementeval_amd.synthetic import blob_mask
+from oracle import mask_oracle as mo
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _to_dev_mask(m: np.ndarray) -> torch.Tensor:
+    return torch.from_numpy(m).unsqueeze(1).contiguous().to(DEV)
+
+
+def _check_tileset(ts: TileMask, want_mask: np.ndarray, prev_tiles=None):
+    torch.cuda.synchronize()
+    got = ts.pixmask[:, 0].cpu().numpy()
+    assert np.array_equal(got, want_mask), "pixel mask differs"
+    tiles = ts.active_tiles().cpu().numpy()
+    want_tiles = mo.tile_list(want_mask)
+    assert np.array_equal(tiles, want_tiles), "tile list differs"
+    assert int(ts.counts[_lib.CNT_TICKET].item()) == 0, "ticket counter not reset"
+    if prev_tiles is not None:
+        assert np.array_equal(ts.stale_tiles().cpu().numpy(), mo.stale_list(prev_tiles, want_tiles))
+    return want_tiles
+
+
+@pytest.mark.parametrize("shape,c,thr", [((1, 264, 352), 5, 0.0), ((2, 37, 53), 3, 0.0),
+                                         ((1, 33, 44), 64, 1e-4), ((1, 16, 16), 1, 0.5)])
+def test_mask_from_delta(shape, c, thr):
+    n, h, w = shape
+    g = torch.Generator().manual_seed(h * w + c)
+    d = torch.randn((n, c, h, w), generator=g) * (torch.rand((n, 1, h, w), generator=g) < 0.07)
+    d[0, :, 0, 0] = 0.0
+    d[0, c - 1, h - 1, w - 1] = 2e-4 if thr < 1e-3 else 0.4     # only the last channel; straddles thr
+    x = d.to(DEV).contiguous(memory_format=torch.channels_last)
+    x = ops.as_nhwc(x)
+    out = torch.zeros((n, 1, h, w), dtype=torch.uint8, device=DEV)
+    ops.mask_from_delta(x, thr, out)
+    torch.cuda.synchronize()
+    assert np.array_equal(out[:, 0].cpu().numpy(), mo.pixel_mask(d.numpy(), thr))
+
+
+@pytest.mark.parametrize("k,s,p", [(1, 1, 0), (3, 1, 1), (3, 2, 1), (5, 1, 2), (5, 2, 2), (7, 1, 3), (7, 2, 3)])
+@pytest.mark.parametrize("n,h,w,dens", [(1, 264, 352, 0.05), (2, 45, 61, 0.02), (1, 8, 8, 0.3)])
+def test_conv_footprint_tiles_and_stale(k, s, p, n, h, w, dens):
+    ho, wo = mo.conv_out_size(h, w, k, s, p)
+    ts = TileMask(n, ho, wo, DEV)
+    prev = np.zeros(0, np.int32)
+    for step in range(3):       # fresh mask per step: exercises the stale list
+        m = np.stack([blob_mask(h, w, dens, seed=1000 * step + 17 * b + k) for b in range(n)])
+        ops.build_mask_tiles(_to_dev_mask(m), None, n, h, w, _lib.FOOT_CONV, k, s, p, ts)
+        prev = _check_tileset(ts, mo.footprint_conv(m, k, s, p), prev)
+
+
+def test_all_active_empty_and_union():
+    n, h, w = 2, 30, 41
+    ts = TileMask(n, h, w, DEV)
+    # NULL mask = every pixel active
+    ops.build_mask_tiles(None, None, n, h, w, _lib.FOOT_CONV, 3, 1, 1, ts)
+    prev = _check_tileset(ts, np.ones((n, h, w), np.uint8))
+    assert prev.size == ts.capacity
+    # empty mask: no tiles, everything stale
+    ops.build_mask_tiles(_to_dev_mask(np.zeros((n, h, w), np.uint8)), None, n, h, w, _lib.FOOT_CONV, 3, 1, 1, ts)
+    prev = _check_tileset(ts, np.zeros((n, h, w), np.uint8), prev)
+    assert ts.stale_tiles().numel() == ts.capacity
+    # union of two masks through a 3x3 footprint
+    a = np.stack([blob_mask(h, w, 0.03, seed=5 + b) for b in range(n)])
+    b = np.stack([blob_mask(h, w, 0.02, seed=50 + b) for b in range(n)])
+    ops.build_mask_tiles(_to_dev_mask(a), _to_dev_mask(b), n, h, w, _lib.FOOT_CONV, 3, 1, 1, ts)
+    _check_tileset(ts, mo.footprint_conv(a | b, 3, 1, 1), prev)
+    # single pixels at the image corners
+    c = np.zeros((n, h, w), np.uint8)
+    c[0, 0, 0] = c[1, h - 1, w - 1] = c[0, h - 1, 0] = 1
+    ops.build_mask_tiles(_to_dev_mask(c), None, n, h, w, _lib.FOOT_CONV, 1, 1, 0, ts)
+    _check_tileset(ts, c)
+
+
+@pytest.mark.parametrize("n,h,w", [(1, 33, 44), (2, 5, 7), (1, 1, 1)])
+def test_up2x_footprint(n, h, w):
+    ts = TileMask(n, 2 * h, 2 * w, DEV)
+    prev = np.zeros(0, np.int32)
+    for step in range(2):
+        m = (np.random.default_rng(step + h).random((n, h, w)) < 0.1).astype(np.uint8)
+        m[0, 0, 0] = 1
+        m[-1, -1, -1] = step
+        ops.build_mask_tiles(_to_dev_mask(m), None, n, h, w, _lib.FOOT_UP2X, 0, 0, 0, ts)
+        prev = _check_tileset(ts, mo.footprint_up2x(m), prev)
+
+
+@pytest.mark.parametrize("k,s,p,op", [(3, 2, 1, 1), (4, 2, 1, 0), (5, 2, 2, 1), (2, 2, 0, 0)])
+def test_tconv_footprint(k, s, p, op):
+    n, h, w = 2, 17, 23
+    ho, wo = (h - 1) * s - 2 * p + k + op, (w - 1) * s - 2 * p + k + op
+    ts = TileMask(n, ho, wo, DEV)
+    m = np.stack([blob_mask(h, w, 0.05, seed=k + b) for b in range(n)])
+    ops.build_mask_tiles(_to_dev_mask(m), None, n, h, w, _lib.FOOT_TCONV, k, s, p, ts)
+    _check_tileset(ts, mo.footprint_tconv(m, k, s, p, ho, wo))
+
+
+def test_large_batch_tile_compaction():
+    # the batched high-resolution configuration: 8 streams of 480x640 -> 38400 tiles
+    n, h, w = 8, 480, 640
+    ts = TileMask(n, h, w, DEV)
+    prev = np.zeros(0, np.int32)
+    for step, dens in enumerate((0.01, 0.20)):
+        m = np.stack([blob_mask(h, w, dens, seed=9000 + 10 * step + b) for b in range(n)])
+        ops.build_mask_tiles(_to_dev_mask(m), None, n, h, w, _lib.FOOT_CONV, 3, 1, 1, ts)
+        prev = _check_tileset(ts, mo.footprint_conv(m, 3, 1, 1), prev)
+
+
+def test_repeated_builds_are_deterministic():
+    n, h, w = 1, 264, 352
+    m = blob_mask(h, w, 0.05, seed=77)[None]
+    dm = _to_dev_mask(m)
+    ts = TileMask(n, h, w, DEV)
+    ref = None
+    for _ in range(20):
+        ops.build_mask_tiles(dm, None, n, h, w, _lib.FOOT_CONV, 5, 1, 2, ts)
+        tiles = ts.active_tiles().cpu().numpy()
+        if ref is None:
+            ref = tiles
+        assert np.array_equal(tiles, ref)
+        assert ts.stale_tiles().numel() == 0

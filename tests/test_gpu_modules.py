@@ -1,0 +1,200 @@
+"""GPU parity of the drop-in module surface (mask_incr_modules / mask_incr_functional)
+and of E2Depth-incr against the CPU oracle.  The first two tests mirror the
+reference's own tests/test_pointops.py."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from maskedincrementeval_amd import _lib, ops
+from maskedincrementeval_amd import mask_incr_functional as mf
+from maskedincrementeval_amd import mask_incr_modules as mm
+from maskedincrementeval_amd.e2depth_incr import ConvLSTMIncr, E2VIDRecurrentIncr
+from maskedincrementeval_amd.masked_types import TileMask
+from maskedincrementeval_amd.synthetic import (event_voxel_delta, gaussian_delta, he_normal_conv_weight,
+                                               seed_module_)
+from oracle import incr_oracle as io
+from oracle import mask_oracle as mo
+from oracle.e2depth_oracle import E2DepthOracle
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+RTOL, ATOL = 1e-4, 1e-5
+
+
+def _cl(t):
+    return t.to(DEV).contiguous(memory_format=torch.channels_last)
+
+
+def _close(got, ref, what="", rtol=RTOL, atol=ATOL):
+    got = got.detach().cpu()
+    err = (got - ref).abs().max().item()
+    assert torch.allclose(got, ref, rtol=rtol, atol=atol), "%s max|diff| = %.3e" % (what, err)
+
+
+def test_accumulate_incr_like_reference():
+    # tests/test_pointops.py:11-22, as a 4-D tensor (1, 1, 40, 80)
+    shape = (1, 1, 40, 80)
+    X = torch.randn(shape, generator=torch.Generator().manual_seed(0))
+    incr = torch.randn(shape, generator=torch.Generator().manual_seed(1))
+    zz = torch.relu(X + incr) - torch.relu(X)
+    act = mm.nnReluIncr()
+    act.forward_refresh_reservoirs(_cl(X))
+    out = act([_cl(incr), None])
+    torch.cuda.synchronize()
+    assert torch.count_nonzero(out[0].cpu() - zz) == 0, "output check"
+    assert torch.count_nonzero(X + incr - act.in_res.reservoir.cpu()) == 0, "incremented_input"
+    assert isinstance(out[1], TileMask)
+
+
+def test_convkxkincr_functional_like_reference():
+    # tests/test_pointops.py:25-35: nnConvIncr(3,5,3,1,1,bias=False), 1x3x25x25, all-ones mask
+    c = mm.nnConvIncr(3, 5, 3, 1, 1, bias=False).to(device=DEV).eval()
+    x = _cl(torch.randn([1, 3, 25, 25], generator=torch.Generator().manual_seed(2)))
+    with torch.no_grad():
+        out_base = c.forward_refresh_reservoirs(x.contiguous())
+        out = c((x, torch.ones_like(x, dtype=bool)))
+    torch.cuda.synchronize()
+    # the reference asserts bit equality against cuDNN; two different summation orders can only
+    # be held to fp32 round-off
+    _close(out[0], out_base.cpu(), "output check", rtol=1e-5, atol=1e-6)
+    _close(out[0], io.conv_incr(x.cpu(), c.weight.detach().cpu(), 1, 1), "vs oracle", rtol=1e-5, atol=1e-6)
+
+
+def test_functional_ops_match_oracle():
+    n, c, h, w = 1, 16, 30, 38
+    d, m = gaussian_delta(n, c, h, w, 0.1, 0.5, seed=3)
+    wt = he_normal_conv_weight(32, c, 3, seed=4)
+    filt = wt.permute(1, 2, 3, 0).contiguous().to(DEV)
+    out = mf.conv2d_from_module([_cl(d), _cl(m.float()).to(torch.uint8)], filt, stride=(2, 2), padding=(1, 1))
+    _close(out[0], io.conv_incr(d, wt, 2, 1), "conv2d_from_module")
+    assert np.array_equal(out[1].pixmask[:, 0].cpu().numpy(), mo.footprint_conv(m[:, 0].numpy(), 3, 2, 1))
+    up = mf.interpolate_from_module([_cl(d), m.to(DEV)])
+    _close(up[0], io.interp_incr(d), "interpolate_from_module")
+    tc = torch.nn.ConvTranspose2d(c, 8, 3, stride=2, padding=1, output_padding=1).to(DEV)
+    tout = mf.transposed_conv2d_from_module([_cl(d), m.to(DEV)], tc)
+    _close(tout[0], io.tconv_incr(d, tc.weight.detach().cpu(), 2, 1, 1), "transposed_conv2d_from_module")
+    bn = torch.nn.BatchNorm2d(c).to(DEV).eval()
+    bn.running_var.uniform_(0.5, 2.0)
+    bn.weight.data.normal_()
+    bout = mf.bn2d_from_module([_cl(d), None], bn)
+    _close(bout[0], io.bn_incr(d, bn.running_var.cpu(), bn.weight.detach().cpu(), bn.eps), "bn2d_from_module")
+    r1, r2 = mf.IncrementReserve(_cl(torch.randn(n, c, h, w))), mf.IncrementReserve(_cl(torch.randn(n, c, h, w)))
+    d2, m2 = gaussian_delta(n, c, h, w, 0.05, 0.5, seed=5)
+    keep = r1.reservoir.clone()
+    pm = mf.IncrPointwiseMultiply([_cl(d), m.to(DEV)], r1, [_cl(d2), m2.to(DEV)], r2)
+    ref = (d2 + r2.reservoir.cpu()) * d + r1.reservoir.cpu() * d2
+    _close(pm[0], ref, "IncrPointwiseMultiply")
+    assert torch.equal(keep, r1.reservoir)
+
+
+@pytest.mark.parametrize("density", [0.01, 0.05, 0.20])
+def test_config2_activation_chain_50_steps(density):
+    """Benchmark configuration 2: 1x64x132x176, conv3x3 64->64 -> incremental LeakyReLU(0.01)
+    -> incremental ReLU, 50 steps with a fresh mask each step: emitted masks exact (staged on
+    the GPU reservoirs), drift against a dense recompute at steps 1 and 50."""
+    n, c, h, w = 1, 64, 132, 176
+    conv = mm.nnConvIncr(c, c, 3, 1, 1).to(DEV).eval()
+    seed_module_(conv, 11)
+    leaky = mm.nnReservedActivation(mm.leaky_relu_op(0.01))
+    relu = mm.nnReservedActivation(torch.relu)
+    x = torch.randn(n, c, h, w, generator=torch.Generator().manual_seed(12))
+    wt, b = conv.weight.detach().cpu(), conv.bias.detach().cpu()
+    with torch.no_grad():
+        y = relu.forward_refresh_reservoirs(leaky.forward_refresh_reservoirs(conv.forward_refresh_reservoirs(_cl(x))))
+    acc = y.clone()
+    o_leaky, o_relu = io.Reserve(io.conv_refresh(x, wt, b, 1, 1)), io.Reserve(None)
+    o_relu.update_reservoir(io.leaky_relu(o_leaky.reservoir))
+    acc_ref = torch.relu(o_relu.reservoir)
+    _close(acc, acc_ref, "refresh")
+    for step in range(50):
+        d, m = gaussian_delta(n, c, h, w, density, 0.2, seed=2000 + step)
+        r_leaky_old = leaky.in_res.reservoir.clone()
+        r_relu_old = relu.in_res.reservoir.clone()
+        with torch.no_grad():
+            a = conv([_cl(d), m.to(DEV)])
+            bq = leaky(a)
+            out = relu(bq)
+        torch.cuda.synchronize()
+        ref = io.act_incr(torch.relu, o_relu, io.act_incr(io.leaky_relu, o_leaky, io.conv_incr(d, wt, 1, 1)))
+        x = x + d
+        acc += out[0]
+        acc_ref += ref
+        if step in (0, 49):
+            _close(out[0], ref, "step %d delta" % step)
+            dense = torch.relu(io.leaky_relu(io.conv_refresh(x, wt, b, 1, 1)))
+            _close(acc, dense, "step %d accumulated vs dense recompute" % step)
+            _close(leaky.in_res.reservoir, o_leaky.reservoir, "step %d reservoir" % step)
+        # structural mask of the conv: exact
+        assert np.array_equal(a[1].pixmask[:, 0].cpu().numpy(), mo.footprint_conv(m[:, 0].numpy(), 3, 1, 1))
+        assert np.array_equal(a[1].active_tiles().cpu().numpy(), mo.tile_list(a[1].pixmask[:, 0].cpu().numpy()))
+        # emitted masks, staged on the GPU-produced reservoir pairs: exact
+        lk = lambda t: F.leaky_relu(t, 0.01)
+        want1 = ((lk(leaky.in_res.reservoir) - lk(r_leaky_old)) != 0).any(1, keepdim=True) & a[1].pixmask.bool()
+        assert torch.equal(bq[1].pixmask.bool(), want1)
+        want2 = ((torch.relu(relu.in_res.reservoir) - torch.relu(r_relu_old)) != 0).any(1, keepdim=True) & want1
+        assert torch.equal(out[1].pixmask.bool(), want2)
+    _close(acc, acc_ref, "accumulated after 50 steps")
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_convlstm_module_matches_oracle(fused):
+    n, cin, hid, h, w = 1, 16, 16, 26, 34
+    cell = ConvLSTMIncr(cin, hid, 3, fused=fused).to(DEV).eval()
+    seed_module_(cell, 21)
+    ref = io.ConvLSTMOracle(cell.Gates.weight.detach().cpu(), cell.Gates.bias.detach().cpu(), hid)
+    x0 = torch.randn(n, cin, h, w, generator=torch.Generator().manual_seed(22))
+    with torch.no_grad():
+        h_d, c_d = cell.forward_refresh_reservoirs(_cl(x0), None)
+    h_r, c_r = ref.refresh(x0)
+    _close(h_d, h_r, "refresh h"), _close(c_d, c_r, "refresh c")
+    for step in range(4):
+        d, m = gaussian_delta(n, cin, h, w, 0.08, 0.3, seed=2300 + step)
+        with torch.no_grad():
+            dh, dc = cell([_cl(d), m.to(DEV)], None)
+        torch.cuda.synchronize()
+        dh_r, dc_r = ref.incr(d)
+        _close(dh[0], dh_r, "dh %d" % step), _close(dc[0], dc_r, "dc %d" % step)
+
+
+def _run_e2depth(h, w, steps, density, fuse, seed=31):
+    model = seed_module_(E2VIDRecurrentIncr(fuse=fuse), seed=seed).to(DEV).eval()
+    oracle = E2DepthOracle(model.state_dict())
+    x0 = torch.randn(1, 5, h, w, generator=torch.Generator().manual_seed(seed + 1)) * 0.5
+    with torch.no_grad():
+        acc = model.forward_refresh_reservoirs(_cl(x0), None)[0].clone()
+    acc_ref = oracle.refresh(x0)
+    _close(acc, acc_ref, "refresh", atol=5e-5)
+    x = x0.clone()
+    for step in range(steps):
+        d, m = event_voxel_delta(1, 5, h, w, density, seed=3000 + step)
+        with torch.no_grad():
+            out, states = model([_cl(d), None], None)      # the reference drivers pass mask None
+        torch.cuda.synchronize()
+        ref = oracle.incr(d)
+        _close(out[0], ref, "step %d" % step)
+        acc += out[0]
+        acc_ref += ref
+        x += d
+        # input mask and head tile list: exact against the oracle definitions
+        pm = mo.pixel_mask(d.numpy(), 0.0)
+        assert np.array_equal(pm, m[:, 0].numpy())
+        head_ts = model.unetrecurrent.head.conv2d._tile_set("out_act" if fuse else "out", 1, h, w, torch.device(DEV))
+        assert np.array_equal(head_ts.active_tiles().cpu().numpy(), mo.tile_list(mo.footprint_conv(pm, 5, 1, 2)))
+    _close(acc, acc_ref, "accumulated")
+    return model, acc, x
+
+
+@pytest.mark.parametrize("fuse", [True, False])
+def test_e2depth_incr_small_matches_oracle(fuse):
+    _run_e2depth(72, 104, steps=4, density=0.05, fuse=fuse)
+
+
+def test_e2depth_incr_full_size_matches_oracle_and_dense():
+    # benchmark configuration 3 at its real size (264x352, 5 %): per-step parity for a few steps,
+    # then refresh + sum of increments == dense forward on the last input (tests/test_network.py:24-31)
+    model, acc, x = _run_e2depth(264, 352, steps=3, density=0.05, fuse=True)
+    fresh = seed_module_(E2VIDRecurrentIncr(), seed=31).to(DEV).eval()
+    with torch.no_grad():
+        dense = fresh.forward_refresh_reservoirs(_cl(x), None)[0]
+    _close(acc, dense.cpu(), "refresh + increments vs dense", atol=5e-5)

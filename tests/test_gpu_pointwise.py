@@ -1,0 +1,183 @@
+"""GPU parity of the point-wise incremental kernels against the CPU oracle, through the
+C ABI: activation increments (ReLU / LeakyReLU bit-exact, sigmoid / tanh within
+rtol 1e-4 / atol 1e-5), product rule, sum, bilinear x2, fused ConvLSTM gates."""
+import numpy as np
+import pytest
+import torch
+
+from maskedincrementeval_amd import _lib, ops
+from maskedincrementeval_amd.masked_types import TileMask
+from maskedincrementeval_amd.synthetic import gaussian_delta
+from oracle import incr_oracle as io
+from oracle import mask_oracle as mo
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+RTOL, ATOL = 1e-4, 1e-5
+
+
+def _dev(t):
+    return ops.as_nhwc(t.to(DEV).contiguous(memory_format=torch.channels_last))
+
+
+def _close(got, ref, what=""):
+    got = got.cpu()
+    err = (got - ref).abs().max().item()
+    assert torch.allclose(got, ref, rtol=RTOL, atol=ATOL), "%s max|diff| = %.3e" % (what, err)
+
+
+def _identity_ts(ts, mask, n, h, w):
+    ops.build_mask_tiles(None if mask is None else mask.to(DEV), None, n, h, w, _lib.FOOT_CONV, 1, 1, 0, ts)
+    return ts
+
+
+def _randn(*shape, seed):
+    return torch.randn(shape, generator=torch.Generator().manual_seed(seed))
+
+
+@pytest.mark.parametrize("kind,slope,op,exact", [
+    (_lib.ACT_RELU, 0.0, torch.relu, True),
+    (_lib.ACT_LEAKY_RELU, 0.01, io.leaky_relu, True),
+    (_lib.ACT_SIGMOID, 0.0, torch.sigmoid, False),
+    (_lib.ACT_TANH, 0.0, torch.tanh, False)])
+@pytest.mark.parametrize("n,c,h,w", [(1, 32, 45, 61), (2, 5, 19, 23), (1, 1, 16, 24)])
+def test_activation_increment(kind, slope, op, exact, n, c, h, w):
+    r0 = _randn(n, c, h, w, seed=c)
+    res_cpu, res_gpu = io.Reserve(r0), _dev(r0.clone())
+    ts = TileMask(n, h, w, DEV)
+    out = ops.new_nhwc(n, c, h, w, DEV)
+    refined = torch.zeros((n, 1, h, w), dtype=torch.uint8, device=DEV)
+    for step in range(4):
+        d, m = gaussian_delta(n, c, h, w, 0.1, 0.7, seed=100 + step + h)
+        _identity_ts(ts, m, n, h, w)
+        r_old = res_gpu.cpu().clone()
+        ops.act_incr(kind, slope, _dev(d), res_gpu, out, ts, refined)
+        torch.cuda.synchronize()
+        ref = io.act_incr(op, res_cpu, d)
+        if exact:
+            # reference tests/test_pointops.py:17-22: zero differing elements, reservoir == X + d
+            assert torch.count_nonzero(out.cpu() - ref) == 0
+            assert torch.count_nonzero(res_gpu.cpu() - res_cpu.reservoir) == 0
+        else:
+            _close(out, ref, "delta")
+            _close(res_gpu, res_cpu.reservoir, "reservoir")
+        # emitted mask, staged on the GPU-produced reservoir pair: exact integer function
+        r_new = res_gpu.cpu()
+        want = ((op(r_new) - op(r_old)) != 0).any(dim=1, keepdim=True) & m.bool()
+        if exact:
+            assert np.array_equal(refined.cpu().numpy(), want.to(torch.uint8).numpy())
+        assert np.array_equal(refined.cpu().numpy(),
+                              (out.cpu() != 0).any(dim=1, keepdim=True).to(torch.uint8).numpy())
+
+
+def test_activation_zero_delta_and_keep_reservoir():
+    n, c, h, w = 1, 16, 24, 24
+    r0 = _randn(n, c, h, w, seed=1)
+    res = _dev(r0.clone())
+    ts = _identity_ts(TileMask(n, h, w, DEV), None, n, h, w)
+    out = ops.new_nhwc(n, c, h, w, DEV)
+    ops.act_incr(_lib.ACT_TANH, 0.0, _dev(torch.zeros(n, c, h, w)), res, out, ts)
+    assert torch.count_nonzero(out) == 0 and torch.equal(res.cpu(), r0)
+    d = _randn(n, c, h, w, seed=2)
+    ops.act_incr(_lib.ACT_RELU, 0.0, _dev(d), res, out, ts, keep_reservoir=True)
+    assert torch.equal(res.cpu(), r0)                       # NonlinearPointOpIncr.forward: no accumulate
+    assert torch.equal(out.cpu(), torch.relu(r0 + d) - torch.relu(r0))
+
+
+@pytest.mark.parametrize("n,c,h,w", [(1, 64, 33, 44), (2, 3, 17, 9)])
+def test_product_rule(n, c, h, w):
+    r1, r2 = _randn(n, c, h, w, seed=3), _randn(n, c, h, w, seed=4)
+    R1, R2 = io.Reserve(r1), io.Reserve(r2)
+    g1, g2 = _dev(r1.clone()), _dev(r2.clone())
+    ts = TileMask(n, h, w, DEV)
+    out = ops.new_nhwc(n, c, h, w, DEV)
+    for step in range(3):
+        d1, m1 = gaussian_delta(n, c, h, w, 0.08, 0.3, seed=200 + step)
+        d2, m2 = gaussian_delta(n, c, h, w, 0.05, 0.3, seed=300 + step)
+        ops.build_mask_tiles(m1.to(DEV), m2.to(DEV), n, h, w, _lib.FOOT_CONV, 1, 1, 0, ts)
+        ops.mul_incr(_dev(d1), m1.to(DEV), g1, _dev(d2), m2.to(DEV), g2, out, ts)
+        torch.cuda.synchronize()
+        _close(out, io.mul_incr(d1, R1, d2, R2), "product")
+        _close(g1, R1.reservoir), _close(g2, R2.reservoir)
+        union = (m1 | m2).bool()
+        assert torch.count_nonzero(out.cpu() * (~union)) == 0
+    # bare IncrPointwiseMultiply: reservoirs untouched
+    before = g1.cpu().clone()
+    ops.mul_incr(_dev(d1), m1.to(DEV), g1, _dev(d2), m2.to(DEV), g2, out, ts, keep_reservoir=True)
+    assert torch.equal(g1.cpu(), before)
+
+
+def test_sum_of_deltas():
+    n, c, h, w = 2, 32, 21, 35
+    ts = TileMask(n, h, w, DEV)
+    out = ops.new_nhwc(n, c, h, w, DEV)
+    for step in range(3):
+        a, ma = gaussian_delta(n, c, h, w, 0.07, 1.0, seed=400 + step)
+        b, mb = gaussian_delta(n, c, h, w, 0.04, 1.0, seed=500 + step)
+        ops.build_mask_tiles(ma.to(DEV), mb.to(DEV), n, h, w, _lib.FOOT_CONV, 1, 1, 0, ts)
+        nan = float("nan")
+        pa = torch.where(ma.bool().expand_as(a), a, torch.full_like(a, nan))
+        ops.add_incr(_dev(pa), ma.to(DEV), _dev(b), mb.to(DEV), out, ts)
+        torch.cuda.synchronize()
+        assert torch.equal(out.cpu(), a + b)
+
+
+@pytest.mark.parametrize("n,c,h,w", [(1, 64, 33, 44), (2, 5, 7, 5), (1, 8, 1, 1)])
+def test_bilinear_up2x_with_skip_sum(n, c, h, w):
+    ts = TileMask(n, 2 * h, 2 * w, DEV)
+    out = ops.new_nhwc(n, c, 2 * h, 2 * w, DEV)
+    for step in range(3):
+        a, ma = gaussian_delta(n, c, h, w, 0.15, 1.0, seed=600 + step)
+        b, mb = gaussian_delta(n, c, h, w, 0.10, 1.0, seed=700 + step)
+        ops.build_mask_tiles(ma.to(DEV), mb.to(DEV), n, h, w, _lib.FOOT_UP2X, 0, 0, 0, ts)
+        ops.upsample2x_incr(_dev(a), ma.to(DEV), _dev(b), mb.to(DEV), ts, out)
+        torch.cuda.synchronize()
+        _close(out, io.interp_incr(a + b), "up2x(a+b)")
+        fp = torch.from_numpy(mo.footprint_up2x((ma | mb)[:, 0].numpy())).bool().unsqueeze(1)
+        assert torch.count_nonzero(out.cpu() * (~fp)) == 0
+    ops.build_mask_tiles(ma.to(DEV), None, n, h, w, _lib.FOOT_UP2X, 0, 0, 0, ts)
+    ops.upsample2x_incr(_dev(a), ma.to(DEV), None, None, ts, out)
+    torch.cuda.synchronize()
+    _close(out, io.interp_incr(a), "up2x(a)")
+
+
+@pytest.mark.parametrize("hid,h,w,with_prev", [(64, 33, 44, False), (16, 19, 27, True), (3, 9, 9, True)])
+def test_fused_convlstm_gates_match_module_chain(hid, h, w, with_prev):
+    """Gate chain of ConvLSTMIncr.forward (e2depth_incr.py:103-117) in one kernel vs the
+    oracle's module-by-module chain; reservoirs are set up from a dense refresh."""
+    n = 1
+    cin = hid
+    wgt = _randn(4 * hid, cin + hid, 3, 3, seed=5) * (0.5 / (cin * 9) ** 0.5)
+    bias = _randn(4 * hid, seed=6) * 0.1
+    cell = io.ConvLSTMOracle(wgt, bias, hid)
+    x0, h0, c0 = _randn(n, cin, h, w, seed=7), _randn(n, hid, h, w, seed=8), _randn(n, hid, h, w, seed=9)
+    cell.refresh(x0, (h0, c0))
+    gates_res = _dev(torch.cat([cell.r[k].reservoir for k in ("sig1", "sig2", "sig3", "tanh1")], 1))
+    cprev_res = _dev(cell.r["m2b"].reservoir.clone())
+    cell_res = _dev(cell.r["tanh2"].reservoir.clone())
+    ts = TileMask(n, h, w, DEV)
+    dh = ops.new_nhwc(n, hid, h, w, DEV)
+    dc = ops.new_nhwc(n, hid, h, w, DEV)
+    acc_h, acc_h_ref = torch.zeros(n, hid, h, w), torch.zeros(n, hid, h, w)
+    for step in range(5):
+        dx, mx = gaussian_delta(n, cin, h, w, 0.1, 0.3, seed=800 + step)
+        prev = None
+        if with_prev:
+            dhp, mh = gaussian_delta(n, hid, h, w, 0.05, 0.2, seed=900 + step)
+            dcp, _ = gaussian_delta(n, hid, h, w, 0.05, 0.2, seed=900 + step)   # same mask as dhp
+            dcp = dcp * 0.5
+            prev = (dhp, dcp)
+        gates_delta = io.conv_incr(torch.cat((dx, prev[0] if prev else torch.zeros(n, hid, h, w)), 1), wgt, 1, 1)
+        gmask = torch.from_numpy(mo.footprint_conv(((mx | mh) if with_prev else mx)[:, 0].numpy(), 3, 1, 1)).unsqueeze(1)
+        _identity_ts(ts, gmask, n, h, w)
+        ops.convlstm_gates_incr(_dev(gates_delta), gates_res, _dev(prev[1]) if prev else None,
+                                mh.to(DEV) if prev else None, cprev_res, cell_res, dh, dc, ts)
+        torch.cuda.synchronize()
+        dh_ref, dc_ref = cell.incr(dx, prev)
+        _close(dh, dh_ref, "dh step %d" % step)
+        _close(dc, dc_ref, "dc step %d" % step)
+        acc_h += dh.cpu()
+        acc_h_ref += dh_ref
+    _close(acc_h, acc_h_ref, "accumulated hidden")
+    _close(cell_res, cell.r["tanh2"].reservoir, "cell reservoir")
+    _close(gates_res[:, :hid], cell.r["sig1"].reservoir, "in-gate reservoir")
