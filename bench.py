@@ -1,0 +1,311 @@
+#!/usr/bin/env python3
+"""Benchmark of the masked incremental inference path on one MI355X.
+
+Workload (the configuration the headline metric is quoted on): E2Depth-incr,
+random-init weights, one event stream of 5x264x352 voxel grids, one dense
+refresh, then incremental steps with 5 % of the pixels carrying a delta
+(Poisson(2) event counts x random polarity x 0.1 per bin, smooth blob masks).
+A "step" is one incremental frame through the whole network; the deltas are
+resident in HBM before the timed region starts and the step is replayed from
+a HIP graph.
+
+Prints ONE JSON line: frames/s (`value`), ms/frame, the roofline of the
+dominant kernel launch (the masked conv layer that takes the most time,
+timed with HIP events on the stream it runs on), a per-layer table, the same
+network run densely through the same kernels (all tiles active), and the CPU
+baseline (the torch-CPU oracle of the reference path on the host cores).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--density", type=float, default=0.05)
+    ap.add_argument("--height", type=int, default=264)
+    ap.add_argument("--width", type=int, default=352)
+    ap.add_argument("--cpu-steps", type=int, default=12, help="incremental steps of the CPU baseline (0 = skip)")
+    ap.add_argument("--no-graph", action="store_true", help="launch kernels eagerly instead of replaying a HIP graph")
+    ap.add_argument("--no-dense", action="store_true", help="skip the all-tiles-active comparator")
+    ap.add_argument("--layer-iters", type=int, default=20, help="timed launches per layer for the roofline table")
+    return ap.parse_args()
+
+
+class LayerProbe:
+    """Times every conv / point-wise entry point of one eager step with HIP events recorded
+    on the stream the kernels are launched on, and derives algorithmic bytes / flops from the
+    tile-set statistics of that step."""
+
+    def __init__(self, ops, torch):
+        self.ops, self.torch = ops, torch
+        self.records = []
+        self._orig = {}
+
+    def _wrap(self, name, describe):
+        orig = getattr(self.ops, name)
+        self._orig[name] = orig
+        torch = self.torch
+
+        def wrapped(*a, **kw):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            r = orig(*a, **kw)
+            e1.record()
+            self.records.append([name, describe(*a, **kw), e0, e1])
+            return r
+        setattr(self.ops, name, wrapped)
+
+    def __enter__(self):
+        def conv_desc(x, xmask, x2, x2mask, filt, k, stride, pad, out_ts, out_delta, reservoir=None, *a, **kw):
+            n, c1, h, w = x.shape
+            c2 = 0 if x2 is None else x2.shape[1]
+            return dict(kind="conv", k=k, s=stride, cin=c1 + c2, cout=filt.shape[3], h=h, w=w, n=n,
+                        xmask=xmask, x2mask=x2mask, ts=out_ts, fused=reservoir is not None)
+
+        def pw_desc(kind, nin, nres):
+            def d(*a, **kw):
+                ts = [t for t in a if hasattr(t, "pixmask") and hasattr(t, "tiles")][-1]
+                t0 = [t for t in a if hasattr(t, "shape") and len(getattr(t, "shape", ())) == 4][0]
+                return dict(kind=kind, c=t0.shape[1], ts=ts, nin=nin, nres=nres)
+            return d
+        self._wrap("conv_masked", conv_desc)
+        self._wrap("act_incr", pw_desc("act", 1, 1))
+        self._wrap("add_incr", pw_desc("add", 2, 0))
+        self._wrap("mul_incr", pw_desc("mul", 2, 2))
+        self._wrap("upsample2x_incr", pw_desc("up2x", 2, 0))
+        self._wrap("convlstm_gates_incr", pw_desc("gates", 4, 6))
+        self._wrap("build_mask_tiles", lambda *a, **kw: dict(kind="tiles", ts=a[-1]))
+        self._wrap("mask_from_delta", lambda d, t, o: dict(kind="mask", c=d.shape[1], npix=d.shape[0] * d.shape[2] * d.shape[3]))
+        return self
+
+    def __exit__(self, *exc):
+        for name, orig in self._orig.items():
+            setattr(self.ops, name, orig)
+
+    def table(self):
+        """One row per launch: ms, algorithmic bytes and flops (counted once per step)."""
+        self.torch.cuda.synchronize()
+        rows = []
+        for name, d, e0, e1 in self.records:
+            ms = e0.elapsed_time(e1)
+            row = dict(op=name, ms=ms)
+            if d["kind"] == "conv":
+                ts = d["ts"]
+                P = d["n"] * d["h"] * d["w"]
+                a_in = P if d["xmask"] is None else int(self._pix(d["xmask"]).sum().item())
+                a_out = int(ts.pixmask.sum().item())
+                cin, cout, k = d["cin"], d["cout"], d["k"]
+                byts = P + a_in * cin * 4 + a_out * cout * 4 + cin * cout * k * k * 4 + ts.capacity * 4
+                if d["fused"]:
+                    byts += 2 * a_out * cout * 4
+                row.update(shape="%dx%d s%d %d->%d @%dx%d" % (k, k, d["s"], cin, cout, ts.h, ts.w),
+                           active_tiles=int(ts.counts[0].item()), tiles=ts.capacity, a_out=a_out,
+                           bytes=byts, flops=2 * a_out * cin * cout * k * k)
+            elif d["kind"] in ("act", "add", "mul", "up2x", "gates"):
+                ts = d["ts"]
+                a = int(ts.pixmask.sum().item())
+                c = d["c"]
+                if d["kind"] == "gates":
+                    hid = c // 4
+                    byts = a * (4 * hid * 4 + 2 * 4 * hid * 4 + 2 * hid * 4 + hid * 4 + 2 * hid * 4)
+                else:
+                    byts = a * c * 4 * (d["nin"] + 2 * d["nres"] + 1)
+                byts += ts.n * ts.h * ts.w
+                row.update(shape="%s C=%d @%dx%d" % (d["kind"], c, ts.h, ts.w), a_out=a, bytes=byts, flops=0,
+                           active_tiles=int(ts.counts[0].item()), tiles=ts.capacity)
+            elif d["kind"] == "tiles":
+                ts = d["ts"]
+                row.update(shape="tiles @%dx%d" % (ts.h, ts.w), bytes=2 * ts.n * ts.h * ts.w + ts.capacity * 8, flops=0)
+            else:
+                row.update(shape="mask C=%d" % d["c"], bytes=d["npix"] * (d["c"] * 4 + 1), flops=0)
+            rows.append(row)
+        return rows
+
+    @staticmethod
+    def _pix(m):
+        return m.pixmask if hasattr(m, "pixmask") else m
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures ONE GPU (independent event streams shard one per GPU with "
+              "no communication); --gpus %d is not run." % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from maskedincrementeval_amd import _lib, ops
+    from maskedincrementeval_amd.e2depth_incr import E2VIDRecurrentIncr
+    from maskedincrementeval_amd.synthetic import event_voxel_delta, seed_module_
+
+    _lib.lib()   # fail loudly if the HIP library is missing
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    H, W, dens = args.height, args.width, args.density
+    cl = lambda t: t.to(dev).contiguous(memory_format=torch.channels_last)
+
+    model = seed_module_(E2VIDRecurrentIncr(), seed=1).to(dev).eval()
+    x0 = torch.randn(1, 5, H, W, generator=torch.Generator().manual_seed(2)) * 0.5
+    n_inputs = 16
+    deltas_cpu = [event_voxel_delta(1, 5, H, W, dens, seed=3000 + i)[0] for i in range(n_inputs)]
+    deltas = [cl(d) for d in deltas_cpu]
+    static_in = cl(torch.zeros(1, 5, H, W))
+
+    def step_eager(m, i):
+        static_in.copy_(deltas[i % n_inputs])
+        return m([static_in, None], None)
+
+    def timed_run(m, tag):
+        with torch.no_grad():
+            m.forward_refresh_reservoirs(cl(x0), None)
+            for i in range(max(args.warmup, 3)):           # also allocates every persistent buffer
+                step_eager(m, i)
+            torch.cuda.synchronize()
+            graph = None
+            if not args.no_graph:
+                side = torch.cuda.Stream()
+                side.wait_stream(torch.cuda.current_stream())
+                with torch.cuda.stream(side):
+                    step_eager(m, 0)
+                torch.cuda.current_stream().wait_stream(side)
+                torch.cuda.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    m([static_in, None], None)
+                for i in range(3):
+                    static_in.copy_(deltas[i % n_inputs])
+                    graph.replay()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for i in range(args.steps):
+                if graph is not None:
+                    static_in.copy_(deltas[i % n_inputs])
+                    graph.replay()
+                else:
+                    step_eager(m, i)
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+        print("[bench] %s: %.3f ms/frame over %d steps (%s)" % (tag, 1e3 * dt / args.steps, args.steps,
+              "eager" if graph is None else "HIP graph"), file=sys.stderr, flush=True)
+        return dt / args.steps
+
+    sec_per_step = timed_run(model, "incremental %.0f%%" % (100 * dens))
+
+    # ---- per-layer roofline table: eager launches with HIP events, several repeats ------------
+    with torch.no_grad():
+        model.forward_refresh_reservoirs(cl(x0), None)
+        step_eager(model, 0)
+        agg = None
+        for it in range(args.layer_iters):
+            with LayerProbe(ops, torch) as probe:
+                step_eager(model, 1 + it)
+            rows = probe.table()
+            if agg is None:
+                agg = rows
+                for r in agg:
+                    r["ms_sum"] = 0.0
+                    r["bytes_sum"] = 0
+                    r["flops_sum"] = 0
+            for r, q in zip(agg, rows):
+                r["ms_sum"] += q["ms"]
+                r["bytes_sum"] += q["bytes"]
+                r["flops_sum"] += q["flops"]
+    layers = []
+    for r in agg:
+        ms = r["ms_sum"] / args.layer_iters
+        byts, fl = r["bytes_sum"] / args.layer_iters, r["flops_sum"] / args.layer_iters
+        layers.append(dict(op=r["op"], shape=r["shape"], us=round(1e3 * ms, 2),
+                           gbs=round(byts / (ms * 1e-3) / 1e9, 1) if ms > 0 else None,
+                           tflops=round(fl / (ms * 1e-3) / 1e12, 2) if ms > 0 else None,
+                           bytes=int(byts), flops=int(fl), active_tiles=r.get("active_tiles"), tiles=r.get("tiles")))
+    convs = [l for l in layers if l["op"] == "conv_masked"]
+    dom = max(convs, key=lambda l: l["us"])
+    mfma_bound = dom["flops"] / max(dom["bytes"], 1) > PEAK_FP32_MFMA_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9)
+    if mfma_bound:
+        roofline = dict(bound="mfma", achieved=dom["tflops"], peak=PEAK_FP32_MFMA_TFLOPS, unit="TFLOP/s",
+                        frac=round(dom["tflops"] / PEAK_FP32_MFMA_TFLOPS, 4), traffic=None)
+    else:
+        roofline = dict(bound="hbm", achieved=dom["gbs"], peak=PEAK_HBM_GBS, unit="GB/s",
+                        frac=round(dom["gbs"] / PEAK_HBM_GBS, 4), traffic=None)
+    roofline.update(kernel="mie_conv_masked %s" % dom["shape"], us=dom["us"],
+                    algorithmic_bytes=dom["bytes"], algorithmic_flops=dom["flops"])
+    tot_us = sum(l["us"] for l in layers)
+    tot_bytes = sum(l["bytes"] for l in layers)
+    tot_flops = sum(l["flops"] for l in layers)
+    print("[bench] per-launch table (eager, HIP events, mean of %d steps):" % args.layer_iters, file=sys.stderr)
+    for l in layers:
+        print("[bench]   %-22s %-34s %9.2f us %8s GB/s %7s TFLOP/s  tiles %s/%s" % (
+            l["op"], l["shape"], l["us"], l["gbs"], l["tflops"], l["active_tiles"], l["tiles"]), file=sys.stderr)
+    print("[bench]   sum of kernels %.1f us; algorithmic %.1f MB, %.2f GFLOP per frame" %
+          (tot_us, tot_bytes / 1e6, tot_flops / 1e9), file=sys.stderr, flush=True)
+
+    # ---- dense comparator: same kernels, every tile active ---------------------------------------
+    dense_sec = None
+    if not args.no_dense:
+        dense_model = seed_module_(E2VIDRecurrentIncr(derive_input_mask=False), seed=1).to(dev).eval()
+        dense_sec = timed_run(dense_model, "dense (all tiles active, same kernels)")
+        del dense_model
+
+    # ---- CPU baseline: the oracle (torch-CPU restatement of the reference path) -----------------
+    cpu = None
+    if args.cpu_steps > 0:
+        from oracle.e2depth_oracle import E2DepthOracle
+        torch.set_num_threads(min(os.cpu_count() or 1, 16))
+        oracle = E2DepthOracle(model.state_dict())
+        with torch.no_grad():
+            oracle.refresh(x0)
+            oracle.incr(deltas_cpu[0])
+            t0 = time.perf_counter()
+            for i in range(args.cpu_steps):
+                oracle.incr(deltas_cpu[(1 + i) % n_inputs])
+            cdt = (time.perf_counter() - t0) / args.cpu_steps
+        cpu = dict(value=round(1.0 / cdt, 3), unit="frames/s", cores=torch.get_num_threads(), kind="port",
+                   ms_per_step=round(1e3 * cdt, 2),
+                   sample="%d incremental steps of the same E2Depth-incr %dx%d workload (dense F.conv2d on the "
+                          "delta, as the reference executes it), torch-CPU fp32" % (args.cpu_steps, H, W))
+        print("[bench] cpu baseline: %.1f ms/frame on %d threads" % (1e3 * cdt, cpu["cores"]), file=sys.stderr, flush=True)
+
+    result = {
+        "metric": "incremental frames/s, E2Depth-incr 264x352 @5% delta density",
+        "value": round(1.0 / sec_per_step, 2),
+        "unit": "frames/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(1e3 * sec_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "E2Depth-incr recurrent UNet, random init, 1x5x%dx%d event voxel deltas, %.0f%% "
+                               "active pixels, 1 dense refresh then incremental steps" % (H, W, 100 * dens),
+                   "density": dens, "height": H, "width": W, "graph": not args.no_graph},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "hbm_frac_whole_frame": round(tot_bytes / sec_per_step / 1e9 / PEAK_HBM_GBS, 5),
+        "algorithmic_mb_per_frame": round(tot_bytes / 1e6, 2),
+        "algorithmic_gflop_per_frame": round(tot_flops / 1e9, 3),
+        "sum_kernel_us": round(tot_us, 1),
+        "dense_same_kernels_ms": None if dense_sec is None else round(1e3 * dense_sec, 4),
+        "speedup_vs_dense": None if dense_sec is None else round(dense_sec / sec_per_step, 3),
+        "layers": layers,
+    }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

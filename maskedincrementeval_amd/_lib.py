@@ -6,6 +6,12 @@ CPU fallback.  If the shared object is missing, `lib()` raises.
 import ctypes
 import os
 
+# torch must be imported before the library is loaded: the PyTorch-ROCm wheel ships its own
+# HIP runtime (soname libamdhip64.so.7); once it is mapped, the loader binds libmie_hip.so to
+# that same runtime, so both share one device context and one set of streams.  In the other
+# order the process ends up with two HIP runtimes and the second one finds no device.
+import torch  # noqa: F401  (import order matters, see above)
+
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "lib", "libmie_hip.so")
 

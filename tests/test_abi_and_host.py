@@ -210,3 +210,11 @@ def test_blob_mask_density_and_determinism():
     vals = torch.unique(ev * 10).round()
     assert (ev[:, :, m2[0, 0] == 0] == 0).all() and torch.allclose(ev * 10, (ev * 10).round(), atol=1e-5)
     assert vals.abs().max() >= 2
+
+
+def test_single_hip_runtime_is_mapped(mie_lib):
+    # libmie_hip.so must bind to the HIP runtime PyTorch-ROCm already loaded; two runtimes in one
+    # process leave the second one without a device
+    with open("/proc/self/maps") as f:
+        paths = {line.split()[-1] for line in f if "libamdhip64" in line}
+    assert len(paths) == 1, paths
