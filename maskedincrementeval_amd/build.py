@@ -13,7 +13,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_DIR = os.path.join(PKG_DIR, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libmie_hip.so")
-SOURCES = ["mie_mask.hip", "mie_pointwise.hip", "mie_conv.hip"]
+SOURCES = ["mie_mask.hip", "mie_pointwise.hip", "mie_conv.hip", "mie_conv_mfma.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
@@ -31,12 +31,7 @@ def find_hipcc():
     raise RuntimeError("hipcc not found (looked at $HIPCC, /opt/rocm/bin/hipcc, PATH)")
 
 
-def build_library(verbose=True):
-    """Compile every HIP source into lib/libmie_hip.so; returns its path."""
-    os.makedirs(LIB_DIR, exist_ok=True)
-    srcs = [os.path.join(CSRC, s) for s in SOURCES]
-    tmp = LIB_PATH + ".tmp"
-    cmd = [find_hipcc()] + HIPCC_FLAGS + srcs + ["-o", tmp]
+def _run(cmd, verbose):
     if verbose:
         print("[build]", " ".join(cmd), flush=True)
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -46,6 +41,26 @@ def build_library(verbose=True):
         raise RuntimeError("hipcc failed:\n" + out)
     if verbose and out.strip():
         print(out, flush=True)
+
+
+def build_library(verbose=True):
+    """Compile every HIP source (one hipcc process per file, in parallel) and link
+    lib/libmie_hip.so; returns its path."""
+    from concurrent.futures import ThreadPoolExecutor
+    os.makedirs(LIB_DIR, exist_ok=True)
+    obj_dir = os.path.join(LIB_DIR, "obj")
+    os.makedirs(obj_dir, exist_ok=True)
+    hipcc = find_hipcc()
+    compile_flags = [f for f in HIPCC_FLAGS if f != "-shared"]
+    jobs = []
+    for s in SOURCES:
+        obj = os.path.join(obj_dir, s.replace(".hip", ".o"))
+        jobs.append(([hipcc] + compile_flags + ["-c", os.path.join(CSRC, s), "-o", obj], obj))
+    with ThreadPoolExecutor(max_workers=min(len(jobs), 8)) as pool:
+        list(pool.map(lambda j: _run(j[0], verbose), jobs))
+    tmp = LIB_PATH + ".tmp"
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc"] + [j[1] for j in jobs] + ["-o", tmp],
+         verbose)
     os.replace(tmp, LIB_PATH)
     return LIB_PATH
 

@@ -1,0 +1,30 @@
+// Arguments shared by the masked-conv kernels (VALU paths in mie_conv.hip, matrix-core
+// path in mie_conv_mfma.hip).
+#pragma once
+#include "mie_common.h"
+
+struct ConvArgs {
+  const float* x; const uint8_t* xm; int c1;
+  const float* x2; const uint8_t* x2m; int c2;
+  int h_in, w_in;
+  const float* filt; int cin_total;
+  int pad, cout;
+  float* out; float* res; int act; float slope;
+  TileSetDev ts;
+};
+
+// Epilogue for one output element.
+static __device__ __forceinline__ void conv_store(const ConvArgs& a, long long off, float acc) {
+  if (a.res) {
+    const float r0 = a.res[off], r1 = r0 + acc;
+    a.res[off] = r1;
+    a.out[off] = mie_act(a.act, a.slope, r1) - mie_act(a.act, a.slope, r0);
+  } else {
+    a.out[off] = acc;
+  }
+}
+
+
+// Launches the matrix-core path for kernel size k (1,3,5,7) and stride s (1,2); the caller
+// has checked c1 % 8 == 0, c2 % 8 == 0 and cout % 32 == 0.
+void mie_launch_conv_mfma(const ConvArgs& a, int k, int s, unsigned cap, hipStream_t st);

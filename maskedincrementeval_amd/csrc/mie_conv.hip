@@ -1,40 +1,17 @@
 // Masked convolution of a delta over active 8x8 output tiles (gfx950).
 //
 // Three code paths, one per arithmetic regime:
-//   mfma    : Cin % 16 == 0 and Cout % 32 == 0 -- per-tile implicit GEMM on
-//             the fp32 matrix cores (v_mfma_f32_32x32x2_f32).  One wave owns
-//             one tile (M = 64 pixels) x 32*NB output channels; the input tile
-//             plus halo is staged in LDS 16 channels at a time, only where the
-//             input pixel mask is set; filter rows stream from L2.
+//   mfma    : Cin % 8 == 0 and Cout % 32 == 0 -- per-tile implicit GEMM on
+//             the fp32 matrix cores (mie_conv_mfma.hip).
 //   valu    : any shape -- thread = one output channel x 16 pixels, input tile
 //             staged in LDS and read as wave-wide broadcasts.
 //   smallco : Cout <= 4 (prediction / flow heads) -- thread = one pixel.
 // All paths share the epilogue: plain delta store, or the fused reservoir
 // update + activation increment.
 #include "mie_common.h"
+#include "mie_conv.h"
 
 namespace {
-
-struct ConvArgs {
-  const float* x; const uint8_t* xm; int c1;
-  const float* x2; const uint8_t* x2m; int c2;
-  int h_in, w_in;
-  const float* filt; int cin_total;
-  int pad, cout;
-  float* out; float* res; int act; float slope;
-  TileSetDev ts;
-};
-
-// Epilogue for one output element.
-__device__ __forceinline__ void conv_store(const ConvArgs& a, long long off, float acc) {
-  if (a.res) {
-    const float r0 = a.res[off], r1 = r0 + acc;
-    a.res[off] = r1;
-    a.out[off] = mie_act(a.act, a.slope, r1) - mie_act(a.act, a.slope, r0);
-  } else {
-    a.out[off] = acc;
-  }
-}
 
 // ---------------------------------------------------------------------------------
 // VALU path.  Block = 256 threads = 64 output channels x 4 pixel groups (two
@@ -155,124 +132,6 @@ __global__ __launch_bounds__(64) void k_conv_smallco(ConvArgs a) {
 }
 
 // ---------------------------------------------------------------------------------
-// MFMA path.  One wave (= one block of 64 threads) per (tile, 32*NB channels).
-//   A (64 pixels x k) comes from LDS: lanes 0-31 hold pixels, the lane half
-//   picks which 4 of the 8 input channels of a sub-chunk it reads as one
-//   ds_read_b128, so one read feeds four k-steps of v_mfma_f32_32x32x2_f32
-//   (k-step j multiplies channel j of the low half and channel 4+j of the
-//   high half).
-//   B (k x 32 channels) comes straight from the filter in L2: lane reads
-//   filt[ci][ky][kx][co0 + lane%32] -- 128-byte rows.
-// LDS row stride CC+4 floats keeps the 16-byte reads of 8 neighbouring pixels
-// on disjoint banks for stride 1 and 2.
-// ---------------------------------------------------------------------------------
-typedef float v16f __attribute__((ext_vector_type(16)));
-
-template <int K, int S, int NB>
-__global__ __launch_bounds__(64) void k_conv_mfma(ConvArgs a) {
-  constexpr int IT = 7 * S + K;
-  constexpr int CC = 16;
-  constexpr int LS = CC + 4;  // LDS floats per staged pixel
-  __shared__ __attribute__((aligned(16))) float s_in[IT * IT * LS];
-  int n, y0, x0;
-  const int tk = mie_pick_tile(a.ts, blockIdx.x, n, y0, x0);
-  if (tk == 0) return;
-  const int lane = threadIdx.x;
-  const int l32 = lane & 31, half = lane >> 5;
-  const int co0 = blockIdx.y * (32 * NB);
-  const int hout = a.ts.h, wout = a.ts.w;
-
-  v16f acc[2][NB];
-#pragma unroll
-  for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[mb][nb][r] = 0.f;
-
-  if (tk == 1) {
-    const int iy0 = y0 * S - a.pad, ix0 = x0 * S - a.pad;
-    // LDS pixel index of this lane's output pixel in m-block mb, tap (0,0)
-    int pbase[2];
-#pragma unroll
-    for (int mb = 0; mb < 2; ++mb) {
-      const int p = mb * 32 + l32;
-      pbase[mb] = ((p >> 3) * S) * IT + (p & 7) * S;
-    }
-    for (int src = 0; src < 2; ++src) {
-      const float* xin = src ? a.x2 : a.x;
-      const uint8_t* xm = src ? a.x2m : a.xm;
-      const int cs = src ? a.c2 : a.c1;
-      const int fbase = src ? a.c1 : 0;
-      if (xin == nullptr || cs == 0) continue;
-      for (int ci0 = 0; ci0 < cs; ci0 += CC) {
-        // stage IT*IT pixels x CC channels (float4 slots), zero where masked
-        for (int idx = lane; idx < IT * IT * (CC / 4); idx += 64) {
-          const int pix = idx / (CC / 4), q4 = idx % (CC / 4);
-          const int iy = iy0 + pix / IT, ix = ix0 + pix % IT;
-          float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-          if (iy >= 0 && iy < a.h_in && ix >= 0 && ix < a.w_in) {
-            const long long po = ((long long)n * a.h_in + iy) * a.w_in + ix;
-            if (xm == nullptr || xm[po])
-              v = *reinterpret_cast<const float4*>(xin + po * cs + ci0 + 4 * q4);
-          }
-          *reinterpret_cast<float4*>(&s_in[pix * LS + 4 * q4]) = v;
-        }
-        __syncthreads();
-#pragma unroll 1
-        for (int ky = 0; ky < K; ++ky) {
-#pragma unroll 1
-          for (int kx = 0; kx < K; ++kx) {
-#pragma unroll
-            for (int q = 0; q < CC / 8; ++q) {
-              float4 av[2];
-#pragma unroll
-              for (int mb = 0; mb < 2; ++mb)
-                av[mb] = *reinterpret_cast<const float4*>(
-                    &s_in[(pbase[mb] + ky * IT + kx) * LS + 8 * q + 4 * half]);
-              float bv[NB][4];
-              const float* wp = a.filt +
-                  ((long long)(fbase + ci0 + 8 * q + 4 * half) * K * K + ky * K + kx) * a.cout +
-                  co0 + l32;
-#pragma unroll
-              for (int j = 0; j < 4; ++j)
-#pragma unroll
-                for (int nb = 0; nb < NB; ++nb)
-                  bv[nb][j] = wp[(long long)j * K * K * a.cout + nb * 32];
-#pragma unroll
-              for (int j = 0; j < 4; ++j)
-#pragma unroll
-                for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-                  for (int mb = 0; mb < 2; ++mb)
-                    acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(
-                        (&av[mb].x)[j], bv[nb][j], acc[mb][nb], 0, 0, 0);
-            }
-          }
-        }
-        __syncthreads();
-      }
-    }
-  }
-  // Epilogue.  acc[mb][nb][r] of this lane is output pixel
-  // p = 32*mb + 8*(r/4) + 4*half + r%4, channel co0 + 32*nb + lane%32.
-#pragma unroll
-  for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int p = mb * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-      const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
-      if (oy >= hout || ox >= wout) continue;
-      const long long ob = (((long long)n * hout + oy) * wout + ox) * a.cout + co0 + l32;
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-        if (tk == 2) a.out[ob + nb * 32] = 0.f;
-        else conv_store(a, ob + nb * 32, acc[mb][nb][r]);
-      }
-    }
-}
-
-// ---------------------------------------------------------------------------------
 // Transposed conv, gather form.  Thread = one output channel x 16 pixels;
 // input values are wave-uniform loads (every lane of a wave reads the same
 // address), filter rows are coalesced over the output channel.
@@ -309,13 +168,8 @@ __global__ __launch_bounds__(256) void k_tconv_valu(ConvArgs a, int K, int S) {
 }
 
 template <int K, int S>
-void launch_conv(const ConvArgs& a, int path, unsigned cap, hipStream_t st) {
-  if (path == MIE_PATH_MFMA) {
-    if (a.cout % 64 == 0)
-      hipLaunchKernelGGL((k_conv_mfma<K, S, 2>), dim3(cap, a.cout / 64), dim3(64), 0, st, a);
-    else
-      hipLaunchKernelGGL((k_conv_mfma<K, S, 1>), dim3(cap, a.cout / 32), dim3(64), 0, st, a);
-  } else if (a.cout <= 4) {
+void launch_conv(const ConvArgs& a, unsigned cap, hipStream_t st) {
+  if (a.cout <= 4) {
     hipLaunchKernelGGL((k_conv_smallco<K, S>), dim3(cap), dim3(64), 0, st, a);
   } else {
     hipLaunchKernelGGL((k_conv_valu<K, S>), dim3(cap, mie_div_up(a.cout, 64)), dim3(256), 0, st, a);
@@ -371,11 +225,11 @@ extern "C" int mie_conv_masked(const float* x, const uint8_t* xmask, int c1, con
               MIE_ERR_INVALID_ARG, "%s: x / x2 / filter must be 16-byte aligned", who);
   rc = check_epilogue(who, out_delta, reservoir, act_kind);
   if (rc != MIE_OK) return rc;
-  const bool mfma_ok = (c1 % 16 == 0) && (c2 % 16 == 0) && (cout % 32 == 0);
+  const bool mfma_ok = (c1 % 8 == 0) && (c2 % 8 == 0) && (cout % 32 == 0);
   MIE_REQUIRE(path == MIE_PATH_AUTO || path == MIE_PATH_VALU || path == MIE_PATH_MFMA,
               MIE_ERR_INVALID_ARG, "%s: unknown path %d", who, path);
   MIE_REQUIRE(path != MIE_PATH_MFMA || mfma_ok, MIE_ERR_UNSUPPORTED,
-              "%s: MFMA path needs c1 %% 16 == 0, c2 %% 16 == 0, cout %% 32 == 0 (c1=%d c2=%d cout=%d)",
+              "%s: MFMA path needs c1 %% 8 == 0, c2 %% 8 == 0, cout %% 32 == 0 (c1=%d c2=%d cout=%d)",
               who, c1, c2, cout);
   if (path == MIE_PATH_AUTO) path = mfma_ok ? MIE_PATH_MFMA : MIE_PATH_VALU;
 
@@ -386,15 +240,19 @@ extern "C" int mie_conv_masked(const float* x, const uint8_t* xmask, int c1, con
   a.slope = slope; a.ts = mie_dev_tileset(out);
   const unsigned cap = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
   hipStream_t st = (hipStream_t)stream;
+  if (path == MIE_PATH_MFMA) {
+    mie_launch_conv_mfma(a, k, stride, cap, st);
+    return mie_check_launch(who);
+  }
   switch (k * 10 + stride) {
-    case 11: launch_conv<1, 1>(a, path, cap, st); break;
-    case 12: launch_conv<1, 2>(a, path, cap, st); break;
-    case 31: launch_conv<3, 1>(a, path, cap, st); break;
-    case 32: launch_conv<3, 2>(a, path, cap, st); break;
-    case 51: launch_conv<5, 1>(a, path, cap, st); break;
-    case 52: launch_conv<5, 2>(a, path, cap, st); break;
-    case 71: launch_conv<7, 1>(a, path, cap, st); break;
-    case 72: launch_conv<7, 2>(a, path, cap, st); break;
+    case 11: launch_conv<1, 1>(a, cap, st); break;
+    case 12: launch_conv<1, 2>(a, cap, st); break;
+    case 31: launch_conv<3, 1>(a, cap, st); break;
+    case 32: launch_conv<3, 2>(a, cap, st); break;
+    case 51: launch_conv<5, 1>(a, cap, st); break;
+    case 52: launch_conv<5, 2>(a, cap, st); break;
+    case 71: launch_conv<7, 1>(a, cap, st); break;
+    case 72: launch_conv<7, 2>(a, cap, st); break;
     default: MIE_REQUIRE(false, MIE_ERR_UNSUPPORTED, "%s: k=%d stride=%d", who, k, stride);
   }
   return mie_check_launch(who);
