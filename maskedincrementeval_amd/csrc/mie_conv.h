@@ -26,5 +26,9 @@ static __device__ __forceinline__ void conv_store(const ConvArgs& a, long long o
 
 
 // Launches the matrix-core path for kernel size k (1,3,5,7) and stride s (1,2); the caller
-// has checked c1 % 8 == 0, c2 % 8 == 0 and cout % 32 == 0.
-void mie_launch_conv_mfma(const ConvArgs& a, int k, int s, unsigned cap, hipStream_t st);
+// has checked that c1 and c2 are multiples of mie_conv_mfma_cin_multiple(k, s) (the channels
+// staged per chunk) and cout of mie_conv_mfma_cout_multiple(k, s).
+// Returns false if no kernel variant takes the shape (nothing is launched then).
+bool mie_launch_conv_mfma(const ConvArgs& a, int k, int s, unsigned cap, hipStream_t st);
+int mie_conv_mfma_cout_multiple(int k, int s);
+int mie_conv_mfma_cin_multiple(int k, int s);

@@ -1,7 +1,7 @@
 // Masked convolution of a delta over active 8x8 output tiles (gfx950).
 //
 // Three code paths, one per arithmetic regime:
-//   mfma    : Cin % 8 == 0 and Cout % 32 == 0 -- per-tile implicit GEMM on
+//   mfma    : Cin % 32 == 0 (16 for stride 2) and Cout % 32 == 0 -- per-tile implicit GEMM on
 //             the fp32 matrix cores (mie_conv_mfma.hip).
 //   valu    : any shape -- thread = one output channel x 16 pixels, input tile
 //             staged in LDS and read as wave-wide broadcasts.
@@ -225,12 +225,14 @@ extern "C" int mie_conv_masked(const float* x, const uint8_t* xmask, int c1, con
               MIE_ERR_INVALID_ARG, "%s: x / x2 / filter must be 16-byte aligned", who);
   rc = check_epilogue(who, out_delta, reservoir, act_kind);
   if (rc != MIE_OK) return rc;
-  const bool mfma_ok = (c1 % 8 == 0) && (c2 % 8 == 0) && (cout % 32 == 0);
+  const int cmul = mie_conv_mfma_cout_multiple(k, stride);
+  const int imul = mie_conv_mfma_cin_multiple(k, stride);
+  const bool mfma_ok = (c1 % imul == 0) && (c2 % imul == 0) && (cout % cmul == 0);
   MIE_REQUIRE(path == MIE_PATH_AUTO || path == MIE_PATH_VALU || path == MIE_PATH_MFMA,
               MIE_ERR_INVALID_ARG, "%s: unknown path %d", who, path);
   MIE_REQUIRE(path != MIE_PATH_MFMA || mfma_ok, MIE_ERR_UNSUPPORTED,
-              "%s: MFMA path needs c1 %% 8 == 0, c2 %% 8 == 0, cout %% 32 == 0 (c1=%d c2=%d cout=%d)",
-              who, c1, c2, cout);
+              "%s: MFMA path needs c1 %% %d == 0, c2 %% %d == 0, cout %% %d == 0 (c1=%d c2=%d cout=%d)",
+              who, imul, imul, cmul, c1, c2, cout);
   if (path == MIE_PATH_AUTO) path = mfma_ok ? MIE_PATH_MFMA : MIE_PATH_VALU;
 
   ConvArgs a;
@@ -241,7 +243,8 @@ extern "C" int mie_conv_masked(const float* x, const uint8_t* xmask, int c1, con
   const unsigned cap = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
   hipStream_t st = (hipStream_t)stream;
   if (path == MIE_PATH_MFMA) {
-    mie_launch_conv_mfma(a, k, stride, cap, st);
+    MIE_REQUIRE(mie_launch_conv_mfma(a, k, stride, cap, st), MIE_ERR_UNSUPPORTED,
+                "%s: no MFMA kernel variant for k=%d stride=%d cout=%d", who, k, stride, cout);
     return mie_check_launch(who);
   }
   switch (k * 10 + stride) {

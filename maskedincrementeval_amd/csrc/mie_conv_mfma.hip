@@ -10,7 +10,7 @@
 //     global loads of chunk c+1 are in flight while chunk c is multiplied.
 //   * B (k x channels): filter rows filt[ci][ky][kx][co..co+31] are read
 //     straight from L2 into registers (each value is used by exactly one wave
-//     of the workgroup), one unit ahead of the MFMAs that consume them.
+//     of the workgroup), three units ahead of the MFMAs that consume them.
 //   * The 4 waves split the workgroup's work WN ways over output channels and
 //     WK = 4/WN ways over k (units = tap x 8-channel sub-chunk, round robin).
 //     Layers with few tiles (33x44 bottleneck: 30 tiles) take WN=1, WK=4 so
@@ -29,11 +29,25 @@ namespace {
 
 typedef float v16f __attribute__((ext_vector_type(16)));
 
+// Channels staged in LDS per chunk, by kernel size and stride (bounded by 64 KB of LDS for
+// two staging buffers of (7*S+K)^2 pixels).
+__host__ __device__ constexpr int stage_channels(int K, int S) {
+  return (S == 1) ? (K <= 5 ? 32 : 16) : (K <= 5 ? 16 : 8);
+}
+
+// Ring size of the B-operand prefetch: the smallest divisor of the units per chunk that is
+// at least 4, so that ring slot (unit % ring) means the same registers in every chunk.
+__host__ __device__ constexpr int ring_size(int upc) {
+  for (int r = 4; r < upc; ++r)
+    if (upc % r == 0) return r;
+  return upc;
+}
+
 template <int K, int S, int WN, int NB>
 __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgs a) {
   constexpr int WK = 4 / WN;
   constexpr int IT = 7 * S + K;                              // input tile edge incl. halo
-  constexpr int CC = (K == 7) ? 8 : (S == 2 ? 16 : 32);      // channels per LDS stage
+  constexpr int CC = stage_channels(K, S);                   // channels per LDS stage
   constexpr int LS = CC + 4;                                 // LDS floats per staged pixel
   constexpr int NPIX = IT * IT;
   constexpr int Q4 = CC / 4;                                 // float4 slots per pixel
@@ -41,7 +55,11 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgs a) {
   constexpr int NLD = (NSLOT + 255) / 256;                   // staging loads per thread
   constexpr int STAGE = NPIX * LS;                           // floats per staging buffer
   constexpr int NQ = CC / 8;                                 // 8-channel sub-chunks per stage
-  constexpr int UNITS = K * K * NQ;                          // (tap, sub-chunk) units per stage
+  static_assert(NQ % WK == 0, "the k-split is over whole sub-chunks");
+  constexpr int NQW = NQ / WK;                               // sub-chunks per wave
+  constexpr int UPC = K * K * NQW;                           // units per chunk and wave
+  constexpr int RING = ring_size(UPC);                       // B operand ring (divides UPC)
+  constexpr int PD = RING - 1;                               // prefetch distance in units
   constexpr int CO_BLK = 32 * NB * WN;
   constexpr int RED = (WK > 1) ? WK * 64 * CO_BLK : 0;
   constexpr int SMEM = (2 * STAGE > RED) ? 2 * STAGE : RED;
@@ -52,18 +70,20 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgs a) {
   const int tk = mie_pick_tile(a.ts, blockIdx.x, n, y0, x0);
   if (tk == 0) return;
   const int tid = threadIdx.x;
-  const int wave = tid >> 6, lane = tid & 63;
+  // wave index as a scalar: everything derived from it (k-split, channel slab) stays in SGPRs
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int l32 = lane & 31, half = lane >> 5;
   const int wn = wave % WN, wk = wave / WN;
   const int co0 = blockIdx.y * CO_BLK;
   const int hout = a.ts.h, wout = a.ts.w;
+  const int cout = a.cout;
 
   if (tk == 2) {  // stale tile: zero this workgroup's channel slab
     for (int idx = tid; idx < 64 * CO_BLK; idx += 256) {
       const int p = idx / CO_BLK, col = idx - p * CO_BLK;
       const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
       if (oy < hout && ox < wout)
-        a.out[(((long long)n * hout + oy) * wout + ox) * a.cout + co0 + col] = 0.f;
+        a.out[(((long long)n * hout + oy) * wout + ox) * cout + co0 + col] = 0.f;
     }
     return;
   }
@@ -78,17 +98,17 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgs a) {
 
   // ---- per-thread staging plan: which pixels / float4 slots this thread copies -------------
   const int iy0 = y0 * S - a.pad, ix0 = x0 * S - a.pad;
-  int st_po[NLD];       // linear input pixel index, -1 = outside the image / beyond the tile
+  int st_po[NLD];       // linear input pixel index
   int st_lds[NLD];      // LDS float offset of the slot
   int st_c4[NLD];       // channel offset of the slot inside the chunk
-  unsigned ok1 = 0u, ok2 = 0u;   // slot readable from x / x2 (pixel mask set)
+  unsigned ok1 = 0u, ok2 = 0u;   // slot readable from x / x2 (inside the image, pixel mask set)
 #pragma unroll
   for (int i = 0; i < NLD; ++i) {
     const int slot = tid + 256 * i;
     const int pix = slot / Q4, q4 = slot - pix * Q4;
     st_lds[i] = pix * LS + 4 * q4;
     st_c4[i] = 4 * q4;
-    st_po[i] = -1;
+    st_po[i] = 0;
     if (slot < NSLOT) {
       const int iy = iy0 + pix / IT, ix = ix0 + pix % IT;
       if (iy >= 0 && iy < a.h_in && ix >= 0 && ix < a.w_in) {
@@ -124,75 +144,93 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgs a) {
       if (tid + 256 * i < NSLOT) *reinterpret_cast<float4*>(dst + st_lds[i]) = st_reg[i];
   };
 
-  // ---- B operand: filter rows for unit u of chunk c ------------------------------------------------
-  const int cob = co0 + wn * (32 * NB) + l32;
-  auto unit_valid = [&](int c, int u) {
-    const bool second = c >= nch1;
-    const int cs = second ? a.c2 : a.c1;
-    const int ci0 = (second ? c - nch1 : c) * CC;
-    return ci0 + 8 * (u % NQ) < cs;
-  };
-  auto load_b = [&](int c, int u, float (&bv)[NB][4]) {
-    const bool second = c >= nch1;
-    const int ci0 = (second ? c - nch1 : c) * CC;
-    const int fb = second ? a.c1 : 0;
-    const int tap = u / NQ, q = u - tap * NQ;
-    const float* wp = a.filt + ((long long)(fb + ci0 + 8 * q + 4 * half) * (K * K) + tap) * a.cout + cob;
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) bv[nb][j] = wp[(long long)j * (K * K) * a.cout + nb * 32];
-  };
-
-  // LDS pixel index of this lane's output pixel in M block mb at tap (0,0)
-  int pbase[2];
+  // ---- operand addressing ------------------------------------------------------------------------
+  // This wave multiplies sub-chunks q = q0w .. q0w+NQW-1 of every chunk.  A unit is one tap of
+  // one sub-chunk: 8 input channels, of which this lane's half handles 4 (channel pairing see
+  // the header).  Everything that depends on the unit index is a compile-time constant times
+  // cout (B) or a compile-time LDS offset (A); the lane-dependent parts are loop invariant.
+  const int q0w = wk * NQW;
+  const int cob0 = co0 + wn * (32 * NB);                       // first column of this wave
+  const int b_lane = (4 * half) * (K * K) * cout + l32;        // lane part of the filter index
+  int a_lane[2];                                               // lane part of the LDS index
 #pragma unroll
   for (int mb = 0; mb < 2; ++mb) {
     const int p = mb * 32 + l32;
-    pbase[mb] = ((p >> 3) * S) * IT + (p & 7) * S;
+    a_lane[mb] = (((p >> 3) * S) * IT + (p & 7) * S) * LS + 8 * q0w + 4 * half;
   }
+  // filter row block of chunk c for this wave (c1 and c2 are multiples of CC: no partial chunks)
+  auto chunk_b = [&](int c) -> const float* {
+    const bool second = c >= nch1;
+    const int ci0 = (second ? c - nch1 : c) * CC;
+    const int fb = second ? a.c1 : 0;
+    return a.filt + (long long)(fb + ci0 + 8 * q0w) * (K * K) * cout + cob0;
+  };
+  float bring[RING][NB][4];
+  auto load_b = [&](const float* ub, int unit, float (&bv)[NB][4]) {
+    const int tap = unit / NQW, qi = unit % NQW;     // compile-time after unrolling
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+        bv[nb][j] = ub[(long long)(((8 * qi + j) * (K * K) + tap) * cout + nb * 32) + b_lane];
+  };
 
-  float bcur[NB][4], bnext[NB][4];
+  // All B loads below are unconditional: a conditional load would make the compiler's wait
+  // counters conservative and collapse the prefetch distance.  After the last chunk the
+  // "next chunk" pointer simply stays on the current one (a few redundant loads).
+  const float* ub_cur = chunk_b(0);
+  const float* ub_next = ub_cur;
   stage_load(0);
-  if (wk < UNITS && unit_valid(0, wk)) load_b(0, wk, bcur);
+#pragma unroll
+  for (int i = 0; i < (PD > 0 ? PD : 1); ++i) load_b(ub_cur, i, bring[i % RING]);
   stage_store(0);
   __syncthreads();
 
   for (int c = 0; c < nch; ++c) {
     const bool more = c + 1 < nch;
-    if (more) stage_load(c + 1);
+    if (more) {
+      ub_next = chunk_b(c + 1);
+      stage_load(c + 1);
+    }
     const float* sin = smem + (c & 1) * STAGE;
-#pragma unroll 1
-    for (int u = wk; u < UNITS; u += WK) {
-      // prefetch B of the next unit (possibly the first unit of the next chunk)
-      int c2 = c, u2 = u + WK;
-      if (u2 >= UNITS) { c2 = c + 1; u2 = wk; }
-      if (c2 < nch && u2 < UNITS && unit_valid(c2, u2)) load_b(c2, u2, bnext);
-      if (unit_valid(c, u)) {
-        const int tap = u / NQ, q = u - tap * NQ;
-        const int ky = tap / K, kx = tap - ky * K;
-        float4 av[2];
+    // A operands are read one unit ahead as well (two register sets); the scheduling barriers
+    // pin "issue the loads for later units, then multiply this unit" so that the compiler can
+    // neither sink the prefetches next to their uses nor hoist them all to the top.
+    float4 av[2][2];
+    auto load_a = [&](int unit, float4 (&dst)[2]) {
+      const int tap = unit / NQW, qi = unit % NQW;
+      const int ky = tap / K, kx = tap - ky * K;
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb)
-          av[mb] = *reinterpret_cast<const float4*>(
-              &sin[(pbase[mb] + ky * IT + kx) * LS + 8 * q + 4 * half]);
+      for (int mb = 0; mb < 2; ++mb)
+        dst[mb] = *reinterpret_cast<const float4*>(&sin[a_lane[mb] + (ky * IT + kx) * LS + 8 * qi]);
+    };
+    load_a(0, av[0]);
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-          for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-            for (int mb = 0; mb < 2; ++mb)
-              acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x2f32((&av[mb].x)[j], bcur[nb][j],
-                                                                 acc[mb][nb], 0, 0, 0);
+    for (int i = 0; i < UPC; ++i) {
+      // B operands of the unit PD ahead (the first units of the next chunk at the end)
+      if (PD > 0) {
+        const int ip = i + PD;
+        if (ip < UPC) load_b(ub_cur, ip, bring[ip % RING]);
+        else load_b(ub_next, ip - UPC, bring[ip % RING]);
       }
+      if (i + 1 < UPC) load_a(i + 1, av[(i + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
+      for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) bcur[nb][j] = bnext[nb][j];
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int mb = 0; mb < 2; ++mb)
+            acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x2f32((&av[i & 1][mb].x)[j], bring[i % RING][nb][j],
+                                                               acc[mb][nb], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (PD == 0) load_b(ub_next, 0, bring[0]);   // ring of one: reload right after use
     }
     if (more) stage_store((c + 1) & 1);
     __syncthreads();
+    ub_cur = ub_next;
   }
+  const int cob = cob0 + l32;
 
   // ---- epilogue -----------------------------------------------------------------------------------
   // acc[mb][nb][r] of this lane is output pixel p = 32*mb + 8*(r/4) + 4*half + r%4,
@@ -234,33 +272,55 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgs a) {
   }
 }
 
+// Launch with the widest channel slab that still gives the chip enough workgroups (256 CUs;
+// aim for >= 2 workgroups per CU when every tile is active), among the wave splits the
+// staging depth of this (K, S) allows.
 template <int K, int S>
-void launch_ks(const ConvArgs& a, unsigned cap, hipStream_t st) {
-  // Pick the widest channel slab that still gives the chip enough workgroups
-  // (256 CUs; aim for >= 2 workgroups per CU when every tile is active).
+bool launch_ks(const ConvArgs& a, unsigned cap, hipStream_t st) {
+  constexpr int NQ = stage_channels(K, S) / 8;
   const long long want = 512;
-  if (a.cout % 256 == 0 && (long long)cap * (a.cout / 256) >= want)
-    hipLaunchKernelGGL((k_conv_mfma<K, S, 4, 2>), dim3(cap, a.cout / 256), dim3(256), 0, st, a);
-  else if (a.cout % 128 == 0 && (long long)cap * (a.cout / 128) >= want)
-    hipLaunchKernelGGL((k_conv_mfma<K, S, 4, 1>), dim3(cap, a.cout / 128), dim3(256), 0, st, a);
-  else if (a.cout % 64 == 0 && (long long)cap * (a.cout / 64) >= want)
-    hipLaunchKernelGGL((k_conv_mfma<K, S, 2, 1>), dim3(cap, a.cout / 64), dim3(256), 0, st, a);
-  else
-    hipLaunchKernelGGL((k_conv_mfma<K, S, 1, 1>), dim3(cap, a.cout / 32), dim3(256), 0, st, a);
+  const int cout = a.cout;
+  if (cout % 256 == 0 && (long long)cap * (cout / 256) >= want) {
+    hipLaunchKernelGGL((k_conv_mfma<K, S, 4, 2>), dim3(cap, cout / 256), dim3(256), 0, st, a);
+    return true;
+  }
+  if (cout % 128 == 0 && ((long long)cap * (cout / 128) >= want || NQ < 2 || cout % 64 != 0)) {
+    hipLaunchKernelGGL((k_conv_mfma<K, S, 4, 1>), dim3(cap, cout / 128), dim3(256), 0, st, a);
+    return true;
+  }
+  if constexpr (NQ >= 2) {
+    if (cout % 64 == 0 && ((long long)cap * (cout / 64) >= want || NQ < 4)) {
+      hipLaunchKernelGGL((k_conv_mfma<K, S, 2, 1>), dim3(cap, cout / 64), dim3(256), 0, st, a);
+      return true;
+    }
+  }
+  if constexpr (NQ >= 4) {
+    hipLaunchKernelGGL((k_conv_mfma<K, S, 1, 1>), dim3(cap, cout / 32), dim3(256), 0, st, a);
+    return true;
+  }
+  return false;
 }
 
 }  // namespace
 
-void mie_launch_conv_mfma(const ConvArgs& a, int k, int s, unsigned cap, hipStream_t st) {
+// Smallest output-channel multiple the matrix-core path takes for (k, s).
+int mie_conv_mfma_cin_multiple(int k, int s) { return stage_channels(k, s); }
+
+int mie_conv_mfma_cout_multiple(int k, int s) {
+  const int nq = stage_channels(k, s) / 8;
+  return nq >= 4 ? 32 : (nq >= 2 ? 64 : 128);
+}
+
+bool mie_launch_conv_mfma(const ConvArgs& a, int k, int s, unsigned cap, hipStream_t st) {
   switch (k * 10 + s) {
-    case 11: launch_ks<1, 1>(a, cap, st); break;
-    case 12: launch_ks<1, 2>(a, cap, st); break;
-    case 31: launch_ks<3, 1>(a, cap, st); break;
-    case 32: launch_ks<3, 2>(a, cap, st); break;
-    case 51: launch_ks<5, 1>(a, cap, st); break;
-    case 52: launch_ks<5, 2>(a, cap, st); break;
-    case 71: launch_ks<7, 1>(a, cap, st); break;
-    case 72: launch_ks<7, 2>(a, cap, st); break;
-    default: break;  // unreachable: the caller validated k and s
+    case 11: return launch_ks<1, 1>(a, cap, st);
+    case 12: return launch_ks<1, 2>(a, cap, st);
+    case 31: return launch_ks<3, 1>(a, cap, st);
+    case 32: return launch_ks<3, 2>(a, cap, st);
+    case 51: return launch_ks<5, 1>(a, cap, st);
+    case 52: return launch_ks<5, 2>(a, cap, st);
+    case 71: return launch_ks<7, 1>(a, cap, st);
+    case 72: return launch_ks<7, 2>(a, cap, st);
+    default: return false;
   }
 }

@@ -1,11 +1,12 @@
 // Pixel masks and ordered active-tile compaction (gfx950).
 //
-// mie_build_mask_tiles is one launch: every wave derives the 64 output-mask
-// bits of one 8x8 tile from the input mask footprint and records whether the
-// tile holds any active pixel (wave ballot); the block that finishes last
-// (ticket counter) turns the per-tile flags into the ascending tile list with
-// a ballot + popcount prefix scan, so the list order is deterministic and no
-// atomics touch the list itself.
+// mie_build_mask_tiles is two launches on the caller's stream: every wave of
+// the first derives the 64 output-mask bits of one 8x8 tile from the input
+// mask footprint and records whether the tile holds any active pixel (wave
+// ballot); the second, a single block, turns the per-tile flags into the
+// ascending tile list with a ballot + popcount prefix scan, so the list order
+// is deterministic and nothing is communicated between workgroups inside a
+// kernel (device-wide fences cost tens of microseconds on this chip).
 #include "mie_common.h"
 
 #include <string.h>
@@ -147,77 +148,75 @@ __device__ int footprint_bit(const BuildArgs& a, int n, int oy, int ox) {
   return bit;
 }
 
-// Ordered compaction of the ids `id(i)` (i in [0, count)) for which keep(i)
-// holds, by the 256 threads of one block: per wave a ballot gives the 64
-// keep-bits, popcount below the lane gives the rank, the four wave totals are
-// exchanged through LDS and a running base carries across chunks.
+// Kernel 1: one wave per output tile.  Lane = pixel of the 8x8 tile: derives its mask bit
+// from the input footprint, writes the output pixel mask, and a wave ballot tells whether
+// the tile holds any active pixel.
+__global__ __launch_bounds__(256) void k_mask_footprint(BuildArgs a) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = blockIdx.x * 4 + wave;
+  if (tile >= a.cap) return;
+  const int tx = tile % a.tiles_x;
+  const int t2 = tile / a.tiles_x;
+  const int ty = t2 % a.tiles_y;
+  const int n = t2 / a.tiles_y;
+  const int oy = ty * MIE_TILE + (lane >> 3), ox = tx * MIE_TILE + (lane & 7);
+  int bit = 0;
+  if (oy < a.h_out && ox < a.w_out) {
+    bit = footprint_bit(a, n, oy, ox);
+    a.out[((long long)n * a.h_out + oy) * a.w_out + ox] = (uint8_t)bit;
+  }
+  const unsigned long long bal = __ballot(bit != 0);
+  if (lane == 0) a.flags[tile] = (bal != 0ull) ? 1u : 0u;
+}
+
+// Ordered compaction of the ids `id(i)` (i in [0, count)) for which keep(i) holds, by the
+// COMPACT_THREADS threads of one block: per wave a ballot gives the 64 keep-bits, popcount
+// below the lane gives the rank, the wave totals are exchanged through LDS and a running
+// base carries across chunks.  The result is in ascending i order without any atomics.
+constexpr int COMPACT_THREADS = 1024;
+constexpr int COMPACT_WAVES = COMPACT_THREADS / 64;
+
 template <typename KeepFn, typename IdFn>
 __device__ int block_compact(int count, KeepFn keep, IdFn id, int32_t* dst, int* s_tot) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   int base = 0;
-  for (int start = 0; start < count; start += 256) {
+  for (int start = 0; start < count; start += COMPACT_THREADS) {
     const int i = start + threadIdx.x;
     const bool k = (i < count) && keep(i);
     const unsigned long long bal = __ballot(k);
     const int rank = __popcll(bal & ((1ull << lane) - 1ull));
     if (lane == 0) s_tot[wave] = __popcll(bal);
     __syncthreads();
-    int off = base;
-    for (int wv = 0; wv < wave; ++wv) off += s_tot[wv];
+    int off = base, all = 0;
+#pragma unroll
+    for (int wv = 0; wv < COMPACT_WAVES; ++wv) {
+      const int t = s_tot[wv];
+      if (wv < wave) off += t;
+      all += t;
+    }
     if (k) dst[off + rank] = id(i);
-    base += s_tot[0] + s_tot[1] + s_tot[2] + s_tot[3];
+    base += all;
     __syncthreads();
   }
   return base;
 }
 
-__global__ __launch_bounds__(256) void k_build_mask_tiles(BuildArgs a) {
-  __shared__ int s_last;
-  __shared__ int s_tot[4];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int tile = blockIdx.x * 4 + wave;
-  if (tile < a.cap) {
-    const int tx = tile % a.tiles_x;
-    const int t2 = tile / a.tiles_x;
-    const int ty = t2 % a.tiles_y;
-    const int n = t2 / a.tiles_y;
-    const int oy = ty * MIE_TILE + (lane >> 3), ox = tx * MIE_TILE + (lane & 7);
-    int bit = 0;
-    if (oy < a.h_out && ox < a.w_out) {
-      bit = footprint_bit(a, n, oy, ox);
-      a.out[((long long)n * a.h_out + oy) * a.w_out + ox] = (uint8_t)bit;
-    }
-    const unsigned long long bal = __ballot(bit != 0);
-    if (lane == 0) a.flags[tile] = (bal != 0ull) ? 1u : 0u;
-  }
-  // Publish this block's flags, then take a ticket; the last block compacts.
-  __threadfence();
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    const int t = atomicAdd(&a.counts[MIE_CNT_TICKET], 1);
-    s_last = (t == (int)gridDim.x - 1);
-  }
-  __syncthreads();
-  if (!s_last) return;
-  __threadfence();
+// Kernel 2 (one block): per-tile flags -> stale list (previous list minus the tiles that are
+// still active) and the new ascending active list.
+__global__ __launch_bounds__(COMPACT_THREADS) void k_compact_tiles(BuildArgs a) {
+  __shared__ int s_tot[COMPACT_WAVES];
   const uint32_t* flags = a.flags;
-  auto flag_of = [&](int t) {
-    return __hip_atomic_load(&flags[t], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
-  };
-  // 1) stale = tiles of the previous list that are not active any more.
   const int n_prev = a.counts[MIE_CNT_ACTIVE];
   const int32_t* prev = a.tiles;
   const int n_stale = block_compact(
-      n_prev, [&](int i) { return !flag_of(prev[i]); }, [&](int i) { return prev[i]; },
+      n_prev, [&](int i) { return flags[prev[i]] == 0u; }, [&](int i) { return prev[i]; },
       a.stale, s_tot);
-  __syncthreads();
-  // 2) new ascending active list.
+  __syncthreads();   // the old list has been consumed; it is overwritten next
   const int n_act = block_compact(
-      a.cap, [&](int i) { return flag_of(i); }, [&](int i) { return i; }, a.tiles, s_tot);
+      a.cap, [&](int i) { return flags[i] != 0u; }, [&](int i) { return i; }, a.tiles, s_tot);
   if (threadIdx.x == 0) {
     a.counts[MIE_CNT_ACTIVE] = n_act;
     a.counts[MIE_CNT_STALE] = n_stale;
-    a.counts[MIE_CNT_TICKET] = 0;
   }
 }
 
@@ -266,6 +265,9 @@ extern "C" int mie_build_mask_tiles(const uint8_t* in_mask, const uint8_t* in_ma
   a.cap = mie_tile_capacity(out->n, out->h, out->w);
   a.tiles = out->tiles; a.stale = out->stale; a.counts = out->counts; a.flags = out->flags;
   const unsigned blocks = (unsigned)mie_div_up(a.cap, 4);
-  hipLaunchKernelGGL(k_build_mask_tiles, dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
+  hipLaunchKernelGGL(k_mask_footprint, dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
+  rc = mie_check_launch("mie_build_mask_tiles");
+  if (rc != MIE_OK) return rc;
+  hipLaunchKernelGGL(k_compact_tiles, dim3(1), dim3(COMPACT_THREADS), 0, (hipStream_t)stream, a);
   return mie_check_launch("mie_build_mask_tiles");
 }

@@ -24,19 +24,36 @@ template <> struct Vec<1> {
   __device__ float& operator[](int) { return v; }
 };
 
-// Slot walker: calls f(px, pixoff, cq) for every in-bounds (pixel, channel
-// vector) slot of the tile; px in [0,64), pixoff = linear pixel index.
+// Slot walker: calls f(px, pixoff, cq) for every in-bounds (pixel, channel vector) slot of
+// the tile that belongs to this block; px in [0,64), pixoff = linear pixel index.  The
+// channel vectors of a tile are split over gridDim.y blocks so that layers with few tiles
+// (33x44: 30 tiles) still put a few hundred workgroups on the chip.
 template <typename F>
 __device__ __forceinline__ void for_tile_slots(const TileSetDev& ts, int n, int y0, int x0,
                                                int cv, F f) {
-  const int total = 64 * cv;
+  const int per = (cv + (int)gridDim.y - 1) / (int)gridDim.y;
+  const int cq0 = (int)blockIdx.y * per;
+  const int cvb = (cv - cq0 < per) ? cv - cq0 : per;
+  if (cvb <= 0) return;
+  const int total = 64 * cvb;
   for (int idx = threadIdx.x; idx < total; idx += 256) {
-    const int px = idx / cv, cq = idx - px * cv;
+    const int px = idx / cvb, cq = cq0 + (idx - px * cvb);
     const int y = y0 + (px >> 3), x = x0 + (px & 7);
     if (y >= ts.h || x >= ts.w) continue;
     const long long pixoff = ((long long)n * ts.h + y) * ts.w + x;
     f(px, pixoff, cq);
   }
+}
+
+// Number of channel splits (gridDim.y) for `cap` tiles and `cv` channel vectors per pixel:
+// aim for >= 1024 workgroups, keep >= 4 vectors x 64 pixels = one slot per thread.
+static inline unsigned channel_splits(int cap, int cv) {
+  int want = (1024 + cap - 1) / cap;
+  int most = cv / 4;
+  if (most < 1) most = 1;
+  if (want > most) want = most;
+  if (want < 1) want = 1;
+  return (unsigned)want;
 }
 
 // ---- activation increment -----------------------------------------------------
@@ -295,11 +312,13 @@ extern "C" int mie_act_incr(int act_kind, float slope, const float* in_delta, fl
   const int keep = (flags & MIE_FLAG_KEEP_RESERVOIR) ? 1 : 0;
   const TileSetDev d = mie_dev_tileset(ts);
   const unsigned grid = (unsigned)mie_tile_capacity(ts->n, ts->h, ts->w);
+  // the refined mask is an any-over-channels inside one block: no channel split then
+  const unsigned ny = out_pixmask ? 1u : channel_splits((int)grid, (c & 3) ? c : c / 4);
   if ((c & 3) == 0)
-    hipLaunchKernelGGL(k_act_incr<4>, dim3(grid), dim3(256), 0, (hipStream_t)stream, d, act_kind,
+    hipLaunchKernelGGL(k_act_incr<4>, dim3(grid, ny), dim3(256), 0, (hipStream_t)stream, d, act_kind,
                        slope, in_delta, reservoir, out_delta, c, out_pixmask, keep);
   else
-    hipLaunchKernelGGL(k_act_incr<1>, dim3(grid), dim3(256), 0, (hipStream_t)stream, d, act_kind,
+    hipLaunchKernelGGL(k_act_incr<1>, dim3(grid, ny), dim3(256), 0, (hipStream_t)stream, d, act_kind,
                        slope, in_delta, reservoir, out_delta, c, out_pixmask, keep);
   return mie_check_launch(who);
 }
@@ -318,10 +337,10 @@ extern "C" int mie_mul_incr(const float* d1, const uint8_t* m1, float* r1, const
   const TileSetDev d = mie_dev_tileset(ts);
   const unsigned grid = (unsigned)mie_tile_capacity(ts->n, ts->h, ts->w);
   if ((c & 3) == 0)
-    hipLaunchKernelGGL(k_mul_incr<4>, dim3(grid), dim3(256), 0, (hipStream_t)stream, d, d1, m1, r1,
+    hipLaunchKernelGGL(k_mul_incr<4>, dim3(grid, channel_splits((int)grid, c / 4)), dim3(256), 0, (hipStream_t)stream, d, d1, m1, r1,
                        d2, m2, r2, out_delta, c, keep);
   else
-    hipLaunchKernelGGL(k_mul_incr<1>, dim3(grid), dim3(256), 0, (hipStream_t)stream, d, d1, m1, r1,
+    hipLaunchKernelGGL(k_mul_incr<1>, dim3(grid, channel_splits((int)grid, c)), dim3(256), 0, (hipStream_t)stream, d, d1, m1, r1,
                        d2, m2, r2, out_delta, c, keep);
   return mie_check_launch(who);
 }
@@ -337,10 +356,10 @@ extern "C" int mie_add_incr(const float* a, const uint8_t* ma, const float* b, c
   const TileSetDev d = mie_dev_tileset(ts);
   const unsigned grid = (unsigned)mie_tile_capacity(ts->n, ts->h, ts->w);
   if ((c & 3) == 0)
-    hipLaunchKernelGGL(k_add_incr<4>, dim3(grid), dim3(256), 0, (hipStream_t)stream, d, a, ma, b,
+    hipLaunchKernelGGL(k_add_incr<4>, dim3(grid, channel_splits((int)grid, c / 4)), dim3(256), 0, (hipStream_t)stream, d, a, ma, b,
                        mb, out_delta, c);
   else
-    hipLaunchKernelGGL(k_add_incr<1>, dim3(grid), dim3(256), 0, (hipStream_t)stream, d, a, ma, b,
+    hipLaunchKernelGGL(k_add_incr<1>, dim3(grid, channel_splits((int)grid, c)), dim3(256), 0, (hipStream_t)stream, d, a, ma, b,
                        mb, out_delta, c);
   return mie_check_launch(who);
 }
@@ -361,10 +380,10 @@ extern "C" int mie_upsample2x_incr(const float* a, const uint8_t* ma, const floa
   const TileSetDev d = mie_dev_tileset(out);
   const unsigned grid = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
   if ((c & 3) == 0)
-    hipLaunchKernelGGL(k_up2x_incr<4>, dim3(grid), dim3(256), 0, (hipStream_t)stream, d, a, ma, b,
+    hipLaunchKernelGGL(k_up2x_incr<4>, dim3(grid, channel_splits((int)grid, c / 4)), dim3(256), 0, (hipStream_t)stream, d, a, ma, b,
                        mb, h_in, w_in, out_delta, c);
   else
-    hipLaunchKernelGGL(k_up2x_incr<1>, dim3(grid), dim3(256), 0, (hipStream_t)stream, d, a, ma, b,
+    hipLaunchKernelGGL(k_up2x_incr<1>, dim3(grid, channel_splits((int)grid, c)), dim3(256), 0, (hipStream_t)stream, d, a, ma, b,
                        mb, h_in, w_in, out_delta, c);
   return mie_check_launch(who);
 }
@@ -389,11 +408,11 @@ extern "C" int mie_convlstm_gates_incr(const float* gates_delta, float* gates_re
   const TileSetDev d = mie_dev_tileset(ts);
   const unsigned grid = (unsigned)mie_tile_capacity(ts->n, ts->h, ts->w);
   if ((hid & 3) == 0)
-    hipLaunchKernelGGL(k_convlstm_gates<4>, dim3(grid), dim3(256), 0, (hipStream_t)stream, d,
+    hipLaunchKernelGGL(k_convlstm_gates<4>, dim3(grid, channel_splits((int)grid, hid / 4)), dim3(256), 0, (hipStream_t)stream, d,
                        gates_delta, gates_res, cprev_delta, cprev_mask, cprev_res, cell_res,
                        h_delta, c_delta, hid);
   else
-    hipLaunchKernelGGL(k_convlstm_gates<1>, dim3(grid), dim3(256), 0, (hipStream_t)stream, d,
+    hipLaunchKernelGGL(k_convlstm_gates<1>, dim3(grid, channel_splits((int)grid, hid)), dim3(256), 0, (hipStream_t)stream, d,
                        gates_delta, gates_res, cprev_delta, cprev_mask, cprev_res, cell_res,
                        h_delta, c_delta, hid);
   return mie_check_launch(who);

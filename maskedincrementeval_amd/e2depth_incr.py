@@ -229,6 +229,7 @@ class ResidualBlockIncr(nn.Module):
         self.relu1 = nnReluIncr()
         self.conv2 = nnConvIncr(out_channels, out_channels, kernel_size=3, stride=1, padding=1, bias=bias)
         self.relu2 = nnReluIncr()
+        self.relu2.refine_mask = not fuse     # the structural mask is passed through when fused
         self.downsample = downsample
         self.add = nnAddIncr()
         self.fuse = fuse
@@ -379,7 +380,7 @@ class BaseUNetIncr(nn.Module):
         self.encoder_input_sizes = [self.base_num_channels * pow(2, i) for i in range(self.num_encoders)]
         self.encoder_output_sizes = [self.base_num_channels * pow(2, i + 1) for i in range(self.num_encoders)]
         op = getattr(torch, activation, 'relu')
-        self.activation = nnReservedActivation(op)
+        self.activation = nnReservedActivation(op, refine_mask=not fuse)
 
     def build_resblocks(self):
         self.resblocks = nn.ModuleList()

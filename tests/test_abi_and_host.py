@@ -82,7 +82,7 @@ def test_invalid_arguments_return_status_not_abort(mie_lib):
                                    ctypes.byref(ts), p, None, 0, 0.0, 0, None) == -1
     assert "aligned" in err()
     # MFMA path on a shape it cannot take
-    assert mie_lib.mie_conv_masked(p, None, 5, None, None, 0, 16, 16, p, 5, 3, 1, 1, 32,
+    assert mie_lib.mie_conv_masked(p, None, 24, None, None, 0, 16, 16, p, 24, 3, 1, 1, 32,
                                    ctypes.byref(ts), p, None, 0, 0.0, _lib.PATH_MFMA, None) == -2
     # activation without a reservoir
     assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 16, 16, p, 16, 3, 1, 1, 32,
