@@ -158,6 +158,24 @@ int mie_conv_masked(const float* x, const uint8_t* xmask, int c1,
                     void* stream);
 
 /*
+ * Dense refresh through the same kernels: for every active tile of `out`
+ * (build it with in_mask = NULL so that every tile is active)
+ *   y = conv2d(x (++ x2), filter, bias, stride, pad);
+ *   reservoir = y (if reservoir != NULL);  out_dense = act(y)
+ * bias may be NULL.  This is the dense pass that (re)fills the cached
+ * pre-activations every 20-100 frames, and the dense comparator of the
+ * incremental path.
+ * Replaces: nnConvIncr.forward_refresh_reservoirs followed by
+ * nnReservedActivation.forward_refresh_reservoirs
+ * (incr_modules/mask_incr_modules.py:182-196,253-256).
+ */
+int mie_conv_refresh(const float* x, int c1, const float* x2, int c2, int h_in,
+                     int w_in, const float* filter, int cin_total, int k,
+                     int stride, int pad, int cout, const float* bias,
+                     const mie_tileset* out, float* out_dense, float* reservoir,
+                     int act_kind, float slope, int path, void* stream);
+
+/*
  * Incremental point-wise non-linearity over the active tiles of ts:
  *   r0 = reservoir; r1 = r0 + in_delta; out_delta = act(r1) - act(r0);
  *   reservoir = r1   (in place)

@@ -28,7 +28,7 @@ CNT_ACTIVE, CNT_STALE, CNT_TICKET, CNT_WORDS = 0, 1, 2, 4
 EXPORTS = (
     "mie_version", "mie_last_error_string", "mie_tile_capacity", "mie_mask_from_delta",
     "mie_build_mask_tiles", "mie_conv_masked", "mie_act_incr", "mie_mul_incr", "mie_add_incr",
-    "mie_upsample2x_incr", "mie_convlstm_gates_incr", "mie_tconv_masked",
+    "mie_upsample2x_incr", "mie_convlstm_gates_incr", "mie_tconv_masked", "mie_conv_refresh",
 )
 
 
@@ -68,6 +68,9 @@ def _declare(l):
     l.mie_conv_masked.restype = ci
     l.mie_conv_masked.argtypes = [vp, vp, ci, vp, vp, ci, ci, ci, vp, ci, ci, ci, ci, ci, tsp, vp,
                                   vp, ci, cf, ci, vp]
+    l.mie_conv_refresh.restype = ci
+    l.mie_conv_refresh.argtypes = [vp, ci, vp, ci, ci, ci, vp, ci, ci, ci, ci, ci, vp, tsp, vp, vp,
+                                   ci, cf, ci, vp]
     l.mie_act_incr.restype = ci
     l.mie_act_incr.argtypes = [ci, cf, vp, vp, vp, ci, tsp, vp, ci, vp]
     l.mie_mul_incr.restype = ci

@@ -10,12 +10,17 @@ struct ConvArgs {
   const float* filt; int cin_total;
   int pad, cout;
   float* out; float* res; int act; float slope;
+  int refresh; const float* bias;   // dense refresh: out = act(acc + bias), res = acc + bias
   TileSetDev ts;
 };
 
-// Epilogue for one output element.
-static __device__ __forceinline__ void conv_store(const ConvArgs& a, long long off, float acc) {
-  if (a.res) {
+// Epilogue for one output element (linear offset off, output channel co).
+static __device__ __forceinline__ void conv_store(const ConvArgs& a, long long off, int co, float acc) {
+  if (a.refresh) {
+    const float v = a.bias ? acc + a.bias[co] : acc;
+    if (a.res) a.res[off] = v;
+    a.out[off] = mie_act(a.act, a.slope, v);
+  } else if (a.res) {
     const float r0 = a.res[off], r1 = r0 + acc;
     a.res[off] = r1;
     a.out[off] = mie_act(a.act, a.slope, r1) - mie_act(a.act, a.slope, r0);

@@ -82,7 +82,7 @@ __global__ __launch_bounds__(256) void k_conv_valu(ConvArgs a) {
     for (int p = 0; p < 16; ++p) {
       const int oy = y0 + 2 * pg + (p >> 3), ox = x0 + (p & 7);
       if (oy < hout && ox < wout)
-        conv_store(a, (((long long)n * hout + oy) * wout + ox) * a.cout + co, acc[p]);
+        conv_store(a, (((long long)n * hout + oy) * wout + ox) * a.cout + co, co, acc[p]);
     }
   }
 }
@@ -128,7 +128,7 @@ __global__ __launch_bounds__(64) void k_conv_smallco(ConvArgs a) {
       }
     }
   }
-  for (int co = 0; co < a.cout; ++co) conv_store(a, obase + co, acc[co]);
+  for (int co = 0; co < a.cout; ++co) conv_store(a, obase + co, co, acc[co]);
 }
 
 // ---------------------------------------------------------------------------------
@@ -163,7 +163,7 @@ __global__ __launch_bounds__(256) void k_tconv_valu(ConvArgs a, int K, int S) {
         for (int ci = 0; ci < a.c1; ++ci) acc += xr[ci] * wp[(long long)ci * K * K * a.cout];
       }
     }
-    conv_store(a, off, acc);
+    conv_store(a, off, co, acc);
   }
 }
 
@@ -176,27 +176,24 @@ void launch_conv(const ConvArgs& a, unsigned cap, hipStream_t st) {
   }
 }
 
-int check_epilogue(const char* who, float* out_delta, float* reservoir, int act_kind) {
+int check_epilogue(const char* who, float* out_delta, float* reservoir, int act_kind,
+                   bool refresh = false) {
   MIE_REQUIRE(out_delta != nullptr, MIE_ERR_INVALID_ARG, "%s: out_delta is NULL", who);
   MIE_REQUIRE(mie_aligned(out_delta, 16) && mie_aligned(reservoir, 16), MIE_ERR_INVALID_ARG,
               "%s: out_delta / reservoir must be 16-byte aligned", who);
   MIE_REQUIRE(act_kind >= MIE_ACT_NONE && act_kind <= MIE_ACT_TANH, MIE_ERR_UNSUPPORTED,
               "%s: unknown activation %d", who, act_kind);
-  MIE_REQUIRE(reservoir != nullptr || act_kind == MIE_ACT_NONE, MIE_ERR_INVALID_ARG,
+  MIE_REQUIRE(refresh || reservoir != nullptr || act_kind == MIE_ACT_NONE, MIE_ERR_INVALID_ARG,
               "%s: activation %d needs a reservoir", who, act_kind);
   return MIE_OK;
 }
 
-}  // namespace
-
-extern "C" int mie_conv_masked(const float* x, const uint8_t* xmask, int c1, const float* x2,
-                               const uint8_t* x2mask, int c2, int h_in, int w_in,
-                               const float* filter, int cin_total, int k, int stride, int pad,
-                               int cout, const mie_tileset* out, float* out_delta,
-                               float* reservoir, int act_kind, float slope, int path,
-                               void* stream) {
+int conv_impl(const char* who, const float* x, const uint8_t* xmask, int c1, const float* x2,
+              const uint8_t* x2mask, int c2, int h_in, int w_in, const float* filter,
+              int cin_total, int k, int stride, int pad, int cout, const mie_tileset* out,
+              float* out_delta, float* reservoir, int act_kind, float slope, int path,
+              bool refresh, const float* bias, void* stream) {
   mie_clear_error();
-  const char* who = "mie_conv_masked";
   int rc = mie_check_tileset(out, who);
   if (rc != MIE_OK) return rc;
   MIE_REQUIRE(x != nullptr && filter != nullptr, MIE_ERR_INVALID_ARG, "%s: NULL pointer", who);
@@ -223,8 +220,9 @@ extern "C" int mie_conv_masked(const float* x, const uint8_t* xmask, int c1, con
               MIE_ERR_CAPACITY, "%s: input too large", who);
   MIE_REQUIRE(mie_aligned(x, 16) && mie_aligned(x2, 16) && mie_aligned(filter, 16),
               MIE_ERR_INVALID_ARG, "%s: x / x2 / filter must be 16-byte aligned", who);
-  rc = check_epilogue(who, out_delta, reservoir, act_kind);
+  rc = check_epilogue(who, out_delta, reservoir, act_kind, refresh);
   if (rc != MIE_OK) return rc;
+  MIE_REQUIRE(mie_aligned(bias, 4), MIE_ERR_INVALID_ARG, "%s: bias must be 4-byte aligned", who);
   const int cmul = mie_conv_mfma_cout_multiple(k, stride);
   const int imul = mie_conv_mfma_cin_multiple(k, stride);
   const bool mfma_ok = (c1 % imul == 0) && (c2 % imul == 0) && (cout % cmul == 0);
@@ -239,7 +237,7 @@ extern "C" int mie_conv_masked(const float* x, const uint8_t* xmask, int c1, con
   a.x = x; a.xm = xmask; a.c1 = c1; a.x2 = x2; a.x2m = x2mask; a.c2 = c2;
   a.h_in = h_in; a.w_in = w_in; a.filt = filter; a.cin_total = cin_total;
   a.pad = pad; a.cout = cout; a.out = out_delta; a.res = reservoir; a.act = act_kind;
-  a.slope = slope; a.ts = mie_dev_tileset(out);
+  a.slope = slope; a.refresh = refresh ? 1 : 0; a.bias = bias; a.ts = mie_dev_tileset(out);
   const unsigned cap = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
   hipStream_t st = (hipStream_t)stream;
   if (path == MIE_PATH_MFMA) {
@@ -259,6 +257,29 @@ extern "C" int mie_conv_masked(const float* x, const uint8_t* xmask, int c1, con
     default: MIE_REQUIRE(false, MIE_ERR_UNSUPPORTED, "%s: k=%d stride=%d", who, k, stride);
   }
   return mie_check_launch(who);
+}
+
+}  // namespace
+
+extern "C" int mie_conv_masked(const float* x, const uint8_t* xmask, int c1, const float* x2,
+                               const uint8_t* x2mask, int c2, int h_in, int w_in,
+                               const float* filter, int cin_total, int k, int stride, int pad,
+                               int cout, const mie_tileset* out, float* out_delta,
+                               float* reservoir, int act_kind, float slope, int path,
+                               void* stream) {
+  return conv_impl("mie_conv_masked", x, xmask, c1, x2, x2mask, c2, h_in, w_in, filter, cin_total,
+                   k, stride, pad, cout, out, out_delta, reservoir, act_kind, slope, path, false,
+                   nullptr, stream);
+}
+
+extern "C" int mie_conv_refresh(const float* x, int c1, const float* x2, int c2, int h_in,
+                                int w_in, const float* filter, int cin_total, int k, int stride,
+                                int pad, int cout, const float* bias, const mie_tileset* out,
+                                float* out_dense, float* reservoir, int act_kind, float slope,
+                                int path, void* stream) {
+  return conv_impl("mie_conv_refresh", x, nullptr, c1, x2, nullptr, c2, h_in, w_in, filter,
+                   cin_total, k, stride, pad, cout, out, out_dense, reservoir, act_kind, slope,
+                   path, true, bias, stream);
 }
 
 extern "C" int mie_tconv_masked(const float* x, const uint8_t* xmask, int cin, int h_in,
@@ -288,7 +309,7 @@ extern "C" int mie_tconv_masked(const float* x, const uint8_t* xmask, int cin, i
   a.x = x; a.xm = xmask; a.c1 = cin; a.x2 = nullptr; a.x2m = nullptr; a.c2 = 0;
   a.h_in = h_in; a.w_in = w_in; a.filt = filter; a.cin_total = cin;
   a.pad = pad; a.cout = cout; a.out = out_delta; a.res = reservoir; a.act = act_kind;
-  a.slope = slope; a.ts = mie_dev_tileset(out);
+  a.slope = slope; a.refresh = 0; a.bias = nullptr; a.ts = mie_dev_tileset(out);
   const unsigned cap = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
   hipLaunchKernelGGL(k_tconv_valu, dim3(cap, mie_div_up(cout, 64)), dim3(256), 0,
                      (hipStream_t)stream, a, k, stride);

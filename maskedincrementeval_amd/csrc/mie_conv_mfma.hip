@@ -245,7 +245,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgs a) {
         if (oy >= hout || ox >= wout) continue;
         const long long ob = (((long long)n * hout + oy) * wout + ox) * a.cout + cob;
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) conv_store(a, ob + nb * 32, acc[mb][nb][r]);
+        for (int nb = 0; nb < NB; ++nb) conv_store(a, ob + nb * 32, cob + nb * 32, acc[mb][nb][r]);
       }
   } else {
     // the trailing barrier of the main loop has retired every read of the staging buffers
@@ -267,7 +267,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgs a) {
       float s = smem[idx];
 #pragma unroll
       for (int k2 = 1; k2 < WK; ++k2) s += smem[k2 * (64 * CO_BLK) + idx];
-      conv_store(a, (((long long)n * hout + oy) * wout + ox) * a.cout + co0 + col, s);
+      conv_store(a, (((long long)n * hout + oy) * wout + ox) * a.cout + co0 + col, co0 + col, s);
     }
   }
 }

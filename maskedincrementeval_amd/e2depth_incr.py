@@ -65,6 +65,8 @@ class ConvLayerIncr(nn.Module):
         return out_incr
 
     def forward_refresh_reservoirs(self, x: DenseT):
+        if self.fuse and self.activation is not None and self.norm not in ['BN', 'IN']:
+            return self.conv2d.forward_refresh_fused(x, self.activation)
         out = self.conv2d.forward_refresh_reservoirs(x)
         if self.norm in ['BN', 'IN']:
             out = self.norm_layer.forward_refresh_reservoirs(out)
@@ -162,10 +164,11 @@ class ConvLSTMIncr(nn.Module, _IncrBuffers):
                     torch.zeros(state_size, device=input_.device).to(memory_format=torch.channels_last),
                     torch.zeros(state_size, device=input_.device).to(memory_format=torch.channels_last))
             prev_state = self.zero_tensors[tuple(state_size)]
+        zero_state = prev_state is self.zero_tensors.get(tuple([batch_size, self.hidden_size] + list(spatial_size)))
         prev_h, prev_c = prev_state
         self._reset_incr()
-        stacked_inputs = torch.cat((input_, prev_h), 1)
-        gates = self.Gates.forward_refresh_reservoirs(stacked_inputs)
+        # the concat is never formed: two-pointer conv input, hidden half skipped when it is zero
+        gates = self.Gates._refresh_forward(input_, None if zero_state else prev_h, path=self.Gates.path)
         in_gate, remember_gate, out_gate, cell_gate = gates.chunk(4, 1)
         if self.fused:
             self.gates_res.update_reservoir(gates)
@@ -248,16 +251,20 @@ class ResidualBlockIncr(nn.Module):
             out_incr = self.bn2(out_incr)
         if self.downsample:
             residual_incr = self.downsample(x_incr)
-        out_incr = self.add(out_incr, residual_incr)
+        # without a down-sampling branch conv2(relu(conv1(x))) reaches every active pixel of x
+        out_incr = self.add(out_incr, residual_incr, a_covers_b=not self.downsample)
         out_incr = self.relu2(out_incr)
         return out_incr
 
     def forward_refresh_reservoirs(self, x):
         residual = x
-        out = self.conv1.forward_refresh_reservoirs(x)
-        if self.norm in ['BN', 'IN']:
-            out = self.bn1.forward_refresh_reservoirs(out)
-        out = self.relu1.forward_refresh_reservoirs(out)
+        if self.fuse and self.norm not in ['BN', 'IN']:
+            out = self.conv1.forward_refresh_fused(x, self.relu1)
+        else:
+            out = self.conv1.forward_refresh_reservoirs(x)
+            if self.norm in ['BN', 'IN']:
+                out = self.bn1.forward_refresh_reservoirs(out)
+            out = self.relu1.forward_refresh_reservoirs(out)
         out = self.conv2.forward_refresh_reservoirs(out)
         if self.norm in ['BN', 'IN']:
             out = self.bn2.forward_refresh_reservoirs(out)
@@ -348,6 +355,8 @@ class UpsampleConvLayerIncr(nn.Module):
 
     def forward_refresh_reservoirs(self, x, skip=None):
         x_upsampled = self.upsample.forward_refresh_reservoirs(x, skip)
+        if self.fuse and self.activation is not None and self.norm not in ['BN', 'IN']:
+            return self.conv2d.forward_refresh_fused(x_upsampled, self.activation)
         out = self.conv2d.forward_refresh_reservoirs(x_upsampled)
         if self.norm in ['BN', 'IN']:
             out = self.norm_layer.forward_refresh_reservoirs(out)

@@ -8,8 +8,9 @@ names, constructor signatures and the two-forward protocol
 
 (reference :13-17).  The incremental forwards run the masked HIP kernels of
 libmie_hip.so on persistent per-module buffers; the mask slot of the result
-is a `TileMask`.  The dense refresh uses torch ops on the GPU (it runs once
-every 20-100 frames in the reference drivers).
+is a `TileMask`.  The dense refresh of the convolutions runs through the same
+kernels with every tile active (bias and the reservoir fill fused in); the
+cheap point-wise parts of the refresh are torch ops on the device.
 """
 import functools
 from typing import Tuple
@@ -68,6 +69,25 @@ class _IncrBuffers:
         b = self._ib().get(key)
         if b is None:
             b = parent.with_pixmask(pix)
+            self._ib()[key] = b
+        return b
+
+    def _dense_tile_set(self, n, h, w, device) -> TileMask:
+        """Tile set with every tile active (built once; survives `_reset_incr`)."""
+        key = ("T", "dense", (n, h, w), str(device))
+        b = self._ib().get(key)
+        if b is None:
+            b = TileMask(n, h, w, device)
+            ops.build_mask_tiles(None, None, n, h, w, _lib.FOOT_CONV, 1, 1, 0, b)
+            self._ib()[key] = b
+        return b
+
+    def _dense_buf(self, name, shape, device) -> torch.Tensor:
+        """Persistent dense output of the refresh pass (not touched by `_reset_incr`)."""
+        key = ("D", name, tuple(shape), str(device))
+        b = self._ib().get(key)
+        if b is None:
+            b = ops.new_nhwc(*shape, device)
             self._ib()[key] = b
         return b
 
@@ -268,18 +288,59 @@ class _ConvIncrMixin(_IncrBuffers):
             x2, pix2, _ = _unpack(x2_incr)
         n, _, h, w = x.shape
         ho, wo = ops.conv_out_size(h, w, k, s, p)
-        ts = self._tile_set(out_name, n, ho, wo, x.device)
         out = self._delta_buf(out_name, (n, self.out_channels, ho, wo), x.device)
-        if x2 is None:
-            m1, m2 = pix, None
-        elif pix is None or pix2 is None:      # one input dense -> every tile active
-            m1 = m2 = None
+        in_tm = x_incr[1] if len(x_incr) > 1 else None
+        if k == 1 and s == 1 and p == 0 and x2 is None and isinstance(in_tm, TileMask):
+            ts = in_tm            # a 1x1 conv reaches exactly the pixels of its input: same tile set
         else:
-            m1, m2 = pix, pix2
-        ops.build_mask_tiles(m1, m2, n, h, w, _lib.FOOT_CONV, k, s, p, ts)
+            ts = self._tile_set(out_name, n, ho, wo, x.device)
+            if x2 is None:
+                m1, m2 = pix, None
+            elif pix is None or pix2 is None:      # one input dense -> every tile active
+                m1 = m2 = None
+            else:
+                m1, m2 = pix, pix2
+            ops.build_mask_tiles(m1, m2, n, h, w, _lib.FOOT_CONV, k, s, p, ts)
         ops.conv_masked(x, pix, x2, pix2, self.conv2d_weights, k, s, p, ts, out, reservoir, act,
                         slope, path)
         return [out, ts]
+
+
+    def _refresh_forward(self, x: DenseT, x2: DenseT = None, activation=None, out=None,
+                         path=_lib.PATH_AUTO) -> DenseT:
+        """Dense pass: conv2d(cat(x, x2), W, b) through the same kernels with every tile
+        active.  With `activation` (an nnReservedActivation) the pre-activation goes straight
+        into its reservoir and the activated tensor is returned.  `out` overrides the result
+        buffer.  CPU tensors take the torch ops (nothing of this package computes on the CPU).
+        """
+        self._reset_incr()
+        if not x.is_cuda:
+            xin = x if x2 is None else torch.cat((x, x2), 1)
+            if xin.shape[1] < self.in_channels:     # absent trailing input (zero hidden state)
+                xin = torch.cat((xin, xin.new_zeros(xin.shape[0], self.in_channels - xin.shape[1],
+                                                    *xin.shape[2:])), 1)
+            y = nn.Conv2d.forward(self, xin)
+            return y if activation is None else activation.forward_refresh_reservoirs(y)
+        k, s, p = self._geometry()
+        x = ops.as_nhwc(x)
+        x2 = None if x2 is None else ops.as_nhwc(x2)
+        n, _, h, w = x.shape
+        ho, wo = ops.conv_out_size(h, w, k, s, p)
+        ts = self._dense_tile_set(n, ho, wo, x.device)
+        shape = (n, self.out_channels, ho, wo)
+        if out is None:
+            out = self._dense_buf("refresh_out", shape, x.device)
+        res, kind, slope = None, _lib.ACT_NONE, 0.0
+        if activation is not None:
+            kind, slope = activation_kind(activation.op)
+            r = activation.in_res.reservoir
+            if r is None or tuple(r.shape) != shape or r.device != x.device:
+                activation.in_res.reservoir = ops.new_nhwc(*shape, x.device)
+            res = activation.in_res.reservoir
+            activation._reset_incr()
+        bias = None if self.bias is None else self.bias.detach()
+        ops.conv_refresh(x, x2, self.conv2d_weights, bias, k, s, p, ts, out, res, kind, slope, path)
+        return out
 
 
 class nnConvIncrBase(nn.Conv2d, _ConvIncrMixin):
@@ -289,8 +350,7 @@ class nnConvIncrBase(nn.Conv2d, _ConvIncrMixin):
         return self._incr_forward(x_incr)
 
     def forward_refresh_reservoirs(self, x):
-        self._reset_incr()
-        return nn.Conv2d.forward(self, x)
+        return self._refresh_forward(x)
 
 
 class nnConvIncr(nn.Conv2d, _ConvIncrMixin):
@@ -327,8 +387,11 @@ class nnConvIncr(nn.Conv2d, _ConvIncrMixin):
     def forward_refresh_reservoirs(self, x):
         # The reference also refreshes self.kf here (:193), a norm and a zero clone
         # that nothing reads because kf.forward is never called (:166).
-        self._reset_incr()
-        return nn.Conv2d.forward(self, x)
+        return self._refresh_forward(x, path=self.path)
+
+    def forward_refresh_fused(self, x, activation: "nnReservedActivation", x2=None):
+        """Dense conv + bias + activation, pre-activation written into activation.in_res."""
+        return self._refresh_forward(x, x2, activation, path=self.path)
 
 
 class nnConvTranspose2dIncr(nn.ConvTranspose2d, _IncrBuffers):
@@ -451,12 +514,17 @@ class nnAddIncr(IncrementMaskModule):
     """Sum of two deltas with the union of their masks (the skip / residual sum the
     reference writes as a tensor add, incr_modules/e2depth_incr.py:220,333)."""
 
-    def forward(self, a_incr: Masked, b_incr: Masked) -> Masked:
-        a, pa, _ = _unpack(a_incr)
+    def forward(self, a_incr: Masked, b_incr: Masked, a_covers_b: bool = False) -> Masked:
+        """a_covers_b: the caller knows that every active pixel of b is active in a (e.g. a is
+        a same-padding conv chain applied to b); a's tile set is then used as is."""
+        a, pa, ta = _unpack(a_incr)
         b, pb, _ = _unpack(b_incr)
         n, c, h, w = a.shape
-        ts = self._tile_set("union", n, h, w, a.device)
-        ops.build_mask_tiles(pa, pb, n, h, w, _lib.FOOT_CONV, 1, 1, 0, ts)
+        if a_covers_b and ta is not None:
+            ts = ta
+        else:
+            ts = self._tile_set("union", n, h, w, a.device)
+            ops.build_mask_tiles(pa, pb, n, h, w, _lib.FOOT_CONV, 1, 1, 0, ts)
         out = self._delta_buf("out", (n, c, h, w), a.device)
         ops.add_incr(a, pa, b, pb, out, ts)
         return [out, ts]

@@ -124,6 +124,24 @@ def conv_masked(x, xmask, x2, x2mask, filt, k, stride, pad, out_ts: TileMask, ou
     return out_delta
 
 
+def conv_refresh(x, x2, filt, bias, k, stride, pad, out_ts: TileMask, out_dense, reservoir=None,
+                 act=_lib.ACT_NONE, slope=0.0, path=_lib.PATH_AUTO):
+    """Dense conv + bias (+ activation, + reservoir fill) over the tiles of out_ts (all active)."""
+    n, c1, h, w = x.shape
+    c2 = 0 if x2 is None else x2.shape[1]
+    _require_gpu(filt, "filter")
+    cin_total, cout = filt.shape[0], filt.shape[3]
+    if tuple(out_dense.shape) != (n, cout, out_ts.h, out_ts.w):
+        raise ValueError("out_dense shape %s, expected %s" % (tuple(out_dense.shape), (n, cout, out_ts.h, out_ts.w)))
+    if bias is not None and (bias.numel() != cout or bias.dtype != torch.float32 or not bias.is_contiguous()):
+        raise ValueError("bias must be contiguous fp32 of %d elements" % cout)
+    check(lib().mie_conv_refresh(
+        nhwc_ptr(x, "x"), c1, nhwc_ptr(x2, "x2"), c2, h, w, filt.data_ptr(), cin_total, k, stride, pad,
+        cout, None if bias is None else bias.data_ptr(), out_ts.ref, nhwc_ptr(out_dense, "out_dense"),
+        nhwc_ptr(reservoir, "reservoir"), act, float(slope), path, _stream(x)))
+    return out_dense
+
+
 def tconv_masked(x, xmask, filt, k, stride, pad, out_ts: TileMask, out_delta, reservoir=None,
                  act=_lib.ACT_NONE, slope=0.0):
     """filt: ConvTranspose2d weight permuted to [Cin, K, K, Cout], contiguous fp32."""
