@@ -136,7 +136,10 @@ int mie_build_mask_tiles(const uint8_t* in_mask, const uint8_t* in_mask2,
  *                                         out_delta = act(r1) - act(r0)
  * (the fused form of nnConvIncr followed by nnReservedActivation).
  * Stale tiles of `out` are zeroed in out_delta.  Inactive input pixels are
- * never read.
+ * never read.  addend (optional, [n, h_out, w_out, cout]) is added to acc first:
+ * a clean delta whose active pixels are covered by `out` -- the residual of a
+ * residual block, or the contribution of a few extra input channels computed
+ * by another launch (conv over a concat = sum of convs over its parts).
  *   x  : [n, h_in, w_in, c1] delta with pixel mask xmask (NULL = all active),
  *        feeds filter input channels [0, c1)
  *   x2 : optional second input [n, h_in, w_in, c2] (NULL, c2 = 0 if absent),
@@ -154,13 +157,13 @@ int mie_conv_masked(const float* x, const uint8_t* xmask, int c1,
                     int h_in, int w_in, const float* filter, int cin_total,
                     int k, int stride, int pad, int cout,
                     const mie_tileset* out, float* out_delta,
-                    float* reservoir, int act_kind, float slope, int path,
-                    void* stream);
+                    const float* addend, float* reservoir, int act_kind,
+                    float slope, int path, void* stream);
 
 /*
  * Dense refresh through the same kernels: for every active tile of `out`
  * (build it with in_mask = NULL so that every tile is active)
- *   y = conv2d(x (++ x2), filter, bias, stride, pad);
+ *   y = conv2d(x (++ x2), filter, bias, stride, pad) (+ addend);
  *   reservoir = y (if reservoir != NULL);  out_dense = act(y)
  * bias may be NULL.  This is the dense pass that (re)fills the cached
  * pre-activations every 20-100 frames, and the dense comparator of the
@@ -172,8 +175,9 @@ int mie_conv_masked(const float* x, const uint8_t* xmask, int c1,
 int mie_conv_refresh(const float* x, int c1, const float* x2, int c2, int h_in,
                      int w_in, const float* filter, int cin_total, int k,
                      int stride, int pad, int cout, const float* bias,
-                     const mie_tileset* out, float* out_dense, float* reservoir,
-                     int act_kind, float slope, int path, void* stream);
+                     const mie_tileset* out, float* out_dense,
+                     const float* addend, float* reservoir, int act_kind,
+                     float slope, int path, void* stream);
 
 /*
  * Incremental point-wise non-linearity over the active tiles of ts:

@@ -67,10 +67,10 @@ def _declare(l):
     l.mie_build_mask_tiles.argtypes = [vp, vp, ci, ci, ci, ci, ci, ci, tsp, vp]
     l.mie_conv_masked.restype = ci
     l.mie_conv_masked.argtypes = [vp, vp, ci, vp, vp, ci, ci, ci, vp, ci, ci, ci, ci, ci, tsp, vp,
-                                  vp, ci, cf, ci, vp]
+                                  vp, vp, ci, cf, ci, vp]
     l.mie_conv_refresh.restype = ci
     l.mie_conv_refresh.argtypes = [vp, ci, vp, ci, ci, ci, vp, ci, ci, ci, ci, ci, vp, tsp, vp, vp,
-                                   ci, cf, ci, vp]
+                                   vp, ci, cf, ci, vp]
     l.mie_act_incr.restype = ci
     l.mie_act_incr.argtypes = [ci, cf, vp, vp, vp, ci, tsp, vp, ci, vp]
     l.mie_mul_incr.restype = ci

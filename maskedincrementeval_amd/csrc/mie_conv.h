@@ -10,12 +10,14 @@ struct ConvArgs {
   const float* filt; int cin_total;
   int pad, cout;
   float* out; float* res; int act; float slope;
+  const float* addend;              // optional delta added to the conv result before the epilogue
   int refresh; const float* bias;   // dense refresh: out = act(acc + bias), res = acc + bias
   TileSetDev ts;
 };
 
 // Epilogue for one output element (linear offset off, output channel co).
 static __device__ __forceinline__ void conv_store(const ConvArgs& a, long long off, int co, float acc) {
+  if (a.addend) acc += a.addend[off];
   if (a.refresh) {
     const float v = a.bias ? acc + a.bias[co] : acc;
     if (a.res) a.res[off] = v;

@@ -191,8 +191,8 @@ int check_epilogue(const char* who, float* out_delta, float* reservoir, int act_
 int conv_impl(const char* who, const float* x, const uint8_t* xmask, int c1, const float* x2,
               const uint8_t* x2mask, int c2, int h_in, int w_in, const float* filter,
               int cin_total, int k, int stride, int pad, int cout, const mie_tileset* out,
-              float* out_delta, float* reservoir, int act_kind, float slope, int path,
-              bool refresh, const float* bias, void* stream) {
+              float* out_delta, const float* addend, float* reservoir, int act_kind, float slope,
+              int path, bool refresh, const float* bias, void* stream) {
   mie_clear_error();
   int rc = mie_check_tileset(out, who);
   if (rc != MIE_OK) return rc;
@@ -222,7 +222,10 @@ int conv_impl(const char* who, const float* x, const uint8_t* xmask, int c1, con
               MIE_ERR_INVALID_ARG, "%s: x / x2 / filter must be 16-byte aligned", who);
   rc = check_epilogue(who, out_delta, reservoir, act_kind, refresh);
   if (rc != MIE_OK) return rc;
-  MIE_REQUIRE(mie_aligned(bias, 4), MIE_ERR_INVALID_ARG, "%s: bias must be 4-byte aligned", who);
+  MIE_REQUIRE(mie_aligned(bias, 4) && mie_aligned(addend, 16), MIE_ERR_INVALID_ARG,
+              "%s: bias must be 4-byte and addend 16-byte aligned", who);
+  MIE_REQUIRE(addend == nullptr || addend != out_delta, MIE_ERR_INVALID_ARG,
+              "%s: addend must not alias out_delta", who);
   const int cmul = mie_conv_mfma_cout_multiple(k, stride);
   const int imul = mie_conv_mfma_cin_multiple(k, stride);
   const bool mfma_ok = (c1 % imul == 0) && (c2 % imul == 0) && (cout % cmul == 0);
@@ -237,7 +240,8 @@ int conv_impl(const char* who, const float* x, const uint8_t* xmask, int c1, con
   a.x = x; a.xm = xmask; a.c1 = c1; a.x2 = x2; a.x2m = x2mask; a.c2 = c2;
   a.h_in = h_in; a.w_in = w_in; a.filt = filter; a.cin_total = cin_total;
   a.pad = pad; a.cout = cout; a.out = out_delta; a.res = reservoir; a.act = act_kind;
-  a.slope = slope; a.refresh = refresh ? 1 : 0; a.bias = bias; a.ts = mie_dev_tileset(out);
+  a.slope = slope; a.addend = addend; a.refresh = refresh ? 1 : 0; a.bias = bias;
+  a.ts = mie_dev_tileset(out);
   const unsigned cap = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
   hipStream_t st = (hipStream_t)stream;
   if (path == MIE_PATH_MFMA) {
@@ -265,21 +269,21 @@ extern "C" int mie_conv_masked(const float* x, const uint8_t* xmask, int c1, con
                                const uint8_t* x2mask, int c2, int h_in, int w_in,
                                const float* filter, int cin_total, int k, int stride, int pad,
                                int cout, const mie_tileset* out, float* out_delta,
-                               float* reservoir, int act_kind, float slope, int path,
-                               void* stream) {
+                               const float* addend, float* reservoir, int act_kind, float slope,
+                               int path, void* stream) {
   return conv_impl("mie_conv_masked", x, xmask, c1, x2, x2mask, c2, h_in, w_in, filter, cin_total,
-                   k, stride, pad, cout, out, out_delta, reservoir, act_kind, slope, path, false,
-                   nullptr, stream);
+                   k, stride, pad, cout, out, out_delta, addend, reservoir, act_kind, slope, path,
+                   false, nullptr, stream);
 }
 
 extern "C" int mie_conv_refresh(const float* x, int c1, const float* x2, int c2, int h_in,
                                 int w_in, const float* filter, int cin_total, int k, int stride,
                                 int pad, int cout, const float* bias, const mie_tileset* out,
-                                float* out_dense, float* reservoir, int act_kind, float slope,
-                                int path, void* stream) {
+                                float* out_dense, const float* addend, float* reservoir,
+                                int act_kind, float slope, int path, void* stream) {
   return conv_impl("mie_conv_refresh", x, nullptr, c1, x2, nullptr, c2, h_in, w_in, filter,
-                   cin_total, k, stride, pad, cout, out, out_dense, reservoir, act_kind, slope,
-                   path, true, bias, stream);
+                   cin_total, k, stride, pad, cout, out, out_dense, addend, reservoir, act_kind,
+                   slope, path, true, bias, stream);
 }
 
 extern "C" int mie_tconv_masked(const float* x, const uint8_t* xmask, int cin, int h_in,
@@ -309,7 +313,7 @@ extern "C" int mie_tconv_masked(const float* x, const uint8_t* xmask, int cin, i
   a.x = x; a.xm = xmask; a.c1 = cin; a.x2 = nullptr; a.x2m = nullptr; a.c2 = 0;
   a.h_in = h_in; a.w_in = w_in; a.filt = filter; a.cin_total = cin;
   a.pad = pad; a.cout = cout; a.out = out_delta; a.res = reservoir; a.act = act_kind;
-  a.slope = slope; a.refresh = 0; a.bias = nullptr; a.ts = mie_dev_tileset(out);
+  a.slope = slope; a.addend = nullptr; a.refresh = 0; a.bias = nullptr; a.ts = mie_dev_tileset(out);
   const unsigned cap = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
   hipLaunchKernelGGL(k_tconv_valu, dim3(cap, mie_div_up(cout, 64)), dim3(256), 0,
                      (hipStream_t)stream, a, k, stride);

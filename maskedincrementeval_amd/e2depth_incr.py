@@ -246,12 +246,15 @@ class ResidualBlockIncr(nn.Module):
             if self.norm in ['BN', 'IN']:
                 out_incr = self.bn1(out_incr)
             out_incr = self.relu1(out_incr)
+        if self.fuse and self.norm not in ['BN', 'IN'] and not self.downsample:
+            # conv2 + residual + relu2 in one kernel: conv2(relu(conv1(x))) reaches every active
+            # pixel of x (two same-padding 3x3), so the residual delta rides in as the addend
+            return self.conv2.forward_fused(out_incr, self.relu2, addend_incr=residual_incr)
         out_incr = self.conv2(out_incr)
         if self.norm in ['BN', 'IN']:
             out_incr = self.bn2(out_incr)
         if self.downsample:
             residual_incr = self.downsample(x_incr)
-        # without a down-sampling branch conv2(relu(conv1(x))) reaches every active pixel of x
         out_incr = self.add(out_incr, residual_incr, a_covers_b=not self.downsample)
         out_incr = self.relu2(out_incr)
         return out_incr
@@ -265,6 +268,8 @@ class ResidualBlockIncr(nn.Module):
             if self.norm in ['BN', 'IN']:
                 out = self.bn1.forward_refresh_reservoirs(out)
             out = self.relu1.forward_refresh_reservoirs(out)
+        if self.fuse and self.norm not in ['BN', 'IN'] and not self.downsample:
+            return self.conv2.forward_refresh_fused(out, self.relu2, addend=residual)
         out = self.conv2.forward_refresh_reservoirs(out)
         if self.norm in ['BN', 'IN']:
             out = self.bn2.forward_refresh_reservoirs(out)

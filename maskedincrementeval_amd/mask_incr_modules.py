@@ -280,7 +280,11 @@ class _ConvIncrMixin(_IncrBuffers):
         return cached[1]
 
     def _incr_forward(self, x_incr: Masked, x2_incr: Masked = None, reservoir=None,
-                      act=_lib.ACT_NONE, slope=0.0, path=_lib.PATH_AUTO, out_name="out") -> Masked:
+                      act=_lib.ACT_NONE, slope=0.0, path=_lib.PATH_AUTO, out_name="out",
+                      addend_incr: Masked = None, filt=None) -> Masked:
+        """addend_incr: delta added to the conv result before the epilogue; the caller
+        guarantees that its active pixels are covered by the conv's output mask.
+        filt: a row slice of conv2d_weights when only part of the input channels is fed."""
         k, s, p = self._geometry()
         x, pix, _ = _unpack(x_incr)
         x2 = pix2 = None
@@ -301,13 +305,14 @@ class _ConvIncrMixin(_IncrBuffers):
             else:
                 m1, m2 = pix, pix2
             ops.build_mask_tiles(m1, m2, n, h, w, _lib.FOOT_CONV, k, s, p, ts)
-        ops.conv_masked(x, pix, x2, pix2, self.conv2d_weights, k, s, p, ts, out, reservoir, act,
-                        slope, path)
+        addend = None if addend_incr is None else ops.as_nhwc(addend_incr[0])
+        ops.conv_masked(x, pix, x2, pix2, self.conv2d_weights if filt is None else filt, k, s, p, ts,
+                        out, reservoir, act, slope, path, addend)
         return [out, ts]
 
 
     def _refresh_forward(self, x: DenseT, x2: DenseT = None, activation=None, out=None,
-                         path=_lib.PATH_AUTO) -> DenseT:
+                         path=_lib.PATH_AUTO, addend: DenseT = None) -> DenseT:
         """Dense pass: conv2d(cat(x, x2), W, b) through the same kernels with every tile
         active.  With `activation` (an nnReservedActivation) the pre-activation goes straight
         into its reservoir and the activated tensor is returned.  `out` overrides the result
@@ -320,6 +325,8 @@ class _ConvIncrMixin(_IncrBuffers):
                 xin = torch.cat((xin, xin.new_zeros(xin.shape[0], self.in_channels - xin.shape[1],
                                                     *xin.shape[2:])), 1)
             y = nn.Conv2d.forward(self, xin)
+            if addend is not None:
+                y = y + addend
             return y if activation is None else activation.forward_refresh_reservoirs(y)
         k, s, p = self._geometry()
         x = ops.as_nhwc(x)
@@ -339,7 +346,8 @@ class _ConvIncrMixin(_IncrBuffers):
             res = activation.in_res.reservoir
             activation._reset_incr()
         bias = None if self.bias is None else self.bias.detach()
-        ops.conv_refresh(x, x2, self.conv2d_weights, bias, k, s, p, ts, out, res, kind, slope, path)
+        ops.conv_refresh(x, x2, self.conv2d_weights, bias, k, s, p, ts, out, res, kind, slope, path,
+                         None if addend is None else ops.as_nhwc(addend))
         return out
 
 
@@ -375,23 +383,24 @@ class nnConvIncr(nn.Conv2d, _ConvIncrMixin):
     def forward(self, x_incr, x2_incr=None):
         return self._incr_forward(x_incr, x2_incr, path=self.path)
 
-    def forward_fused(self, x_incr, activation: "nnReservedActivation", x2_incr=None):
-        """conv + activation increment in one kernel; updates activation.in_res in place."""
+    def forward_fused(self, x_incr, activation: "nnReservedActivation", x2_incr=None,
+                      addend_incr=None, filt=None):
+        """conv (+ addend) + activation increment in one kernel; updates activation.in_res in place."""
         kind, slope = activation_kind(activation.op)
         res = activation.in_res.reservoir
         if res is None:
             raise RuntimeError("fused conv+activation: call forward_refresh_reservoirs first")
         return self._incr_forward(x_incr, x2_incr, reservoir=res, act=kind, slope=slope,
-                                  path=self.path, out_name="out_act")
+                                  path=self.path, out_name="out_act", addend_incr=addend_incr, filt=filt)
 
     def forward_refresh_reservoirs(self, x):
         # The reference also refreshes self.kf here (:193), a norm and a zero clone
         # that nothing reads because kf.forward is never called (:166).
         return self._refresh_forward(x, path=self.path)
 
-    def forward_refresh_fused(self, x, activation: "nnReservedActivation", x2=None):
-        """Dense conv + bias + activation, pre-activation written into activation.in_res."""
-        return self._refresh_forward(x, x2, activation, path=self.path)
+    def forward_refresh_fused(self, x, activation: "nnReservedActivation", x2=None, addend=None):
+        """Dense conv + bias (+ addend) + activation, pre-activation written into activation.in_res."""
+        return self._refresh_forward(x, x2, activation, path=self.path, addend=addend)
 
 
 class nnConvTranspose2dIncr(nn.ConvTranspose2d, _IncrBuffers):

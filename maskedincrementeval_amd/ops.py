@@ -100,7 +100,7 @@ def build_mask_tiles(in_mask, in_mask2, n, h_in, w_in, foot, k, stride, pad, out
 
 
 def conv_masked(x, xmask, x2, x2mask, filt, k, stride, pad, out_ts: TileMask, out_delta,
-                reservoir=None, act=_lib.ACT_NONE, slope=0.0, path=_lib.PATH_AUTO):
+                reservoir=None, act=_lib.ACT_NONE, slope=0.0, path=_lib.PATH_AUTO, addend=None):
     """filt: [Cin_total, K, K, Cout] contiguous fp32."""
     n, c1, h, w = x.shape
     c2 = 0 if x2 is None else x2.shape[1]
@@ -115,17 +115,19 @@ def conv_masked(x, xmask, x2, x2mask, filt, k, stride, pad, out_ts: TileMask, ou
         raise ValueError("out_delta shape %s, expected %s" % (tuple(out_delta.shape), (n, cout, out_ts.h, out_ts.w)))
     if reservoir is not None and reservoir.shape != out_delta.shape:
         raise ValueError("reservoir shape %s != output %s" % (tuple(reservoir.shape), tuple(out_delta.shape)))
+    if addend is not None and addend.shape != out_delta.shape:
+        raise ValueError("addend shape %s != output %s" % (tuple(addend.shape), tuple(out_delta.shape)))
     check(lib().mie_conv_masked(
         nhwc_ptr(x, "x"), pix_ptr(xmask, n, h, w, "xmask"), c1,
         nhwc_ptr(x2, "x2"), pix_ptr(x2mask, n, h, w, "x2mask"), c2, h, w,
         filt.data_ptr(), cin_total, k, stride, pad, cout, out_ts.ref,
-        nhwc_ptr(out_delta, "out_delta"), nhwc_ptr(reservoir, "reservoir"),
+        nhwc_ptr(out_delta, "out_delta"), nhwc_ptr(addend, "addend", cout), nhwc_ptr(reservoir, "reservoir"),
         act, float(slope), path, _stream(x)))
     return out_delta
 
 
 def conv_refresh(x, x2, filt, bias, k, stride, pad, out_ts: TileMask, out_dense, reservoir=None,
-                 act=_lib.ACT_NONE, slope=0.0, path=_lib.PATH_AUTO):
+                 act=_lib.ACT_NONE, slope=0.0, path=_lib.PATH_AUTO, addend=None):
     """Dense conv + bias (+ activation, + reservoir fill) over the tiles of out_ts (all active)."""
     n, c1, h, w = x.shape
     c2 = 0 if x2 is None else x2.shape[1]
@@ -138,7 +140,8 @@ def conv_refresh(x, x2, filt, bias, k, stride, pad, out_ts: TileMask, out_dense,
     check(lib().mie_conv_refresh(
         nhwc_ptr(x, "x"), c1, nhwc_ptr(x2, "x2"), c2, h, w, filt.data_ptr(), cin_total, k, stride, pad,
         cout, None if bias is None else bias.data_ptr(), out_ts.ref, nhwc_ptr(out_dense, "out_dense"),
-        nhwc_ptr(reservoir, "reservoir"), act, float(slope), path, _stream(x)))
+        nhwc_ptr(addend, "addend", cout), nhwc_ptr(reservoir, "reservoir"), act, float(slope), path,
+        _stream(x)))
     return out_dense
 
 

@@ -62,34 +62,34 @@ def test_invalid_arguments_return_status_not_abort(mie_lib):
     err = lambda: mie_lib.mie_last_error_string().decode()
     # NULL tile set
     assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 16, 16, p, 16, 3, 1, 1, 32, None, p,
-                                   None, 0, 0.0, 0, None) == -1
+                                   None, None, 0, 0.0, 0, None) == -1
     assert "tile set is NULL" in err()
     # NULL input pointer
     assert mie_lib.mie_conv_masked(None, None, 16, None, None, 0, 16, 16, p, 16, 3, 1, 1, 32,
-                                   ctypes.byref(ts), p, None, 0, 0.0, 0, None) == -1
+                                   ctypes.byref(ts), p, None, None, 0, 0.0, 0, None) == -1
     # unsupported kernel size and stride (the reference throws std::logic_error, ext_conv.cu:366)
     assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 16, 16, p, 16, 4, 1, 1, 32,
-                                   ctypes.byref(ts), p, None, 0, 0.0, 0, None) == -2
+                                   ctypes.byref(ts), p, None, None, 0, 0.0, 0, None) == -2
     assert "kernel size 4" in err()
     assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 16, 16, p, 16, 3, 3, 1, 32,
-                                   ctypes.byref(ts), p, None, 0, 0.0, 0, None) == -2
+                                   ctypes.byref(ts), p, None, None, 0, 0.0, 0, None) == -2
     # output geometry mismatch
     assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 20, 16, p, 16, 3, 1, 1, 32,
-                                   ctypes.byref(ts), p, None, 0, 0.0, 0, None) == -1
+                                   ctypes.byref(ts), p, None, None, 0, 0.0, 0, None) == -1
     assert "tile set is" in err()
     # misaligned pointer
     assert mie_lib.mie_conv_masked(p + 4, None, 16, None, None, 0, 16, 16, p, 16, 3, 1, 1, 32,
-                                   ctypes.byref(ts), p, None, 0, 0.0, 0, None) == -1
+                                   ctypes.byref(ts), p, None, None, 0, 0.0, 0, None) == -1
     assert "aligned" in err()
     # MFMA path on a shape it cannot take
     assert mie_lib.mie_conv_masked(p, None, 24, None, None, 0, 16, 16, p, 24, 3, 1, 1, 32,
-                                   ctypes.byref(ts), p, None, 0, 0.0, _lib.PATH_MFMA, None) == -2
+                                   ctypes.byref(ts), p, None, None, 0, 0.0, _lib.PATH_MFMA, None) == -2
     # activation without a reservoir
     assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 16, 16, p, 16, 3, 1, 1, 32,
-                                   ctypes.byref(ts), p, None, _lib.ACT_RELU, 0.0, 0, None) == -1
+                                   ctypes.byref(ts), p, None, None, _lib.ACT_RELU, 0.0, 0, None) == -1
     # channels beyond the filter
     assert mie_lib.mie_conv_masked(p, None, 16, p, None, 16, 16, 16, p, 16, 3, 1, 1, 32,
-                                   ctypes.byref(ts), p, None, 0, 0.0, 0, None) == -1
+                                   ctypes.byref(ts), p, None, None, 0, 0.0, 0, None) == -1
     # tile set with a NULL member / zero-sized geometry
     bad, keep2 = _fake_tileset(null="tiles")
     assert mie_lib.mie_act_incr(1, 0.0, p, p, p, 8, ctypes.byref(bad), None, 0, None) == -1

@@ -191,3 +191,40 @@ def test_large_channel_mfma_bottleneck_shapes():
         d, m = gaussian_delta(n, cin, h, w, 0.2, 0.2, seed=cin)
         conv = _Conv(n, cin, cout, h, w, 3, 1, 1, seed=9, path=_lib.PATH_MFMA)
         _close(conv.run(d, m), io.conv_incr(d, conv.w, 1, 1), "%d->%d" % (cin, cout))
+
+
+@pytest.mark.parametrize("pname,path", PATHS)
+def test_addend_rides_into_the_epilogue(pname, path):
+    # residual block tail: relu2(conv2(d) + residual) with the residual delta as the conv's addend
+    n, c, h, w = 1, 32, 40, 56
+    conv = _Conv(n, c, c, h, w, 3, 1, 1, seed=10, path=path)
+    r0 = torch.randn(n, c, h, w, generator=torch.Generator().manual_seed(3))
+    res_gpu, res_cpu = _dev(r0.clone()), io.Reserve(r0)
+    for step in range(3):
+        d, m = gaussian_delta(n, c, h, w, 0.08, 0.5, seed=90 + step)
+        resid = d * 0.5                                   # lives on m, which the 3x3 footprint covers
+        dm = m.to(DEV)
+        ops.build_mask_tiles(dm, None, n, h, w, _lib.FOOT_CONV, 3, 1, 1, conv.ts)
+        ops.conv_masked(_dev(d), dm, None, None, conv.filt, 3, 1, 1, conv.ts, conv.out, res_gpu,
+                        _lib.ACT_RELU, 0.0, path, _dev(resid))
+        torch.cuda.synchronize()
+        ref = io.act_incr(torch.relu, res_cpu, io.conv_incr(d, conv.w, 1, 1) + resid)
+        _close(conv.out, ref, "step %d" % step)
+        _close(res_gpu, res_cpu.reservoir, "reservoir %d" % step)
+
+
+def test_refresh_conv_matches_dense_conv_with_bias():
+    n, cin, cout, h, w = 2, 32, 64, 37, 45
+    g = torch.Generator().manual_seed(5)
+    x, x2 = torch.randn(n, cin, h, w, generator=g), torch.randn(n, cin, h, w, generator=g)
+    wt = he_normal_conv_weight(cout, 2 * cin, 3, 11)
+    bias = torch.randn(cout, generator=g)
+    ts = TileMask(n, h, w, DEV)
+    ops.build_mask_tiles(None, None, n, h, w, _lib.FOOT_CONV, 1, 1, 0, ts)
+    out, res = ops.new_nhwc(n, cout, h, w, DEV), ops.new_nhwc(n, cout, h, w, DEV)
+    for path in (_lib.PATH_VALU, _lib.PATH_MFMA):
+        ops.conv_refresh(_dev(x), _dev(x2), _filt(wt), bias.to(DEV), 3, 1, 1, ts, out, res, _lib.ACT_TANH, 0.0, path)
+        torch.cuda.synchronize()
+        pre = io.conv_refresh(torch.cat((x, x2), 1), wt, bias, 1, 1)
+        _close(res, pre, "reservoir = pre-activation")
+        _close(out, torch.tanh(pre), "activated output")
