@@ -1,0 +1,488 @@
+"""Recurrent multi-resolution EV-FlowNet (ConvGRU) in incremental form.
+
+Restates incr_modules/evflownet_incr.py of the reference on the masked kernels:
+same class names, constructor arguments and sub-module names, the forward /
+forward_refresh_reservoirs pair, stride-2 3x3 encoders each followed by a
+ConvGRU, two residual blocks, decoders with concatenated skips and a 2-channel
+tanh flow head per scale whose prediction is fed to the next decoder.
+
+What differs on purpose:
+* The concat of (previous flow, x, skip) in front of a decoder is never formed
+  for the up-sampling decoders: bilinear x2 is per channel and a conv over a
+  concat is the sum of convs over its parts, so the two wide parts go through
+  the matrix-core conv as two input pointers and the 2-channel flow part through
+  a small conv whose result rides in as the addend of the wide one.
+* `ResidualBlockIncr` of the reference applies ONE activation module (one
+  reservoir) to two different tensors and adds the residual with `+=` on
+  lists (:252-263); here each use has its own reservoir and the residual is a
+  tensor sum, as the dense twin (:285) defines.
+* `ConvGRUIncr.forward` of the reference ignores the reset gate (:58-66).  That
+  is exact when the recurrent state held at refresh time is zero (the drivers
+  pass no state); it is restated as is.
+* Constructor arguments replace the literals of the reference class
+  (`num_bins`, `base_num_channels`, decoder kind), defaults = the reference's.
+"""
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import _lib, ops
+from .masked_types import DenseT, Masked, TileMask
+from .mask_incr_functional import _unpack
+from .mask_incr_modules import (_IncrBuffers, nnAddIncr, nnBatchNorm2dIncr, nnConvIncr,
+                                nnConvTranspose2dIncr, nnReservedActivation, nnReservedMultiplication,
+                                nnSigmoidIncr, nnTanhIncr, nnUpsample2xIncr, activation_kind)
+
+
+def skip_concat(x1, x2):
+    """Reference :9-14 (dense tensors; zero-pads x1 to the size of x2)."""
+    diffY = x2.size()[2] - x1.size()[2]
+    diffX = x2.size()[3] - x1.size()[3]
+    padding = nn.ZeroPad2d((diffX // 2, diffX - diffX // 2, diffY // 2, diffY - diffY // 2))
+    x1 = padding(x1)
+    return torch.cat([x1, x2], dim=1)
+
+
+def _mask_of(x_incr):
+    return x_incr[1] if len(x_incr) > 1 else None
+
+
+class nnCatIncr(nn.Module, _IncrBuffers):
+    """Channel concat of deltas with the union of their masks (torch.cat on the clean delta
+    buffers; used where a kernel takes one input pointer only)."""
+
+    def forward(self, parts):
+        deltas = [ops.as_nhwc(p[0]) for p in parts]
+        n, _, h, w = deltas[0].shape
+        pix = [ops.pixel_mask_of(_mask_of(p), d) for p, d in zip(parts, deltas)]
+        out = ops.as_nhwc(torch.cat(deltas, dim=1))
+        if any(m is None for m in pix):
+            return [out, None]
+        ts = self._tile_set("union", n, h, w, out.device)
+        acc = pix[0]
+        for m in pix[1:-1]:
+            acc = torch.maximum(acc, m)
+        ops.build_mask_tiles(acc, pix[-1] if len(pix) > 1 else None, n, h, w, _lib.FOOT_CONV, 1, 1, 0, ts)
+        return [out, ts]
+
+
+class ConvGRUIncr(nn.Module, _IncrBuffers):
+    """Incremental ConvGRU (reference :18-96)."""
+
+    def __init__(self, input_size, hidden_size, kernel_size, activation=None, fuse=True):
+        super().__init__()
+        padding = kernel_size // 2
+        self.input_size = input_size
+        self.hidden_size = hidden_size
+        self.reset_gate = nnConvIncr(input_size + hidden_size, hidden_size, kernel_size, padding=padding)
+        self.update_gate = nnConvIncr(input_size + hidden_size, hidden_size, kernel_size, padding=padding)
+        self.out_gate = nnConvIncr(input_size + hidden_size, hidden_size, kernel_size, padding=padding)
+        assert activation is None, "ConvGRU activation cannot be set (just for compatibility)"
+        nn.init.orthogonal_(self.reset_gate.weight)
+        nn.init.orthogonal_(self.update_gate.weight)
+        nn.init.orthogonal_(self.out_gate.weight)
+        nn.init.constant_(self.reset_gate.bias, 0.0)
+        nn.init.constant_(self.update_gate.bias, 0.0)
+        nn.init.constant_(self.out_gate.bias, 0.0)
+        self.sigmoid1 = nnSigmoidIncr()
+        self.sigmoid2 = nnSigmoidIncr()
+        self.tanh = nnTanhIncr()
+        self.mult = nnReservedMultiplication()
+        self.add_state = nnAddIncr()
+        self.fuse = fuse
+        if fuse:                       # structural masks are passed through the fused epilogues
+            self.sigmoid1.refine_mask = self.tanh.refine_mask = False
+
+    def _gate(self, conv, act, x_incr, h_incr):
+        if self.fuse:
+            return conv.forward_fused(x_incr, act, h_incr)
+        return act(conv(x_incr, h_incr))
+
+    def forward(self, input_incr, prev_state):
+        """new_state = prev_state + mult(out - prev_state, update)  (reference :47-69)."""
+        update = self._gate(self.update_gate, self.sigmoid1, input_incr, prev_state)
+        out_inputs = self._gate(self.out_gate, self.tanh, input_incr, prev_state)
+        if prev_state is None:
+            new_state = self.mult(out_inputs, update)
+        else:
+            diff = [ops.as_nhwc(out_inputs[0] - prev_state[0]), None]
+            new_state = self.add_state(prev_state, self.mult(diff, update))
+        return new_state, new_state
+
+    def forward_refresh_reservoirs(self, x, prev_state):
+        self._reset_incr()
+        zero_state = prev_state is None
+        if zero_state:
+            state_size = [x.shape[0], self.hidden_size] + list(x.shape[2:])
+            prev_state = torch.zeros(state_size, dtype=x.dtype, device=x.device).to(memory_format=torch.channels_last)
+        h_in = None if zero_state else prev_state
+        update = self.update_gate.forward_refresh_fused(x, self.sigmoid1, h_in)
+        if zero_state:
+            # prev_state * reset is zero whatever the reset gate says: its conv is skipped
+            out_inputs = self.out_gate.forward_refresh_fused(x, self.tanh, None)
+        else:
+            reset = self.reset_gate.forward_refresh_fused(x, self.sigmoid2, h_in)
+            out_inputs = self.out_gate.forward_refresh_fused(x, self.tanh, prev_state * reset)
+        new_state = prev_state + self.mult.forward_refresh_reservoirs(out_inputs - prev_state, update)
+        self.add_state._reset_incr()
+        return new_state, new_state
+
+
+class ConvLayerIncr(nn.Module):
+    """conv -> [BN] -> activation (reference :99-156)."""
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, activation="relu", norm=None,
+                 BN_momentum=0.1, w_scale=None, padding=None, fuse=True):
+        super().__init__()
+        bias = False if norm == "BN" else True
+        if padding is None:
+            padding = kernel_size // 2
+        self.conv2d = nnConvIncr(in_channels, out_channels, kernel_size, stride, padding, bias=bias)
+        if w_scale is not None:
+            nn.init.uniform_(self.conv2d.weight, -w_scale, w_scale)
+            nn.init.zeros_(self.conv2d.bias)
+        self.activation = None
+        if activation is not None and hasattr(torch, activation):
+            self.activation = nnReservedActivation(getattr(torch, activation), refine_mask=not fuse)
+        self.norm = norm
+        if norm == "BN":
+            self.norm_layer = nnBatchNorm2dIncr(out_channels, momentum=BN_momentum)
+        elif norm == "IN":
+            raise NotImplementedError
+        self.fuse = fuse
+
+    def forward(self, x):
+        if self.fuse and self.activation is not None and self.norm not in ["BN", "IN"]:
+            return self.conv2d.forward_fused(x, self.activation)
+        out = self.conv2d(x)
+        if self.norm in ["BN", "IN"]:
+            out = self.norm_layer(out)
+        if self.activation is not None:
+            out = self.activation(out)
+        return out
+
+    def forward_refresh_reservoirs(self, x):
+        if self.fuse and self.activation is not None and self.norm not in ["BN", "IN"]:
+            return self.conv2d.forward_refresh_fused(x, self.activation)
+        out = self.conv2d.forward_refresh_reservoirs(x)
+        if self.norm in ["BN", "IN"]:
+            out = self.norm_layer.forward_refresh_reservoirs(out)
+        if self.activation is not None:
+            out = self.activation.forward_refresh_reservoirs(out)
+        return out
+
+
+class RecurrentConvLayerIncr(nn.Module):
+    """Reference :160-195."""
+
+    def __init__(self, in_channels, out_channels, kernel_size=3, stride=1, activation_ff="relu",
+                 activation_rec=None, norm=None, BN_momentum=0.1, fuse=True):
+        super().__init__()
+        self.conv = ConvLayerIncr(in_channels, out_channels, kernel_size, stride, activation_ff, norm,
+                                  BN_momentum=BN_momentum, fuse=fuse)
+        self.recurrent_block = ConvGRUIncr(input_size=out_channels, hidden_size=out_channels,
+                                           kernel_size=3, activation=activation_rec, fuse=fuse)
+
+    def forward(self, x, prev_state):
+        x = self.conv(x)
+        x, state = self.recurrent_block(x, prev_state)
+        return x, state
+
+    def forward_refresh_reservoirs(self, x, prev_state):
+        x = self.conv.forward_refresh_reservoirs(x)
+        x, state = self.recurrent_block.forward_refresh_reservoirs(x, prev_state)
+        return x, state
+
+
+class ResidualBlockIncr(nn.Module):
+    """conv - act - conv, + residual, act; returns (out2, out1) (reference :198-289)."""
+
+    def __init__(self, in_channels, out_channels, stride=1, activation="relu", downsample=None,
+                 norm=None, BN_momentum=0.1, fuse=True):
+        super().__init__()
+        bias = False if norm == "BN" else True
+        self.conv1 = nnConvIncr(in_channels, out_channels, kernel_size=3, stride=stride, padding=1, bias=bias)
+        self.activation = self.activation2 = None
+        if activation is not None and hasattr(torch, activation):
+            self.activation = nnReservedActivation(getattr(torch, activation), refine_mask=not fuse)
+            self.activation2 = nnReservedActivation(getattr(torch, activation), refine_mask=not fuse)
+        self.norm = norm
+        if norm == "BN":
+            self.bn1 = nnBatchNorm2dIncr(out_channels, momentum=BN_momentum)
+            self.bn2 = nnBatchNorm2dIncr(out_channels, momentum=BN_momentum)
+        elif norm == "IN":
+            raise NotImplementedError
+        self.conv2 = nnConvIncr(out_channels, out_channels, kernel_size=3, stride=1, padding=1, bias=bias)
+        self.downsample = downsample
+        self.add = nnAddIncr()
+        self.fuse = fuse
+
+    def _fusable(self):
+        return self.fuse and self.activation is not None and self.norm not in ["BN", "IN"] and not self.downsample
+
+    def forward(self, x):
+        residual = x
+        if self._fusable():
+            out1 = self.conv1.forward_fused(x, self.activation)
+            return self.conv2.forward_fused(out1, self.activation2, addend_incr=residual), out1
+        out1 = self.conv1(x)
+        if self.norm in ["BN", "IN"]:
+            out1 = self.bn1(out1)
+        if self.activation is not None:
+            out1 = self.activation(out1)
+        out2 = self.conv2(out1)
+        if self.norm in ["BN", "IN"]:
+            out2 = self.bn2(out2)
+        if self.downsample:
+            residual = self.downsample(x)
+        out2 = self.add(out2, residual, a_covers_b=not self.downsample)
+        if self.activation2 is not None:
+            out2 = self.activation2(out2)
+        return out2, out1
+
+    def forward_refresh_reservoirs(self, x):
+        residual = x
+        if self._fusable():
+            out1 = self.conv1.forward_refresh_fused(x, self.activation)
+            return self.conv2.forward_refresh_fused(out1, self.activation2, addend=residual), out1
+        out1 = self.conv1.forward_refresh_reservoirs(x)
+        if self.norm in ["BN", "IN"]:
+            out1 = self.bn1.forward_refresh_reservoirs(out1)
+        if self.activation is not None:
+            out1 = self.activation.forward_refresh_reservoirs(out1)
+        out2 = self.conv2.forward_refresh_reservoirs(out1)
+        if self.norm in ["BN", "IN"]:
+            out2 = self.bn2.forward_refresh_reservoirs(out2)
+        if self.downsample:
+            residual = self.downsample.forward_refresh_reservoirs(x)
+        out2 = self.add.forward_refresh_reservoirs(out2, residual)
+        if self.activation2 is not None:
+            out2 = self.activation2.forward_refresh_reservoirs(out2)
+        return out2, out1
+
+
+class UpsampleConvLayerIncr(nn.Module):
+    """bilinear x2 -> conv -> activation over the parts of a concat (reference :294-343).
+
+    forward / forward_refresh_reservoirs take the list of parts in concat order
+    [previous flow (2 ch, optional), x, skip]; in_channels is the channel count of the concat.
+    """
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, activation="relu",
+                 padding=None, norm=None, fuse=True):
+        super().__init__()
+        bias = False if norm == "BN" else True
+        if padding is None:
+            padding = kernel_size // 2
+        self.conv2d = nnConvIncr(in_channels, out_channels, kernel_size, stride, padding, bias=bias)
+        self.activation = None
+        if activation is not None:
+            self.activation = nnReservedActivation(getattr(torch, activation), refine_mask=not fuse)
+        self.norm = norm
+        if norm == "BN":
+            self.norm_layer = nnBatchNorm2dIncr(out_channels)
+        elif norm == "IN":
+            raise NotImplementedError
+        self.up = nn.ModuleList([nnUpsample2xIncr() for _ in range(3)])
+        self.cat = nnCatIncr()
+        # buffers of the conv over the narrow leading part of the concat (it shares conv2d's filter)
+        self.__dict__["_lead"] = _IncrBuffers()
+        self.fuse = fuse
+
+    def _split_ok(self, parts):
+        wide = parts[-2:]
+        return (self.fuse and self.activation is not None and self.norm not in ["BN", "IN"]
+                and len(parts) in (2, 3) and all(p[0].shape[2:] == parts[0][0].shape[2:] for p in parts)
+                and _mask_of(wide[0]) is not None and _mask_of(wide[1]) is not None)
+
+    def forward(self, parts):
+        ups = [self.up[i](p) for i, p in enumerate(parts)]
+        if not self._split_ok(parts):
+            out = self.conv2d(self.cat(ups))
+            if self.norm in ["BN", "IN"]:
+                out = self.norm_layer(out)
+            return out if self.activation is None else self.activation(out)
+        filt = self.conv2d.conv2d_weights
+        lead_c = 0
+        addend = None
+        if len(ups) == 3:
+            lead_c = ups[0][0].shape[1]
+            # the flow estimate of the previous scale shares the mask of x (it is a 1x1 conv + tanh of
+            # it), so the wide conv's output mask covers this partial result
+            addend = self._lead_conv(ups[0], filt[:lead_c])
+        return self.conv2d.forward_fused(ups[-2], self.activation, ups[-1], addend_incr=addend,
+                                         filt=filt[lead_c:])
+
+    def _lead_conv(self, x_incr, filt):
+        k, s, p = self.conv2d._geometry()
+        x, pix, _ = _unpack(x_incr)
+        n, _, h, w = x.shape
+        ho, wo = ops.conv_out_size(h, w, k, s, p)
+        ts = self._lead._tile_set("lead", n, ho, wo, x.device)
+        out = self._lead._delta_buf("lead", (n, self.conv2d.out_channels, ho, wo), x.device)
+        ops.build_mask_tiles(pix, None, n, h, w, _lib.FOOT_CONV, k, s, p, ts)
+        ops.conv_masked(x, pix, None, None, filt, k, s, p, ts, out)
+        return [out, ts]
+
+    def forward_refresh_reservoirs(self, parts):
+        for m in list(self.up) + [self.cat, self._lead]:
+            m._reset_incr()
+        x = torch.cat([F.interpolate(p, scale_factor=2, mode="bilinear", align_corners=False) for p in parts], 1)
+        if self.fuse and self.activation is not None and self.norm not in ["BN", "IN"]:
+            return self.conv2d.forward_refresh_fused(x, self.activation)
+        out = self.conv2d.forward_refresh_reservoirs(x)
+        if self.norm in ["BN", "IN"]:
+            out = self.norm_layer.forward_refresh_reservoirs(out)
+        if self.activation is not None:
+            out = self.activation.forward_refresh_reservoirs(out)
+        return out
+
+
+class TransposedConvLayerIncr(nn.Module):
+    """Transposed conv (stride 2, output_padding 1) -> activation over the concat of the parts:
+    the decoder kind the benchmark configuration of this network names."""
+
+    def __init__(self, in_channels, out_channels, kernel_size, activation="relu", padding=None, norm=None,
+                 fuse=True):
+        super().__init__()
+        if padding is None:
+            padding = kernel_size // 2
+        self.transposed_conv2d = nnConvTranspose2dIncr(in_channels, out_channels, kernel_size, stride=2,
+                                                       padding=padding, output_padding=1, bias=True)
+        self.activation = None
+        if activation is not None:
+            self.activation = nnReservedActivation(getattr(torch, activation), refine_mask=not fuse)
+        self.cat = nnCatIncr()
+        self.fuse = fuse
+
+    def forward(self, parts):
+        x = self.cat(parts)
+        if self.fuse and self.activation is not None:
+            kind, slope = activation_kind(self.activation.op)
+            return self.transposed_conv2d(x, self.activation.in_res.reservoir, kind, slope)
+        out = self.transposed_conv2d(x)
+        return out if self.activation is None else self.activation(out)
+
+    def forward_refresh_reservoirs(self, parts):
+        self.cat._reset_incr()
+        out = self.transposed_conv2d.forward_refresh_reservoirs(torch.cat(list(parts), 1))
+        if self.activation is not None:
+            out = self.activation.forward_refresh_reservoirs(out)
+        return out
+
+
+class MultiResUNetRecurrentIncr(nn.Module, _IncrBuffers):
+    """EVFlowNet-incr (reference :346-495).  Defaults are the reference's literals
+    (2 input bins, base 32, 4 encoders 64/128/256/512, 2 residual blocks, up-sampling
+    decoders, tanh flow heads); `decoder="transposed"` swaps in transposed-conv decoders."""
+
+    def __init__(self, num_bins=2, base_num_channels=32, num_encoders=4, num_residual_blocks=2,
+                 decoder="upsample", fuse=True, mask_threshold=0.0, derive_input_mask=True):
+        super().__init__()
+        self.final_activation = 'tanh'
+        self.w_scale_pred = None
+        self.num_encoders = num_encoders
+        self.num_residual_blocks = num_residual_blocks
+        self.ff_act, self.rec_act = ['relu', None]
+        self.skip_ftn = skip_concat
+        self.kernel_size = 3
+        self.num_bins = num_bins
+        self.norm = None
+        self.base_num_channels = base_num_channels
+        self.channel_multiplier = 2
+        self.num_output_channels = 2
+        self.decoder_kind = decoder
+        self.fuse = fuse
+        self.mask_threshold = float(mask_threshold)
+        self.derive_input_mask = derive_input_mask
+        self.encoder_input_sizes = [int(self.base_num_channels * pow(self.channel_multiplier, i))
+                                    for i in range(self.num_encoders)]
+        self.encoder_output_sizes = [int(self.base_num_channels * pow(self.channel_multiplier, i + 1))
+                                     for i in range(self.num_encoders)]
+        self.max_num_channels = self.encoder_output_sizes[-1]
+        self.encoders = self.build_recurrent_encoders()
+        self.resblocks = self.build_resblocks()
+        self.decoders = self.build_multires_prediction_decoders()
+        self.preds = self.build_multires_prediction_layer()
+        self.num_states = self.num_encoders
+        self.states = [None] * self.num_states
+
+    def build_recurrent_encoders(self):
+        encoders = nn.ModuleList()
+        for i, (input_size, output_size) in enumerate(zip(self.encoder_input_sizes, self.encoder_output_sizes)):
+            if i == 0:
+                input_size = self.num_bins
+            encoders.append(RecurrentConvLayerIncr(input_size, output_size, kernel_size=self.kernel_size,
+                                                   stride=2, activation_ff=self.ff_act,
+                                                   activation_rec=self.rec_act, norm=self.norm, fuse=self.fuse))
+        return encoders
+
+    def build_resblocks(self):
+        resblocks = nn.ModuleList()
+        for _ in range(self.num_residual_blocks):
+            resblocks.append(ResidualBlockIncr(self.max_num_channels, self.max_num_channels,
+                                               activation=self.ff_act, norm=self.norm, fuse=self.fuse))
+        return resblocks
+
+    def build_multires_prediction_layer(self):
+        preds = nn.ModuleList()
+        for output_size in reversed(self.encoder_input_sizes):
+            preds.append(ConvLayerIncr(output_size, self.num_output_channels, 1,
+                                       activation=self.final_activation, norm=self.norm, fuse=self.fuse))
+        return preds
+
+    def build_multires_prediction_decoders(self):
+        decoders = nn.ModuleList()
+        sizes = zip(reversed(self.encoder_output_sizes), reversed(self.encoder_input_sizes))
+        for i, (input_size, output_size) in enumerate(sizes):
+            prediction_channels = 0 if i == 0 else self.num_output_channels
+            cin = 2 * input_size + prediction_channels
+            if self.decoder_kind == "transposed":
+                decoders.append(TransposedConvLayerIncr(cin, output_size, kernel_size=self.kernel_size,
+                                                        activation=self.ff_act, fuse=self.fuse))
+            else:
+                decoders.append(UpsampleConvLayerIncr(cin, output_size, kernel_size=self.kernel_size,
+                                                      activation=self.ff_act, norm=self.norm, fuse=self.fuse))
+        return decoders
+
+    def forward(self, x_incr):
+        delta = ops.as_nhwc(x_incr[0])
+        mask = _mask_of(x_incr)
+        if mask is None and self.derive_input_mask:
+            n, _, h, w = delta.shape
+            mask = ops.mask_from_delta(delta, self.mask_threshold, self._pix_buf("input", n, h, w, delta.device))
+        x_incr = [delta, mask]
+        states_incr = [None] * self.num_states
+        blocks = []
+        for i, encoder in enumerate(self.encoders):
+            x_incr, state = encoder(x_incr, states_incr[i])
+            blocks.append(x_incr)
+            states_incr[i] = state
+        for resblock in self.resblocks:
+            x_incr, _ = resblock(x_incr)
+        predictions = []
+        for i, (decoder, pred) in enumerate(zip(self.decoders, self.preds)):
+            parts = [x_incr, blocks[self.num_encoders - i - 1]]
+            if i > 0:
+                parts = [predictions[-1]] + parts
+            x_incr = decoder(parts)
+            predictions.append(pred(x_incr))
+        return predictions
+
+    def forward_refresh_reservoirs(self, x):
+        self._reset_incr()
+        blocks = []
+        for i, encoder in enumerate(self.encoders):
+            x, state = encoder.forward_refresh_reservoirs(x, self.states[i])
+            blocks.append(x)
+            self.states[i] = state
+        for resblock in self.resblocks:
+            x, _ = resblock.forward_refresh_reservoirs(x)
+        predictions = []
+        for i, (decoder, pred) in enumerate(zip(self.decoders, self.preds)):
+            parts = [x, blocks[self.num_encoders - i - 1]]
+            if i > 0:
+                parts = [predictions[-1]] + parts
+            x = decoder.forward_refresh_reservoirs(parts)
+            predictions.append(pred.forward_refresh_reservoirs(x))
+        return predictions

@@ -45,6 +45,54 @@ def event_voxel_delta(n, bins, h, w, density, seed) -> "tuple[torch.Tensor, torc
     return counts * sign * 0.1 * m.float(), m
 
 
+class MovingEdges:
+    """Moving-edge event generator: random line segments that translate 1-3 px per step; the
+    pixels a segment sweeps in a step fire events.  Yields (delta NCHW fp32, mask uint8) per
+    step for a 4-channel event image: positive / negative counts and their latest timestamps."""
+
+    def __init__(self, h, w, segments=17, seed=0, thickness=1):
+        self.h, self.w, self.thickness = h, w, thickness
+        self.rng = np.random.default_rng(seed)
+        r = self.rng
+        self.p0 = np.stack([r.uniform(0, h, segments), r.uniform(0, w, segments)], 1)
+        ang = r.uniform(0, 2 * np.pi, segments)
+        length = r.uniform(0.15, 0.5, segments) * min(h, w)
+        self.d = np.stack([np.sin(ang), np.cos(ang)], 1) * length[:, None]
+        vang = r.uniform(0, 2 * np.pi, segments)
+        speed = r.uniform(1.0, 3.0, segments)
+        self.v = np.stack([np.sin(vang), np.cos(vang)], 1) * speed[:, None]
+        self.pol = r.integers(0, 2, segments)
+        self.t = 0
+
+    def _raster(self):
+        m = np.zeros((self.h, self.w), dtype=np.int8)
+        pol = np.zeros((self.h, self.w), dtype=np.int8)
+        for p0, d, pl in zip(self.p0, self.d, self.pol):
+            npts = int(np.hypot(*d)) * 2 + 2
+            ts = np.linspace(0.0, 1.0, npts)
+            ys = np.round(p0[0] + ts * d[0]).astype(int) % self.h
+            xs = np.round(p0[1] + ts * d[1]).astype(int) % self.w
+            for dy in range(self.thickness):
+                m[(ys + dy) % self.h, xs] = 1
+                pol[(ys + dy) % self.h, xs] = pl
+        return m, pol
+
+    def step(self):
+        before, _ = self._raster()
+        self.p0 = self.p0 + self.v
+        self.t += 1
+        after, pol = self._raster()
+        fired = ((after == 1) & (before == 0)) | ((after == 0) & (before == 1))
+        counts = self.rng.poisson(2.0, size=(self.h, self.w)).astype(np.float32) + 1.0
+        d = np.zeros((1, 4, self.h, self.w), dtype=np.float32)
+        d[0, 0] = fired * (pol == 1) * counts
+        d[0, 1] = fired * (pol == 0) * counts
+        d[0, 2] = fired * (pol == 1) * 0.1 * self.t
+        d[0, 3] = fired * (pol == 0) * 0.1 * self.t
+        mask = fired.astype(np.uint8)[None, None]
+        return torch.from_numpy(d) * 0.1, torch.from_numpy(mask)
+
+
 def he_normal_conv_weight(cout, cin, k, seed) -> torch.Tensor:
     """He-normal (std sqrt(2 / (cin * k * k))) conv weight, OIHW."""
     g = torch.Generator().manual_seed(int(seed))
