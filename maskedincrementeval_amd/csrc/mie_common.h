@@ -72,6 +72,8 @@ __device__ __forceinline__ int mie_pick_tile(const TileSetDev& ts, int b,
                                              int& n, int& y0, int& x0) {
   const int n_active = ts.counts[MIE_CNT_ACTIVE];
   const int n_stale = ts.counts[MIE_CNT_STALE];
+  const int cap = ts.n * ts.tiles_y * ts.tiles_x;
+  if (n_active < 0 || n_stale < 0 || n_active > cap || n_stale > cap) return 0;   // corrupt counts
   int tile, kind;
   if (b < n_active) {
     tile = ts.tiles[b];
@@ -82,6 +84,7 @@ __device__ __forceinline__ int mie_pick_tile(const TileSetDev& ts, int b,
   } else {
     return 0;
   }
+  if (tile < 0 || tile >= cap) return 0;    // corrupt list entry: skip rather than touch memory
   const int tx = tile % ts.tiles_x;
   const int t2 = tile / ts.tiles_x;
   const int ty = t2 % ts.tiles_y;

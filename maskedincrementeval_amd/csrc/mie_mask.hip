@@ -206,11 +206,16 @@ __device__ int block_compact(int count, KeepFn keep, IdFn id, int32_t* dst, int*
 __global__ __launch_bounds__(COMPACT_THREADS) void k_compact_tiles(BuildArgs a) {
   __shared__ int s_tot[COMPACT_WAVES];
   const uint32_t* flags = a.flags;
-  const int n_prev = a.counts[MIE_CNT_ACTIVE];
+  // Clamp what comes from memory: a tile set whose counts / list were never initialised must
+  // give a wrong list, never an out-of-bounds access.
+  int n_prev = a.counts[MIE_CNT_ACTIVE];
+  n_prev = n_prev < 0 ? 0 : (n_prev > a.cap ? a.cap : n_prev);
   const int32_t* prev = a.tiles;
+  const int cap = a.cap;
   const int n_stale = block_compact(
-      n_prev, [&](int i) { return flags[prev[i]] == 0u; }, [&](int i) { return prev[i]; },
-      a.stale, s_tot);
+      n_prev,
+      [&](int i) { const int t = prev[i]; return t >= 0 && t < cap && flags[t] == 0u; },
+      [&](int i) { return prev[i]; }, a.stale, s_tot);
   __syncthreads();   // the old list has been consumed; it is overwritten next
   const int n_act = block_compact(
       a.cap, [&](int i) { return flags[i] != 0u; }, [&](int i) { return i; }, a.tiles, s_tot);

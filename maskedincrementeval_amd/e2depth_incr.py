@@ -493,8 +493,10 @@ class E2VIDRecurrentIncr(nn.Module, _IncrBuffers):
     any_c(|delta| > mask_threshold).
     """
 
-    def __init__(self, config=None, fuse=True, mask_threshold: float = 0.0, derive_input_mask=True):
+    def __init__(self, config=None, fuse=True, mask_threshold: float = 0.0, derive_input_mask=True,
+                 async_masks=True):
         super().__init__()
+        self.async_masks = async_masks     # build the tile sets on a second stream, ahead of the convs
         cfg = dict(E2DEPTH_DEFAULT_CONFIG)
         cfg.update(config or {})
         self.num_bins = int(cfg['num_bins'])
@@ -527,9 +529,14 @@ class E2VIDRecurrentIncr(nn.Module, _IncrBuffers):
     def forward(self, event_tensor: Masked, prev_states):
         delta = ops.as_nhwc(event_tensor[0])
         mask = _mask_of(event_tensor)
-        if mask is None and self.derive_input_mask:
-            mask = self.input_mask(delta)
-        img_pred, states = self.unetrecurrent.forward([delta, mask], prev_states)
+        if not self.async_masks:
+            if mask is None and self.derive_input_mask:
+                mask = self.input_mask(delta)
+            return self.unetrecurrent.forward([delta, mask], prev_states)
+        with ops.mask_planner(delta.device):
+            if mask is None and self.derive_input_mask:
+                mask = self.input_mask(delta)
+            img_pred, states = self.unetrecurrent.forward([delta, mask], prev_states)
         return img_pred, states
 
     def forward_refresh_reservoirs(self, event_tensor: DenseT, prev_states):

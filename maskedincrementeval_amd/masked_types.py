@@ -53,6 +53,7 @@ class TileMask:
             self.tiles, self.stale = _parent.tiles, _parent.stale
             self.counts, self.flags = _parent.counts, _parent.flags
         self.parent = _parent
+        self.ready = None      # event of the latest build when it ran on the mask-planning stream
         self.c_struct = _lib.MieTileSet(
             self.n, self.h, self.w, self.pixmask.data_ptr(), self.tiles.data_ptr(),
             self.stale.data_ptr(), self.counts.data_ptr(), self.flags.data_ptr())

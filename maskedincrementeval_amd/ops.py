@@ -17,6 +17,68 @@ def _stream(t: torch.Tensor):
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
+# ---- mask planning on a side stream -------------------------------------------------------------
+# The structural masks / tile lists of a network depend on the input mask only, never on the
+# values, so their builds can run ahead of the convolutions.  Inside `mask_planner()` every
+# mie_build_mask_tiles goes to a second stream (default priority); each tile set carries the
+# event of its build and the first kernel that uses it makes the compute stream wait for it.
+# Pixel masks written on the compute stream (input mask, refined masks) carry an event the
+# other way.  Under HIP-graph capture these waits become edges of the graph.
+_planner = None          # (side stream, device) while active
+_side_streams = {}
+_pix_ready = {}          # data_ptr of a pixel mask written on the compute stream -> event
+
+
+class mask_planner:
+    def __init__(self, device):
+        self.device = torch.device(device)
+
+    def __enter__(self):
+        global _planner
+        if _planner is not None or self.device.type != "cuda":
+            self.nested = True
+            return self
+        self.nested = False
+        side = _side_streams.get(self.device)
+        if side is None:
+            side = torch.cuda.Stream(self.device)
+            _side_streams[self.device] = side
+        ev = torch.cuda.Event()
+        ev.record(torch.cuda.current_stream(self.device))
+        side.wait_event(ev)          # forks from the compute stream (also joins a graph capture)
+        _planner = (side, self.device)
+        return self
+
+    def __exit__(self, *exc):
+        global _planner
+        if self.nested:
+            return False
+        side, dev = _planner
+        _planner = None
+        _pix_ready.clear()
+        ev = torch.cuda.Event()
+        ev.record(side)
+        torch.cuda.current_stream(dev).wait_event(ev)     # join
+        return False
+
+
+def _ready(ts: TileMask):
+    """Make the compute stream wait for the build of `ts` (once)."""
+    root = ts.parent if ts.parent is not None else ts
+    ev = root.__dict__.get("ready")
+    if ev is not None:
+        torch.cuda.current_stream(ts.device).wait_event(ev)
+        root.ready = None
+
+
+def _mark_pix(t: Optional[torch.Tensor]):
+    """A pixel mask was written on the compute stream: builds that read it must wait."""
+    if _planner is not None and t is not None:
+        ev = torch.cuda.Event()
+        ev.record(torch.cuda.current_stream(t.device))
+        _pix_ready[t.data_ptr()] = ev
+
+
 def _require_gpu(t: torch.Tensor, name: str):
     if not t.is_cuda:
         raise RuntimeError("%s must live on the GPU (got %s); this package has no CPU path"
@@ -85,6 +147,7 @@ def mask_from_delta(delta: torch.Tensor, threshold: float, out: torch.Tensor):
     n, c, h, w = delta.shape
     check(lib().mie_mask_from_delta(nhwc_ptr(delta, "delta"), n, h, w, c, float(threshold),
                                     pix_ptr(out, n, h, w, "out"), _stream(delta)))
+    _mark_pix(out)
     return out
 
 
@@ -94,8 +157,27 @@ def build_mask_tiles(in_mask, in_mask2, n, h_in, w_in, foot, k, stride, pad, out
     p2 = pix_ptr(in_mask2, n, h_in, w_in, "in_mask2")
     if p1 is None and p2 is not None:   # "all active" OR anything = all active
         p2 = None
-    st = torch.cuda.current_stream(out.device).cuda_stream
-    check(lib().mie_build_mask_tiles(p1, p2, h_in, w_in, foot, k, stride, pad, out.ref, st))
+    if _planner is None or _planner[1] != out.device:
+        st = torch.cuda.current_stream(out.device).cuda_stream
+        check(lib().mie_build_mask_tiles(p1, p2, h_in, w_in, foot, k, stride, pad, out.ref, st))
+        return out
+    side = _planner[0]
+    root = out.parent if out.parent is not None else out
+    if not root.__dict__.get("built_once"):
+        # a freshly allocated tile set is zero-filled on the compute stream: its first build
+        # on the planning stream must come after that fill
+        ev0 = torch.cuda.Event()
+        ev0.record(torch.cuda.current_stream(out.device))
+        side.wait_event(ev0)
+        root.built_once = True
+    for ptr in (p1, p2):
+        ev = _pix_ready.get(ptr)
+        if ev is not None:
+            side.wait_event(ev)
+    check(lib().mie_build_mask_tiles(p1, p2, h_in, w_in, foot, k, stride, pad, out.ref, side.cuda_stream))
+    ev = torch.cuda.Event()
+    ev.record(side)
+    root.ready = ev
     return out
 
 
@@ -117,6 +199,7 @@ def conv_masked(x, xmask, x2, x2mask, filt, k, stride, pad, out_ts: TileMask, ou
         raise ValueError("reservoir shape %s != output %s" % (tuple(reservoir.shape), tuple(out_delta.shape)))
     if addend is not None and addend.shape != out_delta.shape:
         raise ValueError("addend shape %s != output %s" % (tuple(addend.shape), tuple(out_delta.shape)))
+    _ready(out_ts)
     check(lib().mie_conv_masked(
         nhwc_ptr(x, "x"), pix_ptr(xmask, n, h, w, "xmask"), c1,
         nhwc_ptr(x2, "x2"), pix_ptr(x2mask, n, h, w, "x2mask"), c2, h, w,
@@ -137,6 +220,7 @@ def conv_refresh(x, x2, filt, bias, k, stride, pad, out_ts: TileMask, out_dense,
         raise ValueError("out_dense shape %s, expected %s" % (tuple(out_dense.shape), (n, cout, out_ts.h, out_ts.w)))
     if bias is not None and (bias.numel() != cout or bias.dtype != torch.float32 or not bias.is_contiguous()):
         raise ValueError("bias must be contiguous fp32 of %d elements" % cout)
+    _ready(out_ts)
     check(lib().mie_conv_refresh(
         nhwc_ptr(x, "x"), c1, nhwc_ptr(x2, "x2"), c2, h, w, filt.data_ptr(), cin_total, k, stride, pad,
         cout, None if bias is None else bias.data_ptr(), out_ts.ref, nhwc_ptr(out_dense, "out_dense"),
@@ -155,6 +239,7 @@ def tconv_masked(x, xmask, filt, k, stride, pad, out_ts: TileMask, out_delta, re
     cout = filt.shape[3]
     if tuple(out_delta.shape) != (n, cout, out_ts.h, out_ts.w):
         raise ValueError("out_delta shape %s" % (tuple(out_delta.shape),))
+    _ready(out_ts)
     check(lib().mie_tconv_masked(
         nhwc_ptr(x, "x"), pix_ptr(xmask, n, h, w, "xmask"), cin, h, w, filt.data_ptr(), k, stride,
         pad, cout, out_ts.ref, nhwc_ptr(out_delta, "out_delta"), nhwc_ptr(reservoir, "reservoir"),
@@ -174,11 +259,13 @@ def act_incr(kind, slope, in_delta, reservoir, out_delta, ts: TileMask, out_pixm
     _same_shape("out_delta", out_delta, in_delta)
     if (ts.n, ts.h, ts.w) != (n, h, w):
         raise ValueError("tile set %s does not match delta %s" % ((ts.n, ts.h, ts.w), (n, h, w)))
+    _ready(ts)
     check(lib().mie_act_incr(kind, float(slope), nhwc_ptr(in_delta, "in_delta"),
                              nhwc_ptr(reservoir, "reservoir"), nhwc_ptr(out_delta, "out_delta"), c,
                              ts.ref, pix_ptr(out_pixmask, n, h, w, "out_pixmask"),
                              _lib.FLAG_KEEP_RESERVOIR if keep_reservoir else 0,
                              _stream(in_delta)))
+    _mark_pix(out_pixmask)
     return out_delta
 
 
@@ -186,6 +273,7 @@ def mul_incr(d1, m1, r1, d2, m2, r2, out_delta, ts: TileMask, keep_reservoir=Fal
     n, c, h, w = d1.shape
     for name, t in (("r1", r1), ("d2", d2), ("r2", r2), ("out_delta", out_delta)):
         _same_shape(name, t, d1)
+    _ready(ts)
     check(lib().mie_mul_incr(nhwc_ptr(d1, "d1"), pix_ptr(m1, n, h, w, "m1"), nhwc_ptr(r1, "r1"),
                              nhwc_ptr(d2, "d2"), pix_ptr(m2, n, h, w, "m2"), nhwc_ptr(r2, "r2"),
                              nhwc_ptr(out_delta, "out_delta"), c, ts.ref,
@@ -197,6 +285,7 @@ def add_incr(a, ma, b, mb, out_delta, ts: TileMask):
     n, c, h, w = a.shape
     _same_shape("b", b, a)
     _same_shape("out_delta", out_delta, a)
+    _ready(ts)
     check(lib().mie_add_incr(nhwc_ptr(a, "a"), pix_ptr(ma, n, h, w, "ma"), nhwc_ptr(b, "b"),
                              pix_ptr(mb, n, h, w, "mb"), nhwc_ptr(out_delta, "out_delta"), c,
                              ts.ref, _stream(a)))
@@ -209,6 +298,7 @@ def upsample2x_incr(a, ma, b, mb, out_ts: TileMask, out_delta):
         _same_shape("b", b, a)
     if tuple(out_delta.shape) != (n, c, 2 * h, 2 * w):
         raise ValueError("out_delta shape %s, expected %s" % (tuple(out_delta.shape), (n, c, 2 * h, 2 * w)))
+    _ready(out_ts)
     check(lib().mie_upsample2x_incr(nhwc_ptr(a, "a"), pix_ptr(ma, n, h, w, "ma"),
                                     nhwc_ptr(b, "b"), pix_ptr(mb, n, h, w, "mb"), h, w, c,
                                     out_ts.ref, nhwc_ptr(out_delta, "out_delta"), _stream(a)))
@@ -226,6 +316,7 @@ def convlstm_gates_incr(gates_delta, gates_res, cprev_delta, cprev_mask, cprev_r
                     ("c_delta", c_delta)):
         if tuple(t.shape) != (n, hid, h, w):
             raise ValueError("%s shape %s, expected %s" % (name, tuple(t.shape), (n, hid, h, w)))
+    _ready(ts)
     check(lib().mie_convlstm_gates_incr(
         nhwc_ptr(gates_delta, "gates_delta"), nhwc_ptr(gates_res, "gates_res"),
         nhwc_ptr(cprev_delta, "cprev_delta"), pix_ptr(cprev_mask, n, h, w, "cprev_mask"),

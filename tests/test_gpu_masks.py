@@ -127,3 +127,41 @@ def test_repeated_builds_are_deterministic():
             ref = tiles
         assert np.array_equal(tiles, ref)
         assert ts.stale_tiles().numel() == 0
+
+
+def test_planner_builds_fresh_tile_sets_after_their_zero_fill():
+    # builds on the planning stream must be ordered after the zero-fill of a freshly allocated tile
+    # set, and consumers after the build: many fresh tile sets, each used right away
+    n, h, w = 1, 64, 96
+    m = blob_mask(h, w, 0.1, seed=3)[None]
+    dm = _to_dev_mask(m)
+    want = mo.footprint_conv(m, 3, 1, 1)
+    for rep in range(8):
+        junk = torch.full((4096,), 0x7fffffff, dtype=torch.int32, device=DEV)   # recycled by the allocator
+        del junk
+        with ops.mask_planner(torch.device(DEV)):
+            ts = TileMask(n, h, w, DEV)
+            ops.build_mask_tiles(dm, None, n, h, w, _lib.FOOT_CONV, 3, 1, 1, ts)
+            out = ops.new_nhwc(n, 8, h, w, DEV)
+            res = ops.new_nhwc(n, 8, h, w, DEV)
+            d = torch.ones(n, 8, h, w, device=DEV).contiguous(memory_format=torch.channels_last)
+            ops.act_incr(_lib.ACT_RELU, 0.0, ops.as_nhwc(d), res, out, ts)
+        torch.cuda.synchronize()
+        _check_tileset(ts, want)
+        assert np.array_equal((out[:, 0] != 0).cpu().numpy().astype(np.uint8), want)
+
+
+def test_out_of_range_counts_are_ignored_by_kernels():
+    # counts beyond the capacity (a tile set that was never built) make kernels skip, not read
+    n, h, w = 1, 32, 32
+    ts = TileMask(n, h, w, DEV)
+    ts.counts[_lib.CNT_ACTIVE] = ts.capacity + 7
+    ts.tiles.fill_(-1)
+    out = torch.full((n, 4, h, w), 5.0, device=DEV).contiguous(memory_format=torch.channels_last)
+    res = ops.new_nhwc(n, 4, h, w, DEV)
+    ops.act_incr(_lib.ACT_RELU, 0.0, ops.as_nhwc(torch.ones_like(out)), res, ops.as_nhwc(out), ts)
+    torch.cuda.synchronize()
+    assert torch.count_nonzero(res) == 0
+    # a build on top of it recovers a valid list
+    ops.build_mask_tiles(None, None, n, h, w, _lib.FOOT_CONV, 1, 1, 0, ts)
+    _check_tileset(ts, np.ones((n, h, w), np.uint8))
