@@ -40,6 +40,8 @@ def parse_args():
     ap.add_argument("--no-graph", action="store_true", help="launch kernels eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-dense", action="store_true", help="skip the all-tiles-active comparator")
     ap.add_argument("--layer-iters", type=int, default=20, help="timed launches per layer for the roofline table")
+    ap.add_argument("--sync-masks", action="store_true", help="build tile sets on the compute stream (no planning stream)")
+    ap.add_argument("--sweep", action="store_true", help="also time 1 %% and 20 %% density (reported under \"density_sweep\")")
     return ap.parse_args()
 
 
@@ -157,7 +159,7 @@ def main():
     H, W, dens = args.height, args.width, args.density
     cl = lambda t: t.to(dev).contiguous(memory_format=torch.channels_last)
 
-    model = seed_module_(E2VIDRecurrentIncr(), seed=1).to(dev).eval()
+    model = seed_module_(E2VIDRecurrentIncr(async_masks=not args.sync_masks), seed=1).to(dev).eval()
     x0 = torch.randn(1, 5, H, W, generator=torch.Generator().manual_seed(2)) * 0.5
     n_inputs = 16
     deltas_cpu = [event_voxel_delta(1, 5, H, W, dens, seed=3000 + i)[0] for i in range(n_inputs)]
@@ -282,6 +284,19 @@ def main():
         dense_sec = timed_run(dense_model, "dense (all tiles active, same kernels)")
         del dense_model
 
+    # ---- other densities (same network, same kernels) ------------------------------------------------
+    sweep = None
+    if args.sweep:
+        sweep = {"%.2f" % dens: dict(ms_per_step=round(1e3 * sec_per_step, 4), frames_per_s=round(1 / sec_per_step, 1))}
+        keep = list(deltas)
+        for p in (0.01, 0.20):
+            if abs(p - dens) < 1e-9:
+                continue
+            deltas[:] = [cl(event_voxel_delta(1, 5, H, W, p, seed=3000 + i)[0]) for i in range(n_inputs)]
+            t = timed_run(model, "incremental %.0f%%" % (100 * p))
+            sweep["%.2f" % p] = dict(ms_per_step=round(1e3 * t, 4), frames_per_s=round(1 / t, 1))
+        deltas[:] = keep
+
     # ---- CPU baseline: the oracle (torch-CPU restatement of the reference path) -----------------
     cpu = None
     if args.cpu_steps > 0:
@@ -325,6 +340,7 @@ def main():
         "sum_kernel_us": round(tot_us, 1),
         "dense_same_kernels_ms": None if dense_sec is None else round(1e3 * dense_sec, 4),
         "speedup_vs_dense": None if dense_sec is None else round(dense_sec / sec_per_step, 3),
+        "density_sweep": sweep,
         "layers": layers,
     }
     print(json.dumps(result))

@@ -151,10 +151,7 @@ __device__ int footprint_bit(const BuildArgs& a, int n, int oy, int ox) {
 // Kernel 1: one wave per output tile.  Lane = pixel of the 8x8 tile: derives its mask bit
 // from the input footprint, writes the output pixel mask, and a wave ballot tells whether
 // the tile holds any active pixel.
-__global__ __launch_bounds__(256) void k_mask_footprint(BuildArgs a) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int tile = blockIdx.x * 4 + wave;
-  if (tile >= a.cap) return;
+__device__ __forceinline__ bool tile_footprint(const BuildArgs& a, int tile, int lane) {
   const int tx = tile % a.tiles_x;
   const int t2 = tile / a.tiles_x;
   const int ty = t2 % a.tiles_y;
@@ -165,8 +162,15 @@ __global__ __launch_bounds__(256) void k_mask_footprint(BuildArgs a) {
     bit = footprint_bit(a, n, oy, ox);
     a.out[((long long)n * a.h_out + oy) * a.w_out + ox] = (uint8_t)bit;
   }
-  const unsigned long long bal = __ballot(bit != 0);
-  if (lane == 0) a.flags[tile] = (bal != 0ull) ? 1u : 0u;
+  return __ballot(bit != 0) != 0ull;
+}
+
+__global__ __launch_bounds__(256) void k_mask_footprint(BuildArgs a) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = blockIdx.x * 4 + wave;
+  if (tile >= a.cap) return;
+  const bool any = tile_footprint(a, tile, lane);
+  if (lane == 0) a.flags[tile] = any ? 1u : 0u;
 }
 
 // Ordered compaction of the ids `id(i)` (i in [0, count)) for which keep(i) holds, by the
@@ -203,9 +207,8 @@ __device__ int block_compact(int count, KeepFn keep, IdFn id, int32_t* dst, int*
 
 // Kernel 2 (one block): per-tile flags -> stale list (previous list minus the tiles that are
 // still active) and the new ascending active list.
-__global__ __launch_bounds__(COMPACT_THREADS) void k_compact_tiles(BuildArgs a) {
-  __shared__ int s_tot[COMPACT_WAVES];
-  const uint32_t* flags = a.flags;
+template <typename FlagFn>
+__device__ void compact_lists(const BuildArgs& a, FlagFn flag, int* s_tot) {
   // Clamp what comes from memory: a tile set whose counts / list were never initialised must
   // give a wrong list, never an out-of-bounds access.
   int n_prev = a.counts[MIE_CNT_ACTIVE];
@@ -213,16 +216,40 @@ __global__ __launch_bounds__(COMPACT_THREADS) void k_compact_tiles(BuildArgs a) 
   const int32_t* prev = a.tiles;
   const int cap = a.cap;
   const int n_stale = block_compact(
-      n_prev,
-      [&](int i) { const int t = prev[i]; return t >= 0 && t < cap && flags[t] == 0u; },
+      n_prev, [&](int i) { const int t = prev[i]; return t >= 0 && t < cap && !flag(t); },
       [&](int i) { return prev[i]; }, a.stale, s_tot);
   __syncthreads();   // the old list has been consumed; it is overwritten next
   const int n_act = block_compact(
-      a.cap, [&](int i) { return flags[i] != 0u; }, [&](int i) { return i; }, a.tiles, s_tot);
+      a.cap, [&](int i) { return flag(i); }, [&](int i) { return i; }, a.tiles, s_tot);
   if (threadIdx.x == 0) {
     a.counts[MIE_CNT_ACTIVE] = n_act;
     a.counts[MIE_CNT_STALE] = n_stale;
   }
+}
+
+__global__ __launch_bounds__(COMPACT_THREADS) void k_compact_tiles(BuildArgs a) {
+  __shared__ int s_tot[COMPACT_WAVES];
+  const uint32_t* flags = a.flags;
+  compact_lists(a, [&](int t) { return flags[t] != 0u; }, s_tot);
+}
+
+// Planes of at most SMALL_CAP tiles (the 33x44 plane of a 264x352 frame: 30 tiles): footprint
+// and compaction in ONE block, tile flags handed over through LDS -- one launch instead of two.
+constexpr int SMALL_CAP = 32;
+
+__global__ __launch_bounds__(COMPACT_THREADS) void k_build_small(BuildArgs a) {
+  __shared__ int s_tot[COMPACT_WAVES];
+  __shared__ unsigned s_flag[SMALL_CAP];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int tile = wave; tile < a.cap; tile += COMPACT_WAVES) {
+    const bool any = tile_footprint(a, tile, lane);
+    if (lane == 0) {
+      s_flag[tile] = any ? 1u : 0u;
+      a.flags[tile] = any ? 1u : 0u;
+    }
+  }
+  __syncthreads();
+  compact_lists(a, [&](int t) { return s_flag[t] != 0u; }, s_tot);
 }
 
 extern "C" int mie_build_mask_tiles(const uint8_t* in_mask, const uint8_t* in_mask2,
@@ -269,6 +296,10 @@ extern "C" int mie_build_mask_tiles(const uint8_t* in_mask, const uint8_t* in_ma
   a.tiles_y = mie_div_up(out->h, MIE_TILE); a.tiles_x = mie_div_up(out->w, MIE_TILE);
   a.cap = mie_tile_capacity(out->n, out->h, out->w);
   a.tiles = out->tiles; a.stale = out->stale; a.counts = out->counts; a.flags = out->flags;
+  if (a.cap <= SMALL_CAP) {
+    hipLaunchKernelGGL(k_build_small, dim3(1), dim3(COMPACT_THREADS), 0, (hipStream_t)stream, a);
+    return mie_check_launch("mie_build_mask_tiles");
+  }
   const unsigned blocks = (unsigned)mie_div_up(a.cap, 4);
   hipLaunchKernelGGL(k_mask_footprint, dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
   rc = mie_check_launch("mie_build_mask_tiles");

@@ -494,7 +494,7 @@ class E2VIDRecurrentIncr(nn.Module, _IncrBuffers):
     """
 
     def __init__(self, config=None, fuse=True, mask_threshold: float = 0.0, derive_input_mask=True,
-                 async_masks=True):
+                 async_masks=False):
         super().__init__()
         self.async_masks = async_masks     # build the tile sets on a second stream, ahead of the convs
         cfg = dict(E2DEPTH_DEFAULT_CONFIG)
