@@ -128,6 +128,18 @@ int mie_build_mask_tiles(const uint8_t* in_mask, const uint8_t* in_mask2,
                          int pad, const mie_tileset* out, void* stream);
 
 /*
+ * Re-order a [cin][k][k][cout] filter (cin % 8 == 0) into the layout the
+ * matrix-core kernels stream: P[ci/8][tap][(ci%8)/4][co][ci%4], so that the four
+ * k-steps a lane multiplies per tap come as one 16-byte load.  `packed` has the
+ * size of `filter`; do this once per weight update.
+ * Replaces: convert_filter_out_channels_last
+ * (ext/pointops/pointops_functional.py:13-14), which plays the same role for
+ * the reference kernel.
+ */
+int mie_pack_filter(const float* filter, int cin, int k, int cout, float* packed,
+                    void* stream);
+
+/*
  * Masked convolution of a delta: for every active tile of `out`
  *   acc = conv2d(x (++ x2), filter, bias = none, stride, pad)
  * and then, with reservoir == NULL:      out_delta  = acc
@@ -146,6 +158,10 @@ int mie_build_mask_tiles(const uint8_t* in_mask, const uint8_t* in_mask2,
  *        feeds filter input channels [c1, c1 + c2) -- the concat-free form of
  *        torch.cat((x, h), 1) in ConvLSTMIncr (incr_modules/e2depth_incr.py:100)
  *   filter : [cin_total][k][k][cout], c1 + c2 <= cin_total
+ *   filter_mc : optional copy of the same filter in the matrix-core layout made
+ *        by mie_pack_filter (same size).  The MFMA kernels read only this copy;
+ *        without it MIE_PATH_AUTO takes the VALU kernels and MIE_PATH_MFMA is
+ *        refused.
  *   k in {1,3,5,7}, stride in {1,2}; out->h/w must equal (h_in+2*pad-k)/stride+1
  * Replaces: conv{1,3,5,7}x*_increment_ext(x_incr, mask, filter, out_incr, stride)
  * (ext/pointops/_C_ext/pointops/ops.cpp:51-114, include/ops.h:8-52) and the
@@ -154,7 +170,8 @@ int mie_build_mask_tiles(const uint8_t* in_mask, const uint8_t* in_mask2,
  */
 int mie_conv_masked(const float* x, const uint8_t* xmask, int c1,
                     const float* x2, const uint8_t* x2mask, int c2,
-                    int h_in, int w_in, const float* filter, int cin_total,
+                    int h_in, int w_in, const float* filter,
+                    const float* filter_mc, int cin_total,
                     int k, int stride, int pad, int cout,
                     const mie_tileset* out, float* out_delta,
                     const float* addend, float* reservoir, int act_kind,
@@ -173,7 +190,8 @@ int mie_conv_masked(const float* x, const uint8_t* xmask, int c1,
  * (incr_modules/mask_incr_modules.py:182-196,253-256).
  */
 int mie_conv_refresh(const float* x, int c1, const float* x2, int c2, int h_in,
-                     int w_in, const float* filter, int cin_total, int k,
+                     int w_in, const float* filter, const float* filter_mc,
+                     int cin_total, int k,
                      int stride, int pad, int cout, const float* bias,
                      const mie_tileset* out, float* out_dense,
                      const float* addend, float* reservoir, int act_kind,

@@ -13,7 +13,8 @@ import os
 import torch  # noqa: F401  (import order matters, see above)
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_PKG_DIR, "lib", "libmie_hip.so")
+# MIE_HIP_LIB points at another build of the same library (kernel experiments)
+LIB_PATH = os.environ.get("MIE_HIP_LIB") or os.path.join(_PKG_DIR, "lib", "libmie_hip.so")
 
 MIE_OK = 0
 MIE_TILE = 8
@@ -29,6 +30,7 @@ EXPORTS = (
     "mie_version", "mie_last_error_string", "mie_tile_capacity", "mie_mask_from_delta",
     "mie_build_mask_tiles", "mie_conv_masked", "mie_act_incr", "mie_mul_incr", "mie_add_incr",
     "mie_upsample2x_incr", "mie_convlstm_gates_incr", "mie_tconv_masked", "mie_conv_refresh",
+    "mie_pack_filter",
 )
 
 
@@ -66,10 +68,12 @@ def _declare(l):
     l.mie_build_mask_tiles.restype = ci
     l.mie_build_mask_tiles.argtypes = [vp, vp, ci, ci, ci, ci, ci, ci, tsp, vp]
     l.mie_conv_masked.restype = ci
-    l.mie_conv_masked.argtypes = [vp, vp, ci, vp, vp, ci, ci, ci, vp, ci, ci, ci, ci, ci, tsp, vp,
+    l.mie_conv_masked.argtypes = [vp, vp, ci, vp, vp, ci, ci, ci, vp, vp, ci, ci, ci, ci, ci, tsp, vp,
                                   vp, vp, ci, cf, ci, vp]
+    l.mie_pack_filter.restype = ci
+    l.mie_pack_filter.argtypes = [vp, ci, ci, ci, vp, vp]
     l.mie_conv_refresh.restype = ci
-    l.mie_conv_refresh.argtypes = [vp, ci, vp, ci, ci, ci, vp, ci, ci, ci, ci, ci, vp, tsp, vp, vp,
+    l.mie_conv_refresh.argtypes = [vp, ci, vp, ci, ci, ci, vp, vp, ci, ci, ci, ci, ci, vp, tsp, vp, vp,
                                    vp, ci, cf, ci, vp]
     l.mie_act_incr.restype = ci
     l.mie_act_incr.argtypes = [ci, cf, vp, vp, vp, ci, tsp, vp, ci, vp]

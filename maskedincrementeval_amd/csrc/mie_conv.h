@@ -8,6 +8,7 @@ struct ConvArgs {
   const float* x2; const uint8_t* x2m; int c2;
   int h_in, w_in;
   const float* filt; int cin_total;
+  const float* filt_mc;             // matrix-core copy of the filter (mie_pack_filter) or NULL
   int pad, cout;
   float* out; float* res; int act; float slope;
   const float* addend;              // optional delta added to the conv result before the epilogue

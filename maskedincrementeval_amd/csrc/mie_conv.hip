@@ -190,7 +190,8 @@ int check_epilogue(const char* who, float* out_delta, float* reservoir, int act_
 
 int conv_impl(const char* who, const float* x, const uint8_t* xmask, int c1, const float* x2,
               const uint8_t* x2mask, int c2, int h_in, int w_in, const float* filter,
-              int cin_total, int k, int stride, int pad, int cout, const mie_tileset* out,
+              const float* filter_mc, int cin_total, int k, int stride, int pad, int cout,
+              const mie_tileset* out,
               float* out_delta, const float* addend, float* reservoir, int act_kind, float slope,
               int path, bool refresh, const float* bias, void* stream) {
   mie_clear_error();
@@ -228,17 +229,19 @@ int conv_impl(const char* who, const float* x, const uint8_t* xmask, int c1, con
               "%s: addend must not alias out_delta", who);
   const int cmul = mie_conv_mfma_cout_multiple(k, stride);
   const int imul = mie_conv_mfma_cin_multiple(k, stride);
-  const bool mfma_ok = (c1 % imul == 0) && (c2 % imul == 0) && (cout % cmul == 0);
+  MIE_REQUIRE(mie_aligned(filter_mc, 16), MIE_ERR_INVALID_ARG, "%s: filter_mc must be 16-byte aligned", who);
+  const bool mfma_ok = (filter_mc != nullptr) && (cin_total % 8 == 0) && (c1 % imul == 0) &&
+                       (c2 % imul == 0) && (cout % cmul == 0);
   MIE_REQUIRE(path == MIE_PATH_AUTO || path == MIE_PATH_VALU || path == MIE_PATH_MFMA,
               MIE_ERR_INVALID_ARG, "%s: unknown path %d", who, path);
   MIE_REQUIRE(path != MIE_PATH_MFMA || mfma_ok, MIE_ERR_UNSUPPORTED,
-              "%s: MFMA path needs c1 %% %d == 0, c2 %% %d == 0, cout %% %d == 0 (c1=%d c2=%d cout=%d)",
-              who, imul, imul, cmul, c1, c2, cout);
+              "%s: MFMA path needs filter_mc (mie_pack_filter), c1 %% %d == 0, c2 %% %d == 0, cout %% %d == 0 "
+              "(filter_mc=%p c1=%d c2=%d cout=%d)", who, imul, imul, cmul, (const void*)filter_mc, c1, c2, cout);
   if (path == MIE_PATH_AUTO) path = mfma_ok ? MIE_PATH_MFMA : MIE_PATH_VALU;
 
   ConvArgs a;
   a.x = x; a.xm = xmask; a.c1 = c1; a.x2 = x2; a.x2m = x2mask; a.c2 = c2;
-  a.h_in = h_in; a.w_in = w_in; a.filt = filter; a.cin_total = cin_total;
+  a.h_in = h_in; a.w_in = w_in; a.filt = filter; a.cin_total = cin_total; a.filt_mc = filter_mc;
   a.pad = pad; a.cout = cout; a.out = out_delta; a.res = reservoir; a.act = act_kind;
   a.slope = slope; a.addend = addend; a.refresh = refresh ? 1 : 0; a.bias = bias;
   a.ts = mie_dev_tileset(out);
@@ -265,24 +268,56 @@ int conv_impl(const char* who, const float* x, const uint8_t* xmask, int c1, con
 
 }  // namespace
 
+// P[ci/8][tap][(ci%8)/4][co][ci%4] = F[ci][tap][co]
+__global__ __launch_bounds__(256) void k_pack_filter(const float* __restrict__ f,
+                                                     float* __restrict__ p, int cin, int kk, int cout) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  const long long total = (long long)cin * kk * cout;
+  if (i >= total) return;
+  const int co = (int)(i % cout);
+  const long long t = i / cout;
+  const int tap = (int)(t % kk);
+  const int ci = (int)(t / kk);
+  const long long o = ((((long long)(ci >> 3) * kk + tap) * 2 + ((ci & 7) >> 2)) * cout + co) * 4 + (ci & 3);
+  p[o] = f[i];
+}
+
+extern "C" int mie_pack_filter(const float* filter, int cin, int k, int cout, float* packed,
+                               void* stream) {
+  mie_clear_error();
+  const char* who = "mie_pack_filter";
+  MIE_REQUIRE(filter && packed, MIE_ERR_INVALID_ARG, "%s: NULL pointer", who);
+  MIE_REQUIRE(cin > 0 && k > 0 && cout > 0, MIE_ERR_INVALID_ARG, "%s: sizes must be positive", who);
+  MIE_REQUIRE(cin % 8 == 0, MIE_ERR_UNSUPPORTED, "%s: cin = %d is not a multiple of 8", who, cin);
+  MIE_REQUIRE(mie_aligned(filter, 16) && mie_aligned(packed, 16) && filter != packed,
+              MIE_ERR_INVALID_ARG, "%s: buffers must be 16-byte aligned and distinct", who);
+  const long long total = (long long)cin * k * k * cout;
+  MIE_REQUIRE(total < (1LL << 40), MIE_ERR_CAPACITY, "%s: filter too large", who);
+  hipLaunchKernelGGL(k_pack_filter, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+                     (hipStream_t)stream, filter, packed, cin, k * k, cout);
+  return mie_check_launch(who);
+}
+
 extern "C" int mie_conv_masked(const float* x, const uint8_t* xmask, int c1, const float* x2,
                                const uint8_t* x2mask, int c2, int h_in, int w_in,
-                               const float* filter, int cin_total, int k, int stride, int pad,
-                               int cout, const mie_tileset* out, float* out_delta,
-                               const float* addend, float* reservoir, int act_kind, float slope,
-                               int path, void* stream) {
-  return conv_impl("mie_conv_masked", x, xmask, c1, x2, x2mask, c2, h_in, w_in, filter, cin_total,
+                               const float* filter, const float* filter_mc, int cin_total, int k,
+                               int stride, int pad, int cout, const mie_tileset* out,
+                               float* out_delta, const float* addend, float* reservoir,
+                               int act_kind, float slope, int path, void* stream) {
+  return conv_impl("mie_conv_masked", x, xmask, c1, x2, x2mask, c2, h_in, w_in, filter, filter_mc,
+                   cin_total,
                    k, stride, pad, cout, out, out_delta, addend, reservoir, act_kind, slope, path,
                    false, nullptr, stream);
 }
 
 extern "C" int mie_conv_refresh(const float* x, int c1, const float* x2, int c2, int h_in,
-                                int w_in, const float* filter, int cin_total, int k, int stride,
-                                int pad, int cout, const float* bias, const mie_tileset* out,
+                                int w_in, const float* filter, const float* filter_mc,
+                                int cin_total, int k, int stride, int pad, int cout,
+                                const float* bias, const mie_tileset* out,
                                 float* out_dense, const float* addend, float* reservoir,
                                 int act_kind, float slope, int path, void* stream) {
   return conv_impl("mie_conv_refresh", x, nullptr, c1, x2, nullptr, c2, h_in, w_in, filter,
-                   cin_total, k, stride, pad, cout, out, out_dense, addend, reservoir, act_kind,
+                   filter_mc, cin_total, k, stride, pad, cout, out, out_dense, addend, reservoir, act_kind,
                    slope, path, true, bias, stream);
 }
 
@@ -311,7 +346,7 @@ extern "C" int mie_tconv_masked(const float* x, const uint8_t* xmask, int cin, i
   if (rc != MIE_OK) return rc;
   ConvArgs a;
   a.x = x; a.xm = xmask; a.c1 = cin; a.x2 = nullptr; a.x2m = nullptr; a.c2 = 0;
-  a.h_in = h_in; a.w_in = w_in; a.filt = filter; a.cin_total = cin;
+  a.h_in = h_in; a.w_in = w_in; a.filt = filter; a.cin_total = cin; a.filt_mc = nullptr;
   a.pad = pad; a.cout = cout; a.out = out_delta; a.res = reservoir; a.act = act_kind;
   a.slope = slope; a.addend = nullptr; a.refresh = 0; a.bias = nullptr; a.ts = mie_dev_tileset(out);
   const unsigned cap = (unsigned)mie_tile_capacity(out->n, out->h, out->w);

@@ -8,8 +8,8 @@
 //     rows; pixels whose mask byte is 0 (or that lie outside the image) are
 //     zero-filled without touching HBM.  Staging is double buffered: the
 //     global loads of chunk c+1 are in flight while chunk c is multiplied.
-//   * B (k x channels): filter rows filt[ci][ky][kx][co..co+31] are read
-//     straight from L2 into registers (each value is used by exactly one wave
+//   * B (k x channels): rows of the matrix-core filter copy (mie_pack_filter) are read
+//     straight from L2 into registers, 16 bytes per lane (each value is used by exactly one wave
 //     of the workgroup), three units ahead of the MFMAs that consume them.
 //   * The 4 waves split the workgroup's work WN ways over output channels and
 //     WK = 4/WN ways over k (units = tap x 8-channel sub-chunk, round robin).
@@ -129,11 +129,19 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgs a) {
     const int cs = second ? a.c2 : a.c1;
     const int ci0 = (second ? c - nch1 : c) * CC;
     const unsigned ok = second ? ok2 : ok1;
+    // The loads are unconditional in control flow (a branch around a load makes the compiler's
+    // wait counters conservative: the first MFMAs of a chunk would then wait for the whole
+    // global-memory latency of these loads).  Lanes whose pixel is masked or outside the image
+    // all read one fixed, cache-resident address instead and get zeros selected afterwards,
+    // so inactive pixels still cost no HBM traffic.
+    const float* dummy = a.filt;
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
-      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (((ok >> i) & 1u) && ci0 + st_c4[i] < cs)
-        v = *reinterpret_cast<const float4*>(xin + (long long)st_po[i] * cs + ci0 + st_c4[i]);
+      const bool okb = (ok >> i) & 1u;
+      const float* p = xin + (long long)st_po[i] * cs + ci0 + st_c4[i];
+      p = okb ? p : dummy;
+      float4 v = *reinterpret_cast<const float4*>(p);
+      v.x = okb ? v.x : 0.f; v.y = okb ? v.y : 0.f; v.z = okb ? v.z : 0.f; v.w = okb ? v.w : 0.f;
       st_reg[i] = v;
     }
   };
@@ -151,7 +159,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgs a) {
   // cout (B) or a compile-time LDS offset (A); the lane-dependent parts are loop invariant.
   const int q0w = wk * NQW;
   const int cob0 = co0 + wn * (32 * NB);                       // first column of this wave
-  const int b_lane = (4 * half) * (K * K) * cout + l32;        // lane part of the filter index
+  const int b_lane = (half * cout + l32) * 4;                  // lane part of the packed filter index
   int a_lane[2];                                               // lane part of the LDS index
 #pragma unroll
   for (int mb = 0; mb < 2; ++mb) {
@@ -163,16 +171,19 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgs a) {
     const bool second = c >= nch1;
     const int ci0 = (second ? c - nch1 : c) * CC;
     const int fb = second ? a.c1 : 0;
-    return a.filt + (long long)(fb + ci0 + 8 * q0w) * (K * K) * cout + cob0;
+    return a.filt_mc + ((long long)((fb + ci0) / 8 + q0w) * (K * K) * 2 * cout + cob0) * 4;
   };
+  // Matrix-core filter copy: P[ci/8][tap][(ci%8)/4][co][ci%4].  The four k-steps of a unit are
+  // one 16-byte load per lane, 512 contiguous bytes per half wave.
   float bring[RING][NB][4];
   auto load_b = [&](const float* ub, int unit, float (&bv)[NB][4]) {
     const int tap = unit / NQW, qi = unit % NQW;     // compile-time after unrolling
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-        bv[nb][j] = ub[(long long)(((8 * qi + j) * (K * K) + tap) * cout + nb * 32) + b_lane];
+    for (int nb = 0; nb < NB; ++nb) {
+      const float4 v = *reinterpret_cast<const float4*>(
+          ub + ((long long)((qi * (K * K) + tap) * 2) * cout + nb * 32) * 4 + b_lane);
+      bv[nb][0] = v.x; bv[nb][1] = v.y; bv[nb][2] = v.z; bv[nb][3] = v.w;
+    }
   };
 
   // All B loads below are unconditional: a conditional load would make the compiler's wait
@@ -188,10 +199,9 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgs a) {
 
   for (int c = 0; c < nch; ++c) {
     const bool more = c + 1 < nch;
-    if (more) {
-      ub_next = chunk_b(c + 1);
-      stage_load(c + 1);
-    }
+    const int cn = more ? c + 1 : c;      // after the last chunk: redundant re-load, never stored
+    ub_next = chunk_b(cn);
+    stage_load(cn);
     const float* sin = smem + (c & 1) * STAGE;
     // A operands are read one unit ahead as well (two register sets); the scheduling barriers
     // pin "issue the loads for later units, then multiply this unit" so that the compiler can

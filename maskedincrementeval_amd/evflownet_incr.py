@@ -309,9 +309,9 @@ class UpsampleConvLayerIncr(nn.Module):
             lead_c = ups[0][0].shape[1]
             # the flow estimate of the previous scale shares the mask of x (it is a 1x1 conv + tanh of
             # it), so the wide conv's output mask covers this partial result
-            addend = self._lead_conv(ups[0], filt[:lead_c])
+            addend = self._lead_conv(ups[0], filt.rows(0, lead_c))
         return self.conv2d.forward_fused(ups[-2], self.activation, ups[-1], addend_incr=addend,
-                                         filt=filt[lead_c:])
+                                         filt=filt.rows(lead_c, filt.shape[0]))
 
     def _lead_conv(self, x_incr, filt):
         k, s, p = self.conv2d._geometry()

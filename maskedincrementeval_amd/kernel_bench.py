@@ -68,7 +68,7 @@ def main():
     else:
         mask = None
     x = ops.as_nhwc(x.to(dev).contiguous(memory_format=torch.channels_last))
-    filt = he_normal_conv_weight(cout, cin, k, 0).permute(1, 2, 3, 0).contiguous().to(dev)
+    filt = ops.ConvFilter(he_normal_conv_weight(cout, cin, k, 0).permute(1, 2, 3, 0).contiguous().to(dev))
     ts = TileMask(n, ho, wo, dev)
     ops.build_mask_tiles(mask, None, n, h, w, _lib.FOOT_CONV, k, s, p, ts)
     out = ops.new_nhwc(n, cout, ho, wo, dev)

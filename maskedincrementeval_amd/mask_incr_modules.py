@@ -269,13 +269,14 @@ class _ConvIncrMixin(_IncrBuffers):
         return k, s, p
 
     @property
-    def conv2d_weights(self) -> torch.Tensor:
-        """Filter in the kernel layout [Cin, K, K, Cout], rebuilt when the weight changes."""
+    def conv2d_weights(self) -> "ops.ConvFilter":
+        """Filter in the kernel layouts ([Cin, K, K, Cout] and its matrix-core copy), rebuilt when
+        the weight changes."""
         w = self.weight
         tag = (w.data_ptr(), w._version, str(w.device))
         cached = self.__dict__.get("_filt_cache")
         if cached is None or cached[0] != tag:
-            cached = (tag, w.detach().permute(1, 2, 3, 0).contiguous().float())
+            cached = (tag, ops.ConvFilter(w.detach().permute(1, 2, 3, 0).contiguous().float()))
             self.__dict__["_filt_cache"] = cached
         return cached[1]
 

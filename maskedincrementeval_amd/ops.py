@@ -181,17 +181,65 @@ def build_mask_tiles(in_mask, in_mask2, n, h_in, w_in, foot, k, stride, pad, out
     return out
 
 
-def conv_masked(x, xmask, x2, x2mask, filt, k, stride, pad, out_ts: TileMask, out_delta,
-                reservoir=None, act=_lib.ACT_NONE, slope=0.0, path=_lib.PATH_AUTO, addend=None):
-    """filt: [Cin_total, K, K, Cout] contiguous fp32."""
-    n, c1, h, w = x.shape
-    c2 = 0 if x2 is None else x2.shape[1]
-    if x2 is not None and (x2.shape[0] != n or x2.shape[2:] != x.shape[2:]):
-        raise ValueError("x2 shape %s incompatible with x %s" % (tuple(x2.shape), tuple(x.shape)))
+def pack_filter(filt: torch.Tensor) -> torch.Tensor:
+    """Matrix-core copy of a contiguous fp32 [Cin,K,K,Cout] filter (Cin % 8 == 0), shape
+    [Cin/8, K*K, 2, Cout, 4]: element [b,t,h,co,j] is filt[8b+4h+j, t//K, t%K, co]."""
+    if filt.dim() != 4 or filt.shape[1] != filt.shape[2] or not filt.is_contiguous() or filt.dtype != torch.float32:
+        raise ValueError("filter must be contiguous fp32 [Cin,K,K,Cout], got %s" % (tuple(filt.shape),))
+    _require_gpu(filt, "filter")
+    cin, k, _, cout = filt.shape
+    packed = torch.empty((cin // 8, k * k, 2, cout, 4), dtype=torch.float32, device=filt.device)
+    check(lib().mie_pack_filter(filt.data_ptr(), cin, k, cout, packed.data_ptr(), _stream(filt)))
+    return packed
+
+
+class ConvFilter:
+    """A conv filter as the kernels take it: `plain` [Cin,K,K,Cout] and, when Cin % 8 == 0, `mc`,
+    its matrix-core copy (pack_filter).  Make a new one after every weight update."""
+
+    def __init__(self, plain: torch.Tensor, mc: Optional[torch.Tensor] = None, _packed: bool = False):
+        self.plain = plain
+        self.mc = mc if _packed else (pack_filter(plain) if plain.is_cuda and plain.shape[0] % 8 == 0 else None)
+        self._rows = {}
+
+    @property
+    def shape(self):
+        return self.plain.shape
+
+    def rows(self, lo: int, hi: int) -> "ConvFilter":
+        """The filter of input channels lo..hi-1, made once per range (views of this filter when
+        lo and hi are multiples of 8, else a packed copy of its own)."""
+        sub = self._rows.get((lo, hi))
+        if sub is None:
+            plain = self.plain[lo:hi]
+            if self.mc is not None and lo % 8 == 0 and hi % 8 == 0:
+                sub = ConvFilter(plain, self.mc[lo // 8:hi // 8], _packed=True)
+            else:
+                sub = ConvFilter(plain)
+            self._rows[(lo, hi)] = sub
+        return sub
+
+
+def _filter_args(filt, k):
+    """(plain tensor, pointer of the matrix-core copy or None) of a Tensor or ConvFilter."""
+    mc = None
+    if isinstance(filt, ConvFilter):
+        filt, mc = filt.plain, filt.mc
     if filt.dim() != 4 or filt.shape[1] != k or filt.shape[2] != k or not filt.is_contiguous() \
             or filt.dtype != torch.float32:
         raise ValueError("filter must be contiguous fp32 [Cin,%d,%d,Cout], got %s" % (k, k, tuple(filt.shape)))
     _require_gpu(filt, "filter")
+    return filt, (None if mc is None else mc.data_ptr())
+
+
+def conv_masked(x, xmask, x2, x2mask, filt, k, stride, pad, out_ts: TileMask, out_delta,
+                reservoir=None, act=_lib.ACT_NONE, slope=0.0, path=_lib.PATH_AUTO, addend=None):
+    """filt: ConvFilter, or a contiguous fp32 [Cin_total, K, K, Cout] tensor (VALU kernels only)."""
+    n, c1, h, w = x.shape
+    c2 = 0 if x2 is None else x2.shape[1]
+    if x2 is not None and (x2.shape[0] != n or x2.shape[2:] != x.shape[2:]):
+        raise ValueError("x2 shape %s incompatible with x %s" % (tuple(x2.shape), tuple(x.shape)))
+    filt, mc_ptr = _filter_args(filt, k)
     cin_total, cout = filt.shape[0], filt.shape[3]
     if tuple(out_delta.shape) != (n, cout, out_ts.h, out_ts.w) or out_ts.n != n:
         raise ValueError("out_delta shape %s, expected %s" % (tuple(out_delta.shape), (n, cout, out_ts.h, out_ts.w)))
@@ -203,7 +251,7 @@ def conv_masked(x, xmask, x2, x2mask, filt, k, stride, pad, out_ts: TileMask, ou
     check(lib().mie_conv_masked(
         nhwc_ptr(x, "x"), pix_ptr(xmask, n, h, w, "xmask"), c1,
         nhwc_ptr(x2, "x2"), pix_ptr(x2mask, n, h, w, "x2mask"), c2, h, w,
-        filt.data_ptr(), cin_total, k, stride, pad, cout, out_ts.ref,
+        filt.data_ptr(), mc_ptr, cin_total, k, stride, pad, cout, out_ts.ref,
         nhwc_ptr(out_delta, "out_delta"), nhwc_ptr(addend, "addend", cout), nhwc_ptr(reservoir, "reservoir"),
         act, float(slope), path, _stream(x)))
     return out_delta
@@ -214,7 +262,7 @@ def conv_refresh(x, x2, filt, bias, k, stride, pad, out_ts: TileMask, out_dense,
     """Dense conv + bias (+ activation, + reservoir fill) over the tiles of out_ts (all active)."""
     n, c1, h, w = x.shape
     c2 = 0 if x2 is None else x2.shape[1]
-    _require_gpu(filt, "filter")
+    filt, mc_ptr = _filter_args(filt, k)
     cin_total, cout = filt.shape[0], filt.shape[3]
     if tuple(out_dense.shape) != (n, cout, out_ts.h, out_ts.w):
         raise ValueError("out_dense shape %s, expected %s" % (tuple(out_dense.shape), (n, cout, out_ts.h, out_ts.w)))
@@ -222,8 +270,8 @@ def conv_refresh(x, x2, filt, bias, k, stride, pad, out_ts: TileMask, out_dense,
         raise ValueError("bias must be contiguous fp32 of %d elements" % cout)
     _ready(out_ts)
     check(lib().mie_conv_refresh(
-        nhwc_ptr(x, "x"), c1, nhwc_ptr(x2, "x2"), c2, h, w, filt.data_ptr(), cin_total, k, stride, pad,
-        cout, None if bias is None else bias.data_ptr(), out_ts.ref, nhwc_ptr(out_dense, "out_dense"),
+        nhwc_ptr(x, "x"), c1, nhwc_ptr(x2, "x2"), c2, h, w, filt.data_ptr(), mc_ptr, cin_total, k, stride,
+        pad, cout, None if bias is None else bias.data_ptr(), out_ts.ref, nhwc_ptr(out_dense, "out_dense"),
         nhwc_ptr(addend, "addend", cout), nhwc_ptr(reservoir, "reservoir"), act, float(slope), path,
         _stream(x)))
     return out_dense

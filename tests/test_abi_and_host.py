@@ -61,34 +61,42 @@ def test_invalid_arguments_return_status_not_abort(mie_lib):
     p = (ctypes.addressof(buf) + 15) & ~15
     err = lambda: mie_lib.mie_last_error_string().decode()
     # NULL tile set
-    assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 16, 16, p, 16, 3, 1, 1, 32, None, p,
+    assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 16, 16, p, None, 16, 3, 1, 1, 32, None, p,
                                    None, None, 0, 0.0, 0, None) == -1
     assert "tile set is NULL" in err()
     # NULL input pointer
-    assert mie_lib.mie_conv_masked(None, None, 16, None, None, 0, 16, 16, p, 16, 3, 1, 1, 32,
+    assert mie_lib.mie_conv_masked(None, None, 16, None, None, 0, 16, 16, p, None, 16, 3, 1, 1, 32,
                                    ctypes.byref(ts), p, None, None, 0, 0.0, 0, None) == -1
     # unsupported kernel size and stride (the reference throws std::logic_error, ext_conv.cu:366)
-    assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 16, 16, p, 16, 4, 1, 1, 32,
+    assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 16, 16, p, None, 16, 4, 1, 1, 32,
                                    ctypes.byref(ts), p, None, None, 0, 0.0, 0, None) == -2
     assert "kernel size 4" in err()
-    assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 16, 16, p, 16, 3, 3, 1, 32,
+    assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 16, 16, p, None, 16, 3, 3, 1, 32,
                                    ctypes.byref(ts), p, None, None, 0, 0.0, 0, None) == -2
     # output geometry mismatch
-    assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 20, 16, p, 16, 3, 1, 1, 32,
+    assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 20, 16, p, None, 16, 3, 1, 1, 32,
                                    ctypes.byref(ts), p, None, None, 0, 0.0, 0, None) == -1
     assert "tile set is" in err()
     # misaligned pointer
-    assert mie_lib.mie_conv_masked(p + 4, None, 16, None, None, 0, 16, 16, p, 16, 3, 1, 1, 32,
+    assert mie_lib.mie_conv_masked(p + 4, None, 16, None, None, 0, 16, 16, p, None, 16, 3, 1, 1, 32,
                                    ctypes.byref(ts), p, None, None, 0, 0.0, 0, None) == -1
     assert "aligned" in err()
     # MFMA path on a shape it cannot take
-    assert mie_lib.mie_conv_masked(p, None, 24, None, None, 0, 16, 16, p, 24, 3, 1, 1, 32,
+    assert mie_lib.mie_conv_masked(p, None, 24, None, None, 0, 16, 16, p, None, 24, 3, 1, 1, 32,
                                    ctypes.byref(ts), p, None, None, 0, 0.0, _lib.PATH_MFMA, None) == -2
+    # MFMA path without the matrix-core filter copy
+    assert mie_lib.mie_conv_masked(p, None, 32, None, None, 0, 16, 16, p, None, 32, 3, 1, 1, 32,
+                                   ctypes.byref(ts), p, None, None, 0, 0.0, _lib.PATH_MFMA, None) == -2
+    assert "mie_pack_filter" in err()
+    # filter packing: cin must be a multiple of 8, buffers distinct
+    assert mie_lib.mie_pack_filter(p, 12, 3, 32, p + 4096, None) == -2
+    assert mie_lib.mie_pack_filter(p, 16, 3, 32, p, None) == -1
+    assert mie_lib.mie_pack_filter(p, 16, 3, 32, None, None) == -1
     # activation without a reservoir
-    assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 16, 16, p, 16, 3, 1, 1, 32,
+    assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 16, 16, p, None, 16, 3, 1, 1, 32,
                                    ctypes.byref(ts), p, None, None, _lib.ACT_RELU, 0.0, 0, None) == -1
     # channels beyond the filter
-    assert mie_lib.mie_conv_masked(p, None, 16, p, None, 16, 16, 16, p, 16, 3, 1, 1, 32,
+    assert mie_lib.mie_conv_masked(p, None, 16, p, None, 16, 16, 16, p, None, 16, 3, 1, 1, 32,
                                    ctypes.byref(ts), p, None, None, 0, 0.0, 0, None) == -1
     # tile set with a NULL member / zero-sized geometry
     bad, keep2 = _fake_tileset(null="tiles")
@@ -154,10 +162,10 @@ def test_module_surface_matches_reference_names():
     c = mm.nnConvIncr(3, 5, 3, 1, 1, bias=False)
     assert set(c.state_dict().keys()) == {"weight"}               # nn.Conv2d keys, as in the reference
     assert tuple(c.conv2d_weights.shape) == (3, 3, 3, 5)          # [Cin, K, K, Cout]
-    assert torch.equal(c.conv2d_weights, c.weight.detach().permute(1, 2, 3, 0))
+    assert torch.equal(c.conv2d_weights.plain, c.weight.detach().permute(1, 2, 3, 0))
     with torch.no_grad():
         c.weight.mul_(2.0)
-    assert torch.equal(c.conv2d_weights, c.weight.detach().permute(1, 2, 3, 0))   # follows the weight
+    assert torch.equal(c.conv2d_weights.plain, c.weight.detach().permute(1, 2, 3, 0))   # follows the weight
     with pytest.raises(NotImplementedError):
         mm.nnConvIncr(3, 5, 4)._geometry()
     with pytest.raises(NotImplementedError):

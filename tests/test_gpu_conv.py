@@ -20,7 +20,7 @@ def _dev(t):
 
 
 def _filt(w_oihw):
-    return w_oihw.permute(1, 2, 3, 0).contiguous().to(DEV)
+    return ops.ConvFilter(w_oihw.permute(1, 2, 3, 0).contiguous().to(DEV))
 
 
 def _close(got, ref, what=""):
@@ -228,3 +228,19 @@ def test_refresh_conv_matches_dense_conv_with_bias():
         pre = io.conv_refresh(torch.cat((x, x2), 1), wt, bias, 1, 1)
         _close(res, pre, "reservoir = pre-activation")
         _close(out, torch.tanh(pre), "activated output")
+
+
+def test_pack_filter_layout_and_row_views():
+    cin, k, cout = 24, 3, 40
+    f = torch.arange(cin * k * k * cout, dtype=torch.float32).reshape(cin, k, k, cout).to(DEV)
+    p = ops.pack_filter(f)
+    torch.cuda.synchronize()
+    want = f.reshape(cin // 8, 2, 4, k * k, cout).permute(0, 3, 1, 4, 2).contiguous()    # [b,t,h,co,j]
+    assert torch.equal(p, want)
+    cf = ops.ConvFilter(f)
+    sub = cf.rows(8, 24)
+    assert sub.mc.data_ptr() == cf.mc[1:].data_ptr() and torch.equal(sub.mc, ops.pack_filter(f[8:24].contiguous()))
+    assert cf.rows(8, 24) is sub
+    odd = cf.rows(4, 20)                 # not on an 8-row boundary: a packed copy of its own
+    assert torch.equal(odd.mc, ops.pack_filter(f[4:20].contiguous()))
+    assert ops.ConvFilter(f[:12].contiguous()).mc is None
