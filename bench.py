@@ -41,6 +41,8 @@ def parse_args():
     ap.add_argument("--no-dense", action="store_true", help="skip the all-tiles-active comparator")
     ap.add_argument("--layer-iters", type=int, default=20, help="timed launches per layer for the roofline table")
     ap.add_argument("--sync-masks", action="store_true", help="build tile sets on the compute stream (no planning stream)")
+    ap.add_argument("--kfence-tp", type=float, default=0.0,
+                    help="also time the net with every conv's delta quantiser on (k = tp*||x||); reported under \"kfenced\"")
     ap.add_argument("--sweep", action="store_true", help="also time 1 %% and 20 %% density (reported under \"density_sweep\")")
     return ap.parse_args()
 
@@ -284,6 +286,29 @@ def main():
         dense_sec = timed_run(dense_model, "dense (all tiles active, same kernels)")
         del dense_model
 
+    # ---- lossy variant: delta quantiser in front of every conv ------------------------------------
+    kfenced = None
+    if args.kfence_tp > 0:
+        from maskedincrementeval_amd.mask_incr_modules import set_kfence
+        kf_model = seed_module_(E2VIDRecurrentIncr(async_masks=not args.sync_masks), seed=1).to(dev).eval()
+        set_kfence(kf_model, args.kfence_tp)
+        t = timed_run(kf_model, "quantised deltas (tp = %g)" % args.kfence_tp)
+        # deviation of the accumulated prediction from the exact incremental net, same inputs
+        with torch.no_grad():
+            acc = []
+            for m in (model, kf_model):
+                pred = m.forward_refresh_reservoirs(cl(x0), None)[0].clone()
+                for i in range(n_inputs):
+                    pred += step_eager(m, i)[0][0]
+                acc.append(pred)
+            torch.cuda.synchronize()
+            dev_abs = (acc[0] - acc[1]).abs().max().item()
+        kfenced = dict(tp=args.kfence_tp, ms_per_step=round(1e3 * t, 4), frames_per_s=round(1 / t, 1),
+                       max_abs_deviation_after_16_steps=dev_abs)
+        print("[bench] quantised deltas: max |deviation| of the prediction after %d steps = %.3e" %
+              (n_inputs, dev_abs), file=sys.stderr, flush=True)
+        del kf_model
+
     # ---- other densities (same network, same kernels) ------------------------------------------------
     sweep = None
     if args.sweep:
@@ -341,6 +366,7 @@ def main():
         "dense_same_kernels_ms": None if dense_sec is None else round(1e3 * dense_sec, 4),
         "speedup_vs_dense": None if dense_sec is None else round(dense_sec / sec_per_step, 3),
         "density_sweep": sweep,
+        "kfenced": kfenced,
         "layers": layers,
     }
     print(json.dumps(result))

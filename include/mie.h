@@ -219,6 +219,27 @@ int mie_act_incr(int act_kind, float slope, const float* in_delta,
                  void* stream);
 
 /*
+ * Delta quantiser ("k-fence"): lets multiples of k through and carries the rest
+ * to later steps.  At the active pixels of ts->pixmask, per element
+ *   t = carry + in_delta;  out_delta = k * floor(0.5 + t / k);  carry = t - out_delta
+ * (each operation rounded on its own, true division: bit-identical to the same
+ * expression in fp32 on the host); inactive pixels of active tiles and stale
+ * tiles get out_delta = 0 and keep their carry.  k = *k_dev when k_dev != NULL
+ * (a device scalar, so that a refresh can change k without a host read or a new
+ * graph capture), else k_host; a k that is not positive and finite lets the
+ * delta through unchanged.  A carry that started at zero stays within
+ * [-k/2, k/2], where the dense expression emits 0 as well.  out_pixmask as in
+ * mie_act_incr (refined mask any_c(out_delta != 0)): it is what makes the
+ * following layers sparse again.  out_delta may alias in_delta.
+ * Replaces: KFencedMaskModule.forward / floor_by_k
+ * (incr_modules/mask_incr_modules.py:32-42); k is what
+ * KFencedMaskModule.forward_refresh_reservoirs (:44-48) sets.
+ */
+int mie_kfence_incr(const float* in_delta, float* carry, const float* k_dev,
+                    float k_host, float* out_delta, int c, const mie_tileset* ts,
+                    uint8_t* out_pixmask, void* stream);
+
+/*
  * Incremental point-wise product (product rule with cached operands):
  *   out = (d2 + r2) * d1 + r1 * d2;  r1 += d1;  r2 += d2
  * d1/d2 are read only where their pixel masks m1/m2 (NULL = all active) are

@@ -30,7 +30,7 @@ EXPORTS = (
     "mie_version", "mie_last_error_string", "mie_tile_capacity", "mie_mask_from_delta",
     "mie_build_mask_tiles", "mie_conv_masked", "mie_act_incr", "mie_mul_incr", "mie_add_incr",
     "mie_upsample2x_incr", "mie_convlstm_gates_incr", "mie_tconv_masked", "mie_conv_refresh",
-    "mie_pack_filter",
+    "mie_pack_filter", "mie_kfence_incr",
 )
 
 
@@ -70,6 +70,8 @@ def _declare(l):
     l.mie_conv_masked.restype = ci
     l.mie_conv_masked.argtypes = [vp, vp, ci, vp, vp, ci, ci, ci, vp, vp, ci, ci, ci, ci, ci, tsp, vp,
                                   vp, vp, ci, cf, ci, vp]
+    l.mie_kfence_incr.restype = ci
+    l.mie_kfence_incr.argtypes = [vp, vp, vp, cf, vp, ci, tsp, vp, vp]
     l.mie_pack_filter.restype = ci
     l.mie_pack_filter.argtypes = [vp, ci, ci, ci, vp, vp]
     l.mie_conv_refresh.restype = ci

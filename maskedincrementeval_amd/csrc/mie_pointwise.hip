@@ -105,6 +105,60 @@ __global__ __launch_bounds__(256) void k_act_incr(TileSetDev ts, int kind, float
   }
 }
 
+// ---- delta quantiser (k-fence) ---------------------------------------------------
+// t = carry + d;  f = k * floor(0.5 + t / k);  carry = t - f;  out = f.  Every operation is a
+// separately rounded IEEE fp32 op (no contraction, true division), so the result equals the
+// same expression evaluated op by op on the host.
+template <int VEC>
+__global__ __launch_bounds__(256) void k_kfence_incr(TileSetDev ts, const float* __restrict__ k_dev,
+                                                     float k_host, const float* __restrict__ din,
+                                                     float* __restrict__ carry,
+                                                     float* __restrict__ dout, int c,
+                                                     uint8_t* __restrict__ out_mask) {
+  __shared__ unsigned s_any[64];
+  int n, y0, x0;
+  const int tk = mie_pick_tile(ts, blockIdx.x, n, y0, x0);
+  if (tk == 0) return;
+  if (out_mask) {
+    if (threadIdx.x < 64) s_any[threadIdx.x] = 0u;
+    __syncthreads();
+  }
+  const float k = k_dev ? *k_dev : k_host;
+  const bool fence = k > 0.f && k < INFINITY;     // otherwise the delta passes unchanged
+  const int cv = c / VEC;
+  for_tile_slots(ts, n, y0, x0, cv, [&](int px, long long pixoff, int cq) {
+    const long long off = pixoff * c + (long long)cq * VEC;
+    Vec<VEC> o = Vec<VEC>::zero();
+    if (tk == 1 && ts.pixmask[pixoff]) {
+      Vec<VEC> d = Vec<VEC>::load(din + off);
+      Vec<VEC> r = Vec<VEC>::load(carry + off);
+      unsigned nz = 0u;
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        const float t = __fadd_rn(r[i], d[i]);
+        const float f = fence ? __fmul_rn(k, floorf(__fadd_rn(0.5f, __fdiv_rn(t, k)))) : t;
+        o[i] = f;
+        r[i] = __fsub_rn(t, f);
+        nz |= (f != 0.f) ? 1u : 0u;
+      }
+      r.store(carry + off);
+      if (out_mask && nz) atomicOr(&s_any[px], 1u);
+    }
+    o.store(dout + off);
+  });
+  if (out_mask) {
+    __syncthreads();
+    if (threadIdx.x < 64) {
+      const int px = threadIdx.x;
+      const int y = y0 + (px >> 3), x = x0 + (px & 7);
+      if (y < ts.h && x < ts.w) {
+        const long long pixoff = ((long long)n * ts.h + y) * ts.w + x;
+        out_mask[pixoff] = (uint8_t)((tk == 1 && s_any[px]) ? 1 : 0);
+      }
+    }
+  }
+}
+
 // ---- product rule ---------------------------------------------------------------
 template <int VEC>
 __global__ __launch_bounds__(256) void k_mul_incr(TileSetDev ts, const float* __restrict__ d1,
@@ -320,6 +374,33 @@ extern "C" int mie_act_incr(int act_kind, float slope, const float* in_delta, fl
   else
     hipLaunchKernelGGL(k_act_incr<1>, dim3(grid, ny), dim3(256), 0, (hipStream_t)stream, d, act_kind,
                        slope, in_delta, reservoir, out_delta, c, out_pixmask, keep);
+  return mie_check_launch(who);
+}
+
+extern "C" int mie_kfence_incr(const float* in_delta, float* carry, const float* k_dev, float k_host,
+                               float* out_delta, int c, const mie_tileset* ts,
+                               uint8_t* out_pixmask, void* stream) {
+  mie_clear_error();
+  const char* who = "mie_kfence_incr";
+  int rc = check_pointwise(who, ts, c);
+  if (rc != MIE_OK) return rc;
+  MIE_REQUIRE(in_delta && carry && out_delta, MIE_ERR_INVALID_ARG, "%s: NULL pointer", who);
+  MIE_REQUIRE(carry != in_delta && carry != out_delta, MIE_ERR_INVALID_ARG,
+              "%s: the carry must not alias a delta", who);
+  MIE_REQUIRE(k_dev != nullptr || (k_host > 0.f && k_host < INFINITY), MIE_ERR_INVALID_ARG,
+              "%s: k = %g must be positive and finite", who, (double)k_host);
+  MIE_PTR16(in_delta, who, "in_delta"); MIE_PTR16(carry, who, "carry");
+  MIE_PTR16(out_delta, who, "out_delta");
+  MIE_REQUIRE(mie_aligned(k_dev, 4), MIE_ERR_INVALID_ARG, "%s: k_dev must be 4-byte aligned", who);
+  const TileSetDev d = mie_dev_tileset(ts);
+  const unsigned grid = (unsigned)mie_tile_capacity(ts->n, ts->h, ts->w);
+  const unsigned ny = out_pixmask ? 1u : channel_splits((int)grid, (c & 3) ? c : c / 4);
+  if ((c & 3) == 0)
+    hipLaunchKernelGGL(k_kfence_incr<4>, dim3(grid, ny), dim3(256), 0, (hipStream_t)stream, d, k_dev,
+                       k_host, in_delta, carry, out_delta, c, out_pixmask);
+  else
+    hipLaunchKernelGGL(k_kfence_incr<1>, dim3(grid, ny), dim3(256), 0, (hipStream_t)stream, d, k_dev,
+                       k_host, in_delta, carry, out_delta, c, out_pixmask);
   return mie_check_launch(who);
 }
 

@@ -13,7 +13,7 @@ kernels with every tile active (bias and the reservoir fill fused in); the
 cheap point-wise parts of the refresh are torch ops on the device.
 """
 import functools
-from typing import Tuple
+from typing import Optional, Tuple
 
 import torch
 import torch.nn as nn
@@ -109,9 +109,13 @@ class IncrementMaskModule(nn.Module, _IncrBuffers):
 class KFencedMaskModule(IncrementMaskModule):
     """Delta quantiser: lets multiples of k through, carries the rest (reference :21-47).
 
-    T = Rd + d;  f = k * floor(0.5 + T / k);  Rd = T - f;  returns [f, None].
-    The reference instantiates it in every nnConvIncr but never calls its
-    forward; it is kept as torch ops on the device.
+    T = Rd + d;  f = k * floor(0.5 + T / k);  Rd = T - f;  returns [f, mask of f != 0].
+    One kernel over the active tiles of the input (where d = 0 the carry Rd stays
+    within [-k/2, k/2] and the dense expression emits 0 as well); the refined pixel
+    mask it emits is what makes the layers behind it sparse again.  k is `tp` until
+    a refresh sets it to tp * ||x||_2 (:45), kept in a 1-element device tensor whose
+    address survives later refreshes.  The reference instantiates the module in
+    every nnConvIncr but never calls its forward (:166).
     """
 
     def __init__(self, tp: float = .1):
@@ -124,14 +128,32 @@ class KFencedMaskModule(IncrementMaskModule):
         return self.k * torch.floor(0.5 + T / self.k)
 
     def forward(self, incr: Masked) -> Masked:
-        T1 = self.delta.reservoir + incr[0]
-        f_delta = self.floor_by_k(T1)
-        self.delta.update_reservoir(T1 - f_delta)
-        return f_delta, None
+        d, _, _ = _unpack(incr)
+        n, c, h, w = d.shape
+        if self.delta.reservoir is None or self.delta.reservoir.shape != d.shape:
+            self.delta.update_reservoir(ops.new_nhwc(n, c, h, w, d.device))
+        mask = incr[1] if len(incr) > 1 else None
+        if isinstance(mask, TileMask):
+            ts = mask
+        else:
+            ts = self._tile_set("own", n, h, w, d.device)
+            ops.build_mask_tiles(ops.pixel_mask_of(mask, d), None, n, h, w, _lib.FOOT_CONV, 1, 1, 0, ts)
+        out = self._delta_buf("out", (n, c, h, w), d.device)
+        pix = self._pix_buf("refined", n, h, w, d.device)
+        ops.kfence_incr(d, self.delta.reservoir, self.k, out, ts, pix)
+        return [out, self._view("refined", ts, pix)]
 
     def forward_refresh_reservoirs(self, x: DenseT) -> DenseT:
-        self.k = self.tp * torch.norm(x)
-        self.delta.update_reservoir(torch.zeros_like(x))
+        k = (self.tp * torch.norm(x.detach())).reshape(1).float()
+        if isinstance(self.k, torch.Tensor) and self.k.device == k.device:
+            self.k.copy_(k)
+        else:
+            self.k = k
+        if self.delta.reservoir is not None and self.delta.reservoir.shape == x.shape:
+            self.delta.reservoir.zero_()
+        else:
+            self.delta.update_reservoir(torch.zeros_like(x))
+        self._reset_incr()
         return x
 
 
@@ -374,6 +396,7 @@ class nnConvIncr(nn.Conv2d, _ConvIncrMixin):
                  bias=True):
         nn.Conv2d.__init__(self, in_channels, out_channels, kernel_size, stride, padding, bias=bias)
         self.kf = KFencedMaskModule(0.3)
+        self.use_kf = False          # the reference leaves the quantiser switched off (:166)
         self.path = _lib.PATH_AUTO
 
     def load_state_dict(self, state_dict, strict: bool = True):
@@ -382,11 +405,15 @@ class nnConvIncr(nn.Conv2d, _ConvIncrMixin):
         return ret
 
     def forward(self, x_incr, x2_incr=None):
+        if self.use_kf:
+            x_incr = self.kf(x_incr)
         return self._incr_forward(x_incr, x2_incr, path=self.path)
 
     def forward_fused(self, x_incr, activation: "nnReservedActivation", x2_incr=None,
                       addend_incr=None, filt=None):
         """conv (+ addend) + activation increment in one kernel; updates activation.in_res in place."""
+        if self.use_kf:
+            x_incr = self.kf(x_incr)
         kind, slope = activation_kind(activation.op)
         res = activation.in_res.reservoir
         if res is None:
@@ -395,13 +422,30 @@ class nnConvIncr(nn.Conv2d, _ConvIncrMixin):
                                   path=self.path, out_name="out_act", addend_incr=addend_incr, filt=filt)
 
     def forward_refresh_reservoirs(self, x):
-        # The reference also refreshes self.kf here (:193), a norm and a zero clone
-        # that nothing reads because kf.forward is never called (:166).
+        # The reference refreshes self.kf here unconditionally (:193): a norm and a zero clone
+        # that nothing reads while kf.forward is not called (:166); done only when it is in use.
+        if self.use_kf:
+            self.kf.forward_refresh_reservoirs(x)
         return self._refresh_forward(x, path=self.path)
 
     def forward_refresh_fused(self, x, activation: "nnReservedActivation", x2=None, addend=None):
         """Dense conv + bias (+ addend) + activation, pre-activation written into activation.in_res."""
+        if self.use_kf:
+            self.kf.forward_refresh_reservoirs(x)
         return self._refresh_forward(x, x2, activation, path=self.path, addend=addend)
+
+
+def set_kfence(net: nn.Module, tp: Optional[float]) -> int:
+    """Switch the delta quantiser of every nnConvIncr in `net` on (threshold factor tp, k = tp*||x||
+    at the next refresh) or off (tp None).  Returns the number of convs touched; refresh afterwards."""
+    count = 0
+    for m in net.modules():
+        if isinstance(m, nnConvIncr):
+            m.use_kf = tp is not None
+            if tp is not None:
+                m.kf.tp = float(tp)
+            count += 1
+    return count
 
 
 class nnConvTranspose2dIncr(nn.ConvTranspose2d, _IncrBuffers):

@@ -317,6 +317,28 @@ def act_incr(kind, slope, in_delta, reservoir, out_delta, ts: TileMask, out_pixm
     return out_delta
 
 
+def kfence_incr(in_delta, carry, k, out_delta, ts: TileMask, out_pixmask=None):
+    """k: positive float, or a 1-element fp32 device tensor read by the kernel."""
+    n, c, h, w = in_delta.shape
+    _same_shape("carry", carry, in_delta)
+    _same_shape("out_delta", out_delta, in_delta)
+    if (ts.n, ts.h, ts.w) != (n, h, w):
+        raise ValueError("tile set %s does not match delta %s" % ((ts.n, ts.h, ts.w), (n, h, w)))
+    if isinstance(k, torch.Tensor):
+        if k.numel() != 1 or k.dtype != torch.float32:
+            raise ValueError("k must be a float or a 1-element fp32 tensor")
+        _require_gpu(k, "k")
+        k_dev, k_host = k.data_ptr(), 0.0
+    else:
+        k_dev, k_host = None, float(k)
+    _ready(ts)
+    check(lib().mie_kfence_incr(nhwc_ptr(in_delta, "in_delta"), nhwc_ptr(carry, "carry"), k_dev, k_host,
+                                nhwc_ptr(out_delta, "out_delta"), c, ts.ref,
+                                pix_ptr(out_pixmask, n, h, w, "out_pixmask"), _stream(in_delta)))
+    _mark_pix(out_pixmask)
+    return out_delta
+
+
 def mul_incr(d1, m1, r1, d2, m2, r2, out_delta, ts: TileMask, keep_reservoir=False):
     n, c, h, w = d1.shape
     for name, t in (("r1", r1), ("d2", d2), ("r2", r2), ("out_delta", out_delta)):

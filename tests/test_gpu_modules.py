@@ -61,6 +61,40 @@ def test_convkxkincr_functional_like_reference():
     _close(out[0], io.conv_incr(x.cpu(), c.weight.detach().cpu(), 1, 1), "vs oracle", rtol=1e-5, atol=1e-6)
 
 
+def test_kfenced_conv_restores_sparsity_and_matches_oracle():
+    # nnConvIncr with its quantiser switched on (the reference's commented-out `x_incr = self.kf(x_incr)`,
+    # incr_modules/mask_incr_modules.py:166): k = tp*||x0|| from the refresh (:45), conv of the
+    # quantised delta, carry kept across steps
+    n, cin, cout, h, w = 1, 16, 32, 40, 56
+    conv = mm.nnConvIncr(cin, cout, 3, 1, 1).to(DEV).eval()
+    conv.use_kf, conv.kf.tp = True, 2e-3
+    x0 = torch.randn(n, cin, h, w, generator=torch.Generator().manual_seed(11))
+    with torch.no_grad():
+        conv.forward_refresh_reservoirs(_cl(x0))
+    k_ref = (conv.kf.tp * torch.norm(x0)).float()
+    assert torch.allclose(conv.kf.k.cpu(), k_ref.reshape(1), rtol=1e-6)
+    k_cpu = conv.kf.k.cpu()[0]                       # the value the kernel reads
+    k_ptr = conv.kf.k.data_ptr()
+    carry = io.Reserve(torch.zeros(n, cin, h, w))
+    wt = conv.weight.detach().cpu()
+    for step in range(5):
+        d, m = gaussian_delta(n, cin, h, w, 0.2, 0.08, seed=40 + step)
+        with torch.no_grad():
+            out = conv([_cl(d), m.to(DEV)])
+        torch.cuda.synchronize()
+        f = io.kfenced(carry, k_cpu, d)
+        assert torch.equal(conv.kf.delta.reservoir.cpu(), carry.reservoir)
+        fmask = (f != 0).any(dim=1).to(torch.uint8).numpy()
+        assert 0 < fmask.sum() < m.sum().item()         # the fence removed pixels, not all of them
+        assert np.array_equal(out[1].pixmask[:, 0].cpu().numpy(), mo.footprint_conv(fmask, 3, 1, 1))
+        assert np.array_equal(out[1].active_tiles().cpu().numpy(), mo.tile_list(mo.footprint_conv(fmask, 3, 1, 1)))
+        _close(out[0], io.conv_incr(f, wt, 1, 1), "conv of the quantised delta, step %d" % step)
+    with torch.no_grad():
+        conv.forward_refresh_reservoirs(_cl(2 * x0))        # k follows the refresh in place
+    assert conv.kf.k.data_ptr() == k_ptr and torch.allclose(conv.kf.k.cpu(), 2 * k_ref.reshape(1), rtol=1e-6)
+    assert torch.count_nonzero(conv.kf.delta.reservoir) == 0
+
+
 def test_functional_ops_match_oracle():
     n, c, h, w = 1, 16, 30, 38
     d, m = gaussian_delta(n, c, h, w, 0.1, 0.5, seed=3)

@@ -181,3 +181,52 @@ def test_fused_convlstm_gates_match_module_chain(hid, h, w, with_prev):
     _close(acc_h, acc_h_ref, "accumulated hidden")
     _close(cell_res, cell.r["tanh2"].reservoir, "cell reservoir")
     _close(gates_res[:, :hid], cell.r["sig1"].reservoir, "in-gate reservoir")
+
+
+@pytest.mark.parametrize("n,c,h,w,k_on_device", [(1, 32, 45, 61, True), (2, 5, 19, 23, False), (1, 1, 16, 24, True)])
+def test_kfence_quantiser_is_bit_exact(n, c, h, w, k_on_device):
+    # KFencedMaskModule.forward (incr_modules/mask_incr_modules.py:36-42): f = k*floor(0.5 + T/k),
+    # carry = T - f.  Every op is IEEE fp32, so delta, carry and emitted mask must equal the oracle's
+    kval = 0.173
+    k = torch.tensor([kval], dtype=torch.float32, device=DEV) if k_on_device else kval
+    carry_cpu = io.Reserve(torch.zeros(n, c, h, w))
+    carry_gpu = ops.new_nhwc(n, c, h, w, DEV)
+    ts = TileMask(n, h, w, DEV)
+    out = ops.new_nhwc(n, c, h, w, DEV)
+    refined = torch.zeros((n, 1, h, w), dtype=torch.uint8, device=DEV)
+    total = torch.zeros(n, c, h, w)
+    for step in range(6):
+        d, m = gaussian_delta(n, c, h, w, 0.15, 0.1, seed=300 + step + c)
+        _identity_ts(ts, m, n, h, w)
+        ops.kfence_incr(_dev(d), carry_gpu, k, out, ts, refined)
+        torch.cuda.synchronize()
+        ref = io.kfenced(carry_cpu, torch.tensor(kval), d)
+        total += d
+        assert torch.equal(out.cpu(), ref), "quantised delta differs at step %d" % step
+        assert torch.equal(carry_gpu.cpu(), carry_cpu.reservoir), "carry differs at step %d" % step
+        assert np.array_equal(refined.cpu().numpy(), (ref != 0).any(dim=1, keepdim=True).to(torch.uint8).numpy())
+        # what went through is a multiple of k, and nothing is lost: sum(f) + carry = sum(d)
+        q = out.cpu() / kval
+        assert torch.allclose(q, q.round(), atol=1e-4)
+    assert carry_gpu.abs().max().item() <= 0.5 * kval * (1 + 1e-6)
+
+
+def test_kfence_in_place_and_switched_off():
+    n, c, h, w = 1, 8, 16, 24
+    d, m = gaussian_delta(n, c, h, w, 0.3, 1.0, seed=5)
+    ts = _identity_ts(TileMask(n, h, w, DEV), m, n, h, w)
+    carry = ops.new_nhwc(n, c, h, w, DEV)
+    x = _dev(d.clone())
+    ops.kfence_incr(x, carry, 0.5, x, ts)                       # out aliases in
+    ref = io.kfenced(io.Reserve(torch.zeros(n, c, h, w)), torch.tensor(0.5), d)
+    assert torch.equal(x.cpu(), ref)
+    # a k that is not positive (device scalar): the delta passes, the carry empties
+    kz = torch.zeros(1, device=DEV)
+    out = ops.new_nhwc(n, c, h, w, DEV)
+    carry2 = ops.new_nhwc(n, c, h, w, DEV)
+    ops.kfence_incr(_dev(d), carry2, kz, out, ts)
+    assert torch.equal(out.cpu(), d) and torch.count_nonzero(carry2) == 0
+    with pytest.raises(RuntimeError, match="positive and finite"):
+        ops.kfence_incr(_dev(d), carry2, 0.0, out, ts)
+    with pytest.raises(RuntimeError, match="alias"):
+        ops.kfence_incr(x, x, 0.5, out, ts)
