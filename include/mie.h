@@ -68,6 +68,10 @@ extern "C" {
 /* flags of mie_act_incr / mie_mul_incr */
 #define MIE_FLAG_KEEP_RESERVOIR 1  /* compute the delta, leave reservoirs as is */
 
+/* frame kinds of mie_events_to_frame */
+#define MIE_EVENTS_VOXEL 0      /* num_bins channels, linear weights in time   */
+#define MIE_EVENTS_HISTOGRAM 1  /* 2 channels: counts of p == -1, of p == +1   */
+
 /* counts[] slots of a tile set */
 #define MIE_CNT_ACTIVE 0
 #define MIE_CNT_STALE 1
@@ -309,6 +313,41 @@ int mie_tconv_masked(const float* x, const uint8_t* xmask, int cin, int h_in,
                      int w_in, const float* filter, int k, int stride, int pad,
                      int cout, const mie_tileset* out, float* out_delta,
                      float* reservoir, int act_kind, float slope, void* stream);
+
+/*
+ * Event front end: scatter raw events into a frame, or directly into the DELTA
+ * between the frames of two time windows, in the layout the network consumes.
+ *   events : [n_events][4] doubles (t, x, y, p), the reference's .npy row
+ *            layout; t * t_scale is in the unit of start_* / delta_t
+ *            (t_scale = 1e-9 for nanosecond stamps, util.py:90).  Events off the
+ *            sensor are skipped.
+ *   window : an event belongs to a window iff start < t*t_scale < start + delta_t.
+ *   MIE_EVENTS_VOXEL: ts = (num_bins-1)*(t*t_scale-start)/delta_t; p*(1-frac(ts))
+ *            goes to bin floor(ts), p*frac(ts) to the next bin, p == 0 counts as
+ *            -1 (events_to_voxel_grid_absT, data_fetchers/utils/util.py:78-107;
+ *            with start = first stamp, delta_t = last - first, t_scale = 1 it is
+ *            events_to_voxel_grid, :110-152).
+ *   MIE_EVENTS_HISTOGRAM: channel 0 counts p == -1, channel 1 counts p == +1
+ *            (event_histogram, util.py:62-75).
+ *   delta  : 0 -> out = frame of the window at start_new (start_old unused);
+ *            1 -> out = frame(start_new) - frame(start_old), each event of
+ *            either window visited once (replaces forming both frames and
+ *            `event_tensor - event_tensor_prev`,
+ *            run_e2depth_continuous_dataset.py:66).
+ *   pad_*  : ReflectionPad2d((left, right, top, bottom)) applied to the result
+ *            (run_e2depth_continuous_dataset.py:49), folded into the scatter.
+ *   out    : fp32 [height+pad_top+pad_bottom][width+pad_left+pad_right][channels]
+ *            (one NHWC sample; offset the pointers per sample of a batch),
+ *            fully rewritten (zero where no event lands).
+ *   pixmask: same pixels, 1 where at least one contributing event landed.
+ * Sums use floating-point atomics: a pixel hit by several events can differ in
+ * the last bits between runs (the histogram kind is exact).
+ */
+int mie_events_to_frame(const double* events, int n_events, int kind, int num_bins,
+                        int height, int width, int pad_left, int pad_right,
+                        int pad_top, int pad_bottom, double t_scale,
+                        double start_old, double start_new, double delta_t,
+                        int delta, float* out, uint8_t* pixmask, void* stream);
 
 #ifdef __cplusplus
 }

@@ -21,6 +21,7 @@ MIE_TILE = 8
 
 ACT_NONE, ACT_RELU, ACT_LEAKY_RELU, ACT_SIGMOID, ACT_TANH = 0, 1, 2, 3, 4
 FOOT_CONV, FOOT_UP2X, FOOT_TCONV = 0, 1, 2
+EVENTS_VOXEL, EVENTS_HISTOGRAM = 0, 1
 PATH_AUTO, PATH_VALU, PATH_MFMA = 0, 1, 2
 FLAG_KEEP_RESERVOIR = 1
 CNT_ACTIVE, CNT_STALE, CNT_TICKET, CNT_WORDS = 0, 1, 2, 4
@@ -30,7 +31,7 @@ EXPORTS = (
     "mie_version", "mie_last_error_string", "mie_tile_capacity", "mie_mask_from_delta",
     "mie_build_mask_tiles", "mie_conv_masked", "mie_act_incr", "mie_mul_incr", "mie_add_incr",
     "mie_upsample2x_incr", "mie_convlstm_gates_incr", "mie_tconv_masked", "mie_conv_refresh",
-    "mie_pack_filter", "mie_kfence_incr",
+    "mie_pack_filter", "mie_kfence_incr", "mie_events_to_frame",
 )
 
 
@@ -72,6 +73,9 @@ def _declare(l):
                                   vp, vp, ci, cf, ci, vp]
     l.mie_kfence_incr.restype = ci
     l.mie_kfence_incr.argtypes = [vp, vp, vp, cf, vp, ci, tsp, vp, vp]
+    l.mie_events_to_frame.restype = ci
+    cd = ctypes.c_double
+    l.mie_events_to_frame.argtypes = [vp, ci, ci, ci, ci, ci, ci, ci, ci, ci, cd, cd, cd, cd, ci, vp, vp, vp]
     l.mie_pack_filter.restype = ci
     l.mie_pack_filter.argtypes = [vp, ci, ci, ci, vp, vp]
     l.mie_conv_refresh.restype = ci

@@ -93,6 +93,19 @@ class MovingEdges:
         return torch.from_numpy(d) * 0.1, torch.from_numpy(mask)
 
 
+def random_events(n_events: int, width: int, height: int, t0: float, t1: float, seed: int,
+                  density: float = 0.05, polarity=(0.0, 1.0), t_unit: float = 1e9) -> np.ndarray:
+    """(n, 4) float64 rows (t, x, y, p) sorted by time, the row layout of the reference's event
+    files: stamps uniform in [t0, t1] seconds, stored in 1/t_unit seconds (nanoseconds by default);
+    pixels drawn from a smooth blob mask of the given density; polarity from `polarity`."""
+    rng = np.random.default_rng(seed)
+    ys, xs = np.nonzero(blob_mask(height, width, density, seed))
+    pick = rng.integers(0, ys.size, size=n_events)
+    t = np.sort(rng.uniform(t0, t1, size=n_events)) * t_unit
+    p = rng.choice(np.asarray(polarity, dtype=np.float64), size=n_events)
+    return np.stack([t, xs[pick].astype(np.float64), ys[pick].astype(np.float64), p], axis=1)
+
+
 def he_normal_conv_weight(cout, cin, k, seed) -> torch.Tensor:
     """He-normal (std sqrt(2 / (cin * k * k))) conv weight, OIHW."""
     g = torch.Generator().manual_seed(int(seed))

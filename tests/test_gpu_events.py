@@ -1,0 +1,87 @@
+"""GPU parity of the event front end (mie_events_to_frame through EventFrames) against the numpy
+oracle: frames, frame deltas and touched-pixel masks, with the reflection padding folded in."""
+import numpy as np
+import pytest
+import torch
+
+from maskedincrementeval_amd.event_frontend import EventFrames
+from maskedincrementeval_amd.synthetic import random_events
+from oracle import events_oracle as eo
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+RTOL, ATOL = 1e-4, 1e-5      # several float contributions per pixel, summed in a different order
+
+
+def _nchw(t):
+    return t[0].cpu().numpy()
+
+
+@pytest.mark.parametrize("kind", ["voxelgrid", "histogram"])
+@pytest.mark.parametrize("width,height,pad,n_events", [(346, 260, (3, 3, 2, 2), 60000), (33, 21, (0, 0, 0, 0), 2000),
+                                                       (12, 8, (5, 2, 3, 1), 3000)])
+def test_frames_and_deltas_match_oracle(kind, width, height, pad, n_events):
+    pol = (0.0, 1.0) if kind == "voxelgrid" else (-1.0, 1.0)
+    ev = random_events(n_events, width, height, 0.0, 0.08, seed=width + n_events, density=0.2, polarity=pol)
+    ev[::97, 1] = width + 3            # a few events off the sensor: dropped
+    ev[5::89, 2] = -1.0
+    fe = EventFrames(width, height, num_bins=5, evframe_type=kind, window_size=0.05, pad=pad, device=DEV)
+    fe.set_events(ev)
+    starts = [0.010, 0.011, 0.0125, 0.020]
+    want, wmask = eo.frame(ev, kind, 5, height, width, 0.05, starts[0], pad=pad)
+    got = fe.frame(starts[0])
+    torch.cuda.synchronize()
+    assert got.shape == (1, want.shape[0], height + pad[2] + pad[3], width + pad[0] + pad[1])
+    assert np.allclose(_nchw(got), want, rtol=RTOL, atol=ATOL)
+    if kind == "histogram":
+        assert np.array_equal(_nchw(got), want)            # integer counts: exact
+    assert np.array_equal(fe._fmask[0, 0].cpu().numpy(), wmask)
+    total = want.copy()
+    for s0, s1 in zip(starts[:-1], starts[1:]):
+        d, m = fe.delta(s0, s1)
+        torch.cuda.synchronize()
+        wd, wm = eo.frame_delta(ev, kind, 5, height, width, 0.05, s0, s1, pad=pad)
+        assert np.allclose(_nchw(d), wd, rtol=RTOL, atol=ATOL), np.abs(_nchw(d) - wd).max()
+        assert np.array_equal(m[0, 0].cpu().numpy(), wm)
+        assert not (_nchw(d)[:, wm == 0] != 0).any()       # exactly zero off the mask
+        total += _nchw(d)
+    # accumulated deltas reproduce the frame of the last window
+    assert np.allclose(total, eo.frame(ev, kind, 5, height, width, 0.05, starts[-1], pad=pad)[0], rtol=1e-4, atol=1e-4)
+
+
+def test_empty_and_errors():
+    fe = EventFrames(32, 16, device=DEV)
+    with pytest.raises(RuntimeError, match="set_events"):
+        fe.frame(0.0)
+    fe.set_events(np.zeros((0, 4)))
+    fe._frame.fill_(7.0)
+    assert torch.count_nonzero(fe.frame(0.0)) == 0 and torch.count_nonzero(fe._fmask) == 0
+    with pytest.raises(ValueError):
+        fe.set_events(np.zeros((3, 5)))
+    bad = EventFrames(4, 4, pad=(4, 0, 0, 0), device=DEV)      # reflection needs pad < size
+    bad.set_events(np.zeros((1, 4)))
+    with pytest.raises(RuntimeError, match="padding"):
+        bad.frame(0.0)
+
+
+def test_delta_feeds_the_incremental_network():
+    # the delta and mask of the front end drive E2Depth-incr: refresh on frame(t0), incremental steps
+    # on delta(t_i, t_i+1), against a dense evaluation of the same net on frame(t_last)
+    from maskedincrementeval_amd.e2depth_incr import E2VIDRecurrentIncr
+    from maskedincrementeval_amd.synthetic import seed_module_
+    width, height, pad = 58, 44, (3, 3, 2, 2)             # padded to 64 x 48
+    ev = random_events(8000, width, height, 0.0, 0.07, seed=9, density=0.1)
+    fe = EventFrames(width, height, pad=pad, device=DEV)
+    fe.set_events(ev)
+    cfg = dict(num_bins=5, base_num_channels=8, num_encoders=2, num_residual_blocks=1)
+    net = seed_module_(E2VIDRecurrentIncr(cfg), seed=3).to(DEV).eval()
+    starts = [0.005, 0.006, 0.007, 0.009]
+    with torch.no_grad():
+        pred = net.forward_refresh_reservoirs(fe.frame(starts[0]).clone(), None)[0].clone()
+        for s0, s1 in zip(starts[:-1], starts[1:]):
+            d, m = fe.delta(s0, s1)
+            pred += net([d, m], None)[0][0]
+        dense = seed_module_(E2VIDRecurrentIncr(cfg), seed=3).to(DEV).eval()
+        want = dense.forward_refresh_reservoirs(fe.frame(starts[-1]).clone(), None)[0]
+    torch.cuda.synchronize()
+    assert torch.allclose(pred, want, rtol=1e-3, atol=1e-4), (pred - want).abs().max().item()

@@ -314,3 +314,64 @@ def test_convgru_oracle_is_textbook_cell_at_zero_state():
     upd = torch.sigmoid(F.conv2d(torch.cat([x, z], 1), p["g.update_gate.weight"], p["g.update_gate.bias"], padding=1))
     cand = torch.tanh(F.conv2d(torch.cat([x, z], 1), p["g.out_gate.weight"], p["g.out_gate.bias"], padding=1))
     assert torch.allclose(h, cand * upd, atol=2e-6)
+
+
+# ---- event front end (oracle/events_oracle.py) -------------------------------------------------
+def test_events_oracle_closed_forms():
+    from oracle import events_oracle as eo
+    H, W, B, dT, start = 6, 7, 5, 0.05, 2.0
+    stamp = lambda ts: (start + ts * dT / (B - 1)) * 1e9        # event time with normalised time ts
+    # an event exactly on a bin boundary puts its whole polarity into that bin; p == 0 counts as -1
+    g, m = eo.voxel_grid_abst([[stamp(2.0), 3, 4, 1.0], [stamp(1.0), 0, 0, 0.0]], B, H, W, dT, start)
+    want = np.zeros((B, H, W), np.float32)
+    want[2, 4, 3], want[1, 0, 0] = 1.0, -1.0
+    assert np.allclose(g, want, atol=1e-6) and m.sum() == 2 and m[4, 3] == 1 and m[0, 0] == 1
+    # in between: linear weights (a quarter past bin 1: 0.75 / 0.25), summing to the polarity
+    g, _ = eo.voxel_grid_abst([[stamp(1.25), 2, 1, 1.0]], B, H, W, dT, start)
+    assert np.allclose(g[:, 1, 2], [0, 0.75, 0.25, 0, 0], atol=1e-6)
+    # brute force against a per-event python loop, and window membership
+    rng = np.random.default_rng(0)
+    ev = np.stack([rng.uniform(start - 0.01, start + dT + 0.01, 200) * 1e9, rng.integers(0, W, 200),
+                   rng.integers(0, H, 200), rng.integers(0, 2, 200)], 1).astype(np.float64)
+    g, m = eo.voxel_grid_abst(ev, B, H, W, dT, start)
+    brute = np.zeros((B, H, W), np.float64)
+    hit = np.zeros((H, W), np.uint8)
+    for t, x, y, p in ev:
+        ts = (B - 1) * (t / 1e9 - start) / dT
+        if not (0 < ts < B - 1):
+            continue
+        ti, pol = int(ts), (1.0 if p == 1 else -1.0)
+        brute[ti, int(y), int(x)] += pol * (1 - (ts - ti))
+        brute[ti + 1, int(y), int(x)] += pol * (ts - ti)
+        hit[int(y), int(x)] = 1
+    assert np.allclose(g, brute, atol=1e-5) and np.array_equal(m, hit)
+    assert np.isclose(g.sum(), brute.sum(), atol=1e-4)
+    ev_before = ev.copy()
+    eo.voxel_grid_abst(ev, B, H, W, dT, start)
+    assert np.array_equal(ev, ev_before)                       # the input is left alone
+
+
+def test_events_oracle_histogram_pad_and_delta():
+    from oracle import events_oracle as eo
+    H, W, dT = 9, 11, 0.05
+    rng = np.random.default_rng(1)
+    ev = np.stack([np.sort(rng.uniform(0.0, 0.1, 500)) * 1e9, rng.integers(0, W, 500),
+                   rng.integers(0, H, 500), rng.choice([-1.0, 1.0], 500)], 1)
+    h, m = eo.histogram(ev, H, W, dT, 0.01)
+    inw = (ev[:, 0] / 1e9 > 0.01) & (ev[:, 0] / 1e9 < 0.06)
+    for ch, pol in ((0, -1.0), (1, 1.0)):
+        sel = inw & (ev[:, 3] == pol)
+        cnt = np.bincount((ev[sel, 1] + W * ev[sel, 2]).astype(int), minlength=H * W).reshape(H, W)
+        assert np.array_equal(h[ch], cnt.astype(np.float32))
+    assert np.array_equal(m, (h.sum(0) > 0).astype(np.uint8))
+    # padding is torch's ReflectionPad2d
+    pad = (3, 3, 2, 2)
+    g = eo.voxel_grid_abst(ev, 5, H, W, dT, 0.01)[0]
+    assert np.array_equal(eo.reflect_pad(g, pad), torch.nn.ReflectionPad2d(pad)(torch.from_numpy(g)[None])[0].numpy())
+    # the delta of two windows is the difference of their (padded) frames; it vanishes for equal windows
+    d, dm = eo.frame_delta(ev, "voxelgrid", 5, H, W, dT, 0.01, 0.011, pad=pad)
+    f1 = eo.frame(ev, "voxelgrid", 5, H, W, dT, 0.011, pad=pad)[0]
+    f0 = eo.frame(ev, "voxelgrid", 5, H, W, dT, 0.01, pad=pad)[0]
+    assert np.array_equal(d, f1 - f0) and d.shape == (5, H + 4, W + 6)
+    assert not (d[:, dm == 0] != 0).any()                      # nothing outside the mask
+    assert np.count_nonzero(eo.frame_delta(ev, "voxelgrid", 5, H, W, dT, 0.01, 0.01)[0]) == 0
