@@ -36,6 +36,7 @@ def parse_args():
     ap.add_argument("--density", type=float, default=0.05)
     ap.add_argument("--height", type=int, default=264)
     ap.add_argument("--width", type=int, default=352)
+    ap.add_argument("--batch", type=int, default=1, help="independent event streams per step (8 with 480x640: the batched configuration)")
     ap.add_argument("--cpu-steps", type=int, default=200, help="incremental steps of the CPU baseline (0 = skip)")
     ap.add_argument("--no-graph", action="store_true", help="launch kernels eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-dense", action="store_true", help="skip the all-tiles-active comparator")
@@ -158,15 +159,15 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
     dev = torch.device("cuda:0")
-    H, W, dens = args.height, args.width, args.density
+    H, W, dens, NB = args.height, args.width, args.density, args.batch
     cl = lambda t: t.to(dev).contiguous(memory_format=torch.channels_last)
 
     model = seed_module_(E2VIDRecurrentIncr(async_masks=not args.sync_masks), seed=1).to(dev).eval()
-    x0 = torch.randn(1, 5, H, W, generator=torch.Generator().manual_seed(2)) * 0.5
+    x0 = torch.randn(NB, 5, H, W, generator=torch.Generator().manual_seed(2)) * 0.5
     n_inputs = 16
-    deltas_cpu = [event_voxel_delta(1, 5, H, W, dens, seed=3000 + i)[0] for i in range(n_inputs)]
+    deltas_cpu = [event_voxel_delta(NB, 5, H, W, dens, seed=3000 + i)[0] for i in range(n_inputs)]
     deltas = [cl(d) for d in deltas_cpu]
-    static_in = cl(torch.zeros(1, 5, H, W))
+    static_in = cl(torch.zeros(NB, 5, H, W))
 
     def step_eager(m, i):
         static_in.copy_(deltas[i % n_inputs])
@@ -317,7 +318,7 @@ def main():
         for p in (0.01, 0.20):
             if abs(p - dens) < 1e-9:
                 continue
-            deltas[:] = [cl(event_voxel_delta(1, 5, H, W, p, seed=3000 + i)[0]) for i in range(n_inputs)]
+            deltas[:] = [cl(event_voxel_delta(NB, 5, H, W, p, seed=3000 + i)[0]) for i in range(n_inputs)]
             t = timed_run(model, "incremental %.0f%%" % (100 * p))
             sweep["%.2f" % p] = dict(ms_per_step=round(1e3 * t, 4), frames_per_s=round(1 / t, 1))
         deltas[:] = keep
@@ -335,15 +336,15 @@ def main():
             for i in range(args.cpu_steps):
                 oracle.incr(deltas_cpu[(1 + i) % n_inputs])
             cdt = (time.perf_counter() - t0) / args.cpu_steps
-        cpu = dict(value=round(1.0 / cdt, 3), unit="frames/s", cores=torch.get_num_threads(), kind="port",
+        cpu = dict(value=round(NB / cdt, 3), unit="frames/s", cores=torch.get_num_threads(), kind="port",
                    ms_per_step=round(1e3 * cdt, 2),
                    sample="%d incremental steps of the same E2Depth-incr %dx%d workload (dense F.conv2d on the "
                           "delta, as the reference executes it), torch-CPU fp32" % (args.cpu_steps, H, W))
         print("[bench] cpu baseline: %.1f ms/frame on %d threads" % (1e3 * cdt, cpu["cores"]), file=sys.stderr, flush=True)
 
     result = {
-        "metric": "incremental frames/s, E2Depth-incr 264x352 @5% delta density",
-        "value": round(1.0 / sec_per_step, 2),
+        "metric": "incremental frames/s, E2Depth-incr %dx%d @%g%% delta density" % (H, W, 100 * dens),
+        "value": round(NB / sec_per_step, 2),
         "unit": "frames/s",
         "n_gpus": 1,
         "steps": args.steps,
@@ -354,9 +355,9 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": "E2Depth-incr recurrent UNet, random init, 1x5x%dx%d event voxel deltas, %.0f%% "
-                               "active pixels, 1 dense refresh then incremental steps" % (H, W, 100 * dens),
-                   "density": dens, "height": H, "width": W, "graph": not args.no_graph},
+        "config": {"workload": "E2Depth-incr recurrent UNet, random init, %dx5x%dx%d event voxel deltas, %.0f%% "
+                               "active pixels, 1 dense refresh then incremental steps" % (NB, H, W, 100 * dens),
+                   "density": dens, "height": H, "width": W, "batch": NB, "graph": not args.no_graph},
         "roofline": roofline,
         "cpu_baseline": cpu,
         "hbm_frac_whole_frame": round(tot_bytes / sec_per_step / 1e9 / PEAK_HBM_GBS, 5),

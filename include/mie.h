@@ -68,6 +68,13 @@ extern "C" {
 /* flags of mie_act_incr / mie_mul_incr */
 #define MIE_FLAG_KEEP_RESERVOIR 1  /* compute the delta, leave reservoirs as is */
 
+/* element type of the DELTA buffers of a call (inputs, outputs, addend, and the
+ * matrix-core filter copy).  Reservoirs, bias, the plain filter and every
+ * accumulation are fp32 in both cases.  bf16 values are converted with
+ * round-to-nearest-even.  Pointers to such buffers are `void*` below. */
+#define MIE_DTYPE_F32 0
+#define MIE_DTYPE_BF16 1
+
 /* frame kinds of mie_events_to_frame */
 #define MIE_EVENTS_VOXEL 0      /* num_bins channels, linear weights in time   */
 #define MIE_EVENTS_HISTOGRAM 1  /* 2 channels: counts of p == -1, of p == +1   */
@@ -109,8 +116,8 @@ int mie_tile_capacity(int n, int h, int w);
  * utils/str_sparse_utils.py:10-11); the dilation by the field is the
  * MIE_FOOT_CONV footprint of mie_build_mask_tiles.
  */
-int mie_mask_from_delta(const float* delta, int n, int h, int w, int c,
-                        float threshold, uint8_t* pixmask, void* stream);
+int mie_mask_from_delta(const void* delta, int n, int h, int w, int c,
+                        float threshold, uint8_t* pixmask, int dtype, void* stream);
 
 /*
  * Build the output pixel mask and the ordered active-tile list of an op from
@@ -132,16 +139,19 @@ int mie_build_mask_tiles(const uint8_t* in_mask, const uint8_t* in_mask2,
                          int pad, const mie_tileset* out, void* stream);
 
 /*
- * Re-order a [cin][k][k][cout] filter (cin % 8 == 0) into the layout the
- * matrix-core kernels stream: P[ci/8][tap][(ci%8)/4][co][ci%4], so that the four
- * k-steps a lane multiplies per tap come as one 16-byte load.  `packed` has the
- * size of `filter`; do this once per weight update.
+ * Re-order a fp32 [cin][k][k][cout] filter into the layout the matrix-core
+ * kernels stream, so that the k-steps a lane multiplies per tap come as one
+ * 16-byte load:
+ *   MIE_DTYPE_F32  (cin % 8 == 0):  P[ci/8][tap][(ci%8)/4][co][ci%4], fp32
+ *   MIE_DTYPE_BF16 (cin % 16 == 0): P[ci/16][tap][(ci%16)/8][co][ci%8], bf16
+ * `packed` holds cin*k*k*cout elements of that type; do this once per weight
+ * update.
  * Replaces: convert_filter_out_channels_last
  * (ext/pointops/pointops_functional.py:13-14), which plays the same role for
  * the reference kernel.
  */
-int mie_pack_filter(const float* filter, int cin, int k, int cout, float* packed,
-                    void* stream);
+int mie_pack_filter(const float* filter, int cin, int k, int cout, void* packed,
+                    int dtype, void* stream);
 
 /*
  * Masked convolution of a delta: for every active tile of `out`
@@ -161,25 +171,29 @@ int mie_pack_filter(const float* filter, int cin, int k, int cout, float* packed
  *   x2 : optional second input [n, h_in, w_in, c2] (NULL, c2 = 0 if absent),
  *        feeds filter input channels [c1, c1 + c2) -- the concat-free form of
  *        torch.cat((x, h), 1) in ConvLSTMIncr (incr_modules/e2depth_incr.py:100)
- *   filter : [cin_total][k][k][cout], c1 + c2 <= cin_total
+ *   filter : fp32 [cin_total][k][k][cout], c1 + c2 <= cin_total
  *   filter_mc : optional copy of the same filter in the matrix-core layout made
- *        by mie_pack_filter (same size).  The MFMA kernels read only this copy;
+ *        by mie_pack_filter with the same dtype.  The MFMA kernels read only this copy;
  *        without it MIE_PATH_AUTO takes the VALU kernels and MIE_PATH_MFMA is
  *        refused.
  *   k in {1,3,5,7}, stride in {1,2}; out->h/w must equal (h_in+2*pad-k)/stride+1
+ *   dtype : element type of x, x2, addend, out_delta and filter_mc
+ *        (MIE_DTYPE_BF16: products of bf16 values accumulated in fp32 on the
+ *        matrix cores, v_mfma_f32_32x32x16_bf16; the VALU kernels multiply the
+ *        fp32 `filter`, so give them bf16-representable weights for one result)
  * Replaces: conv{1,3,5,7}x*_increment_ext(x_incr, mask, filter, out_incr, stride)
  * (ext/pointops/_C_ext/pointops/ops.cpp:51-114, include/ops.h:8-52) and the
  * F.conv2d fallback the reference actually runs
  * (incr_modules/mask_incr_modules.py:175-178).
  */
-int mie_conv_masked(const float* x, const uint8_t* xmask, int c1,
-                    const float* x2, const uint8_t* x2mask, int c2,
+int mie_conv_masked(const void* x, const uint8_t* xmask, int c1,
+                    const void* x2, const uint8_t* x2mask, int c2,
                     int h_in, int w_in, const float* filter,
-                    const float* filter_mc, int cin_total,
+                    const void* filter_mc, int cin_total,
                     int k, int stride, int pad, int cout,
-                    const mie_tileset* out, float* out_delta,
-                    const float* addend, float* reservoir, int act_kind,
-                    float slope, int path, void* stream);
+                    const mie_tileset* out, void* out_delta,
+                    const void* addend, float* reservoir, int act_kind,
+                    float slope, int path, int dtype, void* stream);
 
 /*
  * Dense refresh through the same kernels: for every active tile of `out`
@@ -193,13 +207,13 @@ int mie_conv_masked(const float* x, const uint8_t* xmask, int c1,
  * nnReservedActivation.forward_refresh_reservoirs
  * (incr_modules/mask_incr_modules.py:182-196,253-256).
  */
-int mie_conv_refresh(const float* x, int c1, const float* x2, int c2, int h_in,
-                     int w_in, const float* filter, const float* filter_mc,
+int mie_conv_refresh(const void* x, int c1, const void* x2, int c2, int h_in,
+                     int w_in, const float* filter, const void* filter_mc,
                      int cin_total, int k,
                      int stride, int pad, int cout, const float* bias,
-                     const mie_tileset* out, float* out_dense,
-                     const float* addend, float* reservoir, int act_kind,
-                     float slope, int path, void* stream);
+                     const mie_tileset* out, void* out_dense,
+                     const void* addend, float* reservoir, int act_kind,
+                     float slope, int path, int dtype, void* stream);
 
 /*
  * Incremental point-wise non-linearity over the active tiles of ts:
@@ -217,10 +231,10 @@ int mie_conv_refresh(const float* x, int c1, const float* x2, int c2, int h_in,
  * NonlinearPointOpIncr._nonlin + IncrementReserve.accumulate
  * (incr_modules/mask_incr_modules.py:101-103,248-251).
  */
-int mie_act_incr(int act_kind, float slope, const float* in_delta,
-                 float* reservoir, float* out_delta, int c,
+int mie_act_incr(int act_kind, float slope, const void* in_delta,
+                 float* reservoir, void* out_delta, int c,
                  const mie_tileset* ts, uint8_t* out_pixmask, int flags,
-                 void* stream);
+                 int dtype, void* stream);
 
 /*
  * Delta quantiser ("k-fence"): lets multiples of k through and carries the rest
@@ -239,9 +253,9 @@ int mie_act_incr(int act_kind, float slope, const float* in_delta,
  * (incr_modules/mask_incr_modules.py:32-42); k is what
  * KFencedMaskModule.forward_refresh_reservoirs (:44-48) sets.
  */
-int mie_kfence_incr(const float* in_delta, float* carry, const float* k_dev,
-                    float k_host, float* out_delta, int c, const mie_tileset* ts,
-                    uint8_t* out_pixmask, void* stream);
+int mie_kfence_incr(const void* in_delta, float* carry, const float* k_dev,
+                    float k_host, void* out_delta, int c, const mie_tileset* ts,
+                    uint8_t* out_pixmask, int dtype, void* stream);
 
 /*
  * Incremental point-wise product (product rule with cached operands):
@@ -253,19 +267,19 @@ int mie_kfence_incr(const float* in_delta, float* carry, const float* k_dev,
  * Replaces: IncrPointwiseMultiply + nnReservedMultiplication.forward
  * (incr_modules/mask_incr_functional.py:52-54, mask_incr_modules.py:67-75).
  */
-int mie_mul_incr(const float* d1, const uint8_t* m1, float* r1,
-                 const float* d2, const uint8_t* m2, float* r2,
-                 float* out_delta, int c, const mie_tileset* ts, int flags,
-                 void* stream);
+int mie_mul_incr(const void* d1, const uint8_t* m1, float* r1,
+                 const void* d2, const uint8_t* m2, float* r2,
+                 void* out_delta, int c, const mie_tileset* ts, int flags,
+                 int dtype, void* stream);
 
 /*
  * out = a + b over the active tiles of ts (built from the union of ma, mb).
  * Replaces: the skip sum / residual sum on deltas
  * (incr_modules/e2depth_incr.py:220,333).
  */
-int mie_add_incr(const float* a, const uint8_t* ma, const float* b,
-                 const uint8_t* mb, float* out_delta, int c,
-                 const mie_tileset* ts, void* stream);
+int mie_add_incr(const void* a, const uint8_t* ma, const void* b,
+                 const uint8_t* mb, void* out_delta, int c,
+                 const mie_tileset* ts, int dtype, void* stream);
 
 /*
  * Bilinear x2 up-sampling (align_corners = False) of a delta, optionally of
@@ -275,9 +289,10 @@ int mie_add_incr(const float* a, const uint8_t* ma, const float* b,
  * with the skip sum of UNetRecurrentIncr.forward folded in
  * (incr_modules/e2depth_incr.py:429-431).
  */
-int mie_upsample2x_incr(const float* a, const uint8_t* ma, const float* b,
+int mie_upsample2x_incr(const void* a, const uint8_t* ma, const void* b,
                         const uint8_t* mb, int h_in, int w_in, int c,
-                        const mie_tileset* out, float* out_delta, void* stream);
+                        const mie_tileset* out, void* out_delta, int dtype,
+                        void* stream);
 
 /*
  * Fused incremental ConvLSTM gate math for hidden size hid over the active
@@ -293,11 +308,11 @@ int mie_upsample2x_incr(const float* a, const uint8_t* ma, const float* b,
  * pre-activation reservoirs, and writes h_delta, c_delta ([n,h,w,hid]).
  * Replaces: incr_modules/e2depth_incr.py:103-120 (about 25 ATen launches).
  */
-int mie_convlstm_gates_incr(const float* gates_delta, float* gates_res,
-                            const float* cprev_delta, const uint8_t* cprev_mask,
-                            float* cprev_res, float* cell_res, float* h_delta,
-                            float* c_delta, int hid, const mie_tileset* ts,
-                            void* stream);
+int mie_convlstm_gates_incr(const void* gates_delta, float* gates_res,
+                            const void* cprev_delta, const uint8_t* cprev_mask,
+                            float* cprev_res, float* cell_res, void* h_delta,
+                            void* c_delta, int hid, const mie_tileset* ts,
+                            int dtype, void* stream);
 
 /*
  * Masked transposed convolution of a delta (stride s, padding p; the output
@@ -309,10 +324,11 @@ int mie_convlstm_gates_incr(const float* gates_delta, float* gates_res,
  * Replaces: transposed_conv2d_from_module
  * (incr_modules/mask_incr_functional.py:64-66).
  */
-int mie_tconv_masked(const float* x, const uint8_t* xmask, int cin, int h_in,
+int mie_tconv_masked(const void* x, const uint8_t* xmask, int cin, int h_in,
                      int w_in, const float* filter, int k, int stride, int pad,
-                     int cout, const mie_tileset* out, float* out_delta,
-                     float* reservoir, int act_kind, float slope, void* stream);
+                     int cout, const mie_tileset* out, void* out_delta,
+                     float* reservoir, int act_kind, float slope, int dtype,
+                     void* stream);
 
 /*
  * Event front end: scatter raw events into a frame, or directly into the DELTA

@@ -22,6 +22,7 @@ MIE_TILE = 8
 ACT_NONE, ACT_RELU, ACT_LEAKY_RELU, ACT_SIGMOID, ACT_TANH = 0, 1, 2, 3, 4
 FOOT_CONV, FOOT_UP2X, FOOT_TCONV = 0, 1, 2
 EVENTS_VOXEL, EVENTS_HISTOGRAM = 0, 1
+DTYPE_F32, DTYPE_BF16 = 0, 1
 PATH_AUTO, PATH_VALU, PATH_MFMA = 0, 1, 2
 FLAG_KEEP_RESERVOIR = 1
 CNT_ACTIVE, CNT_STALE, CNT_TICKET, CNT_WORDS = 0, 1, 2, 4
@@ -65,34 +66,34 @@ def _declare(l):
     l.mie_tile_capacity.restype = ci
     l.mie_tile_capacity.argtypes = [ci, ci, ci]
     l.mie_mask_from_delta.restype = ci
-    l.mie_mask_from_delta.argtypes = [vp, ci, ci, ci, ci, cf, vp, vp]
+    l.mie_mask_from_delta.argtypes = [vp, ci, ci, ci, ci, cf, vp, ci, vp]
     l.mie_build_mask_tiles.restype = ci
     l.mie_build_mask_tiles.argtypes = [vp, vp, ci, ci, ci, ci, ci, ci, tsp, vp]
     l.mie_conv_masked.restype = ci
     l.mie_conv_masked.argtypes = [vp, vp, ci, vp, vp, ci, ci, ci, vp, vp, ci, ci, ci, ci, ci, tsp, vp,
-                                  vp, vp, ci, cf, ci, vp]
+                                  vp, vp, ci, cf, ci, ci, vp]
     l.mie_kfence_incr.restype = ci
-    l.mie_kfence_incr.argtypes = [vp, vp, vp, cf, vp, ci, tsp, vp, vp]
+    l.mie_kfence_incr.argtypes = [vp, vp, vp, cf, vp, ci, tsp, vp, ci, vp]
     l.mie_events_to_frame.restype = ci
     cd = ctypes.c_double
     l.mie_events_to_frame.argtypes = [vp, ci, ci, ci, ci, ci, ci, ci, ci, ci, cd, cd, cd, cd, ci, vp, vp, vp]
     l.mie_pack_filter.restype = ci
-    l.mie_pack_filter.argtypes = [vp, ci, ci, ci, vp, vp]
+    l.mie_pack_filter.argtypes = [vp, ci, ci, ci, vp, ci, vp]
     l.mie_conv_refresh.restype = ci
     l.mie_conv_refresh.argtypes = [vp, ci, vp, ci, ci, ci, vp, vp, ci, ci, ci, ci, ci, vp, tsp, vp, vp,
-                                   vp, ci, cf, ci, vp]
+                                   vp, ci, cf, ci, ci, vp]
     l.mie_act_incr.restype = ci
-    l.mie_act_incr.argtypes = [ci, cf, vp, vp, vp, ci, tsp, vp, ci, vp]
+    l.mie_act_incr.argtypes = [ci, cf, vp, vp, vp, ci, tsp, vp, ci, ci, vp]
     l.mie_mul_incr.restype = ci
-    l.mie_mul_incr.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, tsp, ci, vp]
+    l.mie_mul_incr.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, tsp, ci, ci, vp]
     l.mie_add_incr.restype = ci
-    l.mie_add_incr.argtypes = [vp, vp, vp, vp, vp, ci, tsp, vp]
+    l.mie_add_incr.argtypes = [vp, vp, vp, vp, vp, ci, tsp, ci, vp]
     l.mie_upsample2x_incr.restype = ci
-    l.mie_upsample2x_incr.argtypes = [vp, vp, vp, vp, ci, ci, ci, tsp, vp, vp]
+    l.mie_upsample2x_incr.argtypes = [vp, vp, vp, vp, ci, ci, ci, tsp, vp, ci, vp]
     l.mie_convlstm_gates_incr.restype = ci
-    l.mie_convlstm_gates_incr.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, ci, tsp, vp]
+    l.mie_convlstm_gates_incr.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, ci, tsp, ci, vp]
     l.mie_tconv_masked.restype = ci
-    l.mie_tconv_masked.argtypes = [vp, vp, ci, ci, ci, vp, ci, ci, ci, ci, tsp, vp, vp, ci, cf, vp]
+    l.mie_tconv_masked.argtypes = [vp, vp, ci, ci, ci, vp, ci, ci, ci, ci, tsp, vp, vp, ci, cf, ci, vp]
 
 
 def lib():

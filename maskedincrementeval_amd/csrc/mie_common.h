@@ -12,6 +12,18 @@
 
 #define MIE_WAVE 64
 
+// bf16 deltas (MIE_DTYPE_BF16): the compiler's native type; conversions from fp32 round to
+// nearest even (v_cvt_pk_bf16_f32 on gfx950), conversions to fp32 are exact.
+typedef __bf16 mie_bf16;
+typedef __bf16 mie_bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 mie_bf16x8 __attribute__((ext_vector_type(8)));
+
+// Scalar load / store of a delta element as fp32.
+static __device__ __forceinline__ float mie_ld(const float* p, long long i) { return p[i]; }
+static __device__ __forceinline__ float mie_ld(const mie_bf16* p, long long i) { return (float)p[i]; }
+static __device__ __forceinline__ void mie_st(float* p, long long i, float v) { p[i] = v; }
+static __device__ __forceinline__ void mie_st(mie_bf16* p, long long i, float v) { p[i] = (mie_bf16)v; }
+
 // ---- host side: error reporting -------------------------------------------
 void mie_set_error(const char* fmt, ...);
 void mie_clear_error();

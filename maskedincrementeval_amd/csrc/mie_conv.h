@@ -3,40 +3,46 @@
 #pragma once
 #include "mie_common.h"
 
-struct ConvArgs {
-  const float* x; const uint8_t* xm; int c1;
-  const float* x2; const uint8_t* x2m; int c2;
+// T = element type of the deltas (inputs, output, addend) and of the matrix-core filter copy:
+// float or mie_bf16.  Reservoirs, bias, the plain filter and all accumulation are fp32.
+template <typename T>
+struct ConvArgsT {
+  const T* x; const uint8_t* xm; int c1;
+  const T* x2; const uint8_t* x2m; int c2;
   int h_in, w_in;
   const float* filt; int cin_total;
-  const float* filt_mc;             // matrix-core copy of the filter (mie_pack_filter) or NULL
+  const T* filt_mc;                 // matrix-core copy of the filter (mie_pack_filter) or NULL
   int pad, cout;
-  float* out; float* res; int act; float slope;
-  const float* addend;              // optional delta added to the conv result before the epilogue
+  T* out; float* res; int act; float slope;
+  const T* addend;                  // optional delta added to the conv result before the epilogue
   int refresh; const float* bias;   // dense refresh: out = act(acc + bias), res = acc + bias
   TileSetDev ts;
 };
+typedef ConvArgsT<float> ConvArgs;
 
 // Epilogue for one output element (linear offset off, output channel co).
-static __device__ __forceinline__ void conv_store(const ConvArgs& a, long long off, int co, float acc) {
-  if (a.addend) acc += a.addend[off];
+template <typename T>
+static __device__ __forceinline__ void conv_store(const ConvArgsT<T>& a, long long off, int co, float acc) {
+  if (a.addend) acc += mie_ld(a.addend, off);
   if (a.refresh) {
     const float v = a.bias ? acc + a.bias[co] : acc;
     if (a.res) a.res[off] = v;
-    a.out[off] = mie_act(a.act, a.slope, v);
+    mie_st(a.out, off, mie_act(a.act, a.slope, v));
   } else if (a.res) {
     const float r0 = a.res[off], r1 = r0 + acc;
     a.res[off] = r1;
-    a.out[off] = mie_act(a.act, a.slope, r1) - mie_act(a.act, a.slope, r0);
+    mie_st(a.out, off, mie_act(a.act, a.slope, r1) - mie_act(a.act, a.slope, r0));
   } else {
-    a.out[off] = acc;
+    mie_st(a.out, off, acc);
   }
 }
 
 
 // Launches the matrix-core path for kernel size k (1,3,5,7) and stride s (1,2); the caller
-// has checked that c1 and c2 are multiples of mie_conv_mfma_cin_multiple(k, s) (the channels
-// staged per chunk) and cout of mie_conv_mfma_cout_multiple(k, s).
+// has checked that c1 and c2 are multiples of mie_conv_mfma_cin_multiple(k, s, dtype) (the
+// channels staged per chunk) and cout of mie_conv_mfma_cout_multiple(k, s).
 // Returns false if no kernel variant takes the shape (nothing is launched then).
-bool mie_launch_conv_mfma(const ConvArgs& a, int k, int s, unsigned cap, hipStream_t st);
+bool mie_launch_conv_mfma(const ConvArgsT<float>& a, int k, int s, unsigned cap, hipStream_t st);
+bool mie_launch_conv_mfma(const ConvArgsT<mie_bf16>& a, int k, int s, unsigned cap, hipStream_t st);
 int mie_conv_mfma_cout_multiple(int k, int s);
-int mie_conv_mfma_cin_multiple(int k, int s);
+int mie_conv_mfma_cin_multiple(int k, int s, int dtype);

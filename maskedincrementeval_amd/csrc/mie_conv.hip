@@ -17,8 +17,8 @@ namespace {
 // VALU path.  Block = 256 threads = 64 output channels x 4 pixel groups (two
 // tile rows each).  CC input channels per LDS stage.
 // ---------------------------------------------------------------------------------
-template <int K, int S>
-__global__ __launch_bounds__(256) void k_conv_valu(ConvArgs a) {
+template <typename T, int K, int S>
+__global__ __launch_bounds__(256) void k_conv_valu(ConvArgsT<T> a) {
   constexpr int IT = 7 * S + K;  // input tile edge incl. halo
   constexpr int CC = 8;
   __shared__ float s_in[IT * IT * CC];
@@ -32,7 +32,7 @@ __global__ __launch_bounds__(256) void k_conv_valu(ConvArgs a) {
     if (co < a.cout)
       for (int p = 0; p < 16; ++p) {
         const int oy = y0 + 2 * pg + (p >> 3), ox = x0 + (p & 7);
-        if (oy < hout && ox < wout) a.out[(((long long)n * hout + oy) * wout + ox) * a.cout + co] = 0.f;
+        if (oy < hout && ox < wout) mie_st(a.out, (((long long)n * hout + oy) * wout + ox) * a.cout + co, 0.f);
       }
     return;
   }
@@ -42,7 +42,7 @@ __global__ __launch_bounds__(256) void k_conv_valu(ConvArgs a) {
   const int iy0 = y0 * S - a.pad, ix0 = x0 * S - a.pad;
 
   for (int src = 0; src < 2; ++src) {
-    const float* xin = src ? a.x2 : a.x;
+    const T* xin = src ? a.x2 : a.x;
     const uint8_t* xm = src ? a.x2m : a.xm;
     const int cs = src ? a.c2 : a.c1;
     const int fbase = src ? a.c1 : 0;
@@ -55,7 +55,7 @@ __global__ __launch_bounds__(256) void k_conv_valu(ConvArgs a) {
         float v = 0.f;
         if (ci0 + cc < cs && iy >= 0 && iy < a.h_in && ix >= 0 && ix < a.w_in) {
           const long long po = ((long long)n * a.h_in + iy) * a.w_in + ix;
-          if (xm == nullptr || xm[po]) v = xin[po * cs + ci0 + cc];
+          if (xm == nullptr || xm[po]) v = mie_ld(xin, po * cs + ci0 + cc);
         }
         s_in[idx] = v;
       }
@@ -90,8 +90,8 @@ __global__ __launch_bounds__(256) void k_conv_valu(ConvArgs a) {
 // ---------------------------------------------------------------------------------
 // Small-Cout path (Cout <= 4): one wave per tile, lane = output pixel.
 // ---------------------------------------------------------------------------------
-template <int K, int S>
-__global__ __launch_bounds__(64) void k_conv_smallco(ConvArgs a) {
+template <typename T, int K, int S>
+__global__ __launch_bounds__(64) void k_conv_smallco(ConvArgsT<T> a) {
   int n, y0, x0;
   const int tk = mie_pick_tile(a.ts, blockIdx.x, n, y0, x0);
   if (tk == 0) return;
@@ -101,12 +101,12 @@ __global__ __launch_bounds__(64) void k_conv_smallco(ConvArgs a) {
   if (oy >= hout || ox >= wout) return;
   const long long obase = (((long long)n * hout + oy) * wout + ox) * a.cout;
   if (tk == 2) {
-    for (int co = 0; co < a.cout; ++co) a.out[obase + co] = 0.f;
+    for (int co = 0; co < a.cout; ++co) mie_st(a.out, obase + co, 0.f);
     return;
   }
   float acc[4] = {0.f, 0.f, 0.f, 0.f};
   for (int src = 0; src < 2; ++src) {
-    const float* xin = src ? a.x2 : a.x;
+    const T* xin = src ? a.x2 : a.x;
     const uint8_t* xm = src ? a.x2m : a.xm;
     const int cs = src ? a.c2 : a.c1;
     const int fbase = src ? a.c1 : 0;
@@ -119,9 +119,9 @@ __global__ __launch_bounds__(64) void k_conv_smallco(ConvArgs a) {
         if (ix < 0 || ix >= a.w_in) continue;
         const long long po = ((long long)n * a.h_in + iy) * a.w_in + ix;
         if (xm != nullptr && !xm[po]) continue;
-        const float* xr = xin + po * cs;
+        const T* xr = xin + po * cs;
         for (int ci = 0; ci < cs; ++ci) {
-          const float xv = xr[ci];
+          const float xv = mie_ld(xr, ci);
           const float* wp = a.filt + ((long long)(fbase + ci) * K * K + ky * K + kx) * a.cout;
           for (int co = 0; co < a.cout; ++co) acc[co] += xv * wp[co];
         }
@@ -136,7 +136,8 @@ __global__ __launch_bounds__(64) void k_conv_smallco(ConvArgs a) {
 // input values are wave-uniform loads (every lane of a wave reads the same
 // address), filter rows are coalesced over the output channel.
 // ---------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void k_tconv_valu(ConvArgs a, int K, int S) {
+template <typename T>
+__global__ __launch_bounds__(256) void k_tconv_valu(ConvArgsT<T> a, int K, int S) {
   int n, y0, x0;
   const int tk = mie_pick_tile(a.ts, blockIdx.x, n, y0, x0);
   if (tk == 0) return;
@@ -148,7 +149,7 @@ __global__ __launch_bounds__(256) void k_tconv_valu(ConvArgs a, int K, int S) {
     const int oy = y0 + 2 * pg + (p >> 3), ox = x0 + (p & 7);
     if (oy >= hout || ox >= wout) continue;
     const long long off = (((long long)n * hout + oy) * wout + ox) * a.cout + co;
-    if (tk == 2) { a.out[off] = 0.f; continue; }
+    if (tk == 2) { mie_st(a.out, off, 0.f); continue; }
     float acc = 0.f;
     for (int ky = 0; ky < K; ++ky) {
       const int ty = oy + a.pad - ky;
@@ -158,25 +159,27 @@ __global__ __launch_bounds__(256) void k_tconv_valu(ConvArgs a, int K, int S) {
         if (tx < 0 || (tx % S) != 0 || tx / S >= a.w_in) continue;
         const long long po = ((long long)n * a.h_in + ty / S) * a.w_in + tx / S;
         if (a.xm != nullptr && !a.xm[po]) continue;
-        const float* xr = a.x + po * a.c1;
+        const T* xr = a.x + po * a.c1;
         const float* wp = a.filt + (long long)(ky * K + kx) * a.cout + co;
-        for (int ci = 0; ci < a.c1; ++ci) acc += xr[ci] * wp[(long long)ci * K * K * a.cout];
+        for (int ci = 0; ci < a.c1; ++ci) acc += mie_ld(xr, ci) * wp[(long long)ci * K * K * a.cout];
       }
     }
     conv_store(a, off, co, acc);
   }
 }
 
-template <int K, int S>
-void launch_conv(const ConvArgs& a, unsigned cap, hipStream_t st) {
+template <typename T, int K, int S>
+void launch_conv(const ConvArgsT<T>& a, unsigned cap, hipStream_t st) {
   if (a.cout <= 4) {
-    hipLaunchKernelGGL((k_conv_smallco<K, S>), dim3(cap), dim3(64), 0, st, a);
+    hipLaunchKernelGGL((k_conv_smallco<T, K, S>), dim3(cap), dim3(64), 0, st, a);
   } else {
-    hipLaunchKernelGGL((k_conv_valu<K, S>), dim3(cap, mie_div_up(a.cout, 64)), dim3(256), 0, st, a);
+    hipLaunchKernelGGL((k_conv_valu<T, K, S>), dim3(cap, mie_div_up(a.cout, 64)), dim3(256), 0, st, a);
   }
 }
 
-int check_epilogue(const char* who, float* out_delta, float* reservoir, int act_kind,
+template <typename T> constexpr int dtype_of() { return sizeof(T) == 4 ? MIE_DTYPE_F32 : MIE_DTYPE_BF16; }
+
+int check_epilogue(const char* who, const void* out_delta, float* reservoir, int act_kind,
                    bool refresh = false) {
   MIE_REQUIRE(out_delta != nullptr, MIE_ERR_INVALID_ARG, "%s: out_delta is NULL", who);
   MIE_REQUIRE(mie_aligned(out_delta, 16) && mie_aligned(reservoir, 16), MIE_ERR_INVALID_ARG,
@@ -188,11 +191,12 @@ int check_epilogue(const char* who, float* out_delta, float* reservoir, int act_
   return MIE_OK;
 }
 
-int conv_impl(const char* who, const float* x, const uint8_t* xmask, int c1, const float* x2,
+template <typename T>
+int conv_impl(const char* who, const T* x, const uint8_t* xmask, int c1, const T* x2,
               const uint8_t* x2mask, int c2, int h_in, int w_in, const float* filter,
-              const float* filter_mc, int cin_total, int k, int stride, int pad, int cout,
+              const T* filter_mc, int cin_total, int k, int stride, int pad, int cout,
               const mie_tileset* out,
-              float* out_delta, const float* addend, float* reservoir, int act_kind, float slope,
+              T* out_delta, const T* addend, float* reservoir, int act_kind, float slope,
               int path, bool refresh, const float* bias, void* stream) {
   mie_clear_error();
   int rc = mie_check_tileset(out, who);
@@ -228,9 +232,10 @@ int conv_impl(const char* who, const float* x, const uint8_t* xmask, int c1, con
   MIE_REQUIRE(addend == nullptr || addend != out_delta, MIE_ERR_INVALID_ARG,
               "%s: addend must not alias out_delta", who);
   const int cmul = mie_conv_mfma_cout_multiple(k, stride);
-  const int imul = mie_conv_mfma_cin_multiple(k, stride);
+  const int imul = mie_conv_mfma_cin_multiple(k, stride, dtype_of<T>());
+  const int pmul = 32 / (int)sizeof(T);       // input channels per block of the matrix-core filter copy
   MIE_REQUIRE(mie_aligned(filter_mc, 16), MIE_ERR_INVALID_ARG, "%s: filter_mc must be 16-byte aligned", who);
-  const bool mfma_ok = (filter_mc != nullptr) && (cin_total % 8 == 0) && (c1 % imul == 0) &&
+  const bool mfma_ok = (filter_mc != nullptr) && (cin_total % pmul == 0) && (c1 % imul == 0) &&
                        (c2 % imul == 0) && (cout % cmul == 0);
   MIE_REQUIRE(path == MIE_PATH_AUTO || path == MIE_PATH_VALU || path == MIE_PATH_MFMA,
               MIE_ERR_INVALID_ARG, "%s: unknown path %d", who, path);
@@ -239,7 +244,7 @@ int conv_impl(const char* who, const float* x, const uint8_t* xmask, int c1, con
               "(filter_mc=%p c1=%d c2=%d cout=%d)", who, imul, imul, cmul, (const void*)filter_mc, c1, c2, cout);
   if (path == MIE_PATH_AUTO) path = mfma_ok ? MIE_PATH_MFMA : MIE_PATH_VALU;
 
-  ConvArgs a;
+  ConvArgsT<T> a;
   a.x = x; a.xm = xmask; a.c1 = c1; a.x2 = x2; a.x2m = x2mask; a.c2 = c2;
   a.h_in = h_in; a.w_in = w_in; a.filt = filter; a.cin_total = cin_total; a.filt_mc = filter_mc;
   a.pad = pad; a.cout = cout; a.out = out_delta; a.res = reservoir; a.act = act_kind;
@@ -253,14 +258,14 @@ int conv_impl(const char* who, const float* x, const uint8_t* xmask, int c1, con
     return mie_check_launch(who);
   }
   switch (k * 10 + stride) {
-    case 11: launch_conv<1, 1>(a, cap, st); break;
-    case 12: launch_conv<1, 2>(a, cap, st); break;
-    case 31: launch_conv<3, 1>(a, cap, st); break;
-    case 32: launch_conv<3, 2>(a, cap, st); break;
-    case 51: launch_conv<5, 1>(a, cap, st); break;
-    case 52: launch_conv<5, 2>(a, cap, st); break;
-    case 71: launch_conv<7, 1>(a, cap, st); break;
-    case 72: launch_conv<7, 2>(a, cap, st); break;
+    case 11: launch_conv<T, 1, 1>(a, cap, st); break;
+    case 12: launch_conv<T, 1, 2>(a, cap, st); break;
+    case 31: launch_conv<T, 3, 1>(a, cap, st); break;
+    case 32: launch_conv<T, 3, 2>(a, cap, st); break;
+    case 51: launch_conv<T, 5, 1>(a, cap, st); break;
+    case 52: launch_conv<T, 5, 2>(a, cap, st); break;
+    case 71: launch_conv<T, 7, 1>(a, cap, st); break;
+    case 72: launch_conv<T, 7, 2>(a, cap, st); break;
     default: MIE_REQUIRE(false, MIE_ERR_UNSUPPORTED, "%s: k=%d stride=%d", who, k, stride);
   }
   return mie_check_launch(who);
@@ -268,9 +273,12 @@ int conv_impl(const char* who, const float* x, const uint8_t* xmask, int c1, con
 
 }  // namespace
 
-// P[ci/8][tap][(ci%8)/4][co][ci%4] = F[ci][tap][co]
-__global__ __launch_bounds__(256) void k_pack_filter(const float* __restrict__ f,
-                                                     float* __restrict__ p, int cin, int kk, int cout) {
+// P[ci/B][tap][(ci%B)/(B/2)][co][ci%(B/2)] = F[ci][tap][co], B = 8 (fp32) or 16 (bf16) input
+// channels per block: the k-steps one MFMA lane multiplies for a tap are 16 contiguous bytes.
+template <typename T>
+__global__ __launch_bounds__(256) void k_pack_filter(const float* __restrict__ f, T* __restrict__ p,
+                                                     int cin, int kk, int cout) {
+  constexpr int B = 32 / (int)sizeof(T), HB = B / 2;
   const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
   const long long total = (long long)cin * kk * cout;
   if (i >= total) return;
@@ -278,55 +286,104 @@ __global__ __launch_bounds__(256) void k_pack_filter(const float* __restrict__ f
   const long long t = i / cout;
   const int tap = (int)(t % kk);
   const int ci = (int)(t / kk);
-  const long long o = ((((long long)(ci >> 3) * kk + tap) * 2 + ((ci & 7) >> 2)) * cout + co) * 4 + (ci & 3);
-  p[o] = f[i];
+  const long long o = ((((long long)(ci / B) * kk + tap) * 2 + (ci % B) / HB) * cout + co) * HB + (ci % HB);
+  mie_st(p, o, f[i]);
 }
 
-extern "C" int mie_pack_filter(const float* filter, int cin, int k, int cout, float* packed,
-                               void* stream) {
-  mie_clear_error();
-  const char* who = "mie_pack_filter";
-  MIE_REQUIRE(filter && packed, MIE_ERR_INVALID_ARG, "%s: NULL pointer", who);
-  MIE_REQUIRE(cin > 0 && k > 0 && cout > 0, MIE_ERR_INVALID_ARG, "%s: sizes must be positive", who);
-  MIE_REQUIRE(cin % 8 == 0, MIE_ERR_UNSUPPORTED, "%s: cin = %d is not a multiple of 8", who, cin);
-  MIE_REQUIRE(mie_aligned(filter, 16) && mie_aligned(packed, 16) && filter != packed,
-              MIE_ERR_INVALID_ARG, "%s: buffers must be 16-byte aligned and distinct", who);
-  const long long total = (long long)cin * k * k * cout;
-  MIE_REQUIRE(total < (1LL << 40), MIE_ERR_CAPACITY, "%s: filter too large", who);
-  hipLaunchKernelGGL(k_pack_filter, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
-                     (hipStream_t)stream, filter, packed, cin, k * k, cout);
+namespace {
+
+template <typename T>
+int tconv_impl(const char* who, const T* x, const uint8_t* xmask, int cin, int h_in, int w_in,
+               const float* filter, int k, int stride, int pad, int cout, const mie_tileset* out,
+               T* out_delta, float* reservoir, int act_kind, float slope, void* stream) {
+  ConvArgsT<T> a;
+  a.x = x; a.xm = xmask; a.c1 = cin; a.x2 = nullptr; a.x2m = nullptr; a.c2 = 0;
+  a.h_in = h_in; a.w_in = w_in; a.filt = filter; a.cin_total = cin; a.filt_mc = nullptr;
+  a.pad = pad; a.cout = cout; a.out = out_delta; a.res = reservoir; a.act = act_kind;
+  a.slope = slope; a.addend = nullptr; a.refresh = 0; a.bias = nullptr; a.ts = mie_dev_tileset(out);
+  const unsigned cap = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
+  hipLaunchKernelGGL(k_tconv_valu<T>, dim3(cap, mie_div_up(cout, 64)), dim3(256), 0,
+                     (hipStream_t)stream, a, k, stride);
   return mie_check_launch(who);
 }
 
-extern "C" int mie_conv_masked(const float* x, const uint8_t* xmask, int c1, const float* x2,
-                               const uint8_t* x2mask, int c2, int h_in, int w_in,
-                               const float* filter, const float* filter_mc, int cin_total, int k,
-                               int stride, int pad, int cout, const mie_tileset* out,
-                               float* out_delta, const float* addend, float* reservoir,
-                               int act_kind, float slope, int path, void* stream) {
-  return conv_impl("mie_conv_masked", x, xmask, c1, x2, x2mask, c2, h_in, w_in, filter, filter_mc,
-                   cin_total,
-                   k, stride, pad, cout, out, out_delta, addend, reservoir, act_kind, slope, path,
-                   false, nullptr, stream);
+}  // namespace
+
+#define MIE_CONV_DTYPE_OK(dtype, who)                                                     \
+  do {                                                                                    \
+    mie_clear_error();                                                                    \
+    MIE_REQUIRE((dtype) == MIE_DTYPE_F32 || (dtype) == MIE_DTYPE_BF16, MIE_ERR_UNSUPPORTED, \
+                "%s: unknown delta dtype %d", who, (int)(dtype));                         \
+  } while (0)
+
+extern "C" int mie_pack_filter(const float* filter, int cin, int k, int cout, void* packed,
+                               int dtype, void* stream) {
+  const char* who = "mie_pack_filter";
+  MIE_CONV_DTYPE_OK(dtype, who);
+  MIE_REQUIRE(filter && packed, MIE_ERR_INVALID_ARG, "%s: NULL pointer", who);
+  MIE_REQUIRE(cin > 0 && k > 0 && cout > 0, MIE_ERR_INVALID_ARG, "%s: sizes must be positive", who);
+  const int blk = dtype == MIE_DTYPE_BF16 ? 16 : 8;
+  MIE_REQUIRE(cin % blk == 0, MIE_ERR_UNSUPPORTED, "%s: cin = %d is not a multiple of %d", who, cin, blk);
+  MIE_REQUIRE(mie_aligned(filter, 16) && mie_aligned(packed, 16) && (const void*)filter != packed,
+              MIE_ERR_INVALID_ARG, "%s: buffers must be 16-byte aligned and distinct", who);
+  const long long total = (long long)cin * k * k * cout;
+  MIE_REQUIRE(total < (1LL << 40), MIE_ERR_CAPACITY, "%s: filter too large", who);
+  const dim3 grid((unsigned)((total + 255) / 256));
+  if (dtype == MIE_DTYPE_BF16)
+    hipLaunchKernelGGL(k_pack_filter<mie_bf16>, grid, dim3(256), 0, (hipStream_t)stream, filter,
+                       (mie_bf16*)packed, cin, k * k, cout);
+  else
+    hipLaunchKernelGGL(k_pack_filter<float>, grid, dim3(256), 0, (hipStream_t)stream, filter,
+                       (float*)packed, cin, k * k, cout);
+  return mie_check_launch(who);
 }
 
-extern "C" int mie_conv_refresh(const float* x, int c1, const float* x2, int c2, int h_in,
-                                int w_in, const float* filter, const float* filter_mc,
+extern "C" int mie_conv_masked(const void* x, const uint8_t* xmask, int c1, const void* x2,
+                               const uint8_t* x2mask, int c2, int h_in, int w_in,
+                               const float* filter, const void* filter_mc, int cin_total, int k,
+                               int stride, int pad, int cout, const mie_tileset* out,
+                               void* out_delta, const void* addend, float* reservoir,
+                               int act_kind, float slope, int path, int dtype, void* stream) {
+  const char* who = "mie_conv_masked";
+  MIE_CONV_DTYPE_OK(dtype, who);
+  if (dtype == MIE_DTYPE_BF16) {
+    typedef mie_bf16 T;
+    return conv_impl<T>(who, (const T*)x, xmask, c1, (const T*)x2, x2mask, c2, h_in, w_in, filter,
+                        (const T*)filter_mc, cin_total, k, stride, pad, cout, out, (T*)out_delta,
+                        (const T*)addend, reservoir, act_kind, slope, path, false, nullptr, stream);
+  }
+  typedef float T;
+  return conv_impl<T>(who, (const T*)x, xmask, c1, (const T*)x2, x2mask, c2, h_in, w_in, filter,
+                      (const T*)filter_mc, cin_total, k, stride, pad, cout, out, (T*)out_delta,
+                      (const T*)addend, reservoir, act_kind, slope, path, false, nullptr, stream);
+}
+
+extern "C" int mie_conv_refresh(const void* x, int c1, const void* x2, int c2, int h_in,
+                                int w_in, const float* filter, const void* filter_mc,
                                 int cin_total, int k, int stride, int pad, int cout,
                                 const float* bias, const mie_tileset* out,
-                                float* out_dense, const float* addend, float* reservoir,
-                                int act_kind, float slope, int path, void* stream) {
-  return conv_impl("mie_conv_refresh", x, nullptr, c1, x2, nullptr, c2, h_in, w_in, filter,
-                   filter_mc, cin_total, k, stride, pad, cout, out, out_dense, addend, reservoir, act_kind,
-                   slope, path, true, bias, stream);
+                                void* out_dense, const void* addend, float* reservoir,
+                                int act_kind, float slope, int path, int dtype, void* stream) {
+  const char* who = "mie_conv_refresh";
+  MIE_CONV_DTYPE_OK(dtype, who);
+  if (dtype == MIE_DTYPE_BF16) {
+    typedef mie_bf16 T;
+    return conv_impl<T>(who, (const T*)x, nullptr, c1, (const T*)x2, nullptr, c2, h_in, w_in, filter,
+                        (const T*)filter_mc, cin_total, k, stride, pad, cout, out, (T*)out_dense,
+                        (const T*)addend, reservoir, act_kind, slope, path, true, bias, stream);
+  }
+  typedef float T;
+  return conv_impl<T>(who, (const T*)x, nullptr, c1, (const T*)x2, nullptr, c2, h_in, w_in, filter,
+                      (const T*)filter_mc, cin_total, k, stride, pad, cout, out, (T*)out_dense,
+                      (const T*)addend, reservoir, act_kind, slope, path, true, bias, stream);
 }
 
-extern "C" int mie_tconv_masked(const float* x, const uint8_t* xmask, int cin, int h_in,
+extern "C" int mie_tconv_masked(const void* x, const uint8_t* xmask, int cin, int h_in,
                                 int w_in, const float* filter, int k, int stride, int pad,
-                                int cout, const mie_tileset* out, float* out_delta,
-                                float* reservoir, int act_kind, float slope, void* stream) {
-  mie_clear_error();
+                                int cout, const mie_tileset* out, void* out_delta,
+                                float* reservoir, int act_kind, float slope, int dtype, void* stream) {
   const char* who = "mie_tconv_masked";
+  MIE_CONV_DTYPE_OK(dtype, who);
   int rc = mie_check_tileset(out, who);
   if (rc != MIE_OK) return rc;
   MIE_REQUIRE(x != nullptr && filter != nullptr, MIE_ERR_INVALID_ARG, "%s: NULL pointer", who);
@@ -344,13 +401,9 @@ extern "C" int mie_tconv_masked(const float* x, const uint8_t* xmask, int cin, i
               "%s: x / filter must be 16-byte aligned", who);
   rc = check_epilogue(who, out_delta, reservoir, act_kind);
   if (rc != MIE_OK) return rc;
-  ConvArgs a;
-  a.x = x; a.xm = xmask; a.c1 = cin; a.x2 = nullptr; a.x2m = nullptr; a.c2 = 0;
-  a.h_in = h_in; a.w_in = w_in; a.filt = filter; a.cin_total = cin; a.filt_mc = nullptr;
-  a.pad = pad; a.cout = cout; a.out = out_delta; a.res = reservoir; a.act = act_kind;
-  a.slope = slope; a.addend = nullptr; a.refresh = 0; a.bias = nullptr; a.ts = mie_dev_tileset(out);
-  const unsigned cap = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
-  hipLaunchKernelGGL(k_tconv_valu, dim3(cap, mie_div_up(cout, 64)), dim3(256), 0,
-                     (hipStream_t)stream, a, k, stride);
-  return mie_check_launch(who);
+  if (dtype == MIE_DTYPE_BF16)
+    return tconv_impl<mie_bf16>(who, (const mie_bf16*)x, xmask, cin, h_in, w_in, filter, k, stride, pad,
+                                cout, out, (mie_bf16*)out_delta, reservoir, act_kind, slope, stream);
+  return tconv_impl<float>(who, (const float*)x, xmask, cin, h_in, w_in, filter, k, stride, pad, cout,
+                           out, (float*)out_delta, reservoir, act_kind, slope, stream);
 }

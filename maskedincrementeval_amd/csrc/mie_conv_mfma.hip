@@ -1,4 +1,8 @@
-// Masked conv on the fp32 matrix cores (v_mfma_f32_32x32x2_f32), gfx950.
+// Masked conv on the matrix cores, gfx950: fp32 deltas with v_mfma_f32_32x32x2_f32, bf16 deltas
+// with v_mfma_f32_32x32x16_bf16 (fp32 accumulation, fp32 reservoirs).  The two element types share
+// one kernel: every operand access is a 16-byte access, which holds 4 fp32 or 8 bf16 channels, so
+// the bf16 kernel is the fp32 kernel with twice the channels per LDS stage, per unit and per load.
+// The text below gives the fp32 numbers.
 //
 // Work decomposition.  One 256-thread workgroup (4 waves) computes one active
 // 8x8 output tile (M = 64 pixels) x CO_BLK output channels as an implicit GEMM
@@ -43,18 +47,35 @@ __host__ __device__ constexpr int ring_size(int upc) {
   return upc;
 }
 
-template <int K, int S, int WN, int NB>
-__global__ __launch_bounds__(256) void k_conv_mfma(ConvArgs a) {
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+// One unit of the contraction on the matrix core: the 16 bytes of A and of B a lane holds.
+__device__ __forceinline__ void mma_unit(v16f& acc, const float4& av, const float4& bv, float) {
+  acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.x, bv.x, acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.y, bv.y, acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.z, bv.z, acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.w, bv.w, acc, 0, 0, 0);
+}
+__device__ __forceinline__ void mma_unit(v16f& acc, const float4& av, const float4& bv, mie_bf16) {
+  const v4f a4 = {av.x, av.y, av.z, av.w}, b4 = {bv.x, bv.y, bv.z, bv.w};
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(mie_bf16x8, a4),
+                                                __builtin_bit_cast(mie_bf16x8, b4), acc, 0, 0, 0);
+}
+
+template <typename T, int K, int S, int WN, int NB>
+__global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
+  constexpr int EPS = 16 / (int)sizeof(T);                   // elements per 16-byte slot (4 / 8)
+  constexpr int SUB = 2 * EPS;                               // channels per unit (8 / 16)
   constexpr int WK = 4 / WN;
   constexpr int IT = 7 * S + K;                              // input tile edge incl. halo
-  constexpr int CC = stage_channels(K, S);                   // channels per LDS stage
-  constexpr int LS = CC + 4;                                 // LDS floats per staged pixel
+  constexpr int CC = stage_channels(K, S) * (4 / (int)sizeof(T));   // channels per LDS stage
+  constexpr int LS = CC + EPS;                               // LDS elements per staged pixel
   constexpr int NPIX = IT * IT;
-  constexpr int Q4 = CC / 4;                                 // float4 slots per pixel
+  constexpr int Q4 = CC / EPS;                               // 16-byte slots per pixel
   constexpr int NSLOT = NPIX * Q4;
   constexpr int NLD = (NSLOT + 255) / 256;                   // staging loads per thread
-  constexpr int STAGE = NPIX * LS;                           // floats per staging buffer
-  constexpr int NQ = CC / 8;                                 // 8-channel sub-chunks per stage
+  constexpr int STAGE = NPIX * LS;                           // elements per staging buffer
+  constexpr int NQ = CC / SUB;                               // sub-chunks (units per tap) per stage
   static_assert(NQ % WK == 0, "the k-split is over whole sub-chunks");
   constexpr int NQW = NQ / WK;                               // sub-chunks per wave
   constexpr int UPC = K * K * NQW;                           // units per chunk and wave
@@ -62,9 +83,11 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgs a) {
   constexpr int PD = RING - 1;                               // prefetch distance in units
   constexpr int CO_BLK = 32 * NB * WN;
   constexpr int RED = (WK > 1) ? WK * 64 * CO_BLK : 0;
-  constexpr int SMEM = (2 * STAGE > RED) ? 2 * STAGE : RED;
+  constexpr int STAGE_F = 2 * STAGE * (int)sizeof(T) / 4;     // both staging buffers, in floats
+  constexpr int SMEM = (STAGE_F > RED) ? STAGE_F : RED;
   static_assert(SMEM * 4 <= 65536, "LDS budget");
   __shared__ __attribute__((aligned(16))) float smem[SMEM];
+  T* const sbuf = reinterpret_cast<T*>(smem);
 
   int n, y0, x0;
   const int tk = mie_pick_tile(a.ts, blockIdx.x, n, y0, x0);
@@ -83,7 +106,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgs a) {
       const int p = idx / CO_BLK, col = idx - p * CO_BLK;
       const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
       if (oy < hout && ox < wout)
-        a.out[(((long long)n * hout + oy) * wout + ox) * cout + co0 + col] = 0.f;
+        mie_st(a.out, (((long long)n * hout + oy) * wout + ox) * cout + co0 + col, 0.f);
     }
     return;
   }
@@ -99,15 +122,15 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgs a) {
   // ---- per-thread staging plan: which pixels / float4 slots this thread copies -------------
   const int iy0 = y0 * S - a.pad, ix0 = x0 * S - a.pad;
   int st_po[NLD];       // linear input pixel index
-  int st_lds[NLD];      // LDS float offset of the slot
+  int st_lds[NLD];      // LDS element offset of the slot
   int st_c4[NLD];       // channel offset of the slot inside the chunk
   unsigned ok1 = 0u, ok2 = 0u;   // slot readable from x / x2 (inside the image, pixel mask set)
 #pragma unroll
   for (int i = 0; i < NLD; ++i) {
     const int slot = tid + 256 * i;
     const int pix = slot / Q4, q4 = slot - pix * Q4;
-    st_lds[i] = pix * LS + 4 * q4;
-    st_c4[i] = 4 * q4;
+    st_lds[i] = pix * LS + EPS * q4;
+    st_c4[i] = EPS * q4;
     st_po[i] = 0;
     if (slot < NSLOT) {
       const int iy = iy0 + pix / IT, ix = ix0 + pix % IT;
@@ -125,7 +148,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgs a) {
   float4 st_reg[NLD];
   auto stage_load = [&](int c) {
     const bool second = c >= nch1;
-    const float* xin = second ? a.x2 : a.x;
+    const T* xin = second ? a.x2 : a.x;
     const int cs = second ? a.c2 : a.c1;
     const int ci0 = (second ? c - nch1 : c) * CC;
     const unsigned ok = second ? ok2 : ok1;
@@ -134,11 +157,11 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgs a) {
     // global-memory latency of these loads).  Lanes whose pixel is masked or outside the image
     // all read one fixed, cache-resident address instead and get zeros selected afterwards,
     // so inactive pixels still cost no HBM traffic.
-    const float* dummy = a.filt;
+    const T* dummy = a.filt_mc;
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
       const bool okb = (ok >> i) & 1u;
-      const float* p = xin + (long long)st_po[i] * cs + ci0 + st_c4[i];
+      const T* p = xin + (long long)st_po[i] * cs + ci0 + st_c4[i];
       p = okb ? p : dummy;
       float4 v = *reinterpret_cast<const float4*>(p);
       v.x = okb ? v.x : 0.f; v.y = okb ? v.y : 0.f; v.z = okb ? v.z : 0.f; v.w = okb ? v.w : 0.f;
@@ -146,7 +169,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgs a) {
     }
   };
   auto stage_store = [&](int buf) {
-    float* dst = smem + buf * STAGE;
+    T* dst = sbuf + buf * STAGE;
 #pragma unroll
     for (int i = 0; i < NLD; ++i)
       if (tid + 256 * i < NSLOT) *reinterpret_cast<float4*>(dst + st_lds[i]) = st_reg[i];
@@ -159,38 +182,36 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgs a) {
   // cout (B) or a compile-time LDS offset (A); the lane-dependent parts are loop invariant.
   const int q0w = wk * NQW;
   const int cob0 = co0 + wn * (32 * NB);                       // first column of this wave
-  const int b_lane = (half * cout + l32) * 4;                  // lane part of the packed filter index
+  const int b_lane = (half * cout + l32) * EPS;                // lane part of the packed filter index
   int a_lane[2];                                               // lane part of the LDS index
 #pragma unroll
   for (int mb = 0; mb < 2; ++mb) {
     const int p = mb * 32 + l32;
-    a_lane[mb] = (((p >> 3) * S) * IT + (p & 7) * S) * LS + 8 * q0w + 4 * half;
+    a_lane[mb] = (((p >> 3) * S) * IT + (p & 7) * S) * LS + SUB * q0w + EPS * half;
   }
   // filter row block of chunk c for this wave (c1 and c2 are multiples of CC: no partial chunks)
-  auto chunk_b = [&](int c) -> const float* {
+  auto chunk_b = [&](int c) -> const T* {
     const bool second = c >= nch1;
     const int ci0 = (second ? c - nch1 : c) * CC;
     const int fb = second ? a.c1 : 0;
-    return a.filt_mc + ((long long)((fb + ci0) / 8 + q0w) * (K * K) * 2 * cout + cob0) * 4;
+    return a.filt_mc + ((long long)((fb + ci0) / SUB + q0w) * (K * K) * 2 * cout + cob0) * EPS;
   };
-  // Matrix-core filter copy: P[ci/8][tap][(ci%8)/4][co][ci%4].  The four k-steps of a unit are
-  // one 16-byte load per lane, 512 contiguous bytes per half wave.
-  float bring[RING][NB][4];
-  auto load_b = [&](const float* ub, int unit, float (&bv)[NB][4]) {
+  // Matrix-core filter copy: P[ci/8][tap][(ci%8)/4][co][ci%4] (fp32; 16 / 8 / 8 for bf16).  The
+  // k-steps of a unit are one 16-byte load per lane, 512 contiguous bytes per half wave.
+  float4 bring[RING][NB];
+  auto load_b = [&](const T* ub, int unit, float4 (&bv)[NB]) {
     const int tap = unit / NQW, qi = unit % NQW;     // compile-time after unrolling
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-      const float4 v = *reinterpret_cast<const float4*>(
-          ub + ((long long)((qi * (K * K) + tap) * 2) * cout + nb * 32) * 4 + b_lane);
-      bv[nb][0] = v.x; bv[nb][1] = v.y; bv[nb][2] = v.z; bv[nb][3] = v.w;
-    }
+    for (int nb = 0; nb < NB; ++nb)
+      bv[nb] = *reinterpret_cast<const float4*>(
+          ub + ((long long)((qi * (K * K) + tap) * 2) * cout + nb * 32) * EPS + b_lane);
   };
 
   // All B loads below are unconditional: a conditional load would make the compiler's wait
   // counters conservative and collapse the prefetch distance.  After the last chunk the
   // "next chunk" pointer simply stays on the current one (a few redundant loads).
-  const float* ub_cur = chunk_b(0);
-  const float* ub_next = ub_cur;
+  const T* ub_cur = chunk_b(0);
+  const T* ub_next = ub_cur;
   stage_load(0);
 #pragma unroll
   for (int i = 0; i < (PD > 0 ? PD : 1); ++i) load_b(ub_cur, i, bring[i % RING]);
@@ -202,7 +223,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgs a) {
     const int cn = more ? c + 1 : c;      // after the last chunk: redundant re-load, never stored
     ub_next = chunk_b(cn);
     stage_load(cn);
-    const float* sin = smem + (c & 1) * STAGE;
+    const T* sin = sbuf + (c & 1) * STAGE;
     // A operands are read one unit ahead as well (two register sets); the scheduling barriers
     // pin "issue the loads for later units, then multiply this unit" so that the compiler can
     // neither sink the prefetches next to their uses nor hoist them all to the top.
@@ -212,7 +233,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgs a) {
       const int ky = tap / K, kx = tap - ky * K;
 #pragma unroll
       for (int mb = 0; mb < 2; ++mb)
-        dst[mb] = *reinterpret_cast<const float4*>(&sin[a_lane[mb] + (ky * IT + kx) * LS + 8 * qi]);
+        dst[mb] = *reinterpret_cast<const float4*>(&sin[a_lane[mb] + (ky * IT + kx) * LS + SUB * qi]);
     };
     load_a(0, av[0]);
 #pragma unroll
@@ -226,13 +247,9 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgs a) {
       if (i + 1 < UPC) load_a(i + 1, av[(i + 1) & 1]);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+      for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-          for (int mb = 0; mb < 2; ++mb)
-            acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x2f32((&av[i & 1][mb].x)[j], bring[i % RING][nb][j],
-                                                               acc[mb][nb], 0, 0, 0);
+        for (int mb = 0; mb < 2; ++mb) mma_unit(acc[mb][nb], av[i & 1][mb], bring[i % RING][nb], T());
       __builtin_amdgcn_sched_barrier(0);
       if (PD == 0) load_b(ub_next, 0, bring[0]);   // ring of one: reload right after use
     }
@@ -285,27 +302,27 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgs a) {
 // Launch with the widest channel slab that still gives the chip enough workgroups (256 CUs;
 // aim for >= 2 workgroups per CU when every tile is active), among the wave splits the
 // staging depth of this (K, S) allows.
-template <int K, int S>
-bool launch_ks(const ConvArgs& a, unsigned cap, hipStream_t st) {
+template <typename T, int K, int S>
+bool launch_ks(const ConvArgsT<T>& a, unsigned cap, hipStream_t st) {
   constexpr int NQ = stage_channels(K, S) / 8;
   const long long want = 512;
   const int cout = a.cout;
   if (cout % 256 == 0 && (long long)cap * (cout / 256) >= want) {
-    hipLaunchKernelGGL((k_conv_mfma<K, S, 4, 2>), dim3(cap, cout / 256), dim3(256), 0, st, a);
+    hipLaunchKernelGGL((k_conv_mfma<T, K, S, 4, 2>), dim3(cap, cout / 256), dim3(256), 0, st, a);
     return true;
   }
   if (cout % 128 == 0 && ((long long)cap * (cout / 128) >= want || NQ < 2 || cout % 64 != 0)) {
-    hipLaunchKernelGGL((k_conv_mfma<K, S, 4, 1>), dim3(cap, cout / 128), dim3(256), 0, st, a);
+    hipLaunchKernelGGL((k_conv_mfma<T, K, S, 4, 1>), dim3(cap, cout / 128), dim3(256), 0, st, a);
     return true;
   }
   if constexpr (NQ >= 2) {
     if (cout % 64 == 0 && ((long long)cap * (cout / 64) >= want || NQ < 4)) {
-      hipLaunchKernelGGL((k_conv_mfma<K, S, 2, 1>), dim3(cap, cout / 64), dim3(256), 0, st, a);
+      hipLaunchKernelGGL((k_conv_mfma<T, K, S, 2, 1>), dim3(cap, cout / 64), dim3(256), 0, st, a);
       return true;
     }
   }
   if constexpr (NQ >= 4) {
-    hipLaunchKernelGGL((k_conv_mfma<K, S, 1, 1>), dim3(cap, cout / 32), dim3(256), 0, st, a);
+    hipLaunchKernelGGL((k_conv_mfma<T, K, S, 1, 1>), dim3(cap, cout / 32), dim3(256), 0, st, a);
     return true;
   }
   return false;
@@ -313,24 +330,37 @@ bool launch_ks(const ConvArgs& a, unsigned cap, hipStream_t st) {
 
 }  // namespace
 
-// Smallest output-channel multiple the matrix-core path takes for (k, s).
-int mie_conv_mfma_cin_multiple(int k, int s) { return stage_channels(k, s); }
+// Input channels staged per chunk: c1 and c2 must be multiples of it.
+int mie_conv_mfma_cin_multiple(int k, int s, int dtype) {
+  return stage_channels(k, s) * (dtype == MIE_DTYPE_BF16 ? 2 : 1);
+}
 
+// Smallest output-channel multiple the matrix-core path takes for (k, s).
 int mie_conv_mfma_cout_multiple(int k, int s) {
   const int nq = stage_channels(k, s) / 8;
   return nq >= 4 ? 32 : (nq >= 2 ? 64 : 128);
 }
 
-bool mie_launch_conv_mfma(const ConvArgs& a, int k, int s, unsigned cap, hipStream_t st) {
+namespace {
+template <typename T>
+bool launch_any(const ConvArgsT<T>& a, int k, int s, unsigned cap, hipStream_t st) {
   switch (k * 10 + s) {
-    case 11: return launch_ks<1, 1>(a, cap, st);
-    case 12: return launch_ks<1, 2>(a, cap, st);
-    case 31: return launch_ks<3, 1>(a, cap, st);
-    case 32: return launch_ks<3, 2>(a, cap, st);
-    case 51: return launch_ks<5, 1>(a, cap, st);
-    case 52: return launch_ks<5, 2>(a, cap, st);
-    case 71: return launch_ks<7, 1>(a, cap, st);
-    case 72: return launch_ks<7, 2>(a, cap, st);
+    case 11: return launch_ks<T, 1, 1>(a, cap, st);
+    case 12: return launch_ks<T, 1, 2>(a, cap, st);
+    case 31: return launch_ks<T, 3, 1>(a, cap, st);
+    case 32: return launch_ks<T, 3, 2>(a, cap, st);
+    case 51: return launch_ks<T, 5, 1>(a, cap, st);
+    case 52: return launch_ks<T, 5, 2>(a, cap, st);
+    case 71: return launch_ks<T, 7, 1>(a, cap, st);
+    case 72: return launch_ks<T, 7, 2>(a, cap, st);
     default: return false;
   }
+}
+}  // namespace
+
+bool mie_launch_conv_mfma(const ConvArgsT<float>& a, int k, int s, unsigned cap, hipStream_t st) {
+  return launch_any<float>(a, k, s, cap, st);
+}
+bool mie_launch_conv_mfma(const ConvArgsT<mie_bf16>& a, int k, int s, unsigned cap, hipStream_t st) {
+  return launch_any<mie_bf16>(a, k, s, cap, st);
 }

@@ -51,29 +51,36 @@ int mie_check_tileset(const mie_tileset* ts, const char* who) {
 // ---- mask from delta ----------------------------------------------------------
 // One thread per pixel walks its channel vector; C is small (<= 1024) and the
 // vector is contiguous, float4 when the row is 16-byte aligned.
+template <typename T>
 __global__ __launch_bounds__(256) void k_mask_from_delta(
-    const float* __restrict__ delta, long long npix, int c, float thr,
+    const T* __restrict__ delta, long long npix, int c, float thr,
     uint8_t* __restrict__ pixmask) {
   const long long p = (long long)blockIdx.x * 256 + threadIdx.x;
   if (p >= npix) return;
-  const float* row = delta + p * c;
+  const T* row = delta + p * c;
   int any = 0;
-  if ((c & 3) == 0) {
-    const float4* r4 = reinterpret_cast<const float4*>(row);
-    for (int i = 0; i < (c >> 2); ++i) {
-      const float4 v = r4[i];
-      any |= (fabsf(v.x) > thr) | (fabsf(v.y) > thr) | (fabsf(v.z) > thr) | (fabsf(v.w) > thr);
+  if constexpr (sizeof(T) == 4) {
+    if ((c & 3) == 0) {
+      const float4* r4 = reinterpret_cast<const float4*>(row);
+      for (int i = 0; i < (c >> 2); ++i) {
+        const float4 v = r4[i];
+        any |= (fabsf(v.x) > thr) | (fabsf(v.y) > thr) | (fabsf(v.z) > thr) | (fabsf(v.w) > thr);
+      }
+    } else {
+      for (int i = 0; i < c; ++i) any |= (fabsf(mie_ld(row, i)) > thr);
     }
   } else {
-    for (int i = 0; i < c; ++i) any |= (fabsf(row[i]) > thr);
+    for (int i = 0; i < c; ++i) any |= (fabsf(mie_ld(row, i)) > thr);
   }
   pixmask[p] = (uint8_t)any;
 }
 
-extern "C" int mie_mask_from_delta(const float* delta, int n, int h, int w, int c,
-                                   float threshold, uint8_t* pixmask, void* stream) {
+extern "C" int mie_mask_from_delta(const void* delta, int n, int h, int w, int c,
+                                   float threshold, uint8_t* pixmask, int dtype, void* stream) {
   mie_clear_error();
   MIE_REQUIRE(delta && pixmask, MIE_ERR_INVALID_ARG, "mie_mask_from_delta: NULL pointer");
+  MIE_REQUIRE(dtype == MIE_DTYPE_F32 || dtype == MIE_DTYPE_BF16, MIE_ERR_UNSUPPORTED,
+              "mie_mask_from_delta: unknown delta dtype %d", dtype);
   MIE_REQUIRE(n > 0 && h > 0 && w > 0 && c > 0, MIE_ERR_INVALID_ARG,
               "mie_mask_from_delta: sizes must be positive (n=%d h=%d w=%d c=%d)", n, h, w, c);
   MIE_REQUIRE(threshold >= 0.f, MIE_ERR_INVALID_ARG, "mie_mask_from_delta: threshold < 0");
@@ -82,8 +89,12 @@ extern "C" int mie_mask_from_delta(const float* delta, int n, int h, int w, int 
   const long long npix = (long long)n * h * w;
   MIE_REQUIRE(npix < 0x7fffffffLL, MIE_ERR_CAPACITY, "mie_mask_from_delta: too many pixels");
   const unsigned blocks = (unsigned)((npix + 255) / 256);
-  hipLaunchKernelGGL(k_mask_from_delta, dim3(blocks), dim3(256), 0, (hipStream_t)stream,
-                     delta, npix, c, threshold, pixmask);
+  if (dtype == MIE_DTYPE_BF16)
+    hipLaunchKernelGGL(k_mask_from_delta<mie_bf16>, dim3(blocks), dim3(256), 0, (hipStream_t)stream,
+                       (const mie_bf16*)delta, npix, c, threshold, pixmask);
+  else
+    hipLaunchKernelGGL(k_mask_from_delta<float>, dim3(blocks), dim3(256), 0, (hipStream_t)stream,
+                       (const float*)delta, npix, c, threshold, pixmask);
   return mie_check_launch("mie_mask_from_delta");
 }
 

@@ -13,6 +13,15 @@ template <> struct Vec<4> {
   float4 v;
   __device__ static Vec load(const float* p) { Vec r; r.v = *reinterpret_cast<const float4*>(p); return r; }
   __device__ void store(float* p) const { *reinterpret_cast<float4*>(p) = v; }
+  // bf16 deltas: 4 values = one 8-byte access, widened to / rounded from fp32 (nearest even)
+  __device__ static Vec load(const mie_bf16* p) {
+    const mie_bf16x4 b = *reinterpret_cast<const mie_bf16x4*>(p);
+    Vec r; r.v = make_float4((float)b[0], (float)b[1], (float)b[2], (float)b[3]); return r;
+  }
+  __device__ void store(mie_bf16* p) const {
+    mie_bf16x4 b; b[0] = (mie_bf16)v.x; b[1] = (mie_bf16)v.y; b[2] = (mie_bf16)v.z; b[3] = (mie_bf16)v.w;
+    *reinterpret_cast<mie_bf16x4*>(p) = b;
+  }
   __device__ static Vec zero() { Vec r; r.v = make_float4(0.f, 0.f, 0.f, 0.f); return r; }
   __device__ float& operator[](int i) { return (&v.x)[i]; }
 };
@@ -20,6 +29,8 @@ template <> struct Vec<1> {
   float v;
   __device__ static Vec load(const float* p) { Vec r; r.v = *p; return r; }
   __device__ void store(float* p) const { *p = v; }
+  __device__ static Vec load(const mie_bf16* p) { Vec r; r.v = (float)*p; return r; }
+  __device__ void store(mie_bf16* p) const { *p = (mie_bf16)v; }
   __device__ static Vec zero() { Vec r; r.v = 0.f; return r; }
   __device__ float& operator[](int) { return v; }
 };
@@ -57,11 +68,11 @@ static inline unsigned channel_splits(int cap, int cv) {
 }
 
 // ---- activation increment -----------------------------------------------------
-template <int VEC>
+template <typename T, int VEC>
 __global__ __launch_bounds__(256) void k_act_incr(TileSetDev ts, int kind, float slope,
-                                                  const float* __restrict__ din,
+                                                  const T* __restrict__ din,
                                                   float* __restrict__ res,
-                                                  float* __restrict__ dout, int c,
+                                                  T* __restrict__ dout, int c,
                                                   uint8_t* __restrict__ out_mask, int keep) {
   __shared__ unsigned s_any[64];
   int n, y0, x0;
@@ -109,11 +120,11 @@ __global__ __launch_bounds__(256) void k_act_incr(TileSetDev ts, int kind, float
 // t = carry + d;  f = k * floor(0.5 + t / k);  carry = t - f;  out = f.  Every operation is a
 // separately rounded IEEE fp32 op (no contraction, true division), so the result equals the
 // same expression evaluated op by op on the host.
-template <int VEC>
+template <typename T, int VEC>
 __global__ __launch_bounds__(256) void k_kfence_incr(TileSetDev ts, const float* __restrict__ k_dev,
-                                                     float k_host, const float* __restrict__ din,
+                                                     float k_host, const T* __restrict__ din,
                                                      float* __restrict__ carry,
-                                                     float* __restrict__ dout, int c,
+                                                     T* __restrict__ dout, int c,
                                                      uint8_t* __restrict__ out_mask) {
   __shared__ unsigned s_any[64];
   int n, y0, x0;
@@ -160,14 +171,14 @@ __global__ __launch_bounds__(256) void k_kfence_incr(TileSetDev ts, const float*
 }
 
 // ---- product rule ---------------------------------------------------------------
-template <int VEC>
-__global__ __launch_bounds__(256) void k_mul_incr(TileSetDev ts, const float* __restrict__ d1,
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void k_mul_incr(TileSetDev ts, const T* __restrict__ d1,
                                                   const uint8_t* __restrict__ m1,
                                                   float* __restrict__ r1,
-                                                  const float* __restrict__ d2,
+                                                  const T* __restrict__ d2,
                                                   const uint8_t* __restrict__ m2,
                                                   float* __restrict__ r2,
-                                                  float* __restrict__ dout, int c, int keep) {
+                                                  T* __restrict__ dout, int c, int keep) {
   int n, y0, x0;
   const int tk = mie_pick_tile(ts, blockIdx.x, n, y0, x0);
   if (tk == 0) return;
@@ -198,12 +209,12 @@ __global__ __launch_bounds__(256) void k_mul_incr(TileSetDev ts, const float* __
 }
 
 // ---- sum ----------------------------------------------------------------------------
-template <int VEC>
-__global__ __launch_bounds__(256) void k_add_incr(TileSetDev ts, const float* __restrict__ a,
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void k_add_incr(TileSetDev ts, const T* __restrict__ a,
                                                   const uint8_t* __restrict__ ma,
-                                                  const float* __restrict__ b,
+                                                  const T* __restrict__ b,
                                                   const uint8_t* __restrict__ mb,
-                                                  float* __restrict__ dout, int c) {
+                                                  T* __restrict__ dout, int c) {
   int n, y0, x0;
   const int tk = mie_pick_tile(ts, blockIdx.x, n, y0, x0);
   if (tk == 0) return;
@@ -238,12 +249,12 @@ __device__ __forceinline__ void up2x_coef(int o, int in_size, int& i0, int& i1, 
   }
 }
 
-template <int VEC>
-__global__ __launch_bounds__(256) void k_up2x_incr(TileSetDev ts, const float* __restrict__ a,
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void k_up2x_incr(TileSetDev ts, const T* __restrict__ a,
                                                    const uint8_t* __restrict__ ma,
-                                                   const float* __restrict__ b,
+                                                   const T* __restrict__ b,
                                                    const uint8_t* __restrict__ mb, int h_in,
-                                                   int w_in, float* __restrict__ dout, int c) {
+                                                   int w_in, T* __restrict__ dout, int c) {
   int n, y0, x0;
   const int tk = mie_pick_tile(ts, blockIdx.x, n, y0, x0);
   if (tk == 0) return;
@@ -286,11 +297,11 @@ __global__ __launch_bounds__(256) void k_up2x_incr(TileSetDev ts, const float* _
 // ---- fused ConvLSTM gates ------------------------------------------------------
 __device__ __forceinline__ float sigm(float v) { return 1.f / (1.f + expf(-v)); }
 
-template <int VEC>
+template <typename T, int VEC>
 __global__ __launch_bounds__(256) void k_convlstm_gates(
-    TileSetDev ts, const float* __restrict__ dg, float* __restrict__ gres,
-    const float* __restrict__ dcp, const uint8_t* __restrict__ mcp, float* __restrict__ cpres,
-    float* __restrict__ cres, float* __restrict__ dh, float* __restrict__ dc, int hid) {
+    TileSetDev ts, const T* __restrict__ dg, float* __restrict__ gres,
+    const T* __restrict__ dcp, const uint8_t* __restrict__ mcp, float* __restrict__ cpres,
+    float* __restrict__ cres, T* __restrict__ dh, T* __restrict__ dc, int hid) {
   int n, y0, x0;
   const int tk = mie_pick_tile(ts, blockIdx.x, n, y0, x0);
   if (tk == 0) return;
@@ -349,15 +360,39 @@ int check_pointwise(const char* who, const mie_tileset* ts, int c) {
 #define MIE_PTR16(p, who, name) \
   MIE_REQUIRE(mie_aligned((p), 16), MIE_ERR_INVALID_ARG, "%s: %s must be 16-byte aligned", who, name)
 
+// Launches KERN<T, VEC> with T from `dtype` and VEC = 4 when c % 4 == 0, else 1.  The kernel
+// arguments are built by ARGS, a macro-local expression list that may use T.
+#define MIE_LAUNCH_POINTWISE(KERN, dtype, c, grid, ny4, ny1, stream, ...)                                   \
+  do {                                                                                                    \
+    if ((dtype) == MIE_DTYPE_BF16) {                                                                      \
+      using T = mie_bf16;                                                                                 \
+      if (((c) & 3) == 0)                                                                                 \
+        hipLaunchKernelGGL((KERN<T, 4>), dim3(grid, ny4), dim3(256), 0, (hipStream_t)(stream), __VA_ARGS__); \
+      else                                                                                                \
+        hipLaunchKernelGGL((KERN<T, 1>), dim3(grid, ny1), dim3(256), 0, (hipStream_t)(stream), __VA_ARGS__); \
+    } else {                                                                                              \
+      using T = float;                                                                                    \
+      if (((c) & 3) == 0)                                                                                 \
+        hipLaunchKernelGGL((KERN<T, 4>), dim3(grid, ny4), dim3(256), 0, (hipStream_t)(stream), __VA_ARGS__); \
+      else                                                                                                \
+        hipLaunchKernelGGL((KERN<T, 1>), dim3(grid, ny1), dim3(256), 0, (hipStream_t)(stream), __VA_ARGS__); \
+    }                                                                                                     \
+  } while (0)
+
+#define MIE_DTYPE_OK(dtype, who)                                                                      \
+  MIE_REQUIRE((dtype) == MIE_DTYPE_F32 || (dtype) == MIE_DTYPE_BF16, MIE_ERR_UNSUPPORTED,              \
+              "%s: unknown delta dtype %d", who, (int)(dtype))
+
 }  // namespace
 
-extern "C" int mie_act_incr(int act_kind, float slope, const float* in_delta, float* reservoir,
-                            float* out_delta, int c, const mie_tileset* ts,
-                            uint8_t* out_pixmask, int flags, void* stream) {
+extern "C" int mie_act_incr(int act_kind, float slope, const void* in_delta, float* reservoir,
+                            void* out_delta, int c, const mie_tileset* ts,
+                            uint8_t* out_pixmask, int flags, int dtype, void* stream) {
   mie_clear_error();
   const char* who = "mie_act_incr";
   int rc = check_pointwise(who, ts, c);
   if (rc != MIE_OK) return rc;
+  MIE_DTYPE_OK(dtype, who);
   MIE_REQUIRE(in_delta && reservoir && out_delta, MIE_ERR_INVALID_ARG, "%s: NULL pointer", who);
   MIE_REQUIRE(act_kind >= MIE_ACT_NONE && act_kind <= MIE_ACT_TANH, MIE_ERR_UNSUPPORTED,
               "%s: unknown activation %d", who, act_kind);
@@ -368,24 +403,21 @@ extern "C" int mie_act_incr(int act_kind, float slope, const float* in_delta, fl
   const unsigned grid = (unsigned)mie_tile_capacity(ts->n, ts->h, ts->w);
   // the refined mask is an any-over-channels inside one block: no channel split then
   const unsigned ny = out_pixmask ? 1u : channel_splits((int)grid, (c & 3) ? c : c / 4);
-  if ((c & 3) == 0)
-    hipLaunchKernelGGL(k_act_incr<4>, dim3(grid, ny), dim3(256), 0, (hipStream_t)stream, d, act_kind,
-                       slope, in_delta, reservoir, out_delta, c, out_pixmask, keep);
-  else
-    hipLaunchKernelGGL(k_act_incr<1>, dim3(grid, ny), dim3(256), 0, (hipStream_t)stream, d, act_kind,
-                       slope, in_delta, reservoir, out_delta, c, out_pixmask, keep);
+  MIE_LAUNCH_POINTWISE(k_act_incr, dtype, c, grid, ny, ny, stream, d, act_kind, slope, (const T*)in_delta,
+                       reservoir, (T*)out_delta, c, out_pixmask, keep);
   return mie_check_launch(who);
 }
 
-extern "C" int mie_kfence_incr(const float* in_delta, float* carry, const float* k_dev, float k_host,
-                               float* out_delta, int c, const mie_tileset* ts,
-                               uint8_t* out_pixmask, void* stream) {
+extern "C" int mie_kfence_incr(const void* in_delta, float* carry, const float* k_dev, float k_host,
+                               void* out_delta, int c, const mie_tileset* ts,
+                               uint8_t* out_pixmask, int dtype, void* stream) {
   mie_clear_error();
   const char* who = "mie_kfence_incr";
   int rc = check_pointwise(who, ts, c);
   if (rc != MIE_OK) return rc;
+  MIE_DTYPE_OK(dtype, who);
   MIE_REQUIRE(in_delta && carry && out_delta, MIE_ERR_INVALID_ARG, "%s: NULL pointer", who);
-  MIE_REQUIRE(carry != in_delta && carry != out_delta, MIE_ERR_INVALID_ARG,
+  MIE_REQUIRE((const void*)carry != in_delta && (void*)carry != out_delta, MIE_ERR_INVALID_ARG,
               "%s: the carry must not alias a delta", who);
   MIE_REQUIRE(k_dev != nullptr || (k_host > 0.f && k_host < INFINITY), MIE_ERR_INVALID_ARG,
               "%s: k = %g must be positive and finite", who, (double)k_host);
@@ -395,63 +427,56 @@ extern "C" int mie_kfence_incr(const float* in_delta, float* carry, const float*
   const TileSetDev d = mie_dev_tileset(ts);
   const unsigned grid = (unsigned)mie_tile_capacity(ts->n, ts->h, ts->w);
   const unsigned ny = out_pixmask ? 1u : channel_splits((int)grid, (c & 3) ? c : c / 4);
-  if ((c & 3) == 0)
-    hipLaunchKernelGGL(k_kfence_incr<4>, dim3(grid, ny), dim3(256), 0, (hipStream_t)stream, d, k_dev,
-                       k_host, in_delta, carry, out_delta, c, out_pixmask);
-  else
-    hipLaunchKernelGGL(k_kfence_incr<1>, dim3(grid, ny), dim3(256), 0, (hipStream_t)stream, d, k_dev,
-                       k_host, in_delta, carry, out_delta, c, out_pixmask);
+  MIE_LAUNCH_POINTWISE(k_kfence_incr, dtype, c, grid, ny, ny, stream, d, k_dev, k_host, (const T*)in_delta,
+                       carry, (T*)out_delta, c, out_pixmask);
   return mie_check_launch(who);
 }
 
-extern "C" int mie_mul_incr(const float* d1, const uint8_t* m1, float* r1, const float* d2,
-                            const uint8_t* m2, float* r2, float* out_delta, int c,
-                            const mie_tileset* ts, int flags, void* stream) {
+extern "C" int mie_mul_incr(const void* d1, const uint8_t* m1, float* r1, const void* d2,
+                            const uint8_t* m2, float* r2, void* out_delta, int c,
+                            const mie_tileset* ts, int flags, int dtype, void* stream) {
   mie_clear_error();
   const char* who = "mie_mul_incr";
   int rc = check_pointwise(who, ts, c);
   if (rc != MIE_OK) return rc;
+  MIE_DTYPE_OK(dtype, who);
   MIE_REQUIRE(d1 && r1 && d2 && r2 && out_delta, MIE_ERR_INVALID_ARG, "%s: NULL pointer", who);
   MIE_PTR16(d1, who, "d1"); MIE_PTR16(r1, who, "r1"); MIE_PTR16(d2, who, "d2");
   MIE_PTR16(r2, who, "r2"); MIE_PTR16(out_delta, who, "out_delta");
   const int keep = (flags & MIE_FLAG_KEEP_RESERVOIR) ? 1 : 0;
   const TileSetDev d = mie_dev_tileset(ts);
   const unsigned grid = (unsigned)mie_tile_capacity(ts->n, ts->h, ts->w);
-  if ((c & 3) == 0)
-    hipLaunchKernelGGL(k_mul_incr<4>, dim3(grid, channel_splits((int)grid, c / 4)), dim3(256), 0, (hipStream_t)stream, d, d1, m1, r1,
-                       d2, m2, r2, out_delta, c, keep);
-  else
-    hipLaunchKernelGGL(k_mul_incr<1>, dim3(grid, channel_splits((int)grid, c)), dim3(256), 0, (hipStream_t)stream, d, d1, m1, r1,
-                       d2, m2, r2, out_delta, c, keep);
+  MIE_LAUNCH_POINTWISE(k_mul_incr, dtype, c, grid, channel_splits((int)grid, c / 4),
+                       channel_splits((int)grid, c), stream, d, (const T*)d1, m1, r1, (const T*)d2, m2, r2,
+                       (T*)out_delta, c, keep);
   return mie_check_launch(who);
 }
 
-extern "C" int mie_add_incr(const float* a, const uint8_t* ma, const float* b, const uint8_t* mb,
-                            float* out_delta, int c, const mie_tileset* ts, void* stream) {
+extern "C" int mie_add_incr(const void* a, const uint8_t* ma, const void* b, const uint8_t* mb,
+                            void* out_delta, int c, const mie_tileset* ts, int dtype, void* stream) {
   mie_clear_error();
   const char* who = "mie_add_incr";
   int rc = check_pointwise(who, ts, c);
   if (rc != MIE_OK) return rc;
+  MIE_DTYPE_OK(dtype, who);
   MIE_REQUIRE(a && b && out_delta, MIE_ERR_INVALID_ARG, "%s: NULL pointer", who);
   MIE_PTR16(a, who, "a"); MIE_PTR16(b, who, "b"); MIE_PTR16(out_delta, who, "out_delta");
   const TileSetDev d = mie_dev_tileset(ts);
   const unsigned grid = (unsigned)mie_tile_capacity(ts->n, ts->h, ts->w);
-  if ((c & 3) == 0)
-    hipLaunchKernelGGL(k_add_incr<4>, dim3(grid, channel_splits((int)grid, c / 4)), dim3(256), 0, (hipStream_t)stream, d, a, ma, b,
-                       mb, out_delta, c);
-  else
-    hipLaunchKernelGGL(k_add_incr<1>, dim3(grid, channel_splits((int)grid, c)), dim3(256), 0, (hipStream_t)stream, d, a, ma, b,
-                       mb, out_delta, c);
+  MIE_LAUNCH_POINTWISE(k_add_incr, dtype, c, grid, channel_splits((int)grid, c / 4),
+                       channel_splits((int)grid, c), stream, d, (const T*)a, ma, (const T*)b, mb,
+                       (T*)out_delta, c);
   return mie_check_launch(who);
 }
 
-extern "C" int mie_upsample2x_incr(const float* a, const uint8_t* ma, const float* b,
+extern "C" int mie_upsample2x_incr(const void* a, const uint8_t* ma, const void* b,
                                    const uint8_t* mb, int h_in, int w_in, int c,
-                                   const mie_tileset* out, float* out_delta, void* stream) {
+                                   const mie_tileset* out, void* out_delta, int dtype, void* stream) {
   mie_clear_error();
   const char* who = "mie_upsample2x_incr";
   int rc = check_pointwise(who, out, c);
   if (rc != MIE_OK) return rc;
+  MIE_DTYPE_OK(dtype, who);
   MIE_REQUIRE(a && out_delta, MIE_ERR_INVALID_ARG, "%s: NULL pointer", who);
   MIE_REQUIRE(b != nullptr || mb == nullptr, MIE_ERR_INVALID_ARG, "%s: mask of absent input b", who);
   MIE_REQUIRE(h_in > 0 && w_in > 0 && out->h == 2 * h_in && out->w == 2 * w_in,
@@ -460,24 +485,22 @@ extern "C" int mie_upsample2x_incr(const float* a, const uint8_t* ma, const floa
   MIE_PTR16(a, who, "a"); MIE_PTR16(b, who, "b"); MIE_PTR16(out_delta, who, "out_delta");
   const TileSetDev d = mie_dev_tileset(out);
   const unsigned grid = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
-  if ((c & 3) == 0)
-    hipLaunchKernelGGL(k_up2x_incr<4>, dim3(grid, channel_splits((int)grid, c / 4)), dim3(256), 0, (hipStream_t)stream, d, a, ma, b,
-                       mb, h_in, w_in, out_delta, c);
-  else
-    hipLaunchKernelGGL(k_up2x_incr<1>, dim3(grid, channel_splits((int)grid, c)), dim3(256), 0, (hipStream_t)stream, d, a, ma, b,
-                       mb, h_in, w_in, out_delta, c);
+  MIE_LAUNCH_POINTWISE(k_up2x_incr, dtype, c, grid, channel_splits((int)grid, c / 4),
+                       channel_splits((int)grid, c), stream, d, (const T*)a, ma, (const T*)b, mb, h_in, w_in,
+                       (T*)out_delta, c);
   return mie_check_launch(who);
 }
 
-extern "C" int mie_convlstm_gates_incr(const float* gates_delta, float* gates_res,
-                                       const float* cprev_delta, const uint8_t* cprev_mask,
-                                       float* cprev_res, float* cell_res, float* h_delta,
-                                       float* c_delta, int hid, const mie_tileset* ts,
+extern "C" int mie_convlstm_gates_incr(const void* gates_delta, float* gates_res,
+                                       const void* cprev_delta, const uint8_t* cprev_mask,
+                                       float* cprev_res, float* cell_res, void* h_delta,
+                                       void* c_delta, int hid, const mie_tileset* ts, int dtype,
                                        void* stream) {
   mie_clear_error();
   const char* who = "mie_convlstm_gates_incr";
   int rc = check_pointwise(who, ts, hid);
   if (rc != MIE_OK) return rc;
+  MIE_DTYPE_OK(dtype, who);
   MIE_REQUIRE(gates_delta && gates_res && cprev_res && cell_res && h_delta && c_delta,
               MIE_ERR_INVALID_ARG, "%s: NULL pointer", who);
   MIE_REQUIRE(cprev_delta != nullptr || cprev_mask == nullptr, MIE_ERR_INVALID_ARG,
@@ -488,13 +511,8 @@ extern "C" int mie_convlstm_gates_incr(const float* gates_delta, float* gates_re
   MIE_PTR16(c_delta, who, "c_delta");
   const TileSetDev d = mie_dev_tileset(ts);
   const unsigned grid = (unsigned)mie_tile_capacity(ts->n, ts->h, ts->w);
-  if ((hid & 3) == 0)
-    hipLaunchKernelGGL(k_convlstm_gates<4>, dim3(grid, channel_splits((int)grid, hid / 4)), dim3(256), 0, (hipStream_t)stream, d,
-                       gates_delta, gates_res, cprev_delta, cprev_mask, cprev_res, cell_res,
-                       h_delta, c_delta, hid);
-  else
-    hipLaunchKernelGGL(k_convlstm_gates<1>, dim3(grid, channel_splits((int)grid, hid)), dim3(256), 0, (hipStream_t)stream, d,
-                       gates_delta, gates_res, cprev_delta, cprev_mask, cprev_res, cell_res,
-                       h_delta, c_delta, hid);
+  MIE_LAUNCH_POINTWISE(k_convlstm_gates, dtype, hid, grid, channel_splits((int)grid, hid / 4),
+                       channel_splits((int)grid, hid), stream, d, (const T*)gates_delta, gates_res,
+                       (const T*)cprev_delta, cprev_mask, cprev_res, cell_res, (T*)h_delta, (T*)c_delta, hid);
   return mie_check_launch(who);
 }

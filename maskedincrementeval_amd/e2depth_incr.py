@@ -127,8 +127,8 @@ class ConvLSTMIncr(nn.Module, _IncrBuffers):
         gates, ts = self.Gates(input_incr, prev_h_incr)
         n, _, h, w = gates.shape
         hid = self.hidden_size
-        dh = self._delta_buf("h", (n, hid, h, w), gates.device)
-        dc = self._delta_buf("c", (n, hid, h, w), gates.device)
+        dh = self._delta_buf("h", (n, hid, h, w), gates.device, gates.dtype)
+        dc = self._delta_buf("c", (n, hid, h, w), gates.device, gates.dtype)
         cp = cpm = None
         if prev_c_incr is not None:
             cp, cpm, _ = _unpack(prev_c_incr)
@@ -147,7 +147,7 @@ class ConvLSTMIncr(nn.Module, _IncrBuffers):
         cell = self.m1(in_gate, cell_gate)
         if prev_c_incr is None:
             # d(f * c_prev) with dc_prev = 0 is df * c_prev: the product rule with a zero delta
-            zero = self._delta_buf("zero_c", tuple(cell[0].shape), cell[0].device)
+            zero = self._delta_buf("zero_c", tuple(cell[0].shape), cell[0].device, cell[0].dtype)
             prev_c_incr = [zero, remember_gate[1]]
         cell = self.add_cell(cell, self.m2(remember_gate, prev_c_incr))
         cell_tanh = self.tanh2(cell)

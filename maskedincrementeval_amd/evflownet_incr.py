@@ -319,7 +319,7 @@ class UpsampleConvLayerIncr(nn.Module):
         n, _, h, w = x.shape
         ho, wo = ops.conv_out_size(h, w, k, s, p)
         ts = self._lead._tile_set("lead", n, ho, wo, x.device)
-        out = self._lead._delta_buf("lead", (n, self.conv2d.out_channels, ho, wo), x.device)
+        out = self._lead._delta_buf("lead", (n, self.conv2d.out_channels, ho, wo), x.device, x.dtype)
         ops.build_mask_tiles(pix, None, n, h, w, _lib.FOOT_CONV, k, s, p, ts)
         ops.conv_masked(x, pix, None, None, filt, k, s, p, ts, out)
         return [out, ts]

@@ -60,6 +60,8 @@ class IncrementReserve:
 
     def update_reservoir(self, x: DenseT):
         x = x.detach()
+        if x.dtype == torch.bfloat16:       # reservoirs stay fp32 when the deltas are bf16
+            x = x.float()
         if (self.reservoir is not None and self.reservoir.shape == x.shape
                 and self.reservoir.device == x.device and self.reservoir.dtype == x.dtype):
             self.reservoir.copy_(x)
@@ -102,7 +104,7 @@ def IncrPointwiseMultiply(x1_incr: Masked, x1: IncrementReserve, x2_incr: Masked
     else:
         ts = TileMask(n, h, w, d1.device)
         ops.build_mask_tiles(p1, p2, n, h, w, _lib.FOOT_CONV, 1, 1, 0, ts)
-    out = ops.new_nhwc(n, c, h, w, d1.device)
+    out = ops.new_nhwc(n, c, h, w, d1.device, d1.dtype)
     ops.mul_incr(d1, p1, x1.reservoir, d2, p2, x2.reservoir, out, ts, keep_reservoir=True)
     return [out, ts]
 
@@ -126,7 +128,7 @@ def conv2d_from_module(x: Masked, conv_weights, stride=(1, 1), padding=(1, 1)) -
     ho, wo = ops.conv_out_size(h, w, k, s, p)
     ts = TileMask(n, ho, wo, delta.device)
     ops.build_mask_tiles(pix, None, n, h, w, _lib.FOOT_CONV, k, s, p, ts)
-    out = ops.new_nhwc(n, conv_weights.shape[3], ho, wo, delta.device)
+    out = ops.new_nhwc(n, conv_weights.shape[3], ho, wo, delta.device, delta.dtype)
     ops.conv_masked(delta, pix, None, None, conv_weights, k, s, p, ts, out)
     return [out, ts]
 
@@ -144,7 +146,7 @@ def transposed_conv2d_from_module(x: Masked, gates: nn.ConvTranspose2d, bias=Tru
     filt = gates.weight.detach().permute(0, 2, 3, 1).contiguous()   # [Cin,K,K,Cout]
     ts = TileMask(n, ho, wo, delta.device)
     ops.build_mask_tiles(pix, None, n, h, w, _lib.FOOT_TCONV, k, s, p, ts)
-    out = ops.new_nhwc(n, filt.shape[3], ho, wo, delta.device)
+    out = ops.new_nhwc(n, filt.shape[3], ho, wo, delta.device, delta.dtype)
     ops.tconv_masked(delta, pix, filt, k, s, p, ts, out)
     return [out, ts]
 
@@ -167,6 +169,6 @@ def interpolate_from_module(x: Masked) -> Masked:
     n, c, h, w = delta.shape
     ts = TileMask(n, 2 * h, 2 * w, delta.device)
     ops.build_mask_tiles(pix, None, n, h, w, _lib.FOOT_UP2X, 0, 0, 0, ts)
-    out = ops.new_nhwc(n, c, 2 * h, 2 * w, delta.device)
+    out = ops.new_nhwc(n, c, 2 * h, 2 * w, delta.device, delta.dtype)
     ops.upsample2x_incr(delta, pix, None, None, ts, out)
     return [out, ts]

@@ -40,11 +40,11 @@ class _IncrBuffers:
             self.__dict__["_incr_bufs"] = d
         return d
 
-    def _delta_buf(self, name, shape, device) -> torch.Tensor:
-        key = ("d", name, tuple(shape), str(device))
+    def _delta_buf(self, name, shape, device, dtype=torch.float32) -> torch.Tensor:
+        key = ("d", name, tuple(shape), str(device), dtype)
         b = self._ib().get(key)
         if b is None:
-            b = ops.new_nhwc(*shape, device)
+            b = ops.new_nhwc(*shape, device, dtype)
             self._ib()[key] = b
         return b
 
@@ -82,12 +82,12 @@ class _IncrBuffers:
             self._ib()[key] = b
         return b
 
-    def _dense_buf(self, name, shape, device) -> torch.Tensor:
+    def _dense_buf(self, name, shape, device, dtype=torch.float32) -> torch.Tensor:
         """Persistent dense output of the refresh pass (not touched by `_reset_incr`)."""
-        key = ("D", name, tuple(shape), str(device))
+        key = ("D", name, tuple(shape), str(device), dtype)
         b = self._ib().get(key)
         if b is None:
-            b = ops.new_nhwc(*shape, device)
+            b = ops.new_nhwc(*shape, device, dtype)
             self._ib()[key] = b
         return b
 
@@ -138,7 +138,7 @@ class KFencedMaskModule(IncrementMaskModule):
         else:
             ts = self._tile_set("own", n, h, w, d.device)
             ops.build_mask_tiles(ops.pixel_mask_of(mask, d), None, n, h, w, _lib.FOOT_CONV, 1, 1, 0, ts)
-        out = self._delta_buf("out", (n, c, h, w), d.device)
+        out = self._delta_buf("out", (n, c, h, w), d.device, d.dtype)
         pix = self._pix_buf("refined", n, h, w, d.device)
         ops.kfence_incr(d, self.delta.reservoir, self.k, out, ts, pix)
         return [out, self._view("refined", ts, pix)]
@@ -152,7 +152,7 @@ class KFencedMaskModule(IncrementMaskModule):
         if self.delta.reservoir is not None and self.delta.reservoir.shape == x.shape:
             self.delta.reservoir.zero_()
         else:
-            self.delta.update_reservoir(torch.zeros_like(x))
+            self.delta.update_reservoir(torch.zeros_like(x, dtype=torch.float32))
         self._reset_incr()
         return x
 
@@ -189,7 +189,7 @@ class nnReservedMultiplication(PointwiseMultiplyIncr):
         else:
             ts = self._tile_set("union", n, h, w, d1.device)
             ops.build_mask_tiles(p1, p2, n, h, w, _lib.FOOT_CONV, 1, 1, 0, ts)
-        out = self._delta_buf("out", (n, c, h, w), d1.device)
+        out = self._delta_buf("out", (n, c, h, w), d1.device, d1.dtype)
         ops.mul_incr(d1, p1, self.x1_res.reservoir, d2, p2, self.x2_res.reservoir, out, ts)
         return [out, ts]
 
@@ -258,7 +258,7 @@ class NonlinearPointOpIncr(IncrementMaskModule):
         else:
             ts = self._tile_set("own", n, h, w, d.device)
             ops.build_mask_tiles(ops.pixel_mask_of(mask, d), None, n, h, w, _lib.FOOT_CONV, 1, 1, 0, ts)
-        out = self._delta_buf("out", (n, c, h, w), d.device)
+        out = self._delta_buf("out", (n, c, h, w), d.device, d.dtype)
         if self.refine_mask:
             pix = self._pix_buf("refined", n, h, w, d.device)
             ops.act_incr(kind, slope, d, res, out, ts, pix, keep_reservoir=keep_reservoir)
@@ -315,7 +315,7 @@ class _ConvIncrMixin(_IncrBuffers):
             x2, pix2, _ = _unpack(x2_incr)
         n, _, h, w = x.shape
         ho, wo = ops.conv_out_size(h, w, k, s, p)
-        out = self._delta_buf(out_name, (n, self.out_channels, ho, wo), x.device)
+        out = self._delta_buf(out_name, (n, self.out_channels, ho, wo), x.device, x.dtype)
         in_tm = x_incr[1] if len(x_incr) > 1 else None
         if k == 1 and s == 1 and p == 0 and x2 is None and isinstance(in_tm, TileMask):
             ts = in_tm            # a 1x1 conv reaches exactly the pixels of its input: same tile set
@@ -359,7 +359,7 @@ class _ConvIncrMixin(_IncrBuffers):
         ts = self._dense_tile_set(n, ho, wo, x.device)
         shape = (n, self.out_channels, ho, wo)
         if out is None:
-            out = self._dense_buf("refresh_out", shape, x.device)
+            out = self._dense_buf("refresh_out", shape, x.device, x.dtype)
         res, kind, slope = None, _lib.ACT_NONE, 0.0
         if activation is not None:
             kind, slope = activation_kind(activation.op)
@@ -472,7 +472,7 @@ class nnConvTranspose2dIncr(nn.ConvTranspose2d, _IncrBuffers):
         n, _, h, w = x.shape
         ho, wo = (h - 1) * s - 2 * p + k + op, (w - 1) * s - 2 * p + k + op
         ts = self._tile_set("out", n, ho, wo, x.device)
-        out = self._delta_buf("out", (n, self.out_channels, ho, wo), x.device)
+        out = self._delta_buf("out", (n, self.out_channels, ho, wo), x.device, x.dtype)
         ops.build_mask_tiles(pix, None, n, h, w, _lib.FOOT_TCONV, k, s, p, ts)
         ops.tconv_masked(x, pix, self._filter(), k, s, p, ts, out, reservoir, act, slope)
         return [out, ts]
@@ -579,7 +579,7 @@ class nnAddIncr(IncrementMaskModule):
         else:
             ts = self._tile_set("union", n, h, w, a.device)
             ops.build_mask_tiles(pa, pb, n, h, w, _lib.FOOT_CONV, 1, 1, 0, ts)
-        out = self._delta_buf("out", (n, c, h, w), a.device)
+        out = self._delta_buf("out", (n, c, h, w), a.device, a.dtype)
         ops.add_incr(a, pa, b, pb, out, ts)
         return [out, ts]
 
@@ -604,7 +604,7 @@ class nnUpsample2xIncr(IncrementMaskModule):
         else:
             m1, m2 = pa, pb
         ops.build_mask_tiles(m1, m2, n, h, w, _lib.FOOT_UP2X, 0, 0, 0, ts)
-        out = self._delta_buf("out", (n, c, 2 * h, 2 * w), a.device)
+        out = self._delta_buf("out", (n, c, 2 * h, 2 * w), a.device, a.dtype)
         ops.upsample2x_incr(a, pa, b, pb, ts, out)
         return [out, ts]
 

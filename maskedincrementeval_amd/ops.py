@@ -85,13 +85,24 @@ def _require_gpu(t: torch.Tensor, name: str):
                            % (name, t.device))
 
 
-def nhwc_ptr(t: Optional[torch.Tensor], name: str, c: Optional[int] = None):
-    """Device pointer of an (N,C,H,W) fp32 tensor stored channels_last; None -> NULL."""
+_DTYPES = {torch.float32: _lib.DTYPE_F32, torch.bfloat16: _lib.DTYPE_BF16}
+
+
+def delta_dtype(t: torch.Tensor) -> int:
+    """MIE_DTYPE_* code of a delta tensor (fp32 or bf16; reservoirs are always fp32)."""
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise ValueError("deltas must be float32 or bfloat16, got %s" % t.dtype) from None
+
+
+def nhwc_ptr(t: Optional[torch.Tensor], name: str, c: Optional[int] = None, dtype=torch.float32):
+    """Device pointer of an (N,C,H,W) tensor of `dtype` stored channels_last; None -> NULL."""
     if t is None:
         return None
     _require_gpu(t, name)
-    if t.dim() != 4 or t.dtype != torch.float32:
-        raise ValueError("%s must be a 4-D float32 tensor, got %s %s" % (name, tuple(t.shape), t.dtype))
+    if t.dim() != 4 or t.dtype != dtype:
+        raise ValueError("%s must be a 4-D %s tensor, got %s %s" % (name, dtype, tuple(t.shape), t.dtype))
     if not t.permute(0, 2, 3, 1).is_contiguous():
         raise ValueError("%s must be channels_last (NHWC in memory); strides %s" % (name, t.stride()))
     if c is not None and t.shape[1] != c:
@@ -100,8 +111,8 @@ def nhwc_ptr(t: Optional[torch.Tensor], name: str, c: Optional[int] = None):
 
 
 def as_nhwc(t: torch.Tensor) -> torch.Tensor:
-    """Return t as fp32 channels_last (copies only if the layout / dtype differs)."""
-    if t.dtype != torch.float32:
+    """Return t as channels_last fp32 (bf16 stays bf16); copies only if the layout / dtype differs."""
+    if t.dtype not in _DTYPES:
         t = t.float()
     if not t.permute(0, 2, 3, 1).is_contiguous():
         t = t.contiguous(memory_format=torch.channels_last)
@@ -110,9 +121,9 @@ def as_nhwc(t: torch.Tensor) -> torch.Tensor:
     return t
 
 
-def new_nhwc(n, c, h, w, device) -> torch.Tensor:
-    """Zero-filled (N,C,H,W) fp32 tensor with NHWC storage."""
-    return torch.zeros((n, h, w, c), dtype=torch.float32, device=device).permute(0, 3, 1, 2)
+def new_nhwc(n, c, h, w, device, dtype=torch.float32) -> torch.Tensor:
+    """Zero-filled (N,C,H,W) tensor with NHWC storage."""
+    return torch.zeros((n, h, w, c), dtype=dtype, device=device).permute(0, 3, 1, 2)
 
 
 def pix_ptr(m, n, h, w, name):
@@ -145,8 +156,8 @@ def pixel_mask_of(mask, like: torch.Tensor) -> Optional[torch.Tensor]:
 # ---- entry points ----------------------------------------------------------------
 def mask_from_delta(delta: torch.Tensor, threshold: float, out: torch.Tensor):
     n, c, h, w = delta.shape
-    check(lib().mie_mask_from_delta(nhwc_ptr(delta, "delta"), n, h, w, c, float(threshold),
-                                    pix_ptr(out, n, h, w, "out"), _stream(delta)))
+    check(lib().mie_mask_from_delta(nhwc_ptr(delta, "delta", dtype=delta.dtype), n, h, w, c, float(threshold),
+                                    pix_ptr(out, n, h, w, "out"), delta_dtype(delta), _stream(delta)))
     _mark_pix(out)
     return out
 
@@ -181,26 +192,41 @@ def build_mask_tiles(in_mask, in_mask2, n, h_in, w_in, foot, k, stride, pad, out
     return out
 
 
-def pack_filter(filt: torch.Tensor) -> torch.Tensor:
-    """Matrix-core copy of a contiguous fp32 [Cin,K,K,Cout] filter (Cin % 8 == 0), shape
-    [Cin/8, K*K, 2, Cout, 4]: element [b,t,h,co,j] is filt[8b+4h+j, t//K, t%K, co]."""
+def pack_filter(filt: torch.Tensor, dtype=torch.float32) -> torch.Tensor:
+    """Matrix-core copy of a contiguous fp32 [Cin,K,K,Cout] filter in `dtype`, shape
+    [Cin/B, K*K, 2, Cout, B/2] with B = 8 (fp32) or 16 (bf16) input channels per block:
+    element [b,t,h,co,j] is filt[B*b + (B/2)*h + j, t//K, t%K, co]."""
     if filt.dim() != 4 or filt.shape[1] != filt.shape[2] or not filt.is_contiguous() or filt.dtype != torch.float32:
         raise ValueError("filter must be contiguous fp32 [Cin,K,K,Cout], got %s" % (tuple(filt.shape),))
     _require_gpu(filt, "filter")
     cin, k, _, cout = filt.shape
-    packed = torch.empty((cin // 8, k * k, 2, cout, 4), dtype=torch.float32, device=filt.device)
-    check(lib().mie_pack_filter(filt.data_ptr(), cin, k, cout, packed.data_ptr(), _stream(filt)))
+    blk = 8 if dtype == torch.float32 else 16
+    packed = torch.empty((cin // blk, k * k, 2, cout, blk // 2), dtype=dtype, device=filt.device)
+    check(lib().mie_pack_filter(filt.data_ptr(), cin, k, cout, packed.data_ptr(), _DTYPES[dtype], _stream(filt)))
     return packed
 
 
 class ConvFilter:
     """A conv filter as the kernels take it: `plain` [Cin,K,K,Cout] and, when Cin % 8 == 0, `mc`,
-    its matrix-core copy (pack_filter).  Make a new one after every weight update."""
+    its matrix-core copy (pack_filter).  For bf16 deltas `for_dtype(torch.bfloat16)` gives the
+    weights rounded to bf16: as fp32 values for the VALU kernels and as the bf16 matrix-core copy
+    (Cin % 16 == 0), both made on first use.  Make a new ConvFilter after every weight update."""
 
     def __init__(self, plain: torch.Tensor, mc: Optional[torch.Tensor] = None, _packed: bool = False):
         self.plain = plain
         self.mc = mc if _packed else (pack_filter(plain) if plain.is_cuda and plain.shape[0] % 8 == 0 else None)
         self._rows = {}
+        self._bf16 = None
+
+    def for_dtype(self, dtype):
+        """(plain fp32 tensor, matrix-core copy | None) for deltas of `dtype`."""
+        if dtype == torch.float32:
+            return self.plain, self.mc
+        if self._bf16 is None:
+            rounded = self.plain.to(torch.bfloat16).float().contiguous()
+            mc = pack_filter(rounded, torch.bfloat16) if rounded.is_cuda and rounded.shape[0] % 16 == 0 else None
+            self._bf16 = (rounded, mc)
+        return self._bf16
 
     @property
     def shape(self):
@@ -220,11 +246,11 @@ class ConvFilter:
         return sub
 
 
-def _filter_args(filt, k):
+def _filter_args(filt, k, dtype=torch.float32):
     """(plain tensor, pointer of the matrix-core copy or None) of a Tensor or ConvFilter."""
     mc = None
     if isinstance(filt, ConvFilter):
-        filt, mc = filt.plain, filt.mc
+        filt, mc = filt.for_dtype(dtype)
     if filt.dim() != 4 or filt.shape[1] != k or filt.shape[2] != k or not filt.is_contiguous() \
             or filt.dtype != torch.float32:
         raise ValueError("filter must be contiguous fp32 [Cin,%d,%d,Cout], got %s" % (k, k, tuple(filt.shape)))
@@ -239,7 +265,8 @@ def conv_masked(x, xmask, x2, x2mask, filt, k, stride, pad, out_ts: TileMask, ou
     c2 = 0 if x2 is None else x2.shape[1]
     if x2 is not None and (x2.shape[0] != n or x2.shape[2:] != x.shape[2:]):
         raise ValueError("x2 shape %s incompatible with x %s" % (tuple(x2.shape), tuple(x.shape)))
-    filt, mc_ptr = _filter_args(filt, k)
+    dt = x.dtype
+    filt, mc_ptr = _filter_args(filt, k, dt)
     cin_total, cout = filt.shape[0], filt.shape[3]
     if tuple(out_delta.shape) != (n, cout, out_ts.h, out_ts.w) or out_ts.n != n:
         raise ValueError("out_delta shape %s, expected %s" % (tuple(out_delta.shape), (n, cout, out_ts.h, out_ts.w)))
@@ -249,11 +276,11 @@ def conv_masked(x, xmask, x2, x2mask, filt, k, stride, pad, out_ts: TileMask, ou
         raise ValueError("addend shape %s != output %s" % (tuple(addend.shape), tuple(out_delta.shape)))
     _ready(out_ts)
     check(lib().mie_conv_masked(
-        nhwc_ptr(x, "x"), pix_ptr(xmask, n, h, w, "xmask"), c1,
-        nhwc_ptr(x2, "x2"), pix_ptr(x2mask, n, h, w, "x2mask"), c2, h, w,
+        nhwc_ptr(x, "x", dtype=dt), pix_ptr(xmask, n, h, w, "xmask"), c1,
+        nhwc_ptr(x2, "x2", dtype=dt), pix_ptr(x2mask, n, h, w, "x2mask"), c2, h, w,
         filt.data_ptr(), mc_ptr, cin_total, k, stride, pad, cout, out_ts.ref,
-        nhwc_ptr(out_delta, "out_delta"), nhwc_ptr(addend, "addend", cout), nhwc_ptr(reservoir, "reservoir"),
-        act, float(slope), path, _stream(x)))
+        nhwc_ptr(out_delta, "out_delta", dtype=dt), nhwc_ptr(addend, "addend", cout, dtype=dt),
+        nhwc_ptr(reservoir, "reservoir"), act, float(slope), path, delta_dtype(x), _stream(x)))
     return out_delta
 
 
@@ -262,7 +289,8 @@ def conv_refresh(x, x2, filt, bias, k, stride, pad, out_ts: TileMask, out_dense,
     """Dense conv + bias (+ activation, + reservoir fill) over the tiles of out_ts (all active)."""
     n, c1, h, w = x.shape
     c2 = 0 if x2 is None else x2.shape[1]
-    filt, mc_ptr = _filter_args(filt, k)
+    dt = x.dtype
+    filt, mc_ptr = _filter_args(filt, k, dt)
     cin_total, cout = filt.shape[0], filt.shape[3]
     if tuple(out_dense.shape) != (n, cout, out_ts.h, out_ts.w):
         raise ValueError("out_dense shape %s, expected %s" % (tuple(out_dense.shape), (n, cout, out_ts.h, out_ts.w)))
@@ -270,10 +298,10 @@ def conv_refresh(x, x2, filt, bias, k, stride, pad, out_ts: TileMask, out_dense,
         raise ValueError("bias must be contiguous fp32 of %d elements" % cout)
     _ready(out_ts)
     check(lib().mie_conv_refresh(
-        nhwc_ptr(x, "x"), c1, nhwc_ptr(x2, "x2"), c2, h, w, filt.data_ptr(), mc_ptr, cin_total, k, stride,
-        pad, cout, None if bias is None else bias.data_ptr(), out_ts.ref, nhwc_ptr(out_dense, "out_dense"),
-        nhwc_ptr(addend, "addend", cout), nhwc_ptr(reservoir, "reservoir"), act, float(slope), path,
-        _stream(x)))
+        nhwc_ptr(x, "x", dtype=dt), c1, nhwc_ptr(x2, "x2", dtype=dt), c2, h, w, filt.data_ptr(), mc_ptr,
+        cin_total, k, stride, pad, cout, None if bias is None else bias.data_ptr(), out_ts.ref,
+        nhwc_ptr(out_dense, "out_dense", dtype=dt), nhwc_ptr(addend, "addend", cout, dtype=dt),
+        nhwc_ptr(reservoir, "reservoir"), act, float(slope), path, delta_dtype(x), _stream(x)))
     return out_dense
 
 
@@ -289,9 +317,9 @@ def tconv_masked(x, xmask, filt, k, stride, pad, out_ts: TileMask, out_delta, re
         raise ValueError("out_delta shape %s" % (tuple(out_delta.shape),))
     _ready(out_ts)
     check(lib().mie_tconv_masked(
-        nhwc_ptr(x, "x"), pix_ptr(xmask, n, h, w, "xmask"), cin, h, w, filt.data_ptr(), k, stride,
-        pad, cout, out_ts.ref, nhwc_ptr(out_delta, "out_delta"), nhwc_ptr(reservoir, "reservoir"),
-        act, float(slope), _stream(x)))
+        nhwc_ptr(x, "x", dtype=x.dtype), pix_ptr(xmask, n, h, w, "xmask"), cin, h, w, filt.data_ptr(), k, stride,
+        pad, cout, out_ts.ref, nhwc_ptr(out_delta, "out_delta", dtype=x.dtype), nhwc_ptr(reservoir, "reservoir"),
+        act, float(slope), delta_dtype(x), _stream(x)))
     return out_delta
 
 
@@ -308,10 +336,11 @@ def act_incr(kind, slope, in_delta, reservoir, out_delta, ts: TileMask, out_pixm
     if (ts.n, ts.h, ts.w) != (n, h, w):
         raise ValueError("tile set %s does not match delta %s" % ((ts.n, ts.h, ts.w), (n, h, w)))
     _ready(ts)
-    check(lib().mie_act_incr(kind, float(slope), nhwc_ptr(in_delta, "in_delta"),
-                             nhwc_ptr(reservoir, "reservoir"), nhwc_ptr(out_delta, "out_delta"), c,
+    dt = in_delta.dtype
+    check(lib().mie_act_incr(kind, float(slope), nhwc_ptr(in_delta, "in_delta", dtype=dt),
+                             nhwc_ptr(reservoir, "reservoir"), nhwc_ptr(out_delta, "out_delta", dtype=dt), c,
                              ts.ref, pix_ptr(out_pixmask, n, h, w, "out_pixmask"),
-                             _lib.FLAG_KEEP_RESERVOIR if keep_reservoir else 0,
+                             _lib.FLAG_KEEP_RESERVOIR if keep_reservoir else 0, delta_dtype(in_delta),
                              _stream(in_delta)))
     _mark_pix(out_pixmask)
     return out_delta
@@ -332,9 +361,11 @@ def kfence_incr(in_delta, carry, k, out_delta, ts: TileMask, out_pixmask=None):
     else:
         k_dev, k_host = None, float(k)
     _ready(ts)
-    check(lib().mie_kfence_incr(nhwc_ptr(in_delta, "in_delta"), nhwc_ptr(carry, "carry"), k_dev, k_host,
-                                nhwc_ptr(out_delta, "out_delta"), c, ts.ref,
-                                pix_ptr(out_pixmask, n, h, w, "out_pixmask"), _stream(in_delta)))
+    dt = in_delta.dtype
+    check(lib().mie_kfence_incr(nhwc_ptr(in_delta, "in_delta", dtype=dt), nhwc_ptr(carry, "carry"), k_dev, k_host,
+                                nhwc_ptr(out_delta, "out_delta", dtype=dt), c, ts.ref,
+                                pix_ptr(out_pixmask, n, h, w, "out_pixmask"), delta_dtype(in_delta),
+                                _stream(in_delta)))
     _mark_pix(out_pixmask)
     return out_delta
 
@@ -344,10 +375,11 @@ def mul_incr(d1, m1, r1, d2, m2, r2, out_delta, ts: TileMask, keep_reservoir=Fal
     for name, t in (("r1", r1), ("d2", d2), ("r2", r2), ("out_delta", out_delta)):
         _same_shape(name, t, d1)
     _ready(ts)
-    check(lib().mie_mul_incr(nhwc_ptr(d1, "d1"), pix_ptr(m1, n, h, w, "m1"), nhwc_ptr(r1, "r1"),
-                             nhwc_ptr(d2, "d2"), pix_ptr(m2, n, h, w, "m2"), nhwc_ptr(r2, "r2"),
-                             nhwc_ptr(out_delta, "out_delta"), c, ts.ref,
-                             _lib.FLAG_KEEP_RESERVOIR if keep_reservoir else 0, _stream(d1)))
+    dt = d1.dtype
+    check(lib().mie_mul_incr(nhwc_ptr(d1, "d1", dtype=dt), pix_ptr(m1, n, h, w, "m1"), nhwc_ptr(r1, "r1"),
+                             nhwc_ptr(d2, "d2", dtype=dt), pix_ptr(m2, n, h, w, "m2"), nhwc_ptr(r2, "r2"),
+                             nhwc_ptr(out_delta, "out_delta", dtype=dt), c, ts.ref,
+                             _lib.FLAG_KEEP_RESERVOIR if keep_reservoir else 0, delta_dtype(d1), _stream(d1)))
     return out_delta
 
 
@@ -356,9 +388,10 @@ def add_incr(a, ma, b, mb, out_delta, ts: TileMask):
     _same_shape("b", b, a)
     _same_shape("out_delta", out_delta, a)
     _ready(ts)
-    check(lib().mie_add_incr(nhwc_ptr(a, "a"), pix_ptr(ma, n, h, w, "ma"), nhwc_ptr(b, "b"),
-                             pix_ptr(mb, n, h, w, "mb"), nhwc_ptr(out_delta, "out_delta"), c,
-                             ts.ref, _stream(a)))
+    dt = a.dtype
+    check(lib().mie_add_incr(nhwc_ptr(a, "a", dtype=dt), pix_ptr(ma, n, h, w, "ma"), nhwc_ptr(b, "b", dtype=dt),
+                             pix_ptr(mb, n, h, w, "mb"), nhwc_ptr(out_delta, "out_delta", dtype=dt), c,
+                             ts.ref, delta_dtype(a), _stream(a)))
     return out_delta
 
 
@@ -369,9 +402,11 @@ def upsample2x_incr(a, ma, b, mb, out_ts: TileMask, out_delta):
     if tuple(out_delta.shape) != (n, c, 2 * h, 2 * w):
         raise ValueError("out_delta shape %s, expected %s" % (tuple(out_delta.shape), (n, c, 2 * h, 2 * w)))
     _ready(out_ts)
-    check(lib().mie_upsample2x_incr(nhwc_ptr(a, "a"), pix_ptr(ma, n, h, w, "ma"),
-                                    nhwc_ptr(b, "b"), pix_ptr(mb, n, h, w, "mb"), h, w, c,
-                                    out_ts.ref, nhwc_ptr(out_delta, "out_delta"), _stream(a)))
+    dt = a.dtype
+    check(lib().mie_upsample2x_incr(nhwc_ptr(a, "a", dtype=dt), pix_ptr(ma, n, h, w, "ma"),
+                                    nhwc_ptr(b, "b", dtype=dt), pix_ptr(mb, n, h, w, "mb"), h, w, c,
+                                    out_ts.ref, nhwc_ptr(out_delta, "out_delta", dtype=dt), delta_dtype(a),
+                                    _stream(a)))
     return out_delta
 
 
@@ -387,12 +422,13 @@ def convlstm_gates_incr(gates_delta, gates_res, cprev_delta, cprev_mask, cprev_r
         if tuple(t.shape) != (n, hid, h, w):
             raise ValueError("%s shape %s, expected %s" % (name, tuple(t.shape), (n, hid, h, w)))
     _ready(ts)
+    dt = gates_delta.dtype
     check(lib().mie_convlstm_gates_incr(
-        nhwc_ptr(gates_delta, "gates_delta"), nhwc_ptr(gates_res, "gates_res"),
-        nhwc_ptr(cprev_delta, "cprev_delta"), pix_ptr(cprev_mask, n, h, w, "cprev_mask"),
+        nhwc_ptr(gates_delta, "gates_delta", dtype=dt), nhwc_ptr(gates_res, "gates_res"),
+        nhwc_ptr(cprev_delta, "cprev_delta", dtype=dt), pix_ptr(cprev_mask, n, h, w, "cprev_mask"),
         nhwc_ptr(cprev_res, "cprev_res"), nhwc_ptr(cell_res, "cell_res"),
-        nhwc_ptr(h_delta, "h_delta"), nhwc_ptr(c_delta, "c_delta"), hid, ts.ref,
-        _stream(gates_delta)))
+        nhwc_ptr(h_delta, "h_delta", dtype=dt), nhwc_ptr(c_delta, "c_delta", dtype=dt), hid, ts.ref,
+        delta_dtype(gates_delta), _stream(gates_delta)))
     return h_delta, c_delta
 
 

@@ -62,58 +62,61 @@ def test_invalid_arguments_return_status_not_abort(mie_lib):
     err = lambda: mie_lib.mie_last_error_string().decode()
     # NULL tile set
     assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 16, 16, p, None, 16, 3, 1, 1, 32, None, p,
-                                   None, None, 0, 0.0, 0, None) == -1
+                                   None, None, 0, 0.0, 0, 0, None) == -1
     assert "tile set is NULL" in err()
     # NULL input pointer
     assert mie_lib.mie_conv_masked(None, None, 16, None, None, 0, 16, 16, p, None, 16, 3, 1, 1, 32,
-                                   ctypes.byref(ts), p, None, None, 0, 0.0, 0, None) == -1
+                                   ctypes.byref(ts), p, None, None, 0, 0.0, 0, 0, None) == -1
     # unsupported kernel size and stride (the reference throws std::logic_error, ext_conv.cu:366)
     assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 16, 16, p, None, 16, 4, 1, 1, 32,
-                                   ctypes.byref(ts), p, None, None, 0, 0.0, 0, None) == -2
+                                   ctypes.byref(ts), p, None, None, 0, 0.0, 0, 0, None) == -2
     assert "kernel size 4" in err()
     assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 16, 16, p, None, 16, 3, 3, 1, 32,
-                                   ctypes.byref(ts), p, None, None, 0, 0.0, 0, None) == -2
+                                   ctypes.byref(ts), p, None, None, 0, 0.0, 0, 0, None) == -2
     # output geometry mismatch
     assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 20, 16, p, None, 16, 3, 1, 1, 32,
-                                   ctypes.byref(ts), p, None, None, 0, 0.0, 0, None) == -1
+                                   ctypes.byref(ts), p, None, None, 0, 0.0, 0, 0, None) == -1
     assert "tile set is" in err()
     # misaligned pointer
     assert mie_lib.mie_conv_masked(p + 4, None, 16, None, None, 0, 16, 16, p, None, 16, 3, 1, 1, 32,
-                                   ctypes.byref(ts), p, None, None, 0, 0.0, 0, None) == -1
+                                   ctypes.byref(ts), p, None, None, 0, 0.0, 0, 0, None) == -1
     assert "aligned" in err()
     # MFMA path on a shape it cannot take
     assert mie_lib.mie_conv_masked(p, None, 24, None, None, 0, 16, 16, p, None, 24, 3, 1, 1, 32,
-                                   ctypes.byref(ts), p, None, None, 0, 0.0, _lib.PATH_MFMA, None) == -2
+                                   ctypes.byref(ts), p, None, None, 0, 0.0, _lib.PATH_MFMA, 0, None) == -2
     # MFMA path without the matrix-core filter copy
     assert mie_lib.mie_conv_masked(p, None, 32, None, None, 0, 16, 16, p, None, 32, 3, 1, 1, 32,
-                                   ctypes.byref(ts), p, None, None, 0, 0.0, _lib.PATH_MFMA, None) == -2
+                                   ctypes.byref(ts), p, None, None, 0, 0.0, _lib.PATH_MFMA, 0, None) == -2
     assert "mie_pack_filter" in err()
     # filter packing: cin must be a multiple of 8, buffers distinct
-    assert mie_lib.mie_pack_filter(p, 12, 3, 32, p + 4096, None) == -2
-    assert mie_lib.mie_pack_filter(p, 16, 3, 32, p, None) == -1
-    assert mie_lib.mie_pack_filter(p, 16, 3, 32, None, None) == -1
+    assert mie_lib.mie_pack_filter(p, 12, 3, 32, p + 4096, 0, None) == -2
+    assert mie_lib.mie_pack_filter(p, 16, 3, 32, p, 0, None) == -1
+    assert mie_lib.mie_pack_filter(p, 16, 3, 32, None, 0, None) == -1
+    assert mie_lib.mie_pack_filter(p, 24, 3, 32, p + 4096, 1, None) == -2      # bf16 blocks hold 16 channels
+    assert mie_lib.mie_pack_filter(p, 16, 3, 32, p + 4096, 7, None) == -2      # unknown dtype
     # activation without a reservoir
     assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 16, 16, p, None, 16, 3, 1, 1, 32,
-                                   ctypes.byref(ts), p, None, None, _lib.ACT_RELU, 0.0, 0, None) == -1
+                                   ctypes.byref(ts), p, None, None, _lib.ACT_RELU, 0.0, 0, 0, None) == -1
     # channels beyond the filter
     assert mie_lib.mie_conv_masked(p, None, 16, p, None, 16, 16, 16, p, None, 16, 3, 1, 1, 32,
-                                   ctypes.byref(ts), p, None, None, 0, 0.0, 0, None) == -1
+                                   ctypes.byref(ts), p, None, None, 0, 0.0, 0, 0, None) == -1
     # tile set with a NULL member / zero-sized geometry
     bad, keep2 = _fake_tileset(null="tiles")
-    assert mie_lib.mie_act_incr(1, 0.0, p, p, p, 8, ctypes.byref(bad), None, 0, None) == -1
+    assert mie_lib.mie_act_incr(1, 0.0, p, p, p, 8, ctypes.byref(bad), None, 0, 0, None) == -1
     zero, keep3 = _fake_tileset(n=0)
-    assert mie_lib.mie_act_incr(1, 0.0, p, p, p, 8, ctypes.byref(zero), None, 0, None) == -1
-    assert mie_lib.mie_act_incr(9, 0.0, p, p, p, 8, ctypes.byref(ts), None, 0, None) == -2
+    assert mie_lib.mie_act_incr(1, 0.0, p, p, p, 8, ctypes.byref(zero), None, 0, 0, None) == -1
+    assert mie_lib.mie_act_incr(9, 0.0, p, p, p, 8, ctypes.byref(ts), None, 0, 0, None) == -2
+    assert mie_lib.mie_act_incr(1, 0.0, p, p, p, 8, ctypes.byref(ts), None, 0, 5, None) == -2   # unknown dtype
     assert mie_lib.mie_build_mask_tiles(None, None, 16, 16, 7, 3, 1, 1, ctypes.byref(ts), None) == -2
     assert mie_lib.mie_build_mask_tiles(None, None, 9, 8, _lib.FOOT_UP2X, 0, 0, 0, ctypes.byref(ts), None) == -1
-    assert mie_lib.mie_upsample2x_incr(p, None, None, None, 9, 8, 4, ctypes.byref(ts), p, None) == -1
-    assert mie_lib.mie_mask_from_delta(p, 1, 4, 4, 4, -1.0, p, None) == -1
-    assert mie_lib.mie_convlstm_gates_incr(p, p, None, p, p, p, p, p, 4, ctypes.byref(ts), None) == -1
-    assert mie_lib.mie_tconv_masked(p, None, 4, 9, 9, p, 3, 2, 1, 4, ctypes.byref(ts), p, None, 0, 0.0, None) == -1
+    assert mie_lib.mie_upsample2x_incr(p, None, None, None, 9, 8, 4, ctypes.byref(ts), p, 0, None) == -1
+    assert mie_lib.mie_mask_from_delta(p, 1, 4, 4, 4, -1.0, p, 0, None) == -1
+    assert mie_lib.mie_convlstm_gates_incr(p, p, None, p, p, p, p, p, 4, ctypes.byref(ts), 0, None) == -1
+    assert mie_lib.mie_tconv_masked(p, None, 4, 9, 9, p, 3, 2, 1, 4, ctypes.byref(ts), p, None, 0, 0.0, 0, None) == -1
 
 
 def test_check_raises_runtime_error(mie_lib):
-    rc = mie_lib.mie_mask_from_delta(None, 1, 4, 4, 4, 0.0, None, None)
+    rc = mie_lib.mie_mask_from_delta(None, 1, 4, 4, 4, 0.0, None, 0, None)
     with pytest.raises(RuntimeError, match="NULL pointer"):
         _lib.check(rc)
     assert issubclass(_lib.MieError, RuntimeError)
