@@ -159,26 +159,32 @@ class ConvLSTMIncr(nn.Module, _IncrBuffers):
         spatial_size = input_.data.size()[2:]
         if prev_state is None:
             state_size = tuple([batch_size, self.hidden_size] + list(spatial_size))
-            if state_size not in self.zero_tensors:
-                self.zero_tensors[state_size] = (
-                    torch.zeros(state_size, device=input_.device).to(memory_format=torch.channels_last),
-                    torch.zeros(state_size, device=input_.device).to(memory_format=torch.channels_last))
-            prev_state = self.zero_tensors[tuple(state_size)]
-        zero_state = prev_state is self.zero_tensors.get(tuple([batch_size, self.hidden_size] + list(spatial_size)))
+            zkey = state_size + (input_.dtype,)
+            if zkey not in self.zero_tensors:
+                self.zero_tensors[zkey] = tuple(
+                    torch.zeros(state_size, device=input_.device, dtype=input_.dtype).to(memory_format=torch.channels_last)
+                    for _ in range(2))
+            prev_state = self.zero_tensors[zkey]
+        zero_state = prev_state is self.zero_tensors.get(
+            tuple([batch_size, self.hidden_size] + list(spatial_size)) + (input_.dtype,))
         prev_h, prev_c = prev_state
         self._reset_incr()
         # the concat is never formed: two-pointer conv input, hidden half skipped when it is zero
-        gates = self.Gates._refresh_forward(input_, None if zero_state else prev_h, path=self.Gates.path)
-        in_gate, remember_gate, out_gate, cell_gate = gates.chunk(4, 1)
         if self.fused:
-            self.gates_res.update_reservoir(gates)
+            # the fp32 gate pre-activations go straight into their reservoir; the state is
+            # computed from them in fp32 and handed on in the dtype of the input
+            self.Gates._refresh_forward(input_, None if zero_state else prev_h, path=self.Gates.path,
+                                        reserve=self.gates_res)
+            in_gate, remember_gate, out_gate, cell_gate = self.gates_res.reservoir.chunk(4, 1)
             self.cprev_res.update_reservoir(prev_c)
             in_gate, remember_gate = torch.sigmoid(in_gate), torch.sigmoid(remember_gate)
             out_gate, cell_gate = torch.sigmoid(out_gate), torch.tanh(cell_gate)
-            cell = in_gate * cell_gate + remember_gate * prev_c
+            cell = in_gate * cell_gate + remember_gate * self.cprev_res.reservoir
             self.cell_res.update_reservoir(cell)
             hidden = out_gate * torch.tanh(cell)
-            return hidden, cell
+            return hidden.to(input_.dtype), cell.to(input_.dtype)
+        gates = self.Gates._refresh_forward(input_, None if zero_state else prev_h, path=self.Gates.path)
+        in_gate, remember_gate, out_gate, cell_gate = gates.chunk(4, 1)
         in_gate = self.sigmoid1.forward_refresh_reservoirs(in_gate)
         remember_gate = self.sigmoid2.forward_refresh_reservoirs(remember_gate)
         out_gate = self.sigmoid3.forward_refresh_reservoirs(out_gate)

@@ -31,6 +31,7 @@ def main():
     ap.add_argument("--density", type=float, default=1.0, help="fraction of active input pixels (1 = dense)")
     ap.add_argument("--fused-act", type=int, default=1, help="1: reservoir + ReLU epilogue, 0: plain delta")
     ap.add_argument("--path", choices=["auto", "valu", "mfma"], default="auto")
+    ap.add_argument("--dtype", choices=["f32", "bf16"], default="f32", help="element type of the deltas and of the matrix-core filter copy")
     ap.add_argument("--iters", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--copy-mb", type=int, default=0, help="run a plain copy of this many MiB instead")
@@ -67,11 +68,13 @@ def main():
         mask = m.to(dev)
     else:
         mask = None
-    x = ops.as_nhwc(x.to(dev).contiguous(memory_format=torch.channels_last))
+    dt = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+    es = 2 if args.dtype == "bf16" else 4
+    x = ops.as_nhwc(x.to(dev).to(dt).contiguous(memory_format=torch.channels_last))
     filt = ops.ConvFilter(he_normal_conv_weight(cout, cin, k, 0).permute(1, 2, 3, 0).contiguous().to(dev))
     ts = TileMask(n, ho, wo, dev)
     ops.build_mask_tiles(mask, None, n, h, w, _lib.FOOT_CONV, k, s, p, ts)
-    out = ops.new_nhwc(n, cout, ho, wo, dev)
+    out = ops.new_nhwc(n, cout, ho, wo, dev, dt)
     res = ops.new_nhwc(n, cout, ho, wo, dev) if args.fused_act else None
     act = _lib.ACT_RELU if args.fused_act else _lib.ACT_NONE
     path = dict(auto=_lib.PATH_AUTO, valu=_lib.PATH_VALU, mfma=_lib.PATH_MFMA)[args.path]
@@ -93,11 +96,11 @@ def main():
     tiles = int(ts.counts[0].item())
     flops = 2 * a_out * cin * cout * k * k
     # algorithmic bytes: mask, active delta, emitted delta, reservoir read+write, filter, tile list
-    byts = n * h * w + a_in * cin * 4 + a_out * cout * 4 + cin * cout * k * k * 4 + ts.capacity * 4
+    byts = n * h * w + a_in * cin * es + a_out * cout * es + cin * cout * k * k * es + ts.capacity * 4
     if args.fused_act:
         byts += 2 * a_out * cout * 4
     print(json.dumps(dict(kernel="mie_conv_masked", shape="%dx%d s%d %d->%d @%dx%d n=%d" % (k, k, s, cin, cout, ho, wo, n),
-                          density=args.density, active_tiles=tiles, tiles=ts.capacity, us=round(us, 2),
+                          dtype=args.dtype, density=args.density, active_tiles=tiles, tiles=ts.capacity, us=round(us, 2),
                           algorithmic_flops=flops, algorithmic_bytes=byts,
                           tile_flops=2 * tiles * 64 * cin * cout * k * k,
                           tflops=round(flops / us / 1e6, 2), gbs=round(byts / us / 1e3, 1), iters=args.iters)))

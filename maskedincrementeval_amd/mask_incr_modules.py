@@ -335,11 +335,13 @@ class _ConvIncrMixin(_IncrBuffers):
 
 
     def _refresh_forward(self, x: DenseT, x2: DenseT = None, activation=None, out=None,
-                         path=_lib.PATH_AUTO, addend: DenseT = None) -> DenseT:
+                         path=_lib.PATH_AUTO, addend: DenseT = None, reserve=None) -> DenseT:
         """Dense pass: conv2d(cat(x, x2), W, b) through the same kernels with every tile
         active.  With `activation` (an nnReservedActivation) the pre-activation goes straight
-        into its reservoir and the activated tensor is returned.  `out` overrides the result
-        buffer.  CPU tensors take the torch ops (nothing of this package computes on the CPU).
+        into its reservoir and the activated tensor is returned; with `reserve` (an
+        IncrementReserve) the fp32 result is also written into that reservoir.  `out` overrides
+        the result buffer.  CPU tensors take the torch ops (nothing of this package computes on
+        the CPU).
         """
         self._reset_incr()
         if not x.is_cuda:
@@ -350,6 +352,8 @@ class _ConvIncrMixin(_IncrBuffers):
             y = nn.Conv2d.forward(self, xin)
             if addend is not None:
                 y = y + addend
+            if reserve is not None:
+                reserve.update_reservoir(y)
             return y if activation is None else activation.forward_refresh_reservoirs(y)
         k, s, p = self._geometry()
         x = ops.as_nhwc(x)
@@ -368,6 +372,11 @@ class _ConvIncrMixin(_IncrBuffers):
                 activation.in_res.reservoir = ops.new_nhwc(*shape, x.device)
             res = activation.in_res.reservoir
             activation._reset_incr()
+        elif reserve is not None:
+            r = reserve.reservoir
+            if r is None or tuple(r.shape) != shape or r.device != x.device:
+                reserve.reservoir = ops.new_nhwc(*shape, x.device)
+            res = reserve.reservoir
         bias = None if self.bias is None else self.bias.detach()
         ops.conv_refresh(x, x2, self.conv2d_weights, bias, k, s, p, ts, out, res, kind, slope, path,
                          None if addend is None else ops.as_nhwc(addend))

@@ -1,0 +1,203 @@
+"""GPU parity of the bf16 variant (bf16 deltas and weights, fp32 reservoirs and accumulation)
+through the C ABI.
+
+Two kinds of checks:
+  * op level, against the CPU oracle evaluated on the SAME bf16-rounded inputs and weights in
+    fp32: the kernels then differ from the oracle only by the summation order inside fp32 and
+    one final rounding to bf16, so results agree to 1-2 bf16 ulps (rtol 2**-7, atol on the
+    scale of the sums); reservoirs are fp32 and held to the fp32 tolerance; exact where the
+    arithmetic is exact (ReLU increment, masks, tile lists, filter packing);
+  * network level, against the fp32 oracle on the un-rounded inputs, within the stated bf16
+    tolerance rtol 2e-2 (of the output range, since a sigmoid output has no small values to
+    be relative to).
+"""
+import numpy as np
+import pytest
+import torch
+
+from maskedincrementeval_amd import _lib, ops
+from maskedincrementeval_amd.e2depth_incr import E2VIDRecurrentIncr
+from maskedincrementeval_amd.masked_types import TileMask
+from maskedincrementeval_amd.synthetic import (event_voxel_delta, gaussian_delta, he_normal_conv_weight,
+                                               seed_module_)
+from oracle import incr_oracle as io
+from oracle import mask_oracle as mo
+from oracle.e2depth_oracle import E2DepthOracle
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+BF = torch.bfloat16
+ULP_RTOL = 2.0 ** -7          # two bf16 ulps
+
+
+def _r(t):
+    """Round to bf16 and back: the value a bf16 buffer holds."""
+    return t.to(BF).float()
+
+
+def _dev(t, dtype=BF):
+    return ops.as_nhwc(t.to(DEV).to(dtype).contiguous(memory_format=torch.channels_last))
+
+
+def _close(got, ref, what, rtol=ULP_RTOL, atol=None):
+    got = got.detach().float().cpu()
+    if atol is None:
+        atol = rtol * ref.abs().max().item()       # sums of many products cancel: scale of the result
+    err = (got - ref).abs().max().item()
+    assert torch.allclose(got, ref, rtol=rtol, atol=atol), "%s max|diff| = %.3e (atol %.3e)" % (what, err, atol)
+
+
+def test_pack_filter_bf16_layout():
+    cin, k, cout = 32, 3, 40
+    f = torch.randn(cin, k, k, cout, generator=torch.Generator().manual_seed(0)).to(DEV)
+    p = ops.pack_filter(f, BF)
+    torch.cuda.synchronize()
+    want = f.to(BF).reshape(cin // 16, 2, 8, k * k, cout).permute(0, 3, 1, 4, 2).contiguous()    # [b,t,h,co,j]
+    assert p.dtype == BF and torch.equal(p, want)
+    cf = ops.ConvFilter(f)
+    plain, mc = cf.for_dtype(BF)
+    assert torch.equal(plain, f.to(BF).float()) and torch.equal(mc, want)
+    assert cf.for_dtype(BF)[1] is mc                              # made once
+    assert ops.ConvFilter(f[:24].contiguous()).for_dtype(BF)[1] is None     # 24 % 16 != 0
+
+
+@pytest.mark.parametrize("path", [_lib.PATH_VALU, _lib.PATH_MFMA])
+@pytest.mark.parametrize("k,s,cin,cout,h,w", [(3, 1, 64, 64, 33, 44), (5, 1, 64, 32, 40, 56), (5, 2, 32, 64, 47, 61),
+                                              (3, 1, 128, 256, 17, 23), (1, 1, 64, 128, 16, 24), (7, 2, 16, 128, 30, 30)])
+def test_conv_bf16_matches_oracle_on_rounded_operands(path, k, s, cin, cout, h, w):
+    n, p = 1, k // 2
+    wt = he_normal_conv_weight(cout, cin, k, seed=k + cin)
+    filt = ops.ConvFilter(wt.permute(1, 2, 3, 0).contiguous().to(DEV))
+    ho, wo = mo.conv_out_size(h, w, k, s, p)
+    ts = TileMask(n, ho, wo, DEV)
+    out = ops.new_nhwc(n, cout, ho, wo, DEV, BF)
+    res = ops.new_nhwc(n, cout, ho, wo, DEV)                        # fp32 reservoir
+    r0 = torch.randn(n, cout, ho, wo, generator=torch.Generator().manual_seed(5))
+    res.copy_(r0)
+    res_cpu = io.Reserve(r0.clone())
+    for step in range(3):
+        d, m = gaussian_delta(n, cin, h, w, 0.15, 0.5, seed=70 + step)
+        x = _dev(d)
+        x[~m.to(DEV).bool().expand_as(x)] = float("nan")          # inactive pixels are never read
+        ops.build_mask_tiles(m.to(DEV), None, n, h, w, _lib.FOOT_CONV, k, s, p, ts)
+        ops.conv_masked(x, m.to(DEV), None, None, filt, k, s, p, ts, out, res, _lib.ACT_RELU, 0.0, path)
+        torch.cuda.synchronize()
+        acc = io.conv_incr(_r(d), _r(wt), s, p)                     # same operands, fp32 sums
+        want = io.act_incr(torch.relu, res_cpu, acc)
+        _close(res, res_cpu.reservoir, "reservoir (fp32) step %d" % step, rtol=1e-4, atol=1e-4)
+        _close(out, want, "delta step %d" % step)
+        assert out.dtype == BF
+        fp = mo.footprint_conv(m[:, 0].numpy(), k, s, p)
+        assert not (out.float().cpu().numpy()[:, :, fp[0] == 0] != 0).any()     # clean outside the mask
+
+
+def test_conv_bf16_two_inputs_addend_and_plain_delta():
+    # concat-free two-pointer conv (64 + 64 channels) with an addend, no reservoir: plain bf16 delta
+    n, c1, c2, cout, h, w = 1, 64, 64, 128, 24, 40
+    wt = he_normal_conv_weight(cout, c1 + c2, 3, seed=3)
+    filt = ops.ConvFilter(wt.permute(1, 2, 3, 0).contiguous().to(DEV))
+    d1, m1 = gaussian_delta(n, c1, h, w, 0.2, 0.4, seed=1)
+    d2, m2 = gaussian_delta(n, c2, h, w, 0.1, 0.4, seed=2)
+    add = _r(torch.randn(n, cout, h, w, generator=torch.Generator().manual_seed(4)) * 0.1)
+    ts = TileMask(n, h, w, DEV)
+    ops.build_mask_tiles(m1.to(DEV), m2.to(DEV), n, h, w, _lib.FOOT_CONV, 3, 1, 1, ts)
+    fp = torch.from_numpy(mo.footprint_conv((m1 | m2)[:, 0].numpy(), 3, 1, 1)).bool()[:, None]
+    add = add * fp                                                   # an addend is a clean delta under the output mask
+    for path in (_lib.PATH_VALU, _lib.PATH_MFMA):
+        out = ops.new_nhwc(n, cout, h, w, DEV, BF)
+        ops.conv_masked(_dev(d1), m1.to(DEV), _dev(d2), m2.to(DEV), filt, 3, 1, 1, ts, out, None,
+                        _lib.ACT_NONE, 0.0, path, addend=_dev(add))
+        torch.cuda.synchronize()
+        want = io.conv_incr(torch.cat((_r(d1), _r(d2)), 1), _r(wt), 1, 1) + add
+        _close(out, want, "two-input conv, path %d" % path)
+    with pytest.raises(ValueError, match="bfloat16"):               # mixed dtypes are refused on the host
+        ops.conv_masked(_dev(d1), m1.to(DEV), _dev(d2, torch.float32), m2.to(DEV), filt, 3, 1, 1, ts, out)
+
+
+def test_pointwise_bf16():
+    n, c, h, w = 2, 32, 21, 37
+    ts = TileMask(n, h, w, DEV)
+    r0 = torch.randn(n, c, h, w, generator=torch.Generator().manual_seed(1))
+    res_cpu, res = io.Reserve(r0.clone()), ops.new_nhwc(n, c, h, w, DEV)
+    res.copy_(r0)
+    out = ops.new_nhwc(n, c, h, w, DEV, BF)
+    refined = torch.zeros((n, 1, h, w), dtype=torch.uint8, device=DEV)
+    for step in range(3):
+        d, m = gaussian_delta(n, c, h, w, 0.1, 0.7, seed=10 + step)
+        ops.build_mask_tiles(m.to(DEV), None, n, h, w, _lib.FOOT_CONV, 1, 1, 0, ts)
+        ops.act_incr(_lib.ACT_RELU, 0.0, _dev(d), res, out, ts, refined)
+        torch.cuda.synchronize()
+        want = io.act_incr(torch.relu, res_cpu, _r(d))
+        # ReLU increment: the fp32 arithmetic is exact-order, the only rounding is the final bf16 one
+        assert torch.equal(res.cpu(), res_cpu.reservoir), "reservoir must be bit-exact fp32"
+        assert torch.equal(out.cpu(), want.to(BF)), "delta must be the bf16 rounding of the fp32 result"
+        assert np.array_equal(refined.cpu().numpy(), (want != 0).any(dim=1, keepdim=True).to(torch.uint8).numpy())
+    # product rule, sum, bilinear x2 on bf16 deltas
+    d1, m1 = gaussian_delta(n, c, h, w, 0.2, 0.5, seed=20)
+    d2, m2 = gaussian_delta(n, c, h, w, 0.2, 0.5, seed=21)
+    both = (m1 | m2)
+    ops.build_mask_tiles(m1.to(DEV), m2.to(DEV), n, h, w, _lib.FOOT_CONV, 1, 1, 0, ts)
+    q1, q2 = torch.randn(n, c, h, w, generator=torch.Generator().manual_seed(22)), torch.randn(n, c, h, w, generator=torch.Generator().manual_seed(23))
+    R1, R2 = io.Reserve(q1.clone()), io.Reserve(q2.clone())
+    g1, g2 = ops.new_nhwc(n, c, h, w, DEV), ops.new_nhwc(n, c, h, w, DEV)
+    g1.copy_(q1), g2.copy_(q2)
+    ops.mul_incr(_dev(d1), m1.to(DEV), g1, _dev(d2), m2.to(DEV), g2, out, ts)
+    _close(out, io.mul_incr(_r(d1), R1, _r(d2), R2), "product rule")
+    _close(g1, R1.reservoir, "r1", rtol=1e-6, atol=1e-6)
+    ops.add_incr(_dev(d1), m1.to(DEV), _dev(d2), m2.to(DEV), out, ts)
+    _close(out, _r(d1) + _r(d2), "sum")
+    up_ts = TileMask(n, 2 * h, 2 * w, DEV)
+    ops.build_mask_tiles(both.to(DEV), None, n, h, w, _lib.FOOT_UP2X, 0, 0, 0, up_ts)
+    up = ops.new_nhwc(n, c, 2 * h, 2 * w, DEV, BF)
+    ops.upsample2x_incr(_dev(d1), m1.to(DEV), _dev(d2), m2.to(DEV), up_ts, up)
+    _close(up, io.interp_incr(_r(d1) + _r(d2)), "bilinear x2 of the sum")
+    # mask from a bf16 delta: exact
+    pix = torch.zeros((n, 1, h, w), dtype=torch.uint8, device=DEV)
+    ops.mask_from_delta(_dev(d1), 0.0, pix)
+    assert np.array_equal(pix[:, 0].cpu().numpy(), mo.pixel_mask(_r(d1).numpy(), 0.0))
+    # quantiser on bf16 deltas: fp32 carry, every op IEEE -> carry exact, delta = bf16 rounding
+    carry_cpu, carry = io.Reserve(torch.zeros(n, c, h, w)), ops.new_nhwc(n, c, h, w, DEV)
+    ops.build_mask_tiles(m1.to(DEV), None, n, h, w, _lib.FOOT_CONV, 1, 1, 0, ts)
+    ops.kfence_incr(_dev(d1), carry, 0.25, out, ts)
+    f = io.kfenced(carry_cpu, torch.tensor(0.25), _r(d1))
+    assert torch.equal(carry.cpu(), carry_cpu.reservoir) and torch.equal(out.cpu(), f.to(BF))
+
+
+def _run_e2depth_bf16(n, h, w, steps, density, cfg=None, seed=31):
+    model = seed_module_(E2VIDRecurrentIncr(cfg), seed=seed).to(DEV).eval()
+    oracle = E2DepthOracle(model.state_dict())
+    x0 = torch.randn(n, 5, h, w, generator=torch.Generator().manual_seed(seed + 1)) * 0.5
+    with torch.no_grad():
+        first = model.forward_refresh_reservoirs(_dev(x0), None)[0]
+    assert first.dtype == BF
+    acc = first.float().clone()
+    acc_ref = oracle.refresh(x0)
+    # the prediction is a sigmoid output in (0, 1): bf16 tolerance 2e-2 of that range
+    _close(acc, acc_ref, "refresh", rtol=2e-2, atol=2e-2)
+    for step in range(steps):
+        d = event_voxel_delta(n, 5, h, w, density, seed=3000 + step)[0]
+        with torch.no_grad():
+            out, _ = model([_dev(d), None], None)
+        torch.cuda.synchronize()
+        assert out[0].dtype == BF
+        ref = oracle.incr(d)
+        _close(out[0], ref, "step %d" % step, rtol=2e-2, atol=2e-2 * max(ref.abs().max().item(), 1e-3))
+        acc += out[0].float()
+        acc_ref += ref
+    _close(acc, acc_ref, "accumulated after %d steps" % steps, rtol=2e-2, atol=2e-2)
+    return model
+
+
+def test_e2depth_incr_bf16_small_matches_fp32_oracle():
+    model = _run_e2depth_bf16(1, 72, 104, steps=6, density=0.05)
+    # every reservoir stayed fp32, every delta buffer is bf16
+    for mod in model.modules():
+        for key, buf in getattr(mod, "__dict__", {}).get("_incr_bufs", {}).items():
+            if key[0] == "d":
+                assert buf.dtype == BF, key
+
+
+def test_e2depth_incr_bf16_batched_high_resolution():
+    # the batched configuration at a quarter of its pixels per stream (8 x 240 x 320): batch-wide tile
+    # compaction, bf16 matrix-core convs on every wide layer, fp32 oracle within the bf16 tolerance
+    _run_e2depth_bf16(8, 240, 320, steps=2, density=0.01)
