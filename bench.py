@@ -25,6 +25,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_BF16_MFMA_TFLOPS = 2500.0
 PEAK_HBM_GBS = 8000.0
 
 
@@ -42,6 +43,8 @@ def parse_args():
     ap.add_argument("--no-dense", action="store_true", help="skip the all-tiles-active comparator")
     ap.add_argument("--layer-iters", type=int, default=20, help="timed launches per layer for the roofline table")
     ap.add_argument("--sync-masks", action="store_true", help="build tile sets on the compute stream (no planning stream)")
+    ap.add_argument("--dtype", choices=["f32", "bf16"], default="f32",
+                    help="element type of deltas and weights (reservoirs and accumulation stay fp32)")
     ap.add_argument("--kfence-tp", type=float, default=0.0,
                     help="also time the net with every conv's delta quantiser on (k = tp*||x||); reported under \"kfenced\"")
     ap.add_argument("--sweep", action="store_true", help="also time 1 %% and 20 %% density (reported under \"density_sweep\")")
@@ -53,8 +56,9 @@ class LayerProbe:
     on the stream the kernels are launched on, and derives algorithmic bytes / flops from the
     tile-set statistics of that step."""
 
-    def __init__(self, ops, torch):
+    def __init__(self, ops, torch, es=4):
         self.ops, self.torch = ops, torch
+        self.es = es            # bytes per delta / weight element (reservoirs are always 4)
         self.records = []
         self._orig = {}
 
@@ -112,7 +116,8 @@ class LayerProbe:
                 a_in = P if d["xmask"] is None else int(self._pix(d["xmask"]).sum().item())
                 a_out = int(ts.pixmask.sum().item())
                 cin, cout, k = d["cin"], d["cout"], d["k"]
-                byts = P + a_in * cin * 4 + a_out * cout * 4 + cin * cout * k * k * 4 + ts.capacity * 4
+                es = self.es
+                byts = P + a_in * cin * es + a_out * cout * es + cin * cout * k * k * es + ts.capacity * 4
                 if d["fused"]:
                     byts += 2 * a_out * cout * 4
                 row.update(shape="%dx%d s%d %d->%d @%dx%d" % (k, k, d["s"], cin, cout, ts.h, ts.w),
@@ -124,9 +129,9 @@ class LayerProbe:
                 c = d["c"]
                 if d["kind"] == "gates":
                     hid = c // 4
-                    byts = a * (4 * hid * 4 + 2 * 4 * hid * 4 + 2 * hid * 4 + hid * 4 + 2 * hid * 4)
+                    byts = a * (4 * hid * self.es + 2 * 4 * hid * 4 + 2 * hid * 4 + hid * 4 + 2 * hid * self.es)
                 else:
-                    byts = a * c * 4 * (d["nin"] + 2 * d["nres"] + 1)
+                    byts = a * c * (self.es * (d["nin"] + 1) + 8 * d["nres"])
                 byts += ts.n * ts.h * ts.w
                 row.update(shape="%s C=%d @%dx%d" % (d["kind"], c, ts.h, ts.w), a_out=a, bytes=byts, flops=0,
                            active_tiles=int(ts.counts[0].item()), tiles=ts.capacity)
@@ -134,7 +139,7 @@ class LayerProbe:
                 ts = d["ts"]
                 row.update(shape="tiles @%dx%d" % (ts.h, ts.w), bytes=2 * ts.n * ts.h * ts.w + ts.capacity * 8, flops=0)
             else:
-                row.update(shape="mask C=%d" % d["c"], bytes=d["npix"] * (d["c"] * 4 + 1), flops=0)
+                row.update(shape="mask C=%d" % d["c"], bytes=d["npix"] * (d["c"] * self.es + 1), flops=0)
             rows.append(row)
         return rows
 
@@ -160,7 +165,10 @@ def main():
         sys.exit(2)
     dev = torch.device("cuda:0")
     H, W, dens, NB = args.height, args.width, args.density, args.batch
-    cl = lambda t: t.to(dev).contiguous(memory_format=torch.channels_last)
+    dt = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+    es = 2 if args.dtype == "bf16" else 4          # bytes per delta / weight element
+    peak_mfma = PEAK_BF16_MFMA_TFLOPS if args.dtype == "bf16" else PEAK_FP32_MFMA_TFLOPS
+    cl = lambda t: t.to(dev).to(dt).contiguous(memory_format=torch.channels_last)
 
     model = seed_module_(E2VIDRecurrentIncr(async_masks=not args.sync_masks), seed=1).to(dev).eval()
     x0 = torch.randn(NB, 5, H, W, generator=torch.Generator().manual_seed(2)) * 0.5
@@ -215,7 +223,7 @@ def main():
         step_eager(model, 0)
         agg = None
         for it in range(args.layer_iters):
-            with LayerProbe(ops, torch) as probe:
+            with LayerProbe(ops, torch, es) as probe:
                 step_eager(model, 1 + it)
             rows = probe.table()
             if agg is None:
@@ -254,10 +262,10 @@ def main():
     dom_us = 1e3 * ev0.elapsed_time(ev1) / reps
     dom = dict(dom, us=round(dom_us, 2), gbs=round(dom["bytes"] / dom_us / 1e3, 1),
                tflops=round(dom["flops"] / dom_us / 1e6, 2))
-    mfma_bound = dom["flops"] / max(dom["bytes"], 1) > PEAK_FP32_MFMA_TFLOPS * 1e12 / (PEAK_HBM_GBS * 1e9)
+    mfma_bound = dom["flops"] / max(dom["bytes"], 1) > peak_mfma * 1e12 / (PEAK_HBM_GBS * 1e9)
     if mfma_bound:
-        roofline = dict(bound="mfma", achieved=dom["tflops"], peak=PEAK_FP32_MFMA_TFLOPS, unit="TFLOP/s",
-                        frac=round(dom["tflops"] / PEAK_FP32_MFMA_TFLOPS, 4), traffic=None)
+        roofline = dict(bound="mfma", achieved=dom["tflops"], peak=peak_mfma, unit="TFLOP/s",
+                        frac=round(dom["tflops"] / peak_mfma, 4), traffic=None)
     else:
         roofline = dict(bound="hbm", achieved=dom["gbs"], peak=PEAK_HBM_GBS, unit="GB/s",
                         frac=round(dom["gbs"] / PEAK_HBM_GBS, 4), traffic=None)
@@ -353,7 +361,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": args.dtype,
         "data": "synthetic",
         "config": {"workload": "E2Depth-incr recurrent UNet, random init, %dx5x%dx%d event voxel deltas, %.0f%% "
                                "active pixels, 1 dense refresh then incremental steps" % (NB, H, W, 100 * dens),

@@ -39,6 +39,20 @@ __host__ __device__ constexpr int stage_channels(int K, int S) {
   return (S == 1) ? (K <= 5 ? 32 : 16) : (K <= 5 ? 16 : 8);
 }
 
+// LDS dwords per row of the staged input tile.  The 16-byte operand reads of 16 neighbouring lanes
+// (8 pixels of one tile row and of the next) must fall on 64 distinct banks: the pixel stride
+// (CC + 4 dwords) spreads one row over every other group of 4 banks, and a row pitch of
+// 32 (mod 64) dwords puts the next row on the groups in between (stride 1).  For stride 2 the
+// pixel stride doubles and every row falls on the same bank groups whatever the pitch; there
+// the two 16-byte halves of a unit are swapped in every other pair of input rows instead
+// (`swz` below), which moves the neighbouring tile row by 4 banks.
+__host__ __device__ constexpr int row_pitch_dw(int it, int ls_dw, int s) {
+  int rp = it * ls_dw;
+  if (s == 1)
+    while (rp % 64 != 32) rp += 4;
+  return rp;
+}
+
 // Ring size of the B-operand prefetch: the smallest divisor of the units per chunk that is
 // at least 4, so that ring slot (unit % ring) means the same registers in every chunk.
 __host__ __device__ constexpr int ring_size(int upc) {
@@ -74,7 +88,8 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   constexpr int Q4 = CC / EPS;                               // 16-byte slots per pixel
   constexpr int NSLOT = NPIX * Q4;
   constexpr int NLD = (NSLOT + 255) / 256;                   // staging loads per thread
-  constexpr int STAGE = NPIX * LS;                           // elements per staging buffer
+  constexpr int RP = row_pitch_dw(IT, LS * (int)sizeof(T) / 4, S) * 4 / (int)sizeof(T);   // elements per tile row
+  constexpr int STAGE = IT * RP;                             // elements per staging buffer
   constexpr int NQ = CC / SUB;                               // sub-chunks (units per tap) per stage
   static_assert(NQ % WK == 0, "the k-split is over whole sub-chunks");
   constexpr int NQW = NQ / WK;                               // sub-chunks per wave
@@ -129,7 +144,9 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   for (int i = 0; i < NLD; ++i) {
     const int slot = tid + 256 * i;
     const int pix = slot / Q4, q4 = slot - pix * Q4;
-    st_lds[i] = pix * LS + EPS * q4;
+    const int lrow = pix / IT;
+    const int swz = (S == 2) ? ((lrow >> 1) & 1) : 0;
+    st_lds[i] = lrow * RP + (pix - lrow * IT) * LS + EPS * (q4 ^ swz);
     st_c4[i] = EPS * q4;
     st_po[i] = 0;
     if (slot < NSLOT) {
@@ -183,11 +200,15 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   const int q0w = wk * NQW;
   const int cob0 = co0 + wn * (32 * NB);                       // first column of this wave
   const int b_lane = (half * cout + l32) * EPS;                // lane part of the packed filter index
-  int a_lane[2];                                               // lane part of the LDS index
+  int a_lane[2][2];                                            // lane part of the LDS index
 #pragma unroll
   for (int mb = 0; mb < 2; ++mb) {
     const int p = mb * 32 + l32;
-    a_lane[mb] = (((p >> 3) * S) * IT + (p & 7) * S) * LS + SUB * q0w + EPS * half;
+    const int rowcol = ((p >> 3) * S) * RP + ((p & 7) * S) * LS + SUB * q0w;
+    // stride 2: tile row r reads input row 2r + ky, whose halves are swapped iff (r + ky/2) is odd
+    const int h0 = (S == 2) ? (half ^ ((p >> 3) & 1)) : half;
+    a_lane[mb][0] = rowcol + EPS * h0;
+    a_lane[mb][1] = rowcol + EPS * (h0 ^ 1);
   }
   // filter row block of chunk c for this wave (c1 and c2 are multiples of CC: no partial chunks)
   auto chunk_b = [&](int c) -> const T* {
@@ -233,7 +254,8 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
       const int ky = tap / K, kx = tap - ky * K;
 #pragma unroll
       for (int mb = 0; mb < 2; ++mb)
-        dst[mb] = *reinterpret_cast<const float4*>(&sin[a_lane[mb] + (ky * IT + kx) * LS + SUB * qi]);
+        dst[mb] = *reinterpret_cast<const float4*>(
+            &sin[a_lane[mb][(S == 2) ? ((ky >> 1) & 1) : 0] + ky * RP + kx * LS + SUB * qi]);
     };
     load_a(0, av[0]);
 #pragma unroll

@@ -201,3 +201,30 @@ def test_e2depth_incr_bf16_batched_high_resolution():
     # the batched configuration at a quarter of its pixels per stream (8 x 240 x 320): batch-wide tile
     # compaction, bf16 matrix-core convs on every wide layer, fp32 oracle within the bf16 tolerance
     _run_e2depth_bf16(8, 240, 320, steps=2, density=0.01)
+
+
+@pytest.mark.parametrize("density", [0.01, 0.20])
+def test_batched_configuration_full_size_accumulation_identity(density):
+    # 8 streams of 5 x 480 x 640, bf16 deltas and weights: too large for the CPU oracle in a test, so
+    # the size-independent property is checked on the device (tests/test_network.py:24-31 pattern):
+    # refresh(x0) + sum of incremental outputs == dense refresh on x0 + sum of deltas, and a
+    # per-sample result agrees with the single-stream run of that sample (streams do not mix).
+    n, h, w, steps = 8, 480, 640, 3
+    model = seed_module_(E2VIDRecurrentIncr(), seed=5).to(DEV).eval()
+    x0 = torch.randn(n, 5, h, w, generator=torch.Generator().manual_seed(6)) * 0.5
+    x = _r(x0).clone()
+    with torch.no_grad():
+        acc = model.forward_refresh_reservoirs(_dev(x0), None)[0].float().clone()
+        for step in range(steps):
+            d = event_voxel_delta(n, 5, h, w, density, seed=4000 + step)[0]
+            out, _ = model([_dev(d), None], None)
+            acc += out[0].float()
+            x = _r(x + _r(d))            # the dense input the deltas add up to, as bf16 holds it
+        fresh = seed_module_(E2VIDRecurrentIncr(), seed=5).to(DEV).eval()
+        dense = fresh.forward_refresh_reservoirs(_dev(x), None)[0].float()
+        single = seed_module_(E2VIDRecurrentIncr(), seed=5).to(DEV).eval()
+        one = single.forward_refresh_reservoirs(_dev(x[3:4]), None)[0].float()
+    torch.cuda.synchronize()
+    _close(acc, dense.cpu(), "refresh + increments vs dense", rtol=2e-2, atol=2e-2)
+    # streams do not mix (the kernel variants picked for 8 streams and for 1 differ in summation order only)
+    _close(one[0], dense[3].cpu(), "sample 3 of the batch vs its single-stream run", rtol=ULP_RTOL, atol=ULP_RTOL)
