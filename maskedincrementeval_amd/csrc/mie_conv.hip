@@ -132,6 +132,51 @@ __global__ __launch_bounds__(64) void k_conv_smallco(ConvArgsT<T> a) {
 }
 
 // ---------------------------------------------------------------------------------
+// 1x1 stride-1 conv with Cout <= 4 and Cin % 4 == 0 (prediction layer 32 -> 1, flow heads): pure
+// bandwidth work.  4 lanes share one pixel and walk its NHWC row in 16-byte (fp32) / 8-byte
+// (bf16) pieces, so a wave reads whole 8-pixel tile rows as contiguous segments; the partial
+// sums meet through two lane exchanges.  Lane `sub` of a pixel stores output channel `sub`.
+// ---------------------------------------------------------------------------------
+static __device__ __forceinline__ float4 load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+static __device__ __forceinline__ float4 load4(const mie_bf16* p) {
+  const mie_bf16x4 b = *reinterpret_cast<const mie_bf16x4*>(p);
+  return make_float4((float)b[0], (float)b[1], (float)b[2], (float)b[3]);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void k_conv1x1_smallco(ConvArgsT<T> a) {
+  int n, y0, x0;
+  const int tk = mie_pick_tile(a.ts, blockIdx.x, n, y0, x0);
+  if (tk == 0) return;
+  const int px = threadIdx.x >> 2, sub = threadIdx.x & 3;
+  const int oy = y0 + (px >> 3), ox = x0 + (px & 7);
+  const int hout = a.ts.h, wout = a.ts.w;
+  const bool inb = oy < hout && ox < wout;
+  const long long po = ((long long)n * hout + oy) * wout + ox;      // input pixel = output pixel
+  if (tk == 2) {
+    if (inb && sub < a.cout) mie_st(a.out, po * a.cout + sub, 0.f);
+    return;
+  }
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  if (inb && (a.xm == nullptr || a.xm[po])) {
+    const T* xr = a.x + po * a.c1;
+    for (int v = sub; v < (a.c1 >> 2); v += 4) {
+      const float4 x = load4(xr + 4 * v);
+      const float* wp = a.filt + (long long)(4 * v) * a.cout;
+      for (int co = 0; co < a.cout; ++co)
+        acc[co] += x.x * wp[co] + x.y * wp[a.cout + co] + x.z * wp[2 * a.cout + co] + x.w * wp[3 * a.cout + co];
+    }
+  }
+#pragma unroll
+  for (int co = 0; co < 4; ++co) {           // every lane of the wave takes part
+    acc[co] += __shfl_xor(acc[co], 1);
+    acc[co] += __shfl_xor(acc[co], 2);
+  }
+  const float mine = sub == 0 ? acc[0] : (sub == 1 ? acc[1] : (sub == 2 ? acc[2] : acc[3]));
+  if (inb && sub < a.cout) conv_store(a, po * a.cout + sub, sub, mine);
+}
+
+// ---------------------------------------------------------------------------------
 // Transposed conv, gather form.  Thread = one output channel x 16 pixels;
 // input values are wave-uniform loads (every lane of a wave reads the same
 // address), filter rows are coalesced over the output channel.
@@ -170,7 +215,9 @@ __global__ __launch_bounds__(256) void k_tconv_valu(ConvArgsT<T> a, int K, int S
 
 template <typename T, int K, int S>
 void launch_conv(const ConvArgsT<T>& a, unsigned cap, hipStream_t st) {
-  if (a.cout <= 4) {
+  if (K == 1 && S == 1 && a.pad == 0 && a.cout <= 4 && a.x2 == nullptr && (a.c1 & 3) == 0) {
+    hipLaunchKernelGGL((k_conv1x1_smallco<T>), dim3(cap), dim3(256), 0, st, a);
+  } else if (a.cout <= 4) {
     hipLaunchKernelGGL((k_conv_smallco<T, K, S>), dim3(cap), dim3(64), 0, st, a);
   } else {
     hipLaunchKernelGGL((k_conv_valu<T, K, S>), dim3(cap, mie_div_up(a.cout, 64)), dim3(256), 0, st, a);

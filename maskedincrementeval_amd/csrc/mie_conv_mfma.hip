@@ -28,6 +28,7 @@
 // LDS row stride CC+4 floats keeps the 16-byte reads of 8 neighbouring pixels
 // on disjoint banks for stride 1 and 2.
 #include "mie_conv.h"
+#include <stdlib.h>
 
 namespace {
 
@@ -321,33 +322,63 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   }
 }
 
-// Launch with the widest channel slab that still gives the chip enough workgroups (256 CUs;
-// aim for >= 2 workgroups per CU when every tile is active), among the wave splits the
-// staging depth of this (K, S) allows.
+// Output channels per workgroup (the slab 32*NB*WN) for a launch of `cap` tiles: the widest of
+// 128 / 64 / 32 that still gives the chip at least 400 workgroups when every tile is active
+// (256 CUs, up to 3 workgroups resident on each), else the narrowest the staging depth of this
+// (K, S) allows.  Measured on MI355X over the layer shapes of both network sizes: wider slabs
+// re-read less of the input tile but leave CUs idle on the small planes; the 256-wide variant
+// (two 32-column blocks per wave) lost to the 128-wide one on every shape and is only taken
+// when forced.  The environment
+// variable MIE_CONV_SLAB (32, 64, 128 or 256) overrides the choice where the shape allows it --
+// a tuning knob for measurements, read once.
+int forced_slab() {
+  static const int v = [] {
+    const char* e = getenv("MIE_CONV_SLAB");
+    return e ? atoi(e) : 0;
+  }();
+  return v;
+}
+
+template <int K, int S>
+int pick_slab(int cout, unsigned cap) {
+  constexpr int NQ = stage_channels(K, S) / 8;
+  const bool ok256 = cout % 256 == 0, ok128 = cout % 128 == 0, ok64 = NQ >= 2 && cout % 64 == 0;
+  const bool ok32 = NQ >= 4 && cout % 32 == 0;
+  const int f = forced_slab();
+  if ((f == 256 && ok256) || (f == 128 && ok128) || (f == 64 && ok64) || (f == 32 && ok32)) return f;
+  const long long want = 400;
+  if (ok128 && ((long long)cap * (cout / 128) >= want || (!ok64 && !ok32))) return 128;
+  if (ok64 && ((long long)cap * (cout / 64) >= want || !ok32)) return 64;
+  if (ok32) return 32;
+  return ok128 ? 128 : 0;
+}
+
 template <typename T, int K, int S>
 bool launch_ks(const ConvArgsT<T>& a, unsigned cap, hipStream_t st) {
   constexpr int NQ = stage_channels(K, S) / 8;
-  const long long want = 512;
   const int cout = a.cout;
-  if (cout % 256 == 0 && (long long)cap * (cout / 256) >= want) {
-    hipLaunchKernelGGL((k_conv_mfma<T, K, S, 4, 2>), dim3(cap, cout / 256), dim3(256), 0, st, a);
-    return true;
-  }
-  if (cout % 128 == 0 && ((long long)cap * (cout / 128) >= want || NQ < 2 || cout % 64 != 0)) {
-    hipLaunchKernelGGL((k_conv_mfma<T, K, S, 4, 1>), dim3(cap, cout / 128), dim3(256), 0, st, a);
-    return true;
-  }
-  if constexpr (NQ >= 2) {
-    if (cout % 64 == 0 && ((long long)cap * (cout / 64) >= want || NQ < 4)) {
-      hipLaunchKernelGGL((k_conv_mfma<T, K, S, 2, 1>), dim3(cap, cout / 64), dim3(256), 0, st, a);
+  switch (pick_slab<K, S>(cout, cap)) {
+    case 256:
+      hipLaunchKernelGGL((k_conv_mfma<T, K, S, 4, 2>), dim3(cap, cout / 256), dim3(256), 0, st, a);
       return true;
-    }
+    case 128:
+      hipLaunchKernelGGL((k_conv_mfma<T, K, S, 4, 1>), dim3(cap, cout / 128), dim3(256), 0, st, a);
+      return true;
+    case 64:
+      if constexpr (NQ >= 2) {
+        hipLaunchKernelGGL((k_conv_mfma<T, K, S, 2, 1>), dim3(cap, cout / 64), dim3(256), 0, st, a);
+        return true;
+      }
+      return false;
+    case 32:
+      if constexpr (NQ >= 4) {
+        hipLaunchKernelGGL((k_conv_mfma<T, K, S, 1, 1>), dim3(cap, cout / 32), dim3(256), 0, st, a);
+        return true;
+      }
+      return false;
+    default:
+      return false;
   }
-  if constexpr (NQ >= 4) {
-    hipLaunchKernelGGL((k_conv_mfma<T, K, S, 1, 1>), dim3(cap, cout / 32), dim3(256), 0, st, a);
-    return true;
-  }
-  return false;
 }
 
 }  // namespace

@@ -79,7 +79,8 @@ def test_conv_paths_match_oracle(pname, path, k, s, p, cin, cout):
 
 
 @pytest.mark.parametrize("cin,cout,k,s,p", [(5, 32, 5, 1, 2), (3, 5, 3, 1, 1), (7, 70, 3, 2, 1), (32, 1, 1, 1, 0),
-                                            (32, 2, 3, 1, 1), (4, 3, 5, 2, 2), (20, 33, 1, 2, 0)])
+                                            (32, 2, 3, 1, 1), (4, 3, 5, 2, 2), (20, 33, 1, 2, 0), (64, 2, 1, 1, 0), (12, 4, 1, 1, 0),
+                                            (6, 3, 1, 1, 0)])
 def test_odd_channel_counts_auto_path(cin, cout, k, s, p):
     # head (Cin=5), prediction (Cout=1), flow heads (Cout=2) and other shapes the MFMA path cannot take
     n, h, w = 1, 41, 29
