@@ -38,11 +38,9 @@ static __device__ __forceinline__ void conv_store(const ConvArgsT<T>& a, long lo
 }
 
 
-// Launches the matrix-core path for kernel size k (1,3,5,7) and stride s (1,2); the caller
-// has checked that c1 and c2 are multiples of mie_conv_mfma_cin_multiple(k, s, dtype) (the
-// channels staged per chunk) and cout of mie_conv_mfma_cout_multiple(k, s).
-// Returns false if no kernel variant takes the shape (nothing is launched then).
+// Launches the matrix-core path for kernel size k (1,3,5,7) and stride s (1,2).  Returns false
+// if no kernel variant takes the shape (nothing is launched then); mie_conv_mfma_takes says so
+// beforehand.
 bool mie_launch_conv_mfma(const ConvArgsT<float>& a, int k, int s, unsigned cap, hipStream_t st);
 bool mie_launch_conv_mfma(const ConvArgsT<mie_bf16>& a, int k, int s, unsigned cap, hipStream_t st);
-int mie_conv_mfma_cout_multiple(int k, int s);
-int mie_conv_mfma_cin_multiple(int k, int s, int dtype);
+bool mie_conv_mfma_takes(int k, int s, int dtype, int c1, int c2, int cout);

@@ -278,17 +278,16 @@ int conv_impl(const char* who, const T* x, const uint8_t* xmask, int c1, const T
               "%s: bias must be 4-byte and addend 16-byte aligned", who);
   MIE_REQUIRE(addend == nullptr || addend != out_delta, MIE_ERR_INVALID_ARG,
               "%s: addend must not alias out_delta", who);
-  const int cmul = mie_conv_mfma_cout_multiple(k, stride);
-  const int imul = mie_conv_mfma_cin_multiple(k, stride, dtype_of<T>());
   const int pmul = 32 / (int)sizeof(T);       // input channels per block of the matrix-core filter copy
   MIE_REQUIRE(mie_aligned(filter_mc, 16), MIE_ERR_INVALID_ARG, "%s: filter_mc must be 16-byte aligned", who);
-  const bool mfma_ok = (filter_mc != nullptr) && (cin_total % pmul == 0) && (c1 % imul == 0) &&
-                       (c2 % imul == 0) && (cout % cmul == 0);
+  const bool mfma_ok = (filter_mc != nullptr) && (cin_total % pmul == 0) &&
+                       mie_conv_mfma_takes(k, stride, dtype_of<T>(), c1, c2, cout);
   MIE_REQUIRE(path == MIE_PATH_AUTO || path == MIE_PATH_VALU || path == MIE_PATH_MFMA,
               MIE_ERR_INVALID_ARG, "%s: unknown path %d", who, path);
   MIE_REQUIRE(path != MIE_PATH_MFMA || mfma_ok, MIE_ERR_UNSUPPORTED,
-              "%s: MFMA path needs filter_mc (mie_pack_filter), c1 %% %d == 0, c2 %% %d == 0, cout %% %d == 0 "
-              "(filter_mc=%p c1=%d c2=%d cout=%d)", who, imul, imul, cmul, (const void*)filter_mc, c1, c2, cout);
+              "%s: MFMA path needs filter_mc (mie_pack_filter) and channel counts in whole staging chunks "
+              "and output slabs for k=%d stride=%d (filter_mc=%p c1=%d c2=%d cout=%d)", who, k, stride,
+              (const void*)filter_mc, c1, c2, cout);
   if (path == MIE_PATH_AUTO) path = mfma_ok ? MIE_PATH_MFMA : MIE_PATH_VALU;
 
   ConvArgsT<T> a;

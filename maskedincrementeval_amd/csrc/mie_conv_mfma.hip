@@ -34,11 +34,16 @@ namespace {
 
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-// Channels staged in LDS per chunk, by kernel size and stride (bounded by 64 KB of LDS for
-// two staging buffers of (7*S+K)^2 pixels).
-__host__ __device__ constexpr int stage_channels(int K, int S) {
-  return (S == 1) ? (K <= 5 ? 32 : 16) : (K <= 5 ? 16 : 8);
+// fp32 channels staged in LDS per chunk (bf16: twice as many), by kernel size and stride, bounded
+// by 64 KB of LDS.  Stride 1 double-buffers the staged tile of (7+K)^2 pixels.  Stride 2 tiles
+// are (14+K)^2 pixels: they are single-buffered (the next chunk waits in registers and is
+// stored between two barriers), which affords the same depth as stride 1 -- and with it the
+// 4-way k-split that fills the chip on planes of a few dozen tiles; HALF is the shallower
+// variant for channel counts that are not a multiple of the full depth.
+__host__ __device__ constexpr int stage_channels(int K, int S, bool HALF = false) {
+  return ((K <= 5) ? 32 : 16) / (HALF ? 2 : 1);
 }
+__host__ __device__ constexpr int stage_buffers(int S) { return S == 1 ? 2 : 1; }
 
 // LDS dwords per row of the staged input tile.  The 16-byte operand reads of 16 neighbouring lanes
 // (8 pixels of one tile row and of the next) must fall on 64 distinct banks: the pixel stride
@@ -77,13 +82,14 @@ __device__ __forceinline__ void mma_unit(v16f& acc, const float4& av, const floa
                                                 __builtin_bit_cast(mie_bf16x8, b4), acc, 0, 0, 0);
 }
 
-template <typename T, int K, int S, int WN, int NB>
+template <typename T, int K, int S, int WN, int NB, bool HALF>
 __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
+  constexpr int NBUF = stage_buffers(S);
   constexpr int EPS = 16 / (int)sizeof(T);                   // elements per 16-byte slot (4 / 8)
   constexpr int SUB = 2 * EPS;                               // channels per unit (8 / 16)
   constexpr int WK = 4 / WN;
   constexpr int IT = 7 * S + K;                              // input tile edge incl. halo
-  constexpr int CC = stage_channels(K, S) * (4 / (int)sizeof(T));   // channels per LDS stage
+  constexpr int CC = stage_channels(K, S, HALF) * (4 / (int)sizeof(T));   // channels per LDS stage
   constexpr int LS = CC + EPS;                               // LDS elements per staged pixel
   constexpr int NPIX = IT * IT;
   constexpr int Q4 = CC / EPS;                               // 16-byte slots per pixel
@@ -99,7 +105,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   constexpr int PD = RING - 1;                               // prefetch distance in units
   constexpr int CO_BLK = 32 * NB * WN;
   constexpr int RED = (WK > 1) ? WK * 64 * CO_BLK : 0;
-  constexpr int STAGE_F = 2 * STAGE * (int)sizeof(T) / 4;     // both staging buffers, in floats
+  constexpr int STAGE_F = NBUF * STAGE * (int)sizeof(T) / 4;  // the staging buffers, in floats
   constexpr int SMEM = (STAGE_F > RED) ? STAGE_F : RED;
   static_assert(SMEM * 4 <= 65536, "LDS budget");
   __shared__ __attribute__((aligned(16))) float smem[SMEM];
@@ -245,7 +251,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
     const int cn = more ? c + 1 : c;      // after the last chunk: redundant re-load, never stored
     ub_next = chunk_b(cn);
     stage_load(cn);
-    const T* sin = sbuf + (c & 1) * STAGE;
+    const T* sin = sbuf + (c % NBUF) * STAGE;
     // A operands are read one unit ahead as well (two register sets); the scheduling barriers
     // pin "issue the loads for later units, then multiply this unit" so that the compiler can
     // neither sink the prefetches next to their uses nor hoist them all to the top.
@@ -276,7 +282,8 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
       __builtin_amdgcn_sched_barrier(0);
       if (PD == 0) load_b(ub_next, 0, bring[0]);   // ring of one: reload right after use
     }
-    if (more) stage_store((c + 1) & 1);
+    if (NBUF == 1) __syncthreads();        // every wave is done reading the only buffer
+    if (more) stage_store((c + 1) % NBUF);
     __syncthreads();
     ub_cur = ub_next;
   }
@@ -339,40 +346,37 @@ int forced_slab() {
   return v;
 }
 
-template <int K, int S>
+template <int K, int S, bool HALF>
 int pick_slab(int cout, unsigned cap) {
-  constexpr int NQ = stage_channels(K, S) / 8;
-  const bool ok256 = cout % 256 == 0, ok128 = cout % 128 == 0, ok64 = NQ >= 2 && cout % 64 == 0;
+  constexpr int NQ = stage_channels(K, S, HALF) / 8;
+  const bool ok128 = cout % 128 == 0, ok64 = NQ >= 2 && cout % 64 == 0;
   const bool ok32 = NQ >= 4 && cout % 32 == 0;
   const int f = forced_slab();
-  if ((f == 256 && ok256) || (f == 128 && ok128) || (f == 64 && ok64) || (f == 32 && ok32)) return f;
+  if ((f == 128 && ok128) || (f == 64 && ok64) || (f == 32 && ok32)) return f;
   const long long want = 400;
   if (ok128 && ((long long)cap * (cout / 128) >= want || (!ok64 && !ok32))) return 128;
   if (ok64 && ((long long)cap * (cout / 64) >= want || !ok32)) return 64;
   if (ok32) return 32;
-  return ok128 ? 128 : 0;
+  return 0;
 }
 
-template <typename T, int K, int S>
-bool launch_ks(const ConvArgsT<T>& a, unsigned cap, hipStream_t st) {
-  constexpr int NQ = stage_channels(K, S) / 8;
+template <typename T, int K, int S, bool HALF>
+bool launch_depth(const ConvArgsT<T>& a, unsigned cap, hipStream_t st) {
+  constexpr int NQ = stage_channels(K, S, HALF) / 8;
   const int cout = a.cout;
-  switch (pick_slab<K, S>(cout, cap)) {
-    case 256:
-      hipLaunchKernelGGL((k_conv_mfma<T, K, S, 4, 2>), dim3(cap, cout / 256), dim3(256), 0, st, a);
-      return true;
+  switch (pick_slab<K, S, HALF>(cout, cap)) {
     case 128:
-      hipLaunchKernelGGL((k_conv_mfma<T, K, S, 4, 1>), dim3(cap, cout / 128), dim3(256), 0, st, a);
+      hipLaunchKernelGGL((k_conv_mfma<T, K, S, 4, 1, HALF>), dim3(cap, cout / 128), dim3(256), 0, st, a);
       return true;
     case 64:
       if constexpr (NQ >= 2) {
-        hipLaunchKernelGGL((k_conv_mfma<T, K, S, 2, 1>), dim3(cap, cout / 64), dim3(256), 0, st, a);
+        hipLaunchKernelGGL((k_conv_mfma<T, K, S, 2, 1, HALF>), dim3(cap, cout / 64), dim3(256), 0, st, a);
         return true;
       }
       return false;
     case 32:
       if constexpr (NQ >= 4) {
-        hipLaunchKernelGGL((k_conv_mfma<T, K, S, 1, 1>), dim3(cap, cout / 32), dim3(256), 0, st, a);
+        hipLaunchKernelGGL((k_conv_mfma<T, K, S, 1, 1, HALF>), dim3(cap, cout / 32), dim3(256), 0, st, a);
         return true;
       }
       return false;
@@ -381,17 +385,33 @@ bool launch_ks(const ConvArgsT<T>& a, unsigned cap, hipStream_t st) {
   }
 }
 
-}  // namespace
-
-// Input channels staged per chunk: c1 and c2 must be multiples of it.
-int mie_conv_mfma_cin_multiple(int k, int s, int dtype) {
-  return stage_channels(k, s) * (dtype == MIE_DTYPE_BF16 ? 2 : 1);
+// Staging depth: the full one when both inputs' channel counts are multiples of it, else
+// (stride 2 only) the half one.
+template <typename T, int K, int S>
+bool launch_ks(const ConvArgsT<T>& a, unsigned cap, hipStream_t st) {
+  constexpr int MULT = 4 / (int)sizeof(T);
+  constexpr int FULL = stage_channels(K, S) * MULT;
+  if (a.c1 % FULL == 0 && a.c2 % FULL == 0 && pick_slab<K, S, false>(a.cout, cap) != 0)
+    return launch_depth<T, K, S, false>(a, cap, st);
+  if constexpr (S == 2) {
+    constexpr int HALFC = stage_channels(K, S, true) * MULT;
+    if (a.c1 % HALFC == 0 && a.c2 % HALFC == 0) return launch_depth<T, K, S, true>(a, cap, st);
+  }
+  return false;
 }
 
-// Smallest output-channel multiple the matrix-core path takes for (k, s).
-int mie_conv_mfma_cout_multiple(int k, int s) {
-  const int nq = stage_channels(k, s) / 8;
-  return nq >= 4 ? 32 : (nq >= 2 ? 64 : 128);
+}  // namespace
+
+// Whether some kernel variant takes the shape: whole staging chunks of input channels (stride 2
+// may fall back to the half depth) and whole output slabs for the wave splits that depth allows.
+bool mie_conv_mfma_takes(int k, int s, int dtype, int c1, int c2, int cout) {
+  const int mult = dtype == MIE_DTYPE_BF16 ? 2 : 1;
+  for (int half = 0; half < (s == 2 ? 2 : 1); ++half) {
+    const int cc = stage_channels(k, s, half != 0), depth = cc * mult, nq = cc / 8;
+    const int cmul = nq >= 4 ? 32 : (nq >= 2 ? 64 : 128);
+    if (c1 % depth == 0 && c2 % depth == 0 && cout % cmul == 0) return true;
+  }
+  return false;
 }
 
 namespace {

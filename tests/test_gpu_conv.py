@@ -57,12 +57,15 @@ PATHS = [("valu", _lib.PATH_VALU), ("mfma", _lib.PATH_MFMA)]
 
 
 def _mfma_takes(k, s, cin, cout):
-    """Shapes the matrix-core path takes: whole staging chunks of input channels
-    (32 for stride 1, 16 for stride 2, halved for 7x7) and whole 32-channel output slabs
-    per wave split the chunk depth allows."""
-    cc = (32 if k <= 5 else 16) if s == 1 else (16 if k <= 5 else 8)
-    cmul = {4: 32, 2: 64, 1: 128}[cc // 8]
-    return cin % cc == 0 and cout % cmul == 0
+    """Shapes the matrix-core path takes (fp32): whole staging chunks of input channels (32, or 16
+    for 7x7; stride 2 may fall back to half of that) and whole output slabs for the wave splits
+    the chunk depth allows (32 / 64 / 128 for 4 / 2 / 1 sub-chunks of 8 channels)."""
+    for half in ((False, True) if s == 2 else (False,)):
+        cc = (32 if k <= 5 else 16) // (2 if half else 1)
+        cmul = {4: 32, 2: 64, 1: 128}[cc // 8]
+        if cin % cc == 0 and cout % cmul == 0:
+            return True
+    return False
 
 
 @pytest.mark.parametrize("pname,path", PATHS)
