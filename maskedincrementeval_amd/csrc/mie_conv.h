@@ -37,6 +37,40 @@ static __device__ __forceinline__ void conv_store(const ConvArgsT<T>& a, long lo
   }
 }
 
+// The same epilogue for N elements of one thread: every reservoir / addend load is issued before
+// the first store, so the loads overlap instead of each waiting for the store before it (the
+// buffers carry no restrict qualifiers: a store may alias a later load as far as the compiler
+// knows).  Elements with ok[i] == false are skipped.
+template <typename T, int N>
+static __device__ __forceinline__ void conv_store_batch(const ConvArgsT<T>& a, const long long (&off)[N],
+                                                        const int (&co)[N], const bool (&ok)[N],
+                                                        float (&acc)[N]) {
+  float r0[N];
+  const bool want_res = a.res != nullptr && !a.refresh;
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    r0[i] = 0.f;
+    if (ok[i]) {
+      if (a.addend) acc[i] += mie_ld(a.addend, off[i]);
+      if (want_res) r0[i] = a.res[off[i]];
+      if (a.refresh && a.bias) acc[i] += a.bias[co[i]];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    if (!ok[i]) continue;
+    if (a.refresh) {
+      if (a.res) a.res[off[i]] = acc[i];
+      mie_st(a.out, off[i], mie_act(a.act, a.slope, acc[i]));
+    } else if (a.res) {
+      const float r1 = r0[i] + acc[i];
+      a.res[off[i]] = r1;
+      mie_st(a.out, off[i], mie_act(a.act, a.slope, r1) - mie_act(a.act, a.slope, r0[i]));
+    } else {
+      mie_st(a.out, off[i], acc[i]);
+    }
+  }
+}
 
 // Launches the matrix-core path for kernel size k (1,3,5,7) and stride s (1,2).  Returns false
 // if no kernel variant takes the shape (nothing is launched then); mie_conv_mfma_takes says so

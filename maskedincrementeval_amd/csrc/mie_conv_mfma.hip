@@ -294,16 +294,26 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   // channel column wn*32*NB + 32*nb + lane%32 of the workgroup's slab.
   if (WK == 1) {
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb)
+    for (int mb = 0; mb < 2; ++mb) {
+      long long off[16 * NB];
+      int co[16 * NB];
+      bool ok[16 * NB];
+      float v[16 * NB];
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int p = mb * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
         const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
-        if (oy >= hout || ox >= wout) continue;
         const long long ob = (((long long)n * hout + oy) * wout + ox) * a.cout + cob;
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) conv_store(a, ob + nb * 32, cob + nb * 32, acc[mb][nb][r]);
+        for (int nb = 0; nb < NB; ++nb) {
+          off[r * NB + nb] = ob + nb * 32;
+          co[r * NB + nb] = cob + nb * 32;
+          ok[r * NB + nb] = oy < hout && ox < wout;
+          v[r * NB + nb] = acc[mb][nb][r];
+        }
       }
+      conv_store_batch<T, 16 * NB>(a, off, co, ok, v);
+    }
   } else {
     // the trailing barrier of the main loop has retired every read of the staging buffers
     float* red = smem + wk * (64 * CO_BLK);
@@ -317,15 +327,25 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
           red[p * CO_BLK + wn * (32 * NB) + nb * 32 + l32] = acc[mb][nb][r];
       }
     __syncthreads();
-    for (int idx = tid; idx < 64 * CO_BLK; idx += 256) {
+    constexpr int PER = 64 * CO_BLK / 256;     // output elements per thread
+    long long off[PER];
+    int co[PER];
+    bool ok[PER];
+    float v[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int idx = tid + 256 * i;
       const int p = idx / CO_BLK, col = idx - p * CO_BLK;
       const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
-      if (oy >= hout || ox >= wout) continue;
-      float s = smem[idx];
+      ok[i] = oy < hout && ox < wout;
+      off[i] = (((long long)n * hout + oy) * wout + ox) * a.cout + co0 + col;
+      co[i] = co0 + col;
+      float sum = smem[idx];
 #pragma unroll
-      for (int k2 = 1; k2 < WK; ++k2) s += smem[k2 * (64 * CO_BLK) + idx];
-      conv_store(a, (((long long)n * hout + oy) * wout + ox) * a.cout + co0 + col, co0 + col, s);
+      for (int k2 = 1; k2 < WK; ++k2) sum += smem[k2 * (64 * CO_BLK) + idx];
+      v[i] = sum;
     }
+    conv_store_batch<T, PER>(a, off, co, ok, v);
   }
 }
 
