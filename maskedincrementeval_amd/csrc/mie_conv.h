@@ -1,5 +1,5 @@
 // Arguments shared by the masked-conv kernels (VALU paths in mie_conv.hip, matrix-core
-// path in mie_conv_mfma.hip).
+// path in mie_conv_mfma_impl.h).
 #pragma once
 #include "mie_common.h"
 

@@ -2,7 +2,7 @@
 //
 // Three code paths, one per arithmetic regime:
 //   mfma    : Cin % 32 == 0 (16 for stride 2) and Cout % 32 == 0 -- per-tile implicit GEMM on
-//             the fp32 matrix cores (mie_conv_mfma.hip).
+//             the matrix cores (mie_conv_mfma_impl.h).
 //   valu    : any shape -- thread = one output channel x 16 pixels, input tile
 //             staged in LDS and read as wave-wide broadcasts.
 //   smallco : Cout <= 4 (prediction / flow heads) -- thread = one pixel.

@@ -1,3 +1,6 @@
+// Kernel and launch templates of the matrix-core conv path, included by one translation unit per
+// element type (mie_conv_mfma_f32.hip, mie_conv_mfma_bf16.hip) so that they compile in parallel.
+//
 // Masked conv on the matrix cores, gfx950: fp32 deltas with v_mfma_f32_32x32x2_f32, bf16 deltas
 // with v_mfma_f32_32x32x16_bf16 (fp32 accumulation, fp32 reservoirs).  The two element types share
 // one kernel: every operand access is a 16-byte access, which holds 4 fp32 or 8 bf16 channels, so
@@ -27,6 +30,7 @@
 // 4+j of the high half; the B operand is loaded with the same pairing).  The
 // LDS row stride CC+4 floats keeps the 16-byte reads of 8 neighbouring pixels
 // on disjoint banks for stride 1 and 2.
+#pragma once
 #include "mie_conv.h"
 #include <stdlib.h>
 
@@ -422,18 +426,6 @@ bool launch_ks(const ConvArgsT<T>& a, unsigned cap, hipStream_t st) {
 
 }  // namespace
 
-// Whether some kernel variant takes the shape: whole staging chunks of input channels (stride 2
-// may fall back to the half depth) and whole output slabs for the wave splits that depth allows.
-bool mie_conv_mfma_takes(int k, int s, int dtype, int c1, int c2, int cout) {
-  const int mult = dtype == MIE_DTYPE_BF16 ? 2 : 1;
-  for (int half = 0; half < (s == 2 ? 2 : 1); ++half) {
-    const int cc = stage_channels(k, s, half != 0), depth = cc * mult, nq = cc / 8;
-    const int cmul = nq >= 4 ? 32 : (nq >= 2 ? 64 : 128);
-    if (c1 % depth == 0 && c2 % depth == 0 && cout % cmul == 0) return true;
-  }
-  return false;
-}
-
 namespace {
 template <typename T>
 bool launch_any(const ConvArgsT<T>& a, int k, int s, unsigned cap, hipStream_t st) {
@@ -451,9 +443,3 @@ bool launch_any(const ConvArgsT<T>& a, int k, int s, unsigned cap, hipStream_t s
 }
 }  // namespace
 
-bool mie_launch_conv_mfma(const ConvArgsT<float>& a, int k, int s, unsigned cap, hipStream_t st) {
-  return launch_any<float>(a, k, s, cap, st);
-}
-bool mie_launch_conv_mfma(const ConvArgsT<mie_bf16>& a, int k, int s, unsigned cap, hipStream_t st) {
-  return launch_any<mie_bf16>(a, k, s, cap, st);
-}
