@@ -25,6 +25,34 @@ template <> struct Vec<4> {
   __device__ static Vec zero() { Vec r; r.v = make_float4(0.f, 0.f, 0.f, 0.f); return r; }
   __device__ float& operator[](int i) { return (&v.x)[i]; }
 };
+// 8 channels: one 16-byte access of a bf16 delta, two of an fp32 buffer
+template <> struct Vec<8> {
+  float v[8];
+  __device__ static Vec load(const float* p) {
+    const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+    Vec r; r.v[0] = a.x; r.v[1] = a.y; r.v[2] = a.z; r.v[3] = a.w; r.v[4] = b.x; r.v[5] = b.y; r.v[6] = b.z; r.v[7] = b.w;
+    return r;
+  }
+  __device__ void store(float* p) const {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+  }
+  __device__ static Vec load(const mie_bf16* p) {
+    const mie_bf16x8 b = *reinterpret_cast<const mie_bf16x8*>(p);
+    Vec r;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r.v[i] = (float)b[i];
+    return r;
+  }
+  __device__ void store(mie_bf16* p) const {
+    mie_bf16x8 b;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) b[i] = (mie_bf16)v[i];
+    *reinterpret_cast<mie_bf16x8*>(p) = b;
+  }
+  __device__ static Vec zero() { Vec r; for (int i = 0; i < 8; ++i) r.v[i] = 0.f; return r; }
+  __device__ float& operator[](int i) { return v[i]; }
+};
 template <> struct Vec<1> {
   float v;
   __device__ static Vec load(const float* p) { Vec r; r.v = *p; return r; }
@@ -362,20 +390,25 @@ int check_pointwise(const char* who, const mie_tileset* ts, int c) {
 
 // Launches KERN<T, VEC> with T from `dtype` and VEC = 4 when c % 4 == 0, else 1.  The kernel
 // arguments are built by ARGS, a macro-local expression list that may use T.
-#define MIE_LAUNCH_POINTWISE(KERN, dtype, c, grid, ny4, ny1, stream, ...)                                   \
+// Launches KERN<T, VEC> with T from `dtype`; VEC = 8 for bf16 deltas with c % 8 == 0 (16-byte
+// delta accesses), else 4 when c % 4 == 0, else 1.  SPLIT: whether the channel vectors of a tile
+// may be spread over gridDim.y.  The kernel arguments may use T.
+#define MIE_LAUNCH_VEC(KERN, T_, VEC_, c, grid, SPLIT, stream, ...)                                        \
+  do {                                                                                                    \
+    using T = T_;                                                                                         \
+    const unsigned ny_ = (SPLIT) ? channel_splits((int)(grid), (c) / (VEC_)) : 1u;                        \
+    hipLaunchKernelGGL((KERN<T, VEC_>), dim3(grid, ny_), dim3(256), 0, (hipStream_t)(stream), __VA_ARGS__); \
+  } while (0)
+
+#define MIE_LAUNCH_POINTWISE(KERN, dtype, c, grid, SPLIT, stream, ...)                                     \
   do {                                                                                                    \
     if ((dtype) == MIE_DTYPE_BF16) {                                                                      \
-      using T = mie_bf16;                                                                                 \
-      if (((c) & 3) == 0)                                                                                 \
-        hipLaunchKernelGGL((KERN<T, 4>), dim3(grid, ny4), dim3(256), 0, (hipStream_t)(stream), __VA_ARGS__); \
-      else                                                                                                \
-        hipLaunchKernelGGL((KERN<T, 1>), dim3(grid, ny1), dim3(256), 0, (hipStream_t)(stream), __VA_ARGS__); \
+      if (((c) & 7) == 0) MIE_LAUNCH_VEC(KERN, mie_bf16, 8, c, grid, SPLIT, stream, __VA_ARGS__);         \
+      else if (((c) & 3) == 0) MIE_LAUNCH_VEC(KERN, mie_bf16, 4, c, grid, SPLIT, stream, __VA_ARGS__);    \
+      else MIE_LAUNCH_VEC(KERN, mie_bf16, 1, c, grid, SPLIT, stream, __VA_ARGS__);                        \
     } else {                                                                                              \
-      using T = float;                                                                                    \
-      if (((c) & 3) == 0)                                                                                 \
-        hipLaunchKernelGGL((KERN<T, 4>), dim3(grid, ny4), dim3(256), 0, (hipStream_t)(stream), __VA_ARGS__); \
-      else                                                                                                \
-        hipLaunchKernelGGL((KERN<T, 1>), dim3(grid, ny1), dim3(256), 0, (hipStream_t)(stream), __VA_ARGS__); \
+      if (((c) & 3) == 0) MIE_LAUNCH_VEC(KERN, float, 4, c, grid, SPLIT, stream, __VA_ARGS__);            \
+      else MIE_LAUNCH_VEC(KERN, float, 1, c, grid, SPLIT, stream, __VA_ARGS__);                           \
     }                                                                                                     \
   } while (0)
 
@@ -402,8 +435,7 @@ extern "C" int mie_act_incr(int act_kind, float slope, const void* in_delta, flo
   const TileSetDev d = mie_dev_tileset(ts);
   const unsigned grid = (unsigned)mie_tile_capacity(ts->n, ts->h, ts->w);
   // the refined mask is an any-over-channels inside one block: no channel split then
-  const unsigned ny = out_pixmask ? 1u : channel_splits((int)grid, (c & 3) ? c : c / 4);
-  MIE_LAUNCH_POINTWISE(k_act_incr, dtype, c, grid, ny, ny, stream, d, act_kind, slope, (const T*)in_delta,
+  MIE_LAUNCH_POINTWISE(k_act_incr, dtype, c, grid, out_pixmask == nullptr, stream, d, act_kind, slope, (const T*)in_delta,
                        reservoir, (T*)out_delta, c, out_pixmask, keep);
   return mie_check_launch(who);
 }
@@ -426,8 +458,7 @@ extern "C" int mie_kfence_incr(const void* in_delta, float* carry, const float* 
   MIE_REQUIRE(mie_aligned(k_dev, 4), MIE_ERR_INVALID_ARG, "%s: k_dev must be 4-byte aligned", who);
   const TileSetDev d = mie_dev_tileset(ts);
   const unsigned grid = (unsigned)mie_tile_capacity(ts->n, ts->h, ts->w);
-  const unsigned ny = out_pixmask ? 1u : channel_splits((int)grid, (c & 3) ? c : c / 4);
-  MIE_LAUNCH_POINTWISE(k_kfence_incr, dtype, c, grid, ny, ny, stream, d, k_dev, k_host, (const T*)in_delta,
+  MIE_LAUNCH_POINTWISE(k_kfence_incr, dtype, c, grid, out_pixmask == nullptr, stream, d, k_dev, k_host, (const T*)in_delta,
                        carry, (T*)out_delta, c, out_pixmask);
   return mie_check_launch(who);
 }
@@ -446,8 +477,7 @@ extern "C" int mie_mul_incr(const void* d1, const uint8_t* m1, float* r1, const 
   const int keep = (flags & MIE_FLAG_KEEP_RESERVOIR) ? 1 : 0;
   const TileSetDev d = mie_dev_tileset(ts);
   const unsigned grid = (unsigned)mie_tile_capacity(ts->n, ts->h, ts->w);
-  MIE_LAUNCH_POINTWISE(k_mul_incr, dtype, c, grid, channel_splits((int)grid, c / 4),
-                       channel_splits((int)grid, c), stream, d, (const T*)d1, m1, r1, (const T*)d2, m2, r2,
+  MIE_LAUNCH_POINTWISE(k_mul_incr, dtype, c, grid, true, stream, d, (const T*)d1, m1, r1, (const T*)d2, m2, r2,
                        (T*)out_delta, c, keep);
   return mie_check_launch(who);
 }
@@ -463,8 +493,7 @@ extern "C" int mie_add_incr(const void* a, const uint8_t* ma, const void* b, con
   MIE_PTR16(a, who, "a"); MIE_PTR16(b, who, "b"); MIE_PTR16(out_delta, who, "out_delta");
   const TileSetDev d = mie_dev_tileset(ts);
   const unsigned grid = (unsigned)mie_tile_capacity(ts->n, ts->h, ts->w);
-  MIE_LAUNCH_POINTWISE(k_add_incr, dtype, c, grid, channel_splits((int)grid, c / 4),
-                       channel_splits((int)grid, c), stream, d, (const T*)a, ma, (const T*)b, mb,
+  MIE_LAUNCH_POINTWISE(k_add_incr, dtype, c, grid, true, stream, d, (const T*)a, ma, (const T*)b, mb,
                        (T*)out_delta, c);
   return mie_check_launch(who);
 }
@@ -485,8 +514,7 @@ extern "C" int mie_upsample2x_incr(const void* a, const uint8_t* ma, const void*
   MIE_PTR16(a, who, "a"); MIE_PTR16(b, who, "b"); MIE_PTR16(out_delta, who, "out_delta");
   const TileSetDev d = mie_dev_tileset(out);
   const unsigned grid = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
-  MIE_LAUNCH_POINTWISE(k_up2x_incr, dtype, c, grid, channel_splits((int)grid, c / 4),
-                       channel_splits((int)grid, c), stream, d, (const T*)a, ma, (const T*)b, mb, h_in, w_in,
+  MIE_LAUNCH_POINTWISE(k_up2x_incr, dtype, c, grid, true, stream, d, (const T*)a, ma, (const T*)b, mb, h_in, w_in,
                        (T*)out_delta, c);
   return mie_check_launch(who);
 }
@@ -511,8 +539,7 @@ extern "C" int mie_convlstm_gates_incr(const void* gates_delta, float* gates_res
   MIE_PTR16(c_delta, who, "c_delta");
   const TileSetDev d = mie_dev_tileset(ts);
   const unsigned grid = (unsigned)mie_tile_capacity(ts->n, ts->h, ts->w);
-  MIE_LAUNCH_POINTWISE(k_convlstm_gates, dtype, hid, grid, channel_splits((int)grid, hid / 4),
-                       channel_splits((int)grid, hid), stream, d, (const T*)gates_delta, gates_res,
+  MIE_LAUNCH_POINTWISE(k_convlstm_gates, dtype, hid, grid, true, stream, d, (const T*)gates_delta, gates_res,
                        (const T*)cprev_delta, cprev_mask, cprev_res, cell_res, (T*)h_delta, (T*)c_delta, hid);
   return mie_check_launch(who);
 }
