@@ -130,6 +130,9 @@ class LayerProbe:
                 if d["kind"] == "gates":
                     hid = c // 4
                     byts = a * (4 * hid * self.es + 2 * 4 * hid * 4 + 2 * hid * 4 + hid * 4 + 2 * hid * self.es)
+                elif d["kind"] == "up2x":
+                    # the two inputs live at a quarter of the output pixels: counted once each
+                    byts = a * c * self.es * (1 + d["nin"] / 4.0)
                 else:
                     byts = a * c * (self.es * (d["nin"] + 1) + 8 * d["nres"])
                 byts += ts.n * ts.h * ts.w

@@ -407,7 +407,8 @@ int check_pointwise(const char* who, const mie_tileset* ts, int c) {
       else if (((c) & 3) == 0) MIE_LAUNCH_VEC(KERN, mie_bf16, 4, c, grid, SPLIT, stream, __VA_ARGS__);    \
       else MIE_LAUNCH_VEC(KERN, mie_bf16, 1, c, grid, SPLIT, stream, __VA_ARGS__);                        \
     } else {                                                                                              \
-      if (((c) & 3) == 0) MIE_LAUNCH_VEC(KERN, float, 4, c, grid, SPLIT, stream, __VA_ARGS__);            \
+      if (((c) & 7) == 0 && (c) >= 64) MIE_LAUNCH_VEC(KERN, float, 8, c, grid, SPLIT, stream, __VA_ARGS__); \
+      else if (((c) & 3) == 0) MIE_LAUNCH_VEC(KERN, float, 4, c, grid, SPLIT, stream, __VA_ARGS__);       \
       else MIE_LAUNCH_VEC(KERN, float, 1, c, grid, SPLIT, stream, __VA_ARGS__);                           \
     }                                                                                                     \
   } while (0)
