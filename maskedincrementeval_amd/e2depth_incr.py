@@ -460,8 +460,12 @@ class UNetRecurrentIncr(BaseUNetIncr):
             x_incr = resblock(x_incr)
         for i, decoder in enumerate(self.decoders):
             x_incr = decoder(x_incr, blocks[self.num_encoders - i - 1])
-        pred_incr = self.pred(self.pred_add(x_incr, head))
-        pred_incr = self.activation(pred_incr)
+        summed = self.pred_add(x_incr, head)
+        if self.fuse and self.norm not in ['BN', 'IN']:
+            # 1x1 conv and output activation in one kernel (the pre-activation reservoir is the activation's)
+            pred_incr = self.pred.conv2d.forward_fused(summed, self.activation)
+        else:
+            pred_incr = self.activation(self.pred(summed))
         return pred_incr, states_incr
 
     def forward_refresh_reservoirs(self, x: DenseT, prev_states):
@@ -479,8 +483,11 @@ class UNetRecurrentIncr(BaseUNetIncr):
             x = resblock.forward_refresh_reservoirs(x)
         for i, decoder in enumerate(self.decoders):
             x = decoder.forward_refresh_reservoirs(x, blocks[self.num_encoders - i - 1])
-        pred = self.pred.forward_refresh_reservoirs(self.pred_add.forward_refresh_reservoirs(x, head))
-        pred = self.activation.forward_refresh_reservoirs(pred)
+        summed = self.pred_add.forward_refresh_reservoirs(x, head)
+        if self.fuse and self.norm not in ['BN', 'IN'] and summed.is_cuda:
+            pred = self.pred.conv2d.forward_refresh_fused(summed, self.activation)
+        else:
+            pred = self.activation.forward_refresh_reservoirs(self.pred.forward_refresh_reservoirs(summed))
         return pred, states
 
 
