@@ -331,6 +331,20 @@ int mie_tconv_masked(const void* x, const uint8_t* xmask, int cin, int h_in,
                      void* stream);
 
 /*
+ * Dense refresh twin of mie_tconv_masked, as mie_conv_refresh is of
+ * mie_conv_masked: out_dense = act(tconv(x) + bias) over the active tiles of
+ * `out` (build it with in_mask = NULL: every tile), reservoir (optional) = the
+ * pre-activation.
+ * Replaces: the conv_transpose2d + bias of TransposedConvLayerIncr's refresh
+ * (incr_modules/e2depth_incr.py:275-282).
+ */
+int mie_tconv_refresh(const void* x, int cin, int h_in, int w_in,
+                      const float* filter, int k, int stride, int pad, int cout,
+                      const float* bias, const mie_tileset* out, void* out_dense,
+                      float* reservoir, int act_kind, float slope, int dtype,
+                      void* stream);
+
+/*
  * Event front end: scatter raw events into a frame, or directly into the DELTA
  * between the frames of two time windows, in the layout the network consumes.
  *   events : [n_events][4] doubles (t, x, y, p), the reference's .npy row

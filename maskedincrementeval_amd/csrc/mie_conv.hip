@@ -341,12 +341,14 @@ namespace {
 template <typename T>
 int tconv_impl(const char* who, const T* x, const uint8_t* xmask, int cin, int h_in, int w_in,
                const float* filter, int k, int stride, int pad, int cout, const mie_tileset* out,
-               T* out_delta, float* reservoir, int act_kind, float slope, void* stream) {
+               T* out_delta, float* reservoir, int act_kind, float slope, bool refresh,
+               const float* bias, void* stream) {
   ConvArgsT<T> a;
   a.x = x; a.xm = xmask; a.c1 = cin; a.x2 = nullptr; a.x2m = nullptr; a.c2 = 0;
   a.h_in = h_in; a.w_in = w_in; a.filt = filter; a.cin_total = cin; a.filt_mc = nullptr;
   a.pad = pad; a.cout = cout; a.out = out_delta; a.res = reservoir; a.act = act_kind;
-  a.slope = slope; a.addend = nullptr; a.refresh = 0; a.bias = nullptr; a.ts = mie_dev_tileset(out);
+  a.slope = slope; a.addend = nullptr; a.refresh = refresh ? 1 : 0; a.bias = bias;
+  a.ts = mie_dev_tileset(out);
   const unsigned cap = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
   hipLaunchKernelGGL(k_tconv_valu<T>, dim3(cap, mie_div_up(cout, 64)), dim3(256), 0,
                      (hipStream_t)stream, a, k, stride);
@@ -424,11 +426,11 @@ extern "C" int mie_conv_refresh(const void* x, int c1, const void* x2, int c2, i
                       (const T*)addend, reservoir, act_kind, slope, path, true, bias, stream);
 }
 
-extern "C" int mie_tconv_masked(const void* x, const uint8_t* xmask, int cin, int h_in,
-                                int w_in, const float* filter, int k, int stride, int pad,
-                                int cout, const mie_tileset* out, void* out_delta,
-                                float* reservoir, int act_kind, float slope, int dtype, void* stream) {
-  const char* who = "mie_tconv_masked";
+namespace {
+int tconv_entry(const char* who, const void* x, const uint8_t* xmask, int cin, int h_in, int w_in,
+                const float* filter, int k, int stride, int pad, int cout, const mie_tileset* out,
+                void* out_delta, float* reservoir, int act_kind, float slope, bool refresh,
+                const float* bias, int dtype, void* stream) {
   MIE_CONV_DTYPE_OK(dtype, who);
   int rc = mie_check_tileset(out, who);
   if (rc != MIE_OK) return rc;
@@ -443,13 +445,31 @@ extern "C" int mie_tconv_masked(const void* x, const uint8_t* xmask, int cin, in
               out->w, hmin, wmin);
   MIE_REQUIRE((long long)out->n * h_in * w_in < 0x7fffffffLL, MIE_ERR_CAPACITY,
               "%s: input too large", who);
-  MIE_REQUIRE(mie_aligned(x, 16) && mie_aligned(filter, 16), MIE_ERR_INVALID_ARG,
-              "%s: x / filter must be 16-byte aligned", who);
-  rc = check_epilogue(who, out_delta, reservoir, act_kind);
+  MIE_REQUIRE(mie_aligned(x, 16) && mie_aligned(filter, 16) && mie_aligned(bias, 4), MIE_ERR_INVALID_ARG,
+              "%s: x / filter must be 16-byte, bias 4-byte aligned", who);
+  rc = check_epilogue(who, out_delta, reservoir, act_kind, refresh);
   if (rc != MIE_OK) return rc;
   if (dtype == MIE_DTYPE_BF16)
     return tconv_impl<mie_bf16>(who, (const mie_bf16*)x, xmask, cin, h_in, w_in, filter, k, stride, pad,
-                                cout, out, (mie_bf16*)out_delta, reservoir, act_kind, slope, stream);
+                                cout, out, (mie_bf16*)out_delta, reservoir, act_kind, slope, refresh, bias,
+                                stream);
   return tconv_impl<float>(who, (const float*)x, xmask, cin, h_in, w_in, filter, k, stride, pad, cout,
-                           out, (float*)out_delta, reservoir, act_kind, slope, stream);
+                           out, (float*)out_delta, reservoir, act_kind, slope, refresh, bias, stream);
+}
+}  // namespace
+
+extern "C" int mie_tconv_masked(const void* x, const uint8_t* xmask, int cin, int h_in,
+                                int w_in, const float* filter, int k, int stride, int pad,
+                                int cout, const mie_tileset* out, void* out_delta,
+                                float* reservoir, int act_kind, float slope, int dtype, void* stream) {
+  return tconv_entry("mie_tconv_masked", x, xmask, cin, h_in, w_in, filter, k, stride, pad, cout, out,
+                     out_delta, reservoir, act_kind, slope, false, nullptr, dtype, stream);
+}
+
+extern "C" int mie_tconv_refresh(const void* x, int cin, int h_in, int w_in, const float* filter,
+                                 int k, int stride, int pad, int cout, const float* bias,
+                                 const mie_tileset* out, void* out_dense, float* reservoir,
+                                 int act_kind, float slope, int dtype, void* stream) {
+  return tconv_entry("mie_tconv_refresh", x, nullptr, cin, h_in, w_in, filter, k, stride, pad, cout, out,
+                     out_dense, reservoir, act_kind, slope, true, bias, dtype, stream);
 }

@@ -98,9 +98,9 @@ static inline unsigned channel_splits(int cap, int cv) {
 // ---- activation increment -----------------------------------------------------
 template <typename T, int VEC>
 __global__ __launch_bounds__(256) void k_act_incr(TileSetDev ts, int kind, float slope,
-                                                  const T* __restrict__ din,
+                                                  const T* din,     // may alias dout (in place)
                                                   float* __restrict__ res,
-                                                  T* __restrict__ dout, int c,
+                                                  T* dout, int c,
                                                   uint8_t* __restrict__ out_mask, int keep) {
   __shared__ unsigned s_any[64];
   int n, y0, x0;
@@ -150,9 +150,9 @@ __global__ __launch_bounds__(256) void k_act_incr(TileSetDev ts, int kind, float
 // same expression evaluated op by op on the host.
 template <typename T, int VEC>
 __global__ __launch_bounds__(256) void k_kfence_incr(TileSetDev ts, const float* __restrict__ k_dev,
-                                                     float k_host, const T* __restrict__ din,
+                                                     float k_host, const T* din,   // may alias dout
                                                      float* __restrict__ carry,
-                                                     T* __restrict__ dout, int c,
+                                                     T* dout, int c,
                                                      uint8_t* __restrict__ out_mask) {
   __shared__ unsigned s_any[64];
   int n, y0, x0;

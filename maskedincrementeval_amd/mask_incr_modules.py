@@ -487,8 +487,21 @@ class nnConvTranspose2dIncr(nn.ConvTranspose2d, _IncrBuffers):
         return [out, ts]
 
     def forward_refresh_reservoirs(self, x):
+        """conv_transpose2d(x, W, b) through the same kernel with every tile active (CPU tensors take
+        the torch op: nothing of this package computes on the CPU)."""
         self._reset_incr()
-        return nn.ConvTranspose2d.forward(self, x)
+        if not x.is_cuda:
+            return nn.ConvTranspose2d.forward(self, x)
+        k = _square(self.kernel_size, "kernel_size")
+        s, p = _square(self.stride, "stride"), _square(self.padding, "padding")
+        op = _square(self.output_padding, "output_padding")
+        x = ops.as_nhwc(x)
+        n, _, h, w = x.shape
+        ho, wo = (h - 1) * s - 2 * p + k + op, (w - 1) * s - 2 * p + k + op
+        ts = self._dense_tile_set(n, ho, wo, x.device)
+        out = self._dense_buf("refresh_out", (n, self.out_channels, ho, wo), x.device, x.dtype)
+        bias = None if self.bias is None else self.bias.detach()
+        return ops.tconv_refresh(x, self._filter(), bias, k, s, p, ts, out)
 
 
 class nnBatchNorm2dIncr(nn.BatchNorm2d):

@@ -323,6 +323,26 @@ def tconv_masked(x, xmask, filt, k, stride, pad, out_ts: TileMask, out_delta, re
     return out_delta
 
 
+def tconv_refresh(x, filt, bias, k, stride, pad, out_ts: TileMask, out_dense, reservoir=None,
+                  act=_lib.ACT_NONE, slope=0.0):
+    """Dense transposed conv + bias (+ activation, + reservoir fill) over the tiles of out_ts (all active)."""
+    n, cin, h, w = x.shape
+    if filt.dim() != 4 or filt.shape[0] != cin or filt.shape[1] != k or not filt.is_contiguous():
+        raise ValueError("filter must be contiguous [Cin,%d,%d,Cout], got %s" % (k, k, tuple(filt.shape)))
+    _require_gpu(filt, "filter")
+    cout = filt.shape[3]
+    if tuple(out_dense.shape) != (n, cout, out_ts.h, out_ts.w):
+        raise ValueError("out_dense shape %s" % (tuple(out_dense.shape),))
+    if bias is not None and (bias.numel() != cout or bias.dtype != torch.float32 or not bias.is_contiguous()):
+        raise ValueError("bias must be contiguous fp32 of %d elements" % cout)
+    _ready(out_ts)
+    check(lib().mie_tconv_refresh(
+        nhwc_ptr(x, "x", dtype=x.dtype), cin, h, w, filt.data_ptr(), k, stride, pad, cout,
+        None if bias is None else bias.data_ptr(), out_ts.ref, nhwc_ptr(out_dense, "out_dense", dtype=x.dtype),
+        nhwc_ptr(reservoir, "reservoir"), act, float(slope), delta_dtype(x), _stream(x)))
+    return out_dense
+
+
 def _same_shape(name, t, ref):
     if t.shape != ref.shape:
         raise ValueError("%s shape %s != %s" % (name, tuple(t.shape), tuple(ref.shape)))

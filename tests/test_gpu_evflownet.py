@@ -88,3 +88,33 @@ def test_evflownet_config4_moving_edges_and_dense_identity():
         dense = fresh.forward_refresh_reservoirs(_cl(x))
     for a, b in zip(acc, dense):
         _close(a, b.cpu(), "refresh + increments vs dense", atol=5e-5)
+
+
+@pytest.mark.parametrize("decoder", ["upsample", "transposed"])
+def test_evflownet_bf16_matches_fp32_oracle(decoder):
+    # bf16 deltas and weights, fp32 reservoirs: every flow scale within rtol 2e-2 of its range (tanh output)
+    h, w = 64, 96
+    bf = torch.bfloat16
+    model = seed_module_(MultiResUNetRecurrentIncr(num_bins=4, decoder=decoder), seed=51).to(DEV).eval()
+    oracle = EVFlowNetOracle(model.state_dict(), decoder=decoder)
+    x0 = torch.randn(1, 4, h, w, generator=torch.Generator().manual_seed(52)) * 0.5
+    with torch.no_grad():
+        acc = [p.float().clone() for p in model.forward_refresh_reservoirs(_cl(x0).to(bf))]
+    acc_ref = oracle.refresh(x0)
+    for a, b in zip(acc, acc_ref):
+        _close(a, b, "refresh", rtol=2e-2, atol=2e-2)
+    for step in range(3):
+        d, m = gaussian_delta(1, 4, h, w, 0.05, 0.3, seed=5400 + step)
+        with torch.no_grad():
+            preds = model([_cl(d).to(bf), None])
+        torch.cuda.synchronize()
+        ref = oracle.incr(d)
+        for s, (a, b) in enumerate(zip(preds, ref)):
+            assert a[0].dtype == bf
+            # a step's delta is a small difference of tanh outputs (|d| < 1e-2 here): held to 5 % of the
+            # step's largest value; the accumulated flow below to 2e-2 of the tanh range
+            _close(a[0].float(), b, "step %d scale %d" % (step, s), rtol=2e-2, atol=5e-2 * max(b.abs().max().item(), 1e-3))
+        acc = [a + p[0].float() for a, p in zip(acc, preds)]
+        acc_ref = [a + b for a, b in zip(acc_ref, ref)]
+    for a, b in zip(acc, acc_ref):
+        _close(a, b, "accumulated", rtol=2e-2, atol=2e-2)

@@ -232,3 +232,31 @@ def test_e2depth_incr_full_size_matches_oracle_and_dense():
     with torch.no_grad():
         dense = fresh.forward_refresh_reservoirs(_cl(x), None)[0]
     _close(acc, dense.cpu(), "refresh + increments vs dense", atol=5e-5)
+
+
+def test_e2depth_incr_empty_frames_between_active_ones():
+    # a frame without any event: every tile list is empty, every output exactly zero, reservoirs
+    # untouched; the frame after it clears the stale tiles of the frame before (clean-delta invariant)
+    h, w = 72, 104
+    model = seed_module_(E2VIDRecurrentIncr(), seed=31).to(DEV).eval()
+    oracle = E2DepthOracle(model.state_dict())
+    x0 = torch.randn(1, 5, h, w, generator=torch.Generator().manual_seed(32)) * 0.5
+    with torch.no_grad():
+        model.forward_refresh_reservoirs(_cl(x0), None)
+    oracle.refresh(x0)
+    zero = torch.zeros(1, 5, h, w)
+    frames = [event_voxel_delta(1, 5, h, w, 0.05, seed=1)[0], zero, zero, event_voxel_delta(1, 5, h, w, 0.02, seed=2)[0]]
+    for i, d in enumerate(frames):
+        with torch.no_grad():
+            out, _ = model([_cl(d), None], None)
+        torch.cuda.synchronize()
+        ref = oracle.incr(d)
+        _close(out[0], ref, "frame %d" % i)
+        if not d.any():
+            assert torch.count_nonzero(out[0]) == 0 and out[1].active_tiles().numel() == 0
+            assert torch.count_nonzero(ref) == 0
+    # every persistent delta buffer is zero outside the active pixels of its tile set after the last frame
+    head = model.unetrecurrent.head.conv2d
+    buf = head._delta_buf("out_act", (1, 32, h, w), torch.device(DEV))
+    ts = head._tile_set("out_act", 1, h, w, torch.device(DEV))
+    assert torch.count_nonzero(buf * (1 - ts.pixmask.float())) == 0
