@@ -89,7 +89,14 @@ class LayerProbe:
                 t0 = [t for t in a if hasattr(t, "shape") and len(getattr(t, "shape", ())) == 4][0]
                 return dict(kind=kind, c=t0.shape[1], ts=ts, nin=nin, nres=nres)
             return d
+        def conv_gates_desc(x, xmask, x2, x2mask, filt, out_ts, *a, **kw):
+            n, c1, h, w = x.shape
+            c2 = 0 if x2 is None else x2.shape[1]
+            return dict(kind="conv", k=3, s=1, cin=c1 + c2, cout=filt.shape[3], h=h, w=w, n=n,
+                        xmask=xmask, x2mask=x2mask, ts=out_ts, fused=True, gates=True)
+
         self._wrap("conv_masked", conv_desc)
+        self._wrap("conv_gates_incr", conv_gates_desc)
         self._wrap("act_incr", pw_desc("act", 1, 1))
         self._wrap("add_incr", pw_desc("add", 2, 0))
         self._wrap("mul_incr", pw_desc("mul", 2, 2))
@@ -117,10 +124,18 @@ class LayerProbe:
                 a_out = int(ts.pixmask.sum().item())
                 cin, cout, k = d["cin"], d["cout"], d["k"]
                 es = self.es
-                byts = P + a_in * cin * es + a_out * cout * es + cin * cout * k * k * es + ts.capacity * 4
-                if d["fused"]:
-                    byts += 2 * a_out * cout * 4
-                row.update(shape="%dx%d s%d %d->%d @%dx%d" % (k, k, d["s"], cin, cout, ts.h, ts.w),
+                byts = P + a_in * cin * es + cin * cout * k * k * es + ts.capacity * 4
+                if d.get("gates"):
+                    # gate reservoirs read + written, cell reservoir read + written, previous cell read,
+                    # hidden and cell deltas written; the 4*hid-channel gate delta never reaches memory
+                    hid = cout // 4
+                    byts += a_out * (2 * cout * 4 + 2 * hid * 4 + hid * 4 + 2 * hid * es)
+                else:
+                    byts += a_out * cout * es
+                    if d["fused"]:
+                        byts += 2 * a_out * cout * 4
+                row.update(shape="%dx%d s%d %d->%d%s @%dx%d" % (k, k, d["s"], cin, cout,
+                                                                 "+lstm" if d.get("gates") else "", ts.h, ts.w),
                            active_tiles=int(ts.counts[0].item()), tiles=ts.capacity, a_out=a_out,
                            bytes=byts, flops=2 * a_out * cin * cout * k * k)
             elif d["kind"] in ("act", "add", "mul", "up2x", "gates"):
@@ -247,7 +262,7 @@ def main():
                            gbs=round(byts / (ms * 1e-3) / 1e9, 1) if ms > 0 else None,
                            tflops=round(fl / (ms * 1e-3) / 1e12, 2) if ms > 0 else None,
                            bytes=int(byts), flops=int(fl), active_tiles=r.get("active_tiles"), tiles=r.get("tiles")))
-    convs = [l for l in layers if l["op"] == "conv_masked"]
+    convs = [l for l in layers if l["op"] in ("conv_masked", "conv_gates_incr")]
     dom = max(convs, key=lambda l: l["us"])
     # Re-time the dominant launch on its own: the same call (same tile set, same buffers)
     # replayed back to back between two HIP events on the launch stream.

@@ -315,6 +315,34 @@ int mie_convlstm_gates_incr(const void* gates_delta, float* gates_res,
                             int dtype, void* stream);
 
 /*
+ * The gates conv of a ConvLSTM and its gate chain in ONE kernel: the 3x3,
+ * stride 1, pad 1 conv of mie_conv_masked (x ++ x2 -> 4*hid channels) whose
+ * epilogue is mie_convlstm_gates_incr, so that the 4*hid-channel gate delta is
+ * never written to memory.  Matrix-core path only: needs filter_mc, c1 and c2
+ * in whole staging chunks (32 channels fp32, 64 bf16) and hid % 8 == 0;
+ * otherwise MIE_ERR_UNSUPPORTED (use the two calls then).
+ *   filter / filter_mc / gates_res : the 4*hid output columns are NOT in the
+ *     order [in | remember | out | cell] x hid of the two-call form but
+ *     interleaved by gate in groups of 8 hidden channels: column
+ *     32*b + 8*g + j  <->  gate g of hidden channel 8*b + j, so that one
+ *     workgroup owns all four gates of its hidden channels.  gates_res
+ *     ([n,h,w,4*hid]) lives in that order too (a refresh through
+ *     mie_conv_refresh with the same filter and a bias in the same order fills
+ *     it consistently).
+ *   cprev_* / cell_res / h_delta / c_delta ([n,h,w,hid]) as in
+ *     mie_convlstm_gates_incr, plain channel order.
+ * Replaces: incr_modules/e2depth_incr.py:100-120 (cat, conv, chunk, the chain).
+ */
+int mie_conv_gates_masked(const void* x, const uint8_t* xmask, int c1,
+                          const void* x2, const uint8_t* x2mask, int c2,
+                          int h_in, int w_in, const float* filter,
+                          const void* filter_mc, int cin_total, int hid,
+                          const mie_tileset* out, float* gates_res,
+                          const void* cprev_delta, const uint8_t* cprev_mask,
+                          float* cprev_res, float* cell_res, void* h_delta,
+                          void* c_delta, int dtype, void* stream);
+
+/*
  * Masked transposed convolution of a delta (stride s, padding p; the output
  * size out->h/w fixes output_padding): out(oy,ox,co) = sum x(iy,ix,ci) *
  * filter[ci][ky][kx][co] over oy = iy*s - p + ky, ox = ix*s - p + kx, with

@@ -16,6 +16,11 @@ struct ConvArgsT {
   T* out; float* res; int act; float slope;
   const T* addend;                  // optional delta added to the conv result before the epilogue
   int refresh; const float* bias;   // dense refresh: out = act(acc + bias), res = acc + bias
+  // ConvLSTM gate chain fused into the epilogue (matrix-core path, GATES kernels): `res` is the gate
+  // pre-activation reservoir in the conv's column order, `out` is unused; the rest as in
+  // mie_convlstm_gates_incr.
+  int hid;
+  const T* g_cpd; const uint8_t* g_cpm; float* g_cpres; float* g_cres; T* g_dh; T* g_dc;
   TileSetDev ts;
 };
 typedef ConvArgsT<float> ConvArgs;
@@ -77,4 +82,33 @@ static __device__ __forceinline__ void conv_store_batch(const ConvArgsT<T>& a, c
 // beforehand.
 bool mie_launch_conv_mfma(const ConvArgsT<float>& a, int k, int s, unsigned cap, hipStream_t st);
 bool mie_launch_conv_mfma(const ConvArgsT<mie_bf16>& a, int k, int s, unsigned cap, hipStream_t st);
+// The 3x3 stride-1 conv of a ConvLSTM with the gate chain as its epilogue (a.hid > 0, a.cout = 4*hid,
+// filter columns in the gate-interleaved order of mie_conv_gates_masked).
+bool mie_launch_conv_gates_mfma(const ConvArgsT<float>& a, unsigned cap, hipStream_t st);
+bool mie_launch_conv_gates_mfma(const ConvArgsT<mie_bf16>& a, unsigned cap, hipStream_t st);
+
+// One element of the ConvLSTM gate chain: pre-activation gate reservoirs r* and their deltas d*, cached
+// previous cell state cp and its delta dP, cached cell state c0.  Updates the reservoirs in place and
+// returns the deltas of the hidden and the cell state (the chain sigmoid1..3 / tanh1 -> m1 + m2 -> tanh2
+// -> m3 of ConvLSTMIncr.forward, incr_modules/e2depth_incr.py:103-120, product rule on cached operands).
+static __device__ __forceinline__ float mie_sigm(float v) { return 1.f / (1.f + expf(-v)); }
+static __device__ __forceinline__ void mie_lstm_gate_chain(float& ri, float& rf, float& ro, float& rg, float di,
+                                                           float df, float dO, float dG, float& cp, float dP,
+                                                           float& cc, float& dh, float& dc) {
+  const float ri1 = ri + di, rf1 = rf + df, ro1 = ro + dO, rg1 = rg + dG;
+  const float si0 = mie_sigm(ri), dsi = mie_sigm(ri1) - si0;
+  const float sf0 = mie_sigm(rf), dsf = mie_sigm(rf1) - sf0;
+  const float so0 = mie_sigm(ro), dso = mie_sigm(ro1) - so0;
+  const float tg0 = tanhf(rg), dtg = tanhf(rg1) - tg0;
+  const float m1 = (dtg + tg0) * dsi + si0 * dtg;       // m1(in_gate, cell_gate)
+  const float m2 = (dP + cp) * dsf + sf0 * dP;          // m2(remember_gate, prev_c)
+  const float dcell = m1 + m2;
+  const float c0 = cc, c1 = c0 + dcell;
+  const float tc0 = tanhf(c0), dtc = tanhf(c1) - tc0;
+  dh = (dtc + tc0) * dso + so0 * dtc;                   // m3(out_gate, tanh(cell))
+  dc = dcell;
+  ri = ri1; rf = rf1; ro = ro1; rg = rg1;
+  cp += dP;
+  cc = c1;
+}
 bool mie_conv_mfma_takes(int k, int s, int dtype, int c1, int c2, int cout);

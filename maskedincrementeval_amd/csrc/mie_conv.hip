@@ -238,13 +238,22 @@ int check_epilogue(const char* who, const void* out_delta, float* reservoir, int
   return MIE_OK;
 }
 
+// Extra operands of the conv with the ConvLSTM gate chain as its epilogue.
+template <typename T>
+struct GatesOperands {
+  int hid;
+  const T* cprev_delta; const uint8_t* cprev_mask; float* cprev_res; float* cell_res;
+  T* h_delta; T* c_delta;
+};
+
 template <typename T>
 int conv_impl(const char* who, const T* x, const uint8_t* xmask, int c1, const T* x2,
               const uint8_t* x2mask, int c2, int h_in, int w_in, const float* filter,
               const T* filter_mc, int cin_total, int k, int stride, int pad, int cout,
               const mie_tileset* out,
               T* out_delta, const T* addend, float* reservoir, int act_kind, float slope,
-              int path, bool refresh, const float* bias, void* stream) {
+              int path, bool refresh, const float* bias, void* stream,
+              const GatesOperands<T>* gates = nullptr) {
   mie_clear_error();
   int rc = mie_check_tileset(out, who);
   if (rc != MIE_OK) return rc;
@@ -272,8 +281,10 @@ int conv_impl(const char* who, const T* x, const uint8_t* xmask, int c1, const T
               MIE_ERR_CAPACITY, "%s: input too large", who);
   MIE_REQUIRE(mie_aligned(x, 16) && mie_aligned(x2, 16) && mie_aligned(filter, 16),
               MIE_ERR_INVALID_ARG, "%s: x / x2 / filter must be 16-byte aligned", who);
-  rc = check_epilogue(who, out_delta, reservoir, act_kind, refresh);
-  if (rc != MIE_OK) return rc;
+  if (gates == nullptr) {
+    rc = check_epilogue(who, out_delta, reservoir, act_kind, refresh);
+    if (rc != MIE_OK) return rc;
+  }
   MIE_REQUIRE(mie_aligned(bias, 4) && mie_aligned(addend, 16), MIE_ERR_INVALID_ARG,
               "%s: bias must be 4-byte and addend 16-byte aligned", who);
   MIE_REQUIRE(addend == nullptr || addend != out_delta, MIE_ERR_INVALID_ARG,
@@ -295,9 +306,22 @@ int conv_impl(const char* who, const T* x, const uint8_t* xmask, int c1, const T
   a.h_in = h_in; a.w_in = w_in; a.filt = filter; a.cin_total = cin_total; a.filt_mc = filter_mc;
   a.pad = pad; a.cout = cout; a.out = out_delta; a.res = reservoir; a.act = act_kind;
   a.slope = slope; a.addend = addend; a.refresh = refresh ? 1 : 0; a.bias = bias;
+  a.hid = 0; a.g_cpd = nullptr; a.g_cpm = nullptr; a.g_cpres = nullptr; a.g_cres = nullptr;
+  a.g_dh = nullptr; a.g_dc = nullptr;
   a.ts = mie_dev_tileset(out);
   const unsigned cap = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
   hipStream_t st = (hipStream_t)stream;
+  if (gates != nullptr) {
+    MIE_REQUIRE(mfma_ok && gates->hid % 8 == 0 && cout == 4 * gates->hid, MIE_ERR_UNSUPPORTED,
+                "%s: needs filter_mc, whole 32-channel (bf16: 64) input chunks and hid %% 8 == 0 "
+                "(c1=%d c2=%d hid=%d)", who, c1, c2, gates->hid);
+    a.hid = gates->hid; a.g_cpd = gates->cprev_delta; a.g_cpm = gates->cprev_mask;
+    a.g_cpres = gates->cprev_res; a.g_cres = gates->cell_res; a.g_dh = gates->h_delta;
+    a.g_dc = gates->c_delta;
+    MIE_REQUIRE(mie_launch_conv_gates_mfma(a, cap, st), MIE_ERR_UNSUPPORTED,
+                "%s: no kernel variant for cout=%d", who, cout);
+    return mie_check_launch(who);
+  }
   if (path == MIE_PATH_MFMA) {
     MIE_REQUIRE(mie_launch_conv_mfma(a, k, stride, cap, st), MIE_ERR_UNSUPPORTED,
                 "%s: no MFMA kernel variant for k=%d stride=%d cout=%d", who, k, stride, cout);
@@ -348,6 +372,8 @@ int tconv_impl(const char* who, const T* x, const uint8_t* xmask, int cin, int h
   a.h_in = h_in; a.w_in = w_in; a.filt = filter; a.cin_total = cin; a.filt_mc = nullptr;
   a.pad = pad; a.cout = cout; a.out = out_delta; a.res = reservoir; a.act = act_kind;
   a.slope = slope; a.addend = nullptr; a.refresh = refresh ? 1 : 0; a.bias = bias;
+  a.hid = 0; a.g_cpd = nullptr; a.g_cpm = nullptr; a.g_cpres = nullptr; a.g_cres = nullptr;
+  a.g_dh = nullptr; a.g_dc = nullptr;
   a.ts = mie_dev_tileset(out);
   const unsigned cap = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
   hipLaunchKernelGGL(k_tconv_valu<T>, dim3(cap, mie_div_up(cout, 64)), dim3(256), 0,
@@ -427,6 +453,28 @@ extern "C" int mie_conv_refresh(const void* x, int c1, const void* x2, int c2, i
 }
 
 namespace {
+template <typename T>
+int conv_gates_entry(const char* who, const void* x, const uint8_t* xmask, int c1, const void* x2,
+                     const uint8_t* x2mask, int c2, int h_in, int w_in, const float* filter,
+                     const void* filter_mc, int cin_total, int hid, const mie_tileset* out,
+                     float* gates_res, const void* cprev_delta, const uint8_t* cprev_mask,
+                     float* cprev_res, float* cell_res, void* h_delta, void* c_delta, void* stream) {
+  MIE_REQUIRE(hid > 0 && hid <= (1 << 20), MIE_ERR_INVALID_ARG, "%s: hid = %d out of range", who, hid);
+  MIE_REQUIRE(gates_res && cprev_res && cell_res && h_delta && c_delta, MIE_ERR_INVALID_ARG,
+              "%s: NULL pointer", who);
+  MIE_REQUIRE(cprev_delta != nullptr || cprev_mask == nullptr, MIE_ERR_INVALID_ARG,
+              "%s: mask of absent cprev_delta", who);
+  MIE_REQUIRE(mie_aligned(gates_res, 16) && mie_aligned(cprev_delta, 16) && mie_aligned(cprev_res, 16) &&
+                  mie_aligned(cell_res, 16) && mie_aligned(h_delta, 16) && mie_aligned(c_delta, 16),
+              MIE_ERR_INVALID_ARG, "%s: buffers must be 16-byte aligned", who);
+  GatesOperands<T> g;
+  g.hid = hid; g.cprev_delta = (const T*)cprev_delta; g.cprev_mask = cprev_mask; g.cprev_res = cprev_res;
+  g.cell_res = cell_res; g.h_delta = (T*)h_delta; g.c_delta = (T*)c_delta;
+  return conv_impl<T>(who, (const T*)x, xmask, c1, (const T*)x2, x2mask, c2, h_in, w_in, filter,
+                      (const T*)filter_mc, cin_total, 3, 1, 1, 4 * hid, out, (T*)nullptr, (const T*)nullptr,
+                      gates_res, MIE_ACT_NONE, 0.f, MIE_PATH_MFMA, false, nullptr, stream, &g);
+}
+
 int tconv_entry(const char* who, const void* x, const uint8_t* xmask, int cin, int h_in, int w_in,
                 const float* filter, int k, int stride, int pad, int cout, const mie_tileset* out,
                 void* out_delta, float* reservoir, int act_kind, float slope, bool refresh,
@@ -472,4 +520,22 @@ extern "C" int mie_tconv_refresh(const void* x, int cin, int h_in, int w_in, con
                                  int act_kind, float slope, int dtype, void* stream) {
   return tconv_entry("mie_tconv_refresh", x, nullptr, cin, h_in, w_in, filter, k, stride, pad, cout, out,
                      out_dense, reservoir, act_kind, slope, true, bias, dtype, stream);
+}
+
+extern "C" int mie_conv_gates_masked(const void* x, const uint8_t* xmask, int c1, const void* x2,
+                                     const uint8_t* x2mask, int c2, int h_in, int w_in,
+                                     const float* filter, const void* filter_mc, int cin_total,
+                                     int hid, const mie_tileset* out, float* gates_res,
+                                     const void* cprev_delta, const uint8_t* cprev_mask,
+                                     float* cprev_res, float* cell_res, void* h_delta,
+                                     void* c_delta, int dtype, void* stream) {
+  const char* who = "mie_conv_gates_masked";
+  MIE_CONV_DTYPE_OK(dtype, who);
+  if (dtype == MIE_DTYPE_BF16)
+    return conv_gates_entry<mie_bf16>(who, x, xmask, c1, x2, x2mask, c2, h_in, w_in, filter, filter_mc,
+                                      cin_total, hid, out, gates_res, cprev_delta, cprev_mask, cprev_res,
+                                      cell_res, h_delta, c_delta, stream);
+  return conv_gates_entry<float>(who, x, xmask, c1, x2, x2mask, c2, h_in, w_in, filter, filter_mc, cin_total,
+                                 hid, out, gates_res, cprev_delta, cprev_mask, cprev_res, cell_res, h_delta,
+                                 c_delta, stream);
 }

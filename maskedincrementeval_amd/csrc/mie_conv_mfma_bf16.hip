@@ -4,3 +4,6 @@
 bool mie_launch_conv_mfma(const ConvArgsT<mie_bf16>& a, int k, int s, unsigned cap, hipStream_t st) {
   return launch_any<mie_bf16>(a, k, s, cap, st);
 }
+bool mie_launch_conv_gates_mfma(const ConvArgsT<mie_bf16>& a, unsigned cap, hipStream_t st) {
+  return launch_gates<mie_bf16>(a, cap, st);
+}

@@ -16,3 +16,6 @@ bool mie_conv_mfma_takes(int k, int s, int dtype, int c1, int c2, int cout) {
 bool mie_launch_conv_mfma(const ConvArgsT<float>& a, int k, int s, unsigned cap, hipStream_t st) {
   return launch_any<float>(a, k, s, cap, st);
 }
+bool mie_launch_conv_gates_mfma(const ConvArgsT<float>& a, unsigned cap, hipStream_t st) {
+  return launch_gates<float>(a, cap, st);
+}

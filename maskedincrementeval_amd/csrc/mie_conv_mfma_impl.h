@@ -86,7 +86,7 @@ __device__ __forceinline__ void mma_unit(v16f& acc, const float4& av, const floa
                                                 __builtin_bit_cast(mie_bf16x8, b4), acc, 0, 0, 0);
 }
 
-template <typename T, int K, int S, int WN, int NB, bool HALF>
+template <typename T, int K, int S, int WN, int NB, bool HALF, bool GATES = false>
 __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   constexpr int NBUF = stage_buffers(S);
   constexpr int EPS = 16 / (int)sizeof(T);                   // elements per 16-byte slot (4 / 8)
@@ -108,7 +108,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   constexpr int RING = ring_size(UPC);                       // B operand ring (divides UPC)
   constexpr int PD = RING - 1;                               // prefetch distance in units
   constexpr int CO_BLK = 32 * NB * WN;
-  constexpr int RED = (WK > 1) ? WK * 64 * CO_BLK : 0;
+  constexpr int RED = (WK > 1 || GATES) ? WK * 64 * CO_BLK : 0;
   constexpr int STAGE_F = NBUF * STAGE * (int)sizeof(T) / 4;  // the staging buffers, in floats
   constexpr int SMEM = (STAGE_F > RED) ? STAGE_F : RED;
   static_assert(SMEM * 4 <= 65536, "LDS budget");
@@ -127,6 +127,19 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   const int hout = a.ts.h, wout = a.ts.w;
   const int cout = a.cout;
 
+  if (GATES && tk == 2) {  // stale tile: zero the hidden / cell deltas of this workgroup's hidden channels
+    constexpr int HC = CO_BLK / 4;
+    for (int idx = tid; idx < 64 * HC; idx += 256) {
+      const int p = idx / HC, hc = idx - p * HC;
+      const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
+      if (oy < hout && ox < wout) {
+        const long long o = (((long long)n * hout + oy) * wout + ox) * a.hid + co0 / 4 + hc;
+        mie_st(a.g_dh, o, 0.f);
+        mie_st(a.g_dc, o, 0.f);
+      }
+    }
+    return;
+  }
   if (tk == 2) {  // stale tile: zero this workgroup's channel slab
     for (int idx = tid; idx < 64 * CO_BLK; idx += 256) {
       const int p = idx / CO_BLK, col = idx - p * CO_BLK;
@@ -296,7 +309,61 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   // ---- epilogue -----------------------------------------------------------------------------------
   // acc[mb][nb][r] of this lane is output pixel p = 32*mb + 8*(r/4) + 4*half + r%4,
   // channel column wn*32*NB + 32*nb + lane%32 of the workgroup's slab.
-  if (WK == 1) {
+  if constexpr (GATES) {
+    // ConvLSTM gate chain as the epilogue.  The filter columns of a slab are interleaved by gate in
+    // groups of 8 hidden channels: column 32*b + 8*g + j of the slab is gate g (in, remember, out,
+    // cell) of hidden channel 8*b + j, so a workgroup owns all four gates of its CO_BLK/4 hidden
+    // channels.  Every wave parks its accumulators in LDS; a thread then sums the k-split partials
+    // of the four gate columns of one (pixel, hidden channel) and runs the chain on the reservoirs.
+    float* red = smem + wk * (64 * CO_BLK);
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int p = mb * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+          red[p * CO_BLK + wn * (32 * NB) + nb * 32 + l32] = acc[mb][nb][r];
+      }
+    __syncthreads();
+    constexpr int HC = CO_BLK / 4;             // hidden channels of this workgroup
+    constexpr int PERG = 64 * HC / 256;        // (pixel, hidden channel) items per thread
+    const int hid = a.hid;
+#pragma unroll
+    for (int i = 0; i < PERG; ++i) {
+      const int idx = tid + 256 * i;
+      const int p = idx / HC, hc = idx - p * HC;
+      const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
+      if (oy >= hout || ox >= wout) continue;
+      const long long pix = ((long long)n * hout + oy) * wout + ox;
+      const long long ho = pix * hid + co0 / 4 + hc;
+      if (!a.ts.pixmask[pix]) {               // inactive pixel of an active tile: clean zeros
+        mie_st(a.g_dh, ho, 0.f);
+        mie_st(a.g_dc, ho, 0.f);
+        continue;
+      }
+      const int colb = (hc >> 3) * 32 + (hc & 7);
+      float dg[4];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        float sum = smem[p * CO_BLK + colb + 8 * g];
+#pragma unroll
+        for (int k2 = 1; k2 < WK; ++k2) sum += smem[k2 * (64 * CO_BLK) + p * CO_BLK + colb + 8 * g];
+        dg[g] = sum;
+      }
+      float* gr = a.res + pix * a.cout + co0 + colb;
+      float ri = gr[0], rf = gr[8], ro = gr[16], rg = gr[24];
+      const bool has_cp = a.g_cpd != nullptr && (a.g_cpm == nullptr || a.g_cpm[pix]);
+      const float dP = has_cp ? mie_ld(a.g_cpd, ho) : 0.f;
+      float cp = a.g_cpres[ho], cc = a.g_cres[ho], dh, dc;
+      mie_lstm_gate_chain(ri, rf, ro, rg, dg[0], dg[1], dg[2], dg[3], cp, dP, cc, dh, dc);
+      gr[0] = ri; gr[8] = rf; gr[16] = ro; gr[24] = rg;
+      if (has_cp) a.g_cpres[ho] = cp;
+      a.g_cres[ho] = cc;
+      mie_st(a.g_dh, ho, dh);
+      mie_st(a.g_dc, ho, dc);
+    }
+  } else if (WK == 1) {
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb) {
       long long off[16 * NB];
@@ -404,6 +471,27 @@ bool launch_depth(const ConvArgsT<T>& a, unsigned cap, hipStream_t st) {
         return true;
       }
       return false;
+    default:
+      return false;
+  }
+}
+
+// The gates conv of a ConvLSTM: 3x3, stride 1, full staging depth, gate chain in the epilogue.
+template <typename T>
+bool launch_gates(const ConvArgsT<T>& a, unsigned cap, hipStream_t st) {
+  constexpr int FULL = stage_channels(3, 1) * (4 / (int)sizeof(T));
+  if (a.c1 % FULL != 0 || a.c2 % FULL != 0 || a.cout != 4 * a.hid || a.hid % 8 != 0) return false;
+  const int cout = a.cout;
+  switch (pick_slab<3, 1, false>(cout, cap)) {
+    case 128:
+      hipLaunchKernelGGL((k_conv_mfma<T, 3, 1, 4, 1, false, true>), dim3(cap, cout / 128), dim3(256), 0, st, a);
+      return true;
+    case 64:
+      hipLaunchKernelGGL((k_conv_mfma<T, 3, 1, 2, 1, false, true>), dim3(cap, cout / 64), dim3(256), 0, st, a);
+      return true;
+    case 32:
+      hipLaunchKernelGGL((k_conv_mfma<T, 3, 1, 1, 1, false, true>), dim3(cap, cout / 32), dim3(256), 0, st, a);
+      return true;
     default:
       return false;
   }

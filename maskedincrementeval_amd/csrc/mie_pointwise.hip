@@ -5,6 +5,7 @@
 // channels of the NHWC row (float4 when C % 4 == 0), so a wave reads whole
 // 8-pixel rows of the tile as contiguous segments.
 #include "mie_common.h"
+#include "mie_conv.h"
 
 namespace {
 
@@ -323,7 +324,6 @@ __global__ __launch_bounds__(256) void k_up2x_incr(TileSetDev ts, const T* __res
 }
 
 // ---- fused ConvLSTM gates ------------------------------------------------------
-__device__ __forceinline__ float sigm(float v) { return 1.f / (1.f + expf(-v)); }
 
 template <typename T, int VEC>
 __global__ __launch_bounds__(256) void k_convlstm_gates(
@@ -348,26 +348,9 @@ __global__ __launch_bounds__(256) void k_convlstm_gates(
       Vec<VEC> cp = Vec<VEC>::load(cpres + off);
       Vec<VEC> cc = Vec<VEC>::load(cres + off);
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        const float ri1 = ri[e] + di[e], rf1 = rf[e] + df[e];
-        const float ro1 = ro[e] + dO[e], rg1 = rg[e] + dG[e];
-        const float si0 = sigm(ri[e]), dsi = sigm(ri1) - si0;
-        const float sf0 = sigm(rf[e]), dsf = sigm(rf1) - sf0;
-        const float so0 = sigm(ro[e]), dso = sigm(ro1) - so0;
-        const float tg0 = tanhf(rg[e]), dtg = tanhf(rg1) - tg0;
-        // m1(in_gate, cell_gate) + m2(remember_gate, prev_c), product rule
-        const float m1 = (dtg + tg0) * dsi + si0 * dtg;
-        const float m2 = (dP[e] + cp[e]) * dsf + sf0 * dP[e];
-        const float dcell = m1 + m2;
-        const float c0 = cc[e], c1 = c0 + dcell;
-        const float tc0 = tanhf(c0), dtc = tanhf(c1) - tc0;
-        // m3(out_gate, tanh(cell))
-        oh[e] = (dtc + tc0) * dso + so0 * dtc;
-        oc[e] = dcell;
-        ri[e] = ri1; rf[e] = rf1; ro[e] = ro1; rg[e] = rg1;
-        cp[e] += dP[e];
-        cc[e] = c1;
-      }
+      for (int e = 0; e < VEC; ++e)
+        mie_lstm_gate_chain(ri[e], rf[e], ro[e], rg[e], di[e], df[e], dO[e], dG[e], cp[e], dP[e], cc[e], oh[e],
+                            oc[e]);
       ri.store(gres + goff); rf.store(gres + goff + hid);
       ro.store(gres + goff + 2 * hid); rg.store(gres + goff + 3 * hid);
       if (has_cp) cp.store(cpres + off);

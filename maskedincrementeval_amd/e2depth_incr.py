@@ -121,9 +121,53 @@ class ConvLSTMIncr(nn.Module, _IncrBuffers):
             return self._forward_fused(input_incr, prev_h_incr, prev_c_incr)
         return self._forward_chain(input_incr, prev_h_incr, prev_c_incr)
 
+    # -- gates conv and gate chain in one kernel ------------------------------------------------
+    def _gates_filter(self):
+        """(ConvFilter, bias) of the gates conv in the gate-interleaved column order."""
+        w = self.Gates.weight
+        tag = (w.data_ptr(), w._version, str(w.device))
+        cached = self.__dict__.get("_gates_filt_cache")
+        if cached is None or cached[0] != tag:
+            perm = ops.gate_interleave_index(self.hidden_size, w.device)
+            filt = ops.ConvFilter(w.detach().permute(1, 2, 3, 0)[..., perm].contiguous().float())
+            bias = None if self.Gates.bias is None else self.Gates.bias.detach()[perm].contiguous().float()
+            cached = (tag, filt, bias)
+            self.__dict__["_gates_filt_cache"] = cached
+        return cached[1], cached[2]
+
+    def _one_kernel_ok(self, x, hidden_present: bool) -> bool:
+        """Whether the conv + gate chain kernel takes this cell: matrix-core shapes only."""
+        chunk = ops.mfma_chunk(x.dtype)
+        return (x.is_cuda and self.kernel_size == 3 and self.hidden_size % 8 == 0
+                and self.input_size % chunk == 0 and (not hidden_present or self.hidden_size % chunk == 0)
+                and self.Gates.path != _lib.PATH_VALU)
+
+    def _forward_one_kernel(self, input_incr, prev_h_incr, prev_c_incr):
+        x, pix, _ = _unpack(input_incr)
+        x2 = pix2 = None
+        if prev_h_incr is not None:
+            x2, pix2, _ = _unpack(prev_h_incr)
+        n, _, h, w = x.shape
+        hid = self.hidden_size
+        ts = self.Gates._conv_tile_set("gates", x, pix, x2, pix2, 3, 1, 1)
+        dh = self._delta_buf("h", (n, hid, h, w), x.device, x.dtype)
+        dc = self._delta_buf("c", (n, hid, h, w), x.device, x.dtype)
+        cp = cpm = None
+        if prev_c_incr is not None:
+            cp, cpm, _ = _unpack(prev_c_incr)
+        filt, _ = self._gates_filter()
+        ops.conv_gates_incr(x, pix, x2, pix2, filt, ts, self.gates_res.reservoir, cp, cpm,
+                            self.cprev_res.reservoir, self.cell_res.reservoir, dh, dc)
+        return [dh, ts], [dc, ts]
+
     def _forward_fused(self, input_incr, prev_h_incr, prev_c_incr):
         if self.gates_res.reservoir is None:
             raise RuntimeError("ConvLSTMIncr: call forward_refresh_reservoirs first")
+        if self.__dict__.get("_gates_interleaved", False):
+            if not self._one_kernel_ok(ops.as_nhwc(input_incr[0]), prev_h_incr is not None):
+                raise RuntimeError("ConvLSTMIncr: the reservoirs were refreshed for the one-kernel form, which "
+                                   "does not take this input (dtype / previous hidden state); refresh again")
+            return self._forward_one_kernel(input_incr, prev_h_incr, prev_c_incr)
         gates, ts = self.Gates(input_incr, prev_h_incr)
         n, _, h, w = gates.shape
         hid = self.hidden_size
@@ -173,9 +217,22 @@ class ConvLSTMIncr(nn.Module, _IncrBuffers):
         if self.fused:
             # the fp32 gate pre-activations go straight into their reservoir; the state is
             # computed from them in fp32 and handed on in the dtype of the input
-            self.Gates._refresh_forward(input_, None if zero_state else prev_h, path=self.Gates.path,
-                                        reserve=self.gates_res)
-            in_gate, remember_gate, out_gate, cell_gate = self.gates_res.reservoir.chunk(4, 1)
+            one_kernel = self._one_kernel_ok(input_, True)
+            self.__dict__["_gates_interleaved"] = one_kernel
+            if one_kernel:
+                # reservoir in the gate-interleaved column order of the conv + gate chain kernel
+                filt, bias = self._gates_filter()
+                self.Gates._refresh_forward(input_, None if zero_state else prev_h, path=self.Gates.path,
+                                            reserve=self.gates_res, filt=filt, bias=bias)
+                g = self.gates_res.reservoir
+                n_, _, h_, w_ = g.shape
+                gv = g.permute(0, 2, 3, 1).reshape(n_, h_, w_, self.hidden_size // 8, 4, 8)
+                in_gate, remember_gate, out_gate, cell_gate = (
+                    gv[..., i, :].reshape(n_, h_, w_, self.hidden_size).permute(0, 3, 1, 2) for i in range(4))
+            else:
+                self.Gates._refresh_forward(input_, None if zero_state else prev_h, path=self.Gates.path,
+                                            reserve=self.gates_res)
+                in_gate, remember_gate, out_gate, cell_gate = self.gates_res.reservoir.chunk(4, 1)
             self.cprev_res.update_reservoir(prev_c)
             in_gate, remember_gate = torch.sigmoid(in_gate), torch.sigmoid(remember_gate)
             out_gate, cell_gate = torch.sigmoid(out_gate), torch.tanh(cell_gate)

@@ -320,22 +320,30 @@ class _ConvIncrMixin(_IncrBuffers):
         if k == 1 and s == 1 and p == 0 and x2 is None and isinstance(in_tm, TileMask):
             ts = in_tm            # a 1x1 conv reaches exactly the pixels of its input: same tile set
         else:
-            ts = self._tile_set(out_name, n, ho, wo, x.device)
-            if x2 is None:
-                m1, m2 = pix, None
-            elif pix is None or pix2 is None:      # one input dense -> every tile active
-                m1 = m2 = None
-            else:
-                m1, m2 = pix, pix2
-            ops.build_mask_tiles(m1, m2, n, h, w, _lib.FOOT_CONV, k, s, p, ts)
+            ts = self._conv_tile_set(out_name, x, pix, x2, pix2, k, s, p)
         addend = None if addend_incr is None else ops.as_nhwc(addend_incr[0])
         ops.conv_masked(x, pix, x2, pix2, self.conv2d_weights if filt is None else filt, k, s, p, ts,
                         out, reservoir, act, slope, path, addend)
         return [out, ts]
 
 
+    def _conv_tile_set(self, name, x, pix, x2, pix2, k, s, p) -> TileMask:
+        """Tile set of the conv output for the (one or two) masked inputs, built for this step."""
+        n, _, h, w = x.shape
+        ho, wo = ops.conv_out_size(h, w, k, s, p)
+        ts = self._tile_set(name, n, ho, wo, x.device)
+        if x2 is None:
+            m1, m2 = pix, None
+        elif pix is None or pix2 is None:      # one input dense -> every tile active
+            m1 = m2 = None
+        else:
+            m1, m2 = pix, pix2
+        ops.build_mask_tiles(m1, m2, n, h, w, _lib.FOOT_CONV, k, s, p, ts)
+        return ts
+
     def _refresh_forward(self, x: DenseT, x2: DenseT = None, activation=None, out=None,
-                         path=_lib.PATH_AUTO, addend: DenseT = None, reserve=None) -> DenseT:
+                         path=_lib.PATH_AUTO, addend: DenseT = None, reserve=None, filt=None,
+                         bias=None) -> DenseT:
         """Dense pass: conv2d(cat(x, x2), W, b) through the same kernels with every tile
         active.  With `activation` (an nnReservedActivation) the pre-activation goes straight
         into its reservoir and the activated tensor is returned; with `reserve` (an
@@ -377,8 +385,10 @@ class _ConvIncrMixin(_IncrBuffers):
             if r is None or tuple(r.shape) != shape or r.device != x.device:
                 reserve.reservoir = ops.new_nhwc(*shape, x.device)
             res = reserve.reservoir
-        bias = None if self.bias is None else self.bias.detach()
-        ops.conv_refresh(x, x2, self.conv2d_weights, bias, k, s, p, ts, out, res, kind, slope, path,
+        if filt is None:     # else: filter and bias in another column order, given together
+            filt = self.conv2d_weights
+            bias = None if self.bias is None else self.bias.detach()
+        ops.conv_refresh(x, x2, filt, bias, k, s, p, ts, out, res, kind, slope, path,
                          None if addend is None else ops.as_nhwc(addend))
         return out
 

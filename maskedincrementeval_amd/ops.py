@@ -452,6 +452,45 @@ def convlstm_gates_incr(gates_delta, gates_res, cprev_delta, cprev_mask, cprev_r
     return h_delta, c_delta
 
 
+def gate_interleave_index(hid: int, device=None) -> torch.Tensor:
+    """Column order of the fused gates conv: entry c' (= 32*b + 8*g + j) holds the column g*hid + 8*b + j of
+    the [in | remember | out | cell] x hid order (gate g of hidden channel 8*b + j)."""
+    cp = torch.arange(4 * hid, device=device)
+    return ((cp % 32) // 8) * hid + (cp // 32) * 8 + cp % 8
+
+
+def conv_gates_incr(x, xmask, x2, x2mask, filt: ConvFilter, out_ts: TileMask, gates_res, cprev_delta, cprev_mask,
+                    cprev_res, cell_res, h_delta, c_delta):
+    """3x3 gates conv of a ConvLSTM with the gate chain as its epilogue; `filt` and `gates_res` are in the
+    gate-interleaved column order (gate_interleave_index)."""
+    n, c1, h, w = x.shape
+    c2 = 0 if x2 is None else x2.shape[1]
+    dt = x.dtype
+    plain, mc_ptr = _filter_args(filt, 3, dt)
+    cin_total, cout = plain.shape[0], plain.shape[3]
+    hid = cout // 4
+    if tuple(gates_res.shape) != (n, cout, h, w):
+        raise ValueError("gates_res shape %s, expected %s" % (tuple(gates_res.shape), (n, cout, h, w)))
+    for name, t in (("cprev_res", cprev_res), ("cell_res", cell_res), ("h_delta", h_delta), ("c_delta", c_delta)):
+        if tuple(t.shape) != (n, hid, h, w):
+            raise ValueError("%s shape %s, expected %s" % (name, tuple(t.shape), (n, hid, h, w)))
+    _ready(out_ts)
+    check(lib().mie_conv_gates_masked(
+        nhwc_ptr(x, "x", dtype=dt), pix_ptr(xmask, n, h, w, "xmask"), c1,
+        nhwc_ptr(x2, "x2", dtype=dt), pix_ptr(x2mask, n, h, w, "x2mask"), c2, h, w,
+        plain.data_ptr(), mc_ptr, cin_total, hid, out_ts.ref, nhwc_ptr(gates_res, "gates_res"),
+        nhwc_ptr(cprev_delta, "cprev_delta", dtype=dt), pix_ptr(cprev_mask, n, h, w, "cprev_mask"),
+        nhwc_ptr(cprev_res, "cprev_res"), nhwc_ptr(cell_res, "cell_res"),
+        nhwc_ptr(h_delta, "h_delta", dtype=dt), nhwc_ptr(c_delta, "c_delta", dtype=dt), delta_dtype(x),
+        _stream(x)))
+    return h_delta, c_delta
+
+
+def mfma_chunk(dtype) -> int:
+    """Input channels per staging chunk of the 3x3 / 5x5 stride-1 matrix-core kernels."""
+    return 32 if dtype == torch.float32 else 64
+
+
 def conv_out_size(h, w, k, stride, pad) -> Tuple[int, int]:
     """Output size formula of the reference wrapper (ext/pointops/pointops_functional.py:25-26)."""
     return (h + 2 * pad - k) // stride + 1, (w + 2 * pad - k) // stride + 1

@@ -172,8 +172,10 @@ def test_config2_activation_chain_50_steps(density):
 
 
 @pytest.mark.parametrize("fused", [True, False])
-def test_convlstm_module_matches_oracle(fused):
-    n, cin, hid, h, w = 1, 16, 16, 26, 34
+@pytest.mark.parametrize("cin,hid", [(16, 16), (32, 32), (64, 32)])
+def test_convlstm_module_matches_oracle(fused, cin, hid):
+    # (32, 32) and (64, 32) take the conv + gate chain kernel when fused, (16, 16) the two-kernel form
+    n, h, w = 1, 26, 34
     cell = ConvLSTMIncr(cin, hid, 3, fused=fused).to(DEV).eval()
     seed_module_(cell, 21)
     ref = io.ConvLSTMOracle(cell.Gates.weight.detach().cpu(), cell.Gates.bias.detach().cpu(), hid)
@@ -182,6 +184,7 @@ def test_convlstm_module_matches_oracle(fused):
         h_d, c_d = cell.forward_refresh_reservoirs(_cl(x0), None)
     h_r, c_r = ref.refresh(x0)
     _close(h_d, h_r, "refresh h"), _close(c_d, c_r, "refresh c")
+    assert cell.__dict__.get("_gates_interleaved", False) == (fused and cin % 32 == 0)
     for step in range(4):
         d, m = gaussian_delta(n, cin, h, w, 0.08, 0.3, seed=2300 + step)
         with torch.no_grad():
@@ -260,3 +263,27 @@ def test_e2depth_incr_empty_frames_between_active_ones():
     buf = head._delta_buf("out_act", (1, 32, h, w), torch.device(DEV))
     ts = head._tile_set("out_act", 1, h, w, torch.device(DEV))
     assert torch.count_nonzero(buf * (1 - ts.pixmask.float())) == 0
+
+
+@pytest.mark.parametrize("cin,hid", [(16, 16), (32, 32)])
+def test_convlstm_with_previous_state_deltas(cin, hid):
+    # non-zero refresh state and non-zero deltas of the previous hidden / cell state (the module
+    # signature allows them, incr_modules/e2depth_incr.py:79,98): two-pointer conv input + m2 term
+    n, h, w = 1, 24, 32
+    cell = seed_module_(ConvLSTMIncr(cin, hid, 3, fused=True), 61).to(DEV).eval()
+    ref = io.ConvLSTMOracle(cell.Gates.weight.detach().cpu(), cell.Gates.bias.detach().cpu(), hid)
+    g = torch.Generator().manual_seed(62)
+    x0, h0, c0 = (torch.randn(n, c, h, w, generator=g) * 0.5 for c in (cin, hid, hid))
+    with torch.no_grad():
+        h_d, c_d = cell.forward_refresh_reservoirs(_cl(x0), (_cl(h0), _cl(c0)))
+    h_r, c_r = ref.refresh(x0, (h0, c0))
+    _close(h_d, h_r, "refresh h"), _close(c_d, c_r, "refresh c")
+    for step in range(3):
+        d, m = gaussian_delta(n, cin, h, w, 0.08, 0.3, seed=6300 + step)
+        dhp, mh = gaussian_delta(n, hid, h, w, 0.05, 0.2, seed=6400 + step)
+        dcp, _ = gaussian_delta(n, hid, h, w, 0.05, 0.2, seed=6400 + step)      # same mask as the hidden delta
+        with torch.no_grad():
+            dh, dc = cell([_cl(d), m.to(DEV)], ([_cl(dhp), mh.to(DEV)], [_cl(dcp), mh.to(DEV)]))
+        torch.cuda.synchronize()
+        dh_r, dc_r = ref.incr(d, (dhp, dcp))
+        _close(dh[0], dh_r, "dh %d" % step), _close(dc[0], dc_r, "dc %d" % step)
