@@ -38,7 +38,7 @@ def parse_args():
     ap.add_argument("--height", type=int, default=264)
     ap.add_argument("--width", type=int, default=352)
     ap.add_argument("--batch", type=int, default=1, help="independent event streams per step (8 with 480x640: the batched configuration)")
-    ap.add_argument("--cpu-steps", type=int, default=200, help="incremental steps of the CPU baseline (0 = skip)")
+    ap.add_argument("--cpu-steps", type=int, default=400, help="incremental steps of the CPU baseline (0 = skip)")
     ap.add_argument("--no-graph", action="store_true", help="launch kernels eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-dense", action="store_true", help="skip the all-tiles-active comparator")
     ap.add_argument("--layer-iters", type=int, default=20, help="timed launches per layer for the roofline table")
