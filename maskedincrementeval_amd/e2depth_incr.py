@@ -143,6 +143,8 @@ class ConvLSTMIncr(nn.Module, _IncrBuffers):
                 and self.Gates.path != _lib.PATH_VALU)
 
     def _forward_one_kernel(self, input_incr, prev_h_incr, prev_c_incr):
+        if self.Gates.use_kf:
+            input_incr = self.Gates.kf(input_incr)
         x, pix, _ = _unpack(input_incr)
         x2 = pix2 = None
         if prev_h_incr is not None:
@@ -213,6 +215,8 @@ class ConvLSTMIncr(nn.Module, _IncrBuffers):
             tuple([batch_size, self.hidden_size] + list(spatial_size)) + (input_.dtype,))
         prev_h, prev_c = prev_state
         self._reset_incr()
+        if self.Gates.use_kf:
+            self.Gates.kf.forward_refresh_reservoirs(input_)
         # the concat is never formed: two-pointer conv input, hidden half skipped when it is zero
         if self.fused:
             # the fp32 gate pre-activations go straight into their reservoir; the state is
