@@ -191,26 +191,43 @@ __global__ __launch_bounds__(256) void k_mask_footprint(BuildArgs a) {
 constexpr int COMPACT_THREADS = 1024;
 constexpr int COMPACT_WAVES = COMPACT_THREADS / 64;
 
+// COMPACT_ITEMS candidates per thread and round (element i = start + j * COMPACT_THREADS + tid), so
+// that a plane of tens of thousands of tiles takes a few rounds of two barriers instead of dozens.
+constexpr int COMPACT_ITEMS = 4;
+
 template <typename KeepFn, typename IdFn>
 __device__ int block_compact(int count, KeepFn keep, IdFn id, int32_t* dst, int* s_tot) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   int base = 0;
-  for (int start = 0; start < count; start += COMPACT_THREADS) {
-    const int i = start + threadIdx.x;
-    const bool k = (i < count) && keep(i);
-    const unsigned long long bal = __ballot(k);
-    const int rank = __popcll(bal & ((1ull << lane) - 1ull));
-    if (lane == 0) s_tot[wave] = __popcll(bal);
-    __syncthreads();
-    int off = base, all = 0;
+  for (int start = 0; start < count; start += COMPACT_THREADS * COMPACT_ITEMS) {
+    bool k[COMPACT_ITEMS];
+    int rank[COMPACT_ITEMS];
 #pragma unroll
-    for (int wv = 0; wv < COMPACT_WAVES; ++wv) {
-      const int t = s_tot[wv];
-      if (wv < wave) off += t;
-      all += t;
+    for (int j = 0; j < COMPACT_ITEMS; ++j) {
+      const int i = start + j * COMPACT_THREADS + threadIdx.x;
+      k[j] = (i < count) && keep(i);
+      const unsigned long long bal = __ballot(k[j]);
+      rank[j] = __popcll(bal & ((1ull << lane) - 1ull));
+      if (lane == 0) s_tot[j * COMPACT_WAVES + wave] = __popcll(bal);
     }
-    if (k) dst[off + rank] = id(i);
-    base += all;
+    __syncthreads();
+    // exclusive prefix over the (j, wave) totals in element order: j major, wave minor
+    int off[COMPACT_ITEMS];
+    int run = base;
+#pragma unroll
+    for (int j = 0; j < COMPACT_ITEMS; ++j) {
+      off[j] = run;
+#pragma unroll
+      for (int wv = 0; wv < COMPACT_WAVES; ++wv) {
+        const int t = s_tot[j * COMPACT_WAVES + wv];
+        if (wv < wave) off[j] += t;
+        run += t;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < COMPACT_ITEMS; ++j)
+      if (k[j]) dst[off[j] + rank[j]] = id(start + j * COMPACT_THREADS + threadIdx.x);
+    base = run;
     __syncthreads();
   }
   return base;
@@ -239,7 +256,7 @@ __device__ void compact_lists(const BuildArgs& a, FlagFn flag, int* s_tot) {
 }
 
 __global__ __launch_bounds__(COMPACT_THREADS) void k_compact_tiles(BuildArgs a) {
-  __shared__ int s_tot[COMPACT_WAVES];
+  __shared__ int s_tot[COMPACT_WAVES * COMPACT_ITEMS];
   const uint32_t* flags = a.flags;
   compact_lists(a, [&](int t) { return flags[t] != 0u; }, s_tot);
 }
@@ -249,7 +266,7 @@ __global__ __launch_bounds__(COMPACT_THREADS) void k_compact_tiles(BuildArgs a) 
 constexpr int SMALL_CAP = 32;
 
 __global__ __launch_bounds__(COMPACT_THREADS) void k_build_small(BuildArgs a) {
-  __shared__ int s_tot[COMPACT_WAVES];
+  __shared__ int s_tot[COMPACT_WAVES * COMPACT_ITEMS];
   __shared__ unsigned s_flag[SMALL_CAP];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   for (int tile = wave; tile < a.cap; tile += COMPACT_WAVES) {
