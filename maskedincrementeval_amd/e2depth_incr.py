@@ -545,7 +545,7 @@ class UNetRecurrentIncr(BaseUNetIncr):
         for i, decoder in enumerate(self.decoders):
             x = decoder.forward_refresh_reservoirs(x, blocks[self.num_encoders - i - 1])
         summed = self.pred_add.forward_refresh_reservoirs(x, head)
-        if self.fuse and self.norm not in ['BN', 'IN'] and summed.is_cuda:
+        if self.fuse and self.norm not in ['BN', 'IN']:
             pred = self.pred.conv2d.forward_refresh_fused(summed, self.activation)
         else:
             pred = self.activation.forward_refresh_reservoirs(self.pred.forward_refresh_reservoirs(summed))

@@ -348,21 +348,10 @@ class _ConvIncrMixin(_IncrBuffers):
         active.  With `activation` (an nnReservedActivation) the pre-activation goes straight
         into its reservoir and the activated tensor is returned; with `reserve` (an
         IncrementReserve) the fp32 result is also written into that reservoir.  `out` overrides
-        the result buffer.  CPU tensors take the torch ops (nothing of this package computes on
-        the CPU).
+        the result buffer.  CPU tensors are refused: this package has no CPU path.
         """
         self._reset_incr()
-        if not x.is_cuda:
-            xin = x if x2 is None else torch.cat((x, x2), 1)
-            if xin.shape[1] < self.in_channels:     # absent trailing input (zero hidden state)
-                xin = torch.cat((xin, xin.new_zeros(xin.shape[0], self.in_channels - xin.shape[1],
-                                                    *xin.shape[2:])), 1)
-            y = nn.Conv2d.forward(self, xin)
-            if addend is not None:
-                y = y + addend
-            if reserve is not None:
-                reserve.update_reservoir(y)
-            return y if activation is None else activation.forward_refresh_reservoirs(y)
+        ops._require_gpu(x, "x")
         k, s, p = self._geometry()
         x = ops.as_nhwc(x)
         x2 = None if x2 is None else ops.as_nhwc(x2)
@@ -497,11 +486,9 @@ class nnConvTranspose2dIncr(nn.ConvTranspose2d, _IncrBuffers):
         return [out, ts]
 
     def forward_refresh_reservoirs(self, x):
-        """conv_transpose2d(x, W, b) through the same kernel with every tile active (CPU tensors take
-        the torch op: nothing of this package computes on the CPU)."""
+        """conv_transpose2d(x, W, b) through the same kernel with every tile active."""
         self._reset_incr()
-        if not x.is_cuda:
-            return nn.ConvTranspose2d.forward(self, x)
+        ops._require_gpu(x, "x")
         k = _square(self.kernel_size, "kernel_size")
         s, p = _square(self.stride, "stride"), _square(self.padding, "padding")
         op = _square(self.output_padding, "output_padding")

@@ -189,13 +189,13 @@ def test_e2depth_module_tree_and_shapes():
     assert tuple(sd[u + "decoders.0.conv2d.weight"].shape) == (128, 256, 5, 5)
     assert tuple(sd[u + "decoders.2.conv2d.weight"].shape) == (32, 64, 5, 5)
     assert tuple(sd[u + "pred.conv2d.weight"].shape) == (1, 32, 1, 1)
-    # dense refresh runs on the CPU (torch ops only) and fills the reservoirs
+    # there is no CPU path: CPU tensors are refused loudly, by the refresh as by the incremental forward
     synthetic.seed_module_(net, 3)
     with torch.no_grad():
-        pred, states = net.forward_refresh_reservoirs(torch.randn(1, 5, 16, 24), None)
-    assert pred.shape == (1, 1, 16, 24) and len(states) == 3
-    assert net.unetrecurrent.head.activation.in_res.reservoir.shape == (1, 32, 16, 24)
-    assert net.unetrecurrent.encoders[2].recurrent_block.gates_res.reservoir.shape == (1, 1024, 2, 3)
+        with pytest.raises(RuntimeError, match="no CPU path"):
+            net.forward_refresh_reservoirs(torch.randn(1, 5, 16, 24), None)
+        with pytest.raises(RuntimeError, match="no CPU path"):
+            net([torch.randn(1, 5, 16, 24), None], None)
 
 
 def test_increment_reserve_keeps_pointer():
