@@ -47,7 +47,10 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 __host__ __device__ constexpr int stage_channels(int K, int S, bool HALF = false) {
   return ((K <= 5) ? 32 : 16) / (HALF ? 2 : 1);
 }
-__host__ __device__ constexpr int stage_buffers(int S) { return S == 1 ? 2 : 1; }
+// bf16 tiles are single-buffered at stride 1 as well: a bf16 workgroup spends a few microseconds on
+// the matrix cores, so what hides its latencies is the number of workgroups resident on the CU (LDS
+// per workgroup halves), not the overlap inside one (measured: +10 % on the 8x480x640 decoder conv).
+__host__ __device__ constexpr int stage_buffers(int S, int elem_size) { return (S == 1 && elem_size == 4) ? 2 : 1; }
 
 // LDS dwords per row of the staged input tile.  The 16-byte operand reads of 16 neighbouring lanes
 // (8 pixels of one tile row and of the next) must fall on 64 distinct banks: the pixel stride
@@ -88,7 +91,7 @@ __device__ __forceinline__ void mma_unit(v16f& acc, const float4& av, const floa
 
 template <typename T, int K, int S, int WN, int NB, bool HALF, bool GATES = false>
 __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
-  constexpr int NBUF = stage_buffers(S);
+  constexpr int NBUF = stage_buffers(S, (int)sizeof(T));
   constexpr int EPS = 16 / (int)sizeof(T);                   // elements per 16-byte slot (4 / 8)
   constexpr int SUB = 2 * EPS;                               // channels per unit (8 / 16)
   constexpr int WK = 4 / WN;
