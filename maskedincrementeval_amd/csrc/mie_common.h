@@ -82,13 +82,16 @@ static inline TileSetDev mie_dev_tileset(const mie_tileset* ts) {
 // (n, y0, x0) = batch index and top-left output pixel of the tile.
 __device__ __forceinline__ int mie_pick_tile(const TileSetDev& ts, int b,
                                              int& n, int& y0, int& x0) {
+  const int cap = ts.n * ts.tiles_y * ts.tiles_x;
+  // the list entry is fetched together with the counts (one memory round trip instead of two);
+  // whether it is valid is decided afterwards
+  const int spec = ts.tiles[(b >= 0 && b < cap) ? b : 0];
   const int n_active = ts.counts[MIE_CNT_ACTIVE];
   const int n_stale = ts.counts[MIE_CNT_STALE];
-  const int cap = ts.n * ts.tiles_y * ts.tiles_x;
   if (n_active < 0 || n_stale < 0 || n_active > cap || n_stale > cap) return 0;   // corrupt counts
   int tile, kind;
   if (b < n_active) {
-    tile = ts.tiles[b];
+    tile = spec;
     kind = 1;
   } else if (b < n_active + n_stale) {
     tile = ts.stale[b - n_active];

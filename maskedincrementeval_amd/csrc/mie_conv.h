@@ -42,39 +42,57 @@ static __device__ __forceinline__ void conv_store(const ConvArgsT<T>& a, long lo
   }
 }
 
-// The same epilogue for N elements of one thread: every reservoir / addend load is issued before
-// the first store, so the loads overlap instead of each waiting for the store before it (the
-// buffers carry no restrict qualifiers: a store may alias a later load as far as the compiler
-// knows).  Elements with ok[i] == false are skipped.
+// The same epilogue for N elements of one thread, in two halves.  conv_epilogue_load issues every
+// reservoir / addend load of the thread as one batch; a kernel calls it long before the values are
+// needed (at its very start: an output element belongs to one thread of one workgroup, nobody else
+// touches its reservoir), so their latency hides behind the contraction.  conv_epilogue_store adds
+// the accumulators and writes.  Elements with ok[i] == false are skipped.
 template <typename T, int N>
-static __device__ __forceinline__ void conv_store_batch(const ConvArgsT<T>& a, const long long (&off)[N],
-                                                        const int (&co)[N], const bool (&ok)[N],
-                                                        float (&acc)[N]) {
-  float r0[N];
+static __device__ __forceinline__ void conv_epilogue_load(const ConvArgsT<T>& a, const long long (&off)[N],
+                                                          const bool (&ok)[N], float (&r0)[N],
+                                                          float (&add)[N]) {
   const bool want_res = a.res != nullptr && !a.refresh;
 #pragma unroll
   for (int i = 0; i < N; ++i) {
     r0[i] = 0.f;
+    add[i] = 0.f;
     if (ok[i]) {
-      if (a.addend) acc[i] += mie_ld(a.addend, off[i]);
+      if (a.addend) add[i] = mie_ld(a.addend, off[i]);
       if (want_res) r0[i] = a.res[off[i]];
-      if (a.refresh && a.bias) acc[i] += a.bias[co[i]];
     }
   }
+}
+
+template <typename T, int N>
+static __device__ __forceinline__ void conv_epilogue_store(const ConvArgsT<T>& a, const long long (&off)[N],
+                                                           const int (&co)[N], const bool (&ok)[N],
+                                                           const float (&acc)[N], const float (&r0)[N],
+                                                           const float (&add)[N]) {
 #pragma unroll
   for (int i = 0; i < N; ++i) {
     if (!ok[i]) continue;
+    float v = acc[i] + add[i];
     if (a.refresh) {
-      if (a.res) a.res[off[i]] = acc[i];
-      mie_st(a.out, off[i], mie_act(a.act, a.slope, acc[i]));
+      if (a.bias) v += a.bias[co[i]];
+      if (a.res) a.res[off[i]] = v;
+      mie_st(a.out, off[i], mie_act(a.act, a.slope, v));
     } else if (a.res) {
-      const float r1 = r0[i] + acc[i];
+      const float r1 = r0[i] + v;
       a.res[off[i]] = r1;
       mie_st(a.out, off[i], mie_act(a.act, a.slope, r1) - mie_act(a.act, a.slope, r0[i]));
     } else {
-      mie_st(a.out, off[i], acc[i]);
+      mie_st(a.out, off[i], v);
     }
   }
+}
+
+template <typename T, int N>
+static __device__ __forceinline__ void conv_store_batch(const ConvArgsT<T>& a, const long long (&off)[N],
+                                                        const int (&co)[N], const bool (&ok)[N],
+                                                        float (&acc)[N]) {
+  float r0[N], add[N];
+  conv_epilogue_load<T, N>(a, off, ok, r0, add);
+  conv_epilogue_store<T, N>(a, off, co, ok, acc, r0, add);
 }
 
 // Launches the matrix-core path for kernel size k (1,3,5,7) and stride s (1,2).  Returns false

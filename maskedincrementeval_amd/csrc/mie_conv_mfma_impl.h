@@ -153,6 +153,26 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
     return;
   }
 
+  // k-split kernels: the thread's share of the output (the elements it reduces and stores at the
+  // end) is fixed by its index, so the reservoir / addend values are fetched right away.
+  constexpr int PER = (WK > 1 && !GATES) ? 64 * CO_BLK / 256 : 1;      // output elements per thread
+  long long e_off[PER];
+  int e_co[PER];
+  bool e_ok[PER];
+  float e_r0[PER], e_add[PER];
+  if (WK > 1 && !GATES) {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int idx = tid + 256 * i;
+      const int p = idx / CO_BLK, col = idx - p * CO_BLK;
+      const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
+      e_ok[i] = oy < hout && ox < wout;
+      e_off[i] = (((long long)n * hout + oy) * wout + ox) * a.cout + co0 + col;
+      e_co[i] = co0 + col;
+    }
+    conv_epilogue_load<T, PER>(a, e_off, e_ok, e_r0, e_add);
+  }
+
   v16f acc[2][NB];
 #pragma unroll
   for (int mb = 0; mb < 2; ++mb)
@@ -401,25 +421,16 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
           red[p * CO_BLK + wn * (32 * NB) + nb * 32 + l32] = acc[mb][nb][r];
       }
     __syncthreads();
-    constexpr int PER = 64 * CO_BLK / 256;     // output elements per thread
-    long long off[PER];
-    int co[PER];
-    bool ok[PER];
     float v[PER];
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const int idx = tid + 256 * i;
-      const int p = idx / CO_BLK, col = idx - p * CO_BLK;
-      const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
-      ok[i] = oy < hout && ox < wout;
-      off[i] = (((long long)n * hout + oy) * wout + ox) * a.cout + co0 + col;
-      co[i] = co0 + col;
       float sum = smem[idx];
 #pragma unroll
       for (int k2 = 1; k2 < WK; ++k2) sum += smem[k2 * (64 * CO_BLK) + idx];
       v[i] = sum;
     }
-    conv_store_batch<T, PER>(a, off, co, ok, v);
+    conv_epilogue_store<T, PER>(a, e_off, e_co, e_ok, v, e_r0, e_add);
   }
 }
 
