@@ -282,6 +282,29 @@ int mie_add_incr(const void* a, const uint8_t* ma, const void* b,
                  const mie_tileset* ts, int dtype, void* stream);
 
 /*
+ * Incremental max pooling: over the active tiles of `out` (built with
+ * MIE_FOOT_CONV for the same k / stride / pad)
+ *   out_delta = maxpool(reservoir + in_delta) - maxpool(reservoir)
+ * with torch's max_pool2d window rule (taps outside the image do not count).
+ * The reservoir ([n,h_in,w_in,c] fp32) is only READ: pooling windows of
+ * neighbouring tiles overlap, so the caller accumulates it afterwards with
+ * mie_accumulate.  in_delta is read at the active pixels of in_mask only.
+ * Replaces: nnMaxPool2dIncr.forward (incr_modules/mask_incr_modules.py:217-219).
+ */
+int mie_maxpool_incr(const void* in_delta, const uint8_t* in_mask,
+                     const float* reservoir, int h_in, int w_in, int c, int k,
+                     int stride, int pad, const mie_tileset* out, void* out_delta,
+                     int dtype, void* stream);
+
+/*
+ * reservoir += in_delta at the active pixels of ts (nothing else is touched).
+ * Replaces: IncrementReserve.accumulate
+ * (incr_modules/mask_incr_functional.py:40-44), a dense add_ over the frame.
+ */
+int mie_accumulate(const void* in_delta, float* reservoir, int c,
+                   const mie_tileset* ts, int dtype, void* stream);
+
+/*
  * Bilinear x2 up-sampling (align_corners = False) of a delta, optionally of
  * the sum of two deltas: out = up2x(a + b).  `out` is the tile set at the
  * output resolution (2*h_in, 2*w_in), built with MIE_FOOT_UP2X.

@@ -33,6 +33,7 @@ EXPORTS = (
     "mie_build_mask_tiles", "mie_conv_masked", "mie_act_incr", "mie_mul_incr", "mie_add_incr",
     "mie_upsample2x_incr", "mie_convlstm_gates_incr", "mie_tconv_masked", "mie_conv_refresh",
     "mie_pack_filter", "mie_kfence_incr", "mie_events_to_frame", "mie_tconv_refresh", "mie_conv_gates_masked",
+    "mie_maxpool_incr", "mie_accumulate",
 )
 
 
@@ -95,6 +96,10 @@ def _declare(l):
     l.mie_conv_gates_masked.restype = ci
     l.mie_conv_gates_masked.argtypes = [vp, vp, ci, vp, vp, ci, ci, ci, vp, vp, ci, ci, tsp, vp, vp, vp, vp, vp,
                                         vp, vp, ci, vp]
+    l.mie_maxpool_incr.restype = ci
+    l.mie_maxpool_incr.argtypes = [vp, vp, vp, ci, ci, ci, ci, ci, ci, tsp, vp, ci, vp]
+    l.mie_accumulate.restype = ci
+    l.mie_accumulate.argtypes = [vp, vp, ci, tsp, ci, vp]
     l.mie_tconv_refresh.restype = ci
     l.mie_tconv_refresh.argtypes = [vp, ci, ci, ci, vp, ci, ci, ci, ci, vp, tsp, vp, vp, ci, cf, ci, vp]
     l.mie_tconv_masked.restype = ci

@@ -323,6 +323,72 @@ __global__ __launch_bounds__(256) void k_up2x_incr(TileSetDev ts, const T* __res
   });
 }
 
+// ---- max pooling increment and masked accumulate ---------------------------------
+// out = pool(R + d) - pool(R) over the active output tiles (window taps outside the image are
+// skipped, which is the -inf padding of torch's max_pool2d); R itself is only read here, the
+// caller accumulates it afterwards with k_accumulate (windows of neighbouring tiles overlap, so
+// an in-place update inside this kernel would race).
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void k_maxpool_incr(TileSetDev ts, const T* __restrict__ din,
+                                                      const uint8_t* __restrict__ dmask,
+                                                      const float* __restrict__ res, int h_in, int w_in,
+                                                      int c, int k, int s, int pad, T* __restrict__ dout) {
+  int n, y0, x0;
+  const int tk = mie_pick_tile(ts, blockIdx.x, n, y0, x0);
+  if (tk == 0) return;
+  const int cv = c / VEC;
+  for_tile_slots(ts, n, y0, x0, cv, [&](int px, long long pixoff, int cq) {
+    const long long off = pixoff * c + (long long)cq * VEC;
+    Vec<VEC> o = Vec<VEC>::zero();
+    if (tk == 1 && ts.pixmask[pixoff]) {
+      const int oy = y0 + (px >> 3), ox = x0 + (px & 7);
+      Vec<VEC> m0, m1;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) m0[e] = m1[e] = -INFINITY;
+      for (int ky = 0; ky < k; ++ky) {
+        const int iy = oy * s - pad + ky;
+        if (iy < 0 || iy >= h_in) continue;
+        for (int kx = 0; kx < k; ++kx) {
+          const int ix = ox * s - pad + kx;
+          if (ix < 0 || ix >= w_in) continue;
+          const long long so = ((long long)n * h_in + iy) * w_in + ix;
+          Vec<VEC> r = Vec<VEC>::load(res + so * c + (long long)cq * VEC);
+          Vec<VEC> d = (dmask == nullptr || dmask[so]) ? Vec<VEC>::load(din + so * c + (long long)cq * VEC)
+                                                       : Vec<VEC>::zero();
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            m0[e] = fmaxf(m0[e], r[e]);
+            m1[e] = fmaxf(m1[e], r[e] + d[e]);
+          }
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) o[e] = m1[e] - m0[e];
+    }
+    o.store(dout + off);
+  });
+}
+
+// R += d at the active pixels of the tile set (IncrementReserve.accumulate without touching the
+// rest of the frame).
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void k_accumulate(TileSetDev ts, const T* __restrict__ din,
+                                                    float* __restrict__ res, int c) {
+  int n, y0, x0;
+  const int tk = mie_pick_tile(ts, blockIdx.x, n, y0, x0);
+  if (tk != 1) return;
+  const int cv = c / VEC;
+  for_tile_slots(ts, n, y0, x0, cv, [&](int, long long pixoff, int cq) {
+    if (!ts.pixmask[pixoff]) return;
+    const long long off = pixoff * c + (long long)cq * VEC;
+    Vec<VEC> r = Vec<VEC>::load(res + off);
+    Vec<VEC> d = Vec<VEC>::load(din + off);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) r[e] += d[e];
+    r.store(res + off);
+  });
+}
+
 // ---- fused ConvLSTM gates ------------------------------------------------------
 
 template <typename T, int VEC>
@@ -525,5 +591,46 @@ extern "C" int mie_convlstm_gates_incr(const void* gates_delta, float* gates_res
   const unsigned grid = (unsigned)mie_tile_capacity(ts->n, ts->h, ts->w);
   MIE_LAUNCH_POINTWISE(k_convlstm_gates, dtype, hid, grid, true, stream, d, (const T*)gates_delta, gates_res,
                        (const T*)cprev_delta, cprev_mask, cprev_res, cell_res, (T*)h_delta, (T*)c_delta, hid);
+  return mie_check_launch(who);
+}
+
+extern "C" int mie_maxpool_incr(const void* in_delta, const uint8_t* in_mask, const float* reservoir,
+                                int h_in, int w_in, int c, int k, int stride, int pad,
+                                const mie_tileset* out, void* out_delta, int dtype, void* stream) {
+  mie_clear_error();
+  const char* who = "mie_maxpool_incr";
+  int rc = check_pointwise(who, out, c);
+  if (rc != MIE_OK) return rc;
+  MIE_DTYPE_OK(dtype, who);
+  MIE_REQUIRE(in_delta && reservoir && out_delta, MIE_ERR_INVALID_ARG, "%s: NULL pointer", who);
+  MIE_REQUIRE(in_delta != out_delta, MIE_ERR_INVALID_ARG, "%s: out_delta must not alias in_delta", who);
+  MIE_REQUIRE(h_in > 0 && w_in > 0 && k >= 1 && k <= 15 && stride >= 1 && stride <= 8 && pad >= 0 &&
+                  2 * pad <= k,
+              MIE_ERR_UNSUPPORTED, "%s: k=%d stride=%d pad=%d not implemented", who, k, stride, pad);
+  MIE_REQUIRE(h_in + 2 * pad >= k && w_in + 2 * pad >= k && out->h == (h_in + 2 * pad - k) / stride + 1 &&
+                  out->w == (w_in + 2 * pad - k) / stride + 1,
+              MIE_ERR_INVALID_ARG, "%s: pooling (%d,%d) with k=%d s=%d p=%d does not give the tile set's (%d,%d)",
+              who, h_in, w_in, k, stride, pad, out->h, out->w);
+  MIE_PTR16(in_delta, who, "in_delta"); MIE_PTR16(reservoir, who, "reservoir");
+  MIE_PTR16(out_delta, who, "out_delta");
+  const TileSetDev d = mie_dev_tileset(out);
+  const unsigned grid = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
+  MIE_LAUNCH_POINTWISE(k_maxpool_incr, dtype, c, grid, true, stream, d, (const T*)in_delta, in_mask, reservoir,
+                       h_in, w_in, c, k, stride, pad, (T*)out_delta);
+  return mie_check_launch(who);
+}
+
+extern "C" int mie_accumulate(const void* in_delta, float* reservoir, int c, const mie_tileset* ts,
+                              int dtype, void* stream) {
+  mie_clear_error();
+  const char* who = "mie_accumulate";
+  int rc = check_pointwise(who, ts, c);
+  if (rc != MIE_OK) return rc;
+  MIE_DTYPE_OK(dtype, who);
+  MIE_REQUIRE(in_delta && reservoir, MIE_ERR_INVALID_ARG, "%s: NULL pointer", who);
+  MIE_PTR16(in_delta, who, "in_delta"); MIE_PTR16(reservoir, who, "reservoir");
+  const TileSetDev d = mie_dev_tileset(ts);
+  const unsigned grid = (unsigned)mie_tile_capacity(ts->n, ts->h, ts->w);
+  MIE_LAUNCH_POINTWISE(k_accumulate, dtype, c, grid, true, stream, d, (const T*)in_delta, reservoir, c);
   return mie_check_launch(who);
 }

@@ -511,8 +511,9 @@ class nnBatchNorm2dIncr(nn.BatchNorm2d):
         return super().forward(x)
 
 
-class nnMaxPool2dIncr(nn.MaxPool2d):
-    """pool(R + d) - pool(R), R += d (reference :210-224); torch ops, not on the hot path."""
+class nnMaxPool2dIncr(nn.MaxPool2d, _IncrBuffers):
+    """pool(R + d) - pool(R), then R += d (reference :210-224): one kernel over the active output
+    tiles and a masked accumulate of the reservoir (square windows, no dilation, floor mode)."""
 
     def __init__(self, kernel_size, stride=None, padding=0):
         nn.MaxPool2d.__init__(self, kernel_size=kernel_size, stride=stride, padding=padding)
@@ -521,11 +522,28 @@ class nnMaxPool2dIncr(nn.MaxPool2d):
         self.mp_res = IncrementReserve()
 
     def forward(self, x_incr: Masked) -> Masked:
-        out = self.functional(self.mp_res.reservoir + x_incr[0]) - self.functional(self.mp_res.reservoir)
-        self.mp_res.accumulate(x_incr)
-        return out, None
+        if self.mp_res.reservoir is None:
+            raise RuntimeError("nnMaxPool2dIncr: call forward_refresh_reservoirs first")
+        if _square(self.dilation, "dilation") != 1 or self.ceil_mode or self.return_indices:
+            raise NotImplementedError("incremental max pooling with dilation / ceil_mode / indices")
+        k = _square(self.kernel_size, "kernel_size")
+        s, p = _square(self.stride, "stride"), _square(self.padding, "padding")
+        x, pix, _ = _unpack(x_incr)
+        n, c, h, w = x.shape
+        ho, wo = ops.conv_out_size(h, w, k, s, p)
+        ts = self._tile_set("out", n, ho, wo, x.device)
+        ops.build_mask_tiles(pix, None, n, h, w, _lib.FOOT_CONV, k, s, p, ts)
+        out = self._delta_buf("out", (n, c, ho, wo), x.device, x.dtype)
+        ops.maxpool_incr(x, pix, self.mp_res.reservoir, k, s, p, ts, out)
+        in_tm = x_incr[1] if len(x_incr) > 1 else None
+        if not isinstance(in_tm, TileMask):
+            in_tm = self._tile_set("in", n, h, w, x.device)
+            ops.build_mask_tiles(pix, None, n, h, w, _lib.FOOT_CONV, 1, 1, 0, in_tm)
+        ops.accumulate(x, self.mp_res.reservoir, in_tm)
+        return [out, ts]
 
     def forward_refresh_reservoirs(self, x: DenseT) -> DenseT:
+        self._reset_incr()
         self.mp_res.update_reservoir(x)
         return super().forward(x)
 

@@ -415,6 +415,29 @@ def add_incr(a, ma, b, mb, out_delta, ts: TileMask):
     return out_delta
 
 
+def maxpool_incr(in_delta, in_mask, reservoir, k, stride, pad, out_ts: TileMask, out_delta):
+    """out_delta = maxpool(reservoir + in_delta) - maxpool(reservoir); the reservoir is only read."""
+    n, c, h, w = in_delta.shape
+    _same_shape("reservoir", reservoir, in_delta)
+    dt = in_delta.dtype
+    _ready(out_ts)
+    check(lib().mie_maxpool_incr(nhwc_ptr(in_delta, "in_delta", dtype=dt), pix_ptr(in_mask, n, h, w, "in_mask"),
+                                 nhwc_ptr(reservoir, "reservoir"), h, w, c, k, stride, pad, out_ts.ref,
+                                 nhwc_ptr(out_delta, "out_delta", c, dtype=dt), delta_dtype(in_delta),
+                                 _stream(in_delta)))
+    return out_delta
+
+
+def accumulate(in_delta, reservoir, ts: TileMask):
+    """reservoir += in_delta at the active pixels of ts."""
+    n, c, h, w = in_delta.shape
+    _same_shape("reservoir", reservoir, in_delta)
+    _ready(ts)
+    check(lib().mie_accumulate(nhwc_ptr(in_delta, "in_delta", dtype=in_delta.dtype), nhwc_ptr(reservoir, "reservoir"),
+                               c, ts.ref, delta_dtype(in_delta), _stream(in_delta)))
+    return reservoir
+
+
 def upsample2x_incr(a, ma, b, mb, out_ts: TileMask, out_delta):
     n, c, h, w = a.shape
     if b is not None:

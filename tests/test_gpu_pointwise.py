@@ -230,3 +230,32 @@ def test_kfence_in_place_and_switched_off():
         ops.kfence_incr(_dev(d), carry2, 0.0, out, ts)
     with pytest.raises(RuntimeError, match="alias"):
         ops.kfence_incr(x, x, 0.5, out, ts)
+
+
+@pytest.mark.parametrize("k,s,p", [(2, 2, 0), (3, 2, 1), (3, 1, 1)])
+@pytest.mark.parametrize("n,c,h,w", [(1, 16, 37, 45), (2, 3, 16, 24)])
+def test_maxpool_increment_and_masked_accumulate(k, s, p, n, c, h, w):
+    # nnMaxPool2dIncr.forward (incr_modules/mask_incr_modules.py:217-219): pool(R + d) - pool(R), R += d.
+    # max and one subtraction of identical fp32 operands: bit-exact against torch's max_pool2d
+    from maskedincrementeval_amd import mask_incr_modules as mm
+    pool = mm.nnMaxPool2dIncr(k, s, p)
+    r0 = _randn(n, c, h, w, seed=k + c)
+    res_cpu = io.Reserve(r0.clone())
+    with torch.no_grad():
+        y0 = pool.forward_refresh_reservoirs(_dev(r0.clone()))
+    assert torch.equal(y0.cpu(), torch.nn.functional.max_pool2d(r0, k, s, p))
+    for step in range(3):
+        d, m = gaussian_delta(n, c, h, w, 0.1, 0.8, seed=500 + step + h)
+        x = _dev(d)
+        x[~m.to(DEV).bool().expand_as(x)] = float("nan")          # inactive pixels are never read
+        out, ts = pool([x, m.to(DEV) if step < 2 else m.expand(n, c, h, w).to(DEV)])
+        torch.cuda.synchronize()
+        want = io.maxpool_incr(res_cpu, d, k, s, p)
+        assert torch.equal(out.cpu(), want), "step %d" % step
+        assert torch.equal(pool.mp_res.reservoir.cpu(), res_cpu.reservoir)
+        assert np.array_equal(ts.pixmask[:, 0].cpu().numpy(), mo.footprint_conv(m[:, 0].numpy(), k, s, p))
+    # dense delta (mask None)
+    d = _randn(n, c, h, w, seed=77) * 0.3
+    out, _ = pool([_dev(d), None])
+    assert torch.equal(out.cpu(), io.maxpool_incr(res_cpu, d, k, s, p))
+    assert torch.equal(pool.mp_res.reservoir.cpu(), res_cpu.reservoir)
