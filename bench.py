@@ -369,7 +369,9 @@ def main():
         print("[bench] cpu baseline: %.1f ms/frame on %d threads" % (1e3 * cdt, cpu["cores"]), file=sys.stderr, flush=True)
 
     result = {
-        "metric": "incremental frames/s, E2Depth-incr %dx%d @%g%% delta density" % (H, W, 100 * dens),
+        # the headline metric's name; `value` is its frames/s part, the HBM GB/s part is in
+        # "hbm_gbs_whole_frame" and per launch in "layers"
+        "metric": "incremental frames/s + HBM GB/s, E2Depth-incr %dx%d @%g%% delta density" % (H, W, 100 * dens),
         "value": round(NB / sec_per_step, 2),
         "unit": "frames/s",
         "n_gpus": 1,
@@ -386,6 +388,7 @@ def main():
                    "density": dens, "height": H, "width": W, "batch": NB, "graph": not args.no_graph},
         "roofline": roofline,
         "cpu_baseline": cpu,
+        "hbm_gbs_whole_frame": round(tot_bytes / sec_per_step / 1e9, 1),
         "hbm_frac_whole_frame": round(tot_bytes / sec_per_step / 1e9 / PEAK_HBM_GBS, 5),
         "algorithmic_mb_per_frame": round(tot_bytes / 1e6, 2),
         "algorithmic_gflop_per_frame": round(tot_flops / 1e9, 3),
