@@ -13,23 +13,36 @@
 //   * A (pixels x k): the input tile plus halo is staged in LDS, CC input
 //     channels at a time, by all 256 threads with 16-byte loads of the NHWC
 //     rows; pixels whose mask byte is 0 (or that lie outside the image) are
-//     zero-filled without touching HBM.  Staging is double buffered: the
-//     global loads of chunk c+1 are in flight while chunk c is multiplied.
-//   * B (k x channels): rows of the matrix-core filter copy (mie_pack_filter) are read
-//     straight from L2 into registers, 16 bytes per lane (each value is used by exactly one wave
-//     of the workgroup), three units ahead of the MFMAs that consume them.
+//     zero-filled without touching HBM.  The global loads of chunk c+1 are in
+//     flight (in registers) while chunk c is multiplied; fp32 stride-1 tiles
+//     also double-buffer the LDS copy, the others store it between two barriers.
+//   * B (k x channels): units of the matrix-core filter copy (mie_pack_filter) are
+//     read straight from L2 into a register ring, 16 bytes per lane (each value is
+//     used by exactly one wave of the workgroup), 3 to 8 units ahead of the MFMAs
+//     that consume them.
 //   * The 4 waves split the workgroup's work WN ways over output channels and
 //     WK = 4/WN ways over k (units = tap x 8-channel sub-chunk, round robin).
 //     Layers with few tiles (33x44 bottleneck: 30 tiles) take WN=1, WK=4 so
 //     that tiles x Cout/32 workgroups of 4 busy waves fill the chip; wide
 //     layers take WN=4.  K-split partial sums meet in LDS and are added in a
 //     fixed order (bit-reproducible).
+//   * Epilogue: plain delta, or reservoir update + activation increment (values
+//     fetched at kernel start in the k-split variants), or -- GATES -- the whole
+//     ConvLSTM gate chain on the four gate columns of each hidden channel.
 // A lane's operand layout: lanes 0-31 = the 32 pixels of an M block, the lane
 // half selects 4 of the 8 channels of a sub-chunk, read as ONE ds_read_b128
 // that feeds 4 k-steps (k-step j pairs channel j of the low half with channel
 // 4+j of the high half; the B operand is loaded with the same pairing).  The
-// LDS row stride CC+4 floats keeps the 16-byte reads of 8 neighbouring pixels
-// on disjoint banks for stride 1 and 2.
+// LDS layout (pixel stride CC+4 dwords, row pitch 32 mod 64 dwords, half swap
+// for stride 2) keeps the 16-byte reads of 16 neighbouring lanes on disjoint banks.
+//
+// What bounds it (measured on MI355X): with the chip full (thousands of
+// workgroups) the fp32 kernel runs at 0.81 of the matrix-core peak.  A single
+// workgroup alone on a CU spends 86 % of each chunk on the matrix cores and about
+// 4 us on tile pick, first staging round trip and epilogue; launches with fewer
+// than a few workgroups per CU are therefore quantised: ceil(workgroups / 256)
+// rounds of one workgroup time.  8-wave workgroups and a 25-deep B ring were
+// tried and changed nothing: a workgroup already owns the CU's four matrix cores.
 #pragma once
 #include "mie_conv.h"
 #include <stdlib.h>
