@@ -1,13 +1,17 @@
 // Masked convolution of a delta over active 8x8 output tiles (gfx950).
 //
-// Three code paths, one per arithmetic regime:
-//   mfma    : Cin % 32 == 0 (16 for stride 2) and Cout % 32 == 0 -- per-tile implicit GEMM on
-//             the matrix cores (mie_conv_mfma_impl.h).
+// Code paths, one per arithmetic regime:
+//   mfma    : input channels in whole staging chunks (32 fp32 / 64 bf16 channels; 16 / 32 for 7x7
+//             and as the fallback depth at stride 2) and Cout % 32 == 0 -- per-tile implicit GEMM
+//             on the matrix cores (mie_conv_mfma_impl.h), optionally with the ConvLSTM gate chain
+//             as its epilogue.
 //   valu    : any shape -- thread = one output channel x 16 pixels, input tile
 //             staged in LDS and read as wave-wide broadcasts.
-//   smallco : Cout <= 4 (prediction / flow heads) -- thread = one pixel.
-// All paths share the epilogue: plain delta store, or the fused reservoir
-// update + activation increment.
+//   smallco : Cout <= 4 (prediction / flow heads) -- thread = one pixel; 1x1 convs of that kind
+//             walk whole NHWC rows with 4 lanes per pixel.
+//   tconv   : transposed conv, gather form.
+// All paths share the epilogue: plain delta store, the fused reservoir update + activation
+// increment, or (dense refresh) bias + activation + reservoir fill.
 #include "mie_common.h"
 #include "mie_conv.h"
 
