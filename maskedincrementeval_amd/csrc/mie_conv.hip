@@ -66,16 +66,20 @@ __global__ __launch_bounds__(256) void k_conv_valu(ConvArgsT<T> a) {
       __syncthreads();
       const int nci = (cs - ci0 < CC) ? cs - ci0 : CC;
       for (int cc = 0; cc < nci; ++cc) {
+        // all K*K filter taps of this input channel first (independent loads, one latency), then the
+        // multiply-adds: a load inside the tap loop would expose the L2 latency K*K times
         const float* wp = a.filt + (long long)(fbase + ci0 + cc) * K * K * a.cout + co;
+        float wv[K * K];
+#pragma unroll
+        for (int t = 0; t < K * K; ++t) wv[t] = (co < a.cout) ? wp[t * a.cout] : 0.f;
 #pragma unroll
         for (int ky = 0; ky < K; ++ky)
 #pragma unroll
           for (int kx = 0; kx < K; ++kx) {
-            const float wv = (co < a.cout) ? wp[(ky * K + kx) * a.cout] : 0.f;
 #pragma unroll
             for (int p = 0; p < 16; ++p) {
               const int py = 2 * pg + (p >> 3), px = p & 7;
-              acc[p] += s_in[((py * S + ky) * IT + px * S + kx) * CC + cc] * wv;
+              acc[p] += s_in[((py * S + ky) * IT + px * S + kx) * CC + cc] * wv[ky * K + kx];
             }
           }
       }
