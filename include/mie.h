@@ -366,6 +366,39 @@ int mie_conv_gates_masked(const void* x, const uint8_t* xmask, int c1,
                           void* c_delta, int dtype, void* stream);
 
 /*
+ * Per-channel scale of a delta over the active tiles of ts: out = in * scale[c]
+ * (inactive pixels of active tiles and stale tiles get zeros).  scale is fp32 [c];
+ * for an eval-mode batch norm it is weight / sqrt(running_var + eps).
+ * out_delta may alias in_delta.
+ * Replaces: bn2d_from_module (incr_modules/mask_incr_functional.py:69-73), the
+ * body of nnBatchNorm2dIncr.forward (incr_modules/mask_incr_modules.py:200-207).
+ */
+int mie_scale_incr(const void* in_delta, const float* scale, void* out_delta,
+                   int c, const mie_tileset* ts, int dtype, void* stream);
+
+/*
+ * Adaptive average pooling of a delta [n,h_in,w_in,c] to [n,h_out,w_out,c] with
+ * torch's window rule (output index o covers [floor(o*in/out), ceil((o+1)*in/out))).
+ * Pixels whose in_mask byte is 0 are not read and add nothing (in_mask NULL =
+ * all active); the divisor is the window size.  Every output element is written.
+ * Replaces: nnAdaptiveAvgPool2dIncr.forward
+ * (incr_modules/mask_incr_modules.py:228-233).
+ */
+int mie_avgpool_incr(const void* in_delta, const uint8_t* in_mask, int n, int h_in,
+                     int w_in, int c, int h_out, int w_out, void* out_delta,
+                     int dtype, void* stream);
+
+/*
+ * Fully connected layer on a delta, bias dropped: out[n][o] = sum_i in[n][i] *
+ * W[o][i].  weight_t is the TRANSPOSED weight, fp32 [f_in][f_out] (make it once
+ * per weight update), so that an input feature's contribution is one contiguous
+ * row; rows of features whose delta is exactly 0 are not read.
+ * Replaces: nnLinearIncr.forward (incr_modules/mask_incr_modules.py:106-116).
+ */
+int mie_linear_incr(const void* in_delta, int n, int f_in, const float* weight_t,
+                    int f_out, void* out_delta, int dtype, void* stream);
+
+/*
  * Masked transposed convolution of a delta (stride s, padding p; the output
  * size out->h/w fixes output_padding): out(oy,ox,co) = sum x(iy,ix,ci) *
  * filter[ci][ky][kx][co] over oy = iy*s - p + ky, ox = ix*s - p + kx, with

@@ -151,16 +151,28 @@ def transposed_conv2d_from_module(x: Masked, gates: nn.ConvTranspose2d, bias=Tru
     return [out, ts]
 
 
+def bn_scale(bnm: nn.BatchNorm2d) -> torch.Tensor:
+    """gamma / sqrt(running_var + eps) as contiguous fp32 [C]."""
+    scale = torch.rsqrt(bnm.running_var.detach().float() + bnm.eps)
+    if bnm.weight is not None:
+        scale = scale * bnm.weight.detach().float()
+    return scale.contiguous()
+
+
 def bn2d_from_module(x: Masked, bnm: nn.BatchNorm2d) -> Masked:
     """Linear part of eval-mode batch norm on a delta: dx * gamma / sqrt(var + eps).
 
     Reference :69-73 (F.batch_norm with zero mean and no bias).  A per-channel
     scale keeps zeros zero, so the mask passes through.
     """
-    scale = torch.rsqrt(bnm.running_var + bnm.eps)
-    if bnm.weight is not None:
-        scale = scale * bnm.weight
-    return [x[0] * scale.view(1, -1, 1, 1), x[1] if len(x) > 1 else None]
+    delta, pix, tm = _unpack(x)
+    n, c, h, w = delta.shape
+    if not isinstance(tm, TileMask):
+        tm = TileMask(n, h, w, delta.device)
+        ops.build_mask_tiles(pix, None, n, h, w, _lib.FOOT_CONV, 1, 1, 0, tm)
+    out = ops.new_nhwc(n, c, h, w, delta.device, delta.dtype)
+    ops.scale_incr(delta, bn_scale(bnm), out, tm)
+    return [out, tm]
 
 
 def interpolate_from_module(x: Masked) -> Masked:

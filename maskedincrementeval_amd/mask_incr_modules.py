@@ -22,7 +22,7 @@ import torch.nn.functional as F
 from . import _lib, ops
 from .masked_types import DenseT, Masked, TileMask
 from .mask_incr_functional import (IncrPointwiseMultiply, IncrementReserve, _square, _unpack,
-                                   bn2d_from_module, conv2d_from_module)
+                                   bn2d_from_module, bn_scale, conv2d_from_module)
 
 
 class _IncrBuffers:
@@ -268,10 +268,26 @@ class NonlinearPointOpIncr(IncrementMaskModule):
 
 
 class nnLinearIncr(nn.Linear):
-    """Fully connected layer on a delta: bias dropped (reference :106-116)."""
+    """Fully connected layer on a delta: bias dropped (reference :106-116).  One kernel that reads only
+    the weight rows of the features whose delta is non-zero; the transposed weight copy it walks is
+    rebuilt when the weight changes."""
+
+    def _weight_t(self) -> torch.Tensor:
+        w = self.weight
+        key = (w.data_ptr(), w._version, w.device)
+        cached = self.__dict__.get("_wt")
+        if cached is None or cached[0] != key:
+            cached = (key, w.detach().float().t().contiguous())
+            self.__dict__["_wt"] = cached
+        return cached[1]
 
     def forward(self, x_incr: Masked) -> Masked:
-        return F.linear(x_incr[0], self.weight, bias=None), None
+        d = x_incr[0]
+        lead = d.shape[:-1]
+        d2 = d.reshape(-1, d.shape[-1]).contiguous()
+        out = torch.empty((d2.shape[0], self.out_features), dtype=d2.dtype, device=d2.device)
+        ops.linear_incr(d2, self._weight_t(), out)
+        return [out.reshape(*lead, self.out_features), None]
 
     def forward_refresh_reservoirs(self, x: DenseT) -> DenseT:
         return super().forward(x)
@@ -501,11 +517,19 @@ class nnConvTranspose2dIncr(nn.ConvTranspose2d, _IncrBuffers):
         return ops.tconv_refresh(x, self._filter(), bias, k, s, p, ts, out)
 
 
-class nnBatchNorm2dIncr(nn.BatchNorm2d):
-    """Reference :200-207."""
+class nnBatchNorm2dIncr(nn.BatchNorm2d, _IncrBuffers):
+    """Reference :200-207: the linear part of the eval-mode batch norm on a delta, one masked kernel into a
+    buffer the module keeps."""
 
     def forward(self, x_incr):
-        return bn2d_from_module(x_incr, self)
+        delta, pix, tm = _unpack(x_incr)
+        n, c, h, w = delta.shape
+        if not isinstance(tm, TileMask):
+            tm = self._tile_set("in", n, h, w, delta.device)
+            ops.build_mask_tiles(pix, None, n, h, w, _lib.FOOT_CONV, 1, 1, 0, tm)
+        out = self._delta_buf("out", (n, c, h, w), delta.device, delta.dtype)
+        ops.scale_incr(delta, bn_scale(self), out, tm)
+        return [out, tm]
 
     def forward_refresh_reservoirs(self, x):
         return super().forward(x)
@@ -549,10 +573,17 @@ class nnMaxPool2dIncr(nn.MaxPool2d, _IncrBuffers):
 
 
 class nnAdaptiveAvgPool2dIncr(nn.AdaptiveAvgPool2d):
-    """Reference :228-233."""
+    """Reference :228-233: adaptive average pooling of a delta; inactive pixels are not read.  The pooled
+    delta is small and dense, so it carries no mask."""
 
     def forward(self, x_incr):
-        return nn.AdaptiveAvgPool2d.forward(self, x_incr[0]), None
+        delta, pix, _ = _unpack(x_incr)
+        n, c, h, w = delta.shape
+        size = self.output_size if isinstance(self.output_size, (tuple, list)) else (self.output_size,) * 2
+        ho, wo = (h if size[0] is None else int(size[0])), (w if size[1] is None else int(size[1]))
+        out = ops.new_nhwc(n, c, ho, wo, delta.device, delta.dtype)
+        ops.avgpool_incr(delta, pix, out)
+        return [out, None]
 
     def forward_refresh_reservoirs(self, x):
         return super().forward(x)

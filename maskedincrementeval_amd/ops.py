@@ -438,6 +438,50 @@ def accumulate(in_delta, reservoir, ts: TileMask):
     return reservoir
 
 
+def scale_incr(in_delta, scale, out_delta, ts: TileMask):
+    """out = in * scale[c] over the active tiles of ts (eval-mode batch norm on a delta); in place allowed."""
+    n, c, h, w = in_delta.shape
+    _same_shape("out_delta", out_delta, in_delta)
+    if scale.dtype != torch.float32 or scale.numel() != c or not scale.is_contiguous():
+        raise ValueError("scale must be contiguous fp32 [%d]" % c)
+    _require_gpu(scale, "scale")
+    _ready(ts)
+    dt = in_delta.dtype
+    check(lib().mie_scale_incr(nhwc_ptr(in_delta, "in_delta", dtype=dt), scale.data_ptr(),
+                               nhwc_ptr(out_delta, "out_delta", c, dtype=dt), c, ts.ref, delta_dtype(in_delta),
+                               _stream(in_delta)))
+    return out_delta
+
+
+def avgpool_incr(in_delta, in_mask, out_delta):
+    """Adaptive average pooling of a delta to the spatial size of out_delta; masked pixels are not read."""
+    n, c, h, w = in_delta.shape
+    if out_delta.shape[:2] != in_delta.shape[:2] or out_delta.dtype != in_delta.dtype:
+        raise ValueError("out_delta %s does not match the input %s" % (tuple(out_delta.shape), tuple(in_delta.shape)))
+    ho, wo = out_delta.shape[2:]
+    dt = in_delta.dtype
+    check(lib().mie_avgpool_incr(nhwc_ptr(in_delta, "in_delta", dtype=dt), pix_ptr(in_mask, n, h, w, "in_mask"),
+                                 n, h, w, c, ho, wo, nhwc_ptr(out_delta, "out_delta", c, dtype=dt),
+                                 delta_dtype(in_delta), _stream(in_delta)))
+    return out_delta
+
+
+def linear_incr(in_delta, weight_t, out_delta):
+    """out[n, o] = sum_i in[n, i] * W[o, i] with weight_t = W.t().contiguous() (fp32 [f_in, f_out])."""
+    if in_delta.dim() != 2 or not in_delta.is_contiguous() or out_delta.dim() != 2 or not out_delta.is_contiguous():
+        raise ValueError("linear_incr takes contiguous 2-D deltas")
+    _require_gpu(in_delta, "in_delta"), _require_gpu(weight_t, "weight_t"), _require_gpu(out_delta, "out_delta")
+    n, f_in = in_delta.shape
+    if weight_t.dtype != torch.float32 or not weight_t.is_contiguous() or weight_t.shape[0] != f_in:
+        raise ValueError("weight_t must be contiguous fp32 [%d, f_out], got %s" % (f_in, tuple(weight_t.shape)))
+    f_out = weight_t.shape[1]
+    if tuple(out_delta.shape) != (n, f_out) or out_delta.dtype != in_delta.dtype:
+        raise ValueError("out_delta must be %s of %s" % ((n, f_out), in_delta.dtype))
+    check(lib().mie_linear_incr(in_delta.data_ptr(), n, f_in, weight_t.data_ptr(), f_out, out_delta.data_ptr(),
+                                delta_dtype(in_delta), _stream(in_delta)))
+    return out_delta
+
+
 def upsample2x_incr(a, ma, b, mb, out_ts: TileMask, out_delta):
     n, c, h, w = a.shape
     if b is not None:

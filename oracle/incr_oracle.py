@@ -64,6 +64,12 @@ def linear_incr(delta, weight):
     return F.linear(delta, weight, bias=None)
 
 
+def avgpool_incr(delta, output_size):
+    """nnAdaptiveAvgPool2dIncr.forward (mask_incr_modules.py:228-233): the pooling is linear, so it
+    applies to the delta as it is."""
+    return F.adaptive_avg_pool2d(delta, output_size)
+
+
 # ---- point-wise ops ----------------------------------------------------------------------------
 def act_incr(op, res: Reserve, delta):
     """nnReservedActivation.forward: op(R + d) - op(R), then R += d

@@ -78,6 +78,27 @@ def test_bn_incr_is_scale_only():
     assert torch.allclose(io.bn_incr(d, var, gamma, 1e-5), ref, atol=1e-6)
 
 
+def test_linear_incr_is_a_matrix_product_without_bias():
+    d, w = _rand(3, 7, seed=40), _rand(5, 7, seed=41)
+    ref = torch.einsum("ni,oi->no", d.double(), w.double())
+    assert torch.allclose(io.linear_incr(d, w).double(), ref, atol=1e-6)
+    assert torch.count_nonzero(io.linear_incr(torch.zeros(2, 7), w)) == 0      # no bias term
+
+
+def test_avgpool_incr_windows():
+    d = _rand(2, 3, 10, 13, seed=42)
+    # global pooling is the plane mean, pooling to the input size the identity
+    assert torch.allclose(io.avgpool_incr(d, 1)[:, :, 0, 0], d.mean((2, 3)), atol=1e-6)
+    assert torch.allclose(io.avgpool_incr(d, (10, 13)), d)
+    # a size that does not divide the plane: windows [floor(o*in/out), ceil((o+1)*in/out)), brute force
+    got = io.avgpool_incr(d, (3, 4))
+    for oy in range(3):
+        for ox in range(4):
+            y0, y1 = (oy * 10) // 3, -((-(oy + 1) * 10) // 3)
+            x0, x1 = (ox * 13) // 4, -((-(ox + 1) * 13) // 4)
+            assert torch.allclose(got[:, :, oy, ox], d[:, :, y0:y1, x0:x1].mean((2, 3)), atol=1e-6)
+
+
 # ---- point-wise ops --------------------------------------------------------------------
 def test_relu_increment_identity_exact():
     # reference tests/test_pointops.py:11-22 (shape (1, 40, 80))
