@@ -278,20 +278,55 @@ __device__ __forceinline__ void up2x_coef(int o, int in_size, int& i0, int& i1, 
   }
 }
 
+// One workgroup per 8x8 output tile (and channel range).  The tile's outputs blend a 6x6 block of source
+// pixels (rows y0/2-1 .. y0/2+4): the block is summed (a + b, masked) into LDS once, fp32, and every
+// output slot then reads its four taps from there -- 36 source pixels fetched per tile instead of
+// 4 per output pixel, which is what the kernel was bound by (load instructions, not bytes).
 template <typename T, int VEC>
 __global__ __launch_bounds__(256) void k_up2x_incr(TileSetDev ts, const T* __restrict__ a,
                                                    const uint8_t* __restrict__ ma,
                                                    const T* __restrict__ b,
                                                    const uint8_t* __restrict__ mb, int h_in,
                                                    int w_in, T* __restrict__ dout, int c) {
+  extern __shared__ __attribute__((aligned(16))) float s_src[];   // [36 source pixels][channels of this block]
+  __shared__ uint8_t s_act[64];                                   // output pixel active (fetched with the sources)
   int n, y0, x0;
   const int tk = mie_pick_tile(ts, blockIdx.x, n, y0, x0);
   if (tk == 0) return;
   const int cv = c / VEC;
+  const int per = (cv + (int)gridDim.y - 1) / (int)gridDim.y;     // the channel split of for_tile_slots
+  const int cq0 = (int)blockIdx.y * per;
+  const int cvb = (cv - cq0 < per) ? cv - cq0 : per;
+  if (cvb <= 0) return;
+  const int cw = cvb * VEC;
+  const int ry0 = (y0 >> 1) - 1, rx0 = (x0 >> 1) - 1;
+  if (tk == 1) {
+    if (threadIdx.x < 64) {
+      const int oy = y0 + ((int)threadIdx.x >> 3), ox = x0 + ((int)threadIdx.x & 7);
+      s_act[threadIdx.x] = (oy < ts.h && ox < ts.w) ? ts.pixmask[((long long)n * ts.h + oy) * ts.w + ox] : 0;
+    }
+    for (int idx = threadIdx.x; idx < 36 * cvb; idx += 256) {
+      const int sp = idx / cvb, cq = idx - sp * cvb;
+      const int sy = ry0 + sp / 6, sx = rx0 + sp % 6;
+      Vec<VEC> t = Vec<VEC>::zero();
+      if (sy >= 0 && sy < h_in && sx >= 0 && sx < w_in) {
+        const long long so = ((long long)n * h_in + sy) * w_in + sx;
+        const long long eo = so * c + (long long)(cq0 + cq) * VEC;
+        if (ma == nullptr || ma[so]) t = Vec<VEC>::load(a + eo);
+        if (b != nullptr && (mb == nullptr || mb[so])) {
+          Vec<VEC> u = Vec<VEC>::load(b + eo);
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) t[e] += u[e];
+        }
+      }
+      t.store(s_src + sp * cw + cq * VEC);
+    }
+    __syncthreads();
+  }
   for_tile_slots(ts, n, y0, x0, cv, [&](int px, long long pixoff, int cq) {
     const long long off = pixoff * c + (long long)cq * VEC;
     Vec<VEC> o = Vec<VEC>::zero();
-    if (tk == 1 && ts.pixmask[pixoff]) {
+    if (tk == 1 && s_act[px]) {
       const int oy = y0 + (px >> 3), ox = x0 + (px & 7);
       int r[2], q[2];
       float lr[2], lq[2];
@@ -303,17 +338,9 @@ __global__ __launch_bounds__(256) void k_up2x_incr(TileSetDev ts, const T* __res
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          const long long so = ((long long)n * h_in + r[i]) * w_in + q[j];
-          Vec<VEC> t = Vec<VEC>::zero();
-          if (ma == nullptr || ma[so]) t = Vec<VEC>::load(a + so * c + (long long)cq * VEC);
-          if (b != nullptr && (mb == nullptr || mb[so])) {
-            Vec<VEC> u = Vec<VEC>::load(b + so * c + (long long)cq * VEC);
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) t[e] += u[e];
-          }
-          v[i][j] = t;
-        }
+        for (int j = 0; j < 2; ++j)
+          v[i][j] = Vec<VEC>::load(static_cast<const float*>(s_src) + ((r[i] - ry0) * 6 + (q[j] - rx0)) * cw +
+                                   (cq - cq0) * VEC);
 #pragma unroll
       for (int e = 0; e < VEC; ++e)
         o[e] = lr[0] * (lq[0] * v[0][0][e] + lq[1] * v[0][1][e]) +
@@ -564,8 +591,23 @@ extern "C" int mie_upsample2x_incr(const void* a, const uint8_t* ma, const void*
   MIE_PTR16(a, who, "a"); MIE_PTR16(b, who, "b"); MIE_PTR16(out_delta, who, "out_delta");
   const TileSetDev d = mie_dev_tileset(out);
   const unsigned grid = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
-  MIE_LAUNCH_POINTWISE(k_up2x_incr, dtype, c, grid, true, stream, d, (const T*)a, ma, (const T*)b, mb, h_in, w_in,
-                       (T*)out_delta, c);
+  // channel vectors per block bounded so that the 36-pixel source block fits 36 KB of LDS
+  const bool bf = dtype == MIE_DTYPE_BF16;
+  const int vec = (c % 8 == 0 && (bf || c >= 64)) ? 8 : (c % 4 == 0 ? 4 : 1);
+  const int cv = c / vec;
+  unsigned ny = channel_splits((int)grid, cv);
+  const unsigned ny_min = (unsigned)mie_div_up(c, 256);
+  if (ny < ny_min) ny = ny_min;
+  const size_t lds = (size_t)36 * mie_div_up(cv, (int)ny) * vec * sizeof(float);
+#define MIE_UP2X_LAUNCH(T_, V_)                                                                              \
+  hipLaunchKernelGGL((k_up2x_incr<T_, V_>), dim3(grid, ny), dim3(256), lds, (hipStream_t)stream, d, (const T_*)a, \
+                     ma, (const T_*)b, mb, h_in, w_in, (T_*)out_delta, c)
+  if (bf) {
+    if (vec == 8) MIE_UP2X_LAUNCH(mie_bf16, 8); else if (vec == 4) MIE_UP2X_LAUNCH(mie_bf16, 4); else MIE_UP2X_LAUNCH(mie_bf16, 1);
+  } else {
+    if (vec == 8) MIE_UP2X_LAUNCH(float, 8); else if (vec == 4) MIE_UP2X_LAUNCH(float, 4); else MIE_UP2X_LAUNCH(float, 1);
+  }
+#undef MIE_UP2X_LAUNCH
   return mie_check_launch(who);
 }
 
