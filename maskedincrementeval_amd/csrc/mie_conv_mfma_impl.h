@@ -173,7 +173,10 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   int e_co[PER];
   bool e_ok[PER];
   float e_r0[PER], e_add[PER];
-  if (WK > 1 && !GATES) {
+  // (bf16: a workgroup's contraction is too short to be worth the registers that hold these values
+  // through it -- they cost a resident workgroup per CU -- so they are fetched after it instead.)
+  constexpr bool EARLY = sizeof(T) == 4;
+  auto epilogue_fetch = [&]() {
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const int idx = tid + 256 * i;
@@ -184,7 +187,8 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
       e_co[i] = co0 + col;
     }
     conv_epilogue_load<T, PER>(a, e_off, e_ok, e_r0, e_add);
-  }
+  };
+  if (WK > 1 && !GATES && EARLY) epilogue_fetch();
 
   v16f acc[2][NB];
 #pragma unroll
@@ -423,6 +427,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
     }
   } else {
     // the trailing barrier of the main loop has retired every read of the staging buffers
+    if (!EARLY) epilogue_fetch();
     float* red = smem + wk * (64 * CO_BLK);
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb)
