@@ -148,9 +148,18 @@ def pixel_mask_of(mask, like: torch.Tensor) -> Optional[torch.Tensor]:
     m = mask
     if m.dim() != 4 or m.shape[0] != n or m.shape[2] != h or m.shape[3] != w:
         raise ValueError("mask shape %s does not match delta %s" % (tuple(m.shape), tuple(like.shape)))
+    # The kernels test mask bytes for non-zero, so a uint8 / bool (N,1,H,W) mask on the device is used
+    # as it is: no copy, and the event of whoever wrote it on the compute stream still names it.
+    if m.shape[1] == 1 and m.is_contiguous() and m.device == like.device:
+        if m.dtype == torch.uint8:
+            return m
+        if m.dtype == torch.bool:
+            return m.view(torch.uint8)
     if m.shape[1] != 1:
         m = m.ne(0).any(dim=1, keepdim=True)
-    return m.ne(0).to(torch.uint8).contiguous().to(like.device)
+    m = m.ne(0).to(torch.uint8).contiguous().to(like.device)
+    _mark_pix(m)          # made on the compute stream: a build on the planning stream must wait for it
+    return m
 
 
 # ---- entry points ----------------------------------------------------------------

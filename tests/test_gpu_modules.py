@@ -287,3 +287,38 @@ def test_convlstm_with_previous_state_deltas(cin, hid):
         torch.cuda.synchronize()
         dh_r, dc_r = ref.incr(d, (dhp, dcp))
         _close(dh[0], dh_r, "dh %d" % step), _close(dc[0], dc_r, "dc %d" % step)
+
+
+@pytest.mark.parametrize("graph", [False, True])
+def test_async_mask_planning_gives_the_same_frames_as_inline_planning(graph):
+    # Tile sets built on the planning stream (eagerly and as edges of a replayed HIP graph) must be the
+    # ones inline planning builds: the same kernels then run over the same tiles, so the predictions
+    # agree bit for bit.  Every step has a fresh mask, so a build that read a mask of the previous
+    # step (or raced with the kernel that writes it) shows up as a difference.
+    h, w, steps = 72, 104, 8
+    a = seed_module_(E2VIDRecurrentIncr(async_masks=True), seed=31).to(DEV).eval()
+    s = seed_module_(E2VIDRecurrentIncr(async_masks=False), seed=31).to(DEV).eval()
+    x0 = torch.randn(1, 5, h, w, generator=torch.Generator().manual_seed(32)) * 0.5
+    deltas = [_cl(event_voxel_delta(1, 5, h, w, 0.03 + 0.02 * (i % 3), seed=4100 + i)[0]) for i in range(steps)]
+    static_in = _cl(torch.zeros(1, 5, h, w))
+    with torch.no_grad():
+        a.forward_refresh_reservoirs(_cl(x0), None)
+        s.forward_refresh_reservoirs(_cl(x0), None)
+        refs = [s([d, None], None)[0][0].clone() for d in deltas]
+        got = []
+        g, g_out = None, None
+        for i, d in enumerate(deltas):
+            static_in.copy_(d)
+            if graph and i == 2:       # two eager steps first: they allocate every persistent buffer
+                torch.cuda.synchronize()
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    g_out = a([static_in, None], None)[0][0]
+            if g is not None:
+                g.replay()
+                got.append(g_out.clone())
+            else:
+                got.append(a([static_in, None], None)[0][0].clone())
+        torch.cuda.synchronize()
+    for i in range(steps):
+        assert torch.equal(got[i], refs[i]), "step %d max|diff| = %.3e" % (i, (got[i] - refs[i]).abs().max().item())
