@@ -199,11 +199,15 @@ def main():
         static_in.copy_(deltas[i % n_inputs])
         return m([static_in, None], None)
 
-    def timed_run(m, tag):
+    output_check = {}
+
+    def timed_run(m, tag, check_against=None):
+        history = []                                       # input index of every step the model takes
         with torch.no_grad():
             m.forward_refresh_reservoirs(cl(x0), None)
             for i in range(max(args.warmup, 3)):           # also allocates every persistent buffer
                 step_eager(m, i)
+                history.append(i)
             torch.cuda.synchronize()
             graph = None
             if not args.no_graph:
@@ -211,14 +215,16 @@ def main():
                 side.wait_stream(torch.cuda.current_stream())
                 with torch.cuda.stream(side):
                     step_eager(m, 0)
+                history.append(0)
                 torch.cuda.current_stream().wait_stream(side)
                 torch.cuda.synchronize()
                 graph = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(graph):
-                    m([static_in, None], None)
+                    graph_out = m([static_in, None], None)[0][0]
                 for i in range(3):
                     static_in.copy_(deltas[i % n_inputs])
                     graph.replay()
+                    history.append(i)
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             for i in range(args.steps):
@@ -229,11 +235,38 @@ def main():
                     step_eager(m, i)
             torch.cuda.synchronize()
             dt = time.perf_counter() - t0
+            history.extend(range(args.steps))
+            if check_against is not None:
+                # The timed configuration (graph replay, planning stream) against the plain one: a second
+                # instance of the network with eager launches and inline mask planning takes the same
+                # steps; the next frames of the two must then agree (same kernels over the same tiles).
+                ref = check_against()
+                ref.forward_refresh_reservoirs(cl(x0), None)
+                for i in history:
+                    ref([deltas[i % n_inputs], None], None)
+                worst = 0.0
+                for i in range(4):
+                    want = ref([deltas[i % n_inputs], None], None)[0][0]
+                    if graph is not None:
+                        static_in.copy_(deltas[i % n_inputs])
+                        graph.replay()
+                        got = graph_out
+                    else:
+                        got = step_eager(m, i)[0][0]
+                    worst = max(worst, (got.float() - want.float()).abs().max().item())
+                torch.cuda.synchronize()
+                output_check.update(max_abs_diff=worst, frames=4, steps_before=len(history),
+                                    against="same network, eager launches, inline mask planning")
+                print("[bench] %s: max |difference| to the eager inline-planning network over 4 frames after %d steps: %.3e"
+                      % (tag, len(history), worst), file=sys.stderr, flush=True)
+                if not worst <= 1e-3:
+                    raise SystemExit("bench: the timed configuration does not reproduce the plain one (%.3e)" % worst)
         print("[bench] %s: %.3f ms/frame over %d steps (%s)" % (tag, 1e3 * dt / args.steps, args.steps,
               "eager" if graph is None else "HIP graph"), file=sys.stderr, flush=True)
         return dt / args.steps
 
-    sec_per_step = timed_run(model, "incremental %.0f%%" % (100 * dens))
+    sec_per_step = timed_run(model, "incremental %.0f%%" % (100 * dens),
+                             check_against=lambda: seed_module_(E2VIDRecurrentIncr(), seed=1).to(dev).eval())
 
     # ---- per-layer roofline table: eager launches with HIP events, several repeats ------------
     with torch.no_grad():
@@ -397,6 +430,7 @@ def main():
         "speedup_vs_dense": None if dense_sec is None else round(dense_sec / sec_per_step, 3),
         "density_sweep": sweep,
         "kfenced": kfenced,
+        "output_check": output_check,
         "layers": layers,
     }
     print(json.dumps(result))
