@@ -42,6 +42,8 @@ def parse_args():
     ap.add_argument("--no-graph", action="store_true", help="launch kernels eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-dense", action="store_true", help="skip the all-tiles-active comparator")
     ap.add_argument("--layer-iters", type=int, default=20, help="timed launches per layer for the roofline table")
+    ap.add_argument("--no-plan-first", dest="plan_first", action="store_false",
+                    help="enqueue each mask build right before its consumer instead of all builds of a step first")
     ap.add_argument("--sync-masks", action="store_true", help="build tile sets on the compute stream (no planning stream)")
     ap.add_argument("--dtype", choices=["f32", "bf16"], default="f32",
                     help="element type of deltas and weights (reservoirs and accumulation stay fp32)")
@@ -188,7 +190,7 @@ def main():
     peak_mfma = PEAK_BF16_MFMA_TFLOPS if args.dtype == "bf16" else PEAK_FP32_MFMA_TFLOPS
     cl = lambda t: t.to(dev).to(dt).contiguous(memory_format=torch.channels_last)
 
-    model = seed_module_(E2VIDRecurrentIncr(async_masks=not args.sync_masks), seed=1).to(dev).eval()
+    model = seed_module_(E2VIDRecurrentIncr(async_masks=not args.sync_masks, plan_first=args.plan_first), seed=1).to(dev).eval()
     x0 = torch.randn(NB, 5, H, W, generator=torch.Generator().manual_seed(2)) * 0.5
     n_inputs = 16
     deltas_cpu = [event_voxel_delta(NB, 5, H, W, dens, seed=3000 + i)[0] for i in range(n_inputs)]
@@ -270,6 +272,7 @@ def main():
 
     # ---- per-layer roofline table: eager launches with HIP events, several repeats ------------
     with torch.no_grad():
+        model.plan_first = False          # one walk per step: the probe times every wrapper call once
         model.forward_refresh_reservoirs(cl(x0), None)
         step_eager(model, 0)
         agg = None
@@ -418,7 +421,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": "E2Depth-incr recurrent UNet, random init, %dx5x%dx%d event voxel deltas, %.0f%% "
                                "active pixels, 1 dense refresh then incremental steps" % (NB, H, W, 100 * dens),
-                   "density": dens, "height": H, "width": W, "batch": NB, "graph": not args.no_graph},
+                   "density": dens, "height": H, "width": W, "batch": NB, "graph": not args.no_graph,
+                   "mask_planning": "inline" if args.sync_masks else ("second stream, builds first" if args.plan_first else "second stream")},
         "roofline": roofline,
         "cpu_baseline": cpu,
         "hbm_gbs_whole_frame": round(tot_bytes / sec_per_step / 1e9, 1),

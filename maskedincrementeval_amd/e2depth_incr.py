@@ -568,9 +568,13 @@ class E2VIDRecurrentIncr(nn.Module, _IncrBuffers):
     """
 
     def __init__(self, config=None, fuse=True, mask_threshold: float = 0.0, derive_input_mask=True,
-                 async_masks=False):
+                 async_masks=False, plan_first=False):
         super().__init__()
         self.async_masks = async_masks     # build the tile sets on a second stream, ahead of the convs
+        # with async_masks: walk the network twice per step, first launching only the mask builds, then
+        # only the other kernels (needs masks that depend on the input mask alone: no refined masks, no
+        # delta quantisers)
+        self.plan_first = plan_first
         cfg = dict(E2DEPTH_DEFAULT_CONFIG)
         cfg.update(config or {})
         self.num_bins = int(cfg['num_bins'])
@@ -610,7 +614,13 @@ class E2VIDRecurrentIncr(nn.Module, _IncrBuffers):
         with ops.mask_planner(delta.device):
             if mask is None and self.derive_input_mask:
                 mask = self.input_mask(delta)
-            img_pred, states = self.unetrecurrent.forward([delta, mask], prev_states)
+            if self.plan_first:
+                with ops.network_pass("plan"):
+                    self.unetrecurrent.forward([delta, mask], prev_states)
+                with ops.network_pass("compute"):
+                    img_pred, states = self.unetrecurrent.forward([delta, mask], prev_states)
+            else:
+                img_pred, states = self.unetrecurrent.forward([delta, mask], prev_states)
         return img_pred, states
 
     def forward_refresh_reservoirs(self, event_tensor: DenseT, prev_states):

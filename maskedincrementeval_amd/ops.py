@@ -9,8 +9,52 @@ from typing import Optional, Tuple
 import torch
 
 from . import _lib
-from ._lib import check, lib
+from ._lib import check
 from .masked_types import TileMask
+
+# ---- planning pass / compute pass -----------------------------------------------------------------
+# A network whose masks depend on the input mask only can be walked twice per step: a planning pass in
+# which only the mask builds are launched (onto the planning stream), then a compute pass in which
+# only the other kernels are.  All builds are then enqueued -- and, in a captured graph, ordered --
+# ahead of the kernels that consume them.  `_phase` is None outside such a walk.
+_phase = None
+_BUILD_ENTRIES = ("mie_build_mask_tiles",)
+
+
+class _PhaseLib:
+    def __init__(self, real):
+        self._real = real
+
+    def __getattr__(self, name):
+        fn = getattr(self._real, name)
+        if name.startswith("mie_") and name not in ("mie_last_error_string", "mie_tile_capacity", "mie_version",
+                                                     "mie_pack_filter"):
+            runs = (name in _BUILD_ENTRIES) == (_phase == "plan")
+            if not runs:
+                return lambda *args: 0
+        return fn
+
+
+def lib():
+    real = _lib.lib()
+    return real if _phase is None else _PhaseLib(real)
+
+
+class network_pass:
+    """`with network_pass("plan")` / `with network_pass("compute")`: see above."""
+
+    def __init__(self, phase):
+        self.phase = phase
+
+    def __enter__(self):
+        global _phase
+        self.prev, _phase = _phase, self.phase
+        return self
+
+    def __exit__(self, *exc):
+        global _phase
+        _phase = self.prev
+        return False
 
 
 def _stream(t: torch.Tensor):
@@ -64,6 +108,8 @@ class mask_planner:
 
 def _ready(ts: TileMask):
     """Make the compute stream wait for the build of `ts` (once)."""
+    if _phase == "plan":
+        return
     root = ts.parent if ts.parent is not None else ts
     ev = root.__dict__.get("ready")
     if ev is not None:
@@ -71,8 +117,13 @@ def _ready(ts: TileMask):
         root.ready = None
 
 
-def _mark_pix(t: Optional[torch.Tensor]):
+def _mark_pix(t: Optional[torch.Tensor], from_values: bool = False):
     """A pixel mask was written on the compute stream: builds that read it must wait."""
+    if t is not None and from_values and _phase is not None:
+        raise RuntimeError("a mask that depends on values (a delta, refined or quantised deltas) cannot be "
+                           "planned ahead: run this network without the planning pass")
+    if _phase == "compute":
+        return
     if _planner is not None and t is not None:
         ev = torch.cuda.Event()
         ev.record(torch.cuda.current_stream(t.device))
@@ -167,7 +218,7 @@ def mask_from_delta(delta: torch.Tensor, threshold: float, out: torch.Tensor):
     n, c, h, w = delta.shape
     check(lib().mie_mask_from_delta(nhwc_ptr(delta, "delta", dtype=delta.dtype), n, h, w, c, float(threshold),
                                     pix_ptr(out, n, h, w, "out"), delta_dtype(delta), _stream(delta)))
-    _mark_pix(out)
+    _mark_pix(out, from_values=True)
     return out
 
 
@@ -177,6 +228,8 @@ def build_mask_tiles(in_mask, in_mask2, n, h_in, w_in, foot, k, stride, pad, out
     p2 = pix_ptr(in_mask2, n, h_in, w_in, "in_mask2")
     if p1 is None and p2 is not None:   # "all active" OR anything = all active
         p2 = None
+    if _phase == "compute":             # built by the planning pass; its event is still attached
+        return out
     if _planner is None or _planner[1] != out.device:
         st = torch.cuda.current_stream(out.device).cuda_stream
         check(lib().mie_build_mask_tiles(p1, p2, h_in, w_in, foot, k, stride, pad, out.ref, st))
@@ -371,7 +424,7 @@ def act_incr(kind, slope, in_delta, reservoir, out_delta, ts: TileMask, out_pixm
                              ts.ref, pix_ptr(out_pixmask, n, h, w, "out_pixmask"),
                              _lib.FLAG_KEEP_RESERVOIR if keep_reservoir else 0, delta_dtype(in_delta),
                              _stream(in_delta)))
-    _mark_pix(out_pixmask)
+    _mark_pix(out_pixmask, from_values=True)
     return out_delta
 
 
@@ -395,7 +448,7 @@ def kfence_incr(in_delta, carry, k, out_delta, ts: TileMask, out_pixmask=None):
                                 nhwc_ptr(out_delta, "out_delta", dtype=dt), c, ts.ref,
                                 pix_ptr(out_pixmask, n, h, w, "out_pixmask"), delta_dtype(in_delta),
                                 _stream(in_delta)))
-    _mark_pix(out_pixmask)
+    _mark_pix(out_pixmask, from_values=True)
     return out_delta
 
 

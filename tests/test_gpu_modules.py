@@ -289,14 +289,15 @@ def test_convlstm_with_previous_state_deltas(cin, hid):
         _close(dh[0], dh_r, "dh %d" % step), _close(dc[0], dc_r, "dc %d" % step)
 
 
+@pytest.mark.parametrize("plan_first", [False, True])
 @pytest.mark.parametrize("graph", [False, True])
-def test_async_mask_planning_gives_the_same_frames_as_inline_planning(graph):
+def test_async_mask_planning_gives_the_same_frames_as_inline_planning(graph, plan_first):
     # Tile sets built on the planning stream (eagerly and as edges of a replayed HIP graph) must be the
     # ones inline planning builds: the same kernels then run over the same tiles, so the predictions
     # agree bit for bit.  Every step has a fresh mask, so a build that read a mask of the previous
     # step (or raced with the kernel that writes it) shows up as a difference.
     h, w, steps = 72, 104, 8
-    a = seed_module_(E2VIDRecurrentIncr(async_masks=True), seed=31).to(DEV).eval()
+    a = seed_module_(E2VIDRecurrentIncr(async_masks=True, plan_first=plan_first), seed=31).to(DEV).eval()
     s = seed_module_(E2VIDRecurrentIncr(async_masks=False), seed=31).to(DEV).eval()
     x0 = torch.randn(1, 5, h, w, generator=torch.Generator().manual_seed(32)) * 0.5
     deltas = [_cl(event_voxel_delta(1, 5, h, w, 0.03 + 0.02 * (i % 3), seed=4100 + i)[0]) for i in range(steps)]
@@ -322,3 +323,17 @@ def test_async_mask_planning_gives_the_same_frames_as_inline_planning(graph):
         torch.cuda.synchronize()
     for i in range(steps):
         assert torch.equal(got[i], refs[i]), "step %d max|diff| = %.3e" % (i, (got[i] - refs[i]).abs().max().item())
+
+
+def test_planning_pass_refuses_masks_that_depend_on_values():
+    # a delta quantiser emits a refined mask from the values it lets through: nothing downstream of it
+    # can be planned before the compute pass has run
+    h, w = 40, 56
+    m = seed_module_(E2VIDRecurrentIncr(async_masks=True, plan_first=True), seed=33).to(DEV).eval()
+    mm.set_kfence(m, 1e-3)
+    x0 = torch.randn(1, 5, h, w, generator=torch.Generator().manual_seed(34))
+    with torch.no_grad():
+        m.forward_refresh_reservoirs(_cl(x0), None)
+        with pytest.raises(RuntimeError, match="cannot be planned ahead"):
+            m([_cl(event_voxel_delta(1, 5, h, w, 0.05, seed=35)[0]), None], None)
+    assert ops._phase is None and ops._planner is None      # both context managers unwound
