@@ -343,9 +343,11 @@ def main():
           (tot_us, tot_bytes / 1e6, tot_flops / 1e9), file=sys.stderr, flush=True)
 
     # ---- dense comparator: same kernels, every tile active ---------------------------------------
+    model.plan_first = args.plan_first
     dense_sec = None
     if not args.no_dense:
-        dense_model = seed_module_(E2VIDRecurrentIncr(derive_input_mask=False), seed=1).to(dev).eval()
+        dense_model = seed_module_(E2VIDRecurrentIncr(derive_input_mask=False, async_masks=not args.sync_masks,
+                                                       plan_first=args.plan_first), seed=1).to(dev).eval()
         dense_sec = timed_run(dense_model, "dense (all tiles active, same kernels)")
         del dense_model
 
