@@ -166,11 +166,16 @@ __global__ __launch_bounds__(256) void k_conv1x1_smallco(ConvArgsT<T> a) {
     return;
   }
   float acc[4] = {0.f, 0.f, 0.f, 0.f};
-  if (inb && (a.xm == nullptr || a.xm[po])) {
-    const T* xr = a.x + po * a.c1;
-    for (int v = sub; v < (a.c1 >> 2); v += 4) {
+  for (int src = 0; src < 2; ++src) {        // x feeds filter rows [0, c1), x2 rows [c1, c1 + c2)
+    const T* xin = src ? a.x2 : a.x;
+    const uint8_t* xm = src ? a.x2m : a.xm;
+    const int cs = src ? a.c2 : a.c1;
+    if (xin == nullptr || !inb || (xm != nullptr && !xm[po])) continue;
+    const T* xr = xin + po * cs;
+    const float* wrow = a.filt + (long long)(src ? a.c1 : 0) * a.cout;
+    for (int v = sub; v < (cs >> 2); v += 4) {
       const float4 x = load4(xr + 4 * v);
-      const float* wp = a.filt + (long long)(4 * v) * a.cout;
+      const float* wp = wrow + (long long)(4 * v) * a.cout;
       for (int co = 0; co < a.cout; ++co)
         acc[co] += x.x * wp[co] + x.y * wp[a.cout + co] + x.z * wp[2 * a.cout + co] + x.w * wp[3 * a.cout + co];
     }
@@ -223,7 +228,7 @@ __global__ __launch_bounds__(256) void k_tconv_valu(ConvArgsT<T> a, int K, int S
 
 template <typename T, int K, int S>
 void launch_conv(const ConvArgsT<T>& a, unsigned cap, hipStream_t st) {
-  if (K == 1 && S == 1 && a.pad == 0 && a.cout <= 4 && a.x2 == nullptr && (a.c1 & 3) == 0) {
+  if (K == 1 && S == 1 && a.pad == 0 && a.cout <= 4 && (a.c1 & 3) == 0 && (a.c2 & 3) == 0) {
     hipLaunchKernelGGL((k_conv1x1_smallco<T>), dim3(cap), dim3(256), 0, st, a);
   } else if (a.cout <= 4) {
     hipLaunchKernelGGL((k_conv_smallco<T, K, S>), dim3(cap), dim3(64), 0, st, a);

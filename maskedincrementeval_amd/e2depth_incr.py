@@ -521,13 +521,23 @@ class UNetRecurrentIncr(BaseUNetIncr):
             x_incr = resblock(x_incr)
         for i, decoder in enumerate(self.decoders):
             x_incr = decoder(x_incr, blocks[self.num_encoders - i - 1])
-        summed = self.pred_add(x_incr, head)
         if self.fuse and self.norm not in ['BN', 'IN']:
-            # 1x1 conv and output activation in one kernel (the pre-activation reservoir is the activation's)
-            pred_incr = self.pred.conv2d.forward_fused(summed, self.activation)
+            # skip sum, 1x1 conv and output activation in one kernel: the conv is linear, so
+            # pred(x + head) is the conv of the two tensors side by side with the filter rows repeated
+            # (the pre-activation reservoir is the activation's)
+            pred_incr = self.pred.conv2d.forward_fused(x_incr, self.activation, x2_incr=head,
+                                                       filt=self._pred_sum_filter())
         else:
-            pred_incr = self.activation(self.pred(summed))
+            pred_incr = self.activation(self.pred(self.pred_add(x_incr, head)))
         return pred_incr, states_incr
+
+    def _pred_sum_filter(self):
+        base = self.pred.conv2d.conv2d_weights
+        cached = self.__dict__.get("_pred_sum_filt")
+        if cached is None or cached[0] is not base:
+            cached = (base, ops.ConvFilter(torch.cat((base.plain, base.plain), 0).contiguous()))
+            self.__dict__["_pred_sum_filt"] = cached
+        return cached[1]
 
     def forward_refresh_reservoirs(self, x: DenseT, prev_states):
         x = self.head.forward_refresh_reservoirs(x)
