@@ -97,7 +97,13 @@ class LayerProbe:
             return dict(kind="conv", k=3, s=1, cin=c1 + c2, cout=filt.shape[3], h=h, w=w, n=n,
                         xmask=xmask, x2mask=x2mask, ts=out_ts, fused=True, gates=True)
 
+        def upconv_desc(a_, amask, b_, bmask, filt, k, pad, out_ts, out_delta, reservoir=None, *a, **kw):
+            n, c, h, w = a_.shape
+            return dict(kind="conv", k=k, s=1, cin=c, cout=filt.shape[3], h=h, w=w, n=n, xmask=amask,
+                        x2mask=bmask, ts=out_ts, fused=reservoir is not None, up=True, two=b_ is not None)
+
         self._wrap("conv_masked", conv_desc)
+        self._wrap("upconv_masked", upconv_desc)
         self._wrap("conv_gates_incr", conv_gates_desc)
         self._wrap("act_incr", pw_desc("act", 1, 1))
         self._wrap("add_incr", pw_desc("add", 2, 0))
@@ -123,6 +129,10 @@ class LayerProbe:
                 ts = d["ts"]
                 P = d["n"] * d["h"] * d["w"]
                 a_in = P if d["xmask"] is None else int(self._pix(d["xmask"]).sum().item())
+                if d.get("up") and d["two"]:
+                    # up2x(a + b) formed on the fly: both half-resolution inputs are read once, nothing in between
+                    a_in += P if d["x2mask"] is None else int(self._pix(d["x2mask"]).sum().item())
+                    P *= 2
                 a_out = int(ts.pixmask.sum().item())
                 cin, cout, k = d["cin"], d["cout"], d["k"]
                 es = self.es
@@ -136,8 +146,8 @@ class LayerProbe:
                     byts += a_out * cout * es
                     if d["fused"]:
                         byts += 2 * a_out * cout * 4
-                row.update(shape="%dx%d s%d %d->%d%s @%dx%d" % (k, k, d["s"], cin, cout,
-                                                                 "+lstm" if d.get("gates") else "", ts.h, ts.w),
+                row.update(shape="%s%dx%d s%d %d->%d%s @%dx%d" % ("up2x+" if d.get("up") else "", k, k, d["s"], cin, cout,
+                                                                   "+lstm" if d.get("gates") else "", ts.h, ts.w),
                            active_tiles=int(ts.counts[0].item()), tiles=ts.capacity, a_out=a_out,
                            bytes=byts, flops=2 * a_out * cin * cout * k * k)
             elif d["kind"] in ("act", "add", "mul", "up2x", "gates"):
@@ -298,7 +308,7 @@ def main():
                            gbs=round(byts / (ms * 1e-3) / 1e9, 1) if ms > 0 else None,
                            tflops=round(fl / (ms * 1e-3) / 1e12, 2) if ms > 0 else None,
                            bytes=int(byts), flops=int(fl), active_tiles=r.get("active_tiles"), tiles=r.get("tiles")))
-    convs = [l for l in layers if l["op"] in ("conv_masked", "conv_gates_incr")]
+    convs = [l for l in layers if l["op"] in ("conv_masked", "conv_gates_incr", "upconv_masked")]
     dom = max(convs, key=lambda l: l["us"])
     # Re-time the dominant launch on its own: the same call (same tile set, same buffers)
     # replayed back to back between two HIP events on the launch stream.

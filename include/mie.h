@@ -399,6 +399,27 @@ int mie_linear_incr(const void* in_delta, int n, int f_in, const float* weight_t
                     int f_out, void* out_delta, int dtype, void* stream);
 
 /*
+ * Bilinear x2 up-sampling (align_corners = False) of a + b followed by the 5x5
+ * stride-1 pad-2 conv of mie_conv_masked, in one kernel: the up-sampled tensor
+ * is never written.  a (mask amask) and the optional b (mask bmask) are
+ * [n,h_in,w_in,c] deltas at HALF the output resolution; `out` is the conv's tile
+ * set at (2*h_in, 2*w_in), built from the up-sampled mask (MIE_FOOT_UP2X, then
+ * MIE_FOOT_CONV).  Matrix-core path only: filter_mc is required, c must be a
+ * multiple of the staging chunk (32 fp32 / 64 bf16 channels) and cout of 32;
+ * otherwise MIE_ERR_UNSUPPORTED (use mie_upsample2x_incr + mie_conv_masked).
+ * Epilogue (addend, reservoir, activation) as in mie_conv_masked.
+ * Replaces: interpolate_from_module + nnConvIncr.forward of
+ * UpsampleConvLayerIncr.forward with the skip sum in front of it
+ * (incr_modules/e2depth_incr.py:306-313, 429-431).
+ */
+int mie_upconv_masked(const void* a, const uint8_t* amask, const void* b,
+                      const uint8_t* bmask, int c, int h_in, int w_in,
+                      const float* filter, const void* filter_mc, int cin_total,
+                      int k, int pad, int cout, const mie_tileset* out,
+                      void* out_delta, const void* addend, float* reservoir,
+                      int act_kind, float slope, int dtype, void* stream);
+
+/*
  * Masked transposed convolution of a delta (stride s, padding p; the output
  * size out->h/w fixes output_padding): out(oy,ox,co) = sum x(iy,ix,ci) *
  * filter[ci][ky][kx][co] over oy = iy*s - p + ky, ox = ix*s - p + kx, with

@@ -33,7 +33,7 @@ EXPORTS = (
     "mie_build_mask_tiles", "mie_conv_masked", "mie_act_incr", "mie_mul_incr", "mie_add_incr",
     "mie_upsample2x_incr", "mie_convlstm_gates_incr", "mie_tconv_masked", "mie_conv_refresh",
     "mie_pack_filter", "mie_kfence_incr", "mie_events_to_frame", "mie_tconv_refresh", "mie_conv_gates_masked",
-    "mie_maxpool_incr", "mie_accumulate", "mie_scale_incr", "mie_avgpool_incr", "mie_linear_incr",
+    "mie_maxpool_incr", "mie_accumulate", "mie_scale_incr", "mie_avgpool_incr", "mie_linear_incr", "mie_upconv_masked",
 )
 
 
@@ -106,6 +106,8 @@ def _declare(l):
     l.mie_avgpool_incr.argtypes = [vp, vp, ci, ci, ci, ci, ci, ci, vp, ci, vp]
     l.mie_linear_incr.restype = ci
     l.mie_linear_incr.argtypes = [vp, ci, ci, vp, ci, vp, ci, vp]
+    l.mie_upconv_masked.restype = ci
+    l.mie_upconv_masked.argtypes = [vp, vp, vp, vp, ci, ci, ci, vp, vp, ci, ci, ci, ci, tsp, vp, vp, vp, ci, cf, ci, vp]
     l.mie_tconv_refresh.restype = ci
     l.mie_tconv_refresh.argtypes = [vp, ci, ci, ci, vp, ci, ci, ci, ci, vp, tsp, vp, vp, ci, cf, ci, vp]
     l.mie_tconv_masked.restype = ci

@@ -104,6 +104,10 @@ bool mie_launch_conv_mfma(const ConvArgsT<mie_bf16>& a, int k, int s, unsigned c
 // filter columns in the gate-interleaved order of mie_conv_gates_masked).
 bool mie_launch_conv_gates_mfma(const ConvArgsT<float>& a, unsigned cap, hipStream_t st);
 bool mie_launch_conv_gates_mfma(const ConvArgsT<mie_bf16>& a, unsigned cap, hipStream_t st);
+// The 5x5 stride-1 pad-2 conv over up2x(a.x + a.x2) (both at half resolution, a.c1 channels each, a.x2
+// optional); a.h_in / a.w_in are the up-sampled size.
+bool mie_launch_conv_up_mfma(const ConvArgsT<float>& a, unsigned cap, hipStream_t st);
+bool mie_launch_conv_up_mfma(const ConvArgsT<mie_bf16>& a, unsigned cap, hipStream_t st);
 
 // One element of the ConvLSTM gate chain: pre-activation gate reservoirs r* and their deltas d*, cached
 // previous cell state cp and its delta dP, cached cell state c0.  Updates the reservoirs in place and

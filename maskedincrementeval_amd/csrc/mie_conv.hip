@@ -535,6 +535,61 @@ extern "C" int mie_tconv_refresh(const void* x, int cin, int h_in, int w_in, con
                      out_dense, reservoir, act_kind, slope, true, bias, dtype, stream);
 }
 
+namespace {
+template <typename T>
+int upconv_entry(const char* who, const void* a_lo, const uint8_t* amask, const void* b_lo, const uint8_t* bmask,
+                 int c, int h_lo, int w_lo, const float* filter, const void* filter_mc, int cin_total, int k,
+                 int pad, int cout, const mie_tileset* out, void* out_delta, const void* addend, float* reservoir,
+                 int act_kind, float slope, void* stream) {
+  int rc = mie_check_tileset(out, who);
+  if (rc != MIE_OK) return rc;
+  MIE_REQUIRE(a_lo && filter && filter_mc, MIE_ERR_INVALID_ARG, "%s: NULL pointer (a, filter and filter_mc are required)", who);
+  MIE_REQUIRE(b_lo != nullptr || bmask == nullptr, MIE_ERR_INVALID_ARG, "%s: mask of absent b", who);
+  MIE_REQUIRE(c > 0 && cout > 0 && h_lo > 0 && w_lo > 0 && cin_total >= c, MIE_ERR_INVALID_ARG,
+              "%s: sizes out of range (c=%d cout=%d cin_total=%d h=%d w=%d)", who, c, cout, cin_total, h_lo, w_lo);
+  MIE_REQUIRE(k == 5 && pad == 2, MIE_ERR_UNSUPPORTED, "%s: only the 5x5 pad-2 conv is implemented (k=%d pad=%d)", who, k, pad);
+  const int chunk = 128 / (int)sizeof(T);      // 32 fp32 / 64 bf16 channels per staged chunk
+  MIE_REQUIRE(c % chunk == 0 && cout % 32 == 0 && cin_total % (32 / (int)sizeof(T)) == 0, MIE_ERR_UNSUPPORTED,
+              "%s: needs c %% %d == 0 and cout %% 32 == 0 (c=%d cout=%d)", who, chunk, c, cout);
+  MIE_REQUIRE(out->h == 2 * h_lo && out->w == 2 * w_lo, MIE_ERR_INVALID_ARG,
+              "%s: the tile set is (%d,%d), twice the input is (%d,%d)", who, out->h, out->w, 2 * h_lo, 2 * w_lo);
+  MIE_REQUIRE((long long)out->n * h_lo * w_lo * c < (1LL << 40) && (long long)out->n * out->h * out->w < 0x7fffffffLL,
+              MIE_ERR_CAPACITY, "%s: input too large", who);
+  MIE_REQUIRE(mie_aligned(a_lo, 16) && mie_aligned(b_lo, 16) && mie_aligned(filter, 16) && mie_aligned(filter_mc, 16) &&
+                  mie_aligned(addend, 16),
+              MIE_ERR_INVALID_ARG, "%s: a / b / filter / filter_mc / addend must be 16-byte aligned", who);
+  MIE_REQUIRE(addend == nullptr || addend != out_delta, MIE_ERR_INVALID_ARG, "%s: addend must not alias out_delta", who);
+  rc = check_epilogue(who, out_delta, reservoir, act_kind, false);
+  if (rc != MIE_OK) return rc;
+  ConvArgsT<T> a;
+  a.x = (const T*)a_lo; a.xm = amask; a.c1 = c; a.x2 = (const T*)b_lo; a.x2m = bmask; a.c2 = b_lo ? c : 0;
+  a.h_in = 2 * h_lo; a.w_in = 2 * w_lo; a.filt = filter; a.cin_total = cin_total; a.filt_mc = (const T*)filter_mc;
+  a.pad = pad; a.cout = cout; a.out = (T*)out_delta; a.res = reservoir; a.act = act_kind;
+  a.slope = slope; a.addend = (const T*)addend; a.refresh = 0; a.bias = nullptr;
+  a.hid = 0; a.g_cpd = nullptr; a.g_cpm = nullptr; a.g_cpres = nullptr; a.g_cres = nullptr;
+  a.g_dh = nullptr; a.g_dc = nullptr;
+  a.ts = mie_dev_tileset(out);
+  const unsigned cap = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
+  MIE_REQUIRE(mie_launch_conv_up_mfma(a, cap, (hipStream_t)stream), MIE_ERR_UNSUPPORTED,
+              "%s: no kernel variant for c=%d cout=%d", who, c, cout);
+  return mie_check_launch(who);
+}
+}  // namespace
+
+extern "C" int mie_upconv_masked(const void* a, const uint8_t* amask, const void* b, const uint8_t* bmask, int c,
+                                 int h_in, int w_in, const float* filter, const void* filter_mc, int cin_total,
+                                 int k, int pad, int cout, const mie_tileset* out, void* out_delta,
+                                 const void* addend, float* reservoir, int act_kind, float slope, int dtype,
+                                 void* stream) {
+  const char* who = "mie_upconv_masked";
+  MIE_CONV_DTYPE_OK(dtype, who);
+  if (dtype == MIE_DTYPE_BF16)
+    return upconv_entry<mie_bf16>(who, a, amask, b, bmask, c, h_in, w_in, filter, filter_mc, cin_total, k, pad, cout,
+                                  out, out_delta, addend, reservoir, act_kind, slope, stream);
+  return upconv_entry<float>(who, a, amask, b, bmask, c, h_in, w_in, filter, filter_mc, cin_total, k, pad, cout, out,
+                             out_delta, addend, reservoir, act_kind, slope, stream);
+}
+
 extern "C" int mie_conv_gates_masked(const void* x, const uint8_t* xmask, int c1, const void* x2,
                                      const uint8_t* x2mask, int c2, int h_in, int w_in,
                                      const float* filter, const void* filter_mc, int cin_total,

@@ -7,3 +7,6 @@ bool mie_launch_conv_mfma(const ConvArgsT<mie_bf16>& a, int k, int s, unsigned c
 bool mie_launch_conv_gates_mfma(const ConvArgsT<mie_bf16>& a, unsigned cap, hipStream_t st) {
   return launch_gates<mie_bf16>(a, cap, st);
 }
+bool mie_launch_conv_up_mfma(const ConvArgsT<mie_bf16>& a, unsigned cap, hipStream_t st) {
+  return launch_up<mie_bf16>(a, cap, st);
+}

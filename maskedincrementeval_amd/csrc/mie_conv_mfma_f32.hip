@@ -19,3 +19,6 @@ bool mie_launch_conv_mfma(const ConvArgsT<float>& a, int k, int s, unsigned cap,
 bool mie_launch_conv_gates_mfma(const ConvArgsT<float>& a, unsigned cap, hipStream_t st) {
   return launch_gates<float>(a, cap, st);
 }
+bool mie_launch_conv_up_mfma(const ConvArgsT<float>& a, unsigned cap, hipStream_t st) {
+  return launch_up<float>(a, cap, st);
+}

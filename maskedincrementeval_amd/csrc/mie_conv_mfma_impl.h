@@ -102,7 +102,42 @@ __device__ __forceinline__ void mma_unit(v16f& acc, const float4& av, const floa
                                                 __builtin_bit_cast(mie_bf16x8, b4), acc, 0, 0, 0);
 }
 
-template <typename T, int K, int S, int WN, int NB, bool HALF, bool GATES = false>
+// Source rows / columns and weights of output index o of a bilinear x2 up-sampling (align_corners =
+// False): src = max(0, o/2 - 0.25), upper index clamped to the last row.
+__device__ __forceinline__ void conv_up2x_coef(int o, int in_size, int& i0, int& i1, float& l0, float& l1) {
+  const int j = o >> 1;
+  if (o & 1) {
+    i0 = j; i1 = (j + 1 < in_size) ? j + 1 : j; l0 = 0.75f; l1 = 0.25f;
+  } else if (j == 0) {
+    i0 = 0; i1 = (1 < in_size) ? 1 : 0; l0 = 1.f; l1 = 0.f;
+  } else {
+    i0 = j - 1; i1 = j; l0 = 0.25f; l1 = 0.75f;
+  }
+}
+// One 16-byte slot of delta elements <-> fp32 values (4 of them, or 8 for bf16).
+__device__ __forceinline__ void slot_to_f32(const float4& raw, float (&f)[4], float) {
+  f[0] = raw.x; f[1] = raw.y; f[2] = raw.z; f[3] = raw.w;
+}
+__device__ __forceinline__ void slot_to_f32(const float4& raw, float (&f)[8], mie_bf16) {
+  const v4f r4 = {raw.x, raw.y, raw.z, raw.w};
+  const mie_bf16x8 b = __builtin_bit_cast(mie_bf16x8, r4);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) f[e] = (float)b[e];
+}
+__device__ __forceinline__ float4 f32_to_slot(const float (&f)[4], float) { return make_float4(f[0], f[1], f[2], f[3]); }
+__device__ __forceinline__ float4 f32_to_slot(const float (&f)[8], mie_bf16) {
+  mie_bf16x8 b;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) b[e] = (mie_bf16)f[e];
+  const v4f r4 = __builtin_bit_cast(v4f, b);
+  return make_float4(r4[0], r4[1], r4[2], r4[3]);
+}
+
+// UP: the conv input is up2x(x + x2), the bilinear x2 up-sampling of the sum of two deltas given at
+// half resolution (x2 optional), and is never formed in memory: per chunk the 8x8 block of source
+// pixels a tile's 12x12 input window blends is summed into LDS (fp32), and the staged tile is expanded
+// from there.  5x5, stride 1, pad 2 only; a.h_in / a.w_in are the up-sampled size.
+template <typename T, int K, int S, int WN, int NB, bool HALF, bool GATES = false, bool UP = false>
 __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   constexpr int NBUF = stage_buffers(S, (int)sizeof(T));
   constexpr int EPS = 16 / (int)sizeof(T);                   // elements per 16-byte slot (4 / 8)
@@ -126,10 +161,14 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   constexpr int CO_BLK = 32 * NB * WN;
   constexpr int RED = (WK > 1 || GATES) ? WK * 64 * CO_BLK : 0;
   constexpr int STAGE_F = NBUF * STAGE * (int)sizeof(T) / 4;  // the staging buffers, in floats
-  constexpr int SMEM = (STAGE_F > RED) ? STAGE_F : RED;
+  constexpr int LOS = CC;                                    // floats per source pixel in LDS
+  constexpr int LO_F = UP ? 64 * LOS : 0;                    // fp32 sums of the 8x8 source block, CC channels
+  static_assert(!UP || (S == 1 && K == 5 && !GATES), "the up-sampling variant is the 5x5 stride-1 conv");
+  constexpr int SMEM = ((STAGE_F > RED) ? STAGE_F : RED) + LO_F;
   static_assert(SMEM * 4 <= 65536, "LDS budget");
   __shared__ __attribute__((aligned(16))) float smem[SMEM];
   T* const sbuf = reinterpret_cast<T*>(smem);
+  float* const s_lo = smem + (SMEM - LO_F);
 
   int n, y0, x0;
   const int tk = mie_pick_tile(a.ts, blockIdx.x, n, y0, x0);
@@ -213,7 +252,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
     st_lds[i] = lrow * RP + (pix - lrow * IT) * LS + EPS * (q4 ^ swz);
     st_c4[i] = EPS * q4;
     st_po[i] = 0;
-    if (slot < NSLOT) {
+    if (!UP && slot < NSLOT) {
       const int iy = iy0 + pix / IT, ix = ix0 + pix % IT;
       if (iy >= 0 && iy < a.h_in && ix >= 0 && ix < a.w_in) {
         const int po = (n * a.h_in + iy) * a.w_in + ix;
@@ -224,10 +263,50 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
     }
   }
   const int nch1 = (a.c1 + CC - 1) / CC;
-  const int nch = nch1 + ((a.x2 != nullptr) ? (a.c2 + CC - 1) / CC : 0);
+  const int nch = nch1 + ((!UP && a.x2 != nullptr) ? (a.c2 + CC - 1) / CC : 0);
+
+  // UP: the source block.  Rows iy0 .. iy0+11 of the up-sampled image (iy0 even) blend source rows
+  // iy0/2 - 1 .. iy0/2 + 6; one 16-byte slot per (source pixel, channel group) and tensor.
+  constexpr int NLO = UP ? (64 * Q4 + 255) / 256 : 1;
+  const int h_lo = a.h_in >> 1, w_lo = a.w_in >> 1;
+  const int lo_y0 = (iy0 >> 1) - 1, lo_x0 = (ix0 >> 1) - 1;
+  int lo_po[NLO];
+  unsigned lo_ok1 = 0u, lo_ok2 = 0u;
+  float4 lo_a[NLO], lo_b[NLO];
+  if (UP) {
+#pragma unroll
+    for (int i = 0; i < NLO; ++i) {
+      const int slot = tid + 256 * i;
+      const int lpix = slot / Q4;
+      const int ly = lo_y0 + (lpix >> 3), lx = lo_x0 + (lpix & 7);
+      lo_po[i] = 0;
+      if (lpix < 64 && ly >= 0 && ly < h_lo && lx >= 0 && lx < w_lo) {
+        const int po = (n * h_lo + ly) * w_lo + lx;
+        lo_po[i] = po;
+        if (a.xm == nullptr || a.xm[po]) lo_ok1 |= 1u << i;
+        if (a.x2 != nullptr && (a.x2m == nullptr || a.x2m[po])) lo_ok2 |= 1u << i;
+      }
+    }
+  }
 
   float4 st_reg[NLD];
   auto stage_load = [&](int c) {
+    if constexpr (UP) {
+      const T* dummy = a.filt_mc;
+#pragma unroll
+      for (int i = 0; i < NLO; ++i) {
+        const int q4 = (tid + 256 * i) % Q4;
+        const long long eo = (long long)lo_po[i] * a.c1 + c * CC + EPS * q4;
+        const bool k1 = (lo_ok1 >> i) & 1u, k2 = (lo_ok2 >> i) & 1u;
+        float4 v = *reinterpret_cast<const float4*>(k1 ? a.x + eo : dummy);
+        float4 u = *reinterpret_cast<const float4*>(k2 ? a.x2 + eo : dummy);
+        v.x = k1 ? v.x : 0.f; v.y = k1 ? v.y : 0.f; v.z = k1 ? v.z : 0.f; v.w = k1 ? v.w : 0.f;
+        u.x = k2 ? u.x : 0.f; u.y = k2 ? u.y : 0.f; u.z = k2 ? u.z : 0.f; u.w = k2 ? u.w : 0.f;
+        lo_a[i] = v;
+        lo_b[i] = u;
+      }
+      return;
+    }
     const bool second = c >= nch1;
     const T* xin = second ? a.x2 : a.x;
     const int cs = second ? a.c2 : a.c1;
@@ -251,6 +330,56 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   };
   auto stage_store = [&](int buf) {
     T* dst = sbuf + buf * STAGE;
+    if constexpr (UP) {
+      // x + x2 of the source block to LDS in fp32 (bit pattern zero = 0 in both element types) ...
+#pragma unroll
+      for (int i = 0; i < NLO; ++i) {
+        const int slot = tid + 256 * i;
+        const int lpix = slot / Q4, q4 = slot - lpix * Q4;
+        float fa[EPS], fb[EPS];
+        slot_to_f32(lo_a[i], fa, T());
+        slot_to_f32(lo_b[i], fb, T());
+        if (lpix < 64) {
+#pragma unroll
+          for (int e = 0; e < EPS; e += 4)
+            *reinterpret_cast<float4*>(&s_lo[lpix * LOS + q4 * EPS + e]) =
+                make_float4(fa[e] + fb[e], fa[e + 1] + fb[e + 1], fa[e + 2] + fb[e + 2], fa[e + 3] + fb[e + 3]);
+        }
+      }
+      __syncthreads();
+      // ... and the staged tile blended from it; pixels outside the up-sampled image are the conv's zero padding
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) {
+        const int slot = tid + 256 * i;
+        if (slot >= NSLOT) continue;
+        const int pix = slot / Q4, q4 = slot - pix * Q4;
+        const int hy = iy0 + pix / IT, hx = ix0 + pix % IT;
+        float o[EPS];
+#pragma unroll
+        for (int e = 0; e < EPS; ++e) o[e] = 0.f;
+        if (hy >= 0 && hy < a.h_in && hx >= 0 && hx < a.w_in) {
+          int r0, r1, q0, q1;
+          float lr0, lr1, lq0, lq1;
+          conv_up2x_coef(hy, h_lo, r0, r1, lr0, lr1);
+          conv_up2x_coef(hx, w_lo, q0, q1, lq0, lq1);
+          const float* v00 = s_lo + ((r0 - lo_y0) * 8 + (q0 - lo_x0)) * LOS + q4 * EPS;
+          const float* v01 = s_lo + ((r0 - lo_y0) * 8 + (q1 - lo_x0)) * LOS + q4 * EPS;
+          const float* v10 = s_lo + ((r1 - lo_y0) * 8 + (q0 - lo_x0)) * LOS + q4 * EPS;
+          const float* v11 = s_lo + ((r1 - lo_y0) * 8 + (q1 - lo_x0)) * LOS + q4 * EPS;
+#pragma unroll
+          for (int e = 0; e < EPS; e += 4) {       // 16-byte LDS reads
+            const float4 t00 = *reinterpret_cast<const float4*>(v00 + e), t01 = *reinterpret_cast<const float4*>(v01 + e);
+            const float4 t10 = *reinterpret_cast<const float4*>(v10 + e), t11 = *reinterpret_cast<const float4*>(v11 + e);
+            o[e] = lr0 * (lq0 * t00.x + lq1 * t01.x) + lr1 * (lq0 * t10.x + lq1 * t11.x);
+            o[e + 1] = lr0 * (lq0 * t00.y + lq1 * t01.y) + lr1 * (lq0 * t10.y + lq1 * t11.y);
+            o[e + 2] = lr0 * (lq0 * t00.z + lq1 * t01.z) + lr1 * (lq0 * t10.z + lq1 * t11.z);
+            o[e + 3] = lr0 * (lq0 * t00.w + lq1 * t01.w) + lr1 * (lq0 * t10.w + lq1 * t11.w);
+          }
+        }
+        *reinterpret_cast<float4*>(dst + st_lds[i]) = f32_to_slot(o, T());
+      }
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < NLD; ++i)
       if (tid + 256 * i < NSLOT) *reinterpret_cast<float4*>(dst + st_lds[i]) = st_reg[i];
@@ -339,7 +468,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
       __builtin_amdgcn_sched_barrier(0);
       if (PD == 0) load_b(ub_next, 0, bring[0]);   // ring of one: reload right after use
     }
-    if (NBUF == 1) __syncthreads();        // every wave is done reading the only buffer
+    if (NBUF == 1 && !UP) __syncthreads();   // every wave is done reading the only buffer (UP: stage_store syncs)
     if (more) stage_store((c + 1) % NBUF);
     __syncthreads();
     ub_cur = ub_next;
@@ -503,6 +632,27 @@ bool launch_depth(const ConvArgsT<T>& a, unsigned cap, hipStream_t st) {
         return true;
       }
       return false;
+    default:
+      return false;
+  }
+}
+
+// The 5x5 stride-1 conv over up2x(x + x2): full staging depth only.
+template <typename T>
+bool launch_up(const ConvArgsT<T>& a, unsigned cap, hipStream_t st) {
+  constexpr int FULL = stage_channels(5, 1) * (4 / (int)sizeof(T));
+  if (a.c1 % FULL != 0) return false;
+  const int cout = a.cout;
+  switch (pick_slab<5, 1, false>(cout, cap)) {
+    case 128:
+      hipLaunchKernelGGL((k_conv_mfma<T, 5, 1, 4, 1, false, false, true>), dim3(cap, cout / 128), dim3(256), 0, st, a);
+      return true;
+    case 64:
+      hipLaunchKernelGGL((k_conv_mfma<T, 5, 1, 2, 1, false, false, true>), dim3(cap, cout / 64), dim3(256), 0, st, a);
+      return true;
+    case 32:
+      hipLaunchKernelGGL((k_conv_mfma<T, 5, 1, 1, 1, false, false, true>), dim3(cap, cout / 32), dim3(256), 0, st, a);
+      return true;
     default:
       return false;
   }

@@ -415,9 +415,10 @@ class UpsampleConvLayerIncr(nn.Module):
         self.fuse = fuse
 
     def forward(self, x_incr: Masked, skip_incr: Masked = None) -> Masked:
-        x_upsampled_incr = self.upsample(x_incr, skip_incr)
         if self.fuse and self.activation is not None and self.norm not in ['BN', 'IN']:
-            return self.conv2d.forward_fused(x_upsampled_incr, self.activation)
+            # up-sampling, skip sum, conv and activation in one kernel where the shape allows it
+            return self.conv2d.forward_fused_upsampled(self.upsample, x_incr, skip_incr, self.activation)
+        x_upsampled_incr = self.upsample(x_incr, skip_incr)
         out_incr = self.conv2d(x_upsampled_incr)
         if self.norm in ['BN', 'IN']:
             out_incr = self.norm_layer(out_incr)

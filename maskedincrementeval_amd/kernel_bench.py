@@ -35,6 +35,8 @@ def main():
     ap.add_argument("--iters", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--copy-mb", type=int, default=0, help="run a plain copy of this many MiB instead")
+    ap.add_argument("--up2x", action="store_true",
+                    help="the conv reads up2x(a + b) of two deltas at half of --h/--w (mie_upconv_masked; 5x5 stride 1)")
     args = ap.parse_args()
     _lib.lib()
     dev = torch.device("cuda:0")
@@ -59,6 +61,8 @@ def main():
 
     n, cin, cout, k, s, h, w = args.n, args.cin, args.cout, args.k, args.stride, args.h, args.w
     p = k // 2
+    if args.up2x:
+        return up2x_conv(args, dev, e0, e1)
     ho, wo = ops.conv_out_size(h, w, k, s, p)
     g = torch.Generator().manual_seed(0)
     x = torch.randn((n, cin, h, w), generator=g)
@@ -104,6 +108,44 @@ def main():
                           algorithmic_flops=flops, algorithmic_bytes=byts,
                           tile_flops=2 * tiles * 64 * cin * cout * k * k,
                           tflops=round(flops / us / 1e6, 2), gbs=round(byts / us / 1e3, 1), iters=args.iters)))
+
+
+def up2x_conv(args, dev, e0, e1):
+    """mie_upconv_masked at output size --h x --w: two dense half-resolution inputs, reservoir + ReLU epilogue."""
+    n, cin, cout, k, h, w = args.n, args.cin, args.cout, args.k, args.h, args.w
+    hl, wl = h // 2, w // 2
+    dt = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+    es = 2 if args.dtype == "bf16" else 4
+    g = torch.Generator().manual_seed(0)
+    a, b = (ops.as_nhwc(torch.randn((n, cin, hl, wl), generator=g).to(dev).to(dt)
+                        .contiguous(memory_format=torch.channels_last)) for _ in range(2))
+    filt = ops.ConvFilter(he_normal_conv_weight(cout, cin, k, 0).permute(1, 2, 3, 0).contiguous().to(dev))
+    ts_up, ts = TileMask(n, 2 * hl, 2 * wl, dev), TileMask(n, 2 * hl, 2 * wl, dev)
+    ops.build_mask_tiles(None, None, n, hl, wl, _lib.FOOT_UP2X, 0, 0, 0, ts_up)
+    ops.build_mask_tiles(ts_up, None, n, 2 * hl, 2 * wl, _lib.FOOT_CONV, k, 1, k // 2, ts)
+    out = ops.new_nhwc(n, cout, 2 * hl, 2 * wl, dev, dt)
+    res = ops.new_nhwc(n, cout, 2 * hl, 2 * wl, dev)
+
+    def launch():
+        ops.upconv_masked(a, None, b, None, filt, k, k // 2, ts, out, res, _lib.ACT_RELU)
+
+    for _ in range(args.warmup):
+        launch()
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(args.iters):
+        launch()
+    e1.record()
+    torch.cuda.synchronize()
+    us = 1e3 * e0.elapsed_time(e1) / args.iters
+    a_out = int(ts.pixmask.sum().item())
+    flops = 2 * a_out * cin * cout * k * k
+    # algorithmic bytes: both half-resolution inputs once, emitted delta, reservoir read + write, filter, tile list
+    byts = 2 * n * hl * wl * (1 + cin * es) + a_out * cout * (es + 8) + cin * cout * k * k * es + ts.capacity * 4
+    print(json.dumps(dict(kernel="mie_upconv_masked", shape="up2x+%dx%d s1 %d->%d @%dx%d n=%d" % (k, k, cin, cout, 2 * hl, 2 * wl, n),
+                          dtype=args.dtype, active_tiles=int(ts.counts[0].item()), tiles=ts.capacity, us=round(us, 2),
+                          algorithmic_flops=flops, algorithmic_bytes=byts, tflops=round(flops / us / 1e6, 2),
+                          gbs=round(byts / us / 1e3, 1), iters=args.iters)))
 
 
 if __name__ == "__main__":

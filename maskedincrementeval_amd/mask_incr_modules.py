@@ -343,6 +343,18 @@ class _ConvIncrMixin(_IncrBuffers):
         return [out, ts]
 
 
+    def _upconv_forward(self, up: "nnUpsample2xIncr", x_incr: Masked, skip_incr: Masked, reservoir, act, slope,
+                        out_name="out_act") -> Masked:
+        """conv over up2x(x + skip) without forming the up-sampled delta (ops.upconv_masked)."""
+        k, s, p = self._geometry()
+        a, pa, b, pb, ts_up = up.plan(x_incr, skip_incr)
+        n, _, h, w = a.shape
+        ts = self._tile_set(out_name, n, 2 * h, 2 * w, a.device)
+        ops.build_mask_tiles(ts_up, None, n, 2 * h, 2 * w, _lib.FOOT_CONV, k, s, p, ts)
+        out = self._delta_buf(out_name, (n, self.out_channels, 2 * h, 2 * w), a.device, a.dtype)
+        ops.upconv_masked(a, pa, b, pb, self.conv2d_weights, k, p, ts, out, reservoir, act, slope)
+        return [out, ts]
+
     def _conv_tile_set(self, name, x, pix, x2, pix2, k, s, p) -> TileMask:
         """Tile set of the conv output for the (one or two) masked inputs, built for this step."""
         n, _, h, w = x.shape
@@ -444,6 +456,27 @@ class nnConvIncr(nn.Conv2d, _ConvIncrMixin):
             raise RuntimeError("fused conv+activation: call forward_refresh_reservoirs first")
         return self._incr_forward(x_incr, x2_incr, reservoir=res, act=kind, slope=slope,
                                   path=self.path, out_name="out_act", addend_incr=addend_incr, filt=filt)
+
+    def forward_fused_upsampled(self, up: "nnUpsample2xIncr", x_incr, skip_incr, activation: "nnReservedActivation"):
+        """bilinear x2 of (x + skip) + conv + activation increment; one kernel when the shape allows it,
+        else the up-sampling kernel followed by forward_fused."""
+        k, s, p = self._geometry()
+        x = x_incr[0]
+        # Measured on MI355X: on planes of up to a few thousand tiles the step is bound by launches and
+        # the one-kernel form wins (2 % of a 264x352 frame); on large planes the extra registers of its
+        # staging cost a resident workgroup per CU and the separate up-sampling kernel is cheaper
+        # (8x480x640 bf16: 858 us against 576 + 150 us for the last decoder).  With more than 4 staged
+        # chunks (256 fp32 channels) the per-chunk blend costs what the saved launch gains: two kernels.
+        tiles = x.shape[0] * ((2 * x.shape[2] + 7) // 8) * ((2 * x.shape[3] + 7) // 8)
+        chunks = x.shape[1] // ops.mfma_chunk(ops.delta_torch_dtype(x))
+        if self.use_kf or tiles > 2048 or chunks > 4 or not ops.upconv_takes(x.shape[1], self.out_channels, k, s, p,
+                                                                self.conv2d_weights, ops.delta_torch_dtype(x)):
+            return self.forward_fused(up(x_incr, skip_incr), activation)
+        kind, slope = activation_kind(activation.op)
+        res = activation.in_res.reservoir
+        if res is None:
+            raise RuntimeError("fused conv+activation: call forward_refresh_reservoirs first")
+        return self._upconv_forward(up, x_incr, skip_incr, res, kind, slope)
 
     def forward_refresh_reservoirs(self, x):
         # The reference refreshes self.kf here unconditionally (:193): a norm and a zero clone
@@ -675,6 +708,22 @@ class nnUpsample2xIncr(IncrementMaskModule):
         out = self._delta_buf("out", (n, c, 2 * h, 2 * w), a.device, a.dtype)
         ops.upsample2x_incr(a, pa, b, pb, ts, out)
         return [out, ts]
+
+    def plan(self, x_incr: Masked, skip_incr: Masked = None):
+        """Only the tile set of the up-sampled delta (for a consumer that up-samples on the fly):
+        returns (a, mask a, b, mask b, tile set at twice the resolution)."""
+        a, pa, _ = _unpack(x_incr)
+        b = pb = None
+        if skip_incr is not None:
+            b, pb, _ = _unpack(skip_incr)
+        n, c, h, w = a.shape
+        ts = self._tile_set("out", n, 2 * h, 2 * w, a.device)
+        if skip_incr is not None and (pa is None or pb is None):
+            m1 = m2 = None
+        else:
+            m1, m2 = pa, pb
+        ops.build_mask_tiles(m1, m2, n, h, w, _lib.FOOT_UP2X, 0, 0, 0, ts)
+        return a, pa, b, pb, ts
 
     def forward_refresh_reservoirs(self, x: DenseT, skip: DenseT = None) -> DenseT:
         self._reset_incr()

@@ -147,6 +147,11 @@ def delta_dtype(t: torch.Tensor) -> int:
         raise ValueError("deltas must be float32 or bfloat16, got %s" % t.dtype) from None
 
 
+def delta_torch_dtype(t: torch.Tensor):
+    """torch dtype a delta travels in: bf16 stays bf16, everything else becomes fp32 (as_nhwc)."""
+    return torch.bfloat16 if t.dtype == torch.bfloat16 else torch.float32
+
+
 def nhwc_ptr(t: Optional[torch.Tensor], name: str, c: Optional[int] = None, dtype=torch.float32):
     """Device pointer of an (N,C,H,W) tensor of `dtype` stored channels_last; None -> NULL."""
     if t is None:
@@ -343,6 +348,34 @@ def conv_masked(x, xmask, x2, x2mask, filt, k, stride, pad, out_ts: TileMask, ou
         filt.data_ptr(), mc_ptr, cin_total, k, stride, pad, cout, out_ts.ref,
         nhwc_ptr(out_delta, "out_delta", dtype=dt), nhwc_ptr(addend, "addend", cout, dtype=dt),
         nhwc_ptr(reservoir, "reservoir"), act, float(slope), path, delta_dtype(x), _stream(x)))
+    return out_delta
+
+
+def upconv_takes(c: int, cout: int, k: int, stride: int, pad: int, filt, dtype) -> bool:
+    """Whether upconv_masked has a kernel for the shape (else: upsample2x_incr + conv_masked)."""
+    return (isinstance(filt, ConvFilter) and k == 5 and stride == 1 and pad == 2 and c % mfma_chunk(dtype) == 0
+            and cout % 32 == 0 and filt.for_dtype(dtype)[1] is not None)
+
+
+def upconv_masked(a, amask, b, bmask, filt, k, pad, out_ts: TileMask, out_delta, reservoir=None,
+                  act=_lib.ACT_NONE, slope=0.0, addend=None):
+    """5x5 conv over up2x(a + b) in one kernel; a, b at half the resolution of out_ts (b may be None)."""
+    n, c, h, w = a.shape
+    dt = a.dtype
+    if b is not None and (b.shape != a.shape or b.dtype != dt):
+        raise ValueError("b %s %s does not match a %s %s" % (tuple(b.shape), b.dtype, tuple(a.shape), dt))
+    plain, mc_ptr = _filter_args(filt, k, dt)
+    cin_total, cout = plain.shape[0], plain.shape[3]
+    if tuple(out_delta.shape) != (n, cout, 2 * h, 2 * w) or out_ts.n != n:
+        raise ValueError("out_delta shape %s, expected %s" % (tuple(out_delta.shape), (n, cout, 2 * h, 2 * w)))
+    if reservoir is not None and reservoir.shape != out_delta.shape:
+        raise ValueError("reservoir shape %s != output %s" % (tuple(reservoir.shape), tuple(out_delta.shape)))
+    _ready(out_ts)
+    check(lib().mie_upconv_masked(
+        nhwc_ptr(a, "a", dtype=dt), pix_ptr(amask, n, h, w, "amask"), nhwc_ptr(b, "b", dtype=dt),
+        pix_ptr(bmask, n, h, w, "bmask"), c, h, w, plain.data_ptr(), mc_ptr, cin_total, k, pad, cout, out_ts.ref,
+        nhwc_ptr(out_delta, "out_delta", dtype=dt), nhwc_ptr(addend, "addend", cout, dtype=dt),
+        nhwc_ptr(reservoir, "reservoir"), act, float(slope), delta_dtype(a), _stream(a)))
     return out_delta
 
 

@@ -248,3 +248,45 @@ def test_pack_filter_layout_and_row_views():
     odd = cf.rows(4, 20)                 # not on an 8-row boundary: a packed copy of its own
     assert torch.equal(odd.mc, ops.pack_filter(f[4:20].contiguous()))
     assert ops.ConvFilter(f[:12].contiguous()).mc is None
+
+
+# 5x5 conv over up2x(a + b) in one kernel (the decoder layers): against interpolate + conv of the oracle,
+# for the three workgroup organisations (32 / 64 / 128 output channels per slab), ragged sizes whose
+# borders exercise the clamped bilinear taps and the conv's zero padding, fresh masks per step (stale
+# tiles), with and without the second input, plain and reservoir + activation epilogue.
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("c,cout,h,w", [(64, 32, 13, 17), (64, 64, 70, 90), (128, 128, 88, 80), (64, 96, 9, 40)])
+def test_upsampled_conv_in_one_kernel(c, cout, h, w, dtype):
+    bf = dtype == torch.bfloat16
+    tol = dict(rtol=2e-2, atol=2e-2) if bf else dict(rtol=RTOL, atol=1e-4)
+    q = (lambda t: t.to(torch.bfloat16).float()) if bf else (lambda t: t)
+    wt = q(he_normal_conv_weight(cout, c, 5, 9))
+    filt = _filt(wt)
+    assert ops.upconv_takes(c, cout, 5, 1, 2, filt, dtype)
+    ts_up, ts = TileMask(1, 2 * h, 2 * w, DEV), TileMask(1, 2 * h, 2 * w, DEV)
+    out = ops.new_nhwc(1, cout, 2 * h, 2 * w, DEV, dtype)
+    r0 = gaussian_delta(1, cout, 2 * h, 2 * w, 1.0, 1.0, seed=3)[0]
+    for step, (da, db, two, with_res) in enumerate([(0.2, 0.1, True, False), (0.03, 0.05, True, False),
+                                                    (0.1, 0.0, False, False), (0.3, 0.2, True, True)]):
+        a, ma = gaussian_delta(1, c, h, w, da, 0.5, seed=100 + step)
+        b, mb = gaussian_delta(1, c, h, w, db, 0.5, seed=200 + step)
+        a, b = q(a), q(b)
+        up = io.interp_incr(a + b if two else a)
+        if bf:
+            up = q(up)            # the staged tile is rounded to bf16, like the up-sampled delta would be
+        ref = io.conv_incr(up, wt, 1, 2)
+        dma, dmb = ma.to(DEV), mb.to(DEV)
+        ops.build_mask_tiles(dma, dmb if two else None, 1, h, w, _lib.FOOT_UP2X, 0, 0, 0, ts_up)
+        ops.build_mask_tiles(ts_up, None, 1, 2 * h, 2 * w, _lib.FOOT_CONV, 5, 1, 2, ts)
+        poison = lambda t, m: torch.where(m.bool().expand_as(t), t, torch.full_like(t, float("nan")))
+        res = _dev(r0).clone() if with_res else None
+        ops.upconv_masked(_dev(poison(a, ma)).to(dtype), dma, _dev(poison(b, mb)).to(dtype) if two else None,
+                          dmb if two else None, filt, 5, 2, ts, out, res,
+                          _lib.ACT_RELU if with_res else _lib.ACT_NONE)
+        torch.cuda.synchronize()
+        got = out.float().cpu()
+        assert torch.isfinite(got).all()
+        want = torch.relu(r0 + ref) - torch.relu(r0) if with_res else ref
+        assert torch.allclose(got, want, **tol), "step %d max|diff| = %.3e" % (step, (got - want).abs().max())
+        if with_res:
+            assert torch.allclose(res.cpu(), r0 + ref, rtol=RTOL, atol=2e-2 if bf else 1e-4)
