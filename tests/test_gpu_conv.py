@@ -290,3 +290,48 @@ def test_upsampled_conv_in_one_kernel(c, cout, h, w, dtype):
         assert torch.allclose(got, want, **tol), "step %d max|diff| = %.3e" % (step, (got - want).abs().max())
         if with_res:
             assert torch.allclose(res.cpu(), r0 + ref, rtol=RTOL, atol=2e-2 if bf else 1e-4)
+
+
+def _random_cases(count, seed):
+    rng = np.random.RandomState(seed)
+    cases = []
+    for i in range(count):
+        k = int(rng.choice([1, 3, 5, 7]))
+        s = int(rng.choice([1, 2]))
+        cin = int(rng.choice([3, 8, 16, 24, 32, 48, 64, 96, 128]))
+        cout = int(rng.choice([1, 2, 5, 16, 32, 40, 64, 96, 128, 160]))
+        h, w = int(rng.randint(k, 70)), int(rng.randint(k, 90))
+        n = int(rng.choice([1, 1, 2, 3]))
+        dens = float(rng.choice([0.0, 0.02, 0.1, 0.4, 1.0]))
+        pad = int(rng.choice([0, k // 2]))
+        cases.append((i, k, s, pad, cin, cout, n, h, w, dens))
+    return cases
+
+
+# A seeded sweep over shapes nobody picked by hand: kernel size, stride, padding (none / same), channel
+# counts on and off the matrix-core path, ragged planes down to the kernel size, batch, density from empty
+# to dense; two steps per case so that tiles go stale.  Auto path, fp32 and bf16.
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", _random_cases(36, seed=2024), ids=lambda c: "k%ds%dp%d_%dto%d_n%d_%dx%d_d%g" % c[1:])
+def test_seeded_random_shapes(case, dtype):
+    i, k, s, pad, cin, cout, n, h, w, dens = case
+    bf = dtype == torch.bfloat16
+    tol = dict(rtol=2e-2, atol=2e-2) if bf else dict(rtol=RTOL, atol=5e-5)
+    q = (lambda t: t.to(torch.bfloat16).float()) if bf else (lambda t: t)
+    wt = q(he_normal_conv_weight(cout, cin, k, 50 + i))
+    filt = _filt(wt)
+    ho, wo = mo.conv_out_size(h, w, k, s, pad)
+    ts = TileMask(n, ho, wo, DEV)
+    out = ops.new_nhwc(n, cout, ho, wo, DEV, dtype)
+    for step, dd in enumerate((dens, dens * 0.5)):
+        d, m = gaussian_delta(n, cin, h, w, dd, 0.5, seed=7000 + 10 * i + step)
+        d = q(d)
+        ref = io.conv_incr(d, wt, s, pad)
+        dm = m.to(DEV)
+        ops.build_mask_tiles(dm, None, n, h, w, _lib.FOOT_CONV, k, s, pad, ts)
+        ops.conv_masked(_dev(d).to(dtype), dm, None, None, filt, k, s, pad, ts, out)
+        torch.cuda.synchronize()
+        got = out.float().cpu()
+        assert torch.allclose(got, ref, **tol), "step %d max|diff| = %.3e" % (step, (got - ref).abs().max())
+        foot = torch.from_numpy(mo.footprint_conv(m[:, 0].numpy(), k, s, pad)).bool().unsqueeze(1)
+        assert torch.count_nonzero(got * (~foot)) == 0
