@@ -44,6 +44,8 @@ def parse_args():
     ap.add_argument("--layer-iters", type=int, default=20, help="timed launches per layer for the roofline table")
     ap.add_argument("--no-plan-first", dest="plan_first", action="store_false",
                     help="enqueue each mask build right before its consumer instead of all builds of a step first")
+    ap.add_argument("--upconv-all", action="store_true",
+                    help="take the one-kernel up-sampling conv for every decoder layer, whatever its size (for measurements)")
     ap.add_argument("--sync-masks", action="store_true", help="build tile sets on the compute stream (no planning stream)")
     ap.add_argument("--dtype", choices=["f32", "bf16"], default="f32",
                     help="element type of deltas and weights (reservoirs and accumulation stay fp32)")
@@ -190,6 +192,8 @@ def main():
     from maskedincrementeval_amd.synthetic import event_voxel_delta, seed_module_
 
     _lib.lib()   # fail loudly if the HIP library is missing
+    if args.upconv_all:
+        ops.upconv_max_tiles = ops.upconv_max_chunks = 1 << 30
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)

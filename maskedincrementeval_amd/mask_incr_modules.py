@@ -462,15 +462,17 @@ class nnConvIncr(nn.Conv2d, _ConvIncrMixin):
         else the up-sampling kernel followed by forward_fused."""
         k, s, p = self._geometry()
         x = x_incr[0]
-        # Measured on MI355X: on planes of up to a few thousand tiles the step is bound by launches and
-        # the one-kernel form wins (2 % of a 264x352 frame); on large planes the extra registers of its
-        # staging cost a resident workgroup per CU and the separate up-sampling kernel is cheaper
-        # (8x480x640 bf16: 858 us against 576 + 150 us for the last decoder).  With more than 4 staged
-        # chunks (256 fp32 channels) the per-chunk blend costs what the saved launch gains: two kernels.
+        # Measured on MI355X.  bf16: the one-kernel form wins at every size (264x352 frame -3 %, 8x480x640
+        # step -6 %).  fp32: on planes of up to a few thousand tiles the step is bound by launches and the
+        # one-kernel form wins (1.5 % of a 264x352 frame) unless the layer has more than 4 staged chunks
+        # (256 channels: the per-chunk blend then costs what the saved launch gains); on large planes the
+        # separate up-sampling kernel is cheaper (8x480x640 step +2 % with the one-kernel form).
+        dt = ops.delta_torch_dtype(x)
         tiles = x.shape[0] * ((2 * x.shape[2] + 7) // 8) * ((2 * x.shape[3] + 7) // 8)
-        chunks = x.shape[1] // ops.mfma_chunk(ops.delta_torch_dtype(x))
-        if self.use_kf or tiles > 2048 or chunks > 4 or not ops.upconv_takes(x.shape[1], self.out_channels, k, s, p,
-                                                                self.conv2d_weights, ops.delta_torch_dtype(x)):
+        chunks = x.shape[1] // ops.mfma_chunk(dt)
+        small = dt == torch.bfloat16 or (tiles <= ops.upconv_max_tiles and chunks <= ops.upconv_max_chunks)
+        if self.use_kf or not small or not ops.upconv_takes(x.shape[1], self.out_channels, k, s, p,
+                                                            self.conv2d_weights, dt):
             return self.forward_fused(up(x_incr, skip_incr), activation)
         kind, slope = activation_kind(activation.op)
         res = activation.in_res.reservoir

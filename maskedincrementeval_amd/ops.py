@@ -351,6 +351,11 @@ def conv_masked(x, xmask, x2, x2mask, filt, k, stride, pad, out_ts: TileMask, ou
     return out_delta
 
 
+# Up to which size fp32 decoder layers take the one-kernel form (see nnConvIncr.forward_fused_upsampled).
+upconv_max_tiles = 2048
+upconv_max_chunks = 4
+
+
 def upconv_takes(c: int, cout: int, k: int, stride: int, pad: int, filt, dtype) -> bool:
     """Whether upconv_masked has a kernel for the shape (else: upsample2x_incr + conv_masked)."""
     return (isinstance(filt, ConvFilter) and k == 5 and stride == 1 and pad == 2 and c % mfma_chunk(dtype) == 0
