@@ -164,11 +164,12 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   constexpr int LOS = CC;                                    // floats per source pixel in LDS
   constexpr int LO_F = UP ? 64 * LOS : 0;                    // fp32 sums of the 8x8 source block, CC channels
   static_assert(!UP || (S == 1 && K == 5 && !GATES), "the up-sampling variant is the 5x5 stride-1 conv");
-  constexpr int SMEM = ((STAGE_F > RED) ? STAGE_F : RED) + LO_F;
+  // the k-split reduction of the epilogue reuses the staging buffers and the source block
+  constexpr int SMEM = (STAGE_F + LO_F > RED) ? STAGE_F + LO_F : RED;
   static_assert(SMEM * 4 <= 65536, "LDS budget");
   __shared__ __attribute__((aligned(16))) float smem[SMEM];
   T* const sbuf = reinterpret_cast<T*>(smem);
-  float* const s_lo = smem + (SMEM - LO_F);
+  float* const s_lo = smem + STAGE_F;
 
   int n, y0, x0;
   const int tk = mie_pick_tile(a.ts, blockIdx.x, n, y0, x0);
