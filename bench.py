@@ -47,6 +47,9 @@ def parse_args():
     ap.add_argument("--upconv-all", action="store_true",
                     help="take the one-kernel up-sampling conv for every decoder layer, whatever its size (for measurements)")
     ap.add_argument("--sync-masks", action="store_true", help="build tile sets on the compute stream (no planning stream)")
+    ap.add_argument("--net", choices=["e2depth", "evflownet"], default="e2depth",
+                    help="e2depth: the headline network (5 bins); evflownet: EVFlowNet-incr, 4 bins, up-sampling decoders "
+                         "(the reference's optical-flow configuration: use --height 256 --width 256 --density 0.03)")
     ap.add_argument("--dtype", choices=["f32", "bf16"], default="f32",
                     help="element type of deltas and weights (reservoirs and accumulation stay fp32)")
     ap.add_argument("--kfence-tp", type=float, default=0.0,
@@ -204,23 +207,40 @@ def main():
     peak_mfma = PEAK_BF16_MFMA_TFLOPS if args.dtype == "bf16" else PEAK_FP32_MFMA_TFLOPS
     cl = lambda t: t.to(dev).to(dt).contiguous(memory_format=torch.channels_last)
 
-    model = seed_module_(E2VIDRecurrentIncr(async_masks=not args.sync_masks, plan_first=args.plan_first), seed=1).to(dev).eval()
-    x0 = torch.randn(NB, 5, H, W, generator=torch.Generator().manual_seed(2)) * 0.5
+    # the two networks differ in their call conventions only: adapters
+    if args.net == "evflownet":
+        from maskedincrementeval_amd.evflownet_incr import MultiResUNetRecurrentIncr
+        BINS, NET_NAME = 4, "EVFlowNet-incr"
+        make_net = lambda **kw: MultiResUNetRecurrentIncr(num_bins=4, **kw)
+        run_net = lambda m, x: m([x, None])
+        out_of = lambda r: r[-1][0]                      # the finest flow scale
+        refresh_net = lambda m, x: m.forward_refresh_reservoirs(x)
+        refresh_out = lambda r: r[-1]
+    else:
+        BINS, NET_NAME = 5, "E2Depth-incr"
+        make_net = E2VIDRecurrentIncr
+        run_net = lambda m, x: m([x, None], None)
+        out_of = lambda r: r[0][0]
+        refresh_net = lambda m, x: m.forward_refresh_reservoirs(x, None)
+        refresh_out = lambda r: r[0]
+
+    model = seed_module_(make_net(async_masks=not args.sync_masks, plan_first=args.plan_first), seed=1).to(dev).eval()
+    x0 = torch.randn(NB, BINS, H, W, generator=torch.Generator().manual_seed(2)) * 0.5
     n_inputs = 16
-    deltas_cpu = [event_voxel_delta(NB, 5, H, W, dens, seed=3000 + i)[0] for i in range(n_inputs)]
+    deltas_cpu = [event_voxel_delta(NB, BINS, H, W, dens, seed=3000 + i)[0] for i in range(n_inputs)]
     deltas = [cl(d) for d in deltas_cpu]
-    static_in = cl(torch.zeros(NB, 5, H, W))
+    static_in = cl(torch.zeros(NB, BINS, H, W))
 
     def step_eager(m, i):
         static_in.copy_(deltas[i % n_inputs])
-        return m([static_in, None], None)
+        return run_net(m, static_in)
 
     output_check = {}
 
     def timed_run(m, tag, check_against=None):
         history = []                                       # input index of every step the model takes
         with torch.no_grad():
-            m.forward_refresh_reservoirs(cl(x0), None)
+            refresh_net(m, cl(x0))
             for i in range(max(args.warmup, 3)):           # also allocates every persistent buffer
                 step_eager(m, i)
                 history.append(i)
@@ -236,7 +256,7 @@ def main():
                 torch.cuda.synchronize()
                 graph = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(graph):
-                    graph_out = m([static_in, None], None)[0][0]
+                    graph_out = out_of(run_net(m, static_in))
                 for i in range(3):
                     static_in.copy_(deltas[i % n_inputs])
                     graph.replay()
@@ -257,18 +277,18 @@ def main():
                 # instance of the network with eager launches and inline mask planning takes the same
                 # steps; the next frames of the two must then agree (same kernels over the same tiles).
                 ref = check_against()
-                ref.forward_refresh_reservoirs(cl(x0), None)
+                refresh_net(ref, cl(x0))
                 for i in history:
-                    ref([deltas[i % n_inputs], None], None)
+                    run_net(ref, deltas[i % n_inputs])
                 worst = 0.0
                 for i in range(4):
-                    want = ref([deltas[i % n_inputs], None], None)[0][0]
+                    want = out_of(run_net(ref, deltas[i % n_inputs]))
                     if graph is not None:
                         static_in.copy_(deltas[i % n_inputs])
                         graph.replay()
                         got = graph_out
                     else:
-                        got = step_eager(m, i)[0][0]
+                        got = out_of(step_eager(m, i))
                     worst = max(worst, (got.float() - want.float()).abs().max().item())
                 torch.cuda.synchronize()
                 output_check.update(max_abs_diff=worst, frames=4, steps_before=len(history),
@@ -282,12 +302,12 @@ def main():
         return dt / args.steps
 
     sec_per_step = timed_run(model, "incremental %.0f%%" % (100 * dens),
-                             check_against=lambda: seed_module_(E2VIDRecurrentIncr(), seed=1).to(dev).eval())
+                             check_against=lambda: seed_module_(make_net(), seed=1).to(dev).eval())
 
     # ---- per-layer roofline table: eager launches with HIP events, several repeats ------------
     with torch.no_grad():
         model.plan_first = False          # one walk per step: the probe times every wrapper call once
-        model.forward_refresh_reservoirs(cl(x0), None)
+        refresh_net(model, cl(x0))
         step_eager(model, 0)
         agg = None
         for it in range(args.layer_iters):
@@ -360,8 +380,8 @@ def main():
     model.plan_first = args.plan_first
     dense_sec = None
     if not args.no_dense:
-        dense_model = seed_module_(E2VIDRecurrentIncr(derive_input_mask=False, async_masks=not args.sync_masks,
-                                                       plan_first=args.plan_first), seed=1).to(dev).eval()
+        dense_model = seed_module_(make_net(derive_input_mask=False, async_masks=not args.sync_masks,
+                                            plan_first=args.plan_first), seed=1).to(dev).eval()
         dense_sec = timed_run(dense_model, "dense (all tiles active, same kernels)")
         del dense_model
 
@@ -369,16 +389,16 @@ def main():
     kfenced = None
     if args.kfence_tp > 0:
         from maskedincrementeval_amd.mask_incr_modules import set_kfence
-        kf_model = seed_module_(E2VIDRecurrentIncr(async_masks=not args.sync_masks), seed=1).to(dev).eval()
+        kf_model = seed_module_(make_net(async_masks=not args.sync_masks), seed=1).to(dev).eval()
         set_kfence(kf_model, args.kfence_tp)
         t = timed_run(kf_model, "quantised deltas (tp = %g)" % args.kfence_tp)
         # deviation of the accumulated prediction from the exact incremental net, same inputs
         with torch.no_grad():
             acc = []
             for m in (model, kf_model):
-                pred = m.forward_refresh_reservoirs(cl(x0), None)[0].clone()
+                pred = refresh_out(refresh_net(m, cl(x0))).clone()
                 for i in range(n_inputs):
-                    pred += step_eager(m, i)[0][0]
+                    pred += out_of(step_eager(m, i))
                 acc.append(pred)
             torch.cuda.synchronize()
             dev_abs = (acc[0] - acc[1]).abs().max().item()
@@ -404,9 +424,13 @@ def main():
     # ---- CPU baseline: the oracle (torch-CPU restatement of the reference path) -----------------
     cpu = None
     if args.cpu_steps > 0:
-        from oracle.e2depth_oracle import E2DepthOracle
         torch.set_num_threads(min(os.cpu_count() or 1, 16))
-        oracle = E2DepthOracle(model.state_dict())
+        if args.net == "evflownet":
+            from oracle.evflownet_oracle import EVFlowNetOracle
+            oracle = EVFlowNetOracle(model.state_dict(), decoder="upsample")
+        else:
+            from oracle.e2depth_oracle import E2DepthOracle
+            oracle = E2DepthOracle(model.state_dict())
         with torch.no_grad():
             oracle.refresh(x0)
             oracle.incr(deltas_cpu[0])
@@ -416,14 +440,14 @@ def main():
             cdt = (time.perf_counter() - t0) / args.cpu_steps
         cpu = dict(value=round(NB / cdt, 3), unit="frames/s", cores=torch.get_num_threads(), kind="port",
                    ms_per_step=round(1e3 * cdt, 2),
-                   sample="%d incremental steps of the same E2Depth-incr %dx%d workload (dense F.conv2d on the "
-                          "delta, as the reference executes it), torch-CPU fp32" % (args.cpu_steps, H, W))
+                   sample="%d incremental steps of the same %s %dx%d workload (dense F.conv2d on the "
+                          "delta, as the reference executes it), torch-CPU fp32" % (args.cpu_steps, NET_NAME, H, W))
         print("[bench] cpu baseline: %.1f ms/frame on %d threads" % (1e3 * cdt, cpu["cores"]), file=sys.stderr, flush=True)
 
     result = {
         # the headline metric's name; `value` is its frames/s part, the HBM GB/s part is in
         # "hbm_gbs_whole_frame" and per launch in "layers"
-        "metric": "incremental frames/s + HBM GB/s, E2Depth-incr %dx%d @%g%% delta density" % (H, W, 100 * dens),
+        "metric": "incremental frames/s + HBM GB/s, %s %dx%d @%g%% delta density" % (NET_NAME, H, W, 100 * dens),
         "value": round(NB / sec_per_step, 2),
         "unit": "frames/s",
         "n_gpus": 1,
@@ -435,8 +459,8 @@ def main():
         "vs_baseline": None,
         "dtype": args.dtype,
         "data": "synthetic",
-        "config": {"workload": "E2Depth-incr recurrent UNet, random init, %dx5x%dx%d event voxel deltas, %.0f%% "
-                               "active pixels, 1 dense refresh then incremental steps" % (NB, H, W, 100 * dens),
+        "config": {"workload": "%s recurrent UNet, random init, %dx%dx%dx%d event voxel deltas, %.0f%% "
+                               "active pixels, 1 dense refresh then incremental steps" % (NET_NAME, NB, BINS, H, W, 100 * dens),
                    "density": dens, "height": H, "width": W, "batch": NB, "graph": not args.no_graph,
                    "mask_planning": "inline" if args.sync_masks else ("second stream, builds first" if args.plan_first else "second stream")},
         "roofline": roofline,

@@ -52,6 +52,10 @@ class nnCatIncr(nn.Module, _IncrBuffers):
     buffers; used where a kernel takes one input pointer only)."""
 
     def forward(self, parts):
+        if ops._planner is not None:
+            # torch.cat / torch.maximum below run on the compute stream and would read pixel masks that the
+            # planning stream is still writing
+            raise NotImplementedError("nnCatIncr under asynchronous mask planning; use async_masks=False")
         deltas = [ops.as_nhwc(p[0]) for p in parts]
         n, _, h, w = deltas[0].shape
         pix = [ops.pixel_mask_of(_mask_of(p), d) for p, d in zip(parts, deltas)]
@@ -377,8 +381,12 @@ class MultiResUNetRecurrentIncr(nn.Module, _IncrBuffers):
     decoders, tanh flow heads); `decoder="transposed"` swaps in transposed-conv decoders."""
 
     def __init__(self, num_bins=2, base_num_channels=32, num_encoders=4, num_residual_blocks=2,
-                 decoder="upsample", fuse=True, mask_threshold=0.0, derive_input_mask=True):
+                 decoder="upsample", fuse=True, mask_threshold=0.0, derive_input_mask=True,
+                 async_masks=False, plan_first=False):
         super().__init__()
+        # async_masks: build the tile sets on a second stream; plan_first: walk the network twice per step,
+        # mask builds first (the masks of this network depend on the input mask only)
+        self.async_masks, self.plan_first = async_masks, plan_first
         self.final_activation = 'tanh'
         self.w_scale_pred = None
         self.num_encoders = num_encoders
@@ -448,6 +456,20 @@ class MultiResUNetRecurrentIncr(nn.Module, _IncrBuffers):
     def forward(self, x_incr):
         delta = ops.as_nhwc(x_incr[0])
         mask = _mask_of(x_incr)
+        if not self.async_masks:
+            return self._forward(delta, mask)
+        with ops.mask_planner(delta.device):
+            if mask is None and self.derive_input_mask:
+                n, _, h, w = delta.shape
+                mask = ops.mask_from_delta(delta, self.mask_threshold, self._pix_buf("input", n, h, w, delta.device))
+            if self.plan_first:
+                with ops.network_pass("plan"):
+                    self._forward(delta, mask)
+                with ops.network_pass("compute"):
+                    return self._forward(delta, mask)
+            return self._forward(delta, mask)
+
+    def _forward(self, delta, mask):
         if mask is None and self.derive_input_mask:
             n, _, h, w = delta.shape
             mask = ops.mask_from_delta(delta, self.mask_threshold, self._pix_buf("input", n, h, w, delta.device))

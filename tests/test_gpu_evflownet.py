@@ -4,6 +4,7 @@ import numpy as np
 import pytest
 import torch
 
+from maskedincrementeval_amd import ops
 from maskedincrementeval_amd.evflownet_incr import ConvGRUIncr, MultiResUNetRecurrentIncr
 from maskedincrementeval_amd.synthetic import MovingEdges, gaussian_delta, seed_module_
 from oracle import mask_oracle as mo
@@ -118,3 +119,48 @@ def test_evflownet_bf16_matches_fp32_oracle(decoder):
         acc_ref = [a + b for a, b in zip(acc_ref, ref)]
     for a, b in zip(acc, acc_ref):
         _close(a, b, "accumulated", rtol=2e-2, atol=2e-2)
+
+
+def test_evflownet_planning_stream_and_pass_reproduce_inline_planning(decoder="upsample"):
+    # tile sets built on the planning stream in a planning pass, replayed from a HIP graph, against inline
+    # planning with eager launches: same kernels over the same tiles, so every flow scale agrees bit for bit
+    h, w, steps = 64, 96, 7
+    a = seed_module_(MultiResUNetRecurrentIncr(num_bins=4, decoder=decoder, async_masks=True, plan_first=True),
+                     seed=51).to(DEV).eval()
+    s = seed_module_(MultiResUNetRecurrentIncr(num_bins=4, decoder=decoder), seed=51).to(DEV).eval()
+    x0 = torch.randn(1, 4, h, w, generator=torch.Generator().manual_seed(52)) * 0.5
+    deltas = [_cl(gaussian_delta(1, 4, h, w, 0.03 + 0.03 * (i % 3), 0.3, seed=5600 + i)[0]) for i in range(steps)]
+    static_in = _cl(torch.zeros(1, 4, h, w))
+    with torch.no_grad():
+        a.forward_refresh_reservoirs(_cl(x0))
+        s.forward_refresh_reservoirs(_cl(x0))
+        refs = [[p[0].clone() for p in s([d, None])] for d in deltas]
+        got, g, g_out = [], None, None
+        for i, d in enumerate(deltas):
+            static_in.copy_(d)
+            if i == 2:
+                torch.cuda.synchronize()
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    g_out = [p[0] for p in a([static_in, None])]
+            if g is not None:
+                g.replay()
+                got.append([t.clone() for t in g_out])
+            else:
+                got.append([p[0].clone() for p in a([static_in, None])])
+        torch.cuda.synchronize()
+    for i in range(steps):
+        for sc, (x, y) in enumerate(zip(got[i], refs[i])):
+            assert torch.equal(x, y), "step %d scale %d max|diff| = %.3e" % (i, sc, (x - y).abs().max().item())
+
+
+def test_concat_layers_refuse_the_planning_stream():
+    # the transposed-conv decoders concatenate with torch ops on the compute stream, which would read pixel
+    # masks the planning stream is still writing: refused, and the planner is unwound
+    h, w = 32, 48
+    m = seed_module_(MultiResUNetRecurrentIncr(num_bins=4, decoder="transposed", async_masks=True), seed=51).to(DEV).eval()
+    with torch.no_grad():
+        m.forward_refresh_reservoirs(_cl(torch.randn(1, 4, h, w, generator=torch.Generator().manual_seed(1))))
+        with pytest.raises(NotImplementedError, match="asynchronous mask planning"):
+            m([_cl(gaussian_delta(1, 4, h, w, 0.05, 0.3, seed=2)[0]), None])
+    assert ops._planner is None and ops._phase is None
