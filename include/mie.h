@@ -196,6 +196,35 @@ int mie_conv_masked(const void* x, const uint8_t* xmask, int c1,
                     float slope, int path, int dtype, void* stream);
 
 /*
+ * mie_conv_masked with a workspace.  On planes of very few tiles (a 16x16
+ * plane is 4 tiles) a conv launch has too few workgroups for the chip; given a
+ * workspace, the matrix-core path then splits the contraction of each
+ * (tile, 32-channel slab) over up to 8 workgroups, which write fp32 partial
+ * sums to the workspace, and a second kernel adds them in a fixed order and
+ * runs the epilogue (results are reproducible run to run, and differ from the
+ * unsplit launch by fp32 rounding of the regrouped sum only).
+ *   workspace : device memory, 16-byte aligned, or NULL (then exactly
+ *        mie_conv_masked); workspace_bytes its size.  A launch is split when
+ *        k = 3, tiles x cout/32 <= 128 (tiles = mie_tile_capacity of `out`), the
+ *        inputs are at least 4 staging chunks deep and the workspace holds at
+ *        least 2 planes of n*h*w*cout floats (8 MiB covers 8 planes of every
+ *        shape that qualifies); otherwise the workspace is not touched.
+ *        Its contents are scratch: undefined after the call, and calls that
+ *        share one workspace must be ordered (same stream).
+ * Has no counterpart in the reference, whose convs run as one launch of
+ * whatever size (ext/pointops/_C_ext/pointops/ext_conv.cu:74-76).
+ */
+int mie_conv_masked_ws(const void* x, const uint8_t* xmask, int c1,
+                       const void* x2, const uint8_t* x2mask, int c2,
+                       int h_in, int w_in, const float* filter,
+                       const void* filter_mc, int cin_total,
+                       int k, int stride, int pad, int cout,
+                       const mie_tileset* out, void* out_delta,
+                       const void* addend, float* reservoir, int act_kind,
+                       float slope, int path, int dtype, void* workspace,
+                       long long workspace_bytes, void* stream);
+
+/*
  * Dense refresh through the same kernels: for every active tile of `out`
  * (build it with in_mask = NULL so that every tile is active)
  *   y = conv2d(x (++ x2), filter, bias, stride, pad) (+ addend);

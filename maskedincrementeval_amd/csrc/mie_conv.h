@@ -21,6 +21,9 @@ struct ConvArgsT {
   // mie_convlstm_gates_incr.
   int hid;
   const T* g_cpd; const uint8_t* g_cpm; float* g_cpres; float* g_cres; T* g_dh; T* g_dc;
+  // Workspace of the matrix-core path for launches of very few tiles (SPLIT kernels): fp32 partial sums,
+  // one plane of n*h*w*cout floats per part.  NULL: such launches are not split.
+  float* ws; long long ws_floats; long long ws_plane;
   TileSetDev ts;
 };
 typedef ConvArgsT<float> ConvArgs;

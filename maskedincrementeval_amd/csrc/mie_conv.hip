@@ -266,7 +266,8 @@ int conv_impl(const char* who, const T* x, const uint8_t* xmask, int c1, const T
               const mie_tileset* out,
               T* out_delta, const T* addend, float* reservoir, int act_kind, float slope,
               int path, bool refresh, const float* bias, void* stream,
-              const GatesOperands<T>* gates = nullptr) {
+              const GatesOperands<T>* gates = nullptr, void* workspace = nullptr,
+              long long workspace_bytes = 0) {
   mie_clear_error();
   int rc = mie_check_tileset(out, who);
   if (rc != MIE_OK) return rc;
@@ -321,6 +322,7 @@ int conv_impl(const char* who, const T* x, const uint8_t* xmask, int c1, const T
   a.slope = slope; a.addend = addend; a.refresh = refresh ? 1 : 0; a.bias = bias;
   a.hid = 0; a.g_cpd = nullptr; a.g_cpm = nullptr; a.g_cpres = nullptr; a.g_cres = nullptr;
   a.g_dh = nullptr; a.g_dc = nullptr;
+  a.ws = nullptr; a.ws_floats = 0; a.ws_plane = 0;
   a.ts = mie_dev_tileset(out);
   const unsigned cap = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
   hipStream_t st = (hipStream_t)stream;
@@ -336,6 +338,11 @@ int conv_impl(const char* who, const T* x, const uint8_t* xmask, int c1, const T
     return mie_check_launch(who);
   }
   if (path == MIE_PATH_MFMA) {
+    MIE_REQUIRE(workspace_bytes >= 0 && (workspace != nullptr || workspace_bytes == 0) &&
+                    mie_aligned(workspace, 16),
+                MIE_ERR_INVALID_ARG, "%s: workspace must be 16-byte aligned with a size >= 0", who);
+    a.ws = (float*)workspace;
+    a.ws_floats = workspace_bytes / 4;
     MIE_REQUIRE(mie_launch_conv_mfma(a, k, stride, cap, st), MIE_ERR_UNSUPPORTED,
                 "%s: no MFMA kernel variant for k=%d stride=%d cout=%d", who, k, stride, cout);
     return mie_check_launch(who);
@@ -387,6 +394,7 @@ int tconv_impl(const char* who, const T* x, const uint8_t* xmask, int cin, int h
   a.slope = slope; a.addend = nullptr; a.refresh = refresh ? 1 : 0; a.bias = bias;
   a.hid = 0; a.g_cpd = nullptr; a.g_cpm = nullptr; a.g_cpres = nullptr; a.g_cres = nullptr;
   a.g_dh = nullptr; a.g_dc = nullptr;
+  a.ws = nullptr; a.ws_floats = 0; a.ws_plane = 0;
   a.ts = mie_dev_tileset(out);
   const unsigned cap = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
   hipLaunchKernelGGL(k_tconv_valu<T>, dim3(cap, mie_div_up(cout, 64)), dim3(256), 0,
@@ -443,6 +451,29 @@ extern "C" int mie_conv_masked(const void* x, const uint8_t* xmask, int c1, cons
   return conv_impl<T>(who, (const T*)x, xmask, c1, (const T*)x2, x2mask, c2, h_in, w_in, filter,
                       (const T*)filter_mc, cin_total, k, stride, pad, cout, out, (T*)out_delta,
                       (const T*)addend, reservoir, act_kind, slope, path, false, nullptr, stream);
+}
+
+extern "C" int mie_conv_masked_ws(const void* x, const uint8_t* xmask, int c1, const void* x2,
+                                  const uint8_t* x2mask, int c2, int h_in, int w_in,
+                                  const float* filter, const void* filter_mc, int cin_total, int k,
+                                  int stride, int pad, int cout, const mie_tileset* out,
+                                  void* out_delta, const void* addend, float* reservoir,
+                                  int act_kind, float slope, int path, int dtype, void* workspace,
+                                  long long workspace_bytes, void* stream) {
+  const char* who = "mie_conv_masked_ws";
+  MIE_CONV_DTYPE_OK(dtype, who);
+  if (dtype == MIE_DTYPE_BF16) {
+    typedef mie_bf16 T;
+    return conv_impl<T>(who, (const T*)x, xmask, c1, (const T*)x2, x2mask, c2, h_in, w_in, filter,
+                        (const T*)filter_mc, cin_total, k, stride, pad, cout, out, (T*)out_delta,
+                        (const T*)addend, reservoir, act_kind, slope, path, false, nullptr, stream, nullptr,
+                        workspace, workspace_bytes);
+  }
+  typedef float T;
+  return conv_impl<T>(who, (const T*)x, xmask, c1, (const T*)x2, x2mask, c2, h_in, w_in, filter,
+                      (const T*)filter_mc, cin_total, k, stride, pad, cout, out, (T*)out_delta,
+                      (const T*)addend, reservoir, act_kind, slope, path, false, nullptr, stream, nullptr,
+                      workspace, workspace_bytes);
 }
 
 extern "C" int mie_conv_refresh(const void* x, int c1, const void* x2, int c2, int h_in,
@@ -568,6 +599,7 @@ int upconv_entry(const char* who, const void* a_lo, const uint8_t* amask, const 
   a.slope = slope; a.addend = (const T*)addend; a.refresh = 0; a.bias = nullptr;
   a.hid = 0; a.g_cpd = nullptr; a.g_cpm = nullptr; a.g_cpres = nullptr; a.g_cres = nullptr;
   a.g_dh = nullptr; a.g_dc = nullptr;
+  a.ws = nullptr; a.ws_floats = 0; a.ws_plane = 0;
   a.ts = mie_dev_tileset(out);
   const unsigned cap = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
   MIE_REQUIRE(mie_launch_conv_up_mfma(a, cap, (hipStream_t)stream), MIE_ERR_UNSUPPORTED,

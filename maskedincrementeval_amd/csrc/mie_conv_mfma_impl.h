@@ -137,7 +137,13 @@ __device__ __forceinline__ float4 f32_to_slot(const float (&f)[8], mie_bf16) {
 // half resolution (x2 optional), and is never formed in memory: per chunk the 8x8 block of source
 // pixels a tile's 12x12 input window blends is summed into LDS (fp32), and the staged tile is expanded
 // from there.  5x5, stride 1, pad 2 only; a.h_in / a.w_in are the up-sampled size.
-template <typename T, int K, int S, int WN, int NB, bool HALF, bool GATES = false, bool UP = false>
+//
+// SPLIT: launches with very few tiles (a 16x16 plane is 4 of them) leave most CUs idle.  The staged
+// chunks of every (tile, slab) are then split over gridDim.z workgroups; each writes its partial sums,
+// fp32 and unactivated, into its own plane of the workspace (a.ws, laid out like the output), and
+// k_conv_split_finish adds the planes in a fixed order and runs the epilogue.  Only the 32-channel
+// slab kernels (WN = 1) have this form.
+template <typename T, int K, int S, int WN, int NB, bool HALF, bool GATES = false, bool UP = false, bool SPLIT = false>
 __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   constexpr int NBUF = stage_buffers(S, (int)sizeof(T));
   constexpr int EPS = 16 / (int)sizeof(T);                   // elements per 16-byte slot (4 / 8)
@@ -171,18 +177,36 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   T* const sbuf = reinterpret_cast<T*>(smem);
   float* const s_lo = smem + STAGE_F;
 
+  // Which (tile, slab, part) this workgroup computes.  SPLIT launches are bound by the filter reaching
+  // the L2s (a 3x3 512->512 filter is 9.4 MB for a few hundred KB of deltas), and each of the 8 XCDs has
+  // an L2 of its own: workgroups are handed to the XCDs round robin in launch order, so the launch
+  // order is permuted to put the workgroups that read one filter slice (one slab, one part, every
+  // tile) on one XCD -- each slice then crosses the fabric once instead of once per tile.
+  int bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
+  if constexpr (SPLIT) {
+    const int gx = gridDim.x, gy = gridDim.y, slices = gy * (int)gridDim.z;
+    if ((slices & 7) == 0) {
+      const int lin = bx + gx * (by + gy * bz);
+      const int xcd = lin & 7, j = lin >> 3;
+      const int q = j / gx;
+      const int sl = q * 8 + xcd;
+      bx = j - q * gx; bz = sl / gy; by = sl - bz * gy;
+    }
+  }
   int n, y0, x0;
-  const int tk = mie_pick_tile(a.ts, blockIdx.x, n, y0, x0);
+  const int tk = mie_pick_tile(a.ts, bx, n, y0, x0);
   if (tk == 0) return;
   const int tid = threadIdx.x;
   // wave index as a scalar: everything derived from it (k-split, channel slab) stays in SGPRs
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int l32 = lane & 31, half = lane >> 5;
   const int wn = wave % WN, wk = wave / WN;
-  const int co0 = blockIdx.y * CO_BLK;
+  const int co0 = by * CO_BLK;
   const int hout = a.ts.h, wout = a.ts.w;
   const int cout = a.cout;
 
+  static_assert(!SPLIT || (WN == 1 && !GATES && !UP), "the split form is the plain 32-channel slab kernel");
+  if (SPLIT && tk == 2) return;      // stale tiles are zeroed by k_conv_split_finish
   if (GATES && tk == 2) {  // stale tile: zero the hidden / cell deltas of this workgroup's hidden channels
     constexpr int HC = CO_BLK / 4;
     for (int idx = tid; idx < 64 * HC; idx += 256) {
@@ -228,7 +252,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
     }
     conv_epilogue_load<T, PER>(a, e_off, e_ok, e_r0, e_add);
   };
-  if (WK > 1 && !GATES && EARLY) epilogue_fetch();
+  if (WK > 1 && !GATES && EARLY && !SPLIT) epilogue_fetch();
 
   v16f acc[2][NB];
 #pragma unroll
@@ -432,20 +456,24 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   // All B loads below are unconditional: a conditional load would make the compiler's wait
   // counters conservative and collapse the prefetch distance.  After the last chunk the
   // "next chunk" pointer simply stays on the current one (a few redundant loads).
-  const T* ub_cur = chunk_b(0);
+  // SPLIT: part blockIdx.z of gridDim.z takes a contiguous range of the chunks (the host keeps
+  // gridDim.z <= nch, so no range is empty)
+  const int c_lo = SPLIT ? bz * nch / (int)gridDim.z : 0;
+  const int c_hi = SPLIT ? (bz + 1) * nch / (int)gridDim.z : nch;
+  const T* ub_cur = chunk_b(c_lo);
   const T* ub_next = ub_cur;
-  stage_load(0);
+  stage_load(c_lo);
 #pragma unroll
   for (int i = 0; i < (PD > 0 ? PD : 1); ++i) load_b(ub_cur, i, bring[i % RING]);
   stage_store(0);
   __syncthreads();
 
-  for (int c = 0; c < nch; ++c) {
-    const bool more = c + 1 < nch;
+  for (int c = c_lo; c < c_hi; ++c) {
+    const bool more = c + 1 < c_hi;
     const int cn = more ? c + 1 : c;      // after the last chunk: redundant re-load, never stored
     ub_next = chunk_b(cn);
     stage_load(cn);
-    const T* sin = sbuf + (c % NBUF) * STAGE;
+    const T* sin = sbuf + ((c - c_lo) % NBUF) * STAGE;
     // A operands are read one unit ahead as well (two register sets); the scheduling barriers
     // pin "issue the loads for later units, then multiply this unit" so that the compiler can
     // neither sink the prefetches next to their uses nor hoist them all to the top.
@@ -477,7 +505,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
       if (PD == 0) load_b(ub_next, 0, bring[0]);   // ring of one: reload right after use
     }
     if (NBUF == 1 && !UP) __syncthreads();   // every wave is done reading the only buffer (UP: stage_store syncs)
-    if (more) stage_store((c + 1) % NBUF);
+    if (more) stage_store((c - c_lo + 1) % NBUF);
     __syncthreads();
     ub_cur = ub_next;
   }
@@ -564,7 +592,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
     }
   } else {
     // the trailing barrier of the main loop has retired every read of the staging buffers
-    if (!EARLY) epilogue_fetch();
+    if (!EARLY && !SPLIT) epilogue_fetch();
     float* red = smem + wk * (64 * CO_BLK);
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb)
@@ -585,8 +613,75 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
       for (int k2 = 1; k2 < WK; ++k2) sum += smem[k2 * (64 * CO_BLK) + idx];
       v[i] = sum;
     }
-    conv_epilogue_store<T, PER>(a, e_off, e_co, e_ok, v, e_r0, e_add);
+    if constexpr (SPLIT) {
+      float* plane = a.ws + (long long)bz * a.ws_plane;
+#pragma unroll
+      for (int i = 0; i < PER; ++i) {
+        const int idx = tid + 256 * i;
+        const int p = idx / CO_BLK, col = idx - p * CO_BLK;
+        const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
+        if (oy < hout && ox < wout) plane[(((long long)n * hout + oy) * wout + ox) * a.cout + co0 + col] = v[i];
+      }
+    } else {
+      conv_epilogue_store<T, PER>(a, e_off, e_co, e_ok, v, e_r0, e_add);
+    }
   }
+}
+
+// Second half of a SPLIT launch: per active tile the `parts` partial planes are added in order and
+// the ordinary epilogue (addend, reservoir, activation) runs; stale tiles are zeroed.  One thread per
+// (pixel, channel), channels fastest.
+template <typename T>
+__global__ __launch_bounds__(256) void k_conv_split_finish(ConvArgsT<T> a, int parts) {
+  int n, y0, x0;
+  const int tk = mie_pick_tile(a.ts, blockIdx.x, n, y0, x0);
+  if (tk == 0) return;
+  const int hout = a.ts.h, wout = a.ts.w, cout = a.cout;
+  const int cb = (cout + (int)gridDim.y - 1) / (int)gridDim.y;      // channels of this block
+  const int c0 = (int)blockIdx.y * cb;
+  const int cn = (cout - c0 < cb) ? cout - c0 : cb;
+  for (int idx = threadIdx.x; idx < 64 * cn; idx += 256) {
+    const int p = idx / cn, co = c0 + (idx - p * cn);
+    const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
+    if (oy >= hout || ox >= wout) continue;
+    const long long off = (((long long)n * hout + oy) * wout + ox) * cout + co;
+    if (tk == 2) {
+      mie_st(a.out, off, 0.f);
+      continue;
+    }
+    float sum = a.ws[off];
+    for (int q = 1; q < parts; ++q) sum += a.ws[(long long)q * a.ws_plane + off];
+    conv_store(a, off, co, sum);
+  }
+}
+
+// A launch is split when it has at most 128 workgroups, at least 4 staged chunks and a workspace:
+// into the largest power of two of parts (up to 8) that keeps the launch at 256 workgroups or fewer (one
+// per CU: measured on MI355X, a second workgroup per CU costs more in per-workgroup set-up than it gains),
+// leaves every part a chunk, and fits the workspace.  Returns false when the launch is not split.
+template <typename T, int K, int S>
+bool launch_split(const ConvArgsT<T>& a0, unsigned cap, hipStream_t st) {
+  constexpr int CC = stage_channels(K, S, false) * (4 / (int)sizeof(T));
+  if (a0.ws == nullptr || a0.refresh || a0.cout % 32 != 0 || a0.c1 % CC != 0 || a0.c2 % CC != 0) return false;
+  const long long groups = (long long)cap * (a0.cout / 32);
+  const int nch = (a0.c1 + a0.c2) / CC;
+  if (groups > 128 || nch < 4) return false;
+  ConvArgsT<T> a = a0;
+  a.ws_plane = (long long)a.ts.n * a.ts.h * a.ts.w * a.cout;
+  static const int most = [] {      // MIE_CONV_SPLIT caps the number of parts (1: never split): a tuning knob, read once
+    const char* e = getenv("MIE_CONV_SPLIT");
+    return e ? atoi(e) : 8;
+  }();
+  int parts = 1;
+  while (2 * parts <= most && 2 * parts <= nch && groups * (2 * parts) <= 256 && (long long)(2 * parts) * a.ws_plane <= a.ws_floats)
+    parts *= 2;
+  if (parts < 2) return false;
+  hipLaunchKernelGGL((k_conv_mfma<T, K, S, 1, 1, false, false, false, true>), dim3(cap, a.cout / 32, parts), dim3(256), 0, st, a);
+  unsigned ny = (unsigned)((1024 + cap - 1) / cap);
+  if (ny > (unsigned)(a.cout / 4)) ny = (unsigned)(a.cout / 4);
+  if (ny < 1) ny = 1;
+  hipLaunchKernelGGL(k_conv_split_finish<T>, dim3(cap, ny), dim3(256), 0, st, a, parts);
+  return true;
 }
 
 // Output channels per workgroup (the slab 32*NB*WN) for a launch of `cap` tiles: the widest of
@@ -710,8 +805,8 @@ bool launch_any(const ConvArgsT<T>& a, int k, int s, unsigned cap, hipStream_t s
   switch (k * 10 + s) {
     case 11: return launch_ks<T, 1, 1>(a, cap, st);
     case 12: return launch_ks<T, 1, 2>(a, cap, st);
-    case 31: return launch_ks<T, 3, 1>(a, cap, st);
-    case 32: return launch_ks<T, 3, 2>(a, cap, st);
+    case 31: return launch_split<T, 3, 1>(a, cap, st) || launch_ks<T, 3, 1>(a, cap, st);
+    case 32: return launch_split<T, 3, 2>(a, cap, st) || launch_ks<T, 3, 2>(a, cap, st);
     case 51: return launch_ks<T, 5, 1>(a, cap, st);
     case 52: return launch_ks<T, 5, 2>(a, cap, st);
     case 71: return launch_ks<T, 7, 1>(a, cap, st);

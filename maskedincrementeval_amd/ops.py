@@ -325,9 +325,28 @@ def _filter_args(filt, k, dtype=torch.float32):
     return filt, (None if mc is None else mc.data_ptr())
 
 
+# Workspace of the matrix-core conv for planes of very few tiles (a 16x16 plane is 4 tiles, 64 workgroups
+# for 512 channels): the library then splits the contraction over up to 8 workgroups per (tile, slab) and
+# needs room for their partial sums.  A launch is split only up to 128 workgroups, i.e. up to 4096
+# tile-channels, so 8 planes of 4096 * 64 floats (8 MiB) cover every case.  One buffer per device: the
+# convs of a device are taken to run on one stream at a time; callers that run convs concurrently on
+# several streams pass buffers of their own (`workspace=`), or False for none.
+SPLIT_WORKSPACE_BYTES = 8 * 4096 * 64 * 4
+split_enabled = True
+_split_ws = {}
+
+
+def split_workspace(device):
+    ws = _split_ws.get(device)
+    if ws is None:
+        ws = _split_ws[device] = torch.empty(SPLIT_WORKSPACE_BYTES // 4, dtype=torch.float32, device=device)
+    return ws
+
+
 def conv_masked(x, xmask, x2, x2mask, filt, k, stride, pad, out_ts: TileMask, out_delta,
-                reservoir=None, act=_lib.ACT_NONE, slope=0.0, path=_lib.PATH_AUTO, addend=None):
-    """filt: ConvFilter, or a contiguous fp32 [Cin_total, K, K, Cout] tensor (VALU kernels only)."""
+                reservoir=None, act=_lib.ACT_NONE, slope=0.0, path=_lib.PATH_AUTO, addend=None, workspace=None):
+    """filt: ConvFilter, or a contiguous fp32 [Cin_total, K, K, Cout] tensor (VALU kernels only).
+    workspace: fp32 tensor for the split form of small launches (None: the device's shared one, False: none)."""
     n, c1, h, w = x.shape
     c2 = 0 if x2 is None else x2.shape[1]
     if x2 is not None and (x2.shape[0] != n or x2.shape[2:] != x.shape[2:]):
@@ -342,12 +361,22 @@ def conv_masked(x, xmask, x2, x2mask, filt, k, stride, pad, out_ts: TileMask, ou
     if addend is not None and addend.shape != out_delta.shape:
         raise ValueError("addend shape %s != output %s" % (tuple(addend.shape), tuple(out_delta.shape)))
     _ready(out_ts)
-    check(lib().mie_conv_masked(
+    if workspace is None:
+        # only launches the library would split get the buffer (k = 3, few tiles): see launch_split
+        small = k == 3 and mc_ptr is not None and out_ts.capacity * (cout // 32) <= 128
+        workspace = split_workspace(x.device) if (split_enabled and small) else False
+    if workspace is False:
+        ws_ptr, ws_bytes = None, 0
+    else:
+        if workspace.dtype != torch.float32 or not workspace.is_contiguous() or workspace.device != x.device:
+            raise ValueError("workspace must be a contiguous fp32 tensor on the device of x")
+        ws_ptr, ws_bytes = workspace.data_ptr(), workspace.numel() * 4
+    check(lib().mie_conv_masked_ws(
         nhwc_ptr(x, "x", dtype=dt), pix_ptr(xmask, n, h, w, "xmask"), c1,
         nhwc_ptr(x2, "x2", dtype=dt), pix_ptr(x2mask, n, h, w, "x2mask"), c2, h, w,
         filt.data_ptr(), mc_ptr, cin_total, k, stride, pad, cout, out_ts.ref,
         nhwc_ptr(out_delta, "out_delta", dtype=dt), nhwc_ptr(addend, "addend", cout, dtype=dt),
-        nhwc_ptr(reservoir, "reservoir"), act, float(slope), path, delta_dtype(x), _stream(x)))
+        nhwc_ptr(reservoir, "reservoir"), act, float(slope), path, delta_dtype(x), ws_ptr, ws_bytes, _stream(x)))
     return out_delta
 
 
