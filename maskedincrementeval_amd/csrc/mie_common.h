@@ -80,17 +80,16 @@ static inline TileSetDev mie_dev_tileset(const mie_tileset* ts) {
 //   returns 0: nothing to do (b beyond active + stale)
 //           1: active tile   2: stale tile (zero its delta)
 // (n, y0, x0) = batch index and top-left output pixel of the tile.
-__device__ __forceinline__ int mie_pick_tile(const TileSetDev& ts, int b,
-                                             int& n, int& y0, int& x0) {
+// The same with the counts and the list entry tiles[b] already loaded by the caller (`spec`; any value
+// if b is not an active position).
+__device__ __forceinline__ int mie_pick_tile_loaded(const TileSetDev& ts, int b, int spec, int n_active,
+                                                    int n_stale, int& n, int& y0, int& x0) {
   const int cap = ts.n * ts.tiles_y * ts.tiles_x;
-  // the list entry is fetched together with the counts (one memory round trip instead of two);
-  // whether it is valid is decided afterwards
-  const int spec = ts.tiles[(b >= 0 && b < cap) ? b : 0];
-  const int n_active = ts.counts[MIE_CNT_ACTIVE];
-  const int n_stale = ts.counts[MIE_CNT_STALE];
   if (n_active < 0 || n_stale < 0 || n_active > cap || n_stale > cap) return 0;   // corrupt counts
   int tile, kind;
-  if (b < n_active) {
+  if (b < 0) {
+    return 0;
+  } else if (b < n_active) {
     tile = spec;
     kind = 1;
   } else if (b < n_active + n_stale) {
@@ -107,6 +106,17 @@ __device__ __forceinline__ int mie_pick_tile(const TileSetDev& ts, int b,
   y0 = ty * MIE_TILE;
   x0 = tx * MIE_TILE;
   return kind;
+}
+
+__device__ __forceinline__ int mie_pick_tile(const TileSetDev& ts, int b,
+                                             int& n, int& y0, int& x0) {
+  const int cap = ts.n * ts.tiles_y * ts.tiles_x;
+  // the list entry is fetched together with the counts (one memory round trip instead of two);
+  // whether it is valid is decided afterwards
+  const int spec = ts.tiles[(b >= 0 && b < cap) ? b : 0];
+  const int n_active = ts.counts[MIE_CNT_ACTIVE];
+  const int n_stale = ts.counts[MIE_CNT_STALE];
+  return mie_pick_tile_loaded(ts, b, spec, n_active, n_stale, n, y0, x0);
 }
 
 __device__ __forceinline__ float mie_act(int kind, float slope, float v) {

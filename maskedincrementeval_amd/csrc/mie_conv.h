@@ -24,6 +24,8 @@ struct ConvArgsT {
   // Workspace of the matrix-core path for launches of very few tiles (SPLIT kernels): fp32 partial sums,
   // one plane of n*h*w*cout floats per part.  NULL: such launches are not split.
   float* ws; long long ws_floats; long long ws_plane;
+  // Matrix-core path: launch order permuted per XCD (number of slab groups, 0 = plain order); set by the launchers.
+  int xcd_fs;
   TileSetDev ts;
 };
 typedef ConvArgsT<float> ConvArgs;

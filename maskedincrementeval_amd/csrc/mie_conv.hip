@@ -305,6 +305,11 @@ int conv_impl(const char* who, const T* x, const uint8_t* xmask, int c1, const T
               "%s: addend must not alias out_delta", who);
   const int pmul = 32 / (int)sizeof(T);       // input channels per block of the matrix-core filter copy
   MIE_REQUIRE(mie_aligned(filter_mc, 16), MIE_ERR_INVALID_ARG, "%s: filter_mc must be 16-byte aligned", who);
+  MIE_REQUIRE(workspace_bytes >= 0 && (workspace != nullptr || workspace_bytes == 0) && mie_aligned(workspace, 16),
+              MIE_ERR_INVALID_ARG, "%s: workspace must be 16-byte aligned, with a size >= 0 (0 if NULL)", who);
+  MIE_REQUIRE(workspace == nullptr || (workspace != (void*)out_delta && workspace != (void*)reservoir &&
+                                       workspace != (const void*)x && workspace != (const void*)x2),
+              MIE_ERR_INVALID_ARG, "%s: workspace must not alias an operand", who);
   const bool mfma_ok = (filter_mc != nullptr) && (cin_total % pmul == 0) &&
                        mie_conv_mfma_takes(k, stride, dtype_of<T>(), c1, c2, cout);
   MIE_REQUIRE(path == MIE_PATH_AUTO || path == MIE_PATH_VALU || path == MIE_PATH_MFMA,
@@ -322,7 +327,7 @@ int conv_impl(const char* who, const T* x, const uint8_t* xmask, int c1, const T
   a.slope = slope; a.addend = addend; a.refresh = refresh ? 1 : 0; a.bias = bias;
   a.hid = 0; a.g_cpd = nullptr; a.g_cpm = nullptr; a.g_cpres = nullptr; a.g_cres = nullptr;
   a.g_dh = nullptr; a.g_dc = nullptr;
-  a.ws = nullptr; a.ws_floats = 0; a.ws_plane = 0;
+  a.ws = nullptr; a.ws_floats = 0; a.ws_plane = 0; a.xcd_fs = 0;
   a.ts = mie_dev_tileset(out);
   const unsigned cap = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
   hipStream_t st = (hipStream_t)stream;
@@ -338,9 +343,6 @@ int conv_impl(const char* who, const T* x, const uint8_t* xmask, int c1, const T
     return mie_check_launch(who);
   }
   if (path == MIE_PATH_MFMA) {
-    MIE_REQUIRE(workspace_bytes >= 0 && (workspace != nullptr || workspace_bytes == 0) &&
-                    mie_aligned(workspace, 16),
-                MIE_ERR_INVALID_ARG, "%s: workspace must be 16-byte aligned with a size >= 0", who);
     a.ws = (float*)workspace;
     a.ws_floats = workspace_bytes / 4;
     MIE_REQUIRE(mie_launch_conv_mfma(a, k, stride, cap, st), MIE_ERR_UNSUPPORTED,
@@ -394,7 +396,7 @@ int tconv_impl(const char* who, const T* x, const uint8_t* xmask, int cin, int h
   a.slope = slope; a.addend = nullptr; a.refresh = refresh ? 1 : 0; a.bias = bias;
   a.hid = 0; a.g_cpd = nullptr; a.g_cpm = nullptr; a.g_cpres = nullptr; a.g_cres = nullptr;
   a.g_dh = nullptr; a.g_dc = nullptr;
-  a.ws = nullptr; a.ws_floats = 0; a.ws_plane = 0;
+  a.ws = nullptr; a.ws_floats = 0; a.ws_plane = 0; a.xcd_fs = 0;
   a.ts = mie_dev_tileset(out);
   const unsigned cap = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
   hipLaunchKernelGGL(k_tconv_valu<T>, dim3(cap, mie_div_up(cout, 64)), dim3(256), 0,
@@ -599,7 +601,7 @@ int upconv_entry(const char* who, const void* a_lo, const uint8_t* amask, const 
   a.slope = slope; a.addend = (const T*)addend; a.refresh = 0; a.bias = nullptr;
   a.hid = 0; a.g_cpd = nullptr; a.g_cpm = nullptr; a.g_cpres = nullptr; a.g_cres = nullptr;
   a.g_dh = nullptr; a.g_dc = nullptr;
-  a.ws = nullptr; a.ws_floats = 0; a.ws_plane = 0;
+  a.ws = nullptr; a.ws_floats = 0; a.ws_plane = 0; a.xcd_fs = 0;
   a.ts = mie_dev_tileset(out);
   const unsigned cap = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
   MIE_REQUIRE(mie_launch_conv_up_mfma(a, cap, (hipStream_t)stream), MIE_ERR_UNSUPPORTED,

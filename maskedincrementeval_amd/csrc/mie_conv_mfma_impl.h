@@ -177,24 +177,53 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   T* const sbuf = reinterpret_cast<T*>(smem);
   float* const s_lo = smem + STAGE_F;
 
-  // Which (tile, slab, part) this workgroup computes.  SPLIT launches are bound by the filter reaching
-  // the L2s (a 3x3 512->512 filter is 9.4 MB for a few hundred KB of deltas), and each of the 8 XCDs has
-  // an L2 of its own: workgroups are handed to the XCDs round robin in launch order, so the launch
-  // order is permuted to put the workgroups that read one filter slice (one slab, one part, every
-  // tile) on one XCD -- each slice then crosses the fabric once instead of once per tile.
-  int bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
-  if constexpr (SPLIT) {
-    const int gx = gridDim.x, gy = gridDim.y, slices = gy * (int)gridDim.z;
-    if ((slices & 7) == 0) {
-      const int lin = bx + gx * (by + gy * bz);
-      const int xcd = lin & 7, j = lin >> 3;
-      const int q = j / gx;
-      const int sl = q * 8 + xcd;
-      bx = j - q * gx; bz = sl / gy; by = sl - bz * gy;
+  // (tile-list position, slab, part) of this workgroup.  Each of the 8 XCDs has an L2 of its own and the
+  // hardware hands workgroups to the XCDs round robin in launch order (x fastest); with a.xcd_fs > 0 the
+  // grid's x extent is a multiple of 8, so the XCD of a workgroup is blockIdx.x % 8, and the launch order
+  // is permuted.  The live (tile, slab) pairs are put in the order (slab group, tile, slab within the
+  // group) -- a.xcd_fs groups of slabs, tiles in list order, i.e. along the rows of the image -- and each
+  // XCD takes a contiguous eighth of it, in that order.  A slab of the filter then reaches 8 / xcd_fs
+  // L2s instead of all 8, an input tile about xcd_fs of them, once, for all slabs of the group at a
+  // time, and neighbouring tiles, which share their halo, meet in one L2 (measured on the 5x5 256->128
+  // conv at 66x88: 65 -> 31 MB fetched per launch).  Active and stale tiles are dealt out separately
+  // (a stale tile costs next to nothing); the shares depend on their numbers, read from the tile set
+  // (one more dependent load at the start of a workgroup: measured, it costs nothing even on launches
+  // of a few dozen workgroups), and idle positions of the capacity-sized grid fall off the end.
+  // (For the SPLIT launches the same idea, one filter slice per XCD, was measured: no gain.)
+  int bx = blockIdx.x, by = blockIdx.y;
+  const int bz = SPLIT ? (int)blockIdx.z : 0;
+  int n, y0, x0, tk;
+  if (!SPLIT && a.xcd_fs > 0) {
+    const int cap = a.ts.n * a.ts.tiles_y * a.ts.tiles_x;
+    const int n_act = a.ts.counts[MIE_CNT_ACTIVE], n_st = a.ts.counts[MIE_CNT_STALE];
+    if (n_act < 0 || n_st < 0 || n_act > cap || n_st > cap) return;
+    const int ns = (int)gridDim.y;
+    const int w_act = n_act * ns, w_st = n_st * ns;          // live workgroups
+    const int c_act = (w_act + 7) >> 3, c_st = (w_st + 7) >> 3;   // per XCD
+    const int xcd = bx & 7;
+    const int slot = by * ((int)gridDim.x >> 3) + (bx >> 3);      // launch order within the XCD
+    const int spg = ns / a.xcd_fs;                           // slabs per group
+    int v, tiles_of_kind;
+    const bool active = slot < c_act;
+    if (active) {
+      v = xcd * c_act + slot;
+      if (v >= w_act) return;
+      tiles_of_kind = n_act;
+    } else {
+      if (slot - c_act >= c_st) return;
+      v = xcd * c_st + (slot - c_act);
+      if (v >= w_st) return;
+      tiles_of_kind = n_st;
     }
+    const int per_group = tiles_of_kind * spg;
+    const int sg = v / per_group, r = v - sg * per_group;
+    const int t = r / spg;
+    by = sg * spg + (r - t * spg);
+    bx = active ? t : n_act + t;
+    tk = mie_pick_tile_loaded(a.ts, bx, active ? a.ts.tiles[t] : 0, n_act, n_st, n, y0, x0);
+  } else {
+    tk = mie_pick_tile(a.ts, bx, n, y0, x0);
   }
-  int n, y0, x0;
-  const int tk = mie_pick_tile(a.ts, bx, n, y0, x0);
   if (tk == 0) return;
   const int tid = threadIdx.x;
   // wave index as a scalar: everything derived from it (k-split, channel slab) stays in SGPRs
@@ -667,6 +696,7 @@ bool launch_split(const ConvArgsT<T>& a0, unsigned cap, hipStream_t st) {
   const int nch = (a0.c1 + a0.c2) / CC;
   if (groups > 128 || nch < 4) return false;
   ConvArgsT<T> a = a0;
+  a.xcd_fs = 0;
   a.ws_plane = (long long)a.ts.n * a.ts.h * a.ts.w * a.cout;
   static const int most = [] {      // MIE_CONV_SPLIT caps the number of parts (1: never split): a tuning knob, read once
     const char* e = getenv("MIE_CONV_SPLIT");
@@ -715,23 +745,53 @@ int pick_slab(int cout, unsigned cap) {
   return 0;
 }
 
+// XCD-aware launch order (see the kernel): chooses the number of slab groups a.xcd_fs in {1, 2, 4, 8}
+// (a divisor of the slab count) that minimises what the 8 L2s fetch in total -- the filter 8 / xcd_fs
+// times plus the input xcd_fs times -- and returns the grid's x extent: the tile capacity rounded up to a
+// multiple of 8, plus 16 (the shares of active and of stale work are rounded up separately).  The
+// environment variable MIE_CONV_XCD forces the number of groups (0: plain launch order, a.xcd_fs = 0) --
+// a tuning knob for measurements, read once.
+template <typename T>
+unsigned xcd_plan(ConvArgsT<T>& a, unsigned cap, int nslabs, int k, bool up = false) {
+  static const int forced = [] {
+    const char* e = getenv("MIE_CONV_XCD");
+    return e ? atoi(e) : -1;
+  }();
+  a.xcd_fs = 0;
+  if (forced == 0) return cap;
+  const double cin = (double)a.c1 + a.c2;
+  const double filt = cin * k * k * a.cout;
+  const double in = (double)a.ts.n * a.h_in * a.w_in * (up ? 0.5 * a.c1 : cin);
+  int best = 1;
+  double cost = 8 * filt + in;
+  for (int fs = 2; fs <= 8; fs *= 2) {
+    if (nslabs % fs != 0) break;
+    const double c = (8 / fs) * filt + fs * in;
+    if (c < cost) cost = c, best = fs;
+  }
+  if (forced > 0 && 8 % forced == 0 && nslabs % forced == 0) best = forced;
+  a.xcd_fs = best;
+  return ((cap + 7u) & ~7u) + 16u;
+}
+
 template <typename T, int K, int S, bool HALF>
-bool launch_depth(const ConvArgsT<T>& a, unsigned cap, hipStream_t st) {
+bool launch_depth(const ConvArgsT<T>& a0, unsigned cap, hipStream_t st) {
   constexpr int NQ = stage_channels(K, S, HALF) / 8;
+  ConvArgsT<T> a = a0;
   const int cout = a.cout;
   switch (pick_slab<K, S, HALF>(cout, cap)) {
     case 128:
-      hipLaunchKernelGGL((k_conv_mfma<T, K, S, 4, 1, HALF>), dim3(cap, cout / 128), dim3(256), 0, st, a);
+      hipLaunchKernelGGL((k_conv_mfma<T, K, S, 4, 1, HALF>), dim3(xcd_plan(a, cap, cout / 128, K), cout / 128), dim3(256), 0, st, a);
       return true;
     case 64:
       if constexpr (NQ >= 2) {
-        hipLaunchKernelGGL((k_conv_mfma<T, K, S, 2, 1, HALF>), dim3(cap, cout / 64), dim3(256), 0, st, a);
+        hipLaunchKernelGGL((k_conv_mfma<T, K, S, 2, 1, HALF>), dim3(xcd_plan(a, cap, cout / 64, K), cout / 64), dim3(256), 0, st, a);
         return true;
       }
       return false;
     case 32:
       if constexpr (NQ >= 4) {
-        hipLaunchKernelGGL((k_conv_mfma<T, K, S, 1, 1, HALF>), dim3(cap, cout / 32), dim3(256), 0, st, a);
+        hipLaunchKernelGGL((k_conv_mfma<T, K, S, 1, 1, HALF>), dim3(xcd_plan(a, cap, cout / 32, K), cout / 32), dim3(256), 0, st, a);
         return true;
       }
       return false;
@@ -742,19 +802,20 @@ bool launch_depth(const ConvArgsT<T>& a, unsigned cap, hipStream_t st) {
 
 // The 5x5 stride-1 conv over up2x(x + x2): full staging depth only.
 template <typename T>
-bool launch_up(const ConvArgsT<T>& a, unsigned cap, hipStream_t st) {
+bool launch_up(const ConvArgsT<T>& a0, unsigned cap, hipStream_t st) {
   constexpr int FULL = stage_channels(5, 1) * (4 / (int)sizeof(T));
-  if (a.c1 % FULL != 0) return false;
+  if (a0.c1 % FULL != 0) return false;
+  ConvArgsT<T> a = a0;
   const int cout = a.cout;
   switch (pick_slab<5, 1, false>(cout, cap)) {
     case 128:
-      hipLaunchKernelGGL((k_conv_mfma<T, 5, 1, 4, 1, false, false, true>), dim3(cap, cout / 128), dim3(256), 0, st, a);
+      hipLaunchKernelGGL((k_conv_mfma<T, 5, 1, 4, 1, false, false, true>), dim3(xcd_plan(a, cap, cout / 128, 5, true), cout / 128), dim3(256), 0, st, a);
       return true;
     case 64:
-      hipLaunchKernelGGL((k_conv_mfma<T, 5, 1, 2, 1, false, false, true>), dim3(cap, cout / 64), dim3(256), 0, st, a);
+      hipLaunchKernelGGL((k_conv_mfma<T, 5, 1, 2, 1, false, false, true>), dim3(xcd_plan(a, cap, cout / 64, 5, true), cout / 64), dim3(256), 0, st, a);
       return true;
     case 32:
-      hipLaunchKernelGGL((k_conv_mfma<T, 5, 1, 1, 1, false, false, true>), dim3(cap, cout / 32), dim3(256), 0, st, a);
+      hipLaunchKernelGGL((k_conv_mfma<T, 5, 1, 1, 1, false, false, true>), dim3(xcd_plan(a, cap, cout / 32, 5, true), cout / 32), dim3(256), 0, st, a);
       return true;
     default:
       return false;
@@ -763,19 +824,20 @@ bool launch_up(const ConvArgsT<T>& a, unsigned cap, hipStream_t st) {
 
 // The gates conv of a ConvLSTM: 3x3, stride 1, full staging depth, gate chain in the epilogue.
 template <typename T>
-bool launch_gates(const ConvArgsT<T>& a, unsigned cap, hipStream_t st) {
+bool launch_gates(const ConvArgsT<T>& a0, unsigned cap, hipStream_t st) {
   constexpr int FULL = stage_channels(3, 1) * (4 / (int)sizeof(T));
-  if (a.c1 % FULL != 0 || a.c2 % FULL != 0 || a.cout != 4 * a.hid || a.hid % 8 != 0) return false;
+  if (a0.c1 % FULL != 0 || a0.c2 % FULL != 0 || a0.cout != 4 * a0.hid || a0.hid % 8 != 0) return false;
+  ConvArgsT<T> a = a0;
   const int cout = a.cout;
   switch (pick_slab<3, 1, false>(cout, cap)) {
     case 128:
-      hipLaunchKernelGGL((k_conv_mfma<T, 3, 1, 4, 1, false, true>), dim3(cap, cout / 128), dim3(256), 0, st, a);
+      hipLaunchKernelGGL((k_conv_mfma<T, 3, 1, 4, 1, false, true>), dim3(xcd_plan(a, cap, cout / 128, 3), cout / 128), dim3(256), 0, st, a);
       return true;
     case 64:
-      hipLaunchKernelGGL((k_conv_mfma<T, 3, 1, 2, 1, false, true>), dim3(cap, cout / 64), dim3(256), 0, st, a);
+      hipLaunchKernelGGL((k_conv_mfma<T, 3, 1, 2, 1, false, true>), dim3(xcd_plan(a, cap, cout / 64, 3), cout / 64), dim3(256), 0, st, a);
       return true;
     case 32:
-      hipLaunchKernelGGL((k_conv_mfma<T, 3, 1, 1, 1, false, true>), dim3(cap, cout / 32), dim3(256), 0, st, a);
+      hipLaunchKernelGGL((k_conv_mfma<T, 3, 1, 1, 1, false, true>), dim3(xcd_plan(a, cap, cout / 32, 3), cout / 32), dim3(256), 0, st, a);
       return true;
     default:
       return false;

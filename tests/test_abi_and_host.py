@@ -100,6 +100,13 @@ def test_invalid_arguments_return_status_not_abort(mie_lib):
     # channels beyond the filter
     assert mie_lib.mie_conv_masked(p, None, 16, p, None, 16, 16, 16, p, None, 16, 3, 1, 1, 32,
                                    ctypes.byref(ts), p, None, None, 0, 0.0, 0, 0, None) == -1
+    # workspace of the split form: misaligned, sized without a pointer, aliasing the output
+    ws_call = lambda ws, nbytes: mie_lib.mie_conv_masked_ws(p, None, 16, None, None, 0, 16, 16, p + 2048, None, 16, 3, 1, 1, 32,
+                                                            ctypes.byref(ts), p + 1024, None, None, 0, 0.0, 0, 0, ws, nbytes, None)
+    assert ws_call(p + 512 + 4, 64) == -1 and "workspace" in err()
+    assert ws_call(None, 64) == -1
+    assert ws_call(p + 512, -1) == -1
+    assert ws_call(p + 1024, 64) == -1 and "alias" in err()
     # tile set with a NULL member / zero-sized geometry
     bad, keep2 = _fake_tileset(null="tiles")
     assert mie_lib.mie_act_incr(1, 0.0, p, p, p, 8, ctypes.byref(bad), None, 0, 0, None) == -1
