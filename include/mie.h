@@ -205,7 +205,7 @@ int mie_conv_masked(const void* x, const uint8_t* xmask, int c1,
  * unsplit launch by fp32 rounding of the regrouped sum only).
  *   workspace : device memory, 16-byte aligned, or NULL (then exactly
  *        mie_conv_masked); workspace_bytes its size.  A launch is split when
- *        k = 3, tiles x cout/32 <= 128 (tiles = mie_tile_capacity of `out`), the
+ *        k = 3 or 5, tiles x cout/32 <= 128 (tiles = mie_tile_capacity of `out`), the
  *        inputs are at least 4 staging chunks deep and the workspace holds at
  *        least 2 planes of n*h*w*cout floats (8 MiB covers 8 planes of every
  *        shape that qualifies); otherwise the workspace is not touched.

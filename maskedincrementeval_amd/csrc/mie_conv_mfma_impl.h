@@ -869,8 +869,8 @@ bool launch_any(const ConvArgsT<T>& a, int k, int s, unsigned cap, hipStream_t s
     case 12: return launch_ks<T, 1, 2>(a, cap, st);
     case 31: return launch_split<T, 3, 1>(a, cap, st) || launch_ks<T, 3, 1>(a, cap, st);
     case 32: return launch_split<T, 3, 2>(a, cap, st) || launch_ks<T, 3, 2>(a, cap, st);
-    case 51: return launch_ks<T, 5, 1>(a, cap, st);
-    case 52: return launch_ks<T, 5, 2>(a, cap, st);
+    case 51: return launch_split<T, 5, 1>(a, cap, st) || launch_ks<T, 5, 1>(a, cap, st);
+    case 52: return launch_split<T, 5, 2>(a, cap, st) || launch_ks<T, 5, 2>(a, cap, st);
     case 71: return launch_ks<T, 7, 1>(a, cap, st);
     case 72: return launch_ks<T, 7, 2>(a, cap, st);
     default: return false;

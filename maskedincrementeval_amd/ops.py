@@ -362,8 +362,8 @@ def conv_masked(x, xmask, x2, x2mask, filt, k, stride, pad, out_ts: TileMask, ou
         raise ValueError("addend shape %s != output %s" % (tuple(addend.shape), tuple(out_delta.shape)))
     _ready(out_ts)
     if workspace is None:
-        # only launches the library would split get the buffer (k = 3, few tiles): see launch_split
-        small = k == 3 and mc_ptr is not None and out_ts.capacity * (cout // 32) <= 128
+        # only launches the library would split get the buffer (k = 3 or 5, few tiles): see launch_split
+        small = k in (3, 5) and mc_ptr is not None and out_ts.capacity * (cout // 32) <= 128
         workspace = split_workspace(x.device) if (split_enabled and small) else False
     if workspace is False:
         ws_ptr, ws_bytes = None, 0

@@ -342,19 +342,20 @@ def test_seeded_random_shapes(case, dtype):
 # Three steps with fresh masks (stale tiles), the last two with reservoir + activation and an addend;
 # checked against the oracle and against the unsplit launch, and the workspace must have been written.
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("k", [3, 5])
 @pytest.mark.parametrize("c1,c2,cout,h,w,s", [(512, 0, 512, 16, 16, 1), (256, 0, 512, 32, 32, 2), (128, 0, 96, 13, 11, 1),
                                               (128, 64, 64, 20, 9, 1), (256, 128, 160, 8, 8, 1), (128, 0, 32, 31, 29, 2),
                                               (256, 0, 256, 32, 32, 1)])
-def test_small_planes_split_the_contraction(c1, c2, cout, h, w, s, dtype):
+def test_small_planes_split_the_contraction(c1, c2, cout, h, w, s, dtype, k):
     bf = dtype == torch.bfloat16
     if bf and (c1 % 64 or c2 % 64 or (c1 + c2) // 64 < 4):
         pytest.skip("fewer than 4 staged chunks of 64 bf16 channels: not split")
     tol = dict(rtol=2e-2, atol=2e-2) if bf else dict(rtol=RTOL, atol=5e-5)
     q = (lambda t: t.to(torch.bfloat16).float()) if bf else (lambda t: t)
     n, cin = 1, c1 + c2
-    wt = q(he_normal_conv_weight(cout, cin, 3, 21))
+    wt = q(he_normal_conv_weight(cout, cin, k, 21))
     filt = _filt(wt)
-    ho, wo = mo.conv_out_size(h, w, 3, s, 1)
+    ho, wo = mo.conv_out_size(h, w, k, s, k // 2)
     ts = TileMask(n, ho, wo, DEV)
     assert ts.capacity * (cout // 32) <= 128
     out, out_plain = ops.new_nhwc(n, cout, ho, wo, DEV, dtype), ops.new_nhwc(n, cout, ho, wo, DEV, dtype)
@@ -365,20 +366,20 @@ def test_small_planes_split_the_contraction(c1, c2, cout, h, w, s, dtype):
         d, m = gaussian_delta(n, cin, h, w, dens, 0.5, seed=300 + step)
         d = q(d)
         add = q(gaussian_delta(n, cout, ho, wo, 1.0, 0.3, seed=400 + step)[0]) if with_res else None
-        ref = io.conv_incr(d, wt, s, 1)
+        ref = io.conv_incr(d, wt, s, k // 2)
         dm = m.to(DEV)
-        ops.build_mask_tiles(dm, None, n, h, w, _lib.FOOT_CONV, 3, s, 1, ts)
+        ops.build_mask_tiles(dm, None, n, h, w, _lib.FOOT_CONV, k, s, k // 2, ts)
         dx = _dev(d).to(dtype)
         x1, x2 = (dx, None) if c2 == 0 else (ops.as_nhwc(dx[:, :c1].contiguous(memory_format=torch.channels_last)),
                                              ops.as_nhwc(dx[:, c1:].contiguous(memory_format=torch.channels_last)))
         dadd = None if add is None else _dev(add).to(dtype)
         for o, r, wsp in ((out, res, ws), (out_plain, res_plain, False)):
-            ops.conv_masked(x1, dm, x2, None if x2 is None else dm, filt, 3, s, 1, ts, o, r if with_res else None,
+            ops.conv_masked(x1, dm, x2, None if x2 is None else dm, filt, k, s, k // 2, ts, o, r if with_res else None,
                             _lib.ACT_RELU if with_res else _lib.ACT_NONE, 0.0, _lib.PATH_MFMA, dadd, workspace=wsp)
         torch.cuda.synchronize()
         got, plain = out.float().cpu(), out_plain.float().cpu()
         if with_res:
-            tiles = torch.from_numpy(mo.footprint_conv(m[:, 0].numpy(), 3, s, 1)).bool()
+            tiles = torch.from_numpy(mo.footprint_conv(m[:, 0].numpy(), k, s, k // 2)).bool()
             tiles = torch.nn.functional.max_pool2d(tiles.float().unsqueeze(1), 8, 8, ceil_mode=True)
             tiles = torch.nn.functional.interpolate(tiles, scale_factor=8)[:, :, :ho, :wo].bool()
             acc = torch.where(tiles, ref + add, torch.zeros_like(ref))      # the addend counts on whole active tiles
