@@ -35,6 +35,11 @@ def main():
     ap.add_argument("--iters", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--copy-mb", type=int, default=0, help="run a plain copy of this many MiB instead")
+    ap.add_argument("--op", choices=["conv", "act", "mul", "add", "up2x", "gates"], default="conv",
+                    help="conv (default), or one of the bandwidth-bound incremental ops on an n x cin x h x w delta: "
+                         "act = reservoir + ReLU increment, mul = product-rule multiply, add = skip sum, "
+                         "up2x = bilinear x2 of a sum of two deltas (h, w = output size), gates = ConvLSTM gate chain "
+                         "(cin = hidden channels)")
     ap.add_argument("--up2x", action="store_true",
                     help="the conv reads up2x(a + b) of two deltas at half of --h/--w (mie_upconv_masked; 5x5 stride 1)")
     args = ap.parse_args()
@@ -61,6 +66,8 @@ def main():
 
     n, cin, cout, k, s, h, w = args.n, args.cin, args.cout, args.k, args.stride, args.h, args.w
     p = k // 2
+    if args.op != "conv":
+        return pointwise(args, dev, e0, e1)
     if args.up2x:
         return up2x_conv(args, dev, e0, e1)
     ho, wo = ops.conv_out_size(h, w, k, s, p)
@@ -146,6 +153,81 @@ def up2x_conv(args, dev, e0, e1):
                           dtype=args.dtype, active_tiles=int(ts.counts[0].item()), tiles=ts.capacity, us=round(us, 2),
                           algorithmic_flops=flops, algorithmic_bytes=byts, tflops=round(flops / us / 1e6, 2),
                           gbs=round(byts / us / 1e3, 1), iters=args.iters)))
+
+
+def pointwise(args, dev, e0, e1):
+    """One bandwidth-bound incremental op.  Algorithmic bytes: every delta, mask byte and reservoir the op must
+    touch on the active pixels, once (A = active pixels, s = element size of the deltas, reservoirs fp32)."""
+    n, c, h, w = args.n, args.cin, args.h, args.w
+    dt = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+    es = 2 if args.dtype == "bf16" else 4
+    g = torch.Generator().manual_seed(0)
+    hi, wi = (h // 2, w // 2) if args.op == "up2x" else (h, w)
+
+    def delta(ch, seed):
+        t = torch.randn((n, ch, hi, wi), generator=g)
+        if args.density < 1.0:
+            m = torch.stack([torch.from_numpy(blob_mask(hi, wi, args.density, seed=seed + b)) for b in range(n)])
+            m = m.view(n, 1, hi, wi)
+            t = t * m.float()
+            mk = m.to(torch.uint8).to(dev)
+        else:
+            mk = None
+        return ops.as_nhwc(t.to(dev).to(dt).contiguous(memory_format=torch.channels_last)), mk
+
+    res = lambda ch: ops.as_nhwc(torch.randn((n, ch, h, w), generator=g).to(dev).contiguous(memory_format=torch.channels_last))
+    ts = TileMask(n, h, w, dev)
+    if args.op == "act":
+        d, m = delta(c, 0)
+        r, out = res(c), ops.new_nhwc(n, c, h, w, dev, dt)
+        ops.build_mask_tiles(m, None, n, h, w, _lib.FOOT_CONV, 1, 1, 0, ts)
+        launch = lambda: ops.act_incr(_lib.ACT_RELU, 0.0, d, r, out, ts)
+        per_px = c * (es + 8 + es) + 1                     # delta in, reservoir read + write, delta out, mask byte
+    elif args.op == "mul":
+        d1, m1 = delta(c, 0)
+        d2, m2 = delta(c, 100)
+        r1, r2, out = res(c), res(c), ops.new_nhwc(n, c, h, w, dev, dt)
+        ops.build_mask_tiles(m1, m2, n, h, w, _lib.FOOT_CONV, 1, 1, 0, ts)
+        launch = lambda: ops.mul_incr(d1, m1, r1, d2, m2, r2, out, ts)
+        per_px = c * (2 * es + 16 + es) + 2                # two deltas, two reservoirs read + write, delta out
+    elif args.op == "add":
+        a, ma = delta(c, 0)
+        b, mb = delta(c, 100)
+        out = ops.new_nhwc(n, c, h, w, dev, dt)
+        ops.build_mask_tiles(ma, mb, n, h, w, _lib.FOOT_CONV, 1, 1, 0, ts)
+        launch = lambda: ops.add_incr(a, ma, b, mb, out, ts)
+        per_px = c * 3 * es + 2
+    elif args.op == "up2x":
+        a, ma = delta(c, 0)
+        b, mb = delta(c, 100)
+        out = ops.new_nhwc(n, c, h, w, dev, dt)
+        ops.build_mask_tiles(ma, mb, n, hi, wi, _lib.FOOT_UP2X, 0, 0, 0, ts)
+        launch = lambda: ops.upsample2x_incr(a, ma, b, mb, ts, out)
+        per_px = c * es + (2 * c * es + 2) / 4.0           # delta out; both inputs at a quarter of the pixels
+    else:
+        gd, m = delta(4 * c, 0)
+        gr, cpr, cr = res(4 * c), res(c), res(c)
+        hd, cd = ops.new_nhwc(n, c, h, w, dev, dt), ops.new_nhwc(n, c, h, w, dev, dt)
+        ops.build_mask_tiles(m, None, n, h, w, _lib.FOOT_CONV, 1, 1, 0, ts)
+        launch = lambda: ops.convlstm_gates_incr(gd, gr, None, None, cpr, cr, hd, cd, ts)
+        # gate deltas, gate reservoirs read + write, cell reservoir read + write, cached previous cell, two deltas out
+        per_px = c * (4 * es + 32 + 8 + 4 + 2 * es) + 1
+    for _ in range(args.warmup):
+        launch()
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(args.iters):
+        launch()
+    e1.record()
+    torch.cuda.synchronize()
+    us = 1e3 * e0.elapsed_time(e1) / args.iters
+    active = int(ts.pixmask.sum().item())
+    byts = int(active * per_px) + ts.capacity * 4
+    print(json.dumps(dict(kernel="mie_%s_incr" % {"gates": "convlstm_gates", "up2x": "upsample2x"}.get(args.op, args.op),
+                          shape="%dx%dx%dx%d" % (n, c, h, w), dtype=args.dtype, density=args.density,
+                          active_pixels=active, active_tiles=int(ts.counts[0].item()), tiles=ts.capacity,
+                          us=round(us, 2), algorithmic_bytes=byts, gbs=round(byts / us / 1e3, 1),
+                          hbm_frac=round(byts / us / 1e3 / 8000.0, 3), iters=args.iters)))
 
 
 if __name__ == "__main__":
