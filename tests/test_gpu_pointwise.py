@@ -259,3 +259,22 @@ def test_maxpool_increment_and_masked_accumulate(k, s, p, n, c, h, w):
     out, _ = pool([_dev(d), None])
     assert torch.equal(out.cpu(), io.maxpool_incr(res_cpu, d, k, s, p))
     assert torch.equal(pool.mp_res.reservoir.cpu(), res_cpu.reservoir)
+
+
+@pytest.mark.parametrize("argv", [["--op", "act"], ["--op", "mul"], ["--op", "add"], ["--op", "up2x"], ["--op", "gates"],
+                                  ["--cin", "32", "--cout", "32", "--k", "3"],
+                                  ["--cin", "64", "--cout", "32", "--k", "5", "--up2x"], ["--copy-mb", "1"]])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_kernel_bench_modes_run_and_report(argv, dtype, monkeypatch, capsys):
+    # the single-kernel benchmark the rocprofv3 counter runs use: every mode launches and prints one JSON line
+    # with a positive duration and the algorithmic bytes of its op
+    import json
+    from maskedincrementeval_amd import kernel_bench
+    small = ["--h", "24", "--w", "40", "--n", "2", "--iters", "2", "--warmup", "1", "--density", "0.3", "--dtype", dtype]
+    if "--cin" not in argv:
+        small += ["--cin", "16"]
+    monkeypatch.setattr("sys.argv", ["kernel_bench"] + argv + small)
+    kernel_bench.main()
+    line = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+    assert line["us"] > 0
+    assert line.get("algorithmic_bytes", line.get("bytes_read", 0)) > 0
