@@ -694,7 +694,9 @@ bool launch_split(const ConvArgsT<T>& a0, unsigned cap, hipStream_t st) {
   if (a0.ws == nullptr || a0.refresh || a0.cout % 32 != 0 || a0.c1 % CC != 0 || a0.c2 % CC != 0) return false;
   const long long groups = (long long)cap * (a0.cout / 32);
   const int nch = (a0.c1 + a0.c2) / CC;
-  if (groups > 128 || nch < 4) return false;
+  static const int max_groups = [] { const char* e = getenv("MIE_CONV_SPLIT_GROUPS"); return e ? atoi(e) : 128; }();
+  static const int max_wgs = [] { const char* e = getenv("MIE_CONV_SPLIT_WGS"); return e ? atoi(e) : 256; }();
+  if (groups > max_groups || nch < 4) return false;
   ConvArgsT<T> a = a0;
   a.xcd_fs = 0;
   a.ws_plane = (long long)a.ts.n * a.ts.h * a.ts.w * a.cout;
@@ -703,7 +705,7 @@ bool launch_split(const ConvArgsT<T>& a0, unsigned cap, hipStream_t st) {
     return e ? atoi(e) : 8;
   }();
   int parts = 1;
-  while (2 * parts <= most && 2 * parts <= nch && groups * (2 * parts) <= 256 && (long long)(2 * parts) * a.ws_plane <= a.ws_floats)
+  while (2 * parts <= most && 2 * parts <= nch && groups * (2 * parts) <= max_wgs && (long long)(2 * parts) * a.ws_plane <= a.ws_floats)
     parts *= 2;
   if (parts < 2) return false;
   hipLaunchKernelGGL((k_conv_mfma<T, K, S, 1, 1, false, false, false, true>), dim3(cap, a.cout / 32, parts), dim3(256), 0, st, a);
