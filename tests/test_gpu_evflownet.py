@@ -91,6 +91,18 @@ def test_evflownet_config4_moving_edges_and_dense_identity():
         _close(a, b.cpu(), "refresh + increments vs dense", atol=5e-5)
 
 
+def test_evflownet_50_steps_of_accumulation():
+    # 50 moving-edge frames accumulated into the same reservoirs: parity per step and scale, and refresh + the 50
+    # increments == dense forward on the accumulated input; reduced frame (64x96: bottleneck planes of 4x6 pixels,
+    # every small-plane form of the conv runs)
+    model, acc, x = _run("upsample", 64, 96, steps=50, edges=True)
+    fresh = seed_module_(MultiResUNetRecurrentIncr(num_bins=4), seed=51).to(DEV).eval()
+    with torch.no_grad():
+        dense = fresh.forward_refresh_reservoirs(_cl(x))
+    for a, b in zip(acc, dense):
+        _close(a, b.cpu(), "refresh + 50 increments vs dense", atol=1e-4)
+
+
 @pytest.mark.parametrize("decoder", ["upsample", "transposed"])
 def test_evflownet_bf16_matches_fp32_oracle(decoder):
     # bf16 deltas and weights, fp32 reservoirs: every flow scale within rtol 2e-2 of its range (tanh output)

@@ -215,7 +215,7 @@ def _run_e2depth(h, w, steps, density, fuse, seed=31):
         x += d
         # input mask and head tile list: exact against the oracle definitions
         pm = mo.pixel_mask(d.numpy(), 0.0)
-        assert np.array_equal(pm, m[:, 0].numpy())
+        assert np.all(pm <= m[:, 0].numpy())     # (an event pixel whose five bins all drew 0 carries no delta)
         head_ts = model.unetrecurrent.head.conv2d._tile_set("out_act" if fuse else "out", 1, h, w, torch.device(DEV))
         assert np.array_equal(head_ts.active_tiles().cpu().numpy(), mo.tile_list(mo.footprint_conv(pm, 5, 1, 2)))
     _close(acc, acc_ref, "accumulated")
@@ -235,6 +235,18 @@ def test_e2depth_incr_full_size_matches_oracle_and_dense():
     with torch.no_grad():
         dense = fresh.forward_refresh_reservoirs(_cl(x), None)[0]
     _close(acc, dense.cpu(), "refresh + increments vs dense", atol=5e-5)
+
+
+def test_e2depth_incr_50_steps_of_accumulation():
+    # 50 successive delta accumulations into the same reservoirs (the reference drivers refresh every 20-100
+    # frames, run_e2depth_continuous_dataset.py:61): parity per step and of the accumulated prediction, and
+    # refresh + 50 increments == dense forward on x0 + the 50 deltas.  Reduced frame (72x104) so that the CPU
+    # oracle takes seconds; at this size the bottleneck planes are 9x13, i.e. the split form of the conv runs too.
+    model, acc, x = _run_e2depth(72, 104, steps=50, density=0.05, fuse=True)
+    fresh = seed_module_(E2VIDRecurrentIncr(), seed=31).to(DEV).eval()
+    with torch.no_grad():
+        dense = fresh.forward_refresh_reservoirs(_cl(x), None)[0]
+    _close(acc, dense.cpu(), "refresh + 50 increments vs dense", atol=1e-4)
 
 
 def test_e2depth_incr_empty_frames_between_active_ones():
