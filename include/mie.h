@@ -367,6 +367,28 @@ int mie_convlstm_gates_incr(const void* gates_delta, float* gates_res,
                             int dtype, void* stream);
 
 /*
+ * Fused incremental ConvGRU gate math for hidden size hid over the active
+ * tiles of ts, for a cell whose state is reset every step (the only way the
+ * reference runs it: new_state = candidate * update, incr_modules/
+ * evflownet_incr.py:58-69 with prev_state None).  gates_delta is
+ * [n,h,w,2*hid]: the delta of the update-gate conv in channels [0, hid) and of
+ * the candidate (out-gate) conv in [hid, 2*hid) -- ONE mie_conv_masked with
+ * the two filters stacked along the output channels, both convs read the same
+ * input.  State kept by the caller ([n,h,w,hid] fp32, updated in place):
+ *   update_res  pre-activation reservoir of the update gate (sigmoid)
+ *   cand_res    pre-activation reservoir of the candidate (tanh)
+ * Computes, per element, sigmoid / tanh increments on those reservoirs and the
+ * product rule of nnReservedMultiplication with its cached operands recomputed
+ * from them, and writes h_delta ([n,h,w,hid]).
+ * Replaces: the second gate conv, two activation increments and the
+ * incremental multiply of ConvGRUIncr.forward
+ * (incr_modules/evflownet_incr.py:58-69, mask_incr_modules.py:67-75).
+ */
+int mie_convgru_gates_incr(const void* gates_delta, float* update_res,
+                           float* cand_res, void* h_delta, int hid,
+                           const mie_tileset* ts, int dtype, void* stream);
+
+/*
  * The gates conv of a ConvLSTM and its gate chain in ONE kernel: the 3x3,
  * stride 1, pad 1 conv of mie_conv_masked (x ++ x2 -> 4*hid channels) whose
  * epilogue is mie_convlstm_gates_incr, so that the 4*hid-channel gate delta is

@@ -454,6 +454,42 @@ __global__ __launch_bounds__(256) void k_convlstm_gates(
   });
 }
 
+// ---- fused ConvGRU gates (state reset each step: new_state = candidate * update) ---------------
+
+// dg is [n,h,w,2*hid]: the update-gate conv delta in channels [0, hid), the candidate conv delta in [hid, 2*hid).
+// Per element: du, dc -> d(sigmoid), d(tanh) on the pre-activation reservoirs, then the product rule with the
+// cached operands recomputed from those reservoirs: dh = (ds + s0) * dt + t0 * ds.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void k_convgru_gates(TileSetDev ts, const T* __restrict__ dg,
+                                                       float* __restrict__ ures, float* __restrict__ cres,
+                                                       T* __restrict__ dh, int hid) {
+  int n, y0, x0;
+  const int tk = mie_pick_tile(ts, blockIdx.x, n, y0, x0);
+  if (tk == 0) return;
+  const int cv = hid / VEC;
+  for_tile_slots(ts, n, y0, x0, cv, [&](int, long long pixoff, int cq) {
+    const long long off = pixoff * hid + (long long)cq * VEC;
+    Vec<VEC> oh = Vec<VEC>::zero();
+    if (tk == 1 && ts.pixmask[pixoff]) {
+      const long long goff = pixoff * 2 * hid + (long long)cq * VEC;
+      Vec<VEC> du = Vec<VEC>::load(dg + goff), ru = Vec<VEC>::load(ures + off);
+      Vec<VEC> dc = Vec<VEC>::load(dg + goff + hid), rc = Vec<VEC>::load(cres + off);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        const float ru1 = ru[e] + du[e], rc1 = rc[e] + dc[e];
+        const float s0 = mie_sigm(ru[e]), ds = mie_sigm(ru1) - s0;
+        const float t0 = tanhf(rc[e]), dt = tanhf(rc1) - t0;
+        oh[e] = (ds + s0) * dt + t0 * ds;             // IncrPointwiseMultiply(candidate, update)
+        ru[e] = ru1;
+        rc[e] = rc1;
+      }
+      ru.store(ures + off);
+      rc.store(cres + off);
+    }
+    oh.store(dh + off);
+  });
+}
+
 int check_pointwise(const char* who, const mie_tileset* ts, int c) {
   int rc = mie_check_tileset(ts, who);
   if (rc != MIE_OK) return rc;
@@ -633,6 +669,26 @@ extern "C" int mie_convlstm_gates_incr(const void* gates_delta, float* gates_res
   const unsigned grid = (unsigned)mie_tile_capacity(ts->n, ts->h, ts->w);
   MIE_LAUNCH_POINTWISE(k_convlstm_gates, dtype, hid, grid, true, stream, d, (const T*)gates_delta, gates_res,
                        (const T*)cprev_delta, cprev_mask, cprev_res, cell_res, (T*)h_delta, (T*)c_delta, hid);
+  return mie_check_launch(who);
+}
+
+extern "C" int mie_convgru_gates_incr(const void* gates_delta, float* update_res, float* cand_res,
+                                      void* h_delta, int hid, const mie_tileset* ts, int dtype,
+                                      void* stream) {
+  mie_clear_error();
+  const char* who = "mie_convgru_gates_incr";
+  int rc = check_pointwise(who, ts, hid);
+  if (rc != MIE_OK) return rc;
+  MIE_DTYPE_OK(dtype, who);
+  MIE_REQUIRE(gates_delta && update_res && cand_res && h_delta, MIE_ERR_INVALID_ARG, "%s: NULL pointer", who);
+  MIE_REQUIRE(update_res != cand_res && gates_delta != h_delta, MIE_ERR_INVALID_ARG,
+              "%s: the two reservoirs, and gates_delta and h_delta, must be distinct", who);
+  MIE_PTR16(gates_delta, who, "gates_delta"); MIE_PTR16(update_res, who, "update_res");
+  MIE_PTR16(cand_res, who, "cand_res"); MIE_PTR16(h_delta, who, "h_delta");
+  const TileSetDev d = mie_dev_tileset(ts);
+  const unsigned grid = (unsigned)mie_tile_capacity(ts->n, ts->h, ts->w);
+  MIE_LAUNCH_POINTWISE(k_convgru_gates, dtype, hid, grid, true, stream, d, (const T*)gates_delta, update_res,
+                       cand_res, (T*)h_delta, hid);
   return mie_check_launch(who);
 }
 

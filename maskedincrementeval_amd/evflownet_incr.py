@@ -73,8 +73,9 @@ class nnCatIncr(nn.Module, _IncrBuffers):
 class ConvGRUIncr(nn.Module, _IncrBuffers):
     """Incremental ConvGRU (reference :18-96)."""
 
-    def __init__(self, input_size, hidden_size, kernel_size, activation=None, fuse=True):
+    def __init__(self, input_size, hidden_size, kernel_size, activation=None, fuse=True, stacked=True):
         super().__init__()
+        self.stacked = stacked          # with fuse: both gate convs as one conv + the gate-math kernel
         padding = kernel_size // 2
         self.input_size = input_size
         self.hidden_size = hidden_size
@@ -102,8 +103,40 @@ class ConvGRUIncr(nn.Module, _IncrBuffers):
             return conv.forward_fused(x_incr, act, h_incr)
         return act(conv(x_incr, h_incr))
 
+    # -- one conv for both gates + one gate-math kernel (state reset each step) -------------------
+    def _stacked_filter(self):
+        """ConvFilter of the update-gate and out-gate filters side by side: columns [0, hid) | [hid, 2*hid)."""
+        wu, wo = self.update_gate.weight, self.out_gate.weight
+        tag = (wu.data_ptr(), wu._version, wo.data_ptr(), wo._version, str(wu.device))
+        cached = self.__dict__.get("_stacked_filt_cache")
+        if cached is None or cached[0] != tag:
+            both = torch.cat((wu.detach(), wo.detach()), 0)                    # [2*hid, cin, k, k]
+            cached = (tag, ops.ConvFilter(both.permute(1, 2, 3, 0).contiguous().float()))
+            self.__dict__["_stacked_filt_cache"] = cached
+        return cached[1]
+
+    def _forward_stacked(self, input_incr):
+        """update and candidate deltas from ONE conv (the two gate convs read the same input), then sigmoid /
+        tanh increments and the incremental product in one kernel (mie_convgru_gates_incr).  The operands of the
+        product are recomputed from the pre-activation reservoirs, so self.mult's own reservoirs are not
+        maintained on this path (as with the fused ConvLSTM cell): switch paths only at a refresh."""
+        conv = self.update_gate
+        k, s, p = conv._geometry()
+        x, pix, _ = _unpack(input_incr)
+        n, _, h, w = x.shape
+        ts = conv._conv_tile_set("out_act", x, pix, None, None, k, s, p)
+        gates = self._delta_buf("gru_gates", (n, 2 * self.hidden_size, h, w), x.device, x.dtype)
+        ops.conv_masked(x, pix, None, None, self._stacked_filter(), k, s, p, ts, gates)
+        new_state = self._delta_buf("gru_state", (n, self.hidden_size, h, w), x.device, x.dtype)
+        ops.convgru_gates_incr(gates, self.sigmoid1.in_res.reservoir, self.tanh.in_res.reservoir, new_state, ts)
+        return [new_state, ts]
+
     def forward(self, input_incr, prev_state):
         """new_state = prev_state + mult(out - prev_state, update)  (reference :47-69)."""
+        if (self.fuse and self.stacked and prev_state is None and not self.update_gate.use_kf
+                and not self.out_gate.use_kf and self.sigmoid1.in_res.reservoir is not None):
+            new_state = self._forward_stacked(input_incr)
+            return new_state, new_state
         update = self._gate(self.update_gate, self.sigmoid1, input_incr, prev_state)
         out_inputs = self._gate(self.out_gate, self.tanh, input_incr, prev_state)
         if prev_state is None:

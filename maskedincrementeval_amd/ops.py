@@ -648,6 +648,23 @@ def convlstm_gates_incr(gates_delta, gates_res, cprev_delta, cprev_mask, cprev_r
     return h_delta, c_delta
 
 
+def convgru_gates_incr(gates_delta, update_res, cand_res, h_delta, ts: TileMask):
+    """ConvGRU gate math on the stacked [update | candidate] conv delta; reservoirs updated in place."""
+    n, c2, h, w = gates_delta.shape
+    hid = c2 // 2
+    if c2 != 2 * hid:
+        raise ValueError("gates tensor needs 2*hid channels, got %d" % c2)
+    for name, t in (("update_res", update_res), ("cand_res", cand_res), ("h_delta", h_delta)):
+        if tuple(t.shape) != (n, hid, h, w):
+            raise ValueError("%s shape %s, expected %s" % (name, tuple(t.shape), (n, hid, h, w)))
+    _ready(ts)
+    dt = gates_delta.dtype
+    check(lib().mie_convgru_gates_incr(nhwc_ptr(gates_delta, "gates_delta", dtype=dt), nhwc_ptr(update_res, "update_res"),
+                                       nhwc_ptr(cand_res, "cand_res"), nhwc_ptr(h_delta, "h_delta", dtype=dt), hid,
+                                       ts.ref, delta_dtype(gates_delta), _stream(gates_delta)))
+    return h_delta
+
+
 def gate_interleave_index(hid: int, device=None) -> torch.Tensor:
     """Column order of the fused gates conv: entry c' (= 32*b + 8*g + j) holds the column g*hid + 8*b + j of
     the [in | remember | out | cell] x hid order (gate g of hidden channel 8*b + j)."""

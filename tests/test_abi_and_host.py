@@ -107,6 +107,10 @@ def test_invalid_arguments_return_status_not_abort(mie_lib):
     assert ws_call(None, 64) == -1
     assert ws_call(p + 512, -1) == -1
     assert ws_call(p + 1024, 64) == -1 and "alias" in err()
+    # ConvGRU gate math: NULL pointer, aliased reservoirs, unknown dtype
+    assert mie_lib.mie_convgru_gates_incr(p, p + 256, None, p + 512, 8, ctypes.byref(ts), 0, None) == -1
+    assert mie_lib.mie_convgru_gates_incr(p, p + 256, p + 256, p + 512, 8, ctypes.byref(ts), 0, None) == -1
+    assert mie_lib.mie_convgru_gates_incr(p, p + 256, p + 1024, p + 512, 8, ctypes.byref(ts), 3, None) == -2
     # tile set with a NULL member / zero-sized geometry
     bad, keep2 = _fake_tileset(null="tiles")
     assert mie_lib.mie_act_incr(1, 0.0, p, p, p, 8, ctypes.byref(bad), None, 0, 0, None) == -1

@@ -24,10 +24,13 @@ def _close(got, ref, what="", rtol=1e-4, atol=1e-5):
     assert torch.allclose(got, ref, rtol=rtol, atol=atol), "%s max|diff| = %.3e" % (what, err)
 
 
-@pytest.mark.parametrize("fuse", [True, False])
-def test_convgru_module_matches_oracle(fuse):
-    n, c, h, w = 1, 32, 20, 28
-    cell = seed_module_(ConvGRUIncr(c, c, 3, fuse=fuse), 41).to(DEV).eval()
+@pytest.mark.parametrize("fuse,stacked", [(True, True), (True, False), (False, False)])
+@pytest.mark.parametrize("c", [32, 12])
+def test_convgru_module_matches_oracle(fuse, stacked, c):
+    # stacked: both gate convs as one conv of 2*hid channels + mie_convgru_gates_incr; c = 12 keeps the conv
+    # off the matrix-core path and the gate kernel on 4-channel vectors
+    n, h, w = 1, 20, 28
+    cell = seed_module_(ConvGRUIncr(c, c, 3, fuse=fuse, stacked=stacked), 41).to(DEV).eval()
     params = {"g." + k: v for k, v in cell.state_dict().items()}
     ref = _ConvGRU({k: v.cpu() for k, v in params.items()}, "g", c)
     x = torch.randn(n, c, h, w, generator=torch.Generator().manual_seed(42))
@@ -40,6 +43,10 @@ def test_convgru_module_matches_oracle(fuse):
             dh, _ = cell([_cl(d), m.to(DEV)], None)
         torch.cuda.synchronize()
         _close(dh[0], ref.incr(d), "step %d" % step)
+        # clean-delta invariant: nothing outside the 3x3 footprint of the input mask
+        foot = torch.from_numpy(mo.footprint_conv(m[:, 0].numpy(), 3, 1, 1)).bool().unsqueeze(1)
+        assert torch.count_nonzero(dh[0].cpu() * (~foot)) == 0
+    assert ("gru_gates" in str(list(cell._ib().keys()))) == (fuse and stacked)
 
 
 def _run(decoder, h, w, steps, edges, fuse=True):
