@@ -114,6 +114,11 @@ bool mie_launch_conv_gates_mfma(const ConvArgsT<mie_bf16>& a, unsigned cap, hipS
 bool mie_launch_conv_up_mfma(const ConvArgsT<float>& a, unsigned cap, hipStream_t st);
 bool mie_launch_conv_up_mfma(const ConvArgsT<mie_bf16>& a, unsigned cap, hipStream_t st);
 
+// Matrix-core conv for layers of at most 8 input channels (the network heads), one input, k in {3, 5}, Cout % 32
+// == 0 (mie_conv_fewcin.hip).  Returns false, launching nothing, for other shapes.
+bool mie_launch_conv_fewcin(const ConvArgsT<float>& a, int k, int s, unsigned cap, hipStream_t st);
+bool mie_launch_conv_fewcin(const ConvArgsT<mie_bf16>& a, int k, int s, unsigned cap, hipStream_t st);
+
 // One element of the ConvLSTM gate chain: pre-activation gate reservoirs r* and their deltas d*, cached
 // previous cell state cp and its delta dP, cached cell state c0.  Updates the reservoirs in place and
 // returns the deltas of the hidden and the cell state (the chain sigmoid1..3 / tanh1 -> m1 + m2 -> tanh2

@@ -318,6 +318,7 @@ int conv_impl(const char* who, const T* x, const uint8_t* xmask, int c1, const T
               "%s: MFMA path needs filter_mc (mie_pack_filter) and channel counts in whole staging chunks "
               "and output slabs for k=%d stride=%d (filter_mc=%p c1=%d c2=%d cout=%d)", who, k, stride,
               (const void*)filter_mc, c1, c2, cout);
+  const bool auto_path = path == MIE_PATH_AUTO;
   if (path == MIE_PATH_AUTO) path = mfma_ok ? MIE_PATH_MFMA : MIE_PATH_VALU;
 
   ConvArgsT<T> a;
@@ -349,6 +350,8 @@ int conv_impl(const char* who, const T* x, const uint8_t* xmask, int c1, const T
                 "%s: no MFMA kernel variant for k=%d stride=%d cout=%d", who, k, stride, cout);
     return mie_check_launch(who);
   }
+  // very few input channels (network heads): a matrix-core kernel of its own, unless the VALU path was asked for
+  if (auto_path && mie_launch_conv_fewcin(a, k, stride, cap, st)) return mie_check_launch(who);
   switch (k * 10 + stride) {
     case 11: launch_conv<T, 1, 1>(a, cap, st); break;
     case 12: launch_conv<T, 1, 2>(a, cap, st); break;

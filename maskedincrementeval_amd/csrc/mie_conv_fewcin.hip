@@ -1,0 +1,143 @@
+// Masked conv on the matrix cores for layers with very few input channels: the network heads (5 or 4
+// event bins -> 32 / 64 channels, 5x5 or 3x3).  Their contraction, K*K*Cin = 36 .. 125, is too short for
+// the staged implicit GEMM of mie_conv_mfma_impl.h (whole chunks of 32 channels, 16-byte channel slots),
+// and on the VALU path they run at a tenth of the vector peak.  Here the whole problem of a workgroup
+// fits LDS at once:
+//   * one 256-thread workgroup = one active 8x8 output tile x 32 output channels;
+//   * the input tile plus halo is staged in fp32, channels padded to 8 (pixel stride 9 floats), inactive
+//     pixels zero-filled without being read; bf16 deltas are widened while staging, so one kernel body
+//     (v_mfma_f32_32x32x2_f32) serves both element types -- products of bf16 values are exact in fp32;
+//   * the filter slab [tap][8 channels][32 columns] is staged from the plain fp32 filter, zero rows for
+//     the padding channels;
+//   * k = (tap, channel pair); wave w multiplies the 32-pixel block w & 1 (tile rows 0-3 / 4-7) for the
+//     taps of parity w >> 1, only the ceil(Cin / 2) channel pairs that exist; the two tap halves meet in
+//     LDS and are added in a fixed order; epilogue as everywhere (addend, reservoir, activation, refresh).
+// One input only (x2 unsupported), stride 1 or 2, K = 3 or 5, Cout % 32 == 0.
+#include "mie_conv.h"
+
+namespace {
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int FC_CH = 8;     // staged channels per pixel
+constexpr int FC_PS = 9;     // LDS floats per staged pixel (odd: the 32 pixels of a block fall on distinct banks)
+
+template <typename T, int K, int S>
+__global__ __launch_bounds__(256) void k_conv_fewcin(ConvArgsT<T> a) {
+  constexpr int IT = 7 * S + K;                  // input tile edge incl. halo
+  constexpr int NPIX = IT * IT;
+  constexpr int IN_F = NPIX * FC_PS;
+  constexpr int W_F = K * K * FC_CH * 32;
+  constexpr int RED_F = 2 * 64 * 16;             // accumulators of the two odd-tap waves
+  static_assert(RED_F <= IN_F + W_F, "the reduction reuses the staging area");
+  __shared__ float smem[IN_F + W_F];
+  float* const s_in = smem;
+  float* const s_w = smem + IN_F;
+
+  int n, y0, x0;
+  const int tk = mie_pick_tile(a.ts, blockIdx.x, n, y0, x0);
+  if (tk == 0) return;
+  const int tid = threadIdx.x;
+  const int hout = a.ts.h, wout = a.ts.w, cout = a.cout, cin = a.c1;
+  const int co0 = blockIdx.y * 32;
+  if (tk == 2) {   // stale tile: zero this workgroup's channel slab
+    for (int idx = tid; idx < 64 * 32; idx += 256) {
+      const int p = idx >> 5, col = idx & 31;
+      const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
+      if (oy < hout && ox < wout) mie_st(a.out, (((long long)n * hout + oy) * wout + ox) * cout + co0 + col, 0.f);
+    }
+    return;
+  }
+
+  // ---- stage the input tile (fp32, 8 channels per pixel) and the filter slab ---------------------
+  // Every global load of the thread is issued before the first LDS store (compile-time trip counts, fully
+  // unrolled): one memory round trip for the whole staging instead of one per loop iteration.
+  const int iy0 = y0 * S - a.pad, ix0 = x0 * S - a.pad;
+  constexpr int NIN = (NPIX * FC_CH + 255) / 256;
+  float vin[NIN], vw[K * K];
+  {
+    const int col = tid & 31, ch = (tid >> 5) & 7;           // filter: thread = (channel, column), one load per tap
+    const float* wp = a.filt + (long long)ch * (K * K) * cout + co0 + col;
+#pragma unroll
+    for (int tap = 0; tap < K * K; ++tap) vw[tap] = (ch < cin) ? wp[(long long)tap * cout] : 0.f;
+  }
+#pragma unroll
+  for (int i = 0; i < NIN; ++i) {
+    const int idx = tid + 256 * i;
+    const int pix = idx >> 3, ch = idx & 7;
+    const int iy = iy0 + pix / IT, ix = ix0 + pix % IT;
+    float v = 0.f;
+    if (pix < NPIX && ch < cin && iy >= 0 && iy < a.h_in && ix >= 0 && ix < a.w_in) {
+      const long long po = ((long long)n * a.h_in + iy) * a.w_in + ix;
+      if (a.xm == nullptr || a.xm[po]) v = mie_ld(a.x, po * cin + ch);
+    }
+    vin[i] = v;
+  }
+#pragma unroll
+  for (int tap = 0; tap < K * K; ++tap) s_w[tap * 256 + tid] = vw[tap];
+#pragma unroll
+  for (int i = 0; i < NIN; ++i) {
+    const int idx = tid + 256 * i;
+    if ((idx >> 3) < NPIX) s_in[(idx >> 3) * FC_PS + (idx & 7)] = vin[i];
+  }
+  __syncthreads();
+
+  // ---- contraction ---------------------------------------------------------------------------------
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int l32 = lane & 31, half = lane >> 5;
+  const int mb = wave & 1, th = wave >> 1;
+  const int prow = mb * 4 + (l32 >> 3), pcol = l32 & 7;
+  const float* pa = s_in + ((prow * S) * IT + pcol * S) * FC_PS + half;
+  const float* pb = s_w + half * 32 + l32;
+  const int npair = (cin + 1) >> 1;
+  v16f acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+  for (int tap = th; tap < K * K; tap += 2) {
+    const int dy = tap / K, dx = tap - dy * K;
+    const float* ta = pa + (dy * IT + dx) * FC_PS;
+    const float* tb = pb + tap * (FC_CH * 32);
+    for (int p = 0; p < npair; ++p)
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ta[2 * p], tb[2 * p * 32], acc, 0, 0, 0);
+  }
+  __syncthreads();                       // every wave is done with the staged operands
+  float* red = smem;
+  if (th == 1) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) red[(mb * 16 + r) * 64 + lane] = acc[r];
+  }
+  __syncthreads();
+  if (th == 1) return;
+
+  // ---- epilogue: lane = output column l32, 16 pixels of the block per lane ---------------------------
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int p = mb * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+    const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
+    if (oy < hout && ox < wout)
+      conv_store(a, (((long long)n * hout + oy) * wout + ox) * cout + co0 + l32, co0 + l32,
+                 acc[r] + red[(mb * 16 + r) * 64 + lane]);
+  }
+}
+
+template <typename T>
+bool launch_fewcin(const ConvArgsT<T>& a, int k, int s, unsigned cap, hipStream_t st) {
+  if (a.x2 != nullptr || a.c1 < 1 || a.c1 > FC_CH || a.cout % 32 != 0) return false;
+  const dim3 grid(cap, a.cout / 32), block(256);
+  switch (k * 10 + s) {
+    case 31: hipLaunchKernelGGL((k_conv_fewcin<T, 3, 1>), grid, block, 0, st, a); return true;
+    case 32: hipLaunchKernelGGL((k_conv_fewcin<T, 3, 2>), grid, block, 0, st, a); return true;
+    case 51: hipLaunchKernelGGL((k_conv_fewcin<T, 5, 1>), grid, block, 0, st, a); return true;
+    case 52: hipLaunchKernelGGL((k_conv_fewcin<T, 5, 2>), grid, block, 0, st, a); return true;
+    default: return false;
+  }
+}
+
+}  // namespace
+
+bool mie_launch_conv_fewcin(const ConvArgsT<float>& a, int k, int s, unsigned cap, hipStream_t st) {
+  return launch_fewcin(a, k, s, cap, st);
+}
+bool mie_launch_conv_fewcin(const ConvArgsT<mie_bf16>& a, int k, int s, unsigned cap, hipStream_t st) {
+  return launch_fewcin(a, k, s, cap, st);
+}
