@@ -394,3 +394,44 @@ def test_small_planes_split_the_contraction(c1, c2, cout, h, w, s, dtype, k):
     # the split form ran: its partial sums replaced the NaN fill of the first planes
     plane = n * ho * wo * cout
     assert torch.isfinite(ws[:plane]).any() and torch.isfinite(ws[plane:2 * plane]).any()
+
+
+# Layers of at most 8 input channels (the network heads) have a matrix-core kernel of their own on the
+# automatic path: against the oracle and against the VALU kernel, every channel count, both kernel sizes and
+# strides, ragged plane, two steps (stale tiles), plain and with reservoir + activation.
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("k,s", [(3, 1), (3, 2), (5, 1), (5, 2)])
+@pytest.mark.parametrize("cin,cout", [(1, 32), (2, 64), (4, 64), (5, 32), (7, 96), (8, 32)])
+def test_few_input_channels_matrix_core_kernel(cin, cout, k, s, dtype):
+    bf = dtype == torch.bfloat16
+    tol = dict(rtol=2e-2, atol=2e-2) if bf else dict(rtol=RTOL, atol=5e-5)
+    q = (lambda t: t.to(torch.bfloat16).float()) if bf else (lambda t: t)
+    n, h, w, p = 2, 29, 43, k // 2
+    wt = q(he_normal_conv_weight(cout, cin, k, 60 + cin))
+    filt = _filt(wt)
+    ho, wo = mo.conv_out_size(h, w, k, s, p)
+    ts = TileMask(n, ho, wo, DEV)
+    out, out_valu = ops.new_nhwc(n, cout, ho, wo, DEV, dtype), ops.new_nhwc(n, cout, ho, wo, DEV, dtype)
+    r0 = gaussian_delta(n, cout, ho, wo, 1.0, 1.0, seed=8)[0]
+    res, res_valu, res_ref = _dev(r0).clone(), _dev(r0).clone(), r0.clone()
+    for step, (dens, with_res) in enumerate([(0.2, False), (0.07, True)]):
+        d, m = gaussian_delta(n, cin, h, w, dens, 0.5, seed=900 + 10 * cin + step)
+        d = q(d)
+        ref = io.conv_incr(d, wt, s, p)
+        dm = m.to(DEV)
+        ops.build_mask_tiles(dm, None, n, h, w, _lib.FOOT_CONV, k, s, p, ts)
+        x = _dev(torch.where(m.bool().expand_as(d), d, torch.full_like(d, float("nan")))).to(dtype)   # inactive pixels are never read
+        for o, r, path in ((out, res, _lib.PATH_AUTO), (out_valu, res_valu, _lib.PATH_VALU)):
+            ops.conv_masked(x, dm, None, None, filt, k, s, p, ts, o, r if with_res else None,
+                            _lib.ACT_RELU if with_res else _lib.ACT_NONE, 0.0, path)
+        torch.cuda.synchronize()
+        got, valu = out.float().cpu(), out_valu.float().cpu()
+        want = torch.relu(res_ref + ref) - torch.relu(res_ref) if with_res else ref
+        if with_res:
+            res_ref = res_ref + ref
+        assert torch.isfinite(got).all()
+        assert torch.allclose(got, want, **tol), "step %d max|diff| = %.3e" % (step, (got - want).abs().max())
+        assert torch.allclose(got, valu, **tol), "step %d vs VALU %.3e" % (step, (got - valu).abs().max())
+        foot = torch.from_numpy(mo.footprint_conv(m[:, 0].numpy(), k, s, p)).bool().unsqueeze(1)
+        assert torch.count_nonzero(got * (~foot)) == 0
+    assert torch.allclose(res.cpu(), res_ref, rtol=RTOL, atol=2e-2 if bf else 1e-4)
