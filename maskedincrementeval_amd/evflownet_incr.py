@@ -364,8 +364,28 @@ class UpsampleConvLayerIncr(nn.Module):
     def forward_refresh_reservoirs(self, parts):
         for m in list(self.up) + [self.cat, self._lead]:
             m._reset_incr()
-        x = torch.cat([F.interpolate(p, scale_factor=2, mode="bilinear", align_corners=False) for p in parts], 1)
-        if self.fuse and self.activation is not None and self.norm not in ["BN", "IN"]:
+        ups = [F.interpolate(p, scale_factor=2, mode="bilinear", align_corners=False) for p in parts]
+        fused = self.fuse and self.activation is not None and self.norm not in ["BN", "IN"]
+        if fused and len(ups) in (2, 3) and not self.conv2d.use_kf:
+            # as in forward: the two wide parts side by side through the two-pointer conv (matrix-core shapes
+            # stay on the matrix cores instead of a VALU conv over the odd channel count of the concat), the
+            # narrow leading part (the 2-channel flow) as a conv of its own whose result rides in as the addend
+            filt = self.conv2d.conv2d_weights
+            lead_c, addend = 0, None
+            if len(ups) == 3:
+                lead_c = ups[0].shape[1]
+                k, s, p = self.conv2d._geometry()
+                lead = ops.as_nhwc(ups[0])
+                n, _, h, w = lead.shape
+                ho, wo = ops.conv_out_size(h, w, k, s, p)
+                ts = self.conv2d._dense_tile_set(n, ho, wo, lead.device)
+                addend = self._lead._dense_buf("lead_refresh", (n, self.conv2d.out_channels, ho, wo), lead.device, lead.dtype)
+                ops.conv_refresh(lead, None, filt.rows(0, lead_c), None, k, s, p, ts, addend)
+            return self.conv2d._refresh_forward(ups[-2], ups[-1], self.activation, path=self.conv2d.path, addend=addend,
+                                                filt=filt.rows(lead_c, filt.shape[0]),
+                                                bias=None if self.conv2d.bias is None else self.conv2d.bias.detach())
+        x = torch.cat(ups, 1)
+        if fused:
             return self.conv2d.forward_refresh_fused(x, self.activation)
         out = self.conv2d.forward_refresh_reservoirs(x)
         if self.norm in ["BN", "IN"]:
