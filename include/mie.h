@@ -455,8 +455,12 @@ int mie_linear_incr(const void* in_delta, int n, int f_in, const float* weight_t
  * is never written.  a (mask amask) and the optional b (mask bmask) are
  * [n,h_in,w_in,c] deltas at HALF the output resolution; `out` is the conv's tile
  * set at (2*h_in, 2*w_in), built from the up-sampled mask (MIE_FOOT_UP2X, then
- * MIE_FOOT_CONV).  Matrix-core path only: filter_mc is required, c must be a
- * multiple of the staging chunk (32 fp32 / 64 bf16 channels) and cout of 32;
+ * MIE_FOOT_CONV).  Matrix-core path only, two forms:
+ *   - filter_mc given, c a multiple of the staging chunk (32 fp32 / 64 bf16
+ *     channels), cout of 32, k = 5, pad = 2;
+ *   - a single input (b = NULL) of c <= 8 channels, k = 3 or 5, pad = k/2, cout
+ *     a multiple of 32 (filter_mc unused): the 2-channel flow estimate in front
+ *     of an EVFlowNet-incr decoder (incr_modules/evflownet_incr.py:463-470);
  * otherwise MIE_ERR_UNSUPPORTED (use mie_upsample2x_incr + mie_conv_masked).
  * Epilogue (addend, reservoir, activation) as in mie_conv_masked.
  * Replaces: interpolate_from_module + nnConvIncr.forward of

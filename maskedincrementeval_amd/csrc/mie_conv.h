@@ -114,10 +114,25 @@ bool mie_launch_conv_gates_mfma(const ConvArgsT<mie_bf16>& a, unsigned cap, hipS
 bool mie_launch_conv_up_mfma(const ConvArgsT<float>& a, unsigned cap, hipStream_t st);
 bool mie_launch_conv_up_mfma(const ConvArgsT<mie_bf16>& a, unsigned cap, hipStream_t st);
 
+// Source rows / columns and weights of output index o of a bilinear x2 up-sampling (align_corners =
+// False): src = max(0, o/2 - 0.25), upper index clamped to the last row.
+static __device__ __forceinline__ void conv_up2x_coef(int o, int in_size, int& i0, int& i1, float& l0, float& l1) {
+  const int j = o >> 1;
+  if (o & 1) {
+    i0 = j; i1 = (j + 1 < in_size) ? j + 1 : j; l0 = 0.75f; l1 = 0.25f;
+  } else if (j == 0) {
+    i0 = 0; i1 = (1 < in_size) ? 1 : 0; l0 = 1.f; l1 = 0.f;
+  } else {
+    i0 = j - 1; i1 = j; l0 = 0.25f; l1 = 0.75f;
+  }
+}
 // Matrix-core conv for layers of at most 8 input channels (the network heads), one input, k in {3, 5}, Cout % 32
 // == 0 (mie_conv_fewcin.hip).  Returns false, launching nothing, for other shapes.
 bool mie_launch_conv_fewcin(const ConvArgsT<float>& a, int k, int s, unsigned cap, hipStream_t st);
 bool mie_launch_conv_fewcin(const ConvArgsT<mie_bf16>& a, int k, int s, unsigned cap, hipStream_t st);
+// The same over up2x(a.x): a.x / a.xm at half resolution, a.h_in / a.w_in the up-sampled size, stride 1.
+bool mie_launch_conv_fewcin_up(const ConvArgsT<float>& a, int k, unsigned cap, hipStream_t st);
+bool mie_launch_conv_fewcin_up(const ConvArgsT<mie_bf16>& a, int k, unsigned cap, hipStream_t st);
 
 // One element of the ConvLSTM gate chain: pre-activation gate reservoirs r* and their deltas d*, cached
 // previous cell state cp and its delta dP, cached cell state c0.  Updates the reservoirs in place and

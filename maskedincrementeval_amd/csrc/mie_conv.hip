@@ -579,14 +579,20 @@ int upconv_entry(const char* who, const void* a_lo, const uint8_t* amask, const 
                  int act_kind, float slope, void* stream) {
   int rc = mie_check_tileset(out, who);
   if (rc != MIE_OK) return rc;
-  MIE_REQUIRE(a_lo && filter && filter_mc, MIE_ERR_INVALID_ARG, "%s: NULL pointer (a, filter and filter_mc are required)", who);
+  MIE_REQUIRE(a_lo && filter, MIE_ERR_INVALID_ARG, "%s: NULL pointer (a and filter are required)", who);
   MIE_REQUIRE(b_lo != nullptr || bmask == nullptr, MIE_ERR_INVALID_ARG, "%s: mask of absent b", who);
   MIE_REQUIRE(c > 0 && cout > 0 && h_lo > 0 && w_lo > 0 && cin_total >= c, MIE_ERR_INVALID_ARG,
               "%s: sizes out of range (c=%d cout=%d cin_total=%d h=%d w=%d)", who, c, cout, cin_total, h_lo, w_lo);
-  MIE_REQUIRE(k == 5 && pad == 2, MIE_ERR_UNSUPPORTED, "%s: only the 5x5 pad-2 conv is implemented (k=%d pad=%d)", who, k, pad);
-  const int chunk = 128 / (int)sizeof(T);      // 32 fp32 / 64 bf16 channels per staged chunk
-  MIE_REQUIRE(c % chunk == 0 && cout % 32 == 0 && cin_total % (32 / (int)sizeof(T)) == 0, MIE_ERR_UNSUPPORTED,
-              "%s: needs c %% %d == 0 and cout %% 32 == 0 (c=%d cout=%d)", who, chunk, c, cout);
+  // a single input of at most 8 channels (the flow estimate in front of an EVFlowNet decoder): 3x3 or 5x5
+  const bool few = c <= 8 && b_lo == nullptr && (k == 3 || k == 5) && pad == k / 2 && cout % 32 == 0;
+  if (!few) {
+    MIE_REQUIRE(k == 5 && pad == 2, MIE_ERR_UNSUPPORTED,
+                "%s: only the 5x5 pad-2 conv is implemented for more than 8 channels or two inputs (k=%d pad=%d)", who, k, pad);
+    MIE_REQUIRE(filter_mc != nullptr, MIE_ERR_INVALID_ARG, "%s: filter_mc is required", who);
+    const int chunk = 128 / (int)sizeof(T);      // 32 fp32 / 64 bf16 channels per staged chunk
+    MIE_REQUIRE(c % chunk == 0 && cout % 32 == 0 && cin_total % (32 / (int)sizeof(T)) == 0, MIE_ERR_UNSUPPORTED,
+                "%s: needs c %% %d == 0 and cout %% 32 == 0 (c=%d cout=%d)", who, chunk, c, cout);
+  }
   MIE_REQUIRE(out->h == 2 * h_lo && out->w == 2 * w_lo, MIE_ERR_INVALID_ARG,
               "%s: the tile set is (%d,%d), twice the input is (%d,%d)", who, out->h, out->w, 2 * h_lo, 2 * w_lo);
   MIE_REQUIRE((long long)out->n * h_lo * w_lo * c < (1LL << 40) && (long long)out->n * out->h * out->w < 0x7fffffffLL,
@@ -607,6 +613,11 @@ int upconv_entry(const char* who, const void* a_lo, const uint8_t* amask, const 
   a.ws = nullptr; a.ws_floats = 0; a.ws_plane = 0; a.xcd_fs = 0;
   a.ts = mie_dev_tileset(out);
   const unsigned cap = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
+  if (few) {
+    MIE_REQUIRE(mie_launch_conv_fewcin_up(a, k, cap, (hipStream_t)stream), MIE_ERR_UNSUPPORTED,
+                "%s: no kernel variant for c=%d cout=%d k=%d", who, c, cout, k);
+    return mie_check_launch(who);
+  }
   MIE_REQUIRE(mie_launch_conv_up_mfma(a, cap, (hipStream_t)stream), MIE_ERR_UNSUPPORTED,
               "%s: no kernel variant for c=%d cout=%d", who, c, cout);
   return mie_check_launch(who);

@@ -13,6 +13,9 @@
 //     taps of parity w >> 1, only the ceil(Cin / 2) channel pairs that exist; the two tap halves meet in
 //     LDS and are added in a fixed order; epilogue as everywhere (addend, reservoir, activation, refresh).
 // One input only (x2 unsupported), stride 1 or 2, K = 3 or 5, Cout % 32 == 0.
+// UP: the input is up2x(x), the bilinear x2 up-sampling of a delta given at half resolution (a.h_in / a.w_in are
+// the up-sampled size): every staged pixel is blended from its four source pixels while staging, the up-sampled
+// tensor is never formed (the 2-channel flow estimate in front of an EVFlowNet decoder).  Stride 1 only.
 #include "mie_conv.h"
 
 namespace {
@@ -22,8 +25,9 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 constexpr int FC_CH = 8;     // staged channels per pixel
 constexpr int FC_PS = 9;     // LDS floats per staged pixel (odd: the 32 pixels of a block fall on distinct banks)
 
-template <typename T, int K, int S>
+template <typename T, int K, int S, bool UP = false>
 __global__ __launch_bounds__(256) void k_conv_fewcin(ConvArgsT<T> a) {
+  static_assert(!UP || S == 1, "the up-sampling form is stride 1");
   constexpr int IT = 7 * S + K;                  // input tile edge incl. halo
   constexpr int NPIX = IT * IT;
   constexpr int IN_F = NPIX * FC_PS;
@@ -68,8 +72,21 @@ __global__ __launch_bounds__(256) void k_conv_fewcin(ConvArgsT<T> a) {
     const int iy = iy0 + pix / IT, ix = ix0 + pix % IT;
     float v = 0.f;
     if (pix < NPIX && ch < cin && iy >= 0 && iy < a.h_in && ix >= 0 && ix < a.w_in) {
-      const long long po = ((long long)n * a.h_in + iy) * a.w_in + ix;
-      if (a.xm == nullptr || a.xm[po]) v = mie_ld(a.x, po * cin + ch);
+      if constexpr (UP) {
+        const int h_lo = a.h_in >> 1, w_lo = a.w_in >> 1;
+        int r[2], q[2];
+        float lr[2], lq[2];
+        conv_up2x_coef(iy, h_lo, r[0], r[1], lr[0], lr[1]);
+        conv_up2x_coef(ix, w_lo, q[0], q[1], lq[0], lq[1]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const long long po = ((long long)n * h_lo + r[j >> 1]) * w_lo + q[j & 1];
+          if (a.xm == nullptr || a.xm[po]) v += lr[j >> 1] * lq[j & 1] * mie_ld(a.x, po * cin + ch);
+        }
+      } else {
+        const long long po = ((long long)n * a.h_in + iy) * a.w_in + ix;
+        if (a.xm == nullptr || a.xm[po]) v = mie_ld(a.x, po * cin + ch);
+      }
     }
     vin[i] = v;
   }
@@ -133,8 +150,25 @@ bool launch_fewcin(const ConvArgsT<T>& a, int k, int s, unsigned cap, hipStream_
   }
 }
 
+template <typename T>
+bool launch_fewcin_up(const ConvArgsT<T>& a, int k, unsigned cap, hipStream_t st) {
+  if (a.x2 != nullptr || a.c1 < 1 || a.c1 > FC_CH || a.cout % 32 != 0 || a.pad != k / 2) return false;
+  const dim3 grid(cap, a.cout / 32), block(256);
+  switch (k) {
+    case 3: hipLaunchKernelGGL((k_conv_fewcin<T, 3, 1, true>), grid, block, 0, st, a); return true;
+    case 5: hipLaunchKernelGGL((k_conv_fewcin<T, 5, 1, true>), grid, block, 0, st, a); return true;
+    default: return false;
+  }
+}
+
 }  // namespace
 
+bool mie_launch_conv_fewcin_up(const ConvArgsT<float>& a, int k, unsigned cap, hipStream_t st) {
+  return launch_fewcin_up(a, k, cap, st);
+}
+bool mie_launch_conv_fewcin_up(const ConvArgsT<mie_bf16>& a, int k, unsigned cap, hipStream_t st) {
+  return launch_fewcin_up(a, k, cap, st);
+}
 bool mie_launch_conv_fewcin(const ConvArgsT<float>& a, int k, int s, unsigned cap, hipStream_t st) {
   return launch_fewcin(a, k, s, cap, st);
 }

@@ -102,18 +102,6 @@ __device__ __forceinline__ void mma_unit(v16f& acc, const float4& av, const floa
                                                 __builtin_bit_cast(mie_bf16x8, b4), acc, 0, 0, 0);
 }
 
-// Source rows / columns and weights of output index o of a bilinear x2 up-sampling (align_corners =
-// False): src = max(0, o/2 - 0.25), upper index clamped to the last row.
-__device__ __forceinline__ void conv_up2x_coef(int o, int in_size, int& i0, int& i1, float& l0, float& l1) {
-  const int j = o >> 1;
-  if (o & 1) {
-    i0 = j; i1 = (j + 1 < in_size) ? j + 1 : j; l0 = 0.75f; l1 = 0.25f;
-  } else if (j == 0) {
-    i0 = 0; i1 = (1 < in_size) ? 1 : 0; l0 = 1.f; l1 = 0.f;
-  } else {
-    i0 = j - 1; i1 = j; l0 = 0.25f; l1 = 0.75f;
-  }
-}
 // One 16-byte slot of delta elements <-> fp32 values (4 of them, or 8 for bf16).
 __device__ __forceinline__ void slot_to_f32(const float4& raw, float (&f)[4], float) {
   f[0] = raw.x; f[1] = raw.y; f[2] = raw.z; f[3] = raw.w;

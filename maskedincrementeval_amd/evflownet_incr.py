@@ -333,7 +333,11 @@ class UpsampleConvLayerIncr(nn.Module):
                 and _mask_of(wide[0]) is not None and _mask_of(wide[1]) is not None)
 
     def forward(self, parts):
-        ups = [self.up[i](p) for i, p in enumerate(parts)]
+        k, s, p = self.conv2d._geometry()
+        # the narrow leading part (the flow estimate) is up-sampled inside its conv when the shape allows it
+        lead_fused = (len(parts) == 3 and self._split_ok(parts) and _mask_of(parts[0]) is not None
+                      and ops.upconv_few_takes(parts[0][0].shape[1], self.conv2d.out_channels, k, s, p))
+        ups = [None if (lead_fused and i == 0) else self.up[i](p_) for i, p_ in enumerate(parts)]
         if not self._split_ok(parts):
             out = self.conv2d(self.cat(ups))
             if self.norm in ["BN", "IN"]:
@@ -343,12 +347,26 @@ class UpsampleConvLayerIncr(nn.Module):
         lead_c = 0
         addend = None
         if len(ups) == 3:
-            lead_c = ups[0][0].shape[1]
+            lead_c = parts[0][0].shape[1]
             # the flow estimate of the previous scale shares the mask of x (it is a 1x1 conv + tanh of
             # it), so the wide conv's output mask covers this partial result
-            addend = self._lead_conv(ups[0], filt.rows(0, lead_c))
+            if lead_fused:
+                addend = self._lead_upconv(parts[0], filt.rows(0, lead_c))
+            else:
+                addend = self._lead_conv(ups[0], filt.rows(0, lead_c))
         return self.conv2d.forward_fused(ups[-2], self.activation, ups[-1], addend_incr=addend,
                                          filt=filt.rows(lead_c, filt.shape[0]))
+
+    def _lead_upconv(self, x_incr, filt):
+        """conv over up2x(x) of the narrow leading part in one kernel (ops.upconv_masked, few-channel form)."""
+        k, s, p = self.conv2d._geometry()
+        a, pa, _, _, ts_up = self.up[0].plan(x_incr, None)
+        n, _, h, w = a.shape
+        ts = self._lead._tile_set("lead", n, 2 * h, 2 * w, a.device)
+        ops.build_mask_tiles(ts_up, None, n, 2 * h, 2 * w, _lib.FOOT_CONV, k, s, p, ts)
+        out = self._lead._delta_buf("lead", (n, self.conv2d.out_channels, 2 * h, 2 * w), a.device, a.dtype)
+        ops.upconv_masked(a, pa, None, None, filt, k, p, ts, out)
+        return [out, ts]
 
     def _lead_conv(self, x_incr, filt):
         k, s, p = self.conv2d._geometry()

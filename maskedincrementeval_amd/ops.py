@@ -391,9 +391,15 @@ def upconv_takes(c: int, cout: int, k: int, stride: int, pad: int, filt, dtype) 
             and cout % 32 == 0 and filt.for_dtype(dtype)[1] is not None)
 
 
+def upconv_few_takes(c: int, cout: int, k: int, stride: int, pad: int) -> bool:
+    """Whether upconv_masked takes a SINGLE input of c channels through its few-channel kernel (3x3 or 5x5)."""
+    return c <= 8 and k in (3, 5) and stride == 1 and pad == k // 2 and cout % 32 == 0
+
+
 def upconv_masked(a, amask, b, bmask, filt, k, pad, out_ts: TileMask, out_delta, reservoir=None,
                   act=_lib.ACT_NONE, slope=0.0, addend=None):
-    """5x5 conv over up2x(a + b) in one kernel; a, b at half the resolution of out_ts (b may be None)."""
+    """conv over up2x(a + b) in one kernel; a, b at half the resolution of out_ts (b may be None): 5x5 for inputs in
+    whole matrix-core chunks, 3x3 or 5x5 for a single input of at most 8 channels."""
     n, c, h, w = a.shape
     dt = a.dtype
     if b is not None and (b.shape != a.shape or b.dtype != dt):

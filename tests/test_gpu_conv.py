@@ -292,6 +292,34 @@ def test_upsampled_conv_in_one_kernel(c, cout, h, w, dtype):
             assert torch.allclose(res.cpu(), r0 + ref, rtol=RTOL, atol=2e-2 if bf else 1e-4)
 
 
+# The same for a single input of very few channels (the flow estimate in front of an EVFlowNet decoder): 3x3 and 5x5.
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("c,cout,k,h,w", [(2, 64, 3, 13, 17), (2, 32, 3, 32, 32), (5, 96, 5, 9, 40), (8, 32, 3, 21, 11)])
+def test_upsampled_conv_few_channels(c, cout, k, h, w, dtype):
+    bf = dtype == torch.bfloat16
+    tol = dict(rtol=2e-2, atol=2e-2) if bf else dict(rtol=RTOL, atol=5e-5)
+    q = (lambda t: t.to(torch.bfloat16).float()) if bf else (lambda t: t)
+    n, p = 2, k // 2
+    wt = q(he_normal_conv_weight(cout, c, k, 19))
+    filt = _filt(wt)
+    assert ops.upconv_few_takes(c, cout, k, 1, p)
+    ts_up, ts = TileMask(n, 2 * h, 2 * w, DEV), TileMask(n, 2 * h, 2 * w, DEV)
+    out = ops.new_nhwc(n, cout, 2 * h, 2 * w, DEV, dtype)
+    for step, dens in enumerate((0.3, 0.05, 1.0)):
+        a, ma = gaussian_delta(n, c, h, w, dens, 0.5, seed=700 + step)
+        a = q(a)
+        ref = io.conv_incr(io.interp_incr(a), wt, 1, p)          # the staged tile stays fp32: no rounding in between
+        dma = ma.to(DEV)
+        ops.build_mask_tiles(dma, None, n, h, w, _lib.FOOT_UP2X, 0, 0, 0, ts_up)
+        ops.build_mask_tiles(ts_up, None, n, 2 * h, 2 * w, _lib.FOOT_CONV, k, 1, p, ts)
+        poisoned = torch.where(ma.bool().expand_as(a), a, torch.full_like(a, float("nan")))
+        ops.upconv_masked(_dev(poisoned).to(dtype), dma, None, None, filt, k, p, ts, out)
+        torch.cuda.synchronize()
+        got = out.float().cpu()
+        assert torch.isfinite(got).all()
+        assert torch.allclose(got, ref, **tol), "step %d max|diff| = %.3e" % (step, (got - ref).abs().max())
+
+
 def _random_cases(count, seed):
     rng = np.random.RandomState(seed)
     cases = []
