@@ -347,6 +347,19 @@ int mie_upsample2x_incr(const void* a, const uint8_t* ma, const void* b,
                         void* stream);
 
 /*
+ * Two independent mie_upsample2x_incr calls of the same geometry (c channels,
+ * [n,h_in,w_in] -> twice that) in one launch: input, mask, tile set and output
+ * of their own each.  For decoders that up-sample the parts of a channel
+ * concat one by one (incr_modules/evflownet_incr.py:294-343 up-samples the
+ * concatenated tensor; here the concat is never formed).
+ */
+int mie_upsample2x_pair_incr(const void* a0, const uint8_t* m0,
+                             const mie_tileset* out0, void* out_delta0,
+                             const void* a1, const uint8_t* m1,
+                             const mie_tileset* out1, void* out_delta1,
+                             int h_in, int w_in, int c, int dtype, void* stream);
+
+/*
  * Fused incremental ConvLSTM gate math for hidden size hid over the active
  * tiles of ts.  gates_delta is [n,h,w,4*hid] in the reference chunk order
  * [in, remember, out, cell] (incr_modules/e2depth_incr.py:103).  State kept

@@ -34,7 +34,7 @@ EXPORTS = (
     "mie_upsample2x_incr", "mie_convlstm_gates_incr", "mie_tconv_masked", "mie_conv_refresh",
     "mie_pack_filter", "mie_kfence_incr", "mie_events_to_frame", "mie_tconv_refresh", "mie_conv_gates_masked",
     "mie_maxpool_incr", "mie_accumulate", "mie_scale_incr", "mie_avgpool_incr", "mie_linear_incr", "mie_upconv_masked",
-    "mie_conv_masked_ws", "mie_convgru_gates_incr",
+    "mie_conv_masked_ws", "mie_convgru_gates_incr", "mie_upsample2x_pair_incr",
 )
 
 
@@ -77,6 +77,8 @@ def _declare(l):
     l.mie_conv_masked_ws.restype = ci
     l.mie_conv_masked_ws.argtypes = [vp, vp, ci, vp, vp, ci, ci, ci, vp, vp, ci, ci, ci, ci, ci, tsp, vp,
                                      vp, vp, ci, cf, ci, ci, vp, ctypes.c_longlong, vp]
+    l.mie_upsample2x_pair_incr.restype = ci
+    l.mie_upsample2x_pair_incr.argtypes = [vp, vp, tsp, vp, vp, vp, tsp, vp, ci, ci, ci, ci, vp]
     l.mie_convgru_gates_incr.restype = ci
     l.mie_convgru_gates_incr.argtypes = [vp, vp, vp, vp, ci, tsp, ci, vp]
     l.mie_kfence_incr.restype = ci

@@ -283,11 +283,10 @@ __device__ __forceinline__ void up2x_coef(int o, int in_size, int& i0, int& i1, 
 // output slot then reads its four taps from there -- 36 source pixels fetched per tile instead of
 // 4 per output pixel, which is what the kernel was bound by (load instructions, not bytes).
 template <typename T, int VEC>
-__global__ __launch_bounds__(256) void k_up2x_incr(TileSetDev ts, const T* __restrict__ a,
-                                                   const uint8_t* __restrict__ ma,
-                                                   const T* __restrict__ b,
-                                                   const uint8_t* __restrict__ mb, int h_in,
-                                                   int w_in, T* __restrict__ dout, int c) {
+__device__ __forceinline__ void up2x_tile(const TileSetDev& ts, const T* __restrict__ a,
+                                          const uint8_t* __restrict__ ma, const T* __restrict__ b,
+                                          const uint8_t* __restrict__ mb, int h_in, int w_in,
+                                          T* __restrict__ dout, int c) {
   extern __shared__ __attribute__((aligned(16))) float s_src[];   // [36 source pixels][channels of this block]
   __shared__ uint8_t s_act[64];                                   // output pixel active (fetched with the sources)
   int n, y0, x0;
@@ -348,6 +347,27 @@ __global__ __launch_bounds__(256) void k_up2x_incr(TileSetDev ts, const T* __res
     }
     o.store(dout + off);
   });
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void k_up2x_incr(TileSetDev ts, const T* __restrict__ a,
+                                                   const uint8_t* __restrict__ ma,
+                                                   const T* __restrict__ b,
+                                                   const uint8_t* __restrict__ mb, int h_in,
+                                                   int w_in, T* __restrict__ dout, int c) {
+  up2x_tile<T, VEC>(ts, a, ma, b, mb, h_in, w_in, dout, c);
+}
+
+// Two independent up-samplings of the same geometry (tensors, masks and tile sets of their own) in one
+// launch: blockIdx.z picks the operand set.  For decoders that up-sample the parts of a concat one by one.
+template <typename T>
+struct Up2xSet {
+  TileSetDev ts; const T* a; const uint8_t* ma; T* out;
+};
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void k_up2x_pair(Up2xSet<T> s0, Up2xSet<T> s1, int h_in, int w_in, int c) {
+  if (blockIdx.z == 0) up2x_tile<T, VEC>(s0.ts, s0.a, s0.ma, (const T*)nullptr, (const uint8_t*)nullptr, h_in, w_in, s0.out, c);
+  else up2x_tile<T, VEC>(s1.ts, s1.a, s1.ma, (const T*)nullptr, (const uint8_t*)nullptr, h_in, w_in, s1.out, c);
 }
 
 // ---- max pooling increment and masked accumulate ---------------------------------
@@ -644,6 +664,48 @@ extern "C" int mie_upsample2x_incr(const void* a, const uint8_t* ma, const void*
     if (vec == 8) MIE_UP2X_LAUNCH(float, 8); else if (vec == 4) MIE_UP2X_LAUNCH(float, 4); else MIE_UP2X_LAUNCH(float, 1);
   }
 #undef MIE_UP2X_LAUNCH
+  return mie_check_launch(who);
+}
+
+extern "C" int mie_upsample2x_pair_incr(const void* a0, const uint8_t* m0, const mie_tileset* out0, void* out_delta0,
+                                        const void* a1, const uint8_t* m1, const mie_tileset* out1, void* out_delta1,
+                                        int h_in, int w_in, int c, int dtype, void* stream) {
+  mie_clear_error();
+  const char* who = "mie_upsample2x_pair_incr";
+  int rc = check_pointwise(who, out0, c);
+  if (rc != MIE_OK) return rc;
+  rc = check_pointwise(who, out1, c);
+  if (rc != MIE_OK) return rc;
+  MIE_DTYPE_OK(dtype, who);
+  MIE_REQUIRE(a0 && a1 && out_delta0 && out_delta1, MIE_ERR_INVALID_ARG, "%s: NULL pointer", who);
+  MIE_REQUIRE(out_delta0 != out_delta1 && out0 != out1 && out0->tiles != out1->tiles, MIE_ERR_INVALID_ARG,
+              "%s: the two outputs and tile sets must be distinct", who);
+  MIE_REQUIRE(h_in > 0 && w_in > 0 && out0->h == 2 * h_in && out0->w == 2 * w_in && out1->h == out0->h &&
+                  out1->w == out0->w && out1->n == out0->n,
+              MIE_ERR_INVALID_ARG, "%s: both outputs must be (n, %d, %d), twice the input", who, 2 * h_in, 2 * w_in);
+  MIE_PTR16(a0, who, "a0"); MIE_PTR16(a1, who, "a1"); MIE_PTR16(out_delta0, who, "out_delta0");
+  MIE_PTR16(out_delta1, who, "out_delta1");
+  const unsigned grid = (unsigned)mie_tile_capacity(out0->n, out0->h, out0->w);
+  const bool bf = dtype == MIE_DTYPE_BF16;
+  const int vec = (c % 8 == 0 && (bf || c >= 64)) ? 8 : (c % 4 == 0 ? 4 : 1);
+  const int cv = c / vec;
+  unsigned ny = channel_splits((int)grid, cv);
+  const unsigned ny_min = (unsigned)mie_div_up(c, 256);
+  if (ny < ny_min) ny = ny_min;
+  const size_t lds = (size_t)36 * mie_div_up(cv, (int)ny) * vec * sizeof(float);
+#define MIE_UP2X_PAIR(T_, V_)                                                                                  \
+  do {                                                                                                         \
+    Up2xSet<T_> s0{mie_dev_tileset(out0), (const T_*)a0, m0, (T_*)out_delta0};                                  \
+    Up2xSet<T_> s1{mie_dev_tileset(out1), (const T_*)a1, m1, (T_*)out_delta1};                                  \
+    hipLaunchKernelGGL((k_up2x_pair<T_, V_>), dim3(grid, ny, 2), dim3(256), lds, (hipStream_t)stream, s0, s1,  \
+                       h_in, w_in, c);                                                                         \
+  } while (0)
+  if (bf) {
+    if (vec == 8) MIE_UP2X_PAIR(mie_bf16, 8); else if (vec == 4) MIE_UP2X_PAIR(mie_bf16, 4); else MIE_UP2X_PAIR(mie_bf16, 1);
+  } else {
+    if (vec == 8) MIE_UP2X_PAIR(float, 8); else if (vec == 4) MIE_UP2X_PAIR(float, 4); else MIE_UP2X_PAIR(float, 1);
+  }
+#undef MIE_UP2X_PAIR
   return mie_check_launch(who);
 }
 

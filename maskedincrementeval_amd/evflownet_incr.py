@@ -337,7 +337,12 @@ class UpsampleConvLayerIncr(nn.Module):
         # the narrow leading part (the flow estimate) is up-sampled inside its conv when the shape allows it
         lead_fused = (len(parts) == 3 and self._split_ok(parts) and _mask_of(parts[0]) is not None
                       and ops.upconv_few_takes(parts[0][0].shape[1], self.conv2d.out_channels, k, s, p))
-        ups = [None if (lead_fused and i == 0) else self.up[i](p_) for i, p_ in enumerate(parts)]
+        ups = [None] * len(parts)
+        if self._split_ok(parts) and parts[-2][0].shape == parts[-1][0].shape and parts[-2][0].dtype == parts[-1][0].dtype:
+            ups[-2], ups[-1] = self._up_pair(len(parts) - 2, parts[-2], parts[-1])      # the two wide parts in one launch
+        for i, p_ in enumerate(parts):
+            if ups[i] is None and not (lead_fused and i == 0):
+                ups[i] = self.up[i](p_)
         if not self._split_ok(parts):
             out = self.conv2d(self.cat(ups))
             if self.norm in ["BN", "IN"]:
@@ -356,6 +361,16 @@ class UpsampleConvLayerIncr(nn.Module):
                 addend = self._lead_conv(ups[0], filt.rows(0, lead_c))
         return self.conv2d.forward_fused(ups[-2], self.activation, ups[-1], addend_incr=addend,
                                          filt=filt.rows(lead_c, filt.shape[0]))
+
+    def _up_pair(self, i, x_incr, y_incr):
+        """self.up[i](x), self.up[i + 1](y) as one launch (ops.upsample2x_pair_incr)."""
+        a, pa, _, _, ts_a = self.up[i].plan(x_incr, None)
+        b, pb, _, _, ts_b = self.up[i + 1].plan(y_incr, None)
+        n, c, h, w = a.shape
+        out_a = self.up[i]._delta_buf("out", (n, c, 2 * h, 2 * w), a.device, a.dtype)
+        out_b = self.up[i + 1]._delta_buf("out", (n, c, 2 * h, 2 * w), b.device, b.dtype)
+        ops.upsample2x_pair_incr(a, pa, ts_a, out_a, b, pb, ts_b, out_b)
+        return [out_a, ts_a], [out_b, ts_b]
 
     def _lead_upconv(self, x_incr, filt):
         """conv over up2x(x) of the narrow leading part in one kernel (ops.upconv_masked, few-channel form)."""

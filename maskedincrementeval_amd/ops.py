@@ -632,6 +632,25 @@ def upsample2x_incr(a, ma, b, mb, out_ts: TileMask, out_delta):
     return out_delta
 
 
+def upsample2x_pair_incr(a0, m0, ts0: TileMask, out0, a1, m1, ts1: TileMask, out1):
+    """Two up-samplings of the same geometry in one launch (own input, mask, tile set and output each)."""
+    n, c, h, w = a0.shape
+    _same_shape("a1", a1, a0)
+    for name, o in (("out0", out0), ("out1", out1)):
+        if tuple(o.shape) != (n, c, 2 * h, 2 * w):
+            raise ValueError("%s shape %s, expected %s" % (name, tuple(o.shape), (n, c, 2 * h, 2 * w)))
+    _ready(ts0)
+    _ready(ts1)
+    dt = a0.dtype
+    if a1.dtype != dt:
+        raise ValueError("the two inputs differ in dtype")
+    check(lib().mie_upsample2x_pair_incr(
+        nhwc_ptr(a0, "a0", dtype=dt), pix_ptr(m0, n, h, w, "m0"), ts0.ref, nhwc_ptr(out0, "out0", dtype=dt),
+        nhwc_ptr(a1, "a1", dtype=dt), pix_ptr(m1, n, h, w, "m1"), ts1.ref, nhwc_ptr(out1, "out1", dtype=dt),
+        h, w, c, delta_dtype(a0), _stream(a0)))
+    return out0, out1
+
+
 def convlstm_gates_incr(gates_delta, gates_res, cprev_delta, cprev_mask, cprev_res, cell_res,
                         h_delta, c_delta, ts: TileMask):
     n, c4, h, w = gates_delta.shape

@@ -278,3 +278,29 @@ def test_kernel_bench_modes_run_and_report(argv, dtype, monkeypatch, capsys):
     line = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
     assert line["us"] > 0
     assert line.get("algorithmic_bytes", line.get("bytes_read", 0)) > 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("c,h,w", [(64, 13, 17), (8, 16, 16), (6, 9, 30)])
+def test_upsample_pair_equals_two_single_launches(c, h, w, dtype):
+    # two up-samplings of the same geometry in one launch: bit-identical to the two separate calls, over
+    # three steps with fresh masks (stale tiles), inactive inputs poisoned
+    from maskedincrementeval_amd.masked_types import TileMask
+    n = 2
+    ts = [TileMask(n, 2 * h, 2 * w, DEV) for _ in range(4)]
+    outs = [ops.new_nhwc(n, c, 2 * h, 2 * w, DEV, dtype) for _ in range(4)]
+    for step in range(3):
+        ins = []
+        for j in range(2):
+            d, m = gaussian_delta(n, c, h, w, (0.3, 0.05, 0.6)[step] * (1 + j) / 2, 0.5, seed=880 + 10 * step + j)
+            x = _dev(torch.where(m.bool().expand_as(d), d, torch.full_like(d, float("nan")))).to(dtype)
+            ins.append((x, m.to(DEV)))
+        for j in range(2):
+            for t in (ts[j], ts[2 + j]):
+                ops.build_mask_tiles(ins[j][1], None, n, h, w, _lib.FOOT_UP2X, 0, 0, 0, t)
+            ops.upsample2x_incr(ins[j][0], ins[j][1], None, None, ts[j], outs[j])
+        ops.upsample2x_pair_incr(ins[0][0], ins[0][1], ts[2], outs[2], ins[1][0], ins[1][1], ts[3], outs[3])
+        torch.cuda.synchronize()
+        for j in range(2):
+            assert torch.isfinite(outs[2 + j].float()).all()
+            assert torch.equal(outs[j], outs[2 + j]), "step %d input %d" % (step, j)
