@@ -127,14 +127,22 @@ __global__ __launch_bounds__(256) void k_conv_fewcin(ConvArgsT<T> a) {
   if (th == 1) return;
 
   // ---- epilogue: lane = output column l32, 16 pixels of the block per lane ---------------------------
+  // (all reservoir / addend loads of the lane as one batch, then the stores: an element-by-element
+  // read-modify-write would be 16 dependent memory round trips)
+  long long off[16];
+  int co[16];
+  bool ok[16];
+  float v[16];
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int p = mb * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
     const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
-    if (oy < hout && ox < wout)
-      conv_store(a, (((long long)n * hout + oy) * wout + ox) * cout + co0 + l32, co0 + l32,
-                 acc[r] + red[(mb * 16 + r) * 64 + lane]);
+    ok[r] = oy < hout && ox < wout;
+    off[r] = (((long long)n * hout + oy) * wout + ox) * cout + co0 + l32;
+    co[r] = co0 + l32;
+    v[r] = acc[r] + red[(mb * 16 + r) * 64 + lane];
   }
+  conv_store_batch<T, 16>(a, off, co, ok, v);
 }
 
 template <typename T>
