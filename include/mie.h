@@ -225,6 +225,37 @@ int mie_conv_masked_ws(const void* x, const uint8_t* xmask, int c1,
                        long long workspace_bytes, void* stream);
 
 /*
+ * mie_conv_masked_ws for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the
+ * same arguments as mie_conv_masked, and the workspace of the split form is an
+ * array of MIE_NOALLOC_WS_BYTES that lives in the library's device image (each
+ * GPU the library runs on holds its own copy until the process ends).  The call
+ * allocates and frees nothing; it looks the array's device address up once per
+ * device, on the first call made with that device current (make that first
+ * call outside of a stream capture).  Results are those of mie_conv_masked_ws
+ * with a workspace of MIE_NOALLOC_WS_BYTES, bit for bit.
+ *   Limit: two partial planes must fit, 2 * n*h*w*cout*4 <= MIE_NOALLOC_WS_BYTES
+ *   (every launch the split form takes is far below that); a larger output is
+ *   refused with MIE_ERR_CAPACITY and nothing is launched -- use
+ *   mie_conv_masked there.
+ *   Sharing: every call on a GPU uses that GPU's one array and leaves its last
+ *   partial sums there.  Nothing in it has to start at zero (each launch
+ *   writes every partial sum it later reads), but calls that overlap on one
+ *   GPU (two streams, two threads) race on it: order them on one stream.
+ * Has no counterpart in the reference; it exists for callers that cannot
+ * allocate.
+ */
+#define MIE_NOALLOC_WS_BYTES (8 * 1024 * 1024)
+int mie_conv_masked_noalloc(const void* x, const uint8_t* xmask, int c1,
+                            const void* x2, const uint8_t* x2mask, int c2,
+                            int h_in, int w_in, const float* filter,
+                            const void* filter_mc, int cin_total,
+                            int k, int stride, int pad, int cout,
+                            const mie_tileset* out, void* out_delta,
+                            const void* addend, float* reservoir, int act_kind,
+                            float slope, int path, int dtype, void* stream);
+
+/*
  * Dense refresh through the same kernels: for every active tile of `out`
  * (build it with in_mask = NULL so that every tile is active)
  *   y = conv2d(x (++ x2), filter, bias, stride, pad) (+ addend);

@@ -18,6 +18,7 @@ LIB_PATH = os.environ.get("MIE_HIP_LIB") or os.path.join(_PKG_DIR, "lib", "libmi
 
 MIE_OK = 0
 MIE_TILE = 8
+NOALLOC_WS_BYTES = 8 * 1024 * 1024
 
 ACT_NONE, ACT_RELU, ACT_LEAKY_RELU, ACT_SIGMOID, ACT_TANH = 0, 1, 2, 3, 4
 FOOT_CONV, FOOT_UP2X, FOOT_TCONV = 0, 1, 2
@@ -34,7 +35,7 @@ EXPORTS = (
     "mie_upsample2x_incr", "mie_convlstm_gates_incr", "mie_tconv_masked", "mie_conv_refresh",
     "mie_pack_filter", "mie_kfence_incr", "mie_events_to_frame", "mie_tconv_refresh", "mie_conv_gates_masked",
     "mie_maxpool_incr", "mie_accumulate", "mie_scale_incr", "mie_avgpool_incr", "mie_linear_incr", "mie_upconv_masked",
-    "mie_conv_masked_ws", "mie_convgru_gates_incr", "mie_upsample2x_pair_incr",
+    "mie_conv_masked_ws", "mie_convgru_gates_incr", "mie_upsample2x_pair_incr", "mie_conv_masked_noalloc",
 )
 
 
@@ -74,6 +75,8 @@ def _declare(l):
     l.mie_conv_masked.restype = ci
     l.mie_conv_masked.argtypes = [vp, vp, ci, vp, vp, ci, ci, ci, vp, vp, ci, ci, ci, ci, ci, tsp, vp,
                                   vp, vp, ci, cf, ci, ci, vp]
+    l.mie_conv_masked_noalloc.restype = ci
+    l.mie_conv_masked_noalloc.argtypes = list(l.mie_conv_masked.argtypes)
     l.mie_conv_masked_ws.restype = ci
     l.mie_conv_masked_ws.argtypes = [vp, vp, ci, vp, vp, ci, ci, ci, vp, vp, ci, ci, ci, ci, ci, tsp, vp,
                                      vp, vp, ci, cf, ci, ci, vp, ctypes.c_longlong, vp]

@@ -14,6 +14,7 @@
 // increment, or (dense refresh) bias + activation + reservoir fill.
 #include "mie_common.h"
 #include "mie_conv.h"
+#include <mutex>
 
 namespace {
 
@@ -479,6 +480,73 @@ extern "C" int mie_conv_masked_ws(const void* x, const uint8_t* xmask, int c1, c
                       (const T*)filter_mc, cin_total, k, stride, pad, cout, out, (T*)out_delta,
                       (const T*)addend, reservoir, act_kind, slope, path, false, nullptr, stream, nullptr,
                       workspace, workspace_bytes);
+}
+
+// ---- the workspace form for callers that cannot allocate ---------------------------------------
+// The split form's partial sums live in a device-resident array instead of a caller workspace.  The
+// array's name is only a host-side handle: its device address differs per GPU and is looked up once
+// per device (with that device current) on the entry point's first call there; kernels and every
+// other use take that address.
+#define MIE_NOALLOC_MAX_DEVICES 64
+static __device__ __align__(256) float scratch[MIE_NOALLOC_WS_BYTES / 4];
+
+namespace {
+int noalloc_scratch(const char* who, float** out) {
+  static float* ptrs[MIE_NOALLOC_MAX_DEVICES];      // zero-initialised; written once per device
+  static bool known[MIE_NOALLOC_MAX_DEVICES];
+  static std::mutex mu;
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  MIE_REQUIRE(e == hipSuccess && dev >= 0 && dev < MIE_NOALLOC_MAX_DEVICES, MIE_ERR_LAUNCH,
+              "%s: no current device (%s)", who, hipGetErrorString(e));
+  std::lock_guard<std::mutex> lock(mu);
+  if (!known[dev]) {
+    float* p = nullptr;
+    e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+    MIE_REQUIRE(e == hipSuccess && p != nullptr, MIE_ERR_LAUNCH,
+                "%s: the device-resident workspace has no address on device %d (%s)", who, dev,
+                hipGetErrorString(e));
+    ptrs[dev] = p;
+    known[dev] = true;
+  }
+  *out = ptrs[dev];
+  return MIE_OK;
+}
+}  // namespace
+
+extern "C" int mie_conv_masked_noalloc(const void* x, const uint8_t* xmask, int c1, const void* x2,
+                                       const uint8_t* x2mask, int c2, int h_in, int w_in,
+                                       const float* filter, const void* filter_mc, int cin_total, int k,
+                                       int stride, int pad, int cout, const mie_tileset* out,
+                                       void* out_delta, const void* addend, float* reservoir,
+                                       int act_kind, float slope, int path, int dtype, void* stream) {
+  const char* who = "mie_conv_masked_noalloc";
+  MIE_CONV_DTYPE_OK(dtype, who);
+  int rc = mie_check_tileset(out, who);
+  if (rc != MIE_OK) return rc;
+  MIE_REQUIRE(cout > 0, MIE_ERR_INVALID_ARG, "%s: cout must be positive", who);
+  // two partial planes of the output must fit: beyond that the launch is no "plane of very few tiles"
+  const long long plane_bytes = (long long)out->n * out->h * out->w * cout * 4;
+  MIE_REQUIRE(2 * plane_bytes <= (long long)MIE_NOALLOC_WS_BYTES, MIE_ERR_CAPACITY,
+              "%s: an output plane of %lld bytes (n=%d h=%d w=%d cout=%d) exceeds the device-resident "
+              "workspace, which holds two planes of at most %lld bytes each; use mie_conv_masked for "
+              "larger outputs", who, plane_bytes, out->n, out->h, out->w, cout,
+              (long long)MIE_NOALLOC_WS_BYTES / 2);
+  float* ws = nullptr;
+  rc = noalloc_scratch(who, &ws);
+  if (rc != MIE_OK) return rc;
+  if (dtype == MIE_DTYPE_BF16) {
+    typedef mie_bf16 T;
+    return conv_impl<T>(who, (const T*)x, xmask, c1, (const T*)x2, x2mask, c2, h_in, w_in, filter,
+                        (const T*)filter_mc, cin_total, k, stride, pad, cout, out, (T*)out_delta,
+                        (const T*)addend, reservoir, act_kind, slope, path, false, nullptr, stream, nullptr,
+                        ws, (long long)MIE_NOALLOC_WS_BYTES);
+  }
+  typedef float T;
+  return conv_impl<T>(who, (const T*)x, xmask, c1, (const T*)x2, x2mask, c2, h_in, w_in, filter,
+                      (const T*)filter_mc, cin_total, k, stride, pad, cout, out, (T*)out_delta,
+                      (const T*)addend, reservoir, act_kind, slope, path, false, nullptr, stream, nullptr,
+                      ws, (long long)MIE_NOALLOC_WS_BYTES);
 }
 
 extern "C" int mie_conv_refresh(const void* x, int c1, const void* x2, int c2, int h_in,
