@@ -97,7 +97,8 @@ typedef struct mie_tileset {
   int32_t* tiles;     /* [capacity]   active tile ids, ascending              */
   int32_t* stale;     /* [capacity]   tiles active last step, inactive now    */
   int32_t* counts;    /* [MIE_CNT_WORDS] active, stale, ticket, reserved      */
-  uint32_t* flags;    /* [capacity]   1 = tile active (scratch of the build)  */
+  uint32_t* flags;    /* [capacity]   16-byte aligned; bit 0 = tile active,
+                         bit 1 = active after the previous build        */
 } mie_tileset;
 
 /* Library version (major*10000 + minor*100 + patch). */
@@ -128,8 +129,13 @@ int mie_mask_from_delta(const void* delta, int n, int h, int w, int c,
  *   foot, k, stride, pad: footprint (MIE_FOOT_*); for MIE_FOOT_UP2X k, stride
  *   and pad are ignored.  Output resolution is out->h, out->w.
  * Writes out->pixmask (every pixel), out->flags, out->tiles (ascending ids),
- * out->stale (tiles that were in out->tiles before this call and are not any
- * more, ascending) and out->counts[ACTIVE, STALE].
+ * out->stale (tiles that were active after the previous build of `out`, as
+ * out->flags remembers it, and are not any more; ascending) and
+ * out->counts[ACTIVE, STALE].
+ * Aliasing: out->pixmask may be in_mask / in_mask2 only for the identity
+ * footprint (MIE_FOOT_CONV, k = 1, stride = 1, pad = 0); any other footprint
+ * reads neighbouring bytes while they are written and is refused with
+ * MIE_ERR_INVALID_ARG.
  * Replaces: the mask argument of conv{1,3,5,7}x*_increment_ext
  * (ext/pointops/_C_ext/pointops/ops.cpp:27-48), which the reference kernel
  * never reads (ext_conv.cu:74-76 synthesises a fake one).
@@ -176,6 +182,10 @@ int mie_pack_filter(const float* filter, int cin, int k, int cout, void* packed,
  *        by mie_pack_filter with the same dtype.  The MFMA kernels read only this copy;
  *        without it MIE_PATH_AUTO takes the VALU kernels and MIE_PATH_MFMA is
  *        refused.
+ *   Aliasing: for k > 1 neither x nor x2 may be out_delta, and neither input
+ *   mask may be out->pixmask (workgroups read the halo of their tile while
+ *   others write it): MIE_ERR_INVALID_ARG.  The same holds for h_delta /
+ *   c_delta of mie_conv_gates_masked.
  *   k in {1,3,5,7}, stride in {1,2}; out->h/w must equal (h_in+2*pad-k)/stride+1
  *   dtype : element type of x, x2, addend, out_delta and filter_mc
  *        (MIE_DTYPE_BF16: products of bf16 values accumulated in fp32 on the

@@ -44,9 +44,10 @@ def _run(cmd, verbose):
         print(out, flush=True)
 
 
-def build_library(verbose=True):
+def build_library(verbose=True, incremental=False):
     """Compile every HIP source (one hipcc process per file, in parallel) and link
-    lib/libmie_hip.so; returns its path."""
+    lib/libmie_hip.so; returns its path.  incremental=True (`--incremental` on the command line)
+    skips sources whose object file is newer than the source and every header."""
     from concurrent.futures import ThreadPoolExecutor
     os.makedirs(LIB_DIR, exist_ok=True)
     obj_dir = os.path.join(LIB_DIR, "obj")
@@ -54,11 +55,17 @@ def build_library(verbose=True):
     hipcc = find_hipcc()
     compile_flags = [f for f in HIPCC_FLAGS if f != "-shared"]
     jobs = []
+    headers = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
+    headers.append(os.path.join(os.path.dirname(PKG_DIR), "include", "mie.h"))
+    newest_header = max(os.path.getmtime(h) for h in headers)
     for s in SOURCES:
         obj = os.path.join(obj_dir, s.replace(".hip", ".o"))
-        jobs.append(([hipcc] + compile_flags + ["-c", os.path.join(CSRC, s), "-o", obj], obj))
+        src = os.path.join(CSRC, s)
+        fresh = (incremental and os.path.exists(obj)
+                 and os.path.getmtime(obj) > max(os.path.getmtime(src), newest_header))
+        jobs.append(([hipcc] + compile_flags + ["-c", src, "-o", obj], obj, fresh))
     with ThreadPoolExecutor(max_workers=min(len(jobs), 8)) as pool:
-        list(pool.map(lambda j: _run(j[0], verbose), jobs))
+        list(pool.map(lambda j: None if j[2] else _run(j[0], verbose), jobs))
     tmp = LIB_PATH + ".tmp"
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc"] + [j[1] for j in jobs] + ["-o", tmp],
          verbose)
@@ -67,5 +74,5 @@ def build_library(verbose=True):
 
 
 if __name__ == "__main__":
-    print(build_library())
+    print(build_library(incremental="--incremental" in sys.argv[1:]))
     sys.exit(0)

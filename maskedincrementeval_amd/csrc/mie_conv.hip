@@ -304,6 +304,19 @@ int conv_impl(const char* who, const T* x, const uint8_t* xmask, int c1, const T
               "%s: bias must be 4-byte and addend 16-byte aligned", who);
   MIE_REQUIRE(addend == nullptr || addend != out_delta, MIE_ERR_INVALID_ARG,
               "%s: addend must not alias out_delta", who);
+  // A workgroup stages the halo of its tile, i.e. pixels that other workgroups of the launch write (their
+  // outputs, and the zeros of stale tiles): only a 1x1 conv, which reads no halo, may run in place.
+  MIE_REQUIRE(k == 1 || ((const void*)x != (const void*)out_delta && (x2 == nullptr || (const void*)x2 != (const void*)out_delta)),
+              MIE_ERR_INVALID_ARG, "%s: x / x2 must not alias out_delta for k > 1", who);
+  MIE_REQUIRE(gates == nullptr ||
+                  ((const void*)x != (const void*)gates->h_delta && (const void*)x != (const void*)gates->c_delta &&
+                   (x2 == nullptr || ((const void*)x2 != (const void*)gates->h_delta &&
+                                      (const void*)x2 != (const void*)gates->c_delta))),
+              MIE_ERR_INVALID_ARG, "%s: x / x2 must not alias h_delta / c_delta (keep two sets of state buffers "
+              "when the state deltas are fed back)", who);
+  MIE_REQUIRE((xmask == nullptr || xmask != (const uint8_t*)out->pixmask || k == 1) &&
+                  (x2mask == nullptr || x2mask != (const uint8_t*)out->pixmask || k == 1),
+              MIE_ERR_INVALID_ARG, "%s: an input mask must not be the output tile set's pixel mask for k > 1", who);
   const int pmul = 32 / (int)sizeof(T);       // input channels per block of the matrix-core filter copy
   MIE_REQUIRE(mie_aligned(filter_mc, 16), MIE_ERR_INVALID_ARG, "%s: filter_mc must be 16-byte aligned", who);
   MIE_REQUIRE(workspace_bytes >= 0 && (workspace != nullptr || workspace_bytes == 0) && mie_aligned(workspace, 16),

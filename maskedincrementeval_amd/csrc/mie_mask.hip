@@ -3,9 +3,10 @@
 // mie_build_mask_tiles is two launches on the caller's stream: every wave of
 // the first derives the 64 output-mask bits of one 8x8 tile from the input
 // mask footprint and records whether the tile holds any active pixel (wave
-// ballot); the second, a single block, turns the per-tile flags into the
-// ascending tile list with a ballot + popcount prefix scan, so the list order
-// is deterministic and nothing is communicated between workgroups inside a
+// ballot); the second turns the per-tile flags into the ascending tile lists
+// with a two-level ballot + popcount prefix scan (one block per 4096 tiles,
+// each counting the flags below its chunk itself), so the list order is
+// deterministic and nothing is communicated between workgroups inside a
 // kernel (device-wide fences cost tens of microseconds on this chip).
 #include "mie_common.h"
 
@@ -43,8 +44,8 @@ int mie_check_tileset(const mie_tileset* ts, const char* who) {
   MIE_REQUIRE(ts->pixmask && ts->tiles && ts->stale && ts->counts && ts->flags,
               MIE_ERR_INVALID_ARG, "%s: tile set has a NULL buffer", who);
   MIE_REQUIRE(mie_aligned(ts->tiles, 4) && mie_aligned(ts->stale, 4) &&
-                  mie_aligned(ts->counts, 4) && mie_aligned(ts->flags, 4),
-              MIE_ERR_INVALID_ARG, "%s: tile set buffers must be 4-byte aligned", who);
+                  mie_aligned(ts->counts, 4) && mie_aligned(ts->flags, 16),
+              MIE_ERR_INVALID_ARG, "%s: tile set buffers must be 4-byte aligned (flags: 16-byte)", who);
   return MIE_OK;
 }
 
@@ -176,89 +177,108 @@ __device__ __forceinline__ bool tile_footprint(const BuildArgs& a, int tile, int
   return __ballot(bit != 0) != 0ull;
 }
 
+// flags[tile]: bit 0 = the tile holds an active pixel after this build, bit 1 = it did after the
+// previous build of this tile set (what makes a tile stale).  A lane reads and writes its own word only.
+__device__ __forceinline__ uint32_t next_flag(uint32_t old, bool any) { return ((old & 1u) << 1) | (any ? 1u : 0u); }
+
 __global__ __launch_bounds__(256) void k_mask_footprint(BuildArgs a) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int tile = blockIdx.x * 4 + wave;
   if (tile >= a.cap) return;
+  const uint32_t old = a.flags[tile];          // issued ahead of the footprint's mask loads
   const bool any = tile_footprint(a, tile, lane);
-  if (lane == 0) a.flags[tile] = any ? 1u : 0u;
+  if (lane == 0) a.flags[tile] = next_flag(old, any);
 }
 
-// Ordered compaction of the ids `id(i)` (i in [0, count)) for which keep(i) holds, by the
-// COMPACT_THREADS threads of one block: per wave a ballot gives the 64 keep-bits, popcount
-// below the lane gives the rank, the wave totals are exchanged through LDS and a running
-// base carries across chunks.  The result is in ascending i order without any atomics.
+// Ordered compaction of the tile flags into the active list (bit 0 set) and the stale list (bit 1
+// set, bit 0 clear), both ascending, by a grid of COMPACT_THREADS-thread blocks without atomics or
+// fences: block b owns the COMPACT_CHUNK flags [b * CHUNK, (b + 1) * CHUNK).  It first counts the two
+// kinds over every flag below its chunk (16-byte loads; at most a few dozen per thread even for tens of
+// thousands of tiles) -- that is its base in either list -- and then ranks its own flags: per wave a
+// ballot gives 64 keep-bits, popcount below the lane the rank inside the wave, and the wave totals
+// meet in LDS.  The last block also writes the two totals.
 constexpr int COMPACT_THREADS = 1024;
 constexpr int COMPACT_WAVES = COMPACT_THREADS / 64;
+constexpr int COMPACT_ITEMS = 4;      // element j * COMPACT_THREADS + tid of the chunk, j < COMPACT_ITEMS
+constexpr int COMPACT_CHUNK = COMPACT_THREADS * COMPACT_ITEMS;
 
-// COMPACT_ITEMS candidates per thread and round (element i = start + j * COMPACT_THREADS + tid), so
-// that a plane of tens of thousands of tiles takes a few rounds of two barriers instead of dozens.
-constexpr int COMPACT_ITEMS = 4;
-
-template <typename KeepFn, typename IdFn>
-__device__ int block_compact(int count, KeepFn keep, IdFn id, int32_t* dst, int* s_tot) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  int base = 0;
-  for (int start = 0; start < count; start += COMPACT_THREADS * COMPACT_ITEMS) {
-    bool k[COMPACT_ITEMS];
-    int rank[COMPACT_ITEMS];
+__device__ __forceinline__ int wave_sum(int v) {
 #pragma unroll
-    for (int j = 0; j < COMPACT_ITEMS; ++j) {
-      const int i = start + j * COMPACT_THREADS + threadIdx.x;
-      k[j] = (i < count) && keep(i);
-      const unsigned long long bal = __ballot(k[j]);
-      rank[j] = __popcll(bal & ((1ull << lane) - 1ull));
-      if (lane == 0) s_tot[j * COMPACT_WAVES + wave] = __popcll(bal);
-    }
-    __syncthreads();
-    // exclusive prefix over the (j, wave) totals in element order: j major, wave minor
-    int off[COMPACT_ITEMS];
-    int run = base;
-#pragma unroll
-    for (int j = 0; j < COMPACT_ITEMS; ++j) {
-      off[j] = run;
-#pragma unroll
-      for (int wv = 0; wv < COMPACT_WAVES; ++wv) {
-        const int t = s_tot[j * COMPACT_WAVES + wv];
-        if (wv < wave) off[j] += t;
-        run += t;
-      }
-    }
-#pragma unroll
-    for (int j = 0; j < COMPACT_ITEMS; ++j)
-      if (k[j]) dst[off[j] + rank[j]] = id(start + j * COMPACT_THREADS + threadIdx.x);
-    base = run;
-    __syncthreads();
-  }
-  return base;
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+  return v;
 }
 
-// Kernel 2 (one block): per-tile flags -> stale list (previous list minus the tiles that are
-// still active) and the new ascending active list.
+// flag(t) returns the flag word of tile t (from memory or, for the one-block build, from LDS).
 template <typename FlagFn>
-__device__ void compact_lists(const BuildArgs& a, FlagFn flag, int* s_tot) {
-  // Clamp what comes from memory: a tile set whose counts / list were never initialised must
-  // give a wrong list, never an out-of-bounds access.
-  int n_prev = a.counts[MIE_CNT_ACTIVE];
-  n_prev = n_prev < 0 ? 0 : (n_prev > a.cap ? a.cap : n_prev);
-  const int32_t* prev = a.tiles;
-  const int cap = a.cap;
-  const int n_stale = block_compact(
-      n_prev, [&](int i) { const int t = prev[i]; return t >= 0 && t < cap && !flag(t); },
-      [&](int i) { return prev[i]; }, a.stale, s_tot);
-  __syncthreads();   // the old list has been consumed; it is overwritten next
-  const int n_act = block_compact(
-      a.cap, [&](int i) { return flag(i); }, [&](int i) { return i; }, a.tiles, s_tot);
-  if (threadIdx.x == 0) {
-    a.counts[MIE_CNT_ACTIVE] = n_act;
-    a.counts[MIE_CNT_STALE] = n_stale;
+__device__ void compact_lists(const BuildArgs& a, FlagFn flag, int chunk, int base_act, int base_st, bool last,
+                              int* s_tot) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  bool ka[COMPACT_ITEMS], ks[COMPACT_ITEMS];
+  int ra[COMPACT_ITEMS], rs[COMPACT_ITEMS];
+#pragma unroll
+  for (int j = 0; j < COMPACT_ITEMS; ++j) {
+    const int t = chunk * COMPACT_CHUNK + j * COMPACT_THREADS + threadIdx.x;
+    const uint32_t f = (t < a.cap) ? flag(t) : 0u;
+    ka[j] = (f & 1u) != 0u;
+    ks[j] = (f & 3u) == 2u;
+    const unsigned long long ba = __ballot(ka[j]), bs = __ballot(ks[j]);
+    const unsigned long long below = (1ull << lane) - 1ull;
+    ra[j] = __popcll(ba & below);
+    rs[j] = __popcll(bs & below);
+    if (lane == 0) {
+      s_tot[j * COMPACT_WAVES + wave] = __popcll(ba);
+      s_tot[COMPACT_ITEMS * COMPACT_WAVES + j * COMPACT_WAVES + wave] = __popcll(bs);
+    }
+  }
+  __syncthreads();
+  // exclusive prefix over the (j, wave) totals in element order: j major, wave minor
+  int run_a = base_act, run_s = base_st;
+#pragma unroll
+  for (int j = 0; j < COMPACT_ITEMS; ++j) {
+    int off_a = run_a, off_s = run_s;
+#pragma unroll
+    for (int wv = 0; wv < COMPACT_WAVES; ++wv) {
+      const int ta = s_tot[j * COMPACT_WAVES + wv];
+      const int tst = s_tot[COMPACT_ITEMS * COMPACT_WAVES + j * COMPACT_WAVES + wv];
+      if (wv < wave) off_a += ta, off_s += tst;
+      run_a += ta;
+      run_s += tst;
+    }
+    const int t = chunk * COMPACT_CHUNK + j * COMPACT_THREADS + threadIdx.x;
+    if (ka[j]) a.tiles[off_a + ra[j]] = t;
+    if (ks[j]) a.stale[off_s + rs[j]] = t;
+  }
+  if (last && threadIdx.x == 0) {
+    a.counts[MIE_CNT_ACTIVE] = run_a;
+    a.counts[MIE_CNT_STALE] = run_s;
   }
 }
 
 __global__ __launch_bounds__(COMPACT_THREADS) void k_compact_tiles(BuildArgs a) {
-  __shared__ int s_tot[COMPACT_WAVES * COMPACT_ITEMS];
+  __shared__ int s_tot[2 * COMPACT_WAVES * COMPACT_ITEMS];
+  __shared__ int s_base[2 * COMPACT_WAVES];
   const uint32_t* flags = a.flags;
-  compact_lists(a, [&](int t) { return flags[t] != 0u; }, s_tot);
+  const int chunk = blockIdx.x;
+  // base = number of active / stale tiles below this chunk (its start is a multiple of 4096 flags)
+  int na = 0, ns = 0;
+  const uint4* f4 = reinterpret_cast<const uint4*>(flags);
+  const int n4 = chunk * (COMPACT_CHUNK / 4);
+  for (int i = threadIdx.x; i < n4; i += COMPACT_THREADS) {
+    const uint4 v = f4[i];
+    na += (int)(v.x & 1u) + (int)(v.y & 1u) + (int)(v.z & 1u) + (int)(v.w & 1u);
+    ns += (int)((v.x & 3u) == 2u) + (int)((v.y & 3u) == 2u) + (int)((v.z & 3u) == 2u) + (int)((v.w & 3u) == 2u);
+  }
+  int base_act = 0, base_st = 0;
+  if (chunk > 0) {      // uniform over the block
+    na = wave_sum(na);
+    ns = wave_sum(ns);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) s_base[wave] = na, s_base[COMPACT_WAVES + wave] = ns;
+    __syncthreads();
+#pragma unroll
+    for (int wv = 0; wv < COMPACT_WAVES; ++wv) base_act += s_base[wv], base_st += s_base[COMPACT_WAVES + wv];
+  }
+  compact_lists(a, [&](int t) { return flags[t]; }, chunk, base_act, base_st, chunk == (int)gridDim.x - 1, s_tot);
 }
 
 // Planes of at most SMALL_CAP tiles (the 33x44 plane of a 264x352 frame: 30 tiles): footprint
@@ -266,18 +286,20 @@ __global__ __launch_bounds__(COMPACT_THREADS) void k_compact_tiles(BuildArgs a) 
 constexpr int SMALL_CAP = 32;
 
 __global__ __launch_bounds__(COMPACT_THREADS) void k_build_small(BuildArgs a) {
-  __shared__ int s_tot[COMPACT_WAVES * COMPACT_ITEMS];
+  __shared__ int s_tot[2 * COMPACT_WAVES * COMPACT_ITEMS];
   __shared__ unsigned s_flag[SMALL_CAP];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   for (int tile = wave; tile < a.cap; tile += COMPACT_WAVES) {
+    const uint32_t old = a.flags[tile];
     const bool any = tile_footprint(a, tile, lane);
     if (lane == 0) {
-      s_flag[tile] = any ? 1u : 0u;
-      a.flags[tile] = any ? 1u : 0u;
+      const uint32_t f = next_flag(old, any);
+      s_flag[tile] = f;
+      a.flags[tile] = f;
     }
   }
   __syncthreads();
-  compact_lists(a, [&](int t) { return s_flag[t] != 0u; }, s_tot);
+  compact_lists(a, [&](int t) { return s_flag[t]; }, 0, 0, 0, true, s_tot);
 }
 
 extern "C" int mie_build_mask_tiles(const uint8_t* in_mask, const uint8_t* in_mask2,
@@ -316,6 +338,12 @@ extern "C" int mie_build_mask_tiles(const uint8_t* in_mask, const uint8_t* in_ma
   } else {
     MIE_REQUIRE(false, MIE_ERR_UNSUPPORTED, "mie_build_mask_tiles: unknown footprint %d", foot);
   }
+  // A lane reads the mask bytes of its footprint while other lanes write theirs: only the 1x1 stride-1
+  // identity footprint (own pixel in, own pixel out) may be built in place.
+  const bool identity = foot == MIE_FOOT_CONV && k == 1 && stride == 1 && pad == 0;
+  MIE_REQUIRE(identity || ((const uint8_t*)out->pixmask != in_mask && (const uint8_t*)out->pixmask != in_mask2),
+              MIE_ERR_INVALID_ARG,
+              "mie_build_mask_tiles: out->pixmask aliases an input mask (allowed for the 1x1 stride-1 footprint only)");
   BuildArgs a;
   a.in = in_mask; a.in2 = in_mask2;
   a.n = out->n; a.h_in = h_in; a.w_in = w_in;
@@ -332,6 +360,7 @@ extern "C" int mie_build_mask_tiles(const uint8_t* in_mask, const uint8_t* in_ma
   hipLaunchKernelGGL(k_mask_footprint, dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
   rc = mie_check_launch("mie_build_mask_tiles");
   if (rc != MIE_OK) return rc;
-  hipLaunchKernelGGL(k_compact_tiles, dim3(1), dim3(COMPACT_THREADS), 0, (hipStream_t)stream, a);
+  hipLaunchKernelGGL(k_compact_tiles, dim3((unsigned)mie_div_up(a.cap, COMPACT_CHUNK)), dim3(COMPACT_THREADS), 0,
+                     (hipStream_t)stream, a);
   return mie_check_launch("mie_build_mask_tiles");
 }

@@ -27,11 +27,20 @@ from .mask_incr_functional import IncrementReserve, _unpack
 from .mask_incr_modules import (_IncrBuffers, nnAddIncr, nnBatchNorm2dIncr, nnConvIncr,
                                 nnConvTranspose2dIncr, nnReluIncr, nnReservedActivation,
                                 nnReservedMultiplication, nnSigmoidIncr, nnTanhIncr,
-                                nnUpsample2xIncr, activation_kind)
+                                nnUpsample2xIncr, activation_kind, activation_op)
 
 
 def _mask_of(x_incr):
     return x_incr[1] if len(x_incr) > 1 else None
+
+
+def _same_mask(a, b) -> bool:
+    """Whether two mask slots name the same pixel mask in memory (None = all active on both sides)."""
+    if a is None or b is None:
+        return a is None and b is None
+    pa = a.pixmask if isinstance(a, TileMask) else a
+    pb = b.pixmask if isinstance(b, TileMask) else b
+    return pa.data_ptr() == pb.data_ptr() and pa.shape == pb.shape and pa.dtype == pb.dtype
 
 
 class ConvLayerIncr(nn.Module):
@@ -43,7 +52,7 @@ class ConvLayerIncr(nn.Module):
         bias = False if norm == 'BN' else True
         self.conv2d = nnConvIncr(in_channels, out_channels, kernel_size, stride, padding, bias=bias)
         if activation is not None:
-            op = getattr(torch, activation, 'relu')
+            op = activation_op(activation)
             self.activation = nnReservedActivation(op)
         else:
             self.activation = None
@@ -114,12 +123,64 @@ class ConvLSTMIncr(nn.Module, _IncrBuffers):
         prev_h_incr = prev_c_incr = None
         if prev_state_incr is not None:
             prev_h_incr, prev_c_incr = prev_state_incr
-            if _mask_of(prev_c_incr) is not _mask_of(prev_h_incr):
-                # the tile set of the gates conv must cover the cell delta too
-                prev_h_incr = [prev_h_incr[0], None]
         if self.fused:
             return self._forward_fused(input_incr, prev_h_incr, prev_c_incr)
         return self._forward_chain(input_incr, prev_h_incr, prev_c_incr)
+
+    # -- state buffers ---------------------------------------------------------------------------
+    # The fused forms return the state deltas in buffers this module owns ([dh, ts], [dc, ts]).  A caller
+    # may feed them back as the next step's previous state, and that step reads them (with a 3x3 halo, and
+    # their pixel mask for the tile-set build) while it writes its own state: it must write elsewhere.  Two
+    # sets of (dh, dc, tile set) are kept and a step takes the one its inputs do not live in.  Each set
+    # has its own stale list, relative to the last step that wrote it, so every buffer stays a clean delta.
+    @staticmethod
+    def _ptrs_of(*state_incrs):
+        used = set()
+        for s_ in state_incrs:
+            if s_ is None:
+                continue
+            used.add(s_[0].data_ptr())
+            m = _mask_of(s_)
+            if isinstance(m, TileMask):
+                used.update((m.tiles.data_ptr(), m.pixmask.data_ptr()))
+            elif torch.is_tensor(m):
+                used.add(m.data_ptr())
+        return used
+
+    def _state_slot(self, prev_h_incr, prev_c_incr) -> int:
+        used = self._ptrs_of(prev_h_incr, prev_c_incr)
+        owned = self.__dict__.setdefault("_slot_ptrs", {})
+        for slot in (0, 1):
+            if not (owned.get(slot, set()) & used):
+                return slot
+        raise RuntimeError("ConvLSTMIncr: the previous state mixes buffers of both of this cell's state sets")
+
+    def _own_slot(self, slot, dh, dc, ts):
+        self.__dict__.setdefault("_slot_ptrs", {})[slot] = {
+            dh.data_ptr(), dc.data_ptr(), ts.tiles.data_ptr(), ts.pixmask.data_ptr()}
+
+    def _cover_prev_c(self, prev_h_incr, prev_c_incr):
+        """The tile set of the gates conv is built from the masks of its two inputs; it must also cover the
+        active pixels of the previous-cell delta.  Returns the mask to build with in place of the hidden
+        one: the hidden mask itself when the cell delta has the same one (the usual case: both come from
+        one earlier step), else the union of the two (all active if either is unmasked)."""
+        if prev_c_incr is None:
+            return None if prev_h_incr is None else _mask_of(prev_h_incr)
+        mh = None if prev_h_incr is None else _mask_of(prev_h_incr)
+        mc = _mask_of(prev_c_incr)
+        if prev_h_incr is not None and _same_mask(mh, mc):
+            return mh
+        if mc is None or (prev_h_incr is not None and mh is None):
+            return None
+        c = ops.as_nhwc(prev_c_incr[0])
+        pc = ops.pixel_mask_of(mc, c)
+        if prev_h_incr is None:
+            return pc
+        n, _, h, w = c.shape
+        ph = ops.pixel_mask_of(mh, c)
+        union = self._tile_set("prev_union", n, h, w, c.device)
+        ops.build_mask_tiles(ph, pc, n, h, w, _lib.FOOT_CONV, 1, 1, 0, union)
+        return union
 
     # -- gates conv and gate chain in one kernel ------------------------------------------------
     def _gates_filter(self):
@@ -142,6 +203,22 @@ class ConvLSTMIncr(nn.Module, _IncrBuffers):
                 and self.input_size % chunk == 0 and (not hidden_present or self.hidden_size % chunk == 0)
                 and self.Gates.path != _lib.PATH_VALU)
 
+    def _gates_tile_set(self, name, x, pix, prev_h_incr, prev_c_incr, pix2):
+        """Tile set of the gates conv for this step: footprint of the input mask and of the previous-state
+        masks (the hidden delta is read through its OWN mask pix2; the build may use a wider one)."""
+        cover = self._cover_prev_c(prev_h_incr, prev_c_incr)
+        n, _, h, w = x.shape
+        ts = self.Gates._tile_set(name, n, h, w, x.device)
+        if prev_h_incr is None and prev_c_incr is None:
+            m1, m2 = pix, None
+        elif pix is None or cover is None:
+            m1 = m2 = None
+        else:
+            m1, m2 = pix, ops.pixel_mask_of(cover, x)
+        k = self.kernel_size
+        ops.build_mask_tiles(m1, m2, n, h, w, _lib.FOOT_CONV, k, 1, k // 2, ts)
+        return ts
+
     def _forward_one_kernel(self, input_incr, prev_h_incr, prev_c_incr):
         if self.Gates.use_kf:
             input_incr = self.Gates.kf(input_incr)
@@ -151,9 +228,12 @@ class ConvLSTMIncr(nn.Module, _IncrBuffers):
             x2, pix2, _ = _unpack(prev_h_incr)
         n, _, h, w = x.shape
         hid = self.hidden_size
-        ts = self.Gates._conv_tile_set("gates", x, pix, x2, pix2, 3, 1, 1)
-        dh = self._delta_buf("h", (n, hid, h, w), x.device, x.dtype)
-        dc = self._delta_buf("c", (n, hid, h, w), x.device, x.dtype)
+        slot = self._state_slot(prev_h_incr, prev_c_incr)
+        sfx = "" if slot == 0 else "_b"
+        ts = self._gates_tile_set("gates" + sfx, x, pix, prev_h_incr, prev_c_incr, pix2)
+        dh = self._delta_buf("h" + sfx, (n, hid, h, w), x.device, x.dtype)
+        dc = self._delta_buf("c" + sfx, (n, hid, h, w), x.device, x.dtype)
+        self._own_slot(slot, dh, dc, ts)
         cp = cpm = None
         if prev_c_incr is not None:
             cp, cpm, _ = _unpack(prev_c_incr)
@@ -170,11 +250,23 @@ class ConvLSTMIncr(nn.Module, _IncrBuffers):
                 raise RuntimeError("ConvLSTMIncr: the reservoirs were refreshed for the one-kernel form, which "
                                    "does not take this input (dtype / previous hidden state); refresh again")
             return self._forward_one_kernel(input_incr, prev_h_incr, prev_c_incr)
-        gates, ts = self.Gates(input_incr, prev_h_incr)
-        n, _, h, w = gates.shape
+        slot = self._state_slot(prev_h_incr, prev_c_incr)
+        sfx = "" if slot == 0 else "_b"
+        if self.Gates.use_kf:
+            input_incr = self.Gates.kf(input_incr)
+        x, pix, _ = _unpack(input_incr)
+        x2 = pix2 = None
+        if prev_h_incr is not None:
+            x2, pix2, _ = _unpack(prev_h_incr)
+        n, _, h, w = x.shape
         hid = self.hidden_size
-        dh = self._delta_buf("h", (n, hid, h, w), gates.device, gates.dtype)
-        dc = self._delta_buf("c", (n, hid, h, w), gates.device, gates.dtype)
+        ts = self._gates_tile_set("out" + sfx, x, pix, prev_h_incr, prev_c_incr, pix2)
+        gates = self.Gates._delta_buf("out", (n, 4 * hid, h, w), x.device, x.dtype)
+        k = self.kernel_size
+        ops.conv_masked(x, pix, x2, pix2, self.Gates.conv2d_weights, k, 1, k // 2, ts, gates, path=self.Gates.path)
+        dh = self._delta_buf("h" + sfx, (n, hid, h, w), gates.device, gates.dtype)
+        dc = self._delta_buf("c" + sfx, (n, hid, h, w), gates.device, gates.dtype)
+        self._own_slot(slot, dh, dc, ts)
         cp = cpm = None
         if prev_c_incr is not None:
             cp, cpm, _ = _unpack(prev_c_incr)
@@ -358,7 +450,7 @@ class TransposedConvLayerIncr(nn.Module):
             in_channels, out_channels, kernel_size, stride=2, padding=padding, output_padding=1, bias=bias)
         self.activation = None
         if activation is not None:
-            op = getattr(torch, activation, 'relu')
+            op = activation_op(activation)
             self.activation = nnReservedActivation(op)
         self.norm = norm
         if norm == 'BN':
@@ -402,7 +494,7 @@ class UpsampleConvLayerIncr(nn.Module):
         bias = False if norm == 'BN' else True
         self.conv2d = nnConvIncr(in_channels, out_channels, kernel_size, stride, padding, bias=bias)
         if activation is not None:
-            op = getattr(torch, activation, 'relu')
+            op = activation_op(activation)
             self.activation = nnReservedActivation(op)
         else:
             self.activation = None
@@ -461,7 +553,7 @@ class BaseUNetIncr(nn.Module):
         assert self.num_output_channels > 0
         self.encoder_input_sizes = [self.base_num_channels * pow(2, i) for i in range(self.num_encoders)]
         self.encoder_output_sizes = [self.base_num_channels * pow(2, i + 1) for i in range(self.num_encoders)]
-        op = getattr(torch, activation, 'relu')
+        op = activation_op(activation)
         self.activation = nnReservedActivation(op, refine_mask=not fuse)
 
     def build_resblocks(self):

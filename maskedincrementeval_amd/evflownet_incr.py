@@ -31,7 +31,7 @@ from .masked_types import DenseT, Masked, TileMask
 from .mask_incr_functional import _unpack
 from .mask_incr_modules import (_IncrBuffers, nnAddIncr, nnBatchNorm2dIncr, nnConvIncr,
                                 nnConvTranspose2dIncr, nnReservedActivation, nnReservedMultiplication,
-                                nnSigmoidIncr, nnTanhIncr, nnUpsample2xIncr, activation_kind)
+                                nnSigmoidIncr, nnTanhIncr, nnUpsample2xIncr, activation_kind, activation_op)
 
 
 def skip_concat(x1, x2):
@@ -136,7 +136,12 @@ class ConvGRUIncr(nn.Module, _IncrBuffers):
         if (self.fuse and self.stacked and prev_state is None and not self.update_gate.use_kf
                 and not self.out_gate.use_kf and self.sigmoid1.in_res.reservoir is not None):
             new_state = self._forward_stacked(input_incr)
+            self.__dict__["_mult_stale"] = True       # self.mult's reservoirs have missed this step
             return new_state, new_state
+        if self.__dict__.get("_mult_stale", False):
+            raise RuntimeError("ConvGRUIncr: steps since the last refresh ran the one-conv form (no previous "
+                               "state), which does not maintain the reservoirs of the module-by-module form; "
+                               "refresh before switching to it")
         update = self._gate(self.update_gate, self.sigmoid1, input_incr, prev_state)
         out_inputs = self._gate(self.out_gate, self.tanh, input_incr, prev_state)
         if prev_state is None:
@@ -148,6 +153,7 @@ class ConvGRUIncr(nn.Module, _IncrBuffers):
 
     def forward_refresh_reservoirs(self, x, prev_state):
         self._reset_incr()
+        self.__dict__["_mult_stale"] = False
         zero_state = prev_state is None
         if zero_state:
             state_size = [x.shape[0], self.hidden_size] + list(x.shape[2:])
@@ -179,8 +185,8 @@ class ConvLayerIncr(nn.Module):
             nn.init.uniform_(self.conv2d.weight, -w_scale, w_scale)
             nn.init.zeros_(self.conv2d.bias)
         self.activation = None
-        if activation is not None and hasattr(torch, activation):
-            self.activation = nnReservedActivation(getattr(torch, activation), refine_mask=not fuse)
+        if activation is not None:
+            self.activation = nnReservedActivation(activation_op(activation), refine_mask=not fuse)
         self.norm = norm
         if norm == "BN":
             self.norm_layer = nnBatchNorm2dIncr(out_channels, momentum=BN_momentum)
@@ -240,9 +246,9 @@ class ResidualBlockIncr(nn.Module):
         bias = False if norm == "BN" else True
         self.conv1 = nnConvIncr(in_channels, out_channels, kernel_size=3, stride=stride, padding=1, bias=bias)
         self.activation = self.activation2 = None
-        if activation is not None and hasattr(torch, activation):
-            self.activation = nnReservedActivation(getattr(torch, activation), refine_mask=not fuse)
-            self.activation2 = nnReservedActivation(getattr(torch, activation), refine_mask=not fuse)
+        if activation is not None:
+            self.activation = nnReservedActivation(activation_op(activation), refine_mask=not fuse)
+            self.activation2 = nnReservedActivation(activation_op(activation), refine_mask=not fuse)
         self.norm = norm
         if norm == "BN":
             self.bn1 = nnBatchNorm2dIncr(out_channels, momentum=BN_momentum)
@@ -314,7 +320,7 @@ class UpsampleConvLayerIncr(nn.Module):
         self.conv2d = nnConvIncr(in_channels, out_channels, kernel_size, stride, padding, bias=bias)
         self.activation = None
         if activation is not None:
-            self.activation = nnReservedActivation(getattr(torch, activation), refine_mask=not fuse)
+            self.activation = nnReservedActivation(activation_op(activation), refine_mask=not fuse)
         self.norm = norm
         if norm == "BN":
             self.norm_layer = nnBatchNorm2dIncr(out_channels)
@@ -441,7 +447,7 @@ class TransposedConvLayerIncr(nn.Module):
                                                        padding=padding, output_padding=1, bias=True)
         self.activation = None
         if activation is not None:
-            self.activation = nnReservedActivation(getattr(torch, activation), refine_mask=not fuse)
+            self.activation = nnReservedActivation(activation_op(activation), refine_mask=not fuse)
         self.cat = nnCatIncr()
         self.fuse = fuse
 

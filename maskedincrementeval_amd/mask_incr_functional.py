@@ -99,7 +99,9 @@ def IncrPointwiseMultiply(x1_incr: Masked, x1: IncrementReserve, x2_incr: Masked
     d1, p1, t1 = _unpack(x1_incr)
     d2, p2, t2 = _unpack(x2_incr)
     n, c, h, w = d1.shape
-    if t1 is not None and t1.shares_tiles_with(t2):
+    # two refined views of one parent share the tile list but not the pixel mask: the kernel gates on ONE pixel
+    # mask, so the operands' own tile set serves only when it is the same mask; else the union is built
+    if t1 is not None and t1.shares_tiles_with(t2) and t1.pixmask.data_ptr() == t2.pixmask.data_ptr():
         ts = t1
     else:
         ts = TileMask(n, h, w, d1.device)

@@ -184,7 +184,7 @@ class nnReservedMultiplication(PointwiseMultiplyIncr):
         if self.x1_res.reservoir is None or self.x2_res.reservoir is None:
             raise RuntimeError("nnReservedMultiplication: call forward_refresh_reservoirs first")
         n, c, h, w = d1.shape
-        if t1 is not None and t1.shares_tiles_with(t2) and t1.pixmask is t2.pixmask:
+        if t1 is not None and t1.shares_tiles_with(t2) and t1.pixmask.data_ptr() == t2.pixmask.data_ptr():
             ts = t1
         else:
             ts = self._tile_set("union", n, h, w, d1.device)
@@ -223,6 +223,22 @@ def activation_kind(op) -> Tuple[int, float]:
         return _lib.ACT_LEAKY_RELU, float(slope)
     raise NotImplementedError(
         "incremental activation for %r has no kernel (supported: relu, leaky_relu, sigmoid, tanh)" % (op,))
+
+
+_ACTIVATION_OPS = {"relu": torch.relu, "sigmoid": torch.sigmoid, "tanh": torch.tanh}
+
+
+def activation_op(name: str):
+    """Unary torch callable for an activation named in a layer constructor ('relu', 'sigmoid', 'tanh',
+    'leaky_relu').  The reference looks the name up with getattr(torch, name, 'relu')
+    (incr_modules/e2depth_incr.py:19), which turns an unknown name into the *string* 'relu' and fails at the
+    first forward; here an unknown name raises at construction."""
+    if name == "leaky_relu":
+        return leaky_relu_op()
+    try:
+        return _ACTIVATION_OPS[name]
+    except KeyError:
+        raise ValueError("unknown activation %r (known: %s, leaky_relu)" % (name, ", ".join(sorted(_ACTIVATION_OPS)))) from None
 
 
 def leaky_relu_op(negative_slope: float = 0.01):

@@ -45,8 +45,8 @@ def test_tile_capacity(mie_lib):
 
 def _fake_tileset(n=1, h=16, w=16, null=None):
     """Tile set with non-NULL but never dereferenced host pointers (validation only)."""
-    buf = ctypes.create_string_buffer(4096)
-    p = ctypes.addressof(buf)
+    buf = ctypes.create_string_buffer(4096 + 16)
+    p = (ctypes.addressof(buf) + 15) & ~15
     vals = dict(pixmask=p, tiles=p, stale=p, counts=p, flags=p)
     if null:
         vals[null] = None
@@ -66,27 +66,27 @@ def test_invalid_arguments_return_status_not_abort(mie_lib):
     assert "tile set is NULL" in err()
     # NULL input pointer
     assert mie_lib.mie_conv_masked(None, None, 16, None, None, 0, 16, 16, p, None, 16, 3, 1, 1, 32,
-                                   ctypes.byref(ts), p, None, None, 0, 0.0, 0, 0, None) == -1
+                                   ctypes.byref(ts), p + 1024, None, None, 0, 0.0, 0, 0, None) == -1
     # unsupported kernel size and stride (the reference throws std::logic_error, ext_conv.cu:366)
     assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 16, 16, p, None, 16, 4, 1, 1, 32,
-                                   ctypes.byref(ts), p, None, None, 0, 0.0, 0, 0, None) == -2
+                                   ctypes.byref(ts), p + 1024, None, None, 0, 0.0, 0, 0, None) == -2
     assert "kernel size 4" in err()
     assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 16, 16, p, None, 16, 3, 3, 1, 32,
-                                   ctypes.byref(ts), p, None, None, 0, 0.0, 0, 0, None) == -2
+                                   ctypes.byref(ts), p + 1024, None, None, 0, 0.0, 0, 0, None) == -2
     # output geometry mismatch
     assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 20, 16, p, None, 16, 3, 1, 1, 32,
-                                   ctypes.byref(ts), p, None, None, 0, 0.0, 0, 0, None) == -1
+                                   ctypes.byref(ts), p + 1024, None, None, 0, 0.0, 0, 0, None) == -1
     assert "tile set is" in err()
     # misaligned pointer
     assert mie_lib.mie_conv_masked(p + 4, None, 16, None, None, 0, 16, 16, p, None, 16, 3, 1, 1, 32,
-                                   ctypes.byref(ts), p, None, None, 0, 0.0, 0, 0, None) == -1
+                                   ctypes.byref(ts), p + 1024, None, None, 0, 0.0, 0, 0, None) == -1
     assert "aligned" in err()
     # MFMA path on a shape it cannot take
     assert mie_lib.mie_conv_masked(p, None, 24, None, None, 0, 16, 16, p, None, 24, 3, 1, 1, 32,
-                                   ctypes.byref(ts), p, None, None, 0, 0.0, _lib.PATH_MFMA, 0, None) == -2
+                                   ctypes.byref(ts), p + 1024, None, None, 0, 0.0, _lib.PATH_MFMA, 0, None) == -2
     # MFMA path without the matrix-core filter copy
     assert mie_lib.mie_conv_masked(p, None, 32, None, None, 0, 16, 16, p, None, 32, 3, 1, 1, 32,
-                                   ctypes.byref(ts), p, None, None, 0, 0.0, _lib.PATH_MFMA, 0, None) == -2
+                                   ctypes.byref(ts), p + 1024, None, None, 0, 0.0, _lib.PATH_MFMA, 0, None) == -2
     assert "mie_pack_filter" in err()
     # filter packing: cin must be a multiple of 8, buffers distinct
     assert mie_lib.mie_pack_filter(p, 12, 3, 32, p + 4096, 0, None) == -2
@@ -96,10 +96,30 @@ def test_invalid_arguments_return_status_not_abort(mie_lib):
     assert mie_lib.mie_pack_filter(p, 16, 3, 32, p + 4096, 7, None) == -2      # unknown dtype
     # activation without a reservoir
     assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 16, 16, p, None, 16, 3, 1, 1, 32,
-                                   ctypes.byref(ts), p, None, None, _lib.ACT_RELU, 0.0, 0, 0, None) == -1
+                                   ctypes.byref(ts), p + 1024, None, None, _lib.ACT_RELU, 0.0, 0, 0, None) == -1
     # channels beyond the filter
     assert mie_lib.mie_conv_masked(p, None, 16, p, None, 16, 16, 16, p, None, 16, 3, 1, 1, 32,
+                                   ctypes.byref(ts), p + 1024, None, None, 0, 0.0, 0, 0, None) == -1
+    # aliasing that would make workgroups race: input == output for k > 1 (allowed for 1x1), an input mask that is
+    # the output tile set's pixel mask, a mask build in place with a footprint wider than the pixel itself
+    assert mie_lib.mie_conv_masked(p, None, 16, None, None, 0, 16, 16, p + 2048, None, 16, 3, 1, 1, 32,
                                    ctypes.byref(ts), p, None, None, 0, 0.0, 0, 0, None) == -1
+    assert "alias" in err()
+    assert mie_lib.mie_conv_masked(p + 512, None, 16, p, None, 16, 16, 16, p + 2048, None, 32, 3, 1, 1, 32,
+                                   ctypes.byref(ts), p, None, None, 0, 0.0, 0, 0, None) == -1
+    assert "alias" in err()
+    assert mie_lib.mie_conv_masked(p, ts.pixmask, 16, None, None, 0, 16, 16, p + 2048, None, 16, 3, 1, 1, 32,
+                                   ctypes.byref(ts), p + 1024, None, None, 0, 0.0, 0, 0, None) == -1
+    assert "pixel mask" in err()
+    assert mie_lib.mie_conv_gates_masked(p, None, 32, p + 512, None, 32, 16, 16, p + 2048, p + 2048, 64, 8,
+                                         ctypes.byref(ts), p + 1024, None, None, p + 1024, p + 1024, p + 512,
+                                         p + 1536, 0, None) == -1
+    assert "h_delta" in err()
+    assert mie_lib.mie_build_mask_tiles(ts.pixmask, None, 16, 16, _lib.FOOT_CONV, 3, 1, 1, ctypes.byref(ts), None) == -1
+    assert "aliases" in err()
+    assert mie_lib.mie_build_mask_tiles(p + 64, ts.pixmask, 16, 16, _lib.FOOT_CONV, 3, 1, 1, ctypes.byref(ts), None) == -1
+    up, keep_up = _fake_tileset(h=32, w=32)
+    assert mie_lib.mie_build_mask_tiles(up.pixmask, None, 16, 16, _lib.FOOT_UP2X, 0, 0, 0, ctypes.byref(up), None) == -1
     # workspace of the split form: misaligned, sized without a pointer, aliasing the output
     ws_call = lambda ws, nbytes: mie_lib.mie_conv_masked_ws(p, None, 16, None, None, 0, 16, 16, p + 2048, None, 16, 3, 1, 1, 32,
                                                             ctypes.byref(ts), p + 1024, None, None, 0, 0.0, 0, 0, ws, nbytes, None)

@@ -290,15 +290,67 @@ def test_convlstm_with_previous_state_deltas(cin, hid):
         h_d, c_d = cell.forward_refresh_reservoirs(_cl(x0), (_cl(h0), _cl(c0)))
     h_r, c_r = ref.refresh(x0, (h0, c0))
     _close(h_d, h_r, "refresh h"), _close(c_d, c_r, "refresh c")
-    for step in range(3):
+    for step in range(4):
         d, m = gaussian_delta(n, cin, h, w, 0.08, 0.3, seed=6300 + step)
         dhp, mh = gaussian_delta(n, hid, h, w, 0.05, 0.2, seed=6400 + step)
-        dcp, _ = gaussian_delta(n, hid, h, w, 0.05, 0.2, seed=6400 + step)      # same mask as the hidden delta
+        if step < 2:
+            # hidden and cell deltas under ONE mask (one device tensor, or two equal copies: the cell then
+            # builds their union): the masked previous-hidden path, pix2 + union tile set
+            dcp, _ = gaussian_delta(n, hid, h, w, 0.05, 0.2, seed=6400 + step)
+            mh_dev = mh.to(DEV)
+            mc_dev = mh_dev if step == 0 else mh.to(DEV)
+            mc = mh
+        else:
+            # different masks for the two: the tile set must cover the union, each delta is read under its own
+            dcp, mc = gaussian_delta(n, hid, h, w, 0.04, 0.2, seed=6500 + step)
+            mh_dev, mc_dev = mh.to(DEV), mc.to(DEV)
+        # inactive pixels of the previous-state deltas are never read
+        nan = float("nan")
+        dhp_dev = _cl(torch.where(mh.bool().expand_as(dhp), dhp, torch.full_like(dhp, nan)))
+        dcp_dev = _cl(torch.where(mc.bool().expand_as(dcp), dcp, torch.full_like(dcp, nan)))
+        if step == 3:      # tile masks in the mask slots
+            tmh, tmc = TileMask(n, h, w, DEV), TileMask(n, h, w, DEV)
+            ops.build_mask_tiles(mh_dev, None, n, h, w, _lib.FOOT_CONV, 1, 1, 0, tmh)
+            ops.build_mask_tiles(mc_dev, None, n, h, w, _lib.FOOT_CONV, 1, 1, 0, tmc)
+            mh_dev, mc_dev = tmh, tmc
         with torch.no_grad():
-            dh, dc = cell([_cl(d), m.to(DEV)], ([_cl(dhp), mh.to(DEV)], [_cl(dcp), mh.to(DEV)]))
+            dh, dc = cell([_cl(d), m.to(DEV)], ([dhp_dev, mh_dev], [dcp_dev, mc_dev]))
         torch.cuda.synchronize()
         dh_r, dc_r = ref.incr(d, (dhp, dcp))
+        assert torch.isfinite(dh[0]).all() and torch.isfinite(dc[0]).all()
         _close(dh[0], dh_r, "dh %d" % step), _close(dc[0], dc_r, "dc %d" % step)
+        if step >= 2:      # the tile set is sparse (not "every tile") and covers the cell delta's pixels
+            assert int(dh[1].counts[0].item()) < dh[1].capacity
+            assert torch.all(dh[1].pixmask.cpu() >= mc)
+
+
+@pytest.mark.parametrize("cin,hid", [(16, 16), (32, 32)])
+def test_convlstm_state_deltas_fed_back(cin, hid):
+    # the returned [dh, ts], [dc, ts] go straight back in as the next step's previous state
+    # (forward(x, prev_states) of the reference, incr_modules/e2depth_incr.py:79,98): the cell must not
+    # write the buffers and the tile set it is reading
+    n, h, w = 1, 40, 48
+    cell = seed_module_(ConvLSTMIncr(cin, hid, 3, fused=True), 71).to(DEV).eval()
+    ref = io.ConvLSTMOracle(cell.Gates.weight.detach().cpu(), cell.Gates.bias.detach().cpu(), hid)
+    g = torch.Generator().manual_seed(72)
+    x0 = torch.randn(n, cin, h, w, generator=g) * 0.5
+    with torch.no_grad():
+        cell.forward_refresh_reservoirs(_cl(x0), None)
+    ref.refresh(x0, None)
+    state, state_r = None, None
+    for step in range(6):
+        d, m = gaussian_delta(n, cin, h, w, 0.04, 0.3, seed=7300 + step)
+        with torch.no_grad():
+            state = cell([_cl(d), m.to(DEV)], state)
+        torch.cuda.synchronize()
+        state_r = ref.incr(d, state_r)
+        _close(state[0][0], state_r[0], "dh %d" % step), _close(state[1][0], state_r[1], "dc %d" % step)
+        # clean delta: zero outside the active pixels of the tile set it is returned with
+        for dlt, ts in state:
+            assert torch.count_nonzero(dlt * (1 - ts.pixmask.float())) == 0
+        if step > 0:
+            assert state[0][0].data_ptr() != prev_ptr      # the two state sets alternate
+        prev_ptr = state[0][0].data_ptr()
 
 
 @pytest.mark.parametrize("plan_first", [False, True])

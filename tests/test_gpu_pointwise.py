@@ -107,6 +107,41 @@ def test_product_rule(n, c, h, w):
     assert torch.equal(g1.cpu(), before)
 
 
+@pytest.mark.parametrize("form", ["functional", "module"])
+def test_product_of_two_refined_views_of_one_tile_set(form):
+    # Two activations applied under ONE tile set each emit a refined pixel mask of their own (a view that
+    # shares the tile list).  The product must cover the union of the two masks: a pixel active in the
+    # second operand only contributes R1 * d2.
+    from maskedincrementeval_amd import mask_incr_functional as mf
+    from maskedincrementeval_amd import mask_incr_modules as mm
+    n, c, h, w = 1, 8, 24, 40
+    parent = TileMask(n, h, w, DEV)
+    base = torch.zeros(n, 1, h, w, dtype=torch.uint8)
+    base[:, :, 2:20, 3:33] = 1
+    ops.build_mask_tiles(base.to(DEV), None, n, h, w, _lib.FOOT_CONV, 1, 1, 0, parent)
+    m1, m2 = torch.zeros_like(base), torch.zeros_like(base)
+    m1[:, :, 2:10, 3:20] = 1            # view 1: upper left part
+    m2[:, :, 6:20, 12:33] = 1           # view 2: lower right part, overlapping view 1
+    v1, v2 = parent.with_pixmask(m1.to(DEV)), parent.with_pixmask(m2.to(DEV))
+    assert v1.shares_tiles_with(v2)
+    d1 = _randn(n, c, h, w, seed=31) * m1.float()
+    d2 = _randn(n, c, h, w, seed=32) * m2.float()
+    r1, r2 = _randn(n, c, h, w, seed=33), _randn(n, c, h, w, seed=34)
+    want = (d2 + r2) * d1 + r1 * d2
+    if form == "functional":
+        R1, R2 = mf.IncrementReserve(_dev(r1)), mf.IncrementReserve(_dev(r2))
+        out, ts = mf.IncrPointwiseMultiply([_dev(d1), v1], R1, [_dev(d2), v2], R2)
+    else:
+        mod = mm.nnReservedMultiplication()
+        mod.forward_refresh_reservoirs(_dev(r1), _dev(r2))
+        out, ts = mod([_dev(d1), v1], [_dev(d2), v2])
+    torch.cuda.synchronize()
+    _close(out, want, "product under the union of two refined masks")
+    only2 = (m2.bool() & ~m1.bool()).expand_as(d1)
+    assert torch.count_nonzero(out.cpu()[only2]) > 0            # the R1 * d2 term is there
+    assert torch.equal(ts.pixmask.cpu(), m1 | m2)
+
+
 def test_sum_of_deltas():
     n, c, h, w = 2, 32, 21, 35
     ts = TileMask(n, h, w, DEV)
