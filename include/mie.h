@@ -471,6 +471,49 @@ int mie_conv_gates_masked(const void* x, const uint8_t* xmask, int c1,
                           void* c_delta, int dtype, void* stream);
 
 /*
+ * Dense refresh of a ConvLSTM cell after its gates conv: gates_res
+ * ([n,h,w,4*hid] fp32) holds the gate pre-activations mie_conv_refresh wrote --
+ * in the order [in | remember | out | cell] x hid, or (interleaved != 0) in the
+ * gate-interleaved order of mie_conv_gates_masked.  Per (pixel, hidden channel):
+ *   cell = sigmoid(in) * tanh(cell_gate) + sigmoid(remember) * prev_c
+ *   h_out = sigmoid(out) * tanh(cell);  c_out = cell
+ *   cprev_res = prev_c;  cell_res = cell      (the reservoirs of the gate chain)
+ * prev_c ([n,h,w,hid], element type `dtype`) may be NULL = zero state, and may
+ * be c_out (the previous refresh's cell state, updated in place); h_out / c_out
+ * are dense tensors of that type.
+ * Replaces: the state math of ConvLSTMIncr.forward_refresh_reservoirs
+ * (incr_modules/e2depth_incr.py:144-166) and its reservoir clones
+ * (incr_modules/mask_incr_functional.py:46-48).
+ */
+int mie_convlstm_gates_refresh(const float* gates_res, int interleaved,
+                               const void* prev_c, float* cprev_res,
+                               float* cell_res, void* h_out, void* c_out, int n,
+                               int h, int w, int hid, int dtype, void* stream);
+
+/*
+ * Dense refresh of a ConvGRU cell after its gate convs: update = sigmoid(update
+ * gate), cand = tanh(out gate), both dense [n,h,w,hid] of type `dtype` as the
+ * fused conv refresh returns them; prev_state may be NULL = zero.
+ *   new_state = prev_state + (cand - prev_state) * update
+ *   diff_res = cand - prev_state;  update_res = update   (optional: the cached
+ *   operands of the incremental product, nnReservedMultiplication)
+ * new_state may be prev_state (updated in place).
+ * Replaces: incr_modules/evflownet_incr.py:84-96.
+ */
+int mie_convgru_gates_refresh(const void* update, const void* cand,
+                              const void* prev_state, float* diff_res,
+                              float* update_res, void* new_state, int n, int h,
+                              int w, int hid, int dtype, void* stream);
+
+/*
+ * out[i] = a[i] * b[i] for count dense elements of type `dtype` (out may alias a
+ * or b): prev_state * reset in front of the candidate conv of a ConvGRU refresh
+ * (incr_modules/evflownet_incr.py:90).
+ */
+int mie_mul_dense(const void* a, const void* b, void* out, long long count,
+                  int dtype, void* stream);
+
+/*
  * Per-channel scale of a delta over the active tiles of ts: out = in * scale[c]
  * (inactive pixels of active tiles and stale tiles get zeros).  scale is fp32 [c];
  * for an eval-mode batch norm it is weight / sqrt(running_var + eps).

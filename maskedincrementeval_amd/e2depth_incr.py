@@ -292,6 +292,24 @@ class ConvLSTMIncr(nn.Module, _IncrBuffers):
         hidden = self.m3(out_gate, cell_tanh)
         return hidden, cell
 
+    def _refresh_state(self, input_, prev_c, interleaved):
+        """Dense (hidden, cell) from the gate pre-activations the conv refresh left in gates_res, and the
+        cell reservoirs of the gate chain, in one kernel."""
+        n, _, h, w = input_.shape
+        dev, hid = input_.device, self.hidden_size
+        for res in (self.cprev_res, self.cell_res):
+            r = res.reservoir
+            if r is None or tuple(r.shape) != (n, hid, h, w) or r.device != dev:
+                res.reservoir = ops.new_nhwc(n, hid, h, w, dev)
+        dt = ops.delta_torch_dtype(input_)
+        hidden = self._dense_buf("h_refresh", (n, hid, h, w), dev, dt)
+        cell = self._dense_buf("c_refresh", (n, hid, h, w), dev, dt)
+        if prev_c is not None:
+            prev_c = ops.as_nhwc(prev_c.to(dt))      # may be `cell` itself (the last refresh's state fed back)
+        ops.convlstm_gates_refresh(self.gates_res.reservoir, interleaved, prev_c, self.cprev_res.reservoir,
+                                   self.cell_res.reservoir, hidden, cell)
+        return hidden, cell
+
     def forward_refresh_reservoirs(self, input_, prev_state):
         batch_size = input_.data.size()[0]
         spatial_size = input_.data.size()[2:]
@@ -320,22 +338,10 @@ class ConvLSTMIncr(nn.Module, _IncrBuffers):
                 filt, bias = self._gates_filter()
                 self.Gates._refresh_forward(input_, None if zero_state else prev_h, path=self.Gates.path,
                                             reserve=self.gates_res, filt=filt, bias=bias)
-                g = self.gates_res.reservoir
-                n_, _, h_, w_ = g.shape
-                gv = g.permute(0, 2, 3, 1).reshape(n_, h_, w_, self.hidden_size // 8, 4, 8)
-                in_gate, remember_gate, out_gate, cell_gate = (
-                    gv[..., i, :].reshape(n_, h_, w_, self.hidden_size).permute(0, 3, 1, 2) for i in range(4))
             else:
                 self.Gates._refresh_forward(input_, None if zero_state else prev_h, path=self.Gates.path,
                                             reserve=self.gates_res)
-                in_gate, remember_gate, out_gate, cell_gate = self.gates_res.reservoir.chunk(4, 1)
-            self.cprev_res.update_reservoir(prev_c)
-            in_gate, remember_gate = torch.sigmoid(in_gate), torch.sigmoid(remember_gate)
-            out_gate, cell_gate = torch.sigmoid(out_gate), torch.tanh(cell_gate)
-            cell = in_gate * cell_gate + remember_gate * self.cprev_res.reservoir
-            self.cell_res.update_reservoir(cell)
-            hidden = out_gate * torch.tanh(cell)
-            return hidden.to(input_.dtype), cell.to(input_.dtype)
+            return self._refresh_state(input_, None if zero_state else prev_c, one_kernel)
         gates = self.Gates._refresh_forward(input_, None if zero_state else prev_h, path=self.Gates.path)
         in_gate, remember_gate, out_gate, cell_gate = gates.chunk(4, 1)
         in_gate = self.sigmoid1.forward_refresh_reservoirs(in_gate)
@@ -647,10 +653,13 @@ class UNetRecurrentIncr(BaseUNetIncr):
             x = resblock.forward_refresh_reservoirs(x)
         for i, decoder in enumerate(self.decoders):
             x = decoder.forward_refresh_reservoirs(x, blocks[self.num_encoders - i - 1])
-        summed = self.pred_add.forward_refresh_reservoirs(x, head)
-        if self.fuse and self.norm not in ['BN', 'IN']:
-            pred = self.pred.conv2d.forward_refresh_fused(summed, self.activation)
+        if self.fuse and self.norm not in ['BN', 'IN'] and not self.pred.conv2d.use_kf:
+            # as in forward: pred(x + head) as the conv of the two tensors side by side
+            conv = self.pred.conv2d
+            pred = conv._refresh_forward(x, head, self.activation, path=conv.path, filt=self._pred_sum_filter(),
+                                         bias=None if conv.bias is None else conv.bias.detach())
         else:
+            summed = self.pred_add.forward_refresh_reservoirs(x, head)
             pred = self.activation.forward_refresh_reservoirs(self.pred.forward_refresh_reservoirs(summed))
         return pred, states
 

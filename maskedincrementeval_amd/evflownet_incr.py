@@ -155,18 +155,26 @@ class ConvGRUIncr(nn.Module, _IncrBuffers):
         self._reset_incr()
         self.__dict__["_mult_stale"] = False
         zero_state = prev_state is None
-        if zero_state:
-            state_size = [x.shape[0], self.hidden_size] + list(x.shape[2:])
-            prev_state = torch.zeros(state_size, dtype=x.dtype, device=x.device).to(memory_format=torch.channels_last)
-        h_in = None if zero_state else prev_state
+        h_in = None if zero_state else ops.as_nhwc(prev_state)
         update = self.update_gate.forward_refresh_fused(x, self.sigmoid1, h_in)
         if zero_state:
             # prev_state * reset is zero whatever the reset gate says: its conv is skipped
             out_inputs = self.out_gate.forward_refresh_fused(x, self.tanh, None)
         else:
             reset = self.reset_gate.forward_refresh_fused(x, self.sigmoid2, h_in)
-            out_inputs = self.out_gate.forward_refresh_fused(x, self.tanh, prev_state * reset)
-        new_state = prev_state + self.mult.forward_refresh_reservoirs(out_inputs - prev_state, update)
+            gated = ops.mul_dense(h_in, reset, self._dense_buf("reset_state", tuple(h_in.shape), h_in.device, h_in.dtype))
+            out_inputs = self.out_gate.forward_refresh_fused(x, self.tanh, gated)
+        # new_state = prev_state + (out - prev_state) * update and the cached operands of self.mult, one kernel
+        n, _, h, w = update.shape
+        shape = (n, self.hidden_size, h, w)
+        for res in (self.mult.x1_res, self.mult.x2_res):
+            r = res.reservoir
+            if r is None or tuple(r.shape) != shape or r.device != update.device:
+                res.reservoir = ops.new_nhwc(*shape, update.device)
+        self.mult._reset_incr()
+        new_state = self._dense_buf("state_refresh", shape, update.device, update.dtype)
+        ops.convgru_gates_refresh(update, out_inputs, h_in, self.mult.x1_res.reservoir, self.mult.x2_res.reservoir,
+                                  new_state)
         self.add_state._reset_incr()
         return new_state, new_state
 
@@ -403,7 +411,7 @@ class UpsampleConvLayerIncr(nn.Module):
     def forward_refresh_reservoirs(self, parts):
         for m in list(self.up) + [self.cat, self._lead]:
             m._reset_incr()
-        ups = [F.interpolate(p, scale_factor=2, mode="bilinear", align_corners=False) for p in parts]
+        ups = [self.up[i].forward_refresh_reservoirs(p) for i, p in enumerate(parts)]
         fused = self.fuse and self.activation is not None and self.norm not in ["BN", "IN"]
         if fused and len(ups) in (2, 3) and not self.conv2d.use_kf:
             # as in forward: the two wide parts side by side through the two-pointer conv (matrix-core shapes

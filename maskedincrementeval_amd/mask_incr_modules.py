@@ -92,6 +92,16 @@ class _IncrBuffers:
         return b
 
     def _reset_incr(self):
+        """Called by every dense refresh; leaves the incremental buffers alone.  They need no reset: a
+        delta buffer is zero outside the active tiles of the step that last wrote it, and the first step
+        after the refresh finds those tiles in its stale list and zeroes them, exactly as between two
+        incremental steps.  (Zero-filling every delta buffer and tile set here cost about as many fill
+        launches per refresh as the refresh has convs.)"""
+        return
+
+    def _zero_incr(self):
+        """Force the all-zero state: delta buffers, pixel masks, tile sets (for callers that rewrite
+        these buffers by hand)."""
         for key, b in self._ib().items():
             if key[0] in ("d", "p"):
                 b.zero_()
@@ -744,7 +754,13 @@ class nnUpsample2xIncr(IncrementMaskModule):
         return a, pa, b, pb, ts
 
     def forward_refresh_reservoirs(self, x: DenseT, skip: DenseT = None) -> DenseT:
+        """up2x(x + skip) of dense tensors through the same kernel with every pixel and tile active."""
         self._reset_incr()
-        if skip is not None:
-            x = x + skip
-        return F.interpolate(x, scale_factor=2, mode="bilinear", align_corners=False)
+        ops._require_gpu(x, "x")
+        a = ops.as_nhwc(x)
+        b = None if skip is None else ops.as_nhwc(skip)
+        n, c, h, w = a.shape
+        ts = self._dense_tile_set(n, 2 * h, 2 * w, a.device)
+        out = self._dense_buf("refresh_out", (n, c, 2 * h, 2 * w), a.device, a.dtype)
+        ops.upsample2x_incr(a, None, b, None, ts, out)
+        return out

@@ -690,6 +690,43 @@ def convgru_gates_incr(gates_delta, update_res, cand_res, h_delta, ts: TileMask)
     return h_delta
 
 
+def convlstm_gates_refresh(gates_res, interleaved: bool, prev_c, cprev_res, cell_res, h_out, c_out):
+    """Dense ConvLSTM state from the gate pre-activations of a refresh; fills the cell reservoirs."""
+    n, hid, h, w = h_out.shape
+    dt = h_out.dtype
+    if tuple(gates_res.shape) != (n, 4 * hid, h, w):
+        raise ValueError("gates_res shape %s, expected %s" % (tuple(gates_res.shape), (n, 4 * hid, h, w)))
+    for name, t in (("cprev_res", cprev_res), ("cell_res", cell_res)):
+        _same_shape(name, t, h_out)
+    check(lib().mie_convlstm_gates_refresh(
+        nhwc_ptr(gates_res, "gates_res"), 1 if interleaved else 0, nhwc_ptr(prev_c, "prev_c", hid, dtype=dt),
+        nhwc_ptr(cprev_res, "cprev_res"), nhwc_ptr(cell_res, "cell_res"), nhwc_ptr(h_out, "h_out", dtype=dt),
+        nhwc_ptr(c_out, "c_out", hid, dtype=dt), n, h, w, hid, delta_dtype(h_out), _stream(h_out)))
+    return h_out, c_out
+
+
+def convgru_gates_refresh(update, cand, prev_state, diff_res, update_res, new_state):
+    """Dense ConvGRU state from the activated gates of a refresh; fills the product's cached operands."""
+    n, hid, h, w = new_state.shape
+    dt = new_state.dtype
+    check(lib().mie_convgru_gates_refresh(
+        nhwc_ptr(update, "update", hid, dtype=dt), nhwc_ptr(cand, "cand", hid, dtype=dt),
+        nhwc_ptr(prev_state, "prev_state", hid, dtype=dt), nhwc_ptr(diff_res, "diff_res", hid),
+        nhwc_ptr(update_res, "update_res", hid), nhwc_ptr(new_state, "new_state", dtype=dt), n, h, w, hid,
+        delta_dtype(new_state), _stream(new_state)))
+    return new_state
+
+
+def mul_dense(a, b, out):
+    """out = a * b, dense tensors of one shape, layout (NHWC) and type."""
+    dt = out.dtype
+    if a.shape != out.shape or b.shape != out.shape:
+        raise ValueError("shapes differ: %s %s %s" % (tuple(a.shape), tuple(b.shape), tuple(out.shape)))
+    check(lib().mie_mul_dense(nhwc_ptr(a, "a", dtype=dt), nhwc_ptr(b, "b", dtype=dt), nhwc_ptr(out, "out", dtype=dt),
+                              out.numel(), delta_dtype(out), _stream(out)))
+    return out
+
+
 def gate_interleave_index(hid: int, device=None) -> torch.Tensor:
     """Column order of the fused gates conv: entry c' (= 32*b + 8*g + j) holds the column g*hid + 8*b + j of
     the [in | remember | out | cell] x hid order (gate g of hidden channel 8*b + j)."""

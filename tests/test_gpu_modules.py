@@ -222,6 +222,78 @@ def _run_e2depth(h, w, steps, density, fuse, seed=31):
     return model, acc, x
 
 
+class _AtenLog(torch.utils._python_dispatch.TorchDispatchMode):
+    """Names of the ATen ops dispatched inside the block (views included)."""
+
+    def __init__(self):
+        super().__init__()
+        self.ops = []
+
+    def __torch_dispatch__(self, func, types, args=(), kwargs=None):
+        self.ops.append(str(func))
+        return func(*args, **(kwargs or {}))
+
+
+# ATen ops that launch nothing: views and metadata
+_VIEW_OPS = ("aten.detach", "aten.permute", "aten.view", "aten._unsafe_view", "aten.reshape", "aten.alias",
+             "aten.as_strided", "aten.slice", "aten.select", "aten.expand", "aten.t.", "aten.transpose",
+             "aten.unsqueeze", "aten.squeeze", "aten.chunk", "aten.split", "aten.narrow", "aten.sym_",
+             "aten.is_", "aten._to_copy.default_noop")
+
+
+def _kernel_ops(log):
+    return [o for o in log.ops if not any(o.startswith(v) for v in _VIEW_OPS)]
+
+
+def test_e2depth_refresh_runs_on_the_library_kernels_and_replays_as_a_graph():
+    # The dense refresh (incr_modules/e2depth_incr.py:442-468): convs, bilinear x2, ConvLSTM state math and the
+    # skip sums all go through libmie_hip; once the buffers exist a refresh dispatches no ATen kernel, so it can
+    # be captured in a HIP graph.  A refresh in the middle of a stream must leave the incremental state
+    # consistent (no buffer is zero-filled: the next step's stale lists clean up).
+    h, w = 72, 104
+    model = seed_module_(E2VIDRecurrentIncr(), seed=31).to(DEV).eval()
+    oracle = E2DepthOracle(model.state_dict())
+    g = torch.Generator().manual_seed(33)
+    x0, x1 = (torch.randn(1, 5, h, w, generator=g) * 0.5 for _ in range(2))
+    static_x = _cl(x0)
+    with torch.no_grad():
+        model.forward_refresh_reservoirs(static_x, None)            # allocates every buffer
+        for step in range(2):
+            d, _ = event_voxel_delta(1, 5, h, w, 0.05, seed=3300 + step)
+            model([_cl(d), None], None)
+        torch.cuda.synchronize()
+        with _AtenLog() as log:
+            pred = model.forward_refresh_reservoirs(static_x, None)[0]
+        assert _kernel_ops(log) == [], "ATen kernels in the refresh: %s" % sorted(set(_kernel_ops(log)))
+        _close(pred, oracle.refresh(x0), "eager refresh")
+        # captured: replay on another input, then incremental steps on top of it
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            model.forward_refresh_reservoirs(static_x, None)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            pred_g = model.forward_refresh_reservoirs(static_x, None)[0]
+        for x in (x1, x0, x1):
+            static_x.copy_(_cl(x))
+            graph.replay()
+            torch.cuda.synchronize()
+            ref = oracle.refresh(x)
+            _close(pred_g, ref, "graph replay of the refresh")
+        acc, acc_ref = pred_g.clone(), ref.clone()
+        for step in range(3):
+            d, _ = event_voxel_delta(1, 5, h, w, 0.05, seed=3400 + step)
+            out, _ = model([_cl(d), None], None)
+            torch.cuda.synchronize()
+            ref_d = oracle.incr(d)
+            _close(out[0], ref_d, "step %d after the replayed refresh" % step)
+            acc += out[0]
+            acc_ref += ref_d
+        _close(acc, acc_ref, "accumulated after the replayed refresh")
+
+
 @pytest.mark.parametrize("fuse", [True, False])
 def test_e2depth_incr_small_matches_oracle(fuse):
     _run_e2depth(72, 104, steps=4, density=0.05, fuse=fuse)
