@@ -588,6 +588,53 @@ int mie_tconv_masked(const void* x, const uint8_t* xmask, int cin, int h_in,
                      void* stream);
 
 /*
+ * The decoder case of mie_tconv_masked on the matrix cores: stride 2, kernel size k
+ * in {3, 5}, padding k/2, output exactly twice the input (output_padding 1), over
+ * one or two inputs (x ++ x2, the concat-free form of a decoder that takes
+ * torch.cat of its parts, incr_modules/evflownet_incr.py:463-470).  The four
+ * sub-pixel phases of the output are four stride-1 contractions over disjoint
+ * tap subsets of the same staged input, so no product is spent on inserted zeros.
+ *   x / x2 : [n,h_in,w_in,c1] / [n,h_in,w_in,c2] deltas with their pixel masks
+ *        (x2 optional); c1, c2 multiples of 32 (bf16: 64), cout of 32
+ *   filter / filter_mc : [cin_total][k][k][cout] as in mie_tconv_masked and its
+ *        matrix-core copy (mie_pack_filter, required); c1 + c2 <= cin_total
+ *   out    : output tile set at (2*h_in, 2*w_in), built with MIE_FOOT_TCONV
+ *        (k, stride 2, pad k/2) from the OR of the input masks
+ *   blocks : tile set at (h_in, w_in) of the 16x16 output blocks the workgroups
+ *        walk, built from out->pixmask with MIE_FOOT_CONV k = 2, stride 2, pad 0
+ *   addend, reservoir, act_kind, slope : epilogue of mie_conv_masked (addend:
+ *        e.g. the contribution of a few more input channels computed by
+ *        mie_tconv_masked, covered by `out`)
+ *   workspace / workspace_bytes : as in mie_conv_masked_ws (planes of very few
+ *        blocks split their contraction over up to 8 workgroups); may be NULL
+ * Replaces: transposed_conv2d_from_module
+ * (incr_modules/mask_incr_functional.py:64-66) inside TransposedConvLayerIncr
+ * (incr_modules/e2depth_incr.py:243-282).
+ */
+int mie_tconv2x_masked(const void* x, const uint8_t* xmask, int c1,
+                       const void* x2, const uint8_t* x2mask, int c2, int h_in,
+                       int w_in, const float* filter, const void* filter_mc,
+                       int cin_total, int k, int cout, const mie_tileset* out,
+                       const mie_tileset* blocks, void* out_delta,
+                       const void* addend, float* reservoir, int act_kind,
+                       float slope, int dtype, void* workspace,
+                       long long workspace_bytes, void* stream);
+
+/*
+ * Dense refresh twin of mie_tconv2x_masked: out_dense = act(tconv(x ++ x2) +
+ * bias (+ addend)) with `out` and `blocks` all active (build both with in_mask =
+ * NULL), reservoir (optional) = the pre-activation.
+ * Replaces: the conv_transpose2d + bias of TransposedConvLayerIncr's refresh
+ * (incr_modules/e2depth_incr.py:275-282).
+ */
+int mie_tconv2x_refresh(const void* x, int c1, const void* x2, int c2, int h_in,
+                        int w_in, const float* filter, const void* filter_mc,
+                        int cin_total, int k, int cout, const float* bias,
+                        const mie_tileset* out, const mie_tileset* blocks,
+                        void* out_dense, const void* addend, float* reservoir,
+                        int act_kind, float slope, int dtype, void* stream);
+
+/*
  * Dense refresh twin of mie_tconv_masked, as mie_conv_refresh is of
  * mie_conv_masked: out_dense = act(tconv(x) + bias) over the active tiles of
  * `out` (build it with in_mask = NULL: every tile), reservoir (optional) = the

@@ -36,7 +36,8 @@ EXPORTS = (
     "mie_pack_filter", "mie_kfence_incr", "mie_events_to_frame", "mie_tconv_refresh", "mie_conv_gates_masked",
     "mie_maxpool_incr", "mie_accumulate", "mie_scale_incr", "mie_avgpool_incr", "mie_linear_incr", "mie_upconv_masked",
     "mie_conv_masked_ws", "mie_convgru_gates_incr", "mie_upsample2x_pair_incr", "mie_conv_masked_noalloc",
-    "mie_convlstm_gates_refresh", "mie_convgru_gates_refresh", "mie_mul_dense",
+    "mie_convlstm_gates_refresh", "mie_convgru_gates_refresh", "mie_mul_dense", "mie_tconv2x_masked",
+    "mie_tconv2x_refresh",
 )
 
 
@@ -82,6 +83,11 @@ def _declare(l):
     l.mie_convgru_gates_refresh.argtypes = [vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp]
     l.mie_mul_dense.restype = ci
     l.mie_mul_dense.argtypes = [vp, vp, vp, ctypes.c_longlong, ci, vp]
+    l.mie_tconv2x_masked.restype = ci
+    l.mie_tconv2x_masked.argtypes = [vp, vp, ci, vp, vp, ci, ci, ci, vp, vp, ci, ci, ci, tsp, tsp, vp, vp, vp, ci, cf, ci,
+                                     vp, ctypes.c_longlong, vp]
+    l.mie_tconv2x_refresh.restype = ci
+    l.mie_tconv2x_refresh.argtypes = [vp, ci, vp, ci, ci, ci, vp, vp, ci, ci, ci, vp, tsp, tsp, vp, vp, vp, ci, cf, ci, vp]
     l.mie_conv_masked_noalloc.restype = ci
     l.mie_conv_masked_noalloc.argtypes = list(l.mie_conv_masked.argtypes)
     l.mie_conv_masked_ws.restype = ci

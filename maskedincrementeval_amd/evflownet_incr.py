@@ -444,7 +444,10 @@ class UpsampleConvLayerIncr(nn.Module):
 
 class TransposedConvLayerIncr(nn.Module):
     """Transposed conv (stride 2, output_padding 1) -> activation over the concat of the parts:
-    the decoder kind the benchmark configuration of this network names."""
+    the decoder kind the benchmark configuration of this network names.  As in the up-sampling
+    decoder the concat [previous flow (2 ch, optional), x, skip] is never formed: the two wide parts
+    are the two input pointers of the matrix-core transposed conv, the narrow leading part goes
+    through the gather kernel and rides in as the addend."""
 
     def __init__(self, in_channels, out_channels, kernel_size, activation="relu", padding=None, norm=None,
                  fuse=True):
@@ -459,17 +462,62 @@ class TransposedConvLayerIncr(nn.Module):
         self.cat = nnCatIncr()
         self.fuse = fuse
 
+    def _split_ok(self, shapes, dtype, masked=True):
+        """Whether the parts (channel counts in `shapes`) run as lead + two-pointer transposed conv."""
+        tc = self.transposed_conv2d
+        k, s, p, op = tc._geometry()
+        lead_c = shapes[0] if len(shapes) == 3 else 0
+        filt = tc._filter()
+        return (self.fuse and self.activation is not None and len(shapes) in (2, 3) and masked
+                and ops.tconv2x_takes(shapes[-2], shapes[-1], tc.out_channels, k, s, p, op,
+                                      filt.rows(lead_c, filt.shape[0]), dtype))
+
     def forward(self, parts):
+        tc = self.transposed_conv2d
+        chans = [p_[0].shape[1] for p_ in parts]
+        same = all(p_[0].shape[2:] == parts[0][0].shape[2:] for p_ in parts)
+        masked = all(_mask_of(p_) is not None for p_ in parts)
+        if same and self._split_ok(chans, ops.delta_torch_dtype(parts[0][0]), masked):
+            filt = tc._filter()
+            lead_c, addend = 0, None
+            if len(parts) == 3:
+                # the flow estimate of the previous scale shares the mask of x (a 1x1 conv + tanh of it), so the
+                # wide conv's output mask covers this partial result
+                lead_c = chans[0]
+                addend = tc.forward(parts[0], filt=filt.rows(0, lead_c), out_name="lead")
+            kind, slope = activation_kind(self.activation.op)
+            return tc.forward(parts[-2], self.activation.in_res.reservoir, kind, slope, x2_incr=parts[-1],
+                              addend_incr=addend, filt=filt.rows(lead_c, filt.shape[0]))
         x = self.cat(parts)
         if self.fuse and self.activation is not None:
             kind, slope = activation_kind(self.activation.op)
-            return self.transposed_conv2d(x, self.activation.in_res.reservoir, kind, slope)
-        out = self.transposed_conv2d(x)
+            return tc(x, self.activation.in_res.reservoir, kind, slope)
+        out = tc(x)
         return out if self.activation is None else self.activation(out)
 
     def forward_refresh_reservoirs(self, parts):
         self.cat._reset_incr()
-        out = self.transposed_conv2d.forward_refresh_reservoirs(torch.cat(list(parts), 1))
+        tc = self.transposed_conv2d
+        parts = list(parts)
+        chans = [p_.shape[1] for p_ in parts]
+        if all(p_.shape[2:] == parts[0].shape[2:] for p_ in parts) and self._split_ok(chans, ops.delta_torch_dtype(parts[0])):
+            filt = tc._filter()
+            lead_c, addend = 0, None
+            if len(parts) == 3:
+                lead_c = chans[0]
+                addend = tc.forward_refresh_reservoirs(parts[0], filt=filt.rows(0, lead_c), bias=None,
+                                                       out_name="lead_refresh")
+            kind, slope = activation_kind(self.activation.op)
+            n, _, h, w = parts[-1].shape
+            shape = (n, tc.out_channels, 2 * h, 2 * w)
+            r = self.activation.in_res.reservoir
+            if r is None or tuple(r.shape) != shape or r.device != parts[-1].device:
+                self.activation.in_res.reservoir = ops.new_nhwc(*shape, parts[-1].device)
+            self.activation._reset_incr()
+            return tc.forward_refresh_reservoirs(parts[-2], parts[-1], addend, filt=filt.rows(lead_c, filt.shape[0]),
+                                                 bias=None if tc.bias is None else tc.bias.detach(),
+                                                 reservoir=self.activation.in_res.reservoir, act=kind, slope=slope)
+        out = tc.forward_refresh_reservoirs(torch.cat(parts, 1))
         if self.activation is not None:
             out = self.activation.forward_refresh_reservoirs(out)
         return out

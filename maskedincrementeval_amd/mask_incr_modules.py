@@ -536,46 +536,85 @@ def set_kfence(net: nn.Module, tp: Optional[float]) -> int:
 class nnConvTranspose2dIncr(nn.ConvTranspose2d, _IncrBuffers):
     """Incremental transposed conv (named but not defined by the reference,
     incr_modules/e2depth_incr.py:248; semantics of transposed_conv2d_from_module,
-    mask_incr_functional.py:64-66)."""
+    mask_incr_functional.py:64-66).  The decoder case -- stride 2, kernel 3 or 5, padding k // 2,
+    output_padding 1, channel counts in whole staging chunks -- runs on the matrix cores
+    (ops.tconv2x_masked: four sub-pixel phases, one or two inputs, optional addend); every other
+    shape takes the gather kernel (ops.tconv_masked)."""
 
-    def _filter(self):
+    def _filter(self) -> "ops.ConvFilter":
         w = self.weight
         tag = (w.data_ptr(), w._version, str(w.device))
         cached = self.__dict__.get("_filt_cache")
         if cached is None or cached[0] != tag:
-            cached = (tag, w.detach().permute(0, 2, 3, 1).contiguous().float())
+            cached = (tag, ops.ConvFilter(w.detach().permute(0, 2, 3, 1).contiguous().float()))
             self.__dict__["_filt_cache"] = cached
         return cached[1]
 
-    def forward(self, x_incr: Masked, reservoir=None, act=_lib.ACT_NONE, slope=0.0) -> Masked:
+    def _geometry(self):
         k = _square(self.kernel_size, "kernel_size")
         s, p = _square(self.stride, "stride"), _square(self.padding, "padding")
         op = _square(self.output_padding, "output_padding")
         if _square(self.dilation, "dilation") != 1 or self.groups != 1:
             raise NotImplementedError("transposed conv with dilation / groups")
+        return k, s, p, op
+
+    def forward(self, x_incr: Masked, reservoir=None, act=_lib.ACT_NONE, slope=0.0, x2_incr: Masked = None,
+                addend_incr: Masked = None, filt=None, out_name="out") -> Masked:
+        """x2_incr: second input (the conv runs over the channel concat of the two without forming it);
+        addend_incr: delta added before the epilogue, covered by the output mask; filt: a row slice of
+        self._filter() when only part of the input channels is fed.  Two inputs and the addend need the
+        matrix-core form."""
+        k, s, p, op = self._geometry()
         x, pix, _ = _unpack(x_incr)
-        n, _, h, w = x.shape
+        x2 = pix2 = None
+        if x2_incr is not None:
+            x2, pix2, _ = _unpack(x2_incr)
+        n, c1, h, w = x.shape
+        c2 = 0 if x2 is None else x2.shape[1]
         ho, wo = (h - 1) * s - 2 * p + k + op, (w - 1) * s - 2 * p + k + op
-        ts = self._tile_set("out", n, ho, wo, x.device)
-        out = self._delta_buf("out", (n, self.out_channels, ho, wo), x.device, x.dtype)
-        ops.build_mask_tiles(pix, None, n, h, w, _lib.FOOT_TCONV, k, s, p, ts)
-        ops.tconv_masked(x, pix, self._filter(), k, s, p, ts, out, reservoir, act, slope)
+        ts = self._tile_set(out_name, n, ho, wo, x.device)
+        out = self._delta_buf(out_name, (n, self.out_channels, ho, wo), x.device, x.dtype)
+        if x2 is not None and (pix is None or pix2 is None):
+            m1 = m2 = None
+        else:
+            m1, m2 = pix, pix2
+        ops.build_mask_tiles(m1, m2, n, h, w, _lib.FOOT_TCONV, k, s, p, ts)
+        filt = self._filter() if filt is None else filt
+        if ops.tconv2x_takes(c1, c2, self.out_channels, k, s, p, op, filt, ops.delta_torch_dtype(x)):
+            blocks = self._tile_set(out_name + "_blocks", n, h, w, x.device)
+            ops.build_mask_tiles(ts, None, n, ho, wo, _lib.FOOT_CONV, 2, 2, 0, blocks)
+            addend = None if addend_incr is None else ops.as_nhwc(addend_incr[0])
+            ops.tconv2x_masked(x, pix, x2, pix2, filt, k, ts, blocks, out, reservoir, act, slope, addend)
+            return [out, ts]
+        if x2 is not None or addend_incr is not None:
+            raise NotImplementedError("transposed conv over two inputs / with an addend needs the matrix-core form "
+                                      "(stride 2, k in {3, 5}, padding k // 2, output_padding 1, channels in whole chunks)")
+        ops.tconv_masked(x, pix, filt, k, s, p, ts, out, reservoir, act, slope)
         return [out, ts]
 
-    def forward_refresh_reservoirs(self, x):
-        """conv_transpose2d(x, W, b) through the same kernel with every tile active."""
+    def forward_refresh_reservoirs(self, x, x2=None, addend=None, filt=None, bias=None, reservoir=None,
+                                   act=_lib.ACT_NONE, slope=0.0, out_name="refresh_out"):
+        """conv_transpose2d(cat(x, x2), W, b) (+ addend) through the same kernels with every tile active."""
         self._reset_incr()
         ops._require_gpu(x, "x")
-        k = _square(self.kernel_size, "kernel_size")
-        s, p = _square(self.stride, "stride"), _square(self.padding, "padding")
-        op = _square(self.output_padding, "output_padding")
+        k, s, p, op = self._geometry()
         x = ops.as_nhwc(x)
-        n, _, h, w = x.shape
+        x2 = None if x2 is None else ops.as_nhwc(x2)
+        n, c1, h, w = x.shape
+        c2 = 0 if x2 is None else x2.shape[1]
         ho, wo = (h - 1) * s - 2 * p + k + op, (w - 1) * s - 2 * p + k + op
         ts = self._dense_tile_set(n, ho, wo, x.device)
-        out = self._dense_buf("refresh_out", (n, self.out_channels, ho, wo), x.device, x.dtype)
-        bias = None if self.bias is None else self.bias.detach()
-        return ops.tconv_refresh(x, self._filter(), bias, k, s, p, ts, out)
+        out = self._dense_buf(out_name, (n, self.out_channels, ho, wo), x.device, x.dtype)
+        if filt is None:
+            filt = self._filter()
+            bias = None if self.bias is None else self.bias.detach()
+        if ops.tconv2x_takes(c1, c2, self.out_channels, k, s, p, op, filt, ops.delta_torch_dtype(x)):
+            blocks = self._dense_tile_set(n, h, w, x.device)
+            return ops.tconv2x_refresh(x, x2, filt, bias, k, ts, blocks, out, reservoir, act, slope,
+                                       None if addend is None else ops.as_nhwc(addend))
+        if x2 is not None or addend is not None:
+            raise NotImplementedError("transposed conv over two inputs / with an addend needs the matrix-core form")
+        return ops.tconv_refresh(x, filt, bias, k, s, p, ts, out, reservoir, act, slope)
 
 
 class nnBatchNorm2dIncr(nn.BatchNorm2d, _IncrBuffers):

@@ -442,8 +442,10 @@ def conv_refresh(x, x2, filt, bias, k, stride, pad, out_ts: TileMask, out_dense,
 
 def tconv_masked(x, xmask, filt, k, stride, pad, out_ts: TileMask, out_delta, reservoir=None,
                  act=_lib.ACT_NONE, slope=0.0):
-    """filt: ConvTranspose2d weight permuted to [Cin, K, K, Cout], contiguous fp32."""
+    """filt: ConvTranspose2d weight permuted to [Cin, K, K, Cout], contiguous fp32 (tensor or ConvFilter)."""
     n, cin, h, w = x.shape
+    if isinstance(filt, ConvFilter):
+        filt = filt.for_dtype(x.dtype)[0]
     if filt.dim() != 4 or filt.shape[0] != cin or filt.shape[1] != k or not filt.is_contiguous():
         raise ValueError("filter must be contiguous [Cin,%d,%d,Cout], got %s" % (k, k, tuple(filt.shape)))
     _require_gpu(filt, "filter")
@@ -462,6 +464,8 @@ def tconv_refresh(x, filt, bias, k, stride, pad, out_ts: TileMask, out_dense, re
                   act=_lib.ACT_NONE, slope=0.0):
     """Dense transposed conv + bias (+ activation, + reservoir fill) over the tiles of out_ts (all active)."""
     n, cin, h, w = x.shape
+    if isinstance(filt, ConvFilter):
+        filt = filt.for_dtype(x.dtype)[0]
     if filt.dim() != 4 or filt.shape[0] != cin or filt.shape[1] != k or not filt.is_contiguous():
         raise ValueError("filter must be contiguous [Cin,%d,%d,Cout], got %s" % (k, k, tuple(filt.shape)))
     _require_gpu(filt, "filter")
@@ -474,6 +478,72 @@ def tconv_refresh(x, filt, bias, k, stride, pad, out_ts: TileMask, out_dense, re
     check(lib().mie_tconv_refresh(
         nhwc_ptr(x, "x", dtype=x.dtype), cin, h, w, filt.data_ptr(), k, stride, pad, cout,
         None if bias is None else bias.data_ptr(), out_ts.ref, nhwc_ptr(out_dense, "out_dense", dtype=x.dtype),
+        nhwc_ptr(reservoir, "reservoir"), act, float(slope), delta_dtype(x), _stream(x)))
+    return out_dense
+
+
+def tconv2x_takes(c1: int, c2: int, cout: int, k: int, stride: int, pad: int, out_pad: int, filt, dtype) -> bool:
+    """Whether tconv2x_masked has a kernel for the layer: stride 2, k in {3, 5}, pad k // 2, output_padding 1,
+    input channels in whole staging chunks, cout % 32 == 0 and a matrix-core filter copy."""
+    chunk = mfma_chunk(dtype)
+    return (isinstance(filt, ConvFilter) and k in (3, 5) and stride == 2 and pad == k // 2 and out_pad == 1
+            and c1 % chunk == 0 and c2 % chunk == 0 and cout % 32 == 0 and filt.for_dtype(dtype)[1] is not None)
+
+
+def _tconv2x_args(x, x2, filt, k, out_ts, block_ts, out, addend, reservoir):
+    n, c1, h, w = x.shape
+    c2 = 0 if x2 is None else x2.shape[1]
+    if x2 is not None and (x2.shape[0] != n or x2.shape[2:] != x.shape[2:] or x2.dtype != x.dtype):
+        raise ValueError("x2 %s incompatible with x %s" % (tuple(x2.shape), tuple(x.shape)))
+    plain, mc_ptr = _filter_args(filt, k, x.dtype)
+    cin_total, cout = plain.shape[0], plain.shape[3]
+    if mc_ptr is None:
+        raise ValueError("tconv2x needs a ConvFilter with a matrix-core copy")
+    if tuple(out.shape) != (n, cout, 2 * h, 2 * w) or (out_ts.n, out_ts.h, out_ts.w) != (n, 2 * h, 2 * w) \
+            or (block_ts.n, block_ts.h, block_ts.w) != (n, h, w):
+        raise ValueError("output %s / tile sets do not match twice the input %s" % (tuple(out.shape), tuple(x.shape)))
+    for name, t in (("addend", addend), ("reservoir", reservoir)):
+        if t is not None and t.shape != out.shape:
+            raise ValueError("%s shape %s != output %s" % (name, tuple(t.shape), tuple(out.shape)))
+    return n, c1, c2, h, w, plain, mc_ptr, cin_total, cout
+
+
+def tconv2x_masked(x, xmask, x2, x2mask, filt, k, out_ts: TileMask, block_ts: TileMask, out_delta, reservoir=None,
+                   act=_lib.ACT_NONE, slope=0.0, addend=None, workspace=None):
+    """Stride-2 transposed conv (k in {3, 5}, pad k // 2, output twice the input) of x ++ x2 on the matrix
+    cores.  out_ts: MIE_FOOT_TCONV tile set of the output; block_ts: tile set of the 16x16 output blocks at
+    input resolution (build_mask_tiles(out_ts, None, ..., FOOT_CONV, 2, 2, 0, block_ts)).
+    workspace: as in conv_masked (None: the device's shared one when the plane is small, False: none)."""
+    n, c1, c2, h, w, plain, mc_ptr, cin_total, cout = _tconv2x_args(x, x2, filt, k, out_ts, block_ts, out_delta,
+                                                                    addend, reservoir)
+    dt = x.dtype
+    _ready(out_ts)
+    _ready(block_ts)
+    if workspace is None:
+        workspace = split_workspace(x.device) if (split_enabled and block_ts.capacity * (cout // 32) <= 128) else False
+    ws_ptr, ws_bytes = (None, 0) if workspace is False else (workspace.data_ptr(), workspace.numel() * 4)
+    check(lib().mie_tconv2x_masked(
+        nhwc_ptr(x, "x", dtype=dt), pix_ptr(xmask, n, h, w, "xmask"), c1, nhwc_ptr(x2, "x2", dtype=dt),
+        pix_ptr(x2mask, n, h, w, "x2mask"), c2, h, w, plain.data_ptr(), mc_ptr, cin_total, k, cout, out_ts.ref,
+        block_ts.ref, nhwc_ptr(out_delta, "out_delta", dtype=dt), nhwc_ptr(addend, "addend", cout, dtype=dt),
+        nhwc_ptr(reservoir, "reservoir"), act, float(slope), delta_dtype(x), ws_ptr, ws_bytes, _stream(x)))
+    return out_delta
+
+
+def tconv2x_refresh(x, x2, filt, bias, k, out_ts: TileMask, block_ts: TileMask, out_dense, reservoir=None,
+                    act=_lib.ACT_NONE, slope=0.0, addend=None):
+    """Dense twin of tconv2x_masked (both tile sets all active): bias, activation and reservoir fill fused."""
+    n, c1, c2, h, w, plain, mc_ptr, cin_total, cout = _tconv2x_args(x, x2, filt, k, out_ts, block_ts, out_dense,
+                                                                    addend, reservoir)
+    dt = x.dtype
+    if bias is not None and (bias.numel() != cout or bias.dtype != torch.float32 or not bias.is_contiguous()):
+        raise ValueError("bias must be contiguous fp32 of %d elements" % cout)
+    _ready(out_ts)
+    _ready(block_ts)
+    check(lib().mie_tconv2x_refresh(
+        nhwc_ptr(x, "x", dtype=dt), c1, nhwc_ptr(x2, "x2", dtype=dt), c2, h, w, plain.data_ptr(), mc_ptr, cin_total, k,
+        cout, None if bias is None else bias.data_ptr(), out_ts.ref, block_ts.ref,
+        nhwc_ptr(out_dense, "out_dense", dtype=dt), nhwc_ptr(addend, "addend", cout, dtype=dt),
         nhwc_ptr(reservoir, "reservoir"), act, float(slope), delta_dtype(x), _stream(x)))
     return out_dense
 

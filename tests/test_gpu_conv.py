@@ -3,6 +3,7 @@ the CPU oracle, through the C ABI.  fp32 tolerance: rtol 1e-4, atol 1e-5."""
 import numpy as np
 import pytest
 import torch
+import torch.nn.functional as F
 
 from maskedincrementeval_amd import _lib, ops
 from maskedincrementeval_amd.masked_types import TileMask
@@ -186,6 +187,76 @@ def test_tconv_matches_oracle(k, s, p, op):
         ops.tconv_masked(_dev(d), m.to(DEV), filt, k, s, p, ts, out)
         torch.cuda.synchronize()
         _close(out, ref, "tconv k%d" % k)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("c1,c2,cout,h,w,k", [
+    (64, 0, 32, 13, 17, 3),        # one input, ragged plane
+    (64, 64, 64, 16, 16, 3),       # two inputs (the concat-free decoder form), 2 chunks: not split
+    (256, 256, 64, 16, 16, 3),     # 4 blocks x 2 slabs, 16 chunks: the contraction is split over workgroups
+    (64, 0, 128, 40, 48, 5),       # 5x5 (the depth network's decoder kind): halo on all sides
+    (128, 128, 32, 9, 20, 5)])
+def test_tconv2x_matrix_core_form(c1, c2, cout, h, w, k, dtype):
+    # stride-2 transposed conv as four sub-pixel phases on the matrix cores, against F.conv_transpose2d of the
+    # concat; three steps with fresh masks (stale blocks), reservoir + ReLU epilogue and an addend
+    if dtype == torch.bfloat16 and (c1 % 64 or c2 % 64):
+        pytest.skip("bf16 chunks hold 64 channels")
+    n, p = 2, k // 2
+    cin = c1 + c2
+    wt = torch.randn(cin, cout, k, k, generator=torch.Generator().manual_seed(k + cin)) * (2.0 / (cin * k * k)) ** 0.5
+    rnd = (lambda t: t.to(dtype).float())
+    wt = rnd(wt)
+    filt = ops.ConvFilter(wt.permute(0, 2, 3, 1).contiguous().to(DEV))
+    ho, wo = 2 * h, 2 * w
+    ts, blocks = TileMask(n, ho, wo, DEV), TileMask(n, h, w, DEV)
+    out = ops.new_nhwc(n, cout, ho, wo, DEV, dtype)
+    r0 = torch.randn(n, cout, ho, wo, generator=torch.Generator().manual_seed(5))
+    res_gpu, res_cpu = _dev(r0.clone()), io.Reserve(r0.clone())
+    tol = dict(rtol=RTOL, atol=ATOL) if dtype == torch.float32 else dict(rtol=2 ** -7, atol=2 ** -7)
+    for step, dens in enumerate((0.10, 0.03, 0.25)):
+        d1, m1 = gaussian_delta(n, c1, h, w, dens, 0.5, seed=900 + step)
+        d1 = rnd(d1)
+        nan = float("nan")
+        x1 = torch.where(m1.bool().expand_as(d1), d1, torch.full_like(d1, nan))      # inactive pixels are never read
+        x2 = m2 = d2 = None
+        full, mask = d1, m1
+        if c2:
+            d2, m2 = gaussian_delta(n, c2, h, w, dens / 2, 0.5, seed=950 + step)
+            d2 = rnd(d2)
+            x2 = torch.where(m2.bool().expand_as(d2), d2, torch.full_like(d2, nan))
+            full, mask = torch.cat((d1, d2), 1), m1 | m2
+        ops.build_mask_tiles(m1.to(DEV), None if m2 is None else m2.to(DEV), n, h, w, _lib.FOOT_TCONV, k, 2, p, ts)
+        ops.build_mask_tiles(ts, None, n, ho, wo, _lib.FOOT_CONV, 2, 2, 0, blocks)
+        want_mask = mo.footprint_tconv(mask[:, 0].numpy(), k, 2, p, ho, wo)
+        assert np.array_equal(ts.pixmask[:, 0].cpu().numpy(), want_mask)
+        add = rnd(torch.randn(n, cout, ho, wo, generator=torch.Generator().manual_seed(70 + step)) * 0.1
+                  * torch.from_numpy(want_mask).unsqueeze(1).float())
+        ops.tconv2x_masked(_dev(x1.to(dtype)), m1.to(DEV), None if x2 is None else _dev(x2.to(dtype)),
+                           None if m2 is None else m2.to(DEV), filt, k, ts, blocks, out, res_gpu, _lib.ACT_RELU, 0.0,
+                           _dev(add.to(dtype)))
+        torch.cuda.synchronize()
+        ref = io.act_incr(torch.relu, res_cpu, io.tconv_incr(full, wt, 2, p, 1) + add)
+        got = out.float().cpu()
+        assert torch.isfinite(got).all()
+        assert torch.allclose(got, ref, **tol), "step %d max|diff| %.3e" % (step, (got - ref).abs().max())
+        assert torch.allclose(res_gpu.cpu(), res_cpu.reservoir, rtol=RTOL, atol=ATOL if dtype == torch.float32 else 1e-4)
+        outside = ~torch.from_numpy(want_mask).bool().unsqueeze(1)
+        assert torch.count_nonzero(got * outside) == 0          # clean delta, stale blocks zeroed
+    # dense refresh twin: bias + activation + reservoir fill
+    dts, dbl = TileMask(n, ho, wo, DEV), TileMask(n, h, w, DEV)
+    ops.build_mask_tiles(None, None, n, ho, wo, _lib.FOOT_CONV, 1, 1, 0, dts)
+    ops.build_mask_tiles(None, None, n, h, w, _lib.FOOT_CONV, 1, 1, 0, dbl)
+    xa = rnd(torch.randn(n, c1, h, w, generator=torch.Generator().manual_seed(80)))
+    xb = rnd(torch.randn(n, c2, h, w, generator=torch.Generator().manual_seed(81))) if c2 else None
+    bias = torch.randn(cout, generator=torch.Generator().manual_seed(82)) * 0.1
+    dense = ops.new_nhwc(n, cout, ho, wo, DEV, dtype)
+    ops.tconv2x_refresh(_dev(xa.to(dtype)), None if xb is None else _dev(xb.to(dtype)), filt, bias.to(DEV), k, dts, dbl,
+                        dense, res_gpu, _lib.ACT_RELU, 0.0)
+    torch.cuda.synchronize()
+    pre = F.conv_transpose2d(xa if xb is None else torch.cat((xa, xb), 1), wt, bias, stride=2, padding=p, output_padding=1)
+    rt = dict(rtol=RTOL, atol=ATOL) if dtype == torch.float32 else dict(rtol=2 ** -7, atol=2 ** -7)
+    assert torch.allclose(res_gpu.cpu(), pre, rtol=1e-4, atol=1e-5 if dtype == torch.float32 else 1e-4)
+    assert torch.allclose(dense.float().cpu(), torch.relu(pre), **rt)
 
 
 def test_large_channel_mfma_bottleneck_shapes():

@@ -88,10 +88,12 @@ def test_evflownet_small_matches_oracle(decoder, fuse):
     _run(decoder, 64, 96, steps=3, edges=False, fuse=fuse)
 
 
-def test_evflownet_config4_moving_edges_and_dense_identity():
-    # benchmark configuration 4: 1x4x256x256, moving-edge deltas (~3 % density), up-sampling decoders
-    model, acc, x = _run("upsample", 256, 256, steps=3, edges=True)
-    fresh = seed_module_(MultiResUNetRecurrentIncr(num_bins=4), seed=51).to(DEV).eval()
+@pytest.mark.parametrize("decoder", ["upsample", "transposed"])
+def test_evflownet_config4_moving_edges_and_dense_identity(decoder):
+    # benchmark configuration 4: 1x4x256x256, moving-edge deltas (~3 % density); transposed-conv decoders as the
+    # configuration words it, up-sampling decoders as the reference file has them
+    model, acc, x = _run(decoder, 256, 256, steps=3, edges=True)
+    fresh = seed_module_(MultiResUNetRecurrentIncr(num_bins=4, decoder=decoder), seed=51).to(DEV).eval()
     with torch.no_grad():
         dense = fresh.forward_refresh_reservoirs(_cl(x))
     for a, b in zip(acc, dense):
@@ -140,7 +142,8 @@ def test_evflownet_bf16_matches_fp32_oracle(decoder):
         _close(a, b, "accumulated", rtol=2e-2, atol=2e-2)
 
 
-def test_evflownet_planning_stream_and_pass_reproduce_inline_planning(decoder="upsample"):
+@pytest.mark.parametrize("decoder", ["upsample", "transposed"])
+def test_evflownet_planning_stream_and_pass_reproduce_inline_planning(decoder):
     # tile sets built on the planning stream in a planning pass, replayed from a HIP graph, against inline
     # planning with eager launches: same kernels over the same tiles, so every flow scale agrees bit for bit
     h, w, steps = 64, 96, 7
@@ -174,10 +177,11 @@ def test_evflownet_planning_stream_and_pass_reproduce_inline_planning(decoder="u
 
 
 def test_concat_layers_refuse_the_planning_stream():
-    # the transposed-conv decoders concatenate with torch ops on the compute stream, which would read pixel
-    # masks the planning stream is still writing: refused, and the planner is unwound
+    # the un-fused transposed-conv decoders concatenate with torch ops on the compute stream, which would read
+    # pixel masks the planning stream is still writing: refused, and the planner is unwound
     h, w = 32, 48
-    m = seed_module_(MultiResUNetRecurrentIncr(num_bins=4, decoder="transposed", async_masks=True), seed=51).to(DEV).eval()
+    m = seed_module_(MultiResUNetRecurrentIncr(num_bins=4, decoder="transposed", async_masks=True, fuse=False),
+                     seed=51).to(DEV).eval()
     with torch.no_grad():
         m.forward_refresh_reservoirs(_cl(torch.randn(1, 4, h, w, generator=torch.Generator().manual_seed(1))))
         with pytest.raises(NotImplementedError, match="asynchronous mask planning"):
