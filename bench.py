@@ -1,23 +1,29 @@
 #!/usr/bin/env python3
 """Benchmark of the masked incremental inference path on one MI355X.
 
-Workload (the configuration the headline metric is quoted on): E2Depth-incr,
+Headline workload (the configuration the metric is quoted on): E2Depth-incr,
 random-init weights, one event stream of 5x264x352 voxel grids, one dense
 refresh, then incremental steps with 5 % of the pixels carrying a delta
 (Poisson(2) event counts x random polarity x 0.1 per bin, smooth blob masks).
 A "step" is one incremental frame through the whole network; the deltas are
 resident in HBM before the timed region starts and the step is replayed from
-a HIP graph.
+a HIP graph.  `--steps` steps are timed between two device synchronisations,
+`--repeats` times over; `ms_per_step` is the median of those repeats.
 
 Prints ONE JSON line: frames/s (`value`), ms/frame, the roofline of the
 dominant kernel launch (the masked conv layer that takes the most time,
 timed with HIP events on the stream it runs on), a per-layer table, the same
-network run densely through the same kernels (all tiles active), and the CPU
-baseline (the torch-CPU oracle of the reference path on the host cores).
+network run densely through the same kernels (all tiles active), 1 % and 20 %
+density, the dense refresh, the other benchmark configurations ("configs":
+single masked conv, activation chain, EVFlowNet-incr with both decoder kinds,
+batched bf16 E2Depth-incr), the lossy frontier (delta quantiser / threshold
+masks: speed against error) and the CPU baseline (the torch-CPU oracle of the
+reference path on the host cores).
 """
 import argparse
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -29,11 +35,16 @@ PEAK_BF16_MFMA_TFLOPS = 2500.0
 PEAK_HBM_GBS = 8000.0
 
 
+def log(msg):
+    print("[bench] " + msg, file=sys.stderr, flush=True)
+
+
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--repeats", type=int, default=10, help="timed repeats of the --steps loop (median reported)")
     ap.add_argument("--density", type=float, default=0.05)
     ap.add_argument("--height", type=int, default=264)
     ap.add_argument("--width", type=int, default=352)
@@ -48,13 +59,17 @@ def parse_args():
                     help="take the one-kernel up-sampling conv for every decoder layer, whatever its size (for measurements)")
     ap.add_argument("--sync-masks", action="store_true", help="build tile sets on the compute stream (no planning stream)")
     ap.add_argument("--net", choices=["e2depth", "evflownet"], default="e2depth",
-                    help="e2depth: the headline network (5 bins); evflownet: EVFlowNet-incr, 4 bins, up-sampling decoders "
-                         "(the reference's optical-flow configuration: use --height 256 --width 256 --density 0.03)")
+                    help="e2depth: the headline network (5 bins); evflownet: EVFlowNet-incr, 4 bins, moving-edge deltas "
+                         "(use --height 256 --width 256)")
+    ap.add_argument("--decoder", choices=["upsample", "transposed"], default="upsample",
+                    help="decoder kind of --net evflownet")
     ap.add_argument("--dtype", choices=["f32", "bf16"], default="f32",
                     help="element type of deltas and weights (reservoirs and accumulation stay fp32)")
-    ap.add_argument("--kfence-tp", type=float, default=0.0,
-                    help="also time the net with every conv's delta quantiser on (k = tp*||x||); reported under \"kfenced\"")
-    ap.add_argument("--sweep", action="store_true", help="also time 1 %% and 20 %% density (reported under \"density_sweep\")")
+    ap.add_argument("--no-sweep", dest="sweep", action="store_false", help="skip the 1 %% / 20 %% density runs")
+    ap.add_argument("--no-configs", dest="configs", action="store_false",
+                    help="skip the other benchmark configurations (single conv, activation chain, EVFlowNet-incr, batched bf16)")
+    ap.add_argument("--no-lossy", dest="lossy", action="store_false", help="skip the lossy frontier")
+    ap.add_argument("--no-refresh", dest="refresh", action="store_false", help="skip the dense-refresh timing")
     return ap.parse_args()
 
 
@@ -107,7 +122,20 @@ class LayerProbe:
             return dict(kind="conv", k=k, s=1, cin=c, cout=filt.shape[3], h=h, w=w, n=n, xmask=amask,
                         x2mask=bmask, ts=out_ts, fused=reservoir is not None, up=True, two=b_ is not None)
 
+        def tconv2x_desc(x, xmask, x2, x2mask, filt, k, out_ts, block_ts, out_delta, reservoir=None, *a, **kw):
+            n, c1, h, w = x.shape
+            c2 = 0 if x2 is None else x2.shape[1]
+            return dict(kind="conv", k=k, s=2, cin=c1 + c2, cout=filt.shape[3], h=h, w=w, n=n, xmask=xmask,
+                        x2mask=x2mask, ts=out_ts, fused=reservoir is not None, tconv=True)
+
+        def tconv_desc(x, xmask, filt, k, stride, pad, out_ts, out_delta, reservoir=None, *a, **kw):
+            n, c1, h, w = x.shape
+            return dict(kind="conv", k=k, s=stride, cin=c1, cout=filt.shape[3], h=h, w=w, n=n, xmask=xmask,
+                        x2mask=None, ts=out_ts, fused=reservoir is not None, tconv=True)
+
         self._wrap("conv_masked", conv_desc)
+        self._wrap("tconv2x_masked", tconv2x_desc)
+        self._wrap("tconv_masked", tconv_desc)
         self._wrap("upconv_masked", upconv_desc)
         self._wrap("conv_gates_incr", conv_gates_desc)
         self._wrap("act_incr", pw_desc("act", 1, 1))
@@ -151,10 +179,15 @@ class LayerProbe:
                     byts += a_out * cout * es
                     if d["fused"]:
                         byts += 2 * a_out * cout * 4
-                row.update(shape="%s%dx%d s%d %d->%d%s @%dx%d" % ("up2x+" if d.get("up") else "", k, k, d["s"], cin, cout,
+                flops = 2 * a_out * cin * cout * k * k
+                if d.get("tconv"):
+                    # stride-s transposed conv: an output pixel meets (k/s)^2 taps on average
+                    flops = 2 * a_out * cin * cout * k * k // (d["s"] * d["s"])
+                row.update(shape="%s%dx%d s%d %d->%d%s @%dx%d" % ("up2x+" if d.get("up") else ("tconv " if d.get("tconv") else ""),
+                                                                   k, k, d["s"], cin, cout,
                                                                    "+lstm" if d.get("gates") else "", ts.h, ts.w),
                            active_tiles=int(ts.counts[0].item()), tiles=ts.capacity, a_out=a_out,
-                           bytes=byts, flops=2 * a_out * cin * cout * k * k)
+                           bytes=byts, flops=flops)
             elif d["kind"] in ("act", "add", "mul", "up2x", "gates"):
                 ts = d["ts"]
                 a = int(ts.pixmask.sum().item())
@@ -183,6 +216,372 @@ class LayerProbe:
         return m.pixmask if hasattr(m, "pixmask") else m
 
 
+
+
+class Workload:
+    """One network configuration: net, frame size, batch, element type, delta generator."""
+
+    def __init__(self, net="e2depth", h=264, w=352, batch=1, density=0.05, dtype="f32", decoder="upsample"):
+        self.net, self.h, self.w, self.batch, self.density, self.dtype, self.decoder = net, h, w, batch, density, dtype, decoder
+
+    def name(self):
+        return "EVFlowNet-incr" if self.net == "evflownet" else "E2Depth-incr"
+
+    def bins(self):
+        return 4 if self.net == "evflownet" else 5
+
+
+class NetBench:
+    """A network instance factory + resident inputs + the timing loops for one Workload."""
+
+    def __init__(self, torch, ops, wl, args, n_inputs=16):
+        from maskedincrementeval_amd.synthetic import MovingEdges, event_voxel_delta
+        self.torch, self.ops, self.wl, self.args = torch, ops, wl, args
+        self.dev = torch.device("cuda:0")
+        self.dt = torch.bfloat16 if wl.dtype == "bf16" else torch.float32
+        self.es = 2 if wl.dtype == "bf16" else 4
+        self.peak_mfma = PEAK_BF16_MFMA_TFLOPS if wl.dtype == "bf16" else PEAK_FP32_MFMA_TFLOPS
+        self.n_inputs = n_inputs
+        nb, bins, h, w = wl.batch, wl.bins(), wl.h, wl.w
+        if wl.net == "evflownet":
+            from maskedincrementeval_amd.evflownet_incr import MultiResUNetRecurrentIncr
+            self.make_net = lambda **kw: MultiResUNetRecurrentIncr(num_bins=4, decoder=wl.decoder, **kw)
+            self.run_net = lambda m, x: m([x, None])
+            self.out_of = lambda r: r[-1][0]                      # the finest flow scale
+            self.refresh_net = lambda m, x: m.forward_refresh_reservoirs(x)
+            self.refresh_out = lambda r: r[-1]
+        else:
+            from maskedincrementeval_amd.e2depth_incr import E2VIDRecurrentIncr
+            self.make_net = E2VIDRecurrentIncr
+            self.run_net = lambda m, x: m([x, None], None)
+            self.out_of = lambda r: r[0][0]
+            self.refresh_net = lambda m, x: m.forward_refresh_reservoirs(x, None)
+            self.refresh_out = lambda r: r[0]
+        self.x0 = torch.randn(nb, bins, h, w, generator=torch.Generator().manual_seed(2)) * 0.5
+        self.static_in = self.cl(torch.zeros(nb, bins, h, w))
+        self.set_density(wl.density)
+
+    def cl(self, t):
+        return t.to(self.dev).to(self.dt).contiguous(memory_format=self.torch.channels_last)
+
+    def set_density(self, p):
+        """(Re)generate the resident input deltas at pixel density p (moving edges: p is nominal)."""
+        from maskedincrementeval_amd.synthetic import MovingEdges, event_voxel_delta
+        torch, wl = self.torch, self.wl
+        if wl.net == "evflownet":
+            gens = [MovingEdges(wl.h, wl.w, seed=53 + b) for b in range(wl.batch)]
+            self.deltas_cpu = [torch.cat([g.step()[0] for g in gens], 0) for _ in range(self.n_inputs)]
+        else:
+            self.deltas_cpu = [event_voxel_delta(wl.batch, wl.bins(), wl.h, wl.w, p, seed=3000 + i)[0]
+                               for i in range(self.n_inputs)]
+        self.deltas = [self.cl(d) for d in self.deltas_cpu]
+        self.measured_density = float(sum((d != 0).any(1).float().mean().item() for d in self.deltas_cpu) / self.n_inputs)
+
+    def new_model(self, seed=1, **kw):
+        from maskedincrementeval_amd.synthetic import seed_module_
+        return seed_module_(self.make_net(**kw), seed=seed).to(self.dev).eval()
+
+    def step_eager(self, m, i):
+        self.static_in.copy_(self.deltas[i % self.n_inputs])
+        return self.run_net(m, self.static_in)
+
+    def timed_run(self, m, tag, steps=None, repeats=None, check_against=None, graph=None):
+        """Refresh, warm up, capture one step in a HIP graph, then time `steps` steps `repeats` times.
+        Returns (median seconds per step, list of the repeats' ms/step, output-check dict)."""
+        torch, args = self.torch, self.args
+        steps = args.steps if steps is None else steps
+        repeats = args.repeats if repeats is None else repeats
+        use_graph = (not args.no_graph) if graph is None else graph
+        history, check = [], {}
+        with torch.no_grad():
+            self.refresh_net(m, self.cl(self.x0))
+            for i in range(max(args.warmup, 3)):           # also allocates every persistent buffer
+                self.step_eager(m, i)
+                history.append(i)
+            torch.cuda.synchronize()
+            g = graph_out = None
+            if use_graph:
+                side = torch.cuda.Stream()
+                side.wait_stream(torch.cuda.current_stream())
+                with torch.cuda.stream(side):
+                    self.step_eager(m, 0)
+                history.append(0)
+                torch.cuda.current_stream().wait_stream(side)
+                torch.cuda.synchronize()
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    graph_out = self.out_of(self.run_net(m, self.static_in))
+                for i in range(3):
+                    self.static_in.copy_(self.deltas[i % self.n_inputs])
+                    g.replay()
+                    history.append(i)
+            per_repeat = []
+            for _ in range(repeats):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for i in range(steps):
+                    if g is not None:
+                        self.static_in.copy_(self.deltas[i % self.n_inputs])
+                        g.replay()
+                    else:
+                        self.step_eager(m, i)
+                torch.cuda.synchronize()
+                per_repeat.append((time.perf_counter() - t0) / steps)
+                history.extend(range(steps))
+            if check_against is not None:
+                # The timed configuration (graph replay, planning stream) against the plain one: a second
+                # instance of the network with eager launches and inline mask planning takes the same
+                # steps; the next frames of the two must then agree (same kernels over the same tiles).
+                ref = check_against()
+                self.refresh_net(ref, self.cl(self.x0))
+                for i in history:
+                    self.run_net(ref, self.deltas[i % self.n_inputs])
+                worst = 0.0
+                for i in range(4):
+                    want = self.out_of(self.run_net(ref, self.deltas[i % self.n_inputs]))
+                    if g is not None:
+                        self.static_in.copy_(self.deltas[i % self.n_inputs])
+                        g.replay()
+                        got = graph_out
+                    else:
+                        got = self.out_of(self.step_eager(m, i))
+                    worst = max(worst, (got.float() - want.float()).abs().max().item())
+                torch.cuda.synchronize()
+                check.update(max_abs_diff=worst, frames=4, steps_before=len(history),
+                             against="same network, eager launches, inline mask planning")
+                log("%s: max |difference| to the eager inline-planning network over 4 frames after %d steps: %.3e"
+                    % (tag, len(history), worst))
+                if not worst <= 1e-3:
+                    raise SystemExit("bench: the timed configuration does not reproduce the plain one (%.3e)" % worst)
+        sec = statistics.median(per_repeat)
+        log("%s: %.3f ms/step median of %d x %d steps (min %.3f, max %.3f; %s)"
+            % (tag, 1e3 * sec, repeats, steps, 1e3 * min(per_repeat), 1e3 * max(per_repeat),
+               "eager" if g is None else "HIP graph"))
+        return sec, [round(1e3 * t, 4) for t in per_repeat], check
+
+    def layer_table(self, model, iters):
+        """Per-launch table of one step: eager launches with HIP events, mean of `iters` steps."""
+        torch, ops = self.torch, self.ops
+        with torch.no_grad():
+            plan_first, model.plan_first = model.plan_first, False   # one walk per step: every wrapper call timed once
+            self.refresh_net(model, self.cl(self.x0))
+            self.step_eager(model, 0)
+            agg = None
+            for it in range(iters):
+                with LayerProbe(ops, torch, self.es) as probe:
+                    self.step_eager(model, 1 + it)
+                rows = probe.table()
+                if agg is None:
+                    agg = rows
+                    for r in agg:
+                        r["ms_sum"], r["bytes_sum"], r["flops_sum"] = 0.0, 0, 0
+                for r, q in zip(agg, rows):
+                    r["ms_sum"] += q["ms"]
+                    r["bytes_sum"] += q["bytes"]
+                    r["flops_sum"] += q["flops"]
+            model.plan_first = plan_first
+        layers = []
+        for r in agg:
+            ms = r["ms_sum"] / iters
+            byts, fl = r["bytes_sum"] / iters, r["flops_sum"] / iters
+            layers.append(dict(op=r["op"], shape=r["shape"], us=round(1e3 * ms, 2),
+                               gbs=round(byts / (ms * 1e-3) / 1e9, 1) if ms > 0 else None,
+                               tflops=round(fl / (ms * 1e-3) / 1e12, 2) if ms > 0 else None,
+                               bytes=int(byts), flops=int(fl), active_tiles=r.get("active_tiles"), tiles=r.get("tiles")))
+        return layers, agg
+
+    def dominant_roofline(self, layers, agg, reps=50):
+        """Roofline of the conv launch that takes the most time, re-timed on its own: the same call (same
+        tile set, same buffers) replayed back to back between two HIP events on the launch stream."""
+        torch = self.torch
+        convs = [l for l in layers if l["op"] in ("conv_masked", "conv_gates_incr", "upconv_masked", "tconv2x_masked")]
+        dom = max(convs, key=lambda l: l["us"])
+        orig, cargs, ckw = agg[layers.index(dom)]["call"]
+        with torch.no_grad():
+            for _ in range(5):
+                orig(*cargs, **ckw)
+            ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            ev0.record()
+            for _ in range(reps):
+                orig(*cargs, **ckw)
+            ev1.record()
+            torch.cuda.synchronize()
+        dom_us = 1e3 * ev0.elapsed_time(ev1) / reps
+        dom = dict(dom, us=round(dom_us, 2), gbs=round(dom["bytes"] / dom_us / 1e3, 1),
+                   tflops=round(dom["flops"] / dom_us / 1e6, 2))
+        mfma_bound = dom["flops"] / max(dom["bytes"], 1) > self.peak_mfma * 1e12 / (PEAK_HBM_GBS * 1e9)
+        if mfma_bound:
+            roofline = dict(bound="mfma", achieved=dom["tflops"], peak=self.peak_mfma, unit="TFLOP/s",
+                            frac=round(dom["tflops"] / self.peak_mfma, 4), traffic=None)
+        else:
+            roofline = dict(bound="hbm", achieved=dom["gbs"], peak=PEAK_HBM_GBS, unit="GB/s",
+                            frac=round(dom["gbs"] / PEAK_HBM_GBS, 4), traffic=None)
+        roofline.update(kernel="mie_%s %s" % (dom["op"].replace("_incr", "").replace("conv_gates", "conv_gates_masked"),
+                                              dom["shape"]), us=dom["us"],
+                        algorithmic_bytes=dom["bytes"], algorithmic_flops=dom["flops"])
+        # HBM bytes per launch of that kernel from the committed rocprofv3 --pmc summary, if it covers this
+        # shape (FETCH_SIZE + WRITE_SIZE, scaled by the copy-kernel calibration)
+        try:
+            with open(os.path.join(ROOT, "profiles", "pmc_traffic.json")) as f:
+                roofline["traffic"] = json.load(f).get(dom["shape"], {}).get("hbm_bytes_per_launch")
+        except OSError:
+            pass
+        return roofline
+
+    def refresh_timing(self, model, reps=30):
+        """The dense refresh (every 20-100 frames in the reference's drivers): eager and replayed from a graph."""
+        torch = self.torch
+        x = self.cl(self.x0)
+        with torch.no_grad():
+            for _ in range(3):
+                self.refresh_net(model, x)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                self.refresh_net(model, x)
+            torch.cuda.synchronize()
+            eager = (time.perf_counter() - t0) / reps
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                self.refresh_net(model, x)
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                self.refresh_net(model, x)
+            for _ in range(3):
+                g.replay()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                g.replay()
+            torch.cuda.synchronize()
+            graph = (time.perf_counter() - t0) / reps
+        log("dense refresh: %.3f ms eager, %.3f ms from a HIP graph" % (1e3 * eager, 1e3 * graph))
+        return dict(ms_eager=round(1e3 * eager, 4), ms_graph=round(1e3 * graph, 4))
+
+
+def event_time(torch, fn, warm=5, reps=50):
+    """Mean microseconds of fn() over `reps` back-to-back calls between two HIP events on the launch stream."""
+    for _ in range(warm):
+        fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return 1e3 * e0.elapsed_time(e1) / reps
+
+
+def config1_single_conv(torch, ops, _lib):
+    """Configuration 1: one masked incremental conv3x3 32 -> 32 on 1x32x264x352 fp32 at 5 % pixel density,
+    plain delta output (no fused epilogue): the launch alone, deltas resident."""
+    from maskedincrementeval_amd.masked_types import TileMask
+    from maskedincrementeval_amd.synthetic import gaussian_delta, he_normal_conv_weight
+    dev = torch.device("cuda:0")
+    n, c, h, w = 1, 32, 264, 352
+    d, m = gaussian_delta(n, c, h, w, 0.05, 0.1, seed=1000)
+    x = ops.as_nhwc(d.to(dev).contiguous(memory_format=torch.channels_last))
+    mask = m.to(dev)
+    filt = ops.ConvFilter(he_normal_conv_weight(c, c, 3, 0).permute(1, 2, 3, 0).contiguous().to(dev))
+    ts = TileMask(n, h, w, dev)
+    ops.build_mask_tiles(mask, None, n, h, w, _lib.FOOT_CONV, 3, 1, 1, ts)
+    out = ops.new_nhwc(n, c, h, w, dev)
+    res = ops.new_nhwc(n, c, h, w, dev)
+    rows = {}
+    for name, r, act in (("delta_only", None, _lib.ACT_NONE), ("fused_reservoir_relu", res, _lib.ACT_RELU)):
+        us = event_time(torch, lambda: ops.conv_masked(x, mask, None, None, filt, 3, 1, 1, ts, out, r, act, 0.0))
+        a_in, a_out = int(mask.sum().item()), int(ts.pixmask.sum().item())
+        byts = n * h * w + a_in * c * 4 + a_out * c * 4 + c * c * 9 * 4 + ts.capacity * 4 + (2 * a_out * c * 4 if r is not None else 0)
+        flops = 2 * a_out * c * c * 9
+        rows[name] = dict(us=round(us, 2), algorithmic_bytes=byts, algorithmic_flops=flops,
+                          gbs=round(byts / us / 1e3, 1), hbm_frac=round(byts / us / 1e3 / PEAK_HBM_GBS, 4),
+                          tflops=round(flops / us / 1e6, 2), active_pixels_in=a_in, active_pixels_out=a_out,
+                          active_tiles=int(ts.counts[0].item()), tiles=ts.capacity)
+    us_build = event_time(torch, lambda: ops.build_mask_tiles(mask, None, n, h, w, _lib.FOOT_CONV, 3, 1, 1, ts))
+    rows["build_mask_tiles_us"] = round(us_build, 2)
+    rows["dense_bytes"], rows["dense_flops"] = 2 * n * c * h * w * 4, 2 * n * h * w * c * c * 9
+    log("config 1 (conv3x3 32->32 @264x352, 5 %%): %.1f us, %.2f MB algorithmic = %.0f GB/s; with reservoir + ReLU %.1f us"
+        % (rows["delta_only"]["us"], rows["delta_only"]["algorithmic_bytes"] / 1e6, rows["delta_only"]["gbs"],
+           rows["fused_reservoir_relu"]["us"]))
+    return rows
+
+
+def config2_activation_chain(torch, ops, _lib):
+    """Configuration 2: masked conv3x3 64 -> 64, incremental LeakyReLU(0.01), incremental ReLU on 1x64x132x176 fp32
+    at 1 / 5 / 20 %, a fresh mask every step: microseconds per step of the chain (mask build + conv with the
+    LeakyReLU increment fused + ReLU increment with its refined mask), eager launches between two HIP events."""
+    from maskedincrementeval_amd import mask_incr_modules as mm
+    from maskedincrementeval_amd.synthetic import gaussian_delta, seed_module_
+    dev = torch.device("cuda:0")
+    n, c, h, w = 1, 64, 132, 176
+    conv = seed_module_(mm.nnConvIncr(c, c, 3, 1, 1), seed=2).to(dev).eval()
+    leaky = mm.nnReservedActivation(mm.leaky_relu_op(0.01), refine_mask=False)
+    relu = mm.nnReluIncr()
+    x0 = torch.randn(n, c, h, w, generator=torch.Generator().manual_seed(20))
+    cl = lambda t: ops.as_nhwc(t.to(dev).contiguous(memory_format=torch.channels_last))
+    out = {}
+    with torch.no_grad():
+        relu.forward_refresh_reservoirs(conv.forward_refresh_fused(cl(x0), leaky))
+        for p in (0.01, 0.05, 0.20):
+            ins = [gaussian_delta(n, c, h, w, p, 0.2, seed=2000 + i) for i in range(8)]
+            ins = [(cl(d), m.to(dev)) for d, m in ins]
+            state = {"i": 0}
+
+            def step():
+                d, m = ins[state["i"] % 8]
+                state["i"] += 1
+                return relu(conv.forward_fused([d, m], leaky))
+            us = event_time(torch, step, warm=8, reps=48)
+            a = sum(int(m.sum().item()) for _, m in ins) / 8.0
+            # algorithmic bytes of the chain: conv (mask, active delta in, delta out, reservoir r+w, filter, tile list)
+            # + ReLU increment (delta in, reservoir r+w, delta out, mask)
+            ts = conv._tile_set("out_act", n, h, w, dev)
+            a_out = int(ts.pixmask.sum().item())
+            byts = (n * h * w + a * c * 4 + a_out * c * 12 + c * c * 9 * 4 + ts.capacity * 4) + (a_out * c * 16 + n * h * w)
+            out["%.2f" % p] = dict(us_per_step=round(us, 2), algorithmic_bytes=int(byts), gbs=round(byts / us / 1e3, 1),
+                                   hbm_frac=round(byts / us / 1e3 / PEAK_HBM_GBS, 4))
+            log("config 2 (conv3x3 64->64 + LeakyReLU + ReLU @132x176, %.0f %%): %.1f us/step, %.0f GB/s algorithmic"
+                % (100 * p, us, byts / us / 1e3))
+    return out
+
+
+def side_config(torch, ops, args, wl, densities, steps, repeats, layer_iters=3, n_inputs=8, dense=True):
+    """ms/step, dominant-kernel roofline and the dense comparator of another network configuration."""
+    nb = NetBench(torch, ops, wl, args, n_inputs=n_inputs)
+    model = nb.new_model(async_masks=not args.sync_masks, plan_first=args.plan_first)
+    rows = {}
+    for p in densities:
+        if abs(p - wl.density) > 1e-12:
+            nb.set_density(p)
+            wl.density = p
+        tag = "%s %dx%dx%d %s%s @%.0f%%" % (wl.name(), wl.batch, wl.h, wl.w, wl.dtype,
+                                          " " + wl.decoder if wl.net == "evflownet" else "", 100 * p)
+        sec, reps_ms, _ = nb.timed_run(model, tag, steps=steps, repeats=repeats)
+        layers, agg = nb.layer_table(model, layer_iters)
+        roof = nb.dominant_roofline(layers, agg, reps=20)
+        rows["%.2f" % p] = dict(ms_per_step=round(1e3 * sec, 4), frames_per_s=round(wl.batch / sec, 1),
+                                repeats_ms=reps_ms, measured_pixel_density=round(nb.measured_density, 4),
+                                algorithmic_gflop_per_step=round(sum(l["flops"] for l in layers) / 1e9, 2),
+                                algorithmic_mb_per_step=round(sum(l["bytes"] for l in layers) / 1e6, 1),
+                                hbm_frac_whole_step=round(sum(l["bytes"] for l in layers) / sec / 1e9 / PEAK_HBM_GBS, 4),
+                                dominant=roof)
+    res = dict(workload="%s %dx%dx%dx%d %s%s" % (wl.name(), wl.batch, wl.bins(), wl.h, wl.w, wl.dtype,
+                                                 ", %s decoders, moving-edge deltas" % wl.decoder if wl.net == "evflownet" else ""),
+               densities=rows)
+    if dense:
+        dm = nb.new_model(derive_input_mask=False, async_masks=not args.sync_masks, plan_first=args.plan_first)
+        dsec, _, _ = nb.timed_run(dm, "  dense (all tiles active, same kernels)", steps=steps, repeats=max(3, repeats // 2))
+        res["dense_same_kernels_ms"] = round(1e3 * dsec, 4)
+        del dm
+    del model, nb
+    torch.cuda.empty_cache()
+    return res
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -191,8 +590,6 @@ def main():
         sys.exit(2)
     import torch
     from maskedincrementeval_amd import _lib, ops
-    from maskedincrementeval_amd.e2depth_incr import E2VIDRecurrentIncr
-    from maskedincrementeval_amd.synthetic import event_voxel_delta, seed_module_
 
     _lib.lib()   # fail loudly if the HIP library is missing
     if args.upconv_all:
@@ -200,226 +597,67 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
-    dev = torch.device("cuda:0")
-    H, W, dens, NB = args.height, args.width, args.density, args.batch
-    dt = torch.bfloat16 if args.dtype == "bf16" else torch.float32
-    es = 2 if args.dtype == "bf16" else 4          # bytes per delta / weight element
-    peak_mfma = PEAK_BF16_MFMA_TFLOPS if args.dtype == "bf16" else PEAK_FP32_MFMA_TFLOPS
-    cl = lambda t: t.to(dev).to(dt).contiguous(memory_format=torch.channels_last)
+    wl = Workload(args.net, args.height, args.width, args.batch, args.density, args.dtype, args.decoder)
+    nb = NetBench(torch, ops, wl, args)
+    H, W, dens, NB, BINS, NET_NAME = wl.h, wl.w, wl.density, wl.batch, wl.bins(), wl.name()
 
-    # the two networks differ in their call conventions only: adapters
-    if args.net == "evflownet":
-        from maskedincrementeval_amd.evflownet_incr import MultiResUNetRecurrentIncr
-        BINS, NET_NAME = 4, "EVFlowNet-incr"
-        make_net = lambda **kw: MultiResUNetRecurrentIncr(num_bins=4, **kw)
-        run_net = lambda m, x: m([x, None])
-        out_of = lambda r: r[-1][0]                      # the finest flow scale
-        refresh_net = lambda m, x: m.forward_refresh_reservoirs(x)
-        refresh_out = lambda r: r[-1]
-    else:
-        BINS, NET_NAME = 5, "E2Depth-incr"
-        make_net = E2VIDRecurrentIncr
-        run_net = lambda m, x: m([x, None], None)
-        out_of = lambda r: r[0][0]
-        refresh_net = lambda m, x: m.forward_refresh_reservoirs(x, None)
-        refresh_out = lambda r: r[0]
+    model = nb.new_model(async_masks=not args.sync_masks, plan_first=args.plan_first)
+    sec_per_step, repeats_ms, output_check = nb.timed_run(model, "incremental %.0f%%" % (100 * dens),
+                                                          check_against=lambda: nb.new_model())
 
-    model = seed_module_(make_net(async_masks=not args.sync_masks, plan_first=args.plan_first), seed=1).to(dev).eval()
-    x0 = torch.randn(NB, BINS, H, W, generator=torch.Generator().manual_seed(2)) * 0.5
-    n_inputs = 16
-    deltas_cpu = [event_voxel_delta(NB, BINS, H, W, dens, seed=3000 + i)[0] for i in range(n_inputs)]
-    deltas = [cl(d) for d in deltas_cpu]
-    static_in = cl(torch.zeros(NB, BINS, H, W))
-
-    def step_eager(m, i):
-        static_in.copy_(deltas[i % n_inputs])
-        return run_net(m, static_in)
-
-    output_check = {}
-
-    def timed_run(m, tag, check_against=None):
-        history = []                                       # input index of every step the model takes
-        with torch.no_grad():
-            refresh_net(m, cl(x0))
-            for i in range(max(args.warmup, 3)):           # also allocates every persistent buffer
-                step_eager(m, i)
-                history.append(i)
-            torch.cuda.synchronize()
-            graph = None
-            if not args.no_graph:
-                side = torch.cuda.Stream()
-                side.wait_stream(torch.cuda.current_stream())
-                with torch.cuda.stream(side):
-                    step_eager(m, 0)
-                history.append(0)
-                torch.cuda.current_stream().wait_stream(side)
-                torch.cuda.synchronize()
-                graph = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(graph):
-                    graph_out = out_of(run_net(m, static_in))
-                for i in range(3):
-                    static_in.copy_(deltas[i % n_inputs])
-                    graph.replay()
-                    history.append(i)
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            for i in range(args.steps):
-                if graph is not None:
-                    static_in.copy_(deltas[i % n_inputs])
-                    graph.replay()
-                else:
-                    step_eager(m, i)
-            torch.cuda.synchronize()
-            dt = time.perf_counter() - t0
-            history.extend(range(args.steps))
-            if check_against is not None:
-                # The timed configuration (graph replay, planning stream) against the plain one: a second
-                # instance of the network with eager launches and inline mask planning takes the same
-                # steps; the next frames of the two must then agree (same kernels over the same tiles).
-                ref = check_against()
-                refresh_net(ref, cl(x0))
-                for i in history:
-                    run_net(ref, deltas[i % n_inputs])
-                worst = 0.0
-                for i in range(4):
-                    want = out_of(run_net(ref, deltas[i % n_inputs]))
-                    if graph is not None:
-                        static_in.copy_(deltas[i % n_inputs])
-                        graph.replay()
-                        got = graph_out
-                    else:
-                        got = out_of(step_eager(m, i))
-                    worst = max(worst, (got.float() - want.float()).abs().max().item())
-                torch.cuda.synchronize()
-                output_check.update(max_abs_diff=worst, frames=4, steps_before=len(history),
-                                    against="same network, eager launches, inline mask planning")
-                print("[bench] %s: max |difference| to the eager inline-planning network over 4 frames after %d steps: %.3e"
-                      % (tag, len(history), worst), file=sys.stderr, flush=True)
-                if not worst <= 1e-3:
-                    raise SystemExit("bench: the timed configuration does not reproduce the plain one (%.3e)" % worst)
-        print("[bench] %s: %.3f ms/frame over %d steps (%s)" % (tag, 1e3 * dt / args.steps, args.steps,
-              "eager" if graph is None else "HIP graph"), file=sys.stderr, flush=True)
-        return dt / args.steps
-
-    sec_per_step = timed_run(model, "incremental %.0f%%" % (100 * dens),
-                             check_against=lambda: seed_module_(make_net(), seed=1).to(dev).eval())
-
-    # ---- per-layer roofline table: eager launches with HIP events, several repeats ------------
-    with torch.no_grad():
-        model.plan_first = False          # one walk per step: the probe times every wrapper call once
-        refresh_net(model, cl(x0))
-        step_eager(model, 0)
-        agg = None
-        for it in range(args.layer_iters):
-            with LayerProbe(ops, torch, es) as probe:
-                step_eager(model, 1 + it)
-            rows = probe.table()
-            if agg is None:
-                agg = rows
-                for r in agg:
-                    r["ms_sum"] = 0.0
-                    r["bytes_sum"] = 0
-                    r["flops_sum"] = 0
-            for r, q in zip(agg, rows):
-                r["ms_sum"] += q["ms"]
-                r["bytes_sum"] += q["bytes"]
-                r["flops_sum"] += q["flops"]
-    layers = []
-    for r in agg:
-        ms = r["ms_sum"] / args.layer_iters
-        byts, fl = r["bytes_sum"] / args.layer_iters, r["flops_sum"] / args.layer_iters
-        layers.append(dict(op=r["op"], shape=r["shape"], us=round(1e3 * ms, 2),
-                           gbs=round(byts / (ms * 1e-3) / 1e9, 1) if ms > 0 else None,
-                           tflops=round(fl / (ms * 1e-3) / 1e12, 2) if ms > 0 else None,
-                           bytes=int(byts), flops=int(fl), active_tiles=r.get("active_tiles"), tiles=r.get("tiles")))
-    convs = [l for l in layers if l["op"] in ("conv_masked", "conv_gates_incr", "upconv_masked")]
-    dom = max(convs, key=lambda l: l["us"])
-    # Re-time the dominant launch on its own: the same call (same tile set, same buffers)
-    # replayed back to back between two HIP events on the launch stream.
-    orig, cargs, ckw = agg[layers.index(dom)]["call"]
-    reps = 50
-    with torch.no_grad():
-        for _ in range(5):
-            orig(*cargs, **ckw)
-        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        ev0.record()
-        for _ in range(reps):
-            orig(*cargs, **ckw)
-        ev1.record()
-        torch.cuda.synchronize()
-    dom_us = 1e3 * ev0.elapsed_time(ev1) / reps
-    dom = dict(dom, us=round(dom_us, 2), gbs=round(dom["bytes"] / dom_us / 1e3, 1),
-               tflops=round(dom["flops"] / dom_us / 1e6, 2))
-    mfma_bound = dom["flops"] / max(dom["bytes"], 1) > peak_mfma * 1e12 / (PEAK_HBM_GBS * 1e9)
-    if mfma_bound:
-        roofline = dict(bound="mfma", achieved=dom["tflops"], peak=peak_mfma, unit="TFLOP/s",
-                        frac=round(dom["tflops"] / peak_mfma, 4), traffic=None)
-    else:
-        roofline = dict(bound="hbm", achieved=dom["gbs"], peak=PEAK_HBM_GBS, unit="GB/s",
-                        frac=round(dom["gbs"] / PEAK_HBM_GBS, 4), traffic=None)
-    roofline.update(kernel="mie_conv_masked %s" % dom["shape"], us=dom["us"],
-                    algorithmic_bytes=dom["bytes"], algorithmic_flops=dom["flops"])
-    # HBM bytes per launch of that kernel from the committed rocprofv3 --pmc summary, if it
-    # covers this shape (FETCH_SIZE + WRITE_SIZE, scaled by the copy-kernel calibration)
-    try:
-        with open(os.path.join(ROOT, "profiles", "pmc_traffic.json")) as f:
-            roofline["traffic"] = json.load(f).get(dom["shape"], {}).get("hbm_bytes_per_launch")
-    except OSError:
-        pass
+    # ---- per-layer roofline table -------------------------------------------------------------------
+    layers, agg = nb.layer_table(model, args.layer_iters)
+    roofline = nb.dominant_roofline(layers, agg)
     tot_us = sum(l["us"] for l in layers)
     tot_bytes = sum(l["bytes"] for l in layers)
     tot_flops = sum(l["flops"] for l in layers)
-    print("[bench] per-launch table (eager, HIP events, mean of %d steps):" % args.layer_iters, file=sys.stderr)
+    log("per-launch table (eager, HIP events, mean of %d steps):" % args.layer_iters)
     for l in layers:
-        print("[bench]   %-22s %-34s %9.2f us %8s GB/s %7s TFLOP/s  tiles %s/%s" % (
-            l["op"], l["shape"], l["us"], l["gbs"], l["tflops"], l["active_tiles"], l["tiles"]), file=sys.stderr)
-    print("[bench]   sum of kernels %.1f us; algorithmic %.1f MB, %.2f GFLOP per frame" %
-          (tot_us, tot_bytes / 1e6, tot_flops / 1e9), file=sys.stderr, flush=True)
+        log("  %-22s %-34s %9.2f us %8s GB/s %7s TFLOP/s  tiles %s/%s" % (
+            l["op"], l["shape"], l["us"], l["gbs"], l["tflops"], l["active_tiles"], l["tiles"]))
+    log("  sum of kernels %.1f us; algorithmic %.1f MB, %.2f GFLOP per frame" % (tot_us, tot_bytes / 1e6, tot_flops / 1e9))
 
     # ---- dense comparator: same kernels, every tile active ---------------------------------------
-    model.plan_first = args.plan_first
     dense_sec = None
     if not args.no_dense:
-        dense_model = seed_module_(make_net(derive_input_mask=False, async_masks=not args.sync_masks,
-                                            plan_first=args.plan_first), seed=1).to(dev).eval()
-        dense_sec = timed_run(dense_model, "dense (all tiles active, same kernels)")
+        dense_model = nb.new_model(derive_input_mask=False, async_masks=not args.sync_masks, plan_first=args.plan_first)
+        dense_sec, _, _ = nb.timed_run(dense_model, "dense (all tiles active, same kernels)", repeats=max(3, args.repeats // 2))
         del dense_model
-
-    # ---- lossy variant: delta quantiser in front of every conv ------------------------------------
-    kfenced = None
-    if args.kfence_tp > 0:
-        from maskedincrementeval_amd.mask_incr_modules import set_kfence
-        kf_model = seed_module_(make_net(async_masks=not args.sync_masks), seed=1).to(dev).eval()
-        set_kfence(kf_model, args.kfence_tp)
-        t = timed_run(kf_model, "quantised deltas (tp = %g)" % args.kfence_tp)
-        # deviation of the accumulated prediction from the exact incremental net, same inputs
-        with torch.no_grad():
-            acc = []
-            for m in (model, kf_model):
-                pred = refresh_out(refresh_net(m, cl(x0))).clone()
-                for i in range(n_inputs):
-                    pred += out_of(step_eager(m, i))
-                acc.append(pred)
-            torch.cuda.synchronize()
-            dev_abs = (acc[0] - acc[1]).abs().max().item()
-        kfenced = dict(tp=args.kfence_tp, ms_per_step=round(1e3 * t, 4), frames_per_s=round(1 / t, 1),
-                       max_abs_deviation_after_16_steps=dev_abs)
-        print("[bench] quantised deltas: max |deviation| of the prediction after %d steps = %.3e" %
-              (n_inputs, dev_abs), file=sys.stderr, flush=True)
-        del kf_model
 
     # ---- other densities (same network, same kernels) ------------------------------------------------
     sweep = None
-    if args.sweep:
-        sweep = {"%.2f" % dens: dict(ms_per_step=round(1e3 * sec_per_step, 4), frames_per_s=round(1 / sec_per_step, 1))}
-        keep = list(deltas)
+    if args.sweep and wl.net == "e2depth":
+        sweep = {"%.2f" % dens: dict(ms_per_step=round(1e3 * sec_per_step, 4), frames_per_s=round(NB / sec_per_step, 1))}
         for p in (0.01, 0.20):
             if abs(p - dens) < 1e-9:
                 continue
-            deltas[:] = [cl(event_voxel_delta(NB, 5, H, W, p, seed=3000 + i)[0]) for i in range(n_inputs)]
-            t = timed_run(model, "incremental %.0f%%" % (100 * p))
-            sweep["%.2f" % p] = dict(ms_per_step=round(1e3 * t, 4), frames_per_s=round(1 / t, 1))
-        deltas[:] = keep
+            nb.set_density(p)
+            t, _, _ = nb.timed_run(model, "incremental %.0f%%" % (100 * p), repeats=max(3, args.repeats // 2))
+            sweep["%.2f" % p] = dict(ms_per_step=round(1e3 * t, 4), frames_per_s=round(NB / t, 1))
+        nb.set_density(dens)
+
+    # ---- dense refresh ---------------------------------------------------------------------------------
+    refresh = nb.refresh_timing(model) if args.refresh else None
+
+    # ---- lossy frontier --------------------------------------------------------------------------------
+    lossy = None
+    if args.lossy and wl.net == "e2depth":
+        from maskedincrementeval_amd.lossy import lossy_frontier
+        lossy = lossy_frontier(nb, model, log)
+
+    # ---- the other benchmark configurations ---------------------------------------------------------
+    configs = None
+    if args.configs:
+        configs = {}
+        configs["c1_single_conv3x3_32to32_264x352_d05"] = config1_single_conv(torch, ops, _lib)
+        configs["c2_conv_leakyrelu_relu_64ch_132x176"] = config2_activation_chain(torch, ops, _lib)
+        short = dict(steps=min(args.steps, 50), repeats=max(3, args.repeats // 2))
+        for dec in ("transposed", "upsample"):
+            configs["c4_evflownet_incr_256x256_%s" % dec] = side_config(
+                torch, ops, args, Workload("evflownet", 256, 256, 1, 0.03, "f32", dec), [0.03], **short)
+        configs["c5_e2depth_incr_bf16_8x480x640"] = side_config(
+            torch, ops, args, Workload("e2depth", 480, 640, 8, 0.01, "bf16"), [0.01, 0.20], n_inputs=4,
+            steps=min(args.steps, 20), repeats=max(3, args.repeats // 2))
 
     # ---- CPU baseline: the oracle (torch-CPU restatement of the reference path) -----------------
     cpu = None
@@ -427,22 +665,22 @@ def main():
         torch.set_num_threads(min(os.cpu_count() or 1, 16))
         if args.net == "evflownet":
             from oracle.evflownet_oracle import EVFlowNetOracle
-            oracle = EVFlowNetOracle(model.state_dict(), decoder="upsample")
+            oracle = EVFlowNetOracle(model.state_dict(), decoder=wl.decoder)
         else:
             from oracle.e2depth_oracle import E2DepthOracle
             oracle = E2DepthOracle(model.state_dict())
         with torch.no_grad():
-            oracle.refresh(x0)
-            oracle.incr(deltas_cpu[0])
+            oracle.refresh(nb.x0)
+            oracle.incr(nb.deltas_cpu[0])
             t0 = time.perf_counter()
             for i in range(args.cpu_steps):
-                oracle.incr(deltas_cpu[(1 + i) % n_inputs])
+                oracle.incr(nb.deltas_cpu[(1 + i) % nb.n_inputs])
             cdt = (time.perf_counter() - t0) / args.cpu_steps
         cpu = dict(value=round(NB / cdt, 3), unit="frames/s", cores=torch.get_num_threads(), kind="port",
                    ms_per_step=round(1e3 * cdt, 2),
                    sample="%d incremental steps of the same %s %dx%d workload (dense F.conv2d on the "
                           "delta, as the reference executes it), torch-CPU fp32" % (args.cpu_steps, NET_NAME, H, W))
-        print("[bench] cpu baseline: %.1f ms/frame on %d threads" % (1e3 * cdt, cpu["cores"]), file=sys.stderr, flush=True)
+        log("cpu baseline: %.1f ms/frame on %d threads" % (1e3 * cdt, cpu["cores"]))
 
     result = {
         # the headline metric's name; `value` is its frames/s part, the HBM GB/s part is in
@@ -462,18 +700,23 @@ def main():
         "config": {"workload": "%s recurrent UNet, random init, %dx%dx%dx%d event voxel deltas, %.0f%% "
                                "active pixels, 1 dense refresh then incremental steps" % (NET_NAME, NB, BINS, H, W, 100 * dens),
                    "density": dens, "height": H, "width": W, "batch": NB, "graph": not args.no_graph,
+                   "timing": "median of %d repeats of %d steps" % (args.repeats, args.steps),
                    "mask_planning": "inline" if args.sync_masks else ("second stream, builds first" if args.plan_first else "second stream")},
         "roofline": roofline,
         "cpu_baseline": cpu,
+        "repeats_ms_per_step": repeats_ms,
         "hbm_gbs_whole_frame": round(tot_bytes / sec_per_step / 1e9, 1),
         "hbm_frac_whole_frame": round(tot_bytes / sec_per_step / 1e9 / PEAK_HBM_GBS, 5),
         "algorithmic_mb_per_frame": round(tot_bytes / 1e6, 2),
         "algorithmic_gflop_per_frame": round(tot_flops / 1e9, 3),
+        "mfma_frac_whole_frame": round(tot_flops / sec_per_step / 1e12 / nb.peak_mfma, 4),
         "sum_kernel_us": round(tot_us, 1),
         "dense_same_kernels_ms": None if dense_sec is None else round(1e3 * dense_sec, 4),
         "speedup_vs_dense": None if dense_sec is None else round(dense_sec / sec_per_step, 3),
         "density_sweep": sweep,
-        "kfenced": kfenced,
+        "refresh": refresh,
+        "lossy_frontier": lossy,
+        "configs": configs,
         "output_check": output_check,
         "layers": layers,
     }

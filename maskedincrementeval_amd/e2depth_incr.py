@@ -220,8 +220,7 @@ class ConvLSTMIncr(nn.Module, _IncrBuffers):
         return ts
 
     def _forward_one_kernel(self, input_incr, prev_h_incr, prev_c_incr):
-        if self.Gates.use_kf:
-            input_incr = self.Gates.kf(input_incr)
+        input_incr = self.Gates.lossy_input(input_incr)
         x, pix, _ = _unpack(input_incr)
         x2 = pix2 = None
         if prev_h_incr is not None:
@@ -252,8 +251,7 @@ class ConvLSTMIncr(nn.Module, _IncrBuffers):
             return self._forward_one_kernel(input_incr, prev_h_incr, prev_c_incr)
         slot = self._state_slot(prev_h_incr, prev_c_incr)
         sfx = "" if slot == 0 else "_b"
-        if self.Gates.use_kf:
-            input_incr = self.Gates.kf(input_incr)
+        input_incr = self.Gates.lossy_input(input_incr)
         x, pix, _ = _unpack(input_incr)
         x2 = pix2 = None
         if prev_h_incr is not None:

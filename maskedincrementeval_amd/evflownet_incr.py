@@ -133,8 +133,8 @@ class ConvGRUIncr(nn.Module, _IncrBuffers):
 
     def forward(self, input_incr, prev_state):
         """new_state = prev_state + mult(out - prev_state, update)  (reference :47-69)."""
-        if (self.fuse and self.stacked and prev_state is None and not self.update_gate.use_kf
-                and not self.out_gate.use_kf and self.sigmoid1.in_res.reservoir is not None):
+        if (self.fuse and self.stacked and prev_state is None and not self.update_gate.lossy
+                and not self.out_gate.lossy and self.sigmoid1.in_res.reservoir is not None):
             new_state = self._forward_stacked(input_incr)
             self.__dict__["_mult_stale"] = True       # self.mult's reservoirs have missed this step
             return new_state, new_state

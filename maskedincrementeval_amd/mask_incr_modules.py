@@ -128,11 +128,15 @@ class KFencedMaskModule(IncrementMaskModule):
     every nnConvIncr but never calls its forward (:166).
     """
 
-    def __init__(self, tp: float = .1):
+    def __init__(self, tp: float = .1, norm: str = "l2"):
         super().__init__()
         self.delta = IncrementReserve()
         self.tp = tp
         self.k = tp
+        # "l2": k = tp * ||x||_2 over the whole tensor, the reference's rule (:45), which grows with the
+        # square root of the tensor size; "rms": k = tp * ||x||_2 / sqrt(numel), a step relative to the
+        # typical magnitude of an element
+        self.norm = norm
 
     def floor_by_k(self, T):
         return self.k * torch.floor(0.5 + T / self.k)
@@ -154,7 +158,11 @@ class KFencedMaskModule(IncrementMaskModule):
         return [out, self._view("refined", ts, pix)]
 
     def forward_refresh_reservoirs(self, x: DenseT) -> DenseT:
-        k = (self.tp * torch.norm(x.detach())).reshape(1).float()
+        k = (self.tp * torch.norm(x.detach().float())).reshape(1)
+        if self.norm == "rms":
+            k = k / float(x.numel()) ** 0.5
+        elif self.norm != "l2":
+            raise ValueError("KFencedMaskModule.norm must be 'l2' or 'rms', got %r" % (self.norm,))
         if isinstance(self.k, torch.Tensor) and self.k.device == k.device:
             self.k.copy_(k)
         else:
@@ -459,6 +467,10 @@ class nnConvIncr(nn.Conv2d, _ConvIncrMixin):
         nn.Conv2d.__init__(self, in_channels, out_channels, kernel_size, stride, padding, bias=bias)
         self.kf = KFencedMaskModule(0.3)
         self.use_kf = False          # the reference leaves the quantiser switched off (:166)
+        # Lossy input mask: pixels whose delta stays within +-in_threshold in every channel are dropped from
+        # the input mask (the reference's mask definition, maxpool(abs(x)) >= thr with field 1,
+        # incr_modules/utils.py:22-25); None = exact masks.  What is dropped is lost (no carry).
+        self.in_threshold = None
         self.path = _lib.PATH_AUTO
 
     def load_state_dict(self, state_dict, strict: bool = True):
@@ -466,16 +478,28 @@ class nnConvIncr(nn.Conv2d, _ConvIncrMixin):
         self.__dict__.pop("_filt_cache", None)
         return ret
 
-    def forward(self, x_incr, x2_incr=None):
+    @property
+    def lossy(self) -> bool:
+        return self.use_kf or self.in_threshold is not None
+
+    def lossy_input(self, x_incr):
+        """The delta quantiser and / or the threshold mask in front of the conv (both off by default)."""
         if self.use_kf:
             x_incr = self.kf(x_incr)
-        return self._incr_forward(x_incr, x2_incr, path=self.path)
+        if self.in_threshold is not None:
+            x = ops.as_nhwc(x_incr[0])
+            n, _, h, w = x.shape
+            pix = ops.mask_from_delta(x, float(self.in_threshold), self._pix_buf("thr_in", n, h, w, x.device))
+            x_incr = [x, pix]
+        return x_incr
+
+    def forward(self, x_incr, x2_incr=None):
+        return self._incr_forward(self.lossy_input(x_incr), x2_incr, path=self.path)
 
     def forward_fused(self, x_incr, activation: "nnReservedActivation", x2_incr=None,
                       addend_incr=None, filt=None):
         """conv (+ addend) + activation increment in one kernel; updates activation.in_res in place."""
-        if self.use_kf:
-            x_incr = self.kf(x_incr)
+        x_incr = self.lossy_input(x_incr)
         kind, slope = activation_kind(activation.op)
         res = activation.in_res.reservoir
         if res is None:
@@ -497,7 +521,7 @@ class nnConvIncr(nn.Conv2d, _ConvIncrMixin):
         tiles = x.shape[0] * ((2 * x.shape[2] + 7) // 8) * ((2 * x.shape[3] + 7) // 8)
         chunks = x.shape[1] // ops.mfma_chunk(dt)
         small = dt == torch.bfloat16 or (tiles <= ops.upconv_max_tiles and chunks <= ops.upconv_max_chunks)
-        if self.use_kf or not small or not ops.upconv_takes(x.shape[1], self.out_channels, k, s, p,
+        if self.lossy or not small or not ops.upconv_takes(x.shape[1], self.out_channels, k, s, p,
                                                             self.conv2d_weights, dt):
             return self.forward_fused(up(x_incr, skip_incr), activation)
         kind, slope = activation_kind(activation.op)
@@ -520,15 +544,27 @@ class nnConvIncr(nn.Conv2d, _ConvIncrMixin):
         return self._refresh_forward(x, x2, activation, path=self.path, addend=addend)
 
 
-def set_kfence(net: nn.Module, tp: Optional[float]) -> int:
-    """Switch the delta quantiser of every nnConvIncr in `net` on (threshold factor tp, k = tp*||x||
-    at the next refresh) or off (tp None).  Returns the number of convs touched; refresh afterwards."""
+def set_kfence(net: nn.Module, tp: Optional[float], norm: str = "l2") -> int:
+    """Switch the delta quantiser of every nnConvIncr in `net` on (threshold factor tp; at the next refresh
+    k = tp*||x||_2, or tp*||x||_2/sqrt(numel) with norm="rms") or off (tp None).  Returns the number of convs
+    touched; refresh afterwards."""
     count = 0
     for m in net.modules():
         if isinstance(m, nnConvIncr):
             m.use_kf = tp is not None
             if tp is not None:
                 m.kf.tp = float(tp)
+                m.kf.norm = norm
+            count += 1
+    return count
+
+
+def set_input_threshold(net: nn.Module, thr: Optional[float]) -> int:
+    """Threshold mask in front of every nnConvIncr of `net` (None: exact masks).  Returns the number of convs."""
+    count = 0
+    for m in net.modules():
+        if isinstance(m, nnConvIncr):
+            m.in_threshold = None if thr is None else float(thr)
             count += 1
     return count
 

@@ -10,6 +10,7 @@ from maskedincrementeval_amd.masked_types import TileMask
 from maskedincrementeval_amd.synthetic import blob_mask, gaussian_delta, he_normal_conv_weight
 from oracle import incr_oracle as io
 from oracle import mask_oracle as mo
+from tolerances import BF16_RTOL, bf16_atol
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -212,7 +213,7 @@ def test_tconv2x_matrix_core_form(c1, c2, cout, h, w, k, dtype):
     out = ops.new_nhwc(n, cout, ho, wo, DEV, dtype)
     r0 = torch.randn(n, cout, ho, wo, generator=torch.Generator().manual_seed(5))
     res_gpu, res_cpu = _dev(r0.clone()), io.Reserve(r0.clone())
-    tol = dict(rtol=RTOL, atol=ATOL) if dtype == torch.float32 else dict(rtol=2 ** -7, atol=2 ** -7)
+    tc_tol = dict(rtol=RTOL, atol=ATOL) if dtype == torch.float32 else dict(rtol=2 ** -7, atol=2 ** -7)
     for step, dens in enumerate((0.10, 0.03, 0.25)):
         d1, m1 = gaussian_delta(n, c1, h, w, dens, 0.5, seed=900 + step)
         d1 = rnd(d1)
@@ -238,7 +239,7 @@ def test_tconv2x_matrix_core_form(c1, c2, cout, h, w, k, dtype):
         ref = io.act_incr(torch.relu, res_cpu, io.tconv_incr(full, wt, 2, p, 1) + add)
         got = out.float().cpu()
         assert torch.isfinite(got).all()
-        assert torch.allclose(got, ref, **tol), "step %d max|diff| %.3e" % (step, (got - ref).abs().max())
+        assert torch.allclose(got, ref, **tc_tol), "step %d max|diff| %.3e" % (step, (got - ref).abs().max())
         assert torch.allclose(res_gpu.cpu(), res_cpu.reservoir, rtol=RTOL, atol=ATOL if dtype == torch.float32 else 1e-4)
         outside = ~torch.from_numpy(want_mask).bool().unsqueeze(1)
         assert torch.count_nonzero(got * outside) == 0          # clean delta, stale blocks zeroed
@@ -329,7 +330,7 @@ def test_pack_filter_layout_and_row_views():
 @pytest.mark.parametrize("c,cout,h,w", [(64, 32, 13, 17), (64, 64, 70, 90), (128, 128, 88, 80), (64, 96, 9, 40)])
 def test_upsampled_conv_in_one_kernel(c, cout, h, w, dtype):
     bf = dtype == torch.bfloat16
-    tol = dict(rtol=2e-2, atol=2e-2) if bf else dict(rtol=RTOL, atol=1e-4)
+    tol = (lambda ref: dict(rtol=BF16_RTOL, atol=bf16_atol(ref, 2.0))) if bf else (lambda ref: dict(rtol=RTOL, atol=ATOL))
     q = (lambda t: t.to(torch.bfloat16).float()) if bf else (lambda t: t)
     wt = q(he_normal_conv_weight(cout, c, 5, 9))
     filt = _filt(wt)
@@ -358,9 +359,9 @@ def test_upsampled_conv_in_one_kernel(c, cout, h, w, dtype):
         got = out.float().cpu()
         assert torch.isfinite(got).all()
         want = torch.relu(r0 + ref) - torch.relu(r0) if with_res else ref
-        assert torch.allclose(got, want, **tol), "step %d max|diff| = %.3e" % (step, (got - want).abs().max())
+        assert torch.allclose(got, want, **tol(want)), "step %d max|diff| = %.3e" % (step, (got - want).abs().max())
         if with_res:
-            assert torch.allclose(res.cpu(), r0 + ref, rtol=RTOL, atol=2e-2 if bf else 1e-4)
+            assert torch.allclose(res.cpu(), r0 + ref, rtol=RTOL, atol=bf16_atol(ref, 2.0) if bf else ATOL)
 
 
 # The same for a single input of very few channels (the flow estimate in front of an EVFlowNet decoder): 3x3 and 5x5.
@@ -368,7 +369,7 @@ def test_upsampled_conv_in_one_kernel(c, cout, h, w, dtype):
 @pytest.mark.parametrize("c,cout,k,h,w", [(2, 64, 3, 13, 17), (2, 32, 3, 32, 32), (5, 96, 5, 9, 40), (8, 32, 3, 21, 11)])
 def test_upsampled_conv_few_channels(c, cout, k, h, w, dtype):
     bf = dtype == torch.bfloat16
-    tol = dict(rtol=2e-2, atol=2e-2) if bf else dict(rtol=RTOL, atol=5e-5)
+    tol = (lambda ref: dict(rtol=BF16_RTOL, atol=bf16_atol(ref, 2.0))) if bf else (lambda ref: dict(rtol=RTOL, atol=ATOL))
     q = (lambda t: t.to(torch.bfloat16).float()) if bf else (lambda t: t)
     n, p = 2, k // 2
     wt = q(he_normal_conv_weight(cout, c, k, 19))
@@ -388,7 +389,7 @@ def test_upsampled_conv_few_channels(c, cout, k, h, w, dtype):
         torch.cuda.synchronize()
         got = out.float().cpu()
         assert torch.isfinite(got).all()
-        assert torch.allclose(got, ref, **tol), "step %d max|diff| = %.3e" % (step, (got - ref).abs().max())
+        assert torch.allclose(got, ref, **tol(ref)), "step %d max|diff| = %.3e" % (step, (got - ref).abs().max())
 
 
 def _random_cases(count, seed):
@@ -415,7 +416,7 @@ def _random_cases(count, seed):
 def test_seeded_random_shapes(case, dtype):
     i, k, s, pad, cin, cout, n, h, w, dens = case
     bf = dtype == torch.bfloat16
-    tol = dict(rtol=2e-2, atol=2e-2) if bf else dict(rtol=RTOL, atol=5e-5)
+    tol = (lambda ref: dict(rtol=BF16_RTOL, atol=bf16_atol(ref, 2.0))) if bf else (lambda ref: dict(rtol=RTOL, atol=ATOL))
     q = (lambda t: t.to(torch.bfloat16).float()) if bf else (lambda t: t)
     wt = q(he_normal_conv_weight(cout, cin, k, 50 + i))
     filt = _filt(wt)
@@ -431,7 +432,7 @@ def test_seeded_random_shapes(case, dtype):
         ops.conv_masked(_dev(d).to(dtype), dm, None, None, filt, k, s, pad, ts, out)
         torch.cuda.synchronize()
         got = out.float().cpu()
-        assert torch.allclose(got, ref, **tol), "step %d max|diff| = %.3e" % (step, (got - ref).abs().max())
+        assert torch.allclose(got, ref, **tol(ref)), "step %d max|diff| = %.3e" % (step, (got - ref).abs().max())
         foot = torch.from_numpy(mo.footprint_conv(m[:, 0].numpy(), k, s, pad)).bool().unsqueeze(1)
         assert torch.count_nonzero(got * (~foot)) == 0
 
@@ -449,7 +450,7 @@ def test_small_planes_split_the_contraction(c1, c2, cout, h, w, s, dtype, k):
     bf = dtype == torch.bfloat16
     if bf and (c1 % 64 or c2 % 64 or (c1 + c2) // 64 < 4):
         pytest.skip("fewer than 4 staged chunks of 64 bf16 channels: not split")
-    tol = dict(rtol=2e-2, atol=2e-2) if bf else dict(rtol=RTOL, atol=5e-5)
+    tol = (lambda ref: dict(rtol=BF16_RTOL, atol=bf16_atol(ref, 2.0))) if bf else (lambda ref: dict(rtol=RTOL, atol=ATOL))
     q = (lambda t: t.to(torch.bfloat16).float()) if bf else (lambda t: t)
     n, cin = 1, c1 + c2
     wt = q(he_normal_conv_weight(cout, cin, k, 21))
@@ -486,10 +487,10 @@ def test_small_planes_split_the_contraction(c1, c2, cout, h, w, s, dtype, k):
             res_ref = res_ref + acc
         else:
             want = ref
-        assert torch.allclose(got, want, **tol), "step %d max|diff| = %.3e" % (step, (got - want).abs().max())
-        assert torch.allclose(got, plain, **tol), "step %d split vs unsplit %.3e" % (step, (got - plain).abs().max())
+        assert torch.allclose(got, want, **tol(want)), "step %d max|diff| = %.3e" % (step, (got - want).abs().max())
+        assert torch.allclose(got, plain, **tol(plain)), "step %d split vs unsplit %.3e" % (step, (got - plain).abs().max())
         if with_res:
-            assert torch.allclose(res.cpu(), res_ref, rtol=RTOL, atol=2e-2 if bf else 1e-4)
+            assert torch.allclose(res.cpu(), res_ref, rtol=RTOL, atol=bf16_atol(ref, 2.0) if bf else ATOL)
     # the split form ran: its partial sums replaced the NaN fill of the first planes
     plane = n * ho * wo * cout
     assert torch.isfinite(ws[:plane]).any() and torch.isfinite(ws[plane:2 * plane]).any()
@@ -503,7 +504,7 @@ def test_small_planes_split_the_contraction(c1, c2, cout, h, w, s, dtype, k):
 @pytest.mark.parametrize("cin,cout", [(1, 32), (2, 64), (4, 64), (5, 32), (7, 96), (8, 32)])
 def test_few_input_channels_matrix_core_kernel(cin, cout, k, s, dtype):
     bf = dtype == torch.bfloat16
-    tol = dict(rtol=2e-2, atol=2e-2) if bf else dict(rtol=RTOL, atol=5e-5)
+    tol = (lambda ref: dict(rtol=BF16_RTOL, atol=bf16_atol(ref, 2.0))) if bf else (lambda ref: dict(rtol=RTOL, atol=ATOL))
     q = (lambda t: t.to(torch.bfloat16).float()) if bf else (lambda t: t)
     n, h, w, p = 2, 29, 43, k // 2
     wt = q(he_normal_conv_weight(cout, cin, k, 60 + cin))
@@ -529,8 +530,8 @@ def test_few_input_channels_matrix_core_kernel(cin, cout, k, s, dtype):
         if with_res:
             res_ref = res_ref + ref
         assert torch.isfinite(got).all()
-        assert torch.allclose(got, want, **tol), "step %d max|diff| = %.3e" % (step, (got - want).abs().max())
-        assert torch.allclose(got, valu, **tol), "step %d vs VALU %.3e" % (step, (got - valu).abs().max())
+        assert torch.allclose(got, want, **tol(want)), "step %d max|diff| = %.3e" % (step, (got - want).abs().max())
+        assert torch.allclose(got, valu, **tol(valu)), "step %d vs VALU %.3e" % (step, (got - valu).abs().max())
         foot = torch.from_numpy(mo.footprint_conv(m[:, 0].numpy(), k, s, p)).bool().unsqueeze(1)
         assert torch.count_nonzero(got * (~foot)) == 0
-    assert torch.allclose(res.cpu(), res_ref, rtol=RTOL, atol=2e-2 if bf else 1e-4)
+    assert torch.allclose(res.cpu(), res_ref, rtol=RTOL, atol=bf16_atol(ref, 2.0) if bf else ATOL)

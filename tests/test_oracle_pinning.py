@@ -294,6 +294,66 @@ def test_e2depth_oracle_accumulation_identity():
     assert torch.allclose(acc, dense, atol=2e-5)
 
 
+def _twin_state(model, twin):
+    """The parameters of an incremental network, loaded strictly into its independent twin."""
+    sd = {k: v for k, v in model.state_dict().items()}
+    twin.load_state_dict(sd, strict=True)          # every parameter name and shape of the module tree
+    return sd
+
+
+def test_e2depth_topology_against_reference_trace_and_independent_twin():
+    # The whole-net oracle's topology, pinned three ways that do not share its code: (1) the incremental
+    # network's state_dict loads strictly into a twin written from plain nn.Conv2d modules; (2) that twin's
+    # conv-by-conv shapes at 1x5x264x352 are the reference's own trace (todo.txt:34-57); (3) the oracle's dense
+    # refresh AND refresh + increments equal the twin's forward -- a skip sum, gate order or residual dropped in
+    # both halves of the oracle cannot hide behind the accumulation identity.
+    from dense_twins import E2DEPTH_CONV_TRACE, E2DepthTwin, conv_trace
+    from maskedincrementeval_amd.e2depth_incr import E2VIDRecurrentIncr
+    from maskedincrementeval_amd.synthetic import event_voxel_delta, seed_module_
+    model = seed_module_(E2VIDRecurrentIncr(), seed=5)
+    twin = E2DepthTwin().eval()
+    params = _twin_state(model, twin)
+    assert conv_trace(twin, torch.zeros(1, 5, 264, 352)) == E2DEPTH_CONV_TRACE
+    net = E2DepthOracle(params)
+    x = _rand(1, 5, 40, 56, seed=210, scale=0.5)
+    with torch.no_grad():
+        assert torch.allclose(net.refresh(x), twin(x), rtol=1e-4, atol=1e-5)
+        acc = net.refresh(x)
+        for t in range(3):
+            d, _ = event_voxel_delta(1, 5, 40, 56, 0.1, seed=220 + t)
+            acc = acc + net.incr(d)
+            x = x + d
+        assert torch.allclose(acc, twin(x), rtol=1e-4, atol=1e-5)
+        # the twin is sensitive to what it pins: without the head skip the prediction moves
+        u = twin.unetrecurrent
+        assert not torch.allclose(twin(x), torch.sigmoid(u.pred.conv2d(torch.zeros(1, 32, 40, 56))), atol=1e-3)
+
+
+@pytest.mark.parametrize("decoder", ["upsample", "transposed"])
+def test_evflownet_topology_against_independent_twin(decoder):
+    from dense_twins import EVFlowNetTwin
+    from maskedincrementeval_amd.evflownet_incr import MultiResUNetRecurrentIncr
+    from maskedincrementeval_amd.synthetic import seed_module_
+    from oracle.evflownet_oracle import EVFlowNetOracle
+    model = seed_module_(MultiResUNetRecurrentIncr(num_bins=4, decoder=decoder), seed=6)
+    twin = EVFlowNetTwin(decoder=decoder).eval()
+    params = _twin_state(model, twin)
+    net = EVFlowNetOracle(params, decoder=decoder)
+    x = _rand(1, 4, 32, 48, seed=230, scale=0.5)
+    with torch.no_grad():
+        flows = twin(x)
+        for a, b in zip(net.refresh(x), flows):
+            assert torch.allclose(a, b, rtol=1e-4, atol=1e-5)
+        net = EVFlowNetOracle(params, decoder=decoder)     # (a second refresh of one instance would start from the first one's state)
+        acc = [p.clone() for p in net.refresh(x)]
+        for t in range(3):
+            d = _rand(1, 4, 32, 48, seed=240 + t, scale=0.2) * (torch.rand(1, 1, 32, 48, generator=torch.Generator().manual_seed(t)) < 0.1)
+            acc = [a + b for a, b in zip(acc, net.incr(d))]
+            x = x + d
+        for a, b in zip(acc, twin(x)):
+            assert torch.allclose(a, b, rtol=1e-4, atol=2e-5)
+
+
 @pytest.mark.parametrize("decoder", ["upsample", "transposed"])
 def test_evflownet_oracle_accumulation_identity(decoder):
     # refresh(x0) + sum of increments == dense(x_T) at every flow scale (zero recurrent state)
