@@ -451,9 +451,9 @@ int mie_convgru_gates_incr(const void* gates_delta, float* update_res,
  * otherwise MIE_ERR_UNSUPPORTED (use the two calls then).
  *   filter / filter_mc / gates_res : the 4*hid output columns are NOT in the
  *     order [in | remember | out | cell] x hid of the two-call form but
- *     interleaved by gate in groups of 8 hidden channels: column
- *     32*b + 8*g + j  <->  gate g of hidden channel 8*b + j, so that one
- *     workgroup owns all four gates of its hidden channels.  gates_res
+ *     interleaved by gate: column 4*hc + g  <->  gate g of hidden channel hc,
+ *     so that one workgroup owns all four gates of its hidden channels and
+ *     reads / writes them as one 16-byte access.  gates_res
  *     ([n,h,w,4*hid]) lives in that order too (a refresh through
  *     mie_conv_refresh with the same filter and a bias in the same order fills
  *     it consistently).

@@ -139,19 +139,29 @@ bool mie_launch_conv_fewcin_up(const ConvArgsT<mie_bf16>& a, int k, unsigned cap
 // returns the deltas of the hidden and the cell state (the chain sigmoid1..3 / tanh1 -> m1 + m2 -> tanh2
 // -> m3 of ConvLSTMIncr.forward, incr_modules/e2depth_incr.py:103-120, product rule on cached operands).
 static __device__ __forceinline__ float mie_sigm(float v) { return 1.f / (1.f + expf(-v)); }
+// Gate chain: sigmoid and tanh through the hardware exponential (v_exp_f32) and reciprocal (v_rcp_f32), about
+// 1e-7 absolute error each -- far inside the 1e-5 the results are held to -- at a third of the instructions
+// of expf / tanhf / IEEE division; with ten evaluations per (pixel, hidden channel) the chain was bound by
+// them.  The same functions serve the dense refresh, so that refresh and increments see one sigmoid.
+static __device__ __forceinline__ float mie_gate_sigm(float v) {
+  return __builtin_amdgcn_rcpf(1.f + __expf(-v));
+}
+static __device__ __forceinline__ float mie_gate_tanh(float v) {
+  return 1.f - 2.f * __builtin_amdgcn_rcpf(1.f + __expf(2.f * v));     // exp overflow -> rcp(inf) = 0 -> 1
+}
 static __device__ __forceinline__ void mie_lstm_gate_chain(float& ri, float& rf, float& ro, float& rg, float di,
                                                            float df, float dO, float dG, float& cp, float dP,
                                                            float& cc, float& dh, float& dc) {
   const float ri1 = ri + di, rf1 = rf + df, ro1 = ro + dO, rg1 = rg + dG;
-  const float si0 = mie_sigm(ri), dsi = mie_sigm(ri1) - si0;
-  const float sf0 = mie_sigm(rf), dsf = mie_sigm(rf1) - sf0;
-  const float so0 = mie_sigm(ro), dso = mie_sigm(ro1) - so0;
-  const float tg0 = tanhf(rg), dtg = tanhf(rg1) - tg0;
+  const float si0 = mie_gate_sigm(ri), dsi = mie_gate_sigm(ri1) - si0;
+  const float sf0 = mie_gate_sigm(rf), dsf = mie_gate_sigm(rf1) - sf0;
+  const float so0 = mie_gate_sigm(ro), dso = mie_gate_sigm(ro1) - so0;
+  const float tg0 = mie_gate_tanh(rg), dtg = mie_gate_tanh(rg1) - tg0;
   const float m1 = (dtg + tg0) * dsi + si0 * dtg;       // m1(in_gate, cell_gate)
   const float m2 = (dP + cp) * dsf + sf0 * dP;          // m2(remember_gate, prev_c)
   const float dcell = m1 + m2;
   const float c0 = cc, c1 = c0 + dcell;
-  const float tc0 = tanhf(c0), dtc = tanhf(c1) - tc0;
+  const float tc0 = mie_gate_tanh(c0), dtc = mie_gate_tanh(c1) - tc0;
   dh = (dtc + tc0) * dso + so0 * dtc;                   // m3(out_gate, tanh(cell))
   dc = dcell;
   ri = ri1; rf = rf1; ro = ro1; rg = rg1;

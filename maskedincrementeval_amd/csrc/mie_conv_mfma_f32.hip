@@ -22,3 +22,12 @@ bool mie_launch_conv_gates_mfma(const ConvArgsT<float>& a, unsigned cap, hipStre
 bool mie_launch_conv_up_mfma(const ConvArgsT<float>& a, unsigned cap, hipStream_t st) {
   return launch_up<float>(a, cap, st);
 }
+
+#ifdef MIE_WG_PROFILE
+// Measurement builds only: where the fp32 kernels of this translation unit write their workgroup timelines
+// (NULL switches the stamps off).  The buffer needs 128 bytes per workgroup of the launches it covers.
+extern "C" __attribute__((visibility("default"))) int mie_set_profile_buffer(void* p) {
+  long long* q = (long long*)p;
+  return hipMemcpyToSymbol(HIP_SYMBOL(mie_prof_buf), &q, sizeof(q)) == hipSuccess ? 0 : -4;
+}
+#endif

@@ -46,10 +46,33 @@
 #pragma once
 #include "mie_conv.h"
 #include <stdlib.h>
+#include <type_traits>
 
 namespace {
 
 typedef float v16f __attribute__((ext_vector_type(16)));
+#ifndef MIE_PIPE
+#define MIE_PIPE 1
+#endif
+
+// Build-time instrumentation (-DMIE_WG_PROFILE, measurement builds only): thread 0 of every workgroup
+// records the 100 MHz device clock at the stages of its life into a buffer handed over with
+// mie_set_profile_buffer, 16 slots per workgroup (slot 15 = number of stamps).  Compiled out otherwise.
+#ifdef MIE_WG_PROFILE
+static __device__ long long* mie_prof_buf;       // set by mie_set_profile_buffer (measurement builds only)
+#define MIE_STAMP(k)                                                                                   \
+  do {                                                                                                 \
+    if (mie_prof_buf != nullptr && threadIdx.x == 0 && (k) < 15) {                                     \
+      long long* slot_ = mie_prof_buf + (((long long)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 16; \
+      slot_[(k)] = (long long)wall_clock64();                                                          \
+      if ((k) == 0) slot_[12] = (long long)clock64();                                                  \
+      if ((k) == 14) slot_[13] = (long long)clock64();                                                 \
+      slot_[15] = (k) + 1;                                                                             \
+    }                                                                                                  \
+  } while (0)
+#else
+#define MIE_STAMP(k) do { } while (0)
+#endif
 
 // fp32 channels staged in LDS per chunk (bf16: twice as many), by kernel size and stride, bounded
 // by 64 KB of LDS.  Stride 1 double-buffers the staged tile of (7+K)^2 pixels.  Stride 2 tiles
@@ -100,6 +123,23 @@ __device__ __forceinline__ void mma_unit(v16f& acc, const float4& av, const floa
   const v4f a4 = {av.x, av.y, av.z, av.w}, b4 = {bv.x, bv.y, bv.z, bv.w};
   acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(mie_bf16x8, a4),
                                                 __builtin_bit_cast(mie_bf16x8, b4), acc, 0, 0, 0);
+}
+
+// The same for the two pixel blocks of a tile against one B operand, the k-steps of the two accumulators
+// interleaved: consecutive MFMAs are independent, so none waits for the result of the one before it.
+__device__ __forceinline__ void mma_unit2(v16f& acc0, v16f& acc1, const float4& a0, const float4& a1, const float4& bv, float) {
+  acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.x, bv.x, acc0, 0, 0, 0);
+  acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1.x, bv.x, acc1, 0, 0, 0);
+  acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.y, bv.y, acc0, 0, 0, 0);
+  acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1.y, bv.y, acc1, 0, 0, 0);
+  acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.z, bv.z, acc0, 0, 0, 0);
+  acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1.z, bv.z, acc1, 0, 0, 0);
+  acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.w, bv.w, acc0, 0, 0, 0);
+  acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1.w, bv.w, acc1, 0, 0, 0);
+}
+__device__ __forceinline__ void mma_unit2(v16f& acc0, v16f& acc1, const float4& a0, const float4& a1, const float4& bv, mie_bf16) {
+  mma_unit(acc0, a0, bv, mie_bf16());
+  mma_unit(acc1, a1, bv, mie_bf16());
 }
 
 // One 16-byte slot of delta elements <-> fp32 values (4 of them, or 8 for bf16).
@@ -178,6 +218,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   // (one more dependent load at the start of a workgroup: measured, it costs nothing even on launches
   // of a few dozen workgroups), and idle positions of the capacity-sized grid fall off the end.
   // (For the SPLIT launches the same idea, one filter slice per XCD, was measured: no gain.)
+  MIE_STAMP(0);
   int bx = blockIdx.x, by = blockIdx.y;
   const int bz = SPLIT ? (int)blockIdx.z : 0;
   int n, y0, x0, tk;
@@ -213,6 +254,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
     tk = mie_pick_tile(a.ts, bx, n, y0, x0);
   }
   if (tk == 0) return;
+  MIE_STAMP(1);
   const int tid = threadIdx.x;
   // wave index as a scalar: everything derived from it (k-split, channel slab) stays in SGPRs
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
@@ -479,17 +521,25 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   const int c_hi = SPLIT ? (bz + 1) * nch / (int)gridDim.z : nch;
   const T* ub_cur = chunk_b(c_lo);
   const T* ub_next = ub_cur;
+  MIE_STAMP(2);
   stage_load(c_lo);
 #pragma unroll
   for (int i = 0; i < (PD > 0 ? PD : 1); ++i) load_b(ub_cur, i, bring[i % RING]);
   stage_store(0);
   __syncthreads();
+  MIE_STAMP(3);
 
+  // Double-buffered kernels pipeline the chunk hand-over into the contraction: the next chunk's global loads
+  // (and their address arithmetic) are issued once the first unit's MFMAs are in flight, and its LDS stores
+  // go out under the MFMAs of the last unit, so that between two chunks the matrix cores only wait for the
+  // barrier and the first operand read.  (Without it every boundary idled them for about 0.5 us: stores,
+  // barrier, some 70 address instructions, loads, first LDS read, all after the last MFMA had been issued.)
+  constexpr bool PIPE = MIE_PIPE && NBUF == 2 && !UP && UPC >= 4;
   for (int c = c_lo; c < c_hi; ++c) {
     const bool more = c + 1 < c_hi;
     const int cn = more ? c + 1 : c;      // after the last chunk: redundant re-load, never stored
     ub_next = chunk_b(cn);
-    stage_load(cn);
+    if (!PIPE) stage_load(cn);
     const T* sin = sbuf + ((c - c_lo) % NBUF) * STAGE;
     // A operands are read one unit ahead as well (two register sets); the scheduling barriers
     // pin "issue the loads for later units, then multiply this unit" so that the compiler can
@@ -507,24 +557,41 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
 #pragma unroll
     for (int i = 0; i < UPC; ++i) {
       // B operands of the unit PD ahead (the first units of the next chunk at the end)
+#ifndef MIE_EXP_NOB
       if (PD > 0) {
         const int ip = i + PD;
         if (ip < UPC) load_b(ub_cur, ip, bring[ip % RING]);
         else load_b(ub_next, ip - UPC, bring[ip % RING]);
       }
+#endif
+#ifndef MIE_EXP_NOA
       if (i + 1 < UPC) load_a(i + 1, av[(i + 1) & 1]);
+#endif
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mb = 0; mb < 2; ++mb) mma_unit(acc[mb][nb], av[i & 1][mb], bring[i % RING][nb], T());
+      for (int nb = 0; nb < NB; ++nb) mma_unit2(acc[0][nb], acc[1][nb], av[i & 1][0], av[i & 1][1], bring[i % RING][nb], T());
       __builtin_amdgcn_sched_barrier(0);
       if (PD == 0) load_b(ub_next, 0, bring[0]);   // ring of one: reload right after use
+#ifndef MIE_EXP_NOSTAGE
+      if (PIPE && i == 0) {
+        stage_load(cn);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (PIPE && i == UPC - 2) {
+        if (more) stage_store((c - c_lo + 1) % NBUF);    // the other buffer: nobody reads it during this chunk
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#endif
     }
-    if (NBUF == 1 && !UP) __syncthreads();   // every wave is done reading the only buffer (UP: stage_store syncs)
-    if (more) stage_store((c - c_lo + 1) % NBUF);
+    if (!PIPE) {
+      if (NBUF == 1 && !UP) __syncthreads();   // every wave is done reading the only buffer (UP: stage_store syncs)
+      if (more) stage_store((c - c_lo + 1) % NBUF);
+    }
+#ifndef MIE_EXP_NOBARRIER
     __syncthreads();
+#endif
     ub_cur = ub_next;
+    MIE_STAMP(4 + (c - c_lo));
   }
   const int cob = cob0 + l32;
 
@@ -532,11 +599,10 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   // acc[mb][nb][r] of this lane is output pixel p = 32*mb + 8*(r/4) + 4*half + r%4,
   // channel column wn*32*NB + 32*nb + lane%32 of the workgroup's slab.
   if constexpr (GATES) {
-    // ConvLSTM gate chain as the epilogue.  The filter columns of a slab are interleaved by gate in
-    // groups of 8 hidden channels: column 32*b + 8*g + j of the slab is gate g (in, remember, out,
-    // cell) of hidden channel 8*b + j, so a workgroup owns all four gates of its CO_BLK/4 hidden
-    // channels.  Every wave parks its accumulators in LDS; a thread then sums the k-split partials
-    // of the four gate columns of one (pixel, hidden channel) and runs the chain on the reservoirs.
+    // ConvLSTM gate chain as the epilogue.  The filter columns are interleaved by gate: column 4*hc + g is
+    // gate g (in, remember, out, cell) of hidden channel hc, so a workgroup owns all four gates of its
+    // CO_BLK/4 hidden channels.  Every wave parks its accumulators in LDS; a thread then sums the k-split
+    // partials of the four gate columns of one (pixel, hidden channel) and runs the chain on the reservoirs.
     float* red = smem + wk * (64 * CO_BLK);
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb)
@@ -564,22 +630,21 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
         mie_st(a.g_dc, ho, 0.f);
         continue;
       }
-      const int colb = (hc >> 3) * 32 + (hc & 7);
-      float dg[4];
+      // the four gates of a hidden channel are four adjacent columns: one 16-byte access each for the k-split
+      // partials in LDS and for the gate reservoir
+      float4 dg = *reinterpret_cast<const float4*>(&smem[p * CO_BLK + 4 * hc]);
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        float sum = smem[p * CO_BLK + colb + 8 * g];
-#pragma unroll
-        for (int k2 = 1; k2 < WK; ++k2) sum += smem[k2 * (64 * CO_BLK) + p * CO_BLK + colb + 8 * g];
-        dg[g] = sum;
+      for (int k2 = 1; k2 < WK; ++k2) {
+        const float4 part = *reinterpret_cast<const float4*>(&smem[k2 * (64 * CO_BLK) + p * CO_BLK + 4 * hc]);
+        dg.x += part.x; dg.y += part.y; dg.z += part.z; dg.w += part.w;
       }
-      float* gr = a.res + pix * a.cout + co0 + colb;
-      float ri = gr[0], rf = gr[8], ro = gr[16], rg = gr[24];
+      float4* gr = reinterpret_cast<float4*>(a.res + pix * a.cout + co0 + 4 * hc);
+      float4 rr = *gr;
       const bool has_cp = a.g_cpd != nullptr && (a.g_cpm == nullptr || a.g_cpm[pix]);
       const float dP = has_cp ? mie_ld(a.g_cpd, ho) : 0.f;
       float cp = a.g_cpres[ho], cc = a.g_cres[ho], dh, dc;
-      mie_lstm_gate_chain(ri, rf, ro, rg, dg[0], dg[1], dg[2], dg[3], cp, dP, cc, dh, dc);
-      gr[0] = ri; gr[8] = rf; gr[16] = ro; gr[24] = rg;
+      mie_lstm_gate_chain(rr.x, rr.y, rr.z, rr.w, dg.x, dg.y, dg.z, dg.w, cp, dP, cc, dh, dc);
+      *gr = rr;
       if (has_cp) a.g_cpres[ho] = cp;
       a.g_cres[ho] = cc;
       mie_st(a.g_dh, ho, dh);
@@ -643,6 +708,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
       conv_epilogue_store<T, PER>(a, e_off, e_co, e_ok, v, e_r0, e_add);
     }
   }
+  MIE_STAMP(14);
 }
 
 // Second half of a SPLIT launch: per active tile the `parts` partial planes are added in order and

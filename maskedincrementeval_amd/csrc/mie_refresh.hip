@@ -18,18 +18,18 @@ __global__ __launch_bounds__(256) void k_convlstm_gates_refresh(
   if (idx >= total) return;
   const long long pix = idx / hid;
   const int hc = (int)(idx - pix * hid);
-  // gate columns of this hidden channel: [in | remember | out | cell] x hid, or interleaved by gate in
-  // groups of 8 hidden channels (column 32*b + 8*g + j <-> gate g of hidden channel 8*b + j)
-  const int col0 = interleaved ? ((hc >> 3) * 32 + (hc & 7)) : hc;
-  const int step = interleaved ? 8 : hid;
+  // gate columns of this hidden channel: [in | remember | out | cell] x hid, or interleaved by gate
+  // (column 4*hc + g <-> gate g of hidden channel hc)
+  const int col0 = interleaved ? 4 * hc : hc;
+  const int step = interleaved ? 1 : hid;
   const float* g = gates_res + pix * (4LL * hid) + col0;
-  const float gi = mie_sigm(g[0]), gf = mie_sigm(g[step]), go = mie_sigm(g[2 * step]);
-  const float gg = tanhf(g[3 * step]);
+  const float gi = mie_gate_sigm(g[0]), gf = mie_gate_sigm(g[step]), go = mie_gate_sigm(g[2 * step]);
+  const float gg = mie_gate_tanh(g[3 * step]);
   const float cp = prev_c ? mie_ld(prev_c, idx) : 0.f;
   const float cell = gi * gg + gf * cp;
   cprev_res[idx] = cp;
   cell_res[idx] = cell;
-  mie_st(h_out, idx, go * tanhf(cell));
+  mie_st(h_out, idx, go * mie_gate_tanh(cell));
   mie_st(c_out, idx, cell);
 }
 

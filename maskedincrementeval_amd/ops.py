@@ -798,10 +798,10 @@ def mul_dense(a, b, out):
 
 
 def gate_interleave_index(hid: int, device=None) -> torch.Tensor:
-    """Column order of the fused gates conv: entry c' (= 32*b + 8*g + j) holds the column g*hid + 8*b + j of
-    the [in | remember | out | cell] x hid order (gate g of hidden channel 8*b + j)."""
+    """Column order of the fused gates conv: entry c' (= 4*hc + g) holds the column g*hid + hc of the
+    [in | remember | out | cell] x hid order (gate g of hidden channel hc)."""
     cp = torch.arange(4 * hid, device=device)
-    return ((cp % 32) // 8) * hid + (cp // 32) * 8 + cp % 8
+    return (cp % 4) * hid + cp // 4
 
 
 def conv_gates_incr(x, xmask, x2, x2mask, filt: ConvFilter, out_ts: TileMask, gates_res, cprev_delta, cprev_mask,
