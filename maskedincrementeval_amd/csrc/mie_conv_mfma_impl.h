@@ -36,13 +36,18 @@
 // LDS layout (pixel stride CC+4 dwords, row pitch 32 mod 64 dwords, half swap
 // for stride 2) keeps the 16-byte reads of 16 neighbouring lanes on disjoint banks.
 //
-// What bounds it (measured on MI355X): with the chip full (thousands of
-// workgroups) the fp32 kernel runs at 0.81 of the matrix-core peak.  A single
-// workgroup alone on a CU spends 86 % of each chunk on the matrix cores and about
-// 4 us on tile pick, first staging round trip and epilogue; launches with fewer
-// than a few workgroups per CU are therefore quantised: ceil(workgroups / 256)
-// rounds of one workgroup time.  8-wave workgroups and a 25-deep B ring were
-// tried and changed nothing: a workgroup already owns the CU's four matrix cores.
+// What bounds it (measured on MI355X).  A register-only loop of the same MFMAs sustains 27.2 ns per
+// v_mfma_f32_32x32x2_f32 and wave (64 cycles at 2.36 GHz; 152-155 TFLOP/s over the chip, constant or random
+// operands alike) -- and 13.8 ns per v_mfma_f32_32x32x16_bf16 with constant operands but 20.6 ns (1.63 PFLOP/s,
+// 0.65 of the nominal peak) with random ones: the bf16 rate is power-limited by the data.  In this kernel a
+// 3x3 chunk of 72 MFMAs per wave takes 2.92 us = 40.6 ns per MFMA (one workgroup per CU, 3x3 256->256 at
+// 33x44), a 5x5 chunk of 200 about 6.2 us = 31 ns.  Builds with parts of the loop compiled out (timing only)
+// put the 3x3 kernel at 28.8 us complete, 27.6 without the A reads from LDS, 24.3 without any load, store or
+// barrier in the loop; of those 24.3 us, 5.6 are tile pick, first staging round trip and epilogue.  The
+// chunk hand-over, the B prefetch depth, the staging depth (64 channels per chunk), 8-wave workgroups, a
+// third resident workgroup per CU (registers cut to fit) and splitting the contraction of the decoder convs
+// over two or four workgroups were each built and measured: none moved a layer by more than 2 %, the last
+// three for the worse.  Launches of a few workgroups per CU stay quantised: ceil(workgroups / 256) rounds.
 #pragma once
 #include "mie_conv.h"
 #include <stdlib.h>
@@ -529,69 +534,106 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   __syncthreads();
   MIE_STAMP(3);
 
-  // Double-buffered kernels pipeline the chunk hand-over into the contraction: the next chunk's global loads
-  // (and their address arithmetic) are issued once the first unit's MFMAs are in flight, and its LDS stores
-  // go out under the MFMAs of the last unit, so that between two chunks the matrix cores only wait for the
-  // barrier and the first operand read.  (Without it every boundary idled them for about 0.5 us: stores,
-  // barrier, some 70 address instructions, loads, first LDS read, all after the last MFMA had been issued.)
-  constexpr bool PIPE = MIE_PIPE && NBUF == 2 && !UP && UPC >= 4;
-  for (int c = c_lo; c < c_hi; ++c) {
-    const bool more = c + 1 < c_hi;
-    const int cn = more ? c + 1 : c;      // after the last chunk: redundant re-load, never stored
-    ub_next = chunk_b(cn);
-    if (!PIPE) stage_load(cn);
-    const T* sin = sbuf + ((c - c_lo) % NBUF) * STAGE;
-    // A operands are read one unit ahead as well (two register sets); the scheduling barriers
-    // pin "issue the loads for later units, then multiply this unit" so that the compiler can
-    // neither sink the prefetches next to their uses nor hoist them all to the top.
-    float4 av[2][2];
-    auto load_a = [&](int unit, float4 (&dst)[2]) {
-      const int tap = unit / NQW, qi = unit % NQW;
-      const int ky = tap / K, kx = tap - ky * K;
+  // A operand of unit `unit` from the staged chunk at `sin` (one 16-byte LDS read per pixel block).
+  auto load_a = [&](const T* sin, int unit, float4 (&dst)[2]) {
+    const int tap = unit / NQW, qi = unit % NQW;
+    const int ky = tap / K, kx = tap - ky * K;
 #pragma unroll
-      for (int mb = 0; mb < 2; ++mb)
-        dst[mb] = *reinterpret_cast<const float4*>(
-            &sin[a_lane[mb][(S == 2) ? ((ky >> 1) & 1) : 0] + ky * RP + kx * LS + SUB * qi]);
-    };
-    load_a(0, av[0]);
+    for (int mb = 0; mb < 2; ++mb)
+      dst[mb] = *reinterpret_cast<const float4*>(
+          &sin[a_lane[mb][(S == 2) ? ((ky >> 1) & 1) : 0] + ky * RP + kx * LS + SUB * qi]);
+  };
+
+  // Double-buffered kernels fold the chunk hand-over into the contraction, so that the matrix cores run
+  // through it:
+  //   * the next chunk's addresses are computed and its global loads issued right after the MFMAs of the
+  //     first unit (an opaque copy of the chunk index keeps the compiler from hoisting the ~70 address
+  //     instructions in front of them, where they ran with the matrix cores idle);
+  //   * its LDS stores go out under the unit before the last but one;
+  //   * the barrier sits between the last two units: by then every wave holds the A operands of its last
+  //     unit in registers, so the barrier, and the LDS read of the next chunk's first operands (a register
+  //     set of their own) behind it, pass under the last unit's MFMAs.
+  // Measured on MI355X this ordering is worth under 1 % against "loads at the top of the chunk, stores and
+  // barrier at its end": what a chunk loses against its MFMA time is not the hand-over (see the header).
+  constexpr bool PIPE = MIE_PIPE && NBUF == 2 && !UP && UPC >= 8;
+  if constexpr (PIPE) {
+    float4 av[2][2], av0[2];
+    load_a(sbuf, 0, av0);
+    for (int c = c_lo; c < c_hi; ++c) {
+      const bool more = c + 1 < c_hi;
+      const T* sin = sbuf + ((c - c_lo) & 1) * STAGE;
+      const T* sin_next = sbuf + ((c - c_lo + 1) & 1) * STAGE;
 #pragma unroll
-    for (int i = 0; i < UPC; ++i) {
-      // B operands of the unit PD ahead (the first units of the next chunk at the end)
-#ifndef MIE_EXP_NOB
-      if (PD > 0) {
-        const int ip = i + PD;
-        if (ip < UPC) load_b(ub_cur, ip, bring[ip % RING]);
-        else load_b(ub_next, ip - UPC, bring[ip % RING]);
-      }
-#endif
-#ifndef MIE_EXP_NOA
-      if (i + 1 < UPC) load_a(i + 1, av[(i + 1) & 1]);
-#endif
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) mma_unit2(acc[0][nb], acc[1][nb], av[i & 1][0], av[i & 1][1], bring[i % RING][nb], T());
-      __builtin_amdgcn_sched_barrier(0);
-      if (PD == 0) load_b(ub_next, 0, bring[0]);   // ring of one: reload right after use
-#ifndef MIE_EXP_NOSTAGE
-      if (PIPE && i == 0) {
-        stage_load(cn);
+      for (int i = 0; i < UPC; ++i) {
+        if (PD > 0) {
+          const int ip = i + PD;
+          if (ip < UPC) load_b(ub_cur, ip, bring[ip % RING]);
+          else load_b(ub_next, ip - UPC, bring[ip % RING]);
+        }
+        if (i + 1 < UPC) load_a(sin, i + 1, av[(i + 1) & 1]);
         __builtin_amdgcn_sched_barrier(0);
-      }
-      if (PIPE && i == UPC - 2) {
-        if (more) stage_store((c - c_lo + 1) % NBUF);    // the other buffer: nobody reads it during this chunk
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          if (i == 0) mma_unit2(acc[0][nb], acc[1][nb], av0[0], av0[1], bring[0][nb], T());
+          else mma_unit2(acc[0][nb], acc[1][nb], av[i & 1][0], av[i & 1][1], bring[i % RING][nb], T());
+        }
         __builtin_amdgcn_sched_barrier(0);
+        if (i == 0) {
+          int cn = more ? c + 1 : c;      // after the last chunk: redundant re-load, never stored
+          asm volatile("" : "+s"(cn));
+          ub_next = chunk_b(cn);
+          stage_load(cn);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        if (i == UPC - 3) {
+          if (more) stage_store((c - c_lo + 1) & 1);    // the other buffer: nobody reads it during this chunk
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        if (i == UPC - 2) {
+          // every wave has its last operands of this chunk (the wait for them is part of the barrier)
+          __syncthreads();
+          load_a(sin_next, 0, av0);       // after the last chunk: read and dropped
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
-#endif
+      ub_cur = ub_next;
+      MIE_STAMP(4 + (c - c_lo));
     }
-    if (!PIPE) {
+    // (the epilogue reuses the staging buffers: every read of them that matters was waited for in front of the
+    // last barrier; the operand read behind it returns whatever a faster wave has parked there, and is dropped)
+  } else {
+    for (int c = c_lo; c < c_hi; ++c) {
+      const bool more = c + 1 < c_hi;
+      const int cn = more ? c + 1 : c;      // after the last chunk: redundant re-load, never stored
+      ub_next = chunk_b(cn);
+      stage_load(cn);
+      const T* sin = sbuf + ((c - c_lo) % NBUF) * STAGE;
+      // A operands are read one unit ahead as well (two register sets); the scheduling barriers
+      // pin "issue the loads for later units, then multiply this unit" so that the compiler can
+      // neither sink the prefetches next to their uses nor hoist them all to the top.
+      float4 av[2][2];
+      load_a(sin, 0, av[0]);
+#pragma unroll
+      for (int i = 0; i < UPC; ++i) {
+        // B operands of the unit PD ahead (the first units of the next chunk at the end)
+        if (PD > 0) {
+          const int ip = i + PD;
+          if (ip < UPC) load_b(ub_cur, ip, bring[ip % RING]);
+          else load_b(ub_next, ip - UPC, bring[ip % RING]);
+        }
+        if (i + 1 < UPC) load_a(sin, i + 1, av[(i + 1) & 1]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) mma_unit2(acc[0][nb], acc[1][nb], av[i & 1][0], av[i & 1][1], bring[i % RING][nb], T());
+        __builtin_amdgcn_sched_barrier(0);
+        if (PD == 0) load_b(ub_next, 0, bring[0]);   // ring of one: reload right after use
+      }
       if (NBUF == 1 && !UP) __syncthreads();   // every wave is done reading the only buffer (UP: stage_store syncs)
       if (more) stage_store((c - c_lo + 1) % NBUF);
+      __syncthreads();
+      ub_cur = ub_next;
+      MIE_STAMP(4 + (c - c_lo));
     }
-#ifndef MIE_EXP_NOBARRIER
-    __syncthreads();
-#endif
-    ub_cur = ub_next;
-    MIE_STAMP(4 + (c - c_lo));
   }
   const int cob = cob0 + l32;
 
@@ -673,7 +715,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
       conv_store_batch<T, 16 * NB>(a, off, co, ok, v);
     }
   } else {
-    // the trailing barrier of the main loop has retired every read of the staging buffers
+    // the last barrier of the main loop has retired every read of the staging buffers that is used
     if (!EARLY && !SPLIT) epilogue_fetch();
     float* red = smem + wk * (64 * CO_BLK);
 #pragma unroll

@@ -133,11 +133,39 @@ __device__ __forceinline__ void up2x_src(int o, int in_size, int& i0, int& i1) {
   }
 }
 
+// k x k window of a conv with the window size known at compile time: every load is issued from a clamped
+// address and masked afterwards, so the K * K loads of a lane are independent and go out back to back.
+template <int K>
+__device__ __forceinline__ int conv_window_bit(const BuildArgs& a, int n, int iy0, int ix0) {
+  const uint8_t* base = a.in + (long long)n * a.h_in * a.w_in;
+  const uint8_t* base2 = a.in2 ? a.in2 + (long long)n * a.h_in * a.w_in : nullptr;
+  int bit = 0;
+#pragma unroll
+  for (int ky = 0; ky < K; ++ky) {
+    const int iy = iy0 + ky;
+    const bool oky = iy >= 0 && iy < a.h_in;
+    const int row = (oky ? iy : 0) * a.w_in;
+#pragma unroll
+    for (int kx = 0; kx < K; ++kx) {
+      const int ix = ix0 + kx;
+      const bool ok = oky && ix >= 0 && ix < a.w_in;
+      const int o = row + (ok ? ix : 0);
+      int v = base[o];
+      if (base2) v |= base2[o];
+      bit |= ok ? v : 0;
+    }
+  }
+  return bit != 0;
+}
+
 __device__ int footprint_bit(const BuildArgs& a, int n, int oy, int ox) {
   if (a.in == nullptr) return 1;
   int bit = 0;
   if (a.foot == MIE_FOOT_CONV) {
     const int iy0 = oy * a.s - a.p, ix0 = ox * a.s - a.p;
+    if (a.k == 5) return conv_window_bit<5>(a, n, iy0, ix0);
+    if (a.k == 3) return conv_window_bit<3>(a, n, iy0, ix0);
+    if (a.k == 1) return conv_window_bit<1>(a, n, iy0, ix0);
     for (int ky = 0; ky < a.k; ++ky)
       for (int kx = 0; kx < a.k; ++kx) bit |= mask_at(a, n, iy0 + ky, ix0 + kx);
   } else if (a.foot == MIE_FOOT_UP2X) {

@@ -35,11 +35,12 @@ def main():
     ap.add_argument("--iters", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--copy-mb", type=int, default=0, help="run a plain copy of this many MiB instead")
-    ap.add_argument("--op", choices=["conv", "act", "mul", "add", "up2x", "gates"], default="conv",
+    ap.add_argument("--op", choices=["conv", "act", "mul", "add", "up2x", "gates", "mask"], default="conv",
                     help="conv (default), or one of the bandwidth-bound incremental ops on an n x cin x h x w delta: "
                          "act = reservoir + ReLU increment, mul = product-rule multiply, add = skip sum, "
                          "up2x = bilinear x2 of a sum of two deltas (h, w = output size), gates = ConvLSTM gate chain "
-                         "(cin = hidden channels)")
+                         "(cin = hidden channels), mask = the tile-mask build of a k x k conv (footprint pass + ordered "
+                         "tile compaction) over an n x h x w pixel mask")
     ap.add_argument("--up2x", action="store_true",
                     help="the conv reads up2x(a + b) of two deltas at half of --h/--w (mie_upconv_masked; 5x5 stride 1)")
     args = ap.parse_args()
@@ -66,6 +67,8 @@ def main():
 
     n, cin, cout, k, s, h, w = args.n, args.cin, args.cout, args.k, args.stride, args.h, args.w
     p = k // 2
+    if args.op == "mask":
+        return mask_build(args, dev, e0, e1)
     if args.op != "conv":
         return pointwise(args, dev, e0, e1)
     if args.up2x:
@@ -115,6 +118,33 @@ def main():
                           algorithmic_flops=flops, algorithmic_bytes=byts,
                           tile_flops=2 * tiles * 64 * cin * cout * k * k,
                           tflops=round(flops / us / 1e6, 2), gbs=round(byts / us / 1e3, 1), iters=args.iters)))
+
+
+def mask_build(args, dev, e0, e1):
+    """The tile-mask build in front of a k x k conv: dilated pixel mask + tile flags (k_mask_footprint), then the
+    ascending active / stale tile lists (k_compact_tiles).  Algorithmic bytes: input and output pixel masks, one
+    flag word per tile read and written, the tile list."""
+    n, k, s, h, w = args.n, args.k, args.stride, args.h, args.w
+    p = k // 2
+    ho, wo = ops.conv_out_size(h, w, k, s, p)
+    m = torch.stack([torch.from_numpy(blob_mask(h, w, args.density, seed=b)) for b in range(n)]).view(n, 1, h, w)
+    mask = m.to(torch.uint8).to(dev)
+    ts = TileMask(n, ho, wo, dev)
+    launch = lambda: ops.build_mask_tiles(mask, None, n, h, w, _lib.FOOT_CONV, k, s, p, ts)
+    for _ in range(args.warmup):
+        launch()
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(args.iters):
+        launch()
+    e1.record()
+    torch.cuda.synchronize()
+    us = 1e3 * e0.elapsed_time(e1) / args.iters
+    tiles = int(ts.counts[0].item())
+    byts = n * h * w + n * ho * wo + ts.capacity * 8 + tiles * 4
+    print(json.dumps(dict(kernel="mie_build_mask_tiles", shape="%dx%d s%d @%dx%d n=%d" % (k, k, s, h, w, n),
+                          density=args.density, active_tiles=tiles, tiles=ts.capacity, us=round(us, 2),
+                          algorithmic_bytes=byts, gbs=round(byts / us / 1e3, 1), iters=args.iters)))
 
 
 def up2x_conv(args, dev, e0, e1):
