@@ -332,6 +332,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   int st_lds[NLD];      // LDS element offset of the slot
   int st_c4[NLD];       // channel offset of the slot inside the chunk
   unsigned ok1 = 0u, ok2 = 0u;   // slot readable from x / x2 (inside the image, pixel mask set)
+  unsigned inb = 0u;             // slot inside the image
 #pragma unroll
   for (int i = 0; i < NLD; ++i) {
     const int slot = tid + 256 * i;
@@ -344,10 +345,8 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
     if (!UP && slot < NSLOT) {
       const int iy = iy0 + pix / IT, ix = ix0 + pix % IT;
       if (iy >= 0 && iy < a.h_in && ix >= 0 && ix < a.w_in) {
-        const int po = (n * a.h_in + iy) * a.w_in + ix;
-        st_po[i] = po;
-        if (a.xm == nullptr || a.xm[po]) ok1 |= 1u << i;
-        if (a.x2 != nullptr && (a.x2m == nullptr || a.x2m[po])) ok2 |= 1u << i;
+        st_po[i] = (n * a.h_in + iy) * a.w_in + ix;
+        inb |= 1u << i;
       }
     }
   }
@@ -360,7 +359,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   const int h_lo = a.h_in >> 1, w_lo = a.w_in >> 1;
   const int lo_y0 = (iy0 >> 1) - 1, lo_x0 = (ix0 >> 1) - 1;
   int lo_po[NLO];
-  unsigned lo_ok1 = 0u, lo_ok2 = 0u;
+  unsigned lo_ok1 = 0u, lo_ok2 = 0u, lo_inb = 0u;
   float4 lo_a[NLO], lo_b[NLO];
   if (UP) {
 #pragma unroll
@@ -370,23 +369,26 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
       const int ly = lo_y0 + (lpix >> 3), lx = lo_x0 + (lpix & 7);
       lo_po[i] = 0;
       if (lpix < 64 && ly >= 0 && ly < h_lo && lx >= 0 && lx < w_lo) {
-        const int po = (n * h_lo + ly) * w_lo + lx;
-        lo_po[i] = po;
-        if (a.xm == nullptr || a.xm[po]) lo_ok1 |= 1u << i;
-        if (a.x2 != nullptr && (a.x2m == nullptr || a.x2m[po])) lo_ok2 |= 1u << i;
+        lo_po[i] = (n * h_lo + ly) * w_lo + lx;
+        lo_inb |= 1u << i;
       }
     }
   }
 
+  // The pixel-mask bytes a workgroup needs are one more dependent round trip at its start (tile id -> mask
+  // bytes -> input loads).  The loads of its FIRST chunk therefore go out for every pixel inside the image,
+  // before the mask bytes are there (`first`), and the masked pixels are zeroed when the bytes have arrived
+  // (stage_mask_first); from the second chunk on a masked pixel is not fetched at all, as before.
   float4 st_reg[NLD];
-  auto stage_load = [&](int c) {
+  auto stage_load = [&](int c, bool first = false) {
     if constexpr (UP) {
       const T* dummy = a.filt_mc;
 #pragma unroll
       for (int i = 0; i < NLO; ++i) {
         const int q4 = (tid + 256 * i) % Q4;
         const long long eo = (long long)lo_po[i] * a.c1 + c * CC + EPS * q4;
-        const bool k1 = (lo_ok1 >> i) & 1u, k2 = (lo_ok2 >> i) & 1u;
+        const bool k1 = ((first ? lo_inb : lo_ok1) >> i) & 1u;
+        const bool k2 = first ? (a.x2 != nullptr && ((lo_inb >> i) & 1u)) : ((lo_ok2 >> i) & 1u);
         float4 v = *reinterpret_cast<const float4*>(k1 ? a.x + eo : dummy);
         float4 u = *reinterpret_cast<const float4*>(k2 ? a.x2 + eo : dummy);
         v.x = k1 ? v.x : 0.f; v.y = k1 ? v.y : 0.f; v.z = k1 ? v.z : 0.f; v.w = k1 ? v.w : 0.f;
@@ -400,7 +402,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
     const T* xin = second ? a.x2 : a.x;
     const int cs = second ? a.c2 : a.c1;
     const int ci0 = (second ? c - nch1 : c) * CC;
-    const unsigned ok = second ? ok2 : ok1;
+    const unsigned ok = first ? inb : (second ? ok2 : ok1);
     // The loads are unconditional in control flow (a branch around a load makes the compiler's
     // wait counters conservative: the first MFMAs of a chunk would then wait for the whole
     // global-memory latency of these loads).  Lanes whose pixel is masked or outside the image
@@ -527,9 +529,46 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   const T* ub_cur = chunk_b(c_lo);
   const T* ub_next = ub_cur;
   MIE_STAMP(2);
-  stage_load(c_lo);
+  stage_load(c_lo, true);
+  // the pixel-mask bytes, behind the first chunk's loads (pixel 0 stands in for slots outside the image, so that
+  // these loads are unconditional too)
+  {
+    const bool m1 = a.xm != nullptr, has2 = a.x2 != nullptr, m2 = has2 && a.x2m != nullptr;
+    if constexpr (UP) {
+#pragma unroll
+      for (int i = 0; i < NLO; ++i) {
+        const unsigned b = (lo_inb >> i) & 1u;
+        const unsigned v1 = m1 ? (unsigned)(a.xm[lo_po[i]] != 0) : 1u;
+        const unsigned v2 = m2 ? (unsigned)(a.x2m[lo_po[i]] != 0) : (has2 ? 1u : 0u);
+        lo_ok1 |= (b & v1) << i;
+        lo_ok2 |= (b & v2) << i;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) {
+        const unsigned b = (inb >> i) & 1u;
+        const unsigned v1 = m1 ? (unsigned)(a.xm[st_po[i]] != 0) : 1u;
+        const unsigned v2 = m2 ? (unsigned)(a.x2m[st_po[i]] != 0) : (has2 ? 1u : 0u);
+        ok1 |= (b & v1) << i;
+        ok2 |= (b & v2) << i;
+      }
+    }
+  }
 #pragma unroll
   for (int i = 0; i < (PD > 0 ? PD : 1); ++i) load_b(ub_cur, i, bring[i % RING]);
+  // zero what the first chunk's loads fetched of masked pixels
+  if constexpr (UP) {
+#pragma unroll
+    for (int i = 0; i < NLO; ++i) {
+      if (!((lo_ok1 >> i) & 1u)) lo_a[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (!((lo_ok2 >> i) & 1u)) lo_b[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+  } else {
+    const unsigned ok = (c_lo >= nch1) ? ok2 : ok1;
+#pragma unroll
+    for (int i = 0; i < NLD; ++i)
+      if (!((ok >> i) & 1u)) st_reg[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+  }
   stage_store(0);
   __syncthreads();
   MIE_STAMP(3);
