@@ -227,6 +227,55 @@ __global__ __launch_bounds__(256) void k_tconv_valu(ConvArgsT<T> a, int K, int S
   }
 }
 
+// The decoder geometry (3x3, stride 2, pad 1, output exactly twice the input) over very few input
+// channels -- the 2-channel flow estimate in front of an EVFlowNet decoder, whose result rides into the
+// matrix-core transposed conv as its addend.  An output pixel (oy, ox) sees the taps of its sub-pixel
+// phase only: ky = 1 for even oy, ky in {0, 2} for odd oy (input row (oy + 1 - ky) / 2), the same in x,
+// so 1, 2 or 4 taps -- no division, no modulo.  A thread owns 4 adjacent output channels of one pixel
+// (16-byte filter loads, the input values are broadcast loads); a workgroup one 8x8 output tile.
+template <typename T>
+__global__ __launch_bounds__(256) void k_tconv2x_fewcin(ConvArgsT<T> a) {
+  int n, y0, x0;
+  const int tk = mie_pick_tile(a.ts, blockIdx.x, n, y0, x0);
+  if (tk == 0) return;
+  const int hout = a.ts.h, wout = a.ts.w, cout = a.cout, c1 = a.c1;
+  const int G = cout >> 2;
+  for (int idx = threadIdx.x; idx < 64 * G; idx += 256) {
+    const int p = idx / G, g = idx - p * G;
+    const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
+    if (oy >= hout || ox >= wout) continue;
+    const long long off = (((long long)n * hout + oy) * wout + ox) * cout + 4 * g;
+    if (tk == 2) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) mie_st(a.out, off + e, 0.f);
+      continue;
+    }
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    const int nky = (oy & 1) ? 2 : 1, nkx = (ox & 1) ? 2 : 1;
+    for (int iky = 0; iky < nky; ++iky) {
+      const int ky = (oy & 1) ? 2 * iky : 1;
+      const int iy = (oy + 1 - ky) >> 1;
+      if (iy >= a.h_in) continue;
+      for (int ikx = 0; ikx < nkx; ++ikx) {
+        const int kx = (ox & 1) ? 2 * ikx : 1;
+        const int ix = (ox + 1 - kx) >> 1;
+        if (ix >= a.w_in) continue;
+        const long long po = ((long long)n * a.h_in + iy) * a.w_in + ix;
+        if (a.xm != nullptr && !a.xm[po]) continue;
+        const T* xr = a.x + po * c1;
+        const float* wp = a.filt + (long long)(ky * 3 + kx) * cout + 4 * g;
+        for (int ci = 0; ci < c1; ++ci) {
+          const float xv = mie_ld(xr, ci);
+          const float4 w4 = *reinterpret_cast<const float4*>(wp + (long long)ci * 9 * cout);
+          acc[0] += xv * w4.x; acc[1] += xv * w4.y; acc[2] += xv * w4.z; acc[3] += xv * w4.w;
+        }
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) conv_store(a, off + e, 4 * g + e, acc[e]);
+  }
+}
+
 template <typename T, int K, int S>
 void launch_conv(const ConvArgsT<T>& a, unsigned cap, hipStream_t st) {
   if (K == 1 && S == 1 && a.pad == 0 && a.cout <= 4 && (a.c1 & 3) == 0 && (a.c2 & 3) == 0) {
@@ -416,8 +465,12 @@ int tconv_impl(const char* who, const T* x, const uint8_t* xmask, int cin, int h
   a.ws = nullptr; a.ws_floats = 0; a.ws_plane = 0; a.xcd_fs = 0;
   a.ts = mie_dev_tileset(out);
   const unsigned cap = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
-  hipLaunchKernelGGL(k_tconv_valu<T>, dim3(cap, mie_div_up(cout, 64)), dim3(256), 0,
-                     (hipStream_t)stream, a, k, stride);
+  if (k == 3 && stride == 2 && pad == 1 && out->h == 2 * h_in && out->w == 2 * w_in && cin <= 8 && cout % 4 == 0 &&
+      mie_aligned(filter, 16))
+    hipLaunchKernelGGL(k_tconv2x_fewcin<T>, dim3(cap), dim3(256), 0, (hipStream_t)stream, a);
+  else
+    hipLaunchKernelGGL(k_tconv_valu<T>, dim3(cap, mie_div_up(cout, 64)), dim3(256), 0,
+                       (hipStream_t)stream, a, k, stride);
   return mie_check_launch(who);
 }
 

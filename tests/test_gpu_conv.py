@@ -191,6 +191,33 @@ def test_tconv_matches_oracle(k, s, p, op):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("cin,cout,h,w", [(2, 32, 16, 16), (2, 64, 13, 21), (8, 20, 7, 9), (1, 4, 33, 5)])
+def test_tconv2x_few_channel_form(cin, cout, h, w, dtype):
+    """The decoder geometry over very few input channels (the flow lead of an EVFlowNet decoder) takes a kernel
+    of its own: against the oracle, over three steps with moving masks (stale tiles are zeroed), ragged planes."""
+    n, k, s, p, op = 2, 3, 2, 1, 1
+    wt = torch.randn(cin, cout, k, k, generator=torch.Generator().manual_seed(cin + cout)) * 0.3
+    if dtype == torch.bfloat16:
+        wt = wt.to(dtype).float()
+    ho, wo = 2 * h, 2 * w
+    ts = TileMask(n, ho, wo, DEV)
+    out = ops.new_nhwc(n, cout, ho, wo, DEV, dtype)
+    filt = wt.permute(0, 2, 3, 1).contiguous().to(DEV)
+    for step in range(3):
+        d, m = gaussian_delta(n, cin, h, w, 0.06, 0.5, seed=10 * step + cin)
+        if dtype == torch.bfloat16:
+            d = d.to(dtype).float()
+        ref = io.tconv_incr(d, wt, s, p, op)
+        ops.build_mask_tiles(m.to(DEV), None, n, h, w, _lib.FOOT_TCONV, k, s, p, ts)
+        ops.tconv_masked(_dev(d).to(dtype), m.to(DEV), filt, k, s, p, ts, out)
+        torch.cuda.synchronize()
+        if dtype == torch.bfloat16:
+            assert torch.allclose(out.float().cpu(), ref, rtol=2.0 ** -7, atol=bf16_atol(ref, 1)), "step %d" % step
+        else:
+            _close(out, ref, "tconv2x few-channel step %d" % step)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("c1,c2,cout,h,w,k", [
     (64, 0, 32, 13, 17, 3),        # one input, ragged plane
     (64, 64, 64, 16, 16, 3),       # two inputs (the concat-free decoder form), 2 chunks: not split
