@@ -376,9 +376,10 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   }
 
   // The pixel-mask bytes a workgroup needs are one more dependent round trip at its start (tile id -> mask
-  // bytes -> input loads).  The loads of its FIRST chunk therefore go out for every pixel inside the image,
-  // before the mask bytes are there (`first`), and the masked pixels are zeroed when the bytes have arrived
-  // (stage_mask_first); from the second chunk on a masked pixel is not fetched at all, as before.
+  // bytes -> input loads).  Where the contraction has at least four chunks, the loads of the FIRST chunk
+  // therefore go out for every pixel inside the image, before the mask bytes are there (`first`), and the
+  // masked pixels are zeroed when the bytes have arrived; from the second chunk on -- and in layers of fewer
+  // chunks, where that would be a large share of the reads -- a masked pixel is not fetched at all.
   float4 st_reg[NLD];
   auto stage_load = [&](int c, bool first = false) {
     if constexpr (UP) {
@@ -529,7 +530,8 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   const T* ub_cur = chunk_b(c_lo);
   const T* ub_next = ub_cur;
   MIE_STAMP(2);
-  stage_load(c_lo, true);
+  const bool early = c_hi - c_lo >= 4;      // uniform over the workgroup
+  if (early) stage_load(c_lo, true);
   // the pixel-mask bytes, behind the first chunk's loads (pixel 0 stands in for slots outside the image, so that
   // these loads are unconditional too)
   {
@@ -554,10 +556,12 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
       }
     }
   }
+  if (!early) stage_load(c_lo);
 #pragma unroll
   for (int i = 0; i < (PD > 0 ? PD : 1); ++i) load_b(ub_cur, i, bring[i % RING]);
   // zero what the first chunk's loads fetched of masked pixels
-  if constexpr (UP) {
+  if (!early) {
+  } else if constexpr (UP) {
 #pragma unroll
     for (int i = 0; i < NLO; ++i) {
       if (!((lo_ok1 >> i) & 1u)) lo_a[i] = make_float4(0.f, 0.f, 0.f, 0.f);
