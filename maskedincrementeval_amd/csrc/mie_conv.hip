@@ -232,7 +232,8 @@ __global__ __launch_bounds__(256) void k_tconv_valu(ConvArgsT<T> a, int K, int S
 // matrix-core transposed conv as its addend.  An output pixel (oy, ox) sees the taps of its sub-pixel
 // phase only: ky = 1 for even oy, ky in {0, 2} for odd oy (input row (oy + 1 - ky) / 2), the same in x,
 // so 1, 2 or 4 taps -- no division, no modulo.  A thread owns 4 adjacent output channels of one pixel
-// (16-byte filter loads, the input values are broadcast loads); a workgroup one 8x8 output tile.
+// (16-byte filter loads, the input values are broadcast loads); the workgroups of grid row x share one
+// 8x8 output tile.
 template <typename T>
 __global__ __launch_bounds__(256) void k_tconv2x_fewcin(ConvArgsT<T> a) {
   int n, y0, x0;
@@ -240,7 +241,9 @@ __global__ __launch_bounds__(256) void k_tconv2x_fewcin(ConvArgsT<T> a) {
   if (tk == 0) return;
   const int hout = a.ts.h, wout = a.ts.w, cout = a.cout, c1 = a.c1;
   const int G = cout >> 2;
-  for (int idx = threadIdx.x; idx < 64 * G; idx += 256) {
+  // one (pixel, channel group) per thread: grid y covers the 64 * G items of a tile, so that a tile's
+  // dependent loads are one chain deep whatever the channel count
+  for (int idx = blockIdx.y * 256 + threadIdx.x; idx < 64 * G; idx += 256 * gridDim.y) {
     const int p = idx / G, g = idx - p * G;
     const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
     if (oy >= hout || ox >= wout) continue;
@@ -467,7 +470,7 @@ int tconv_impl(const char* who, const T* x, const uint8_t* xmask, int cin, int h
   const unsigned cap = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
   if (k == 3 && stride == 2 && pad == 1 && out->h == 2 * h_in && out->w == 2 * w_in && cin <= 8 && cout % 4 == 0 &&
       mie_aligned(filter, 16))
-    hipLaunchKernelGGL(k_tconv2x_fewcin<T>, dim3(cap), dim3(256), 0, (hipStream_t)stream, a);
+    hipLaunchKernelGGL(k_tconv2x_fewcin<T>, dim3(cap, mie_div_up(16 * cout, 256)), dim3(256), 0, (hipStream_t)stream, a);
   else
     hipLaunchKernelGGL(k_tconv_valu<T>, dim3(cap, mie_div_up(cout, 64)), dim3(256), 0,
                        (hipStream_t)stream, a, k, stride);
