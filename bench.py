@@ -392,7 +392,9 @@ class NetBench:
 
     def dominant_roofline(self, layers, agg, reps=50):
         """Roofline of the conv launch that takes the most time, re-timed on its own: the same call (same
-        tile set, same buffers) replayed back to back between two HIP events on the launch stream."""
+        tile set, same buffers) replayed `reps` times on the launch stream, each launch between two HIP events
+        of its own, so that the figure is the kernel's duration and not the 3-4 us from the end of one launch
+        to the start of the next (what a kernel trace reports as the kernel's average duration)."""
         torch = self.torch
         convs = [l for l in layers if l["op"] in ("conv_masked", "conv_gates_incr", "upconv_masked", "tconv2x_masked")]
         dom = max(convs, key=lambda l: l["us"])
@@ -400,13 +402,17 @@ class NetBench:
         with torch.no_grad():
             for _ in range(5):
                 orig(*cargs, **ckw)
+            evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
             ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             ev0.record()
-            for _ in range(reps):
+            for ea, eb in evs:
+                ea.record()
                 orig(*cargs, **ckw)
+                eb.record()
             ev1.record()
             torch.cuda.synchronize()
-        dom_us = 1e3 * ev0.elapsed_time(ev1) / reps
+        dom_us = 1e3 * sum(ea.elapsed_time(eb) for ea, eb in evs) / reps
+        self.dominant_back_to_back_us = round(1e3 * ev0.elapsed_time(ev1) / reps, 2)
         dom = dict(dom, us=round(dom_us, 2), gbs=round(dom["bytes"] / dom_us / 1e3, 1),
                    tflops=round(dom["flops"] / dom_us / 1e6, 2))
         mfma_bound = dom["flops"] / max(dom["bytes"], 1) > self.peak_mfma * 1e12 / (PEAK_HBM_GBS * 1e9)
@@ -418,7 +424,8 @@ class NetBench:
                             frac=round(dom["gbs"] / PEAK_HBM_GBS, 4), traffic=None)
         roofline.update(kernel="mie_%s %s" % (dom["op"].replace("_incr", "").replace("conv_gates", "conv_gates_masked"),
                                               dom["shape"]), us=dom["us"],
-                        algorithmic_bytes=dom["bytes"], algorithmic_flops=dom["flops"])
+                        algorithmic_bytes=dom["bytes"], algorithmic_flops=dom["flops"],
+                        us_back_to_back=self.dominant_back_to_back_us)
         # HBM bytes per launch of that kernel from the committed rocprofv3 --pmc summary, if it covers this
         # shape (FETCH_SIZE + WRITE_SIZE, scaled by the copy-kernel calibration)
         try:
