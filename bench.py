@@ -410,7 +410,13 @@ class NetBench:
                 orig(*cargs, **ckw)
                 eb.record()
             ev1.record()
+            # what an event pair reads with nothing between its two records
+            empty = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+            for ea, eb in empty:
+                ea.record()
+                eb.record()
             torch.cuda.synchronize()
+        self.event_pair_us = round(1e3 * sum(ea.elapsed_time(eb) for ea, eb in empty) / reps, 2)
         dom_us = 1e3 * sum(ea.elapsed_time(eb) for ea, eb in evs) / reps
         self.dominant_back_to_back_us = round(1e3 * ev0.elapsed_time(ev1) / reps, 2)
         dom = dict(dom, us=round(dom_us, 2), gbs=round(dom["bytes"] / dom_us / 1e3, 1),
@@ -425,7 +431,7 @@ class NetBench:
         roofline.update(kernel="mie_%s %s" % (dom["op"].replace("_incr", "").replace("conv_gates", "conv_gates_masked"),
                                               dom["shape"]), us=dom["us"],
                         algorithmic_bytes=dom["bytes"], algorithmic_flops=dom["flops"],
-                        us_back_to_back=self.dominant_back_to_back_us)
+                        us_back_to_back=self.dominant_back_to_back_us, us_empty_event_pair=self.event_pair_us)
         # HBM bytes per launch of that kernel from the committed rocprofv3 --pmc summary, if it covers this
         # shape (FETCH_SIZE + WRITE_SIZE, scaled by the copy-kernel calibration)
         try:
