@@ -23,6 +23,18 @@ static __device__ __forceinline__ float mie_ld(const float* p, long long i) { re
 static __device__ __forceinline__ float mie_ld(const mie_bf16* p, long long i) { return (float)p[i]; }
 static __device__ __forceinline__ void mie_st(float* p, long long i, float v) { p[i] = v; }
 static __device__ __forceinline__ void mie_st(mie_bf16* p, long long i, float v) { p[i] = (mie_bf16)v; }
+// Four adjacent elements at once (i a multiple of 4, p + i 16-byte / 8-byte aligned).
+static __device__ __forceinline__ float4 mie_ld4(const float* p, long long i) { return *reinterpret_cast<const float4*>(p + i); }
+static __device__ __forceinline__ float4 mie_ld4(const mie_bf16* p, long long i) {
+  const mie_bf16x4 b = *reinterpret_cast<const mie_bf16x4*>(p + i);
+  return make_float4((float)b[0], (float)b[1], (float)b[2], (float)b[3]);
+}
+static __device__ __forceinline__ void mie_st4(float* p, long long i, const float4& v) { *reinterpret_cast<float4*>(p + i) = v; }
+static __device__ __forceinline__ void mie_st4(mie_bf16* p, long long i, const float4& v) {
+  mie_bf16x4 b;
+  b[0] = (mie_bf16)v.x; b[1] = (mie_bf16)v.y; b[2] = (mie_bf16)v.z; b[3] = (mie_bf16)v.w;
+  *reinterpret_cast<mie_bf16x4*>(p + i) = b;
+}
 
 // ---- host side: error reporting -------------------------------------------
 void mie_set_error(const char* fmt, ...);

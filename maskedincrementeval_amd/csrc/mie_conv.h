@@ -91,6 +91,53 @@ static __device__ __forceinline__ void conv_epilogue_store(const ConvArgsT<T>& a
   }
 }
 
+// The same for N groups of four adjacent output channels of one pixel each (off[i] = offset of the first of
+// the four, a multiple of 4; co[i] its channel): 16-byte reservoir accesses, 16- / 8-byte delta accesses.
+template <typename T, int N>
+static __device__ __forceinline__ void conv_epilogue_load4(const ConvArgsT<T>& a, const long long (&off)[N],
+                                                           const bool (&ok)[N], float4 (&r0)[N], float4 (&add)[N]) {
+  const bool want_res = a.res != nullptr && !a.refresh;
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    r0[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    add[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (ok[i]) {
+      if (a.addend) add[i] = mie_ld4(a.addend, off[i]);
+      if (want_res) r0[i] = mie_ld4(a.res, off[i]);
+    }
+  }
+}
+
+template <typename T, int N>
+static __device__ __forceinline__ void conv_epilogue_store4(const ConvArgsT<T>& a, const long long (&off)[N],
+                                                            const int (&co)[N], const bool (&ok)[N],
+                                                            const float4 (&acc)[N], const float4 (&r0)[N],
+                                                            const float4 (&add)[N]) {
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    if (!ok[i]) continue;
+    float4 v = make_float4(acc[i].x + add[i].x, acc[i].y + add[i].y, acc[i].z + add[i].z, acc[i].w + add[i].w);
+    if (a.refresh) {
+      if (a.bias) {
+        v.x += a.bias[co[i]]; v.y += a.bias[co[i] + 1]; v.z += a.bias[co[i] + 2]; v.w += a.bias[co[i] + 3];
+      }
+      if (a.res) mie_st4(a.res, off[i], v);
+      mie_st4(a.out, off[i], make_float4(mie_act(a.act, a.slope, v.x), mie_act(a.act, a.slope, v.y),
+                                         mie_act(a.act, a.slope, v.z), mie_act(a.act, a.slope, v.w)));
+    } else if (a.res) {
+      const float4 r1 = make_float4(r0[i].x + v.x, r0[i].y + v.y, r0[i].z + v.z, r0[i].w + v.w);
+      mie_st4(a.res, off[i], r1);
+      mie_st4(a.out, off[i],
+              make_float4(mie_act(a.act, a.slope, r1.x) - mie_act(a.act, a.slope, r0[i].x),
+                          mie_act(a.act, a.slope, r1.y) - mie_act(a.act, a.slope, r0[i].y),
+                          mie_act(a.act, a.slope, r1.z) - mie_act(a.act, a.slope, r0[i].z),
+                          mie_act(a.act, a.slope, r1.w) - mie_act(a.act, a.slope, r0[i].w)));
+    } else {
+      mie_st4(a.out, off[i], v);
+    }
+  }
+}
+
 template <typename T, int N>
 static __device__ __forceinline__ void conv_store_batch(const ConvArgsT<T>& a, const long long (&off)[N],
                                                         const int (&co)[N], const bool (&ok)[N],

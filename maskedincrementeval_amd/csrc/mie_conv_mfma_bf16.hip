@@ -10,3 +10,11 @@ bool mie_launch_conv_gates_mfma(const ConvArgsT<mie_bf16>& a, unsigned cap, hipS
 bool mie_launch_conv_up_mfma(const ConvArgsT<mie_bf16>& a, unsigned cap, hipStream_t st) {
   return launch_up<mie_bf16>(a, cap, st);
 }
+
+#ifdef MIE_WG_PROFILE
+// Measurement builds only: the same for the bf16 kernels of this translation unit.
+extern "C" __attribute__((visibility("default"))) int mie_set_profile_buffer_bf16(void* p) {
+  long long* q = (long long*)p;
+  return hipMemcpyToSymbol(HIP_SYMBOL(mie_prof_buf), &q, sizeof(q)) == hipSuccess ? 0 : -4;
+}
+#endif

@@ -198,7 +198,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   constexpr int RING = ring_size(UPC);                       // B operand ring (divides UPC)
   constexpr int PD = RING - 1;                               // prefetch distance in units
   constexpr int CO_BLK = 32 * NB * WN;
-  constexpr int RED = (WK > 1 || GATES) ? WK * 64 * CO_BLK : 0;
+  constexpr int RED = WK * 64 * CO_BLK;                      // every wave parks its accumulators here for the epilogue
   constexpr int STAGE_F = NBUF * STAGE * (int)sizeof(T) / 4;  // the staging buffers, in floats
   constexpr int LOS = CC;                                    // floats per source pixel in LDS
   constexpr int LO_F = UP ? 64 * LOS : 0;                    // fp32 sums of the 8x8 source block, CC channels
@@ -294,29 +294,33 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
     return;
   }
 
-  // k-split kernels: the thread's share of the output (the elements it reduces and stores at the
-  // end) is fixed by its index, so the reservoir / addend values are fetched right away.
-  constexpr int PER = (WK > 1 && !GATES) ? 64 * CO_BLK / 256 : 1;      // output elements per thread
+  // Epilogue (all but the gate chain): every wave parks its accumulators in LDS, and a thread then owns groups of
+  // four adjacent output channels of a pixel -- 16-byte reads of the k-split partial sums, 16-byte reservoir
+  // accesses, 16- / 8-byte delta accesses.  A thread's share of the output is fixed by its index, so in the k-split
+  // fp32 kernels the reservoir / addend values are fetched right away and have the whole contraction to arrive.
+  constexpr int QPP = CO_BLK / 4;                            // groups of four channels per pixel
+  constexpr int PER = GATES ? 1 : 64 * QPP / 256;            // groups per thread
   long long e_off[PER];
   int e_co[PER];
   bool e_ok[PER];
-  float e_r0[PER], e_add[PER];
+  float4 e_r0[PER], e_add[PER];
   // (bf16: a workgroup's contraction is too short to be worth the registers that hold these values
-  // through it -- they cost a resident workgroup per CU -- so they are fetched after it instead.)
-  constexpr bool EARLY = sizeof(T) == 4;
+  // through it -- they cost a resident workgroup per CU -- so they are fetched after it instead; the same
+  // holds for the 128-column slabs, whose threads own 8 groups.)
+  constexpr bool EARLY = sizeof(T) == 4 && WK > 1;
   auto epilogue_fetch = [&]() {
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const int idx = tid + 256 * i;
-      const int p = idx / CO_BLK, col = idx - p * CO_BLK;
+      const int p = idx / QPP, col = 4 * (idx - p * QPP);
       const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
       e_ok[i] = oy < hout && ox < wout;
       e_off[i] = (((long long)n * hout + oy) * wout + ox) * a.cout + co0 + col;
       e_co[i] = co0 + col;
     }
-    conv_epilogue_load<T, PER>(a, e_off, e_ok, e_r0, e_add);
+    if (!SPLIT) conv_epilogue_load4<T, PER>(a, e_off, e_ok, e_r0, e_add);
   };
-  if (WK > 1 && !GATES && EARLY && !SPLIT) epilogue_fetch();
+  if (!GATES && EARLY && !SPLIT) epilogue_fetch();
 
   v16f acc[2][NB];
 #pragma unroll
@@ -678,7 +682,6 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
       MIE_STAMP(4 + (c - c_lo));
     }
   }
-  const int cob = cob0 + l32;
 
   // ---- epilogue -----------------------------------------------------------------------------------
   // acc[mb][nb][r] of this lane is output pixel p = 32*mb + 8*(r/4) + 4*half + r%4,
@@ -735,31 +738,9 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
       mie_st(a.g_dh, ho, dh);
       mie_st(a.g_dc, ho, dc);
     }
-  } else if (WK == 1) {
-#pragma unroll
-    for (int mb = 0; mb < 2; ++mb) {
-      long long off[16 * NB];
-      int co[16 * NB];
-      bool ok[16 * NB];
-      float v[16 * NB];
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int p = mb * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-        const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
-        const long long ob = (((long long)n * hout + oy) * wout + ox) * a.cout + cob;
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-          off[r * NB + nb] = ob + nb * 32;
-          co[r * NB + nb] = cob + nb * 32;
-          ok[r * NB + nb] = oy < hout && ox < wout;
-          v[r * NB + nb] = acc[mb][nb][r];
-        }
-      }
-      conv_store_batch<T, 16 * NB>(a, off, co, ok, v);
-    }
   } else {
     // the last barrier of the main loop has retired every read of the staging buffers that is used
-    if (!EARLY && !SPLIT) epilogue_fetch();
+    if (!EARLY || SPLIT) epilogue_fetch();
     float* red = smem + wk * (64 * CO_BLK);
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb)
@@ -771,26 +752,25 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
           red[p * CO_BLK + wn * (32 * NB) + nb * 32 + l32] = acc[mb][nb][r];
       }
     __syncthreads();
-    float v[PER];
+    float4 v[PER];
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
-      const int idx = tid + 256 * i;
-      float sum = smem[idx];
+      const int idx = tid + 256 * i;             // group idx: pixel idx / QPP, channels 4 * (idx % QPP) ...
+      float4 sum = *reinterpret_cast<const float4*>(&smem[4 * idx]);
 #pragma unroll
-      for (int k2 = 1; k2 < WK; ++k2) sum += smem[k2 * (64 * CO_BLK) + idx];
+      for (int k2 = 1; k2 < WK; ++k2) {
+        const float4 part = *reinterpret_cast<const float4*>(&smem[k2 * (64 * CO_BLK) + 4 * idx]);
+        sum.x += part.x; sum.y += part.y; sum.z += part.z; sum.w += part.w;
+      }
       v[i] = sum;
     }
     if constexpr (SPLIT) {
       float* plane = a.ws + (long long)bz * a.ws_plane;
 #pragma unroll
-      for (int i = 0; i < PER; ++i) {
-        const int idx = tid + 256 * i;
-        const int p = idx / CO_BLK, col = idx - p * CO_BLK;
-        const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
-        if (oy < hout && ox < wout) plane[(((long long)n * hout + oy) * wout + ox) * a.cout + co0 + col] = v[i];
-      }
+      for (int i = 0; i < PER; ++i)
+        if (e_ok[i]) *reinterpret_cast<float4*>(plane + e_off[i]) = v[i];
     } else {
-      conv_epilogue_store<T, PER>(a, e_off, e_co, e_ok, v, e_r0, e_add);
+      conv_epilogue_store4<T, PER>(a, e_off, e_co, e_ok, v, e_r0, e_add);
     }
   }
   MIE_STAMP(14);
