@@ -272,24 +272,24 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   static_assert(!SPLIT || (WN == 1 && !GATES && !UP), "the split form is the plain 32-channel slab kernel");
   if (SPLIT && tk == 2) return;      // stale tiles are zeroed by k_conv_split_finish
   if (GATES && tk == 2) {  // stale tile: zero the hidden / cell deltas of this workgroup's hidden channels
-    constexpr int HC = CO_BLK / 4;
-    for (int idx = tid; idx < 64 * HC; idx += 256) {
-      const int p = idx / HC, hc = idx - p * HC;
+    constexpr int HG = CO_BLK / 16;          // groups of four hidden channels
+    for (int idx = tid; idx < 64 * HG; idx += 256) {
+      const int p = idx / HG, g4 = idx - p * HG;
       const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
       if (oy < hout && ox < wout) {
-        const long long o = (((long long)n * hout + oy) * wout + ox) * a.hid + co0 / 4 + hc;
-        mie_st(a.g_dh, o, 0.f);
-        mie_st(a.g_dc, o, 0.f);
+        const long long o = (((long long)n * hout + oy) * wout + ox) * a.hid + co0 / 4 + 4 * g4;
+        mie_st4(a.g_dh, o, make_float4(0.f, 0.f, 0.f, 0.f));
+        mie_st4(a.g_dc, o, make_float4(0.f, 0.f, 0.f, 0.f));
       }
     }
     return;
   }
   if (tk == 2) {  // stale tile: zero this workgroup's channel slab
-    for (int idx = tid; idx < 64 * CO_BLK; idx += 256) {
-      const int p = idx / CO_BLK, col = idx - p * CO_BLK;
+    for (int idx = tid; idx < 16 * CO_BLK; idx += 256) {       // groups of four channels
+      const int p = idx / (CO_BLK / 4), col = 4 * (idx - p * (CO_BLK / 4));
       const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
       if (oy < hout && ox < wout)
-        mie_st(a.out, (((long long)n * hout + oy) * wout + ox) * cout + co0 + col, 0.f);
+        mie_st4(a.out, (((long long)n * hout + oy) * wout + ox) * cout + co0 + col, make_float4(0.f, 0.f, 0.f, 0.f));
     }
     return;
   }
@@ -702,41 +702,58 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
           red[p * CO_BLK + wn * (32 * NB) + nb * 32 + l32] = acc[mb][nb][r];
       }
     __syncthreads();
+    // An item is one pixel x four adjacent hidden channels: their 16 gate columns are four 16-byte groups in LDS
+    // and 64 contiguous bytes of the gate reservoir, their cell / previous-cell reservoirs one 16-byte group each,
+    // their state deltas 16 (fp32) or 8 (bf16) bytes.
     constexpr int HC = CO_BLK / 4;             // hidden channels of this workgroup
-    constexpr int PERG = 64 * HC / 256;        // (pixel, hidden channel) items per thread
+    constexpr int HG = HC / 4;                 // groups of four of them
+    constexpr int NIT = 64 * HG;               // items of the tile
+    constexpr int PERG = (NIT + 255) / 256;    // items per thread (the 32-column slab has 128 items: half the threads idle)
     const int hid = a.hid;
+    const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
     for (int i = 0; i < PERG; ++i) {
       const int idx = tid + 256 * i;
-      const int p = idx / HC, hc = idx - p * HC;
+      if (idx >= NIT) continue;
+      const int p = idx / HG, g4 = idx - p * HG;
       const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
       if (oy >= hout || ox >= wout) continue;
       const long long pix = ((long long)n * hout + oy) * wout + ox;
-      const long long ho = pix * hid + co0 / 4 + hc;
+      const long long ho = pix * hid + co0 / 4 + 4 * g4;
       if (!a.ts.pixmask[pix]) {               // inactive pixel of an active tile: clean zeros
-        mie_st(a.g_dh, ho, 0.f);
-        mie_st(a.g_dc, ho, 0.f);
+        mie_st4(a.g_dh, ho, zero4);
+        mie_st4(a.g_dc, ho, zero4);
         continue;
       }
-      // the four gates of a hidden channel are four adjacent columns: one 16-byte access each for the k-split
-      // partials in LDS and for the gate reservoir
-      float4 dg = *reinterpret_cast<const float4*>(&smem[p * CO_BLK + 4 * hc]);
+      float4 dg[4], rr[4];
+      float4* gr = reinterpret_cast<float4*>(a.res + pix * a.cout + co0 + 16 * g4);
 #pragma unroll
-      for (int k2 = 1; k2 < WK; ++k2) {
-        const float4 part = *reinterpret_cast<const float4*>(&smem[k2 * (64 * CO_BLK) + p * CO_BLK + 4 * hc]);
-        dg.x += part.x; dg.y += part.y; dg.z += part.z; dg.w += part.w;
+      for (int j = 0; j < 4; ++j) {
+        rr[j] = gr[j];
+        dg[j] = *reinterpret_cast<const float4*>(&smem[p * CO_BLK + 16 * g4 + 4 * j]);
+#pragma unroll
+        for (int k2 = 1; k2 < WK; ++k2) {
+          const float4 part = *reinterpret_cast<const float4*>(&smem[k2 * (64 * CO_BLK) + p * CO_BLK + 16 * g4 + 4 * j]);
+          dg[j].x += part.x; dg[j].y += part.y; dg[j].z += part.z; dg[j].w += part.w;
+        }
       }
-      float4* gr = reinterpret_cast<float4*>(a.res + pix * a.cout + co0 + 4 * hc);
-      float4 rr = *gr;
       const bool has_cp = a.g_cpd != nullptr && (a.g_cpm == nullptr || a.g_cpm[pix]);
-      const float dP = has_cp ? mie_ld(a.g_cpd, ho) : 0.f;
-      float cp = a.g_cpres[ho], cc = a.g_cres[ho], dh, dc;
-      mie_lstm_gate_chain(rr.x, rr.y, rr.z, rr.w, dg.x, dg.y, dg.z, dg.w, cp, dP, cc, dh, dc);
-      *gr = rr;
-      if (has_cp) a.g_cpres[ho] = cp;
-      a.g_cres[ho] = cc;
-      mie_st(a.g_dh, ho, dh);
-      mie_st(a.g_dc, ho, dc);
+      const float4 dP4 = has_cp ? mie_ld4(a.g_cpd, ho) : zero4;
+      const float4 cp4 = *reinterpret_cast<const float4*>(a.g_cpres + ho);
+      const float4 cc4 = *reinterpret_cast<const float4*>(a.g_cres + ho);
+      float cp[4] = {cp4.x, cp4.y, cp4.z, cp4.w}, cc[4] = {cc4.x, cc4.y, cc4.z, cc4.w};
+      const float dP[4] = {dP4.x, dP4.y, dP4.z, dP4.w};
+      float dh[4], dc[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        mie_lstm_gate_chain(rr[j].x, rr[j].y, rr[j].z, rr[j].w, dg[j].x, dg[j].y, dg[j].z, dg[j].w, cp[j], dP[j], cc[j],
+                            dh[j], dc[j]);
+        gr[j] = rr[j];
+      }
+      if (has_cp) *reinterpret_cast<float4*>(a.g_cpres + ho) = make_float4(cp[0], cp[1], cp[2], cp[3]);
+      *reinterpret_cast<float4*>(a.g_cres + ho) = make_float4(cc[0], cc[1], cc[2], cc[3]);
+      mie_st4(a.g_dh, ho, make_float4(dh[0], dh[1], dh[2], dh[3]));
+      mie_st4(a.g_dc, ho, make_float4(dc[0], dc[1], dc[2], dc[3]));
     }
   } else {
     // the last barrier of the main loop has retired every read of the staging buffers that is used
