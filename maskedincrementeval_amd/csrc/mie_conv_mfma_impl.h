@@ -802,21 +802,31 @@ __global__ __launch_bounds__(256) void k_conv_split_finish(ConvArgsT<T> a, int p
   const int tk = mie_pick_tile(a.ts, blockIdx.x, n, y0, x0);
   if (tk == 0) return;
   const int hout = a.ts.h, wout = a.ts.w, cout = a.cout;
-  const int cb = (cout + (int)gridDim.y - 1) / (int)gridDim.y;      // channels of this block
+  const int cb = (((cout + (int)gridDim.y - 1) / (int)gridDim.y) + 3) & ~3;      // channels of this block (whole groups of four)
   const int c0 = (int)blockIdx.y * cb;
   const int cn = (cout - c0 < cb) ? cout - c0 : cb;
-  for (int idx = threadIdx.x; idx < 64 * cn; idx += 256) {
-    const int p = idx / cn, co = c0 + (idx - p * cn);
+  const int qn = cn >> 2;                                             // groups of four adjacent channels
+  for (int idx = threadIdx.x; idx < 64 * qn; idx += 256) {
+    const int p = idx / qn, co = c0 + 4 * (idx - p * qn);
     const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
     if (oy >= hout || ox >= wout) continue;
     const long long off = (((long long)n * hout + oy) * wout + ox) * cout + co;
     if (tk == 2) {
-      mie_st(a.out, off, 0.f);
+      mie_st4(a.out, off, make_float4(0.f, 0.f, 0.f, 0.f));
       continue;
     }
-    float sum = a.ws[off];
-    for (int q = 1; q < parts; ++q) sum += a.ws[(long long)q * a.ws_plane + off];
-    conv_store(a, off, co, sum);
+    float4 sum = *reinterpret_cast<const float4*>(a.ws + off);
+    for (int q = 1; q < parts; ++q) {
+      const float4 part = *reinterpret_cast<const float4*>(a.ws + (long long)q * a.ws_plane + off);
+      sum.x += part.x; sum.y += part.y; sum.z += part.z; sum.w += part.w;
+    }
+    const long long offs[1] = {off};
+    const int cos[1] = {co};
+    const bool oks[1] = {true};
+    const float4 accs[1] = {sum};
+    float4 r0[1], add[1];
+    conv_epilogue_load4<T, 1>(a, offs, oks, r0, add);
+    conv_epilogue_store4<T, 1>(a, offs, cos, oks, accs, r0, add);
   }
 }
 

@@ -50,7 +50,7 @@ __global__ __launch_bounds__(256) void k_tconv_mfma(ConvArgsT<T> a, TileSetDev p
   constexpr int RING = ring_size(UPC);
   constexpr int PD = RING - 1;
   constexpr int CO_BLK = 32 * WN;
-  constexpr int RED = (WK > 1) ? WK * 64 * CO_BLK : 0;       // one phase at a time
+  constexpr int RED = WK * 64 * CO_BLK;                      // the accumulators of one phase, parked for the epilogue
   constexpr int STAGE_F = NBUF * STAGE * (int)sizeof(T) / 4;
   constexpr int SMEM = STAGE_F > RED ? STAGE_F : RED;
   static_assert(SMEM * 4 <= 65536, "LDS budget");
@@ -72,10 +72,11 @@ __global__ __launch_bounds__(256) void k_tconv_mfma(ConvArgsT<T> a, TileSetDev p
 
   if (tk == 2) {                                             // stale block: zero this workgroup's slab of its 16x16 pixels
     if (SPLIT) return;                                       // (the finish kernel zeroes the stale output tiles)
-    for (int idx = tid; idx < 256 * CO_BLK; idx += 256) {
-      const int p = idx / CO_BLK, col = idx - p * CO_BLK;
+    for (int idx = tid; idx < 64 * CO_BLK; idx += 256) {      // groups of four channels
+      const int p = idx / (CO_BLK / 4), col = 4 * (idx - p * (CO_BLK / 4));
       const int oy = 2 * y0 + (p >> 4), ox = 2 * x0 + (p & 15);
-      if (oy < hout && ox < wout) mie_st(a.out, (((long long)n * hout + oy) * wout + ox) * cout + co0 + col, 0.f);
+      if (oy < hout && ox < wout)
+        mie_st4(a.out, (((long long)n * hout + oy) * wout + ox) * cout + co0 + col, make_float4(0.f, 0.f, 0.f, 0.f));
     }
     return;
   }
@@ -218,62 +219,50 @@ __global__ __launch_bounds__(256) void k_tconv_mfma(ConvArgsT<T> a, TileSetDev p
   auto epilogue = [&](auto PH) {
     constexpr int ph = decltype(PH)::value;
     constexpr int py = ph >> 1, px = ph & 1;
-    if constexpr (WK == 1) {
+    // every wave parks the phase's accumulators in LDS; a thread then owns groups of four adjacent output channels
+    // of a pixel (16-byte reads of the k-split partial sums, 16-byte reservoir accesses, 16- / 8-byte delta accesses)
+    constexpr int QPP = CO_BLK / 4;
+    constexpr int PER = 64 * QPP / 256;
+    float* red = smem + wk * (64 * CO_BLK);
 #pragma unroll
-      for (int mb = 0; mb < 2; ++mb) {
-        long long off[16];
-        int co[16];
-        bool ok[16];
-        float v[16];
+    for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int p = mb * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-          const int iy = y0 + (p >> 3), ix = x0 + (p & 7);
-          off[r] = (((long long)n * hout + 2 * iy + py) * wout + 2 * ix + px) * cout + cob0 + l32;
-          co[r] = cob0 + l32;
-          ok[r] = iy < a.h_in && ix < a.w_in;
-          v[r] = acc[ph][mb][r];
-        }
-        conv_store_batch<T, 16>(a, off, co, ok, v);
+      for (int r = 0; r < 16; ++r) {
+        const int p = mb * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+        red[p * CO_BLK + wn * 32 + l32] = acc[ph][mb][r];
       }
-    } else {
-      constexpr int PER = 64 * CO_BLK / 256;
-      float* red = smem + wk * (64 * CO_BLK);
+    __syncthreads();
+    long long off[PER];
+    int co[PER];
+    bool ok[PER];
+    float4 v[PER];
 #pragma unroll
-      for (int mb = 0; mb < 2; ++mb)
+    for (int i = 0; i < PER; ++i) {
+      const int idx = tid + 256 * i;
+      const int p = idx / QPP, col = 4 * (idx - p * QPP);
+      const int iy = y0 + (p >> 3), ix = x0 + (p & 7);
+      ok[i] = iy < a.h_in && ix < a.w_in;
+      off[i] = (((long long)n * hout + 2 * iy + py) * wout + 2 * ix + px) * cout + co0 + col;
+      co[i] = co0 + col;
+      float4 sum = *reinterpret_cast<const float4*>(&smem[4 * idx]);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int p = mb * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-          red[p * CO_BLK + wn * 32 + l32] = acc[ph][mb][r];
-        }
-      __syncthreads();
-      long long off[PER];
-      int co[PER];
-      bool ok[PER];
-      float v[PER];
-#pragma unroll
-      for (int i = 0; i < PER; ++i) {
-        const int idx = tid + 256 * i;
-        const int p = idx / CO_BLK, col = idx - p * CO_BLK;
-        const int iy = y0 + (p >> 3), ix = x0 + (p & 7);
-        ok[i] = iy < a.h_in && ix < a.w_in;
-        off[i] = (((long long)n * hout + 2 * iy + py) * wout + 2 * ix + px) * cout + co0 + col;
-        co[i] = co0 + col;
-        float sum = smem[idx];
-#pragma unroll
-        for (int k2 = 1; k2 < WK; ++k2) sum += smem[k2 * (64 * CO_BLK) + idx];
-        v[i] = sum;
+      for (int k2 = 1; k2 < WK; ++k2) {
+        const float4 part = *reinterpret_cast<const float4*>(&smem[k2 * (64 * CO_BLK) + 4 * idx]);
+        sum.x += part.x; sum.y += part.y; sum.z += part.z; sum.w += part.w;
       }
-      if constexpr (SPLIT) {
-        float* plane = a.ws + (long long)bz * a.ws_plane;
-#pragma unroll
-        for (int i = 0; i < PER; ++i)
-          if (ok[i]) plane[off[i]] = v[i];
-      } else {
-        conv_store_batch<T, PER>(a, off, co, ok, v);
-      }
-      __syncthreads();                   // the next phase overwrites the reduction buffers
+      v[i] = sum;
     }
+    if constexpr (SPLIT) {
+      float* plane = a.ws + (long long)bz * a.ws_plane;
+#pragma unroll
+      for (int i = 0; i < PER; ++i)
+        if (ok[i]) *reinterpret_cast<float4*>(plane + off[i]) = v[i];
+    } else {
+      float4 r0[PER], add[PER];
+      conv_epilogue_load4<T, PER>(a, off, ok, r0, add);
+      conv_epilogue_store4<T, PER>(a, off, co, ok, v, r0, add);
+    }
+    __syncthreads();                   // the next phase overwrites the parked accumulators
   };
   epilogue(std::integral_constant<int, 0>{});
   epilogue(std::integral_constant<int, 1>{});
