@@ -32,9 +32,9 @@ __global__ __launch_bounds__(256) void k_conv_fewcin(ConvArgsT<T> a) {
   constexpr int NPIX = IT * IT;
   constexpr int IN_F = NPIX * FC_PS;
   constexpr int W_F = K * K * FC_CH * 32;
-  constexpr int RED_F = 2 * 64 * 16;             // accumulators of the two odd-tap waves
-  static_assert(RED_F <= IN_F + W_F, "the reduction reuses the staging area");
-  __shared__ float smem[IN_F + W_F];
+  constexpr int RED_F = 2 * 64 * 32;             // the accumulators of the two tap halves, parked for the epilogue
+  constexpr int SMEM_F = (IN_F + W_F > RED_F) ? IN_F + W_F : RED_F;      // (they reuse the staging area)
+  __shared__ float smem[SMEM_F];
   float* const s_in = smem;
   float* const s_w = smem + IN_F;
 
@@ -45,10 +45,11 @@ __global__ __launch_bounds__(256) void k_conv_fewcin(ConvArgsT<T> a) {
   const int hout = a.ts.h, wout = a.ts.w, cout = a.cout, cin = a.c1;
   const int co0 = blockIdx.y * 32;
   if (tk == 2) {   // stale tile: zero this workgroup's channel slab
-    for (int idx = tid; idx < 64 * 32; idx += 256) {
-      const int p = idx >> 5, col = idx & 31;
+    for (int idx = tid; idx < 64 * 8; idx += 256) {        // groups of four channels
+      const int p = idx >> 3, col = 4 * (idx & 7);
       const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
-      if (oy < hout && ox < wout) mie_st(a.out, (((long long)n * hout + oy) * wout + ox) * cout + co0 + col, 0.f);
+      if (oy < hout && ox < wout)
+        mie_st4(a.out, (((long long)n * hout + oy) * wout + ox) * cout + co0 + col, make_float4(0.f, 0.f, 0.f, 0.f));
     }
     return;
   }
@@ -118,31 +119,34 @@ __global__ __launch_bounds__(256) void k_conv_fewcin(ConvArgsT<T> a) {
       acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ta[2 * p], tb[2 * p * 32], acc, 0, 0, 0);
   }
   __syncthreads();                       // every wave is done with the staged operands
-  float* red = smem;
-  if (th == 1) {
-#pragma unroll
-    for (int r = 0; r < 16; ++r) red[(mb * 16 + r) * 64 + lane] = acc[r];
-  }
-  __syncthreads();
-  if (th == 1) return;
-
-  // ---- epilogue: lane = output column l32, 16 pixels of the block per lane ---------------------------
-  // (all reservoir / addend loads of the lane as one batch, then the stores: an element-by-element
-  // read-modify-write would be 16 dependent memory round trips)
-  long long off[16];
-  int co[16];
-  bool ok[16];
-  float v[16];
+  // ---- epilogue: the two tap halves park their accumulators in LDS; a thread then owns groups of four adjacent
+  // output channels of a pixel (16-byte reads of the two partial sums, 16-byte reservoir accesses, 16- / 8-byte
+  // delta accesses; all reservoir / addend loads of the thread as one batch, then the stores)
+  float* red = smem + th * (64 * 32);
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int p = mb * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-    const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
-    ok[r] = oy < hout && ox < wout;
-    off[r] = (((long long)n * hout + oy) * wout + ox) * cout + co0 + l32;
-    co[r] = co0 + l32;
-    v[r] = acc[r] + red[(mb * 16 + r) * 64 + lane];
+    red[p * 32 + l32] = acc[r];
   }
-  conv_store_batch<T, 16>(a, off, co, ok, v);
+  __syncthreads();
+  long long off[2];
+  int co[2];
+  bool ok[2];
+  float4 v[2], r0[2], add[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int idx = tid + 256 * i;
+    const int p = idx >> 3, col = 4 * (idx & 7);
+    const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
+    ok[i] = oy < hout && ox < wout;
+    off[i] = (((long long)n * hout + oy) * wout + ox) * cout + co0 + col;
+    co[i] = co0 + col;
+    const float4 s0 = *reinterpret_cast<const float4*>(&smem[4 * idx]);
+    const float4 s1 = *reinterpret_cast<const float4*>(&smem[64 * 32 + 4 * idx]);
+    v[i] = make_float4(s0.x + s1.x, s0.y + s1.y, s0.z + s1.z, s0.w + s1.w);
+  }
+  conv_epilogue_load4<T, 2>(a, off, ok, r0, add);
+  conv_epilogue_store4<T, 2>(a, off, co, ok, v, r0, add);
 }
 
 template <typename T>
