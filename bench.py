@@ -475,18 +475,34 @@ class NetBench:
         return dict(ms_eager=round(1e3 * eager, 4), ms_graph=round(1e3 * graph, 4))
 
 
-def event_time(torch, fn, warm=5, reps=50):
-    """Mean microseconds of fn() over `reps` back-to-back calls between two HIP events on the launch stream."""
+def event_time(torch, fn, warm=5, reps=50, replays=7):
+    """Microseconds of fn(): `reps` calls captured in one HIP graph (launches of 5-15 us are otherwise bound by
+    the host's call rate, not by the GPU), the graph replayed `replays` times between HIP events on the launch
+    stream; the median replay divided by `reps`."""
     for _ in range(warm):
         fn()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
-    e0.record()
-    for _ in range(reps):
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
         fn()
-    e1.record()
+    torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
-    return 1e3 * e0.elapsed_time(e1) / reps
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for _ in range(reps):
+            fn()
+    g.replay()
+    torch.cuda.synchronize()
+    times = []
+    for _ in range(replays):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        times.append(1e3 * e0.elapsed_time(e1) / reps)
+    return float(statistics.median(times))
 
 
 def config1_single_conv(torch, ops, _lib):
