@@ -74,6 +74,13 @@ extern "C" {
  * round-to-nearest-even.  Pointers to such buffers are `void*` below. */
 #define MIE_DTYPE_F32 0
 #define MIE_DTYPE_BF16 1
+/* fp32 deltas whose matrix-core contraction runs on the bf16 instruction at fp32 accuracy: every input and
+ * weight is split into three bf16 terms (hi + mid + lo, all 24 significant bits) and the six term products
+ * that matter are accumulated in fp32 -- what is dropped is below 2^-26 of |x*w| per product, a quarter of
+ * the rounding step of an fp32 multiply-add.  Taken by mie_pack_filter and by the `dtype` of
+ * mie_conv_masked / _ws / _noalloc, mie_conv_refresh, mie_upconv_masked and mie_conv_gates_masked, with
+ * filter_mc packed for it; every buffer is what it is for MIE_DTYPE_F32.  Shapes: mie_conv_f32x3_takes. */
+#define MIE_DTYPE_F32_BF16X3 2
 
 /* frame kinds of mie_events_to_frame */
 #define MIE_EVENTS_VOXEL 0      /* num_bins channels, linear weights in time   */
@@ -150,14 +157,24 @@ int mie_build_mask_tiles(const uint8_t* in_mask, const uint8_t* in_mask2,
  * 16-byte load:
  *   MIE_DTYPE_F32  (cin % 8 == 0):  P[ci/8][tap][(ci%8)/4][co][ci%4], fp32
  *   MIE_DTYPE_BF16 (cin % 16 == 0): P[ci/16][tap][(ci%16)/8][co][ci%8], bf16
- * `packed` holds cin*k*k*cout elements of that type; do this once per weight
- * update.
+ *   MIE_DTYPE_F32_BF16X3 (cin % 16 == 0): P[ci/16][tap][term][(ci%16)/8][co][ci%8], bf16,
+ *        term 0 / 1 / 2 = the weight rounded to bf16, the rest of it rounded to bf16, what is left
+ * `packed` holds cin*k*k*cout elements of that type (three times that many bf16 for
+ * MIE_DTYPE_F32_BF16X3); do this once per weight update.
  * Replaces: convert_filter_out_channels_last
  * (ext/pointops/pointops_functional.py:13-14), which plays the same role for
  * the reference kernel.
  */
 int mie_pack_filter(const float* filter, int cin, int k, int cout, void* packed,
                     int dtype, void* stream);
+
+/*
+ * 1 if the matrix-core conv takes this shape with dtype MIE_DTYPE_F32_BF16X3 (k = 3 or 5, stride 1,
+ * c1, c2 and cout multiples of 32), else 0: such a call must then be made with MIE_DTYPE_F32 and the
+ * fp32 filter copy.  No counterpart in the reference (it has one arithmetic, cuDNN's or its own
+ * kernel's fp32: ext/pointops/_C_ext/pointops/ext_conv.cu:74-76).
+ */
+int mie_conv_f32x3_takes(int k, int stride, int c1, int c2, int cout);
 
 /*
  * Masked convolution of a delta: for every active tile of `out`

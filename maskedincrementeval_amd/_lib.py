@@ -23,7 +23,7 @@ NOALLOC_WS_BYTES = 8 * 1024 * 1024
 ACT_NONE, ACT_RELU, ACT_LEAKY_RELU, ACT_SIGMOID, ACT_TANH = 0, 1, 2, 3, 4
 FOOT_CONV, FOOT_UP2X, FOOT_TCONV = 0, 1, 2
 EVENTS_VOXEL, EVENTS_HISTOGRAM = 0, 1
-DTYPE_F32, DTYPE_BF16 = 0, 1
+DTYPE_F32, DTYPE_BF16, DTYPE_F32_BF16X3 = 0, 1, 2
 PATH_AUTO, PATH_VALU, PATH_MFMA = 0, 1, 2
 FLAG_KEEP_RESERVOIR = 1
 CNT_ACTIVE, CNT_STALE, CNT_TICKET, CNT_WORDS = 0, 1, 2, 4
@@ -37,7 +37,7 @@ EXPORTS = (
     "mie_maxpool_incr", "mie_accumulate", "mie_scale_incr", "mie_avgpool_incr", "mie_linear_incr", "mie_upconv_masked",
     "mie_conv_masked_ws", "mie_convgru_gates_incr", "mie_upsample2x_pair_incr", "mie_conv_masked_noalloc",
     "mie_convlstm_gates_refresh", "mie_convgru_gates_refresh", "mie_mul_dense", "mie_tconv2x_masked",
-    "mie_tconv2x_refresh",
+    "mie_tconv2x_refresh", "mie_conv_f32x3_takes",
 )
 
 
@@ -102,6 +102,8 @@ def _declare(l):
     l.mie_events_to_frame.restype = ci
     cd = ctypes.c_double
     l.mie_events_to_frame.argtypes = [vp, ci, ci, ci, ci, ci, ci, ci, ci, ci, cd, cd, cd, cd, ci, vp, vp, vp]
+    l.mie_conv_f32x3_takes.restype = ci
+    l.mie_conv_f32x3_takes.argtypes = [ci, ci, ci, ci, ci]
     l.mie_pack_filter.restype = ci
     l.mie_pack_filter.argtypes = [vp, ci, ci, ci, vp, ci, vp]
     l.mie_conv_refresh.restype = ci

@@ -26,6 +26,9 @@ struct ConvArgsT {
   float* ws; long long ws_floats; long long ws_plane;
   // Matrix-core path: launch order permuted per XCD (number of slab groups, 0 = plain order); set by the launchers.
   int xcd_fs;
+  // Matrix-core path, fp32 deltas: filt_mc is the three-term bf16 copy and the contraction runs as six bf16 products
+  // per term pair (MIE_DTYPE_F32_BF16X3).
+  int x3;
   TileSetDev ts;
 };
 typedef ConvArgsT<float> ConvArgs;
@@ -216,3 +219,5 @@ static __device__ __forceinline__ void mie_lstm_gate_chain(float& ri, float& rf,
   cc = c1;
 }
 bool mie_conv_mfma_takes(int k, int s, int dtype, int c1, int c2, int cout);
+// The same for the three-term form of fp32 deltas (MIE_DTYPE_F32_BF16X3).
+bool mie_conv_x3_takes(int k, int s, int c1, int c2, int cout);

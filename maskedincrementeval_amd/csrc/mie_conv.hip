@@ -320,7 +320,7 @@ int conv_impl(const char* who, const T* x, const uint8_t* xmask, int c1, const T
               T* out_delta, const T* addend, float* reservoir, int act_kind, float slope,
               int path, bool refresh, const float* bias, void* stream,
               const GatesOperands<T>* gates = nullptr, void* workspace = nullptr,
-              long long workspace_bytes = 0) {
+              long long workspace_bytes = 0, bool x3 = false) {
   mie_clear_error();
   int rc = mie_check_tileset(out, who);
   if (rc != MIE_OK) return rc;
@@ -376,8 +376,15 @@ int conv_impl(const char* who, const T* x, const uint8_t* xmask, int c1, const T
   MIE_REQUIRE(workspace == nullptr || (workspace != (void*)out_delta && workspace != (void*)reservoir &&
                                        workspace != (const void*)x && workspace != (const void*)x2),
               MIE_ERR_INVALID_ARG, "%s: workspace must not alias an operand", who);
-  const bool mfma_ok = (filter_mc != nullptr) && (cin_total % pmul == 0) &&
-                       mie_conv_mfma_takes(k, stride, dtype_of<T>(), c1, c2, cout);
+  MIE_REQUIRE(!x3 || (sizeof(T) == 4 && path != MIE_PATH_VALU), MIE_ERR_INVALID_ARG,
+              "%s: MIE_DTYPE_F32_BF16X3 is a mode of the matrix-core path for fp32 deltas", who);
+  const bool mfma_ok = x3 ? (filter_mc != nullptr && cin_total % 16 == 0 && mie_conv_x3_takes(k, stride, c1, c2, cout))
+                          : ((filter_mc != nullptr) && (cin_total % pmul == 0) &&
+                             mie_conv_mfma_takes(k, stride, dtype_of<T>(), c1, c2, cout));
+  MIE_REQUIRE(!x3 || mfma_ok, MIE_ERR_UNSUPPORTED,
+              "%s: MIE_DTYPE_F32_BF16X3 needs filter_mc packed in that layout, k = 3 or 5, stride 1 and channel counts "
+              "that are multiples of 32 (k=%d stride=%d c1=%d c2=%d cout=%d); see mie_conv_f32x3_takes", who, k, stride,
+              c1, c2, cout);
   MIE_REQUIRE(path == MIE_PATH_AUTO || path == MIE_PATH_VALU || path == MIE_PATH_MFMA,
               MIE_ERR_INVALID_ARG, "%s: unknown path %d", who, path);
   MIE_REQUIRE(path != MIE_PATH_MFMA || mfma_ok, MIE_ERR_UNSUPPORTED,
@@ -394,7 +401,7 @@ int conv_impl(const char* who, const T* x, const uint8_t* xmask, int c1, const T
   a.slope = slope; a.addend = addend; a.refresh = refresh ? 1 : 0; a.bias = bias;
   a.hid = 0; a.g_cpd = nullptr; a.g_cpm = nullptr; a.g_cpres = nullptr; a.g_cres = nullptr;
   a.g_dh = nullptr; a.g_dc = nullptr;
-  a.ws = nullptr; a.ws_floats = 0; a.ws_plane = 0; a.xcd_fs = 0;
+  a.ws = nullptr; a.ws_floats = 0; a.ws_plane = 0; a.xcd_fs = 0; a.x3 = x3 ? 1 : 0;
   a.ts = mie_dev_tileset(out);
   const unsigned cap = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
   hipStream_t st = (hipStream_t)stream;
@@ -451,6 +458,29 @@ __global__ __launch_bounds__(256) void k_pack_filter(const float* __restrict__ f
   mie_st(p, o, f[i]);
 }
 
+// The three-term copy for MIE_DTYPE_F32_BF16X3: every weight as hi + mid + lo in bf16 (each rounded to nearest even),
+// P[ci/16][tap][term][(ci%16)/8][co][ci%8].
+__global__ __launch_bounds__(256) void k_pack_filter_x3(const float* __restrict__ f, mie_bf16* __restrict__ p,
+                                                        int cin, int kk, int cout) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  const long long total = (long long)cin * kk * cout;
+  if (i >= total) return;
+  const int co = (int)(i % cout);
+  const long long t = i / cout;
+  const int tap = (int)(t % kk);
+  const int ci = (int)(t / kk);
+  const float v = f[i];
+  const mie_bf16 hi = (mie_bf16)v;
+  const float r1 = v - (float)hi;
+  const mie_bf16 mid = (mie_bf16)r1;
+  const mie_bf16 lo = (mie_bf16)(r1 - (float)mid);
+  const long long o = (((((long long)(ci / 16) * kk + tap) * 3) * 2 + (ci % 16) / 8) * cout + co) * 8 + (ci % 8);
+  const long long term = 2LL * cout * 8;
+  p[o] = hi;
+  p[o + term] = mid;
+  p[o + 2 * term] = lo;
+}
+
 namespace {
 
 template <typename T>
@@ -465,7 +495,7 @@ int tconv_impl(const char* who, const T* x, const uint8_t* xmask, int cin, int h
   a.slope = slope; a.addend = nullptr; a.refresh = refresh ? 1 : 0; a.bias = bias;
   a.hid = 0; a.g_cpd = nullptr; a.g_cpm = nullptr; a.g_cpres = nullptr; a.g_cres = nullptr;
   a.g_dh = nullptr; a.g_dc = nullptr;
-  a.ws = nullptr; a.ws_floats = 0; a.ws_plane = 0; a.xcd_fs = 0;
+  a.ws = nullptr; a.ws_floats = 0; a.ws_plane = 0; a.xcd_fs = 0; a.x3 = 0;
   a.ts = mie_dev_tileset(out);
   const unsigned cap = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
   if (k == 3 && stride == 2 && pad == 1 && out->h == 2 * h_in && out->w == 2 * w_in && cin <= 8 && cout % 4 == 0 &&
@@ -485,21 +515,38 @@ int tconv_impl(const char* who, const T* x, const uint8_t* xmask, int cin, int h
     MIE_REQUIRE((dtype) == MIE_DTYPE_F32 || (dtype) == MIE_DTYPE_BF16, MIE_ERR_UNSUPPORTED, \
                 "%s: unknown delta dtype %d", who, (int)(dtype));                         \
   } while (0)
+// The entry points of the matrix-core conv also take MIE_DTYPE_F32_BF16X3: fp32 deltas, three-term filter copy.
+#define MIE_CONV_DTYPE_X3_OK(dtype, who, x3)                                              \
+  do {                                                                                    \
+    if ((dtype) == MIE_DTYPE_F32_BF16X3) {                                                \
+      x3 = true;                                                                          \
+      dtype = MIE_DTYPE_F32;                                                              \
+    }                                                                                     \
+    MIE_CONV_DTYPE_OK(dtype, who);                                                        \
+  } while (0)
+
+extern "C" int mie_conv_f32x3_takes(int k, int stride, int c1, int c2, int cout) {
+  return mie_conv_x3_takes(k, stride, c1, c2, cout) ? 1 : 0;
+}
 
 extern "C" int mie_pack_filter(const float* filter, int cin, int k, int cout, void* packed,
                                int dtype, void* stream) {
   const char* who = "mie_pack_filter";
-  MIE_CONV_DTYPE_OK(dtype, who);
+  bool x3 = false;
+  MIE_CONV_DTYPE_X3_OK(dtype, who, x3);
   MIE_REQUIRE(filter && packed, MIE_ERR_INVALID_ARG, "%s: NULL pointer", who);
   MIE_REQUIRE(cin > 0 && k > 0 && cout > 0, MIE_ERR_INVALID_ARG, "%s: sizes must be positive", who);
-  const int blk = dtype == MIE_DTYPE_BF16 ? 16 : 8;
+  const int blk = (dtype == MIE_DTYPE_BF16 || x3) ? 16 : 8;
   MIE_REQUIRE(cin % blk == 0, MIE_ERR_UNSUPPORTED, "%s: cin = %d is not a multiple of %d", who, cin, blk);
   MIE_REQUIRE(mie_aligned(filter, 16) && mie_aligned(packed, 16) && (const void*)filter != packed,
               MIE_ERR_INVALID_ARG, "%s: buffers must be 16-byte aligned and distinct", who);
   const long long total = (long long)cin * k * k * cout;
   MIE_REQUIRE(total < (1LL << 40), MIE_ERR_CAPACITY, "%s: filter too large", who);
   const dim3 grid((unsigned)((total + 255) / 256));
-  if (dtype == MIE_DTYPE_BF16)
+  if (x3)
+    hipLaunchKernelGGL(k_pack_filter_x3, grid, dim3(256), 0, (hipStream_t)stream, filter, (mie_bf16*)packed, cin,
+                       k * k, cout);
+  else if (dtype == MIE_DTYPE_BF16)
     hipLaunchKernelGGL(k_pack_filter<mie_bf16>, grid, dim3(256), 0, (hipStream_t)stream, filter,
                        (mie_bf16*)packed, cin, k * k, cout);
   else
@@ -515,7 +562,8 @@ extern "C" int mie_conv_masked(const void* x, const uint8_t* xmask, int c1, cons
                                void* out_delta, const void* addend, float* reservoir,
                                int act_kind, float slope, int path, int dtype, void* stream) {
   const char* who = "mie_conv_masked";
-  MIE_CONV_DTYPE_OK(dtype, who);
+  bool x3 = false;
+  MIE_CONV_DTYPE_X3_OK(dtype, who, x3);
   if (dtype == MIE_DTYPE_BF16) {
     typedef mie_bf16 T;
     return conv_impl<T>(who, (const T*)x, xmask, c1, (const T*)x2, x2mask, c2, h_in, w_in, filter,
@@ -525,7 +573,7 @@ extern "C" int mie_conv_masked(const void* x, const uint8_t* xmask, int c1, cons
   typedef float T;
   return conv_impl<T>(who, (const T*)x, xmask, c1, (const T*)x2, x2mask, c2, h_in, w_in, filter,
                       (const T*)filter_mc, cin_total, k, stride, pad, cout, out, (T*)out_delta,
-                      (const T*)addend, reservoir, act_kind, slope, path, false, nullptr, stream);
+                      (const T*)addend, reservoir, act_kind, slope, path, false, nullptr, stream, nullptr, nullptr, 0, x3);
 }
 
 extern "C" int mie_conv_masked_ws(const void* x, const uint8_t* xmask, int c1, const void* x2,
@@ -536,7 +584,8 @@ extern "C" int mie_conv_masked_ws(const void* x, const uint8_t* xmask, int c1, c
                                   int act_kind, float slope, int path, int dtype, void* workspace,
                                   long long workspace_bytes, void* stream) {
   const char* who = "mie_conv_masked_ws";
-  MIE_CONV_DTYPE_OK(dtype, who);
+  bool x3 = false;
+  MIE_CONV_DTYPE_X3_OK(dtype, who, x3);
   if (dtype == MIE_DTYPE_BF16) {
     typedef mie_bf16 T;
     return conv_impl<T>(who, (const T*)x, xmask, c1, (const T*)x2, x2mask, c2, h_in, w_in, filter,
@@ -548,7 +597,7 @@ extern "C" int mie_conv_masked_ws(const void* x, const uint8_t* xmask, int c1, c
   return conv_impl<T>(who, (const T*)x, xmask, c1, (const T*)x2, x2mask, c2, h_in, w_in, filter,
                       (const T*)filter_mc, cin_total, k, stride, pad, cout, out, (T*)out_delta,
                       (const T*)addend, reservoir, act_kind, slope, path, false, nullptr, stream, nullptr,
-                      workspace, workspace_bytes);
+                      workspace, workspace_bytes, x3);
 }
 
 // ---- the workspace form for callers that cannot allocate ---------------------------------------
@@ -590,7 +639,8 @@ extern "C" int mie_conv_masked_noalloc(const void* x, const uint8_t* xmask, int 
                                        void* out_delta, const void* addend, float* reservoir,
                                        int act_kind, float slope, int path, int dtype, void* stream) {
   const char* who = "mie_conv_masked_noalloc";
-  MIE_CONV_DTYPE_OK(dtype, who);
+  bool x3 = false;
+  MIE_CONV_DTYPE_X3_OK(dtype, who, x3);
   int rc = mie_check_tileset(out, who);
   if (rc != MIE_OK) return rc;
   MIE_REQUIRE(cout > 0, MIE_ERR_INVALID_ARG, "%s: cout must be positive", who);
@@ -615,7 +665,7 @@ extern "C" int mie_conv_masked_noalloc(const void* x, const uint8_t* xmask, int 
   return conv_impl<T>(who, (const T*)x, xmask, c1, (const T*)x2, x2mask, c2, h_in, w_in, filter,
                       (const T*)filter_mc, cin_total, k, stride, pad, cout, out, (T*)out_delta,
                       (const T*)addend, reservoir, act_kind, slope, path, false, nullptr, stream, nullptr,
-                      ws, (long long)MIE_NOALLOC_WS_BYTES);
+                      ws, (long long)MIE_NOALLOC_WS_BYTES, x3);
 }
 
 extern "C" int mie_conv_refresh(const void* x, int c1, const void* x2, int c2, int h_in,
@@ -625,7 +675,8 @@ extern "C" int mie_conv_refresh(const void* x, int c1, const void* x2, int c2, i
                                 void* out_dense, const void* addend, float* reservoir,
                                 int act_kind, float slope, int path, int dtype, void* stream) {
   const char* who = "mie_conv_refresh";
-  MIE_CONV_DTYPE_OK(dtype, who);
+  bool x3 = false;
+  MIE_CONV_DTYPE_X3_OK(dtype, who, x3);
   if (dtype == MIE_DTYPE_BF16) {
     typedef mie_bf16 T;
     return conv_impl<T>(who, (const T*)x, nullptr, c1, (const T*)x2, nullptr, c2, h_in, w_in, filter,
@@ -635,7 +686,7 @@ extern "C" int mie_conv_refresh(const void* x, int c1, const void* x2, int c2, i
   typedef float T;
   return conv_impl<T>(who, (const T*)x, nullptr, c1, (const T*)x2, nullptr, c2, h_in, w_in, filter,
                       (const T*)filter_mc, cin_total, k, stride, pad, cout, out, (T*)out_dense,
-                      (const T*)addend, reservoir, act_kind, slope, path, true, bias, stream);
+                      (const T*)addend, reservoir, act_kind, slope, path, true, bias, stream, nullptr, nullptr, 0, x3);
 }
 
 namespace {
@@ -644,7 +695,8 @@ int conv_gates_entry(const char* who, const void* x, const uint8_t* xmask, int c
                      const uint8_t* x2mask, int c2, int h_in, int w_in, const float* filter,
                      const void* filter_mc, int cin_total, int hid, const mie_tileset* out,
                      float* gates_res, const void* cprev_delta, const uint8_t* cprev_mask,
-                     float* cprev_res, float* cell_res, void* h_delta, void* c_delta, void* stream) {
+                     float* cprev_res, float* cell_res, void* h_delta, void* c_delta, void* stream,
+                     bool x3 = false) {
   MIE_REQUIRE(hid > 0 && hid <= (1 << 20), MIE_ERR_INVALID_ARG, "%s: hid = %d out of range", who, hid);
   MIE_REQUIRE(gates_res && cprev_res && cell_res && h_delta && c_delta, MIE_ERR_INVALID_ARG,
               "%s: NULL pointer", who);
@@ -658,7 +710,7 @@ int conv_gates_entry(const char* who, const void* x, const uint8_t* xmask, int c
   g.cell_res = cell_res; g.h_delta = (T*)h_delta; g.c_delta = (T*)c_delta;
   return conv_impl<T>(who, (const T*)x, xmask, c1, (const T*)x2, x2mask, c2, h_in, w_in, filter,
                       (const T*)filter_mc, cin_total, 3, 1, 1, 4 * hid, out, (T*)nullptr, (const T*)nullptr,
-                      gates_res, MIE_ACT_NONE, 0.f, MIE_PATH_MFMA, false, nullptr, stream, &g);
+                      gates_res, MIE_ACT_NONE, 0.f, MIE_PATH_MFMA, false, nullptr, stream, &g, nullptr, 0, x3);
 }
 
 int tconv_entry(const char* who, const void* x, const uint8_t* xmask, int cin, int h_in, int w_in,
@@ -713,7 +765,7 @@ template <typename T>
 int upconv_entry(const char* who, const void* a_lo, const uint8_t* amask, const void* b_lo, const uint8_t* bmask,
                  int c, int h_lo, int w_lo, const float* filter, const void* filter_mc, int cin_total, int k,
                  int pad, int cout, const mie_tileset* out, void* out_delta, const void* addend, float* reservoir,
-                 int act_kind, float slope, void* stream) {
+                 int act_kind, float slope, void* stream, bool x3 = false) {
   int rc = mie_check_tileset(out, who);
   if (rc != MIE_OK) return rc;
   MIE_REQUIRE(a_lo && filter, MIE_ERR_INVALID_ARG, "%s: NULL pointer (a and filter are required)", who);
@@ -727,7 +779,7 @@ int upconv_entry(const char* who, const void* a_lo, const uint8_t* amask, const 
                 "%s: only the 5x5 pad-2 conv is implemented for more than 8 channels or two inputs (k=%d pad=%d)", who, k, pad);
     MIE_REQUIRE(filter_mc != nullptr, MIE_ERR_INVALID_ARG, "%s: filter_mc is required", who);
     const int chunk = 128 / (int)sizeof(T);      // 32 fp32 / 64 bf16 channels per staged chunk
-    MIE_REQUIRE(c % chunk == 0 && cout % 32 == 0 && cin_total % (32 / (int)sizeof(T)) == 0, MIE_ERR_UNSUPPORTED,
+    MIE_REQUIRE(c % chunk == 0 && cout % 32 == 0 && cin_total % (x3 ? 16 : 32 / (int)sizeof(T)) == 0, MIE_ERR_UNSUPPORTED,
                 "%s: needs c %% %d == 0 and cout %% 32 == 0 (c=%d cout=%d)", who, chunk, c, cout);
   }
   MIE_REQUIRE(out->h == 2 * h_lo && out->w == 2 * w_lo, MIE_ERR_INVALID_ARG,
@@ -747,7 +799,7 @@ int upconv_entry(const char* who, const void* a_lo, const uint8_t* amask, const 
   a.slope = slope; a.addend = (const T*)addend; a.refresh = 0; a.bias = nullptr;
   a.hid = 0; a.g_cpd = nullptr; a.g_cpm = nullptr; a.g_cpres = nullptr; a.g_cres = nullptr;
   a.g_dh = nullptr; a.g_dc = nullptr;
-  a.ws = nullptr; a.ws_floats = 0; a.ws_plane = 0; a.xcd_fs = 0;
+  a.ws = nullptr; a.ws_floats = 0; a.ws_plane = 0; a.xcd_fs = 0; a.x3 = (x3 && !few) ? 1 : 0;
   a.ts = mie_dev_tileset(out);
   const unsigned cap = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
   if (few) {
@@ -767,12 +819,13 @@ extern "C" int mie_upconv_masked(const void* a, const uint8_t* amask, const void
                                  const void* addend, float* reservoir, int act_kind, float slope, int dtype,
                                  void* stream) {
   const char* who = "mie_upconv_masked";
-  MIE_CONV_DTYPE_OK(dtype, who);
+  bool x3 = false;
+  MIE_CONV_DTYPE_X3_OK(dtype, who, x3);
   if (dtype == MIE_DTYPE_BF16)
     return upconv_entry<mie_bf16>(who, a, amask, b, bmask, c, h_in, w_in, filter, filter_mc, cin_total, k, pad, cout,
                                   out, out_delta, addend, reservoir, act_kind, slope, stream);
   return upconv_entry<float>(who, a, amask, b, bmask, c, h_in, w_in, filter, filter_mc, cin_total, k, pad, cout, out,
-                             out_delta, addend, reservoir, act_kind, slope, stream);
+                             out_delta, addend, reservoir, act_kind, slope, stream, x3);
 }
 
 extern "C" int mie_conv_gates_masked(const void* x, const uint8_t* xmask, int c1, const void* x2,
@@ -783,12 +836,13 @@ extern "C" int mie_conv_gates_masked(const void* x, const uint8_t* xmask, int c1
                                      float* cprev_res, float* cell_res, void* h_delta,
                                      void* c_delta, int dtype, void* stream) {
   const char* who = "mie_conv_gates_masked";
-  MIE_CONV_DTYPE_OK(dtype, who);
+  bool x3 = false;
+  MIE_CONV_DTYPE_X3_OK(dtype, who, x3);
   if (dtype == MIE_DTYPE_BF16)
     return conv_gates_entry<mie_bf16>(who, x, xmask, c1, x2, x2mask, c2, h_in, w_in, filter, filter_mc,
                                       cin_total, hid, out, gates_res, cprev_delta, cprev_mask, cprev_res,
                                       cell_res, h_delta, c_delta, stream);
   return conv_gates_entry<float>(who, x, xmask, c1, x2, x2mask, c2, h_in, w_in, filter, filter_mc, cin_total,
                                  hid, out, gates_res, cprev_delta, cprev_mask, cprev_res, cell_res, h_delta,
-                                 c_delta, stream);
+                                 c_delta, stream, x3);
 }

@@ -13,6 +13,8 @@ bool mie_conv_mfma_takes(int k, int s, int dtype, int c1, int c2, int cout) {
   return false;
 }
 
+bool mie_conv_x3_takes(int k, int s, int c1, int c2, int cout) { return x3_takes(k, s, c1, c2, cout); }
+
 bool mie_launch_conv_mfma(const ConvArgsT<float>& a, int k, int s, unsigned cap, hipStream_t st) {
   return launch_any<float>(a, k, s, cap, st);
 }

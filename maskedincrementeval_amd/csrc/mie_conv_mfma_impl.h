@@ -109,10 +109,17 @@ __host__ __device__ constexpr int row_pitch_dw(int it, int ls_dw, int s) {
 
 // Ring size of the B-operand prefetch: the smallest divisor of the units per chunk that is
 // at least 4, so that ring slot (unit % ring) means the same registers in every chunk.
-__host__ __device__ constexpr int ring_size(int upc) {
-  for (int r = 4; r < upc; ++r)
+__host__ __device__ constexpr int ring_size(int upc, int least = 4) {
+  for (int r = least; r < upc; ++r)
     if (upc % r == 0) return r;
   return upc;
+}
+
+// Unit positions per chunk for the k-split over taps: at least n, padded until the ring size is at most 6
+// (the extra positions hold no unit for any wave and compile to nothing).
+__host__ __device__ constexpr int pad_units(int n) {
+  while (ring_size(n) > 6) ++n;
+  return n;
 }
 
 typedef float v4f __attribute__((ext_vector_type(4)));
@@ -147,6 +154,37 @@ __device__ __forceinline__ void mma_unit2(v16f& acc0, v16f& acc1, const float4& 
   mma_unit(acc1, a1, bv, mie_bf16());
 }
 
+// X3 (fp32 deltas multiplied as three bf16 terms each): v = hi + mid + lo with every term rounded to nearest
+// even, so |mid| <= 2^-9 |v|, |lo| <= 2^-18 |v| and the three terms carry all 24 bits of v.  The six products
+// hi*hi, hi*mid, mid*hi, hi*lo, mid*mid, lo*hi are exact in the fp32 accumulator's input; what is left out
+// (mid*lo, lo*mid, lo*lo) is below 2^-26 of |a*b|, a quarter of fp32's own rounding step.
+__device__ __forceinline__ void split3(const float (&f)[8], float4 (&pl)[3]) {
+  mie_bf16x8 b0, b1, b2;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const mie_bf16 hi = (mie_bf16)f[e];
+    const float r1 = f[e] - (float)hi;
+    const mie_bf16 mid = (mie_bf16)r1;
+    const float r2 = r1 - (float)mid;
+    b0[e] = hi; b1[e] = mid; b2[e] = (mie_bf16)r2;
+  }
+  const v4f r0 = __builtin_bit_cast(v4f, b0), r1 = __builtin_bit_cast(v4f, b1), r2 = __builtin_bit_cast(v4f, b2);
+  pl[0] = make_float4(r0[0], r0[1], r0[2], r0[3]);
+  pl[1] = make_float4(r1[0], r1[1], r1[2], r1[3]);
+  pl[2] = make_float4(r2[0], r2[1], r2[2], r2[3]);
+}
+// One unit (16 input channels of a tap) of the X3 contraction for the two pixel blocks of a tile: six bf16 MFMAs
+// per block, smallest terms first, the two accumulators interleaved.
+__device__ __forceinline__ void mma_unit2_x3(v16f& acc0, v16f& acc1, const float4 (&a0)[3], const float4 (&a1)[3],
+                                             const float4 (&b)[3]) {
+  mma_unit(acc0, a0[2], b[0], mie_bf16()); mma_unit(acc1, a1[2], b[0], mie_bf16());
+  mma_unit(acc0, a0[1], b[1], mie_bf16()); mma_unit(acc1, a1[1], b[1], mie_bf16());
+  mma_unit(acc0, a0[0], b[2], mie_bf16()); mma_unit(acc1, a1[0], b[2], mie_bf16());
+  mma_unit(acc0, a0[1], b[0], mie_bf16()); mma_unit(acc1, a1[1], b[0], mie_bf16());
+  mma_unit(acc0, a0[0], b[1], mie_bf16()); mma_unit(acc1, a1[0], b[1], mie_bf16());
+  mma_unit(acc0, a0[0], b[0], mie_bf16()); mma_unit(acc1, a1[0], b[0], mie_bf16());
+}
+
 // One 16-byte slot of delta elements <-> fp32 values (4 of them, or 8 for bf16).
 __device__ __forceinline__ void slot_to_f32(const float4& raw, float (&f)[4], float) {
   f[0] = raw.x; f[1] = raw.y; f[2] = raw.z; f[3] = raw.w;
@@ -176,30 +214,46 @@ __device__ __forceinline__ float4 f32_to_slot(const float (&f)[8], mie_bf16) {
 // fp32 and unactivated, into its own plane of the workspace (a.ws, laid out like the output), and
 // k_conv_split_finish adds the planes in a fixed order and runs the epilogue.  Only the 32-channel
 // slab kernels (WN = 1) have this form.
-template <typename T, int K, int S, int WN, int NB, bool HALF, bool GATES = false, bool UP = false, bool SPLIT = false>
+//
+// X3 (fp32 deltas only): the contraction runs on the bf16 matrix-core instruction at fp32 accuracy.  Every staged
+// input value and every filter value is split into three bf16 terms (split3; the filter once, by
+// mie_pack_filter); the staged tile is three bf16 planes in LDS, a unit is 16 input channels of a tap, and
+// its six significant term products are six v_mfma_f32_32x32x16_bf16 per pixel block -- 6 x 32 cycles for what
+// eight v_mfma_f32_32x32x2_f32 take 8 x 64 cycles to do.  Chunks of 32 channels (two units per tap); the k-split
+// of the 32-column slab kernels (WK = 4) is over (sub-chunk, tap parity).  Global loads, masks, epilogue: fp32.
+template <typename T, int K, int S, int WN, int NB, bool HALF, bool GATES = false, bool UP = false, bool SPLIT = false,
+          bool X3 = false>
 __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
-  constexpr int NBUF = stage_buffers(S, (int)sizeof(T));
-  constexpr int EPS = 16 / (int)sizeof(T);                   // elements per 16-byte slot (4 / 8)
+  static_assert(!X3 || (sizeof(T) == 4 && S == 1 && !HALF && (K == 3 || K == 5)), "X3: fp32 deltas, 3x3 / 5x5, stride 1");
+  using TL = std::conditional_t<X3, mie_bf16, T>;            // element type in LDS and on the matrix cores
+  constexpr int PL = X3 ? 3 : 1;                             // operand planes (terms per value)
+  constexpr int GPS = X3 ? 2 : 1;                            // 16-byte global loads per staging slot
+  constexpr int NBUF = X3 ? (K == 3 ? 2 : 1) : stage_buffers(S, (int)sizeof(T));
+  constexpr int EPS = 16 / (int)sizeof(TL);                  // elements per 16-byte slot (4 / 8)
   constexpr int SUB = 2 * EPS;                               // channels per unit (8 / 16)
   constexpr int WK = 4 / WN;
   constexpr int IT = 7 * S + K;                              // input tile edge incl. halo
-  constexpr int CC = stage_channels(K, S, HALF) * (4 / (int)sizeof(T));   // channels per LDS stage
+  constexpr int CC = X3 ? 32 : stage_channels(K, S, HALF) * (4 / (int)sizeof(T));   // channels per LDS stage
   constexpr int LS = CC + EPS;                               // LDS elements per staged pixel
   constexpr int NPIX = IT * IT;
   constexpr int Q4 = CC / EPS;                               // 16-byte slots per pixel
   constexpr int NSLOT = NPIX * Q4;
-  constexpr int NLD = (NSLOT + 255) / 256;                   // staging loads per thread
-  constexpr int RP = row_pitch_dw(IT, LS * (int)sizeof(T) / 4, S) * 4 / (int)sizeof(T);   // elements per tile row
-  constexpr int STAGE = IT * RP;                             // elements per staging buffer
+  constexpr int NLD = (NSLOT + 255) / 256;                   // staging slots per thread
+  constexpr int RP = row_pitch_dw(IT, LS * (int)sizeof(TL) / 4, S) * 4 / (int)sizeof(TL);   // elements per tile row
+  constexpr int STAGE = IT * RP;                             // elements per plane of a staging buffer
   constexpr int NQ = CC / SUB;                               // sub-chunks (units per tap) per stage
-  static_assert(NQ % WK == 0, "the k-split is over whole sub-chunks");
-  constexpr int NQW = NQ / WK;                               // sub-chunks per wave
-  constexpr int UPC = K * K * NQW;                           // units per chunk and wave
-  constexpr int RING = ring_size(UPC);                       // B operand ring (divides UPC)
+  // k-split: over whole sub-chunks (every wave takes NQW of them, for every tap), or -- more waves than sub-chunks,
+  // X3 only -- one sub-chunk and every TP-th tap per wave (the last position of a chunk is then empty for some waves)
+  constexpr bool TPAR = WK > NQ;
+  static_assert(TPAR ? (X3 && WK % NQ == 0) : (NQ % WK == 0), "the k-split is over whole sub-chunks, or over taps");
+  constexpr int TP = TPAR ? WK / NQ : 1;                     // tap classes
+  constexpr int NQW = TPAR ? 1 : NQ / WK;                    // sub-chunks per wave
+  constexpr int UPC = TPAR ? pad_units((K * K + TP - 1) / TP) : K * K * NQW;   // unit positions per chunk and wave
+  constexpr int RING = (X3 && ring_size(UPC) > 6) ? ring_size(UPC, 3) : ring_size(UPC);   // B operand ring (divides UPC)
   constexpr int PD = RING - 1;                               // prefetch distance in units
   constexpr int CO_BLK = 32 * NB * WN;
   constexpr int RED = WK * 64 * CO_BLK;                      // every wave parks its accumulators here for the epilogue
-  constexpr int STAGE_F = NBUF * STAGE * (int)sizeof(T) / 4;  // the staging buffers, in floats
+  constexpr int STAGE_F = NBUF * PL * STAGE * (int)sizeof(TL) / 4;  // the staging buffers, in floats
   constexpr int LOS = CC;                                    // floats per source pixel in LDS
   constexpr int LO_F = UP ? 64 * LOS : 0;                    // fp32 sums of the 8x8 source block, CC channels
   static_assert(!UP || (S == 1 && K == 5 && !GATES), "the up-sampling variant is the 5x5 stride-1 conv");
@@ -207,7 +261,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   constexpr int SMEM = (STAGE_F + LO_F > RED) ? STAGE_F + LO_F : RED;
   static_assert(SMEM * 4 <= 65536, "LDS budget");
   __shared__ __attribute__((aligned(16))) float smem[SMEM];
-  T* const sbuf = reinterpret_cast<T*>(smem);
+  TL* const sbuf = reinterpret_cast<TL*>(smem);
   float* const s_lo = smem + STAGE_F;
 
   // (tile-list position, slab, part) of this workgroup.  Each of the 8 XCDs has an L2 of its own and the
@@ -364,7 +418,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   const int lo_y0 = (iy0 >> 1) - 1, lo_x0 = (ix0 >> 1) - 1;
   int lo_po[NLO];
   unsigned lo_ok1 = 0u, lo_ok2 = 0u, lo_inb = 0u;
-  float4 lo_a[NLO], lo_b[NLO];
+  float4 lo_a[NLO][GPS], lo_b[NLO][GPS];
   if (UP) {
 #pragma unroll
     for (int i = 0; i < NLO; ++i) {
@@ -384,7 +438,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   // therefore go out for every pixel inside the image, before the mask bytes are there (`first`), and the
   // masked pixels are zeroed when the bytes have arrived; from the second chunk on -- and in layers of fewer
   // chunks, where that would be a large share of the reads -- a masked pixel is not fetched at all.
-  float4 st_reg[NLD];
+  float4 st_reg[NLD][GPS];
   auto stage_load = [&](int c, bool first = false) {
     if constexpr (UP) {
       const T* dummy = a.filt_mc;
@@ -394,12 +448,15 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
         const long long eo = (long long)lo_po[i] * a.c1 + c * CC + EPS * q4;
         const bool k1 = ((first ? lo_inb : lo_ok1) >> i) & 1u;
         const bool k2 = first ? (a.x2 != nullptr && ((lo_inb >> i) & 1u)) : ((lo_ok2 >> i) & 1u);
-        float4 v = *reinterpret_cast<const float4*>(k1 ? a.x + eo : dummy);
-        float4 u = *reinterpret_cast<const float4*>(k2 ? a.x2 + eo : dummy);
-        v.x = k1 ? v.x : 0.f; v.y = k1 ? v.y : 0.f; v.z = k1 ? v.z : 0.f; v.w = k1 ? v.w : 0.f;
-        u.x = k2 ? u.x : 0.f; u.y = k2 ? u.y : 0.f; u.z = k2 ? u.z : 0.f; u.w = k2 ? u.w : 0.f;
-        lo_a[i] = v;
-        lo_b[i] = u;
+#pragma unroll
+        for (int g = 0; g < GPS; ++g) {
+          float4 v = *reinterpret_cast<const float4*>(k1 ? a.x + eo + 4 * g : dummy);
+          float4 u = *reinterpret_cast<const float4*>(k2 ? a.x2 + eo + 4 * g : dummy);
+          v.x = k1 ? v.x : 0.f; v.y = k1 ? v.y : 0.f; v.z = k1 ? v.z : 0.f; v.w = k1 ? v.w : 0.f;
+          u.x = k2 ? u.x : 0.f; u.y = k2 ? u.y : 0.f; u.z = k2 ? u.z : 0.f; u.w = k2 ? u.w : 0.f;
+          lo_a[i][g] = v;
+          lo_b[i][g] = u;
+        }
       }
       return;
     }
@@ -419,13 +476,28 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
       const bool okb = (ok >> i) & 1u;
       const T* p = xin + (long long)st_po[i] * cs + ci0 + st_c4[i];
       p = okb ? p : dummy;
-      float4 v = *reinterpret_cast<const float4*>(p);
-      v.x = okb ? v.x : 0.f; v.y = okb ? v.y : 0.f; v.z = okb ? v.z : 0.f; v.w = okb ? v.w : 0.f;
-      st_reg[i] = v;
+#pragma unroll
+      for (int g = 0; g < GPS; ++g) {
+        float4 v = *reinterpret_cast<const float4*>(p + 4 * g);
+        v.x = okb ? v.x : 0.f; v.y = okb ? v.y : 0.f; v.z = okb ? v.z : 0.f; v.w = okb ? v.w : 0.f;
+        st_reg[i][g] = v;
+      }
+    }
+  };
+  // one staged slot to LDS: as it is, or (X3) its eight fp32 values as three bf16 planes
+  auto store_slot = [&](TL* dst, const float4 (&raw)[GPS]) {
+    if constexpr (X3) {
+      const float f[8] = {raw[0].x, raw[0].y, raw[0].z, raw[0].w, raw[1].x, raw[1].y, raw[1].z, raw[1].w};
+      float4 pl[3];
+      split3(f, pl);
+#pragma unroll
+      for (int q = 0; q < 3; ++q) *reinterpret_cast<float4*>(dst + q * STAGE) = pl[q];
+    } else {
+      *reinterpret_cast<float4*>(dst) = raw[0];
     }
   };
   auto stage_store = [&](int buf) {
-    T* dst = sbuf + buf * STAGE;
+    TL* dst = sbuf + buf * (PL * STAGE);
     if constexpr (UP) {
       // x + x2 of the source block to LDS in fp32 (bit pattern zero = 0 in both element types) ...
 #pragma unroll
@@ -433,8 +505,15 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
         const int slot = tid + 256 * i;
         const int lpix = slot / Q4, q4 = slot - lpix * Q4;
         float fa[EPS], fb[EPS];
-        slot_to_f32(lo_a[i], fa, T());
-        slot_to_f32(lo_b[i], fb, T());
+        if constexpr (X3) {
+          const float ta[8] = {lo_a[i][0].x, lo_a[i][0].y, lo_a[i][0].z, lo_a[i][0].w, lo_a[i][1].x, lo_a[i][1].y, lo_a[i][1].z, lo_a[i][1].w};
+          const float tb[8] = {lo_b[i][0].x, lo_b[i][0].y, lo_b[i][0].z, lo_b[i][0].w, lo_b[i][1].x, lo_b[i][1].y, lo_b[i][1].z, lo_b[i][1].w};
+#pragma unroll
+          for (int e = 0; e < 8; ++e) fa[e] = ta[e], fb[e] = tb[e];
+        } else {
+          slot_to_f32(lo_a[i][0], fa, T());
+          slot_to_f32(lo_b[i][0], fb, T());
+        }
         if (lpix < 64) {
 #pragma unroll
           for (int e = 0; e < EPS; e += 4)
@@ -479,13 +558,21 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
           }
         }
         const int lrow = pix / IT;
-        *reinterpret_cast<float4*>(dst + lrow * RP + (pix - lrow * IT) * LS + EPS * q4) = f32_to_slot(o, T());
+        TL* d = dst + lrow * RP + (pix - lrow * IT) * LS + EPS * q4;
+        if constexpr (X3) {
+          float4 pl[3];
+          split3(o, pl);
+#pragma unroll
+          for (int q = 0; q < 3; ++q) *reinterpret_cast<float4*>(d + q * STAGE) = pl[q];
+        } else {
+          *reinterpret_cast<float4*>(d) = f32_to_slot(o, T());
+        }
       }
       return;
     }
 #pragma unroll
     for (int i = 0; i < NLD; ++i)
-      if (tid + 256 * i < NSLOT) *reinterpret_cast<float4*>(dst + st_lds[i]) = st_reg[i];
+      if (tid + 256 * i < NSLOT) store_slot(dst + st_lds[i], st_reg[i]);
   };
 
   // ---- operand addressing ------------------------------------------------------------------------
@@ -493,7 +580,12 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   // one sub-chunk: 8 input channels, of which this lane's half handles 4 (channel pairing see
   // the header).  Everything that depends on the unit index is a compile-time constant times
   // cout (B) or a compile-time LDS offset (A); the lane-dependent parts are loop invariant.
-  const int q0w = wk * NQW;
+  const int q0w = TPAR ? wk % NQ : wk * NQW;
+  const int par = TPAR ? wk / NQ : 0;                          // tap class of this wave (scalar)
+  // (tap, sub-chunk) of unit position `unit`; with the k-split over taps the tap depends on the wave and the last
+  // position may hold no unit (tap >= K*K): it then multiplies nothing and prefetches the last tap once more
+  auto unit_tap = [&](int unit) { return TPAR ? unit * TP + par : unit / NQW; };
+  auto unit_sub = [&](int unit) { return TPAR ? 0 : unit % NQW; };
   const int cob0 = co0 + wn * (32 * NB);                       // first column of this wave
   const int b_lane = (half * cout + l32) * EPS;                // lane part of the packed filter index
   int a_lane[2][2];                                            // lane part of the LDS index
@@ -507,21 +599,28 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
     a_lane[mb][1] = rowcol + EPS * (h0 ^ 1);
   }
   // filter row block of chunk c for this wave (c1 and c2 are multiples of CC: no partial chunks)
-  auto chunk_b = [&](int c) -> const T* {
+  auto chunk_b = [&](int c) -> const TL* {
     const bool second = c >= nch1;
     const int ci0 = (second ? c - nch1 : c) * CC;
     const int fb = second ? a.c1 : 0;
-    return a.filt_mc + ((long long)((fb + ci0) / SUB + q0w) * (K * K) * 2 * cout + cob0) * EPS;
+    return reinterpret_cast<const TL*>(a.filt_mc) +
+           ((long long)((fb + ci0) / SUB + q0w) * (K * K) * (PL * 2) * cout + cob0) * EPS;
   };
-  // Matrix-core filter copy: P[ci/8][tap][(ci%8)/4][co][ci%4] (fp32; 16 / 8 / 8 for bf16).  The
-  // k-steps of a unit are one 16-byte load per lane, 512 contiguous bytes per half wave.
-  float4 bring[RING][NB];
-  auto load_b = [&](const T* ub, int unit, float4 (&bv)[NB]) {
-    const int tap = unit / NQW, qi = unit % NQW;     // compile-time after unrolling
+  // Matrix-core filter copy: P[ci/8][tap][(ci%8)/4][co][ci%4] (fp32; 16 / 8 / 8 for bf16; X3: the bf16 layout with
+  // the three term planes of a (block, tap) next to each other, P[ci/16][tap][term][(ci%16)/8][co][ci%8]).  The
+  // k-steps of a unit are one 16-byte load per lane (and term), 512 contiguous bytes per half wave.
+  float4 bring[RING][NB][PL];
+  auto load_b = [&](const TL* ub, int unit, float4 (&bv)[NB][PL]) {
+    if (TPAR && unit * TP >= K * K) return;          // padding position: no unit for any wave
+    int tap = unit_tap(unit);                        // compile-time after unrolling, but for the k-split over taps
+    const int qi = unit_sub(unit);
+    if (TPAR && tap >= K * K) tap = K * K - 1;
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
-      bv[nb] = *reinterpret_cast<const float4*>(
-          ub + ((long long)((qi * (K * K) + tap) * 2) * cout + nb * 32) * EPS + b_lane);
+#pragma unroll
+      for (int q = 0; q < PL; ++q)
+        bv[nb][q] = *reinterpret_cast<const float4*>(
+            ub + ((long long)(((qi * (K * K) + tap) * PL + q) * 2) * cout + nb * 32) * EPS + b_lane);
   };
 
   // All B loads below are unconditional: a conditional load would make the compiler's wait
@@ -531,8 +630,8 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   // gridDim.z <= nch, so no range is empty)
   const int c_lo = SPLIT ? bz * nch / (int)gridDim.z : 0;
   const int c_hi = SPLIT ? (bz + 1) * nch / (int)gridDim.z : nch;
-  const T* ub_cur = chunk_b(c_lo);
-  const T* ub_next = ub_cur;
+  const TL* ub_cur = chunk_b(c_lo);
+  const TL* ub_next = ub_cur;
   MIE_STAMP(2);
   const bool early = c_hi - c_lo >= 4;      // uniform over the workgroup
   if (early) stage_load(c_lo, true);
@@ -567,28 +666,46 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   if (!early) {
   } else if constexpr (UP) {
 #pragma unroll
-    for (int i = 0; i < NLO; ++i) {
-      if (!((lo_ok1 >> i) & 1u)) lo_a[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (!((lo_ok2 >> i) & 1u)) lo_b[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-    }
+    for (int i = 0; i < NLO; ++i)
+#pragma unroll
+      for (int g = 0; g < GPS; ++g) {
+        if (!((lo_ok1 >> i) & 1u)) lo_a[i][g] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (!((lo_ok2 >> i) & 1u)) lo_b[i][g] = make_float4(0.f, 0.f, 0.f, 0.f);
+      }
   } else {
     const unsigned ok = (c_lo >= nch1) ? ok2 : ok1;
 #pragma unroll
     for (int i = 0; i < NLD; ++i)
-      if (!((ok >> i) & 1u)) st_reg[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+      for (int g = 0; g < GPS; ++g)
+        if (!((ok >> i) & 1u)) st_reg[i][g] = make_float4(0.f, 0.f, 0.f, 0.f);
   }
   stage_store(0);
   __syncthreads();
   MIE_STAMP(3);
 
   // A operand of unit `unit` from the staged chunk at `sin` (one 16-byte LDS read per pixel block).
-  auto load_a = [&](const T* sin, int unit, float4 (&dst)[2]) {
-    const int tap = unit / NQW, qi = unit % NQW;
+  auto load_a = [&](const TL* sin, int unit, float4 (&dst)[2][PL]) {
+    if (TPAR && unit * TP >= K * K) return;
+    int tap = unit_tap(unit);
+    const int qi = unit_sub(unit);
+    if (TPAR && tap >= K * K) tap = K * K - 1;
     const int ky = tap / K, kx = tap - ky * K;
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb)
-      dst[mb] = *reinterpret_cast<const float4*>(
-          &sin[a_lane[mb][(S == 2) ? ((ky >> 1) & 1) : 0] + ky * RP + kx * LS + SUB * qi]);
+#pragma unroll
+      for (int q = 0; q < PL; ++q)
+        dst[mb][q] = *reinterpret_cast<const float4*>(
+            &sin[q * STAGE + a_lane[mb][(S == 2) ? ((ky >> 1) & 1) : 0] + ky * RP + kx * LS + SUB * qi]);
+  };
+  // the MFMAs of one unit position
+  auto mma = [&](int unit, const float4 (&av)[2][PL], const float4 (&bv)[NB][PL]) {
+    if (TPAR && (unit * TP >= K * K || unit_tap(unit) >= K * K)) return;     // uniform over the wave
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      if constexpr (X3) mma_unit2_x3(acc[0][nb], acc[1][nb], av[0], av[1], bv[nb]);
+      else mma_unit2(acc[0][nb], acc[1][nb], av[0][0], av[1][0], bv[nb][0], T());
+    }
   };
 
   // Double-buffered kernels fold the chunk hand-over into the contraction, so that the matrix cores run
@@ -604,12 +721,12 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   // barrier at its end": what a chunk loses against its MFMA time is not the hand-over (see the header).
   constexpr bool PIPE = MIE_PIPE && NBUF == 2 && !UP && UPC >= 8;
   if constexpr (PIPE) {
-    float4 av[2][2], av0[2];
+    float4 av[2][2][PL], av0[2][PL];
     load_a(sbuf, 0, av0);
     for (int c = c_lo; c < c_hi; ++c) {
       const bool more = c + 1 < c_hi;
-      const T* sin = sbuf + ((c - c_lo) & 1) * STAGE;
-      const T* sin_next = sbuf + ((c - c_lo + 1) & 1) * STAGE;
+      const TL* sin = sbuf + ((c - c_lo) & 1) * (PL * STAGE);
+      const TL* sin_next = sbuf + ((c - c_lo + 1) & 1) * (PL * STAGE);
 #pragma unroll
       for (int i = 0; i < UPC; ++i) {
         if (PD > 0) {
@@ -619,11 +736,8 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
         }
         if (i + 1 < UPC) load_a(sin, i + 1, av[(i + 1) & 1]);
         __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-          if (i == 0) mma_unit2(acc[0][nb], acc[1][nb], av0[0], av0[1], bring[0][nb], T());
-          else mma_unit2(acc[0][nb], acc[1][nb], av[i & 1][0], av[i & 1][1], bring[i % RING][nb], T());
-        }
+        if (i == 0) mma(0, av0, bring[0]);
+        else mma(i, av[i & 1], bring[i % RING]);
         __builtin_amdgcn_sched_barrier(0);
         if (i == 0) {
           int cn = more ? c + 1 : c;      // after the last chunk: redundant re-load, never stored
@@ -654,11 +768,11 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
       const int cn = more ? c + 1 : c;      // after the last chunk: redundant re-load, never stored
       ub_next = chunk_b(cn);
       stage_load(cn);
-      const T* sin = sbuf + ((c - c_lo) % NBUF) * STAGE;
+      const TL* sin = sbuf + ((c - c_lo) % NBUF) * (PL * STAGE);
       // A operands are read one unit ahead as well (two register sets); the scheduling barriers
       // pin "issue the loads for later units, then multiply this unit" so that the compiler can
       // neither sink the prefetches next to their uses nor hoist them all to the top.
-      float4 av[2][2];
+      float4 av[2][2][PL];
       load_a(sin, 0, av[0]);
 #pragma unroll
       for (int i = 0; i < UPC; ++i) {
@@ -670,8 +784,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
         }
         if (i + 1 < UPC) load_a(sin, i + 1, av[(i + 1) & 1]);
         __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) mma_unit2(acc[0][nb], acc[1][nb], av[i & 1][0], av[i & 1][1], bring[i % RING][nb], T());
+        mma(i, av[i & 1], bring[i % RING]);
         __builtin_amdgcn_sched_barrier(0);
         if (PD == 0) load_b(ub_next, 0, bring[0]);   // ring of one: reload right after use
       }
@@ -854,7 +967,14 @@ bool launch_split(const ConvArgsT<T>& a0, unsigned cap, hipStream_t st) {
   while (2 * parts <= most && 2 * parts <= nch && groups * (2 * parts) <= max_wgs && (long long)(2 * parts) * a.ws_plane <= a.ws_floats)
     parts *= 2;
   if (parts < 2) return false;
-  hipLaunchKernelGGL((k_conv_mfma<T, K, S, 1, 1, false, false, false, true>), dim3(cap, a.cout / 32, parts), dim3(256), 0, st, a);
+  bool x3 = false;
+  if constexpr (sizeof(T) == 4 && S == 1 && (K == 3 || K == 5)) x3 = a.x3 != 0;
+  if (x3) {
+    if constexpr (sizeof(T) == 4 && S == 1 && (K == 3 || K == 5))
+      hipLaunchKernelGGL((k_conv_mfma<T, K, S, 1, 1, false, false, false, true, true>), dim3(cap, a.cout / 32, parts), dim3(256), 0, st, a);
+  } else {
+    hipLaunchKernelGGL((k_conv_mfma<T, K, S, 1, 1, false, false, false, true>), dim3(cap, a.cout / 32, parts), dim3(256), 0, st, a);
+  }
   unsigned ny = (unsigned)((1024 + cap - 1) / cap);
   if (ny > (unsigned)(a.cout / 4)) ny = (unsigned)(a.cout / 4);
   if (ny < 1) ny = 1;
@@ -922,6 +1042,42 @@ unsigned xcd_plan(ConvArgsT<T>& a, unsigned cap, int nslabs, int k, bool up = fa
   return ((cap + 7u) & ~7u) + 16u;
 }
 
+// X3 kernels (fp32 deltas, a.x3 set, the filter copy in the three-term layout): 3x3 / 5x5, stride 1, input channels in
+// whole chunks of 32, output slabs of 128 / 64 / 32 columns by the same rule as above.
+inline int pick_slab_x3(int cout, unsigned cap) {
+  const bool ok128 = cout % 128 == 0, ok64 = cout % 64 == 0, ok32 = cout % 32 == 0;
+  const int f = forced_slab();
+  if ((f == 128 && ok128) || (f == 64 && ok64) || (f == 32 && ok32)) return f;
+  const long long want = 400;
+  if (ok128 && ((long long)cap * (cout / 128) >= want || (!ok64 && !ok32))) return 128;
+  if (ok64 && ((long long)cap * (cout / 64) >= want || !ok32)) return 64;
+  if (ok32) return 32;
+  return 0;
+}
+inline bool x3_takes(int k, int s, int c1, int c2, int cout) {
+  return (k == 3 || k == 5) && s == 1 && c1 % 32 == 0 && c2 % 32 == 0 && cout % 32 == 0;
+}
+
+template <int K, bool GATES, bool UP>
+bool launch_x3(const ConvArgsT<float>& a0, unsigned cap, hipStream_t st) {
+  ConvArgsT<float> a = a0;
+  const int cout = a.cout;
+  if (!x3_takes(K, 1, a.c1, UP ? 0 : a.c2, cout)) return false;
+  switch (pick_slab_x3(cout, cap)) {
+    case 128:
+      hipLaunchKernelGGL((k_conv_mfma<float, K, 1, 4, 1, false, GATES, UP, false, true>), dim3(xcd_plan(a, cap, cout / 128, K, UP), cout / 128), dim3(256), 0, st, a);
+      return true;
+    case 64:
+      hipLaunchKernelGGL((k_conv_mfma<float, K, 1, 2, 1, false, GATES, UP, false, true>), dim3(xcd_plan(a, cap, cout / 64, K, UP), cout / 64), dim3(256), 0, st, a);
+      return true;
+    case 32:
+      hipLaunchKernelGGL((k_conv_mfma<float, K, 1, 1, 1, false, GATES, UP, false, true>), dim3(xcd_plan(a, cap, cout / 32, K, UP), cout / 32), dim3(256), 0, st, a);
+      return true;
+    default:
+      return false;
+  }
+}
+
 template <typename T, int K, int S, bool HALF>
 bool launch_depth(const ConvArgsT<T>& a0, unsigned cap, hipStream_t st) {
   constexpr int NQ = stage_channels(K, S, HALF) / 8;
@@ -951,6 +1107,9 @@ bool launch_depth(const ConvArgsT<T>& a0, unsigned cap, hipStream_t st) {
 // The 5x5 stride-1 conv over up2x(x + x2): full staging depth only.
 template <typename T>
 bool launch_up(const ConvArgsT<T>& a0, unsigned cap, hipStream_t st) {
+  if constexpr (sizeof(T) == 4) {
+    if (a0.x3) return launch_x3<5, false, true>(a0, cap, st);
+  }
   constexpr int FULL = stage_channels(5, 1) * (4 / (int)sizeof(T));
   if (a0.c1 % FULL != 0) return false;
   ConvArgsT<T> a = a0;
@@ -973,6 +1132,9 @@ bool launch_up(const ConvArgsT<T>& a0, unsigned cap, hipStream_t st) {
 // The gates conv of a ConvLSTM: 3x3, stride 1, full staging depth, gate chain in the epilogue.
 template <typename T>
 bool launch_gates(const ConvArgsT<T>& a0, unsigned cap, hipStream_t st) {
+  if constexpr (sizeof(T) == 4) {
+    if (a0.x3) return a0.cout == 4 * a0.hid && a0.hid % 8 == 0 && launch_x3<3, true, false>(a0, cap, st);
+  }
   constexpr int FULL = stage_channels(3, 1) * (4 / (int)sizeof(T));
   if (a0.c1 % FULL != 0 || a0.c2 % FULL != 0 || a0.cout != 4 * a0.hid || a0.hid % 8 != 0) return false;
   ConvArgsT<T> a = a0;
@@ -1012,6 +1174,14 @@ bool launch_ks(const ConvArgsT<T>& a, unsigned cap, hipStream_t st) {
 namespace {
 template <typename T>
 bool launch_any(const ConvArgsT<T>& a, int k, int s, unsigned cap, hipStream_t st) {
+  if constexpr (sizeof(T) == 4) {
+    if (a.x3) {
+      if (s != 1) return false;
+      if (k == 3) return launch_split<T, 3, 1>(a, cap, st) || launch_x3<3, false, false>(a, cap, st);
+      if (k == 5) return launch_split<T, 5, 1>(a, cap, st) || launch_x3<5, false, false>(a, cap, st);
+      return false;
+    }
+  }
   switch (k * 10 + s) {
     case 11: return launch_ks<T, 1, 1>(a, cap, st);
     case 12: return launch_ks<T, 1, 2>(a, cap, st);

@@ -352,7 +352,7 @@ int tconv2x_impl(const char* who, const void* x, const uint8_t* xmask, int c1, c
   a.pad = k / 2; a.cout = cout; a.out = (T*)out_delta; a.res = reservoir; a.act = act_kind; a.slope = slope;
   a.addend = (const T*)addend; a.refresh = refresh ? 1 : 0; a.bias = bias;
   a.hid = 0; a.g_cpd = nullptr; a.g_cpm = nullptr; a.g_cpres = nullptr; a.g_cres = nullptr; a.g_dh = nullptr; a.g_dc = nullptr;
-  a.ws = (float*)workspace; a.ws_floats = workspace_bytes / 4; a.ws_plane = 0; a.xcd_fs = 0;
+  a.ws = (float*)workspace; a.ws_floats = workspace_bytes / 4; a.ws_plane = 0; a.xcd_fs = 0; a.x3 = 0;
   a.ts = mie_dev_tileset(out);
   const TileSetDev pts = mie_dev_tileset(blocks);
   const bool ok = (k == 3) ? launch_tconv<T, 3>(a, pts, (hipStream_t)stream) : launch_tconv<T, 5>(a, pts, (hipStream_t)stream);

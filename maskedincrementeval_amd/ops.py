@@ -4,6 +4,7 @@ Each function checks shapes / layouts on the host, pulls raw device pointers
 and the current HIP stream out of torch, and calls one entry point of
 include/mie.h.  torch is used for memory and streams only.
 """
+import os
 from typing import Optional, Tuple
 
 import torch
@@ -259,18 +260,40 @@ def build_mask_tiles(in_mask, in_mask2, n, h_in, w_in, foot, k, stride, pad, out
     return out
 
 
-def pack_filter(filt: torch.Tensor, dtype=torch.float32) -> torch.Tensor:
+def pack_filter(filt: torch.Tensor, dtype=torch.float32, x3: bool = False) -> torch.Tensor:
     """Matrix-core copy of a contiguous fp32 [Cin,K,K,Cout] filter in `dtype`, shape
     [Cin/B, K*K, 2, Cout, B/2] with B = 8 (fp32) or 16 (bf16) input channels per block:
-    element [b,t,h,co,j] is filt[B*b + (B/2)*h + j, t//K, t%K, co]."""
+    element [b,t,h,co,j] is filt[B*b + (B/2)*h + j, t//K, t%K, co].
+    x3=True: the three-term bf16 copy of an fp32 filter (MIE_DTYPE_F32_BF16X3), shape [Cin/16, K*K, 3, 2, Cout, 8]:
+    [b,t,0] + [b,t,1] + [b,t,2] is the fp32 weight, each term rounded to bf16."""
     if filt.dim() != 4 or filt.shape[1] != filt.shape[2] or not filt.is_contiguous() or filt.dtype != torch.float32:
         raise ValueError("filter must be contiguous fp32 [Cin,K,K,Cout], got %s" % (tuple(filt.shape),))
     _require_gpu(filt, "filter")
     cin, k, _, cout = filt.shape
+    if x3:
+        packed = torch.empty((cin // 16, k * k, 3, 2, cout, 8), dtype=torch.bfloat16, device=filt.device)
+        check(lib().mie_pack_filter(filt.data_ptr(), cin, k, cout, packed.data_ptr(), _lib.DTYPE_F32_BF16X3, _stream(filt)))
+        return packed
     blk = 8 if dtype == torch.float32 else 16
     packed = torch.empty((cin // blk, k * k, 2, cout, blk // 2), dtype=dtype, device=filt.device)
     check(lib().mie_pack_filter(filt.data_ptr(), cin, k, cout, packed.data_ptr(), _DTYPES[dtype], _stream(filt)))
     return packed
+
+
+# How the matrix-core kernels multiply fp32 deltas: "bf16x3" = every value as three bf16 terms, six term products
+# per multiply on the bf16 matrix-core instruction (fp32 accuracy: what is dropped is below 2^-26 of a product; about
+# twice the rate of the fp32 instruction), where the library has that form (3x3 / 5x5, stride 1, channel counts in
+# multiples of 32); "native" = v_mfma_f32_32x32x2_f32 everywhere.  Environment variable MIE_F32_MATMUL.
+f32_matmul = os.environ.get("MIE_F32_MATMUL", "bf16x3")
+
+
+def f32x3_takes(k: int, stride: int, c1: int, c2: int, cout: int) -> bool:
+    """Whether a conv of this shape on fp32 deltas runs in the three-term bf16 form under the current setting."""
+    if f32_matmul != "bf16x3":
+        if f32_matmul != "native":
+            raise ValueError("ops.f32_matmul must be 'bf16x3' or 'native', not %r" % (f32_matmul,))
+        return False
+    return bool(lib().mie_conv_f32x3_takes(k, stride, c1, c2, cout))
 
 
 class ConvFilter:
@@ -284,10 +307,16 @@ class ConvFilter:
         self.mc = mc if _packed else (pack_filter(plain) if plain.is_cuda and plain.shape[0] % 8 == 0 else None)
         self._rows = {}
         self._bf16 = None
+        self._x3 = None
 
-    def for_dtype(self, dtype):
-        """(plain fp32 tensor, matrix-core copy | None) for deltas of `dtype`."""
+    def for_dtype(self, dtype, x3: bool = False):
+        """(plain fp32 tensor, matrix-core copy | None) for deltas of `dtype`; x3: the three-term copy for fp32
+        deltas (Cin % 16 == 0), made on first use."""
         if dtype == torch.float32:
+            if x3 and self.plain.is_cuda and self.plain.shape[0] % 16 == 0:
+                if self._x3 is None:
+                    self._x3 = pack_filter(self.plain.contiguous(), x3=True)
+                return self.plain, self._x3
             return self.plain, self.mc
         if self._bf16 is None:
             rounded = self.plain.to(torch.bfloat16).float().contiguous()
@@ -313,16 +342,24 @@ class ConvFilter:
         return sub
 
 
-def _filter_args(filt, k, dtype=torch.float32):
-    """(plain tensor, pointer of the matrix-core copy or None) of a Tensor or ConvFilter."""
+def _filter_args(filt, k, dtype=torch.float32, x3_shape=None, with_code=False):
+    """(plain tensor, pointer of the matrix-core copy or None) of a Tensor or ConvFilter; with_code: a third value,
+    the MIE_DTYPE_* code of the call.  x3_shape = (stride, c1, c2, cout): fp32 deltas take the three-term bf16 form
+    (its filter copy, its code) where the setting (f32_matmul) and the library allow it."""
     mc = None
+    code = _DTYPES.get(dtype)
     if isinstance(filt, ConvFilter):
-        filt, mc = filt.for_dtype(dtype)
+        x3 = (x3_shape is not None and dtype == torch.float32 and filt.plain.shape[0] % 16 == 0
+              and f32x3_takes(k, *x3_shape))
+        filt, mc = filt.for_dtype(dtype, x3)
+        if x3:
+            code = _lib.DTYPE_F32_BF16X3
     if filt.dim() != 4 or filt.shape[1] != k or filt.shape[2] != k or not filt.is_contiguous() \
             or filt.dtype != torch.float32:
         raise ValueError("filter must be contiguous fp32 [Cin,%d,%d,Cout], got %s" % (k, k, tuple(filt.shape)))
     _require_gpu(filt, "filter")
-    return filt, (None if mc is None else mc.data_ptr())
+    ptr = None if mc is None else mc.data_ptr()
+    return (filt, ptr, code) if with_code else (filt, ptr)
 
 
 # Workspace of the matrix-core conv for planes of very few tiles (a 16x16 plane is 4 tiles, 64 workgroups
@@ -352,7 +389,8 @@ def conv_masked(x, xmask, x2, x2mask, filt, k, stride, pad, out_ts: TileMask, ou
     if x2 is not None and (x2.shape[0] != n or x2.shape[2:] != x.shape[2:]):
         raise ValueError("x2 shape %s incompatible with x %s" % (tuple(x2.shape), tuple(x.shape)))
     dt = x.dtype
-    filt, mc_ptr = _filter_args(filt, k, dt)
+    filt, mc_ptr, code = _filter_args(filt, k, dt, (stride, c1, c2, filt.shape[3]) if path != _lib.PATH_VALU else None,
+                                      with_code=True)
     cin_total, cout = filt.shape[0], filt.shape[3]
     if tuple(out_delta.shape) != (n, cout, out_ts.h, out_ts.w) or out_ts.n != n:
         raise ValueError("out_delta shape %s, expected %s" % (tuple(out_delta.shape), (n, cout, out_ts.h, out_ts.w)))
@@ -376,7 +414,7 @@ def conv_masked(x, xmask, x2, x2mask, filt, k, stride, pad, out_ts: TileMask, ou
         nhwc_ptr(x2, "x2", dtype=dt), pix_ptr(x2mask, n, h, w, "x2mask"), c2, h, w,
         filt.data_ptr(), mc_ptr, cin_total, k, stride, pad, cout, out_ts.ref,
         nhwc_ptr(out_delta, "out_delta", dtype=dt), nhwc_ptr(addend, "addend", cout, dtype=dt),
-        nhwc_ptr(reservoir, "reservoir"), act, float(slope), path, delta_dtype(x), ws_ptr, ws_bytes, _stream(x)))
+        nhwc_ptr(reservoir, "reservoir"), act, float(slope), path, code, ws_ptr, ws_bytes, _stream(x)))
     return out_delta
 
 
@@ -404,7 +442,8 @@ def upconv_masked(a, amask, b, bmask, filt, k, pad, out_ts: TileMask, out_delta,
     dt = a.dtype
     if b is not None and (b.shape != a.shape or b.dtype != dt):
         raise ValueError("b %s %s does not match a %s %s" % (tuple(b.shape), b.dtype, tuple(a.shape), dt))
-    plain, mc_ptr = _filter_args(filt, k, dt)
+    plain, mc_ptr, code = _filter_args(filt, k, dt, (1, c, 0, filt.shape[3]) if (k == 5 and c > 8) else None,
+                                       with_code=True)
     cin_total, cout = plain.shape[0], plain.shape[3]
     if tuple(out_delta.shape) != (n, cout, 2 * h, 2 * w) or out_ts.n != n:
         raise ValueError("out_delta shape %s, expected %s" % (tuple(out_delta.shape), (n, cout, 2 * h, 2 * w)))
@@ -415,7 +454,7 @@ def upconv_masked(a, amask, b, bmask, filt, k, pad, out_ts: TileMask, out_delta,
         nhwc_ptr(a, "a", dtype=dt), pix_ptr(amask, n, h, w, "amask"), nhwc_ptr(b, "b", dtype=dt),
         pix_ptr(bmask, n, h, w, "bmask"), c, h, w, plain.data_ptr(), mc_ptr, cin_total, k, pad, cout, out_ts.ref,
         nhwc_ptr(out_delta, "out_delta", dtype=dt), nhwc_ptr(addend, "addend", cout, dtype=dt),
-        nhwc_ptr(reservoir, "reservoir"), act, float(slope), delta_dtype(a), _stream(a)))
+        nhwc_ptr(reservoir, "reservoir"), act, float(slope), code, _stream(a)))
     return out_delta
 
 
@@ -425,7 +464,8 @@ def conv_refresh(x, x2, filt, bias, k, stride, pad, out_ts: TileMask, out_dense,
     n, c1, h, w = x.shape
     c2 = 0 if x2 is None else x2.shape[1]
     dt = x.dtype
-    filt, mc_ptr = _filter_args(filt, k, dt)
+    filt, mc_ptr, code = _filter_args(filt, k, dt, (stride, c1, c2, filt.shape[3]) if path != _lib.PATH_VALU else None,
+                                      with_code=True)
     cin_total, cout = filt.shape[0], filt.shape[3]
     if tuple(out_dense.shape) != (n, cout, out_ts.h, out_ts.w):
         raise ValueError("out_dense shape %s, expected %s" % (tuple(out_dense.shape), (n, cout, out_ts.h, out_ts.w)))
@@ -436,7 +476,7 @@ def conv_refresh(x, x2, filt, bias, k, stride, pad, out_ts: TileMask, out_dense,
         nhwc_ptr(x, "x", dtype=dt), c1, nhwc_ptr(x2, "x2", dtype=dt), c2, h, w, filt.data_ptr(), mc_ptr,
         cin_total, k, stride, pad, cout, None if bias is None else bias.data_ptr(), out_ts.ref,
         nhwc_ptr(out_dense, "out_dense", dtype=dt), nhwc_ptr(addend, "addend", cout, dtype=dt),
-        nhwc_ptr(reservoir, "reservoir"), act, float(slope), path, delta_dtype(x), _stream(x)))
+        nhwc_ptr(reservoir, "reservoir"), act, float(slope), path, code, _stream(x)))
     return out_dense
 
 
@@ -811,7 +851,7 @@ def conv_gates_incr(x, xmask, x2, x2mask, filt: ConvFilter, out_ts: TileMask, ga
     n, c1, h, w = x.shape
     c2 = 0 if x2 is None else x2.shape[1]
     dt = x.dtype
-    plain, mc_ptr = _filter_args(filt, 3, dt)
+    plain, mc_ptr, code = _filter_args(filt, 3, dt, (1, c1, c2, filt.shape[3]), with_code=True)
     cin_total, cout = plain.shape[0], plain.shape[3]
     hid = cout // 4
     if tuple(gates_res.shape) != (n, cout, h, w):
@@ -826,7 +866,7 @@ def conv_gates_incr(x, xmask, x2, x2mask, filt: ConvFilter, out_ts: TileMask, ga
         plain.data_ptr(), mc_ptr, cin_total, hid, out_ts.ref, nhwc_ptr(gates_res, "gates_res"),
         nhwc_ptr(cprev_delta, "cprev_delta", dtype=dt), pix_ptr(cprev_mask, n, h, w, "cprev_mask"),
         nhwc_ptr(cprev_res, "cprev_res"), nhwc_ptr(cell_res, "cell_res"),
-        nhwc_ptr(h_delta, "h_delta", dtype=dt), nhwc_ptr(c_delta, "c_delta", dtype=dt), delta_dtype(x),
+        nhwc_ptr(h_delta, "h_delta", dtype=dt), nhwc_ptr(c_delta, "c_delta", dtype=dt), code,
         _stream(x)))
     return h_delta, c_delta
 
