@@ -157,32 +157,42 @@ __device__ __forceinline__ void mma_unit2(v16f& acc0, v16f& acc1, const float4& 
 // X3 (fp32 deltas multiplied as three bf16 terms each): v = hi + mid + lo with every term rounded to nearest
 // even, so |mid| <= 2^-9 |v|, |lo| <= 2^-18 |v| and the three terms carry all 24 bits of v.  The six products
 // hi*hi, hi*mid, mid*hi, hi*lo, mid*mid, lo*hi are exact in the fp32 accumulator's input; what is left out
-// (mid*lo, lo*mid, lo*lo) is below 2^-26 of |a*b|, a quarter of fp32's own rounding step.
+// (mid*lo, lo*mid, lo*lo) is at most 2^-23 of |a*b| and typically 2^-26 (an fp32 multiply-add rounds at 2^-24); the
+// measured error of whole convs against fp64 is no larger than that of the fp32 instruction.
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef __bf16 mie_bf16x2 __attribute__((ext_vector_type(2)));
+// two values at a time: one packed conversion per term, the bf16 pair widened again with a shift and a mask
+__device__ __forceinline__ void split3_pair(float f0, float f1, float& p0, float& p1, float& p2) {
+  const v2f v = {f0, f1};
+  const mie_bf16x2 hi = __builtin_convertvector(v, mie_bf16x2);
+  const unsigned uh = __builtin_bit_cast(unsigned, hi);
+  const v2f r1 = {f0 - __builtin_bit_cast(float, uh << 16), f1 - __builtin_bit_cast(float, uh & 0xffff0000u)};
+  const mie_bf16x2 mid = __builtin_convertvector(r1, mie_bf16x2);
+  const unsigned um = __builtin_bit_cast(unsigned, mid);
+  const v2f r2 = {r1[0] - __builtin_bit_cast(float, um << 16), r1[1] - __builtin_bit_cast(float, um & 0xffff0000u)};
+  const mie_bf16x2 lo = __builtin_convertvector(r2, mie_bf16x2);
+  p0 = __builtin_bit_cast(float, hi);
+  p1 = __builtin_bit_cast(float, mid);
+  p2 = __builtin_bit_cast(float, lo);
+}
 __device__ __forceinline__ void split3(const float (&f)[8], float4 (&pl)[3]) {
-  mie_bf16x8 b0, b1, b2;
-#pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const mie_bf16 hi = (mie_bf16)f[e];
-    const float r1 = f[e] - (float)hi;
-    const mie_bf16 mid = (mie_bf16)r1;
-    const float r2 = r1 - (float)mid;
-    b0[e] = hi; b1[e] = mid; b2[e] = (mie_bf16)r2;
-  }
-  const v4f r0 = __builtin_bit_cast(v4f, b0), r1 = __builtin_bit_cast(v4f, b1), r2 = __builtin_bit_cast(v4f, b2);
-  pl[0] = make_float4(r0[0], r0[1], r0[2], r0[3]);
-  pl[1] = make_float4(r1[0], r1[1], r1[2], r1[3]);
-  pl[2] = make_float4(r2[0], r2[1], r2[2], r2[3]);
+  split3_pair(f[0], f[1], pl[0].x, pl[1].x, pl[2].x);
+  split3_pair(f[2], f[3], pl[0].y, pl[1].y, pl[2].y);
+  split3_pair(f[4], f[5], pl[0].z, pl[1].z, pl[2].z);
+  split3_pair(f[6], f[7], pl[0].w, pl[1].w, pl[2].w);
 }
 // One unit (16 input channels of a tap) of the X3 contraction for the two pixel blocks of a tile: six bf16 MFMAs
-// per block, smallest terms first, the two accumulators interleaved.
-__device__ __forceinline__ void mma_unit2_x3(v16f& acc0, v16f& acc1, const float4 (&a0)[3], const float4 (&a1)[3],
-                                             const float4 (&b)[3]) {
-  mma_unit(acc0, a0[2], b[0], mie_bf16()); mma_unit(acc1, a1[2], b[0], mie_bf16());
-  mma_unit(acc0, a0[1], b[1], mie_bf16()); mma_unit(acc1, a1[1], b[1], mie_bf16());
-  mma_unit(acc0, a0[0], b[2], mie_bf16()); mma_unit(acc1, a1[0], b[2], mie_bf16());
-  mma_unit(acc0, a0[1], b[0], mie_bf16()); mma_unit(acc1, a1[1], b[0], mie_bf16());
-  mma_unit(acc0, a0[0], b[1], mie_bf16()); mma_unit(acc1, a1[0], b[1], mie_bf16());
+// per block.  The three large products (hi*hi, mid*hi, hi*mid) and the three small ones (lo*hi, mid*mid, hi*lo, 2^-16 of
+// the first) go to accumulators of their own, added in the epilogue: four independent chains, so that no MFMA
+// waits for the one issued just before it, and the small terms are summed among themselves.
+__device__ __forceinline__ void mma_unit2_x3(v16f& acc0, v16f& acc1, v16f& sm0, v16f& sm1, const float4 (&a0)[3],
+                                             const float4 (&a1)[3], const float4 (&b)[3]) {
   mma_unit(acc0, a0[0], b[0], mie_bf16()); mma_unit(acc1, a1[0], b[0], mie_bf16());
+  mma_unit(sm0, a0[2], b[0], mie_bf16());  mma_unit(sm1, a1[2], b[0], mie_bf16());
+  mma_unit(acc0, a0[1], b[0], mie_bf16()); mma_unit(acc1, a1[1], b[0], mie_bf16());
+  mma_unit(sm0, a0[1], b[1], mie_bf16());  mma_unit(sm1, a1[1], b[1], mie_bf16());
+  mma_unit(acc0, a0[0], b[1], mie_bf16()); mma_unit(acc1, a1[0], b[1], mie_bf16());
+  mma_unit(sm0, a0[0], b[2], mie_bf16());  mma_unit(sm1, a1[0], b[2], mie_bf16());
 }
 
 // One 16-byte slot of delta elements <-> fp32 values (4 of them, or 8 for bf16).
@@ -361,7 +371,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   // (bf16: a workgroup's contraction is too short to be worth the registers that hold these values
   // through it -- they cost a resident workgroup per CU -- so they are fetched after it instead; the same
   // holds for the 128-column slabs, whose threads own 8 groups.)
-  constexpr bool EARLY = sizeof(T) == 4 && WK > 1;
+  constexpr bool EARLY = sizeof(T) == 4 && WK > 1 && !(X3 && K == 5);
   auto epilogue_fetch = [&]() {
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
@@ -377,12 +387,16 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   if (!GATES && EARLY && !SPLIT) epilogue_fetch();
 
   v16f acc[2][NB];
+  v16f accs[X3 ? 2 : 1][X3 ? NB : 1];      // X3: the small term products
 #pragma unroll
   for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[mb][nb][r] = 0.f;
+      for (int r = 0; r < 16; ++r) {
+        acc[mb][nb][r] = 0.f;
+        if (X3) accs[mb][nb][r] = 0.f;
+      }
 
   // ---- per-thread staging plan: which pixels / float4 slots this thread copies -------------
   const int iy0 = y0 * S - a.pad, ix0 = x0 * S - a.pad;
@@ -439,6 +453,31 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   // masked pixels are zeroed when the bytes have arrived; from the second chunk on -- and in layers of fewer
   // chunks, where that would be a large share of the reads -- a masked pixel is not fetched at all.
   float4 st_reg[NLD][GPS];
+  auto load_slots = [&](float4 (&regs)[NLD][GPS], int c, bool first) {
+    const bool second = c >= nch1;
+    const T* xin = second ? a.x2 : a.x;
+    const int cs = second ? a.c2 : a.c1;
+    const int ci0 = (second ? c - nch1 : c) * CC;
+    const unsigned ok = first ? inb : (second ? ok2 : ok1);
+    // The loads are unconditional in control flow (a branch around a load makes the compiler's
+    // wait counters conservative: the first MFMAs of a chunk would then wait for the whole
+    // global-memory latency of these loads).  Lanes whose pixel is masked or outside the image
+    // all read one fixed, cache-resident address instead and get zeros selected afterwards,
+    // so inactive pixels still cost no HBM traffic.
+    const T* dummy = a.filt_mc;
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+      const bool okb = (ok >> i) & 1u;
+      const T* p = xin + (long long)st_po[i] * cs + ci0 + st_c4[i];
+      p = okb ? p : dummy;
+#pragma unroll
+      for (int g = 0; g < GPS; ++g) {
+        float4 v = *reinterpret_cast<const float4*>(p + 4 * g);
+        v.x = okb ? v.x : 0.f; v.y = okb ? v.y : 0.f; v.z = okb ? v.z : 0.f; v.w = okb ? v.w : 0.f;
+        regs[i][g] = v;
+      }
+    }
+  };
   auto stage_load = [&](int c, bool first = false) {
     if constexpr (UP) {
       const T* dummy = a.filt_mc;
@@ -460,29 +499,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
       }
       return;
     }
-    const bool second = c >= nch1;
-    const T* xin = second ? a.x2 : a.x;
-    const int cs = second ? a.c2 : a.c1;
-    const int ci0 = (second ? c - nch1 : c) * CC;
-    const unsigned ok = first ? inb : (second ? ok2 : ok1);
-    // The loads are unconditional in control flow (a branch around a load makes the compiler's
-    // wait counters conservative: the first MFMAs of a chunk would then wait for the whole
-    // global-memory latency of these loads).  Lanes whose pixel is masked or outside the image
-    // all read one fixed, cache-resident address instead and get zeros selected afterwards,
-    // so inactive pixels still cost no HBM traffic.
-    const T* dummy = a.filt_mc;
-#pragma unroll
-    for (int i = 0; i < NLD; ++i) {
-      const bool okb = (ok >> i) & 1u;
-      const T* p = xin + (long long)st_po[i] * cs + ci0 + st_c4[i];
-      p = okb ? p : dummy;
-#pragma unroll
-      for (int g = 0; g < GPS; ++g) {
-        float4 v = *reinterpret_cast<const float4*>(p + 4 * g);
-        v.x = okb ? v.x : 0.f; v.y = okb ? v.y : 0.f; v.z = okb ? v.z : 0.f; v.w = okb ? v.w : 0.f;
-        st_reg[i][g] = v;
-      }
-    }
+    load_slots(st_reg, c, first);
   };
   // one staged slot to LDS: as it is, or (X3) its eight fp32 values as three bf16 planes
   auto store_slot = [&](TL* dst, const float4 (&raw)[GPS]) {
@@ -495,6 +512,12 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
     } else {
       *reinterpret_cast<float4*>(dst) = raw[0];
     }
+  };
+  auto store_slots = [&](const float4 (&regs)[NLD][GPS], int buf) {
+    TL* dst = sbuf + buf * (PL * STAGE);
+#pragma unroll
+    for (int i = 0; i < NLD; ++i)
+      if (tid + 256 * i < NSLOT) store_slot(dst + st_lds[i], regs[i]);
   };
   auto stage_store = [&](int buf) {
     TL* dst = sbuf + buf * (PL * STAGE);
@@ -528,7 +551,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
       // (two workgroups per CU either way) and run 1.5 % faster for it; in the bf16 kernels they cost
       // one or two resident workgroups, so there an opaque zero makes them a per-chunk computation.
       int opaque = 0;
-      if (sizeof(T) == 2) asm volatile("" : "+v"(opaque));
+      if (sizeof(T) == 2 || X3) asm volatile("" : "+v"(opaque));
 #pragma unroll
       for (int i = 0; i < NLD; ++i) {
         const int slot = tid + 256 * i + opaque;
@@ -570,9 +593,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
       }
       return;
     }
-#pragma unroll
-    for (int i = 0; i < NLD; ++i)
-      if (tid + 256 * i < NSLOT) store_slot(dst + st_lds[i], st_reg[i]);
+    store_slots(st_reg, buf);
   };
 
   // ---- operand addressing ------------------------------------------------------------------------
@@ -703,7 +724,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
     if (TPAR && (unit * TP >= K * K || unit_tap(unit) >= K * K)) return;     // uniform over the wave
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
-      if constexpr (X3) mma_unit2_x3(acc[0][nb], acc[1][nb], av[0], av[1], bv[nb]);
+      if constexpr (X3) mma_unit2_x3(acc[0][nb], acc[1][nb], accs[0][nb], accs[1][nb], av[0], av[1], bv[nb]);
       else mma_unit2(acc[0][nb], acc[1][nb], av[0][0], av[1][0], bv[nb][0], T());
     }
   };
@@ -740,7 +761,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
         else mma(i, av[i & 1], bring[i % RING]);
         __builtin_amdgcn_sched_barrier(0);
         if (i == 0) {
-          int cn = more ? c + 1 : c;      // after the last chunk: redundant re-load, never stored
+          int cn = __builtin_amdgcn_readfirstlane(more ? c + 1 : c);      // after the last chunk: redundant re-load, never stored
           asm volatile("" : "+s"(cn));
           ub_next = chunk_b(cn);
           stage_load(cn);
@@ -799,6 +820,14 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   // ---- epilogue -----------------------------------------------------------------------------------
   // acc[mb][nb][r] of this lane is output pixel p = 32*mb + 8*(r/4) + 4*half + r%4,
   // channel column wn*32*NB + 32*nb + lane%32 of the workgroup's slab.
+  if constexpr (X3) {
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[mb][nb][r] += accs[mb][nb][r];
+  }
   if constexpr (GATES) {
     // ConvLSTM gate chain as the epilogue.  The filter columns are interleaved by gate: column 4*hc + g is
     // gate g (in, remember, out, cell) of hidden channel hc, so a workgroup owns all four gates of its
