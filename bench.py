@@ -70,6 +70,11 @@ def parse_args():
                     help="skip the other benchmark configurations (single conv, activation chain, EVFlowNet-incr, batched bf16)")
     ap.add_argument("--no-lossy", dest="lossy", action="store_false", help="skip the lossy frontier")
     ap.add_argument("--no-refresh", dest="refresh", action="store_false", help="skip the dense-refresh timing")
+    ap.add_argument("--f32-matmul", choices=["bf16x3", "native"], default=None,
+                    help="how the matrix-core kernels multiply fp32 deltas (default: the library setting, bf16x3 = "
+                         "three bf16 terms per value on the bf16 instruction, fp32 accuracy)")
+    ap.add_argument("--no-native", dest="native", action="store_false",
+                    help="skip the comparison run with the fp32 matrix-core instruction")
     return ap.parse_args()
 
 
@@ -422,7 +427,17 @@ class NetBench:
         dom = dict(dom, us=round(dom_us, 2), gbs=round(dom["bytes"] / dom_us / 1e3, 1),
                    tflops=round(dom["flops"] / dom_us / 1e6, 2))
         mfma_bound = dom["flops"] / max(dom["bytes"], 1) > self.peak_mfma * 1e12 / (PEAK_HBM_GBS * 1e9)
-        if mfma_bound:
+        x3 = self.wl.dtype == "f32" and self._takes_x3(dom)
+        if mfma_bound and x3:
+            # fp32 deltas multiplied as three bf16 terms: six bf16 matrix-core products per algorithmic multiply, so
+            # the bound is the bf16 peak over six; the fraction of the fp32 instruction's peak is given beside it
+            peak = round(PEAK_BF16_MFMA_TFLOPS / 6.0, 1)
+            roofline = dict(bound="mfma", achieved=dom["tflops"], peak=peak, unit="TFLOP/s",
+                            frac=round(dom["tflops"] / peak, 4), traffic=None,
+                            peak_basis="bf16 matrix-core peak %.0f TFLOP/s / 6 term products per fp32 multiply" % PEAK_BF16_MFMA_TFLOPS,
+                            executed_bf16_tflops=round(6 * dom["tflops"], 1),
+                            frac_of_fp32_mfma_peak=round(dom["tflops"] / PEAK_FP32_MFMA_TFLOPS, 4))
+        elif mfma_bound:
             roofline = dict(bound="mfma", achieved=dom["tflops"], peak=self.peak_mfma, unit="TFLOP/s",
                             frac=round(dom["tflops"] / self.peak_mfma, 4), traffic=None)
         else:
@@ -440,6 +455,16 @@ class NetBench:
         except OSError:
             pass
         return roofline
+
+    def _takes_x3(self, layer):
+        """Whether the launch of a per-launch table row ran in the three-term bf16 form (its shape string is
+        "KxK sS CIN->COUT..." with the input channels of the first operand)."""
+        import re
+        m = re.search(r"(\d)x\d s(\d) (\d+)->(\d+)", layer["shape"])
+        if m is None:
+            return False
+        k, s_, cin, cout = (int(g) for g in m.groups())
+        return self.ops.f32x3_takes(k, s_, cin, 0, cout)
 
     def refresh_timing(self, model, reps=30):
         """The dense refresh (every 20-100 frames in the reference's drivers): eager and replayed from a graph."""
@@ -623,6 +648,8 @@ def main():
     _lib.lib()   # fail loudly if the HIP library is missing
     if args.upconv_all:
         ops.upconv_max_tiles = ops.upconv_max_chunks = 1 << 30
+    if args.f32_matmul is not None:
+        ops.f32_matmul = args.f32_matmul
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
@@ -645,6 +672,18 @@ def main():
         log("  %-22s %-34s %9.2f us %8s GB/s %7s TFLOP/s  tiles %s/%s" % (
             l["op"], l["shape"], l["us"], l["gbs"], l["tflops"], l["active_tiles"], l["tiles"]))
     log("  sum of kernels %.1f us; algorithmic %.1f MB, %.2f GFLOP per frame" % (tot_us, tot_bytes / 1e6, tot_flops / 1e9))
+
+    # ---- the same network with the fp32 matrix-core instruction (v_mfma_f32_32x32x2_f32) ------------------
+    native = None
+    if args.native and args.dtype == "f32" and ops.f32_matmul == "bf16x3":
+        ops.f32_matmul = "native"
+        try:
+            nat_model = nb.new_model(async_masks=not args.sync_masks, plan_first=args.plan_first)
+            nat_sec, _, _ = nb.timed_run(nat_model, "incremental, fp32 matrix-core instruction", repeats=max(3, args.repeats // 2))
+            del nat_model
+        finally:
+            ops.f32_matmul = "bf16x3"
+        native = dict(ms_per_step=round(1e3 * nat_sec, 4), frames_per_s=round(NB / nat_sec, 1))
 
     # ---- dense comparator: same kernels, every tile active ---------------------------------------
     dense_sec = None
@@ -730,6 +769,7 @@ def main():
                                "active pixels, 1 dense refresh then incremental steps" % (NET_NAME, NB, BINS, H, W, 100 * dens),
                    "density": dens, "height": H, "width": W, "batch": NB, "graph": not args.no_graph,
                    "timing": "median of %d repeats of %d steps" % (args.repeats, args.steps),
+                   "f32_matmul": ops.f32_matmul if args.dtype == "f32" else None,
                    "mask_planning": "inline" if args.sync_masks else ("second stream, builds first" if args.plan_first else "second stream")},
         "roofline": roofline,
         "cpu_baseline": cpu,
@@ -740,6 +780,7 @@ def main():
         "algorithmic_gflop_per_frame": round(tot_flops / 1e9, 3),
         "mfma_frac_whole_frame": round(tot_flops / sec_per_step / 1e12 / nb.peak_mfma, 4),
         "sum_kernel_us": round(tot_us, 1),
+        "f32_native_mfma": native,
         "dense_same_kernels_ms": None if dense_sec is None else round(1e3 * dense_sec, 4),
         "speedup_vs_dense": None if dense_sec is None else round(dense_sec / sec_per_step, 3),
         "density_sweep": sweep,

@@ -16,6 +16,12 @@ LIB_PATH = os.path.join(LIB_DIR, "libmie_hip.so")
 SOURCES = ["mie_mask.hip", "mie_pointwise.hip", "mie_conv.hip", "mie_conv_mfma_f32.hip",
            "mie_conv_mfma_bf16.hip", "mie_conv_fewcin.hip", "mie_events.hip", "mie_tail.hip", "mie_refresh.hip", "mie_tconv_mfma.hip"]
 
+# Per-source additions.  The fp32 matrix-core kernels unroll their unit loops completely (up to 196 positions);
+# without the higher threshold the compiler gives up on the longest ones (the 128-column 5x5 / 7x7 kernels), their
+# operand ring is then indexed at run time and ends up in scratch memory (measured: 5.7 instead of 2.0 ms on the
+# 8x120x160 5x5 conv).  The other sources are faster with the default.
+EXTRA_FLAGS = {"mie_conv_mfma_f32.hip": ["-mllvm", "-pragma-unroll-threshold=65536"]}
+
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     "-fvisibility=hidden", "-fno-gpu-rdc",
@@ -63,7 +69,7 @@ def build_library(verbose=True, incremental=False):
         src = os.path.join(CSRC, s)
         fresh = (incremental and os.path.exists(obj)
                  and os.path.getmtime(obj) > max(os.path.getmtime(src), newest_header))
-        jobs.append(([hipcc] + compile_flags + ["-c", src, "-o", obj], obj, fresh))
+        jobs.append(([hipcc] + compile_flags + EXTRA_FLAGS.get(s, []) + ["-c", src, "-o", obj], obj, fresh))
     with ThreadPoolExecutor(max_workers=min(len(jobs), 8)) as pool:
         list(pool.map(lambda j: None if j[2] else _run(j[0], verbose), jobs))
     tmp = LIB_PATH + ".tmp"

@@ -233,6 +233,9 @@ __device__ __forceinline__ float4 f32_to_slot(const float (&f)[8], mie_bf16) {
 // of the 32-column slab kernels (WK = 4) is over (sub-chunk, tap parity).  Global loads, masks, epilogue: fp32.
 template <typename T, int K, int S, int WN, int NB, bool HALF, bool GATES = false, bool UP = false, bool SPLIT = false,
           bool X3 = false>
+// (Build with -mllvm -pragma-unroll-threshold=65536: the unit loop of the 128-column 5x5 / 7x7 kernels is 100 / 196
+// positions long, and where the compiler refuses to unroll it the operand ring is indexed at run time and lands in
+// scratch memory -- a factor of three in time.)
 __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   static_assert(!X3 || (sizeof(T) == 4 && S == 1 && !HALF && (K == 3 || K == 5)), "X3: fp32 deltas, 3x3 / 5x5, stride 1");
   using TL = std::conditional_t<X3, mie_bf16, T>;            // element type in LDS and on the matrix cores
@@ -364,27 +367,29 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   // fp32 kernels the reservoir / addend values are fetched right away and have the whole contraction to arrive.
   constexpr int QPP = CO_BLK / 4;                            // groups of four channels per pixel
   constexpr int PER = GATES ? 1 : 64 * QPP / 256;            // groups per thread
-  long long e_off[PER];
-  int e_co[PER];
-  bool e_ok[PER];
-  float4 e_r0[PER], e_add[PER];
+  constexpr int PB = PER > 4 ? 4 : PER;                      // groups per pass of the epilogue (registers)
+  long long e_off[PB];
+  int e_co[PB];
+  bool e_ok[PB];
+  float4 e_r0[PB], e_add[PB];
   // (bf16: a workgroup's contraction is too short to be worth the registers that hold these values
   // through it -- they cost a resident workgroup per CU -- so they are fetched after it instead; the same
   // holds for the 128-column slabs, whose threads own 8 groups.)
   constexpr bool EARLY = sizeof(T) == 4 && WK > 1 && !(X3 && K == 5);
-  auto epilogue_fetch = [&]() {
+  static_assert(!EARLY || PER == PB, "the early fetch covers a thread's whole share");
+  auto epilogue_fetch = [&](int h0) {
 #pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int idx = tid + 256 * i;
+    for (int i = 0; i < PB; ++i) {
+      const int idx = tid + 256 * (h0 + i);
       const int p = idx / QPP, col = 4 * (idx - p * QPP);
       const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
       e_ok[i] = oy < hout && ox < wout;
       e_off[i] = (((long long)n * hout + oy) * wout + ox) * a.cout + co0 + col;
       e_co[i] = co0 + col;
     }
-    if (!SPLIT) conv_epilogue_load4<T, PER>(a, e_off, e_ok, e_r0, e_add);
+    if (!SPLIT) conv_epilogue_load4<T, PB>(a, e_off, e_ok, e_r0, e_add);
   };
-  if (!GATES && EARLY && !SPLIT) epilogue_fetch();
+  if (!GATES && EARLY && !SPLIT) epilogue_fetch(0);
 
   v16f acc[2][NB];
   v16f accs[X3 ? 2 : 1][X3 ? NB : 1];      // X3: the small term products
@@ -899,7 +904,6 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
     }
   } else {
     // the last barrier of the main loop has retired every read of the staging buffers that is used
-    if (!EARLY || SPLIT) epilogue_fetch();
     float* red = smem + wk * (64 * CO_BLK);
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb)
@@ -911,25 +915,29 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
           red[p * CO_BLK + wn * (32 * NB) + nb * 32 + l32] = acc[mb][nb][r];
       }
     __syncthreads();
-    float4 v[PER];
 #pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int idx = tid + 256 * i;             // group idx: pixel idx / QPP, channels 4 * (idx % QPP) ...
-      float4 sum = *reinterpret_cast<const float4*>(&smem[4 * idx]);
+    for (int h0 = 0; h0 < PER; h0 += PB) {       // the 128-column slabs in two passes of four groups per thread
+      if (!EARLY || SPLIT) epilogue_fetch(h0);
+      float4 v[PB];
 #pragma unroll
-      for (int k2 = 1; k2 < WK; ++k2) {
-        const float4 part = *reinterpret_cast<const float4*>(&smem[k2 * (64 * CO_BLK) + 4 * idx]);
-        sum.x += part.x; sum.y += part.y; sum.z += part.z; sum.w += part.w;
+      for (int i = 0; i < PB; ++i) {
+        const int idx = tid + 256 * (h0 + i);      // group idx: pixel idx / QPP, channels 4 * (idx % QPP) ...
+        float4 sum = *reinterpret_cast<const float4*>(&smem[4 * idx]);
+#pragma unroll
+        for (int k2 = 1; k2 < WK; ++k2) {
+          const float4 part = *reinterpret_cast<const float4*>(&smem[k2 * (64 * CO_BLK) + 4 * idx]);
+          sum.x += part.x; sum.y += part.y; sum.z += part.z; sum.w += part.w;
+        }
+        v[i] = sum;
       }
-      v[i] = sum;
-    }
-    if constexpr (SPLIT) {
-      float* plane = a.ws + (long long)bz * a.ws_plane;
+      if constexpr (SPLIT) {
+        float* plane = a.ws + (long long)bz * a.ws_plane;
 #pragma unroll
-      for (int i = 0; i < PER; ++i)
-        if (e_ok[i]) *reinterpret_cast<float4*>(plane + e_off[i]) = v[i];
-    } else {
-      conv_epilogue_store4<T, PER>(a, e_off, e_co, e_ok, v, e_r0, e_add);
+        for (int i = 0; i < PB; ++i)
+          if (e_ok[i]) *reinterpret_cast<float4*>(plane + e_off[i]) = v[i];
+      } else {
+        conv_epilogue_store4<T, PB>(a, e_off, e_co, e_ok, v, e_r0, e_add);
+      }
     }
   }
   MIE_STAMP(14);

@@ -32,3 +32,19 @@ def pytest_collection_modifyitems(config, items):
 def mie_lib():
     from maskedincrementeval_amd import _lib
     return _lib.lib()
+
+
+@pytest.fixture(autouse=True)
+def _f32_matmul_mode(request):
+    """Tests parametrized over `f32mode` run with ops.f32_matmul set to it: "bf16x3" (fp32 deltas multiplied as three
+    bf16 terms on the bf16 matrix-core instruction, the default) or "native" (the fp32 instruction)."""
+    spec = getattr(request.node, "callspec", None)
+    mode = spec.params.get("f32mode") if spec is not None else None
+    if mode is None:
+        yield
+        return
+    from maskedincrementeval_amd import ops
+    old = ops.f32_matmul
+    ops.f32_matmul = mode
+    yield
+    ops.f32_matmul = old

@@ -73,7 +73,8 @@ def _mfma_takes(k, s, cin, cout):
 @pytest.mark.parametrize("pname,path", PATHS)
 @pytest.mark.parametrize("k,s,p", [(1, 1, 0), (3, 1, 1), (3, 2, 1), (5, 1, 2), (5, 2, 2), (7, 1, 3), (7, 2, 3)])
 @pytest.mark.parametrize("cin,cout", [(32, 32), (32, 64), (64, 128)])
-def test_conv_paths_match_oracle(pname, path, k, s, p, cin, cout):
+@pytest.mark.parametrize("f32mode", ["bf16x3", "native"])
+def test_conv_paths_match_oracle(pname, path, k, s, p, cin, cout, f32mode):
     if path == _lib.PATH_MFMA and not _mfma_takes(k, s, cin, cout):
         pytest.skip("shape not taken by the matrix-core path (falls to the VALU path)")
     n, h, w = 2, 37, 45      # ragged: not multiples of the 8x8 tile
@@ -122,7 +123,8 @@ def test_inactive_pixels_are_never_read_and_output_is_clean(pname, path):
 
 
 @pytest.mark.parametrize("pname,path", PATHS)
-def test_two_pointer_input_equals_concat(pname, path):
+@pytest.mark.parametrize("f32mode", ["bf16x3", "native"])
+def test_two_pointer_input_equals_concat(pname, path, f32mode):
     # ConvLSTM gates: conv over cat(x, h) without forming the concat (e2depth_incr.py:100-101)
     n, c1, c2, cout, h, w = 1, 32, 32, 128, 33, 44
     dx, mx = gaussian_delta(n, c1, h, w, 0.05, 0.3, seed=60)
@@ -140,7 +142,8 @@ def test_two_pointer_input_equals_concat(pname, path):
                                           (_lib.ACT_LEAKY_RELU, 0.01, io.leaky_relu),
                                           (_lib.ACT_SIGMOID, 0.0, torch.sigmoid),
                                           (_lib.ACT_TANH, 0.0, torch.tanh)])
-def test_fused_conv_activation_epilogue(pname, path, act, slope, op):
+@pytest.mark.parametrize("f32mode", ["bf16x3", "native"])
+def test_fused_conv_activation_epilogue(pname, path, act, slope, op, f32mode):
     n, cin, cout, h, w = 1, 32, 32, 40, 48
     conv = _Conv(n, cin, cout, h, w, 3, 1, 1, seed=8, path=path)
     r0 = torch.randn(n, cout, h, w, generator=torch.Generator().manual_seed(1))
@@ -287,7 +290,8 @@ def test_tconv2x_matrix_core_form(c1, c2, cout, h, w, k, dtype):
     assert torch.allclose(dense.float().cpu(), torch.relu(pre), **rt)
 
 
-def test_large_channel_mfma_bottleneck_shapes():
+@pytest.mark.parametrize("f32mode", ["bf16x3", "native"])
+def test_large_channel_mfma_bottleneck_shapes(f32mode):
     # 256 -> 256 3x3 at 33x44 (residual blocks) and 512 -> 1024 gates: K = 2304 / 4608 contractions
     n, h, w = 1, 33, 44
     for cin, cout in ((256, 256), (512, 1024)):
@@ -297,7 +301,8 @@ def test_large_channel_mfma_bottleneck_shapes():
 
 
 @pytest.mark.parametrize("pname,path", PATHS)
-def test_addend_rides_into_the_epilogue(pname, path):
+@pytest.mark.parametrize("f32mode", ["bf16x3", "native"])
+def test_addend_rides_into_the_epilogue(pname, path, f32mode):
     # residual block tail: relu2(conv2(d) + residual) with the residual delta as the conv's addend
     n, c, h, w = 1, 32, 40, 56
     conv = _Conv(n, c, c, h, w, 3, 1, 1, seed=10, path=path)
@@ -316,7 +321,8 @@ def test_addend_rides_into_the_epilogue(pname, path):
         _close(res_gpu, res_cpu.reservoir, "reservoir %d" % step)
 
 
-def test_refresh_conv_matches_dense_conv_with_bias():
+@pytest.mark.parametrize("f32mode", ["bf16x3", "native"])
+def test_refresh_conv_matches_dense_conv_with_bias(f32mode):
     n, cin, cout, h, w = 2, 32, 64, 37, 45
     g = torch.Generator().manual_seed(5)
     x, x2 = torch.randn(n, cin, h, w, generator=g), torch.randn(n, cin, h, w, generator=g)
@@ -355,7 +361,8 @@ def test_pack_filter_layout_and_row_views():
 # tiles), with and without the second input, plain and reservoir + activation epilogue.
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("c,cout,h,w", [(64, 32, 13, 17), (64, 64, 70, 90), (128, 128, 88, 80), (64, 96, 9, 40)])
-def test_upsampled_conv_in_one_kernel(c, cout, h, w, dtype):
+@pytest.mark.parametrize("f32mode", ["bf16x3", "native"])
+def test_upsampled_conv_in_one_kernel(c, cout, h, w, dtype, f32mode):
     bf = dtype == torch.bfloat16
     tol = (lambda ref: dict(rtol=BF16_RTOL, atol=bf16_atol(ref, 2.0))) if bf else (lambda ref: dict(rtol=RTOL, atol=ATOL))
     q = (lambda t: t.to(torch.bfloat16).float()) if bf else (lambda t: t)
@@ -473,7 +480,8 @@ def test_seeded_random_shapes(case, dtype):
 @pytest.mark.parametrize("c1,c2,cout,h,w,s", [(512, 0, 512, 16, 16, 1), (256, 0, 512, 32, 32, 2), (128, 0, 96, 13, 11, 1),
                                               (128, 64, 64, 20, 9, 1), (256, 128, 160, 8, 8, 1), (128, 0, 32, 31, 29, 2),
                                               (256, 0, 256, 32, 32, 1)])
-def test_small_planes_split_the_contraction(c1, c2, cout, h, w, s, dtype, k):
+@pytest.mark.parametrize("f32mode", ["bf16x3", "native"])
+def test_small_planes_split_the_contraction(c1, c2, cout, h, w, s, dtype, k, f32mode):
     bf = dtype == torch.bfloat16
     if bf and (c1 % 64 or c2 % 64 or (c1 + c2) // 64 < 4):
         pytest.skip("fewer than 4 staged chunks of 64 bf16 channels: not split")

@@ -173,7 +173,8 @@ def test_config2_activation_chain_50_steps(density):
 
 @pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("cin,hid", [(16, 16), (32, 32), (64, 32)])
-def test_convlstm_module_matches_oracle(fused, cin, hid):
+@pytest.mark.parametrize("f32mode", ["bf16x3", "native"])
+def test_convlstm_module_matches_oracle(fused, cin, hid, f32mode):
     # (32, 32) and (64, 32) take the conv + gate chain kernel when fused, (16, 16) the two-kernel form
     n, h, w = 1, 26, 34
     cell = ConvLSTMIncr(cin, hid, 3, fused=fused).to(DEV).eval()
@@ -295,7 +296,8 @@ def test_e2depth_refresh_runs_on_the_library_kernels_and_replays_as_a_graph():
 
 
 @pytest.mark.parametrize("fuse", [True, False])
-def test_e2depth_incr_small_matches_oracle(fuse):
+@pytest.mark.parametrize("f32mode", ["bf16x3", "native"])
+def test_e2depth_incr_small_matches_oracle(fuse, f32mode):
     _run_e2depth(72, 104, steps=4, density=0.05, fuse=fuse)
 
 

@@ -177,7 +177,8 @@ def test_bilinear_up2x_with_skip_sum(n, c, h, w):
 
 
 @pytest.mark.parametrize("hid,h,w,with_prev", [(64, 33, 44, False), (16, 19, 27, True), (3, 9, 9, True)])
-def test_fused_convlstm_gates_match_module_chain(hid, h, w, with_prev):
+@pytest.mark.parametrize("f32mode", ["bf16x3", "native"])
+def test_fused_convlstm_gates_match_module_chain(hid, h, w, with_prev, f32mode):
     """Gate chain of ConvLSTMIncr.forward (e2depth_incr.py:103-117) in one kernel vs the
     oracle's module-by-module chain; reservoirs are set up from a dense refresh."""
     n = 1
