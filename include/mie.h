@@ -169,8 +169,8 @@ int mie_pack_filter(const float* filter, int cin, int k, int cout, void* packed,
                     int dtype, void* stream);
 
 /*
- * 1 if the matrix-core conv takes this shape with dtype MIE_DTYPE_F32_BF16X3 (k = 3 or 5, stride 1,
- * c1, c2 and cout multiples of 32), else 0: such a call must then be made with MIE_DTYPE_F32 and the
+ * 1 if the matrix-core conv takes this shape with dtype MIE_DTYPE_F32_BF16X3 (k = 3 or 5 at stride 1 with
+ * c1, c2 multiples of 32, or k = 5 at stride 2 with multiples of 16; cout a multiple of 32), else 0: such a call must then be made with MIE_DTYPE_F32 and the
  * fp32 filter copy.  No counterpart in the reference (it has one arithmetic, cuDNN's or its own
  * kernel's fp32: ext/pointops/_C_ext/pointops/ext_conv.cu:74-76).
  */

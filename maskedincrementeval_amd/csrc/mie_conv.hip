@@ -382,8 +382,8 @@ int conv_impl(const char* who, const T* x, const uint8_t* xmask, int c1, const T
                           : ((filter_mc != nullptr) && (cin_total % pmul == 0) &&
                              mie_conv_mfma_takes(k, stride, dtype_of<T>(), c1, c2, cout));
   MIE_REQUIRE(!x3 || mfma_ok, MIE_ERR_UNSUPPORTED,
-              "%s: MIE_DTYPE_F32_BF16X3 needs filter_mc packed in that layout, k = 3 or 5, stride 1 and channel counts "
-              "that are multiples of 32 (k=%d stride=%d c1=%d c2=%d cout=%d); see mie_conv_f32x3_takes", who, k, stride,
+              "%s: MIE_DTYPE_F32_BF16X3 needs filter_mc packed in that layout, k = 3 or 5 and channel counts "
+              "in whole chunks (32, stride 2: 16; k=%d stride=%d c1=%d c2=%d cout=%d); see mie_conv_f32x3_takes", who, k, stride,
               c1, c2, cout);
   MIE_REQUIRE(path == MIE_PATH_AUTO || path == MIE_PATH_VALU || path == MIE_PATH_MFMA,
               MIE_ERR_INVALID_ARG, "%s: unknown path %d", who, path);

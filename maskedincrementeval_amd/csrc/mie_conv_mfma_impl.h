@@ -229,24 +229,25 @@ __device__ __forceinline__ float4 f32_to_slot(const float (&f)[8], mie_bf16) {
 // input value and every filter value is split into three bf16 terms (split3; the filter once, by
 // mie_pack_filter); the staged tile is three bf16 planes in LDS, a unit is 16 input channels of a tap, and
 // its six significant term products are six v_mfma_f32_32x32x16_bf16 per pixel block -- 6 x 32 cycles for what
-// eight v_mfma_f32_32x32x2_f32 take 8 x 64 cycles to do.  Chunks of 32 channels (two units per tap); the k-split
-// of the 32-column slab kernels (WK = 4) is over (sub-chunk, tap parity).  Global loads, masks, epilogue: fp32.
+// eight v_mfma_f32_32x32x2_f32 take 8 x 64 cycles to do.  Chunks of 32 channels (two units per tap; stride 2, whose
+// staged tile is four times the size: 16 channels, one unit per tap); where the k-split has more waves than a tap
+// has units it is over (sub-chunk, tap class).  Global loads, masks, epilogue: fp32.
 template <typename T, int K, int S, int WN, int NB, bool HALF, bool GATES = false, bool UP = false, bool SPLIT = false,
           bool X3 = false>
 // (Build with -mllvm -pragma-unroll-threshold=65536: the unit loop of the 128-column 5x5 / 7x7 kernels is 100 / 196
 // positions long, and where the compiler refuses to unroll it the operand ring is indexed at run time and lands in
 // scratch memory -- a factor of three in time.)
 __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
-  static_assert(!X3 || (sizeof(T) == 4 && S == 1 && !HALF && (K == 3 || K == 5)), "X3: fp32 deltas, 3x3 / 5x5, stride 1");
+  static_assert(!X3 || (sizeof(T) == 4 && !HALF && (K == 3 || K == 5)), "X3: fp32 deltas, 3x3 / 5x5");
   using TL = std::conditional_t<X3, mie_bf16, T>;            // element type in LDS and on the matrix cores
   constexpr int PL = X3 ? 3 : 1;                             // operand planes (terms per value)
   constexpr int GPS = X3 ? 2 : 1;                            // 16-byte global loads per staging slot
-  constexpr int NBUF = X3 ? (K == 3 ? 2 : 1) : stage_buffers(S, (int)sizeof(T));
+  constexpr int NBUF = X3 ? ((K == 3 && S == 1) ? 2 : 1) : stage_buffers(S, (int)sizeof(T));
   constexpr int EPS = 16 / (int)sizeof(TL);                  // elements per 16-byte slot (4 / 8)
   constexpr int SUB = 2 * EPS;                               // channels per unit (8 / 16)
   constexpr int WK = 4 / WN;
   constexpr int IT = 7 * S + K;                              // input tile edge incl. halo
-  constexpr int CC = X3 ? 32 : stage_channels(K, S, HALF) * (4 / (int)sizeof(T));   // channels per LDS stage
+  constexpr int CC = X3 ? (S == 2 ? 16 : 32) : stage_channels(K, S, HALF) * (4 / (int)sizeof(T));   // channels per LDS stage
   constexpr int LS = CC + EPS;                               // LDS elements per staged pixel
   constexpr int NPIX = IT * IT;
   constexpr int Q4 = CC / EPS;                               // 16-byte slots per pixel
@@ -1092,23 +1093,25 @@ inline int pick_slab_x3(int cout, unsigned cap) {
   return 0;
 }
 inline bool x3_takes(int k, int s, int c1, int c2, int cout) {
+  // (3x3 stride 2 was measured too: no faster than the fp32 instruction, 15-29 us either way, and it has a split form)
+  if (s == 2) return k == 5 && c1 % 16 == 0 && c2 % 16 == 0 && cout % 32 == 0;
   return (k == 3 || k == 5) && s == 1 && c1 % 32 == 0 && c2 % 32 == 0 && cout % 32 == 0;
 }
 
-template <int K, bool GATES, bool UP>
+template <int K, bool GATES, bool UP, int S = 1>
 bool launch_x3(const ConvArgsT<float>& a0, unsigned cap, hipStream_t st) {
   ConvArgsT<float> a = a0;
   const int cout = a.cout;
-  if (!x3_takes(K, 1, a.c1, UP ? 0 : a.c2, cout)) return false;
+  if (!x3_takes(K, S, a.c1, UP ? 0 : a.c2, cout)) return false;
   switch (pick_slab_x3(cout, cap)) {
     case 128:
-      hipLaunchKernelGGL((k_conv_mfma<float, K, 1, 4, 1, false, GATES, UP, false, true>), dim3(xcd_plan(a, cap, cout / 128, K, UP), cout / 128), dim3(256), 0, st, a);
+      hipLaunchKernelGGL((k_conv_mfma<float, K, S, 4, 1, false, GATES, UP, false, true>), dim3(xcd_plan(a, cap, cout / 128, K, UP), cout / 128), dim3(256), 0, st, a);
       return true;
     case 64:
-      hipLaunchKernelGGL((k_conv_mfma<float, K, 1, 2, 1, false, GATES, UP, false, true>), dim3(xcd_plan(a, cap, cout / 64, K, UP), cout / 64), dim3(256), 0, st, a);
+      hipLaunchKernelGGL((k_conv_mfma<float, K, S, 2, 1, false, GATES, UP, false, true>), dim3(xcd_plan(a, cap, cout / 64, K, UP), cout / 64), dim3(256), 0, st, a);
       return true;
     case 32:
-      hipLaunchKernelGGL((k_conv_mfma<float, K, 1, 1, 1, false, GATES, UP, false, true>), dim3(xcd_plan(a, cap, cout / 32, K, UP), cout / 32), dim3(256), 0, st, a);
+      hipLaunchKernelGGL((k_conv_mfma<float, K, S, 1, 1, false, GATES, UP, false, true>), dim3(xcd_plan(a, cap, cout / 32, K, UP), cout / 32), dim3(256), 0, st, a);
       return true;
     default:
       return false;
@@ -1213,9 +1216,9 @@ template <typename T>
 bool launch_any(const ConvArgsT<T>& a, int k, int s, unsigned cap, hipStream_t st) {
   if constexpr (sizeof(T) == 4) {
     if (a.x3) {
-      if (s != 1) return false;
-      if (k == 3) return launch_split<T, 3, 1>(a, cap, st) || launch_x3<3, false, false>(a, cap, st);
-      if (k == 5) return launch_split<T, 5, 1>(a, cap, st) || launch_x3<5, false, false>(a, cap, st);
+      if (k == 3 && s == 1) return launch_split<T, 3, 1>(a, cap, st) || launch_x3<3, false, false>(a, cap, st);
+      if (k == 5 && s == 1) return launch_split<T, 5, 1>(a, cap, st) || launch_x3<5, false, false>(a, cap, st);
+      if (k == 5 && s == 2) return launch_x3<5, false, false, 2>(a, cap, st);     // (no split form at stride 2)
       return false;
     }
   }

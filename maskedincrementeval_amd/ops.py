@@ -389,8 +389,12 @@ def conv_masked(x, xmask, x2, x2mask, filt, k, stride, pad, out_ts: TileMask, ou
     if x2 is not None and (x2.shape[0] != n or x2.shape[2:] != x.shape[2:]):
         raise ValueError("x2 shape %s incompatible with x %s" % (tuple(x2.shape), tuple(x.shape)))
     dt = x.dtype
-    filt, mc_ptr, code = _filter_args(filt, k, dt, (stride, c1, c2, filt.shape[3]) if path != _lib.PATH_VALU else None,
-                                      with_code=True)
+    # launches the library would split over the contraction (k = 3 or 5, few tiles: see launch_split); at stride 2
+    # only the fp32-instruction kernels have that form, and it is worth more there than the three-term arithmetic
+    small = k in (3, 5) and out_ts.capacity * (filt.shape[3] // 32) <= 128
+    want_split = small and split_enabled and workspace is not False
+    x3_shape = (stride, c1, c2, filt.shape[3]) if (path != _lib.PATH_VALU and not (stride == 2 and want_split)) else None
+    filt, mc_ptr, code = _filter_args(filt, k, dt, x3_shape, with_code=True)
     cin_total, cout = filt.shape[0], filt.shape[3]
     if tuple(out_delta.shape) != (n, cout, out_ts.h, out_ts.w) or out_ts.n != n:
         raise ValueError("out_delta shape %s, expected %s" % (tuple(out_delta.shape), (n, cout, out_ts.h, out_ts.w)))
@@ -400,9 +404,8 @@ def conv_masked(x, xmask, x2, x2mask, filt, k, stride, pad, out_ts: TileMask, ou
         raise ValueError("addend shape %s != output %s" % (tuple(addend.shape), tuple(out_delta.shape)))
     _ready(out_ts)
     if workspace is None:
-        # only launches the library would split get the buffer (k = 3 or 5, few tiles): see launch_split
-        small = k in (3, 5) and mc_ptr is not None and out_ts.capacity * (cout // 32) <= 128
-        workspace = split_workspace(x.device) if (split_enabled and small) else False
+        # only launches the library would split get the buffer
+        workspace = split_workspace(x.device) if (split_enabled and small and mc_ptr is not None) else False
     if workspace is False:
         ws_ptr, ws_bytes = None, 0
     else:

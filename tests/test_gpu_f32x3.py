@@ -81,7 +81,10 @@ def test_library_says_which_shapes_take_the_three_term_form():
     L = _lib.lib()
     assert L.mie_conv_f32x3_takes(3, 1, 64, 64, 256) == 1
     assert L.mie_conv_f32x3_takes(5, 1, 256, 0, 128) == 1
-    assert L.mie_conv_f32x3_takes(5, 2, 64, 0, 128) == 0          # stride 2: fp32 instruction
+    assert L.mie_conv_f32x3_takes(5, 2, 64, 0, 128) == 1
+    assert L.mie_conv_f32x3_takes(5, 2, 48, 16, 64) == 1          # stride 2: chunks of 16 channels
+    assert L.mie_conv_f32x3_takes(3, 2, 64, 0, 64) == 0           # 3x3 stride 2 stays on the fp32 instruction
+    assert L.mie_conv_f32x3_takes(7, 2, 64, 0, 64) == 0
     assert L.mie_conv_f32x3_takes(3, 1, 48, 0, 64) == 0           # 48 input channels: not whole chunks
     assert L.mie_conv_f32x3_takes(1, 1, 64, 0, 64) == 0
     old = ops.f32_matmul
@@ -114,11 +117,11 @@ def test_three_term_dtype_is_refused_where_it_has_no_kernel():
     assert call(_lib.PATH_AUTO, 1, 1, ts) == 0
     rc = call(_lib.PATH_VALU, 1, 1, ts)
     assert rc != 0 and "matrix-core" in _err()
-    ts2 = TileMask(n, 8, 8, DEV)
-    ops.build_mask_tiles(None, None, n, h, w, _lib.FOOT_CONV, k, 2, 1, ts2)
-    out2 = ops.new_nhwc(n, c, 8, 8, DEV)
-    rc = L.mie_conv_masked(ops.nhwc_ptr(x, "x"), None, c, None, None, 0, h, w, plain.data_ptr(), mc3.data_ptr(), c, k, 2, 1, c,
-                           ts2.ref, ops.nhwc_ptr(out2, "out"), None, None, _lib.ACT_NONE, 0.0, _lib.PATH_AUTO,
+    # a 1x1 conv has no three-term kernel
+    w1 = _filt(he_normal_conv_weight(c, c, 1, 2))
+    plain1, mc1 = w1.for_dtype(torch.float32, x3=True)
+    rc = L.mie_conv_masked(ops.nhwc_ptr(x, "x"), None, c, None, None, 0, h, w, plain1.data_ptr(), mc1.data_ptr(), c, 1, 1, 0, c,
+                           ts.ref, ops.nhwc_ptr(out, "out"), None, None, _lib.ACT_NONE, 0.0, _lib.PATH_AUTO,
                            _lib.DTYPE_F32_BF16X3, None)
     assert rc != 0 and "mie_conv_f32x3_takes" in _err()
     # the pointwise entry points know two delta types only
