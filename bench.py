@@ -451,7 +451,7 @@ class NetBench:
         # shape (FETCH_SIZE + WRITE_SIZE, scaled by the copy-kernel calibration)
         try:
             with open(os.path.join(ROOT, "profiles", "pmc_traffic.json")) as f:
-                roofline["traffic"] = json.load(f).get(dom["shape"], {}).get("hbm_bytes_per_launch")
+                roofline["traffic"] = json.load(f).get(dom["shape"] + (" bf16x3" if x3 else ""), {}).get("hbm_bytes_per_launch")
         except OSError:
             pass
         return roofline
