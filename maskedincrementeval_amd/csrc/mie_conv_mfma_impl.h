@@ -5,7 +5,9 @@
 // with v_mfma_f32_32x32x16_bf16 (fp32 accumulation, fp32 reservoirs).  The two element types share
 // one kernel: every operand access is a 16-byte access, which holds 4 fp32 or 8 bf16 channels, so
 // the bf16 kernel is the fp32 kernel with twice the channels per LDS stage, per unit and per load.
-// The text below gives the fp32 numbers.
+// The text below gives the fp32 numbers.  A third form, X3, multiplies fp32 deltas on the bf16 instruction at fp32
+// accuracy (three bf16 terms per value, six term products per multiply): it is described at the kernel template and
+// is what fp32 deltas take by default wherever it exists.
 //
 // Work decomposition.  One 256-thread workgroup (4 waves) computes one active
 // 8x8 output tile (M = 64 pixels) x CO_BLK output channels as an implicit GEMM
@@ -48,6 +50,10 @@
 // third resident workgroup per CU (registers cut to fit) and splitting the contraction of the decoder convs
 // over two or four workgroups were each built and measured: none moved a layer by more than 2 %, the last
 // three for the worse.  Launches of a few workgroups per CU stay quantised: ceil(workgroups / 256) rounds.
+// The X3 form does the same 3x3 chunk's work in 54 MFMAs of 32 cycles, 0.95 us, and takes 2.4 us for it: with one wave
+// per SIMD nothing overlaps that wave's own staging work (88 VALU instructions to split a chunk's values, address
+// arithmetic, waits -- the load counter is in order, so a filter prefetch behind the staging loads waits for them).
+// A three-chunk software pipeline with two staging register sets changed nothing (19.8 us either way) and was removed.
 #pragma once
 #include "mie_conv.h"
 #include <stdlib.h>
