@@ -1088,10 +1088,23 @@ unsigned xcd_plan(ConvArgsT<T>& a, unsigned cap, int nslabs, int k, bool up = fa
 
 // X3 kernels (fp32 deltas, a.x3 set, the filter copy in the three-term layout): 3x3 / 5x5, stride 1, input channels in
 // whole chunks of 32, output slabs of 128 / 64 / 32 columns by the same rule as above.
-inline int pick_slab_x3(int cout, unsigned cap) {
+// Stride 1 first looks for the widest slab that makes the launch one round of more than half a chip of workgroups
+// (129 .. 256): measured on MI355X, one workgroup per CU with twice the columns beats one and a half rounds of the
+// narrow ones (5x5 256->128 at 66x88: 198 workgroups of 64 columns 61-65 us, 396 of 32 columns 71-74 us; 3x3 gates conv
+// 256+256->1024 at 33x44: 240 of 128 columns 53 us, 480 of 64 columns 57 us); at stride 2, whose workgroups are short,
+// it does not (28 vs 29 us).
+inline int pick_slab_x3(int cout, unsigned cap, int s) {
   const bool ok128 = cout % 128 == 0, ok64 = cout % 64 == 0, ok32 = cout % 32 == 0;
   const int f = forced_slab();
   if ((f == 128 && ok128) || (f == 64 && ok64) || (f == 32 && ok32)) return f;
+  if (s == 1) {
+    const int widths[3] = {128, 64, 32};
+    const bool oks[3] = {ok128, ok64, ok32};
+    for (int i = 0; i < 3; ++i) {
+      const long long wgs = (long long)cap * (cout / widths[i]);
+      if (oks[i] && wgs > 128 && wgs <= 256) return widths[i];
+    }
+  }
   const long long want = 400;
   if (ok128 && ((long long)cap * (cout / 128) >= want || (!ok64 && !ok32))) return 128;
   if (ok64 && ((long long)cap * (cout / 64) >= want || !ok32)) return 64;
@@ -1109,7 +1122,7 @@ bool launch_x3(const ConvArgsT<float>& a0, unsigned cap, hipStream_t st) {
   ConvArgsT<float> a = a0;
   const int cout = a.cout;
   if (!x3_takes(K, S, a.c1, UP ? 0 : a.c2, cout)) return false;
-  switch (pick_slab_x3(cout, cap)) {
+  switch (pick_slab_x3(cout, cap, S)) {
     case 128:
       hipLaunchKernelGGL((k_conv_mfma<float, K, S, 4, 1, false, GATES, UP, false, true>), dim3(xcd_plan(a, cap, cout / 128, K, UP), cout / 128), dim3(256), 0, st, a);
       return true;
