@@ -38,19 +38,21 @@ class _Case:
         self.out = [ops.new_nhwc(n, cout, self.ho, self.wo, DEV), ops.new_nhwc(n, cout, self.ho, self.wo, DEV)]
         torch.cuda.synchronize()
 
-    def args(self, which):
-        plain, mc = self.filt.for_dtype(torch.float32)
+    def args(self, which, x3=False):
+        """x3: fp32 deltas multiplied as three bf16 terms (MIE_DTYPE_F32_BF16X3 and the filter copy packed for it)."""
+        plain, mc = self.filt.for_dtype(torch.float32, x3=x3)
         return [self.d.data_ptr(), self.m.data_ptr(), self.cin, None, None, 0, self.h, self.w,
                 plain.data_ptr(), mc.data_ptr(), self.cin, self.k, self.s, self.p, self.cout, self.ts.ref,
                 self.out[which].data_ptr(), None, self.res[which].data_ptr(), _lib.ACT_RELU, 0.0,
-                _lib.PATH_AUTO, _lib.DTYPE_F32]
+                _lib.PATH_AUTO, _lib.DTYPE_F32_BF16X3 if x3 else _lib.DTYPE_F32]
 
 
 def _stream():
     return torch.cuda.current_stream(torch.device(DEV)).cuda_stream
 
 
-def test_noalloc_matches_workspace_form_on_two_calls():
+@pytest.mark.parametrize("x3", [False, True], ids=["fp32_instruction", "three_bf16_terms"])
+def test_noalloc_matches_workspace_form_on_two_calls(x3):
     lib = _lib.lib()
     # 512 -> 256 on a 16x16 plane (4 tiles x 8 slabs, 16 chunks: split 8 ways), then a smaller 256 -> 128 conv
     # on an 8x24 plane (3 tiles x 4 slabs, 8 chunks): the second call finds the first call's partial sums
@@ -59,9 +61,9 @@ def test_noalloc_matches_workspace_form_on_two_calls():
     ws = torch.full((_lib.NOALLOC_WS_BYTES // 4,), float("nan"), dtype=torch.float32, device=DEV)
     torch.cuda.synchronize()
     for case in (big, small):
-        _lib.check(lib.mie_conv_masked_ws(*case.args(0), ws.data_ptr(), ws.numel() * 4, _stream()))
+        _lib.check(lib.mie_conv_masked_ws(*case.args(0, x3), ws.data_ptr(), ws.numel() * 4, _stream()))
         before = torch.cuda.memory_stats(DEV)["allocation.all.allocated"]
-        _lib.check(lib.mie_conv_masked_noalloc(*case.args(1), _stream()))
+        _lib.check(lib.mie_conv_masked_noalloc(*case.args(1, x3), _stream()))
         torch.cuda.synchronize()
         assert torch.cuda.memory_stats(DEV)["allocation.all.allocated"] == before
         assert torch.equal(case.out[0], case.out[1]), "delta differs from the workspace form"
