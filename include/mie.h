@@ -78,8 +78,9 @@ extern "C" {
  * weight is split into three bf16 terms (hi + mid + lo, all 24 significant bits) and the six term products
  * that matter are accumulated in fp32 -- what is dropped is below 2^-26 of |x*w| per product, a quarter of
  * the rounding step of an fp32 multiply-add.  Taken by mie_pack_filter and by the `dtype` of
- * mie_conv_masked / _ws / _noalloc, mie_conv_refresh, mie_upconv_masked and mie_conv_gates_masked, with
- * filter_mc packed for it; every buffer is what it is for MIE_DTYPE_F32.  Shapes: mie_conv_f32x3_takes. */
+ * mie_conv_masked / _ws / _noalloc, mie_conv_refresh, mie_upconv_masked, mie_conv_gates_masked (shapes:
+ * mie_conv_f32x3_takes) and mie_tconv2x_masked / mie_tconv2x_refresh (c1, c2 multiples of 64), with filter_mc
+ * packed for it; every buffer is what it is for MIE_DTYPE_F32. */
 #define MIE_DTYPE_F32_BF16X3 2
 
 /* frame kinds of mie_events_to_frame */
@@ -612,7 +613,7 @@ int mie_tconv_masked(const void* x, const uint8_t* xmask, int cin, int h_in,
  * sub-pixel phases of the output are four stride-1 contractions over disjoint
  * tap subsets of the same staged input, so no product is spent on inserted zeros.
  *   x / x2 : [n,h_in,w_in,c1] / [n,h_in,w_in,c2] deltas with their pixel masks
- *        (x2 optional); c1, c2 multiples of 32 (bf16: 64), cout of 32
+ *        (x2 optional); c1, c2 multiples of 32 (bf16 and MIE_DTYPE_F32_BF16X3: 64), cout of 32
  *   filter / filter_mc : [cin_total][k][k][cout] as in mie_tconv_masked and its
  *        matrix-core copy (mie_pack_filter, required); c1 + c2 <= cin_total
  *   out    : output tile set at (2*h_in, 2*w_in), built with MIE_FOOT_TCONV

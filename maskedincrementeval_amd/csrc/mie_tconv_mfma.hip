@@ -26,37 +26,46 @@ namespace {
 __host__ __device__ constexpr int tc_phase(int k, int pad) { return (((k - pad) % 2) + 2) % 2; }
 __host__ __device__ constexpr int tc_shift(int k, int pad) { return (tc_phase(k, pad) + pad - k) / 2; }   // numerator is even
 
-template <typename T, int K, int WN, bool SPLIT>
+// X3 (fp32 deltas): the three-term bf16 form of k_conv_mfma -- staged values and weights as hi + mid + lo in bf16, six
+// v_mfma_f32_32x32x16_bf16 products per multiply, fp32 accuracy; chunks of 64 channels (four units per tap, so that the
+// k-split stays over whole sub-chunks and every tap's phase is known at compile time), three bf16 planes in LDS,
+// single-buffered.  With the accumulators of four phases it needs 140-176 registers beside them: one workgroup per CU
+// (forcing two makes it spill and costs 1 % of the EVFlowNet frame; as it is the form gains 1-2 % there).
+template <typename T, int K, int WN, bool SPLIT, bool X3 = false>
 __global__ __launch_bounds__(256) void k_tconv_mfma(ConvArgsT<T> a, TileSetDev pts) {
+  static_assert(!X3 || sizeof(T) == 4, "X3: fp32 deltas");
+  using TL = std::conditional_t<X3, mie_bf16, T>;            // element type in LDS and on the matrix cores
+  constexpr int PL = X3 ? 3 : 1;                             // operand planes (terms per value)
+  constexpr int GPS = X3 ? 2 : 1;                            // 16-byte global loads per staging slot
   constexpr int PAD = K / 2;
   constexpr int LO = (K == 5) ? 1 : 0;                       // halo above / left of the block (shifts reach -LO .. +1)
-  constexpr int NBUF = stage_buffers(1, (int)sizeof(T));
-  constexpr int EPS = 16 / (int)sizeof(T);
+  constexpr int NBUF = X3 ? 1 : stage_buffers(1, (int)sizeof(T));
+  constexpr int EPS = 16 / (int)sizeof(TL);
   constexpr int SUB = 2 * EPS;
   constexpr int WK = 4 / WN;
   constexpr int IT = 8 + LO + 1;
-  constexpr int CC = stage_channels(K, 1) * (4 / (int)sizeof(T));
+  constexpr int CC = X3 ? 64 : stage_channels(K, 1) * (4 / (int)sizeof(T));
   constexpr int LS = CC + EPS;
   constexpr int NPIX = IT * IT;
   constexpr int Q4 = CC / EPS;
   constexpr int NSLOT = NPIX * Q4;
   constexpr int NLD = (NSLOT + 255) / 256;
-  constexpr int RP = row_pitch_dw(IT, LS * (int)sizeof(T) / 4, 1) * 4 / (int)sizeof(T);
-  constexpr int STAGE = IT * RP;
+  constexpr int RP = row_pitch_dw(IT, LS * (int)sizeof(TL) / 4, 1) * 4 / (int)sizeof(TL);
+  constexpr int STAGE = IT * RP;                             // elements per plane of a staging buffer
   constexpr int NQ = CC / SUB;
   static_assert(NQ % WK == 0, "the k-split is over whole sub-chunks");
   constexpr int NQW = NQ / WK;
   constexpr int UPC = K * K * NQW;
-  constexpr int RING = ring_size(UPC);
+  constexpr int RING = (X3 && ring_size(UPC) > 6) ? ring_size(UPC, 3) : ring_size(UPC);
   constexpr int PD = RING - 1;
   constexpr int CO_BLK = 32 * WN;
   constexpr int RED = WK * 64 * CO_BLK;                      // the accumulators of one phase, parked for the epilogue
-  constexpr int STAGE_F = NBUF * STAGE * (int)sizeof(T) / 4;
+  constexpr int STAGE_F = NBUF * PL * STAGE * (int)sizeof(TL) / 4;
   constexpr int SMEM = STAGE_F > RED ? STAGE_F : RED;
   static_assert(SMEM * 4 <= 65536, "LDS budget");
   static_assert(!SPLIT || WN == 1, "the split form is the 32-channel slab kernel");
   __shared__ __attribute__((aligned(16))) float smem[SMEM];
-  T* const sbuf = reinterpret_cast<T*>(smem);
+  TL* const sbuf = reinterpret_cast<TL*>(smem);
 
   int n, y0, x0;                                             // block origin in INPUT coordinates
   const int tk = mie_pick_tile(pts, blockIdx.x, n, y0, x0);
@@ -114,7 +123,7 @@ __global__ __launch_bounds__(256) void k_tconv_mfma(ConvArgsT<T> a, TileSetDev p
   const int nch1 = a.c1 / CC;
   const int nch = nch1 + (a.x2 != nullptr ? a.c2 / CC : 0);
 
-  float4 st_reg[NLD];
+  float4 st_reg[NLD][GPS];
   auto stage_load = [&](int c) {
     const bool second = c >= nch1;
     const T* xin = second ? a.x2 : a.x;
@@ -127,16 +136,30 @@ __global__ __launch_bounds__(256) void k_tconv_mfma(ConvArgsT<T> a, TileSetDev p
       const bool okb = (ok >> i) & 1u;
       const T* p = xin + (long long)st_po[i] * cs + ci0 + st_c4[i];
       p = okb ? p : dummy;
-      float4 v = *reinterpret_cast<const float4*>(p);
-      v.x = okb ? v.x : 0.f; v.y = okb ? v.y : 0.f; v.z = okb ? v.z : 0.f; v.w = okb ? v.w : 0.f;
-      st_reg[i] = v;
+#pragma unroll
+      for (int g = 0; g < GPS; ++g) {
+        float4 v = *reinterpret_cast<const float4*>(p + 4 * g);
+        v.x = okb ? v.x : 0.f; v.y = okb ? v.y : 0.f; v.z = okb ? v.z : 0.f; v.w = okb ? v.w : 0.f;
+        st_reg[i][g] = v;
+      }
     }
   };
   auto stage_store = [&](int buf) {
-    T* dst = sbuf + buf * STAGE;
+    TL* dst = sbuf + buf * (PL * STAGE);
 #pragma unroll
     for (int i = 0; i < NLD; ++i)
-      if (tid + 256 * i < NSLOT) *reinterpret_cast<float4*>(dst + st_lds[i]) = st_reg[i];
+      if (tid + 256 * i < NSLOT) {
+        if constexpr (X3) {
+          const float f[8] = {st_reg[i][0].x, st_reg[i][0].y, st_reg[i][0].z, st_reg[i][0].w,
+                              st_reg[i][1].x, st_reg[i][1].y, st_reg[i][1].z, st_reg[i][1].w};
+          float4 pl[3];
+          split3(f, pl);
+#pragma unroll
+          for (int q = 0; q < 3; ++q) *reinterpret_cast<float4*>(dst + q * STAGE + st_lds[i]) = pl[q];
+        } else {
+          *reinterpret_cast<float4*>(dst + st_lds[i]) = st_reg[i][0];
+        }
+      }
   };
 
   // ---- operand addressing --------------------------------------------------------------------------------
@@ -149,22 +172,24 @@ __global__ __launch_bounds__(256) void k_tconv_mfma(ConvArgsT<T> a, TileSetDev p
     const int p = mb * 32 + l32;
     a_lane[mb] = (p >> 3) * RP + (p & 7) * LS + SUB * q0w + EPS * half;
   }
-  auto chunk_b = [&](int c) -> const T* {
+  auto chunk_b = [&](int c) -> const TL* {
     const bool second = c >= nch1;
     const int ci0 = (second ? c - nch1 : c) * CC;
     const int fb = second ? a.c1 : 0;
-    return a.filt_mc + ((long long)((fb + ci0) / SUB + q0w) * (K * K) * 2 * cout + cob0) * EPS;
+    return reinterpret_cast<const TL*>(a.filt_mc) + ((long long)((fb + ci0) / SUB + q0w) * (K * K) * (PL * 2) * cout + cob0) * EPS;
   };
-  float4 bring[RING];
-  auto load_b = [&](const T* ub, int unit, float4& bv) {
+  float4 bring[RING][PL];
+  auto load_b = [&](const TL* ub, int unit, float4 (&bv)[PL]) {
     const int tap = unit / NQW, qi = unit % NQW;
-    bv = *reinterpret_cast<const float4*>(ub + ((long long)((qi * (K * K) + tap) * 2) * cout) * EPS + b_lane);
+#pragma unroll
+    for (int q = 0; q < PL; ++q)
+      bv[q] = *reinterpret_cast<const float4*>(ub + ((long long)(((qi * (K * K) + tap) * PL + q) * 2) * cout) * EPS + b_lane);
   };
 
   const int c_lo = SPLIT ? bz * nch / (int)gridDim.z : 0;
   const int c_hi = SPLIT ? (bz + 1) * nch / (int)gridDim.z : nch;
-  const T* ub_cur = chunk_b(c_lo);
-  const T* ub_next = ub_cur;
+  const TL* ub_cur = chunk_b(c_lo);
+  const TL* ub_next = ub_cur;
   stage_load(c_lo);
 #pragma unroll
   for (int i = 0; i < (PD > 0 ? PD : 1); ++i) load_b(ub_cur, i, bring[i % RING]);
@@ -176,15 +201,17 @@ __global__ __launch_bounds__(256) void k_tconv_mfma(ConvArgsT<T> a, TileSetDev p
     const int cn = more ? c + 1 : c;
     ub_next = chunk_b(cn);
     stage_load(cn);
-    const T* sin = sbuf + ((c - c_lo) % NBUF) * STAGE;
-    float4 av[2][2];
-    auto load_a = [&](int unit, float4 (&dst)[2]) {
+    const TL* sin = sbuf + ((c - c_lo) % NBUF) * (PL * STAGE);
+    float4 av[2][2][PL];
+    auto load_a = [&](int unit, float4 (&dst)[2][PL]) {
       const int tap = unit / NQW, qi = unit % NQW;
       const int ky = tap / K, kx = tap - ky * K;
       const int dy = tc_shift(ky, PAD) + LO, dx = tc_shift(kx, PAD) + LO;
 #pragma unroll
       for (int mb = 0; mb < 2; ++mb)
-        dst[mb] = *reinterpret_cast<const float4*>(&sin[a_lane[mb] + dy * RP + dx * LS + SUB * qi]);
+#pragma unroll
+        for (int q = 0; q < PL; ++q)
+          dst[mb][q] = *reinterpret_cast<const float4*>(&sin[q * STAGE + a_lane[mb] + dy * RP + dx * LS + SUB * qi]);
     };
     load_a(0, av[0]);
 #pragma unroll
@@ -200,8 +227,20 @@ __global__ __launch_bounds__(256) void k_tconv_mfma(ConvArgsT<T> a, TileSetDev p
         const int tap = i / NQW;
         const int ky = tap / K, kx = tap - ky * K;
         const int ph = tc_phase(ky, PAD) * 2 + tc_phase(kx, PAD);      // compile-time after unrolling
+        if constexpr (X3) {
+          // the six significant term products of the unit, the two pixel blocks interleaved (smallest terms first)
+          const auto& A = av[i & 1];
+          const auto& B = bring[i % RING];
+          mma_unit(acc[ph][0], A[0][2], B[0], mie_bf16()); mma_unit(acc[ph][1], A[1][2], B[0], mie_bf16());
+          mma_unit(acc[ph][0], A[0][1], B[1], mie_bf16()); mma_unit(acc[ph][1], A[1][1], B[1], mie_bf16());
+          mma_unit(acc[ph][0], A[0][0], B[2], mie_bf16()); mma_unit(acc[ph][1], A[1][0], B[2], mie_bf16());
+          mma_unit(acc[ph][0], A[0][1], B[0], mie_bf16()); mma_unit(acc[ph][1], A[1][1], B[0], mie_bf16());
+          mma_unit(acc[ph][0], A[0][0], B[1], mie_bf16()); mma_unit(acc[ph][1], A[1][0], B[1], mie_bf16());
+          mma_unit(acc[ph][0], A[0][0], B[0], mie_bf16()); mma_unit(acc[ph][1], A[1][0], B[0], mie_bf16());
+        } else {
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb) mma_unit(acc[ph][mb], av[i & 1][mb], bring[i % RING], T());
+          for (int mb = 0; mb < 2; ++mb) mma_unit(acc[ph][mb], av[i & 1][mb][0], bring[i % RING][0], T());
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
       if (PD == 0) load_b(ub_next, 0, bring[0]);
@@ -270,9 +309,9 @@ __global__ __launch_bounds__(256) void k_tconv_mfma(ConvArgsT<T> a, TileSetDev p
   epilogue(std::integral_constant<int, 3>{});
 }
 
-template <typename T, int K>
+template <typename T, int K, bool X3 = false>
 bool launch_tconv(const ConvArgsT<T>& a0, const TileSetDev& pts, hipStream_t st) {
-  constexpr int CC = stage_channels(K, 1) * (4 / (int)sizeof(T));
+  constexpr int CC = X3 ? 64 : stage_channels(K, 1) * (4 / (int)sizeof(T));
   if (a0.filt_mc == nullptr || a0.c1 % CC != 0 || a0.c2 % CC != 0 || a0.cout % 32 != 0) return false;
   ConvArgsT<T> a = a0;
   a.xcd_fs = 0;
@@ -287,7 +326,7 @@ bool launch_tconv(const ConvArgsT<T>& a0, const TileSetDev& pts, hipStream_t st)
     while (2 * parts <= 8 && 2 * parts <= nch && groups * (2 * parts) <= 256 && (long long)(2 * parts) * a.ws_plane <= a.ws_floats)
       parts *= 2;
     if (parts >= 2) {
-      hipLaunchKernelGGL((k_tconv_mfma<T, K, 1, true>), dim3(cap_p, cout / 32, parts), dim3(256), 0, st, a, pts);
+      hipLaunchKernelGGL((k_tconv_mfma<T, K, 1, true, X3>), dim3(cap_p, cout / 32, parts), dim3(256), 0, st, a, pts);
       unsigned ny = (unsigned)((1024 + cap_out - 1) / cap_out);
       if (ny > (unsigned)(cout / 4)) ny = (unsigned)(cout / 4);
       if (ny < 1) ny = 1;
@@ -296,12 +335,14 @@ bool launch_tconv(const ConvArgsT<T>& a0, const TileSetDev& pts, hipStream_t st)
     }
   }
   a.ws = nullptr;
-  if (cout % 128 == 0 && (long long)cap_p * (cout / 128) >= 400)
-    hipLaunchKernelGGL((k_tconv_mfma<T, K, 4, false>), dim3(cap_p, cout / 128), dim3(256), 0, st, a, pts);
+  // (the 128-column kernel holds 4 phases x 2 blocks of accumulators and a four-column operand ring: in the three-term
+  // form it would spill, so that form stops at 64 columns)
+  if (!X3 && cout % 128 == 0 && (long long)cap_p * (cout / 128) >= 400)
+    hipLaunchKernelGGL((k_tconv_mfma<T, K, 4, false, false>), dim3(cap_p, cout / 128), dim3(256), 0, st, a, pts);
   else if (cout % 64 == 0 && (long long)cap_p * (cout / 64) >= 400)
-    hipLaunchKernelGGL((k_tconv_mfma<T, K, 2, false>), dim3(cap_p, cout / 64), dim3(256), 0, st, a, pts);
+    hipLaunchKernelGGL((k_tconv_mfma<T, K, 2, false, X3>), dim3(cap_p, cout / 64), dim3(256), 0, st, a, pts);
   else
-    hipLaunchKernelGGL((k_tconv_mfma<T, K, 1, false>), dim3(cap_p, cout / 32), dim3(256), 0, st, a, pts);
+    hipLaunchKernelGGL((k_tconv_mfma<T, K, 1, false, X3>), dim3(cap_p, cout / 32), dim3(256), 0, st, a, pts);
   return true;
 }
 
@@ -310,7 +351,7 @@ int tconv2x_impl(const char* who, const void* x, const uint8_t* xmask, int c1, c
                  const uint8_t* x2mask, int c2, int h_in, int w_in, const float* filter, const void* filter_mc,
                  int cin_total, int k, int cout, const mie_tileset* out, const mie_tileset* blocks,
                  void* out_delta, const void* addend, float* reservoir, int act_kind, float slope, bool refresh,
-                 const float* bias, void* workspace, long long workspace_bytes, void* stream) {
+                 const float* bias, void* workspace, long long workspace_bytes, void* stream, bool x3 = false) {
   int rc = mie_check_tileset(out, who);
   if (rc != MIE_OK) return rc;
   rc = mie_check_tileset(blocks, who);
@@ -323,8 +364,9 @@ int tconv2x_impl(const char* who, const void* x, const uint8_t* xmask, int c1, c
   MIE_REQUIRE((x2 != nullptr) == (c2 > 0) && (x2 != nullptr || x2mask == nullptr), MIE_ERR_INVALID_ARG,
               "%s: x2, c2 and x2mask must be given together", who);
   MIE_REQUIRE(k == 3 || k == 5, MIE_ERR_UNSUPPORTED, "%s: kernel size %d not implemented (3, 5)", who, k);
-  const int chunk = 128 / (int)sizeof(T);
-  MIE_REQUIRE(c1 % chunk == 0 && c2 % chunk == 0 && cout % 32 == 0 && cin_total % (32 / (int)sizeof(T)) == 0,
+  MIE_REQUIRE(!x3 || sizeof(T) == 4, MIE_ERR_INVALID_ARG, "%s: MIE_DTYPE_F32_BF16X3 is a form of fp32 deltas", who);
+  const int chunk = x3 ? 64 : 128 / (int)sizeof(T);
+  MIE_REQUIRE(c1 % chunk == 0 && c2 % chunk == 0 && cout % 32 == 0 && cin_total % (x3 ? 16 : 32 / (int)sizeof(T)) == 0,
               MIE_ERR_UNSUPPORTED, "%s: needs c1, c2 %% %d == 0 and cout %% 32 == 0 (c1=%d c2=%d cout=%d)", who, chunk,
               c1, c2, cout);
   MIE_REQUIRE(out->h == 2 * h_in && out->w == 2 * w_in && blocks->h == h_in && blocks->w == w_in && blocks->n == out->n,
@@ -352,10 +394,16 @@ int tconv2x_impl(const char* who, const void* x, const uint8_t* xmask, int c1, c
   a.pad = k / 2; a.cout = cout; a.out = (T*)out_delta; a.res = reservoir; a.act = act_kind; a.slope = slope;
   a.addend = (const T*)addend; a.refresh = refresh ? 1 : 0; a.bias = bias;
   a.hid = 0; a.g_cpd = nullptr; a.g_cpm = nullptr; a.g_cpres = nullptr; a.g_cres = nullptr; a.g_dh = nullptr; a.g_dc = nullptr;
-  a.ws = (float*)workspace; a.ws_floats = workspace_bytes / 4; a.ws_plane = 0; a.xcd_fs = 0; a.x3 = 0;
+  a.ws = (float*)workspace; a.ws_floats = workspace_bytes / 4; a.ws_plane = 0; a.xcd_fs = 0; a.x3 = x3 ? 1 : 0;
   a.ts = mie_dev_tileset(out);
   const TileSetDev pts = mie_dev_tileset(blocks);
-  const bool ok = (k == 3) ? launch_tconv<T, 3>(a, pts, (hipStream_t)stream) : launch_tconv<T, 5>(a, pts, (hipStream_t)stream);
+  bool ok;
+  if constexpr (sizeof(T) == 4) {
+    if (x3) ok = (k == 3) ? launch_tconv<T, 3, true>(a, pts, (hipStream_t)stream) : launch_tconv<T, 5, true>(a, pts, (hipStream_t)stream);
+    else ok = (k == 3) ? launch_tconv<T, 3>(a, pts, (hipStream_t)stream) : launch_tconv<T, 5>(a, pts, (hipStream_t)stream);
+  } else {
+    ok = (k == 3) ? launch_tconv<T, 3>(a, pts, (hipStream_t)stream) : launch_tconv<T, 5>(a, pts, (hipStream_t)stream);
+  }
   MIE_REQUIRE(ok, MIE_ERR_UNSUPPORTED, "%s: no kernel variant for c1=%d c2=%d cout=%d", who, c1, c2, cout);
   return mie_check_launch(who);
 }
@@ -369,6 +417,8 @@ extern "C" int mie_tconv2x_masked(const void* x, const uint8_t* xmask, int c1, c
                                   int dtype, void* workspace, long long workspace_bytes, void* stream) {
   const char* who = "mie_tconv2x_masked";
   mie_clear_error();
+  const bool x3 = dtype == MIE_DTYPE_F32_BF16X3;
+  if (x3) dtype = MIE_DTYPE_F32;
   MIE_REQUIRE(dtype == MIE_DTYPE_F32 || dtype == MIE_DTYPE_BF16, MIE_ERR_UNSUPPORTED, "%s: unknown delta dtype %d", who, dtype);
   if (dtype == MIE_DTYPE_BF16)
     return tconv2x_impl<mie_bf16>(who, x, xmask, c1, x2, x2mask, c2, h_in, w_in, filter, filter_mc, cin_total, k, cout, out,
@@ -376,7 +426,7 @@ extern "C" int mie_tconv2x_masked(const void* x, const uint8_t* xmask, int c1, c
                                   workspace_bytes, stream);
   return tconv2x_impl<float>(who, x, xmask, c1, x2, x2mask, c2, h_in, w_in, filter, filter_mc, cin_total, k, cout, out, blocks,
                              out_delta, addend, reservoir, act_kind, slope, false, nullptr, workspace, workspace_bytes,
-                             stream);
+                             stream, x3);
 }
 
 extern "C" int mie_tconv2x_refresh(const void* x, int c1, const void* x2, int c2, int h_in, int w_in, const float* filter,
@@ -385,10 +435,12 @@ extern "C" int mie_tconv2x_refresh(const void* x, int c1, const void* x2, int c2
                                    float* reservoir, int act_kind, float slope, int dtype, void* stream) {
   const char* who = "mie_tconv2x_refresh";
   mie_clear_error();
+  const bool x3 = dtype == MIE_DTYPE_F32_BF16X3;
+  if (x3) dtype = MIE_DTYPE_F32;
   MIE_REQUIRE(dtype == MIE_DTYPE_F32 || dtype == MIE_DTYPE_BF16, MIE_ERR_UNSUPPORTED, "%s: unknown delta dtype %d", who, dtype);
   if (dtype == MIE_DTYPE_BF16)
     return tconv2x_impl<mie_bf16>(who, x, nullptr, c1, x2, nullptr, c2, h_in, w_in, filter, filter_mc, cin_total, k, cout, out,
                                   blocks, out_dense, addend, reservoir, act_kind, slope, true, bias, nullptr, 0, stream);
   return tconv2x_impl<float>(who, x, nullptr, c1, x2, nullptr, c2, h_in, w_in, filter, filter_mc, cin_total, k, cout, out, blocks,
-                             out_dense, addend, reservoir, act_kind, slope, true, bias, nullptr, 0, stream);
+                             out_dense, addend, reservoir, act_kind, slope, true, bias, nullptr, 0, stream, x3);
 }

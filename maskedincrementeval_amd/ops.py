@@ -538,7 +538,15 @@ def _tconv2x_args(x, x2, filt, k, out_ts, block_ts, out, addend, reservoir):
     c2 = 0 if x2 is None else x2.shape[1]
     if x2 is not None and (x2.shape[0] != n or x2.shape[2:] != x.shape[2:] or x2.dtype != x.dtype):
         raise ValueError("x2 %s incompatible with x %s" % (tuple(x2.shape), tuple(x.shape)))
-    plain, mc_ptr = _filter_args(filt, k, x.dtype)
+    # fp32 deltas in the three-term bf16 form where the setting asks for it and the channel counts are whole chunks of 64
+    x3 = (x.dtype == torch.float32 and isinstance(filt, ConvFilter) and f32_matmul == "bf16x3"
+          and c1 % 64 == 0 and c2 % 64 == 0 and filt.shape[3] % 32 == 0)
+    if x3:
+        plain, mc = filt.for_dtype(torch.float32, x3=True)
+        mc_ptr, code = mc.data_ptr(), _lib.DTYPE_F32_BF16X3
+    else:
+        plain, mc_ptr = _filter_args(filt, k, x.dtype)
+        code = delta_dtype(x)
     cin_total, cout = plain.shape[0], plain.shape[3]
     if mc_ptr is None:
         raise ValueError("tconv2x needs a ConvFilter with a matrix-core copy")
@@ -548,7 +556,7 @@ def _tconv2x_args(x, x2, filt, k, out_ts, block_ts, out, addend, reservoir):
     for name, t in (("addend", addend), ("reservoir", reservoir)):
         if t is not None and t.shape != out.shape:
             raise ValueError("%s shape %s != output %s" % (name, tuple(t.shape), tuple(out.shape)))
-    return n, c1, c2, h, w, plain, mc_ptr, cin_total, cout
+    return n, c1, c2, h, w, plain, mc_ptr, cin_total, cout, code
 
 
 def tconv2x_masked(x, xmask, x2, x2mask, filt, k, out_ts: TileMask, block_ts: TileMask, out_delta, reservoir=None,
@@ -557,7 +565,7 @@ def tconv2x_masked(x, xmask, x2, x2mask, filt, k, out_ts: TileMask, block_ts: Ti
     cores.  out_ts: MIE_FOOT_TCONV tile set of the output; block_ts: tile set of the 16x16 output blocks at
     input resolution (build_mask_tiles(out_ts, None, ..., FOOT_CONV, 2, 2, 0, block_ts)).
     workspace: as in conv_masked (None: the device's shared one when the plane is small, False: none)."""
-    n, c1, c2, h, w, plain, mc_ptr, cin_total, cout = _tconv2x_args(x, x2, filt, k, out_ts, block_ts, out_delta,
+    n, c1, c2, h, w, plain, mc_ptr, cin_total, cout, code = _tconv2x_args(x, x2, filt, k, out_ts, block_ts, out_delta,
                                                                     addend, reservoir)
     dt = x.dtype
     _ready(out_ts)
@@ -569,14 +577,14 @@ def tconv2x_masked(x, xmask, x2, x2mask, filt, k, out_ts: TileMask, block_ts: Ti
         nhwc_ptr(x, "x", dtype=dt), pix_ptr(xmask, n, h, w, "xmask"), c1, nhwc_ptr(x2, "x2", dtype=dt),
         pix_ptr(x2mask, n, h, w, "x2mask"), c2, h, w, plain.data_ptr(), mc_ptr, cin_total, k, cout, out_ts.ref,
         block_ts.ref, nhwc_ptr(out_delta, "out_delta", dtype=dt), nhwc_ptr(addend, "addend", cout, dtype=dt),
-        nhwc_ptr(reservoir, "reservoir"), act, float(slope), delta_dtype(x), ws_ptr, ws_bytes, _stream(x)))
+        nhwc_ptr(reservoir, "reservoir"), act, float(slope), code, ws_ptr, ws_bytes, _stream(x)))
     return out_delta
 
 
 def tconv2x_refresh(x, x2, filt, bias, k, out_ts: TileMask, block_ts: TileMask, out_dense, reservoir=None,
                     act=_lib.ACT_NONE, slope=0.0, addend=None):
     """Dense twin of tconv2x_masked (both tile sets all active): bias, activation and reservoir fill fused."""
-    n, c1, c2, h, w, plain, mc_ptr, cin_total, cout = _tconv2x_args(x, x2, filt, k, out_ts, block_ts, out_dense,
+    n, c1, c2, h, w, plain, mc_ptr, cin_total, cout, code = _tconv2x_args(x, x2, filt, k, out_ts, block_ts, out_dense,
                                                                     addend, reservoir)
     dt = x.dtype
     if bias is not None and (bias.numel() != cout or bias.dtype != torch.float32 or not bias.is_contiguous()):
@@ -587,7 +595,7 @@ def tconv2x_refresh(x, x2, filt, bias, k, out_ts: TileMask, block_ts: TileMask, 
         nhwc_ptr(x, "x", dtype=dt), c1, nhwc_ptr(x2, "x2", dtype=dt), c2, h, w, plain.data_ptr(), mc_ptr, cin_total, k,
         cout, None if bias is None else bias.data_ptr(), out_ts.ref, block_ts.ref,
         nhwc_ptr(out_dense, "out_dense", dtype=dt), nhwc_ptr(addend, "addend", cout, dtype=dt),
-        nhwc_ptr(reservoir, "reservoir"), act, float(slope), delta_dtype(x), _stream(x)))
+        nhwc_ptr(reservoir, "reservoir"), act, float(slope), code, _stream(x)))
     return out_dense
 
 

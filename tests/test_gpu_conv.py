@@ -227,7 +227,8 @@ def test_tconv2x_few_channel_form(cin, cout, h, w, dtype):
     (256, 256, 64, 16, 16, 3),     # 4 blocks x 2 slabs, 16 chunks: the contraction is split over workgroups
     (64, 0, 128, 40, 48, 5),       # 5x5 (the depth network's decoder kind): halo on all sides
     (128, 128, 32, 9, 20, 5)])
-def test_tconv2x_matrix_core_form(c1, c2, cout, h, w, k, dtype):
+@pytest.mark.parametrize("f32mode", ["bf16x3", "native"])
+def test_tconv2x_matrix_core_form(c1, c2, cout, h, w, k, dtype, f32mode):
     # stride-2 transposed conv as four sub-pixel phases on the matrix cores, against F.conv_transpose2d of the
     # concat; three steps with fresh masks (stale blocks), reservoir + ReLU epilogue and an addend
     if dtype == torch.bfloat16 and (c1 % 64 or c2 % 64):
