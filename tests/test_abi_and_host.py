@@ -260,3 +260,25 @@ def test_single_hip_runtime_is_mapped(mie_lib):
     with open("/proc/self/maps") as f:
         paths = {line.split()[-1] for line in f if "libamdhip64" in line}
     assert len(paths) == 1, paths
+
+
+def test_python_constants_mirror_the_header():
+    """Every MIE_* code the Python side passes is the value include/mie.h defines (the dtype codes included: a
+    mismatch would silently select another arithmetic)."""
+    import re
+    hdr = open(os.path.join(ROOT, "include", "mie.h")).read()
+    defs = {m.group(1): int(m.group(2)) for m in re.finditer(r"#define\s+(MIE_[A-Z0-9_]+)\s+(-?\d+)\b", hdr)}
+    pairs = [("MIE_DTYPE_F32", _lib.DTYPE_F32), ("MIE_DTYPE_BF16", _lib.DTYPE_BF16),
+             ("MIE_DTYPE_F32_BF16X3", _lib.DTYPE_F32_BF16X3), ("MIE_PATH_AUTO", _lib.PATH_AUTO),
+             ("MIE_PATH_VALU", _lib.PATH_VALU), ("MIE_PATH_MFMA", _lib.PATH_MFMA), ("MIE_FOOT_CONV", _lib.FOOT_CONV),
+             ("MIE_FOOT_UP2X", _lib.FOOT_UP2X), ("MIE_FOOT_TCONV", _lib.FOOT_TCONV)]
+    for name, value in pairs:
+        assert defs[name] == value, name
+
+
+def test_three_term_shape_query_needs_no_gpu(mie_lib):
+    """mie_conv_f32x3_takes is host logic: which conv shapes run fp32 deltas in the three-term bf16 form."""
+    takes = mie_lib.mie_conv_f32x3_takes
+    assert takes(3, 1, 64, 64, 256) == 1 and takes(5, 1, 256, 0, 128) == 1 and takes(5, 2, 32, 0, 64) == 1
+    assert takes(3, 2, 64, 0, 64) == 0 and takes(7, 1, 64, 0, 64) == 0 and takes(1, 1, 64, 0, 64) == 0
+    assert takes(3, 1, 48, 0, 64) == 0 and takes(3, 1, 64, 0, 48) == 0 and takes(5, 2, 24, 0, 64) == 0
