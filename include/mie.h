@@ -80,7 +80,9 @@ extern "C" {
  * the rounding step of an fp32 multiply-add.  Taken by mie_pack_filter and by the `dtype` of
  * mie_conv_masked / _ws / _noalloc, mie_conv_refresh, mie_upconv_masked, mie_conv_gates_masked (shapes:
  * mie_conv_f32x3_takes) and mie_tconv2x_masked / mie_tconv2x_refresh (c1, c2 multiples of 64), with filter_mc
- * packed for it; every buffer is what it is for MIE_DTYPE_F32. */
+ * packed for it; every buffer is what it is for MIE_DTYPE_F32.  Values must be finite and below the bf16
+ * maximum (3.39e38): an infinity, or a value that rounds to one in bf16, splits into inf - inf and gives
+ * NaN where the fp32 instruction would give an infinity. */
 #define MIE_DTYPE_F32_BF16X3 2
 
 /* frame kinds of mie_events_to_frame */
