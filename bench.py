@@ -770,6 +770,12 @@ def main():
                    "density": dens, "height": H, "width": W, "batch": NB, "graph": not args.no_graph,
                    "timing": "median of %d repeats of %d steps" % (args.repeats, args.steps),
                    "f32_matmul": ops.f32_matmul if args.dtype == "f32" else None,
+                   "arithmetic": (("fp32 deltas, reservoirs and accumulators; matrix-core products as three bf16 terms per "
+                                   "value, six term products per multiply (error against fp64 no larger than the fp32 "
+                                   "instruction's: tests/test_gpu_f32x3.py); the same frame with the fp32 matrix-core "
+                                   "instruction is timed in f32_native_mfma") if ops.f32_matmul == "bf16x3"
+                                  else "fp32 deltas, reservoirs, accumulators and matrix-core instruction") if args.dtype == "f32"
+                   else "bf16 deltas and weights, fp32 reservoirs and accumulators",
                    "mask_planning": "inline" if args.sync_masks else ("second stream, builds first" if args.plan_first else "second stream")},
         "roofline": roofline,
         "cpu_baseline": cpu,
