@@ -771,7 +771,7 @@ def main():
                    "timing": "median of %d repeats of %d steps" % (args.repeats, args.steps),
                    "f32_matmul": ops.f32_matmul if args.dtype == "f32" else None,
                    "arithmetic": (("fp32 deltas, reservoirs and accumulators; matrix-core products as three bf16 terms per "
-                                   "value, six term products per multiply (error against fp64 no larger than the fp32 "
+                                   "value, six term products per multiply (error against fp64 0.6-1.1 of the fp32 "
                                    "instruction's: tests/test_gpu_f32x3.py); the same frame with the fp32 matrix-core "
                                    "instruction is timed in f32_native_mfma") if ops.f32_matmul == "bf16x3"
                                   else "fp32 deltas, reservoirs, accumulators and matrix-core instruction") if args.dtype == "f32"
