@@ -44,7 +44,7 @@ def test_three_term_filter_copy_sums_to_the_weights_exactly():
 
 @pytest.mark.parametrize("cin,cout,k,h,w,density", [(64, 64, 3, 40, 40, 1.0), (64, 32, 5, 33, 47, 0.3), (256, 256, 3, 33, 44, 1.0),
                                                       (256, 128, 5, 34, 42, 1.0), (128, 96, 3, 20, 28, 0.5)])
-def test_error_against_fp64_is_no_larger_than_the_fp32_instructions(cin, cout, k, h, w, density):
+def test_error_against_fp64_beside_the_fp32_instructions(cin, cout, k, h, w, density):
     p = k // 2
     torch.manual_seed(cin + cout + k)
     x = torch.randn(1, cin, h, w)
@@ -72,7 +72,8 @@ def test_error_against_fp64_is_no_larger_than_the_fp32_instructions(cin, cout, k
             err[mode] = (e.max().item(), (e / bound.clamp_min(1e-30)).max().item())
     finally:
         ops.f32_matmul = old
-    # relative to sum |x||w| both stay within a few fp32 rounding steps; the three-term form is not the worse one
+    # relative to sum |x||w| both stay within a few fp32 rounding steps, and the three-term form within a quarter of the
+    # fp32 instruction's error (it is the smaller one where both kernels split the contraction the same way)
     assert err["bf16x3"][1] < 4e-7 and err["native"][1] < 4e-7, err
     assert err["bf16x3"][0] <= 1.25 * err["native"][0] + 1e-7, err
 
