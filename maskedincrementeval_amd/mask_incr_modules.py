@@ -513,14 +513,18 @@ class nnConvIncr(nn.Conv2d, _ConvIncrMixin):
         k, s, p = self._geometry()
         x = x_incr[0]
         # Measured on MI355X.  bf16: the one-kernel form wins at every size (264x352 frame -3 %, 8x480x640
-        # step -6 %).  fp32: on planes of up to a few thousand tiles the step is bound by launches and the
-        # one-kernel form wins (1.5 % of a 264x352 frame) unless the layer has more than 4 staged chunks
-        # (256 channels: the per-chunk blend then costs what the saved launch gains); on large planes the
-        # separate up-sampling kernel is cheaper (8x480x640 step +2 % with the one-kernel form).
+        # step -6 %).  fp32 on the fp32 matrix-core instruction: on planes of up to a few thousand tiles the step
+        # is bound by launches and the one-kernel form wins (1.5 % of a 264x352 frame) unless the layer has more
+        # than 4 staged chunks (256 channels: the per-chunk blend then costs what the saved launch gains); on
+        # large planes the separate up-sampling kernel is cheaper (8x480x640 step +2 % with the one-kernel form).
+        # fp32 in the three-term form: the one-kernel form wins at every size and depth (264x352 frame -0.4 %,
+        # 8x480x640 step -1.8 %).
         dt = ops.delta_torch_dtype(x)
         tiles = x.shape[0] * ((2 * x.shape[2] + 7) // 8) * ((2 * x.shape[3] + 7) // 8)
         chunks = x.shape[1] // ops.mfma_chunk(dt)
-        small = dt == torch.bfloat16 or (tiles <= ops.upconv_max_tiles and chunks <= ops.upconv_max_chunks)
+        three_term = dt == torch.float32 and ops.f32x3_takes(k, s, x.shape[1], 0, self.out_channels)
+        small = (dt == torch.bfloat16 or three_term
+                 or (tiles <= ops.upconv_max_tiles and chunks <= ops.upconv_max_chunks))
         if self.lossy or not small or not ops.upconv_takes(x.shape[1], self.out_channels, k, s, p,
                                                             self.conv2d_weights, dt):
             return self.forward_fused(up(x_incr, skip_incr), activation)

@@ -421,7 +421,8 @@ def conv_masked(x, xmask, x2, x2mask, filt, k, stride, pad, out_ts: TileMask, ou
     return out_delta
 
 
-# Up to which size fp32 decoder layers take the one-kernel form (see nnConvIncr.forward_fused_upsampled).
+# Up to which size fp32 decoder layers take the one-kernel form where they run on the fp32 matrix-core instruction
+# (see nnConvIncr.forward_fused_upsampled; in the three-term form they always do).
 upconv_max_tiles = 2048
 upconv_max_chunks = 4
 
