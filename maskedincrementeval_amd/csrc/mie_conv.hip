@@ -155,7 +155,7 @@ static __device__ __forceinline__ float4 load4(const mie_bf16* p) {
 template <typename T>
 __global__ __launch_bounds__(256) void k_conv1x1_smallco(ConvArgsT<T> a) {
   int n, y0, x0;
-  const int tk = mie_pick_tile(a.ts, blockIdx.x, n, y0, x0);
+  const int tk = mie_pick_tile(a.ts, blockIdx.x + conv_args_entry_zero(a), n, y0, x0);
   if (tk == 0) return;
   const int px = threadIdx.x >> 2, sub = threadIdx.x & 3;
   const int oy = y0 + (px >> 3), ox = x0 + (px & 7);
@@ -237,7 +237,7 @@ __global__ __launch_bounds__(256) void k_tconv_valu(ConvArgsT<T> a, int K, int S
 template <typename T>
 __global__ __launch_bounds__(256) void k_tconv2x_fewcin(ConvArgsT<T> a) {
   int n, y0, x0;
-  const int tk = mie_pick_tile(a.ts, blockIdx.x, n, y0, x0);
+  const int tk = mie_pick_tile(a.ts, blockIdx.x + conv_args_entry_zero(a), n, y0, x0);
   if (tk == 0) return;
   const int hout = a.ts.h, wout = a.ts.w, cout = a.cout, c1 = a.c1;
   const int G = cout >> 2;

@@ -39,7 +39,7 @@ __global__ __launch_bounds__(256) void k_conv_fewcin(ConvArgsT<T> a) {
   float* const s_w = smem + IN_F;
 
   int n, y0, x0;
-  const int tk = mie_pick_tile(a.ts, blockIdx.x, n, y0, x0);
+  const int tk = mie_pick_tile(a.ts, blockIdx.x + conv_args_entry_zero(a), n, y0, x0);
   if (tk == 0) return;
   const int tid = threadIdx.x;
   const int hout = a.ts.h, wout = a.ts.w, cout = a.cout, cin = a.c1;

@@ -298,8 +298,9 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
   // (one more dependent load at the start of a workgroup: measured, it costs nothing even on launches
   // of a few dozen workgroups), and idle positions of the capacity-sized grid fall off the end.
   // (For the SPLIT launches the same idea, one filter slice per XCD, was measured: no gain.)
+  const int entry_zero = conv_args_entry_zero(a);      // every line of the argument block, fetched in one batch
   MIE_STAMP(0);
-  int bx = blockIdx.x, by = blockIdx.y;
+  int bx = blockIdx.x + entry_zero, by = blockIdx.y;
   const int bz = SPLIT ? (int)blockIdx.z : 0;
   int n, y0, x0, tk;
   if (!SPLIT && a.xcd_fs > 0) {
@@ -957,7 +958,7 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
 template <typename T>
 __global__ __launch_bounds__(256) void k_conv_split_finish(ConvArgsT<T> a, int parts) {
   int n, y0, x0;
-  const int tk = mie_pick_tile(a.ts, blockIdx.x, n, y0, x0);
+  const int tk = mie_pick_tile(a.ts, blockIdx.x + conv_args_entry_zero(a), n, y0, x0);
   if (tk == 0) return;
   const int hout = a.ts.h, wout = a.ts.w, cout = a.cout;
   const int cb = (((cout + (int)gridDim.y - 1) / (int)gridDim.y) + 3) & ~3;      // channels of this block (whole groups of four)

@@ -68,7 +68,7 @@ __global__ __launch_bounds__(256) void k_tconv_mfma(ConvArgsT<T> a, TileSetDev p
   TL* const sbuf = reinterpret_cast<TL*>(smem);
 
   int n, y0, x0;                                             // block origin in INPUT coordinates
-  const int tk = mie_pick_tile(pts, blockIdx.x, n, y0, x0);
+  const int tk = mie_pick_tile(pts, blockIdx.x + conv_args_entry_zero(a), n, y0, x0);
   if (tk == 0) return;
   const int by = blockIdx.y, bz = SPLIT ? (int)blockIdx.z : 0;
   const int tid = threadIdx.x;
