@@ -53,7 +53,10 @@
 // The X3 form does the same 3x3 chunk's work in 54 MFMAs of 32 cycles, 0.95 us, and takes 2.4 us for it: with one wave
 // per SIMD nothing overlaps that wave's own staging work (88 VALU instructions to split a chunk's values, address
 // arithmetic, waits -- the load counter is in order, so a filter prefetch behind the staging loads waits for them).
-// A three-chunk software pipeline with two staging register sets changed nothing (19.8 us either way) and was removed.
+// A three-chunk software pipeline with two staging register sets changed nothing (19.8 us either way) and was removed;
+// so were two extra waves that did all the staging with loads in flight four chunks ahead (chunk 2.2 -> 1.9 us, but a
+// longer head: 20.8 -> 20.5 us).  With every filter load and LDS read of the loop made cache-resident on top of that
+// (timing only) the chunk still takes 1.5 us: the staging latency is 0.3 us of it, all memory effects 0.7 us.
 #pragma once
 #include "mie_conv.h"
 #include <stdlib.h>
