@@ -566,9 +566,11 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
       // The taps' LDS offsets and weights depend on the tile only, and the compiler computes them once
       // and keeps 40 registers alive through the contraction.  fp32 kernels have the registers to spare
       // (two workgroups per CU either way) and run 1.5 % faster for it; in the bf16 kernels they cost
-      // one or two resident workgroups, so there an opaque zero makes them a per-chunk computation.
+      // one or two resident workgroups, so there an opaque zero makes them a per-chunk computation.  The three-term
+      // kernels: the 32-column one would pass 256 registers and lose its second workgroup; the wider ones have the
+      // room (252) and keep the values (decoder 0 of the 264x352 frame 73 -> 70 us).
       int opaque = 0;
-      if (sizeof(T) == 2 || X3) asm volatile("" : "+v"(opaque));
+      if (sizeof(T) == 2 || (X3 && WN == 1)) asm volatile("" : "+v"(opaque));
 #pragma unroll
       for (int i = 0; i < NLD; ++i) {
         const int slot = tid + 256 * i + opaque;
