@@ -10,15 +10,19 @@ resident in HBM before the timed region starts and the step is replayed from
 a HIP graph.  `--steps` steps are timed between two device synchronisations,
 `--repeats` times over; `ms_per_step` is the median of those repeats.
 
-Prints ONE JSON line: frames/s (`value`), ms/frame, the roofline of the
-dominant kernel launch (the masked conv layer that takes the most time,
-timed with HIP events on the stream it runs on), a per-layer table, the same
-network run densely through the same kernels (all tiles active), 1 % and 20 %
-density, the dense refresh, the other benchmark configurations ("configs":
-single masked conv, activation chain, EVFlowNet-incr with both decoder kinds,
-batched bf16 E2Depth-incr), the lossy frontier (delta quantiser / threshold
-masks: speed against error) and the CPU baseline (the torch-CPU oracle of the
-reference path on the host cores).
+Prints ONE compact JSON line on stdout (kept under 6000 characters: asserted by
+tests/test_bench_line.py): frames/s (`value`), ms/frame, the roofline of the
+dominant kernel launch (the masked conv layer that takes the most time, timed
+with HIP events on the stream it runs on), the CPU baseline (the torch-CPU
+oracle of the reference path on the host cores), a check of the first steps
+against that oracle, and a {time, roofline fraction} summary of everything
+else that is measured: the same network run densely through the same kernels
+(all tiles active), 1 % and 20 % density, the dense refresh, the other
+benchmark configurations (single masked conv, activation chain, EVFlowNet-incr
+with both decoder kinds, batched bf16 E2Depth-incr) and the lossy frontier
+(delta quantiser / threshold masks: speed against error).  The full tables
+(per-launch table, every configuration with its repeats, every lossy point) go
+to `--detail-file` (default gpurun_out/bench_detail.json) and to stderr.
 """
 import argparse
 import json
@@ -75,6 +79,9 @@ def parse_args():
                          "three bf16 terms per value on the bf16 instruction, fp32 accuracy)")
     ap.add_argument("--no-native", dest="native", action="store_false",
                     help="skip the comparison run with the fp32 matrix-core instruction")
+    ap.add_argument("--detail-file", default=os.path.join(ROOT, "gpurun_out", "bench_detail.json"),
+                    help="where the full tables go (per-launch table, configurations, lossy frontier); stdout carries "
+                         "one compact JSON line")
     return ap.parse_args()
 
 
@@ -728,7 +735,7 @@ def main():
             steps=min(args.steps, 20), repeats=max(3, args.repeats // 2))
 
     # ---- CPU baseline: the oracle (torch-CPU restatement of the reference path) -----------------
-    cpu = None
+    cpu = oracle_check = None
     if args.cpu_steps > 0:
         torch.set_num_threads(min(os.cpu_count() or 1, 16))
         if args.net == "evflownet":
@@ -738,11 +745,41 @@ def main():
             from oracle.e2depth_oracle import E2DepthOracle
             oracle = E2DepthOracle(model.state_dict())
         with torch.no_grad():
-            oracle.refresh(nb.x0)
-            oracle.incr(nb.deltas_cpu[0])
+            # The oracle as the checker: a fresh instance of the timed network (same weights) takes the dense refresh
+            # and the first incremental steps of the CPU run, and every output must match the oracle's.
+            n_chk = 3
+            chk = nb.new_model(async_masks=not args.sync_masks, plan_first=args.plan_first)
+            if args.dtype == "f32":
+                rtol, atol_of = 1e-4, lambda ref: 1e-5
+            else:
+                rtol, atol_of = 2e-2, lambda ref: 3 * 2.0 ** -8 * max(float(ref.abs().max()), 1e-3)
+            worst = 0.0
+
+            def compare(got, ref, what):
+                nonlocal worst
+                got = got.float().cpu()
+                err = (got - ref).abs().max().item()
+                worst = max(worst, err)
+                if not torch.allclose(got, ref, rtol=rtol, atol=atol_of(ref)):
+                    raise SystemExit("bench: %s differs from the CPU oracle (max |difference| %.3e)" % (what, err))
+
+            ref0 = oracle.refresh(nb.x0)
+            got0 = nb.refresh_out(nb.refresh_net(chk, nb.cl(nb.x0)))
+            if args.net == "evflownet":
+                ref0 = ref0[-1]
+            compare(got0, ref0, "the dense refresh")
+            for i in range(n_chk):
+                ref = oracle.incr(nb.deltas_cpu[i % nb.n_inputs])
+                if args.net == "evflownet":
+                    ref = ref[-1]
+                compare(nb.out_of(nb.step_eager(chk, i)), ref, "incremental step %d" % i)
+            oracle_check = dict(max_abs_diff=worst, steps=n_chk, rtol=rtol, atol=atol_of(ref),
+                                against="CPU oracle, same weights and inputs: dense refresh + %d incremental steps" % n_chk)
+            log("oracle check: refresh + %d steps, max |difference| %.3e" % (n_chk, worst))
+            del chk
             t0 = time.perf_counter()
             for i in range(args.cpu_steps):
-                oracle.incr(nb.deltas_cpu[(1 + i) % nb.n_inputs])
+                oracle.incr(nb.deltas_cpu[(n_chk + i) % nb.n_inputs])
             cdt = (time.perf_counter() - t0) / args.cpu_steps
         cpu = dict(value=round(NB / cdt, 3), unit="frames/s", cores=torch.get_num_threads(), kind="port",
                    ms_per_step=round(1e3 * cdt, 2),
@@ -750,9 +787,11 @@ def main():
                           "delta, as the reference executes it), torch-CPU fp32" % (args.cpu_steps, NET_NAME, H, W))
         log("cpu baseline: %.1f ms/frame on %d threads" % (1e3 * cdt, cpu["cores"]))
 
-    result = {
-        # the headline metric's name; `value` is its frames/s part, the HBM GB/s part is in
-        # "hbm_gbs_whole_frame" and per launch in "layers"
+    x3 = args.dtype == "f32" and ops.f32_matmul == "bf16x3"
+    # one basis for every matrix-core fraction of the line: the peak of the instruction that runs (for fp32 deltas
+    # in the three-term form the bf16 peak over the six term products of a multiply)
+    mfma_peak = PEAK_BF16_MFMA_TFLOPS / 6.0 if x3 else nb.peak_mfma
+    detail = {
         "metric": "incremental frames/s + HBM GB/s, %s %dx%d @%g%% delta density" % (NET_NAME, H, W, 100 * dens),
         "value": round(NB / sec_per_step, 2),
         "unit": "frames/s",
@@ -770,22 +809,17 @@ def main():
                    "density": dens, "height": H, "width": W, "batch": NB, "graph": not args.no_graph,
                    "timing": "median of %d repeats of %d steps" % (args.repeats, args.steps),
                    "f32_matmul": ops.f32_matmul if args.dtype == "f32" else None,
-                   "arithmetic": (("fp32 deltas, reservoirs and accumulators; matrix-core products as three bf16 terms per "
-                                   "value, six term products per multiply (error against fp64 0.6-1.1 of the fp32 "
-                                   "instruction's: tests/test_gpu_f32x3.py); the same frame with the fp32 matrix-core "
-                                   "instruction is timed in f32_native_mfma") if ops.f32_matmul == "bf16x3"
-                                  else "fp32 deltas, reservoirs, accumulators and matrix-core instruction") if args.dtype == "f32"
-                   else "bf16 deltas and weights, fp32 reservoirs and accumulators",
+                   "arithmetic": ARITHMETIC["bf16" if args.dtype == "bf16" else ops.f32_matmul],
                    "mask_planning": "inline" if args.sync_masks else ("second stream, builds first" if args.plan_first else "second stream")},
         "roofline": roofline,
         "cpu_baseline": cpu,
         "repeats_ms_per_step": repeats_ms,
-        "hbm_gbs_whole_frame": round(tot_bytes / sec_per_step / 1e9, 1),
-        "hbm_frac_whole_frame": round(tot_bytes / sec_per_step / 1e9 / PEAK_HBM_GBS, 5),
-        "algorithmic_mb_per_frame": round(tot_bytes / 1e6, 2),
-        "algorithmic_gflop_per_frame": round(tot_flops / 1e9, 3),
-        "mfma_frac_whole_frame": round(tot_flops / sec_per_step / 1e12 / nb.peak_mfma, 4),
-        "sum_kernel_us": round(tot_us, 1),
+        "whole_frame": {"algorithmic_mb": round(tot_bytes / 1e6, 2), "algorithmic_gflop": round(tot_flops / 1e9, 3),
+                        "hbm_gbs": round(tot_bytes / sec_per_step / 1e9, 1),
+                        "hbm_frac": round(tot_bytes / sec_per_step / 1e9 / PEAK_HBM_GBS, 5),
+                        "mfma_tflops": round(tot_flops / sec_per_step / 1e12, 2),
+                        "mfma_frac": round(tot_flops / sec_per_step / 1e12 / mfma_peak, 4),
+                        "mfma_peak_tflops": round(mfma_peak, 1), "sum_kernel_us": round(tot_us, 1)},
         "f32_native_mfma": native,
         "dense_same_kernels_ms": None if dense_sec is None else round(1e3 * dense_sec, 4),
         "speedup_vs_dense": None if dense_sec is None else round(dense_sec / sec_per_step, 3),
@@ -794,9 +828,97 @@ def main():
         "lossy_frontier": lossy,
         "configs": configs,
         "output_check": output_check,
+        "oracle_check": oracle_check,
         "layers": layers,
     }
-    print(json.dumps(result))
+    # The bulky tables go to a side file and to stderr; stdout carries one compact line.
+    try:
+        os.makedirs(os.path.dirname(os.path.abspath(args.detail_file)), exist_ok=True)
+        with open(args.detail_file, "w") as f:
+            json.dump(detail, f, indent=1)
+        log("full tables written to %s" % args.detail_file)
+    except OSError as e:
+        log("could not write %s: %s" % (args.detail_file, e))
+        args.detail_file = None
+    log("detail: " + json.dumps({k: detail[k] for k in ("configs", "lossy_frontier", "density_sweep", "refresh")}))
+    print(compact_line(detail, args.detail_file))
+
+
+ARITHMETIC = {
+    "bf16x3": "fp32 deltas, reservoirs, accumulators; matrix-core products as three bf16 terms per value "
+              "(six term products per multiply, fp32-class error: tests/test_gpu_f32x3.py)",
+    "native": "fp32 deltas, reservoirs, accumulators and matrix-core instruction",
+    "bf16": "bf16 deltas and weights, fp32 reservoirs and accumulators",
+}
+LINE_LIMIT = 6000        # characters of the stdout line (the driver keeps the tail of stdout only)
+
+
+def _pick(d, keys):
+    return None if d is None else {k: d[k] for k in keys if k in d}
+
+
+def compact_line(detail, detail_file=None):
+    """The one JSON line of stdout: the contract keys, `roofline`, `cpu_baseline` and a summary of everything else
+    (one {ms_per_step | us, frac, bound, kernel} entry per configuration and density).  The per-launch table, the
+    lossy frontier, per-repeat lists and the full `configs` block stay in `detail` (side file, stderr)."""
+    line = {k: detail[k] for k in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step",
+                                   "higher_is_better", "scaling", "vs_baseline", "dtype", "data")}
+    line["config"] = detail["config"]
+    roof = detail["roofline"]
+    line["roofline"] = _pick(roof, ("bound", "achieved", "peak", "unit", "frac", "traffic", "kernel", "us", "peak_basis",
+                                    "frac_of_fp32_mfma_peak", "algorithmic_bytes", "algorithmic_flops"))
+    line["cpu_baseline"] = detail["cpu_baseline"]
+    line["whole_frame"] = detail.get("whole_frame")
+    nat = detail.get("f32_native_mfma")
+    line["f32_native_mfma_ms"] = None if nat is None else nat["ms_per_step"]
+    line["dense_same_kernels_ms"] = detail.get("dense_same_kernels_ms")
+    line["speedup_vs_dense"] = detail.get("speedup_vs_dense")
+    sweep = detail.get("density_sweep")
+    line["density_sweep_ms"] = None if sweep is None else {p: r["ms_per_step"] for p, r in sweep.items()}
+    ref = detail.get("refresh")
+    line["refresh_ms"] = None if ref is None else ref["ms_graph"]
+    lossy = detail.get("lossy_frontier")
+    if lossy is not None:
+        best = max((r for r in lossy["points"] if r["method"] != "exact"), key=lambda r: r["speedup"], default=None)
+        line["lossy"] = dict(exact_ms=lossy["exact_inline_ms_per_step"], captured=lossy.get("captured"),
+                             reaches_5x=bool(lossy["reaches_5x"]),
+                             fastest=_pick(best, ("method", "param", "ms_per_step", "speedup", "max_abs_deviation")),
+                             threshold_0p01=_pick(next((r for r in lossy["points"] if r["method"] == "threshold"
+                                                        and r["param"] == 1e-2), None),
+                                                  ("ms_per_step", "speedup", "max_abs_deviation")))
+    cfgs = detail.get("configs")
+    if cfgs is not None:
+        out = {}
+        for name, c in cfgs.items():
+            if "densities" in c:                      # a network configuration
+                for p, r in c["densities"].items():
+                    d = r["dominant"]
+                    out["%s@%s" % (name, p)] = dict(ms_per_step=r["ms_per_step"], frac=d["frac"], bound=d["bound"],
+                                                    kernel=d["kernel"], us=d["us"])
+                out[name + "@dense"] = c.get("dense_same_kernels_ms")
+            elif "delta_only" in c:                   # the single conv
+                for form in ("delta_only", "fused_reservoir_relu"):
+                    out["%s/%s" % (name, form)] = dict(us=c[form]["us"], frac=c[form]["hbm_frac"], bound="hbm",
+                                                       kernel="mie_conv_masked 3x3 s1 32->32 @264x352")
+            else:                                      # the activation chain, one entry per density
+                for p, r in c.items():
+                    if isinstance(r, dict):
+                        out["%s@%s" % (name, p)] = dict(us=r["us_per_step"], frac=r["hbm_frac"], bound="hbm",
+                                                        kernel="conv3x3 64->64 + LeakyReLU + ReLU increments")
+        out["note"] = "c1/c2: us per call from a replayed HIP graph of 48-50 identical calls (kernel time, not host call rate)"
+        line["configs"] = out
+    line["output_check"] = _pick(detail.get("output_check"), ("max_abs_diff", "frames", "against"))
+    line["oracle_check"] = detail.get("oracle_check")
+    line["detail_file"] = detail_file
+    text = json.dumps(line)
+    if len(text) > LINE_LIMIT:
+        # never let the line outgrow what the driver keeps: drop the optional parts, largest first
+        for key in ("configs", "lossy", "whole_frame", "density_sweep_ms", "output_check"):
+            line[key] = None
+            text = json.dumps(line)
+            if len(text) <= LINE_LIMIT:
+                break
+    return text
 
 
 if __name__ == "__main__":
