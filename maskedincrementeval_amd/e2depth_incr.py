@@ -309,6 +309,8 @@ class ConvLSTMIncr(nn.Module, _IncrBuffers):
         return hidden, cell
 
     def forward_refresh_reservoirs(self, input_, prev_state):
+        """Dense (hidden, cell).  With fused=True both are views of buffers this module owns and the next refresh
+        overwrites them in place (the reference returns fresh tensors): clone what must outlive it."""
         batch_size = input_.data.size()[0]
         spatial_size = input_.data.size()[2:]
         if prev_state is None:
@@ -323,6 +325,9 @@ class ConvLSTMIncr(nn.Module, _IncrBuffers):
             tuple([batch_size, self.hidden_size] + list(spatial_size)) + (input_.dtype,))
         prev_h, prev_c = prev_state
         self._reset_incr()
+        # buffer ownership of the two state sets is told by raw addresses: forget them here, so that an address the
+        # allocator has reused since (a shape or device change frees the old buffers) cannot be mistaken for one
+        self.__dict__.pop("_slot_ptrs", None)
         if self.Gates.use_kf:
             self.Gates.kf.forward_refresh_reservoirs(input_)
         # the concat is never formed: two-pointer conv input, hidden half skipped when it is zero

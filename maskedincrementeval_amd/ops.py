@@ -542,8 +542,10 @@ def _tconv2x_args(x, x2, filt, k, out_ts, block_ts, out, addend, reservoir):
     if x2 is not None and (x2.shape[0] != n or x2.shape[2:] != x.shape[2:] or x2.dtype != x.dtype):
         raise ValueError("x2 %s incompatible with x %s" % (tuple(x2.shape), tuple(x.shape)))
     # fp32 deltas in the three-term bf16 form where the setting asks for it and the channel counts are whole chunks of 64
+    # (the same conditions under which ConvFilter.for_dtype hands out the three-term copy: else the fp32 copy and code)
     x3 = (x.dtype == torch.float32 and isinstance(filt, ConvFilter) and f32_matmul == "bf16x3"
-          and c1 % 64 == 0 and c2 % 64 == 0 and filt.shape[3] % 32 == 0)
+          and c1 % 64 == 0 and c2 % 64 == 0 and filt.shape[3] % 32 == 0
+          and filt.plain.is_cuda and filt.plain.shape[0] % 16 == 0)
     if x3:
         plain, mc = filt.for_dtype(torch.float32, x3=True)
         mc_ptr, code = mc.data_ptr(), _lib.DTYPE_F32_BF16X3

@@ -10,6 +10,7 @@ from maskedincrementeval_amd.synthetic import MovingEdges, gaussian_delta, seed_
 from oracle import mask_oracle as mo
 from tolerances import BF16_RTOL, bf16_atol
 from oracle.evflownet_oracle import EVFlowNetOracle, _ConvGRU
+import mask_chain
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -61,12 +62,13 @@ def _run(decoder, h, w, steps, edges, fuse=True):
         _close(a, b, "refresh")
     gen = MovingEdges(h, w, seed=53) if edges else None
     x = x0.clone()
+    prev_lists, sets_checked = {}, 0
     for step in range(steps):
         if edges:
             d, m = gen.step()
         else:
             d, m = gaussian_delta(1, 4, h, w, 0.05, 0.3, seed=5400 + step)
-        with torch.no_grad():
+        with torch.no_grad(), mask_chain.BuildRecorder() as rec:
             preds = model([_cl(d), None])           # the reference drivers pass no mask
         torch.cuda.synchronize()
         ref = oracle.incr(d)
@@ -75,9 +77,17 @@ def _run(decoder, h, w, steps, edges, fuse=True):
         acc = [a + p[0] for a, p in zip(acc, preds)]
         acc_ref = [a + b for a, b in zip(acc_ref, ref)]
         x = x + d
+        pm = mo.pixel_mask(d.numpy(), 0.0)
         enc0 = model.encoders[0].conv.conv2d._tile_set("out_act" if fuse else "out", 1, h // 2, w // 2, torch.device(DEV))
-        want = mo.tile_list(mo.footprint_conv(mo.pixel_mask(d.numpy(), 0.0), 3, 2, 1))
+        want = mo.tile_list(mo.footprint_conv(pm, 3, 2, 1))
         assert np.array_equal(enc0.active_tiles().cpu().numpy(), want)
+        if fuse:
+            # every tile set of the step in situ (pixel mask, ascending tile list, stale list) against the chained
+            # footprints of the input pixel mask, and the named layers against the chain of the network definition
+            seeds = {model._pix_buf("input", 1, h, w, torch.device(DEV)).data_ptr(): pm}
+            sets_checked += mask_chain.check_recorded_builds(rec.calls, seeds, prev_lists, "step %d" % step)
+            sets_checked += mask_chain.check_evflownet_layers(model, pm, "step %d" % step)
+    assert not fuse or sets_checked >= 30 * steps
     for a, b in zip(acc, acc_ref):
         _close(a, b, "accumulated")
     return model, acc, x
@@ -94,11 +104,24 @@ def test_evflownet_config4_moving_edges_and_dense_identity(decoder):
     # benchmark configuration 4: 1x4x256x256, moving-edge deltas (~3 % density); transposed-conv decoders as the
     # configuration words it, up-sampling decoders as the reference file has them
     model, acc, x = _run(decoder, 256, 256, steps=3, edges=True)
+    _dense_identity(decoder, acc, x)
+
+
+def _dense_identity(decoder, acc, x):
     fresh = seed_module_(MultiResUNetRecurrentIncr(num_bins=4, decoder=decoder), seed=51).to(DEV).eval()
     with torch.no_grad():
         dense = fresh.forward_refresh_reservoirs(_cl(x))
     for a, b in zip(acc, dense):
         _close(a, b.cpu(), "refresh + increments vs dense")
+
+
+@pytest.mark.parametrize("decoder", ["upsample", "transposed"])
+def test_evflownet_config4_100_steps_of_accumulation(decoder):
+    # benchmark configuration 4 as it is worded: 100 moving-edge frames at 1x4x256x256 accumulated into the same
+    # reservoirs; every step and flow scale against the CPU oracle, every tile set of every step against the mask
+    # oracle, and refresh + the 100 increments == dense forward on the accumulated input
+    model, acc, x = _run(decoder, 256, 256, steps=100, edges=True)
+    _dense_identity(decoder, acc, x)
 
 
 def test_evflownet_50_steps_of_accumulation():

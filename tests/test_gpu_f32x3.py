@@ -128,3 +128,86 @@ def test_three_term_dtype_is_refused_where_it_has_no_kernel():
     # the pointwise entry points know two delta types only
     rc = L.mie_mask_from_delta(ops.nhwc_ptr(x, "x"), n, h, w, c, 0.0, ts.pixmask.data_ptr(), _lib.DTYPE_F32_BF16X3, None)
     assert rc != 0
+
+
+def _conv_both_modes(x, wt, k, modes=("native", "bf16x3")):
+    n, cin, h, w = x.shape
+    cout, p = wt.shape[0], k // 2
+    ts = TileMask(n, h, w, DEV)
+    ops.build_mask_tiles(None, None, n, h, w, _lib.FOOT_CONV, k, 1, p, ts)
+    outs = {}
+    old = ops.f32_matmul
+    try:
+        for mode in modes:
+            ops.f32_matmul = mode
+            out = ops.new_nhwc(n, cout, h, w, DEV)
+            ops.conv_masked(_dev(x), None, None, None, _filt(wt), k, 1, p, ts, out, path=_lib.PATH_MFMA, workspace=False)
+            torch.cuda.synchronize()
+            outs[mode] = out.cpu()
+    finally:
+        ops.f32_matmul = old
+    return outs
+
+
+@pytest.mark.parametrize("lo_exp,hi_exp", [(-12, 12), (-30, 30), (-36, -30)])
+def test_error_bound_holds_over_many_decades_of_magnitude(lo_exp, hi_exp):
+    # Inputs and weights whose magnitudes span many decades -- per input channel a scale 10^e on the delta and,
+    # in the first two cases, 10^-e on the weights, so that every channel contributes O(1) products from operands
+    # between 1e-30 and 1e+30; in the last case all operands are tiny (1e-36 .. 1e-30): the second and third bf16
+    # terms of such values (2^-9 and 2^-18 of them) reach the subnormal range.  The error against fp64 must stay
+    # within a few fp32 rounding steps of sum |x||w| for the three-term form exactly as for the fp32 instruction.
+    cin, cout, k, h, w = 64, 64, 3, 24, 24
+    g = torch.Generator().manual_seed(11)
+    exps = torch.linspace(lo_exp, hi_exp, cin, dtype=torch.float64)
+    sx = (10.0 ** exps).view(1, cin, 1, 1)
+    x = (torch.randn(1, cin, h, w, generator=g, dtype=torch.float64) * sx).float()
+    wt = torch.randn(cout, cin, k, k, generator=g, dtype=torch.float64)
+    if hi_exp > 0:
+        wt = wt / sx.view(1, cin, 1, 1)
+    wt = wt.float()
+    assert torch.isfinite(x).all() and torch.isfinite(wt).all()
+    ref = F.conv2d(x.double(), wt.double(), padding=k // 2)
+    bound = F.conv2d(x.double().abs(), wt.double().abs(), padding=k // 2)
+    outs = _conv_both_modes(x, wt, k)
+    rel = {m: ((o.double() - ref).abs() / bound.clamp_min(1e-300)).max().item() for m, o in outs.items()}
+    # (fp32 results below the normal range lose bits in any arithmetic: the tiny case is compared where |ref| is normal)
+    assert rel["native"] < 4e-7 and rel["bf16x3"] < 4e-7, rel
+    assert torch.isfinite(outs["bf16x3"]).all()
+
+
+def test_non_finite_deltas_never_come_out_as_finite_numbers():
+    # The three-term split does not carry non-finite values (inf - inf is NaN), and a value of 3.39e38 or more rounds to
+    # an infinite first term.  What the library guarantees, and this test pins: an output whose window holds such a
+    # value is non-finite in BOTH arithmetic forms (never a finite wrong number), outputs whose windows hold none
+    # are unaffected, and with f32_matmul = "native" the result is what an IEEE fp32 conv gives (inf stays inf).
+    cin, cout, k, h, w = 32, 32, 3, 24, 24
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(1, cin, h, w, generator=g)
+    wt = torch.randn(cout, cin, k, k, generator=g).abs() + 0.1          # positive weights: inf * w = inf, no cancellation
+    clean = _conv_both_modes(x, wt, k)
+    bad = x.clone()
+    bad[0, 3, 5, 7] = float("inf")
+    bad[0, 9, 17, 4] = float("-inf")
+    bad[0, 20, 11, 19] = float("nan")
+    bad[0, 1, 20, 20] = 3.4e38                                            # finite, rounds to an infinite bf16 term
+    touched = torch.zeros(1, 1, h, w)
+    for (y, x_) in ((5, 7), (17, 4), (11, 19), (20, 20)):
+        touched[0, 0, y, x_] = 1
+    touched = (F.max_pool2d(touched, k, 1, k // 2) > 0).expand(1, cout, h, w)
+    outs = _conv_both_modes(bad, wt, k)
+    ieee = F.conv2d(bad, wt, padding=k // 2)
+    for mode in ("native", "bf16x3"):
+        o = outs[mode]
+        assert torch.equal(o[~touched], clean[mode][~touched]), mode + ": outputs away from the non-finite values changed"
+    # native: IEEE propagation, as torch's fp32 conv has it (inf where it has inf, nan where it has nan)
+    nat = outs["native"]
+    assert torch.equal(torch.isnan(nat), torch.isnan(ieee)) and torch.equal(torch.isinf(nat), torch.isinf(ieee))
+    assert torch.equal(nat[torch.isinf(ieee)], ieee[torch.isinf(ieee)])
+    # three-term form: every output the IEEE conv makes non-finite is non-finite (NaN in place of inf is allowed) ...
+    x3 = outs["bf16x3"]
+    assert (~torch.isfinite(x3[~torch.isfinite(ieee)])).all()
+    # ... and so is every output whose window holds the 3.4e38 value, which the fp32 conv still carries
+    near_big = torch.zeros(1, 1, h, w)
+    near_big[0, 0, 20, 20] = 1
+    near_big = (F.max_pool2d(near_big, k, 1, k // 2) > 0).expand(1, cout, h, w)
+    assert (~torch.isfinite(x3[near_big])).all()

@@ -62,10 +62,14 @@ def test_noalloc_matches_workspace_form_on_two_calls(x3):
     torch.cuda.synchronize()
     for case in (big, small):
         _lib.check(lib.mie_conv_masked_ws(*case.args(0, x3), ws.data_ptr(), ws.numel() * 4, _stream()))
+        # no allocation: neither through torch's caching allocator nor behind its back (hipMalloc / hipFree in the
+        # library would move the device's free byte count, which torch's statistics do not see)
         before = torch.cuda.memory_stats(DEV)["allocation.all.allocated"]
+        free_before = torch.cuda.mem_get_info(DEV)[0]
         _lib.check(lib.mie_conv_masked_noalloc(*case.args(1, x3), _stream()))
         torch.cuda.synchronize()
         assert torch.cuda.memory_stats(DEV)["allocation.all.allocated"] == before
+        assert torch.cuda.mem_get_info(DEV)[0] == free_before
         assert torch.equal(case.out[0], case.out[1]), "delta differs from the workspace form"
         assert torch.equal(case.res[0], case.res[1]), "reservoir differs from the workspace form"
         # and both are the conv: against the CPU oracle (fp32: rtol 1e-4, atol 1e-5)
@@ -75,6 +79,34 @@ def test_noalloc_matches_workspace_form_on_two_calls(x3):
         assert torch.allclose(case.res[1].cpu(), res.reservoir, rtol=1e-4, atol=1e-5)
     # the caller workspace was really used by the form compared against (the launches were split)
     assert torch.isfinite(ws[:16 * 16 * 256 * 2]).all()
+
+
+def test_noalloc_runs_under_graph_capture():
+    # the callers it is for: a captured HIP graph may not allocate.  After a warm-up call (which looks the array's
+    # address up) the entry point is captured, replayed three times with the program's own work in between, and
+    # every replay must reproduce the eager result bit for bit.
+    lib = _lib.lib()
+    case = _Case(1, 256, 128, 8, 24, 3, 1, seed=41)
+    _lib.check(lib.mie_conv_masked_noalloc(*case.args(0), _stream()))          # warm-up, eager: the result to match
+    torch.cuda.synchronize()
+    want_out, want_res = case.out[0].clone(), case.res[0].clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        _lib.check(lib.mie_conv_masked_noalloc(*case.args(1), side.cuda_stream))
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info(DEV)[0]
+    with torch.cuda.graph(graph):
+        _lib.check(lib.mie_conv_masked_noalloc(*case.args(1), _stream()))
+    for _ in range(3):
+        case.res[1].copy_(_dev(case.r0_cpu.clone()))       # the reservoir is updated in place: start each replay alike
+        case.out[1].zero_()                                  # (inactive tiles are not written: they stay zero)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(case.out[1], want_out) and torch.equal(case.res[1], want_res)
+    assert torch.cuda.mem_get_info(DEV)[0] >= free_before - (1 << 20)           # (the graph object itself is host-side)
 
 
 def test_noalloc_rejects_outputs_beyond_its_workspace():
