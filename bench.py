@@ -840,7 +840,6 @@ def main():
     except OSError as e:
         log("could not write %s: %s" % (args.detail_file, e))
         args.detail_file = None
-    log("detail: " + json.dumps({k: detail[k] for k in ("configs", "lossy_frontier", "density_sweep", "refresh")}))
     print(compact_line(detail, args.detail_file))
 
 

@@ -156,6 +156,33 @@ int mie_build_mask_tiles(const uint8_t* in_mask, const uint8_t* in_mask2,
                          int pad, const mie_tileset* out, void* stream);
 
 /*
+ * A sequence of mie_build_mask_tiles calls as one launch: the tile sets of a whole network, whose structural
+ * masks are all footprints of footprints of the input pixel mask.  ops[i] holds the arguments of the i-th call;
+ * the result -- every out[i].pixmask, flags, tiles, stale, counts -- is what the n_ops calls would leave when
+ * issued in order on the stream.  An in_mask / in_mask2 that is the pixmask of an earlier op's `out` is taken
+ * from that op (the chain never goes through memory); any other is read from memory once.  All ops share one
+ * batch size out.n.  One workgroup per sample walks the chain on bitmaps in LDS; with one sample and at most 4096
+ * tiles per set that is the only launch, otherwise a second kernel ranks all the lists.
+ * Limits: conv footprints of stride 1 or 2, transposed-conv footprints of stride 2 (MIE_ERR_UNSUPPORTED
+ * otherwise); ops plus masks read from memory <= MIE_PLAN_MAX_STEPS, and the masks alive at one time must fit the
+ * LDS of a workgroup as bitmaps (MIE_ERR_CAPACITY: split the plan, or fall back to mie_build_mask_tiles).  ops is
+ * host memory, read during the call only.
+ * Replaces: nothing in the reference, which propagates no masks (every module returns None in the mask slot,
+ * incr_modules/mask_incr_modules.py:41,103,178); the mask definitions are those of mie_build_mask_tiles
+ * (incr_modules/utils.py:22-25, utils/str_sparse_utils.py:10-11).
+ */
+#define MIE_PLAN_MAX_STEPS 40
+typedef struct mie_plan_op {
+  const uint8_t* in_mask;    /* as in mie_build_mask_tiles (NULL = every input pixel active) */
+  const uint8_t* in_mask2;
+  int32_t h_in, w_in;
+  int32_t foot, k, stride, pad;
+  mie_tileset out;
+} mie_plan_op;
+
+int mie_build_mask_plan(const mie_plan_op* ops, int n_ops, void* stream);
+
+/*
  * Re-order a fp32 [cin][k][k][cout] filter into the layout the matrix-core
  * kernels stream, so that the k-steps a lane multiplies per tap come as one
  * 16-byte load:

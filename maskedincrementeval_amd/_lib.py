@@ -37,8 +37,9 @@ EXPORTS = (
     "mie_maxpool_incr", "mie_accumulate", "mie_scale_incr", "mie_avgpool_incr", "mie_linear_incr", "mie_upconv_masked",
     "mie_conv_masked_ws", "mie_convgru_gates_incr", "mie_upsample2x_pair_incr", "mie_conv_masked_noalloc",
     "mie_convlstm_gates_refresh", "mie_convgru_gates_refresh", "mie_mul_dense", "mie_tconv2x_masked",
-    "mie_tconv2x_refresh", "mie_conv_f32x3_takes",
+    "mie_tconv2x_refresh", "mie_conv_f32x3_takes", "mie_build_mask_plan",
 )
+PLAN_MAX_STEPS = 40
 
 
 class MieTileSet(ctypes.Structure):
@@ -47,6 +48,16 @@ class MieTileSet(ctypes.Structure):
         ("n", ctypes.c_int32), ("h", ctypes.c_int32), ("w", ctypes.c_int32),
         ("pixmask", ctypes.c_void_p), ("tiles", ctypes.c_void_p), ("stale", ctypes.c_void_p),
         ("counts", ctypes.c_void_p), ("flags", ctypes.c_void_p),
+    ]
+
+
+class MiePlanOp(ctypes.Structure):
+    """struct mie_plan_op of include/mie.h: the arguments of one mie_build_mask_tiles call."""
+    _fields_ = [
+        ("in_mask", ctypes.c_void_p), ("in_mask2", ctypes.c_void_p),
+        ("h_in", ctypes.c_int32), ("w_in", ctypes.c_int32),
+        ("foot", ctypes.c_int32), ("k", ctypes.c_int32), ("stride", ctypes.c_int32), ("pad", ctypes.c_int32),
+        ("out", MieTileSet),
     ]
 
 
@@ -74,6 +85,8 @@ def _declare(l):
     l.mie_mask_from_delta.argtypes = [vp, ci, ci, ci, ci, cf, vp, ci, vp]
     l.mie_build_mask_tiles.restype = ci
     l.mie_build_mask_tiles.argtypes = [vp, vp, ci, ci, ci, ci, ci, ci, tsp, vp]
+    l.mie_build_mask_plan.restype = ci
+    l.mie_build_mask_plan.argtypes = [ctypes.POINTER(MiePlanOp), ci, vp]
     l.mie_conv_masked.restype = ci
     l.mie_conv_masked.argtypes = [vp, vp, ci, vp, vp, ci, ci, ci, vp, vp, ci, ci, ci, ci, ci, tsp, vp,
                                   vp, vp, ci, cf, ci, ci, vp]

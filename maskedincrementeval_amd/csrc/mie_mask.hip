@@ -282,11 +282,9 @@ __device__ void compact_lists(const BuildArgs& a, FlagFn flag, int chunk, int ba
   }
 }
 
-__global__ __launch_bounds__(COMPACT_THREADS) void k_compact_tiles(BuildArgs a) {
-  __shared__ int s_tot[2 * COMPACT_WAVES * COMPACT_ITEMS];
-  __shared__ int s_base[2 * COMPACT_WAVES];
+// One chunk of the compaction of a tile set: block `chunk` of `nchunks`.
+__device__ void compact_chunk(const BuildArgs& a, int chunk, int nchunks, int* s_tot, int* s_base) {
   const uint32_t* flags = a.flags;
-  const int chunk = blockIdx.x;
   // base = number of active / stale tiles below this chunk (its start is a multiple of 4096 flags)
   int na = 0, ns = 0;
   const uint4* f4 = reinterpret_cast<const uint4*>(flags);
@@ -306,7 +304,13 @@ __global__ __launch_bounds__(COMPACT_THREADS) void k_compact_tiles(BuildArgs a) 
 #pragma unroll
     for (int wv = 0; wv < COMPACT_WAVES; ++wv) base_act += s_base[wv], base_st += s_base[COMPACT_WAVES + wv];
   }
-  compact_lists(a, [&](int t) { return flags[t]; }, chunk, base_act, base_st, chunk == (int)gridDim.x - 1, s_tot);
+  compact_lists(a, [&](int t) { return flags[t]; }, chunk, base_act, base_st, chunk == nchunks - 1, s_tot);
+}
+
+__global__ __launch_bounds__(COMPACT_THREADS) void k_compact_tiles(BuildArgs a) {
+  __shared__ int s_tot[2 * COMPACT_WAVES * COMPACT_ITEMS];
+  __shared__ int s_base[2 * COMPACT_WAVES];
+  compact_chunk(a, blockIdx.x, (int)gridDim.x, s_tot, s_base);
 }
 
 // Planes of at most SMALL_CAP tiles (the 33x44 plane of a 264x352 frame: 30 tiles): footprint
@@ -391,4 +395,718 @@ extern "C" int mie_build_mask_tiles(const uint8_t* in_mask, const uint8_t* in_ma
   hipLaunchKernelGGL(k_compact_tiles, dim3((unsigned)mie_div_up(a.cap, COMPACT_CHUNK)), dim3(COMPACT_THREADS), 0,
                      (hipStream_t)stream, a);
   return mie_check_launch("mie_build_mask_tiles");
+}
+
+// ---- every tile set of a network in two launches ------------------------------------------------
+// mie_build_mask_plan runs a sequence of mie_build_mask_tiles calls -- every structural mask of a network is a chain
+// of footprints of the input pixel mask -- as two kernels.  In the first, a workgroup keeps the pixel masks of one
+// sample's chain as BITMAPS in LDS (a 264x352 plane is 11.6 KB): a footprint is then a handful of word operations
+// per 32 pixels -- the window of a conv is the OR of the rows it covers, shifted left and right (stride 2: the even
+// bits of that, compressed); bilinear x2 and the stride-2 transposed conv interleave two such ORs bit by bit --
+// instead of k*k byte loads per pixel, and no launch or memory round trip separates one mask of the chain from the
+// next.  That part is so cheap that several workgroups per sample each walk the whole chain on their own and share
+// only what goes to memory: of every set's pixel mask (bytes, 16 per store where the rows allow it) and tile flags a
+// workgroup writes its slice, so the stores of a large plane do not queue up behind one CU.  The second kernel
+// ranks the lists of all sets, one block per 4096 tiles of each (as k_compact_tiles).  Slots of LDS are handed out
+// on the host by lifetime (a mask is dropped after its last reader).
+namespace {
+
+constexpr int PLAN_THREADS = COMPACT_THREADS;
+constexpr int PLAN_MAX_SHARES = 64;                    // workgroups per sample
+constexpr int PLAN_PIXELS_PER_SHARE = 8192;            // of the plan's largest plane: 128 tiles, so a thread owns at most one
+constexpr int PLAN_STEP_LOAD = 0, PLAN_STEP_FOOT = 1;
+constexpr int PLAN_IN_NONE = -1, PLAN_IN_ALL = -2;
+
+struct PlanStep {
+  int kind;                 // PLAN_STEP_LOAD: bytes -> bitmap; PLAN_STEP_FOOT: footprint of one or two bitmaps
+  int in1, in2;             // LDS word offsets of the input bitmaps (PLAN_IN_*)
+  int out;                  // LDS word offset of the bitmap this step makes
+  int h_in, w_in, h_out, w_out;
+  int geom;                 // foot | k << 8 | stride << 16 | pad << 24
+  int flag_off, flag_cnt;   // this step's part of the workgroup's flag area in LDS: first word, words
+  int key;                  // which specialised form of the footprint runs (PLAN_KEY_*), chosen on the host
+  unsigned m_words, m_units, m_tiles;   // plan_magic of the words per row, the 16-pixel units per row, the tiles per row
+  int pad_;
+  const uint8_t* ext;       // LOAD: the mask in memory, [n, h_out, w_out]
+  uint8_t* pixmask;
+  uint32_t* flags;
+};
+
+struct PlanArgs {
+  int n_steps, n, flag_words, pad1_;
+#ifdef MIE_PLAN_PROFILE
+  int* dbg;                // measurement builds only: 2 ticks per step
+#endif
+  PlanStep st[MIE_PLAN_MAX_STEPS];
+};
+constexpr int PLAN_HEAD = MIE_PLAN_MAX_STEPS * (int)(sizeof(PlanStep) / 4);     // words of LDS in front of the bitmaps: the steps
+
+// a step's fields, read from LDS (the same address in every lane), as scalars
+__device__ __forceinline__ int plan_uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
+template <typename P>
+__device__ __forceinline__ P* plan_uni(P* p) {
+  const unsigned long long v = reinterpret_cast<unsigned long long>(p);
+  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)v), hi = __builtin_amdgcn_readfirstlane((unsigned)(v >> 32));
+  return reinterpret_cast<P*>(((unsigned long long)hi << 32) | lo);
+}
+__device__ __forceinline__ PlanStep plan_uni(const PlanStep& s) {
+  PlanStep u;
+  u.kind = plan_uni(s.kind); u.in1 = plan_uni(s.in1); u.in2 = plan_uni(s.in2); u.out = plan_uni(s.out);
+  u.h_in = plan_uni(s.h_in); u.w_in = plan_uni(s.w_in); u.h_out = plan_uni(s.h_out); u.w_out = plan_uni(s.w_out);
+  u.geom = plan_uni(s.geom); u.flag_off = plan_uni(s.flag_off); u.flag_cnt = plan_uni(s.flag_cnt); u.key = plan_uni(s.key);
+  u.m_words = (unsigned)plan_uni((int)s.m_words); u.m_units = (unsigned)plan_uni((int)s.m_units);
+  u.m_tiles = (unsigned)plan_uni((int)s.m_tiles); u.pad_ = 0;
+  u.ext = plan_uni(s.ext); u.pixmask = plan_uni(s.pixmask); u.flags = plan_uni(s.flags);
+  return u;
+}
+
+// bit x of the result = bit (x + t) of the row whose words around the current one are prev, cur, next (|t| < 32):
+// 32 bits out of the middle of two adjacent words (v_alignbit_b32), no branch on the sign of t
+__device__ __forceinline__ uint32_t plan_shift(uint32_t prev, uint32_t cur, uint32_t next, int t) {
+  const uint32_t hi = t >= 0 ? next : cur, lo = t >= 0 ? cur : prev;
+  return __builtin_amdgcn_alignbit(hi, lo, (uint32_t)t & 31u);
+}
+// bits 0, 2, 4, ... of x packed into the low half
+__device__ __forceinline__ uint32_t plan_even_bits(uint32_t x) {
+  x &= 0x55555555u;
+  x = (x | (x >> 1)) & 0x33333333u;
+  x = (x | (x >> 2)) & 0x0f0f0f0fu;
+  x = (x | (x >> 4)) & 0x00ff00ffu;
+  x = (x | (x >> 8)) & 0x0000ffffu;
+  return x;
+}
+// bit i of the low half of x moved to bit 2i
+__device__ __forceinline__ uint32_t plan_spread(uint32_t x) {
+  x &= 0x0000ffffu;
+  x = (x | (x << 8)) & 0x00ff00ffu;
+  x = (x | (x << 4)) & 0x0f0f0f0fu;
+  x = (x | (x << 2)) & 0x33333333u;
+  x = (x | (x << 1)) & 0x55555555u;
+  return x;
+}
+// four mask bytes -> four bits (a byte counts when it is not zero)
+__device__ __forceinline__ uint32_t plan_nibble(uint32_t v) {
+  const uint32_t t = (v | ((v | 0x80808080u) - 0x01010101u)) & 0x80808080u;     // bit 7 of every non-zero byte
+  return ((t >> 7) & 1u) | ((t >> 14) & 2u) | ((t >> 21) & 4u) | ((t >> 28) & 8u);
+}
+// four bits -> four bytes of 0 / 1
+__device__ __forceinline__ uint32_t plan_bytes(uint32_t nib) {
+  return (nib & 1u) | ((nib & 2u) << 7) | ((nib & 4u) << 14) | ((nib & 8u) << 21);
+}
+
+// The input of a step: one bitmap, or (TWO) the OR of two.  Every load below goes out unconditionally from a clamped
+// address and is masked afterwards, so that the loads of a whole window are in flight together instead of one row
+// after the other.
+template <bool TWO>
+struct PlanRowAcc {
+  const uint32_t* b1;
+  const uint32_t* b2;
+  int ww, h;
+  __device__ __forceinline__ uint32_t at(int y, int j) const {
+    return TWO ? (b1[y * ww + j] | b2[y * ww + j]) : b1[y * ww + j];
+  }
+  // row y if it exists, else all zeros: (clamped row, mask)
+  __device__ __forceinline__ int row(int y, uint32_t& m) const {
+    const bool ok = y >= 0 && y < h;
+    m = ok ? 0xffffffffu : 0u;
+    return ok ? y : 0;
+  }
+};
+
+// One output word of a footprint step: pixels 32*j .. 32*j+31 of row oy.  K = 0: kernel size read at run time.
+struct PlanGeom { int k, p; };
+template <int FOOT, int K, int S, bool TWO>
+__device__ __forceinline__ uint32_t plan_foot_word(const PlanGeom& g, const PlanRowAcc<TWO>& in, int oy, int j) {
+  // kernel size and padding: compile-time constants for the common footprints (K > 0: "same" padding K / 2)
+  const PlanGeom s = {K > 0 ? K : g.k, K > 0 ? K / 2 : g.p};
+  const int k = s.k;
+  const int ww = in.ww, h = in.h;
+  if (FOOT == MIE_FOOT_CONV && S == 1) {
+    const int lo = -s.p;
+    const bool okp = j > 0, okc = j < ww, okn = j + 1 < ww;
+    const int jp = okp ? j - 1 : 0, jc = okc ? j : 0, jn = okn ? j + 1 : 0;
+    uint32_t vp = 0u, vc = 0u, vn = 0u;
+#pragma unroll
+    for (int ky = 0; ky < k; ++ky) {
+      uint32_t m;
+      const int iy = in.row(oy - s.p + ky, m);
+      vp |= in.at(iy, jp) & m;
+      vc |= in.at(iy, jc) & m;
+      vn |= in.at(iy, jn) & m;
+    }
+    vp = okp ? vp : 0u; vc = okc ? vc : 0u; vn = okn ? vn : 0u;
+    uint32_t r = 0u;
+#pragma unroll
+    for (int t = 0; t < k; ++t) r |= plan_shift(vp, vc, vn, lo + t);
+    return r;
+  }
+  if (FOOT == MIE_FOOT_CONV) {
+    // stride 2: the window OR at input positions 64*j .. 64*j+63, of which the even ones are the outputs
+    const int lo = -s.p;
+    const int j0 = 2 * j - 1;
+    bool ok[4];
+    int jj[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      ok[q] = j0 + q >= 0 && j0 + q < ww;
+      jj[q] = ok[q] ? j0 + q : 0;
+    }
+    uint32_t v[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int ky = 0; ky < k; ++ky) {
+      uint32_t m;
+      const int iy = in.row(2 * oy - s.p + ky, m);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) v[q] |= in.at(iy, jj[q]) & m;
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) v[q] = ok[q] ? v[q] : 0u;
+    uint32_t d0 = 0u, d1 = 0u;
+#pragma unroll
+    for (int t = 0; t < k; ++t) {
+      d0 |= plan_shift(v[0], v[1], v[2], lo + t);
+      d1 |= plan_shift(v[1], v[2], v[3], lo + t);
+    }
+    return plan_even_bits(d0) | (plan_even_bits(d1) << 16);
+  }
+  const int js = j >> 1, sh = 16 * (j & 1);
+  const bool okp = js > 0, okc = js < ww, okn = js + 1 < ww;
+  const int jp = okp ? js - 1 : 0, jc = okc ? js : 0, jn = okn ? js + 1 : 0;
+  uint32_t vp = 0u, vc = 0u, vn = 0u;
+  if (FOOT == MIE_FOOT_UP2X) {
+    // out[2m] = in[m-1] | in[m], out[2m+1] = in[m] | in[m+1], rows and columns alike (clamping at the border adds
+    // nothing: the clamped neighbour is the pixel itself)
+    int r0, r1;
+    up2x_src(oy, h, r0, r1);
+    vp = in.at(r0, jp) | in.at(r1, jp);
+    vc = in.at(r0, jc) | in.at(r1, jc);
+    vn = in.at(r0, jn) | in.at(r1, jn);
+    vp = okp ? vp : 0u; vc = okc ? vc : 0u; vn = okn ? vn : 0u;
+    const uint32_t ev = vc | plan_shift(vp, vc, vn, -1), od = vc | plan_shift(vp, vc, vn, 1);
+    return plan_spread(ev >> sh) | (plan_spread(od >> sh) << 1);
+  }
+  // MIE_FOOT_TCONV, stride 2: output 2m + e sees input m + (e + p - kk) / 2 for the taps kk with e + p - kk even
+  const int e = oy & 1, m_ = oy >> 1;
+#pragma unroll
+  for (int ky = 0; ky < k; ++ky) {
+    const int d2 = e + s.p - ky;
+    uint32_t m;
+    const int iy = in.row(m_ + (d2 >> 1), m);
+    m = (d2 & 1) ? 0u : m;
+    vp |= in.at(iy, jp) & m;
+    vc |= in.at(iy, jc) & m;
+    vn |= in.at(iy, jn) & m;
+  }
+  vp = okp ? vp : 0u; vc = okc ? vc : 0u; vn = okn ? vn : 0u;
+  uint32_t ev = 0u, od = 0u;
+#pragma unroll
+  for (int kx = 0; kx < k; ++kx) {
+    const int d2 = s.p - kx;
+    if (d2 & 1) od |= plan_shift(vp, vc, vn, (d2 + 1) >> 1);
+    else ev |= plan_shift(vp, vc, vn, d2 >> 1);
+  }
+  return plan_spread(ev >> sh) | (plan_spread(od >> sh) << 1);
+}
+
+// floor(a / d) with m = plan_magic(d) = ceil(2^32 / d) worked out on the host: one multiply instead of a division by a
+// run-time value.  Exact while a * d < 2^32 (the excess of m over 2^32 / d is below one, so the quotient is off by less
+// than a / 2^32 < 1 / d); the planes of a plan are held to 2^20 pixels per sample and 2^11 per row for that.  d = 1
+// has no 32-bit magic number: a itself, by a select.
+inline unsigned plan_magic(int d) { return d <= 1 ? 0u : (unsigned)(0xffffffffu / (unsigned)d + 1u); }
+__device__ __forceinline__ int plan_div(int a, unsigned m) {
+  const int q = (int)__umulhi((unsigned)a, m);
+  return m == 0u ? a : q;
+}
+
+// Threads of a workgroup by role: the first PLAN_COMPUTE make the bitmap of a step while PLAN_PIX others write the
+// pixel mask of the step before it and the last PLAN_FLG its tile flags, so that none waits for another's
+// instruction stream: a step is a few hundred instructions of each kind and nothing else to hide them behind.
+constexpr int PLAN_COMPUTE = 640;
+constexpr int PLAN_PIX = 192;
+constexpr int PLAN_FLG = PLAN_THREADS - PLAN_COMPUTE - PLAN_PIX;
+
+// specialised forms of the footprint (kernel size, stride and "same" padding K / 2 at compile time)
+enum { PLAN_KEY_GENERIC = 0, PLAN_KEY_C11, PLAN_KEY_C31, PLAN_KEY_C51, PLAN_KEY_C32, PLAN_KEY_C52, PLAN_KEY_UP, PLAN_KEY_T32, PLAN_KEY_T52 };
+
+// the bitmap of a footprint step: compute thread r of nthr takes words r, r + nthr, ...
+template <int FOOT, int K, int S, bool TWO>
+__device__ __forceinline__ void plan_foot_all(const PlanStep& s, const uint32_t* bm, uint32_t* out, int r, int nthr) {
+  PlanRowAcc<TWO> in;
+  in.b1 = bm + s.in1;
+  in.b2 = bm + ((TWO && s.in2 >= 0) ? s.in2 : s.in1);
+  in.ww = (s.w_in + 31) >> 5;
+  in.h = s.h_in;
+  const int ho = s.h_out, wo = s.w_out, wwo = (wo + 31) >> 5;
+  PlanGeom g;
+  g.k = (s.geom >> 8) & 255; g.p = (s.geom >> 24) & 255;
+  for (int wd = r; wd < ho * wwo; wd += nthr) {
+    const int y = plan_div(wd, s.m_words), j = wd - y * wwo;
+    const int left = wo - 32 * j;
+    const uint32_t valid = left >= 32 ? 0xffffffffu : ((1u << left) - 1u);
+    out[wd] = plan_foot_word<FOOT, K, S, TWO>(g, in, y, j) & valid;
+  }
+}
+template <int FOOT, int K, int S>
+__device__ __forceinline__ void plan_foot_any(const PlanStep& s, const uint32_t* bm, uint32_t* out, int r, int nthr) {
+  if (s.in2 >= 0) plan_foot_all<FOOT, K, S, true>(s, bm, out, r, nthr);
+  else plan_foot_all<FOOT, K, S, false>(s, bm, out, r, nthr);
+}
+
+__device__ void plan_compute(const PlanStep& s, const uint32_t* bm, uint32_t* out, int r, int nthr) {
+  const int ho = s.h_out, wo = s.w_out, wwo = (wo + 31) >> 5;
+  if (s.in1 == PLAN_IN_ALL) {
+    for (int wd = r; wd < ho * wwo; wd += nthr) {
+      const int j = wd - plan_div(wd, s.m_words) * wwo;
+      const int left = wo - 32 * j;
+      out[wd] = left >= 32 ? 0xffffffffu : ((1u << left) - 1u);
+    }
+    return;
+  }
+  switch (s.key) {       // uniform over the workgroup
+    case PLAN_KEY_C11: plan_foot_any<MIE_FOOT_CONV, 1, 1>(s, bm, out, r, nthr); break;
+    case PLAN_KEY_C31: plan_foot_any<MIE_FOOT_CONV, 3, 1>(s, bm, out, r, nthr); break;
+    case PLAN_KEY_C51: plan_foot_any<MIE_FOOT_CONV, 5, 1>(s, bm, out, r, nthr); break;
+    case PLAN_KEY_C32: plan_foot_any<MIE_FOOT_CONV, 3, 2>(s, bm, out, r, nthr); break;
+    case PLAN_KEY_C52: plan_foot_any<MIE_FOOT_CONV, 5, 2>(s, bm, out, r, nthr); break;
+    case PLAN_KEY_UP: plan_foot_any<MIE_FOOT_UP2X, 1, 1>(s, bm, out, r, nthr); break;
+    case PLAN_KEY_T32: plan_foot_any<MIE_FOOT_TCONV, 3, 2>(s, bm, out, r, nthr); break;
+    case PLAN_KEY_T52: plan_foot_any<MIE_FOOT_TCONV, 5, 2>(s, bm, out, r, nthr); break;
+    default: {
+      const int foot = s.geom & 255, ss = (s.geom >> 16) & 255;
+      if (foot == MIE_FOOT_TCONV) plan_foot_all<MIE_FOOT_TCONV, 0, 2, true>(s, bm, out, r, nthr);
+      else if (ss == 1) plan_foot_all<MIE_FOOT_CONV, 0, 1, true>(s, bm, out, r, nthr);
+      else plan_foot_all<MIE_FOOT_CONV, 0, 2, true>(s, bm, out, r, nthr);
+    }
+  }
+}
+
+// What a step leaves in memory, from its bitmap `out`.  The pixel mask, as bytes: this workgroup's slice (share of
+// shares), by threads r of nthr.
+__device__ void plan_write_pixels(const PlanStep& s, const uint32_t* out, int n, int share, int shares, int r, int nthr) {
+  const int ho = s.h_out, wo = s.w_out, wwo = (wo + 31) >> 5;
+  const int first = share * nthr + r, stride = shares * nthr;
+  uint8_t* pm = s.pixmask + (long long)n * ho * wo;
+  if ((wo & 15) == 0) {
+    const int per_row = wo >> 4, units = ho * per_row;
+    for (int u = first; u < units; u += stride) {
+      const int y = plan_div(u, s.m_units), q = u - y * per_row;
+      const uint32_t b16 = out[y * wwo + (q >> 1)] >> (16 * (q & 1));
+      const uint4 v = make_uint4(plan_bytes(b16 & 15u), plan_bytes((b16 >> 4) & 15u), plan_bytes((b16 >> 8) & 15u),
+                                 plan_bytes((b16 >> 12) & 15u));
+      *reinterpret_cast<uint4*>(pm + (long long)y * wo + 16 * q) = v;
+    }
+  } else if ((wo & 3) == 0) {
+    const int per_row = wo >> 2, units = ho * per_row;
+    for (int u = first; u < units; u += stride) {
+      const int y = plan_div(u, s.m_units), q = u - y * per_row;
+      const uint32_t nib = (out[y * wwo + (q >> 3)] >> (4 * (q & 7))) & 15u;
+      *reinterpret_cast<uint32_t*>(pm + (long long)y * wo + 4 * q) = plan_bytes(nib);
+    }
+  } else {
+    for (int u = first; u < ho * wo; u += stride) {
+      const int y = plan_div(u, s.m_units), x = u - y * wo;
+      pm[u] = (uint8_t)((out[y * wwo + (x >> 5)] >> (x & 31)) & 1u);
+    }
+  }
+}
+
+// The tile flags: tile (ty, tx) is byte tx % 4 of word tx / 4 in rows 8*ty .. 8*ty+7.  A flag word is written by the one
+// thread that owns its tile -- word f of this step's flag area is tile f * shares + share -- from the old value fetched
+// at the start.
+__device__ void plan_write_flags(const PlanStep& s, const uint32_t* out, const uint32_t* s_old, int n, int share, int shares,
+                                 int r, int nthr) {
+  const int ho = s.h_out, wo = s.w_out, wwo = (wo + 31) >> 5;
+  const int tiles_y = (ho + MIE_TILE - 1) / MIE_TILE, tiles_x = (wo + MIE_TILE - 1) / MIE_TILE;
+  const int tpp = tiles_y * tiles_x;
+  for (int f = r; f < s.flag_cnt; f += nthr) {
+    const int t = f * shares + share;
+    if (t >= tpp) break;
+    const int ty = plan_div(t, s.m_tiles), tx = t - ty * tiles_x;
+    uint32_t any = 0u;
+#pragma unroll
+    for (int q = 0; q < MIE_TILE; ++q) {
+      const int y = ty * MIE_TILE + q;
+      any |= out[(y < ho ? y : ho - 1) * wwo + (tx >> 2)] & (y < ho ? 0xffffffffu : 0u);
+    }
+    s.flags[n * tpp + t] = next_flag(s_old[s.flag_off + f], ((any >> (8 * (tx & 3))) & 0xffu) != 0u);
+  }
+}
+
+__global__ __launch_bounds__(PLAN_THREADS) void k_plan_bits(PlanArgs a) {
+  extern __shared__ __attribute__((aligned(16))) uint32_t plan_lds[];
+  // The steps first go from the argument block to LDS in one batch: read where they are used, every step's fields
+  // would be a cache miss of their own in a chain where nothing else hides it.
+  PlanStep* steps = reinterpret_cast<PlanStep*>(plan_lds);
+  uint32_t* bm = plan_lds + PLAN_HEAD;
+  const int n = blockIdx.y, tid = threadIdx.x;
+  {
+    const uint32_t* src = reinterpret_cast<const uint32_t*>(&a.st[0]);
+    const int nw = a.n_steps * (int)(sizeof(PlanStep) / 4);
+    for (int i = tid; i < nw; i += PLAN_THREADS) plan_lds[i] = src[i];
+  }
+  __syncthreads();
+  // sample blockIdx.y; share blockIdx.x of gridDim.x of everything that is written to memory
+  const int share = blockIdx.x, shares = gridDim.x;
+  // The tile flags this workgroup owns -- tiles share, share + shares, ... of every set -- hold the previous build's
+  // state and are needed when a step is written out.  Asked for step by step, each would be a memory round trip that
+  // nothing hides; so all of them are fetched now, in one batch behind which the first mask's loads queue up, into the
+  // LDS area in front of the bitmaps (word flag_off + f of a step = tile f * shares + share).
+  uint32_t* s_old = bm;
+  bm += a.flag_words;
+  for (int u = tid; u < a.flag_words; u += PLAN_THREADS) {
+    int q = 0;
+    for (int i = 1; i < a.n_steps; ++i)
+      if (steps[i].flag_off <= u) q = i;            // the last step whose area starts at or below u (areas are in step order)
+    const PlanStep& sq = steps[q];
+    const int tpp = ((sq.h_out + MIE_TILE - 1) / MIE_TILE) * ((sq.w_out + MIE_TILE - 1) / MIE_TILE);
+    const int t = (u - sq.flag_off) * shares + share;
+    s_old[u] = (sq.kind == PLAN_STEP_FOOT && t < tpp) ? sq.flags[n * tpp + t] : 0u;
+  }
+  // role of this wave: 0 = bitmaps, 1 = pixel masks, 2 = tile flags (uniform over a wave: the limits are multiples of 64)
+  const int role = tid < PLAN_COMPUTE ? 0 : (tid < PLAN_COMPUTE + PLAN_PIX ? 1 : 2);
+  int pending = -1;                                    // the footprint step that is not written out yet
+  for (int i = 0; i < a.n_steps; ++i) {
+#ifdef MIE_PLAN_PROFILE
+    const long long t_step = wall_clock64();
+#endif
+    const PlanStep s = plan_uni(steps[i]);
+    uint32_t* out = bm + s.out;
+    const int ho = s.h_out, wo = s.w_out, wwo = (wo + 31) >> 5;
+    if (s.kind == PLAN_STEP_LOAD) {
+      const uint8_t* src = s.ext + (long long)n * ho * wo;
+      for (int wd = tid; wd < ho * wwo; wd += PLAN_THREADS) {
+        const int y = plan_div(wd, s.m_words), j = wd - y * wwo;
+        const int x0 = 32 * j, nb = (wo - x0 < 32) ? wo - x0 : 32;
+        const uint8_t* row = src + (long long)y * wo + x0;
+        uint32_t bits = 0u;
+        if ((wo & 15) == 0) {           // rows start on 16-byte boundaries and hold whole groups of 16 pixels
+          const uint4* r16 = reinterpret_cast<const uint4*>(row);
+          const uint4 v0 = r16[0];
+          bits = plan_nibble(v0.x) | (plan_nibble(v0.y) << 4) | (plan_nibble(v0.z) << 8) | (plan_nibble(v0.w) << 12);
+          if (nb > 16) {
+            const uint4 v1 = r16[1];
+            bits |= (plan_nibble(v1.x) | (plan_nibble(v1.y) << 4) | (plan_nibble(v1.z) << 8) | (plan_nibble(v1.w) << 12)) << 16;
+          }
+        } else if ((wo & 3) == 0) {     // 4-byte boundaries
+          const uint32_t* r4 = reinterpret_cast<const uint32_t*>(row);
+          for (int q = 0; q < (nb >> 2); ++q) bits |= plan_nibble(r4[q]) << (4 * q);
+        } else {
+          for (int b = 0; b < nb; ++b) bits |= (row[b] != 0 ? 1u : 0u) << b;
+        }
+        out[wd] = bits;
+      }
+      __syncthreads();
+      continue;
+    }
+    // The compute waves make this step's bitmap while the others put the step before it into memory.  (They read that
+    // step's slot while this step's is written, and the step after this one writes its own one barrier later: the host
+    // keeps all three apart -- a slot is handed on one step after its last reader.)
+    if (role == 0) {
+      plan_compute(s, bm, out, tid, PLAN_COMPUTE);
+    } else if (pending >= 0) {
+      const PlanStep sp = plan_uni(steps[pending]);
+      if (role == 1) plan_write_pixels(sp, bm + sp.out, n, share, shares, tid - PLAN_COMPUTE, PLAN_PIX);
+      else plan_write_flags(sp, bm + sp.out, s_old, n, share, shares, tid - PLAN_COMPUTE - PLAN_PIX, PLAN_FLG);
+    }
+#ifdef MIE_PLAN_PROFILE
+    // measurement builds only: ticks of the 100 MHz clock of this step in workgroup (0, 0), first thread of each role
+    if (blockIdx.x == 0 && n == 0 && (tid == 0 || tid == PLAN_COMPUTE || tid == PLAN_COMPUTE + PLAN_PIX))
+      reinterpret_cast<int32_t*>(a.dbg)[3 * i + role] = (int)(wall_clock64() - t_step);
+#endif
+    __syncthreads();
+    pending = i;
+  }
+  if (pending >= 0) {       // the last step, by everybody
+    const PlanStep sp = plan_uni(steps[pending]);
+    plan_write_pixels(sp, bm + sp.out, n, share, shares, tid, PLAN_THREADS);
+    plan_write_flags(sp, bm + sp.out, s_old, n, share, shares, tid, PLAN_THREADS);
+  }
+}
+
+// The lists of every set of a plan: block b is chunk b - first_chunk[i] of the compaction of set i (as
+// k_compact_tiles).  The table of first chunks is a few cache lines read in one go; a block then touches only the
+// line of its own set.
+struct PlanCompactSet {
+  int32_t* tiles;
+  int32_t* stale;
+  int32_t* counts;
+  uint32_t* flags;
+  int cap, pad_;
+};
+struct PlanCompactArgs {
+  int n_sets, pad_;
+  int first_chunk[MIE_PLAN_MAX_STEPS + 2];     // first_chunk[n_sets] = number of blocks
+  PlanCompactSet set[MIE_PLAN_MAX_STEPS];
+};
+
+__global__ __launch_bounds__(COMPACT_THREADS) void k_plan_compact(PlanCompactArgs a) {
+  __shared__ int s_tot[2 * COMPACT_WAVES * COMPACT_ITEMS];
+  __shared__ int s_base[2 * COMPACT_WAVES];
+  const int b = blockIdx.x;
+  int i = 0;
+#pragma unroll 1
+  for (int q = 1; q < a.n_sets; ++q)
+    if (a.first_chunk[q] <= b) i = q;
+  const PlanCompactSet& st = a.set[i];
+  BuildArgs ba;
+  ba.cap = st.cap;
+  ba.tiles = st.tiles; ba.stale = st.stale; ba.counts = st.counts; ba.flags = st.flags;
+  compact_chunk(ba, b - a.first_chunk[i], a.first_chunk[i + 1] - a.first_chunk[i], s_tot, s_base);
+}
+
+// Host side: LDS words of a plane's bitmap.
+inline long long plan_words(int h, int w) { return (long long)h * ((w + 31) / 32); }
+
+// First-fit allocator over the bitmap area (word offsets), free blocks kept sorted and coalesced.
+struct PlanArena {
+  struct Blk { long long off, size; };
+  Blk free_[2 * MIE_PLAN_MAX_STEPS + 2];
+  int nfree = 0;
+  long long top = 0;          // high-water mark
+  long long alloc(long long size) {
+    for (int i = 0; i < nfree; ++i)
+      if (free_[i].size >= size) {
+        const long long off = free_[i].off;
+        free_[i].off += size;
+        free_[i].size -= size;
+        if (free_[i].size == 0) {
+          for (int j = i; j + 1 < nfree; ++j) free_[j] = free_[j + 1];
+          --nfree;
+        }
+        return off;
+      }
+    // grow: extend a free block that ends at the top, else start a new one there
+    if (nfree > 0 && free_[nfree - 1].off + free_[nfree - 1].size == top) {
+      const long long off = free_[nfree - 1].off;
+      top = off + size;
+      --nfree;
+      return off;
+    }
+    const long long off = top;
+    top += size;
+    return off;
+  }
+  void release(long long off, long long size) {
+    int i = 0;
+    while (i < nfree && free_[i].off < off) ++i;
+    for (int j = nfree; j > i; --j) free_[j] = free_[j - 1];
+    free_[i] = {off, size};
+    ++nfree;
+    if (i + 1 < nfree && free_[i].off + free_[i].size == free_[i + 1].off) {
+      free_[i].size += free_[i + 1].size;
+      for (int j = i + 1; j + 1 < nfree; ++j) free_[j] = free_[j + 1];
+      --nfree;
+    }
+    if (i > 0 && free_[i - 1].off + free_[i - 1].size == free_[i].off) {
+      free_[i - 1].size += free_[i].size;
+      for (int j = i; j + 1 < nfree; ++j) free_[j] = free_[j + 1];
+      --nfree;
+    }
+  }
+};
+
+// LDS a workgroup may use on the current device, and the opt-in for more than 64 KB of it (once per process).
+int plan_lds_limit(long long need_bytes, const char* who) {
+  static int limit[64];
+  static long long opted[64];
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  MIE_REQUIRE(e == hipSuccess && dev >= 0 && dev < 64, MIE_ERR_LAUNCH, "%s: no current device (%s)", who, hipGetErrorString(e));
+  if (limit[dev] == 0) {
+    int v = 0;
+    e = hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, dev);
+    MIE_REQUIRE(e == hipSuccess && v > 0, MIE_ERR_LAUNCH, "%s: cannot read the LDS size of device %d (%s)", who, dev, hipGetErrorString(e));
+    limit[dev] = v;
+  }
+  MIE_REQUIRE(need_bytes <= limit[dev], MIE_ERR_CAPACITY,
+              "%s: the masks of this plan need %lld bytes of LDS at once, the device offers %d per workgroup; "
+              "build the plan in parts, or with mie_build_mask_tiles", who, need_bytes, limit[dev]);
+  if (need_bytes > 65536 && need_bytes > opted[dev]) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(k_plan_bits), hipFuncAttributeMaxDynamicSharedMemorySize, limit[dev]);
+    MIE_REQUIRE(e == hipSuccess, MIE_ERR_CAPACITY, "%s: the device refuses %d bytes of dynamic LDS (%s)", who, limit[dev],
+                hipGetErrorString(e));
+    opted[dev] = limit[dev];
+  }
+  return MIE_OK;
+}
+
+}  // namespace
+
+extern "C" int mie_build_mask_plan(const mie_plan_op* ops, int n_ops, void* stream) {
+  const char* who = "mie_build_mask_plan";
+  mie_clear_error();
+  MIE_REQUIRE(ops != nullptr && n_ops > 0, MIE_ERR_INVALID_ARG, "%s: no ops", who);
+  MIE_REQUIRE(n_ops <= MIE_PLAN_MAX_STEPS, MIE_ERR_CAPACITY, "%s: %d ops, at most %d per call", who, n_ops, MIE_PLAN_MAX_STEPS);
+  PlanArgs a;
+  memset(&a, 0, sizeof(a));
+  a.n = ops[0].out.n;
+  // masks in LDS: pointer -> (slot offset, words, step index of the last reader)
+  struct Slot { const uint8_t* ptr; long long off, words; int h, w, last; };
+  Slot slots[2 * MIE_PLAN_MAX_STEPS];
+  int nslots = 0;
+  // which op reads a mask last (by pointer), so that its slot can be handed on afterwards
+  auto last_reader = [&](const uint8_t* p, int from) {
+    int last = from;
+    for (int j = from; j < n_ops; ++j)
+      if (ops[j].in_mask == p || ops[j].in_mask2 == p) last = j;
+    return last;
+  };
+  auto find_slot = [&](const uint8_t* p) -> Slot* {
+    for (int i = nslots - 1; i >= 0; --i)      // the latest mask at this address
+      if (slots[i].ptr == p) return &slots[i];
+    return nullptr;
+  };
+  PlanArena arena;
+  long long total_chunks = 0, max_pixels = 0, max_tiles = 0;
+  for (int i = 0; i < n_ops; ++i) {
+    const mie_plan_op& op = ops[i];
+    int rc = mie_check_tileset(&op.out, who);
+    if (rc != MIE_OK) return rc;
+    MIE_REQUIRE(op.out.n == a.n, MIE_ERR_INVALID_ARG, "%s: op %d has batch size %d, op 0 has %d", who, i, op.out.n, a.n);
+    MIE_REQUIRE(op.h_in > 0 && op.w_in > 0, MIE_ERR_INVALID_ARG, "%s: op %d: input size (%d,%d) must be positive", who, i,
+                op.h_in, op.w_in);
+    MIE_REQUIRE(op.in_mask != nullptr || op.in_mask2 == nullptr, MIE_ERR_INVALID_ARG, "%s: op %d: in_mask2 given without in_mask", who, i);
+    MIE_REQUIRE((long long)a.n * op.h_in * op.w_in < 0x7fffffffLL, MIE_ERR_CAPACITY, "%s: op %d: more than 2^31 input pixels", who, i);
+    MIE_REQUIRE(op.w_in <= 2048 && op.out.w <= 2048 && (long long)op.h_in * op.w_in <= (1 << 20) &&
+                    (long long)op.out.h * op.out.w <= (1 << 20),
+                MIE_ERR_CAPACITY, "%s: op %d: planes of up to 2048 pixels per row and 2^20 pixels per sample (use mie_build_mask_tiles)", who, i);
+    const int k = op.k, st = op.stride, pad = op.pad;
+    if (op.foot == MIE_FOOT_CONV) {
+      MIE_REQUIRE(k >= 1 && k <= 15 && (st == 1 || st == 2) && pad >= 0 && pad < 16, MIE_ERR_UNSUPPORTED,
+                  "%s: op %d: conv footprint k=%d stride=%d pad=%d (strides 1 and 2 only)", who, i, k, st, pad);
+      const int ho = (op.h_in + 2 * pad - k) / st + 1, wo = (op.w_in + 2 * pad - k) / st + 1;
+      MIE_REQUIRE(op.h_in + 2 * pad >= k && op.w_in + 2 * pad >= k && ho == op.out.h && wo == op.out.w, MIE_ERR_INVALID_ARG,
+                  "%s: op %d: conv output of (%d,%d) k=%d s=%d p=%d is (%d,%d), tile set is (%d,%d)", who, i, op.h_in, op.w_in, k,
+                  st, pad, ho, wo, op.out.h, op.out.w);
+    } else if (op.foot == MIE_FOOT_UP2X) {
+      MIE_REQUIRE(op.out.h == 2 * op.h_in && op.out.w == 2 * op.w_in, MIE_ERR_INVALID_ARG,
+                  "%s: op %d: up2x of (%d,%d) is not (%d,%d)", who, i, op.h_in, op.w_in, op.out.h, op.out.w);
+    } else if (op.foot == MIE_FOOT_TCONV) {
+      MIE_REQUIRE(k >= 1 && k <= 15 && st == 2 && pad >= 0 && pad < 16, MIE_ERR_UNSUPPORTED,
+                  "%s: op %d: tconv footprint k=%d stride=%d pad=%d (stride 2 only)", who, i, k, st, pad);
+      const int hmin = (op.h_in - 1) * st - 2 * pad + k, wmin = (op.w_in - 1) * st - 2 * pad + k;
+      MIE_REQUIRE(op.out.h >= hmin && op.out.h < hmin + st && op.out.w >= wmin && op.out.w < wmin + st, MIE_ERR_INVALID_ARG,
+                  "%s: op %d: tconv output (%d,%d) not in [(%d,%d), +stride)", who, i, op.out.h, op.out.w, hmin, wmin);
+    } else {
+      MIE_REQUIRE(false, MIE_ERR_UNSUPPORTED, "%s: op %d: unknown footprint %d", who, i, op.foot);
+    }
+    // (as in mie_build_mask_tiles: only the identity footprint may be built in place)
+    const bool identity = op.foot == MIE_FOOT_CONV && k == 1 && st == 1 && pad == 0;
+    MIE_REQUIRE(identity || ((const uint8_t*)op.out.pixmask != op.in_mask && (const uint8_t*)op.out.pixmask != op.in_mask2),
+                MIE_ERR_INVALID_ARG, "%s: op %d: out.pixmask aliases an input mask (allowed for the 1x1 stride-1 footprint only)", who, i);
+    // inputs: a mask an earlier op of this plan wrote is still in LDS; any other is loaded from memory first
+    int in_off[2] = {PLAN_IN_NONE, PLAN_IN_NONE};
+    const uint8_t* ins[2] = {op.in_mask, op.in_mask2};
+    if (op.in_mask == nullptr) in_off[0] = PLAN_IN_ALL;
+    for (int q = 0; q < 2 && op.in_mask != nullptr; ++q) {
+      if (ins[q] == nullptr) continue;
+      Slot* sl = find_slot(ins[q]);
+      if (sl == nullptr || sl->last < i) {
+        // not in LDS (never was, or its slot has been handed on): load it
+        MIE_REQUIRE(a.n_steps < MIE_PLAN_MAX_STEPS && nslots < 2 * MIE_PLAN_MAX_STEPS, MIE_ERR_CAPACITY,
+                    "%s: more than %d steps (ops plus masks loaded from memory); build the plan in parts", who, MIE_PLAN_MAX_STEPS);
+        Slot ns;
+        ns.ptr = ins[q]; ns.h = op.h_in; ns.w = op.w_in; ns.words = plan_words(op.h_in, op.w_in);
+        ns.last = last_reader(ins[q], i);
+        // (a later op of the plan may overwrite this address: then the mask in LDS is the old one from there on)
+        for (int j = i; j < ns.last; ++j)
+          if (ops[j].out.pixmask == ins[q]) { ns.last = j; break; }
+        ns.off = arena.alloc(ns.words);
+        PlanStep& ld = a.st[a.n_steps++];
+        ld.kind = PLAN_STEP_LOAD;
+        ld.in1 = ld.in2 = PLAN_IN_NONE;
+        ld.out = (int)ns.off;
+        ld.h_in = ld.h_out = op.h_in; ld.w_in = ld.w_out = op.w_in;
+        ld.m_words = plan_magic((op.w_in + 31) / 32);
+        ld.ext = ins[q];
+        slots[nslots++] = ns;
+        sl = &slots[nslots - 1];
+      }
+      MIE_REQUIRE(sl->h == op.h_in && sl->w == op.w_in, MIE_ERR_INVALID_ARG,
+                  "%s: op %d reads a mask of (%d,%d) as (%d,%d)", who, i, sl->h, sl->w, op.h_in, op.w_in);
+      in_off[q] = (int)sl->off;
+    }
+    if (in_off[0] == PLAN_IN_ALL) in_off[1] = PLAN_IN_NONE;
+    MIE_REQUIRE(a.n_steps < MIE_PLAN_MAX_STEPS && nslots < 2 * MIE_PLAN_MAX_STEPS, MIE_ERR_CAPACITY,
+                "%s: more than %d steps (ops plus masks loaded from memory); build the plan in parts", who, MIE_PLAN_MAX_STEPS);
+    // the output's slot: every input of this op is still alive, so it cannot land on one of them
+    Slot os;
+    os.ptr = op.out.pixmask; os.h = op.out.h; os.w = op.out.w; os.words = plan_words(op.out.h, op.out.w);
+    os.last = last_reader(op.out.pixmask, i);
+    for (int j = i + 1; j < os.last; ++j)
+      if (ops[j].out.pixmask == op.out.pixmask) { os.last = j; break; }      // rewritten before its last reader
+    os.off = arena.alloc(os.words);
+    PlanStep& ft = a.st[a.n_steps++];
+    ft.kind = PLAN_STEP_FOOT;
+    ft.in1 = in_off[0]; ft.in2 = in_off[1];
+    ft.out = (int)os.off;
+    ft.h_in = op.h_in; ft.w_in = op.w_in; ft.h_out = op.out.h; ft.w_out = op.out.w;
+    ft.geom = op.foot | (k << 8) | (st << 16) | (pad << 24);
+    ft.pixmask = op.out.pixmask;
+    ft.flags = op.out.flags;
+    ft.m_words = plan_magic((op.out.w + 31) / 32);
+    ft.m_units = plan_magic(op.out.w % 16 == 0 ? op.out.w / 16 : (op.out.w % 4 == 0 ? op.out.w / 4 : op.out.w));
+    ft.m_tiles = plan_magic(mie_div_up(op.out.w, MIE_TILE));
+    // the specialised forms have kernel size, stride and the padding k / 2 built in
+    ft.key = PLAN_KEY_GENERIC;
+    if (op.foot == MIE_FOOT_UP2X) ft.key = PLAN_KEY_UP;
+    else if (pad == k / 2) {
+      if (op.foot == MIE_FOOT_CONV && st == 1) ft.key = k == 1 ? PLAN_KEY_C11 : k == 3 ? PLAN_KEY_C31 : k == 5 ? PLAN_KEY_C51 : PLAN_KEY_GENERIC;
+      if (op.foot == MIE_FOOT_CONV && st == 2) ft.key = k == 3 ? PLAN_KEY_C32 : k == 5 ? PLAN_KEY_C52 : PLAN_KEY_GENERIC;
+      if (op.foot == MIE_FOOT_TCONV) ft.key = k == 3 ? PLAN_KEY_T32 : k == 5 ? PLAN_KEY_T52 : PLAN_KEY_GENERIC;
+    }
+    slots[nslots++] = os;
+    // Slots whose last reader was the PREVIOUS op are free from here on: one op late, because the kernel has no
+    // barrier between the end of a step (threads still reading its output slot while they write the pixel mask and
+    // the flags) and the compute phase of the next step, which writes that step's output slot.  With the release
+    // delayed, the slot a step writes was last read at least one whole step -- and its barrier -- earlier.
+    for (int q = 0; q < nslots; ++q)
+      if (slots[q].last >= 0 && slots[q].last < i && slots[q].words > 0) {
+        arena.release(slots[q].off, slots[q].words);
+        slots[q].words = 0;
+        slots[q].last = -1;
+      }
+    const int cap = mie_tile_capacity(op.out.n, op.out.h, op.out.w);
+    total_chunks += mie_div_up(cap, COMPACT_CHUNK);
+    if ((long long)op.out.h * op.out.w > max_pixels) max_pixels = (long long)op.out.h * op.out.w;
+    if (cap / op.out.n > max_tiles) max_tiles = cap / op.out.n;
+  }
+  // workgroups per sample: a slice of the largest plane's stores each, and never more than one tile flag per thread
+  long long shares = (max_pixels + PLAN_PIXELS_PER_SHARE - 1) / PLAN_PIXELS_PER_SHARE;
+  if (shares * PLAN_THREADS < max_tiles) shares = (max_tiles + PLAN_THREADS - 1) / PLAN_THREADS;
+  // the flag area of a workgroup: per set, the tiles it owns (every shares-th one)
+  for (int i = 0; i < a.n_steps; ++i) {
+    PlanStep& stp = a.st[i];
+    stp.flag_off = a.flag_words;
+    stp.flag_cnt = 0;
+    if (stp.kind != PLAN_STEP_FOOT) continue;
+    const long long tpp = (long long)mie_div_up(stp.h_out, MIE_TILE) * mie_div_up(stp.w_out, MIE_TILE);
+    stp.flag_cnt = (int)((tpp + shares - 1) / shares);
+    a.flag_words += stp.flag_cnt;
+  }
+  MIE_REQUIRE(shares <= PLAN_MAX_SHARES, MIE_ERR_CAPACITY,
+              "%s: a plane of %lld pixels (%lld tiles) per sample is beyond the plan's %d workgroups per sample; use "
+              "mie_build_mask_tiles", who, max_pixels, max_tiles, PLAN_MAX_SHARES);
+  const long long lds_bytes = (PLAN_HEAD + a.flag_words + arena.top) * 4;
+  int rc = plan_lds_limit(lds_bytes, who);
+  if (rc != MIE_OK) return rc;
+#ifdef MIE_PLAN_PROFILE
+  a.dbg = reinterpret_cast<int*>(ops[n_ops - 1].out.stale) + (mie_tile_capacity(a.n, ops[n_ops - 1].out.h, ops[n_ops - 1].out.w) - 3 * MIE_PLAN_MAX_STEPS);
+#endif
+  hipLaunchKernelGGL(k_plan_bits, dim3((unsigned)shares, (unsigned)a.n), dim3(PLAN_THREADS), (size_t)lds_bytes,
+                     (hipStream_t)stream, a);
+  rc = mie_check_launch(who);
+  if (rc != MIE_OK) return rc;
+  PlanCompactArgs c;
+  memset(&c, 0, sizeof(c));
+  for (int i = 0; i < n_ops; ++i) {
+    const mie_tileset& ts = ops[i].out;
+    PlanCompactSet& st = c.set[c.n_sets];
+    st.tiles = ts.tiles; st.stale = ts.stale; st.counts = ts.counts; st.flags = ts.flags;
+    st.cap = mie_tile_capacity(ts.n, ts.h, ts.w);
+    c.first_chunk[c.n_sets + 1] = c.first_chunk[c.n_sets] + mie_div_up(st.cap, COMPACT_CHUNK);
+    ++c.n_sets;
+  }
+  hipLaunchKernelGGL(k_plan_compact, dim3((unsigned)total_chunks), dim3(COMPACT_THREADS), 0, (hipStream_t)stream, c);
+  return mie_check_launch(who);
 }

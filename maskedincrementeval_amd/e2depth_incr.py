@@ -17,6 +17,8 @@ are deliberate:
 * `BaseE2VID` (an un-vendored dependency of the reference, :4) is replaced
   by a plain config dict on `E2VIDRecurrentIncr`.
 """
+import contextlib
+
 import torch
 import torch.nn as nn
 import torch.nn.functional as F
@@ -722,11 +724,12 @@ class E2VIDRecurrentIncr(nn.Module, _IncrBuffers):
     def forward(self, event_tensor: Masked, prev_states):
         delta = ops.as_nhwc(event_tensor[0])
         mask = _mask_of(event_tensor)
-        if not self.async_masks:
+        if not self.async_masks and not self.plan_first:
             if mask is None and self.derive_input_mask:
                 mask = self.input_mask(delta)
             return self.unetrecurrent.forward([delta, mask], prev_states)
-        with ops.mask_planner(delta.device):
+        # (plan_first without async_masks: the planning pass runs on the compute stream, ahead of the compute pass)
+        with (ops.mask_planner(delta.device) if self.async_masks else contextlib.nullcontext()):
             if mask is None and self.derive_input_mask:
                 mask = self.input_mask(delta)
             if self.plan_first:

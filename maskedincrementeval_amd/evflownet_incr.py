@@ -22,6 +22,8 @@ What differs on purpose:
 * Constructor arguments replace the literals of the reference class
   (`num_bins`, `base_num_channels`, decoder kind), defaults = the reference's.
 """
+import contextlib
+
 import torch
 import torch.nn as nn
 import torch.nn.functional as F
@@ -604,9 +606,10 @@ class MultiResUNetRecurrentIncr(nn.Module, _IncrBuffers):
     def forward(self, x_incr):
         delta = ops.as_nhwc(x_incr[0])
         mask = _mask_of(x_incr)
-        if not self.async_masks:
+        if not self.async_masks and not self.plan_first:
             return self._forward(delta, mask)
-        with ops.mask_planner(delta.device):
+        # (plan_first without async_masks: the planning pass runs on the compute stream, ahead of the compute pass)
+        with (ops.mask_planner(delta.device) if self.async_masks else contextlib.nullcontext()):
             if mask is None and self.derive_input_mask:
                 n, _, h, w = delta.shape
                 mask = ops.mask_from_delta(delta, self.mask_threshold, self._pix_buf("input", n, h, w, delta.device))

@@ -41,6 +41,18 @@ def lib():
     return real if _phase is None else _PhaseLib(real)
 
 
+# The builds of a planning pass are not launched one by one: they are collected and handed to the library as
+# plans (mie_build_mask_plan: the whole chain of footprints on bitmaps in LDS, two kernels per plan).  With
+# `plan_split_first` the first build goes out as a plan of its own -- its tile set is what the first kernel of the
+# compute pass waits for -- and the rest as one plan, or as several where the library says one is too long; a part
+# the library does not take as a plan (a footprint it has no bitmap form for, masks too large for LDS) is built set
+# by set as before.  `fused_plan = False` restores one mie_build_mask_tiles launch pair per set.
+fused_plan = os.environ.get("MIE_FUSED_PLAN", "1") != "0"
+plan_split_first = os.environ.get("MIE_PLAN_SPLIT_FIRST", "0") != "0"
+_plan_batch = None       # [(p1, p2, h_in, w_in, foot, k, stride, pad, out TileMask)] while a planning pass collects
+_plan_cache = {}         # signature of a batch -> [("plan", ctypes array, n) | ("single", index)] parts
+
+
 class network_pass:
     """`with network_pass("plan")` / `with network_pass("compute")`: see above."""
 
@@ -48,14 +60,97 @@ class network_pass:
         self.phase = phase
 
     def __enter__(self):
-        global _phase
+        global _phase, _plan_batch
         self.prev, _phase = _phase, self.phase
+        if self.phase == "plan" and fused_plan:
+            _plan_batch = []
         return self
 
     def __exit__(self, *exc):
-        global _phase
-        _phase = self.prev
+        global _phase, _plan_batch
+        batch, _plan_batch = _plan_batch, None
+        try:
+            if self.phase == "plan" and batch and exc[0] is None:
+                _launch_plan(batch)
+        finally:
+            _phase = self.prev
         return False
+
+
+def _plan_ops(batch):
+    arr = (_lib.MiePlanOp * len(batch))()
+    for op, (p1, p2, h_in, w_in, foot, k, stride, pad, out) in zip(arr, batch):
+        op.in_mask, op.in_mask2, op.h_in, op.w_in = p1, p2, h_in, w_in
+        op.foot, op.k, op.stride, op.pad = foot, k, stride, pad
+        op.out = out.c_struct
+    return arr
+
+
+def _launch_plan(batch):
+    """Enqueue the collected builds: on the planning stream when one is active (with the waits and events a
+    single build would get), else on the current stream."""
+    real = _lib.lib()
+    dev = batch[0][-1].device
+    side = _planner[0] if (_planner is not None and _planner[1] == dev) else None
+    if side is not None:
+        fresh = False
+        for b in batch:
+            root = b[-1].parent if b[-1].parent is not None else b[-1]
+            if not root.__dict__.get("built_once"):
+                root.built_once = fresh = True
+        if fresh:       # freshly allocated tile sets are zero-filled on the compute stream
+            ev0 = torch.cuda.Event()
+            ev0.record(torch.cuda.current_stream(dev))
+            side.wait_event(ev0)
+        for b in batch:
+            for ptr in b[:2]:
+                ev = _pix_ready.get(ptr)
+                if ev is not None:
+                    side.wait_event(ev)
+        stream = side.cuda_stream
+    else:
+        stream = torch.cuda.current_stream(dev).cuda_stream
+    sig = (plan_split_first,) + tuple(b[:8] + (b[8].pixmask.data_ptr(), b[8].tiles.data_ptr()) for b in batch)
+    parts = _plan_cache.get(sig)
+
+    def single(b):
+        p1, p2, h_in, w_in, foot, k, stride, pad, out = b
+        check(real.mie_build_mask_tiles(p1, p2, h_in, w_in, foot, k, stride, pad, out.ref, stream))
+
+    if parts is None:
+        # first use of this batch: find parts the library takes (a refused plan launches nothing)
+        parts = []
+        todo = [(0, 1), (1, len(batch))] if (len(batch) > 1 and plan_split_first) else [(0, len(batch))]
+        while todo:
+            lo, hi = todo.pop(0)
+            if lo >= hi:
+                continue
+            arr = _plan_ops(batch[lo:hi])
+            rc = real.mie_build_mask_plan(arr, hi - lo, stream)
+            if rc == 0:
+                parts.append(("plan", arr, hi - lo, lo))
+            elif rc == -3 and hi - lo > 1:               # MIE_ERR_CAPACITY: too long or too much LDS -- halve it
+                mid = (lo + hi) // 2
+                todo = [(lo, mid), (mid, hi)] + todo
+            elif rc in (-2, -3):                          # no bitmap form for this footprint / plane too large
+                for i in range(lo, hi):
+                    single(batch[i])
+                    parts.append(("single", None, 1, i))
+            else:
+                check(rc)
+        _plan_cache[sig] = parts
+    else:
+        for kind, arr, n_ops, lo in parts:
+            if kind == "plan":
+                check(real.mie_build_mask_plan(arr, n_ops, stream))
+            else:
+                single(batch[lo])
+    if side is not None:
+        ev = torch.cuda.Event()
+        ev.record(side)
+        for b in batch:
+            root = b[-1].parent if b[-1].parent is not None else b[-1]
+            root.ready = ev
 
 
 def _stream(t: torch.Tensor):
@@ -235,6 +330,9 @@ def build_mask_tiles(in_mask, in_mask2, n, h_in, w_in, foot, k, stride, pad, out
     if p1 is None and p2 is not None:   # "all active" OR anything = all active
         p2 = None
     if _phase == "compute":             # built by the planning pass; its event is still attached
+        return out
+    if _phase == "plan" and _plan_batch is not None:
+        _plan_batch.append((p1, p2, h_in, w_in, foot, k, stride, pad, out))
         return out
     if _planner is None or _planner[1] != out.device:
         st = torch.cuda.current_stream(out.device).cuda_stream

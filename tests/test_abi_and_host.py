@@ -146,6 +146,38 @@ def test_invalid_arguments_return_status_not_abort(mie_lib):
     assert mie_lib.mie_tconv_masked(p, None, 4, 9, 9, p, 3, 2, 1, 4, ctypes.byref(ts), p, None, 0, 0.0, 0, None) == -1
 
 
+def test_mask_plan_rejects_what_it_cannot_run(mie_lib):
+    # host-side validation of mie_build_mask_plan: every call below returns before anything is launched
+    err = lambda: mie_lib.mie_last_error_string().decode()
+    ts, keep = _fake_tileset()
+    half, keep_h = _fake_tileset(h=8, w=8)
+    two, keep_2 = _fake_tileset(n=2)
+    buf = ctypes.create_string_buffer(4096)
+    p = (ctypes.addressof(buf) + 15) & ~15
+
+    def plan(*ops_):
+        arr = (_lib.MiePlanOp * max(len(ops_), 1))()
+        for o, (m1, m2, h, w, foot, k, s, pad, out) in zip(arr, ops_):
+            o.in_mask, o.in_mask2, o.h_in, o.w_in, o.foot, o.k, o.stride, o.pad, o.out = m1, m2, h, w, foot, k, s, pad, out
+        return mie_lib.mie_build_mask_plan(arr, len(ops_), None)
+    conv = (p, None, 16, 16, _lib.FOOT_CONV, 3, 1, 1, ts)
+    assert plan() == -1 and "no ops" in err()
+    assert mie_lib.mie_build_mask_plan(None, 3, None) == -1
+    assert plan(*([conv] * (_lib.PLAN_MAX_STEPS + 1))) == -3 and "at most" in err()
+    assert plan((p, None, 16, 16, _lib.FOOT_CONV, 3, 3, 1, ts)) == -2 and "strides 1 and 2" in err()
+    assert plan((p, None, 16, 16, _lib.FOOT_TCONV, 3, 1, 1, ts)) == -2 and "stride 2 only" in err()
+    assert plan((p, None, 16, 16, 9, 3, 1, 1, ts)) == -2 and "unknown footprint" in err()
+    assert plan((p, None, 20, 16, _lib.FOOT_CONV, 3, 1, 1, ts)) == -1 and "tile set is" in err()
+    assert plan((p, None, 16, 16, _lib.FOOT_UP2X, 0, 0, 0, ts)) == -1 and "up2x" in err()
+    assert plan((None, p, 16, 16, _lib.FOOT_CONV, 3, 1, 1, ts)) == -1 and "in_mask2 given without in_mask" in err()
+    assert plan(conv, (p, None, 16, 16, _lib.FOOT_CONV, 3, 1, 1, two)) == -1 and "batch size" in err()
+    assert plan((ts.pixmask, None, 16, 16, _lib.FOOT_CONV, 3, 1, 1, ts)) == -1 and "aliases" in err()
+    # a mask of an earlier op read at another size than it was built with
+    assert plan(conv, (ts.pixmask, None, 15, 15, _lib.FOOT_CONV, 3, 2, 1, half)) == -1 and "reads a mask of" in err()
+    bad, keep_b = _fake_tileset(null="flags")
+    assert plan((p, None, 16, 16, _lib.FOOT_CONV, 3, 1, 1, bad)) == -1
+
+
 def test_check_raises_runtime_error(mie_lib):
     rc = mie_lib.mie_mask_from_delta(None, 1, 4, 4, 4, 0.0, None, 0, None)
     with pytest.raises(RuntimeError, match="NULL pointer"):
@@ -271,7 +303,8 @@ def test_python_constants_mirror_the_header():
     pairs = [("MIE_DTYPE_F32", _lib.DTYPE_F32), ("MIE_DTYPE_BF16", _lib.DTYPE_BF16),
              ("MIE_DTYPE_F32_BF16X3", _lib.DTYPE_F32_BF16X3), ("MIE_PATH_AUTO", _lib.PATH_AUTO),
              ("MIE_PATH_VALU", _lib.PATH_VALU), ("MIE_PATH_MFMA", _lib.PATH_MFMA), ("MIE_FOOT_CONV", _lib.FOOT_CONV),
-             ("MIE_FOOT_UP2X", _lib.FOOT_UP2X), ("MIE_FOOT_TCONV", _lib.FOOT_TCONV)]
+             ("MIE_FOOT_UP2X", _lib.FOOT_UP2X), ("MIE_FOOT_TCONV", _lib.FOOT_TCONV),
+             ("MIE_PLAN_MAX_STEPS", _lib.PLAN_MAX_STEPS)]
     for name, value in pairs:
         assert defs[name] == value, name
 

@@ -165,3 +165,126 @@ def test_out_of_range_counts_are_ignored_by_kernels():
     # a build on top of it recovers a valid list
     ops.build_mask_tiles(None, None, n, h, w, _lib.FOOT_CONV, 1, 1, 0, ts)
     _check_tileset(ts, np.ones((n, h, w), np.uint8))
+
+
+# ---- mie_build_mask_plan: a chain of builds as one launch ----------------------------------------------------
+def _plan_chain(n, h, w):
+    """(name, inputs, foot, k, s, p) of a chain that covers every footprint kind the plan has a bitmap form for: same-size
+    and shrinking convs, strided convs, unions of two masks, an all-active input, bilinear x2, transposed convs of
+    kernel 2 / 3 / 5 at stride 2, an identity footprint, and masks read again long after they were built."""
+    c2 = lambda v, k, p: (v + 2 * p - k) // 2 + 1
+    h2, w2 = c2(h, 5, 2), c2(w, 5, 2)
+    h4, w4 = c2(h2, 3, 1), c2(w2, 3, 1)
+    return [
+        # name     inputs            foot            k  s  p   output plane
+        ("a",      ("x",),           _lib.FOOT_CONV, 5, 1, 2, (h, w)),
+        ("b",      ("a",),           _lib.FOOT_CONV, 5, 2, 2, (h2, w2)),
+        ("c",      ("b",),           _lib.FOOT_CONV, 3, 1, 1, (h2, w2)),
+        ("d",      ("c",),           _lib.FOOT_CONV, 3, 2, 1, (h4, w4)),
+        ("e",      ("d", "y4"),      _lib.FOOT_CONV, 7, 1, 3, (h4, w4)),           # union with a mask from memory
+        ("f",      ("e",),           _lib.FOOT_UP2X, 0, 0, 0, (2 * h4, 2 * w4)),
+        ("g",      ("e",),           _lib.FOOT_TCONV, 3, 2, 1, (2 * h4, 2 * w4)),  # output_padding 1
+        ("g5",     ("e",),           _lib.FOOT_TCONV, 5, 2, 2, (2 * h4 - 1, 2 * w4 - 1)),
+        ("g2",     ("d",),           _lib.FOOT_TCONV, 2, 2, 0, (2 * h4, 2 * w4)),
+        ("u",      ("f", "g"),       _lib.FOOT_CONV, 1, 1, 0, (2 * h4, 2 * w4)),   # union, identity footprint
+        ("v",      ("u",),           _lib.FOOT_CONV, 3, 1, 0, (2 * h4 - 2, 2 * w4 - 2)),   # no padding: the plane shrinks
+        ("blocks", ("u",),           _lib.FOOT_CONV, 2, 2, 0, (h4, w4)),           # even kernel (block sets of the tconv)
+        ("all",    (None,),          _lib.FOOT_CONV, 3, 1, 1, (h, w)),             # NULL mask: every pixel active
+        ("late",   ("a", "x"),       _lib.FOOT_CONV, 3, 1, 1, (h, w)),             # first mask of the chain, read last
+    ]
+
+
+def _plan_inputs(n, h, w, step):
+    c2 = lambda v, k, p: (v + 2 * p - k) // 2 + 1
+    h4, w4 = c2(c2(h, 5, 2), 3, 1), c2(c2(w, 5, 2), 3, 1)
+    dens = [0.03, 0.0, 0.2][step % 3]                      # sparse, empty (everything stale), dense
+    x = np.stack([blob_mask(h, w, dens, seed=100 * step + b) if dens > 0 else np.zeros((h, w), np.uint8) for b in range(n)])
+    y4 = np.stack([blob_mask(h4, w4, 0.05, seed=900 + 100 * step + b) for b in range(n)])
+    return {"x": x, "y4": y4}
+
+
+def _run_chain(chain, sets, inputs_dev, n, planned):
+    """Build the chain into `sets` (name -> TileMask): one mie_build_mask_plan call, or one build per set."""
+    shape_of = {name: plane for name, _, _, _, _, _, plane in chain}
+    batch = []
+    for name, ins, foot, k, s, p, (ho, wo) in chain:
+        srcs = [None if i is None else (inputs_dev[i] if i in inputs_dev else sets[i].pixmask) for i in ins]
+        hi, wi = (ho, wo) if ins[0] is None else tuple(srcs[0].shape[2:])
+        p1 = None if srcs[0] is None else srcs[0].data_ptr()
+        p2 = srcs[1].data_ptr() if len(srcs) > 1 else None
+        batch.append((p1, p2, hi, wi, foot, k, s, p, sets[name]))
+    lib = _lib.lib()
+    st = torch.cuda.current_stream().cuda_stream
+    if planned:
+        arr = ops._plan_ops(batch)
+        _lib.check(lib.mie_build_mask_plan(arr, len(batch), st))
+    else:
+        for p1, p2, hi, wi, foot, k, s, p, out in batch:
+            _lib.check(lib.mie_build_mask_tiles(p1, p2, hi, wi, foot, k, s, p, out.ref, st))
+
+
+@pytest.mark.parametrize("n,h,w", [(1, 264, 352), (1, 70, 94), (3, 37, 53), (2, 128, 160), (1, 33, 44)])
+def test_mask_plan_equals_the_builds_it_replaces(n, h, w):
+    # one launch for the whole chain against one mie_build_mask_tiles call per set, over three steps with fresh masks
+    # (sparse, empty, dense: the stale lists see everything): every buffer of every tile set must match bit for bit,
+    # and both match the numpy oracle.  Planes with rows that are multiples of 16 bytes, of 4 bytes and of neither;
+    # one sample (lists ranked in the same launch) and several (second kernel).
+    chain = _plan_chain(n, h, w)
+    mk = lambda: {name: TileMask(n, plane[0], plane[1], DEV) for name, _, _, _, _, _, plane in chain}
+    seq, plan = mk(), mk()
+    prev = {}
+    for step in range(3):
+        inputs = _plan_inputs(n, h, w, step)
+        dev = {k_: _to_dev_mask(v) for k_, v in inputs.items()}
+        _run_chain(chain, seq, dev, n, planned=False)
+        _run_chain(chain, plan, dev, n, planned=True)
+        torch.cuda.synchronize()
+        want = dict(inputs)
+        for name, ins, foot, k, s, p, (ho, wo) in chain:
+            a, b = seq[name], plan[name]
+            na, ns = int(a.counts[0].item()), int(a.counts[1].item())
+            tag = "step %d set %s" % (step, name)
+            assert torch.equal(a.pixmask, b.pixmask), tag + ": pixel mask"
+            assert torch.equal(a.counts, b.counts), tag + ": counts %s vs %s" % (a.counts.tolist(), b.counts.tolist())
+            assert torch.equal(a.flags, b.flags), tag + ": flags"
+            assert torch.equal(a.tiles[:na], b.tiles[:na]), tag + ": active list"
+            assert torch.equal(a.stale[:ns], b.stale[:ns]), tag + ": stale list"
+            # and the oracle (the chain restated with numpy)
+            if ins[0] is None:
+                src = np.ones((n, ho, wo), np.uint8)
+            else:
+                src = want[ins[0]] if len(ins) == 1 else (want[ins[0]] | want[ins[1]])
+            if foot == _lib.FOOT_CONV:
+                m = mo.footprint_conv(src, k, s, p)
+            elif foot == _lib.FOOT_UP2X:
+                m = mo.footprint_up2x(src)
+            else:
+                m = mo.footprint_tconv(src, k, s, p, ho, wo)
+            want[name] = m
+            prev[name] = _check_tileset(b, m, prev.get(name))
+
+
+def test_mask_plan_of_a_large_plane_and_many_samples():
+    # 8 samples of 480x640 (38 400 tiles per set: the lists are ranked by the second kernel, ten blocks per set) and a
+    # chain whose masks need more than 64 KB of LDS at once; a device that offers less refuses the plan with
+    # MIE_ERR_CAPACITY and launches nothing
+    n, h, w = 8, 480, 640
+    x = np.stack([blob_mask(h, w, 0.01, seed=7 + b) for b in range(n)])
+    xd = _to_dev_mask(x)
+    names = [("a", 5, 1, 2, (h, w)), ("b", 5, 2, 2, (240, 320)), ("c", 3, 1, 1, (240, 320))]
+    sets = {nm: TileMask(n, pl[0], pl[1], DEV) for nm, _, _, _, pl in names}
+    batch, src, hi, wi = [], xd, h, w
+    for nm, k, s, p, pl in names:
+        batch.append((src.data_ptr(), None, hi, wi, _lib.FOOT_CONV, k, s, p, sets[nm]))
+        src, (hi, wi) = sets[nm].pixmask, pl
+    batch.append((sets["a"].pixmask.data_ptr(), xd.data_ptr(), h, w, _lib.FOOT_CONV, 3, 1, 1, TileMask(n, h, w, DEV)))
+    rc = _lib.lib().mie_build_mask_plan(ops._plan_ops(batch), len(batch), torch.cuda.current_stream().cuda_stream)
+    if rc == -3:
+        assert "LDS" in _lib.lib().mie_last_error_string().decode()
+        pytest.skip("this device offers a workgroup less LDS than the plan needs")
+    _lib.check(rc)
+    m = x
+    for nm, k, s, p, pl in names:
+        m = mo.footprint_conv(m, k, s, p)
+        _check_tileset(sets[nm], m)
+    _check_tileset(batch[-1][-1], mo.footprint_conv(mo.footprint_conv(x, 5, 1, 2) | x, 3, 1, 1))
