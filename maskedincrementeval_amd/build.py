@@ -14,7 +14,7 @@ CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_DIR = os.path.join(PKG_DIR, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libmie_hip.so")
 SOURCES = ["mie_mask.hip", "mie_pointwise.hip", "mie_conv.hip", "mie_conv_mfma_f32.hip",
-           "mie_conv_mfma_bf16.hip", "mie_conv_fewcin.hip", "mie_events.hip", "mie_tail.hip", "mie_refresh.hip", "mie_tconv_mfma.hip"]
+           "mie_conv_mfma_bf16.hip", "mie_upconv_persist.hip", "mie_conv_fewcin.hip", "mie_events.hip", "mie_tail.hip", "mie_refresh.hip", "mie_tconv_mfma.hip"]
 
 # Per-source additions.  The fp32 matrix-core kernels unroll their unit loops completely (up to 196 positions);
 # without the higher threshold the compiler gives up on the longest ones (the 128-column 5x5 / 7x7 kernels), their

@@ -178,6 +178,10 @@ bool mie_launch_conv_gates_mfma(const ConvArgsT<mie_bf16>& a, unsigned cap, hipS
 bool mie_launch_conv_up_mfma(const ConvArgsT<float>& a, unsigned cap, hipStream_t st);
 bool mie_launch_conv_up_mfma(const ConvArgsT<mie_bf16>& a, unsigned cap, hipStream_t st);
 
+// The same for bf16 deltas, 64 -> 32 channels, on planes of many tiles: a persistent kernel (mie_upconv_persist.hip).
+// Returns false, launching nothing, for other shapes.
+bool mie_launch_upconv_persist(const ConvArgsT<mie_bf16>& a, unsigned cap, hipStream_t st);
+
 // Source rows / columns and weights of output index o of a bilinear x2 up-sampling (align_corners =
 // False): src = max(0, o/2 - 0.25), upper index clamped to the last row.
 static __device__ __forceinline__ void conv_up2x_coef(int o, int in_size, int& i0, int& i1, float& l0, float& l1) {
@@ -189,6 +193,15 @@ static __device__ __forceinline__ void conv_up2x_coef(int o, int in_size, int& i
   } else {
     i0 = j - 1; i1 = j; l0 = 0.25f; l1 = 0.75f;
   }
+}
+// One value of the up-sampled tile from its four source values (t00 t01 / t10 t11) with column weights lq0, lq1 and row
+// weights lr0, lr1: horizontal first, then vertical, every product and sum rounded where it is written here, so that
+// every kernel that forms the tile (per pixel, or rows and columns separately) gets the same bits.
+static __device__ __forceinline__ float conv_up2x_h(float lq0, float lq1, float t0, float t1) {
+  return __fmaf_rn(lq0, t0, __fmul_rn(lq1, t1));
+}
+static __device__ __forceinline__ float conv_up2x_v(float lr0, float lr1, float h0, float h1) {
+  return __fmaf_rn(lr0, h0, __fmul_rn(lr1, h1));
 }
 // Matrix-core conv for layers of at most 8 input channels (the network heads), one input, k in {3, 5}, Cout % 32
 // == 0 (mie_conv_fewcin.hip).  Returns false, launching nothing, for other shapes.

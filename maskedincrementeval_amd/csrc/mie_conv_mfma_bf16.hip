@@ -8,7 +8,8 @@ bool mie_launch_conv_gates_mfma(const ConvArgsT<mie_bf16>& a, unsigned cap, hipS
   return launch_gates<mie_bf16>(a, cap, st);
 }
 bool mie_launch_conv_up_mfma(const ConvArgsT<mie_bf16>& a, unsigned cap, hipStream_t st) {
-  return launch_up<mie_bf16>(a, cap, st);
+  // 64 -> 32 channels on a large plane: the persistent kernel (mie_upconv_persist.hip)
+  return mie_launch_upconv_persist(a, cap, st) || launch_up<mie_bf16>(a, cap, st);
 }
 
 #ifdef MIE_WG_PROFILE

@@ -593,10 +593,10 @@ __global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
           for (int e = 0; e < EPS; e += 4) {       // 16-byte LDS reads
             const float4 t00 = *reinterpret_cast<const float4*>(v00 + e), t01 = *reinterpret_cast<const float4*>(v01 + e);
             const float4 t10 = *reinterpret_cast<const float4*>(v10 + e), t11 = *reinterpret_cast<const float4*>(v11 + e);
-            o[e] = lr0 * (lq0 * t00.x + lq1 * t01.x) + lr1 * (lq0 * t10.x + lq1 * t11.x);
-            o[e + 1] = lr0 * (lq0 * t00.y + lq1 * t01.y) + lr1 * (lq0 * t10.y + lq1 * t11.y);
-            o[e + 2] = lr0 * (lq0 * t00.z + lq1 * t01.z) + lr1 * (lq0 * t10.z + lq1 * t11.z);
-            o[e + 3] = lr0 * (lq0 * t00.w + lq1 * t01.w) + lr1 * (lq0 * t10.w + lq1 * t11.w);
+            o[e] = conv_up2x_v(lr0, lr1, conv_up2x_h(lq0, lq1, t00.x, t01.x), conv_up2x_h(lq0, lq1, t10.x, t11.x));
+            o[e + 1] = conv_up2x_v(lr0, lr1, conv_up2x_h(lq0, lq1, t00.y, t01.y), conv_up2x_h(lq0, lq1, t10.y, t11.y));
+            o[e + 2] = conv_up2x_v(lr0, lr1, conv_up2x_h(lq0, lq1, t00.z, t01.z), conv_up2x_h(lq0, lq1, t10.z, t11.z));
+            o[e + 3] = conv_up2x_v(lr0, lr1, conv_up2x_h(lq0, lq1, t00.w, t01.w), conv_up2x_h(lq0, lq1, t10.w, t11.w));
           }
         }
         const int lrow = pix / IT;

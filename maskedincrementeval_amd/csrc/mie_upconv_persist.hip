@@ -1,0 +1,358 @@
+// The last decoder of the batched bf16 network -- 5x5 conv over up2x(a + b), 64 -> 32 channels, bf16 deltas -- as a
+// persistent kernel (gfx950).
+//
+// Per 8x8 output tile this layer holds 0.7 us of matrix-core work (1600 x 32 per pixel) against 22 KB of reservoir and
+// delta traffic and a chain of dependent memory round trips -- tile id, mask bytes, source pixels, filter, reservoir --
+// that a one-tile workgroup walks once per tile: at four resident workgroups per CU each lives 14 us for those 0.7.
+// Here 512 workgroups stay resident (two per CU) and walk the tile list:
+//   * the filter never moves again: a wave owns 16 of the 64 input channels for all 25 taps, which is 25 x 16 bytes
+//     per lane -- 100 registers -- loaded once per workgroup instead of once per tile (102 KB per tile from L2);
+//   * the next tile's source pixels, mask bytes and list entry are asked for while the current tile is blended and
+//     multiplied, this tile's reservoir values before its contraction: no load is waited for where it is issued;
+//   * staging buffer, source block and the k-split reduction buffer have LDS of their own (72 KB), so a tile takes
+//     three barriers;
+//   * and, what counts most, a tile costs fewer instructions: this layer is bound by instruction issue (the one-tile
+//     kernel spends about 1900 issue slots per wave and tile, the bilinear blend of the 12 x 12 x 64 staged values
+//     first among them).  The blend here is separable -- a thread owns one column, eight channels and six rows of the
+//     staged tile, forms the column-blended values of its five source rows once and takes every output row from two
+//     of them -- tile coordinates come from multiplications instead of divisions, and the epilogue's cases (reservoir,
+//     activation) are template arguments.
+// Arithmetic, operand layouts and summation order are those of k_conv_mfma<bf16, 5, 1, 1, 1, ..., UP> (32-column
+// slab, four-way k-split added in wave order, fp32 blend of the fp32 sums a + b), so the two kernels agree bit for bit.
+// XCD-aware order: workgroup b lives on XCD b % 8; each XCD takes a contiguous eighth of the tile list and its 64
+// workgroups walk it side by side, so neighbouring tiles, which share their halo, meet in one L2 at about the same time.
+#include "mie_conv.h"
+
+#include <stdlib.h>
+
+namespace {
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+constexpr int C = 64;                 // input channels (one staged chunk of bf16)
+constexpr int COUT = 32;              // output channels (one slab)
+constexpr int K = 5;
+constexpr int EPS = 8;                // bf16 elements per 16-byte slot
+constexpr int Q4 = C / EPS;           // slots per pixel
+constexpr int IT = 7 + K;             // staged tile edge (12)
+constexpr int NPIX = IT * IT;
+constexpr int NSLOT = NPIX * Q4;      // 1152
+constexpr int NLD = (NSLOT + 255) / 256;
+constexpr int LS = C + EPS;           // staged elements per pixel (72)
+constexpr int RP = 960;               // staged elements per tile row: 12 * 72 = 864, raised to 480 dwords = 32 (mod 64)
+constexpr int STAGE = IT * RP;        // bf16 elements
+constexpr int LO_F = 64 * C;          // floats of the 8x8 source block
+constexpr int RED_F = 4 * 64 * COUT;  // floats of the k-split reduction buffer
+constexpr int GRID = 512;             // resident workgroups: two per CU
+static_assert(RP % 8 == 0 && (RP / 2) % 64 == 32, "row pitch: 32 dwords modulo 64");
+static_assert(STAGE * 2 + LO_F * 4 + RED_F * 4 <= 80 * 1024, "two workgroups per CU");
+
+__device__ __forceinline__ void bf16x8_to_f32(const float4& raw, float (&f)[8]) {
+  const v4f r4 = {raw.x, raw.y, raw.z, raw.w};
+  const mie_bf16x8 b = __builtin_bit_cast(mie_bf16x8, r4);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) f[e] = (float)b[e];
+}
+__device__ __forceinline__ float4 f32_to_bf16x8(const float (&f)[8]) {
+  mie_bf16x8 b;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) b[e] = (mie_bf16)f[e];
+  const v4f r4 = __builtin_bit_cast(v4f, b);
+  return make_float4(r4[0], r4[1], r4[2], r4[3]);
+}
+__device__ __forceinline__ void mma(v16f& acc, const float4& av, const float4& bv) {
+  const v4f a4 = {av.x, av.y, av.z, av.w}, b4 = {bv.x, bv.y, bv.z, bv.w};
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(mie_bf16x8, a4), __builtin_bit_cast(mie_bf16x8, b4), acc, 0, 0, 0);
+}
+
+// (batch index, top-left output pixel) of tile id `tile`; divisions by the tile grid as multiplications by
+// ceil(2^32 / d) (exact while tile * d < 2^32: tile ids stay below 2^30 / d here, see the launcher)
+struct TileGrid { int tiles_x, tiles_y; unsigned mx, my; };
+struct TilePos { int n, y0, x0; };
+__device__ __forceinline__ int div_magic(int a, int d, unsigned m) { return d == 1 ? a : (int)__umulhi((unsigned)a, m); }
+__device__ __forceinline__ TilePos tile_pos(const TileGrid& g, int tile) {
+  TilePos p;
+  const int t2 = div_magic(tile, g.tiles_x, g.mx);
+  p.x0 = (tile - t2 * g.tiles_x) * MIE_TILE;
+  p.n = div_magic(t2, g.tiles_y, g.my);
+  p.y0 = (t2 - p.n * g.tiles_y) * MIE_TILE;
+  return p;
+}
+
+// epilogue of one group of four adjacent channels, its cases fixed at compile time
+template <bool RES, int ACT>
+__device__ __forceinline__ void epilogue4(const ConvArgsT<mie_bf16>& a, long long off, const float4& v, const float4& r0) {
+  if (!RES) {
+    mie_st4(a.out, off, v);
+    return;
+  }
+  const float4 r1 = make_float4(r0.x + v.x, r0.y + v.y, r0.z + v.z, r0.w + v.w);
+  mie_st4(a.res, off, r1);
+  mie_st4(a.out, off, make_float4(mie_act(ACT, a.slope, r1.x) - mie_act(ACT, a.slope, r0.x),
+                                  mie_act(ACT, a.slope, r1.y) - mie_act(ACT, a.slope, r0.y),
+                                  mie_act(ACT, a.slope, r1.z) - mie_act(ACT, a.slope, r0.z),
+                                  mie_act(ACT, a.slope, r1.w) - mie_act(ACT, a.slope, r0.w)));
+}
+
+template <bool RES, int ACT>
+__global__ __launch_bounds__(256, 2) void k_upconv64_persist(ConvArgsT<mie_bf16> a) {
+  __shared__ __attribute__((aligned(16))) mie_bf16 s_stage[STAGE];
+  __shared__ __attribute__((aligned(16))) float s_lo[LO_F];
+  __shared__ __attribute__((aligned(16))) float s_red[RED_F];
+  const int entry_zero = conv_args_entry_zero(a);
+  const int bid = blockIdx.x + entry_zero;
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int l32 = lane & 31, half = lane >> 5;
+  const int cap = a.ts.n * a.ts.tiles_y * a.ts.tiles_x;
+  const int n_act = a.ts.counts[MIE_CNT_ACTIVE], n_st = a.ts.counts[MIE_CNT_STALE];
+  if (n_act < 0 || n_st < 0 || n_act > cap || n_st > cap) return;       // corrupt counts
+  const int hout = a.ts.h, wout = a.ts.w;
+  const int h_lo = a.h_in >> 1, w_lo = a.w_in >> 1;
+  TileGrid grid;
+  grid.tiles_x = a.ts.tiles_x; grid.tiles_y = a.ts.tiles_y;
+  grid.mx = 0xffffffffu / (unsigned)grid.tiles_x + 1u;
+  grid.my = 0xffffffffu / (unsigned)grid.tiles_y + 1u;
+
+  // ---- stale tiles: zero this layer's delta there (the whole grid shares them) ----------------------------------
+  for (int s = bid; s < n_st; s += GRID) {
+    const int tile = a.ts.stale[s];
+    if (tile < 0 || tile >= cap) continue;
+    const TilePos tp = tile_pos(grid, tile);
+    for (int idx = tid; idx < 64 * (COUT / 4); idx += 256) {
+      const int p = idx / (COUT / 4), col = 4 * (idx - p * (COUT / 4));
+      const int oy = tp.y0 + (p >> 3), ox = tp.x0 + (p & 7);
+      if (oy < hout && ox < wout)
+        mie_st4(a.out, (((long long)tp.n * hout + oy) * wout + ox) * COUT + col, make_float4(0.f, 0.f, 0.f, 0.f));
+    }
+  }
+
+  // ---- this workgroup's walk over the active list ------------------------------------------------------------------
+  const int xcd = bid & 7, per = GRID >> 3;
+  const int c_act = (n_act + 7) >> 3;
+  const int t_hi = (xcd + 1) * c_act < n_act ? (xcd + 1) * c_act : n_act;
+  int t = xcd * c_act + (bid >> 3);
+  if (t >= t_hi) return;
+  auto list_entry = [&](int pos) -> int {     // tile id at list position pos of this walk, -1 past its end
+    const int v = a.ts.tiles[pos < t_hi ? pos : t_hi - 1];
+    return (pos < t_hi && v >= 0 && v < cap) ? v : -1;
+  };
+
+  // ---- the filter: this wave's 16 input channels of every tap, for good ----------------------------------------
+  // matrix-core filter copy P[ci/16][tap][(ci%16)/8][co][ci%8]: a lane's 16 bytes of unit (sub-chunk `wave`, tap)
+  float4 bfrag[K * K];
+  {
+    const mie_bf16* fb = a.filt_mc + ((long long)wave * (K * K) * 2 * COUT) * EPS + (half * COUT + l32) * EPS;
+#pragma unroll
+    for (int tap = 0; tap < K * K; ++tap) bfrag[tap] = *reinterpret_cast<const float4*>(fb + (long long)tap * 2 * COUT * EPS);
+  }
+
+  // ---- per-thread constants of the staging plan -------------------------------------------------------------------
+  // source block: 64 pixels x 8 slots per tensor; this thread copies slot q4 of pixels lp0 and lp0 + 32
+  const int q4 = tid & 7, lp0 = tid >> 3;
+  // operand reads: pixel p = 32 * mb + l32 of the tile, channels 16 * wave + 8 * half ...
+  int a_lane[2];
+#pragma unroll
+  for (int mb = 0; mb < 2; ++mb) {
+    const int p = mb * 32 + l32;
+    a_lane[mb] = (p >> 3) * RP + (p & 7) * LS + 16 * wave + EPS * half;
+  }
+  const bool m1 = a.xm != nullptr, has2 = a.x2 != nullptr, m2 = has2 && a.x2m != nullptr;
+  const mie_bf16* dummy = a.filt_mc;      // masked lanes read one cache-resident address
+
+  // source pixels and mask bits of a tile, into registers (loads unconditional in control flow)
+  auto load_src = [&](int tile, float4 (&ra)[2], float4 (&rb)[2], unsigned& ok_a, unsigned& ok_b) {
+    ok_a = ok_b = 0u;
+    const TilePos tp = tile_pos(grid, tile < 0 ? 0 : tile);
+    const int lo_y0 = ((tp.y0 - 2) >> 1) - 1, lo_x0 = ((tp.x0 - 2) >> 1) - 1;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int lp = lp0 + 32 * i;
+      const int ly = lo_y0 + (lp >> 3), lx = lo_x0 + (lp & 7);
+      const bool inb = tile >= 0 && ly >= 0 && ly < h_lo && lx >= 0 && lx < w_lo;
+      const long long po = inb ? ((long long)tp.n * h_lo + ly) * w_lo + lx : 0;
+      const long long eo = po * C + EPS * q4;
+      const unsigned v1 = m1 ? (unsigned)(a.xm[po] != 0) : 1u;
+      const unsigned v2 = m2 ? (unsigned)(a.x2m[po] != 0) : (has2 ? 1u : 0u);
+      ra[i] = *reinterpret_cast<const float4*>(inb ? a.x + eo : dummy);
+      rb[i] = *reinterpret_cast<const float4*>((inb && has2) ? a.x2 + eo : dummy);
+      ok_a |= (inb ? v1 : 0u) << i;
+      ok_b |= (inb ? v2 : 0u) << i;
+    }
+  };
+
+  int tile = list_entry(t);
+  int tile_next = list_entry(t + per);
+  float4 ra[2], rb[2];
+  unsigned ok_a, ok_b;
+  load_src(tile, ra, rb, ok_a, ok_b);
+
+  while (tile >= 0) {
+    const TilePos tp = tile_pos(grid, tile);
+    const int n = tp.n, y0 = tp.y0, x0 = tp.x0;
+    const int iy0 = y0 - 2, ix0 = x0 - 2;
+    const int lo_y0 = (iy0 >> 1) - 1, lo_x0 = (ix0 >> 1) - 1;
+
+    // A. a + b of the source block to LDS, fp32 (masked pixels: the raw registers are zeroed, bit pattern 0 = 0.0)
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const bool ka = (ok_a >> i) & 1u, kb = (ok_b >> i) & 1u;
+      const float4 za = ka ? ra[i] : make_float4(0.f, 0.f, 0.f, 0.f), zb = kb ? rb[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+      float fa[8], fb[8];
+      bf16x8_to_f32(za, fa);
+      bf16x8_to_f32(zb, fb);
+      float* d = s_lo + (lp0 + 32 * i) * C + q4 * EPS;
+      *reinterpret_cast<float4*>(d) = make_float4(fa[0] + fb[0], fa[1] + fb[1], fa[2] + fb[2], fa[3] + fb[3]);
+      *reinterpret_cast<float4*>(d + 4) = make_float4(fa[4] + fb[4], fa[5] + fb[5], fa[6] + fb[6], fa[7] + fb[7]);
+    }
+
+    // B. this tile's reservoir values: asked for now, used after the contraction
+    long long e_off[2];
+    bool e_ok[2];
+    float4 e_r0[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int idx = tid + 256 * i;
+      const int p = idx >> 3, col = 4 * (idx & 7);
+      const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
+      e_ok[i] = oy < hout && ox < wout;
+      e_off[i] = (((long long)n * hout + oy) * wout + ox) * COUT + col;
+      e_r0[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (RES && e_ok[i]) e_r0[i] = *reinterpret_cast<const float4*>(a.res + e_off[i]);
+    }
+
+    // C. the next tile's source pixels and the list entry after it
+    t += per;
+    const int tile_nn = list_entry(t + per);
+    load_src(tile_next, ra, rb, ok_a, ok_b);
+    __syncthreads();                                   // (1) the source block is in LDS
+
+    // D. the staged tile, blended from the source block.  Thread u < 192 owns column pcol, channels 8 * sq .. and rows
+    // 6 * rh .. 6 * rh + 5 of the 12 x 12 tile: the column blend of its five source rows (local rows 3 * rh .. 3 * rh + 4 of
+    // the 8 x 8 block) once, then every output row from two of them.  Row 2m of the up-sampled image takes source rows
+    // (m - 1, m) with weights (1/4, 3/4), row 2m + 1 rows (m, m + 1) with (3/4, 1/4); at the image border the missing
+    // neighbour is the row itself, i.e. weights (0, 1) / (1, 0) on the pair as it lies in the block (rows outside the image
+    // are stored as zeros); rows and columns outside the up-sampled image are the conv's zero padding: weights (0, 0).
+    if (tid < 192) {
+      const int sq = tid & 7, cu = tid >> 3;
+      const int rh = cu >= IT ? 1 : 0, pcol = cu - IT * rh;
+      const int hx = ix0 + pcol;
+      int c0 = 0, c1 = 0;
+      float lq0 = 0.f, lq1 = 0.f;
+      if (hx >= 0 && hx < a.w_in) conv_up2x_coef(hx, w_lo, c0, c1, lq0, lq1);
+      else c0 = c1 = lo_x0 < 0 ? 0 : lo_x0;
+      const float* s0 = s_lo + ((3 * rh) * 8 + (c0 - lo_x0)) * C + sq * EPS;
+      const float* s1 = s_lo + ((3 * rh) * 8 + (c1 - lo_x0)) * C + sq * EPS;
+      float hb[5][EPS];
+#pragma unroll
+      for (int r = 0; r < 5; ++r)
+#pragma unroll
+        for (int e = 0; e < EPS; e += 4) {
+          const float4 t0 = *reinterpret_cast<const float4*>(s0 + r * 8 * C + e), t1 = *reinterpret_cast<const float4*>(s1 + r * 8 * C + e);
+          hb[r][e] = conv_up2x_h(lq0, lq1, t0.x, t1.x);
+          hb[r][e + 1] = conv_up2x_h(lq0, lq1, t0.y, t1.y);
+          hb[r][e + 2] = conv_up2x_h(lq0, lq1, t0.z, t1.z);
+          hb[r][e + 3] = conv_up2x_h(lq0, lq1, t0.w, t1.w);
+        }
+#pragma unroll
+      for (int i = 0; i < 6; ++i) {
+        const int pr = 6 * rh + i;
+        const int hy = iy0 + pr, m = hy >> 1;
+        const bool odd = (i & 1) != 0;                       // iy0 is even: row parity is the parity of i
+        const int ra_ = (i >> 1) + (odd ? 1 : 0);            // first row of the pair, relative to 3 * rh
+        float lr0 = odd ? 0.75f : 0.25f, lr1 = odd ? 0.25f : 0.75f;
+        if (odd ? (m + 1 >= h_lo) : (m == 0)) lr0 = odd ? 1.f : 0.f, lr1 = odd ? 0.f : 1.f;
+        if (hy < 0 || hy >= a.h_in) lr0 = lr1 = 0.f;
+        float o[EPS];
+#pragma unroll
+        for (int e = 0; e < EPS; ++e) o[e] = conv_up2x_v(lr0, lr1, hb[ra_][e], hb[ra_ + 1][e]);
+        *reinterpret_cast<float4*>(s_stage + pr * RP + pcol * LS + EPS * sq) = f32_to_bf16x8(o);
+      }
+    }
+    __syncthreads();                                   // (2) the staged tile is in LDS
+
+    // E. the contraction: 25 units (taps) of this wave's sub-chunk, two pixel blocks each
+    v16f acc[2];
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[mb][r] = 0.f;
+    {
+      float4 av[2][2];
+      av[0][0] = *reinterpret_cast<const float4*>(&s_stage[a_lane[0]]);
+      av[0][1] = *reinterpret_cast<const float4*>(&s_stage[a_lane[1]]);
+#pragma unroll
+      for (int tap = 0; tap < K * K; ++tap) {
+        if (tap + 1 < K * K) {
+          const int ky = (tap + 1) / K, kx = (tap + 1) - ky * K;
+          av[(tap + 1) & 1][0] = *reinterpret_cast<const float4*>(&s_stage[a_lane[0] + ky * RP + kx * LS]);
+          av[(tap + 1) & 1][1] = *reinterpret_cast<const float4*>(&s_stage[a_lane[1] + ky * RP + kx * LS]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        mma(acc[0], av[tap & 1][0], bfrag[tap]);
+        mma(acc[1], av[tap & 1][1], bfrag[tap]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+
+    // F. the four k-split partial sums meet in LDS (a buffer of its own: nobody has to be waited for first)
+    {
+      float* red = s_red + wave * (64 * COUT);
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int p = mb * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+          red[p * COUT + l32] = acc[mb][r];
+        }
+    }
+    __syncthreads();                                   // (3) the partial sums are in LDS
+    {
+      float4 v[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int idx = tid + 256 * i;
+        float4 sum = *reinterpret_cast<const float4*>(&s_red[4 * idx]);
+#pragma unroll
+        for (int k2 = 1; k2 < 4; ++k2) {
+          const float4 part = *reinterpret_cast<const float4*>(&s_red[k2 * (64 * COUT) + 4 * idx]);
+          sum.x += part.x; sum.y += part.y; sum.z += part.z; sum.w += part.w;
+        }
+        v[i] = sum;
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        if (e_ok[i]) epilogue4<RES, ACT>(a, e_off[i], v[i], e_r0[i]);
+    }
+    // (the next tile's barriers (1) and (2) stand between these reads of s_red and its next writes, barrier (3) between
+    // this tile's reads of s_lo / s_stage and their next writes)
+    tile = tile_next;
+    tile_next = tile_nn;
+  }
+}
+
+}  // namespace
+
+// Takes the shape of the batched bf16 network's last decoder on planes large enough to keep the resident grid busy
+// (launches nothing and returns false otherwise; MIE_UPCONV_PERSIST=0 switches the kernel off, for measurements).
+bool mie_launch_upconv_persist(const ConvArgsT<mie_bf16>& a, unsigned cap, hipStream_t st) {
+  static const bool enabled = [] {
+    const char* e = getenv("MIE_UPCONV_PERSIST");
+    return e == nullptr || atoi(e) != 0;
+  }();
+  if (!enabled || a.c1 != C || a.cout != COUT || a.pad != 2 || a.refresh || a.filt_mc == nullptr || a.x3 || a.addend != nullptr) return false;
+  if (a.x2 != nullptr && a.c2 != C) return false;
+  if (cap < 4u * GRID || cap > (1u << 20)) return false;      // small planes: one tile per workgroup is as good
+  const dim3 g(GRID), b(256);
+  if (a.res == nullptr) {
+    hipLaunchKernelGGL((k_upconv64_persist<false, MIE_ACT_NONE>), g, b, 0, st, a);
+    return true;
+  }
+  switch (a.act) {
+    case MIE_ACT_NONE: hipLaunchKernelGGL((k_upconv64_persist<true, MIE_ACT_NONE>), g, b, 0, st, a); return true;
+    case MIE_ACT_RELU: hipLaunchKernelGGL((k_upconv64_persist<true, MIE_ACT_RELU>), g, b, 0, st, a); return true;
+    case MIE_ACT_LEAKY_RELU: hipLaunchKernelGGL((k_upconv64_persist<true, MIE_ACT_LEAKY_RELU>), g, b, 0, st, a); return true;
+    default: return false;                                      // sigmoid / tanh epilogues: the one-tile kernel
+  }
+}

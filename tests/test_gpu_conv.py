@@ -571,3 +571,55 @@ def test_few_input_channels_matrix_core_kernel(cin, cout, k, s, dtype):
         foot = torch.from_numpy(mo.footprint_conv(m[:, 0].numpy(), k, s, p)).bool().unsqueeze(1)
         assert torch.count_nonzero(got * (~foot)) == 0
     assert torch.allclose(res.cpu(), res_ref, rtol=RTOL, atol=bf16_atol(ref, 2.0) if bf else ATOL)
+
+
+# The persistent form of the 64 -> 32 bf16 up-sampling conv (the last decoder of the batched network) takes planes of
+# at least 2048 tiles.  Same inputs once as a batch of three ragged frames (2250 tiles: the persistent kernel) and once
+# frame by frame (750 tiles each: one workgroup per tile) must agree bit for bit -- deltas and reservoirs -- over three
+# steps with fresh masks (stale tiles, an empty step), one and two inputs, with and without the reservoir epilogue;
+# and both match the oracle.
+def test_persistent_upsampled_conv_agrees_with_the_one_tile_kernel():
+    bf = torch.bfloat16
+    n, c, cout, h, w = 3, 64, 32, 100, 118                   # output 200 x 236: 25 x 30 tiles per frame, ragged right edge
+    q = lambda t: t.to(bf).float()
+    wt = q(he_normal_conv_weight(cout, c, 5, 9))
+    filt = _filt(wt)
+    assert _lib.tile_capacity(n, 2 * h, 2 * w) >= 2048 > _lib.tile_capacity(1, 2 * h, 2 * w)
+    big = dict(up=TileMask(n, 2 * h, 2 * w, DEV), ts=TileMask(n, 2 * h, 2 * w, DEV), out=ops.new_nhwc(n, cout, 2 * h, 2 * w, DEV, bf))
+    one = [dict(up=TileMask(1, 2 * h, 2 * w, DEV), ts=TileMask(1, 2 * h, 2 * w, DEV), out=ops.new_nhwc(1, cout, 2 * h, 2 * w, DEV, bf))
+           for _ in range(n)]
+    r0 = gaussian_delta(n, cout, 2 * h, 2 * w, 1.0, 1.0, seed=3)[0]
+    res_big = _dev(r0).clone()
+    res_one = [_dev(r0[i:i + 1]).clone() for i in range(n)]
+    res_ref = r0.clone()
+    for step, (da, db, two, with_res) in enumerate([(0.2, 0.1, True, True), (0.0, 0.0, True, False), (0.05, 0.0, False, True),
+                                                    (0.3, 0.2, True, False)]):
+        a, ma = gaussian_delta(n, c, h, w, da, 0.5, seed=100 + step) if da > 0 else (torch.zeros(n, c, h, w), torch.zeros(n, 1, h, w, dtype=torch.uint8))
+        b, mb = gaussian_delta(n, c, h, w, db, 0.5, seed=200 + step) if db > 0 else (torch.zeros(n, c, h, w), torch.zeros(n, 1, h, w, dtype=torch.uint8))
+        a, b = q(a), q(b)
+        ref = io.conv_incr(q(io.interp_incr(a + b if two else a)), wt, 1, 2)
+        act = _lib.ACT_RELU if with_res else _lib.ACT_NONE
+
+        def run(sets, ad, am, bd, bm, res):
+            nn = ad.shape[0]
+            ops.build_mask_tiles(am, bm if two else None, nn, h, w, _lib.FOOT_UP2X, 0, 0, 0, sets["up"])
+            ops.build_mask_tiles(sets["up"], None, nn, 2 * h, 2 * w, _lib.FOOT_CONV, 5, 1, 2, sets["ts"])
+            ops.upconv_masked(ad, am, bd if two else None, bm if two else None, filt, 5, 2, sets["ts"], sets["out"],
+                              res if with_res else None, act)
+        ad, bd, am, bm = _dev(a).to(bf), _dev(b).to(bf), ma.to(DEV), mb.to(DEV)
+        run(big, ad, am, bd, bm, res_big)
+        for i in range(n):
+            run(one[i], ad[i:i + 1].contiguous(memory_format=torch.channels_last), am[i:i + 1].contiguous(),
+                bd[i:i + 1].contiguous(memory_format=torch.channels_last), bm[i:i + 1].contiguous(), res_one[i])
+        torch.cuda.synchronize()
+        for i in range(n):
+            assert torch.equal(big["out"][i:i + 1], one[i]["out"]), "step %d frame %d: delta" % (step, i)
+            assert torch.equal(res_big[i:i + 1], res_one[i]), "step %d frame %d: reservoir" % (step, i)
+        got = big["out"].float().cpu()
+        want = torch.relu(res_ref + ref) - torch.relu(res_ref) if with_res else ref
+        assert torch.allclose(got, want, rtol=BF16_RTOL, atol=bf16_atol(want, 2.0)), "step %d max|diff| = %.3e" % (step, (got - want).abs().max())
+        if with_res:
+            res_ref = res_ref + ref
+            assert torch.allclose(res_big.cpu(), res_ref, rtol=RTOL, atol=bf16_atol(ref, 2.0))
+        # clean delta: zero outside the active pixels of the tile set
+        assert torch.count_nonzero(big["out"].float() * (1 - big["ts"].pixmask.float())) == 0

@@ -498,3 +498,57 @@ def test_planning_pass_refuses_masks_that_depend_on_values():
         with pytest.raises(RuntimeError, match="cannot be planned ahead"):
             m([_cl(event_voxel_delta(1, 5, h, w, 0.05, seed=35)[0]), None], None)
     assert ops._phase is None and ops._planner is None      # both context managers unwound
+
+
+@pytest.mark.parametrize("knob", ["threshold", "kfence"])
+def test_value_dependent_masks_replay_from_a_graph(knob):
+    # A network whose masks depend on the values (threshold masks in front of every conv, incr_modules/utils.py:22-25; the
+    # delta quantiser, incr_modules/mask_incr_modules.py:21-47) cannot be planned ahead, but it can be captured: every
+    # mask build is a launch on the compute stream and no launch reads device data on the host.  Eight steps with fresh
+    # inputs replayed from ONE captured graph must reproduce the eager network bit for bit (predictions and, for the
+    # thresholded network, the number of tiles every step left active in the last decoder), with the program's own
+    # work between the replays.
+    h, w, steps = 72, 104, 8
+    nets = []
+    for _ in range(2):
+        m = seed_module_(E2VIDRecurrentIncr(), seed=31).to(DEV).eval()
+        if knob == "threshold":
+            mm.set_input_threshold(m, 3e-3)
+        else:
+            mm.set_kfence(m, 0.05, norm="rms")
+        nets.append(m)
+    eager, captured = nets
+    x0 = torch.randn(1, 5, h, w, generator=torch.Generator().manual_seed(32)) * 0.5
+    deltas = [_cl(event_voxel_delta(1, 5, h, w, 0.03 + 0.02 * (i % 3), seed=4300 + i)[0]) for i in range(steps)]
+    static_in = _cl(torch.zeros(1, 5, h, w))
+    last = lambda m: m.unetrecurrent.decoders[2].conv2d
+    with torch.no_grad():
+        eager.forward_refresh_reservoirs(_cl(x0), None)
+        captured.forward_refresh_reservoirs(_cl(x0), None)
+        refs, ref_tiles = [], []
+        for d in deltas:
+            refs.append(eager([d, None], None)[0][0].clone())
+            ref_tiles.append([int(b.counts[0].item()) for k_, b in last(eager)._ib().items() if k_[0] == "t"])
+        got, got_tiles = [], []
+        g = g_out = None
+        for i, d in enumerate(deltas):
+            static_in.copy_(d)
+            if i == 2:                # two eager steps first: they allocate every persistent buffer
+                torch.cuda.synchronize()
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    g_out = captured([static_in, None], None)[0][0]
+            if g is not None:
+                g.replay()
+                got.append(g_out.clone())
+            else:
+                got.append(captured([static_in, None], None)[0][0].clone())
+            got_tiles.append([int(b.counts[0].item()) for k_, b in last(captured)._ib().items() if k_[0] == "t"])
+    torch.cuda.synchronize()
+    for i in range(steps):
+        assert torch.equal(got[i], refs[i]), "step %d max|diff| = %.3e" % (i, (got[i] - refs[i]).abs().max().item())
+        assert got_tiles[i] == ref_tiles[i], "step %d: active tiles %s vs %s" % (i, got_tiles[i], ref_tiles[i])
+    if knob == "threshold":
+        # the masks did depend on the values: the thresholded network runs fewer tiles than the plane holds
+        cap = max(b.capacity for k_, b in last(captured)._ib().items() if k_[0] == "t")
+        assert min(max(t) for t in got_tiles) < cap
