@@ -55,6 +55,9 @@ def parse_args():
     ap.add_argument("--batch", type=int, default=1, help="independent event streams per step (8 with 480x640: the batched configuration)")
     ap.add_argument("--cpu-steps", type=int, default=400, help="incremental steps of the CPU baseline (0 = skip)")
     ap.add_argument("--no-graph", action="store_true", help="launch kernels eagerly instead of replaying a HIP graph")
+    ap.add_argument("--copy-input", action="store_true",
+                    help="one captured graph and a device-to-device copy of the next delta into its input buffer before every "
+                         "replay (default: one graph per resident input, no copy)")
     ap.add_argument("--no-dense", action="store_true", help="skip the all-tiles-active comparator")
     ap.add_argument("--layer-iters", type=int, default=20, help="timed launches per layer for the roofline table")
     ap.add_argument("--no-plan-first", dest="plan_first", action="store_false",
@@ -297,6 +300,13 @@ class NetBench:
         self.static_in.copy_(self.deltas[i % self.n_inputs])
         return self.run_net(m, self.static_in)
 
+    def _replay(self, graphs, i):
+        if len(graphs) == 1:
+            self.static_in.copy_(self.deltas[i % self.n_inputs])
+            graphs[0].replay()
+        else:
+            graphs[i % self.n_inputs].replay()
+
     def timed_run(self, m, tag, steps=None, repeats=None, check_against=None, graph=None):
         """Refresh, warm up, capture one step in a HIP graph, then time `steps` steps `repeats` times.
         Returns (median seconds per step, list of the repeats' ms/step, output-check dict)."""
@@ -311,8 +321,11 @@ class NetBench:
                 self.step_eager(m, i)
                 history.append(i)
             torch.cuda.synchronize()
-            g = graph_out = None
+            graphs = graph_out = None
             if use_graph:
+                # One captured graph per resident input: a step then reads its delta where it lies, as it would from the
+                # buffer an event front end writes, and no copy into a fixed input buffer is timed (--copy-input: one
+                # graph, input copied in front of every replay).
                 side = torch.cuda.Stream()
                 side.wait_stream(torch.cuda.current_stream())
                 with torch.cuda.stream(side):
@@ -320,21 +333,22 @@ class NetBench:
                 history.append(0)
                 torch.cuda.current_stream().wait_stream(side)
                 torch.cuda.synchronize()
-                g = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(g):
-                    graph_out = self.out_of(self.run_net(m, self.static_in))
+                graphs = []
+                for src in ([self.static_in] if args.copy_input else self.deltas):
+                    g = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(g):
+                        graph_out = self.out_of(self.run_net(m, src))
+                    graphs.append(g)
                 for i in range(3):
-                    self.static_in.copy_(self.deltas[i % self.n_inputs])
-                    g.replay()
+                    self._replay(graphs, i)
                     history.append(i)
             per_repeat = []
             for _ in range(repeats):
                 torch.cuda.synchronize()
                 t0 = time.perf_counter()
                 for i in range(steps):
-                    if g is not None:
-                        self.static_in.copy_(self.deltas[i % self.n_inputs])
-                        g.replay()
+                    if graphs is not None:
+                        self._replay(graphs, i)
                     else:
                         self.step_eager(m, i)
                 torch.cuda.synchronize()
@@ -351,9 +365,8 @@ class NetBench:
                 worst = 0.0
                 for i in range(4):
                     want = self.out_of(self.run_net(ref, self.deltas[i % self.n_inputs]))
-                    if g is not None:
-                        self.static_in.copy_(self.deltas[i % self.n_inputs])
-                        g.replay()
+                    if graphs is not None:
+                        self._replay(graphs, i)
                         got = graph_out
                     else:
                         got = self.out_of(self.step_eager(m, i))
@@ -368,7 +381,7 @@ class NetBench:
         sec = statistics.median(per_repeat)
         log("%s: %.3f ms/step median of %d x %d steps (min %.3f, max %.3f; %s)"
             % (tag, 1e3 * sec, repeats, steps, 1e3 * min(per_repeat), 1e3 * max(per_repeat),
-               "eager" if g is None else "HIP graph"))
+               "eager" if graphs is None else "HIP graph"))
         return sec, [round(1e3 * t, 4) for t in per_repeat], check
 
     def layer_table(self, model, iters):
@@ -806,7 +819,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": "%s recurrent UNet, random init, %dx%dx%dx%d event voxel deltas, %.0f%% "
                                "active pixels, 1 dense refresh then incremental steps" % (NET_NAME, NB, BINS, H, W, 100 * dens),
-                   "density": dens, "height": H, "width": W, "batch": NB, "graph": not args.no_graph,
+                   "density": dens, "height": H, "width": W, "batch": NB, "graph": not args.no_graph, "input": "copied per step" if args.copy_input else "read in place",
                    "timing": "median of %d repeats of %d steps" % (args.repeats, args.steps),
                    "f32_matmul": ops.f32_matmul if args.dtype == "f32" else None,
                    "arithmetic": ARITHMETIC["bf16" if args.dtype == "bf16" else ops.f32_matmul],
