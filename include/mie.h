@@ -731,6 +731,19 @@ int mie_events_to_frame(const double* events, int n_events, int kind, int num_bi
                         double start_old, double start_new, double delta_t,
                         int delta, float* out, uint8_t* pixmask, void* stream);
 
+/*
+ * mie_events_to_frame with the frame also delivered as bf16, for the networks that run on bf16 deltas
+ * (MIE_DTYPE_BF16): `sums` is the fp32 frame exactly as mie_events_to_frame leaves it in `out` (the
+ * atomic sums need fp32), `out` [same shape] receives every element of it rounded to nearest even, in
+ * the same stream -- the cast a caller would otherwise run as a separate pass over the frame
+ * (`event_tensor.to(...)` after data_fetchers/utils/util.py:107).  out != sums, 8-byte aligned.
+ */
+int mie_events_to_frame_bf16(const double* events, int n_events, int kind, int num_bins,
+                             int height, int width, int pad_left, int pad_right,
+                             int pad_top, int pad_bottom, double t_scale,
+                             double start_old, double start_new, double delta_t,
+                             int delta, float* sums, void* out, uint8_t* pixmask, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -33,7 +33,7 @@ EXPORTS = (
     "mie_version", "mie_last_error_string", "mie_tile_capacity", "mie_mask_from_delta",
     "mie_build_mask_tiles", "mie_conv_masked", "mie_act_incr", "mie_mul_incr", "mie_add_incr",
     "mie_upsample2x_incr", "mie_convlstm_gates_incr", "mie_tconv_masked", "mie_conv_refresh",
-    "mie_pack_filter", "mie_kfence_incr", "mie_events_to_frame", "mie_tconv_refresh", "mie_conv_gates_masked",
+    "mie_pack_filter", "mie_kfence_incr", "mie_events_to_frame", "mie_events_to_frame_bf16", "mie_tconv_refresh", "mie_conv_gates_masked",
     "mie_maxpool_incr", "mie_accumulate", "mie_scale_incr", "mie_avgpool_incr", "mie_linear_incr", "mie_upconv_masked",
     "mie_conv_masked_ws", "mie_convgru_gates_incr", "mie_upsample2x_pair_incr", "mie_conv_masked_noalloc",
     "mie_convlstm_gates_refresh", "mie_convgru_gates_refresh", "mie_mul_dense", "mie_tconv2x_masked",
@@ -115,6 +115,8 @@ def _declare(l):
     l.mie_events_to_frame.restype = ci
     cd = ctypes.c_double
     l.mie_events_to_frame.argtypes = [vp, ci, ci, ci, ci, ci, ci, ci, ci, ci, cd, cd, cd, cd, ci, vp, vp, vp]
+    l.mie_events_to_frame_bf16.restype = ci
+    l.mie_events_to_frame_bf16.argtypes = [vp, ci, ci, ci, ci, ci, ci, ci, ci, ci, cd, cd, cd, cd, ci, vp, vp, vp, vp]
     l.mie_conv_f32x3_takes.restype = ci
     l.mie_conv_f32x3_takes.argtypes = [ci, ci, ci, ci, ci]
     l.mie_pack_filter.restype = ci

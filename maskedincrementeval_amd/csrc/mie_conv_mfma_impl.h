@@ -133,6 +133,18 @@ __host__ __device__ constexpr int pad_units(int n) {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
+// Waves per SIMD the register allocation must leave room for.  The stride-2 5x5 bf16 kernels stage a 19x19 tile
+// (52 KB of LDS: three workgroups fit a CU) and spend two thirds of a workgroup's life outside the MFMA loop
+// (tile pick, mask bytes, the one staging round trip, a 128-column epilogue), so a third resident workgroup
+// is what fills the matrix cores; their natural allocation (172 registers) stops at two.
+#ifndef MIE_S2_WAVES
+#define MIE_S2_WAVES 3
+#endif
+__host__ __device__ constexpr int conv_min_waves(int elem_size, int K, int S, bool HALF, bool GATES, bool UP, bool SPLIT,
+                                                 bool X3) {
+  return (elem_size == 2 && S == 2 && K == 5 && !HALF && !GATES && !UP && !SPLIT && !X3) ? MIE_S2_WAVES : 1;
+}
+
 // One unit of the contraction on the matrix core: the 16 bytes of A and of B a lane holds.
 __device__ __forceinline__ void mma_unit(v16f& acc, const float4& av, const float4& bv, float) {
   acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.x, bv.x, acc, 0, 0, 0);
@@ -247,7 +259,7 @@ template <typename T, int K, int S, int WN, int NB, bool HALF, bool GATES = fals
 // (Build with -mllvm -pragma-unroll-threshold=65536: the unit loop of the 128-column 5x5 / 7x7 kernels is 100 / 196
 // positions long, and where the compiler refuses to unroll it the operand ring is indexed at run time and lands in
 // scratch memory -- a factor of three in time.)
-__global__ __launch_bounds__(256) void k_conv_mfma(ConvArgsT<T> a) {
+__global__ __launch_bounds__(256, conv_min_waves((int)sizeof(T), K, S, HALF, GATES, UP, SPLIT, X3)) void k_conv_mfma(ConvArgsT<T> a) {
   static_assert(!X3 || (sizeof(T) == 4 && !HALF && (K == 3 || K == 5)), "X3: fp32 deltas, 3x3 / 5x5");
   using TL = std::conditional_t<X3, mie_bf16, T>;            // element type in LDS and on the matrix cores
   constexpr int PL = X3 ? 3 : 1;                             // operand planes (terms per value)

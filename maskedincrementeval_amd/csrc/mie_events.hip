@@ -94,6 +94,17 @@ __global__ __launch_bounds__(256) void k_events_scatter(EventArgs a) {
     }
 }
 
+// fp32 sums -> bf16 elements (round to nearest even), four per thread; the sums are zero where no event landed
+__global__ __launch_bounds__(256) void k_events_round(const float* __restrict__ acc, long long n, mie_bf16* __restrict__ out) {
+  const long long i = ((long long)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (i + 4 <= n) {
+    const float4 v = *reinterpret_cast<const float4*>(acc + i);
+    mie_st4(out, i, v);
+  } else {
+    for (long long j = i; j < n; ++j) out[j] = (mie_bf16)acc[j];
+  }
+}
+
 }  // namespace
 
 extern "C" int mie_events_to_frame(const double* events, int n_events, int kind, int num_bins,
@@ -134,5 +145,23 @@ extern "C" int mie_events_to_frame(const double* events, int n_events, int kind,
   a.t_scale = t_scale; a.start_old = start_old; a.start_new = start_new; a.delta_t = delta_t;
   a.delta = delta ? 1 : 0; a.out = out; a.pixmask = pixmask;
   hipLaunchKernelGGL(k_events_scatter, dim3((unsigned)((n_events + 255) / 256)), dim3(256), 0, s, a);
+  return mie_check_launch(who);
+}
+
+extern "C" int mie_events_to_frame_bf16(const double* events, int n_events, int kind, int num_bins,
+                                        int height, int width, int pad_left, int pad_right, int pad_top,
+                                        int pad_bottom, double t_scale, double start_old,
+                                        double start_new, double delta_t, int delta, float* sums,
+                                        void* out, uint8_t* pixmask, void* stream) {
+  const char* who = "mie_events_to_frame_bf16";
+  int rc = mie_events_to_frame(events, n_events, kind, num_bins, height, width, pad_left, pad_right, pad_top,
+                               pad_bottom, t_scale, start_old, start_new, delta_t, delta, sums, pixmask, stream);
+  if (rc != MIE_OK) return rc;
+  MIE_REQUIRE(out != nullptr && mie_aligned(out, 8), MIE_ERR_INVALID_ARG, "%s: out must be 8-byte aligned", who);
+  MIE_REQUIRE(out != (void*)sums, MIE_ERR_INVALID_ARG, "%s: out and sums are different buffers", who);
+  const int channels = kind == MIE_EVENTS_HISTOGRAM ? 2 : num_bins;
+  const long long n = (long long)(height + pad_top + pad_bottom) * (width + pad_left + pad_right) * channels;
+  hipLaunchKernelGGL(k_events_round, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, (hipStream_t)stream, sums, n,
+                     reinterpret_cast<mie_bf16*>(out));
   return mie_check_launch(who);
 }

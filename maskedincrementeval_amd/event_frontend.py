@@ -29,11 +29,13 @@ class EventFrames:
     window_size: window length in seconds (the reference's 0.05); t_scale converts the
     event stamps to seconds (1e-9 for the nanosecond stamps of the reference's .npy files);
     pad = (left, right, top, bottom) reflection padding.
+    dtype: element type of the frames handed out -- torch.float32, or torch.bfloat16 for the networks that run
+    on bf16 deltas (the fp32 sums are rounded in the same stream, mie_events_to_frame_bf16).
     """
 
     def __init__(self, width: int, height: int, num_bins: int = 5, evframe_type: str = "voxelgrid",
                  window_size: float = 0.05, t_scale: float = 1e-9, pad: Sequence[int] = (3, 3, 2, 2),
-                 device="cuda:0"):
+                 device="cuda:0", dtype=torch.float32):
         if evframe_type not in ("voxelgrid", "histogram"):
             raise NotImplementedError(evframe_type)
         self.kind = _lib.EVENTS_VOXEL if evframe_type == "voxelgrid" else _lib.EVENTS_HISTOGRAM
@@ -44,10 +46,15 @@ class EventFrames:
         self.device = torch.device(device)
         self.out_h = self.height + self.pad[2] + self.pad[3]
         self.out_w = self.width + self.pad[0] + self.pad[1]
+        if dtype not in (torch.float32, torch.bfloat16):
+            raise NotImplementedError("EventFrames: frames are float32 or bfloat16, not %s" % (dtype,))
+        self.dtype = dtype
         self._events = None
         self._n = 0
-        self._frame = ops.new_nhwc(1, self.channels, self.out_h, self.out_w, self.device)
-        self._delta = ops.new_nhwc(1, self.channels, self.out_h, self.out_w, self.device)
+        self._frame = ops.new_nhwc(1, self.channels, self.out_h, self.out_w, self.device, dtype)
+        self._delta = ops.new_nhwc(1, self.channels, self.out_h, self.out_w, self.device, dtype)
+        # bf16 frames: the fp32 sums the scatter accumulates (float atomics), kept beside the rounded frame
+        self._sums = ops.new_nhwc(1, self.channels, self.out_h, self.out_w, self.device) if dtype != torch.float32 else None
         self._mask = torch.zeros((1, 1, self.out_h, self.out_w), dtype=torch.uint8, device=self.device)
         self._fmask = torch.zeros_like(self._mask)
 
@@ -65,11 +72,14 @@ class EventFrames:
         if self._events is None:
             raise RuntimeError("EventFrames: call set_events first")
         stream = torch.cuda.current_stream(self.device).cuda_stream
-        check(lib().mie_events_to_frame(
-            self._events.data_ptr() if self._n else None, self._n, self.kind, self.num_bins, self.height,
-            self.width, self.pad[0], self.pad[1], self.pad[2], self.pad[3], self.t_scale, float(start_old),
-            float(start_new), self.window_size, 1 if delta else 0, ops.nhwc_ptr(out, "out"), mask.data_ptr(),
-            stream))
+        head = (self._events.data_ptr() if self._n else None, self._n, self.kind, self.num_bins, self.height,
+                self.width, self.pad[0], self.pad[1], self.pad[2], self.pad[3], self.t_scale, float(start_old),
+                float(start_new), self.window_size, 1 if delta else 0)
+        if self._sums is None:
+            check(lib().mie_events_to_frame(*head, ops.nhwc_ptr(out, "out"), mask.data_ptr(), stream))
+        else:
+            check(lib().mie_events_to_frame_bf16(*head, ops.nhwc_ptr(self._sums, "sums"), ops.nhwc_ptr(out, "out", dtype=self.dtype),
+                                                 mask.data_ptr(), stream))
 
     def frame(self, start: float) -> torch.Tensor:
         """Dense (1, C, H', W') channels_last frame of the window (start, start + window_size)."""

@@ -49,6 +49,30 @@ def test_frames_and_deltas_match_oracle(kind, width, height, pad, n_events):
     assert np.allclose(total, eo.frame(ev, kind, 5, height, width, 0.05, starts[-1], pad=pad)[0], rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("kind", ["voxelgrid", "histogram"])
+@pytest.mark.parametrize("width,height,pad", [(346, 260, (3, 3, 2, 2)), (33, 21, (0, 0, 0, 0)), (13, 7, (2, 1, 3, 0))])
+def test_bf16_frames_are_the_rounded_fp32_sums(kind, width, height, pad):
+    # mie_events_to_frame_bf16: the fp32 sums as the plain entry point leaves them (against the oracle) and, in the
+    # same call, every element rounded to nearest even (exactly what .to(bfloat16) makes of those sums)
+    pol = (0.0, 1.0) if kind == "voxelgrid" else (-1.0, 1.0)
+    ev = random_events(20000, width, height, 0.0, 0.08, seed=width, density=0.3, polarity=pol)
+    fe = EventFrames(width, height, num_bins=5, evframe_type=kind, window_size=0.05, pad=pad, device=DEV, dtype=torch.bfloat16)
+    fe.set_events(ev)
+    got = fe.frame(0.01)
+    torch.cuda.synchronize()
+    assert got.dtype == torch.bfloat16 and got.permute(0, 2, 3, 1).is_contiguous()
+    want, wmask = eo.frame(ev, kind, 5, height, width, 0.05, 0.01, pad=pad)
+    assert np.allclose(_nchw(fe._sums), want, rtol=RTOL, atol=ATOL)
+    assert torch.equal(got, fe._sums.to(torch.bfloat16))
+    assert np.array_equal(fe._fmask[0, 0].cpu().numpy(), wmask)
+    d, m = fe.delta(0.01, 0.0125)
+    torch.cuda.synchronize()
+    wd, wm = eo.frame_delta(ev, kind, 5, height, width, 0.05, 0.01, 0.0125, pad=pad)
+    assert np.allclose(_nchw(fe._sums), wd, rtol=RTOL, atol=ATOL)
+    assert torch.equal(d, fe._sums.to(torch.bfloat16)) and np.array_equal(m[0, 0].cpu().numpy(), wm)
+    assert not (_nchw(d.float())[:, wm == 0] != 0).any()
+
+
 def test_empty_and_errors():
     fe = EventFrames(32, 16, device=DEV)
     with pytest.raises(RuntimeError, match="set_events"):
@@ -62,6 +86,8 @@ def test_empty_and_errors():
     bad.set_events(np.zeros((1, 4)))
     with pytest.raises(RuntimeError, match="padding"):
         bad.frame(0.0)
+    with pytest.raises(NotImplementedError):
+        EventFrames(32, 16, device=DEV, dtype=torch.float16)
 
 
 def test_delta_feeds_the_incremental_network():
