@@ -216,8 +216,13 @@ int mie_conv_f32x3_takes(int k, int stride, int c1, int c2, int cout);
  *                                         out_delta = act(r1) - act(r0)
  * (the fused form of nnConvIncr followed by nnReservedActivation).
  * Stale tiles of `out` are zeroed in out_delta.  Inactive input pixels are
- * never read.  addend (optional, [n, h_out, w_out, cout]) is added to acc first:
- * a clean delta whose active pixels are covered by `out` -- the residual of a
+ * never read.  out->pixmask must hold every output pixel whose window contains
+ * an active input pixel (mie_build_mask_tiles / mie_build_mask_plan make exactly
+ * that set; a superset is fine): at the other pixels of an active tile acc is
+ * zero by construction, and the matrix-core kernels write out_delta = 0 there
+ * without touching the reservoir.  addend (optional, [n, h_out, w_out, cout]) is
+ * added to acc first:
+ * a clean delta whose active pixels lie in out->pixmask -- the residual of a
  * residual block, or the contribution of a few extra input channels computed
  * by another launch (conv over a concat = sum of convs over its parts).
  *   x  : [n, h_in, w_in, c1] delta with pixel mask xmask (NULL = all active),

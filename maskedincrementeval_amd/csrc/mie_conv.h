@@ -110,6 +110,10 @@ static __device__ __forceinline__ void conv_epilogue_store(const ConvArgsT<T>& a
 
 // The same for N groups of four adjacent output channels of one pixel each (off[i] = offset of the first of
 // the four, a multiple of 4; co[i] its channel): 16-byte reservoir accesses, 16- / 8-byte delta accesses.
+// Pixels of an active tile that lie outside the output pixel mask (live[i] false; the mask covers every pixel whose
+// window holds an active input pixel, so acc and addend are exactly zero there) keep their reservoir untouched -- r1 =
+// r0 + 0 would store the value just read -- and get a zero delta: conv_epilogue_load4 fetches nothing for them
+// (pass live as its ok), conv_epilogue_store4 writes the zeros.  A dense refresh treats every pixel as live.
 template <typename T, int N>
 static __device__ __forceinline__ void conv_epilogue_load4(const ConvArgsT<T>& a, const long long (&off)[N],
                                                            const bool (&ok)[N], float4 (&r0)[N], float4 (&add)[N]) {
@@ -129,10 +133,14 @@ template <typename T, int N>
 static __device__ __forceinline__ void conv_epilogue_store4(const ConvArgsT<T>& a, const long long (&off)[N],
                                                             const int (&co)[N], const bool (&ok)[N],
                                                             const float4 (&acc)[N], const float4 (&r0)[N],
-                                                            const float4 (&add)[N]) {
+                                                            const float4 (&add)[N], const bool (&live)[N]) {
 #pragma unroll
   for (int i = 0; i < N; ++i) {
     if (!ok[i]) continue;
+    if (!live[i]) {
+      mie_st4(a.out, off[i], make_float4(0.f, 0.f, 0.f, 0.f));
+      continue;
+    }
     float4 v = make_float4(acc[i].x + add[i].x, acc[i].y + add[i].y, acc[i].z + add[i].z, acc[i].w + add[i].w);
     if (a.refresh) {
       if (a.bias) {
@@ -153,6 +161,14 @@ static __device__ __forceinline__ void conv_epilogue_store4(const ConvArgsT<T>& 
       mie_st4(a.out, off[i], v);
     }
   }
+}
+
+template <typename T, int N>
+static __device__ __forceinline__ void conv_epilogue_store4(const ConvArgsT<T>& a, const long long (&off)[N],
+                                                            const int (&co)[N], const bool (&ok)[N],
+                                                            const float4 (&acc)[N], const float4 (&r0)[N],
+                                                            const float4 (&add)[N]) {
+  conv_epilogue_store4<T, N>(a, off, co, ok, acc, r0, add, ok);
 }
 
 template <typename T, int N>

@@ -54,6 +54,16 @@ __global__ __launch_bounds__(256) void k_conv_fewcin(ConvArgsT<T> a) {
     return;
   }
 
+  // pixels of this thread's two epilogue groups that lie in the output pixel mask (elsewhere the sums are exactly
+  // zero: no reservoir access, a zero delta); the bytes are asked for before the staging loads
+  bool live[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int p = (tid + 256 * i) >> 3;
+    const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
+    live[i] = oy < hout && ox < wout && (a.refresh || a.ts.pixmask[((long long)n * hout + oy) * wout + ox] != 0);
+  }
+
   // ---- stage the input tile (fp32, 8 channels per pixel) and the filter slab ---------------------
   // Every global load of the thread is issued before the first LDS store (compile-time trip counts, fully
   // unrolled): one memory round trip for the whole staging instead of one per loop iteration.
@@ -145,8 +155,8 @@ __global__ __launch_bounds__(256) void k_conv_fewcin(ConvArgsT<T> a) {
     const float4 s1 = *reinterpret_cast<const float4*>(&smem[64 * 32 + 4 * idx]);
     v[i] = make_float4(s0.x + s1.x, s0.y + s1.y, s0.z + s1.z, s0.w + s1.w);
   }
-  conv_epilogue_load4<T, 2>(a, off, ok, r0, add);
-  conv_epilogue_store4<T, 2>(a, off, co, ok, v, r0, add);
+  conv_epilogue_load4<T, 2>(a, off, live, r0, add);
+  conv_epilogue_store4<T, 2>(a, off, co, ok, v, r0, add, live);
 }
 
 template <typename T>

@@ -142,7 +142,8 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 #endif
 __host__ __device__ constexpr int conv_min_waves(int elem_size, int K, int S, bool HALF, bool GATES, bool UP, bool SPLIT,
                                                  bool X3) {
-  return (elem_size == 2 && S == 2 && K == 5 && !HALF && !GATES && !UP && !SPLIT && !X3) ? MIE_S2_WAVES : 1;
+  if (X3) return 2;      // 64 accumulator registers: the three-term kernels sit at the edge of two waves per SIMD
+  return (elem_size == 2 && S == 2 && K == 5 && !HALF && !GATES && !UP && !SPLIT) ? MIE_S2_WAVES : 1;
 }
 
 // One unit of the contraction on the matrix core: the 16 bytes of A and of B a lane holds.
@@ -394,8 +395,19 @@ __global__ __launch_bounds__(256, conv_min_waves((int)sizeof(T), K, S, HALF, GAT
   constexpr int PB = PER > 4 ? 4 : PER;                      // groups per pass of the epilogue (registers)
   long long e_off[PB];
   int e_co[PB];
-  bool e_ok[PB];
+  bool e_ok[PB], e_live[PB];
   float4 e_r0[PB], e_add[PB];
+  // bit g: group g of this thread lies on a pixel of the output pixel mask.  Elsewhere in an active tile the sums are
+  // exactly zero: no reservoir access, a zero delta.  (The bytes are asked for here, long before the epilogue needs them.)
+  unsigned live_bits = 0u;
+  if (!GATES && !SPLIT) {
+#pragma unroll
+    for (int g = 0; g < PER; ++g) {
+      const int p = (tid + 256 * g) / QPP;
+      const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
+      if (oy < hout && ox < wout && (a.refresh || a.ts.pixmask[((long long)n * hout + oy) * wout + ox] != 0)) live_bits |= 1u << g;
+    }
+  }
   // (bf16: a workgroup's contraction is too short to be worth the registers that hold these values
   // through it -- they cost a resident workgroup per CU -- so they are fetched after it instead; the same
   // holds for the 128-column slabs, whose threads own 8 groups.)
@@ -408,10 +420,11 @@ __global__ __launch_bounds__(256, conv_min_waves((int)sizeof(T), K, S, HALF, GAT
       const int p = idx / QPP, col = 4 * (idx - p * QPP);
       const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
       e_ok[i] = oy < hout && ox < wout;
+      e_live[i] = SPLIT ? e_ok[i] : ((live_bits >> (h0 + i)) & 1u) != 0;
       e_off[i] = (((long long)n * hout + oy) * wout + ox) * a.cout + co0 + col;
       e_co[i] = co0 + col;
     }
-    if (!SPLIT) conv_epilogue_load4<T, PB>(a, e_off, e_ok, e_r0, e_add);
+    if (!SPLIT) conv_epilogue_load4<T, PB>(a, e_off, e_live, e_r0, e_add);
   };
   if (!GATES && EARLY && !SPLIT) epilogue_fetch(0);
 
@@ -962,7 +975,7 @@ __global__ __launch_bounds__(256, conv_min_waves((int)sizeof(T), K, S, HALF, GAT
         for (int i = 0; i < PB; ++i)
           if (e_ok[i]) *reinterpret_cast<float4*>(plane + e_off[i]) = v[i];
       } else {
-        conv_epilogue_store4<T, PB>(a, e_off, e_co, e_ok, v, e_r0, e_add);
+        conv_epilogue_store4<T, PB>(a, e_off, e_co, e_ok, v, e_r0, e_add, e_live);
       }
     }
   }

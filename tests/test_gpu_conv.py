@@ -501,7 +501,9 @@ def test_small_planes_split_the_contraction(c1, c2, cout, h, w, s, dtype, k, f32
     for step, (dens, with_res) in enumerate([(0.3, False), (0.05, True), (0.6, True)]):
         d, m = gaussian_delta(n, cin, h, w, dens, 0.5, seed=300 + step)
         d = q(d)
-        add = q(gaussian_delta(n, cout, ho, wo, 1.0, 0.3, seed=400 + step)[0]) if with_res else None
+        foot = torch.from_numpy(mo.footprint_conv(m[:, 0].numpy(), k, s, k // 2)).bool().unsqueeze(1)
+        # an addend is a clean delta on pixels of the output mask
+        add = q(gaussian_delta(n, cout, ho, wo, 1.0, 0.3, seed=400 + step)[0]) * foot if with_res else None
         ref = io.conv_incr(d, wt, s, k // 2)
         dm = m.to(DEV)
         ops.build_mask_tiles(dm, None, n, h, w, _lib.FOOT_CONV, k, s, k // 2, ts)
@@ -515,10 +517,7 @@ def test_small_planes_split_the_contraction(c1, c2, cout, h, w, s, dtype, k, f32
         torch.cuda.synchronize()
         got, plain = out.float().cpu(), out_plain.float().cpu()
         if with_res:
-            tiles = torch.from_numpy(mo.footprint_conv(m[:, 0].numpy(), k, s, k // 2)).bool()
-            tiles = torch.nn.functional.max_pool2d(tiles.float().unsqueeze(1), 8, 8, ceil_mode=True)
-            tiles = torch.nn.functional.interpolate(tiles, scale_factor=8)[:, :, :ho, :wo].bool()
-            acc = torch.where(tiles, ref + add, torch.zeros_like(ref))      # the addend counts on whole active tiles
+            acc = ref + add
             want = torch.relu(res_ref + acc) - torch.relu(res_ref)
             res_ref = res_ref + acc
         else:
