@@ -524,6 +524,23 @@ int mie_conv_gates_masked(const void* x, const uint8_t* xmask, int c1,
                           void* c_delta, int dtype, void* stream);
 
 /*
+ * mie_conv_gates_masked with a workspace.  On planes of few tiles (tiles x 4*hid/32 <= 128, inputs at least 4 staging
+ * chunks deep) the contraction runs as a split 3x3 conv of the two inputs -- up to 8 workgroups per (tile, 32-column
+ * slab) write fp32 partial sums of the gate columns to the workspace -- and a second kernel adds them in a fixed order
+ * and runs the gate chain.  workspace NULL (workspace_bytes 0): exactly mie_conv_gates_masked.  Workspace rules as
+ * in mie_conv_masked_ws.  No counterpart in the reference (incr_modules/e2depth_incr.py:100-120 is one conv launch).
+ */
+int mie_conv_gates_masked_ws(const void* x, const uint8_t* xmask, int c1,
+                             const void* x2, const uint8_t* x2mask, int c2,
+                             int h_in, int w_in, const float* filter,
+                             const void* filter_mc, int cin_total, int hid,
+                             const mie_tileset* out, float* gates_res,
+                             const void* cprev_delta, const uint8_t* cprev_mask,
+                             float* cprev_res, float* cell_res, void* h_delta,
+                             void* c_delta, int dtype, void* workspace,
+                             long long workspace_bytes, void* stream);
+
+/*
  * Dense refresh of a ConvLSTM cell after its gates conv: gates_res
  * ([n,h,w,4*hid] fp32) holds the gate pre-activations mie_conv_refresh wrote --
  * in the order [in | remember | out | cell] x hid, or (interleaved != 0) in the
@@ -623,6 +640,21 @@ int mie_upconv_masked(const void* a, const uint8_t* amask, const void* b,
                       int k, int pad, int cout, const mie_tileset* out,
                       void* out_delta, const void* addend, float* reservoir,
                       int act_kind, float slope, int dtype, void* stream);
+
+/*
+ * mie_upconv_masked with a workspace, as mie_conv_masked_ws is to mie_conv_masked: on planes of few tiles (tiles x
+ * cout/32 <= 128, c at least 4 staging chunks) the contraction of each (tile, 32-channel slab) is split over up to 8
+ * workgroups that write fp32 partial sums to the workspace, and a second kernel adds them in a fixed order and runs the
+ * epilogue.  workspace NULL (workspace_bytes 0): exactly mie_upconv_masked.  The few-channel form is never split.
+ * No counterpart in the reference (one launch per conv whatever its size, incr_modules/e2depth_incr.py:306-313).
+ */
+int mie_upconv_masked_ws(const void* a, const uint8_t* amask, const void* b,
+                         const uint8_t* bmask, int c, int h_in, int w_in,
+                         const float* filter, const void* filter_mc, int cin_total,
+                         int k, int pad, int cout, const mie_tileset* out,
+                         void* out_delta, const void* addend, float* reservoir,
+                         int act_kind, float slope, int dtype, void* workspace,
+                         long long workspace_bytes, void* stream);
 
 /*
  * Masked transposed convolution of a delta (stride s, padding p; the output

@@ -412,6 +412,8 @@ int conv_impl(const char* who, const T* x, const uint8_t* xmask, int c1, const T
     a.hid = gates->hid; a.g_cpd = gates->cprev_delta; a.g_cpm = gates->cprev_mask;
     a.g_cpres = gates->cprev_res; a.g_cres = gates->cell_res; a.g_dh = gates->h_delta;
     a.g_dc = gates->c_delta;
+    a.ws = (float*)workspace;
+    a.ws_floats = workspace_bytes / 4;
     MIE_REQUIRE(mie_launch_conv_gates_mfma(a, cap, st), MIE_ERR_UNSUPPORTED,
                 "%s: no kernel variant for cout=%d", who, cout);
     return mie_check_launch(who);
@@ -695,8 +697,8 @@ int conv_gates_entry(const char* who, const void* x, const uint8_t* xmask, int c
                      const uint8_t* x2mask, int c2, int h_in, int w_in, const float* filter,
                      const void* filter_mc, int cin_total, int hid, const mie_tileset* out,
                      float* gates_res, const void* cprev_delta, const uint8_t* cprev_mask,
-                     float* cprev_res, float* cell_res, void* h_delta, void* c_delta, void* stream,
-                     bool x3 = false) {
+                     float* cprev_res, float* cell_res, void* h_delta, void* c_delta, void* workspace,
+                     long long workspace_bytes, void* stream, bool x3 = false) {
   MIE_REQUIRE(hid > 0 && hid <= (1 << 20), MIE_ERR_INVALID_ARG, "%s: hid = %d out of range", who, hid);
   MIE_REQUIRE(gates_res && cprev_res && cell_res && h_delta && c_delta, MIE_ERR_INVALID_ARG,
               "%s: NULL pointer", who);
@@ -710,7 +712,7 @@ int conv_gates_entry(const char* who, const void* x, const uint8_t* xmask, int c
   g.cell_res = cell_res; g.h_delta = (T*)h_delta; g.c_delta = (T*)c_delta;
   return conv_impl<T>(who, (const T*)x, xmask, c1, (const T*)x2, x2mask, c2, h_in, w_in, filter,
                       (const T*)filter_mc, cin_total, 3, 1, 1, 4 * hid, out, (T*)nullptr, (const T*)nullptr,
-                      gates_res, MIE_ACT_NONE, 0.f, MIE_PATH_MFMA, false, nullptr, stream, &g, nullptr, 0, x3);
+                      gates_res, MIE_ACT_NONE, 0.f, MIE_PATH_MFMA, false, nullptr, stream, &g, workspace, workspace_bytes, x3);
 }
 
 int tconv_entry(const char* who, const void* x, const uint8_t* xmask, int cin, int h_in, int w_in,
@@ -765,7 +767,7 @@ template <typename T>
 int upconv_entry(const char* who, const void* a_lo, const uint8_t* amask, const void* b_lo, const uint8_t* bmask,
                  int c, int h_lo, int w_lo, const float* filter, const void* filter_mc, int cin_total, int k,
                  int pad, int cout, const mie_tileset* out, void* out_delta, const void* addend, float* reservoir,
-                 int act_kind, float slope, void* stream, bool x3 = false) {
+                 int act_kind, float slope, void* workspace, long long workspace_bytes, void* stream, bool x3 = false) {
   int rc = mie_check_tileset(out, who);
   if (rc != MIE_OK) return rc;
   MIE_REQUIRE(a_lo && filter, MIE_ERR_INVALID_ARG, "%s: NULL pointer (a and filter are required)", who);
@@ -790,6 +792,11 @@ int upconv_entry(const char* who, const void* a_lo, const uint8_t* amask, const 
                   mie_aligned(addend, 16),
               MIE_ERR_INVALID_ARG, "%s: a / b / filter / filter_mc / addend must be 16-byte aligned", who);
   MIE_REQUIRE(addend == nullptr || addend != out_delta, MIE_ERR_INVALID_ARG, "%s: addend must not alias out_delta", who);
+  MIE_REQUIRE(workspace_bytes >= 0 && (workspace != nullptr || workspace_bytes == 0) && mie_aligned(workspace, 16),
+              MIE_ERR_INVALID_ARG, "%s: workspace must be 16-byte aligned, with a size >= 0 (0 if NULL)", who);
+  MIE_REQUIRE(workspace == nullptr || (workspace != out_delta && workspace != (void*)reservoir && workspace != a_lo &&
+                                       workspace != b_lo && workspace != addend),
+              MIE_ERR_INVALID_ARG, "%s: workspace must not alias an operand", who);
   rc = check_epilogue(who, out_delta, reservoir, act_kind, false);
   if (rc != MIE_OK) return rc;
   ConvArgsT<T> a;
@@ -799,7 +806,8 @@ int upconv_entry(const char* who, const void* a_lo, const uint8_t* amask, const 
   a.slope = slope; a.addend = (const T*)addend; a.refresh = 0; a.bias = nullptr;
   a.hid = 0; a.g_cpd = nullptr; a.g_cpm = nullptr; a.g_cpres = nullptr; a.g_cres = nullptr;
   a.g_dh = nullptr; a.g_dc = nullptr;
-  a.ws = nullptr; a.ws_floats = 0; a.ws_plane = 0; a.xcd_fs = 0; a.x3 = (x3 && !few) ? 1 : 0;
+  a.ws = few ? nullptr : (float*)workspace; a.ws_floats = few ? 0 : workspace_bytes / 4; a.ws_plane = 0; a.xcd_fs = 0;
+  a.x3 = (x3 && !few) ? 1 : 0;
   a.ts = mie_dev_tileset(out);
   const unsigned cap = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
   if (few) {
@@ -813,19 +821,51 @@ int upconv_entry(const char* who, const void* a_lo, const uint8_t* amask, const 
 }
 }  // namespace
 
-extern "C" int mie_upconv_masked(const void* a, const uint8_t* amask, const void* b, const uint8_t* bmask, int c,
-                                 int h_in, int w_in, const float* filter, const void* filter_mc, int cin_total,
-                                 int k, int pad, int cout, const mie_tileset* out, void* out_delta,
-                                 const void* addend, float* reservoir, int act_kind, float slope, int dtype,
-                                 void* stream) {
+extern "C" int mie_upconv_masked_ws(const void* a, const uint8_t* amask, const void* b, const uint8_t* bmask, int c,
+                                    int h_in, int w_in, const float* filter, const void* filter_mc, int cin_total,
+                                    int k, int pad, int cout, const mie_tileset* out, void* out_delta,
+                                    const void* addend, float* reservoir, int act_kind, float slope, int dtype,
+                                    void* workspace, long long workspace_bytes, void* stream) {
   const char* who = "mie_upconv_masked";
   bool x3 = false;
   MIE_CONV_DTYPE_X3_OK(dtype, who, x3);
   if (dtype == MIE_DTYPE_BF16)
     return upconv_entry<mie_bf16>(who, a, amask, b, bmask, c, h_in, w_in, filter, filter_mc, cin_total, k, pad, cout,
-                                  out, out_delta, addend, reservoir, act_kind, slope, stream);
+                                  out, out_delta, addend, reservoir, act_kind, slope, workspace, workspace_bytes, stream);
   return upconv_entry<float>(who, a, amask, b, bmask, c, h_in, w_in, filter, filter_mc, cin_total, k, pad, cout, out,
-                             out_delta, addend, reservoir, act_kind, slope, stream, x3);
+                             out_delta, addend, reservoir, act_kind, slope, workspace, workspace_bytes, stream, x3);
+}
+
+extern "C" int mie_upconv_masked(const void* a, const uint8_t* amask, const void* b, const uint8_t* bmask, int c,
+                                 int h_in, int w_in, const float* filter, const void* filter_mc, int cin_total,
+                                 int k, int pad, int cout, const mie_tileset* out, void* out_delta,
+                                 const void* addend, float* reservoir, int act_kind, float slope, int dtype,
+                                 void* stream) {
+  return mie_upconv_masked_ws(a, amask, b, bmask, c, h_in, w_in, filter, filter_mc, cin_total, k, pad, cout, out,
+                              out_delta, addend, reservoir, act_kind, slope, dtype, nullptr, 0, stream);
+}
+
+extern "C" int mie_conv_gates_masked_ws(const void* x, const uint8_t* xmask, int c1, const void* x2,
+                                        const uint8_t* x2mask, int c2, int h_in, int w_in,
+                                        const float* filter, const void* filter_mc, int cin_total,
+                                        int hid, const mie_tileset* out, float* gates_res,
+                                        const void* cprev_delta, const uint8_t* cprev_mask,
+                                        float* cprev_res, float* cell_res, void* h_delta,
+                                        void* c_delta, int dtype, void* workspace, long long workspace_bytes,
+                                        void* stream) {
+  const char* who = "mie_conv_gates_masked";
+  bool x3 = false;
+  MIE_CONV_DTYPE_X3_OK(dtype, who, x3);
+  MIE_REQUIRE(workspace == nullptr || (workspace != (void*)gates_res && workspace != (void*)cprev_res && workspace != (void*)cell_res &&
+                                       workspace != h_delta && workspace != c_delta && workspace != cprev_delta),
+              MIE_ERR_INVALID_ARG, "%s: workspace must not alias an operand", who);
+  if (dtype == MIE_DTYPE_BF16)
+    return conv_gates_entry<mie_bf16>(who, x, xmask, c1, x2, x2mask, c2, h_in, w_in, filter, filter_mc,
+                                      cin_total, hid, out, gates_res, cprev_delta, cprev_mask, cprev_res,
+                                      cell_res, h_delta, c_delta, workspace, workspace_bytes, stream);
+  return conv_gates_entry<float>(who, x, xmask, c1, x2, x2mask, c2, h_in, w_in, filter, filter_mc, cin_total,
+                                 hid, out, gates_res, cprev_delta, cprev_mask, cprev_res, cell_res, h_delta,
+                                 c_delta, workspace, workspace_bytes, stream, x3);
 }
 
 extern "C" int mie_conv_gates_masked(const void* x, const uint8_t* xmask, int c1, const void* x2,
@@ -835,14 +875,7 @@ extern "C" int mie_conv_gates_masked(const void* x, const uint8_t* xmask, int c1
                                      const void* cprev_delta, const uint8_t* cprev_mask,
                                      float* cprev_res, float* cell_res, void* h_delta,
                                      void* c_delta, int dtype, void* stream) {
-  const char* who = "mie_conv_gates_masked";
-  bool x3 = false;
-  MIE_CONV_DTYPE_X3_OK(dtype, who, x3);
-  if (dtype == MIE_DTYPE_BF16)
-    return conv_gates_entry<mie_bf16>(who, x, xmask, c1, x2, x2mask, c2, h_in, w_in, filter, filter_mc,
-                                      cin_total, hid, out, gates_res, cprev_delta, cprev_mask, cprev_res,
-                                      cell_res, h_delta, c_delta, stream);
-  return conv_gates_entry<float>(who, x, xmask, c1, x2, x2mask, c2, h_in, w_in, filter, filter_mc, cin_total,
-                                 hid, out, gates_res, cprev_delta, cprev_mask, cprev_res, cell_res, h_delta,
-                                 c_delta, stream, x3);
+  return mie_conv_gates_masked_ws(x, xmask, c1, x2, x2mask, c2, h_in, w_in, filter, filter_mc, cin_total, hid, out,
+                                  gates_res, cprev_delta, cprev_mask, cprev_res, cell_res, h_delta, c_delta, dtype,
+                                  nullptr, 0, stream);
 }

@@ -237,6 +237,35 @@ __device__ __forceinline__ float4 f32_to_slot(const float (&f)[8], mie_bf16) {
   return make_float4(r4[0], r4[1], r4[2], r4[3]);
 }
 
+// The gate chain of one item of a gates conv -- pixel `pix`, four adjacent hidden channels whose state values start at
+// element `ho` and whose 16 gate columns start at element `go` of the gate reservoir -- given the conv sums dg of those
+// columns: reservoirs updated, state deltas written.
+template <typename T>
+__device__ __forceinline__ void conv_gates_item(const ConvArgsT<T>& a, long long pix, long long ho, long long go, const float4 (&dg)[4]) {
+  const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+  float4 rr[4];
+  float4* gr = reinterpret_cast<float4*>(a.res + go);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) rr[j] = gr[j];
+  const bool has_cp = a.g_cpd != nullptr && (a.g_cpm == nullptr || a.g_cpm[pix]);
+  const float4 dP4 = has_cp ? mie_ld4(a.g_cpd, ho) : zero4;
+  const float4 cp4 = *reinterpret_cast<const float4*>(a.g_cpres + ho);
+  const float4 cc4 = *reinterpret_cast<const float4*>(a.g_cres + ho);
+  float cp[4] = {cp4.x, cp4.y, cp4.z, cp4.w}, cc[4] = {cc4.x, cc4.y, cc4.z, cc4.w};
+  const float dP[4] = {dP4.x, dP4.y, dP4.z, dP4.w};
+  float dh[4], dc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    mie_lstm_gate_chain(rr[j].x, rr[j].y, rr[j].z, rr[j].w, dg[j].x, dg[j].y, dg[j].z, dg[j].w, cp[j], dP[j], cc[j],
+                        dh[j], dc[j]);
+    gr[j] = rr[j];
+  }
+  if (has_cp) *reinterpret_cast<float4*>(a.g_cpres + ho) = make_float4(cp[0], cp[1], cp[2], cp[3]);
+  *reinterpret_cast<float4*>(a.g_cres + ho) = make_float4(cc[0], cc[1], cc[2], cc[3]);
+  mie_st4(a.g_dh, ho, make_float4(dh[0], dh[1], dh[2], dh[3]));
+  mie_st4(a.g_dc, ho, make_float4(dc[0], dc[1], dc[2], dc[3]));
+}
+
 // UP: the conv input is up2x(x + x2), the bilinear x2 up-sampling of the sum of two deltas given at
 // half resolution (x2 optional), and is never formed in memory: per chunk the 8x8 block of source
 // pixels a tile's 12x12 input window blends is summed into LDS (fp32), and the staged tile is expanded
@@ -361,7 +390,7 @@ __global__ __launch_bounds__(256, conv_min_waves((int)sizeof(T), K, S, HALF, GAT
   const int hout = a.ts.h, wout = a.ts.w;
   const int cout = a.cout;
 
-  static_assert(!SPLIT || (WN == 1 && !GATES && !UP), "the split form is the plain 32-channel slab kernel");
+  static_assert(!SPLIT || (WN == 1 && !GATES), "the split form is a 32-channel slab kernel (the gates conv splits as a plain conv)");
   if (SPLIT && tk == 2) return;      // stale tiles are zeroed by k_conv_split_finish
   if (GATES && tk == 2) {  // stale tile: zero the hidden / cell deltas of this workgroup's hidden channels
     constexpr int HG = CO_BLK / 16;          // groups of four hidden channels
@@ -911,11 +940,9 @@ __global__ __launch_bounds__(256, conv_min_waves((int)sizeof(T), K, S, HALF, GAT
         mie_st4(a.g_dc, ho, zero4);
         continue;
       }
-      float4 dg[4], rr[4];
-      float4* gr = reinterpret_cast<float4*>(a.res + pix * a.cout + co0 + 16 * g4);
+      float4 dg[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        rr[j] = gr[j];
         dg[j] = *reinterpret_cast<const float4*>(&smem[p * CO_BLK + 16 * g4 + 4 * j]);
 #pragma unroll
         for (int k2 = 1; k2 < WK; ++k2) {
@@ -923,23 +950,7 @@ __global__ __launch_bounds__(256, conv_min_waves((int)sizeof(T), K, S, HALF, GAT
           dg[j].x += part.x; dg[j].y += part.y; dg[j].z += part.z; dg[j].w += part.w;
         }
       }
-      const bool has_cp = a.g_cpd != nullptr && (a.g_cpm == nullptr || a.g_cpm[pix]);
-      const float4 dP4 = has_cp ? mie_ld4(a.g_cpd, ho) : zero4;
-      const float4 cp4 = *reinterpret_cast<const float4*>(a.g_cpres + ho);
-      const float4 cc4 = *reinterpret_cast<const float4*>(a.g_cres + ho);
-      float cp[4] = {cp4.x, cp4.y, cp4.z, cp4.w}, cc[4] = {cc4.x, cc4.y, cc4.z, cc4.w};
-      const float dP[4] = {dP4.x, dP4.y, dP4.z, dP4.w};
-      float dh[4], dc[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        mie_lstm_gate_chain(rr[j].x, rr[j].y, rr[j].z, rr[j].w, dg[j].x, dg[j].y, dg[j].z, dg[j].w, cp[j], dP[j], cc[j],
-                            dh[j], dc[j]);
-        gr[j] = rr[j];
-      }
-      if (has_cp) *reinterpret_cast<float4*>(a.g_cpres + ho) = make_float4(cp[0], cp[1], cp[2], cp[3]);
-      *reinterpret_cast<float4*>(a.g_cres + ho) = make_float4(cc[0], cc[1], cc[2], cc[3]);
-      mie_st4(a.g_dh, ho, make_float4(dh[0], dh[1], dh[2], dh[3]));
-      mie_st4(a.g_dc, ho, make_float4(dc[0], dc[1], dc[2], dc[3]));
+      conv_gates_item<T>(a, pix, ho, pix * a.cout + co0 + 16 * g4, dg);
     }
   } else {
     // the last barrier of the main loop has retired every read of the staging buffers that is used
@@ -1019,30 +1030,83 @@ __global__ __launch_bounds__(256) void k_conv_split_finish(ConvArgsT<T> a, int p
   }
 }
 
+// Second half of a split gates conv: per active tile the partial planes of the 4 * hid gate columns are added in
+// order and the ConvLSTM gate chain runs on the sums; stale tiles get zero state deltas.  One thread per (pixel, four
+// adjacent hidden channels), blockIdx.y over groups of hidden channels.
+template <typename T>
+__global__ __launch_bounds__(256) void k_gates_split_finish(ConvArgsT<T> a, int parts) {
+  int n, y0, x0;
+  const int tk = mie_pick_tile(a.ts, blockIdx.x + conv_args_entry_zero(a), n, y0, x0);
+  if (tk == 0) return;
+  const int hout = a.ts.h, wout = a.ts.w, hid = a.hid;
+  const int hg_all = hid / 4;                                         // groups of four hidden channels
+  const int hgb = (hg_all + (int)gridDim.y - 1) / (int)gridDim.y;      // groups of this block
+  const int g_lo = (int)blockIdx.y * hgb;
+  const int gn = (hg_all - g_lo < hgb) ? hg_all - g_lo : hgb;
+  const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int idx = threadIdx.x; idx < 64 * gn; idx += 256) {
+    const int p = idx / gn, g4 = g_lo + (idx - p * gn);
+    const int oy = y0 + (p >> 3), ox = x0 + (p & 7);
+    if (oy >= hout || ox >= wout) continue;
+    const long long pix = ((long long)n * hout + oy) * wout + ox;
+    const long long ho = pix * hid + 4 * g4;
+    if (tk == 2 || !a.ts.pixmask[pix]) {
+      mie_st4(a.g_dh, ho, zero4);
+      mie_st4(a.g_dc, ho, zero4);
+      continue;
+    }
+    const long long go = pix * a.cout + 16 * g4;
+    float4 dg[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      dg[j] = *reinterpret_cast<const float4*>(a.ws + go + 4 * j);
+      for (int q = 1; q < parts; ++q) {
+        const float4 part = *reinterpret_cast<const float4*>(a.ws + (long long)q * a.ws_plane + go + 4 * j);
+        dg[j].x += part.x; dg[j].y += part.y; dg[j].z += part.z; dg[j].w += part.w;
+      }
+    }
+    conv_gates_item<T>(a, pix, ho, go, dg);
+  }
+}
+
 // A launch is split when it has at most 128 workgroups, at least 4 staged chunks and a workspace:
 // into the largest power of two of parts (up to 8) that keeps the launch at 256 workgroups or fewer (one
 // per CU: measured on MI355X, a second workgroup per CU costs more in per-workgroup set-up than it gains),
 // leaves every part a chunk, and fits the workspace.  Returns false when the launch is not split.
-template <typename T, int K, int S>
-bool launch_split(const ConvArgsT<T>& a0, unsigned cap, hipStream_t st) {
-  constexpr int CC = stage_channels(K, S, false) * (4 / (int)sizeof(T));
-  if (a0.ws == nullptr || a0.refresh || a0.cout % 32 != 0 || a0.c1 % CC != 0 || a0.c2 % CC != 0) return false;
-  const long long groups = (long long)cap * (a0.cout / 32);
-  const int nch = (a0.c1 + a0.c2) / CC;
+// Number of parts (0: the launch is not split) for `groups` (tile, slab) pairs of `nch` staged chunks each; sets the
+// plane size of the workspace.
+template <typename T>
+int split_parts(ConvArgsT<T>& a, long long groups, int nch) {
   static const int max_groups = [] { const char* e = getenv("MIE_CONV_SPLIT_GROUPS"); return e ? atoi(e) : 128; }();
   static const int max_wgs = [] { const char* e = getenv("MIE_CONV_SPLIT_WGS"); return e ? atoi(e) : 256; }();
-  if (groups > max_groups || nch < 4) return false;
-  ConvArgsT<T> a = a0;
-  a.xcd_fs = 0;
-  a.ws_plane = (long long)a.ts.n * a.ts.h * a.ts.w * a.cout;
   static const int most = [] {      // MIE_CONV_SPLIT caps the number of parts (1: never split): a tuning knob, read once
     const char* e = getenv("MIE_CONV_SPLIT");
     return e ? atoi(e) : 8;
   }();
+  if (a.ws == nullptr || groups > max_groups || nch < 4) return 0;
+  a.xcd_fs = 0;
+  a.ws_plane = (long long)a.ts.n * a.ts.h * a.ts.w * a.cout;
   int parts = 1;
   while (2 * parts <= most && 2 * parts <= nch && groups * (2 * parts) <= max_wgs && (long long)(2 * parts) * a.ws_plane <= a.ws_floats)
     parts *= 2;
-  if (parts < 2) return false;
+  return parts < 2 ? 0 : parts;
+}
+
+template <typename T>
+void launch_split_finish(const ConvArgsT<T>& a, unsigned cap, int parts, hipStream_t st) {
+  unsigned ny = (unsigned)((1024 + cap - 1) / cap);
+  if (ny > (unsigned)(a.cout / 4)) ny = (unsigned)(a.cout / 4);
+  if (ny < 1) ny = 1;
+  hipLaunchKernelGGL(k_conv_split_finish<T>, dim3(cap, ny), dim3(256), 0, st, a, parts);
+}
+
+template <typename T, int K, int S>
+bool launch_split(const ConvArgsT<T>& a0, unsigned cap, hipStream_t st) {
+  constexpr int CC = stage_channels(K, S, false) * (4 / (int)sizeof(T));
+  if (a0.ws == nullptr || a0.refresh || a0.cout % 32 != 0 || a0.c1 % CC != 0 || a0.c2 % CC != 0) return false;
+  ConvArgsT<T> a = a0;
+  const int parts = split_parts(a, (long long)cap * (a0.cout / 32), (a0.c1 + a0.c2) / CC);
+  if (parts == 0) return false;
   bool x3 = false;
   if constexpr (sizeof(T) == 4 && S == 1 && (K == 3 || K == 5)) x3 = a.x3 != 0;
   if (x3) {
@@ -1051,10 +1115,54 @@ bool launch_split(const ConvArgsT<T>& a0, unsigned cap, hipStream_t st) {
   } else {
     hipLaunchKernelGGL((k_conv_mfma<T, K, S, 1, 1, false, false, false, true>), dim3(cap, a.cout / 32, parts), dim3(256), 0, st, a);
   }
+  launch_split_finish(a, cap, parts, st);
+  return true;
+}
+
+// The split form of the 5x5 conv over up2x(x + x2): the chunks of the (summed) input split as above, the plain finish.
+template <typename T>
+bool launch_up_split(const ConvArgsT<T>& a0, unsigned cap, hipStream_t st) {
+  constexpr int CC = stage_channels(5, 1, false) * (4 / (int)sizeof(T));
+  static const bool on = [] { const char* e = getenv("MIE_CONV_SPLIT_UP"); return e == nullptr || atoi(e) != 0; }();   // tuning knob
+  if (!on || a0.ws == nullptr || a0.cout % 32 != 0 || a0.c1 % CC != 0) return false;
+  ConvArgsT<T> a = a0;
+  const int parts = split_parts(a, (long long)cap * (a0.cout / 32), a0.c1 / CC);
+  if (parts == 0) return false;
+  bool x3 = false;
+  if constexpr (sizeof(T) == 4) x3 = a.x3 != 0;
+  if (x3) {
+    if constexpr (sizeof(T) == 4)
+      hipLaunchKernelGGL((k_conv_mfma<T, 5, 1, 1, 1, false, false, true, true, true>), dim3(cap, a.cout / 32, parts), dim3(256), 0, st, a);
+  } else {
+    hipLaunchKernelGGL((k_conv_mfma<T, 5, 1, 1, 1, false, false, true, true>), dim3(cap, a.cout / 32, parts), dim3(256), 0, st, a);
+  }
+  launch_split_finish(a, cap, parts, st);
+  return true;
+}
+
+// The split form of a ConvLSTM's gates conv: the contraction as a plain split 3x3 conv of the two inputs (the partial
+// sums of all 4 * hid gate columns go to the workspace), then the gate chain in the finish kernel.
+template <typename T>
+bool launch_gates_split(const ConvArgsT<T>& a0, unsigned cap, hipStream_t st) {
+  constexpr int CC = stage_channels(3, 1, false) * (4 / (int)sizeof(T));
+  static const bool on = [] { const char* e = getenv("MIE_CONV_SPLIT_GATES"); return e == nullptr || atoi(e) != 0; }();   // tuning knob
+  if (!on || a0.ws == nullptr || a0.cout != 4 * a0.hid || a0.hid % 8 != 0 || a0.c1 % CC != 0 || a0.c2 % CC != 0) return false;
+  ConvArgsT<T> a = a0;
+  const int parts = split_parts(a, (long long)cap * (a0.cout / 32), (a0.c1 + a0.c2) / CC);
+  // (two parts do not pay for the second launch: E2Depth-incr 128x128 frame 0.2685 -> 0.2699 ms, measured; four do)
+  if (parts < 4) return false;
+  bool x3 = false;
+  if constexpr (sizeof(T) == 4) x3 = a.x3 != 0;
+  if (x3) {
+    if constexpr (sizeof(T) == 4)
+      hipLaunchKernelGGL((k_conv_mfma<T, 3, 1, 1, 1, false, false, false, true, true>), dim3(cap, a.cout / 32, parts), dim3(256), 0, st, a);
+  } else {
+    hipLaunchKernelGGL((k_conv_mfma<T, 3, 1, 1, 1, false, false, false, true>), dim3(cap, a.cout / 32, parts), dim3(256), 0, st, a);
+  }
   unsigned ny = (unsigned)((1024 + cap - 1) / cap);
-  if (ny > (unsigned)(a.cout / 4)) ny = (unsigned)(a.cout / 4);
+  if (ny > (unsigned)(a.hid / 4)) ny = (unsigned)(a.hid / 4);
   if (ny < 1) ny = 1;
-  hipLaunchKernelGGL(k_conv_split_finish<T>, dim3(cap, ny), dim3(256), 0, st, a, parts);
+  hipLaunchKernelGGL(k_gates_split_finish<T>, dim3(cap, ny), dim3(256), 0, st, a, parts);
   return true;
 }
 
@@ -1198,6 +1306,7 @@ bool launch_depth(const ConvArgsT<T>& a0, unsigned cap, hipStream_t st) {
 // The 5x5 stride-1 conv over up2x(x + x2): full staging depth only.
 template <typename T>
 bool launch_up(const ConvArgsT<T>& a0, unsigned cap, hipStream_t st) {
+  if (launch_up_split<T>(a0, cap, st)) return true;
   if constexpr (sizeof(T) == 4) {
     if (a0.x3) return launch_x3<5, false, true>(a0, cap, st);
   }
@@ -1223,6 +1332,7 @@ bool launch_up(const ConvArgsT<T>& a0, unsigned cap, hipStream_t st) {
 // The gates conv of a ConvLSTM: 3x3, stride 1, full staging depth, gate chain in the epilogue.
 template <typename T>
 bool launch_gates(const ConvArgsT<T>& a0, unsigned cap, hipStream_t st) {
+  if (launch_gates_split<T>(a0, cap, st)) return true;
   if constexpr (sizeof(T) == 4) {
     if (a0.x3) return a0.cout == 4 * a0.hid && a0.hid % 8 == 0 && launch_x3<3, true, false>(a0, cap, st);
   }

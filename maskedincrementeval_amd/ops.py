@@ -42,13 +42,13 @@ def lib():
 
 
 # The builds of a planning pass are not launched one by one: they are collected and handed to the library as
-# plans (mie_build_mask_plan: the whole chain of footprints on bitmaps in LDS, two kernels per plan).  With
-# `plan_split_first` the first build goes out as a plan of its own -- its tile set is what the first kernel of the
-# compute pass waits for -- and the rest as one plan, or as several where the library says one is too long; a part
-# the library does not take as a plan (a footprint it has no bitmap form for, masks too large for LDS) is built set
-# by set as before.  `fused_plan = False` restores one mie_build_mask_tiles launch pair per set.
+# plans (mie_build_mask_plan: the whole chain of footprints on bitmaps in LDS, two kernels per plan).  A plan the
+# library says is too long goes out in halves; a part the library does not take as a plan (a footprint it has no
+# bitmap form for, masks too large for LDS) is built set by set as before.  `fused_plan = False` restores one
+# mie_build_mask_tiles launch pair per set.  (Measured and not kept: the first one or two builds as a plan of their
+# own with an event of their own, so that the first convs run beside the plan of the rest -- every extra dependency
+# between the two streams costs 5-10 us of idle time in the replayed graph, more than the overlap wins.)
 fused_plan = os.environ.get("MIE_FUSED_PLAN", "1") != "0"
-plan_split_first = os.environ.get("MIE_PLAN_SPLIT_FIRST", "0") != "0"
 _plan_batch = None       # [(p1, p2, h_in, w_in, foot, k, stride, pad, out TileMask)] while a planning pass collects
 _plan_cache = {}         # signature of a batch -> [("plan", ctypes array, n) | ("single", index)] parts
 
@@ -110,7 +110,7 @@ def _launch_plan(batch):
         stream = side.cuda_stream
     else:
         stream = torch.cuda.current_stream(dev).cuda_stream
-    sig = (plan_split_first,) + tuple(b[:8] + (b[8].pixmask.data_ptr(), b[8].tiles.data_ptr()) for b in batch)
+    sig = tuple(b[:8] + (b[8].pixmask.data_ptr(), b[8].tiles.data_ptr()) for b in batch)
     parts = _plan_cache.get(sig)
 
     def single(b):
@@ -120,7 +120,7 @@ def _launch_plan(batch):
     if parts is None:
         # first use of this batch: find parts the library takes (a refused plan launches nothing)
         parts = []
-        todo = [(0, 1), (1, len(batch))] if (len(batch) > 1 and plan_split_first) else [(0, len(batch))]
+        todo = [(0, len(batch))]
         while todo:
             lo, hi = todo.pop(0)
             if lo >= hi:
@@ -480,6 +480,18 @@ def split_workspace(device):
     return ws
 
 
+def _workspace_args(workspace, small: bool, device):
+    """(pointer, bytes) of the split form's workspace: None -> the device's shared buffer where the launch is small
+    enough to be split, False -> none."""
+    if workspace is None:
+        workspace = split_workspace(device) if (split_enabled and small) else False
+    if workspace is False:
+        return None, 0
+    if workspace.dtype != torch.float32 or not workspace.is_contiguous() or workspace.device != device:
+        raise ValueError("workspace must be a contiguous fp32 tensor on the device of the operands")
+    return workspace.data_ptr(), workspace.numel() * 4
+
+
 def conv_masked(x, xmask, x2, x2mask, filt, k, stride, pad, out_ts: TileMask, out_delta,
                 reservoir=None, act=_lib.ACT_NONE, slope=0.0, path=_lib.PATH_AUTO, addend=None, workspace=None):
     """filt: ConvFilter, or a contiguous fp32 [Cin_total, K, K, Cout] tensor (VALU kernels only).
@@ -503,15 +515,8 @@ def conv_masked(x, xmask, x2, x2mask, filt, k, stride, pad, out_ts: TileMask, ou
     if addend is not None and addend.shape != out_delta.shape:
         raise ValueError("addend shape %s != output %s" % (tuple(addend.shape), tuple(out_delta.shape)))
     _ready(out_ts)
-    if workspace is None:
-        # only launches the library would split get the buffer
-        workspace = split_workspace(x.device) if (split_enabled and small and mc_ptr is not None) else False
-    if workspace is False:
-        ws_ptr, ws_bytes = None, 0
-    else:
-        if workspace.dtype != torch.float32 or not workspace.is_contiguous() or workspace.device != x.device:
-            raise ValueError("workspace must be a contiguous fp32 tensor on the device of x")
-        ws_ptr, ws_bytes = workspace.data_ptr(), workspace.numel() * 4
+    # only launches the library would split get the shared buffer
+    ws_ptr, ws_bytes = _workspace_args(workspace, small and mc_ptr is not None, x.device)
     check(lib().mie_conv_masked_ws(
         nhwc_ptr(x, "x", dtype=dt), pix_ptr(xmask, n, h, w, "xmask"), c1,
         nhwc_ptr(x2, "x2", dtype=dt), pix_ptr(x2mask, n, h, w, "x2mask"), c2, h, w,
@@ -539,9 +544,9 @@ def upconv_few_takes(c: int, cout: int, k: int, stride: int, pad: int) -> bool:
 
 
 def upconv_masked(a, amask, b, bmask, filt, k, pad, out_ts: TileMask, out_delta, reservoir=None,
-                  act=_lib.ACT_NONE, slope=0.0, addend=None):
+                  act=_lib.ACT_NONE, slope=0.0, addend=None, workspace=None):
     """conv over up2x(a + b) in one kernel; a, b at half the resolution of out_ts (b may be None): 5x5 for inputs in
-    whole matrix-core chunks, 3x3 or 5x5 for a single input of at most 8 channels."""
+    whole matrix-core chunks, 3x3 or 5x5 for a single input of at most 8 channels.  workspace: as in conv_masked."""
     n, c, h, w = a.shape
     dt = a.dtype
     if b is not None and (b.shape != a.shape or b.dtype != dt):
@@ -554,11 +559,12 @@ def upconv_masked(a, amask, b, bmask, filt, k, pad, out_ts: TileMask, out_delta,
     if reservoir is not None and reservoir.shape != out_delta.shape:
         raise ValueError("reservoir shape %s != output %s" % (tuple(reservoir.shape), tuple(out_delta.shape)))
     _ready(out_ts)
-    check(lib().mie_upconv_masked(
+    ws_ptr, ws_bytes = _workspace_args(workspace, c > 8 and mc_ptr is not None and out_ts.capacity * (cout // 32) <= 128, a.device)
+    check(lib().mie_upconv_masked_ws(
         nhwc_ptr(a, "a", dtype=dt), pix_ptr(amask, n, h, w, "amask"), nhwc_ptr(b, "b", dtype=dt),
         pix_ptr(bmask, n, h, w, "bmask"), c, h, w, plain.data_ptr(), mc_ptr, cin_total, k, pad, cout, out_ts.ref,
         nhwc_ptr(out_delta, "out_delta", dtype=dt), nhwc_ptr(addend, "addend", cout, dtype=dt),
-        nhwc_ptr(reservoir, "reservoir"), act, float(slope), code, _stream(a)))
+        nhwc_ptr(reservoir, "reservoir"), act, float(slope), code, ws_ptr, ws_bytes, _stream(a)))
     return out_delta
 
 
@@ -959,9 +965,9 @@ def gate_interleave_index(hid: int, device=None) -> torch.Tensor:
 
 
 def conv_gates_incr(x, xmask, x2, x2mask, filt: ConvFilter, out_ts: TileMask, gates_res, cprev_delta, cprev_mask,
-                    cprev_res, cell_res, h_delta, c_delta):
+                    cprev_res, cell_res, h_delta, c_delta, workspace=None):
     """3x3 gates conv of a ConvLSTM with the gate chain as its epilogue; `filt` and `gates_res` are in the
-    gate-interleaved column order (gate_interleave_index)."""
+    gate-interleaved column order (gate_interleave_index).  workspace: as in conv_masked."""
     n, c1, h, w = x.shape
     c2 = 0 if x2 is None else x2.shape[1]
     dt = x.dtype
@@ -974,13 +980,14 @@ def conv_gates_incr(x, xmask, x2, x2mask, filt: ConvFilter, out_ts: TileMask, ga
         if tuple(t.shape) != (n, hid, h, w):
             raise ValueError("%s shape %s, expected %s" % (name, tuple(t.shape), (n, hid, h, w)))
     _ready(out_ts)
-    check(lib().mie_conv_gates_masked(
+    ws_ptr, ws_bytes = _workspace_args(workspace, mc_ptr is not None and out_ts.capacity * (cout // 32) <= 128, x.device)
+    check(lib().mie_conv_gates_masked_ws(
         nhwc_ptr(x, "x", dtype=dt), pix_ptr(xmask, n, h, w, "xmask"), c1,
         nhwc_ptr(x2, "x2", dtype=dt), pix_ptr(x2mask, n, h, w, "x2mask"), c2, h, w,
         plain.data_ptr(), mc_ptr, cin_total, hid, out_ts.ref, nhwc_ptr(gates_res, "gates_res"),
         nhwc_ptr(cprev_delta, "cprev_delta", dtype=dt), pix_ptr(cprev_mask, n, h, w, "cprev_mask"),
         nhwc_ptr(cprev_res, "cprev_res"), nhwc_ptr(cell_res, "cell_res"),
-        nhwc_ptr(h_delta, "h_delta", dtype=dt), nhwc_ptr(c_delta, "c_delta", dtype=dt), code,
+        nhwc_ptr(h_delta, "h_delta", dtype=dt), nhwc_ptr(c_delta, "c_delta", dtype=dt), code, ws_ptr, ws_bytes,
         _stream(x)))
     return h_delta, c_delta
 

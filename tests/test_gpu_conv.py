@@ -399,6 +399,57 @@ def test_upsampled_conv_in_one_kernel(c, cout, h, w, dtype, f32mode):
             assert torch.allclose(res.cpu(), r0 + ref, rtol=RTOL, atol=bf16_atol(ref, 2.0) if bf else ATOL)
 
 
+# Up-sampling decoder convs on planes of few tiles: the contraction is split over workgroups through a workspace
+# (mie_upconv_masked_ws) and a second kernel runs the epilogue.  Against the oracle and against the unsplit launch;
+# three steps with fresh masks (stale tiles), reservoir + activation on the last two.
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("c,cout,h,w,two", [(256, 128, 16, 16, True), (128, 64, 12, 20, True), (256, 32, 9, 7, False)])
+@pytest.mark.parametrize("f32mode", ["bf16x3", "native"])
+def test_small_upsampled_planes_split_the_contraction(c, cout, h, w, two, dtype, f32mode):
+    bf = dtype == torch.bfloat16
+    if bf and c // 64 < 4:
+        pytest.skip("fewer than 4 staged chunks of 64 bf16 channels: not split")
+    tol = (lambda ref: dict(rtol=BF16_RTOL, atol=bf16_atol(ref, 2.0))) if bf else (lambda ref: dict(rtol=RTOL, atol=ATOL))
+    q = (lambda t: t.to(torch.bfloat16).float()) if bf else (lambda t: t)
+    wt = q(he_normal_conv_weight(cout, c, 5, 19))
+    filt = _filt(wt)
+    ho, wo = 2 * h, 2 * w
+    ts_up, ts = TileMask(1, ho, wo, DEV), TileMask(1, ho, wo, DEV)
+    assert ts.capacity * (cout // 32) <= 128
+    out, out_plain = ops.new_nhwc(1, cout, ho, wo, DEV, dtype), ops.new_nhwc(1, cout, ho, wo, DEV, dtype)
+    ws = torch.full((ops.SPLIT_WORKSPACE_BYTES // 4,), float("nan"), device=DEV)
+    r0 = gaussian_delta(1, cout, ho, wo, 1.0, 1.0, seed=7)[0]
+    res, res_plain, res_ref = _dev(r0).clone(), _dev(r0).clone(), r0.clone()
+    for step, (da, db, with_res) in enumerate([(0.3, 0.2, False), (0.05, 0.02, True), (0.5, 0.4, True)]):
+        a, ma = gaussian_delta(1, c, h, w, da, 0.5, seed=500 + step)
+        b, mb = gaussian_delta(1, c, h, w, db, 0.5, seed=600 + step)
+        a, b = q(a), q(b)
+        up = io.interp_incr(a + b if two else a)
+        if bf:
+            up = q(up)
+        ref = io.conv_incr(up, wt, 1, 2)
+        dma, dmb = ma.to(DEV), mb.to(DEV)
+        ops.build_mask_tiles(dma, dmb if two else None, 1, h, w, _lib.FOOT_UP2X, 0, 0, 0, ts_up)
+        ops.build_mask_tiles(ts_up, None, 1, ho, wo, _lib.FOOT_CONV, 5, 1, 2, ts)
+        poison = lambda t, m: torch.where(m.bool().expand_as(t), t, torch.full_like(t, float("nan")))
+        xa, xb = _dev(poison(a, ma)).to(dtype), (_dev(poison(b, mb)).to(dtype) if two else None)
+        for o, r, wsp in ((out, res, ws), (out_plain, res_plain, False)):
+            ops.upconv_masked(xa, dma, xb, dmb if two else None, filt, 5, 2, ts, o, r if with_res else None,
+                              _lib.ACT_RELU if with_res else _lib.ACT_NONE, workspace=wsp)
+        torch.cuda.synchronize()
+        got, plain = out.float().cpu(), out_plain.float().cpu()
+        assert torch.isfinite(got).all()
+        want = torch.relu(res_ref + ref) - torch.relu(res_ref) if with_res else ref
+        if with_res:
+            res_ref = res_ref + ref
+        assert torch.allclose(got, want, **tol(want)), "step %d max|diff| = %.3e" % (step, (got - want).abs().max())
+        assert torch.allclose(got, plain, **tol(plain)), "step %d split vs unsplit %.3e" % (step, (got - plain).abs().max())
+        if with_res:
+            assert torch.allclose(res.cpu(), res_ref, rtol=RTOL, atol=bf16_atol(ref, 2.0) if bf else ATOL)
+    plane = ho * wo * cout
+    assert torch.isfinite(ws[:plane]).any() and torch.isfinite(ws[plane:2 * plane]).any()      # the split form ran
+
+
 # The same for a single input of very few channels (the flow estimate in front of an EVFlowNet decoder): 3x3 and 5x5.
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("c,cout,k,h,w", [(2, 64, 3, 13, 17), (2, 32, 3, 32, 32), (5, 96, 5, 9, 40), (8, 32, 3, 21, 11)])

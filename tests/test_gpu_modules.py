@@ -374,6 +374,48 @@ def test_e2depth_incr_empty_frames_between_active_ones():
     assert torch.count_nonzero(buf * (1 - ts.pixmask.float())) == 0
 
 
+@pytest.mark.parametrize("cin,hid,h,w", [(128, 128, 16, 8), (64, 64, 12, 20), (256, 256, 8, 8)])
+@pytest.mark.parametrize("f32mode", ["bf16x3", "native"])
+def test_convlstm_on_a_small_plane_splits_the_gates_conv(cin, hid, h, w, f32mode):
+    # planes of few tiles: the gates conv runs as a split contraction (partial sums in the workspace) and the gate
+    # chain in a second kernel (mie_conv_gates_masked_ws).  Against the oracle, and against a twin cell whose launches
+    # are not split; previous-state deltas from the second step on (two-input contraction, previous-cell term).
+    n = 1
+    cells = [seed_module_(ConvLSTMIncr(cin, hid, 3, fused=True), 81).to(DEV).eval() for _ in range(2)]
+    ref = io.ConvLSTMOracle(cells[0].Gates.weight.detach().cpu(), cells[0].Gates.bias.detach().cpu(), hid)
+    x0 = torch.randn(n, cin, h, w, generator=torch.Generator().manual_seed(82)) * 0.5
+    with torch.no_grad():
+        for cell in cells:
+            h_d, c_d = cell.forward_refresh_reservoirs(_cl(x0), None)
+    h_r, c_r = ref.refresh(x0)
+    _close(h_d, h_r, "refresh h"), _close(c_d, c_r, "refresh c")
+    ws = ops.split_workspace(torch.device(DEV))
+    ws.fill_(float("nan"))
+    for step in range(4):
+        d, m = gaussian_delta(n, cin, h, w, (0.4, 0.05, 0.7, 0.2)[step], 0.3, seed=8300 + step)
+        prev, prev_ref = None, None
+        if step >= 1:
+            dhp, mh = gaussian_delta(n, hid, h, w, 0.2, 0.2, seed=8400 + step)
+            dcp, mc = gaussian_delta(n, hid, h, w, 0.1, 0.2, seed=8500 + step)
+            prev = lambda: ([_cl(dhp), mh.to(DEV)], [_cl(dcp), mc.to(DEV)])
+            prev_ref = (dhp, dcp)
+        outs = []
+        for cell, split in zip(cells, (True, False)):
+            ops.split_enabled = split
+            try:
+                with torch.no_grad():
+                    outs.append(cell([_cl(d), m.to(DEV)], None if prev is None else prev()))
+            finally:
+                ops.split_enabled = True
+        torch.cuda.synchronize()
+        dh_r, dc_r = ref.incr(d, prev_ref) if prev_ref is not None else ref.incr(d)
+        for (dh, dc), what in zip(outs, ("split", "one launch")):
+            assert torch.isfinite(dh[0]).all() and torch.isfinite(dc[0]).all()
+            _close(dh[0], dh_r, "%s dh %d" % (what, step)), _close(dc[0], dc_r, "%s dc %d" % (what, step))
+    plane = n * h * w * 4 * hid
+    assert torch.isfinite(ws[:plane]).any() and torch.isfinite(ws[plane:2 * plane]).any()      # the split form ran
+
+
 @pytest.mark.parametrize("cin,hid", [(16, 16), (32, 32)])
 def test_convlstm_with_previous_state_deltas(cin, hid):
     # non-zero refresh state and non-zero deltas of the previous hidden / cell state (the module
