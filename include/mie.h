@@ -657,6 +657,32 @@ int mie_upconv_masked_ws(const void* a, const uint8_t* amask, const void* b,
                          long long workspace_bytes, void* stream);
 
 /*
+ * The tail of E2Depth-incr in one kernel: the last decoder -- mie_upconv_masked, 5x5 over up2x(a + b), c = 64 -> cout =
+ * 32 channels, reservoir + activation -- whose activation increment y is NOT stored, followed by the one-channel 1x1
+ * prediction conv over y + skip (skip: the head's output delta, [n, 2*h_in, 2*w_in, cout], clean outside skip_mask, NULL
+ * mask = every pixel), the update of the prediction's pre-activation reservoir and its activation increment:
+ *   r1 = reservoir + conv;  y = act(r1) - act(reservoir)  (rounded to the delta type);  reservoir = r1
+ *   z  = sum_c pred_filter[c] * y[c] + pred_filter[cout + c] * skip[c]
+ *   p1 = pred_reservoir + z;  pred_delta = pred_act(p1) - pred_act(pred_reservoir);  pred_reservoir = p1
+ * at every pixel of the active tiles of `out`, zeros in pred_delta ([n, 2*h_in, 2*w_in], element type `dtype`) on its
+ * stale tiles.  `out` is the tile set of the PREDICTION: the union of the decoder's output set and the set of skip
+ * (mie_build_mask_tiles with both as inputs, MIE_FOOT_CONV k = 1); the decoder's conv runs on all of its tiles.
+ * pred_filter: fp32 [2][cout], the prediction conv's weights for y and for skip (the same row twice for
+ * pred(x + head)).  Implemented for MIE_DTYPE_BF16, c = 64, cout = 32, decoder activations none / ReLU / leaky ReLU,
+ * on planes of 2048 .. 2^20 tiles; MIE_ERR_UNSUPPORTED otherwise (run mie_upconv_masked and mie_conv_masked).
+ * Replaces: the last UpsampleConvLayerIncr, the skip sum, the prediction layer and the output activation of
+ * UNetRecurrentIncr.forward (incr_modules/e2depth_incr.py:429-435).
+ */
+int mie_upconv_pred_masked(const void* a, const uint8_t* amask, const void* b,
+                           const uint8_t* bmask, int c, int h_in, int w_in,
+                           const float* filter, const void* filter_mc, int cin_total,
+                           int cout, const mie_tileset* out, float* reservoir,
+                           int act_kind, float slope, const void* skip,
+                           const uint8_t* skip_mask, const float* pred_filter,
+                           float* pred_reservoir, int pred_act, float pred_slope,
+                           void* pred_delta, int dtype, void* stream);
+
+/*
  * Masked transposed convolution of a delta (stride s, padding p; the output
  * size out->h/w fixes output_padding): out(oy,ox,co) = sum x(iy,ix,ci) *
  * filter[ci][ky][kx][co] over oy = iy*s - p + ky, ox = ix*s - p + kx, with

@@ -34,7 +34,7 @@ EXPORTS = (
     "mie_build_mask_tiles", "mie_conv_masked", "mie_act_incr", "mie_mul_incr", "mie_add_incr",
     "mie_upsample2x_incr", "mie_convlstm_gates_incr", "mie_tconv_masked", "mie_conv_refresh",
     "mie_pack_filter", "mie_kfence_incr", "mie_events_to_frame", "mie_events_to_frame_bf16", "mie_tconv_refresh", "mie_conv_gates_masked", "mie_conv_gates_masked_ws",
-    "mie_maxpool_incr", "mie_accumulate", "mie_scale_incr", "mie_avgpool_incr", "mie_linear_incr", "mie_upconv_masked", "mie_upconv_masked_ws",
+    "mie_maxpool_incr", "mie_accumulate", "mie_scale_incr", "mie_avgpool_incr", "mie_linear_incr", "mie_upconv_masked", "mie_upconv_masked_ws", "mie_upconv_pred_masked",
     "mie_conv_masked_ws", "mie_convgru_gates_incr", "mie_upsample2x_pair_incr", "mie_conv_masked_noalloc",
     "mie_convlstm_gates_refresh", "mie_convgru_gates_refresh", "mie_mul_dense", "mie_tconv2x_masked",
     "mie_tconv2x_refresh", "mie_conv_f32x3_takes", "mie_build_mask_plan",
@@ -152,6 +152,9 @@ def _declare(l):
     l.mie_linear_incr.argtypes = [vp, ci, ci, vp, ci, vp, ci, vp]
     l.mie_upconv_masked.restype = ci
     l.mie_upconv_masked.argtypes = [vp, vp, vp, vp, ci, ci, ci, vp, vp, ci, ci, ci, ci, tsp, vp, vp, vp, ci, cf, ci, vp]
+    l.mie_upconv_pred_masked.restype = ci
+    l.mie_upconv_pred_masked.argtypes = [vp, vp, vp, vp, ci, ci, ci, vp, vp, ci, ci, tsp, vp, ci, cf, vp, vp, vp, vp, ci, cf,
+                                         vp, ci, vp]
     l.mie_upconv_masked_ws.restype = ci
     l.mie_upconv_masked_ws.argtypes = [vp, vp, vp, vp, ci, ci, ci, vp, vp, ci, ci, ci, ci, tsp, vp, vp, vp, ci, cf, ci, vp,
                                        ctypes.c_longlong, vp]

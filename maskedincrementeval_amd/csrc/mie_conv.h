@@ -197,6 +197,12 @@ bool mie_launch_conv_up_mfma(const ConvArgsT<mie_bf16>& a, unsigned cap, hipStre
 // The same for bf16 deltas, 64 -> 32 channels, on planes of many tiles: a persistent kernel (mie_upconv_persist.hip).
 // Returns false, launching nothing, for other shapes.
 bool mie_launch_upconv_persist(const ConvArgsT<mie_bf16>& a, unsigned cap, hipStream_t st);
+// ... with the network's tail fused in: the layer's activation increment is not stored; the 1x1 prediction conv over it
+// and over `skip` (32 channels, same resolution), the prediction's reservoir update and its activation increment
+// (one channel, pred_out) run in the epilogue.  pred_w: [2][32] fp32 (weights of the layer's output, of skip).
+bool mie_launch_upconv_pred_persist(const ConvArgsT<mie_bf16>& a, const mie_bf16* skip, const uint8_t* skip_mask,
+                                    const float* pred_w, float* pred_res, mie_bf16* pred_out, int pred_act,
+                                    float pred_slope, unsigned cap, hipStream_t st);
 
 // Source rows / columns and weights of output index o of a bilinear x2 up-sampling (align_corners =
 // False): src = max(0, o/2 - 0.25), upper index clamped to the last row.

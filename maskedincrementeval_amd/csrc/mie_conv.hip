@@ -845,6 +845,51 @@ extern "C" int mie_upconv_masked(const void* a, const uint8_t* amask, const void
                               out_delta, addend, reservoir, act_kind, slope, dtype, nullptr, 0, stream);
 }
 
+extern "C" int mie_upconv_pred_masked(const void* a_lo, const uint8_t* amask, const void* b_lo, const uint8_t* bmask,
+                                      int c, int h_in, int w_in, const float* filter, const void* filter_mc,
+                                      int cin_total, int cout, const mie_tileset* out, float* reservoir, int act_kind,
+                                      float slope, const void* skip, const uint8_t* skip_mask, const float* pred_filter,
+                                      float* pred_reservoir, int pred_act, float pred_slope, void* pred_delta,
+                                      int dtype, void* stream) {
+  mie_clear_error();
+  const char* who = "mie_upconv_pred_masked";
+  int rc = mie_check_tileset(out, who);
+  if (rc != MIE_OK) return rc;
+  MIE_REQUIRE(dtype == MIE_DTYPE_BF16 && c == 64 && cout == 32, MIE_ERR_UNSUPPORTED,
+              "%s: implemented for bf16 deltas, 64 -> 32 channels (dtype=%d c=%d cout=%d)", who, dtype, c, cout);
+  MIE_REQUIRE(a_lo && filter && filter_mc && reservoir && skip && pred_filter && pred_reservoir && pred_delta,
+              MIE_ERR_INVALID_ARG, "%s: NULL pointer", who);
+  MIE_REQUIRE(b_lo != nullptr || bmask == nullptr, MIE_ERR_INVALID_ARG, "%s: mask of absent b", who);
+  MIE_REQUIRE(h_in > 0 && w_in > 0 && cin_total >= c && cin_total % 16 == 0, MIE_ERR_INVALID_ARG,
+              "%s: sizes out of range (cin_total=%d h=%d w=%d)", who, cin_total, h_in, w_in);
+  MIE_REQUIRE(out->h == 2 * h_in && out->w == 2 * w_in, MIE_ERR_INVALID_ARG,
+              "%s: the tile set is (%d,%d), twice the input is (%d,%d)", who, out->h, out->w, 2 * h_in, 2 * w_in);
+  MIE_REQUIRE((long long)out->n * out->h * out->w < 0x7fffffffLL, MIE_ERR_CAPACITY, "%s: input too large", who);
+  MIE_REQUIRE(mie_aligned(a_lo, 16) && mie_aligned(b_lo, 16) && mie_aligned(filter, 16) && mie_aligned(filter_mc, 16) &&
+                  mie_aligned(reservoir, 16) && mie_aligned(skip, 16) && mie_aligned(pred_filter, 16) &&
+                  mie_aligned(pred_reservoir, 4) && mie_aligned(pred_delta, 2),
+              MIE_ERR_INVALID_ARG, "%s: misaligned operand", who);
+  MIE_REQUIRE((act_kind == MIE_ACT_NONE || act_kind == MIE_ACT_RELU || act_kind == MIE_ACT_LEAKY_RELU) &&
+                  pred_act >= MIE_ACT_NONE && pred_act <= MIE_ACT_TANH,
+              MIE_ERR_UNSUPPORTED, "%s: activation %d / %d not implemented", who, act_kind, pred_act);
+  MIE_REQUIRE(pred_delta != skip && pred_delta != a_lo && pred_delta != b_lo && (void*)pred_reservoir != (void*)reservoir,
+              MIE_ERR_INVALID_ARG, "%s: outputs must not alias inputs", who);
+  ConvArgsT<mie_bf16> a;
+  a.x = (const mie_bf16*)a_lo; a.xm = amask; a.c1 = c; a.x2 = (const mie_bf16*)b_lo; a.x2m = bmask; a.c2 = b_lo ? c : 0;
+  a.h_in = 2 * h_in; a.w_in = 2 * w_in; a.filt = filter; a.cin_total = cin_total; a.filt_mc = (const mie_bf16*)filter_mc;
+  a.pad = 2; a.cout = cout; a.out = nullptr; a.res = reservoir; a.act = act_kind;
+  a.slope = slope; a.addend = nullptr; a.refresh = 0; a.bias = nullptr;
+  a.hid = 0; a.g_cpd = nullptr; a.g_cpm = nullptr; a.g_cpres = nullptr; a.g_cres = nullptr;
+  a.g_dh = nullptr; a.g_dc = nullptr;
+  a.ws = nullptr; a.ws_floats = 0; a.ws_plane = 0; a.xcd_fs = 0; a.x3 = 0;
+  a.ts = mie_dev_tileset(out);
+  const unsigned cap = (unsigned)mie_tile_capacity(out->n, out->h, out->w);
+  MIE_REQUIRE(mie_launch_upconv_pred_persist(a, (const mie_bf16*)skip, skip_mask, pred_filter, pred_reservoir,
+                                             (mie_bf16*)pred_delta, pred_act, pred_slope, cap, (hipStream_t)stream),
+              MIE_ERR_UNSUPPORTED, "%s: planes of fewer than 2048 tiles (or more than 2^20) take the separate kernels", who);
+  return mie_check_launch(who);
+}
+
 extern "C" int mie_conv_gates_masked_ws(const void* x, const uint8_t* xmask, int c1, const void* x2,
                                         const uint8_t* x2mask, int c2, int h_in, int w_in,
                                         const float* filter, const void* filter_mc, int cin_total,

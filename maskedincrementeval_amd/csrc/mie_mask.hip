@@ -941,7 +941,15 @@ extern "C" int mie_build_mask_plan(const mie_plan_op* ops, int n_ops, void* stre
   memset(&a, 0, sizeof(a));
   a.n = ops[0].out.n;
   // masks in LDS: pointer -> (slot offset, words, step index of the last reader)
-  struct Slot { const uint8_t* ptr; long long off, words; int h, w, last; };
+  struct Slot { const uint8_t* ptr; long long off, words; int h, w, last, born, rec; };
+  // Every allocation of the walk below, with the ops during which it is held (born .. rel, both included): the walk
+  // runs twice -- first with a first-fit allocator, which fragments (the short-lived input mask of a UNet leaves a hole
+  // that small masks then chop up, and the two full-resolution masks at the end of the chain no longer fit into it);
+  // then, if that is tighter, with offsets packed off line from the recorded lifetimes, largest masks first.
+  struct AllocRec { long long words, off; int born, rel; };
+  AllocRec recs[2 * MIE_PLAN_MAX_STEPS];
+  int nrec = 0;
+  bool replay = false;
   Slot slots[2 * MIE_PLAN_MAX_STEPS];
   int nslots = 0;
   // which op reads a mask last (by pointer), so that its slot can be handed on afterwards
@@ -958,6 +966,17 @@ extern "C" int mie_build_mask_plan(const mie_plan_op* ops, int n_ops, void* stre
   };
   PlanArena arena;
   long long total_chunks = 0, max_pixels = 0, max_tiles = 0;
+  int alloc_no = 0;
+  auto slot_alloc = [&](long long words, int born) -> int {      // returns the record index; recs[..].off is the offset
+    const int id = alloc_no++;
+    if (!replay) {
+      recs[id].words = words; recs[id].born = born; recs[id].rel = n_ops;
+      recs[id].off = arena.alloc(words);
+      nrec = alloc_no;
+    }
+    return id;
+  };
+  auto walk = [&]() -> int {
   for (int i = 0; i < n_ops; ++i) {
     const mie_plan_op& op = ops[i];
     int rc = mie_check_tileset(&op.out, who);
@@ -1007,11 +1026,13 @@ extern "C" int mie_build_mask_plan(const mie_plan_op* ops, int n_ops, void* stre
                     "%s: more than %d steps (ops plus masks loaded from memory); build the plan in parts", who, MIE_PLAN_MAX_STEPS);
         Slot ns;
         ns.ptr = ins[q]; ns.h = op.h_in; ns.w = op.w_in; ns.words = plan_words(op.h_in, op.w_in);
+        ns.born = i;
         ns.last = last_reader(ins[q], i);
         // (a later op of the plan may overwrite this address: then the mask in LDS is the old one from there on)
         for (int j = i; j < ns.last; ++j)
           if (ops[j].out.pixmask == ins[q]) { ns.last = j; break; }
-        ns.off = arena.alloc(ns.words);
+        ns.rec = slot_alloc(ns.words, i);
+        ns.off = recs[ns.rec].off;
         PlanStep& ld = a.st[a.n_steps++];
         ld.kind = PLAN_STEP_LOAD;
         ld.in1 = ld.in2 = PLAN_IN_NONE;
@@ -1035,7 +1056,28 @@ extern "C" int mie_build_mask_plan(const mie_plan_op* ops, int n_ops, void* stre
     os.last = last_reader(op.out.pixmask, i);
     for (int j = i + 1; j < os.last; ++j)
       if (ops[j].out.pixmask == op.out.pixmask) { os.last = j; break; }      // rewritten before its last reader
-    os.off = arena.alloc(os.words);
+    os.born = i;
+    // A union (the 1x1 footprint of two masks) is a word-by-word OR: it may overwrite an input that nobody reads after
+    // this op -- provided that input is at least two ops old, so that the writer waves of the op before this one, which
+    // still read THEIR op's output while this op computes, are not looking at it.  Saves a slot of the plane's size
+    // (the full-resolution union at the end of a UNet is what decides whether the chain fits the LDS in one plan).
+    os.off = -1;
+    if (identity && op.in_mask != nullptr && op.in_mask2 != nullptr) {
+      for (int q = 1; q >= 0 && os.off < 0; --q) {
+        Slot* sl = find_slot(ins[q]);
+        if (sl != nullptr && sl->off == in_off[q] && sl->words == os.words && sl->last == i && sl->born <= i - 2 &&
+            ins[q] != (const uint8_t*)op.out.pixmask) {
+          os.off = sl->off;
+          os.rec = sl->rec;       // the memory is the output's now: one allocation, held on
+          sl->words = 0;
+          sl->last = -1;
+        }
+      }
+    }
+    if (os.off < 0) {
+      os.rec = slot_alloc(os.words, i);
+      os.off = recs[os.rec].off;
+    }
     PlanStep& ft = a.st[a.n_steps++];
     ft.kind = PLAN_STEP_FOOT;
     ft.in1 = in_off[0]; ft.in2 = in_off[1];
@@ -1062,7 +1104,10 @@ extern "C" int mie_build_mask_plan(const mie_plan_op* ops, int n_ops, void* stre
     // delayed, the slot a step writes was last read at least one whole step -- and its barrier -- earlier.
     for (int q = 0; q < nslots; ++q)
       if (slots[q].last >= 0 && slots[q].last < i && slots[q].words > 0) {
-        arena.release(slots[q].off, slots[q].words);
+        if (!replay) {
+          arena.release(slots[q].off, slots[q].words);
+          recs[slots[q].rec].rel = i;
+        }
         slots[q].words = 0;
         slots[q].last = -1;
       }
@@ -1071,8 +1116,56 @@ extern "C" int mie_build_mask_plan(const mie_plan_op* ops, int n_ops, void* stre
     if ((long long)op.out.h * op.out.w > max_pixels) max_pixels = (long long)op.out.h * op.out.w;
     if (cap / op.out.n > max_tiles) max_tiles = cap / op.out.n;
   }
+  return MIE_OK;
+  };
+  int rc = walk();
+  if (rc != MIE_OK) return rc;
+  {
+    // off-line packing: largest first, each at the lowest offset where it meets no allocation whose lifetime overlaps
+    int order[2 * MIE_PLAN_MAX_STEPS];
+    long long packed[2 * MIE_PLAN_MAX_STEPS];
+    for (int i = 0; i < nrec; ++i) order[i] = i;
+    for (int i = 1; i < nrec; ++i)
+      for (int j = i; j > 0 && (recs[order[j]].words > recs[order[j - 1]].words ||
+                                (recs[order[j]].words == recs[order[j - 1]].words && recs[order[j]].born < recs[order[j - 1]].born)); --j) {
+        const int t = order[j]; order[j] = order[j - 1]; order[j - 1] = t;
+      }
+    long long top = 0;
+    for (int oi = 0; oi < nrec; ++oi) {
+      const AllocRec& r = recs[order[oi]];
+      long long off = 0;
+      for (bool moved = true; moved;) {
+        moved = false;
+        for (int oj = 0; oj < oi; ++oj) {
+          const AllocRec& q = recs[order[oj]];
+          const long long qo = packed[order[oj]];
+          if (r.born <= q.rel && q.born <= r.rel && off < qo + q.words && qo < off + r.words) {
+            off = qo + q.words;
+            moved = true;
+          }
+        }
+      }
+      packed[order[oi]] = off;
+      if (off + r.words > top) top = off + r.words;
+    }
+    if (top < arena.top) {
+      for (int i = 0; i < nrec; ++i) recs[i].off = packed[i];
+      arena.top = top;
+      replay = true;
+      memset(&a, 0, sizeof(a));
+      a.n = ops[0].out.n;
+      nslots = 0; alloc_no = 0; total_chunks = 0; max_pixels = 0; max_tiles = 0;
+      rc = walk();
+      if (rc != MIE_OK) return rc;
+    }
+  }
   // workgroups per sample: a slice of the largest plane's stores each, and never more than one tile flag per thread
   long long shares = (max_pixels + PLAN_PIXELS_PER_SHARE - 1) / PLAN_PIXELS_PER_SHARE;
+  // Every workgroup walks the whole chain of its sample (and loads every mask that comes from memory): with a batch of
+  // samples there are workgroups enough without many per sample, and more than one per CU would only queue (a
+  // workgroup of a large plane takes most of a CU's LDS).
+  static const int max_wgs = [] { const char* e = getenv("MIE_PLAN_WGS"); return e ? atoi(e) : 256; }();      // tuning knob
+  if (shares * a.n > max_wgs) shares = max_wgs / a.n > 0 ? max_wgs / a.n : 1;
   if (shares * PLAN_THREADS < max_tiles) shares = (max_tiles + PLAN_THREADS - 1) / PLAN_THREADS;
   // the flag area of a workgroup: per set, the tiles it owns (every shares-th one)
   for (int i = 0; i < a.n_steps; ++i) {
@@ -1088,7 +1181,7 @@ extern "C" int mie_build_mask_plan(const mie_plan_op* ops, int n_ops, void* stre
               "%s: a plane of %lld pixels (%lld tiles) per sample is beyond the plan's %d workgroups per sample; use "
               "mie_build_mask_tiles", who, max_pixels, max_tiles, PLAN_MAX_SHARES);
   const long long lds_bytes = (PLAN_HEAD + a.flag_words + arena.top) * 4;
-  int rc = plan_lds_limit(lds_bytes, who);
+  rc = plan_lds_limit(lds_bytes, who);
   if (rc != MIE_OK) return rc;
 #ifdef MIE_PLAN_PROFILE
   a.dbg = reinterpret_cast<int*>(ops[n_ops - 1].out.stale) + (mie_tile_capacity(a.n, ops[n_ops - 1].out.h, ops[n_ops - 1].out.w) - 3 * MIE_PLAN_MAX_STEPS);

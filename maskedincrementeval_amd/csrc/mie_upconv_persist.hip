@@ -80,6 +80,12 @@ __device__ __forceinline__ TilePos tile_pos(const TileGrid& g, int tile) {
   return p;
 }
 
+// v of another lane, chosen by a DPP control word (lanes without a source read 0)
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+
 // epilogue of one group of four adjacent channels, its cases fixed at compile time
 template <bool RES, int ACT>
 __device__ __forceinline__ void epilogue4(const ConvArgsT<mie_bf16>& a, long long off, const float4& v, const float4& r0) {
@@ -95,8 +101,24 @@ __device__ __forceinline__ void epilogue4(const ConvArgsT<mie_bf16>& a, long lon
                                   mie_act(ACT, a.slope, r1.w) - mie_act(ACT, a.slope, r0.w)));
 }
 
-template <bool RES, int ACT>
-__global__ __launch_bounds__(256, 2) void k_upconv64_persist(ConvArgsT<mie_bf16> a) {
+// PRED: the network's tail rides along.  The layer's activation increment y (32 channels, rounded to bf16 as the
+// delta it would have been stored as) is not written; instead the 1x1 prediction conv over y and over a second
+// 32-channel delta at the same resolution (the head's output: pred(x + head) = w . y + w . head, the conv being
+// linear) is summed over the eight lanes that share a pixel, added to the prediction's pre-activation reservoir, and
+// the one-channel activation increment is the output.
+struct PredTail {
+  const mie_bf16* skip;        // [n, h, w, 32] delta, clean outside skip_mask
+  const uint8_t* skip_mask;    // may be NULL: every pixel
+  const float* w;              // [2][32]: weights of y, weights of skip
+  float* res;                  // [n, h, w] pre-activation reservoir of the prediction
+  mie_bf16* out;               // [n, h, w] prediction delta
+  int act;
+  float slope;
+};
+
+template <bool RES, int ACT, bool PRED = false>
+__global__ __launch_bounds__(256, 2) void k_upconv64_persist(ConvArgsT<mie_bf16> a, PredTail pt) {
+  static_assert(!PRED || RES, "the fused tail needs the layer's reservoir");
   __shared__ __attribute__((aligned(16))) mie_bf16 s_stage[STAGE];
   __shared__ __attribute__((aligned(16))) float s_lo[LO_F];
   __shared__ __attribute__((aligned(16))) float s_red[RED_F];
@@ -120,6 +142,11 @@ __global__ __launch_bounds__(256, 2) void k_upconv64_persist(ConvArgsT<mie_bf16>
     const int tile = a.ts.stale[s];
     if (tile < 0 || tile >= cap) continue;
     const TilePos tp = tile_pos(grid, tile);
+    if (PRED) {
+      const int oy = tp.y0 + (tid >> 3), ox = tp.x0 + (tid & 7);
+      if (tid < 64 && oy < hout && ox < wout) pt.out[((long long)tp.n * hout + oy) * wout + ox] = (mie_bf16)0.f;
+      continue;
+    }
     for (int idx = tid; idx < 64 * (COUT / 4); idx += 256) {
       const int p = idx / (COUT / 4), col = 4 * (idx - p * (COUT / 4));
       const int oy = tp.y0 + (p >> 3), ox = tp.x0 + (p & 7);
@@ -146,6 +173,13 @@ __global__ __launch_bounds__(256, 2) void k_upconv64_persist(ConvArgsT<mie_bf16>
     const mie_bf16* fb = a.filt_mc + ((long long)wave * (K * K) * 2 * COUT) * EPS + (half * COUT + l32) * EPS;
 #pragma unroll
     for (int tap = 0; tap < K * K; ++tap) bfrag[tap] = *reinterpret_cast<const float4*>(fb + (long long)tap * 2 * COUT * EPS);
+  }
+
+  // ---- the tail's weights of this thread's four channels (its column group is the same in both epilogue groups) ----
+  float4 pw_y = make_float4(0.f, 0.f, 0.f, 0.f), pw_s = pw_y;
+  if (PRED) {
+    pw_y = *reinterpret_cast<const float4*>(pt.w + 4 * (tid & 7));
+    pw_s = *reinterpret_cast<const float4*>(pt.w + COUT + 4 * (tid & 7));
   }
 
   // ---- per-thread constants of the staging plan -------------------------------------------------------------------
@@ -211,6 +245,9 @@ __global__ __launch_bounds__(256, 2) void k_upconv64_persist(ConvArgsT<mie_bf16>
     long long e_off[2];
     bool e_ok[2];
     float4 e_r0[2];
+    long long t_pix[2];          // PRED: pixel index, the second delta's four channels, the prediction's reservoir value
+    float4 t_skip[2];
+    float t_p0[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int idx = tid + 256 * i;
@@ -220,6 +257,18 @@ __global__ __launch_bounds__(256, 2) void k_upconv64_persist(ConvArgsT<mie_bf16>
       e_off[i] = (((long long)n * hout + oy) * wout + ox) * COUT + col;
       e_r0[i] = make_float4(0.f, 0.f, 0.f, 0.f);
       if (RES && e_ok[i]) e_r0[i] = *reinterpret_cast<const float4*>(a.res + e_off[i]);
+      if (PRED) {
+        const long long pix = ((long long)n * hout + oy) * wout + ox;
+        t_pix[i] = pix;
+        t_skip[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        t_p0[i] = 0.f;
+        if (e_ok[i]) {
+          const bool on = pt.skip_mask == nullptr || pt.skip_mask[pix] != 0;
+          const mie_bf16x4 sv = *reinterpret_cast<const mie_bf16x4*>(pt.skip + pix * COUT + col);
+          if (on) t_skip[i] = make_float4((float)sv[0], (float)sv[1], (float)sv[2], (float)sv[3]);
+          if ((tid & 7) == 0) t_p0[i] = pt.res[pix];
+        }
+      }
     }
 
     // C. the next tile's source pixels and the list entry after it
@@ -321,9 +370,37 @@ __global__ __launch_bounds__(256, 2) void k_upconv64_persist(ConvArgsT<mie_bf16>
         }
         v[i] = sum;
       }
+      if constexpr (PRED) {
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
-        if (e_ok[i]) epilogue4<RES, ACT>(a, e_off[i], v[i], e_r0[i]);
+        for (int i = 0; i < 2; ++i) {
+          const float4 r0 = e_r0[i];
+          const float4 r1 = make_float4(r0.x + v[i].x, r0.y + v[i].y, r0.z + v[i].z, r0.w + v[i].w);
+          if (e_ok[i]) mie_st4(a.res, e_off[i], r1);
+          // the increment as the bf16 delta it would be stored as
+          const float y0_ = (float)(mie_bf16)(mie_act(ACT, a.slope, r1.x) - mie_act(ACT, a.slope, r0.x));
+          const float y1_ = (float)(mie_bf16)(mie_act(ACT, a.slope, r1.y) - mie_act(ACT, a.slope, r0.y));
+          const float y2_ = (float)(mie_bf16)(mie_act(ACT, a.slope, r1.z) - mie_act(ACT, a.slope, r0.z));
+          const float y3_ = (float)(mie_bf16)(mie_act(ACT, a.slope, r1.w) - mie_act(ACT, a.slope, r0.w));
+          float z = pw_y.x * y0_ + pw_y.y * y1_ + pw_y.z * y2_ + pw_y.w * y3_;
+          z += pw_s.x * t_skip[i].x + pw_s.y * t_skip[i].y + pw_s.z * t_skip[i].z + pw_s.w * t_skip[i].w;
+          if (!e_ok[i]) z = 0.f;
+          // the eight lanes of a pixel, by data-parallel moves inside the wave's rows of 16 (no LDS round trip):
+          // neighbours within quads, then the quad four lanes up -- complete in the lanes 0 and 8 of a row, the ones
+          // that own the pixel's prediction
+          z += dpp_f32<0xB1>(z);               // quad_perm [1,0,3,2]
+          z += dpp_f32<0x4E>(z);               // quad_perm [2,3,0,1]
+          z += dpp_f32<0x104>(z);              // row_shl:4 (lane l reads lane l + 4)
+          if (e_ok[i] && (tid & 7) == 0) {
+            const float p1 = t_p0[i] + z;
+            pt.res[t_pix[i]] = p1;
+            pt.out[t_pix[i]] = (mie_bf16)(mie_act(pt.act, pt.slope, p1) - mie_act(pt.act, pt.slope, t_p0[i]));
+          }
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+          if (e_ok[i]) epilogue4<RES, ACT>(a, e_off[i], v[i], e_r0[i]);
+      }
     }
     // (the next tile's barriers (1) and (2) stand between these reads of s_red and its next writes, barrier (3) between
     // this tile's reads of s_lo / s_stage and their next writes)
@@ -336,23 +413,45 @@ __global__ __launch_bounds__(256, 2) void k_upconv64_persist(ConvArgsT<mie_bf16>
 
 // Takes the shape of the batched bf16 network's last decoder on planes large enough to keep the resident grid busy
 // (launches nothing and returns false otherwise; MIE_UPCONV_PERSIST=0 switches the kernel off, for measurements).
-bool mie_launch_upconv_persist(const ConvArgsT<mie_bf16>& a, unsigned cap, hipStream_t st) {
+static bool persist_takes(const ConvArgsT<mie_bf16>& a, unsigned cap) {
   static const bool enabled = [] {
     const char* e = getenv("MIE_UPCONV_PERSIST");
     return e == nullptr || atoi(e) != 0;
   }();
   if (!enabled || a.c1 != C || a.cout != COUT || a.pad != 2 || a.refresh || a.filt_mc == nullptr || a.x3 || a.addend != nullptr) return false;
   if (a.x2 != nullptr && a.c2 != C) return false;
-  if (cap < 4u * GRID || cap > (1u << 20)) return false;      // small planes: one tile per workgroup is as good
+  return cap >= 4u * GRID && cap <= (1u << 20);      // small planes: one tile per workgroup is as good
+}
+
+bool mie_launch_upconv_persist(const ConvArgsT<mie_bf16>& a, unsigned cap, hipStream_t st) {
+  if (!persist_takes(a, cap)) return false;
   const dim3 g(GRID), b(256);
+  const PredTail none = {};
   if (a.res == nullptr) {
-    hipLaunchKernelGGL((k_upconv64_persist<false, MIE_ACT_NONE>), g, b, 0, st, a);
+    hipLaunchKernelGGL((k_upconv64_persist<false, MIE_ACT_NONE>), g, b, 0, st, a, none);
     return true;
   }
   switch (a.act) {
-    case MIE_ACT_NONE: hipLaunchKernelGGL((k_upconv64_persist<true, MIE_ACT_NONE>), g, b, 0, st, a); return true;
-    case MIE_ACT_RELU: hipLaunchKernelGGL((k_upconv64_persist<true, MIE_ACT_RELU>), g, b, 0, st, a); return true;
-    case MIE_ACT_LEAKY_RELU: hipLaunchKernelGGL((k_upconv64_persist<true, MIE_ACT_LEAKY_RELU>), g, b, 0, st, a); return true;
+    case MIE_ACT_NONE: hipLaunchKernelGGL((k_upconv64_persist<true, MIE_ACT_NONE>), g, b, 0, st, a, none); return true;
+    case MIE_ACT_RELU: hipLaunchKernelGGL((k_upconv64_persist<true, MIE_ACT_RELU>), g, b, 0, st, a, none); return true;
+    case MIE_ACT_LEAKY_RELU: hipLaunchKernelGGL((k_upconv64_persist<true, MIE_ACT_LEAKY_RELU>), g, b, 0, st, a, none); return true;
     default: return false;                                      // sigmoid / tanh epilogues: the one-tile kernel
+  }
+}
+
+// The same with the network's tail fused in (a.out is not written): see PredTail.
+bool mie_launch_upconv_pred_persist(const ConvArgsT<mie_bf16>& a, const mie_bf16* skip, const uint8_t* skip_mask,
+                                    const float* pred_w, float* pred_res, mie_bf16* pred_out, int pred_act,
+                                    float pred_slope, unsigned cap, hipStream_t st) {
+  if (!persist_takes(a, cap) || a.res == nullptr) return false;
+  PredTail pt;
+  pt.skip = skip; pt.skip_mask = skip_mask; pt.w = pred_w; pt.res = pred_res; pt.out = pred_out; pt.act = pred_act;
+  pt.slope = pred_slope;
+  const dim3 g(GRID), b(256);
+  switch (a.act) {
+    case MIE_ACT_NONE: hipLaunchKernelGGL((k_upconv64_persist<true, MIE_ACT_NONE, true>), g, b, 0, st, a, pt); return true;
+    case MIE_ACT_RELU: hipLaunchKernelGGL((k_upconv64_persist<true, MIE_ACT_RELU, true>), g, b, 0, st, a, pt); return true;
+    case MIE_ACT_LEAKY_RELU: hipLaunchKernelGGL((k_upconv64_persist<true, MIE_ACT_LEAKY_RELU, true>), g, b, 0, st, a, pt); return true;
+    default: return false;
   }
 }

@@ -624,6 +624,9 @@ class UNetRecurrentIncr(BaseUNetIncr):
         for resblock in self.resblocks:
             x_incr = resblock(x_incr)
         for i, decoder in enumerate(self.decoders):
+            if i == self.num_encoders - 1 and self._tail_is_fusable(decoder, x_incr, head):
+                # last decoder, skip sum, prediction conv and output activation in one kernel
+                return self._fused_tail(decoder, x_incr, blocks[0], head), states_incr
             x_incr = decoder(x_incr, blocks[self.num_encoders - i - 1])
         if self.fuse and self.norm not in ['BN', 'IN']:
             # skip sum, 1x1 conv and output activation in one kernel: the conv is linear, so
@@ -634,6 +637,55 @@ class UNetRecurrentIncr(BaseUNetIncr):
         else:
             pred_incr = self.activation(self.pred(self.pred_add(x_incr, head)))
         return pred_incr, states_incr
+
+    def _tail_is_fusable(self, decoder, x_incr, head) -> bool:
+        """The shape ops.upconv_pred_masked takes: up-sampling decoder 64 -> 32 with a ReLU-kind activation on bf16
+        deltas, exact masks, one prediction channel, a plane of at least 2048 tiles."""
+        if not (self.fuse and self.norm not in ['BN', 'IN'] and isinstance(decoder, UpsampleConvLayerIncr)
+                and decoder.activation is not None and self.num_output_channels == 1):
+            return False
+        conv, pconv = decoder.conv2d, self.pred.conv2d
+        if conv.lossy or pconv.lossy or not isinstance(head[1] if len(head) > 1 else None, TileMask):
+            return False
+        x = x_incr[0]
+        k, s, p = conv._geometry()
+        tiles = x.shape[0] * ((2 * x.shape[2] + 7) // 8) * ((2 * x.shape[3] + 7) // 8)
+        try:
+            kind, _ = activation_kind(decoder.activation.op)
+        except NotImplementedError:
+            return False
+        return ops.upconv_pred_takes(x.shape[1], conv.out_channels, k, s, p, conv.conv2d_weights,
+                                     ops.delta_torch_dtype(x), tiles, kind)
+
+    def _fused_tail(self, decoder, x_incr, skip_incr, head):
+        conv, pconv, up = decoder.conv2d, self.pred.conv2d, decoder.upsample
+        k, s, p = conv._geometry()
+        a, pa, b, pb, ts_up = up.plan(x_incr, skip_incr)
+        n, _, h, w = a.shape
+        H, W = 2 * h, 2 * w
+        ts_dec = conv._tile_set("out_act", n, H, W, a.device)           # the decoder's own output set ...
+        ops.build_mask_tiles(ts_up, None, n, H, W, _lib.FOOT_CONV, k, s, p, ts_dec)
+        ts_pred = pconv._tile_set("out_act", n, H, W, a.device)          # ... and the prediction's: its union with the head's
+        ops.build_mask_tiles(ts_dec, head[1], n, H, W, _lib.FOOT_CONV, 1, 1, 0, ts_pred)
+        res, pres = decoder.activation.in_res.reservoir, self.activation.in_res.reservoir
+        if res is None or pres is None:
+            raise RuntimeError("fused tail: call forward_refresh_reservoirs first")
+        kind, slope = activation_kind(decoder.activation.op)
+        pkind, pslope = activation_kind(self.activation.op)
+        out = pconv._delta_buf("out_act", (n, 1, H, W), a.device, a.dtype)
+        ops.upconv_pred_masked(a, pa, b, pb, conv.conv2d_weights, ts_pred, res, kind, slope, ops.as_nhwc(head[0]), head[1],
+                               self._pred_tail_weights(), pres, pkind, pslope, out)
+        return [out, ts_pred]
+
+    def _pred_tail_weights(self):
+        base = self.pred.conv2d.conv2d_weights
+        cached = self.__dict__.get("_pred_tail_w")
+        if cached is None or cached[0] is not base:
+            # [Cin, 1, 1, 1] -> (1, Cin), rounded to bf16 like every weight a bf16 network multiplies
+            row = base.for_dtype(torch.bfloat16)[0].reshape(1, -1).float()
+            cached = (base, torch.cat((row, row), 0).contiguous())
+            self.__dict__["_pred_tail_w"] = cached
+        return cached[1]
 
     def _pred_sum_filter(self):
         base = self.pred.conv2d.conv2d_weights

@@ -568,6 +568,49 @@ def upconv_masked(a, amask, b, bmask, filt, k, pad, out_ts: TileMask, out_delta,
     return out_delta
 
 
+# Planes the fused tail kernel takes (the persistent last-decoder kernel: tiles of the whole batch).
+UPCONV_PRED_MIN_TILES, UPCONV_PRED_MAX_TILES = 2048, 1 << 20
+upconv_pred_enabled = os.environ.get("MIE_UPCONV_PRED", "1") != "0"
+
+
+def upconv_pred_takes(c: int, cout: int, k: int, stride: int, pad: int, filt, dtype, tiles: int, act: int) -> bool:
+    """Whether upconv_pred_masked has a kernel for this last-decoder shape (else: upconv_masked + conv_masked)."""
+    return (upconv_pred_enabled and dtype == torch.bfloat16 and c == 64 and cout == 32 and k == 5 and stride == 1
+            and pad == 2 and UPCONV_PRED_MIN_TILES <= tiles <= UPCONV_PRED_MAX_TILES
+            and act in (_lib.ACT_NONE, _lib.ACT_RELU, _lib.ACT_LEAKY_RELU)
+            and isinstance(filt, ConvFilter) and filt.for_dtype(dtype)[1] is not None)
+
+
+def upconv_pred_masked(a, amask, b, bmask, filt, out_ts: TileMask, reservoir, act, slope, skip, skip_mask, pred_w,
+                       pred_res, pred_act, pred_slope, pred_out):
+    """Last decoder (5x5 conv over up2x(a + b), 64 -> 32 bf16 channels, reservoir + activation) with the 1x1
+    prediction conv over (its increment + skip), the prediction's reservoir and activation increment in its epilogue.
+    out_ts: the prediction's tile set; pred_w: fp32 [2, 32] (weights of the increment, of skip); pred_res fp32 and
+    pred_out bf16, both (N, 1, 2H, 2W)."""
+    n, c, h, w = a.shape
+    dt = a.dtype
+    if b is not None and (b.shape != a.shape or b.dtype != dt):
+        raise ValueError("b %s %s does not match a %s %s" % (tuple(b.shape), b.dtype, tuple(a.shape), dt))
+    plain, mc_ptr, code = _filter_args(filt, 5, dt, None, with_code=True)
+    cin_total, cout = plain.shape[0], plain.shape[3]
+    full = (n, cout, 2 * h, 2 * w)
+    if tuple(reservoir.shape) != full or tuple(skip.shape) != full or skip.dtype != dt:
+        raise ValueError("reservoir %s / skip %s %s, expected %s %s" % (tuple(reservoir.shape), tuple(skip.shape), skip.dtype, full, dt))
+    if tuple(pred_res.shape) != (n, 1, 2 * h, 2 * w) or tuple(pred_out.shape) != (n, 1, 2 * h, 2 * w) or pred_out.dtype != dt:
+        raise ValueError("prediction buffers must be (%d, 1, %d, %d)" % (n, 2 * h, 2 * w))
+    if pred_w.dtype != torch.float32 or tuple(pred_w.shape) != (2, cout) or not pred_w.is_contiguous():
+        raise ValueError("pred_w must be contiguous fp32 (2, %d)" % cout)
+    _require_gpu(pred_w, "pred_w")
+    _ready(out_ts)
+    check(lib().mie_upconv_pred_masked(
+        nhwc_ptr(a, "a", dtype=dt), pix_ptr(amask, n, h, w, "amask"), nhwc_ptr(b, "b", dtype=dt),
+        pix_ptr(bmask, n, h, w, "bmask"), c, h, w, plain.data_ptr(), mc_ptr, cin_total, cout, out_ts.ref,
+        nhwc_ptr(reservoir, "reservoir"), act, float(slope), nhwc_ptr(skip, "skip", dtype=dt),
+        pix_ptr(skip_mask, n, 2 * h, 2 * w, "skip_mask"), pred_w.data_ptr(), nhwc_ptr(pred_res, "pred_res"), pred_act,
+        float(pred_slope), nhwc_ptr(pred_out, "pred_out", dtype=dt), code, _stream(a)))
+    return pred_out
+
+
 def conv_refresh(x, x2, filt, bias, k, stride, pad, out_ts: TileMask, out_dense, reservoir=None,
                  act=_lib.ACT_NONE, slope=0.0, path=_lib.PATH_AUTO, addend=None):
     """Dense conv + bias (+ activation, + reservoir fill) over the tiles of out_ts (all active)."""

@@ -673,3 +673,66 @@ def test_persistent_upsampled_conv_agrees_with_the_one_tile_kernel():
             assert torch.allclose(res_big.cpu(), res_ref, rtol=RTOL, atol=bf16_atol(ref, 2.0))
         # clean delta: zero outside the active pixels of the tile set
         assert torch.count_nonzero(big["out"].float() * (1 - big["ts"].pixmask.float())) == 0
+
+
+def test_fused_tail_equals_decoder_then_prediction():
+    # mie_upconv_pred_masked: last decoder + 1x1 prediction over (its increment + a second delta) + sigmoid increment in
+    # one kernel, against the two launches it replaces (same decoder arithmetic: the decoder's reservoir must come out
+    # bit-equal; the prediction's 64-term sum is regrouped, fp32) and against a CPU restatement.  Four steps with
+    # fresh masks: stale tiles of the prediction's set, an empty step, one input only.
+    bf = torch.bfloat16
+    n, c, cout, h, w = 3, 64, 32, 100, 118
+    H, W = 2 * h, 2 * w
+    q = lambda t: t.to(bf).float()
+    wt = q(he_normal_conv_weight(cout, c, 5, 9))
+    filt = _filt(wt)
+    pw = q(torch.randn(cout, generator=torch.Generator().manual_seed(4)) * 0.3)      # bf16 networks carry bf16 weights
+    pred_filt = _filt(torch.cat((pw, pw)).reshape(1, 2 * cout, 1, 1))                  # [1, 64, 1, 1] -> rows repeated
+    pred_w = torch.stack((pw, pw)).contiguous().to(DEV)
+    assert ops.upconv_pred_takes(c, cout, 5, 1, 2, filt, bf, _lib.tile_capacity(n, H, W), _lib.ACT_RELU)
+    sets = [dict(up=TileMask(n, H, W, DEV), dec=TileMask(n, H, W, DEV), pred=TileMask(n, H, W, DEV)) for _ in range(2)]
+    y_buf = ops.new_nhwc(n, cout, H, W, DEV, bf)
+    outs = [ops.new_nhwc(n, 1, H, W, DEV, bf) for _ in range(2)]
+    r0 = gaussian_delta(n, cout, H, W, 1.0, 1.0, seed=3)[0]
+    p0 = gaussian_delta(n, 1, H, W, 1.0, 1.0, seed=5)[0]
+    res = [_dev(r0).clone() for _ in range(2)]
+    pres = [_dev(p0).clone() for _ in range(2)]
+    res_ref, pres_ref = r0.clone(), p0.clone()
+    for step, (da, db, ds, two) in enumerate([(0.2, 0.1, 0.1, True), (0.0, 0.0, 0.0, True), (0.05, 0.0, 0.3, False), (0.3, 0.2, 0.02, True)]):
+        zeros = lambda ch, hh, ww: (torch.zeros(n, ch, hh, ww), torch.zeros(n, 1, hh, ww, dtype=torch.uint8))
+        a, ma = gaussian_delta(n, c, h, w, da, 0.5, seed=100 + step) if da > 0 else zeros(c, h, w)
+        b, mb = gaussian_delta(n, c, h, w, db, 0.5, seed=200 + step) if db > 0 else zeros(c, h, w)
+        sk, ms = gaussian_delta(n, cout, H, W, ds, 0.5, seed=300 + step) if ds > 0 else zeros(cout, H, W)
+        a, b, sk = q(a), q(b), q(sk)
+        ad, bd, am, bm = _dev(a).to(bf), _dev(b).to(bf), ma.to(DEV), mb.to(DEV)
+        skd, msd = _dev(sk).to(bf), ms.to(DEV)
+        for s_ in sets:
+            ops.build_mask_tiles(am, bm if two else None, n, h, w, _lib.FOOT_UP2X, 0, 0, 0, s_["up"])
+            ops.build_mask_tiles(s_["up"], None, n, H, W, _lib.FOOT_CONV, 5, 1, 2, s_["dec"])
+            ops.build_mask_tiles(s_["dec"], msd, n, H, W, _lib.FOOT_CONV, 1, 1, 0, s_["pred"])
+        # the two launches
+        ops.upconv_masked(ad, am, bd if two else None, bm if two else None, filt, 5, 2, sets[0]["dec"], y_buf, res[0], _lib.ACT_RELU)
+        ops.conv_masked(y_buf, sets[0]["dec"], skd, msd, pred_filt, 1, 1, 0, sets[0]["pred"], outs[0], pres[0], _lib.ACT_SIGMOID)
+        # the one
+        ops.upconv_pred_masked(ad, am, bd if two else None, bm if two else None, filt, sets[1]["pred"], res[1], _lib.ACT_RELU, 0.0,
+                               skd, msd, pred_w, pres[1], _lib.ACT_SIGMOID, 0.0, outs[1])
+        torch.cuda.synchronize()
+        # CPU restatement
+        conv = io.conv_incr(q(io.interp_incr(a + b if two else a)), wt, 1, 2)
+        y = q(torch.relu(res_ref + conv) - torch.relu(res_ref))
+        res_ref = res_ref + conv
+        z = ((y + sk) * pw.view(1, -1, 1, 1)).sum(1, keepdim=True)
+        want = torch.sigmoid(pres_ref + z) - torch.sigmoid(pres_ref)
+        pres_ref = pres_ref + z
+        assert torch.equal(res[0], res[1]), "step %d: decoder reservoir" % step
+        assert torch.allclose(pres[0], pres[1], rtol=1e-5, atol=1e-5), "step %d: prediction reservoir %.3e" % (step, (pres[0] - pres[1]).abs().max())
+        assert torch.allclose(outs[0].float(), outs[1].float(), rtol=2 ** -7, atol=2 ** -9), "step %d: prediction delta %.3e" % (
+            step, (outs[0].float() - outs[1].float()).abs().max())
+        # (the GPU's y differs from the CPU's by a bf16 rounding step where the conv sums differ in their last bits: a few
+        # 1e-4 per step on a reservoir of order 1, carried over the steps)
+        assert torch.allclose(pres[1].cpu(), pres_ref, rtol=1e-3, atol=4e-3), "step %d: reservoir vs CPU %.3e" % (
+            step, (pres[1].cpu() - pres_ref).abs().max())
+        assert torch.allclose(outs[1].float().cpu(), want, rtol=BF16_RTOL, atol=2e-3), "step %d: delta vs CPU %.3e" % (
+            step, (outs[1].float().cpu() - want).abs().max())
+        # clean delta: zero outside the pixels of the prediction's tile set
+        assert torch.count_nonzero(outs[1].float() * (1 - sets[1]["pred"].pixmask.float())) == 0
