@@ -137,6 +137,11 @@ class LayerProbe:
             return dict(kind="conv", k=k, s=1, cin=c, cout=filt.shape[3], h=h, w=w, n=n, xmask=amask,
                         x2mask=bmask, ts=out_ts, fused=reservoir is not None, up=True, two=b_ is not None)
 
+        def upconv_pred_desc(a_, amask, b_, bmask, filt, out_ts, reservoir, act, slope, skip, skip_mask, *a, **kw):
+            n, c, h, w = a_.shape
+            return dict(kind="conv", k=5, s=1, cin=c, cout=filt.shape[3], h=h, w=w, n=n, xmask=amask, x2mask=bmask,
+                        ts=out_ts, fused=True, up=True, two=b_ is not None, pred=True, skip_mask=skip_mask)
+
         def tconv2x_desc(x, xmask, x2, x2mask, filt, k, out_ts, block_ts, out_delta, reservoir=None, *a, **kw):
             n, c1, h, w = x.shape
             c2 = 0 if x2 is None else x2.shape[1]
@@ -152,6 +157,7 @@ class LayerProbe:
         self._wrap("tconv2x_masked", tconv2x_desc)
         self._wrap("tconv_masked", tconv_desc)
         self._wrap("upconv_masked", upconv_desc)
+        self._wrap("upconv_pred_masked", upconv_pred_desc)
         self._wrap("conv_gates_incr", conv_gates_desc)
         self._wrap("act_incr", pw_desc("act", 1, 1))
         self._wrap("add_incr", pw_desc("add", 2, 0))
@@ -190,17 +196,23 @@ class LayerProbe:
                     # hidden and cell deltas written; the 4*hid-channel gate delta never reaches memory
                     hid = cout // 4
                     byts += a_out * (2 * cout * 4 + 2 * hid * 4 + hid * 4 + 2 * hid * es)
+                elif d.get("pred"):
+                    # fused tail: the layer's reservoir read + written, its delta never stored; the second delta of the
+                    # prediction conv read where its mask is set; prediction reservoir read + written, prediction delta
+                    a_skip = a_out if d["skip_mask"] is None else int(self._pix(d["skip_mask"]).sum().item())
+                    byts += 2 * a_out * cout * 4 + a_skip * cout * es + a_out * (8 + es)
                 else:
                     byts += a_out * cout * es
                     if d["fused"]:
                         byts += 2 * a_out * cout * 4
-                flops = 2 * a_out * cin * cout * k * k
+                flops = 2 * a_out * cin * cout * k * k + (4 * a_out * cout if d.get("pred") else 0)
                 if d.get("tconv"):
                     # stride-s transposed conv: an output pixel meets (k/s)^2 taps on average
                     flops = 2 * a_out * cin * cout * k * k // (d["s"] * d["s"])
                 row.update(shape="%s%dx%d s%d %d->%d%s @%dx%d" % ("up2x+" if d.get("up") else ("tconv " if d.get("tconv") else ""),
                                                                    k, k, d["s"], cin, cout,
-                                                                   "+lstm" if d.get("gates") else "", ts.h, ts.w),
+                                                                   "+lstm" if d.get("gates") else ("+pred" if d.get("pred") else ""),
+                                                                   ts.h, ts.w),
                            active_tiles=int(ts.counts[0].item()), tiles=ts.capacity, a_out=a_out,
                            bytes=byts, flops=flops)
             elif d["kind"] in ("act", "add", "mul", "up2x", "gates"):
@@ -421,7 +433,7 @@ class NetBench:
         of its own, so that the figure is the kernel's duration and not the 3-4 us from the end of one launch
         to the start of the next (what a kernel trace reports as the kernel's average duration)."""
         torch = self.torch
-        convs = [l for l in layers if l["op"] in ("conv_masked", "conv_gates_incr", "upconv_masked", "tconv2x_masked")]
+        convs = [l for l in layers if l["op"] in ("conv_masked", "conv_gates_incr", "upconv_masked", "upconv_pred_masked", "tconv2x_masked")]
         dom = max(convs, key=lambda l: l["us"])
         orig, cargs, ckw = agg[layers.index(dom)]["call"]
         with torch.no_grad():
