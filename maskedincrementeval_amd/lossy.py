@@ -113,7 +113,7 @@ def lossy_frontier(nb, exact_model, log, steps=50, time_steps=50, repeats=5):
         del m
     torch.cuda.empty_cache()
     best = [r for r in rows if r["speedup"] >= 5.0]
-    return dict(steps=steps, exact_inline_ms_per_step=round(1e3 * t_exact, 4),
+    return dict(steps=steps, exact_inline_ms_per_step=round(1e3 * t_exact, 4), captured=True,
                 note="prediction is a sigmoid output in (0, 1); deviation is of refresh + sum of %d increments "
                      "against the exact incremental network on the same inputs" % steps,
                 reaches_5x=[dict(method=r["method"], param=r["param"], max_abs_deviation=r["max_abs_deviation"])
