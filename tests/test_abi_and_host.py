@@ -178,6 +178,43 @@ def test_mask_plan_rejects_what_it_cannot_run(mie_lib):
     assert plan((p, None, 16, 16, _lib.FOOT_CONV, 3, 1, 1, bad)) == -1
 
 
+def test_newer_entry_points_reject_bad_arguments(mie_lib):
+    # host-side validation of the fused tail, the workspace forms and the bf16 event frame: every call returns before
+    # anything is launched
+    err = lambda: mie_lib.mie_last_error_string().decode()
+    big, keep = _fake_tileset(h=32, w=32)
+    buf = ctypes.create_string_buffer(8192)
+    p = (ctypes.addressof(buf) + 255) & ~255
+    q = p + 1024
+    BF16, F32 = 1, 0
+
+    def pred(c=64, cout=32, dtype=BF16, act=1, h=16, w=16, skip=q, out=big, pdelta=p + 2048):
+        return mie_lib.mie_upconv_pred_masked(p, None, None, None, c, h, w, p, p, c, cout, ctypes.byref(out), p + 512, act, 0.0,
+                                              skip, None, p + 768, p + 1280, 3, 0.0, pdelta, dtype, None)
+    assert pred(dtype=F32) == -2 and "bf16" in err()
+    assert pred(c=128) == -2 and pred(cout=64) == -2
+    assert pred(skip=None) == -1 and "NULL" in err()
+    assert pred(h=15) == -1 and "twice the input" in err()
+    assert pred(act=3) == -2 and "activation" in err()                # sigmoid on the decoder: the separate kernels
+    assert pred(pdelta=q) == -1 and "alias" in err()
+
+    # workspace forms: alignment, size without a pointer, aliasing
+    up = lambda ws, nbytes: mie_lib.mie_upconv_masked_ws(p, None, None, None, 64, 16, 16, p, p, 64, 5, 2, 32, ctypes.byref(big),
+                                                         p + 4096, None, None, 0, 0.0, F32, ws, nbytes, None)
+    assert up(p + 5000 + 4, 1024) == -1 and "workspace" in err()
+    assert up(None, 1024) == -1 and "workspace" in err()
+    assert up(p + 4096, 1024) == -1 and "alias" in err()
+    gates = lambda ws, nbytes: mie_lib.mie_conv_gates_masked_ws(p, None, 32, q, None, 32, 32, 32, p, p, 64, 32, ctypes.byref(big),
+                                                                p + 512, None, None, p + 1024, p + 1536, p + 2048, p + 2560,
+                                                                F32, ws, nbytes, None)
+    assert gates(p + 2048, 4096) == -1 and "alias" in err()
+    assert gates(p + 6000 + 4, 64) == -1 and "workspace" in err()
+
+    # bf16 event frame: the rounded frame is a buffer of its own
+    ev = lambda out: mie_lib.mie_events_to_frame_bf16(None, 0, 0, 5, 8, 8, 0, 0, 0, 0, 1.0, 0.0, 0.0, -1.0, 0, p, out, q, None)
+    assert ev(p + 4096) == -1 and "window length" in err()             # the base entry point's checks come first
+
+
 def test_check_raises_runtime_error(mie_lib):
     rc = mie_lib.mie_mask_from_delta(None, 1, 4, 4, 4, 0.0, None, 0, None)
     with pytest.raises(RuntimeError, match="NULL pointer"):

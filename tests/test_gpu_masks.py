@@ -288,3 +288,59 @@ def test_mask_plan_of_a_large_plane_and_many_samples():
         m = mo.footprint_conv(m, k, s, p)
         _check_tileset(sets[nm], m)
     _check_tileset(batch[-1][-1], mo.footprint_conv(mo.footprint_conv(x, 5, 1, 2) | x, 3, 1, 1))
+
+
+def test_mask_plan_holds_a_whole_unet_chain_at_full_resolution():
+    # The 18 tile sets of E2Depth-incr at 8 x 480 x 640 in ONE plan: four full-resolution bitmaps of 38.4 KB live at
+    # its end (head, the up-sampled mask, the last decoder's, their union), which fits a CU's 160 KB only with the LDS
+    # slots packed from their lifetimes and the final union written in place over the head's bitmap.  Two steps with
+    # different masks (stale lists); every set against the chained mask oracle.
+    import mask_chain
+    n, h, w = 8, 480, 640
+    c2 = lambda v: (v + 4 - 5) // 2 + 1
+    planes = [(h, w)]
+    for _ in range(3):
+        planes.append((c2(planes[-1][0]), c2(planes[-1][1])))
+    S = lambda pl: TileMask(n, pl[0], pl[1], DEV)
+    sets = {"head": S(planes[0])}
+    ops_ = [("head", ("x", None), planes[0], _lib.FOOT_CONV, 5, 1, 2)]
+    prev = "head"
+    for i in range(3):
+        sets["enc%d.conv" % i], sets["enc%d.gates" % i] = S(planes[i + 1]), S(planes[i + 1])
+        ops_.append(("enc%d.conv" % i, (prev, None), planes[i], _lib.FOOT_CONV, 5, 2, 2))
+        ops_.append(("enc%d.gates" % i, ("enc%d.conv" % i, None), planes[i + 1], _lib.FOOT_CONV, 3, 1, 1))
+        prev = "enc%d.gates" % i
+    for j in range(2):
+        for c in ("conv1", "conv2"):
+            name = "res%d.%s" % (j, c)
+            sets[name] = S(planes[3])
+            ops_.append((name, (prev, None), planes[3], _lib.FOOT_CONV, 3, 1, 1))
+            prev = name
+    for i in range(3):
+        lo, hi = planes[3 - i], planes[2 - i]
+        sets["dec%d.up" % i], sets["dec%d.conv" % i] = S(hi), S(hi)
+        ops_.append(("dec%d.up" % i, (prev, "enc%d.gates" % (2 - i)), lo, _lib.FOOT_UP2X, 0, 0, 0))
+        ops_.append(("dec%d.conv" % i, ("dec%d.up" % i, None), hi, _lib.FOOT_CONV, 5, 1, 2))
+        prev = "dec%d.conv" % i
+    sets["pred"] = S(planes[0])
+    ops_.append(("pred", (prev, "head"), planes[0], _lib.FOOT_CONV, 1, 1, 0))
+    assert len(ops_) == 18
+    prev_lists = {}
+    for step, dens in enumerate((0.01, 0.002)):
+        x = np.stack([blob_mask(h, w, dens, seed=40 * step + b) for b in range(n)])
+        xd = _to_dev_mask(x)
+        ptr = lambda nm: None if nm is None else (xd.data_ptr() if nm == "x" else sets[nm].pixmask.data_ptr())
+        batch = [(ptr(a), ptr(b), pl[0], pl[1], foot, k, s, p, sets[name]) for name, (a, b), pl, foot, k, s, p in ops_]
+        rc = _lib.lib().mie_build_mask_plan(ops._plan_ops(batch), len(batch), torch.cuda.current_stream().cuda_stream)
+        if rc == -3:
+            assert "LDS" in _lib.lib().mie_last_error_string().decode()
+            pytest.skip("this device offers a workgroup less LDS than the chain needs")
+        _lib.check(rc)
+        torch.cuda.synchronize()
+        want = mask_chain.e2depth_chain(mo.footprint_conv(x, 1, 1, 0))
+        for name in sets:
+            _check_tileset(sets[name], want[name])
+            tiles = mo.tile_list(want[name])
+            assert np.array_equal(sets[name].stale_tiles().cpu().numpy(),
+                                  mo.stale_list(prev_lists.get(name, np.zeros(0, dtype=np.int32)), tiles)), name
+            prev_lists[name] = tiles
