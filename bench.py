@@ -55,6 +55,10 @@ def parse_args():
     ap.add_argument("--batch", type=int, default=1, help="independent event streams per step (8 with 480x640: the batched configuration)")
     ap.add_argument("--cpu-steps", type=int, default=400, help="incremental steps of the CPU baseline (0 = skip)")
     ap.add_argument("--no-graph", action="store_true", help="launch kernels eagerly instead of replaying a HIP graph")
+    ap.add_argument("--plan-ahead", choices=["streams", "fork", "off"], default="fork",
+                    help="plan the next step's tile sets beside this step's kernels: 'streams' = planning and compute "
+                         "halves as two graphs on two streams, ordered by events between the replays; 'fork' = one graph "
+                         "per step with the plan forked inside it; 'off' = every step plans its own tile sets first")
     ap.add_argument("--copy-input", action="store_true",
                     help="one captured graph and a device-to-device copy of the next delta into its input buffer before every "
                          "replay (default: one graph per resident input, no copy)")
@@ -274,6 +278,9 @@ class NetBench:
             from maskedincrementeval_amd.evflownet_incr import MultiResUNetRecurrentIncr
             self.make_net = lambda **kw: MultiResUNetRecurrentIncr(num_bins=4, decoder=wl.decoder, **kw)
             self.run_net = lambda m, x: m([x, None])
+            self.run_pipe = lambda m, x, nxt, par: m.forward_pipelined([x, None], [nxt, None], par)
+            self.run_planned = lambda m, x, par: m.forward_planned([x, None], par)
+            self.run_plan = lambda m, x, par: m.plan_ahead([x, None], par)
             self.out_of = lambda r: r[-1][0]                      # the finest flow scale
             self.refresh_net = lambda m, x: m.forward_refresh_reservoirs(x)
             self.refresh_out = lambda r: r[-1]
@@ -281,6 +288,9 @@ class NetBench:
             from maskedincrementeval_amd.e2depth_incr import E2VIDRecurrentIncr
             self.make_net = E2VIDRecurrentIncr
             self.run_net = lambda m, x: m([x, None], None)
+            self.run_pipe = lambda m, x, nxt, par: m.forward_pipelined([x, None], [nxt, None], par)
+            self.run_planned = lambda m, x, par: m.forward_planned([x, None], par)
+            self.run_plan = lambda m, x, par: m.plan_ahead([x, None], par)
             self.out_of = lambda r: r[0][0]
             self.refresh_net = lambda m, x: m.forward_refresh_reservoirs(x, None)
             self.refresh_out = lambda r: r[0]
@@ -312,28 +322,67 @@ class NetBench:
         self.static_in.copy_(self.deltas[i % self.n_inputs])
         return self.run_net(m, self.static_in)
 
-    def _replay(self, graphs, i):
-        if len(graphs) == 1:
-            self.static_in.copy_(self.deltas[i % self.n_inputs])
-            graphs[0].replay()
-        else:
-            graphs[i % self.n_inputs].replay()
+    def plan_ahead_mode(self):
+        a = self.args
+        return None if (a.plan_ahead == "off" or a.copy_input) else a.plan_ahead
 
-    def timed_run(self, m, tag, steps=None, repeats=None, check_against=None, graph=None):
-        """Refresh, warm up, capture one step in a HIP graph, then time `steps` steps `repeats` times.
+    def timed_run(self, m, tag, steps=None, repeats=None, check_against=None, graph=None, plan_ahead="default"):
+        """Refresh, warm up, capture one step per resident input in a HIP graph, then time `steps` steps `repeats`
+        times.  The inputs are taken cyclically by one running step counter.  plan_ahead "fork": the graph of
+        input i holds step i and, forked beside it, the plan of input i + 1's tile sets (forward_pipelined);
+        "streams": the two halves are graphs of their own, replayed on two streams with events between them
+        (forward_planned / plan_ahead); None: every step plans its own tile sets first (forward).
         Returns (median seconds per step, list of the repeats' ms/step, output-check dict)."""
         torch, args = self.torch, self.args
         steps = args.steps if steps is None else steps
         repeats = args.repeats if repeats is None else repeats
         use_graph = (not args.no_graph) if graph is None else graph
+        pipe = self.plan_ahead_mode() if plan_ahead == "default" else plan_ahead
+        n_in = self.n_inputs
+        assert n_in % 2 == 0
         history, check = [], {}
+        k = 0                                                # running step counter: input k % n_in
+        plan_stream = torch.cuda.Stream() if pipe == "streams" else None
+        planned = [torch.cuda.Event(), torch.cuda.Event()]   # by parity: the tile sets of the step of that parity are built
+        computed = [torch.cuda.Event(), torch.cuda.Event()]  # by parity: the step of that parity has run
+
+        def two_streams(i, compute, plan):
+            """Step i on the current stream; beside it, on the planning stream, the plan of step i + 1 -- which
+            overwrites what step i - 1 read, so it waits for that step's event."""
+            cur, p = torch.cuda.current_stream(), i % 2
+            cur.wait_event(planned[p])
+            out = compute(i)
+            computed[p].record(cur)
+            with torch.cuda.stream(plan_stream):
+                plan_stream.wait_event(computed[1 - p])
+                plan((i + 1) % n_in)
+                planned[1 - p].record(plan_stream)
+            return out
+
+        def eager(kk):
+            i = kk % n_in
+            if pipe == "fork":
+                return self.run_pipe(m, self.deltas[i], self.deltas[(i + 1) % n_in], i % 2)
+            if pipe == "streams":
+                return two_streams(i, lambda j: self.run_planned(m, self.deltas[j], j % 2),
+                                   lambda j: self.run_plan(m, self.deltas[j], j % 2))
+            self.static_in.copy_(self.deltas[i])
+            return self.run_net(m, self.static_in)
+
+        def capture(fn):
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                r = fn()
+            return g, r
         with torch.no_grad():
             self.refresh_net(m, self.cl(self.x0))
-            for i in range(max(args.warmup, 3)):           # also allocates every persistent buffer
-                self.step_eager(m, i)
-                history.append(i)
+            warm = -(-max(args.warmup, 3) // n_in) * n_in    # whole cycles; also allocates every persistent buffer
+            for _ in range(warm):
+                eager(k)
+                history.append(k % n_in)
+                k += 1
             torch.cuda.synchronize()
-            graphs = graph_out = None
+            replay = graph_outs = None
             if use_graph:
                 # One captured graph per resident input: a step then reads its delta where it lies, as it would from the
                 # buffer an event front end writes, and no copy into a fixed input buffer is timed (--copy-input: one
@@ -341,47 +390,71 @@ class NetBench:
                 side = torch.cuda.Stream()
                 side.wait_stream(torch.cuda.current_stream())
                 with torch.cuda.stream(side):
-                    self.step_eager(m, 0)
-                history.append(0)
+                    for _ in range(n_in):
+                        eager(k)
+                        history.append(k % n_in)
+                        k += 1
                 torch.cuda.current_stream().wait_stream(side)
                 torch.cuda.synchronize()
-                graphs = []
-                for src in ([self.static_in] if args.copy_input else self.deltas):
-                    g = torch.cuda.CUDAGraph()
-                    with torch.cuda.graph(g):
-                        graph_out = self.out_of(self.run_net(m, src))
+                graphs, graph_outs = [], []
+                if pipe == "streams":
+                    plans = [None] * n_in
+                    for i in range(n_in):                   # in the order of the steps: the networks check it
+                        g, r = capture(lambda: self.run_planned(m, self.deltas[i], i % 2))
+                        graphs.append(g)
+                        graph_outs.append(self.out_of(r))
+                        j = (i + 1) % n_in
+                        plans[j], _ = capture(lambda: self.run_plan(m, self.deltas[j], j % 2))
+                    replay = lambda kk: two_streams(kk % n_in, lambda i: graphs[i].replay(), lambda j: plans[j].replay())
+                elif pipe == "fork":
+                    for i in range(n_in):
+                        g, r = capture(lambda: self.run_pipe(m, self.deltas[i], self.deltas[(i + 1) % n_in], i % 2))
+                        graphs.append(g)
+                        graph_outs.append(self.out_of(r))
+                    replay = lambda kk: graphs[kk % n_in].replay()
+                elif args.copy_input:
+                    g, r = capture(lambda: self.run_net(m, self.static_in))
                     graphs.append(g)
-                for i in range(3):
-                    self._replay(graphs, i)
-                    history.append(i)
+                    graph_outs.append(self.out_of(r))
+
+                    def replay(kk):
+                        self.static_in.copy_(self.deltas[kk % n_in])
+                        graphs[0].replay()
+                else:
+                    for i in range(n_in):
+                        g, r = capture(lambda: self.run_net(m, self.deltas[i]))
+                        graphs.append(g)
+                        graph_outs.append(self.out_of(r))
+                    replay = lambda kk: graphs[kk % n_in].replay()
+                for _ in range(n_in):
+                    replay(k)
+                    history.append(k % n_in)
+                    k += 1
+            step = replay if replay is not None else eager
             per_repeat = []
             for _ in range(repeats):
                 torch.cuda.synchronize()
                 t0 = time.perf_counter()
-                for i in range(steps):
-                    if graphs is not None:
-                        self._replay(graphs, i)
-                    else:
-                        self.step_eager(m, i)
+                for _ in range(steps):
+                    step(k)
+                    k += 1
                 torch.cuda.synchronize()
                 per_repeat.append((time.perf_counter() - t0) / steps)
-                history.extend(range(steps))
+                history.extend((k - steps + j) % n_in for j in range(steps))
             if check_against is not None:
-                # The timed configuration (graph replay, planning stream) against the plain one: a second
+                # The timed configuration (graph replay, planning ahead) against the plain one: a second
                 # instance of the network with eager launches and inline mask planning takes the same
                 # steps; the next frames of the two must then agree (same kernels over the same tiles).
                 ref = check_against()
                 self.refresh_net(ref, self.cl(self.x0))
                 for i in history:
-                    self.run_net(ref, self.deltas[i % self.n_inputs])
+                    self.run_net(ref, self.deltas[i])
                 worst = 0.0
-                for i in range(4):
-                    want = self.out_of(self.run_net(ref, self.deltas[i % self.n_inputs]))
-                    if graphs is not None:
-                        self._replay(graphs, i)
-                        got = graph_out
-                    else:
-                        got = self.out_of(self.step_eager(m, i))
+                for _ in range(4):
+                    want = self.out_of(self.run_net(ref, self.deltas[k % n_in]))
+                    got = step(k)
+                    got = graph_outs[k % len(graph_outs)] if replay is not None else self.out_of(got)
+                    k += 1
                     worst = max(worst, (got.float() - want.float()).abs().max().item())
                 torch.cuda.synchronize()
                 check.update(max_abs_diff=worst, frames=4, steps_before=len(history),
@@ -844,7 +917,10 @@ def main():
                    "timing": "median of %d repeats of %d steps" % (args.repeats, args.steps),
                    "f32_matmul": ops.f32_matmul if args.dtype == "f32" else None,
                    "arithmetic": ARITHMETIC["bf16" if args.dtype == "bf16" else ops.f32_matmul],
-                   "mask_planning": "inline" if args.sync_masks else ("second stream, builds first" if args.plan_first else "second stream")},
+                   "mask_planning": {"streams": "one step ahead: plan and compute halves are graphs of their own on two streams, events between the replays",
+                                     "fork": "one step ahead: the next step's plan forked inside this step's graph",
+                                     None: ("inline" if args.sync_masks else ("second stream, builds first" if args.plan_first else "second stream"))
+                                     }[nb.plan_ahead_mode()]},
         "roofline": roofline,
         "cpu_baseline": cpu,
         "repeats_ms_per_step": repeats_ms,

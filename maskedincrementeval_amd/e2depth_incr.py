@@ -793,6 +793,42 @@ class E2VIDRecurrentIncr(nn.Module, _IncrBuffers):
                 img_pred, states = self.unetrecurrent.forward([delta, mask], prev_states)
         return img_pred, states
 
+    def _lookahead_parts(self, delta):
+        n, _, h, w = delta.shape
+
+        def make_mask(d):
+            return self.input_mask(d) if self.derive_input_mask else None
+
+        def mask_buffer(d):
+            return self._pix_buf("input", n, h, w, d.device) if self.derive_input_mask else None
+        return (self.__dict__.setdefault("_pipe", {}), make_mask, mask_buffer,
+                lambda d, m: self.unetrecurrent.forward([d, m], None))
+
+    def forward_pipelined(self, event_tensor: Masked, next_event_tensor: Masked, parity: int):
+        """forward(event_tensor, None) with the tile sets of the NEXT step -- whose delta, next_event_tensor, must
+        already hold its values -- planned on a second stream while this step computes (ops.pipelined_step: the
+        plan, 7 % of a 264x352 step, leaves the critical path).  parity alternates 0 / 1 from call to call; the
+        next call must be for the delta announced here.  None as next_event_tensor: no look-ahead (last step).
+        Exact masks only (no delta quantiser, no thresholds), previous states None."""
+        delta = ops.as_nhwc(event_tensor[0])
+        nxt = None if next_event_tensor is None else ops.as_nhwc(next_event_tensor[0])
+        state, make_mask, mask_buffer, walk = self._lookahead_parts(delta)
+        return ops.pipelined_step(state, parity, delta, nxt, make_mask, mask_buffer, walk)
+
+    def plan_ahead(self, event_tensor: Masked, parity: int) -> None:
+        """The planning half of forward_pipelined, on the current stream: input mask and every tile set of the step
+        that will take event_tensor with this parity (ops.plan_step_ahead has the ordering the caller owes)."""
+        delta = ops.as_nhwc(event_tensor[0])
+        state, make_mask, _, walk = self._lookahead_parts(delta)
+        ops.plan_step_ahead(state, parity, delta, make_mask, walk)
+
+    def forward_planned(self, event_tensor: Masked, parity: int):
+        """The compute half: forward(event_tensor, None) over the tile sets plan_ahead built for this parity."""
+        delta = ops.as_nhwc(event_tensor[0])
+        state, make_mask, mask_buffer, walk = self._lookahead_parts(delta)
+        return ops.run_planned_step(state, parity, delta, make_mask, mask_buffer, walk)
+
     def forward_refresh_reservoirs(self, event_tensor: DenseT, prev_states):
+        ops.drop_lookahead(self)
         img_pred, states = self.unetrecurrent.forward_refresh_reservoirs(event_tensor, prev_states)
         return img_pred, states

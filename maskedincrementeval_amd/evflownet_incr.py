@@ -642,7 +642,42 @@ class MultiResUNetRecurrentIncr(nn.Module, _IncrBuffers):
             predictions.append(pred(x_incr))
         return predictions
 
+    def _lookahead_parts(self, delta):
+        n, _, h, w = delta.shape
+
+        def make_mask(d):
+            if not self.derive_input_mask:
+                return None
+            return ops.mask_from_delta(d, self.mask_threshold, self._pix_buf("input", n, h, w, d.device))
+
+        def mask_buffer(d):
+            return self._pix_buf("input", n, h, w, d.device) if self.derive_input_mask else None
+        return self.__dict__.setdefault("_pipe", {}), make_mask, mask_buffer, self._forward
+
+    def forward_pipelined(self, x_incr, next_x_incr, parity: int):
+        """forward(x_incr) with the tile sets of the NEXT step -- whose delta, next_x_incr[0], must already hold its
+        values -- planned on a second stream while this step computes (ops.pipelined_step).  parity alternates
+        0 / 1 from call to call; the next call must be for the delta announced here; None: no look-ahead."""
+        delta = ops.as_nhwc(x_incr[0])
+        nxt = None if next_x_incr is None else ops.as_nhwc(next_x_incr[0])
+        state, make_mask, mask_buffer, walk = self._lookahead_parts(delta)
+        return ops.pipelined_step(state, parity, delta, nxt, make_mask, mask_buffer, walk)
+
+    def plan_ahead(self, x_incr, parity: int) -> None:
+        """The planning half of forward_pipelined, on the current stream: input mask and every tile set of the step
+        that will take x_incr with this parity (ops.plan_step_ahead has the ordering the caller owes)."""
+        delta = ops.as_nhwc(x_incr[0])
+        state, make_mask, _, walk = self._lookahead_parts(delta)
+        ops.plan_step_ahead(state, parity, delta, make_mask, walk)
+
+    def forward_planned(self, x_incr, parity: int):
+        """The compute half: forward(x_incr) over the tile sets plan_ahead built for this parity."""
+        delta = ops.as_nhwc(x_incr[0])
+        state, make_mask, mask_buffer, walk = self._lookahead_parts(delta)
+        return ops.run_planned_step(state, parity, delta, make_mask, mask_buffer, walk)
+
     def forward_refresh_reservoirs(self, x):
+        ops.drop_lookahead(self)
         self._reset_incr()
         blocks = []
         for i, encoder in enumerate(self.encoders):

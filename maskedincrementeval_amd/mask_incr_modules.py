@@ -30,7 +30,9 @@ class _IncrBuffers:
 
     Deltas written by the kernels live in fixed buffers (stable pointers, zero
     outside the active tiles); `_reset_incr` returns them to the all-zero state
-    a dense refresh implies.
+    a dense refresh implies.  Delta buffers, tile sets and pixel masks exist once per
+    `ops.buffer_parity` (0 unless a network is run with its next step planned ahead,
+    ops.pipelined_step).
     """
 
     def _ib(self):
@@ -41,7 +43,7 @@ class _IncrBuffers:
         return d
 
     def _delta_buf(self, name, shape, device, dtype=torch.float32) -> torch.Tensor:
-        key = ("d", name, tuple(shape), str(device), dtype)
+        key = ("d", name, tuple(shape), str(device), dtype, ops.buffer_parity)
         b = self._ib().get(key)
         if b is None:
             b = ops.new_nhwc(*shape, device, dtype)
@@ -49,7 +51,7 @@ class _IncrBuffers:
         return b
 
     def _tile_set(self, name, n, h, w, device) -> TileMask:
-        key = ("t", name, (n, h, w), str(device))
+        key = ("t", name, (n, h, w), str(device), ops.buffer_parity)
         b = self._ib().get(key)
         if b is None:
             b = TileMask(n, h, w, device)
@@ -57,7 +59,7 @@ class _IncrBuffers:
         return b
 
     def _pix_buf(self, name, n, h, w, device) -> torch.Tensor:
-        key = ("p", name, (n, h, w), str(device))
+        key = ("p", name, (n, h, w), str(device), ops.buffer_parity)
         b = self._ib().get(key)
         if b is None:
             b = torch.zeros((n, 1, h, w), dtype=torch.uint8, device=device)

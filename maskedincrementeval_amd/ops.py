@@ -153,6 +153,130 @@ def _launch_plan(batch):
             root.ready = ev
 
 
+# ---- planning one step ahead ---------------------------------------------------------------------
+# The tile sets of a step depend on that step's input mask alone, so where the next input is already there (a
+# recorded sequence, a batch job, a front end that runs ahead) they can be built while the CURRENT step computes: the
+# plan then leaves the critical path altogether.  Two generations of every tile set, pixel mask and delta buffer
+# exist for that (`buffer_parity` is part of their keys in _IncrBuffers): the step of parity p reads the sets of
+# parity p while the plan of the next step writes those of parity 1 - p.  Reservoirs are shared.  A delta buffer of
+# parity p is next written two steps later, under a tile set whose previous build was the one it was last written
+# under -- so stale lists stay right -- PROVIDED every plan is followed by its step: a set built twice with no
+# compute pass between the builds forgets which tiles still hold data.  run_planned_step therefore refuses a delta that
+# is not the one the plan of its parity was made for (same pointer and shape), and plan_step_ahead refuses sets whose
+# last plan was never run.  (Under graph capture these checks see the capture order only: replay the captured steps in the
+# cyclic order they were captured in.)
+buffer_parity = 0
+_lookahead_streams = {}
+
+
+def _delta_key(t):
+    return (t.data_ptr(), tuple(t.shape), t.dtype)
+
+
+def _check_lookahead_context(parity):
+    if _phase is not None or _planner is not None:
+        raise RuntimeError("planning one step ahead: not inside a planning pass or a mask_planner block")
+    if parity not in (0, 1):
+        raise ValueError("parity must be 0 or 1")
+
+
+def plan_step_ahead(state: dict, parity: int, delta: torch.Tensor, make_mask, walk):
+    """Build, on the CURRENT stream, the input mask and every tile set of the step that will run `delta` with
+    `parity`.  It writes the buffers of that parity only, so it may run beside the step before it (other parity) --
+    but not before the step two back (same parity) has finished, and the step it plans must wait for it: the caller
+    orders that with events (pipelined_step does, with a fork and a join; with two streams of one's own, the planning
+    stream waits for the event recorded after step k - 1 before planning step k + 1, and the compute stream waits for
+    the event recorded after that plan before step k + 1).
+    state: a dict the caller keeps per network instance; make_mask(delta) -> the input pixel mask (or None: every
+    pixel), written into the parity's buffer; walk(delta, mask) -> one walk of the network."""
+    global buffer_parity
+    _check_lookahead_context(parity)
+    pending = state.setdefault("planned", {})
+    if pending.get(parity) is not None:
+        raise RuntimeError("planning one step ahead: the step planned for parity %d was never run" % parity)
+    try:
+        buffer_parity = parity
+        mask = make_mask(delta)
+        with network_pass("plan"):
+            walk(delta, mask)
+        pending[parity] = _delta_key(delta)
+    finally:
+        buffer_parity = 0
+
+
+def run_planned_step(state: dict, parity: int, delta: torch.Tensor, make_mask, mask_buffer, walk):
+    """The compute pass of the step plan_step_ahead planned for (parity, delta), on the current stream.  If nothing was
+    planned for this parity (the first step of a sequence) the plan is made here first.  A plan for another delta
+    (other pointer or shape) than the one passed is refused.  mask_buffer(delta) -> the parity's input-mask buffer
+    without recomputing it."""
+    global buffer_parity
+    _check_lookahead_context(parity)
+    pending = state.setdefault("planned", {})
+    try:
+        buffer_parity = parity
+        if pending.get(parity) == _delta_key(delta):
+            mask = mask_buffer(delta)
+        elif pending.get(parity) is None:
+            mask = make_mask(delta)
+            with network_pass("plan"):
+                walk(delta, mask)
+        else:
+            raise RuntimeError("planning one step ahead: the tile sets of parity %d were planned for another delta than "
+                               "the one passed now; run the step that was announced as next" % parity)
+        pending[parity] = None
+        with network_pass("compute"):
+            return walk(delta, mask)
+    finally:
+        buffer_parity = 0
+
+
+def pipelined_step(state: dict, parity: int, delta: torch.Tensor, next_delta: Optional[torch.Tensor],
+                   make_mask, mask_buffer, walk):
+    """run_planned_step(parity, delta) with plan_step_ahead(1 - parity, next_delta) forked onto a second stream beside
+    it and joined behind it -- one call, and one graph if captured.  (In a captured graph the fork and the join are
+    edges between streams, and on this hardware they cost about half of what the overlap gains; two graphs on two
+    streams of the caller's, ordered by events between the replays, keep all of it.)"""
+    _check_lookahead_context(parity)
+    dev = delta.device
+    cur = torch.cuda.current_stream(dev)
+    pending = state.setdefault("planned", {})
+    fork = None
+    if next_delta is not None:
+        if pending.get(1 - parity) is not None:
+            raise RuntimeError("planning one step ahead: the step planned for parity %d was never run" % (1 - parity))
+        if pending.get(parity) not in (None, _delta_key(delta)):
+            raise RuntimeError("planning one step ahead: the tile sets of parity %d were planned for another delta than "
+                               "the one passed now; run the step that was announced as next" % parity)
+        fork = torch.cuda.Event()
+        fork.record(cur)
+    # this step's kernels are enqueued first: the look-ahead depends on none of them
+    out = run_planned_step(state, parity, delta, make_mask, mask_buffer, walk)
+    if fork is not None:
+        side = _lookahead_streams.get(dev)
+        if side is None:
+            side = _lookahead_streams[dev] = torch.cuda.Stream(dev)
+        side.wait_event(fork)                          # fork (joins a graph capture, too)
+        with torch.cuda.stream(side):
+            plan_step_ahead(state, 1 - parity, next_delta, make_mask, walk)
+        ev = torch.cuda.Event()
+        ev.record(side)
+        cur.wait_event(ev)                             # join
+    return out
+
+
+def drop_lookahead(net):
+    """Called by a network's dense refresh: the sequence starts anew.  If a step was planned ahead and never run, its
+    tile sets were built without a compute pass behind them, and the next build would no longer know which tiles of
+    their delta buffers hold data: every incremental buffer of the network is then put back to the all-zero state
+    (pass None as the next delta of the last step before a refresh and nothing has to be zeroed)."""
+    state = net.__dict__.pop("_pipe", None)
+    if state and any(v is not None for v in state.get("planned", {}).values()):
+        for m in net.modules():
+            zero = getattr(m, "_zero_incr", None)
+            if zero is not None:
+                zero()
+
+
 def _stream(t: torch.Tensor):
     return torch.cuda.current_stream(t.device).cuda_stream
 

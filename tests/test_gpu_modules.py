@@ -594,3 +594,132 @@ def test_value_dependent_masks_replay_from_a_graph(knob):
         # the masks did depend on the values: the thresholded network runs fewer tiles than the plane holds
         cap = max(b.capacity for k_, b in last(captured)._ib().items() if k_[0] == "t")
         assert min(max(t) for t in got_tiles) < cap
+
+
+@pytest.mark.parametrize("net", ["e2depth", "evflownet_transposed", "evflownet_upsample"])
+def test_planning_one_step_ahead_reproduces_plain_steps(net):
+    # forward_pipelined: the tile sets of step t + 1 are planned on a second stream while step t computes, in a second
+    # generation of every tile set / delta buffer (ops.pipelined_step).  Against the same network stepped plainly, bit
+    # for bit: 7 eager steps with fresh masks (stale tiles in both generations), a dense refresh with a plan still
+    # pending (buffers are zeroed), then four resident inputs captured as four graphs -- each holds its step and the
+    # plan of the next input -- and replayed cyclically for three rounds, with the program's own work in between.
+    from maskedincrementeval_amd.evflownet_incr import MultiResUNetRecurrentIncr
+    from maskedincrementeval_amd.synthetic import MovingEdges
+    if net == "e2depth":
+        h, w, c = 72, 104, 5
+        make = lambda: seed_module_(E2VIDRecurrentIncr(), seed=31).to(DEV).eval()
+        plain = lambda m, d: m([d, None], None)[0][0]
+        piped = lambda m, d, nx, p: m.forward_pipelined([d, None], None if nx is None else [nx, None], p)[0][0]
+        refresh = lambda m, x: m.forward_refresh_reservoirs(x, None)
+        deltas = [_cl(event_voxel_delta(1, c, h, w, 0.02 + 0.03 * (i % 3), seed=5300 + i)[0]) for i in range(12)]
+    else:
+        h, w, c = 64, 96, 4
+        kind = net.split("_")[1]
+        make = lambda: seed_module_(MultiResUNetRecurrentIncr(num_bins=c, decoder=kind), seed=41).to(DEV).eval()
+        plain = lambda m, d: m([d, None])[-1][0]
+        piped = lambda m, d, nx, p: m.forward_pipelined([d, None], None if nx is None else [nx, None], p)[-1][0]
+        refresh = lambda m, x: m.forward_refresh_reservoirs(x)
+        gen = MovingEdges(h, w, seed=7)
+        deltas = [_cl(gen.step()[0]) for _ in range(12)]
+    a, b = make(), make()
+    x0 = _cl(torch.randn(1, c, h, w, generator=torch.Generator().manual_seed(33)) * 0.5)
+    with torch.no_grad():
+        refresh(a, x0), refresh(b, x0)
+        for i in range(7):
+            want = plain(a, deltas[i]).clone()
+            got = piped(b, deltas[i], deltas[i + 1], i % 2).clone()     # (after step 6 the plan of deltas[7] stays pending)
+            assert torch.equal(got, want), "eager step %d: %.3e" % (i, (got - want).abs().max().item())
+        # a step that is not the one announced is refused, loudly
+        with pytest.raises(RuntimeError, match="announced as next"):
+            piped(b, deltas[9], None, 1)
+        refresh(a, x0), refresh(b, x0)
+        res = deltas[8:12]
+        for i in range(4):                                              # eager round: allocates nothing new, primes the cycle
+            want = plain(a, res[i]).clone()
+            got = piped(b, res[i], res[(i + 1) % 4], i % 2).clone()
+            assert torch.equal(got, want), "round 0 step %d" % i
+        torch.cuda.synchronize()
+        graphs, outs = [], []
+        for i in range(4):
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                outs.append(piped(b, res[i], res[(i + 1) % 4], i % 2))
+            graphs.append(g)
+        for rnd in range(3):
+            for i in range(4):
+                want = plain(a, res[i]).clone()
+                graphs[i].replay()
+                got = outs[i].clone()
+                assert torch.equal(got, want), "replay round %d step %d: %.3e" % (rnd, i, (got - want).abs().max().item())
+    torch.cuda.synchronize()
+    assert ops.buffer_parity == 0 and ops._phase is None
+
+
+@pytest.mark.parametrize("net", ["e2depth", "evflownet_transposed"])
+def test_plan_and_compute_halves_on_two_streams_reproduce_plain_steps(net):
+    # plan_ahead / forward_planned: the two halves of forward_pipelined with the caller's own streams and events.  The
+    # planning stream waits for the event recorded after step k - 1 before it plans step k + 1 (same buffers as
+    # step k - 1), the compute stream waits for the event recorded after that plan.  Eager for a round, then each half
+    # captured as a graph of its own (no edge between streams inside any graph) and replayed for three rounds.
+    from maskedincrementeval_amd.evflownet_incr import MultiResUNetRecurrentIncr
+    from maskedincrementeval_amd.synthetic import MovingEdges
+    if net == "e2depth":
+        h, w, c = 72, 104, 5
+        make = lambda: seed_module_(E2VIDRecurrentIncr(), seed=31).to(DEV).eval()
+        plain = lambda m, d: m([d, None], None)[0][0]
+        out_of = lambda r: r[0][0]
+        refresh = lambda m, x: m.forward_refresh_reservoirs(x, None)
+        res = [_cl(event_voxel_delta(1, c, h, w, 0.02 + 0.03 * (i % 3), seed=5400 + i)[0]) for i in range(4)]
+    else:
+        h, w, c = 64, 96, 4
+        make = lambda: seed_module_(MultiResUNetRecurrentIncr(num_bins=c, decoder="transposed"), seed=41).to(DEV).eval()
+        plain = lambda m, d: m([d, None])[-1][0]
+        out_of = lambda r: r[-1][0]
+        refresh = lambda m, x: m.forward_refresh_reservoirs(x)
+        gen = MovingEdges(h, w, seed=9)
+        res = [_cl(gen.step()[0]) for _ in range(4)]
+    a, b = make(), make()
+    x0 = _cl(torch.randn(1, c, h, w, generator=torch.Generator().manual_seed(35)) * 0.5)
+    cur, side = torch.cuda.current_stream(), torch.cuda.Stream()
+    planned = [torch.cuda.Event(), torch.cuda.Event()]        # by parity: the plan of the step of that parity is made
+    computed = [torch.cuda.Event(), torch.cuda.Event()]       # by parity: the step of that parity has run
+
+    def step(i, compute, plan):
+        p = i % 2
+        cur.wait_event(planned[p])
+        out = compute(i)
+        computed[p].record(cur)
+        with torch.cuda.stream(side):
+            side.wait_event(computed[1 - p])                  # step i - 1 read the buffers this plan overwrites
+            plan((i + 1) % 4)
+            planned[1 - p].record(side)
+        return out
+
+    with torch.no_grad():
+        refresh(a, x0), refresh(b, x0)
+        torch.cuda.synchronize()
+        for rnd in range(2):
+            for i in range(4):
+                want = plain(a, res[i]).clone()
+                got = out_of(step(i, lambda j: b.forward_planned([res[j], None], j % 2),
+                                  lambda j: b.plan_ahead([res[j], None], j % 2))).clone()
+                assert torch.equal(got, want), "eager round %d step %d: %.3e" % (rnd, i, (got - want).abs().max().item())
+        torch.cuda.synchronize()
+        g_comp, g_plan, outs = [], [None] * 4, []
+        for i in range(4):                                     # capture order = the order the state checks expect
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                outs.append(out_of(b.forward_planned([res[i], None], i % 2)))
+            g_comp.append(g)
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                b.plan_ahead([res[(i + 1) % 4], None], (i + 1) % 2)
+            g_plan[(i + 1) % 4] = g
+        for rnd in range(3):
+            for i in range(4):
+                want = plain(a, res[i]).clone()
+                step(i, lambda j: g_comp[j].replay(), lambda j: g_plan[j].replay())
+                got = outs[i].clone()
+                assert torch.equal(got, want), "replay round %d step %d: %.3e" % (rnd, i, (got - want).abs().max().item())
+    torch.cuda.synchronize()
+    assert ops.buffer_parity == 0 and ops._phase is None
