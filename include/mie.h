@@ -183,6 +183,17 @@ typedef struct mie_plan_op {
 int mie_build_mask_plan(const mie_plan_op* ops, int n_ops, void* stream);
 
 /*
+ * mie_build_mask_plan with a cap on the workgroups of its first kernel, for a plan that runs BESIDE other kernels --
+ * the next step's tile sets built on a second stream while this step's convs run.  A plan workgroup is 1024 threads
+ * and most of a CU's LDS; at the default (up to 256 workgroups, one round of the chip) it takes the CUs from the
+ * convs it runs beside: at 8x480x640 the first stride-2 encoder went from 43 to 107 us.  With 64 the plan takes
+ * longer, which nothing waits for, and the step of 8 frames 2.20 instead of 2.25 ms.  Same results as
+ * mie_build_mask_plan; max_workgroups > 0 (values above the default cap mean the default).
+ * Replaces: nothing in the reference (see mie_build_mask_plan).
+ */
+int mie_build_mask_plan_wgs(const mie_plan_op* ops, int n_ops, int max_workgroups, void* stream);
+
+/*
  * Re-order a fp32 [cin][k][k][cout] filter into the layout the matrix-core
  * kernels stream, so that the k-steps a lane multiplies per tap come as one
  * 16-byte load:

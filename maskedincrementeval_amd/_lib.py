@@ -37,7 +37,7 @@ EXPORTS = (
     "mie_maxpool_incr", "mie_accumulate", "mie_scale_incr", "mie_avgpool_incr", "mie_linear_incr", "mie_upconv_masked", "mie_upconv_masked_ws", "mie_upconv_pred_masked",
     "mie_conv_masked_ws", "mie_convgru_gates_incr", "mie_upsample2x_pair_incr", "mie_conv_masked_noalloc",
     "mie_convlstm_gates_refresh", "mie_convgru_gates_refresh", "mie_mul_dense", "mie_tconv2x_masked",
-    "mie_tconv2x_refresh", "mie_conv_f32x3_takes", "mie_build_mask_plan",
+    "mie_tconv2x_refresh", "mie_conv_f32x3_takes", "mie_build_mask_plan", "mie_build_mask_plan_wgs",
 )
 PLAN_MAX_STEPS = 40
 
@@ -87,6 +87,8 @@ def _declare(l):
     l.mie_build_mask_tiles.argtypes = [vp, vp, ci, ci, ci, ci, ci, ci, tsp, vp]
     l.mie_build_mask_plan.restype = ci
     l.mie_build_mask_plan.argtypes = [ctypes.POINTER(MiePlanOp), ci, vp]
+    l.mie_build_mask_plan_wgs.restype = ci
+    l.mie_build_mask_plan_wgs.argtypes = [ctypes.POINTER(MiePlanOp), ci, ci, vp]
     l.mie_conv_masked.restype = ci
     l.mie_conv_masked.argtypes = [vp, vp, ci, vp, vp, ci, ci, ci, vp, vp, ci, ci, ci, ci, ci, tsp, vp,
                                   vp, vp, ci, cf, ci, ci, vp]

@@ -932,8 +932,23 @@ int plan_lds_limit(long long need_bytes, const char* who) {
 
 }  // namespace
 
+namespace {
+int build_mask_plan(const char* who, const mie_plan_op* ops, int n_ops, int wg_cap, void* stream);
+}
+
 extern "C" int mie_build_mask_plan(const mie_plan_op* ops, int n_ops, void* stream) {
-  const char* who = "mie_build_mask_plan";
+  return build_mask_plan("mie_build_mask_plan", ops, n_ops, 0, stream);
+}
+
+extern "C" int mie_build_mask_plan_wgs(const mie_plan_op* ops, int n_ops, int max_workgroups, void* stream) {
+  const char* who = "mie_build_mask_plan_wgs";
+  mie_clear_error();
+  MIE_REQUIRE(max_workgroups > 0, MIE_ERR_INVALID_ARG, "%s: max_workgroups %d", who, max_workgroups);
+  return build_mask_plan(who, ops, n_ops, max_workgroups, stream);
+}
+
+namespace {
+int build_mask_plan(const char* who, const mie_plan_op* ops, int n_ops, int wg_cap, void* stream) {
   mie_clear_error();
   MIE_REQUIRE(ops != nullptr && n_ops > 0, MIE_ERR_INVALID_ARG, "%s: no ops", who);
   MIE_REQUIRE(n_ops <= MIE_PLAN_MAX_STEPS, MIE_ERR_CAPACITY, "%s: %d ops, at most %d per call", who, n_ops, MIE_PLAN_MAX_STEPS);
@@ -1165,7 +1180,8 @@ extern "C" int mie_build_mask_plan(const mie_plan_op* ops, int n_ops, void* stre
   // samples there are workgroups enough without many per sample, and more than one per CU would only queue (a
   // workgroup of a large plane takes most of a CU's LDS).
   static const int max_wgs = [] { const char* e = getenv("MIE_PLAN_WGS"); return e ? atoi(e) : 256; }();      // tuning knob
-  if (shares * a.n > max_wgs) shares = max_wgs / a.n > 0 ? max_wgs / a.n : 1;
+  const int wgs = (wg_cap > 0 && wg_cap < max_wgs) ? wg_cap : max_wgs;     // a caller's cap: the plan runs beside other kernels
+  if (shares * a.n > wgs) shares = wgs / a.n > 0 ? wgs / a.n : 1;
   if (shares * PLAN_THREADS < max_tiles) shares = (max_tiles + PLAN_THREADS - 1) / PLAN_THREADS;
   // the flag area of a workgroup: per set, the tiles it owns (every shares-th one)
   for (int i = 0; i < a.n_steps; ++i) {
@@ -1203,3 +1219,4 @@ extern "C" int mie_build_mask_plan(const mie_plan_op* ops, int n_ops, void* stre
   hipLaunchKernelGGL(k_plan_compact, dim3((unsigned)total_chunks), dim3(COMPACT_THREADS), 0, (hipStream_t)stream, c);
   return mie_check_launch(who);
 }
+}  // namespace

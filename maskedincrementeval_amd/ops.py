@@ -110,8 +110,12 @@ def _launch_plan(batch):
         stream = side.cuda_stream
     else:
         stream = torch.cuda.current_stream(dev).cuda_stream
-    sig = tuple(b[:8] + (b[8].pixmask.data_ptr(), b[8].tiles.data_ptr()) for b in batch)
+    sig = tuple(b[:8] + (b[8].pixmask.data_ptr(), b[8].tiles.data_ptr()) for b in batch) + (_plan_wgs,)
     parts = _plan_cache.get(sig)
+    if _plan_wgs:
+        build_plan = lambda arr, n: real.mie_build_mask_plan_wgs(arr, n, _plan_wgs, stream)
+    else:
+        build_plan = lambda arr, n: real.mie_build_mask_plan(arr, n, stream)
 
     def single(b):
         p1, p2, h_in, w_in, foot, k, stride, pad, out = b
@@ -126,7 +130,7 @@ def _launch_plan(batch):
             if lo >= hi:
                 continue
             arr = _plan_ops(batch[lo:hi])
-            rc = real.mie_build_mask_plan(arr, hi - lo, stream)
+            rc = build_plan(arr, hi - lo)
             if rc == 0:
                 parts.append(("plan", arr, hi - lo, lo))
             elif rc == -3 and hi - lo > 1:               # MIE_ERR_CAPACITY: too long or too much LDS -- halve it
@@ -142,7 +146,7 @@ def _launch_plan(batch):
     else:
         for kind, arr, n_ops, lo in parts:
             if kind == "plan":
-                check(real.mie_build_mask_plan(arr, n_ops, stream))
+                check(build_plan(arr, n_ops))
             else:
                 single(batch[lo])
     if side is not None:
@@ -167,6 +171,10 @@ def _launch_plan(batch):
 # cyclic order they were captured in.)
 buffer_parity = 0
 _lookahead_streams = {}
+# A plan made ahead runs beside the convs of the step before it and nothing waits for it: it is held to this many
+# workgroups (mie_build_mask_plan_wgs), so that the chip stays with the convs.  0: the library's own cap.
+LOOKAHEAD_PLAN_WGS = int(os.environ.get("MIE_LOOKAHEAD_PLAN_WGS", "64"))      # tuning knob, read once
+_plan_wgs = 0
 
 
 def _delta_key(t):
@@ -194,14 +202,15 @@ def plan_step_ahead(state: dict, parity: int, delta: torch.Tensor, make_mask, wa
     pending = state.setdefault("planned", {})
     if pending.get(parity) is not None:
         raise RuntimeError("planning one step ahead: the step planned for parity %d was never run" % parity)
+    global _plan_wgs
     try:
-        buffer_parity = parity
+        buffer_parity, _plan_wgs = parity, LOOKAHEAD_PLAN_WGS
         mask = make_mask(delta)
         with network_pass("plan"):
             walk(delta, mask)
         pending[parity] = _delta_key(delta)
     finally:
-        buffer_parity = 0
+        buffer_parity = _plan_wgs = 0
 
 
 def run_planned_step(state: dict, parity: int, delta: torch.Tensor, make_mask, mask_buffer, walk):

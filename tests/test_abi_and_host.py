@@ -163,6 +163,9 @@ def test_mask_plan_rejects_what_it_cannot_run(mie_lib):
     conv = (p, None, 16, 16, _lib.FOOT_CONV, 3, 1, 1, ts)
     assert plan() == -1 and "no ops" in err()
     assert mie_lib.mie_build_mask_plan(None, 3, None) == -1
+    one = (_lib.MiePlanOp * 1)()
+    assert mie_lib.mie_build_mask_plan_wgs(one, 1, 0, None) == -1 and "max_workgroups" in err()
+    assert mie_lib.mie_build_mask_plan_wgs(None, 1, 8, None) == -1 and "no ops" in err()
     assert plan(*([conv] * (_lib.PLAN_MAX_STEPS + 1))) == -3 and "at most" in err()
     assert plan((p, None, 16, 16, _lib.FOOT_CONV, 3, 3, 1, ts)) == -2 and "strides 1 and 2" in err()
     assert plan((p, None, 16, 16, _lib.FOOT_TCONV, 3, 1, 1, ts)) == -2 and "stride 2 only" in err()

@@ -203,8 +203,9 @@ def _plan_inputs(n, h, w, step):
     return {"x": x, "y4": y4}
 
 
-def _run_chain(chain, sets, inputs_dev, n, planned):
-    """Build the chain into `sets` (name -> TileMask): one mie_build_mask_plan call, or one build per set."""
+def _run_chain(chain, sets, inputs_dev, n, planned, wgs=0):
+    """Build the chain into `sets` (name -> TileMask): one mie_build_mask_plan call (wgs > 0: mie_build_mask_plan_wgs
+    with that cap), or one build per set."""
     shape_of = {name: plane for name, _, _, _, _, _, plane in chain}
     batch = []
     for name, ins, foot, k, s, p, (ho, wo) in chain:
@@ -217,7 +218,10 @@ def _run_chain(chain, sets, inputs_dev, n, planned):
     st = torch.cuda.current_stream().cuda_stream
     if planned:
         arr = ops._plan_ops(batch)
-        _lib.check(lib.mie_build_mask_plan(arr, len(batch), st))
+        if wgs:
+            _lib.check(lib.mie_build_mask_plan_wgs(arr, len(batch), wgs, st))
+        else:
+            _lib.check(lib.mie_build_mask_plan(arr, len(batch), st))
     else:
         for p1, p2, hi, wi, foot, k, s, p, out in batch:
             _lib.check(lib.mie_build_mask_tiles(p1, p2, hi, wi, foot, k, s, p, out.ref, st))
@@ -262,6 +266,31 @@ def test_mask_plan_equals_the_builds_it_replaces(n, h, w):
                 m = mo.footprint_tconv(src, k, s, p, ho, wo)
             want[name] = m
             prev[name] = _check_tileset(b, m, prev.get(name))
+
+
+@pytest.mark.parametrize("n,h,w,wgs", [(1, 264, 352, 1), (1, 264, 352, 3), (4, 240, 320, 4), (4, 240, 320, 9),
+                                       (3, 37, 53, 64), (2, 128, 160, 100000)])
+def test_mask_plan_held_to_few_workgroups_builds_the_same_sets(n, h, w, wgs):
+    # mie_build_mask_plan_wgs: the plan that runs beside other kernels, its first kernel capped at `wgs` workgroups --
+    # one per sample, fewer than samples (the cap is then one per sample), an odd share count, and a cap above the
+    # default.  Three steps with fresh masks; every buffer of every set bit-equal to the uncapped plan's.
+    chain = _plan_chain(n, h, w)
+    mk = lambda: {name: TileMask(n, plane[0], plane[1], DEV) for name, _, _, _, _, _, plane in chain}
+    full, capped = mk(), mk()
+    for step in range(3):
+        dev = {k_: _to_dev_mask(v) for k_, v in _plan_inputs(n, h, w, step).items()}
+        _run_chain(chain, full, dev, n, planned=True)
+        _run_chain(chain, capped, dev, n, planned=True, wgs=wgs)
+        torch.cuda.synchronize()
+        for name, *_ in chain:
+            a, b = full[name], capped[name]
+            na, ns = int(a.counts[0].item()), int(a.counts[1].item())
+            tag = "step %d set %s" % (step, name)
+            assert torch.equal(a.pixmask, b.pixmask), tag + ": pixel mask"
+            assert torch.equal(a.counts, b.counts), tag + ": counts"
+            assert torch.equal(a.flags, b.flags), tag + ": flags"
+            assert torch.equal(a.tiles[:na], b.tiles[:na]), tag + ": active list"
+            assert torch.equal(a.stale[:ns], b.stale[:ns]), tag + ": stale list"
 
 
 def test_mask_plan_of_a_large_plane_and_many_samples():
