@@ -147,6 +147,8 @@ int mie_mask_from_delta(const void* delta, int n, int h, int w, int c,
  * footprint (MIE_FOOT_CONV, k = 1, stride = 1, pad = 0); any other footprint
  * reads neighbouring bytes while they are written and is refused with
  * MIE_ERR_INVALID_ARG.
+ * Sets of 33 to 4096 tiles are built in one launch: the workgroup that finishes last (a ticket in
+ * out->counts[MIE_CNT_TICKET], zero between calls) ranks the lists.
  * Replaces: the mask argument of conv{1,3,5,7}x*_increment_ext
  * (ext/pointops/_C_ext/pointops/ops.cpp:27-48), which the reference kernel
  * never reads (ext_conv.cu:74-76 synthesises a fake one).
@@ -154,6 +156,23 @@ int mie_mask_from_delta(const void* delta, int n, int h, int w, int c,
 int mie_build_mask_tiles(const uint8_t* in_mask, const uint8_t* in_mask2,
                          int h_in, int w_in, int foot, int k, int stride,
                          int pad, const mie_tileset* out, void* stream);
+
+/*
+ * mie_mask_from_delta(delta -> thr_mask) followed by mie_build_mask_tiles(thr_mask, in_mask2, conv footprint k /
+ * stride / pad -> out) as ONE launch (two above 4096 tiles), for networks whose masks depend on values: a conv with
+ * a thresholded input mask otherwise pays three or four launches of 4-14 us each before it can start.  delta is
+ * [out->n, h_in, w_in, c] of `dtype` (MIE_DTYPE_F32 / MIE_DTYPE_BF16), 16-byte aligned; thr_mask [out->n, h_in, w_in]
+ * receives the thresholded input mask (a pixel is active when |delta| > threshold in any channel), which the conv
+ * takes as its input pixel mask; in_mask2 (may be NULL) is OR-ed in before the footprint, as in
+ * mie_build_mask_tiles.  Results are bit-equal to the two calls.  Limits: stride + pad <= k and
+ * 7 * stride + k <= 24 (MIE_ERR_UNSUPPORTED otherwise: use the two calls); thr_mask, in_mask2 and out->pixmask are
+ * three distinct buffers.  Uses out->counts[MIE_CNT_TICKET], which is zero between calls.
+ * Replaces: the mask a thresholded module derives from its input, maxpool(abs(x)) >= thr with field 1
+ * (incr_modules/utils.py:22-25), chained with the footprint of the conv that reads it.
+ */
+int mie_build_mask_tiles_thresholded(const void* delta, int c, int dtype, float threshold, uint8_t* thr_mask,
+                                     const uint8_t* in_mask2, int h_in, int w_in, int k, int stride, int pad,
+                                     const mie_tileset* out, void* stream);
 
 /*
  * A sequence of mie_build_mask_tiles calls as one launch: the tile sets of a whole network, whose structural

@@ -30,7 +30,7 @@ CNT_ACTIVE, CNT_STALE, CNT_TICKET, CNT_WORDS = 0, 1, 2, 4
 
 # every symbol include/mie.h declares
 EXPORTS = (
-    "mie_version", "mie_last_error_string", "mie_tile_capacity", "mie_mask_from_delta",
+    "mie_version", "mie_last_error_string", "mie_tile_capacity", "mie_mask_from_delta", "mie_build_mask_tiles_thresholded",
     "mie_build_mask_tiles", "mie_conv_masked", "mie_act_incr", "mie_mul_incr", "mie_add_incr",
     "mie_upsample2x_incr", "mie_convlstm_gates_incr", "mie_tconv_masked", "mie_conv_refresh",
     "mie_pack_filter", "mie_kfence_incr", "mie_events_to_frame", "mie_events_to_frame_bf16", "mie_tconv_refresh", "mie_conv_gates_masked", "mie_conv_gates_masked_ws",
@@ -83,6 +83,8 @@ def _declare(l):
     l.mie_tile_capacity.argtypes = [ci, ci, ci]
     l.mie_mask_from_delta.restype = ci
     l.mie_mask_from_delta.argtypes = [vp, ci, ci, ci, ci, cf, vp, ci, vp]
+    l.mie_build_mask_tiles_thresholded.restype = ci
+    l.mie_build_mask_tiles_thresholded.argtypes = [vp, ci, ci, cf, vp, vp, ci, ci, ci, ci, ci, tsp, vp]
     l.mie_build_mask_tiles.restype = ci
     l.mie_build_mask_tiles.argtypes = [vp, vp, ci, ci, ci, ci, ci, ci, tsp, vp]
     l.mie_build_mask_plan.restype = ci

@@ -334,6 +334,207 @@ __global__ __launch_bounds__(COMPACT_THREADS) void k_build_small(BuildArgs a) {
   compact_lists(a, [&](int t) { return s_flag[t]; }, 0, 0, 0, true, s_tot);
 }
 
+// ---- one launch for planes of up to TICKET_CAP tiles ----------------------------------------------
+// The footprint kernel's workgroups take a ticket from counts[MIE_CNT_TICKET] when their flags are written; the one
+// that draws the last ticket puts the counter back to zero and ranks the two lists from the flags of all of them.
+// Nobody waits for anybody: every other workgroup has left by then.  The lists are what k_compact_tiles writes.
+// Flags are stored and, by the last workgroup, loaded as device-scope atomics, which go through to the level the
+// XCDs share; a workgroup waits for its flag stores to complete before it draws its ticket.  (A device-scope
+// release / acquire fence pair would order ordinary stores as well, but it writes back and invalidates the whole L2
+// of the XCD -- with a step's deltas in it that cost 8 us per build, more than the launch it saves.)  The pixel masks
+// are ordinary stores: nothing in the kernel reads another workgroup's.
+constexpr int TICKET_CAP = 4096;
+constexpr int TICKET_THREADS = 256;
+constexpr int TICKET_ITEMS = TICKET_CAP / TICKET_THREADS;      // consecutive flags per thread
+
+__device__ __forceinline__ void store_flag(uint32_t* flags, int tile, uint32_t f) {
+  __hip_atomic_store(flags + tile, f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// true in exactly one workgroup of the grid: the one whose ticket is the last
+__device__ __forceinline__ bool last_workgroup(int32_t* counts, int* s_last) {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");      // this thread's flag stores have completed
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const int t = __hip_atomic_fetch_add(&counts[MIE_CNT_TICKET], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const bool last = t == (int)gridDim.x - 1;
+    if (last) __hip_atomic_store(&counts[MIE_CNT_TICKET], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // all drawn
+    *s_last = last ? 1 : 0;
+  }
+  __syncthreads();
+  return *s_last != 0;
+}
+
+// the two lists of a set of at most TICKET_CAP tiles, by the first TICKET_THREADS threads of one workgroup (all of its
+// threads call)
+__device__ void compact_by_one(const BuildArgs& a, int* s_w) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  uint32_t f[TICKET_ITEMS];
+  int na = 0, ns = 0;
+#pragma unroll
+  for (int j = 0; j < TICKET_ITEMS; ++j) {
+    const int t = tid * TICKET_ITEMS + j;
+    f[j] = (tid < TICKET_THREADS && t < a.cap) ? __hip_atomic_load(a.flags + t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+    na += (int)(f[j] & 1u);
+    ns += (int)((f[j] & 3u) == 2u);
+  }
+  // exclusive prefix over the threads: inside the wave by shuffles, wave totals through LDS
+  int ia = na, is = ns;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int ua = __shfl_up(ia, o), us = __shfl_up(is, o);
+    if (lane >= o) ia += ua, is += us;
+  }
+  if (lane == 63 && wave < TICKET_THREADS / 64) s_w[wave] = ia, s_w[4 + wave] = is;
+  __syncthreads();
+  if (tid >= TICKET_THREADS) return;      // a wider workgroup: its other waves only meet the barrier
+  int pa = ia - na, ps = is - ns, ta = 0, tst = 0;
+#pragma unroll
+  for (int wv = 0; wv < TICKET_THREADS / 64; ++wv) {
+    if (wv < wave) pa += s_w[wv], ps += s_w[4 + wv];
+    ta += s_w[wv];
+    tst += s_w[4 + wv];
+  }
+#pragma unroll
+  for (int j = 0; j < TICKET_ITEMS; ++j) {
+    const int t = tid * TICKET_ITEMS + j;
+    if (f[j] & 1u) a.tiles[pa++] = t;
+    if ((f[j] & 3u) == 2u) a.stale[ps++] = t;
+  }
+  if (tid == 0) {
+    a.counts[MIE_CNT_ACTIVE] = ta;
+    a.counts[MIE_CNT_STALE] = tst;
+  }
+}
+
+// k_mask_footprint + k_compact_tiles for sets of up to TICKET_CAP tiles
+__global__ __launch_bounds__(TICKET_THREADS) void k_mask_footprint_lists(BuildArgs a) {
+  __shared__ int s_w[8];
+  __shared__ int s_last;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = blockIdx.x * 4 + wave;
+  if (tile < a.cap) {
+    const uint32_t old = a.flags[tile];
+    const bool any = tile_footprint(a, tile, lane);
+    if (lane == 0) store_flag(a.flags, tile, next_flag(old, any));
+  }
+  if (last_workgroup(a.counts, &s_last)) compact_by_one(a, s_w);
+}
+
+// ---- threshold mask + footprint (+ lists) in one launch -------------------------------------------
+// What mie_mask_from_delta followed by mie_build_mask_tiles (conv footprint) leave, for the thresholded masks of
+// the lossy networks: one workgroup per output tile tests the input pixels of its tile's windows against the
+// threshold itself, straight from the delta, keeps the bits in LDS, writes the bytes of the input pixels it owns (the
+// 8s x 8s block under its tile; the last row / column of tiles owns through the plane's edge) and forms the footprint
+// from LDS.  Pixels in the halo of a window are tested by up to four workgroups; a delta plane of these networks is
+// at most a few MB and the launch is bound by latency -- so the test is a flat loop over (pixel, 4-channel group)
+// pairs with eight loads in flight per thread and no exchange between lanes (a hit sets the pixel's byte in LDS).
+struct ThrArgs {
+  BuildArgs b;          // b.in is unused (the mask comes from delta); b.in2 as in mie_build_mask_tiles
+  const void* delta;
+  uint8_t* thr_mask;    // [n, h_in, w_in]: the thresholded mask, as mie_mask_from_delta writes it
+  int c;
+  int vec_shift;        // log2(c / 4) when c / 4 is a power of two, else -1
+  float thr;
+  int lists;            // 1: the last workgroup ranks the lists
+};
+constexpr int THR_EDGE = 24;      // largest region edge: 7 * s + k (+ the rows no window reaches)
+constexpr int THR_UNROLL = 8;
+constexpr int TICKET_MAX_WGS = 128;      // more workgroups than this queue up at the ticket counter: two launches then
+
+template <typename T>
+__global__ __launch_bounds__(1024) void k_build_thresholded(ThrArgs a) {
+  __shared__ uint8_t s_in[THR_EDGE * THR_EDGE];
+  __shared__ int s_w[8];
+  __shared__ int s_last;
+  const BuildArgs& b = a.b;
+  const int tid = threadIdx.x, nthr = blockDim.x, lane = tid & 63;
+  const int tile = blockIdx.x;                    // the grid is one workgroup per tile
+  const int tx = tile % b.tiles_x, t2 = tile / b.tiles_x, ty = t2 % b.tiles_y, n = t2 / b.tiles_y;
+  uint32_t old = 0;
+  if (tid == 0) old = b.flags[tile];
+  const int r0 = ty * MIE_TILE * b.s - b.p, c0 = tx * MIE_TILE * b.s - b.p;
+  const int own_r0 = ty * MIE_TILE * b.s, own_c0 = tx * MIE_TILE * b.s;
+  const int own_r1 = (ty == b.tiles_y - 1) ? b.h_in : own_r0 + MIE_TILE * b.s;
+  const int own_c1 = (tx == b.tiles_x - 1) ? b.w_in : own_c0 + MIE_TILE * b.s;
+  const int win = 7 * b.s + b.k;
+  const int rows = max(r0 + win, own_r1) - r0, cols = max(c0 + win, own_c1) - c0;
+  const int npx = rows * cols;
+  const unsigned col_magic = (65536u + (unsigned)cols - 1u) / (unsigned)cols;      // p / cols for p < 576, cols <= 24
+  const T* plane = static_cast<const T*>(a.delta) + (long long)n * b.h_in * b.w_in * a.c;
+  for (int i = tid; i < npx; i += nthr) s_in[i] = 0;
+  __syncthreads();
+  if ((a.c & 3) == 0) {
+    const int nvec = a.c >> 2, total = npx * nvec;
+    for (int base = tid; base < total; base += THR_UNROLL * nthr) {
+      float4 v[THR_UNROLL];
+      int pp[THR_UNROLL];
+#pragma unroll
+      for (int u = 0; u < THR_UNROLL; ++u) {
+        const int idx = base + u * nthr;
+        const int p = a.vec_shift >= 0 ? (idx >> a.vec_shift) : idx / nvec;
+        const int q = idx - p * nvec;
+        const int ry = (int)(((unsigned)p * col_magic) >> 16), rx = p - ry * cols;
+        const int iy = r0 + ry, ix = c0 + rx;
+        const bool inside = idx < total && iy >= 0 && iy < b.h_in && ix >= 0 && ix < b.w_in;
+        pp[u] = inside ? p : -1;
+        // every load goes out, from a clamped address: eight independent loads, no branch between them
+        v[u] = mie_ld4(plane + (inside ? ((long long)iy * b.w_in + ix) * a.c + 4 * q : 0ll), 0);
+      }
+#pragma unroll
+      for (int u = 0; u < THR_UNROLL; ++u) {
+        const bool hit = (fabsf(v[u].x) > a.thr) | (fabsf(v[u].y) > a.thr) | (fabsf(v[u].z) > a.thr) | (fabsf(v[u].w) > a.thr);
+        if (pp[u] >= 0 && hit) s_in[pp[u]] = 1;
+      }
+    }
+  } else {      // channel counts that are no multiple of 4 (a network's input): one thread per pixel
+    for (int p = tid; p < npx; p += nthr) {
+      const int ry = (int)(((unsigned)p * col_magic) >> 16), rx = p - ry * cols;
+      const int iy = r0 + ry, ix = c0 + rx;
+      if (iy < 0 || iy >= b.h_in || ix < 0 || ix >= b.w_in) continue;
+      const T* row = plane + ((long long)iy * b.w_in + ix) * a.c;
+      int any = 0;
+      for (int i = 0; i < a.c; ++i) any |= (fabsf(mie_ld(row, i)) > a.thr);
+      if (any) s_in[p] = 1;
+    }
+  }
+  __syncthreads();
+  for (int p = tid; p < npx; p += nthr) {
+    const int ry = (int)(((unsigned)p * col_magic) >> 16), rx = p - ry * cols;
+    const int iy = r0 + ry, ix = c0 + rx;
+    if (iy >= own_r0 && iy < min(own_r1, b.h_in) && ix >= own_c0 && ix < min(own_c1, b.w_in))
+      a.thr_mask[((long long)n * b.h_in + iy) * b.w_in + ix] = s_in[p];
+  }
+  if (tid < 64) {
+    const int py = lane >> 3, px = lane & 7;
+    const int oy = ty * MIE_TILE + py, ox = tx * MIE_TILE + px;
+    int bit = 0;
+    if (oy < b.h_out && ox < b.w_out) {
+      for (int ky = 0; ky < b.k; ++ky)
+        for (int kx = 0; kx < b.k; ++kx) bit |= s_in[(py * b.s + ky) * cols + px * b.s + kx];
+      if (b.in2) {
+        const uint8_t* m2 = b.in2 + (long long)n * b.h_in * b.w_in;
+        for (int ky = 0; ky < b.k; ++ky) {
+          const int iy = oy * b.s - b.p + ky;
+          if (iy < 0 || iy >= b.h_in) continue;
+          for (int kx = 0; kx < b.k; ++kx) {
+            const int ix = ox * b.s - b.p + kx;
+            if (ix >= 0 && ix < b.w_in) bit |= m2[iy * b.w_in + ix];
+          }
+        }
+      }
+      bit = bit != 0;
+      b.out[((long long)n * b.h_out + oy) * b.w_out + ox] = (uint8_t)bit;
+    }
+    const bool any = __ballot(bit != 0) != 0ull;
+    if (lane == 0) {
+      if (a.lists) store_flag(b.flags, tile, next_flag(old, any));
+      else b.flags[tile] = next_flag(old, any);
+    }
+  }
+  if (a.lists && last_workgroup(b.counts, &s_last)) compact_by_one(b, s_w);
+}
+
 extern "C" int mie_build_mask_tiles(const uint8_t* in_mask, const uint8_t* in_mask2,
                                     int h_in, int w_in, int foot, int k, int stride,
                                     int pad, const mie_tileset* out, void* stream) {
@@ -389,12 +590,71 @@ extern "C" int mie_build_mask_tiles(const uint8_t* in_mask, const uint8_t* in_ma
     return mie_check_launch("mie_build_mask_tiles");
   }
   const unsigned blocks = (unsigned)mie_div_up(a.cap, 4);
+  static const int ticket_wgs = [] { const char* e = getenv("MIE_BUILD_TICKET"); return e ? atoi(e) : TICKET_MAX_WGS; }();   // tuning knob
+  if ((int)blocks <= ticket_wgs && a.cap <= TICKET_CAP) {
+    hipLaunchKernelGGL(k_mask_footprint_lists, dim3(blocks), dim3(TICKET_THREADS), 0, (hipStream_t)stream, a);
+    return mie_check_launch("mie_build_mask_tiles");
+  }
   hipLaunchKernelGGL(k_mask_footprint, dim3(blocks), dim3(256), 0, (hipStream_t)stream, a);
   rc = mie_check_launch("mie_build_mask_tiles");
   if (rc != MIE_OK) return rc;
   hipLaunchKernelGGL(k_compact_tiles, dim3((unsigned)mie_div_up(a.cap, COMPACT_CHUNK)), dim3(COMPACT_THREADS), 0,
                      (hipStream_t)stream, a);
   return mie_check_launch("mie_build_mask_tiles");
+}
+
+extern "C" int mie_build_mask_tiles_thresholded(const void* delta, int c, int dtype, float threshold, uint8_t* thr_mask,
+                                                const uint8_t* in_mask2, int h_in, int w_in, int k, int stride, int pad,
+                                                const mie_tileset* out, void* stream) {
+  const char* who = "mie_build_mask_tiles_thresholded";
+  mie_clear_error();
+  int rc = mie_check_tileset(out, who);
+  if (rc != MIE_OK) return rc;
+  MIE_REQUIRE(delta && thr_mask, MIE_ERR_INVALID_ARG, "%s: NULL pointer", who);
+  MIE_REQUIRE(dtype == MIE_DTYPE_F32 || dtype == MIE_DTYPE_BF16, MIE_ERR_UNSUPPORTED, "%s: unknown delta dtype %d", who, dtype);
+  MIE_REQUIRE(h_in > 0 && w_in > 0 && c > 0, MIE_ERR_INVALID_ARG, "%s: sizes must be positive (h=%d w=%d c=%d)", who, h_in, w_in, c);
+  MIE_REQUIRE(threshold >= 0.f, MIE_ERR_INVALID_ARG, "%s: threshold < 0", who);
+  MIE_REQUIRE(mie_aligned(delta, 16), MIE_ERR_INVALID_ARG, "%s: delta must be 16-byte aligned", who);
+  MIE_REQUIRE((long long)out->n * h_in * w_in < 0x7fffffffLL, MIE_ERR_CAPACITY, "%s: more than 2^31 input pixels", who);
+  MIE_REQUIRE(k >= 1 && stride >= 1 && pad >= 0, MIE_ERR_UNSUPPORTED, "%s: conv footprint k=%d stride=%d pad=%d", who, k, stride, pad);
+  // a workgroup owns the input block under its tile and must find it inside its tile's windows
+  MIE_REQUIRE(stride + pad <= k && 7 * stride + k + (stride - 1 - pad > 0 ? stride - 1 - pad : 0) <= THR_EDGE,
+              MIE_ERR_UNSUPPORTED, "%s: no one-launch form for k=%d stride=%d pad=%d (mie_mask_from_delta + mie_build_mask_tiles take it)",
+              who, k, stride, pad);
+  const int ho = (h_in + 2 * pad - k) / stride + 1, wo = (w_in + 2 * pad - k) / stride + 1;
+  MIE_REQUIRE(h_in + 2 * pad >= k && w_in + 2 * pad >= k && ho == out->h && wo == out->w, MIE_ERR_INVALID_ARG,
+              "%s: conv output of (%d,%d) k=%d s=%d p=%d is (%d,%d), tile set is (%d,%d)", who, h_in, w_in, k, stride, pad,
+              ho, wo, out->h, out->w);
+  MIE_REQUIRE(thr_mask != out->pixmask && in_mask2 != out->pixmask && in_mask2 != thr_mask, MIE_ERR_INVALID_ARG,
+              "%s: thr_mask, in_mask2 and out->pixmask must be three buffers", who);
+  ThrArgs a;
+  memset(&a, 0, sizeof(a));
+  BuildArgs& b = a.b;
+  b.in = nullptr; b.in2 = in_mask2;
+  b.n = out->n; b.h_in = h_in; b.w_in = w_in;
+  b.foot = MIE_FOOT_CONV; b.k = k; b.s = stride; b.p = pad;
+  b.out = out->pixmask; b.h_out = out->h; b.w_out = out->w;
+  b.tiles_y = mie_div_up(out->h, MIE_TILE); b.tiles_x = mie_div_up(out->w, MIE_TILE);
+  b.cap = mie_tile_capacity(out->n, out->h, out->w);
+  b.tiles = out->tiles; b.stale = out->stale; b.counts = out->counts; b.flags = out->flags;
+  a.delta = delta; a.thr_mask = thr_mask; a.c = c; a.thr = threshold;
+  a.vec_shift = -1;
+  if ((c & 3) == 0 && ((c >> 2) & ((c >> 2) - 1)) == 0)
+    for (a.vec_shift = 0; (1 << a.vec_shift) < (c >> 2); ++a.vec_shift) {}
+  static const int ticket_wgs = [] { const char* e = getenv("MIE_BUILD_TICKET"); return e ? atoi(e) : TICKET_MAX_WGS; }();   // tuning knob
+  a.lists = b.cap <= ticket_wgs && b.cap <= TICKET_CAP ? 1 : 0;
+  // deep planes of few tiles (at most two workgroups per CU): more threads per tile, so that a thread's loads go out in
+  // one round
+  const int threads = (b.cap <= 512 && (long long)(7 * stride + k) * (7 * stride + k) * (c / 4) > THR_UNROLL * 256) ? 1024 : 256;
+  if (dtype == MIE_DTYPE_BF16)
+    hipLaunchKernelGGL(k_build_thresholded<mie_bf16>, dim3((unsigned)b.cap), dim3(threads), 0, (hipStream_t)stream, a);
+  else
+    hipLaunchKernelGGL(k_build_thresholded<float>, dim3((unsigned)b.cap), dim3(threads), 0, (hipStream_t)stream, a);
+  rc = mie_check_launch(who);
+  if (rc != MIE_OK || a.lists) return rc;
+  hipLaunchKernelGGL(k_compact_tiles, dim3((unsigned)mie_div_up(b.cap, COMPACT_CHUNK)), dim3(COMPACT_THREADS), 0,
+                     (hipStream_t)stream, b);
+  return mie_check_launch(who);
 }
 
 // ---- every tile set of a network in two launches ------------------------------------------------

@@ -491,7 +491,7 @@ class nnConvIncr(nn.Conv2d, _ConvIncrMixin):
         if self.in_threshold is not None:
             x = ops.as_nhwc(x_incr[0])
             n, _, h, w = x.shape
-            pix = ops.mask_from_delta(x, float(self.in_threshold), self._pix_buf("thr_in", n, h, w, x.device))
+            pix = ops.threshold_mask_lazy(x, float(self.in_threshold), self._pix_buf("thr_in", n, h, w, x.device))
             x_incr = [x, pix]
         return x_incr
 

@@ -420,6 +420,8 @@ def pix_ptr(m, n, h, w, name):
         raise ValueError("%s must be a contiguous uint8 (%d,1,%d,%d) mask, got %s %s"
                          % (name, n, h, w, tuple(t.shape), t.dtype))
     _require_gpu(t, name)
+    if _pending_thr:
+        _force_threshold_mask(t)
     return t.data_ptr()
 
 
@@ -456,8 +458,53 @@ def mask_from_delta(delta: torch.Tensor, threshold: float, out: torch.Tensor):
     return out
 
 
+# Thresholded masks whose kernel has not been launched yet: data pointer of the mask buffer -> (delta, threshold,
+# buffer).  threshold_mask_lazy leaves the launch to the first reader of the buffer.  If that reader is the build of a
+# conv's tile set, threshold test, footprint and lists go out as one launch (mie_build_mask_tiles_thresholded); any
+# other reader (pix_ptr) launches mie_mask_from_delta first.
+_pending_thr = {}
+fused_threshold_build = os.environ.get("MIE_FUSED_THRESHOLD_BUILD", "1") != "0"      # tuning knob, read once
+
+
+def threshold_mask_lazy(delta: torch.Tensor, threshold: float, out: torch.Tensor):
+    """mask_from_delta(delta, threshold, out) whose launch waits for the first reader of `out` (delta must keep its
+    values until then: call this right before the op that reads the mask)."""
+    if not fused_threshold_build:
+        return mask_from_delta(delta, threshold, out)
+    _mark_pix(out, from_values=True)
+    _pending_thr[out.data_ptr()] = (delta, float(threshold), out)
+    return out
+
+
+def _force_threshold_mask(t: torch.Tensor):
+    ent = _pending_thr.pop(t.data_ptr(), None)
+    if ent is not None:
+        mask_from_delta(*ent)
+
+
+def _thresholded_build(in_mask, in_mask2, n, h_in, w_in, foot, k, stride, pad, out: TileMask) -> bool:
+    """The one-launch form of a pending threshold mask + the build that reads it, where the library has one."""
+    t = in_mask.pixmask if isinstance(in_mask, TileMask) else in_mask
+    ent = None if t is None else _pending_thr.get(t.data_ptr())
+    if ent is None:
+        return False
+    delta, thr, buf = ent
+    if (foot != _lib.FOOT_CONV or stride + pad > k or 7 * stride + k + max(0, stride - 1 - pad) > 24
+            or _phase is not None or (_planner is not None and _planner[1] == out.device)
+            or tuple(delta.shape) != (n, delta.shape[1], h_in, w_in)):
+        return False
+    del _pending_thr[t.data_ptr()]
+    p2 = pix_ptr(in_mask2, n, h_in, w_in, "in_mask2")
+    check(lib().mie_build_mask_tiles_thresholded(
+        nhwc_ptr(delta, "delta", dtype=delta.dtype), delta.shape[1], delta_dtype(delta), thr,
+        buf.data_ptr(), p2, h_in, w_in, k, stride, pad, out.ref, _stream(delta)))
+    return True
+
+
 def build_mask_tiles(in_mask, in_mask2, n, h_in, w_in, foot, k, stride, pad, out: TileMask):
     """in_mask / in_mask2: None | TileMask | uint8 (N,1,H,W)."""
+    if _pending_thr and _thresholded_build(in_mask, in_mask2, n, h_in, w_in, foot, k, stride, pad, out):
+        return out
     p1 = pix_ptr(in_mask, n, h_in, w_in, "in_mask")
     p2 = pix_ptr(in_mask2, n, h_in, w_in, "in_mask2")
     if p1 is None and p2 is not None:   # "all active" OR anything = all active

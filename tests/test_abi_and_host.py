@@ -213,6 +213,19 @@ def test_newer_entry_points_reject_bad_arguments(mie_lib):
     assert gates(p + 2048, 4096) == -1 and "alias" in err()
     assert gates(p + 6000 + 4, 64) == -1 and "workspace" in err()
 
+    # threshold mask + build in one launch: footprints it has no form for, aliasing, sizes
+    half, keep_h = _fake_tileset(h=8, w=8)
+    thr = lambda k=3, s=2, pad=1, mask=q, m2=None, t=0.1, c=4, dtype=F32, ts=half: mie_lib.mie_build_mask_tiles_thresholded(
+        p, c, dtype, t, mask, m2, 16, 16, k, s, pad, ctypes.byref(ts), None)
+    assert thr(k=1, s=2, pad=0) == -2 and "no one-launch form" in err()
+    assert thr(k=11, s=2, pad=5) == -2
+    assert thr(mask=None) == -1 and "NULL" in err()
+    assert thr(t=-0.5) == -1 and "threshold" in err()
+    assert thr(c=0) == -1 and thr(dtype=2) == -2
+    assert thr(mask=half.pixmask) == -1 and "three buffers" in err()
+    assert thr(m2=q) == -1 and "three buffers" in err()
+    assert thr(k=3, s=1, pad=1) == -1 and "tile set is" in err()
+
     # bf16 event frame: the rounded frame is a buffer of its own
     ev = lambda out: mie_lib.mie_events_to_frame_bf16(None, 0, 0, 5, 8, 8, 0, 0, 0, 0, 1.0, 0.0, 0.0, -1.0, 0, p, out, q, None)
     assert ev(p + 4096) == -1 and "window length" in err()             # the base entry point's checks come first

@@ -58,6 +58,55 @@ def test_conv_footprint_tiles_and_stale(k, s, p, n, h, w, dens):
         prev = _check_tileset(ts, mo.footprint_conv(m, k, s, p), prev)
 
 
+@pytest.mark.parametrize("k,s,p", [(1, 1, 0), (3, 1, 1), (3, 2, 1), (5, 1, 2), (5, 2, 2), (7, 1, 3), (3, 1, 0), (5, 2, 1), (3, 1, 2)])
+@pytest.mark.parametrize("n,h,w,c,dt,second", [(1, 33, 44, 256, torch.float32, False), (2, 45, 61, 5, torch.float32, True),
+                                               (1, 132, 176, 64, torch.bfloat16, True), (4, 264, 352, 4, torch.float32, False),
+                                               (1, 66, 88, 24, torch.bfloat16, False), (3, 9, 70, 2, torch.bfloat16, True)])
+def test_threshold_mask_footprint_and_lists_in_one_launch(k, s, p, n, h, w, c, dt, second):
+    # mie_build_mask_tiles_thresholded against the numpy oracle (threshold mask, union, conv footprint, tile and stale
+    # lists) over three steps with fresh deltas: one lane per pixel (c not a multiple of 4) up to 16 lanes per pixel
+    # (c = 256), both element types, a second mask OR-ed in, planes whose last tiles are partial, windows with and
+    # without padding, 5808 tiles (lists by the separate ranking kernel) and fewer (ticket).  The thresholded input
+    # mask comes out as mie_mask_from_delta writes it.
+    thr = 0.05
+    ho, wo = mo.conv_out_size(h, w, k, s, p)
+    ts = TileMask(n, ho, wo, DEV)
+    thr_mask = torch.full((n, 1, h, w), 7, dtype=torch.uint8, device=DEV)
+    prev = np.zeros(0, np.int32)
+    for step in range(3):
+        g = torch.Generator().manual_seed(1000 * step + h + c + k)
+        d = torch.randn((n, c, h, w), generator=g) * (torch.rand((n, 1, h, w), generator=g) < [0.03, 0.0, 0.3][step])
+        d = d * (torch.rand((n, c, h, w), generator=g) < 0.5)              # most channels of an active pixel are zero
+        d[0, c - 1, h - 1, w - 1] = 0.051                                   # last channel of the last pixel, just above
+        d[0, 0, 0, 0] = 0.049                                               # just below
+        d = d.to(dt).float()
+        x = ops.as_nhwc(d.to(DEV).to(dt).contiguous(memory_format=torch.channels_last))
+        m2 = np.stack([blob_mask(h, w, 0.02, seed=77 * step + b) for b in range(n)]) if second else None
+        m2d = _to_dev_mask(m2) if second else None
+        _lib.check(_lib.lib().mie_build_mask_tiles_thresholded(
+            x.data_ptr(), c, ops.delta_dtype(x), thr, thr_mask.data_ptr(), None if m2d is None else m2d.data_ptr(),
+            h, w, k, s, p, ts.ref, torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        want_in = mo.pixel_mask(d.numpy(), thr)
+        assert np.array_equal(thr_mask[:, 0].cpu().numpy(), want_in), "step %d: thresholded input mask" % step
+        src = want_in | m2 if second else want_in
+        prev = _check_tileset(ts, mo.footprint_conv(src, k, s, p), prev)
+
+
+def test_thresholded_build_refuses_footprints_without_a_one_launch_form():
+    ts = TileMask(1, 8, 8, DEV)
+    x = torch.zeros((1, 16, 16, 4), device=DEV)
+    m = torch.zeros((1, 1, 16, 16), dtype=torch.uint8, device=DEV)
+    lib = _lib.lib()
+    st = torch.cuda.current_stream().cuda_stream
+    assert lib.mie_build_mask_tiles_thresholded(x.data_ptr(), 4, _lib.DTYPE_F32, 0.1, m.data_ptr(), None, 16, 16, 1, 2, 0, ts.ref, st) == -2
+    assert "no one-launch form" in lib.mie_last_error_string().decode()
+    assert lib.mie_build_mask_tiles_thresholded(x.data_ptr(), 4, _lib.DTYPE_F32, 0.1, ts.pixmask.data_ptr(), None, 16, 16, 3, 2, 1, ts.ref, st) == -1
+    assert lib.mie_build_mask_tiles_thresholded(x.data_ptr(), 4, _lib.DTYPE_F32, -1.0, m.data_ptr(), None, 16, 16, 3, 2, 1, ts.ref, st) == -1
+    assert lib.mie_build_mask_tiles_thresholded(x.data_ptr(), 4, _lib.DTYPE_F32, 0.1, m.data_ptr(), None, 16, 16, 3, 1, 1, ts.ref, st) == -1   # output size
+    torch.cuda.synchronize()
+
+
 def test_all_active_empty_and_union():
     n, h, w = 2, 30, 41
     ts = TileMask(n, h, w, DEV)

@@ -596,6 +596,52 @@ def test_value_dependent_masks_replay_from_a_graph(knob):
         assert min(max(t) for t in got_tiles) < cap
 
 
+def test_thresholded_network_with_one_launch_builds_equals_the_separate_launches():
+    # Threshold masks in front of every conv: with ops.fused_threshold_build the threshold test, the footprint and the
+    # tile lists of a conv go out as one launch (mie_build_mask_tiles_thresholded) instead of mie_mask_from_delta +
+    # mie_build_mask_tiles.  Same predictions bit for bit over six steps, same thresholded input masks and tile lists
+    # in every conv (the gates convs take a second mask, the decoders read up-sampled deltas, the head has 5 channels).
+    h, w, steps = 72, 104, 6
+    nets = []
+    for _ in range(2):
+        m = seed_module_(E2VIDRecurrentIncr(), seed=31).to(DEV).eval()
+        mm.set_input_threshold(m, 3e-3)
+        nets.append(m)
+    fused, plain = nets
+    x0 = torch.randn(1, 5, h, w, generator=torch.Generator().manual_seed(32)) * 0.5
+    deltas = [_cl(event_voxel_delta(1, 5, h, w, 0.03 + 0.02 * (i % 3), seed=4400 + i)[0]) for i in range(steps)]
+    keep = ops.fused_threshold_build
+    try:
+        with torch.no_grad():
+            for m in nets:
+                m.forward_refresh_reservoirs(_cl(x0), None)
+            for i, d in enumerate(deltas):
+                ops.fused_threshold_build = True
+                a = fused([d, None], None)[0][0].clone()
+                assert not ops._pending_thr, "a thresholded mask was never launched"
+                ops.fused_threshold_build = False
+                b = plain([d, None], None)[0][0].clone()
+                assert torch.equal(a, b), "step %d max|diff| = %.3e" % (i, (a - b).abs().max().item())
+                checked = 0
+                for (na, ma), (nb_, mb) in zip(fused.named_modules(), plain.named_modules()):
+                    if not isinstance(ma, mm.nnConvIncr):
+                        continue
+                    for key, ba in ma._ib().items():
+                        bb = mb._ib()[key]
+                        if key[0] == "p":                                   # pixel-mask buffers (thresholded inputs)
+                            assert torch.equal(ba, bb), "step %d %s %s" % (i, na, key)
+                            checked += 1
+                        elif key[0] == "t":                                 # tile sets
+                            assert torch.equal(ba.counts[:2], bb.counts[:2]), "step %d %s %s counts" % (i, na, key)
+                            n_act = int(ba.counts[0].item())
+                            assert torch.equal(ba.tiles[:n_act], bb.tiles[:n_act]) and torch.equal(ba.pixmask, bb.pixmask)
+                            checked += 1
+                assert checked >= 20
+    finally:
+        ops.fused_threshold_build = keep
+    torch.cuda.synchronize()
+
+
 @pytest.mark.parametrize("net", ["e2depth", "evflownet_transposed", "evflownet_upsample"])
 def test_planning_one_step_ahead_reproduces_plain_steps(net):
     # forward_pipelined: the tile sets of step t + 1 are planned on a second stream while step t computes, in a second
