@@ -69,6 +69,10 @@ def parse_args():
     ap.add_argument("--upconv-all", action="store_true",
                     help="take the one-kernel up-sampling conv for every decoder layer, whatever its size (for measurements)")
     ap.add_argument("--sync-masks", action="store_true", help="build tile sets on the compute stream (no planning stream)")
+    ap.add_argument("--in-threshold", type=float, default=None,
+                    help="run the network with a threshold mask in front of every conv (a lossy variant: pixels whose delta stays "
+                         "within the threshold are dropped for the step); value-dependent masks are built inline, so "
+                         "--sync-masks --no-plan-first --plan-ahead off are implied and the oracle check is skipped")
     ap.add_argument("--net", choices=["e2depth", "evflownet"], default="e2depth",
                     help="e2depth: the headline network (5 bins); evflownet: EVFlowNet-incr, 4 bins, moving-edge deltas "
                          "(use --height 256 --width 256)")
@@ -316,7 +320,14 @@ class NetBench:
 
     def new_model(self, seed=1, **kw):
         from maskedincrementeval_amd.synthetic import seed_module_
-        return seed_module_(self.make_net(**kw), seed=seed).to(self.dev).eval()
+        thr = getattr(self.args, "in_threshold", None)
+        if thr is not None:
+            kw.pop("async_masks", None), kw.pop("plan_first", None)
+        m = seed_module_(self.make_net(**kw), seed=seed).to(self.dev).eval()
+        if thr is not None:
+            from maskedincrementeval_amd.mask_incr_modules import set_input_threshold
+            set_input_threshold(m, thr)
+        return m
 
     def step_eager(self, m, i):
         self.static_in.copy_(self.deltas[i % self.n_inputs])
@@ -324,7 +335,7 @@ class NetBench:
 
     def plan_ahead_mode(self):
         a = self.args
-        return None if (a.plan_ahead == "off" or a.copy_input) else a.plan_ahead
+        return None if (a.plan_ahead == "off" or a.copy_input or getattr(a, "in_threshold", None) is not None) else a.plan_ahead
 
     def timed_run(self, m, tag, steps=None, repeats=None, check_against=None, graph=None, plan_ahead="default"):
         """Refresh, warm up, capture one step per resident input in a HIP graph, then time `steps` steps `repeats`
@@ -843,7 +854,7 @@ def main():
 
     # ---- CPU baseline: the oracle (torch-CPU restatement of the reference path) -----------------
     cpu = oracle_check = None
-    if args.cpu_steps > 0:
+    if args.cpu_steps > 0 and args.in_threshold is None:       # the oracle restates the exact network
         torch.set_num_threads(min(os.cpu_count() or 1, 16))
         if args.net == "evflownet":
             from oracle.evflownet_oracle import EVFlowNetOracle
@@ -919,8 +930,10 @@ def main():
                    "arithmetic": ARITHMETIC["bf16" if args.dtype == "bf16" else ops.f32_matmul],
                    "mask_planning": {"streams": "one step ahead: plan and compute halves are graphs of their own on two streams, events between the replays",
                                      "fork": "one step ahead: the next step's plan forked inside this step's graph",
-                                     None: ("inline" if args.sync_masks else ("second stream, builds first" if args.plan_first else "second stream"))
-                                     }[nb.plan_ahead_mode()]},
+                                     None: ("inline" if (args.sync_masks or args.in_threshold is not None) else
+                                            ("second stream, builds first" if args.plan_first else "second stream"))
+                                     }[nb.plan_ahead_mode()],
+                   **({"in_threshold": args.in_threshold} if args.in_threshold is not None else {})},
         "roofline": roofline,
         "cpu_baseline": cpu,
         "repeats_ms_per_step": repeats_ms,
