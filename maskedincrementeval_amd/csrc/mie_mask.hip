@@ -643,9 +643,10 @@ extern "C" int mie_build_mask_tiles_thresholded(const void* delta, int c, int dt
     for (a.vec_shift = 0; (1 << a.vec_shift) < (c >> 2); ++a.vec_shift) {}
   static const int ticket_wgs = [] { const char* e = getenv("MIE_BUILD_TICKET"); return e ? atoi(e) : TICKET_MAX_WGS; }();   // tuning knob
   a.lists = b.cap <= ticket_wgs && b.cap <= TICKET_CAP ? 1 : 0;
-  // deep planes of few tiles (at most two workgroups per CU): more threads per tile, so that a thread's loads go out in
-  // one round
-  const int threads = (b.cap <= 512 && (long long)(7 * stride + k) * (7 * stride + k) * (c / 4) > THR_UNROLL * 256) ? 1024 : 256;
+  // deep planes of few tiles (fewer workgroups than CUs): more threads per tile, so that a thread's loads go out in one
+  // round (thresholded 264x352 frame, cap 0 / 128 / 512 / 2048: 0.504 / 0.485 / 0.490 / 0.501 ms)
+  static const int wide_cap = [] { const char* e = getenv("MIE_THR_WIDE_CAP"); return e ? atoi(e) : 128; }();      // tuning knob
+  const int threads = (b.cap <= wide_cap && (long long)(7 * stride + k) * (7 * stride + k) * (c / 4) > THR_UNROLL * 256) ? 1024 : 256;
   if (dtype == MIE_DTYPE_BF16)
     hipLaunchKernelGGL(k_build_thresholded<mie_bf16>, dim3((unsigned)b.cap), dim3(threads), 0, (hipStream_t)stream, a);
   else
