@@ -442,15 +442,17 @@ class NetBench:
                     history.append(k % n_in)
                     k += 1
             step = replay if replay is not None else eager
-            per_repeat = []
+            per_repeat, enqueue = [], []
             for _ in range(repeats):
                 torch.cuda.synchronize()
                 t0 = time.perf_counter()
                 for _ in range(steps):
                     step(k)
                     k += 1
+                t_host = time.perf_counter()
                 torch.cuda.synchronize()
                 per_repeat.append((time.perf_counter() - t0) / steps)
+                enqueue.append((t_host - t0) / steps)
                 history.extend((k - steps + j) % n_in for j in range(steps))
             if check_against is not None:
                 # The timed configuration (graph replay, planning ahead) against the plain one: a second
@@ -475,9 +477,10 @@ class NetBench:
                 if not worst <= 1e-3:
                     raise SystemExit("bench: the timed configuration does not reproduce the plain one (%.3e)" % worst)
         sec = statistics.median(per_repeat)
-        log("%s: %.3f ms/step median of %d x %d steps (min %.3f, max %.3f; %s)"
+        log("%s: %.3f ms/step median of %d x %d steps (min %.3f, max %.3f; %s; the host has enqueued a step after %.3f ms)"
             % (tag, 1e3 * sec, repeats, steps, 1e3 * min(per_repeat), 1e3 * max(per_repeat),
-               "eager" if graphs is None else "HIP graph"))
+               "eager" if graphs is None else "HIP graph", 1e3 * statistics.median(enqueue)))
+        check["host_enqueue_ms_per_step"] = round(1e3 * statistics.median(enqueue), 4)
         return sec, [round(1e3 * t, 4) for t in per_repeat], check
 
     def layer_table(self, model, iters):
