@@ -648,7 +648,7 @@ def test_planning_one_step_ahead_reproduces_plain_steps(net):
     # generation of every tile set / delta buffer (ops.pipelined_step).  Against the same network stepped plainly, bit
     # for bit: 7 eager steps with fresh masks (stale tiles in both generations), a dense refresh with a plan still
     # pending (buffers are zeroed), then four resident inputs captured as four graphs -- each holds its step and the
-    # plan of the next input -- and replayed cyclically for three rounds, with the program's own work in between.
+    # plan of the next input -- and replayed cyclically three times over, with the program's own work in between.
     from maskedincrementeval_amd.evflownet_incr import MultiResUNetRecurrentIncr
     from maskedincrementeval_amd.synthetic import MovingEdges
     if net == "e2depth":
@@ -680,10 +680,10 @@ def test_planning_one_step_ahead_reproduces_plain_steps(net):
             piped(b, deltas[9], None, 1)
         refresh(a, x0), refresh(b, x0)
         res = deltas[8:12]
-        for i in range(4):                                              # eager round: allocates nothing new, primes the cycle
+        for i in range(4):                                              # eager cycle: allocates nothing new, primes the graphs
             want = plain(a, res[i]).clone()
             got = piped(b, res[i], res[(i + 1) % 4], i % 2).clone()
-            assert torch.equal(got, want), "round 0 step %d" % i
+            assert torch.equal(got, want), "first cycle, step %d" % i
         torch.cuda.synchronize()
         graphs, outs = [], []
         for i in range(4):
@@ -696,7 +696,7 @@ def test_planning_one_step_ahead_reproduces_plain_steps(net):
                 want = plain(a, res[i]).clone()
                 graphs[i].replay()
                 got = outs[i].clone()
-                assert torch.equal(got, want), "replay round %d step %d: %.3e" % (rnd, i, (got - want).abs().max().item())
+                assert torch.equal(got, want), "replay cycle %d step %d: %.3e" % (rnd, i, (got - want).abs().max().item())
     torch.cuda.synchronize()
     assert ops.buffer_parity == 0 and ops._phase is None
 
@@ -705,8 +705,8 @@ def test_planning_one_step_ahead_reproduces_plain_steps(net):
 def test_plan_and_compute_halves_on_two_streams_reproduce_plain_steps(net):
     # plan_ahead / forward_planned: the two halves of forward_pipelined with the caller's own streams and events.  The
     # planning stream waits for the event recorded after step k - 1 before it plans step k + 1 (same buffers as
-    # step k - 1), the compute stream waits for the event recorded after that plan.  Eager for a round, then each half
-    # captured as a graph of its own (no edge between streams inside any graph) and replayed for three rounds.
+    # step k - 1), the compute stream waits for the event recorded after that plan.  Eager for two cycles, then each half
+    # captured as a graph of its own (no edge between streams inside any graph) and replayed three times over.
     from maskedincrementeval_amd.evflownet_incr import MultiResUNetRecurrentIncr
     from maskedincrementeval_amd.synthetic import MovingEdges
     if net == "e2depth":
@@ -749,7 +749,7 @@ def test_plan_and_compute_halves_on_two_streams_reproduce_plain_steps(net):
                 want = plain(a, res[i]).clone()
                 got = out_of(step(i, lambda j: b.forward_planned([res[j], None], j % 2),
                                   lambda j: b.plan_ahead([res[j], None], j % 2))).clone()
-                assert torch.equal(got, want), "eager round %d step %d: %.3e" % (rnd, i, (got - want).abs().max().item())
+                assert torch.equal(got, want), "eager cycle %d step %d: %.3e" % (rnd, i, (got - want).abs().max().item())
         torch.cuda.synchronize()
         g_comp, g_plan, outs = [], [None] * 4, []
         for i in range(4):                                     # capture order = the order the state checks expect
@@ -766,6 +766,6 @@ def test_plan_and_compute_halves_on_two_streams_reproduce_plain_steps(net):
                 want = plain(a, res[i]).clone()
                 step(i, lambda j: g_comp[j].replay(), lambda j: g_plan[j].replay())
                 got = outs[i].clone()
-                assert torch.equal(got, want), "replay round %d step %d: %.3e" % (rnd, i, (got - want).abs().max().item())
+                assert torch.equal(got, want), "replay cycle %d step %d: %.3e" % (rnd, i, (got - want).abs().max().item())
     torch.cuda.synchronize()
     assert ops.buffer_parity == 0 and ops._phase is None
