@@ -55,10 +55,12 @@ def parse_args():
     ap.add_argument("--batch", type=int, default=1, help="independent event streams per step (8 with 480x640: the batched configuration)")
     ap.add_argument("--cpu-steps", type=int, default=400, help="incremental steps of the CPU baseline (0 = skip)")
     ap.add_argument("--no-graph", action="store_true", help="launch kernels eagerly instead of replaying a HIP graph")
-    ap.add_argument("--plan-ahead", choices=["streams", "fork", "off"], default="fork",
-                    help="plan the next step's tile sets beside this step's kernels: 'streams' = planning and compute "
-                         "halves as two graphs on two streams, ordered by events between the replays; 'fork' = one graph "
-                         "per step with the plan forked inside it; 'off' = every step plans its own tile sets first")
+    ap.add_argument("--plan-ahead", choices=["host", "streams", "fork", "off"], default="host",
+                    help="plan the next step's tile sets beside this step's kernels: 'host' = planning and compute halves "
+                         "as two graphs on two streams, the host keeps their order (it launches a half after the event it "
+                         "depends on has fired); 'streams' = the same with the order kept by event waits on the GPU; "
+                         "'fork' = one graph per step with the plan forked inside it; 'off' = every step plans its own "
+                         "tile sets first")
     ap.add_argument("--copy-input", action="store_true",
                     help="one captured graph and a device-to-device copy of the next delta into its input buffer before every "
                          "replay (default: one graph per resident input, no copy)")
@@ -341,8 +343,9 @@ class NetBench:
         """Refresh, warm up, capture one step per resident input in a HIP graph, then time `steps` steps `repeats`
         times.  The inputs are taken cyclically by one running step counter.  plan_ahead "fork": the graph of
         input i holds step i and, forked beside it, the plan of input i + 1's tile sets (forward_pipelined);
-        "streams": the two halves are graphs of their own, replayed on two streams with events between them
-        (forward_planned / plan_ahead); None: every step plans its own tile sets first (forward).
+        "streams" / "host": the two halves are graphs of their own, replayed on two streams (forward_planned /
+        plan_ahead, ops.LookaheadStepper), ordered by event waits on the GPU / by the host; None: every step plans
+        its own tile sets first (forward).
         Returns (median seconds per step, list of the repeats' ms/step, output-check dict)."""
         torch, args = self.torch, self.args
         steps = args.steps if steps is None else steps
@@ -353,22 +356,13 @@ class NetBench:
         assert n_in % 2 == 0
         history, check = [], {}
         k = 0                                                # running step counter: input k % n_in
-        plan_stream = torch.cuda.Stream() if pipe == "streams" else None
-        planned = [torch.cuda.Event(), torch.cuda.Event()]   # by parity: the tile sets of the step of that parity are built
-        computed = [torch.cuda.Event(), torch.cuda.Event()]  # by parity: the step of that parity has run
+        stepper = None
+        if pipe in ("streams", "host"):     # the two halves on two streams: orderings as GPU-side waits / kept by the host
+            stepper = self.ops.LookaheadStepper(self.dev, host_ordered=(pipe == "host"))
+            pipe = "streams"
 
         def two_streams(i, compute, plan):
-            """Step i on the current stream; beside it, on the planning stream, the plan of step i + 1 -- which
-            overwrites what step i - 1 read, so it waits for that step's event."""
-            cur, p = torch.cuda.current_stream(), i % 2
-            cur.wait_event(planned[p])
-            out = compute(i)
-            computed[p].record(cur)
-            with torch.cuda.stream(plan_stream):
-                plan_stream.wait_event(computed[1 - p])
-                plan((i + 1) % n_in)
-                planned[1 - p].record(plan_stream)
-            return out
+            return stepper.step(i, lambda: compute(i), lambda: plan((i + 1) % n_in))
 
         def eager(kk):
             i = kk % n_in
@@ -932,6 +926,7 @@ def main():
                    "f32_matmul": ops.f32_matmul if args.dtype == "f32" else None,
                    "arithmetic": ARITHMETIC["bf16" if args.dtype == "bf16" else ops.f32_matmul],
                    "mask_planning": {"streams": "one step ahead: plan and compute halves are graphs of their own on two streams, events between the replays",
+                                     "host": "one step ahead: plan and compute halves are graphs of their own on two streams, the host keeps their order (it waits for the plan's event before it launches the step, for the step before last before it launches the plan)",
                                      "fork": "one step ahead: the next step's plan forked inside this step's graph",
                                      None: ("inline" if (args.sync_masks or args.in_threshold is not None) else
                                             ("second stream, builds first" if args.plan_first else "second stream"))

@@ -701,12 +701,13 @@ def test_planning_one_step_ahead_reproduces_plain_steps(net):
     assert ops.buffer_parity == 0 and ops._phase is None
 
 
+@pytest.mark.parametrize("host_ordered", [True, False])
 @pytest.mark.parametrize("net", ["e2depth", "evflownet_transposed"])
-def test_plan_and_compute_halves_on_two_streams_reproduce_plain_steps(net):
-    # plan_ahead / forward_planned: the two halves of forward_pipelined with the caller's own streams and events.  The
-    # planning stream waits for the event recorded after step k - 1 before it plans step k + 1 (same buffers as
-    # step k - 1), the compute stream waits for the event recorded after that plan.  Eager for two cycles, then each half
-    # captured as a graph of its own (no edge between streams inside any graph) and replayed three times over.
+def test_plan_and_compute_halves_on_two_streams_reproduce_plain_steps(net, host_ordered):
+    # plan_ahead / forward_planned: the two halves of forward_pipelined on two streams (ops.LookaheadStepper).  The plan
+    # of step k + 1 follows the event recorded after step k - 1 (same buffers as step k - 1), step k + 1 the event
+    # recorded after that plan -- as waits on the GPU, or with the host waiting before it launches.  Eager for two cycles,
+    # then each half captured as a graph of its own (no edge between streams inside any graph) and replayed three times.
     from maskedincrementeval_amd.evflownet_incr import MultiResUNetRecurrentIncr
     from maskedincrementeval_amd.synthetic import MovingEdges
     if net == "e2depth":
@@ -726,20 +727,10 @@ def test_plan_and_compute_halves_on_two_streams_reproduce_plain_steps(net):
         res = [_cl(gen.step()[0]) for _ in range(4)]
     a, b = make(), make()
     x0 = _cl(torch.randn(1, c, h, w, generator=torch.Generator().manual_seed(35)) * 0.5)
-    cur, side = torch.cuda.current_stream(), torch.cuda.Stream()
-    planned = [torch.cuda.Event(), torch.cuda.Event()]        # by parity: the plan of the step of that parity is made
-    computed = [torch.cuda.Event(), torch.cuda.Event()]       # by parity: the step of that parity has run
+    stepper = ops.LookaheadStepper(DEV, host_ordered=host_ordered)
 
     def step(i, compute, plan):
-        p = i % 2
-        cur.wait_event(planned[p])
-        out = compute(i)
-        computed[p].record(cur)
-        with torch.cuda.stream(side):
-            side.wait_event(computed[1 - p])                  # step i - 1 read the buffers this plan overwrites
-            plan((i + 1) % 4)
-            planned[1 - p].record(side)
-        return out
+        return stepper.step(i, lambda: compute(i), lambda: plan((i + 1) % 4))
 
     with torch.no_grad():
         refresh(a, x0), refresh(b, x0)
