@@ -473,7 +473,7 @@ class NetBench:
         sec = statistics.median(per_repeat)
         log("%s: %.3f ms/step median of %d x %d steps (min %.3f, max %.3f; %s; the host has enqueued a step after %.3f ms)"
             % (tag, 1e3 * sec, repeats, steps, 1e3 * min(per_repeat), 1e3 * max(per_repeat),
-               "eager" if graphs is None else "HIP graph", 1e3 * statistics.median(enqueue)))
+               "eager" if replay is None else "HIP graph", 1e3 * statistics.median(enqueue)))
         check["host_enqueue_ms_per_step"] = round(1e3 * statistics.median(enqueue), 4)
         return sec, [round(1e3 * t, 4) for t in per_repeat], check
 
