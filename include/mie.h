@@ -147,8 +147,8 @@ int mie_mask_from_delta(const void* delta, int n, int h, int w, int c,
  * footprint (MIE_FOOT_CONV, k = 1, stride = 1, pad = 0); any other footprint
  * reads neighbouring bytes while they are written and is refused with
  * MIE_ERR_INVALID_ARG.
- * Sets of 33 to 4096 tiles are built in one launch: the workgroup that finishes last (a ticket in
- * out->counts[MIE_CNT_TICKET], zero between calls) ranks the lists.
+ * Sets of 33 to 512 tiles are built in one launch: the workgroup that finishes last (a ticket in
+ * out->counts[MIE_CNT_TICKET], zero between calls) ranks the lists; larger sets take a second launch for that.
  * Replaces: the mask argument of conv{1,3,5,7}x*_increment_ext
  * (ext/pointops/_C_ext/pointops/ops.cpp:27-48), which the reference kernel
  * never reads (ext_conv.cu:74-76 synthesises a fake one).
@@ -159,7 +159,8 @@ int mie_build_mask_tiles(const uint8_t* in_mask, const uint8_t* in_mask2,
 
 /*
  * mie_mask_from_delta(delta -> thr_mask) followed by mie_build_mask_tiles(thr_mask, in_mask2, conv footprint k /
- * stride / pad -> out) as ONE launch (two above 4096 tiles), for networks whose masks depend on values: a conv with
+ * stride / pad -> out) as ONE launch (two above 128 tiles: the lists then have a launch of their own), for networks whose
+ * masks depend on values: a conv with
  * a thresholded input mask otherwise pays three or four launches of 4-14 us each before it can start.  delta is
  * [out->n, h_in, w_in, c] of `dtype` (MIE_DTYPE_F32 / MIE_DTYPE_BF16), 16-byte aligned; thr_mask [out->n, h_in, w_in]
  * receives the thresholded input mask (a pixel is active when |delta| > threshold in any channel), which the conv
