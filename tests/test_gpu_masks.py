@@ -30,15 +30,23 @@ def _check_tileset(ts: TileMask, want_mask: np.ndarray, prev_tiles=None):
     return want_tiles
 
 
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("shape,c,thr", [((1, 264, 352), 5, 0.0), ((2, 37, 53), 3, 0.0),
-                                         ((1, 33, 44), 64, 1e-4), ((1, 16, 16), 1, 0.5)])
-def test_mask_from_delta(shape, c, thr):
+                                         ((1, 33, 44), 64, 1e-4), ((1, 16, 16), 1, 0.5),
+                                         ((3, 7, 9), 13, 0.0), ((1, 5, 13), 2, 0.5), ((2, 33, 41), 18, 0.0)])
+def test_mask_from_delta(shape, c, thr, dt):
+    # thread-per-pixel rows (multiples of 4 channels, many channels) and the contiguous-span form (few channels that
+    # are no multiple of 4), pixel counts that are no multiple of 64, a delta whose last 16-byte load would run past
+    # its end, one active channel per pixel
     n, h, w = shape
     g = torch.Generator().manual_seed(h * w + c)
     d = torch.randn((n, c, h, w), generator=g) * (torch.rand((n, 1, h, w), generator=g) < 0.07)
+    d = d * (torch.rand((n, c, h, w), generator=g) < 0.4)         # most channels of an active pixel are zero
     d[0, :, 0, 0] = 0.0
-    d[0, c - 1, h - 1, w - 1] = 2e-4 if thr < 1e-3 else 0.4     # only the last channel; straddles thr
-    x = d.to(DEV).contiguous(memory_format=torch.channels_last)
+    d[0, c - 1, h - 1, w - 1] = 2e-4 if thr < 1e-3 else 0.75    # only the last channel of the last pixel
+    d[0, 0, 0, 1] = 0.25                                          # below the larger threshold
+    d = d.to(dt).float()
+    x = d.to(dt).to(DEV).contiguous(memory_format=torch.channels_last)
     x = ops.as_nhwc(x)
     out = torch.zeros((n, 1, h, w), dtype=torch.uint8, device=DEV)
     ops.mask_from_delta(x, thr, out)
