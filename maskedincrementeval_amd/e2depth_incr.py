@@ -774,6 +774,7 @@ class E2VIDRecurrentIncr(nn.Module, _IncrBuffers):
         return ops.mask_from_delta(delta, self.mask_threshold, pix)
 
     def forward(self, event_tensor: Masked, prev_states):
+        ops.require_no_lookahead(self)
         delta = ops.as_nhwc(event_tensor[0])
         mask = _mask_of(event_tensor)
         if not self.async_masks and not self.plan_first:

@@ -604,6 +604,7 @@ class MultiResUNetRecurrentIncr(nn.Module, _IncrBuffers):
         return decoders
 
     def forward(self, x_incr):
+        ops.require_no_lookahead(self)
         delta = ops.as_nhwc(x_incr[0])
         mask = _mask_of(x_incr)
         if not self.async_masks and not self.plan_first:

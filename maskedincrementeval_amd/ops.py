@@ -313,6 +313,16 @@ class LookaheadStepper:
         return out
 
 
+def require_no_lookahead(net):
+    """Called by a network's plain forward: a step that was planned ahead must be run (forward_planned /
+    forward_pipelined) or dropped by a refresh first -- a plain step would rebuild tile sets of that plan without a
+    compute pass between the two builds, and their stale lists would no longer describe the delta buffers."""
+    state = net.__dict__.get("_pipe")
+    if state and any(v is not None for v in state.get("planned", {}).values()):
+        raise RuntimeError("a step of this network was planned ahead and has not run: run it (forward_planned / "
+                           "forward_pipelined) or refresh the reservoirs before stepping plainly")
+
+
 def drop_lookahead(net):
     """Called by a network's dense refresh: the sequence starts anew.  If a step was planned ahead and never run, its
     tile sets were built without a compute pass behind them, and the next build would no longer know which tiles of

@@ -675,9 +675,11 @@ def test_planning_one_step_ahead_reproduces_plain_steps(net):
             want = plain(a, deltas[i]).clone()
             got = piped(b, deltas[i], deltas[i + 1], i % 2).clone()     # (after step 6 the plan of deltas[7] stays pending)
             assert torch.equal(got, want), "eager step %d: %.3e" % (i, (got - want).abs().max().item())
-        # a step that is not the one announced is refused, loudly
+        # a step that is not the one announced is refused, loudly, and so is a plain step while a plan is pending
         with pytest.raises(RuntimeError, match="announced as next"):
             piped(b, deltas[9], None, 1)
+        with pytest.raises(RuntimeError, match="planned ahead and has not run"):
+            plain(b, deltas[7])
         refresh(a, x0), refresh(b, x0)
         res = deltas[8:12]
         for i in range(4):                                              # eager cycle: allocates nothing new, primes the graphs
