@@ -47,7 +47,7 @@ def canned_detail(n_layers=60, n_lossy=12):
                                     "the delta, as the reference executes it), torch-CPU fp32"),
         "repeats_ms_per_step": [0.573] * 10,
         "whole_frame": dict(algorithmic_mb=258.5, algorithmic_gflop=53.3, hbm_gbs=451.0, hbm_frac=0.0564,
-                            mfma_tflops=93.0, mfma_frac=0.2232, mfma_peak_tflops=416.7, sum_kernel_us=512.0),
+                            mfma_tflops=93.0, mfma_frac=0.2232, mfma_peak_tflops=416.7, sum_eager_launch_us=512.0),
         "f32_native_mfma": dict(ms_per_step=0.809, frames_per_s=1236.0),
         "dense_same_kernels_ms": 0.618, "speedup_vs_dense": 1.079,
         "density_sweep": {p: dict(ms_per_step=0.55, frames_per_s=1800.0) for p in ("0.01", "0.05", "0.20")},
