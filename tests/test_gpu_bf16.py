@@ -203,6 +203,46 @@ def test_e2depth_incr_bf16_batched_high_resolution():
     _run_e2depth_bf16(8, 240, 320, steps=2, density=0.01)
 
 
+@pytest.mark.parametrize("n,h,w", [(8, 120, 160), (8, 480, 640)])
+def test_batched_bf16_network_planned_one_step_ahead_reproduces_plain_steps(n, h, w):
+    # The batched bf16 network with the next step's tile sets planned beside the step (plan_ahead / forward_planned on
+    # two streams, the host keeping the order): eight samples, so the plan made ahead is the capped one
+    # (mie_build_mask_plan_wgs, 8 workgroups per sample), and at 480x640 the last decoder is the persistent kernel with
+    # the prediction in its epilogue.  Bit-equal to the same network stepped plainly, eager and from graphs.
+    make = lambda: seed_module_(E2VIDRecurrentIncr(), seed=31).to(DEV).eval()
+    a, b = make(), make()
+    x0 = torch.randn(n, 5, h, w, generator=torch.Generator().manual_seed(41)) * 0.5
+    res = [_dev(event_voxel_delta(n, 5, h, w, 0.01 + 0.02 * (i % 2), seed=6100 + i)[0]) for i in range(4)]
+    stepper = ops.LookaheadStepper(DEV)
+    step = lambda i, compute, plan: stepper.step(i, lambda: compute(i), lambda: plan((i + 1) % 4))
+    with torch.no_grad():
+        a.forward_refresh_reservoirs(_dev(x0), None), b.forward_refresh_reservoirs(_dev(x0), None)
+        torch.cuda.synchronize()
+        for i in range(4):
+            want = a([res[i], None], None)[0][0].clone()
+            got = step(i, lambda j: b.forward_planned([res[j], None], j % 2),
+                       lambda j: b.plan_ahead([res[j], None], j % 2))[0][0].clone()
+            assert got.dtype == BF and torch.equal(got, want), "eager step %d: %.3e" % (i, (got.float() - want.float()).abs().max().item())
+        torch.cuda.synchronize()
+        g_comp, g_plan, outs = [], [None] * 4, []
+        for i in range(4):
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                outs.append(b.forward_planned([res[i], None], i % 2)[0][0])
+            g_comp.append(g)
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                b.plan_ahead([res[(i + 1) % 4], None], (i + 1) % 2)
+            g_plan[(i + 1) % 4] = g
+        for cycle in range(2):
+            for i in range(4):
+                want = a([res[i], None], None)[0][0].clone()
+                step(i, lambda j: g_comp[j].replay(), lambda j: g_plan[j].replay())
+                got = outs[i].clone()
+                assert torch.equal(got, want), "replay %d.%d: %.3e" % (cycle, i, (got.float() - want.float()).abs().max().item())
+    torch.cuda.synchronize()
+
+
 @pytest.mark.parametrize("density", [0.01, 0.20])
 def test_batched_configuration_full_size_accumulation_identity(density):
     # 8 streams of 5 x 480 x 640, bf16 deltas and weights: too large for the CPU oracle in a test, so

@@ -704,7 +704,7 @@ def test_planning_one_step_ahead_reproduces_plain_steps(net):
 
 
 @pytest.mark.parametrize("host_ordered", [True, False])
-@pytest.mark.parametrize("net", ["e2depth", "evflownet_transposed"])
+@pytest.mark.parametrize("net", ["e2depth", "e2depth_264x352", "evflownet_transposed"])
 def test_plan_and_compute_halves_on_two_streams_reproduce_plain_steps(net, host_ordered):
     # plan_ahead / forward_planned: the two halves of forward_pipelined on two streams (ops.LookaheadStepper).  The plan
     # of step k + 1 follows the event recorded after step k - 1 (same buffers as step k - 1), step k + 1 the event
@@ -712,8 +712,8 @@ def test_plan_and_compute_halves_on_two_streams_reproduce_plain_steps(net, host_
     # then each half captured as a graph of its own (no edge between streams inside any graph) and replayed three times.
     from maskedincrementeval_amd.evflownet_incr import MultiResUNetRecurrentIncr
     from maskedincrementeval_amd.synthetic import MovingEdges
-    if net == "e2depth":
-        h, w, c = 72, 104, 5
+    if net.startswith("e2depth"):
+        h, w, c = (264, 352, 5) if net.endswith("264x352") else (72, 104, 5)      # (the headline frame size)
         make = lambda: seed_module_(E2VIDRecurrentIncr(), seed=31).to(DEV).eval()
         plain = lambda m, d: m([d, None], None)[0][0]
         out_of = lambda r: r[0][0]
